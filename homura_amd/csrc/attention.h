@@ -1,0 +1,18 @@
+// Internal launch interface of the GQA decode attention kernel, shared with the decode plan.
+#pragma once
+#include "hm_common.h"
+
+struct AttnArgs {
+    const float *q = nullptr;          // [B][H][hd]
+    const uint16_t *kcache = nullptr;  // [B][kvh][max_len][hd] bf16
+    const uint16_t *vcache = nullptr;
+    float *out = nullptr;              // [B][H*hd]
+    int B = 0, H = 0, kvh = 0, hd = 0, max_len = 0, kv_len = 0;
+    float scale = 1.f;
+    // Decode-plan mode: kv_len = state->pos + 1 is read on the device and the grid is sized
+    // for max_len with a fixed chunk (workgroups past the live range exit at once).
+    const DecodeState *state = nullptr;
+    int fixed_chunk = 0;
+};
+
+int gqa_decode_attn_launch(hm_ctx *ctx, const AttnArgs &a);

@@ -1,0 +1,410 @@
+// Weight-streaming matmul for batch-1 decode: f32 activations x bf16 weights, f32 accumulate.
+//
+// Two weight layouts are served:
+//   [N][K] ("stream layout", K contiguous): one wavefront owns whole output rows, every lane
+//       streams 16-byte pieces of the row, partial dot products are folded with a wavefront
+//       butterfly. No cross-workgroup reduction, fixed summation order.
+//   [K][N] (the layout the reference hands its kernels): lanes own adjacent output columns,
+//       K is split across the waves of a workgroup (LDS) and across workgroups (workspace +
+//       last-arriver fold in fixed order).
+// These are HBM-bandwidth kernels: algorithmic traffic is K*N*2 bytes of weights per call.
+#include "gemv_bf16.h"
+
+// ─────────────────────────── [N][K] stream layout ───────────────────────────
+
+namespace {
+
+constexpr int GEMV_THREADS = 256;
+constexpr int GEMV_WAVES = GEMV_THREADS / WAVE;
+
+// Stage the activation vector(s) in LDS, optionally applying
+//   residual add:  r = x + res          (reference src/hf/emitter.rs:787)
+//   RMSNorm:       (r * rsqrt(mean(r^2) + eps)) * w   (src/graph_builder/emit_linalg.rs:7-26)
+// Every workgroup performs the same arithmetic in the same order, so all of them see
+// bit-identical activations.
+template <int MT>
+__device__ __forceinline__ void stage_activations(float *xs, const float *__restrict__ x,
+                                                  const float *__restrict__ res,
+                                                  const float *__restrict__ norm_w, float eps,
+                                                  int K, float *__restrict__ resid_out,
+                                                  bool write_resid) {
+    __shared__ float red[GEMV_WAVES];
+    const int tid = threadIdx.x;
+    for (int m = 0; m < MT; m++) {
+        float ss = 0.f;
+        for (int k = tid; k < K; k += GEMV_THREADS) {
+            float v = x[(size_t)m * K + k];
+            if (res) v = v + res[(size_t)m * K + k];
+            xs[m * K + k] = v;
+            ss += v * v;
+        }
+        if (norm_w) {
+            ss = wave_sum(ss);
+            __syncthreads();
+            if ((tid & (WAVE - 1)) == 0) red[tid / WAVE] = ss;
+            __syncthreads();
+            float tot = 0.f;
+#pragma unroll
+            for (int w = 0; w < GEMV_WAVES; w++) tot += red[w];
+            float inv = 1.0f / sqrtf(tot / (float)K + eps);
+            for (int k = tid; k < K; k += GEMV_THREADS) {
+                float v = xs[m * K + k];
+                if (write_resid && resid_out) resid_out[(size_t)m * K + k] = v;
+                xs[m * K + k] = (v * inv) * norm_w[k];
+            }
+        } else if (write_resid && resid_out) {
+            for (int k = tid; k < K; k += GEMV_THREADS) resid_out[(size_t)m * K + k] = xs[m * K + k];
+        }
+    }
+    __syncthreads();
+}
+
+__device__ __forceinline__ float dot8(const u32x4 w, const float *xv, float acc) {
+    acc = fmaf(bf16_lo(w.x), xv[0], acc);
+    acc = fmaf(bf16_hi(w.x), xv[1], acc);
+    acc = fmaf(bf16_lo(w.y), xv[2], acc);
+    acc = fmaf(bf16_hi(w.y), xv[3], acc);
+    acc = fmaf(bf16_lo(w.z), xv[4], acc);
+    acc = fmaf(bf16_hi(w.z), xv[5], acc);
+    acc = fmaf(bf16_lo(w.w), xv[6], acc);
+    acc = fmaf(bf16_hi(w.w), xv[7], acc);
+    return acc;
+}
+
+// R rows per wavefront per step, MT activation rows.
+template <int R, int MT, int EPI>
+__global__ __launch_bounds__(GEMV_THREADS) void gemv_bf16_nk_kernel(GemvArgs a) {
+    extern __shared__ float xs[];  // [MT][K]
+    const int K = a.K, N = a.N;
+    stage_activations<MT>(xs, a.x, a.prologue_residual, a.norm_w, a.eps, K, a.resid_out,
+                          blockIdx.x == 0);
+
+    const int lane = threadIdx.x & (WAVE - 1);
+    const int wave = threadIdx.x / WAVE;
+    const int groups = (N + R - 1) / R;
+    const int nchunks = (K + 511) / 512;
+    const int gstride = gridDim.x * GEMV_WAVES;
+
+    float best_v = -INFINITY;
+    int best_i = -1;
+
+    for (int g = blockIdx.x * GEMV_WAVES + wave; g < groups; g += gstride) {
+        const int row0 = g * R;
+        float acc[R][MT];
+#pragma unroll
+        for (int r = 0; r < R; r++)
+#pragma unroll
+            for (int m = 0; m < MT; m++) acc[r][m] = 0.f;
+
+        const uint16_t *wrow[R];
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            int row = row0 + r < N ? row0 + r : N - 1;  // clamp: tail rows re-read a valid row
+            wrow[r] = a.w + (size_t)row * K;
+        }
+
+#pragma unroll 2
+        for (int c = 0; c < nchunks; c++) {
+            const int k = (c * WAVE + lane) * 8;
+            if (k < K) {
+                u32x4 wv[R];
+#pragma unroll
+                for (int r = 0; r < R; r++) wv[r] = ld128_stream(wrow[r] + k);
+#pragma unroll
+                for (int m = 0; m < MT; m++) {
+                    float xv[8];
+                    const f32x4 x0 = *reinterpret_cast<const f32x4 *>(xs + m * K + k);
+                    const f32x4 x1 = *reinterpret_cast<const f32x4 *>(xs + m * K + k + 4);
+                    xv[0] = x0.x; xv[1] = x0.y; xv[2] = x0.z; xv[3] = x0.w;
+                    xv[4] = x1.x; xv[5] = x1.y; xv[6] = x1.z; xv[7] = x1.w;
+#pragma unroll
+                    for (int r = 0; r < R; r++) acc[r][m] = dot8(wv[r], xv, acc[r][m]);
+                }
+            }
+        }
+
+#pragma unroll
+        for (int r = 0; r < R; r++)
+#pragma unroll
+            for (int m = 0; m < MT; m++) acc[r][m] = wave_sum(acc[r][m]);
+
+        if (EPI == GEMV_EPI_SILU_MUL_PAIRS) {
+            // rows come in (gate_i, up_i) pairs; output index = row / 2
+            // (reference src/hf/emitter.rs:794-799: silu(gate) * up).
+#pragma unroll
+            for (int r = 0; r < R; r += 2) {
+                const int row = row0 + r;
+                if (lane == r && row < N) {
+#pragma unroll
+                    for (int m = 0; m < MT; m++) {
+                        float gte = acc[r][m], up = acc[r + 1][m];
+                        float s = gte / (1.0f + expf(-gte));
+                        a.out[(size_t)m * (N / 2) + row / 2] = s * up;
+                    }
+                }
+            }
+        } else {
+#pragma unroll
+            for (int r = 0; r < R; r++) {
+                const int row = row0 + r;
+                if (lane == r && row < N) {
+#pragma unroll
+                    for (int m = 0; m < MT; m++) {
+                        float v = acc[r][m];
+                        if (EPI == GEMV_EPI_RESIDUAL) v = a.epilogue_residual[(size_t)m * N + row] + v;
+                        a.out[(size_t)m * N + row] = v;
+                    }
+                }
+            }
+            if (EPI == GEMV_EPI_ARGMAX) {
+                // running (max, last index) over this wavefront's rows (ascending); m == 0 only.
+                // Of equal maxima the later row wins (Rust Iterator::max_by, reference
+                // src/generate.rs:735-742). NaN logits are not ordered here.
+#pragma unroll
+                for (int r = 0; r < R; r++) {
+                    const int row = row0 + r;
+                    const float v = acc[r][0];
+                    if (row < N && (best_i < 0 || v >= best_v)) {
+                        best_v = v;
+                        best_i = row;
+                    }
+                }
+            }
+        }
+    }
+
+    if (EPI == GEMV_EPI_ARGMAX) {
+        // all lanes of a wavefront hold the same (best_v, best_i); fold the waves of the
+        // workgroup through LDS and emit one candidate per workgroup.
+        __shared__ float wv[GEMV_WAVES];
+        __shared__ int wi[GEMV_WAVES];
+        if (lane == 0) {
+            wv[wave] = best_v;
+            wi[wave] = best_i;
+        }
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            float bv = -INFINITY;
+            int bi = -1;
+            for (int w = 0; w < GEMV_WAVES; w++) {
+                if (wi[w] < 0) continue;
+                if (bi < 0 || wv[w] > bv || (wv[w] == bv && wi[w] > bi)) {
+                    bv = wv[w];
+                    bi = wi[w];
+                }
+            }
+            a.argmax_val[blockIdx.x] = bv;
+            a.argmax_idx[blockIdx.x] = bi;
+        }
+    }
+}
+
+template <int R, int MT>
+int launch_nk(hm_ctx *ctx, const GemvArgs &a, int epi, int grid, size_t lds) {
+    dim3 g(grid), b(GEMV_THREADS);
+    switch (epi) {
+    case GEMV_EPI_NONE:
+        hipLaunchKernelGGL((gemv_bf16_nk_kernel<R, MT, GEMV_EPI_NONE>), g, b, lds, ctx->stream, a);
+        break;
+    case GEMV_EPI_RESIDUAL:
+        hipLaunchKernelGGL((gemv_bf16_nk_kernel<R, MT, GEMV_EPI_RESIDUAL>), g, b, lds, ctx->stream, a);
+        break;
+    case GEMV_EPI_SILU_MUL_PAIRS:
+        hipLaunchKernelGGL((gemv_bf16_nk_kernel<R, MT, GEMV_EPI_SILU_MUL_PAIRS>), g, b, lds, ctx->stream, a);
+        break;
+    case GEMV_EPI_ARGMAX:
+        hipLaunchKernelGGL((gemv_bf16_nk_kernel<R, MT, GEMV_EPI_ARGMAX>), g, b, lds, ctx->stream, a);
+        break;
+    default:
+        return hm_set_error(ctx, HM_ERR_INVALID, "gemv: unknown epilogue %d", epi);
+    }
+    HM_LAUNCH_CHECK(ctx);
+    return HM_OK;
+}
+
+}  // namespace
+
+int gemv_bf16_nk_grid(const hm_ctx *ctx, int N, int R) {
+    const int groups = (N + R - 1) / R;
+    int wgs = (groups + GEMV_WAVES - 1) / GEMV_WAVES;
+    const int cap = ctx->num_cus * 8;  // 8 workgroups (32 waves) per CU keep the loads deep
+    return wgs < cap ? wgs : cap;
+}
+
+int gemv_bf16_nk_launch(hm_ctx *ctx, GemvArgs a, int M, int epi) {
+    HM_REQUIRE(ctx, a.K > 0 && a.N > 0 && a.K % 8 == 0, "gemv_bf16_nk: K=%d must be a positive multiple of 8", a.K);
+    HM_REQUIRE(ctx, M >= 1 && M <= 8, "gemv_bf16_nk: M=%d outside 1..8", M);
+    HM_REQUIRE(ctx, (size_t)a.K * 4 <= 64 * 1024, "gemv_bf16_nk: K=%d too large for the LDS stage", a.K);
+    HM_REQUIRE(ctx, ((uintptr_t)a.w % 16) == 0 && ((uintptr_t)a.x % 16) == 0, "gemv_bf16_nk: pointers must be 16-byte aligned");
+    if (epi == GEMV_EPI_SILU_MUL_PAIRS) HM_REQUIRE(ctx, a.N % 2 == 0, "gemv: paired epilogue needs even N");
+    if (epi == GEMV_EPI_ARGMAX) HM_REQUIRE(ctx, M == 1 && a.argmax_val && a.argmax_idx, "gemv: argmax epilogue needs M == 1 and candidate buffers");
+    const int out_n = epi == GEMV_EPI_SILU_MUL_PAIRS ? a.N / 2 : a.N;
+    int m0 = 0;
+    while (m0 < M) {
+        GemvArgs b = a;
+        b.x = a.x + (size_t)m0 * a.K;
+        if (a.prologue_residual) b.prologue_residual = a.prologue_residual + (size_t)m0 * a.K;
+        if (a.resid_out) b.resid_out = a.resid_out + (size_t)m0 * a.K;
+        if (a.epilogue_residual) b.epilogue_residual = a.epilogue_residual + (size_t)m0 * a.N;
+        b.out = a.out + (size_t)m0 * out_n;
+        int rc;
+        if (M - m0 >= 4 && (size_t)4 * a.K * 4 <= 64 * 1024) {
+            const int grid = gemv_bf16_nk_grid(ctx, a.N, 2);
+            rc = launch_nk<2, 4>(ctx, b, epi, grid, (size_t)4 * a.K * 4);
+            m0 += 4;
+        } else {
+            int grid = gemv_bf16_nk_grid(ctx, a.N, 4);
+            if (epi == GEMV_EPI_ARGMAX && grid > a.argmax_cap) grid = a.argmax_cap;
+            rc = launch_nk<4, 1>(ctx, b, epi, grid, (size_t)a.K * 4);
+            m0 += 1;
+        }
+        if (rc != HM_OK) return rc;
+    }
+    return HM_OK;
+}
+
+// ─────────────────────────── [K][N] reference layout ───────────────────────────
+
+namespace {
+
+constexpr int KN_COLS_PER_LANE = 4;                    // 8-byte loads
+constexpr int KN_STRIP = WAVE * KN_COLS_PER_LANE;      // 256 columns per workgroup
+
+// grid = (strips, ksplit). Each wave of the workgroup walks rows k = kbeg + wave, +4, ...
+// of the workgroup's K slice; partials are folded over the 4 waves in LDS, written to the
+// workspace, and the last workgroup to arrive for a strip folds the ksplit partials in
+// ascending order (deterministic) into out.
+__global__ __launch_bounds__(GEMV_THREADS) void gemv_bf16_kn_kernel(
+    const float *__restrict__ x, const uint16_t *__restrict__ w, float *__restrict__ out,
+    float *__restrict__ partial, unsigned int *__restrict__ counters, int K, int N, int kslice) {
+    __shared__ float red[GEMV_WAVES][KN_STRIP];
+    __shared__ bool is_last;
+    const int lane = threadIdx.x & (WAVE - 1);
+    const int wave = threadIdx.x / WAVE;
+    const int strip = blockIdx.x, ks = blockIdx.y, ksplit = gridDim.y;
+    const int col = strip * KN_STRIP + lane * KN_COLS_PER_LANE;
+    const int kbeg = ks * kslice;
+    const int kend = min(K, kbeg + kslice);
+
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+    if (col < N) {
+#pragma unroll 4
+        for (int k = kbeg + wave; k < kend; k += GEMV_WAVES) {
+            const u32x2 wv = __builtin_nontemporal_load(
+                reinterpret_cast<const u32x2 *>(w + (size_t)k * N + col));
+            const float xk = x[k];
+            acc[0] = fmaf(bf16_lo(wv.x), xk, acc[0]);
+            acc[1] = fmaf(bf16_hi(wv.x), xk, acc[1]);
+            acc[2] = fmaf(bf16_lo(wv.y), xk, acc[2]);
+            acc[3] = fmaf(bf16_hi(wv.y), xk, acc[3]);
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < 4; j++) red[wave][lane * 4 + j] = acc[j];
+    __syncthreads();
+    const int t = threadIdx.x;  // 256 threads <-> 256 columns
+    const int c = strip * KN_STRIP + t;
+    float s = (red[0][t] + red[1][t]) + (red[2][t] + red[3][t]);
+    if (ksplit == 1) {
+        if (c < N) out[c] = s;
+        return;
+    }
+    if (c < N) partial[(size_t)ks * N + c] = s;
+    __threadfence();
+    __syncthreads();
+    if (t == 0) {
+        unsigned int prev = atomicAdd(&counters[strip], 1u);
+        is_last = (prev == (unsigned int)(ksplit - 1));
+    }
+    __syncthreads();
+    if (!is_last) return;
+    __threadfence();
+    if (c < N) {
+        float tot = 0.f;
+        for (int j = 0; j < ksplit; j++) tot += __builtin_nontemporal_load(&partial[(size_t)j * N + c]);
+        out[c] = tot;
+    }
+    if (t == 0) counters[strip] = 0u;  // leave the counter ready for the next call
+}
+
+// [K][N] -> [N][K] through a 64x64 LDS tile (both sides coalesced).
+// Output row n lands at dst row n * row_mult + row_off (1, 0 = plain transpose; 2, 0 / 2, 1
+// interleave two matrices row by row).
+__global__ __launch_bounds__(256) void pack_kn_to_nk_kernel(const uint16_t *__restrict__ src,
+                                                            uint16_t *__restrict__ dst, int K,
+                                                            int N, int row_mult, int row_off) {
+    __shared__ uint16_t tile[64][66];
+    const int n0 = blockIdx.x * 64, k0 = blockIdx.y * 64;
+    const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+    for (int i = ty; i < 64; i += 4) {
+        int k = k0 + i, n = n0 + tx;
+        tile[i][tx] = (k < K && n < N) ? src[(size_t)k * N + n] : (uint16_t)0;
+    }
+    __syncthreads();
+    for (int i = ty; i < 64; i += 4) {
+        int n = n0 + i, k = k0 + tx;
+        if (n < N && k < K) dst[((size_t)n * row_mult + row_off) * K + k] = tile[tx][i];
+    }
+}
+
+}  // namespace
+
+int pack_bf16_kn_to_nk_strided(hm_ctx *ctx, const uint16_t *d_w_kn, uint16_t *d_dst, int K, int N,
+                               int row_mult, int row_off) {
+    HM_REQUIRE(ctx, d_w_kn && d_dst && K > 0 && N > 0 && row_mult >= 1 && row_off >= 0 && row_off < row_mult,
+               "pack_bf16_kn_to_nk: bad arguments");
+    dim3 grid((N + 63) / 64, (K + 63) / 64);
+    hipLaunchKernelGGL(pack_kn_to_nk_kernel, grid, dim3(256), 0, ctx->stream, d_w_kn, d_dst, K, N,
+                       row_mult, row_off);
+    HM_LAUNCH_CHECK(ctx);
+    return HM_OK;
+}
+
+extern "C" {
+
+int hm_gemv_bf16_nk(hm_ctx *ctx, const float *d_x, const uint16_t *d_w_nk, float *d_out, int M,
+                    int K, int N) {
+    HM_CHECK_CTX(ctx);
+    HM_REQUIRE(ctx, d_x && d_w_nk && d_out, "hm_gemv_bf16_nk: NULL pointer");
+    GemvArgs a{};
+    a.x = d_x;
+    a.w = d_w_nk;
+    a.out = d_out;
+    a.K = K;
+    a.N = N;
+    return gemv_bf16_nk_launch(ctx, a, M, GEMV_EPI_NONE);
+}
+
+int hm_gemv_bf16(hm_ctx *ctx, const float *d_x, const uint16_t *d_w_kn, float *d_out, int M, int K,
+                 int N) {
+    HM_CHECK_CTX(ctx);
+    HM_REQUIRE(ctx, d_x && d_w_kn && d_out, "hm_gemv_bf16: NULL pointer");
+    HM_REQUIRE(ctx, M >= 1 && M <= 8, "hm_gemv_bf16: M=%d outside 1..8", M);
+    HM_REQUIRE(ctx, K > 0 && N > 0 && N % 4 == 0, "hm_gemv_bf16: need K > 0 and N %% 4 == 0 (K=%d N=%d)", K, N);
+    HM_REQUIRE(ctx, ((uintptr_t)d_w_kn % 8) == 0, "hm_gemv_bf16: weight pointer must be 8-byte aligned");
+    const int strips = (N + KN_STRIP - 1) / KN_STRIP;
+    HM_REQUIRE(ctx, (size_t)strips <= ctx->num_counters, "hm_gemv_bf16: N=%d too wide", N);
+    // enough workgroups for ~2 per CU, but at least 16 K rows per workgroup
+    int ksplit = (2 * ctx->num_cus + strips - 1) / strips;
+    int max_split = (K + 15) / 16;
+    if (ksplit > max_split) ksplit = max_split;
+    if (ksplit < 1) ksplit = 1;
+    while ((size_t)ksplit * N * sizeof(float) > ctx->workspace_bytes && ksplit > 1) ksplit--;
+    int kslice = (K + ksplit - 1) / ksplit;
+    kslice = (kslice + GEMV_WAVES - 1) / GEMV_WAVES * GEMV_WAVES;
+    ksplit = (K + kslice - 1) / kslice;
+    for (int m = 0; m < M; m++) {
+        hipLaunchKernelGGL(gemv_bf16_kn_kernel, dim3(strips, ksplit), dim3(GEMV_THREADS), 0,
+                           ctx->stream, d_x + (size_t)m * K, d_w_kn, d_out + (size_t)m * N,
+                           (float *)ctx->workspace, ctx->counters, K, N, kslice);
+        HM_LAUNCH_CHECK(ctx);
+    }
+    return HM_OK;
+}
+
+int hm_pack_bf16_kn_to_nk(hm_ctx *ctx, const uint16_t *d_w_kn, uint16_t *d_w_nk, int K, int N) {
+    HM_CHECK_CTX(ctx);
+    return pack_bf16_kn_to_nk_strided(ctx, d_w_kn, d_w_nk, K, N, 1, 0);
+}
+
+}  // extern "C"

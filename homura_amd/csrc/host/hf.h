@@ -1,0 +1,101 @@
+// HF-style decoder model on the GPU plan: TransformerConfig, TransformerWeights, the plan
+// emitters and HfModel (reference src/hf/config.rs, src/hf/weights.rs, src/hf/emitter.rs,
+// src/hf/emitter_quant.rs, src/hf/model.rs).
+#pragma once
+
+#include <memory>
+#include <string>
+#include <vector>
+
+#include "runtime.h"
+
+namespace homura {
+
+// reference TransformerConfig (src/hf/config.rs:11-73)
+struct TransformerConfig {
+    int hidden_size = 0, intermediate_size = 0, num_attention_heads = 0, num_hidden_layers = 0;
+    int num_key_value_heads = 0;  // 0 => MHA
+    int vocab_size = 0;
+    double rms_norm_eps = 1e-6;
+    double rope_theta = 10000.0;
+    int max_position_embeddings = 2048;
+    bool tie_word_embeddings = false;
+    int head_dim_opt = 0;  // 0 => hidden_size / num_attention_heads
+
+    int kv_heads() const { return num_key_value_heads ? num_key_value_heads : num_attention_heads; }
+    int head_dim() const { return head_dim_opt ? head_dim_opt : hidden_size / num_attention_heads; }
+    int gqa_repeat() const { return num_attention_heads / kv_heads(); }
+    int q_dim() const { return num_attention_heads * head_dim(); }
+    int kv_dim() const { return kv_heads() * head_dim(); }
+};
+
+// One entry of TransformerWeights::to_slot_buffers (src/hf/weights.rs:63-116 / :136-183):
+// what the host hands over for this slot.
+struct WeightSlotInfo {
+    std::string name;
+    DType dtype;
+    int64_t dim0 = 0, dim1 = 0;  // bf16/f32 matrices: [K][N] as the reference keeps them;
+                                 // quantised: dim0 = N rows, dim1 = K (raw blocks [N][K/32])
+    size_t bytes = 0;
+};
+
+// Scratch that the reference's fused kernels keep internal (attention output before the
+// O projection, the MLP's residual and activation) plus the LM-head argmax candidates.
+struct PlanScratch {
+    Buffer attn_flat, resid, act, cand_val, cand_idx;
+    Buffer normed, gate, up, down, q_raw, k_raw, v_raw;  // quantised plan only
+    int cand_cap = 0;
+};
+
+class HfModel {
+  public:
+    static std::unique_ptr<HfModel> create(hm_ctx *ctx, const TransformerConfig &cfg,
+                                           DType weight_dtype, bool has_qk_norm);
+    ~HfModel();
+
+    const TransformerConfig &config() const { return cfg_; }
+    const std::vector<WeightSlotInfo> &weight_slot_infos() const { return infos_; }
+    // Upload one slot (host pointer, exact byte size). bf16 matrices arrive [K][N] and are
+    // re-packed once into the K-contiguous stream layout; quantised blocks stay as they are.
+    int set_weight(int slot, const void *h_data, size_t bytes);
+    // reference HfModel::ensure_compiled (src/hf/model.rs:148-160) + RoPE tables (:62-66)
+    int finalize(int max_seq_len);
+
+    // reference HfModel::run_kv (src/hf/model.rs:198-218); multi-token input is consumed one
+    // token per plan step. h_logits: [n_ids][vocab] or NULL.
+    int run_kv(const int64_t *h_ids, int n_ids, float *h_logits);
+    int init_kv_cache(const float *const *h_kv, int seq_len);
+    int reset_kv_cache();
+    int kv_cache_len() const;
+    int generate_greedy(const int64_t *h_prompt, int n_prompt, int n_new, int32_t *h_tokens);
+    int bench_decode(int64_t first_id, int n_steps, float *ms_out, int32_t *h_tokens);
+    int profile_step(int64_t token_id, std::vector<StepProfile> &out);
+    ExecutionPlan *plan() { return plan_.get(); }
+
+  private:
+    HfModel() = default;
+    int emit_transformer_plan();        // reference src/hf/emitter.rs:867-1050
+    int emit_transformer_plan_quant();  // reference src/hf/emitter_quant.rs:1142-1503
+    int step_inputs(std::vector<Buffer *> &inputs);
+    int check_ids(const int64_t *ids, int n, std::vector<int32_t> &out);
+
+    hm_ctx *ctx_ = nullptr;
+    TransformerConfig cfg_;
+    DType weight_dtype_ = DType::BF16;
+    bool has_qk_norm_ = false;
+    bool finalized_ = false;
+    int max_seq_len_ = 0;
+    std::vector<WeightSlotInfo> infos_;
+    std::vector<Buffer> weight_bufs_;   // in weight_slots order, device resident
+    std::vector<bool> weight_set_;
+    // packed storage the bf16 weight slot buffers are views of
+    struct LayerPacked { Buffer qkv, o, gate_up, down; };
+    std::vector<LayerPacked> packed_;
+    Buffer lm_head_packed_;
+    Buffer rope_cos_, rope_sin_;        // [max_position][head_dim] f32
+    Buffer ids_view_, mask_view_;
+    std::shared_ptr<PlanScratch> scratch_;
+    std::unique_ptr<ExecutionPlan> plan_;
+};
+
+}  // namespace homura

@@ -1,0 +1,661 @@
+// HfModel and the bf16 plan emitter on the GPU runtime (see hf.h).
+#include "hf.h"
+
+#include <cmath>
+
+#include "../attention.h"
+#include "../gemv_bf16.h"
+#include "../light_ops.h"
+
+namespace homura {
+
+namespace {
+
+// reference precompute_rope_cos_sin (src/hf/precompute.rs:10-40): f64 angle
+// pos / theta^(2i/head_dim), rounded to f32, both halves of a row identical.
+void precompute_rope_cos_sin(int head_dim, int max_seq_len, double theta, std::vector<float> &cosv,
+                             std::vector<float> &sinv) {
+    const int half = head_dim / 2;
+    cosv.assign((size_t)max_seq_len * head_dim, 0.f);
+    sinv.assign((size_t)max_seq_len * head_dim, 0.f);
+    for (int pos = 0; pos < max_seq_len; pos++)
+        for (int i = 0; i < half; i++) {
+            const double freq = 1.0 / std::pow(theta, 2.0 * (double)i / (double)head_dim);
+            const double angle = (double)pos * freq;
+            const float c = (float)std::cos(angle), s = (float)std::sin(angle);
+            cosv[(size_t)pos * head_dim + i] = c;
+            cosv[(size_t)pos * head_dim + half + i] = c;
+            sinv[(size_t)pos * head_dim + i] = s;
+            sinv[(size_t)pos * head_dim + half + i] = s;
+        }
+}
+
+}  // namespace
+
+std::unique_ptr<HfModel> HfModel::create(hm_ctx *ctx, const TransformerConfig &cfg,
+                                         DType weight_dtype, bool has_qk_norm) {
+    auto fail = [&](const char *msg) -> std::unique_ptr<HfModel> {
+        hm_set_error(ctx, HM_ERR_INVALID, "hm_model_create: %s", msg);
+        return nullptr;
+    };
+    if (cfg.hidden_size <= 0 || cfg.intermediate_size <= 0 || cfg.num_attention_heads <= 0 ||
+        cfg.num_hidden_layers <= 0 || cfg.vocab_size <= 0)
+        return fail("config has a non-positive dimension");
+    if (cfg.num_attention_heads % cfg.kv_heads() != 0) return fail("heads not divisible by kv heads");
+    if (cfg.head_dim() != 128 && cfg.head_dim() != 64) return fail("head_dim must be 64 or 128");
+    if (cfg.gqa_repeat() > 8) return fail("GQA group larger than 8");
+    if (cfg.hidden_size % 32 || cfg.intermediate_size % 32 || cfg.q_dim() % 32)
+        return fail("hidden, intermediate and q dims must be multiples of 32");
+    if (weight_dtype != DType::BF16 && weight_dtype != DType::Q8_0 && weight_dtype != DType::Q4_0)
+        return fail("projection dtype must be BF16, Q8_0 or Q4_0");
+
+    std::unique_ptr<HfModel> m(new HfModel());
+    m->ctx_ = ctx;
+    m->cfg_ = cfg;
+    m->weight_dtype_ = weight_dtype;
+    m->has_qk_norm_ = has_qk_norm;
+
+    // Slot order = TransformerWeights::to_slot_buffers (src/hf/weights.rs:63-116) for bf16,
+    // to_slot_buffers_quant (:136-183) for block-quantised projections; models without bias.
+    const int64_t hidden = cfg.hidden_size, inter = cfg.intermediate_size, vocab = cfg.vocab_size;
+    const int64_t qd = cfg.q_dim(), kvd = cfg.kv_dim(), hd = cfg.head_dim();
+    const bool quant = dtype_is_quantized(weight_dtype);
+    auto &v = m->infos_;
+    auto f32_vec = [&](const std::string &name, int64_t n) {
+        v.push_back(WeightSlotInfo{name, DType::F32, n, 1, (size_t)n * 4});
+    };
+    auto proj = [&](const std::string &name, int64_t K, int64_t N) {
+        if (quant)
+            v.push_back(WeightSlotInfo{name, weight_dtype, N, K,
+                                       dtype_bytes_for_elements(weight_dtype, (size_t)(N * K), nullptr)});
+        else
+            v.push_back(WeightSlotInfo{name, DType::BF16, K, N, (size_t)(K * N) * 2});
+    };
+    v.push_back(WeightSlotInfo{"model.embed_tokens.weight", DType::F32, vocab, hidden,
+                               (size_t)(vocab * hidden) * 4});
+    for (int l = 0; l < cfg.num_hidden_layers; l++) {
+        const std::string p = "model.layers." + std::to_string(l) + ".";
+        f32_vec(p + "input_layernorm.weight", hidden);
+        proj(p + "self_attn.q_proj.weight", hidden, qd);
+        proj(p + "self_attn.k_proj.weight", hidden, kvd);
+        proj(p + "self_attn.v_proj.weight", hidden, kvd);
+        if (has_qk_norm) {
+            f32_vec(p + "self_attn.q_norm.weight", hd);
+            f32_vec(p + "self_attn.k_norm.weight", hd);
+        }
+        proj(p + "self_attn.o_proj.weight", qd, hidden);
+        f32_vec(p + "post_attention_layernorm.weight", hidden);
+        proj(p + "mlp.gate_proj.weight", hidden, inter);
+        proj(p + "mlp.up_proj.weight", hidden, inter);
+        proj(p + "mlp.down_proj.weight", inter, hidden);
+    }
+    f32_vec("model.norm.weight", hidden);
+    if (quant)  // the quantised plan keeps the LM head in f32 (src/hf/weights.rs:174-180)
+        v.push_back(WeightSlotInfo{"lm_head.weight", DType::F32, hidden, vocab, (size_t)(hidden * vocab) * 4});
+    else
+        v.push_back(WeightSlotInfo{"lm_head.weight", DType::BF16, hidden, vocab, (size_t)(hidden * vocab) * 2});
+
+    m->weight_bufs_.resize(v.size());
+    m->weight_set_.assign(v.size(), false);
+    m->packed_.resize(cfg.num_hidden_layers);
+    return m;
+}
+
+HfModel::~HfModel() {
+    if (ctx_) hm_sync(ctx_);
+}
+
+int HfModel::set_weight(int slot, const void *h_data, size_t bytes) {
+    if (slot < 0 || slot >= (int)infos_.size())
+        return hm_set_error(ctx_, HM_ERR_INVALID, "weight slot %d out of range (have %zu)", slot, infos_.size());
+    const WeightSlotInfo &info = infos_[slot];
+    if (bytes != info.bytes)  // the reference panics on a weight byte-size mismatch
+                              // (src/hf/emitter_quant.rs:1462-1478)
+        return hm_set_error(ctx_, HM_ERR_INVALID, "weight %s: expected %zu bytes, got %zu",
+                            info.name.c_str(), info.bytes, bytes);
+    if (finalized_) return hm_set_error(ctx_, HM_ERR_STATE, "model already finalized");
+    if (!h_data) return hm_set_error(ctx_, HM_ERR_INVALID, "weight %s: NULL data", info.name.c_str());
+
+    if (info.dtype != DType::BF16) {
+        // f32 vectors / tables and raw quantised blocks are stored as they come
+        Buffer b = Buffer::alloc_bytes(ctx_, bytes, {info.dim0, info.dim1}, info.dtype);
+        if (!b) return HM_ERR_OOM;
+        int rc = hm_upload(ctx_, b.ptr(), h_data, bytes);
+        if (rc != HM_OK) return rc;
+        weight_bufs_[slot] = std::move(b);
+        weight_set_[slot] = true;
+        return HM_OK;
+    }
+
+    // bf16 projection [K][N]: stage, then transpose into its place in the packed stream buffers
+    const int K = (int)info.dim0, N = (int)info.dim1;
+    const int hidden = cfg_.hidden_size, inter = cfg_.intermediate_size;
+    const int qd = cfg_.q_dim(), kvd = cfg_.kv_dim();
+    Buffer staging = Buffer::alloc_bytes(ctx_, bytes, {K, N}, DType::BF16);
+    if (!staging) return HM_ERR_OOM;
+    int rc = hm_upload(ctx_, staging.ptr(), h_data, bytes);
+    if (rc != HM_OK) return rc;
+
+    uint16_t *dst = nullptr;
+    int row_mult = 1, row_off = 0;
+    auto ensure = [&](Buffer &b, int64_t rows, int64_t cols) -> bool {
+        if (!b) b = Buffer::alloc(ctx_, {rows, cols}, DType::BF16);
+        return (bool)b;
+    };
+    const std::string &nm = info.name;
+    auto ends_with = [&](const char *suffix) {
+        const std::string s(suffix);
+        return nm.size() >= s.size() && nm.compare(nm.size() - s.size(), s.size(), s) == 0;
+    };
+    if (nm == "lm_head.weight") {
+        if (!ensure(lm_head_packed_, cfg_.vocab_size, hidden)) return HM_ERR_OOM;
+        dst = lm_head_packed_.as<uint16_t>();
+    } else {
+        const size_t p0 = std::string("model.layers.").size();
+        const int layer = std::atoi(nm.c_str() + p0);
+        LayerPacked &lp = packed_[layer];
+        if (ends_with("q_proj.weight") || ends_with("k_proj.weight") || ends_with("v_proj.weight")) {
+            if (!ensure(lp.qkv, qd + 2 * kvd, hidden)) return HM_ERR_OOM;
+            const size_t row0 = ends_with("q_proj.weight") ? 0 : ends_with("k_proj.weight") ? qd : qd + kvd;
+            dst = lp.qkv.as<uint16_t>() + row0 * hidden;
+        } else if (ends_with("o_proj.weight")) {
+            if (!ensure(lp.o, hidden, qd)) return HM_ERR_OOM;
+            dst = lp.o.as<uint16_t>();
+        } else if (ends_with("gate_proj.weight") || ends_with("up_proj.weight")) {
+            // rows interleaved (gate_0, up_0, gate_1, up_1, ...) so one wavefront finishes
+            // silu(gate_i) * up_i without a second pass
+            if (!ensure(lp.gate_up, 2 * (int64_t)inter, hidden)) return HM_ERR_OOM;
+            dst = lp.gate_up.as<uint16_t>();
+            row_mult = 2;
+            row_off = ends_with("up_proj.weight") ? 1 : 0;
+        } else if (ends_with("down_proj.weight")) {
+            if (!ensure(lp.down, hidden, inter)) return HM_ERR_OOM;
+            dst = lp.down.as<uint16_t>();
+        } else {
+            return hm_set_error(ctx_, HM_ERR_INVALID, "unexpected bf16 weight %s", nm.c_str());
+        }
+    }
+    rc = pack_bf16_kn_to_nk_strided(ctx_, staging.as<uint16_t>(), dst, K, N, row_mult, row_off);
+    if (rc != HM_OK) return rc;
+    if ((rc = hm_sync(ctx_)) != HM_OK) return rc;
+    // the slot buffer is a view of the packed rows ([N][K], K contiguous; interleaved slots
+    // have a doubled row stride)
+    weight_bufs_[slot] = Buffer::view(dst + (size_t)row_off * K, (size_t)N * K * 2 * row_mult, {N, K},
+                                      {(int64_t)K * row_mult, 1}, DType::BF16);
+    weight_set_[slot] = true;
+    return HM_OK;
+}
+
+int HfModel::finalize(int max_seq_len) {
+    if (finalized_) return HM_OK;
+    for (size_t i = 0; i < weight_set_.size(); i++)
+        if (!weight_set_[i])  // reference: "missing weight: {key}" (src/hf/weights.rs:276-282)
+            return hm_set_error(ctx_, HM_ERR_STATE, "missing weight: %s", infos_[i].name.c_str());
+    if (max_seq_len <= 0 || max_seq_len > cfg_.max_position_embeddings)
+        return hm_set_error(ctx_, HM_ERR_INVALID, "max_seq_len %d outside 1..max_position_embeddings=%d",
+                            max_seq_len, cfg_.max_position_embeddings);
+    max_seq_len_ = max_seq_len;
+
+    std::vector<float> cosv, sinv;
+    precompute_rope_cos_sin(cfg_.head_dim(), cfg_.max_position_embeddings, cfg_.rope_theta, cosv, sinv);
+    rope_cos_ = Buffer::alloc(ctx_, {cfg_.max_position_embeddings, cfg_.head_dim()}, DType::F32);
+    rope_sin_ = Buffer::alloc(ctx_, {cfg_.max_position_embeddings, cfg_.head_dim()}, DType::F32);
+    if (!rope_cos_ || !rope_sin_) return HM_ERR_OOM;
+    int rc = hm_upload(ctx_, rope_cos_.ptr(), cosv.data(), cosv.size() * 4);
+    if (rc == HM_OK) rc = hm_upload(ctx_, rope_sin_.ptr(), sinv.data(), sinv.size() * 4);
+    if (rc != HM_OK) return rc;
+
+    scratch_ = std::make_shared<PlanScratch>();
+    PlanScratch &s = *scratch_;
+    s.attn_flat = Buffer::alloc(ctx_, {cfg_.q_dim()}, DType::F32);
+    s.resid = Buffer::alloc(ctx_, {cfg_.hidden_size}, DType::F32);
+    s.act = Buffer::alloc(ctx_, {cfg_.intermediate_size}, DType::F32);
+    s.cand_cap = 4096;
+    s.cand_val = Buffer::alloc(ctx_, {s.cand_cap}, DType::F32);
+    s.cand_idx = Buffer::alloc(ctx_, {s.cand_cap}, DType::F32);
+    if (!s.attn_flat || !s.resid || !s.act || !s.cand_val || !s.cand_idx) return HM_ERR_OOM;
+
+    rc = dtype_is_quantized(weight_dtype_) ? emit_transformer_plan_quant() : emit_transformer_plan();
+    if (rc != HM_OK) return rc;
+    rc = plan_->prepare(std::max(max_seq_len, 16));
+    if (rc != HM_OK) return rc;
+    rc = plan_->ensure_kv_cache(max_seq_len_);
+    if (rc != HM_OK) return rc;
+    ids_view_ = Buffer::view(plan_->forced_ids(), (size_t)plan_->out_capacity() * 4, {1, DIM_DYNAMIC},
+                             {1, 1}, DType::I64);
+    mask_view_ = Buffer::view(plan_->state(), sizeof(DecodeState), {1, 1, 1, DIM_DYNAMIC}, {1, 1, 1, 1},
+                              DType::F32);
+    finalized_ = true;
+    return hm_sync(ctx_);
+}
+
+// ── bf16 plan ────────────────────────────────────────────────────────────────
+// Slot order and step list follow assign_transformer_slots / emit_transformer_plan
+// (reference src/hf/emitter.rs:74-498, :902-1014) for a model without biases.
+int HfModel::emit_transformer_plan() {
+    const TransformerConfig c = cfg_;
+    const int64_t hidden = c.hidden_size, inter = c.intermediate_size, vocab = c.vocab_size;
+    const int64_t H = c.num_attention_heads, kvh = c.kv_heads(), hd = c.head_dim();
+    const int64_t qd = c.q_dim(), kvd = c.kv_dim();
+    const int L = c.num_hidden_layers;
+    const float eps = (float)c.rms_norm_eps;
+    const bool qkn = has_qk_norm_;
+    const int64_t D = DIM_DYNAMIC;
+
+    std::vector<SlotDesc> descs;
+    auto alloc = [&](std::vector<int64_t> shape, DType dt, const std::string &name) -> size_t {
+        descs.push_back(SlotDesc{std::move(shape), dt, name});
+        return descs.size() - 1;
+    };
+    std::vector<size_t> input_slots, weight_slots, past_kv, present_kv;
+
+    const size_t input_ids = alloc({1, D}, DType::I64, "input_ids");
+    const size_t mask = alloc({1, 1, D, D}, DType::F32, "mask");
+    const size_t cos_s = alloc({D, hd}, DType::F32, "cos");
+    const size_t sin_s = alloc({D, hd}, DType::F32, "sin");
+    input_slots = {input_ids, mask, cos_s, sin_s};
+    const size_t embed_w = alloc({vocab, hidden}, DType::F32, "embed_tokens");
+    weight_slots.push_back(embed_w);
+    const size_t embed_out = alloc({1, D, hidden}, DType::F32, "embed_out");
+
+    struct LayerSlots {
+        size_t hidden_in, input_ln, q_w, k_w, v_w, q_norm, k_norm, o_w, post_ln, gate_w, up_w, down_w;
+        size_t q, k, v, past_k, past_v, present_k, present_v, attn_out, hidden_out;
+    };
+    std::vector<LayerSlots> ls(L);
+    for (int i = 0; i < L; i++) {
+        LayerSlots &s = ls[i];
+        const std::string p = "l" + std::to_string(i) + ".";
+        s.hidden_in = i == 0 ? embed_out : ls[i - 1].hidden_out;
+        auto w = [&](std::vector<int64_t> shape, DType dt, const std::string &n) {
+            size_t slot = alloc(std::move(shape), dt, p + n);
+            weight_slots.push_back(slot);
+            return slot;
+        };
+        s.input_ln = w({hidden}, DType::F32, "input_ln");
+        s.q_w = w({hidden, qd}, DType::BF16, "q_w");
+        s.k_w = w({hidden, kvd}, DType::BF16, "k_w");
+        s.v_w = w({hidden, kvd}, DType::BF16, "v_w");
+        s.q_norm = s.k_norm = (size_t)-1;
+        if (qkn) {
+            s.q_norm = w({hd}, DType::F32, "q_norm");
+            s.k_norm = w({hd}, DType::F32, "k_norm");
+        }
+        s.o_w = w({qd, hidden}, DType::BF16, "o_w");
+        s.post_ln = w({hidden}, DType::F32, "post_ln");
+        s.gate_w = w({hidden, inter}, DType::BF16, "gate_w");
+        s.up_w = w({hidden, inter}, DType::BF16, "up_w");
+        s.down_w = w({inter, hidden}, DType::BF16, "down_w");
+        s.q = alloc({1, D, H, hd}, DType::F32, p + "q");
+        s.k = alloc({1, kvh, D, hd}, DType::F32, p + "k");
+        s.v = alloc({1, kvh, D, hd}, DType::F32, p + "v");
+        s.past_k = alloc({1, kvh, D, hd}, DType::BF16, p + "past_k");
+        s.past_v = alloc({1, kvh, D, hd}, DType::BF16, p + "past_v");
+        past_kv.push_back(s.past_k);
+        past_kv.push_back(s.past_v);
+        input_slots.push_back(s.past_k);
+        input_slots.push_back(s.past_v);
+        s.present_k = alloc({1, kvh, D, hd}, DType::BF16, p + "present_k");
+        s.present_v = alloc({1, kvh, D, hd}, DType::BF16, p + "present_v");
+        present_kv.push_back(s.present_k);
+        present_kv.push_back(s.present_v);
+        s.attn_out = alloc({1, D, hidden}, DType::F32, p + "attn_out");
+        s.hidden_out = alloc({1, D, hidden}, DType::F32, p + "hidden_out");
+    }
+    const size_t final_norm = alloc({hidden}, DType::F32, "final_norm");
+    weight_slots.push_back(final_norm);
+    const size_t lm_head = alloc({hidden, vocab}, DType::BF16, "lm_head");
+    weight_slots.push_back(lm_head);
+    const size_t logits = alloc({1, D, vocab}, DType::F32, "logits");
+    std::vector<size_t> output_slots{logits};
+    output_slots.insert(output_slots.end(), present_kv.begin(), present_kv.end());
+
+    if (weight_slots.size() != infos_.size())
+        return hm_set_error(ctx_, HM_ERR_STATE, "plan expects %zu weights, model lists %zu",
+                            weight_slots.size(), infos_.size());
+
+    // attention split: ~2 workgroups per CU when the cache is full, at least 32 rows each
+    int att_chunk;
+    {
+        const int pairs = (int)kvh;
+        const int want = (2 * ctx_->num_cus + pairs - 1) / pairs;
+        att_chunk = (max_seq_len_ + want - 1) / want;
+        att_chunk = std::max(32, (att_chunk + 31) / 32 * 32);
+        att_chunk = std::min(att_chunk, 1024);
+    }
+
+    std::shared_ptr<PlanScratch> scr = scratch_;
+    std::vector<CompiledKernel> kernels;
+    std::vector<KernelStep> steps;
+    const double kv_bytes_full = 2.0 * kvh * max_seq_len_ * hd * 2;
+
+    // --- Embedding kernel (reference src/hf/emitter.rs:902-909) ---
+    {
+        CompiledKernel k;
+        k.ops_label = "Embed";
+        k.algorithmic_bytes = hidden * 4.0 * 2;
+        k.launch = [=](const StepContext &sc) -> int {
+            Buffer *table = sc.pool[sc.step.input_slots[1]];
+            Buffer *out = sc.pool[sc.step.output_slots[0]];
+            sc.plan->count_launches(1);
+            return embed_step_launch(sc.ctx, sc.plan->state(), sc.plan->forced_ids(), table->as<float>(),
+                                     out->as<float>(), (int)vocab, (int)hidden);
+        };
+        kernels.push_back(std::move(k));
+        steps.push_back(KernelStep::kernel(kernels.size() - 1, {input_ids, embed_w}, {embed_out}));
+    }
+
+    for (int i = 0; i < L; i++) {
+        const LayerSlots &s = ls[i];
+        // --- QKV + QK-norm + RoPE kernel (reference src/hf/emitter.rs:915-948) ---
+        {
+            CompiledKernel k;
+            k.ops_label = qkn ? "QKV+QKNorm+RoPE" : "QKV+RoPE";
+            k.algorithmic_bytes = (double)hidden * (qd + 2 * kvd) * 2;
+            const int layer = i;
+            k.launch = [=](const StepContext &sc) -> int {
+                const auto &in = sc.step.input_slots;
+                Buffer *h = sc.pool[in[0]], *ln_w = sc.pool[in[1]], *q_w = sc.pool[in[2]];
+                Buffer *cosb = sc.pool[in[5]], *sinb = sc.pool[in[6]];
+                Buffer *q = sc.pool[sc.step.output_slots[0]], *kk = sc.pool[sc.step.output_slots[1]],
+                       *vv = sc.pool[sc.step.output_slots[2]];
+                GemvArgs g;
+                g.x = h->as<float>();
+                g.w = q_w->as<uint16_t>();  // q|k|v rows are adjacent in the packed buffer
+                g.out = q->as<float>();     // q|k|v outputs are adjacent too (aliased slots)
+                g.K = (int)hidden;
+                g.N = (int)(qd + 2 * kvd);
+                g.norm_w = ln_w->as<float>();
+                g.eps = eps;
+                int rc = gemv_bf16_nk_launch(sc.ctx, g, 1, GEMV_EPI_NONE);
+                if (rc != HM_OK) return rc;
+                KvCache *cache = sc.plan->kv_cache();
+                QkRopeArgs r;
+                r.q = q->as<float>();
+                r.k = kk->as<float>();
+                r.v = vv->as<float>();
+                if (qkn) {
+                    r.qw = sc.pool[in[7]]->as<float>();
+                    r.kw = sc.pool[in[8]]->as<float>();
+                }
+                r.cos = cosb->as<float>();
+                r.sin = sinb->as<float>();
+                r.S = 1;
+                r.H = (int)H;
+                r.kvh = (int)kvh;
+                r.hd = (int)hd;
+                r.eps = eps;
+                r.kcache = cache->key_ptr(layer);
+                r.vcache = cache->value_ptr(layer);
+                r.max_len = cache->max_len();
+                r.state = sc.plan->state();
+                sc.plan->count_launches(2);
+                return qknorm_rope_launch(sc.ctx, r);
+            };
+            kernels.push_back(std::move(k));
+            std::vector<size_t> in{s.hidden_in, s.input_ln, s.q_w, s.k_w, s.v_w, cos_s, sin_s};
+            if (qkn) {
+                in.push_back(s.q_norm);
+                in.push_back(s.k_norm);
+            }
+            steps.push_back(KernelStep::kernel(kernels.size() - 1, in, {s.q, s.k, s.v}));
+        }
+        // --- KV concat native ops (reference src/hf/emitter.rs:950-965) ---
+        for (int kv = 0; kv < 2; kv++) {
+            KernelStep st;
+            st.input_slots = {kv ? s.past_v : s.past_k, kv ? s.v : s.k};
+            st.output_slots = {kv ? s.present_v : s.present_k};
+            st.native_op = NativeOp{NativeOpKind::Concat, 2};
+            steps.push_back(st);
+        }
+        // --- Attention + O projection kernel (reference src/hf/emitter.rs:967-980) ---
+        {
+            CompiledKernel k;
+            k.ops_label = "Attn";
+            k.algorithmic_bytes = (double)qd * hidden * 2 + kv_bytes_full;
+            k.launch = [=](const StepContext &sc) -> int {
+                const auto &in = sc.step.input_slots;
+                Buffer *q = sc.pool[in[0]], *pk = sc.pool[in[1]], *pv = sc.pool[in[2]], *o_w = sc.pool[in[4]];
+                Buffer *out = sc.pool[sc.step.output_slots[0]];
+                AttnArgs a;
+                a.q = q->as<float>();
+                a.kcache = pk->as<uint16_t>();
+                a.vcache = pv->as<uint16_t>();
+                a.out = scr->attn_flat.as<float>();
+                a.B = 1;
+                a.H = (int)H;
+                a.kvh = (int)kvh;
+                a.hd = (int)hd;
+                a.max_len = sc.plan->kv_cache()->max_len();
+                a.kv_len = 1;
+                a.scale = (float)(1.0 / std::sqrt((double)hd));  // f64 -> f32 constant, emitter.rs:719
+                a.state = sc.plan->state();
+                a.fixed_chunk = att_chunk;
+                int rc = gqa_decode_attn_launch(sc.ctx, a);
+                if (rc != HM_OK) return rc;
+                GemvArgs g;
+                g.x = scr->attn_flat.as<float>();
+                g.w = o_w->as<uint16_t>();
+                g.out = out->as<float>();
+                g.K = (int)qd;
+                g.N = (int)hidden;
+                sc.plan->count_launches(2);
+                return gemv_bf16_nk_launch(sc.ctx, g, 1, GEMV_EPI_NONE);
+            };
+            kernels.push_back(std::move(k));
+            steps.push_back(KernelStep::kernel(kernels.size() - 1,
+                                               {s.q, s.present_k, s.present_v, mask, s.o_w}, {s.attn_out}));
+        }
+        // --- residual + MLP kernel (reference src/hf/emitter.rs:982-996) ---
+        {
+            CompiledKernel k;
+            k.ops_label = "MLP";
+            k.algorithmic_bytes = 3.0 * hidden * inter * 2;
+            k.launch = [=](const StepContext &sc) -> int {
+                const auto &in = sc.step.input_slots;
+                Buffer *h = sc.pool[in[0]], *attn_out = sc.pool[in[1]], *ln_w = sc.pool[in[2]];
+                Buffer *gate_w = sc.pool[in[3]], *down_w = sc.pool[in[5]];
+                Buffer *out = sc.pool[sc.step.output_slots[0]];
+                GemvArgs g;  // gate|up interleaved rows, silu(gate)*up in the epilogue
+                g.x = h->as<float>();
+                g.prologue_residual = attn_out->as<float>();
+                g.norm_w = ln_w->as<float>();
+                g.eps = eps;
+                g.resid_out = scr->resid.as<float>();
+                g.w = gate_w->as<uint16_t>();
+                g.out = scr->act.as<float>();
+                g.K = (int)hidden;
+                g.N = (int)(2 * inter);
+                int rc = gemv_bf16_nk_launch(sc.ctx, g, 1, GEMV_EPI_SILU_MUL_PAIRS);
+                if (rc != HM_OK) return rc;
+                GemvArgs d;
+                d.x = scr->act.as<float>();
+                d.w = down_w->as<uint16_t>();
+                d.out = out->as<float>();
+                d.K = (int)inter;
+                d.N = (int)hidden;
+                d.epilogue_residual = scr->resid.as<float>();
+                sc.plan->count_launches(2);
+                return gemv_bf16_nk_launch(sc.ctx, d, 1, GEMV_EPI_RESIDUAL);
+            };
+            kernels.push_back(std::move(k));
+            steps.push_back(KernelStep::kernel(
+                kernels.size() - 1, {s.hidden_in, s.attn_out, s.post_ln, s.gate_w, s.up_w, s.down_w},
+                {s.hidden_out}));
+        }
+    }
+    // --- LM head kernel (reference src/hf/emitter.rs:999-1014) + the greedy pick of
+    //     src/generate.rs:735-742 taken on the device ---
+    {
+        CompiledKernel k;
+        k.ops_label = "LMHead";
+        k.algorithmic_bytes = (double)hidden * vocab * 2 + vocab * 4.0;
+        k.launch = [=](const StepContext &sc) -> int {
+            const auto &in = sc.step.input_slots;
+            Buffer *h = sc.pool[in[0]], *nw = sc.pool[in[1]], *w = sc.pool[in[2]];
+            Buffer *out = sc.pool[sc.step.output_slots[0]];
+            GemvArgs g;
+            g.x = h->as<float>();
+            g.norm_w = nw->as<float>();
+            g.eps = eps;
+            g.w = w->as<uint16_t>();
+            g.out = out->as<float>();
+            g.K = (int)hidden;
+            g.N = (int)vocab;
+            g.argmax_val = scr->cand_val.as<float>();
+            g.argmax_idx = scr->cand_idx.as<int>();
+            g.argmax_cap = scr->cand_cap;
+            int rc = gemv_bf16_nk_launch(sc.ctx, g, 1, GEMV_EPI_ARGMAX);
+            if (rc != HM_OK) return rc;
+            const int ncand = std::min(gemv_bf16_nk_grid(sc.ctx, (int)vocab, 4), scr->cand_cap);
+            sc.plan->count_launches(2);
+            return finish_step_launch(sc.ctx, sc.plan->state(), scr->cand_val.as<float>(),
+                                      scr->cand_idx.as<int>(), ncand, sc.plan->out_tokens(),
+                                      sc.plan->out_capacity());
+        };
+        kernels.push_back(std::move(k));
+        steps.push_back(KernelStep::kernel(kernels.size() - 1, {ls[L - 1].hidden_out, final_norm, lm_head},
+                                           {logits}));
+    }
+
+    const size_t num_slots = descs.size();
+    plan_.reset(new ExecutionPlan(ctx_, std::move(kernels), std::move(steps), num_slots, input_slots,
+                                  weight_slots, output_slots, std::move(descs)));
+    KvPlanInfo info;
+    info.num_layers = L;
+    info.num_heads = (int)kvh;
+    info.head_dim = (int)hd;
+    info.past_kv_input_slots = past_kv;
+    info.present_kv_output_slots = present_kv;
+    plan_->set_kv_info(info);
+    for (int i = 0; i < L; i++) {  // q|k|v of a layer share one allocation
+        plan_->alias_slot(ls[i].k, ls[i].q, (size_t)qd * 4);
+        plan_->alias_slot(ls[i].v, ls[i].q, (size_t)(qd + kvd) * 4);
+    }
+    return HM_OK;
+}
+
+int HfModel::emit_transformer_plan_quant() {
+    return hm_set_error(ctx_, HM_ERR_INVALID, "quantised transformer plan is not built yet");
+}
+
+// ── running ──────────────────────────────────────────────────────────────────
+
+int HfModel::step_inputs(std::vector<Buffer *> &inputs) {
+    inputs = {&ids_view_, &mask_view_, &rope_cos_, &rope_sin_};
+    return HM_OK;
+}
+
+int HfModel::check_ids(const int64_t *ids, int n, std::vector<int32_t> &out) {
+    out.resize(n);
+    for (int i = 0; i < n; i++) {
+        if (ids[i] < 0 || ids[i] >= cfg_.vocab_size)
+            return hm_set_error(ctx_, HM_ERR_INVALID, "token id %lld outside the vocabulary (%d)",
+                                (long long)ids[i], cfg_.vocab_size);
+        out[i] = (int32_t)ids[i];
+    }
+    return HM_OK;
+}
+
+int HfModel::run_kv(const int64_t *h_ids, int n_ids, float *h_logits) {
+    if (!finalized_) return hm_set_error(ctx_, HM_ERR_STATE, "model not finalized");
+    if (n_ids <= 0 || !h_ids) return hm_set_error(ctx_, HM_ERR_INVALID, "run_kv: no input ids");
+    if (kv_cache_len() + n_ids > max_seq_len_)
+        return hm_set_error(ctx_, HM_ERR_STATE, "KV cache full (%d + %d > %d)", kv_cache_len(), n_ids, max_seq_len_);
+    std::vector<int32_t> ids;
+    int rc = check_ids(h_ids, n_ids, ids);
+    if (rc != HM_OK) return rc;
+    if (n_ids > plan_->out_capacity())
+        return hm_set_error(ctx_, HM_ERR_INVALID, "run_kv: %d ids exceed the step capacity %d", n_ids, plan_->out_capacity());
+    if ((rc = plan_->arm(ids.data(), n_ids)) != HM_OK) return rc;
+    std::vector<Buffer *> inputs;
+    step_inputs(inputs);
+    const size_t logits_slot = plan_->output_slots()[0];
+    for (int i = 0; i < n_ids; i++) {
+        if ((rc = plan_->run_kv(inputs, weight_bufs_, max_seq_len_)) != HM_OK) return rc;
+        if (h_logits) {
+            rc = hm_download(ctx_, h_logits + (size_t)i * cfg_.vocab_size, plan_->slot(logits_slot)->ptr(),
+                             (size_t)cfg_.vocab_size * 4);
+            if (rc != HM_OK) return rc;
+        }
+    }
+    return hm_sync(ctx_);
+}
+
+int HfModel::init_kv_cache(const float *const *h_kv, int seq_len) {
+    if (!finalized_) return hm_set_error(ctx_, HM_ERR_STATE, "model not finalized");
+    return plan_->init_kv_cache(h_kv, seq_len, max_seq_len_);
+}
+
+int HfModel::reset_kv_cache() {
+    if (!finalized_) return hm_set_error(ctx_, HM_ERR_STATE, "model not finalized");
+    plan_->reset_kv_cache();
+    return HM_OK;
+}
+
+int HfModel::kv_cache_len() const { return plan_ ? plan_->kv_cache_len() : 0; }
+
+int HfModel::generate_greedy(const int64_t *h_prompt, int n_prompt, int n_new, int32_t *h_tokens) {
+    if (!finalized_) return hm_set_error(ctx_, HM_ERR_STATE, "model not finalized");
+    if (n_prompt <= 0 || n_new <= 0 || !h_prompt || !h_tokens)
+        return hm_set_error(ctx_, HM_ERR_INVALID, "generate_greedy: bad arguments");
+    const int steps = n_prompt + n_new - 1;
+    if (kv_cache_len() + steps > max_seq_len_)  // the reference's loop stops at max_seq_len
+                                                // (src/generate.rs:188-194); here it is an error
+        return hm_set_error(ctx_, HM_ERR_STATE, "KV cache full (%d + %d > %d)", kv_cache_len(), steps, max_seq_len_);
+    if (steps > plan_->out_capacity())
+        return hm_set_error(ctx_, HM_ERR_INVALID, "generate_greedy: %d steps exceed capacity %d", steps, plan_->out_capacity());
+    std::vector<int32_t> ids;
+    int rc = check_ids(h_prompt, n_prompt, ids);
+    if (rc != HM_OK) return rc;
+    if ((rc = plan_->arm(ids.data(), n_prompt)) != HM_OK) return rc;
+    std::vector<Buffer *> inputs;
+    step_inputs(inputs);
+    for (int i = 0; i < steps; i++)
+        if ((rc = plan_->run_kv(inputs, weight_bufs_, max_seq_len_)) != HM_OK) return rc;
+    // the pick after prompt token n_prompt-1 is generated token 0
+    return hm_download(ctx_, h_tokens, plan_->out_tokens() + (n_prompt - 1), (size_t)n_new * 4);
+}
+
+int HfModel::bench_decode(int64_t first_id, int n_steps, float *ms_out, int32_t *h_tokens) {
+    if (!finalized_) return hm_set_error(ctx_, HM_ERR_STATE, "model not finalized");
+    if (n_steps <= 0 || n_steps > plan_->out_capacity())
+        return hm_set_error(ctx_, HM_ERR_INVALID, "bench_decode: bad step count %d", n_steps);
+    if (kv_cache_len() + n_steps > max_seq_len_)
+        return hm_set_error(ctx_, HM_ERR_STATE, "KV cache full (%d + %d > %d)", kv_cache_len(), n_steps, max_seq_len_);
+    std::vector<int32_t> ids;
+    int rc = check_ids(&first_id, 1, ids);
+    if (rc != HM_OK) return rc;
+    if ((rc = plan_->arm(ids.data(), 1)) != HM_OK) return rc;
+    std::vector<Buffer *> inputs;
+    step_inputs(inputs);
+    hipEvent_t e0, e1;
+    HM_HIP(ctx_, hipEventCreate(&e0));
+    HM_HIP(ctx_, hipEventCreate(&e1));
+    HM_HIP(ctx_, hipEventRecord(e0, ctx_->stream));
+    for (int i = 0; i < n_steps; i++)
+        if ((rc = plan_->run_kv(inputs, weight_bufs_, max_seq_len_)) != HM_OK) break;
+    if (rc == HM_OK) {
+        HM_HIP(ctx_, hipEventRecord(e1, ctx_->stream));
+        HM_HIP(ctx_, hipEventSynchronize(e1));
+        HM_HIP(ctx_, hipEventElapsedTime(ms_out, e0, e1));
+    }
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    if (rc != HM_OK) return rc;
+    if (h_tokens) rc = hm_download(ctx_, h_tokens, plan_->out_tokens(), (size_t)n_steps * 4);
+    return rc;
+}
+
+int HfModel::profile_step(int64_t token_id, std::vector<StepProfile> &out) {
+    if (!finalized_) return hm_set_error(ctx_, HM_ERR_STATE, "model not finalized");
+    std::vector<int32_t> ids;
+    int rc = check_ids(&token_id, 1, ids);
+    if (rc != HM_OK) return rc;
+    if ((rc = plan_->arm(ids.data(), 1)) != HM_OK) return rc;
+    std::vector<Buffer *> inputs;
+    step_inputs(inputs);
+    return plan_->profile_step(inputs, weight_bufs_, max_seq_len_, out);
+}
+
+}  // namespace homura

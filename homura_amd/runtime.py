@@ -1,0 +1,292 @@
+"""Python handles over the C boundary: Context / DeviceBuffer for the kernel-level entry
+points, HfModel for the C++ host classes that mirror the reference's
+HfModel -> ExecutionPlan -> KvCache stack (reference src/hf/model.rs, src/runtime.rs).
+"""
+from __future__ import annotations
+
+import ctypes as C
+from dataclasses import dataclass
+
+import numpy as np
+
+from . import _ffi
+
+DTYPE_F32, DTYPE_BF16, DTYPE_Q8_0, DTYPE_Q4_0, DTYPE_I64 = 0, 1, 2, 3, 4
+
+
+class HomuraError(RuntimeError):
+    """A C entry point returned a negative status; `.code` carries it."""
+
+    def __init__(self, code: int, message: str):
+        super().__init__(f"[{code}] {message}")
+        self.code = code
+
+
+class DeviceBuffer:
+    """An HBM allocation owned by a Context (freed explicitly or with the context)."""
+
+    def __init__(self, ctx: "Context", ptr: int, nbytes: int):
+        self.ctx, self.ptr, self.nbytes = ctx, ptr, nbytes
+
+    def upload(self, arr: np.ndarray) -> "DeviceBuffer":
+        a = np.ascontiguousarray(arr)
+        if a.nbytes > self.nbytes:
+            raise ValueError(f"upload of {a.nbytes} bytes into a buffer of {self.nbytes}")
+        self.ctx._check(self.ctx.lib.hm_upload(self.ctx.h, self.ptr, a.ctypes.data, a.nbytes))
+        return self
+
+    def download(self, dtype, shape=None) -> np.ndarray:
+        dtype = np.dtype(dtype)
+        n = self.nbytes // dtype.itemsize if shape is None else int(np.prod(shape))
+        out = np.empty(n, dtype=dtype)
+        if out.nbytes > self.nbytes:
+            raise ValueError("download larger than the buffer")
+        self.ctx._check(self.ctx.lib.hm_download(self.ctx.h, out.ctypes.data, self.ptr, out.nbytes))
+        return out if shape is None else out.reshape(shape)
+
+    def free(self):
+        if self.ptr:
+            self.ctx._check(self.ctx.lib.hm_free(self.ctx.h, self.ptr))
+            self.ptr = 0
+
+
+class Context:
+    """One GPU + one HIP stream (hm_ctx)."""
+
+    def __init__(self, device: int = 0):
+        self.lib = _ffi.load()
+        self.h = self.lib.hm_init(device)
+        if not self.h:
+            raise HomuraError(-2, (self.lib.hm_last_error(None) or b"hm_init failed").decode())
+        self._bufs: list[DeviceBuffer] = []
+
+    def _check(self, rc: int):
+        if rc != 0:
+            raise HomuraError(rc, (self.lib.hm_last_error(self.h) or b"").decode())
+
+    def close(self):
+        if self.h:
+            self.lib.hm_destroy(self.h)
+            self.h = None
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        for b in self._bufs:
+            if b.ptr:
+                try:
+                    b.free()
+                except HomuraError:
+                    pass
+        self.close()
+
+    # memory
+    def alloc(self, nbytes: int) -> DeviceBuffer:
+        p = C.c_void_p()
+        self._check(self.lib.hm_alloc(self.h, nbytes, C.byref(p)))
+        b = DeviceBuffer(self, p.value, max(nbytes, 1))
+        self._bufs.append(b)
+        return b
+
+    def to_device(self, arr: np.ndarray) -> DeviceBuffer:
+        a = np.ascontiguousarray(arr)
+        return self.alloc(a.nbytes).upload(a)
+
+    def empty(self, n: int, dtype=np.float32) -> DeviceBuffer:
+        return self.alloc(int(n) * np.dtype(dtype).itemsize)
+
+    def sync(self):
+        self._check(self.lib.hm_sync(self.h))
+
+    def device_name(self) -> str:
+        buf = C.create_string_buffer(128)
+        self._check(self.lib.hm_device_name(self.h, buf, 128))
+        return buf.value.decode()
+
+    # timing on the context stream
+    def time_ms(self, fn, iters: int = 1, warmup: int = 0) -> float:
+        """Average milliseconds per call of `fn` measured with HIP events on the stream."""
+        e0, e1 = C.c_void_p(), C.c_void_p()
+        self._check(self.lib.hm_event_create(self.h, C.byref(e0)))
+        self._check(self.lib.hm_event_create(self.h, C.byref(e1)))
+        try:
+            for _ in range(warmup):
+                fn()
+            self._check(self.lib.hm_event_record(self.h, e0))
+            for _ in range(iters):
+                fn()
+            self._check(self.lib.hm_event_record(self.h, e1))
+            ms = C.c_float()
+            self._check(self.lib.hm_event_elapsed_ms(self.h, e0, e1, C.byref(ms)))
+            return ms.value / iters
+        finally:
+            self.lib.hm_event_destroy(self.h, e0)
+            self.lib.hm_event_destroy(self.h, e1)
+
+    # kernel-level entry points (thin: pointer plumbing only)
+    def gemv_bf16(self, x, w_kn, out, M, K, N):
+        self._check(self.lib.hm_gemv_bf16(self.h, x.ptr, w_kn.ptr, out.ptr, M, K, N))
+
+    def pack_bf16_kn_to_nk(self, w_kn, w_nk, K, N):
+        self._check(self.lib.hm_pack_bf16_kn_to_nk(self.h, w_kn.ptr, w_nk.ptr, K, N))
+
+    def gemv_bf16_nk(self, x, w_nk, out, M, K, N):
+        self._check(self.lib.hm_gemv_bf16_nk(self.h, x.ptr, w_nk.ptr, out.ptr, M, K, N))
+
+    def gemv_q8_0(self, x, w, out, M, K, N):
+        self._check(self.lib.hm_gemv_q8_0(self.h, x.ptr, w.ptr, out.ptr, M, K, N))
+
+    def gemv_q4_0(self, x, w, out, M, K, N):
+        self._check(self.lib.hm_gemv_q4_0(self.h, x.ptr, w.ptr, out.ptr, M, K, N))
+
+    def dequant_q8_0(self, blocks, out, nblocks):
+        self._check(self.lib.hm_dequant_q8_0(self.h, blocks.ptr, out.ptr, nblocks))
+
+    def dequant_q4_0(self, blocks, out, nblocks):
+        self._check(self.lib.hm_dequant_q4_0(self.h, blocks.ptr, out.ptr, nblocks))
+
+    def gemm_bf16(self, a, b, c, M, K, N):
+        self._check(self.lib.hm_gemm_bf16(self.h, a.ptr, b.ptr, c.ptr, M, K, N))
+
+    def kv_append(self, kc, vc, k, v, B, kvh, hd, max_len, pos, n_new):
+        self._check(self.lib.hm_kv_append(self.h, kc.ptr, vc.ptr, k.ptr, v.ptr, B, kvh, hd,
+                                          max_len, pos, n_new))
+
+    def gqa_decode_attn(self, q, kc, vc, out, B, H, kvh, hd, max_len, kv_len, scale):
+        self._check(self.lib.hm_gqa_decode_attn(self.h, q.ptr, kc.ptr, vc.ptr, out.ptr, B, H, kvh,
+                                                hd, max_len, kv_len, scale))
+
+    def rmsnorm(self, x, w, out, rows, dim, eps):
+        self._check(self.lib.hm_rmsnorm(self.h, x.ptr, w.ptr, out.ptr, rows, dim, eps))
+
+    def qknorm_rope(self, q, k, qw, kw, cos, sin, S, H, kvh, hd, eps):
+        self._check(self.lib.hm_qknorm_rope(self.h, q.ptr, k.ptr, qw.ptr if qw else None,
+                                            kw.ptr if kw else None, cos.ptr, sin.ptr, S, H, kvh,
+                                            hd, eps))
+
+    def silu_mul(self, g, u, out, n):
+        self._check(self.lib.hm_silu_mul(self.h, g.ptr, u.ptr, out.ptr, n))
+
+    def add(self, a, b, out, n):
+        self._check(self.lib.hm_add(self.h, a.ptr, b.ptr, out.ptr, n))
+
+    def embed(self, ids, table, out, n_ids, vocab, hidden):
+        self._check(self.lib.hm_embed(self.h, ids.ptr, table.ptr, out.ptr, n_ids, vocab, hidden))
+
+    def argmax(self, values, n, out):
+        self._check(self.lib.hm_argmax(self.h, values.ptr, n, out.ptr))
+
+
+@dataclass
+class TransformerConfig:
+    """Field-for-field the reference's TransformerConfig (src/hf/config.rs:11-73)."""
+    hidden_size: int
+    intermediate_size: int
+    num_attention_heads: int
+    num_hidden_layers: int
+    vocab_size: int
+    num_key_value_heads: int | None = None
+    rms_norm_eps: float = 1e-6
+    rope_theta: float = 10_000.0
+    max_position_embeddings: int = 2048
+    tie_word_embeddings: bool = False
+    head_dim: int | None = None
+
+    def kv_heads(self) -> int:
+        return self.num_key_value_heads or self.num_attention_heads
+
+    def get_head_dim(self) -> int:
+        return self.head_dim or self.hidden_size // self.num_attention_heads
+
+    def gqa_repeat(self) -> int:
+        return self.num_attention_heads // self.kv_heads()
+
+    def to_c(self) -> _ffi.HmTransformerConfig:
+        return _ffi.HmTransformerConfig(
+            self.hidden_size, self.intermediate_size, self.num_attention_heads,
+            self.num_hidden_layers, self.num_key_value_heads or 0, self.vocab_size,
+            self.head_dim or 0, self.max_position_embeddings, int(self.tie_word_embeddings),
+            self.rms_norm_eps, self.rope_theta)
+
+
+class HfModel:
+    """Handle on the C++ HfModel (reference src/hf/model.rs:17-268): weights are handed over
+    in TransformerWeights::to_slot_buffers order, then run_kv / generate run on the GPU."""
+
+    def __init__(self, ctx: Context, config: TransformerConfig, weight_dtype: int = DTYPE_BF16,
+                 has_qk_norm: bool = False):
+        self.ctx, self.config, self.lib = ctx, config, ctx.lib
+        cfg = config.to_c()
+        self.h = self.lib.hm_model_create(ctx.h, C.byref(cfg), weight_dtype, int(has_qk_norm))
+        if not self.h:
+            raise HomuraError(-1, (self.lib.hm_last_error(ctx.h) or b"").decode())
+
+    def _check(self, rc: int):
+        if rc < 0:
+            raise HomuraError(rc, (self.lib.hm_last_error(self.ctx.h) or b"").decode())
+        return rc
+
+    def close(self):
+        if self.h:
+            self.lib.hm_model_destroy(self.h)
+            self.h = None
+
+    def weight_slots(self):
+        """[(name, dtype, dim0, dim1, nbytes)] in upload order."""
+        out = []
+        n = self._check(self.lib.hm_model_num_weight_slots(self.h))
+        for i in range(n):
+            name = C.create_string_buffer(96)
+            dt, d0, d1, nb = C.c_int(), C.c_int64(), C.c_int64(), C.c_size_t()
+            self._check(self.lib.hm_model_weight_slot_info(self.h, i, name, 96, C.byref(dt),
+                                                           C.byref(d0), C.byref(d1), C.byref(nb)))
+            out.append((name.value.decode(), dt.value, d0.value, d1.value, nb.value))
+        return out
+
+    def set_weight(self, slot: int, arr: np.ndarray):
+        a = np.ascontiguousarray(arr)
+        self._check(self.lib.hm_model_set_weight(self.h, slot, a.ctypes.data, a.nbytes))
+
+    def finalize(self, max_seq_len: int):
+        self._check(self.lib.hm_model_finalize(self.h, max_seq_len))
+
+    def init_kv_cache(self, kv_buffers: list[np.ndarray], seq_len: int):
+        arrs = [np.ascontiguousarray(b, dtype=np.float32) for b in kv_buffers]
+        ptrs = (_ffi.c_f32_p * len(arrs))(*[a.ctypes.data_as(_ffi.c_f32_p) for a in arrs])
+        self._check(self.lib.hm_model_init_kv_cache(self.h, ptrs, seq_len))
+
+    def reset_kv_cache(self):
+        self._check(self.lib.hm_model_reset_kv_cache(self.h))
+
+    def kv_cache_len(self) -> int:
+        return self._check(self.lib.hm_model_kv_cache_len(self.h))
+
+    def run_kv(self, input_ids, want_logits: bool = True):
+        ids = np.ascontiguousarray(input_ids, dtype=np.int64).reshape(-1)
+        logits = np.empty((len(ids), self.config.vocab_size), dtype=np.float32) if want_logits else None
+        self._check(self.lib.hm_model_run_kv(
+            self.h, ids.ctypes.data_as(C.POINTER(C.c_int64)), len(ids),
+            logits.ctypes.data_as(_ffi.c_f32_p) if want_logits else None))
+        return logits
+
+    def generate_greedy(self, prompt_ids, n_new: int) -> np.ndarray:
+        ids = np.ascontiguousarray(prompt_ids, dtype=np.int64).reshape(-1)
+        out = np.empty(n_new, dtype=np.int32)
+        self._check(self.lib.hm_model_generate_greedy(
+            self.h, ids.ctypes.data_as(C.POINTER(C.c_int64)), len(ids), n_new,
+            out.ctypes.data_as(C.POINTER(C.c_int32))))
+        return out
+
+    def bench_decode(self, first_id: int, n_steps: int):
+        ms = C.c_float()
+        toks = np.empty(n_steps, dtype=np.int32)
+        self._check(self.lib.hm_model_bench_decode(self.h, first_id, n_steps, C.byref(ms),
+                                                   toks.ctypes.data_as(C.POINTER(C.c_int32))))
+        return ms.value, toks
+
+    def profile_step(self, token_id: int):
+        recs = (_ffi.HmKernelProfile * 32)()
+        n = self._check(self.lib.hm_model_profile_step(self.h, token_id, recs, 32))
+        return [dict(label=recs[i].label.decode(), ms=recs[i].ms, launches=recs[i].launches,
+                     bytes=recs[i].bytes) for i in range(n)]

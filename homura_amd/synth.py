@@ -1,0 +1,61 @@
+"""Deterministic synthetic tensors (numpy views of the library's host-side generator).
+
+Same bits on every platform: the generator is integer arithmetic (see csrc/synth.cpp).
+Seeds used by the BASELINE configurations live here so tests and bench agree.
+"""
+from __future__ import annotations
+
+import numpy as np
+
+from . import _ffi
+
+SEED_CFG1 = 0xC0FFEE01  # single bf16 GEMV 896 x 4864
+SEED_CFG2 = 0xC0FFEE02  # Qwen3-0.6B-shape decode
+SEED_CFG3 = 0xC0FFEE03  # Q8_0 GEMV 2048 -> 5632
+SEED_CFG4 = 0xC0FFEE04  # Q4_0 GEMV 1536 -> 151936
+SEED_CFG5 = 0xC0FFEE05  # prefill GEMM + long-context attention
+
+
+def _ptr(a: np.ndarray):
+    return a.ctypes.data
+
+
+def normal_f32(seed: int, n: int, scale: float = 1.0, first: int = 0) -> np.ndarray:
+    out = np.empty(n, dtype=np.float32)
+    _ffi.load().hm_synth_normal_f32(seed, first, n, scale, _ptr(out))
+    return out
+
+
+def normal_bf16(seed: int, n: int, scale: float = 1.0, first: int = 0) -> np.ndarray:
+    """bf16 bit patterns (uint16) of round-to-nearest-even(N(0,1) * scale)."""
+    out = np.empty(n, dtype=np.uint16)
+    _ffi.load().hm_synth_normal_bf16(seed, first, n, scale, _ptr(out))
+    return out
+
+
+def token_ids(seed: int, n: int, vocab: int) -> np.ndarray:
+    out = np.empty(n, dtype=np.int64)
+    _ffi.load().hm_synth_token_ids(seed, n, vocab, _ptr(out))
+    return out
+
+
+def q8_0_blocks(seed: int, n_blocks: int, d_scale: float = 0.01) -> np.ndarray:
+    out = np.empty(n_blocks * 34, dtype=np.uint8)
+    _ffi.load().hm_synth_q8_0(seed, n_blocks, d_scale, _ptr(out))
+    return out
+
+
+def q4_0_blocks(seed: int, n_blocks: int, d_scale: float = 0.01) -> np.ndarray:
+    out = np.empty(n_blocks * 18, dtype=np.uint8)
+    _ffi.load().hm_synth_q4_0(seed, n_blocks, d_scale, _ptr(out))
+    return out
+
+
+def bf16_to_f32(bits: np.ndarray) -> np.ndarray:
+    return (bits.astype(np.uint32) << 16).view(np.float32)
+
+
+def f32_to_bf16_rne(x: np.ndarray) -> np.ndarray:
+    u = np.ascontiguousarray(x, dtype=np.float32).view(np.uint32).astype(np.uint64)
+    lsb = (u >> 16) & 1
+    return ((u + 0x7FFF + lsb) >> 16).astype(np.uint16)

@@ -1,0 +1,252 @@
+/*
+ * homura_amd — MI355X (gfx950) kernels for Homura's batch-1 decode hot path.
+ *
+ * This header is the drop-in boundary. In the reference every heavy op is a symbol
+ * `_mlir__mlir_ciface_k{idx}(void** args)` in a dlopen'ed CPU kernel library, called by
+ * `CompiledGraph::run_with_output_bufs` (reference src/runtime.rs:930-1037) with memref
+ * descriptors built by `build_memref_descriptor` (src/runtime.rs:664-698). Here the same
+ * ops are plain C entry points over HBM-resident buffers: pointers named `d_*` are device
+ * pointers obtained from hm_alloc(); everything else is host memory. Each entry point cites
+ * the reference kernel it stands in for.
+ *
+ * Conventions
+ *  - every function returns HM_OK (0) or a negative HM_ERR_*; hm_last_error() gives the text.
+ *    (The reference's kernels return void and panic in Rust; a GPU call can fail, so the
+ *    boundary carries a status.)
+ *  - one hm_ctx = one GPU + one HIP stream; all kernels are enqueued on that stream and are
+ *    asynchronous; hm_download() and hm_sync() are the blocking calls. One host thread per
+ *    context at a time (the reference serialises runs under a Mutex, src/hf/model.rs:205).
+ *  - activations, norms, logits are f32; bf16 values travel as uint16_t (top half of an f32,
+ *    reference src/hf/safetensors.rs:105-115); quantised weights are raw GGUF block bytes.
+ */
+#ifndef HOMURA_AMD_H
+#define HOMURA_AMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* every declaration below is exported from libhomura_amd.so */
+#pragma GCC visibility push(default)
+
+#define HM_OK 0
+#define HM_ERR_INVALID (-1) /* bad argument / shape the kernels do not support */
+#define HM_ERR_HIP (-2)     /* a HIP runtime call failed */
+#define HM_ERR_OOM (-3)     /* device allocation failed */
+#define HM_ERR_STATE (-4)   /* call made in the wrong state (e.g. KV cache full) */
+
+typedef struct hm_ctx hm_ctx;
+
+/* ── context, memory, stream (replaces the reference's Vec<u8>-backed Buffer,
+ *    src/runtime.rs:35-299, for device residency) ───────────────────────────── */
+hm_ctx *hm_init(int device);       /* NULL on failure: see hm_last_error(NULL) */
+void hm_destroy(hm_ctx *ctx);
+const char *hm_last_error(hm_ctx *ctx); /* ctx may be NULL for hm_init failures */
+int hm_alloc(hm_ctx *ctx, size_t bytes, void **d_out);
+int hm_free(hm_ctx *ctx, void *d_ptr);
+int hm_upload(hm_ctx *ctx, void *d_dst, const void *h_src, size_t bytes);
+int hm_download(hm_ctx *ctx, void *h_dst, const void *d_src, size_t bytes);
+int hm_copy(hm_ctx *ctx, void *d_dst, const void *d_src, size_t bytes);
+int hm_fill_zero(hm_ctx *ctx, void *d_dst, size_t bytes);
+int hm_sync(hm_ctx *ctx);
+void *hm_stream(hm_ctx *ctx); /* the context's hipStream_t */
+int hm_device_name(hm_ctx *ctx, char *buf, size_t buflen);
+
+/* HIP-event timing on the context stream (the GPU-side analogue of the reference's
+ * HOMURA_PROFILE Instant timers, src/runtime.rs:1676-1681). */
+int hm_event_create(hm_ctx *ctx, void **ev_out);
+int hm_event_destroy(hm_ctx *ctx, void *ev);
+int hm_event_record(hm_ctx *ctx, void *ev);
+int hm_event_elapsed_ms(hm_ctx *ctx, void *ev_start, void *ev_stop, float *ms_out);
+
+/* ── heavy ops ─────────────────────────────────────────────────────────────── */
+
+/* bf16-weight matmul, reference GraphBuilder::emit_matmul 3D x 2D arm with the mixed
+ * f32 x bf16 region (src/graph_builder/emit_linalg.rs:1328-1339, :1928-2008, :2224-2307):
+ * out[m,n] = sum_k x[m,k] * f32(W[k,n]); x f32 [M,K], W bf16 [K,N] row-major (the layout
+ * the reference hands its kernels, src/hf/weights.rs:225-261), out f32 [M,N].
+ * M <= 8. K % 8 == 0, N % 8 == 0. */
+int hm_gemv_bf16(hm_ctx *ctx, const float *d_x, const uint16_t *d_w_kn, float *d_out, int M,
+                 int K, int N);
+
+/* One-time re-pack of a [K,N] bf16 weight into the K-contiguous [N,K] stream layout
+ * (which is also HuggingFace's native [out,in] layout, i.e. the reference's load-time
+ * transpose_2d of src/hf/weights.rs:225-261 undone). */
+int hm_pack_bf16_kn_to_nk(hm_ctx *ctx, const uint16_t *d_w_kn, uint16_t *d_w_nk, int K, int N);
+
+/* Same contraction as hm_gemv_bf16 on the [N,K] stream layout. M <= 8, K % 8 == 0. */
+int hm_gemv_bf16_nk(hm_ctx *ctx, const float *d_x, const uint16_t *d_w_nk, float *d_out, int M,
+                    int K, int N);
+
+/* Q8_0 dequant-matmul, reference emit_dequant_matmul_q8_0
+ * (src/graph_builder/emit_quant.rs:30-142): weight = raw GGUF blocks [N][K/32] x 34 bytes
+ * (LE f16 d + 32 int8), out[m,n] = sum_k x[m,k] * (q * d). M <= 8, K % 32 == 0. */
+int hm_gemv_q8_0(hm_ctx *ctx, const float *d_x, const uint8_t *d_w_blocks, float *d_out, int M,
+                 int K, int N);
+
+/* Q4_0 dequant-matmul. The reference parses the type (src/gguf.rs:28,116,141) but has no
+ * kernel for it (src/gguf.rs:94-108); blocks are ggml block_q4_0: [N][K/32] x 18 bytes
+ * (LE f16 d + 16 bytes, byte j = element j low nibble, element j+16 high nibble),
+ * w = (q - 8) * d. M <= 8, K % 32 == 0. */
+int hm_gemv_q4_0(hm_ctx *ctx, const float *d_x, const uint8_t *d_w_blocks, float *d_out, int M,
+                 int K, int N);
+
+/* Block dequantisation to f32, reference dequant_q8_0 (src/gguf.rs:817-831): one f32
+ * multiply per element, bit-exact with the CPU. hm_dequant_q4_0 is its Q4_0 analogue. */
+int hm_dequant_q8_0(hm_ctx *ctx, const uint8_t *d_blocks, float *d_out, size_t nblocks);
+int hm_dequant_q4_0(hm_ctx *ctx, const uint8_t *d_blocks, float *d_out, size_t nblocks);
+
+/* Prefill-chunk GEMM on the matrix cores: the reference runs the same emit_matmul with
+ * seq > 1 (docs/kv-cache.md:31-37); here A bf16 [M,K], B bf16 [K,N] (reference layout),
+ * C f32 [M,N], f32 accumulate. M % 128 == 0, N % 128 == 0, K % 32 == 0. */
+int hm_gemm_bf16(hm_ctx *ctx, const uint16_t *d_a_mk, const uint16_t *d_b_kn, float *d_c, int M,
+                 int K, int N);
+
+/* ── KV cache + attention ──────────────────────────────────────────────────── */
+
+/* KvCache::append_key / append_value (src/runtime.rs:521-568) on an HBM cache
+ * [B][kvh][max_len][hd] bf16: rows d_k/d_v f32 [B][kvh][n_new][hd] (BHSD, as the
+ * reference's QKV kernel emits them) are rounded to bf16 (nearest-even) and written at
+ * row `pos`. Fails with HM_ERR_STATE when pos + n_new > max_len (the reference panics
+ * "KV cache full"). */
+int hm_kv_append(hm_ctx *ctx, uint16_t *d_kcache, uint16_t *d_vcache, const float *d_k,
+                 const float *d_v, int B, int kvh, int hd, int max_len, int pos, int n_new);
+
+/* Decode attention, the attention part of reference emit_attention_kernel
+ * (src/hf/emitter.rs:709-737; emit_gqa_qk_transpose / emit_softmax / emit_gqa_av,
+ * src/graph_builder/emit_linalg.rs:93-245, :509-528): one query row per sequence,
+ * q f32 [B][H][hd]; K,V bf16 caches [B][kvh][max_len][hd] of which rows [0,kv_len) are
+ * attended (the all-zero decode mask of src/hf/precompute.rs:49-64); kv head = h / (H/kvh);
+ * scores * scale, softmax in f32, out f32 [B][H*hd]. hd == 128 or 64. */
+int hm_gqa_decode_attn(hm_ctx *ctx, const float *d_q, const uint16_t *d_kcache,
+                       const uint16_t *d_vcache, float *d_out, int B, int H, int kvh, int hd,
+                       int max_len, int kv_len, float scale);
+
+/* ── light ops ─────────────────────────────────────────────────────────────── */
+
+/* emit_rms_norm (src/graph_builder/emit_linalg.rs:7-26): out = (x * rsqrt(mean(x^2)+eps)) * w
+ * per row; x,out f32 [rows][dim], w f32 [dim]. */
+int hm_rmsnorm(hm_ctx *ctx, const float *d_x, const float *d_w, float *d_out, int rows, int dim,
+               float eps);
+
+/* The per-head QK-norm + emit_rope_half tail of emit_qkv_kernel (src/hf/emitter.rs:629-644,
+ * src/graph_builder/emit_linalg.rs:315-342), in place: q f32 [S][H][hd], k f32 [S][kvh][hd];
+ * d_qw/d_kw f32 [hd] or NULL (no QK-norm); cos/sin f32 [S][hd] (rows already sliced for the
+ * positions, src/hf/precompute.rs:73-101). */
+int hm_qknorm_rope(hm_ctx *ctx, float *d_q, float *d_k, const float *d_qw, const float *d_kw,
+                   const float *d_cos, const float *d_sin, int S, int H, int kvh, int hd,
+                   float eps);
+
+/* silu(gate) * up (src/graph_builder/emit_arithmetic.rs:101-107, src/hf/emitter.rs:797-799). */
+int hm_silu_mul(hm_ctx *ctx, const float *d_gate, const float *d_up, float *d_out, size_t n);
+/* residual add (src/hf/emitter.rs:787, :804). */
+int hm_add(hm_ctx *ctx, const float *d_a, const float *d_b, float *d_out, size_t n);
+/* emit_embed_kernel (src/hf/emitter.rs:506-537): out[i,:] = table[ids[i],:]. */
+int hm_embed(hm_ctx *ctx, const int64_t *d_ids, const float *d_table, float *d_out, int n_ids,
+             int vocab, int hidden);
+/* greedy pick of src/generate.rs:457-468 / :735-742: index of the maximum; of equal maxima
+ * the LAST (Rust Iterator::max_by). Writes one int32 to d_index_out. */
+int hm_argmax(hm_ctx *ctx, const float *d_values, int n, int32_t *d_index_out);
+
+/* ── host-side mirror of Model / ExecutionPlan / KvCache, C view ─────────────
+ * The C++ classes in homura_amd/csrc/host/ keep the reference's names (HfModel,
+ * ExecutionPlan, KernelStep, KvCache, Buffer); these functions are their C handles. */
+
+typedef struct hm_model hm_model;
+
+/* reference TransformerConfig (src/hf/config.rs:11-73) */
+typedef struct {
+    int hidden_size;
+    int intermediate_size;
+    int num_attention_heads;
+    int num_hidden_layers;
+    int num_key_value_heads; /* 0 => num_attention_heads */
+    int vocab_size;
+    int head_dim;            /* 0 => hidden_size / num_attention_heads */
+    int max_position_embeddings;
+    int tie_word_embeddings;
+    double rms_norm_eps;
+    double rope_theta;
+} hm_transformer_config;
+
+#define HM_DTYPE_F32 0
+#define HM_DTYPE_BF16 1
+#define HM_DTYPE_Q8_0 2
+#define HM_DTYPE_Q4_0 3
+#define HM_DTYPE_I64 4
+
+/* HfModel::load_with_dtype / load_gguf stand-in (src/hf/model.rs:46-145) for weights that
+ * are already in host memory: create, hand over every weight slot in
+ * TransformerWeights::to_slot_buffers order (src/hf/weights.rs:63-116, :136-183), finalize.
+ * `weight_dtype` is the dtype of the seven projections (BF16, Q8_0 or Q4_0). */
+hm_model *hm_model_create(hm_ctx *ctx, const hm_transformer_config *cfg, int weight_dtype,
+                          int has_qk_norm);
+void hm_model_destroy(hm_model *m);
+int hm_model_num_weight_slots(hm_model *m);
+/* name is copied into buf; dtype/rows/cols describe the host buffer expected for the slot */
+int hm_model_weight_slot_info(hm_model *m, int slot, char *name_buf, size_t buflen, int *dtype,
+                              int64_t *dim0, int64_t *dim1, size_t *bytes);
+int hm_model_set_weight(hm_model *m, int slot, const void *h_data, size_t bytes);
+/* ensure_compiled (src/hf/model.rs:148-160): builds the ExecutionPlan, RoPE tables, packs. */
+int hm_model_finalize(hm_model *m, int max_seq_len);
+
+/* ExecutionPlan::init_kv_cache (src/runtime.rs:1898-1938): h_kv = 2*layers host buffers
+ * (K,V alternating) of f32 [1][kvh][seq_len][hd]; rounds to bf16 into the HBM cache. */
+int hm_model_init_kv_cache(hm_model *m, const float *const *h_kv, int seq_len);
+int hm_model_reset_kv_cache(hm_model *m);  /* src/runtime.rs:1941-1945 */
+int hm_model_kv_cache_len(hm_model *m);    /* src/runtime.rs:1948-1950 */
+
+/* HfModel::run_kv (src/hf/model.rs:198-218) -> ExecutionPlan::run_kv
+ * (src/runtime.rs:1580-1892): n_ids new tokens on top of the cache; h_logits receives
+ * [n_ids][vocab] f32 (may be NULL to skip the download). Advances the cache by n_ids. */
+int hm_model_run_kv(hm_model *m, const int64_t *h_ids, int n_ids, float *h_logits);
+
+/* The greedy loop of generate_streaming_core (src/generate.rs:187-270) with pure argmax:
+ * the prompt is consumed as incremental prefill through run_kv, then n_new tokens are
+ * produced with the argmax taken on the device and fed straight back, no per-token host
+ * round trip. h_tokens_out receives n_new ids. */
+int hm_model_generate_greedy(hm_model *m, const int64_t *h_prompt, int n_prompt, int n_new,
+                             int32_t *h_tokens_out);
+
+/* Timed decode for benchmarking: runs `n_steps` decode steps starting from token `first_id`
+ * (greedy feedback on device), returns total milliseconds measured with HIP events on the
+ * context stream. */
+int hm_model_bench_decode(hm_model *m, int64_t first_id, int n_steps, float *ms_out,
+                          int32_t *h_tokens_out);
+
+/* Per-kernel profile of one decode step (HOMURA_PROFILE analogue): fills up to `cap`
+ * records; returns the number written. */
+typedef struct {
+    char label[32]; /* "Embed", "QKV", "KVConcat", "Attn", "O", "GateUp", "Down", "LMHead", ... */
+    float ms;       /* summed over layers */
+    int launches;
+    double bytes;   /* algorithmic bytes moved by these launches */
+} hm_kernel_profile;
+int hm_model_profile_step(hm_model *m, int64_t token_id, hm_kernel_profile *out, int cap);
+
+/* ── deterministic synthetic data (host side, no GPU needed) ─────────────────
+ * Counter-based generator shared by tests and benchmarks: sample i of stream `seed` uses
+ * outputs 3i..3i+2 of the splitmix64 sequence seeded with `seed`; a normal variate is the
+ * centred sum of the twelve 16-bit fields of those outputs (Irwin-Hall, unit variance),
+ * computed in integers so that every platform produces the same bits. */
+void hm_synth_normal_f32(uint64_t seed, uint64_t first, size_t n, float scale, float *out);
+void hm_synth_normal_bf16(uint64_t seed, uint64_t first, size_t n, float scale, uint16_t *out);
+void hm_synth_token_ids(uint64_t seed, size_t n, int vocab, int64_t *out);
+/* n_blocks Q8_0 blocks: q uniform in [-127,127], d = f16(|N(0,1)| * d_scale) */
+void hm_synth_q8_0(uint64_t seed, size_t n_blocks, float d_scale, uint8_t *out);
+/* n_blocks Q4_0 blocks: nibbles uniform in [0,15], d = f16(|N(0,1)| * d_scale) */
+void hm_synth_q4_0(uint64_t seed, size_t n_blocks, float d_scale, uint8_t *out);
+uint16_t hm_f32_to_bf16_rne(float v);
+uint16_t hm_f32_to_f16_rne(float v);
+
+const char *hm_version(void);
+
+#pragma GCC visibility pop
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* HOMURA_AMD_H */

@@ -1,0 +1,840 @@
+/*
+ * CPU oracle for the batch-1 decode hot path of edg-l/homura.
+ *
+ * THIS FILE IS TEST INFRASTRUCTURE. It is a plain-C restatement of what the
+ * reference's generated CPU kernels compute, written from the reference's Rust
+ * sources (cited per function as file:line, relative to the reference tree).
+ * Only the test-suite, the smoke check and the CPU-baseline leg of the
+ * benchmark may call it; the product library never links or loads it.
+ *
+ * Pinning status (which independent evidence fixes each function):
+ *   orc_f16_to_f32 ........ exhaustive vs numpy float16 (65536 patterns) + 0x3C00/0x3800/0x3400
+ *   orc_dequant_q8_0 ...... single f32 multiply; reference KAT d=1,q=1..32
+ *   orc_gemv_q8_0 ......... reference KAT (528 per output) + fp64 brute force
+ *   orc_dequant_q4_0 / orc_gemv_q4_0 .. PARITY UNPINNED in the reference (it has no
+ *                           Q4_0 kernel); pinned only by the published ggml block_q4_0
+ *                           layout and the formula w=(q-8)*d, cross-checked with an
+ *                           independent numpy decode.
+ *   orc_matmul_* .......... reference exact vectors ([[19,22],[43,50]], identity cases),
+ *                           fp64 brute force
+ *   orc_rms_norm* ......... reference rms_norm_basic + closed form
+ *   orc_silu_mul .......... reference silu_basic closed form
+ *   orc_softmax* .......... reference softmax vectors ([.0900,.2447,.6652], sigma=1/(1+e))
+ *   orc_rope_tables ....... reference rope_basic_values
+ *   orc_rope_half ......... PARITY UNPINNED by a reference value test (none feeds
+ *                           emit_rope_half); pinned by the rotate_half closed form,
+ *                           identity at position 0 and pairwise norm preservation.
+ *   orc_gqa_attention ..... reference repeat_kv head order, uniform-K => mean(V),
+ *                           one-hot score => that V row, fp64 brute force
+ *   orc_kv_* .............. reference KvCache exact arrays
+ *   orc_argmax_last ....... reference greedy vector + Rust max_by tie rule
+ *   orc_model_run_kv ...... composition of the above following the reference's step list;
+ *                           end-to-end logits of a real checkpoint are PARITY UNPINNED
+ *                           (the reference's golden files for that are not shipped).
+ */
+#include <math.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+#include <stdio.h>
+
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+#define ORC_API __attribute__((visibility("default")))
+
+/* ───────────────────────── scalar conversions ───────────────────────── */
+
+/* src/gguf.rs:781-810 — IEEE half bits to f32, subnormals/inf/NaN handled by hand. */
+ORC_API float orc_f16_to_f32(uint16_t bits) {
+    uint32_t sign = (bits >> 15) & 1u;
+    uint32_t exp = (bits >> 10) & 0x1Fu;
+    uint32_t frac = bits & 0x3FFu;
+    uint32_t out;
+    if (exp == 0) {
+        if (frac == 0) {
+            out = sign << 31;
+        } else {
+            int e = 0;
+            uint32_t f = frac;
+            while ((f & 0x400u) == 0) {
+                f <<= 1;
+                e -= 1;
+            }
+            f &= 0x3FFu;
+            uint32_t exp32 = (uint32_t)(127 - 15 + 1 + e);
+            out = (sign << 31) | (exp32 << 23) | (f << 13);
+        }
+    } else if (exp == 31) {
+        out = (sign << 31) | (0xFFu << 23) | (frac << 13);
+    } else {
+        uint32_t exp32 = (uint32_t)((int)exp - 15 + 127);
+        out = (sign << 31) | (exp32 << 23) | (frac << 13);
+    }
+    float r;
+    memcpy(&r, &out, 4);
+    return r;
+}
+
+/* Array form of the above (results stored as bits, so signalling NaNs survive the trip). */
+ORC_API void orc_f16_to_f32_array(const uint16_t *bits, size_t n, float *out) {
+    for (size_t i = 0; i < n; i++) out[i] = orc_f16_to_f32(bits[i]);
+}
+
+/* src/hf/safetensors.rs:105-115, src/hf/weights.rs:197-204 — bf16 is the top half of an f32. */
+static inline float bf16_to_f32(uint16_t b) {
+    uint32_t u = (uint32_t)b << 16;
+    float r;
+    memcpy(&r, &u, 4);
+    return r;
+}
+ORC_API float orc_bf16_to_f32(uint16_t b) { return bf16_to_f32(b); }
+
+/* src/hf/weights.rs:206-214 — f32 to bf16 by truncation (used for the tied LM head). */
+ORC_API uint16_t orc_f32_to_bf16_trunc(float v) {
+    uint32_t u;
+    memcpy(&u, &v, 4);
+    return (uint16_t)(u >> 16);
+}
+
+/* Round-to-nearest-even f32 to bf16. Not in the reference (its KV cache is f32,
+ * src/runtime.rs:1593-1599); used for the documented bf16-KV deviation so that the
+ * oracle and the GPU round new K/V rows identically. */
+ORC_API uint16_t orc_f32_to_bf16_rne(float v) {
+    uint32_t u;
+    memcpy(&u, &v, 4);
+    if ((u & 0x7F800000u) == 0x7F800000u && (u & 0x007FFFFFu)) return (uint16_t)((u >> 16) | 0x40u);
+    uint32_t lsb = (u >> 16) & 1u;
+    u += 0x7FFFu + lsb;
+    return (uint16_t)(u >> 16);
+}
+
+/* ───────────────────────── block dequantisation ───────────────────────── */
+
+/* src/gguf.rs:817-831 — Q8_0: 34-byte blocks, LE f16 scale then 32 int8; x = q * d. */
+ORC_API void orc_dequant_q8_0(const uint8_t *src, size_t nblocks, float *dst) {
+#pragma omp parallel for schedule(static)
+    for (size_t b = 0; b < nblocks; b++) {
+        const uint8_t *blk = src + b * 34;
+        float d = orc_f16_to_f32((uint16_t)(blk[0] | (blk[1] << 8)));
+        for (int j = 0; j < 32; j++) {
+            int8_t q = (int8_t)blk[2 + j];
+            dst[b * 32 + j] = (float)q * d;
+        }
+    }
+}
+
+/* Q4_0 — absent from the reference (src/gguf.rs:94-108 rejects it; sizes only at :116,:141).
+ * ggml block_q4_0: LE f16 d, then 16 bytes; byte j carries element j in its low nibble and
+ * element j+16 in its high nibble; x = (q - 8) * d. The low-then-high nibble order is the
+ * same convention the reference uses for Q4_K (src/gguf.rs:864-878). */
+ORC_API void orc_dequant_q4_0(const uint8_t *src, size_t nblocks, float *dst) {
+#pragma omp parallel for schedule(static)
+    for (size_t b = 0; b < nblocks; b++) {
+        const uint8_t *blk = src + b * 18;
+        float d = orc_f16_to_f32((uint16_t)(blk[0] | (blk[1] << 8)));
+        for (int j = 0; j < 16; j++) {
+            int lo = (blk[2 + j] & 0x0F) - 8;
+            int hi = (blk[2 + j] >> 4) - 8;
+            dst[b * 32 + j] = (float)lo * d;
+            dst[b * 32 + j + 16] = (float)hi * d;
+        }
+    }
+}
+
+/* ───────────────────────── matmul family ───────────────────────── */
+
+/* src/graph_builder/mod.rs:60-75 — forall tile over N: max(16, pow2_floor(N / (1.5*cores))). */
+static int tile_parallel_n_tile(int n, int cores) {
+    int target = cores + cores / 2;
+    int ideal = target > 0 ? n / target : n;
+    int t = 1;
+    if (ideal > 1) {
+        t = 1;
+        while ((t << 1) <= ideal) t <<= 1;
+    }
+    if (t < 16) t = 16;
+    return t;
+}
+
+static int host_cores(void) {
+#ifdef _OPENMP
+    return omp_get_max_threads();
+#else
+    return 1;
+#endif
+}
+
+/* src/graph_builder/emit_linalg.rs:1328-1339, :1928-2008, :2224-2307 with the TileParallel
+ * schedule of src/compiler.rs:1585-1597: out[m,n] = sum_k x[m,k] * f32(W[k,n]); the
+ * accumulator starts at zero, N is tiled across threads, K runs ascending in the outer loop
+ * and N is innermost, so every output sums its K terms in ascending order. bf16 widens by a
+ * 16-bit shift; mul+add may contract to FMA (src/compiler.rs:89-111). */
+ORC_API void orc_matmul_f32_bf16(const float *x, const uint16_t *w_kn, float *out, int M, int K,
+                                 int N) {
+    int n_tile = tile_parallel_n_tile(N, host_cores());
+    int tiles = (N + n_tile - 1) / n_tile;
+#pragma omp parallel for schedule(dynamic, 1)
+    for (int t = 0; t < tiles; t++) {
+        int n0 = t * n_tile;
+        int n1 = n0 + n_tile < N ? n0 + n_tile : N;
+        for (int m = 0; m < M; m++) {
+            float *o = out + (size_t)m * N;
+            for (int n = n0; n < n1; n++) o[n] = 0.0f;
+            const float *xr = x + (size_t)m * K;
+            for (int k = 0; k < K; k++) {
+                float xk = xr[k];
+                const uint16_t *wr = w_kn + (size_t)k * N;
+                for (int n = n0; n < n1; n++) o[n] += xk * bf16_to_f32(wr[n]);
+            }
+        }
+    }
+}
+
+/* Same contraction with f32 weights (the quantised plan keeps the LM head in f32:
+ * src/hf/emitter_quant.rs:1399-1440, src/hf/weights.rs:174-180). */
+ORC_API void orc_matmul_f32_f32(const float *x, const float *w_kn, float *out, int M, int K,
+                                int N) {
+    int n_tile = tile_parallel_n_tile(N, host_cores());
+    int tiles = (N + n_tile - 1) / n_tile;
+#pragma omp parallel for schedule(dynamic, 1)
+    for (int t = 0; t < tiles; t++) {
+        int n0 = t * n_tile;
+        int n1 = n0 + n_tile < N ? n0 + n_tile : N;
+        for (int m = 0; m < M; m++) {
+            float *o = out + (size_t)m * N;
+            for (int n = n0; n < n1; n++) o[n] = 0.0f;
+            const float *xr = x + (size_t)m * K;
+            for (int k = 0; k < K; k++) {
+                float xk = xr[k];
+                const float *wr = w_kn + (size_t)k * N;
+                for (int n = n0; n < n1; n++) o[n] += xk * wr[n];
+            }
+        }
+    }
+}
+
+/* bf16 x bf16 GEMM of the prefill chunk: the reference runs the same mixed matmul with both
+ * operands widened to f32 (src/graph_builder/emit_linalg.rs:2238-2267). */
+ORC_API void orc_matmul_bf16_bf16(const uint16_t *a_mk, const uint16_t *b_kn, float *out, int M,
+                                  int K, int N) {
+#pragma omp parallel for schedule(dynamic, 1)
+    for (int m = 0; m < M; m++) {
+        float *o = out + (size_t)m * N;
+        for (int n = 0; n < N; n++) o[n] = 0.0f;
+        for (int k = 0; k < K; k++) {
+            float ak = bf16_to_f32(a_mk[(size_t)m * K + k]);
+            const uint16_t *br = b_kn + (size_t)k * N;
+            for (int n = 0; n < N; n++) o[n] += ak * bf16_to_f32(br[n]);
+        }
+    }
+}
+
+/* src/graph_builder/emit_quant.rs:30-142 — per output: for each 32-block, dequantise
+ * (f32(q) * f32(d)), multiply by 32 activations, horizontal add, then acc += dot, blocks
+ * in ascending order. Weight bytes are [N][K/32] blocks of 34. */
+ORC_API void orc_gemv_q8_0(const float *x, const uint8_t *w, float *out, int M, int K, int N) {
+    int nb = K / 32;
+#pragma omp parallel for schedule(static)
+    for (int n = 0; n < N; n++) {
+        for (int m = 0; m < M; m++) {
+            const float *xr = x + (size_t)m * K;
+            float acc = 0.0f;
+            for (int kb = 0; kb < nb; kb++) {
+                const uint8_t *blk = w + ((size_t)n * nb + kb) * 34;
+                float d = orc_f16_to_f32((uint16_t)(blk[0] | (blk[1] << 8)));
+                float dot = 0.0f;
+                for (int j = 0; j < 32; j++) {
+                    float dq = (float)(int8_t)blk[2 + j] * d;
+                    dot += dq * xr[kb * 32 + j];
+                }
+                acc += dot;
+            }
+            out[(size_t)m * N + n] = acc;
+        }
+    }
+}
+
+/* Q4_0 analogue of the above (no reference kernel; see orc_dequant_q4_0). */
+ORC_API void orc_gemv_q4_0(const float *x, const uint8_t *w, float *out, int M, int K, int N) {
+    int nb = K / 32;
+#pragma omp parallel for schedule(static)
+    for (int n = 0; n < N; n++) {
+        for (int m = 0; m < M; m++) {
+            const float *xr = x + (size_t)m * K;
+            float acc = 0.0f;
+            for (int kb = 0; kb < nb; kb++) {
+                const uint8_t *blk = w + ((size_t)n * nb + kb) * 18;
+                float d = orc_f16_to_f32((uint16_t)(blk[0] | (blk[1] << 8)));
+                float dot = 0.0f;
+                for (int j = 0; j < 16; j++) {
+                    float lo = (float)((blk[2 + j] & 0x0F) - 8) * d;
+                    dot += lo * xr[kb * 32 + j];
+                }
+                for (int j = 0; j < 16; j++) {
+                    float hi = (float)((blk[2 + j] >> 4) - 8) * d;
+                    dot += hi * xr[kb * 32 + 16 + j];
+                }
+                acc += dot;
+            }
+            out[(size_t)m * N + n] = acc;
+        }
+    }
+}
+
+/* ───────────────────────── light ops ───────────────────────── */
+
+/* src/graph_builder/emit_linalg.rs:7-26 with reduce_mean :379-498 —
+ * (x * rsqrt(sum(x*x)/count + eps)) * w, f32 throughout, sequential sum. */
+ORC_API void orc_rms_norm(const float *x, const float *w, float *out, int rows, int dim,
+                          float eps) {
+    for (int r = 0; r < rows; r++) {
+        const float *xr = x + (size_t)r * dim;
+        float s = 0.0f;
+        for (int i = 0; i < dim; i++) s += xr[i] * xr[i];
+        float var = s / (float)dim;
+        float inv = 1.0f / sqrtf(var + eps);
+        for (int i = 0; i < dim; i++) out[(size_t)r * dim + i] = (xr[i] * inv) * w[i];
+    }
+}
+
+/* src/hf/emitter_quant.rs:713-791 and src/graph_builder/emit_linalg.rs:33-56 — the quantised
+ * plan's variant: sum of squares in f64, mean = sum * (1/dim) in f64, truncate to f32,
+ * + eps, 1 / sqrt. */
+ORC_API void orc_rms_norm_f64acc(const float *x, const float *w, float *out, int rows, int dim,
+                                 float eps) {
+    double inv_n = 1.0 / (double)dim;
+    for (int r = 0; r < rows; r++) {
+        const float *xr = x + (size_t)r * dim;
+        double s = 0.0;
+        for (int i = 0; i < dim; i++) s += (double)xr[i] * (double)xr[i];
+        float mean = (float)(s * inv_n);
+        float scale = 1.0f / sqrtf(mean + eps);
+        for (int i = 0; i < dim; i++) out[(size_t)r * dim + i] = (xr[i] * scale) * w[i];
+    }
+}
+
+/* src/graph_builder/emit_linalg.rs:33-56 — the graph-builder variant used for the quantised
+ * plan's QK-norm (src/hf/emitter_quant.rs:869-878) and LM-head norm (:1411): x*x in f32,
+ * widened to f64, mean = f64 sum / count, truncated to f32, + eps, rsqrt. */
+ORC_API void orc_rms_norm_f64mean(const float *x, const float *w, float *out, int rows, int dim,
+                                  float eps) {
+    for (int r = 0; r < rows; r++) {
+        const float *xr = x + (size_t)r * dim;
+        double s = 0.0;
+        for (int i = 0; i < dim; i++) s += (double)(xr[i] * xr[i]);
+        float var = (float)(s / (double)dim);
+        float inv = 1.0f / sqrtf(var + eps);
+        for (int i = 0; i < dim; i++) out[(size_t)r * dim + i] = (xr[i] * inv) * w[i];
+    }
+}
+
+/* src/graph_builder/emit_arithmetic.rs:101-107 and src/hf/emitter.rs:797-799 —
+ * silu(g) * u with silu(g) = g / (1 + exp(-g)). */
+ORC_API void orc_silu_mul(const float *gate, const float *up, float *out, size_t n) {
+    for (size_t i = 0; i < n; i++) {
+        float g = gate[i];
+        out[i] = (g / (1.0f + expf(-g))) * up[i];
+    }
+}
+
+ORC_API void orc_add(const float *a, const float *b, float *out, size_t n) {
+    for (size_t i = 0; i < n; i++) out[i] = a[i] + b[i];
+}
+
+/* src/graph_builder/emit_linalg.rs:509-528 — max, subtract, exp, sum, divide. */
+ORC_API void orc_softmax(const float *x, float *out, int rows, int n) {
+    for (int r = 0; r < rows; r++) {
+        const float *xr = x + (size_t)r * n;
+        float *o = out + (size_t)r * n;
+        float mx = -INFINITY;
+        for (int i = 0; i < n; i++) mx = xr[i] > mx ? xr[i] : mx;
+        float s = 0.0f;
+        for (int i = 0; i < n; i++) {
+            o[i] = expf(xr[i] - mx);
+            s += o[i];
+        }
+        for (int i = 0; i < n; i++) o[i] = o[i] / s;
+    }
+}
+
+/* src/graph_builder/emit_linalg.rs:534-555 — same with the sum of exps taken in f64. */
+ORC_API void orc_softmax_f64acc(const float *x, float *out, int rows, int n) {
+    for (int r = 0; r < rows; r++) {
+        const float *xr = x + (size_t)r * n;
+        float *o = out + (size_t)r * n;
+        float mx = -INFINITY;
+        for (int i = 0; i < n; i++) mx = xr[i] > mx ? xr[i] : mx;
+        double s = 0.0;
+        for (int i = 0; i < n; i++) {
+            o[i] = expf(xr[i] - mx);
+            s += (double)o[i];
+        }
+        float sf = (float)s;
+        for (int i = 0; i < n; i++) o[i] = o[i] / sf;
+    }
+}
+
+/* src/hf/precompute.rs:10-40 — cos/sin tables [max_pos][head_dim], f64 angle
+ * pos / theta^(2i/head_dim), both halves duplicated. */
+ORC_API void orc_rope_tables(int head_dim, int max_pos, double theta, float *cos_out,
+                             float *sin_out) {
+    int half = head_dim / 2;
+    for (int pos = 0; pos < max_pos; pos++) {
+        for (int i = 0; i < half; i++) {
+            double freq = 1.0 / pow(theta, 2.0 * (double)i / (double)head_dim);
+            double angle = (double)pos * freq;
+            float c = (float)cos(angle);
+            float s = (float)sin(angle);
+            cos_out[(size_t)pos * head_dim + i] = c;
+            cos_out[(size_t)pos * head_dim + half + i] = c;
+            sin_out[(size_t)pos * head_dim + i] = s;
+            sin_out[(size_t)pos * head_dim + half + i] = s;
+        }
+    }
+}
+
+/* src/hf/precompute.rs:49-64 — mask[i][j] = -inf where j > i + past, else 0. */
+ORC_API void orc_causal_mask(int seq, int past, float *mask) {
+    int total = seq + past;
+    for (int i = 0; i < seq; i++)
+        for (int j = 0; j < total; j++) mask[(size_t)i * total + j] = (j > i + past) ? -INFINITY : 0.0f;
+}
+
+/* src/graph_builder/emit_linalg.rs:315-342 — x*cos + rotate_half(x)*sin with
+ * rotate_half(x) = cat(-x[hd/2:], x[:hd/2]); x is [S][heads][hd], cos/sin [S][hd]. In place. */
+ORC_API void orc_rope_half(float *x, const float *cosv, const float *sinv, int S, int heads,
+                           int hd) {
+    int half = hd / 2;
+    float tmp[1024];
+    for (int s = 0; s < S; s++) {
+        const float *c = cosv + (size_t)s * hd;
+        const float *sn = sinv + (size_t)s * hd;
+        for (int h = 0; h < heads; h++) {
+            float *v = x + ((size_t)s * heads + h) * hd;
+            for (int i = 0; i < half; i++) {
+                tmp[i] = -v[half + i];
+                tmp[half + i] = v[i];
+            }
+            for (int i = 0; i < hd; i++) v[i] = v[i] * c[i] + tmp[i] * sn[i];
+        }
+    }
+}
+
+/* src/hf/emitter.rs:506-537, src/graph_builder/emit_linalg.rs:252-254 — row gather. */
+ORC_API void orc_embed(const int64_t *ids, int n_ids, const float *table, int hidden, float *out) {
+    for (int i = 0; i < n_ids; i++)
+        memcpy(out + (size_t)i * hidden, table + (size_t)ids[i] * hidden, (size_t)hidden * 4);
+}
+
+/* src/generate.rs:457-468, :735-742 — Iterator::max_by keeps the LAST of equal maxima;
+ * comparisons involving NaN count as equal. */
+ORC_API int orc_argmax_last(const float *v, int n) {
+    int best = 0;
+    for (int i = 1; i < n; i++) {
+        /* max_by replaces the running maximum unless it compares Greater than the candidate */
+        int greater = v[best] > v[i]; /* false for NaN on either side (=> Equal => replace) */
+        if (!greater) best = i;
+    }
+    return best;
+}
+
+/* ───────────────────────── attention ───────────────────────── */
+
+/* src/hf/emitter.rs:709-737 using src/graph_builder/emit_linalg.rs:93-245 —
+ * q [S][H][hd] (BSHD), K/V views [kvh][total][hd] with a head stride in elements
+ * (src/runtime.rs:600-625), mask [S][total]; scores = Q.K^T over hd with kv head h / g,
+ * scaled by (float)(1/sqrt(hd)), + mask, softmax (f32 or f64-sum), out = P.V;
+ * out [S][H*hd]. `scores_scratch` must hold H*S*total floats. */
+ORC_API void orc_gqa_attention(const float *q, const float *k, const float *v, const float *mask,
+                               float *out, int S, int H, int kvh, int hd, int total,
+                               long head_stride, int f64_softmax, float *scores_scratch) {
+    int g = H / kvh;
+    float scale = (float)(1.0 / sqrt((double)hd));
+#pragma omp parallel for schedule(static)
+    for (int h = 0; h < H; h++) {
+        const float *kh = k + (size_t)(h / g) * head_stride;
+        const float *vh = v + (size_t)(h / g) * head_stride;
+        for (int m = 0; m < S; m++) {
+            const float *qv = q + ((size_t)m * H + h) * hd;
+            float *sc = scores_scratch + ((size_t)h * S + m) * total;
+            for (int n = 0; n < total; n++) {
+                float acc = 0.0f;
+                const float *kr = kh + (size_t)n * hd;
+                for (int d = 0; d < hd; d++) acc += qv[d] * kr[d];
+                sc[n] = acc * scale + mask[(size_t)m * total + n];
+            }
+            if (f64_softmax)
+                orc_softmax_f64acc(sc, sc, 1, total);
+            else
+                orc_softmax(sc, sc, 1, total);
+            float *o = out + ((size_t)m * H + h) * hd;
+            for (int d = 0; d < hd; d++) o[d] = 0.0f;
+            for (int n = 0; n < total; n++) {
+                float p = sc[n];
+                const float *vr = vh + (size_t)n * hd;
+                for (int d = 0; d < hd; d++) o[d] += p * vr[d];
+            }
+        }
+    }
+}
+
+/* ───────────────────────── KV cache ───────────────────────── */
+
+/* src/runtime.rs:355-650 — per layer two f32 buffers [1][heads][max_len][hd], zero-filled. */
+typedef struct {
+    int layers, heads, max_len, hd;
+    int current_len, new_tokens;
+    int round_bf16; /* documented deviation: round appended rows to bf16 (RNE) */
+    float **key;
+    float **value;
+} orc_kv_cache;
+
+ORC_API orc_kv_cache *orc_kv_new(int layers, int heads, int max_len, int hd, int round_bf16) {
+    orc_kv_cache *c = (orc_kv_cache *)calloc(1, sizeof(*c));
+    c->layers = layers;
+    c->heads = heads;
+    c->max_len = max_len;
+    c->hd = hd;
+    c->round_bf16 = round_bf16;
+    c->key = (float **)calloc((size_t)layers, sizeof(float *));
+    c->value = (float **)calloc((size_t)layers, sizeof(float *));
+    size_t n = (size_t)heads * max_len * hd;
+    for (int l = 0; l < layers; l++) {
+        c->key[l] = (float *)calloc(n, sizeof(float));
+        c->value[l] = (float *)calloc(n, sizeof(float));
+    }
+    return c;
+}
+
+ORC_API void orc_kv_free(orc_kv_cache *c) {
+    if (!c) return;
+    for (int l = 0; l < c->layers; l++) {
+        free(c->key[l]);
+        free(c->value[l]);
+    }
+    free(c->key);
+    free(c->value);
+    free(c);
+}
+
+static int kv_append_into(orc_kv_cache *c, float *dst, const float *src, int new_seq) {
+    /* src/runtime.rs:521-568: rows [h][new_seq][hd] go to row current_len of each head */
+    if (c->current_len + new_seq > c->max_len) return -1; /* reference panics "KV cache full" */
+    c->new_tokens = new_seq;
+    for (int h = 0; h < c->heads; h++) {
+        float *d = dst + ((size_t)h * c->max_len + c->current_len) * c->hd;
+        const float *s = src + (size_t)h * new_seq * c->hd;
+        size_t cnt = (size_t)new_seq * c->hd;
+        if (c->round_bf16) {
+            for (size_t i = 0; i < cnt; i++) d[i] = bf16_to_f32(orc_f32_to_bf16_rne(s[i]));
+        } else {
+            memcpy(d, s, cnt * 4);
+        }
+    }
+    return 0;
+}
+
+ORC_API int orc_kv_append_key(orc_kv_cache *c, int layer, const float *new_k, int new_seq) {
+    return kv_append_into(c, c->key[layer], new_k, new_seq);
+}
+ORC_API int orc_kv_append_value(orc_kv_cache *c, int layer, const float *new_v, int new_seq) {
+    return kv_append_into(c, c->value[layer], new_v, new_seq);
+}
+/* src/runtime.rs:635-638 */
+ORC_API void orc_kv_advance_by(orc_kv_cache *c, int n) {
+    c->current_len += n;
+    c->new_tokens = 0;
+}
+/* src/runtime.rs:642-644 */
+ORC_API void orc_kv_reset(orc_kv_cache *c, int initial_len) { c->current_len = initial_len; }
+ORC_API int orc_kv_current_len(const orc_kv_cache *c) { return c->current_len; }
+/* src/runtime.rs:575-625 — zero-copy views cover [0, current_len + new_tokens). */
+ORC_API const float *orc_kv_key_ptr(const orc_kv_cache *c, int layer) { return c->key[layer]; }
+ORC_API const float *orc_kv_value_ptr(const orc_kv_cache *c, int layer) { return c->value[layer]; }
+ORC_API int orc_kv_view_len(const orc_kv_cache *c) { return c->current_len + c->new_tokens; }
+ORC_API long orc_kv_head_stride(const orc_kv_cache *c) { return (long)c->max_len * c->hd; }
+
+/* src/runtime.rs:479-518 (test-only `view`): contiguous copy [heads][current_len][hd]. */
+ORC_API void orc_kv_view_copy(const orc_kv_cache *c, int layer, float *k_out, float *v_out) {
+    for (int h = 0; h < c->heads; h++)
+        for (int s = 0; s < c->current_len; s++) {
+            size_t so = ((size_t)h * c->max_len + s) * c->hd;
+            size_t dof = ((size_t)h * c->current_len + s) * c->hd;
+            memcpy(k_out + dof, c->key[layer] + so, (size_t)c->hd * 4);
+            memcpy(v_out + dof, c->value[layer] + so, (size_t)c->hd * 4);
+        }
+}
+
+/* src/runtime.rs:1898-1938 — bulk-load prefill K/V ([heads][seq][hd] per buffer). */
+ORC_API int orc_kv_init_from(orc_kv_cache *c, int layer, const float *k, const float *v,
+                             int seq_len) {
+    if (seq_len > c->max_len) return -1;
+    for (int h = 0; h < c->heads; h++) {
+        size_t so = (size_t)h * seq_len * c->hd;
+        size_t dof = (size_t)h * c->max_len * c->hd;
+        size_t cnt = (size_t)seq_len * c->hd;
+        if (c->round_bf16) {
+            for (size_t i = 0; i < cnt; i++) {
+                c->key[layer][dof + i] = bf16_to_f32(orc_f32_to_bf16_rne(k[so + i]));
+                c->value[layer][dof + i] = bf16_to_f32(orc_f32_to_bf16_rne(v[so + i]));
+            }
+        } else {
+            memcpy(c->key[layer] + dof, k + so, cnt * 4);
+            memcpy(c->value[layer] + dof, v + so, cnt * 4);
+        }
+    }
+    c->current_len = seq_len;
+    return 0;
+}
+
+/* ───────────────────────── whole decode step ───────────────────────── */
+
+enum { ORC_W_BF16 = 1, ORC_W_Q8_0 = 2, ORC_W_Q4_0 = 3 };
+
+typedef struct {
+    int hidden, inter, heads, kv_heads, head_dim, layers, vocab;
+    float eps;
+    int weight_kind; /* ORC_W_* for the seven projections */
+    int has_qk_norm;
+} orc_config;
+
+/* Weight pointers in the order of TransformerWeights::to_slot_buffers
+ * (src/hf/weights.rs:63-116; no-bias models): embed, per layer {input_ln, q, k, v,
+ * [q_norm, k_norm], o, post_ln, gate, up, down}, final_norm, lm_head.
+ * bf16 projections are [K][N] (transposed at load, src/hf/weights.rs:225-261);
+ * quantised ones are raw [N][K/32] blocks (src/hf/weights.rs:136-194).
+ * lm_head is bf16 [hidden][vocab] in the bf16 plan and f32 [hidden][vocab] in the quant plan. */
+typedef struct {
+    const float *input_ln, *q_norm, *k_norm, *post_ln;
+    const void *q, *k, *v, *o, *gate, *up, *down;
+} orc_layer_weights;
+
+typedef struct {
+    orc_config cfg;
+    const float *embed;
+    orc_layer_weights *layers;
+    const float *final_norm;
+    const void *lm_head;
+    const float *rope_cos, *rope_sin; /* [max_pos][head_dim] */
+    int max_pos;
+    orc_kv_cache *kv;
+    /* scratch */
+    float *h, *normed, *q, *k, *v, *attn_flat, *attn_out, *resid, *gate, *up, *act, *down,
+        *scores, *mask;
+    int scratch_seq, scratch_total;
+} orc_model;
+
+ORC_API orc_model *orc_model_new(const orc_config *cfg) {
+    orc_model *m = (orc_model *)calloc(1, sizeof(*m));
+    m->cfg = *cfg;
+    m->layers = (orc_layer_weights *)calloc((size_t)cfg->layers, sizeof(orc_layer_weights));
+    return m;
+}
+
+ORC_API void orc_model_set_global(orc_model *m, const float *embed, const float *final_norm,
+                                  const void *lm_head, const float *rope_cos,
+                                  const float *rope_sin, int max_pos) {
+    m->embed = embed;
+    m->final_norm = final_norm;
+    m->lm_head = lm_head;
+    m->rope_cos = rope_cos;
+    m->rope_sin = rope_sin;
+    m->max_pos = max_pos;
+}
+
+ORC_API void orc_model_set_layer(orc_model *m, int l, const float *input_ln, const void *q,
+                                 const void *k, const void *v, const float *q_norm,
+                                 const float *k_norm, const void *o, const float *post_ln,
+                                 const void *gate, const void *up, const void *down) {
+    orc_layer_weights *w = &m->layers[l];
+    w->input_ln = input_ln;
+    w->q = q;
+    w->k = k;
+    w->v = v;
+    w->q_norm = q_norm;
+    w->k_norm = k_norm;
+    w->o = o;
+    w->post_ln = post_ln;
+    w->gate = gate;
+    w->up = up;
+    w->down = down;
+}
+
+ORC_API void orc_model_attach_kv(orc_model *m, orc_kv_cache *kv) { m->kv = kv; }
+
+static void free_scratch(orc_model *m) {
+    free(m->h); free(m->normed); free(m->q); free(m->k); free(m->v); free(m->attn_flat);
+    free(m->attn_out); free(m->resid); free(m->gate); free(m->up); free(m->act); free(m->down);
+    free(m->scores); free(m->mask);
+    m->h = m->normed = m->q = m->k = m->v = m->attn_flat = m->attn_out = m->resid = NULL;
+    m->gate = m->up = m->act = m->down = m->scores = m->mask = NULL;
+}
+
+ORC_API void orc_model_free(orc_model *m) {
+    if (!m) return;
+    free_scratch(m);
+    free(m->layers);
+    free(m);
+}
+
+static void ensure_scratch(orc_model *m, int S, int total) {
+    if (m->h && S <= m->scratch_seq && total <= m->scratch_total) return;
+    free_scratch(m);
+    const orc_config *c = &m->cfg;
+    size_t s = (size_t)S;
+    int qd = c->heads * c->head_dim, kvd = c->kv_heads * c->head_dim;
+    m->h = (float *)malloc(s * c->hidden * 4);
+    m->normed = (float *)malloc(s * c->hidden * 4);
+    m->q = (float *)malloc(s * qd * 4);
+    m->k = (float *)malloc(s * kvd * 4);
+    m->v = (float *)malloc(s * kvd * 4);
+    m->attn_flat = (float *)malloc(s * qd * 4);
+    m->attn_out = (float *)malloc(s * c->hidden * 4);
+    m->resid = (float *)malloc(s * c->hidden * 4);
+    m->gate = (float *)malloc(s * c->inter * 4);
+    m->up = (float *)malloc(s * c->inter * 4);
+    m->act = (float *)malloc(s * c->inter * 4);
+    m->down = (float *)malloc(s * c->hidden * 4);
+    m->scores = (float *)malloc((size_t)c->heads * s * total * 4);
+    m->mask = (float *)malloc(s * total * 4);
+    m->scratch_seq = S;
+    m->scratch_total = total;
+}
+
+static void proj(const orc_model *m, const float *x, const void *w, float *out, int M, int K,
+                 int N) {
+    switch (m->cfg.weight_kind) {
+    case ORC_W_BF16: orc_matmul_f32_bf16(x, (const uint16_t *)w, out, M, K, N); break;
+    case ORC_W_Q8_0: orc_gemv_q8_0(x, (const uint8_t *)w, out, M, K, N); break;
+    case ORC_W_Q4_0: orc_gemv_q4_0(x, (const uint8_t *)w, out, M, K, N); break;
+    default: abort();
+    }
+}
+
+/* [S][heads][hd] -> [heads][S][hd] (the BSHD->BHSD transposes of src/hf/emitter.rs:648-649) */
+static void to_bhsd(const float *src, float *dst, int S, int heads, int hd) {
+    for (int s = 0; s < S; s++)
+        for (int h = 0; h < heads; h++)
+            memcpy(dst + ((size_t)h * S + s) * hd, src + ((size_t)s * heads + h) * hd,
+                   (size_t)hd * 4);
+}
+
+/* One pass of ExecutionPlan::run_kv (src/runtime.rs:1580-1892) over the step list built by
+ * emit_transformer_plan (src/hf/emitter.rs:902-1014) or, for quantised projections,
+ * emit_transformer_plan_quant (src/hf/emitter_quant.rs:1211-1440), with the inputs prepared
+ * as HfModel::run_kv does (src/hf/model.rs:198-218): positions past..past+S, causal mask.
+ * Writes logits [S][vocab]; returns 0, or -1 when the KV cache would overflow. */
+ORC_API int orc_model_run_kv(orc_model *m, const int64_t *ids, int S, float *logits) {
+    const orc_config *c = &m->cfg;
+    orc_kv_cache *kv = m->kv;
+    int past = kv->current_len;
+    int total = past + S;
+    if (total > kv->max_len || total > m->max_pos) return -1;
+    ensure_scratch(m, S, total);
+    int hd = c->head_dim, qd = c->heads * hd, kvd = c->kv_heads * hd;
+    int quant = c->weight_kind != ORC_W_BF16;
+    const float *cosv = m->rope_cos + (size_t)past * hd; /* slice_rope_for_positions */
+    const float *sinv = m->rope_sin + (size_t)past * hd;
+    orc_causal_mask(S, past, m->mask);
+    float *kb = (float *)malloc((size_t)S * kvd * 4);
+    float *vb = (float *)malloc((size_t)S * kvd * 4);
+
+    orc_embed(ids, S, m->embed, c->hidden, m->h);
+    for (int l = 0; l < c->layers; l++) {
+        const orc_layer_weights *w = &m->layers[l];
+        /* QKV kernel: src/hf/emitter.rs:549-673 (quant: RMSNorm :713-791, QuantMM x3,
+         * PostQKV :802-912) */
+        if (quant)
+            orc_rms_norm_f64acc(m->h, w->input_ln, m->normed, S, c->hidden, c->eps);
+        else
+            orc_rms_norm(m->h, w->input_ln, m->normed, S, c->hidden, c->eps);
+        proj(m, m->normed, w->q, m->q, S, c->hidden, qd);
+        proj(m, m->normed, w->k, m->k, S, c->hidden, kvd);
+        proj(m, m->normed, w->v, m->v, S, c->hidden, kvd);
+        if (c->has_qk_norm) {
+            if (quant) {
+                orc_rms_norm_f64mean(m->q, w->q_norm, m->q, S * c->heads, hd, c->eps);
+                orc_rms_norm_f64mean(m->k, w->k_norm, m->k, S * c->kv_heads, hd, c->eps);
+            } else {
+                orc_rms_norm(m->q, w->q_norm, m->q, S * c->heads, hd, c->eps);
+                orc_rms_norm(m->k, w->k_norm, m->k, S * c->kv_heads, hd, c->eps);
+            }
+        }
+        orc_rope_half(m->q, cosv, sinv, S, c->heads, hd);
+        orc_rope_half(m->k, cosv, sinv, S, c->kv_heads, hd);
+        to_bhsd(m->k, kb, S, c->kv_heads, hd);
+        to_bhsd(m->v, vb, S, c->kv_heads, hd);
+        /* KV concat steps: src/runtime.rs:1729-1755 */
+        if (orc_kv_append_key(kv, l, kb, S) || orc_kv_append_value(kv, l, vb, S)) {
+            free(kb); free(vb);
+            return -1;
+        }
+        /* Attention kernel: src/hf/emitter.rs:683-758 (quant: AttnBody :922-975 + QuantMM O) */
+        orc_gqa_attention(m->q, orc_kv_key_ptr(kv, l), orc_kv_value_ptr(kv, l), m->mask,
+                          m->attn_flat, S, c->heads, c->kv_heads, hd, total,
+                          orc_kv_head_stride(kv), quant, m->scores);
+        proj(m, m->attn_flat, w->o, m->attn_out, S, qd, c->hidden);
+        /* MLP kernel: src/hf/emitter.rs:767-822 (quant: Residual+Norm :985-1071, QuantMM
+         * gate/up, SiLU*Up :1077-1103, QuantMM down, ResAdd :1109-1134) */
+        orc_add(m->h, m->attn_out, m->resid, (size_t)S * c->hidden);
+        if (quant)
+            orc_rms_norm_f64acc(m->resid, w->post_ln, m->normed, S, c->hidden, c->eps);
+        else
+            orc_rms_norm(m->resid, w->post_ln, m->normed, S, c->hidden, c->eps);
+        proj(m, m->normed, w->gate, m->gate, S, c->hidden, c->inter);
+        proj(m, m->normed, w->up, m->up, S, c->hidden, c->inter);
+        orc_silu_mul(m->gate, m->up, m->act, (size_t)S * c->inter);
+        proj(m, m->act, w->down, m->down, S, c->inter, c->hidden);
+        orc_add(m->resid, m->down, m->h, (size_t)S * c->hidden);
+    }
+    /* LM head: src/hf/emitter.rs:828-862 (bf16 weights, f32 RMSNorm); the quantised plan
+     * (src/hf/emitter_quant.rs:1399-1440) uses the f64-mean RMSNorm and an f32 weight. */
+    if (quant) {
+        orc_rms_norm_f64mean(m->h, m->final_norm, m->normed, S, c->hidden, c->eps);
+        orc_matmul_f32_f32(m->normed, (const float *)m->lm_head, logits, S, c->hidden, c->vocab);
+    } else {
+        orc_rms_norm(m->h, m->final_norm, m->normed, S, c->hidden, c->eps);
+        orc_matmul_f32_bf16(m->normed, (const uint16_t *)m->lm_head, logits, S, c->hidden,
+                            c->vocab);
+    }
+    /* src/runtime.rs:1875-1880 — one advance after all layers appended */
+    orc_kv_advance_by(kv, S);
+    free(kb);
+    free(vb);
+    return 0;
+}
+
+/* Greedy loop of src/generate.rs:187-270 restricted to pure argmax (repetition penalty 1.0):
+ * prompt tokens are fed one at a time through run_kv (incremental prefill on an existing
+ * cache, src/hf/model.rs:321-336); the argmax after the last prompt token is generated
+ * token 0. Optionally records the top1-top2 logit margin of every generated token. */
+ORC_API int orc_generate_greedy(orc_model *m, const int64_t *prompt, int n_prompt, int n_new,
+                                int32_t *out_tokens, float *margins) {
+    float *logits = (float *)malloc((size_t)m->cfg.vocab * 4);
+    int64_t tok = 0;
+    int produced = 0;
+    for (int i = 0; i < n_prompt + n_new - 1 && produced < n_new; i++) {
+        tok = i < n_prompt ? prompt[i] : tok;
+        if (orc_model_run_kv(m, &tok, 1, logits)) {
+            free(logits);
+            return -1;
+        }
+        if (i >= n_prompt - 1) {
+            int best = orc_argmax_last(logits, m->cfg.vocab);
+            if (margins) {
+                float second = -INFINITY;
+                for (int j = 0; j < m->cfg.vocab; j++)
+                    if (j != best && logits[j] > second) second = logits[j];
+                margins[produced] = logits[best] - second;
+            }
+            out_tokens[produced++] = best;
+            tok = best;
+        }
+    }
+    free(logits);
+    return produced;
+}
+
+ORC_API int orc_num_threads(void) { return host_cores(); }

@@ -1,0 +1,316 @@
+"""GPU parity of every kernel-level entry point of the C boundary against the CPU oracle, on the
+same seeded inputs. Bit-exact for byte/integer work (dequantisation, KV append, argmax,
+embedding); max relative error <= 1e-2 for matmul/attention outputs, where
+    rel = |gpu - ref| / max(|ref|, 1e-3 * max|ref|)
+(the floor keeps outputs that happen to land near zero from dividing by nothing)."""
+import math
+
+import numpy as np
+import pytest
+
+from homura_amd import HomuraError, synth
+
+pytestmark = pytest.mark.gpu
+
+TOL = 1e-2
+
+
+def rel_err(a, b):
+    a = np.asarray(a, np.float64).reshape(-1)
+    b = np.asarray(b, np.float64).reshape(-1)
+    floor = 1e-3 * max(np.abs(b).max(), 1e-30)
+    return float(np.max(np.abs(a - b) / np.maximum(np.abs(b), floor)))
+
+
+def say(msg):
+    print(msg, flush=True)
+
+
+# ── bf16 GEMV (reference emit_matmul with bf16 weights) ───────────────────────
+
+@pytest.mark.parametrize("M,K,N", [(1, 896, 4864),   # BASELINE config 1
+                                   (1, 1024, 4096), (1, 3072, 1024), (1, 2048, 1024),
+                                   (3, 896, 4864), (5, 1024, 1024), (8, 256, 136),
+                                   (1, 40, 12), (2, 8, 8)])
+def test_gemv_bf16_both_layouts(ctx, oracle, M, K, N):
+    say(f"gemv_bf16 M={M} K={K} N={N}")
+    x = synth.normal_f32(synth.SEED_CFG1, M * K).reshape(M, K)
+    w = synth.normal_bf16(synth.SEED_CFG1 + 1, K * N, 0.02).reshape(K, N)
+    want = oracle.matmul_f32_bf16(x, w, M, K, N)
+    dx, dw, dout = ctx.to_device(x), ctx.to_device(w), ctx.empty(M * N)
+    ctx.gemv_bf16(dx, dw, dout, M, K, N)
+    got = dout.download(np.float32, (M, N))
+    assert rel_err(got, want) < TOL
+    # a second call must see clean split-K counters
+    ctx.gemv_bf16(dx, dw, dout, M, K, N)
+    assert np.array_equal(dout.download(np.float32, (M, N)), got)
+    if K % 8 == 0:
+        dnk, dout2 = ctx.empty(K * N, np.uint16), ctx.empty(M * N)
+        ctx.pack_bf16_kn_to_nk(dw, dnk, K, N)
+        assert np.array_equal(dnk.download(np.uint16, (N, K)), w.T)  # pure data movement: exact
+        ctx.gemv_bf16_nk(dx, dnk, dout2, M, K, N)
+        assert rel_err(dout2.download(np.float32, (M, N)), want) < TOL
+        dnk.free(); dout2.free()
+    for b in (dx, dw, dout):
+        b.free()
+
+
+def test_gemv_bf16_reference_vectors(ctx, golden):
+    """The reference's exact matmul vectors (integers are bf16-representable)."""
+    g = golden["matmul_2d_known_values"]
+    a = np.zeros((2, 8), np.float32)
+    b = np.zeros((8, 8), np.float32)
+    a[:, :2] = g["a"]
+    b[:2, :2] = g["b"]
+    bits = (b.view(np.uint32) >> 16).astype(np.uint16)
+    dx, dw, dout = ctx.to_device(a), ctx.to_device(bits), ctx.empty(16)
+    ctx.gemv_bf16(dx, dw, dout, 2, 8, 8)
+    got = dout.download(np.float32, (2, 8))
+    assert np.array_equal(got[:, :2], np.array(g["expected"], np.float32))
+    assert np.all(got[:, 2:] == 0)
+
+
+# ── Q8_0 / Q4_0 ───────────────────────────────────────────────────────────────
+
+def test_dequant_bit_exact(ctx, oracle):
+    nb = 8192 + 3
+    for kind, bb, gen, dq, orc in (("q8_0", 34, synth.q8_0_blocks, ctx.dequant_q8_0, oracle.dequant_q8_0),
+                                   ("q4_0", 18, synth.q4_0_blocks, ctx.dequant_q4_0, oracle.dequant_q4_0)):
+        say(f"dequant {kind}")
+        raw = gen(77, nb)
+        blk = raw.reshape(nb, bb)
+        # scales that exercise f16 subnormals, zero, max, inf and NaN
+        for i, bits in enumerate([0x0001, 0x03FF, 0x0000, 0x8000, 0x7BFF, 0x7C00, 0xFC00, 0x7E00, 0x0400]):
+            blk[i, 0], blk[i, 1] = bits & 0xFF, bits >> 8
+        want = orc(raw)
+        d_in, d_out = ctx.to_device(raw), ctx.empty(nb * 32)
+        dq(d_in, d_out, nb)
+        got = d_out.download(np.float32)
+        nan = np.isnan(want)
+        assert np.array_equal(np.isnan(got), nan)
+        assert np.array_equal(got[~nan].view(np.uint32), want[~nan].view(np.uint32))
+        d_in.free(); d_out.free()
+
+
+def test_q8_0_reference_kat(ctx, golden):
+    g = golden["emit_q8_0_correctness"]
+    N, K = g["N"], g["K"]
+    raw = np.zeros((N, 34), np.uint8)
+    raw[:, 0], raw[:, 1] = g["scale_bits"] & 0xFF, g["scale_bits"] >> 8
+    raw[:, 2:] = np.arange(1, 33, dtype=np.uint8)
+    dx, dw, dout = ctx.to_device(np.ones(K, np.float32)), ctx.to_device(raw), ctx.empty(N)
+    ctx.gemv_q8_0(dx, dw, dout, 1, K, N)
+    assert np.all(dout.download(np.float32) == g["expected_each"])
+
+
+@pytest.mark.parametrize("kind,M,K,N", [("q8_0", 1, 2048, 5632),    # BASELINE config 3
+                                        ("q4_0", 1, 1536, 151936),  # BASELINE config 4
+                                        ("q8_0", 1, 2048, 2048), ("q8_0", 1, 5632, 2048),
+                                        ("q8_0", 2, 4096, 77), ("q8_0", 1, 32, 5), ("q8_0", 1, 96, 1),
+                                        ("q4_0", 3, 2048, 260), ("q4_0", 1, 32, 7), ("q4_0", 1, 8960, 64)])
+def test_quant_gemv(ctx, oracle, kind, M, K, N):
+    say(f"gemv_{kind} M={M} K={K} N={N}")
+    nb = N * (K // 32)
+    seed = synth.SEED_CFG3 if kind == "q8_0" else synth.SEED_CFG4
+    raw = (synth.q8_0_blocks if kind == "q8_0" else synth.q4_0_blocks)(seed, nb, 0.01)
+    x = synth.normal_f32(seed + 1, M * K).reshape(M, K)
+    want = (oracle.gemv_q8_0 if kind == "q8_0" else oracle.gemv_q4_0)(x, raw, M, K, N)
+    dx, dw, dout = ctx.to_device(x), ctx.to_device(raw), ctx.empty(M * N)
+    (ctx.gemv_q8_0 if kind == "q8_0" else ctx.gemv_q4_0)(dx, dw, dout, M, K, N)
+    got = dout.download(np.float32, (M, N))
+    assert rel_err(got, want) < TOL
+    for b in (dx, dw, dout):
+        b.free()
+
+
+# ── prefill GEMM (MFMA) ───────────────────────────────────────────────────────
+
+@pytest.mark.parametrize("M,K,N", [(512, 2048, 8192),  # BASELINE config 5a
+                                   (128, 32, 128), (256, 96, 384)])
+def test_gemm_bf16_mfma(ctx, oracle, M, K, N):
+    say(f"gemm_bf16 M={M} K={K} N={N}")
+    a = synth.normal_bf16(synth.SEED_CFG5, M * K, 1.0).reshape(M, K)
+    b = synth.normal_bf16(synth.SEED_CFG5 + 1, K * N, 0.02).reshape(K, N)
+    want = oracle.matmul_bf16_bf16(a, b, M, K, N)
+    da, db, dc = ctx.to_device(a), ctx.to_device(b), ctx.empty(M * N)
+    ctx.gemm_bf16(da, db, dc, M, K, N)
+    got = dc.download(np.float32, (M, N))
+    assert rel_err(got, want) < TOL
+    for buf in (da, db, dc):
+        buf.free()
+
+
+def test_gemm_identity_exact(ctx):
+    """A = I (bf16) picks rows of B exactly: catches a wrong fragment layout or transposition."""
+    M = K = 128
+    N = 256
+    a = np.zeros((M, K), np.float32)
+    a[np.arange(M), (np.arange(M) * 37) % K] = 1.0  # a permutation matrix
+    b = synth.normal_bf16(5, K * N, 1.0).reshape(K, N)
+    da, db, dc = ctx.to_device((a.view(np.uint32) >> 16).astype(np.uint16)), ctx.to_device(b), ctx.empty(M * N)
+    ctx.gemm_bf16(da, db, dc, M, K, N)
+    got = dc.download(np.float32, (M, N))
+    assert np.array_equal(got, synth.bf16_to_f32(b)[(np.arange(M) * 37) % K])
+
+
+# ── KV cache append + decode attention ────────────────────────────────────────
+
+def test_kv_append_reference_arrays(ctx, golden):
+    g = golden["kv_cache_multi_token_append"]
+    heads, max_len, hd = g["heads"], g["max_len"], g["head_dim"]
+    kc, vc = ctx.empty(heads * max_len * hd, np.uint16), ctx.empty(heads * max_len * hd, np.uint16)
+    ctx._check(ctx.lib.hm_fill_zero(ctx.h, kc.ptr, kc.nbytes))
+    ctx._check(ctx.lib.hm_fill_zero(ctx.h, vc.ptr, vc.nbytes))
+    k3, v3 = ctx.to_device(np.array(g["k3"], np.float32)), ctx.to_device(np.array(g["v3"], np.float32))
+    ctx.kv_append(kc, vc, k3, v3, 1, heads, hd, max_len, 0, 3)
+    k1, v1 = ctx.to_device(np.array(g["k1"], np.float32)), ctx.to_device(np.array(g["v1"], np.float32))
+    ctx.kv_append(kc, vc, k1, v1, 1, heads, hd, max_len, 3, 1)
+    cache = synth.bf16_to_f32(kc.download(np.uint16)).reshape(heads, max_len, hd)
+    assert np.array_equal(cache[:, :4].reshape(-1), np.array(g["view_k_after_4"], np.float32))
+    assert np.all(cache[:, 4:] == 0)
+    # the reference panics "KV cache full"; here it is an error status and nothing is written
+    with pytest.raises(HomuraError) as e:
+        ctx.kv_append(kc, vc, k3, v3, 1, heads, hd, max_len, 6, 3)
+    assert e.value.code == -4 and "KV cache full" in str(e.value)
+
+
+def test_kv_append_rounds_to_nearest_even(ctx, oracle):
+    lib = oracle.load()
+    x = synth.normal_f32(9, 2 * 4 * 128)
+    x[:3] = [1.0 + 2 ** -8, 1.0 + 3 * 2 ** -8, -1.0 - 2 ** -8]  # exact ties
+    kc, vc = ctx.empty(2 * 8 * 128, np.uint16), ctx.empty(2 * 8 * 128, np.uint16)
+    dk = ctx.to_device(x)
+    ctx.kv_append(kc, vc, dk, dk, 1, 2, 128, 8, 2, 4)
+    got = kc.download(np.uint16).reshape(2, 8, 128)[:, 2:6].reshape(-1)
+    want = np.array([lib.orc_f32_to_bf16_rne(float(v)) for v in x], np.uint16)
+    assert np.array_equal(got, want)
+    assert np.array_equal(vc.download(np.uint16).reshape(2, 8, 128)[:, 2:6].reshape(-1), want)
+
+
+@pytest.mark.parametrize("B,H,kvh,hd,max_len,kv_len", [
+    (8, 12, 2, 128, 4096, 4096),   # BASELINE config 5b
+    (1, 16, 8, 128, 2048, 1025),   # Qwen3-0.6B decode shape
+    (1, 16, 8, 128, 1152, 1),      # first token
+    (2, 14, 2, 64, 300, 33),       # Qwen2.5-0.5B heads (g = 7), ragged length
+    (1, 4, 4, 128, 64, 64),        # MHA (g = 1), single split
+    (3, 32, 4, 64, 512, 511)])     # g = 8
+def test_gqa_decode_attn(ctx, oracle, B, H, kvh, hd, max_len, kv_len):
+    say(f"gqa_decode_attn B={B} H={H} kvh={kvh} hd={hd} max_len={max_len} kv_len={kv_len}")
+    q = synth.normal_f32(synth.SEED_CFG5 + 2, B * H * hd).reshape(B, H, hd)
+    kb = synth.normal_bf16(synth.SEED_CFG5 + 3, B * kvh * max_len * hd).reshape(B, kvh, max_len, hd)
+    vb = synth.normal_bf16(synth.SEED_CFG5 + 4, B * kvh * max_len * hd).reshape(B, kvh, max_len, hd)
+    scale = 1.0 / math.sqrt(hd)
+    dq, dk, dv, dout = ctx.to_device(q), ctx.to_device(kb), ctx.to_device(vb), ctx.empty(B * H * hd)
+    ctx.gqa_decode_attn(dq, dk, dv, dout, B, H, kvh, hd, max_len, kv_len, scale)
+    got = dout.download(np.float32, (B, H * hd))
+    mask = np.zeros((1, kv_len), np.float32)  # decode: every cached row is attended
+    for b in range(B):
+        want = oracle.gqa_attention(q[b:b + 1], synth.bf16_to_f32(kb[b]), synth.bf16_to_f32(vb[b]), mask)
+        assert rel_err(got[b], want) < TOL, f"sequence {b}"
+    # repeat: the split counters must have been left clean
+    ctx.gqa_decode_attn(dq, dk, dv, dout, B, H, kvh, hd, max_len, kv_len, scale)
+    assert np.array_equal(dout.download(np.float32, (B, H * hd)), got)
+    for buf in (dq, dk, dv, dout):
+        buf.free()
+
+
+def test_attention_uniform_keys_give_mean_of_values(ctx):
+    B, H, kvh, hd, L = 1, 4, 2, 128, 200
+    q = synth.normal_f32(1, H * hd)
+    k = np.zeros((kvh, L, hd), np.uint16)
+    vb = synth.normal_bf16(2, kvh * L * hd).reshape(kvh, L, hd)
+    dq, dk, dv, dout = ctx.to_device(q), ctx.to_device(k), ctx.to_device(vb), ctx.empty(H * hd)
+    ctx.gqa_decode_attn(dq, dk, dv, dout, B, H, kvh, hd, L, L, 0.1)
+    got = dout.download(np.float32, (H, hd))
+    mean = synth.bf16_to_f32(vb).astype(np.float64).mean(axis=1)
+    for h in range(H):
+        assert np.allclose(got[h], mean[h // 2], atol=1e-5)  # heads h0,h0,h1,h1 (floordiv map)
+
+
+# ── light ops ─────────────────────────────────────────────────────────────────
+
+def test_rmsnorm(ctx, oracle, golden):
+    g = golden["rms_norm_basic"]
+    dx, dw, dout = ctx.to_device(np.array(g["input"], np.float32)), ctx.to_device(np.array(g["weight"], np.float32)), ctx.empty(4)
+    ctx.rmsnorm(dx, dw, dout, 1, 4, g["eps"])
+    want = np.array(g["input"]) / math.sqrt(g["mean_square"] + g["eps"])
+    assert np.allclose(dout.download(np.float32), want, atol=g["tolerance"])
+    x = synth.normal_f32(3, 5 * 1024).reshape(5, 1024)
+    w = synth.normal_f32(4, 1024)
+    dx, dw, dout = ctx.to_device(x), ctx.to_device(w), ctx.empty(5 * 1024)
+    ctx.rmsnorm(dx, dw, dout, 5, 1024, 1e-6)
+    assert rel_err(dout.download(np.float32, (5, 1024)), oracle.rms_norm(x, w, 1e-6)) < 1e-4
+
+
+@pytest.mark.parametrize("S,H,kvh,hd,qk_norm", [(1, 16, 8, 128, True), (3, 14, 2, 64, False), (2, 4, 4, 128, True)])
+def test_qknorm_rope(ctx, oracle, S, H, kvh, hd, qk_norm):
+    q = synth.normal_f32(5, S * H * hd).reshape(S, H, hd)
+    k = synth.normal_f32(6, S * kvh * hd).reshape(S, kvh, hd)
+    qw, kw = synth.normal_f32(7, hd), synth.normal_f32(8, hd)
+    cos, sin = oracle.rope_tables(hd, 2048, 1e6)
+    pos = [1029 + i for i in range(S)]
+    wq = oracle.rms_norm(q, qw, 1e-6) if qk_norm else q
+    wk = oracle.rms_norm(k, kw, 1e-6) if qk_norm else k
+    wq, wk = oracle.rope_half(wq, cos[pos], sin[pos]), oracle.rope_half(wk, cos[pos], sin[pos])
+    dq, dk = ctx.to_device(q), ctx.to_device(k)
+    dqw, dkw = (ctx.to_device(qw), ctx.to_device(kw)) if qk_norm else (None, None)
+    dc, ds = ctx.to_device(cos[pos]), ctx.to_device(sin[pos])
+    ctx.qknorm_rope(dq, dk, dqw, dkw, dc, ds, S, H, kvh, hd, 1e-6)
+    assert rel_err(dq.download(np.float32, q.shape), wq) < 1e-4
+    assert rel_err(dk.download(np.float32, k.shape), wk) < 1e-4
+
+
+def test_silu_add_embed(ctx, oracle, golden):
+    g = synth.normal_f32(10, 3072) * 3
+    u = synth.normal_f32(11, 3072)
+    dg, du, dout = ctx.to_device(g), ctx.to_device(u), ctx.empty(3072)
+    ctx.silu_mul(dg, du, dout, 3072)
+    assert rel_err(dout.download(np.float32), oracle.silu_mul(g, u)) < 1e-5
+    ctx.add(dg, du, dout, 3072)
+    assert np.array_equal(dout.download(np.float32), g + u)  # one f32 add: exact
+    e = golden["embedding_basic"]
+    table = np.array(e["table"], np.float32)
+    ids = np.array(e["ids"], np.int64)
+    dt, di, do = ctx.to_device(table), ctx.to_device(ids), ctx.empty(4 * 3)
+    ctx.embed(di, dt, do, 4, 4, 3)
+    assert np.array_equal(do.download(np.float32, (4, 3)), np.array(e["expected"], np.float32))
+
+
+def test_argmax_tie_rule(ctx, oracle, golden):
+    cases = [np.array(golden["sample_token_greedy"]["logits"], np.float32),
+             np.array([3.0, 1.0, 3.0, 2.0, 3.0, 0.0], np.float32),
+             np.array([-np.inf, -np.inf], np.float32),
+             np.array([1.0, np.nan, 0.5], np.float32),
+             np.array([1.0, 2.0, np.nan], np.float32)]
+    big = synth.normal_f32(12, 151936)
+    top = float(big.max()) + 1.0
+    big[[7, 70000, 151000]] = top            # three equal maxima: the last one wins
+    cases.append(big)
+    big2 = big.copy()
+    big2[100000] = np.nan                     # a NaN discards everything before it
+    cases.append(big2)
+    dout = ctx.empty(1, np.int32)
+    for c in cases:
+        dv = ctx.to_device(c)
+        ctx.argmax(dv, c.size, dout)
+        assert int(dout.download(np.int32)[0]) == oracle.argmax_last(c)
+        dv.free()
+    assert oracle.argmax_last(big) == 151000 and oracle.argmax_last(big2) == 151000
+
+
+# ── error behaviour ───────────────────────────────────────────────────────────
+
+def test_bad_arguments_are_errors_not_faults(ctx):
+    d = ctx.empty(64)
+    with pytest.raises(HomuraError) as e:
+        ctx.gemv_q8_0(d, d, d, 1, 48, 4)          # K not a multiple of 32
+    assert e.value.code == -1
+    with pytest.raises(HomuraError):
+        ctx.gemv_bf16(d, d, d, 9, 8, 8)           # M out of range
+    with pytest.raises(HomuraError):
+        ctx.gemm_bf16(d, d, d, 100, 32, 128)      # M not a multiple of 128
+    with pytest.raises(HomuraError):
+        ctx.gqa_decode_attn(d, d, d, d, 1, 6, 4, 128, 16, 4, 1.0)  # heads not divisible
+    with pytest.raises(HomuraError):
+        ctx.gqa_decode_attn(d, d, d, d, 1, 4, 4, 128, 16, 17, 1.0)  # kv_len > max_len
+    ctx.sync()
