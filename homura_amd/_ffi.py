@@ -88,10 +88,13 @@ SIGNATURES = {
     "hm_model_init_kv_cache": (_I, [_P, C.POINTER(c_f32_p), _I]),
     "hm_model_reset_kv_cache": (_I, [_P]),
     "hm_model_kv_cache_len": (_I, [_P]),
+    "hm_model_set_graph": (_I, [_P, _I]),
     "hm_model_run_kv": (_I, [_P, C.POINTER(C.c_int64), _I, c_f32_p]),
     "hm_model_generate_greedy": (_I, [_P, C.POINTER(C.c_int64), _I, _I, C.POINTER(C.c_int32)]),
     "hm_model_bench_decode": (_I, [_P, C.c_int64, _I, c_f32_p, C.POINTER(C.c_int32)]),
     "hm_model_profile_step": (_I, [_P, C.c_int64, C.POINTER(HmKernelProfile), _I]),
+    "hm_model_time_kernels": (_I, [_P, _I, C.POINTER(HmKernelProfile), _I]),
+    "hm_model_launches_per_step": (_I, [_P]),
     "hm_synth_normal_f32": (None, [C.c_uint64, C.c_uint64, _SZ, C.c_float, _P]),
     "hm_synth_normal_bf16": (None, [C.c_uint64, C.c_uint64, _SZ, C.c_float, _P]),
     "hm_synth_token_ids": (None, [C.c_uint64, _SZ, _I, _P]),

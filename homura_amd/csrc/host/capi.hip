@@ -85,6 +85,12 @@ int hm_model_kv_cache_len(hm_model *m) {
     return m->impl->kv_cache_len();
 }
 
+int hm_model_set_graph(hm_model *m, int on) {
+    if (!m) return HM_ERR_INVALID;
+    if (!m->impl->plan()) return hm_set_error(m->ctx, HM_ERR_STATE, "model not finalized");
+    return m->impl->plan()->enable_graph(on != 0);
+}
+
 int hm_model_run_kv(hm_model *m, const int64_t *h_ids, int n_ids, float *h_logits) {
     if (!m) return HM_ERR_INVALID;
     return m->impl->run_kv(h_ids, n_ids, h_logits);
@@ -103,11 +109,33 @@ int hm_model_bench_decode(hm_model *m, int64_t first_id, int n_steps, float *ms_
     return m->impl->bench_decode(first_id, n_steps, ms_out, h_tokens_out);
 }
 
+static int fill_profiles(const std::vector<StepProfile> &prof, hm_kernel_profile *out, int cap);
+
+int hm_model_time_kernels(hm_model *m, int rounds, hm_kernel_profile *out, int cap) {
+    if (!m) return HM_ERR_INVALID;
+    std::vector<StepProfile> prof;
+    int rc = m->impl->time_kernels(rounds, prof);
+    if (rc != HM_OK) return rc;
+    return fill_profiles(prof, out, cap);
+}
+
+int hm_model_launches_per_step(hm_model *m) {
+    if (!m) return HM_ERR_INVALID;
+    if (!m->impl->plan()) return hm_set_error(m->ctx, HM_ERR_STATE, "model not finalized");
+    return m->impl->plan()->launches_per_step();
+}
+
 int hm_model_profile_step(hm_model *m, int64_t token_id, hm_kernel_profile *out, int cap) {
     if (!m) return HM_ERR_INVALID;
     std::vector<StepProfile> prof;
     int rc = m->impl->profile_step(token_id, prof);
     if (rc != HM_OK) return rc;
+    return fill_profiles(prof, out, cap);
+}
+
+}  // extern "C"
+
+static int fill_profiles(const std::vector<StepProfile> &prof, hm_kernel_profile *out, int cap) {
     int n = 0;
     for (auto &p : prof) {
         if (n >= cap) break;
@@ -120,5 +148,3 @@ int hm_model_profile_step(hm_model *m, int64_t token_id, hm_kernel_profile *out,
     }
     return n;
 }
-
-}  // extern "C"

@@ -70,6 +70,7 @@ class HfModel {
     int generate_greedy(const int64_t *h_prompt, int n_prompt, int n_new, int32_t *h_tokens);
     int bench_decode(int64_t first_id, int n_steps, float *ms_out, int32_t *h_tokens);
     int profile_step(int64_t token_id, std::vector<StepProfile> &out);
+    int time_kernels(int rounds, std::vector<StepProfile> &out);
     ExecutionPlan *plan() { return plan_.get(); }
 
   private:

@@ -327,20 +327,22 @@ int HfModel::emit_transformer_plan() {
     std::shared_ptr<PlanScratch> scr = scratch_;
     std::vector<CompiledKernel> kernels;
     std::vector<KernelStep> steps;
-    const double kv_bytes_full = 2.0 * kvh * max_seq_len_ * hd * 2;
+    auto gemv_bytes = [](double K, double N, double out_n) { return K * N * 2 + K * 4 + out_n * 4; };
 
     // --- Embedding kernel (reference src/hf/emitter.rs:902-909) ---
     {
         CompiledKernel k;
         k.ops_label = "Embed";
-        k.algorithmic_bytes = hidden * 4.0 * 2;
-        k.launch = [=](const StepContext &sc) -> int {
+        DeviceLaunch l;
+        l.name = "embed";
+        l.bytes_fixed = hidden * 4.0 * 2;
+        l.fn = [=](const StepContext &sc) -> int {
             Buffer *table = sc.pool[sc.step.input_slots[1]];
             Buffer *out = sc.pool[sc.step.output_slots[0]];
-            sc.plan->count_launches(1);
             return embed_step_launch(sc.ctx, sc.plan->state(), sc.plan->forced_ids(), table->as<float>(),
                                      out->as<float>(), (int)vocab, (int)hidden);
         };
+        k.launches.push_back(std::move(l));
         kernels.push_back(std::move(k));
         steps.push_back(KernelStep::kernel(kernels.size() - 1, {input_ids, embed_w}, {embed_out}));
     }
@@ -351,35 +353,39 @@ int HfModel::emit_transformer_plan() {
         {
             CompiledKernel k;
             k.ops_label = qkn ? "QKV+QKNorm+RoPE" : "QKV+RoPE";
-            k.algorithmic_bytes = (double)hidden * (qd + 2 * kvd) * 2;
             const int layer = i;
-            k.launch = [=](const StepContext &sc) -> int {
+            DeviceLaunch g1;
+            g1.name = "gemv_bf16[qkv]";
+            g1.bytes_fixed = gemv_bytes(hidden, qd + 2 * kvd, qd + 2 * kvd) + hidden * 4.0;
+            g1.fn = [=](const StepContext &sc) -> int {
                 const auto &in = sc.step.input_slots;
-                Buffer *h = sc.pool[in[0]], *ln_w = sc.pool[in[1]], *q_w = sc.pool[in[2]];
-                Buffer *cosb = sc.pool[in[5]], *sinb = sc.pool[in[6]];
-                Buffer *q = sc.pool[sc.step.output_slots[0]], *kk = sc.pool[sc.step.output_slots[1]],
-                       *vv = sc.pool[sc.step.output_slots[2]];
                 GemvArgs g;
-                g.x = h->as<float>();
-                g.w = q_w->as<uint16_t>();  // q|k|v rows are adjacent in the packed buffer
-                g.out = q->as<float>();     // q|k|v outputs are adjacent too (aliased slots)
+                g.x = sc.pool[in[0]]->as<float>();
+                g.w = sc.pool[in[2]]->as<uint16_t>();  // q|k|v rows are adjacent in the packed buffer
+                g.out = sc.pool[sc.step.output_slots[0]]->as<float>();  // q|k|v outputs adjacent too
                 g.K = (int)hidden;
                 g.N = (int)(qd + 2 * kvd);
-                g.norm_w = ln_w->as<float>();
+                g.norm_w = sc.pool[in[1]]->as<float>();
                 g.eps = eps;
-                int rc = gemv_bf16_nk_launch(sc.ctx, g, 1, GEMV_EPI_NONE);
-                if (rc != HM_OK) return rc;
+                return gemv_bf16_nk_launch(sc.ctx, g, 1, GEMV_EPI_NONE);
+            };
+            k.launches.push_back(std::move(g1));
+            DeviceLaunch g2;
+            g2.name = qkn ? "qknorm_rope_append" : "rope_append";
+            g2.bytes_fixed = (qd + 2 * kvd) * 4.0 * 2 + 2 * kvd * 2.0 + 2 * hd * 4.0;
+            g2.fn = [=](const StepContext &sc) -> int {
+                const auto &in = sc.step.input_slots;
                 KvCache *cache = sc.plan->kv_cache();
                 QkRopeArgs r;
-                r.q = q->as<float>();
-                r.k = kk->as<float>();
-                r.v = vv->as<float>();
+                r.q = sc.pool[sc.step.output_slots[0]]->as<float>();
+                r.k = sc.pool[sc.step.output_slots[1]]->as<float>();
+                r.v = sc.pool[sc.step.output_slots[2]]->as<float>();
                 if (qkn) {
                     r.qw = sc.pool[in[7]]->as<float>();
                     r.kw = sc.pool[in[8]]->as<float>();
                 }
-                r.cos = cosb->as<float>();
-                r.sin = sinb->as<float>();
+                r.cos = sc.pool[in[5]]->as<float>();
+                r.sin = sc.pool[in[6]]->as<float>();
                 r.S = 1;
                 r.H = (int)H;
                 r.kvh = (int)kvh;
@@ -389,9 +395,9 @@ int HfModel::emit_transformer_plan() {
                 r.vcache = cache->value_ptr(layer);
                 r.max_len = cache->max_len();
                 r.state = sc.plan->state();
-                sc.plan->count_launches(2);
                 return qknorm_rope_launch(sc.ctx, r);
             };
+            k.launches.push_back(std::move(g2));
             kernels.push_back(std::move(k));
             std::vector<size_t> in{s.hidden_in, s.input_ln, s.q_w, s.k_w, s.v_w, cos_s, sin_s};
             if (qkn) {
@@ -412,15 +418,16 @@ int HfModel::emit_transformer_plan() {
         {
             CompiledKernel k;
             k.ops_label = "Attn";
-            k.algorithmic_bytes = (double)qd * hidden * 2 + kv_bytes_full;
-            k.launch = [=](const StepContext &sc) -> int {
+            DeviceLaunch a1;
+            a1.name = "gqa_decode_attn";
+            a1.bytes_fixed = qd * 4.0 * 2;
+            a1.bytes_per_kv_row = 2.0 * kvh * hd * 2;
+            a1.fn = [=](const StepContext &sc) -> int {
                 const auto &in = sc.step.input_slots;
-                Buffer *q = sc.pool[in[0]], *pk = sc.pool[in[1]], *pv = sc.pool[in[2]], *o_w = sc.pool[in[4]];
-                Buffer *out = sc.pool[sc.step.output_slots[0]];
                 AttnArgs a;
-                a.q = q->as<float>();
-                a.kcache = pk->as<uint16_t>();
-                a.vcache = pv->as<uint16_t>();
+                a.q = sc.pool[in[0]]->as<float>();
+                a.kcache = sc.pool[in[1]]->as<uint16_t>();
+                a.vcache = sc.pool[in[2]]->as<uint16_t>();
                 a.out = scr->attn_flat.as<float>();
                 a.B = 1;
                 a.H = (int)H;
@@ -431,17 +438,22 @@ int HfModel::emit_transformer_plan() {
                 a.scale = (float)(1.0 / std::sqrt((double)hd));  // f64 -> f32 constant, emitter.rs:719
                 a.state = sc.plan->state();
                 a.fixed_chunk = att_chunk;
-                int rc = gqa_decode_attn_launch(sc.ctx, a);
-                if (rc != HM_OK) return rc;
+                return gqa_decode_attn_launch(sc.ctx, a);
+            };
+            k.launches.push_back(std::move(a1));
+            DeviceLaunch a2;
+            a2.name = "gemv_bf16[o]";
+            a2.bytes_fixed = gemv_bytes(qd, hidden, hidden);
+            a2.fn = [=](const StepContext &sc) -> int {
                 GemvArgs g;
                 g.x = scr->attn_flat.as<float>();
-                g.w = o_w->as<uint16_t>();
-                g.out = out->as<float>();
+                g.w = sc.pool[sc.step.input_slots[4]]->as<uint16_t>();
+                g.out = sc.pool[sc.step.output_slots[0]]->as<float>();
                 g.K = (int)qd;
                 g.N = (int)hidden;
-                sc.plan->count_launches(2);
                 return gemv_bf16_nk_launch(sc.ctx, g, 1, GEMV_EPI_NONE);
             };
+            k.launches.push_back(std::move(a2));
             kernels.push_back(std::move(k));
             steps.push_back(KernelStep::kernel(kernels.size() - 1,
                                                {s.q, s.present_k, s.present_v, mask, s.o_w}, {s.attn_out}));
@@ -450,34 +462,38 @@ int HfModel::emit_transformer_plan() {
         {
             CompiledKernel k;
             k.ops_label = "MLP";
-            k.algorithmic_bytes = 3.0 * hidden * inter * 2;
-            k.launch = [=](const StepContext &sc) -> int {
+            DeviceLaunch m1;
+            m1.name = "gemv_bf16[gate_up+silu]";
+            m1.bytes_fixed = gemv_bytes(hidden, 2 * inter, inter) + hidden * 4.0 * 3;
+            m1.fn = [=](const StepContext &sc) -> int {
                 const auto &in = sc.step.input_slots;
-                Buffer *h = sc.pool[in[0]], *attn_out = sc.pool[in[1]], *ln_w = sc.pool[in[2]];
-                Buffer *gate_w = sc.pool[in[3]], *down_w = sc.pool[in[5]];
-                Buffer *out = sc.pool[sc.step.output_slots[0]];
                 GemvArgs g;  // gate|up interleaved rows, silu(gate)*up in the epilogue
-                g.x = h->as<float>();
-                g.prologue_residual = attn_out->as<float>();
-                g.norm_w = ln_w->as<float>();
+                g.x = sc.pool[in[0]]->as<float>();
+                g.prologue_residual = sc.pool[in[1]]->as<float>();
+                g.norm_w = sc.pool[in[2]]->as<float>();
                 g.eps = eps;
                 g.resid_out = scr->resid.as<float>();
-                g.w = gate_w->as<uint16_t>();
+                g.w = sc.pool[in[3]]->as<uint16_t>();
                 g.out = scr->act.as<float>();
                 g.K = (int)hidden;
                 g.N = (int)(2 * inter);
-                int rc = gemv_bf16_nk_launch(sc.ctx, g, 1, GEMV_EPI_SILU_MUL_PAIRS);
-                if (rc != HM_OK) return rc;
+                return gemv_bf16_nk_launch(sc.ctx, g, 1, GEMV_EPI_SILU_MUL_PAIRS);
+            };
+            k.launches.push_back(std::move(m1));
+            DeviceLaunch m2;
+            m2.name = "gemv_bf16[down+residual]";
+            m2.bytes_fixed = gemv_bytes(inter, hidden, hidden) + hidden * 4.0;
+            m2.fn = [=](const StepContext &sc) -> int {
                 GemvArgs d;
                 d.x = scr->act.as<float>();
-                d.w = down_w->as<uint16_t>();
-                d.out = out->as<float>();
+                d.w = sc.pool[sc.step.input_slots[5]]->as<uint16_t>();
+                d.out = sc.pool[sc.step.output_slots[0]]->as<float>();
                 d.K = (int)inter;
                 d.N = (int)hidden;
                 d.epilogue_residual = scr->resid.as<float>();
-                sc.plan->count_launches(2);
                 return gemv_bf16_nk_launch(sc.ctx, d, 1, GEMV_EPI_RESIDUAL);
             };
+            k.launches.push_back(std::move(m2));
             kernels.push_back(std::move(k));
             steps.push_back(KernelStep::kernel(
                 kernels.size() - 1, {s.hidden_in, s.attn_out, s.post_ln, s.gate_w, s.up_w, s.down_w},
@@ -489,30 +505,36 @@ int HfModel::emit_transformer_plan() {
     {
         CompiledKernel k;
         k.ops_label = "LMHead";
-        k.algorithmic_bytes = (double)hidden * vocab * 2 + vocab * 4.0;
-        k.launch = [=](const StepContext &sc) -> int {
+        DeviceLaunch h1;
+        h1.name = "gemv_bf16[lm_head+argmax]";
+        h1.bytes_fixed = gemv_bytes(hidden, vocab, vocab) + hidden * 4.0;
+        h1.fn = [=](const StepContext &sc) -> int {
             const auto &in = sc.step.input_slots;
-            Buffer *h = sc.pool[in[0]], *nw = sc.pool[in[1]], *w = sc.pool[in[2]];
-            Buffer *out = sc.pool[sc.step.output_slots[0]];
             GemvArgs g;
-            g.x = h->as<float>();
-            g.norm_w = nw->as<float>();
+            g.x = sc.pool[in[0]]->as<float>();
+            g.norm_w = sc.pool[in[1]]->as<float>();
             g.eps = eps;
-            g.w = w->as<uint16_t>();
-            g.out = out->as<float>();
+            g.w = sc.pool[in[2]]->as<uint16_t>();
+            g.out = sc.pool[sc.step.output_slots[0]]->as<float>();
             g.K = (int)hidden;
             g.N = (int)vocab;
             g.argmax_val = scr->cand_val.as<float>();
             g.argmax_idx = scr->cand_idx.as<int>();
             g.argmax_cap = scr->cand_cap;
-            int rc = gemv_bf16_nk_launch(sc.ctx, g, 1, GEMV_EPI_ARGMAX);
-            if (rc != HM_OK) return rc;
+            return gemv_bf16_nk_launch(sc.ctx, g, 1, GEMV_EPI_ARGMAX);
+        };
+        k.launches.push_back(std::move(h1));
+        DeviceLaunch h2;
+        h2.name = "finish_step";
+        h2.moves_cursor = true;
+        h2.bytes_fixed = 64;
+        h2.fn = [=](const StepContext &sc) -> int {
             const int ncand = std::min(gemv_bf16_nk_grid(sc.ctx, (int)vocab, 4), scr->cand_cap);
-            sc.plan->count_launches(2);
             return finish_step_launch(sc.ctx, sc.plan->state(), scr->cand_val.as<float>(),
                                       scr->cand_idx.as<int>(), ncand, sc.plan->out_tokens(),
                                       sc.plan->out_capacity());
         };
+        k.launches.push_back(std::move(h2));
         kernels.push_back(std::move(k));
         steps.push_back(KernelStep::kernel(kernels.size() - 1, {ls[L - 1].hidden_out, final_norm, lm_head},
                                            {logits}));
@@ -645,6 +667,16 @@ int HfModel::bench_decode(int64_t first_id, int n_steps, float *ms_out, int32_t 
     if (rc != HM_OK) return rc;
     if (h_tokens) rc = hm_download(ctx_, h_tokens, plan_->out_tokens(), (size_t)n_steps * 4);
     return rc;
+}
+
+int HfModel::time_kernels(int rounds, std::vector<StepProfile> &out) {
+    if (!finalized_) return hm_set_error(ctx_, HM_ERR_STATE, "model not finalized");
+    int32_t tok = 0;
+    int rc = plan_->arm(&tok, 1);
+    if (rc != HM_OK) return rc;
+    std::vector<Buffer *> inputs;
+    step_inputs(inputs);
+    return plan_->time_kernels(inputs, weight_bufs_, max_seq_len_, rounds, out);
 }
 
 int HfModel::profile_step(int64_t token_id, std::vector<StepProfile> &out) {

@@ -146,17 +146,32 @@ struct StepContext {
     const std::vector<Buffer *> &pool;  // slot -> buffer (inputs, weights, intermediates)
     const KernelStep &step;
 };
+// One HIP kernel launch inside a compiled kernel, named so that timings and byte counts can be
+// reported per device kernel.
+struct DeviceLaunch {
+    std::string name;                 // e.g. "gemv_bf16[qkv]", "gqa_decode_attn"
+    double bytes_fixed = 0;           // algorithmic bytes per launch (weights + activations)
+    double bytes_per_kv_row = 0;      // plus this much per cached row (attention)
+    bool moves_cursor = false;        // advances the DecodeState (must run exactly once per step)
+    std::function<int(const StepContext &)> fn;
+};
 struct CompiledKernel {
     std::string ops_label;  // "Embed", "QKV+QKNorm+RoPE", "Attn", "MLP", "LMHead", "QuantMM[q]", ...
-    std::function<int(const StepContext &)> launch;
-    double algorithmic_bytes = 0;  // bytes one call has to move (weights + KV at full cache)
+    std::vector<DeviceLaunch> launches;
+    int launch(const StepContext &sc) const {
+        for (const auto &l : launches) {
+            int rc = l.fn(sc);
+            if (rc != HM_OK) return rc;
+        }
+        return HM_OK;
+    }
 };
 
 struct StepProfile {
-    std::string label;
-    float ms = 0;
+    std::string label;  // device kernel name
+    float ms = 0;       // summed over the launches
     int launches = 0;
-    double bytes = 0;
+    double bytes = 0;   // algorithmic bytes summed over the launches
 };
 
 // Ordered kernel dispatch with slot routing (reference ExecutionPlan, src/runtime.rs:1113-1951).
@@ -204,9 +219,17 @@ class ExecutionPlan {
     int enable_graph(bool on);
     bool graph_enabled() const { return use_graph_; }
 
-    // Per-kernel timing of one step (HOMURA_PROFILE analogue, reference src/runtime.rs:1849-1873)
+    // Per-kernel timing of one step (HOMURA_PROFILE analogue, reference src/runtime.rs:1849-1873):
+    // HIP events around every device launch of a real decode step.
     int profile_step(const std::vector<Buffer *> &inputs, std::vector<Buffer> &weights,
                      int max_seq_len, std::vector<StepProfile> &out);
+    // Kernel-by-kernel timing for roofline figures: for every device-kernel name, all its
+    // launches of the step (one per layer, i.e. different weights each time, so nothing is
+    // cache-resident) are issued back to back `rounds` times between two HIP events. Launches
+    // that move the cursor are skipped. Leaves activations and the current cache row in an
+    // unspecified state: call when the decode is over.
+    int time_kernels(const std::vector<Buffer *> &inputs, std::vector<Buffer> &weights,
+                     int max_seq_len, int rounds, std::vector<StepProfile> &out);
 
     const std::vector<KernelStep> &steps() const { return steps_; }
     const std::vector<CompiledKernel> &kernels() const { return kernels_; }
@@ -217,8 +240,7 @@ class ExecutionPlan {
     size_t num_slots() const { return num_slots_; }
     Buffer *slot(size_t s) { return pool_[s]; }
     hm_ctx *ctx() const { return ctx_; }
-    int launches_per_step() const { return launches_per_step_; }
-    void count_launches(int n) { launch_counter_ += n; }
+    int launches_per_step() const;
 
   private:
     int bind(const std::vector<Buffer *> &inputs, std::vector<Buffer> &weights);
@@ -243,8 +265,6 @@ class ExecutionPlan {
     bool use_graph_ = false;
     hipGraph_t graph_ = nullptr;
     hipGraphExec_t graph_exec_ = nullptr;
-    int launches_per_step_ = 0;
-    int launch_counter_ = 0;
 };
 
 }  // namespace homura

@@ -326,12 +326,20 @@ int ExecutionPlan::bind(const std::vector<Buffer *> &inputs, std::vector<Buffer>
     return HM_OK;
 }
 
+int ExecutionPlan::launches_per_step() const {
+    int n = 0;
+    for (const auto &st : steps_)
+        if (st.native_op.kind == NativeOpKind::None) n += (int)kernels_[st.kernel_idx].launches.size();
+    return n;
+}
+
 int ExecutionPlan::run_steps(std::vector<StepProfile> *profile) {
     hipEvent_t e0 = nullptr, e1 = nullptr;
     if (profile) {
         HM_HIP(ctx_, hipEventCreate(&e0));
         HM_HIP(ctx_, hipEventCreate(&e1));
     }
+    const int kv_rows = kv_cache_ ? kv_cache_->current_len() + kv_cache_->new_tokens() : 0;
     std::map<std::string, size_t> by_label;
     for (size_t step_idx = 0; step_idx < steps_.size(); step_idx++) {
         const KernelStep &step = steps_[step_idx];
@@ -348,32 +356,83 @@ int ExecutionPlan::run_steps(std::vector<StepProfile> *profile) {
             if (!pool_[s])  // reference panics with the same message (src/runtime.rs:1700-1705)
                 return hm_set_error(ctx_, HM_ERR_STATE, "buffer slot %zu not populated at step %zu", s, step_idx);
         const CompiledKernel &k = kernels_[step.kernel_idx];
-        const int before = launch_counter_;
-        if (profile) HM_HIP(ctx_, hipEventRecord(e0, ctx_->stream));
         StepContext sc{ctx_, this, pool_, step};
-        int rc = k.launch(sc);
-        if (rc != HM_OK) return rc;
-        if (profile) {
+        if (!profile) {
+            int rc = k.launch(sc);
+            if (rc != HM_OK) return rc;
+            continue;
+        }
+        for (const DeviceLaunch &l : k.launches) {
+            HM_HIP(ctx_, hipEventRecord(e0, ctx_->stream));
+            int rc = l.fn(sc);
+            if (rc != HM_OK) return rc;
             HM_HIP(ctx_, hipEventRecord(e1, ctx_->stream));
             HM_HIP(ctx_, hipEventSynchronize(e1));
             float ms = 0;
             HM_HIP(ctx_, hipEventElapsedTime(&ms, e0, e1));
-            auto it = by_label.find(k.ops_label);
+            auto it = by_label.find(l.name);
             if (it == by_label.end()) {
-                by_label[k.ops_label] = profile->size();
-                profile->push_back(StepProfile{k.ops_label, 0.f, 0, 0.0});
-                it = by_label.find(k.ops_label);
+                by_label[l.name] = profile->size();
+                profile->push_back(StepProfile{l.name, 0.f, 0, 0.0});
+                it = by_label.find(l.name);
             }
             StepProfile &p = (*profile)[it->second];
             p.ms += ms;
-            p.launches += launch_counter_ - before;
-            p.bytes += k.algorithmic_bytes;
+            p.launches += 1;
+            p.bytes += l.bytes_fixed + l.bytes_per_kv_row * kv_rows;
         }
     }
     if (profile) {
         (void)hipEventDestroy(e0);
         (void)hipEventDestroy(e1);
     }
+    return HM_OK;
+}
+
+int ExecutionPlan::time_kernels(const std::vector<Buffer *> &inputs, std::vector<Buffer> &weights,
+                                int max_seq_len, int rounds, std::vector<StepProfile> &out) {
+    if (!prepared_) return hm_set_error(ctx_, HM_ERR_STATE, "plan not prepared");
+    if (rounds < 1) return hm_set_error(ctx_, HM_ERR_INVALID, "time_kernels: rounds must be >= 1");
+    int rc = ensure_kv_cache(max_seq_len);
+    if (rc != HM_OK) return rc;
+    if (kv_cache_->current_len() + 1 > kv_cache_->max_len())
+        return hm_set_error(ctx_, HM_ERR_STATE, "KV cache full (%d + 1 > %d)", kv_cache_->current_len(), kv_cache_->max_len());
+    if ((rc = bind(inputs, weights)) != HM_OK) return rc;
+    const int kv_rows = kv_cache_->current_len() + 1;
+    std::vector<std::string> names;
+    for (const auto &st : steps_) {
+        if (st.native_op.kind != NativeOpKind::None) continue;
+        for (const auto &l : kernels_[st.kernel_idx].launches)
+            if (!l.moves_cursor && std::find(names.begin(), names.end(), l.name) == names.end())
+                names.push_back(l.name);
+    }
+    hipEvent_t e0, e1;
+    HM_HIP(ctx_, hipEventCreate(&e0));
+    HM_HIP(ctx_, hipEventCreate(&e1));
+    for (const auto &name : names) {
+        StepProfile p{name, 0.f, 0, 0.0};
+        for (int r = -1; r < rounds; r++) {  // round -1 is an untimed warm-up
+            if (r == 0) HM_HIP(ctx_, hipEventRecord(e0, ctx_->stream));
+            for (const auto &st : steps_) {
+                if (st.native_op.kind != NativeOpKind::None) continue;
+                StepContext sc{ctx_, this, pool_, st};
+                for (const auto &l : kernels_[st.kernel_idx].launches) {
+                    if (l.name != name) continue;
+                    if ((rc = l.fn(sc)) != HM_OK) return rc;
+                    if (r >= 0) {
+                        p.launches++;
+                        p.bytes += l.bytes_fixed + l.bytes_per_kv_row * kv_rows;
+                    }
+                }
+            }
+        }
+        HM_HIP(ctx_, hipEventRecord(e1, ctx_->stream));
+        HM_HIP(ctx_, hipEventSynchronize(e1));
+        HM_HIP(ctx_, hipEventElapsedTime(&p.ms, e0, e1));
+        out.push_back(p);
+    }
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
     return HM_OK;
 }
 
@@ -391,7 +450,6 @@ int ExecutionPlan::run_kv(const std::vector<Buffer *> &inputs, std::vector<Buffe
     if ((rc = bind(inputs, weights)) != HM_OK) return rc;
     if (use_graph_) {
         if (!graph_exec_) {
-            launch_counter_ = 0;
             HM_HIP(ctx_, hipStreamBeginCapture(ctx_->stream, hipStreamCaptureModeRelaxed));
             rc = run_steps(nullptr);
             hipGraph_t g = nullptr;
@@ -403,14 +461,11 @@ int ExecutionPlan::run_kv(const std::vector<Buffer *> &inputs, std::vector<Buffe
             HM_HIP(ctx_, e);
             graph_ = g;
             HM_HIP(ctx_, hipGraphInstantiate(&graph_exec_, graph_, nullptr, nullptr, 0));
-            launches_per_step_ = launch_counter_;
         }
         HM_HIP(ctx_, hipGraphLaunch(graph_exec_, ctx_->stream));
     } else {
-        launch_counter_ = 0;
         rc = run_steps(nullptr);
         if (rc != HM_OK) return rc;
-        launches_per_step_ = launch_counter_;
     }
     // one advance after all layers appended (reference src/runtime.rs:1875-1880)
     kv_cache_->advance_by(kv_cache_->new_tokens());
@@ -424,7 +479,6 @@ int ExecutionPlan::profile_step(const std::vector<Buffer *> &inputs, std::vector
     if (rc != HM_OK) return rc;
     if ((rc = kv_cache_->note_appended(1)) != HM_OK) return rc;
     if ((rc = bind(inputs, weights)) != HM_OK) return rc;
-    launch_counter_ = 0;
     rc = run_steps(&out);
     if (rc != HM_OK) return rc;
     kv_cache_->advance_by(kv_cache_->new_tokens());

@@ -256,6 +256,10 @@ class HfModel:
         ptrs = (_ffi.c_f32_p * len(arrs))(*[a.ctypes.data_as(_ffi.c_f32_p) for a in arrs])
         self._check(self.lib.hm_model_init_kv_cache(self.h, ptrs, seq_len))
 
+    def set_graph(self, on: bool):
+        """Replay each decode step from a captured HIP graph instead of launching kernel by kernel."""
+        self._check(self.lib.hm_model_set_graph(self.h, int(on)))
+
     def reset_kv_cache(self):
         self._check(self.lib.hm_model_reset_kv_cache(self.h))
 
@@ -285,8 +289,22 @@ class HfModel:
                                                    toks.ctypes.data_as(C.POINTER(C.c_int32))))
         return ms.value, toks
 
-    def profile_step(self, token_id: int):
-        recs = (_ffi.HmKernelProfile * 32)()
-        n = self._check(self.lib.hm_model_profile_step(self.h, token_id, recs, 32))
+    @staticmethod
+    def _records(recs, n):
         return [dict(label=recs[i].label.decode(), ms=recs[i].ms, launches=recs[i].launches,
                      bytes=recs[i].bytes) for i in range(n)]
+
+    def profile_step(self, token_id: int):
+        """One real decode step with HIP events around every device launch."""
+        recs = (_ffi.HmKernelProfile * 32)()
+        n = self._check(self.lib.hm_model_profile_step(self.h, token_id, recs, 32))
+        return self._records(recs, n)
+
+    def time_kernels(self, rounds: int):
+        """Per device kernel: its per-layer launches back to back, `rounds` times (see header)."""
+        recs = (_ffi.HmKernelProfile * 32)()
+        n = self._check(self.lib.hm_model_time_kernels(self.h, rounds, recs, 32))
+        return self._records(recs, n)
+
+    def launches_per_step(self) -> int:
+        return self._check(self.lib.hm_model_launches_per_step(self.h))

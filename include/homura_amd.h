@@ -199,6 +199,10 @@ int hm_model_init_kv_cache(hm_model *m, const float *const *h_kv, int seq_len);
 int hm_model_reset_kv_cache(hm_model *m);  /* src/runtime.rs:1941-1945 */
 int hm_model_kv_cache_len(hm_model *m);    /* src/runtime.rs:1948-1950 */
 
+/* Replay every decode step from one captured HIP graph (on != 0) or launch kernel by kernel.
+ * No counterpart in the reference (its plan is a host loop over dlsym'ed functions). */
+int hm_model_set_graph(hm_model *m, int on);
+
 /* HfModel::run_kv (src/hf/model.rs:198-218) -> ExecutionPlan::run_kv
  * (src/runtime.rs:1580-1892): n_ids new tokens on top of the cache; h_logits receives
  * [n_ids][vocab] f32 (may be NULL to skip the download). Advances the cache by n_ids. */
@@ -217,15 +221,22 @@ int hm_model_generate_greedy(hm_model *m, const int64_t *h_prompt, int n_prompt,
 int hm_model_bench_decode(hm_model *m, int64_t first_id, int n_steps, float *ms_out,
                           int32_t *h_tokens_out);
 
-/* Per-kernel profile of one decode step (HOMURA_PROFILE analogue): fills up to `cap`
- * records; returns the number written. */
+/* Per-kernel profile of one decode step (HOMURA_PROFILE analogue, reference
+ * src/runtime.rs:1849-1873): HIP events around every device launch; one record per device
+ * kernel name. Fills up to `cap` records; returns the number written. */
 typedef struct {
-    char label[32]; /* "Embed", "QKV", "KVConcat", "Attn", "O", "GateUp", "Down", "LMHead", ... */
-    float ms;       /* summed over layers */
+    char label[32]; /* "gemv_bf16[qkv]", "gqa_decode_attn", "gemv_bf16[lm_head+argmax]", ... */
+    float ms;       /* summed over the launches */
     int launches;
     double bytes;   /* algorithmic bytes moved by these launches */
 } hm_kernel_profile;
 int hm_model_profile_step(hm_model *m, int64_t token_id, hm_kernel_profile *out, int cap);
+/* Roofline timing: per device kernel name, all of the step's launches of that kernel (one per
+ * layer, different weights each) back to back, `rounds` times, between two HIP events.
+ * Disturbs activations and the current cache row: call after the decode. */
+int hm_model_time_kernels(hm_model *m, int rounds, hm_kernel_profile *out, int cap);
+/* Number of HIP kernel launches one decode step issues. */
+int hm_model_launches_per_step(hm_model *m);
 
 /* ── deterministic synthetic data (host side, no GPU needed) ─────────────────
  * Counter-based generator shared by tests and benchmarks: sample i of stream `seed` uses

