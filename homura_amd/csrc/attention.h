@@ -13,6 +13,12 @@ struct AttnArgs {
     // for max_len with a fixed chunk (workgroups past the live range exit at once).
     const DecodeState *state = nullptr;
     int fixed_chunk = 0;
+    // Fused prologue (decode plan, B == 1): when qkv_raw is set, q is ignored; the kernel applies
+    // QK-norm + RoPE to the raw projection row and appends the new K/V row to the caches.
+    const float *qkv_raw = nullptr;  // [H*hd | kvh*hd | kvh*hd]
+    const float *qw = nullptr, *kw = nullptr;
+    const float *cos_tab = nullptr, *sin_tab = nullptr;  // [max_pos][hd]
+    float eps = 0.f;
 };
 
 int gqa_decode_attn_launch(hm_ctx *ctx, const AttnArgs &a);

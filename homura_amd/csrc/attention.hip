@@ -5,8 +5,8 @@
 // its KV head (the reference's `h floordiv g` map, src/graph_builder/emit_linalg.rs:123-127),
 // so each K/V row is read from HBM once. Rows are streamed with 16-byte loads: HD/8 lanes
 // cover a row, 64/(HD/8) rows per wavefront instruction. Scores live in LDS; softmax is f32.
-// Partial (o, max, sum) triples go to the workspace and the last workgroup to arrive for a
-// (batch, kv head) folds them in split order, so the result does not depend on timing.
+// Partial (o, max, sum) triples go to the workspace and a second, tiny kernel folds them per
+// (batch, kv head) in split order, so the result does not depend on timing.
 // Algorithmic HBM traffic: 2 * kv_len * HD * 2 bytes per (batch, kv head).
 #include "attention.h"
 
@@ -22,58 +22,149 @@ __device__ __forceinline__ void unpack8(const u32x4 w, float *f) {
     f[6] = bf16_lo(w.w); f[7] = bf16_hi(w.w);
 }
 
+constexpr int NRG_MAX = 8;  // row groups per wavefront held in registers (K and V each)
+
+// Optional prologue fused into the attention kernel (decode plan, batch 1): the raw q|k|v row
+// produced by the QKV projection goes through the per-head QK-norm and RoPE of the reference's
+// QKV kernel (src/hf/emitter.rs:629-644) here, and the workgroup that owns the last live split
+// rounds the new K/V row to bf16, appends it to the cache (KvCache::append_key/append_value,
+// src/runtime.rs:521-568) and uses the rounded values itself.
+struct AttnFuse {
+    const float *qkv_raw;   // [H*hd | kvh*hd | kvh*hd] f32
+    const float *qw, *kw;   // [hd] or nullptr
+    const float *cos_tab;   // [max_pos][hd]
+    const float *sin_tab;
+    float eps;
+};
+
+// One wavefront: optional RMSNorm over hd, then x*cos + rotate_half(x)*sin; lane i < hd/2 owns
+// the rotation pair (i, i + hd/2) and gets its two results back in (o_lo, o_hi).
+template <int HD>
+__device__ __forceinline__ void norm_rope_row(const float *__restrict__ src,
+                                              const float *__restrict__ nw,
+                                              const float *__restrict__ c,
+                                              const float *__restrict__ sn, float eps, int lane,
+                                              float &o_lo, float &o_hi) {
+    constexpr int HALF = HD / 2;
+    const bool on = lane < HALF;
+    float lo = on ? src[lane] : 0.f, hi = on ? src[lane + HALF] : 0.f;
+    const float c_lo = on ? c[lane] : 0.f, c_hi = on ? c[lane + HALF] : 0.f;
+    const float s_lo = on ? sn[lane] : 0.f, s_hi = on ? sn[lane + HALF] : 0.f;
+    const float w_lo = (on && nw) ? nw[lane] : 1.f, w_hi = (on && nw) ? nw[lane + HALF] : 1.f;
+    if (nw) {
+        const float ss = wave_sum(lo * lo + hi * hi);
+        const float inv = 1.0f / sqrtf(ss / (float)HD + eps);
+        lo = (lo * inv) * w_lo;
+        hi = (hi * inv) * w_hi;
+    }
+    o_lo = lo * c_lo + (-hi) * s_lo;
+    o_hi = hi * c_hi + lo * s_hi;
+}
+
 template <int HD, int G>
 __global__ __launch_bounds__(ATT_THREADS) void gqa_decode_attn_kernel(
-    const float *__restrict__ q, const uint16_t *__restrict__ kcache,
-    const uint16_t *__restrict__ vcache, float *__restrict__ out, float *__restrict__ part_o,
-    float *__restrict__ part_ml, unsigned int *__restrict__ counters, int kvh, int max_len,
-    int kv_len_arg, int chunk, float scale, const DecodeState *__restrict__ state) {
-    constexpr int LPR = HD / 8;    // lanes per row
+    const float *__restrict__ q, uint16_t *__restrict__ kcache, uint16_t *__restrict__ vcache,
+    float *__restrict__ out, float *__restrict__ part_o, float *__restrict__ part_ml, int kvh,
+    int max_len, int kv_len_arg, int chunk, float scale, const DecodeState *__restrict__ state,
+    int lds_front, AttnFuse fuse) {
+    constexpr int LPR = HD / 8;      // lanes per row
     constexpr int RPI = WAVE / LPR;  // rows per wavefront instruction
     extern __shared__ float sm[];
-    float *sc = sm;                          // [G][chunk] scores, then probabilities
-    float *red = sm + (size_t)G * chunk;     // [ATT_WAVES][G][HD]
+    float *sc = sm;               // [G][chunk] scores, then probabilities; later the fold's (m,l)
+    float *red = sm + lds_front;  // [ATT_WAVES][G][HD]
+    __shared__ float qs[G][HD];
+    __shared__ float knew[HD], vnew[HD];
     __shared__ float s_m[G], s_l[G];
-    __shared__ bool is_last;
 
     const int tid = threadIdx.x, lane = tid & (WAVE - 1), wave = tid / WAVE;
     const int sub = lane / LPR, dl = lane % LPR;
-    const int kv_len = state ? state->pos + 1 : kv_len_arg;
     const int split = blockIdx.x, kvhd = blockIdx.y, b = blockIdx.z;
-    const int nsplit = (kv_len + chunk - 1) / chunk;  // live splits; the grid may be larger
-    if (split >= nsplit) return;
     const int H = kvh * G;
     const int n0 = split * chunk;
-    const int cnt = min(kv_len, n0 + chunk) - n0;
     const size_t head_base = ((size_t)b * kvh + kvhd) * max_len * HD;
     const uint16_t *kbase = kcache + head_base + (size_t)n0 * HD + dl * 8;
     const uint16_t *vbase = vcache + head_base + (size_t)n0 * HD + dl * 8;
+    const int nrg = chunk / (ATT_WAVES * RPI);  // row groups per wavefront (<= NRG_MAX)
+    const int row_cap = min(chunk, max_len - n0);  // rows of this chunk that exist in the cache
+
+    // ── every K and V row of the chunk is requested before anything waits ──
+    u32x4 kreg[NRG_MAX], vreg[NRG_MAX];
+#pragma unroll
+    for (int i = 0; i < NRG_MAX; i++) {
+        const int row = (i * ATT_WAVES + wave) * RPI + sub;
+        const bool ok = i < nrg && row < row_cap;
+        kreg[i] = ok ? ld128_stream(kbase + (size_t)row * HD) : u32x4{0u, 0u, 0u, 0u};
+        vreg[i] = ok ? ld128_stream(vbase + (size_t)row * HD) : u32x4{0u, 0u, 0u, 0u};
+    }
+
+    const int kv_len = state ? state->pos + 1 : kv_len_arg;
+    const int nsplit = (kv_len + chunk - 1) / chunk;  // live splits; the grid may be larger
+    if (split >= nsplit) return;
+    const int cnt = min(kv_len, n0 + chunk) - n0;
+    const bool fused = fuse.qkv_raw != nullptr;
+    const int pos = kv_len - 1;
+    const bool owner = fused && split == nsplit - 1;  // this chunk holds the new row
+    const int new_row = pos - n0;
+
+    // ── queries (and, for the owner, the new K/V row) into LDS ──
+    if (fused) {
+        const float *c = fuse.cos_tab + (size_t)pos * HD;
+        const float *sn = fuse.sin_tab + (size_t)pos * HD;
+        constexpr int HALF = HD / 2;
+        for (int t = wave; t < G + 2; t += ATT_WAVES) {
+            if (t < G) {
+                float lo, hi;
+                norm_rope_row<HD>(fuse.qkv_raw + (size_t)(kvhd * G + t) * HD, fuse.qw, c, sn, fuse.eps,
+                                  lane, lo, hi);
+                if (lane < HALF) {
+                    qs[t][lane] = lo;
+                    qs[t][lane + HALF] = hi;
+                }
+            } else if (owner && t == G) {
+                float lo, hi;
+                norm_rope_row<HD>(fuse.qkv_raw + (size_t)H * HD + (size_t)kvhd * HD, fuse.kw, c, sn,
+                                  fuse.eps, lane, lo, hi);
+                // round to bf16 exactly once; cache and this kernel use the same rounded values
+                if (lane < HALF) {
+                    uint16_t *dst = kcache + head_base + (size_t)pos * HD;
+                    const uint16_t r_lo = f32_to_bf16_rne_dev(lo), r_hi = f32_to_bf16_rne_dev(hi);
+                    dst[lane] = r_lo;
+                    dst[lane + HALF] = r_hi;
+                    knew[lane] = __uint_as_float((uint32_t)r_lo << 16);
+                    knew[lane + HALF] = __uint_as_float((uint32_t)r_hi << 16);
+                }
+            } else if (owner && t == G + 1) {
+                const float *src = fuse.qkv_raw + (size_t)(H + kvh) * HD + (size_t)kvhd * HD;
+                uint16_t *dst = vcache + head_base + (size_t)pos * HD;
+                for (int i = lane; i < HD; i += WAVE) {
+                    const uint16_t r = f32_to_bf16_rne_dev(src[i]);
+                    dst[i] = r;
+                    vnew[i] = __uint_as_float((uint32_t)r << 16);
+                }
+            }
+        }
+    } else {
+        for (int i = tid; i < G * HD; i += ATT_THREADS)
+            qs[i / HD][i % HD] = q[((size_t)b * H + kvhd * G) * HD + i];
+    }
+    __syncthreads();
 
     float qv[G][8];
 #pragma unroll
-    for (int gi = 0; gi < G; gi++) {
-        const float *qp = q + ((size_t)b * H + kvhd * G + gi) * HD + dl * 8;
-        const f32x4 a = *reinterpret_cast<const f32x4 *>(qp);
-        const f32x4 c = *reinterpret_cast<const f32x4 *>(qp + 4);
-        qv[gi][0] = a.x; qv[gi][1] = a.y; qv[gi][2] = a.z; qv[gi][3] = a.w;
-        qv[gi][4] = c.x; qv[gi][5] = c.y; qv[gi][6] = c.z; qv[gi][7] = c.w;
-    }
+    for (int gi = 0; gi < G; gi++)
+#pragma unroll
+        for (int e = 0; e < 8; e++) qv[gi][e] = qs[gi][dl * 8 + e];
 
-    // ── scores = (Q.K^T) * scale ──
-    constexpr int U = 4;
-    const int ngroups = (cnt + RPI - 1) / RPI;
-    for (int rg0 = wave; rg0 < ngroups; rg0 += ATT_WAVES * U) {
-        u32x4 kv[U];
+    // ── scores = (Q.K^T) * scale; rows outside the live range (and the not-yet-written new
+    //    row) are dropped here ──
 #pragma unroll
-        for (int u = 0; u < U; u++) {
-            const int row = (rg0 + u * ATT_WAVES) * RPI + sub;
-            kv[u] = row < cnt ? ld128_stream(kbase + (size_t)row * HD) : u32x4{0u, 0u, 0u, 0u};
-        }
-#pragma unroll
-        for (int u = 0; u < U; u++) {
-            const int row = (rg0 + u * ATT_WAVES) * RPI + sub;
+    for (int i = 0; i < NRG_MAX; i++) {
+        if (i < nrg) {
+            const int row = (i * ATT_WAVES + wave) * RPI + sub;
+            const bool live = row < cnt && !(owner && row == new_row);
+            if (!live) vreg[i] = u32x4{0u, 0u, 0u, 0u};  // stale rows may hold anything
             float kf[8];
-            unpack8(kv[u], kf);
+            unpack8(kreg[i], kf);
 #pragma unroll
             for (int gi = 0; gi < G; gi++) {
                 float p = 0.f;
@@ -81,8 +172,19 @@ __global__ __launch_bounds__(ATT_THREADS) void gqa_decode_attn_kernel(
                 for (int e = 0; e < 8; e++) p = fmaf(kf[e], qv[gi][e], p);
 #pragma unroll
                 for (int off = LPR / 2; off >= 1; off >>= 1) p += __shfl_xor(p, off, WAVE);
-                if (dl == 0 && row < cnt) sc[gi * chunk + row] = p * scale;
+                if (dl == 0 && live) sc[gi * chunk + row] = p * scale;
             }
+        }
+    }
+    if (owner && wave == 0) {  // the new row's score from the rounded values in LDS
+#pragma unroll
+        for (int gi = 0; gi < G; gi++) {
+            float p = 0.f;
+#pragma unroll
+            for (int e = 0; e < 8; e++) p = fmaf(knew[dl * 8 + e], qv[gi][e], p);
+#pragma unroll
+            for (int off = LPR / 2; off >= 1; off >>= 1) p += __shfl_xor(p, off, WAVE);
+            if (lane == 0) sc[gi * chunk + new_row] = p * scale;
         }
     }
     __syncthreads();
@@ -113,25 +215,26 @@ __global__ __launch_bounds__(ATT_THREADS) void gqa_decode_attn_kernel(
     for (int gi = 0; gi < G; gi++)
 #pragma unroll
         for (int e = 0; e < 8; e++) acc[gi][e] = 0.f;
-
-    for (int rg0 = wave; rg0 < ngroups; rg0 += ATT_WAVES * U) {
-        u32x4 vv[U];
 #pragma unroll
-        for (int u = 0; u < U; u++) {
-            const int row = (rg0 + u * ATT_WAVES) * RPI + sub;
-            vv[u] = row < cnt ? ld128_stream(vbase + (size_t)row * HD) : u32x4{0u, 0u, 0u, 0u};
-        }
-#pragma unroll
-        for (int u = 0; u < U; u++) {
-            const int row = (rg0 + u * ATT_WAVES) * RPI + sub;
+    for (int i = 0; i < NRG_MAX; i++) {
+        if (i < nrg) {
+            const int row = (i * ATT_WAVES + wave) * RPI + sub;
             float vf[8];
-            unpack8(vv[u], vf);
+            unpack8(vreg[i], vf);
 #pragma unroll
             for (int gi = 0; gi < G; gi++) {
                 const float p = row < cnt ? sc[gi * chunk + row] : 0.f;
 #pragma unroll
                 for (int e = 0; e < 8; e++) acc[gi][e] = fmaf(p, vf[e], acc[gi][e]);
             }
+        }
+    }
+    if (owner && wave == 0 && sub == 0) {
+#pragma unroll
+        for (int gi = 0; gi < G; gi++) {
+            const float p = sc[gi * chunk + new_row];
+#pragma unroll
+            for (int e = 0; e < 8; e++) acc[gi][e] = fmaf(p, vnew[dl * 8 + e], acc[gi][e]);
         }
     }
     // fold the RPI row-subgroups of the wavefront, then the waves of the workgroup
@@ -171,30 +274,57 @@ __global__ __launch_bounds__(ATT_THREADS) void gqa_decode_attn_kernel(
         pml[tid * 2] = s_m[tid];
         pml[tid * 2 + 1] = s_l[tid];
     }
-    __threadfence();
-    __syncthreads();
-    if (tid == 0) {
-        const unsigned int prev = atomicAdd(&counters[pair], 1u);
-        is_last = prev == (unsigned int)(nsplit - 1);
-    }
-    __syncthreads();
-    if (!is_last) return;
-    __threadfence();
+}
+
+// Second half of the split attention: one workgroup per (batch, kv head) folds the partial
+// (o, max, sum) triples in ascending split order. A separate launch instead of a
+// "last workgroup to arrive" fold: the kernel boundary orders the partial writes, so no
+// device-scope fence (a full L2 write-back + invalidate on this chip) is needed.
+template <int HD, int G>
+__global__ __launch_bounds__(ATT_THREADS) void gqa_decode_fold_kernel(
+    float *__restrict__ out, const float *__restrict__ part_o, const float *__restrict__ part_ml,
+    int kvh, int kv_len_arg, int chunk, const DecodeState *__restrict__ state) {
+    extern __shared__ float s_ml[];  // [nsplit][G][2]
+    const int tid = threadIdx.x;
+    const int kvhd = blockIdx.x, b = blockIdx.y;
+    const int H = kvh * G;
+    const int kv_len = state ? state->pos + 1 : kv_len_arg;
+    const int nsplit = (kv_len + chunk - 1) / chunk;
+    if (nsplit == 1) return;  // the attention kernel wrote the final result itself
+    const size_t pair = (size_t)b * kvh + kvhd;
     const float *ao = part_o + pair * nsplit * G * HD;
     const float *aml = part_ml + pair * nsplit * G * 2;
-    for (int i = tid; i < G * HD; i += ATT_THREADS) {
+    for (int i = tid; i < nsplit * G * 2; i += ATT_THREADS) s_ml[i] = aml[i];
+    for (int i0 = 0; i0 < G * HD; i0 += ATT_THREADS) {
+        const int i = i0 + tid;
         const int gi = i / HD, d = i % HD;
-        float M = -INFINITY;
-        for (int s = 0; s < nsplit; s++) M = fmaxf(M, aml[((size_t)s * G + gi) * 2]);
-        float L = 0.f, O = 0.f;
-        for (int s = 0; s < nsplit; s++) {
-            const float wgt = expf(aml[((size_t)s * G + gi) * 2] - M);
-            L = fmaf(wgt, aml[((size_t)s * G + gi) * 2 + 1], L);
-            O = fmaf(wgt, ao[((size_t)s * G + gi) * HD + d], O);
+        constexpr int FB = 16;  // splits fetched per batch, all loads of a batch in flight together
+        float L = 0.f, O = 0.f, M = -INFINITY;
+        bool have_m = false;
+        for (int s0 = 0; s0 < nsplit; s0 += FB) {
+            float o[FB];
+#pragma unroll
+            for (int u = 0; u < FB; u++)
+                o[u] = (i < G * HD && s0 + u < nsplit) ? ao[((size_t)(s0 + u) * G + gi) * HD + d] : 0.f;
+            if (!have_m) {
+                __syncthreads();  // s_ml complete (uniform across the block)
+                if (i < G * HD)
+                    for (int s = 0; s < nsplit; s++) M = fmaxf(M, s_ml[(s * G + gi) * 2]);
+                have_m = true;
+            }
+            if (i < G * HD) {
+#pragma unroll
+                for (int u = 0; u < FB; u++) {
+                    if (s0 + u < nsplit) {
+                        const float wgt = expf(s_ml[((s0 + u) * G + gi) * 2] - M);
+                        L = fmaf(wgt, s_ml[((s0 + u) * G + gi) * 2 + 1], L);
+                        O = fmaf(wgt, o[u], O);
+                    }
+                }
+            }
         }
-        out[((size_t)b * H + kvhd * G + gi) * HD + d] = O / L;
+        if (i < G * HD) out[((size_t)b * H + kvhd * G + gi) * HD + d] = O / L;
     }
-    if (tid == 0) counters[pair] = 0u;
 }
 
 // KvCache::append_key / append_value (reference src/runtime.rs:521-568) with the cache in
@@ -215,14 +345,25 @@ __global__ void kv_append_kernel(uint16_t *__restrict__ kc, uint16_t *__restrict
 
 template <int HD, int G>
 int launch_attn(hm_ctx *ctx, const AttnArgs &a, int nsplit, int chunk) {
-    const size_t lds = ((size_t)G * chunk + (size_t)ATT_WAVES * G * HD) * sizeof(float);
+    // scores [G][chunk] + wave partials [4][G][HD]
+    const size_t front = (size_t)G * chunk;
+    const size_t lds = (front + (size_t)ATT_WAVES * G * HD) * sizeof(float);
     const size_t pairs = (size_t)a.B * a.kvh;
     float *part_o = (float *)ctx->workspace;
     float *part_ml = part_o + pairs * nsplit * G * HD;
+    AttnFuse f{a.qkv_raw, a.qw, a.kw, a.cos_tab, a.sin_tab, a.eps};
     hipLaunchKernelGGL((gqa_decode_attn_kernel<HD, G>), dim3(nsplit, a.kvh, a.B), dim3(ATT_THREADS),
-                       lds, ctx->stream, a.q, a.kcache, a.vcache, a.out, part_o, part_ml,
-                       ctx->counters, a.kvh, a.max_len, a.kv_len, chunk, a.scale, a.state);
+                       lds, ctx->stream, a.q, const_cast<uint16_t *>(a.kcache),
+                       const_cast<uint16_t *>(a.vcache), a.out, part_o, part_ml, a.kvh, a.max_len,
+                       a.kv_len, chunk, a.scale, a.state, (int)front, f);
     HM_LAUNCH_CHECK(ctx);
+    if (nsplit > 1) {  // nsplit is the grid's split count: 1 means no call can ever need a fold
+        const size_t fold_lds = (size_t)nsplit * G * 2 * sizeof(float);
+        HM_REQUIRE(ctx, fold_lds <= 64 * 1024, "gqa_decode_attn: too many splits (%d)", nsplit);
+        hipLaunchKernelGGL((gqa_decode_fold_kernel<HD, G>), dim3(a.kvh, a.B), dim3(ATT_THREADS), fold_lds,
+                           ctx->stream, a.out, part_o, part_ml, a.kvh, a.kv_len, chunk, a.state);
+        HM_LAUNCH_CHECK(ctx);
+    }
     return HM_OK;
 }
 
@@ -245,26 +386,32 @@ int dispatch_g(hm_ctx *ctx, const AttnArgs &a, int g, int nsplit, int chunk) {
 }  // namespace
 
 int gqa_decode_attn_launch(hm_ctx *ctx, const AttnArgs &a) {
-    HM_REQUIRE(ctx, a.q && a.kcache && a.vcache && a.out, "gqa_decode_attn: NULL pointer");
+    HM_REQUIRE(ctx, a.kcache && a.vcache && a.out, "gqa_decode_attn: NULL pointer");
     HM_REQUIRE(ctx, a.B > 0 && a.H > 0 && a.kvh > 0 && a.H % a.kvh == 0, "gqa_decode_attn: bad head counts H=%d kvh=%d", a.H, a.kvh);
     HM_REQUIRE(ctx, a.hd == 128 || a.hd == 64, "gqa_decode_attn: head_dim %d not supported (64, 128)", a.hd);
     if (!a.state) HM_REQUIRE(ctx, a.kv_len >= 1 && a.kv_len <= a.max_len, "gqa_decode_attn: kv_len=%d outside 1..max_len=%d", a.kv_len, a.max_len);
-    HM_REQUIRE(ctx, ((uintptr_t)a.q % 16) == 0 && ((uintptr_t)a.kcache % 16) == 0 && ((uintptr_t)a.vcache % 16) == 0, "gqa_decode_attn: pointers must be 16-byte aligned");
+    HM_REQUIRE(ctx, ((uintptr_t)a.kcache % 16) == 0 && ((uintptr_t)a.vcache % 16) == 0, "gqa_decode_attn: caches must be 16-byte aligned");
     const int g = a.H / a.kvh;
     const size_t pairs = (size_t)a.B * a.kvh;
-    HM_REQUIRE(ctx, pairs <= ctx->num_counters, "gqa_decode_attn: B*kvh=%zu too large", pairs);
-    // Aim at ~2 workgroups per CU; a workgroup takes at least 32 rows and at most 1024.
+    // A workgroup keeps its whole chunk in registers: 32..128 rows. Aim at about one workgroup
+    // per CU over the rows that can be live.
     const int rows_step = 32;
     const int span = a.state ? a.max_len : a.kv_len;  // rows the grid has to be able to cover
     int chunk = a.fixed_chunk;
     if (chunk <= 0) {
-        int want = (int)((2 * (size_t)ctx->num_cus + pairs - 1) / pairs);
+        int want = (int)(((size_t)ctx->num_cus + pairs - 1) / pairs);
         chunk = (span + want - 1) / want;
         chunk = (chunk + rows_step - 1) / rows_step * rows_step;
-        if (chunk < rows_step) chunk = rows_step;
-        if (chunk > 1024) chunk = 1024;
     }
-    HM_REQUIRE(ctx, chunk % 16 == 0 && chunk <= 1024, "gqa_decode_attn: bad chunk %d", chunk);
+    if (chunk < rows_step) chunk = rows_step;
+    if (chunk > 128) chunk = 128;
+    HM_REQUIRE(ctx, chunk % rows_step == 0, "gqa_decode_attn: chunk %d must be a multiple of 32", chunk);
+    if (a.qkv_raw) {
+        HM_REQUIRE(ctx, a.B == 1 && a.state && a.cos_tab && a.sin_tab, "gqa_decode_attn: the fused prologue needs batch 1, a decode cursor and RoPE tables");
+        HM_REQUIRE(ctx, (a.qw == nullptr) == (a.kw == nullptr), "gqa_decode_attn: q and k norm weights must come together");
+    } else {
+        HM_REQUIRE(ctx, a.q != nullptr, "gqa_decode_attn: NULL query");
+    }
     int nsplit = (span + chunk - 1) / chunk;
     const size_t ws_need = pairs * nsplit * g * (a.hd + 2) * sizeof(float);
     HM_REQUIRE(ctx, ws_need <= ctx->workspace_bytes, "gqa_decode_attn: workspace too small (%zu bytes needed)", ws_need);

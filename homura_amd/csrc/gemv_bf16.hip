@@ -30,6 +30,48 @@ __device__ __forceinline__ void stage_activations(float *xs, const float *__rest
                                                   bool write_resid) {
     __shared__ float red[GEMV_WAVES];
     const int tid = threadIdx.x;
+    constexpr int XMAX = 16;  // K <= 4096 keeps a thread's elements in registers
+    if (K <= XMAX * GEMV_THREADS) {
+        for (int m = 0; m < MT; m++) {
+            // every global load of the prologue is issued before anything waits on one
+            float xv[XMAX], rv[XMAX], wv[XMAX];
+#pragma unroll
+            for (int j = 0; j < XMAX; j++) {
+                const int k = tid + j * GEMV_THREADS;
+                const bool ok = k < K;
+                xv[j] = ok ? x[(size_t)m * K + k] : 0.f;
+                rv[j] = (ok && res) ? res[(size_t)m * K + k] : 0.f;
+                wv[j] = (ok && norm_w) ? norm_w[k] : 0.f;
+            }
+            float ss = 0.f;
+#pragma unroll
+            for (int j = 0; j < XMAX; j++) {
+                if (res) xv[j] = xv[j] + rv[j];
+                ss += xv[j] * xv[j];
+            }
+            float inv = 1.f;
+            if (norm_w) {
+                ss = wave_sum(ss);
+                if (m > 0) __syncthreads();
+                if ((tid & (WAVE - 1)) == 0) red[tid / WAVE] = ss;
+                __syncthreads();
+                float tot = 0.f;
+#pragma unroll
+                for (int w = 0; w < GEMV_WAVES; w++) tot += red[w];
+                inv = 1.0f / sqrtf(tot / (float)K + eps);
+            }
+#pragma unroll
+            for (int j = 0; j < XMAX; j++) {
+                const int k = tid + j * GEMV_THREADS;
+                if (k < K) {
+                    if (write_resid && resid_out) resid_out[(size_t)m * K + k] = xv[j];
+                    xs[m * K + k] = norm_w ? (xv[j] * inv) * wv[j] : xv[j];
+                }
+            }
+        }
+        __syncthreads();
+        return;
+    }
     for (int m = 0; m < MT; m++) {
         float ss = 0.f;
         for (int k = tid; k < K; k += GEMV_THREADS) {
@@ -199,6 +241,163 @@ __global__ __launch_bounds__(GEMV_THREADS) void gemv_bf16_nk_kernel(GemvArgs a) 
     }
 }
 
+// Latency-ordered variant for one activation row and a matrix small enough that every
+// wavefront owns exactly one group of R rows: the wavefront's whole weight slice (R rows x NC
+// chunks of 512 k) is requested first, the activation prologue (residual add, RMSNorm) runs
+// while those loads are in flight, and only then does anything wait. One HBM round trip per
+// kernel instead of two.
+template <int R, int NC>
+__global__ __launch_bounds__(GEMV_THREADS) void gemv_bf16_nk_oneshot_kernel(GemvArgs a, int epi) {
+    extern __shared__ float xs[];  // [K]
+    __shared__ float red[GEMV_WAVES];
+    const int K = a.K, N = a.N;
+    const int tid = threadIdx.x;
+    const int lane = tid & (WAVE - 1);
+    const int wave = tid / WAVE;
+    const int row0 = (blockIdx.x * GEMV_WAVES + wave) * R;
+    constexpr int NX = 2 * NC;  // K <= 512 * NC: a thread stages at most NX activation elements
+
+    // Loads return to a wavefront in issue order, so the (small, needed-first) activation loads
+    // go out before the weight stream and can be consumed while the weights are still in flight.
+    float xv[NX], rv[NX], nw[NX];
+#pragma unroll
+    for (int j = 0; j < NX; j++) {
+        const int k = tid + j * GEMV_THREADS;
+        const bool ok = k < K;
+        xv[j] = ok ? a.x[k] : 0.f;
+        rv[j] = (ok && a.prologue_residual) ? a.prologue_residual[k] : 0.f;
+        nw[j] = (ok && a.norm_w) ? a.norm_w[k] : 0.f;
+    }
+    u32x4 wv[NC][R];
+#pragma unroll
+    for (int c = 0; c < NC; c++) {
+        const int k = (c * WAVE + lane) * 8;
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            const int row = row0 + r < N ? row0 + r : N - 1;  // clamp: stays inside the matrix
+            wv[c][r] = k < K ? ld128_stream(a.w + (size_t)row * K + k) : u32x4{0u, 0u, 0u, 0u};
+        }
+    }
+
+    // residual add (reference src/hf/emitter.rs:787) and RMSNorm
+    // (src/graph_builder/emit_linalg.rs:7-26); identical arithmetic in every workgroup
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < NX; j++) {
+        if (a.prologue_residual) xv[j] = xv[j] + rv[j];
+        ss += xv[j] * xv[j];
+    }
+    float inv = 1.f;
+    if (a.norm_w) {
+        ss = wave_sum(ss);
+        if (lane == 0) red[wave] = ss;
+        __syncthreads();
+        float tot = 0.f;
+#pragma unroll
+        for (int w = 0; w < GEMV_WAVES; w++) tot += red[w];
+        inv = 1.0f / sqrtf(tot / (float)K + a.eps);
+    }
+#pragma unroll
+    for (int j = 0; j < NX; j++) {
+        const int k = tid + j * GEMV_THREADS;
+        if (k < K) {
+            if (blockIdx.x == 0 && a.resid_out) a.resid_out[k] = xv[j];
+            xs[k] = a.norm_w ? (xv[j] * inv) * nw[j] : xv[j];
+        }
+    }
+    __syncthreads();
+
+    float acc[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) acc[r] = 0.f;
+#pragma unroll
+    for (int c = 0; c < NC; c++) {
+        const int k = (c * WAVE + lane) * 8;
+        if (k < K) {
+            float xv[8];
+            const f32x4 x0 = *reinterpret_cast<const f32x4 *>(xs + k);
+            const f32x4 x1 = *reinterpret_cast<const f32x4 *>(xs + k + 4);
+            xv[0] = x0.x; xv[1] = x0.y; xv[2] = x0.z; xv[3] = x0.w;
+            xv[4] = x1.x; xv[5] = x1.y; xv[6] = x1.z; xv[7] = x1.w;
+#pragma unroll
+            for (int r = 0; r < R; r++) acc[r] = dot8(wv[c][r], xv, acc[r]);
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < R; r++) acc[r] = wave_sum(acc[r]);
+
+    if (epi == GEMV_EPI_SILU_MUL_PAIRS) {
+        if constexpr (R % 2 == 0) {
+#pragma unroll
+            for (int r = 0; r < R; r += 2) {
+                const int row = row0 + r;
+                if (lane == r && row < N) {
+                    const float gte = acc[r], up = acc[r + 1];
+                    a.out[row / 2] = (gte / (1.0f + expf(-gte))) * up;
+                }
+            }
+        }
+    } else {
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            const int row = row0 + r;
+            if (lane == r && row < N) {
+                float v = acc[r];
+                if (epi == GEMV_EPI_RESIDUAL) v = a.epilogue_residual[row] + v;
+                a.out[row] = v;
+            }
+        }
+    }
+}
+
+template <int R, int NC>
+int launch_oneshot(hm_ctx *ctx, const GemvArgs &a, int epi) {
+    const int groups = (a.N + R - 1) / R;
+    const int grid = (groups + GEMV_WAVES - 1) / GEMV_WAVES;
+    hipLaunchKernelGGL((gemv_bf16_nk_oneshot_kernel<R, NC>), dim3(grid), dim3(GEMV_THREADS),
+                       (size_t)a.K * 4, ctx->stream, a, epi);
+    HM_LAUNCH_CHECK(ctx);
+    return HM_OK;
+}
+
+// Pick rows-per-wavefront so that the launch is about one workgroup per CU (each wavefront
+// then has its whole slice in flight at once), within 16 outstanding 16-byte loads per lane.
+// Returns false when the shape does not fit the one-shot kernel.
+bool try_oneshot(hm_ctx *ctx, const GemvArgs &a, int epi, int *rc) {
+    const int nc_exact = (a.K + 511) / 512;
+    if (nc_exact > 8 || epi == GEMV_EPI_ARGMAX) return false;
+    static const int max_loads = [] {  // outstanding 16-byte loads per lane; HOMURA_GEMV_LOADS overrides
+        const char *e = getenv("HOMURA_GEMV_LOADS");
+        const int v = e ? atoi(e) : 4;
+        return v < 2 ? 2 : (v > 16 ? 16 : v);
+    }();
+    const int nc = (nc_exact + 1) / 2 * 2;  // instantiated for 2, 4, 6, 8 chunks
+    const int cand[5] = {8, 6, 4, 2, 1};
+    int r_pick = 0;
+    for (int i = 0; i < 5; i++) {
+        const int r = cand[i];
+        if (r * nc > max_loads && r > (epi == GEMV_EPI_SILU_MUL_PAIRS ? 2 : 1)) continue;
+        if (epi == GEMV_EPI_SILU_MUL_PAIRS && (r % 2)) continue;
+        const int wgs = ((a.N + r - 1) / r + GEMV_WAVES - 1) / GEMV_WAVES;
+        if (wgs >= ctx->num_cus) {
+            r_pick = r;
+            break;
+        }
+        if (!r_pick || r < r_pick) r_pick = r;  // too few rows for a full chip: smallest R
+    }
+    if (!r_pick) return false;
+    // a matrix this large is better served by the persistent kernel (more waves per CU)
+    const int wgs = ((a.N + r_pick - 1) / r_pick + GEMV_WAVES - 1) / GEMV_WAVES;
+    if (wgs > 4 * ctx->num_cus) return false;
+#define HM_ONESHOT(RR, CC) \
+    if (r_pick == RR && nc == CC) { *rc = launch_oneshot<RR, CC>(ctx, a, epi); return true; }
+    HM_ONESHOT(1, 2) HM_ONESHOT(1, 4) HM_ONESHOT(1, 6) HM_ONESHOT(1, 8)
+    HM_ONESHOT(2, 2) HM_ONESHOT(2, 4) HM_ONESHOT(2, 6) HM_ONESHOT(2, 8)
+    HM_ONESHOT(4, 2) HM_ONESHOT(4, 4) HM_ONESHOT(6, 2) HM_ONESHOT(8, 2)
+#undef HM_ONESHOT
+    return false;
+}
+
 template <int R, int MT>
 int launch_nk(hm_ctx *ctx, const GemvArgs &a, int epi, int grid, size_t lds) {
     dim3 g(grid), b(GEMV_THREADS);
@@ -253,9 +452,11 @@ int gemv_bf16_nk_launch(hm_ctx *ctx, GemvArgs a, int M, int epi) {
             rc = launch_nk<2, 4>(ctx, b, epi, grid, (size_t)4 * a.K * 4);
             m0 += 4;
         } else {
-            int grid = gemv_bf16_nk_grid(ctx, a.N, 4);
-            if (epi == GEMV_EPI_ARGMAX && grid > a.argmax_cap) grid = a.argmax_cap;
-            rc = launch_nk<4, 1>(ctx, b, epi, grid, (size_t)a.K * 4);
+            if (!try_oneshot(ctx, b, epi, &rc)) {
+                int grid = gemv_bf16_nk_grid(ctx, a.N, 4);
+                if (epi == GEMV_EPI_ARGMAX && grid > a.argmax_cap) grid = a.argmax_cap;
+                rc = launch_nk<4, 1>(ctx, b, epi, grid, (size_t)a.K * 4);
+            }
             m0 += 1;
         }
         if (rc != HM_OK) return rc;

@@ -2,6 +2,7 @@
 #include "hf.h"
 
 #include <cmath>
+#include <cstdlib>
 
 #include "../attention.h"
 #include "../gemv_bf16.h"
@@ -314,15 +315,10 @@ int HfModel::emit_transformer_plan() {
         return hm_set_error(ctx_, HM_ERR_STATE, "plan expects %zu weights, model lists %zu",
                             weight_slots.size(), infos_.size());
 
-    // attention split: ~2 workgroups per CU when the cache is full, at least 32 rows each
-    int att_chunk;
-    {
-        const int pairs = (int)kvh;
-        const int want = (2 * ctx_->num_cus + pairs - 1) / pairs;
-        att_chunk = (max_seq_len_ + want - 1) / want;
-        att_chunk = std::max(32, (att_chunk + 31) / 32 * 32);
-        att_chunk = std::min(att_chunk, 1024);
-    }
+    // attention split: rows per workgroup (kept in registers); HOMURA_ATT_CHUNK overrides
+    int att_chunk = 64;
+    if (const char *e = std::getenv("HOMURA_ATT_CHUNK")) att_chunk = std::atoi(e);
+    att_chunk = std::min(128, std::max(32, att_chunk / 32 * 32));
 
     std::shared_ptr<PlanScratch> scr = scratch_;
     std::vector<CompiledKernel> kernels;
@@ -353,7 +349,9 @@ int HfModel::emit_transformer_plan() {
         {
             CompiledKernel k;
             k.ops_label = qkn ? "QKV+QKNorm+RoPE" : "QKV+RoPE";
-            const int layer = i;
+            // The QK-norm, RoPE and cache append of this reference kernel run in the prologue of
+            // the attention kernel that follows (same arithmetic, one launch fewer); the q|k|v
+            // slots therefore hold the raw projections.
             DeviceLaunch g1;
             g1.name = "gemv_bf16[qkv]";
             g1.bytes_fixed = gemv_bytes(hidden, qd + 2 * kvd, qd + 2 * kvd) + hidden * 4.0;
@@ -370,34 +368,6 @@ int HfModel::emit_transformer_plan() {
                 return gemv_bf16_nk_launch(sc.ctx, g, 1, GEMV_EPI_NONE);
             };
             k.launches.push_back(std::move(g1));
-            DeviceLaunch g2;
-            g2.name = qkn ? "qknorm_rope_append" : "rope_append";
-            g2.bytes_fixed = (qd + 2 * kvd) * 4.0 * 2 + 2 * kvd * 2.0 + 2 * hd * 4.0;
-            g2.fn = [=](const StepContext &sc) -> int {
-                const auto &in = sc.step.input_slots;
-                KvCache *cache = sc.plan->kv_cache();
-                QkRopeArgs r;
-                r.q = sc.pool[sc.step.output_slots[0]]->as<float>();
-                r.k = sc.pool[sc.step.output_slots[1]]->as<float>();
-                r.v = sc.pool[sc.step.output_slots[2]]->as<float>();
-                if (qkn) {
-                    r.qw = sc.pool[in[7]]->as<float>();
-                    r.kw = sc.pool[in[8]]->as<float>();
-                }
-                r.cos = sc.pool[in[5]]->as<float>();
-                r.sin = sc.pool[in[6]]->as<float>();
-                r.S = 1;
-                r.H = (int)H;
-                r.kvh = (int)kvh;
-                r.hd = (int)hd;
-                r.eps = eps;
-                r.kcache = cache->key_ptr(layer);
-                r.vcache = cache->value_ptr(layer);
-                r.max_len = cache->max_len();
-                r.state = sc.plan->state();
-                return qknorm_rope_launch(sc.ctx, r);
-            };
-            k.launches.push_back(std::move(g2));
             kernels.push_back(std::move(k));
             std::vector<size_t> in{s.hidden_in, s.input_ln, s.q_w, s.k_w, s.v_w, cos_s, sin_s};
             if (qkn) {
@@ -419,13 +389,22 @@ int HfModel::emit_transformer_plan() {
             CompiledKernel k;
             k.ops_label = "Attn";
             DeviceLaunch a1;
-            a1.name = "gqa_decode_attn";
-            a1.bytes_fixed = qd * 4.0 * 2;
+            a1.name = qkn ? "qknorm_rope_append+gqa_attn" : "rope_append+gqa_attn";
+            a1.bytes_fixed = (qd + 2 * kvd) * 4.0 + qd * 4.0 + 2 * kvd * 2.0;
             a1.bytes_per_kv_row = 2.0 * kvh * hd * 2;
+            a1.hip_launches = 2;  // split attention + fold
+            const size_t q_norm_slot = s.q_norm, k_norm_slot = s.k_norm;
             a1.fn = [=](const StepContext &sc) -> int {
                 const auto &in = sc.step.input_slots;
                 AttnArgs a;
-                a.q = sc.pool[in[0]]->as<float>();
+                a.qkv_raw = sc.pool[in[0]]->as<float>();  // q|k|v raw rows are adjacent
+                if (qkn) {
+                    a.qw = sc.pool[q_norm_slot]->as<float>();
+                    a.kw = sc.pool[k_norm_slot]->as<float>();
+                }
+                a.cos_tab = sc.pool[cos_s]->as<float>();
+                a.sin_tab = sc.pool[sin_s]->as<float>();
+                a.eps = eps;
                 a.kcache = sc.pool[in[1]]->as<uint16_t>();
                 a.vcache = sc.pool[in[2]]->as<uint16_t>();
                 a.out = scr->attn_flat.as<float>();

@@ -153,6 +153,7 @@ struct DeviceLaunch {
     double bytes_fixed = 0;           // algorithmic bytes per launch (weights + activations)
     double bytes_per_kv_row = 0;      // plus this much per cached row (attention)
     bool moves_cursor = false;        // advances the DecodeState (must run exactly once per step)
+    int hip_launches = 1;             // HIP kernels this entry enqueues
     std::function<int(const StepContext &)> fn;
 };
 struct CompiledKernel {

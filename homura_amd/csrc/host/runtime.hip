@@ -329,7 +329,8 @@ int ExecutionPlan::bind(const std::vector<Buffer *> &inputs, std::vector<Buffer>
 int ExecutionPlan::launches_per_step() const {
     int n = 0;
     for (const auto &st : steps_)
-        if (st.native_op.kind == NativeOpKind::None) n += (int)kernels_[st.kernel_idx].launches.size();
+        if (st.native_op.kind == NativeOpKind::None)
+            for (const auto &l : kernels_[st.kernel_idx].launches) n += l.hip_launches;
     return n;
 }
 
