@@ -12,7 +12,8 @@ enum GemvEpilogue {
 
 struct GemvArgs {
     const float *x = nullptr;                  // [M][K]
-    const uint16_t *w = nullptr;               // [N][K] bf16
+    const void *w = nullptr;                   // [N][K] bf16 (or f32 when w_f32)
+    bool w_f32 = false;
     float *out = nullptr;                      // [M][N] (or [M][N/2] for the paired epilogue)
     int K = 0, N = 0;
     // prologue: r = x + prologue_residual (optional), then RMSNorm with norm_w (optional)
@@ -35,3 +36,4 @@ int gemv_bf16_nk_launch(hm_ctx *ctx, GemvArgs a, int M, int epi);
 // n * row_mult + row_off.
 int pack_bf16_kn_to_nk_strided(hm_ctx *ctx, const uint16_t *d_w_kn, uint16_t *d_dst, int K, int N,
                                int row_mult, int row_off);
+int pack_f32_kn_to_nk(hm_ctx *ctx, const float *d_w_kn, float *d_dst, int K, int N);

@@ -113,9 +113,21 @@ __device__ __forceinline__ float dot8(const u32x4 w, const float *xv, float acc)
     return acc;
 }
 
-// R rows per wavefront per step, MT activation rows.
-template <int R, int MT, int EPI>
+__device__ __forceinline__ float dot4_f32(const u32x4 w, const float *xv, float acc) {
+    acc = fmaf(__uint_as_float(w.x), xv[0], acc);
+    acc = fmaf(__uint_as_float(w.y), xv[1], acc);
+    acc = fmaf(__uint_as_float(w.z), xv[2], acc);
+    acc = fmaf(__uint_as_float(w.w), xv[3], acc);
+    return acc;
+}
+
+// R rows per wavefront per step, MT activation rows. WF32: weights are f32 (4 per 16-byte
+// load) instead of bf16 (8 per load); same contraction (reference make_mixed_matmul_region with
+// an f32 right-hand side, src/graph_builder/emit_linalg.rs:2224-2307).
+template <int R, int MT, int EPI, bool WF32>
 __global__ __launch_bounds__(GEMV_THREADS) void gemv_bf16_nk_kernel(GemvArgs a) {
+    constexpr int EPL = WF32 ? 4 : 8;  // elements per lane per load
+    constexpr int ESZ = WF32 ? 4 : 2;
     extern __shared__ float xs[];  // [MT][K]
     const int K = a.K, N = a.N;
     stage_activations<MT>(xs, a.x, a.prologue_residual, a.norm_w, a.eps, K, a.resid_out,
@@ -124,7 +136,7 @@ __global__ __launch_bounds__(GEMV_THREADS) void gemv_bf16_nk_kernel(GemvArgs a) 
     const int lane = threadIdx.x & (WAVE - 1);
     const int wave = threadIdx.x / WAVE;
     const int groups = (N + R - 1) / R;
-    const int nchunks = (K + 511) / 512;
+    const int nchunks = (K + WAVE * EPL - 1) / (WAVE * EPL);
     const int gstride = gridDim.x * GEMV_WAVES;
 
     float best_v = -INFINITY;
@@ -138,29 +150,32 @@ __global__ __launch_bounds__(GEMV_THREADS) void gemv_bf16_nk_kernel(GemvArgs a) 
 #pragma unroll
             for (int m = 0; m < MT; m++) acc[r][m] = 0.f;
 
-        const uint16_t *wrow[R];
+        const char *wrow[R];
 #pragma unroll
         for (int r = 0; r < R; r++) {
             int row = row0 + r < N ? row0 + r : N - 1;  // clamp: tail rows re-read a valid row
-            wrow[r] = a.w + (size_t)row * K;
+            wrow[r] = reinterpret_cast<const char *>(a.w) + (size_t)row * K * ESZ;
         }
 
 #pragma unroll 2
         for (int c = 0; c < nchunks; c++) {
-            const int k = (c * WAVE + lane) * 8;
+            const int k = (c * WAVE + lane) * EPL;
             if (k < K) {
                 u32x4 wv[R];
 #pragma unroll
-                for (int r = 0; r < R; r++) wv[r] = ld128_stream(wrow[r] + k);
+                for (int r = 0; r < R; r++) wv[r] = ld128_stream(wrow[r] + (size_t)k * ESZ);
 #pragma unroll
                 for (int m = 0; m < MT; m++) {
                     float xv[8];
                     const f32x4 x0 = *reinterpret_cast<const f32x4 *>(xs + m * K + k);
-                    const f32x4 x1 = *reinterpret_cast<const f32x4 *>(xs + m * K + k + 4);
                     xv[0] = x0.x; xv[1] = x0.y; xv[2] = x0.z; xv[3] = x0.w;
-                    xv[4] = x1.x; xv[5] = x1.y; xv[6] = x1.z; xv[7] = x1.w;
+                    if (!WF32) {
+                        const f32x4 x1 = *reinterpret_cast<const f32x4 *>(xs + m * K + k + 4);
+                        xv[4] = x1.x; xv[5] = x1.y; xv[6] = x1.z; xv[7] = x1.w;
+                    }
 #pragma unroll
-                    for (int r = 0; r < R; r++) acc[r][m] = dot8(wv[r], xv, acc[r][m]);
+                    for (int r = 0; r < R; r++)
+                        acc[r][m] = WF32 ? dot4_f32(wv[r], xv, acc[r][m]) : dot8(wv[r], xv, acc[r][m]);
                 }
             }
         }
@@ -275,7 +290,8 @@ __global__ __launch_bounds__(GEMV_THREADS) void gemv_bf16_nk_oneshot_kernel(Gemv
 #pragma unroll
         for (int r = 0; r < R; r++) {
             const int row = row0 + r < N ? row0 + r : N - 1;  // clamp: stays inside the matrix
-            wv[c][r] = k < K ? ld128_stream(a.w + (size_t)row * K + k) : u32x4{0u, 0u, 0u, 0u};
+            wv[c][r] = k < K ? ld128_stream(static_cast<const uint16_t *>(a.w) + (size_t)row * K + k)
+                             : u32x4{0u, 0u, 0u, 0u};
         }
     }
 
@@ -365,7 +381,7 @@ int launch_oneshot(hm_ctx *ctx, const GemvArgs &a, int epi) {
 // Returns false when the shape does not fit the one-shot kernel.
 bool try_oneshot(hm_ctx *ctx, const GemvArgs &a, int epi, int *rc) {
     const int nc_exact = (a.K + 511) / 512;
-    if (nc_exact > 8 || epi == GEMV_EPI_ARGMAX) return false;
+    if (nc_exact > 8 || epi == GEMV_EPI_ARGMAX || a.w_f32) return false;
     static const int max_loads = [] {  // outstanding 16-byte loads per lane; HOMURA_GEMV_LOADS overrides
         const char *e = getenv("HOMURA_GEMV_LOADS");
         const int v = e ? atoi(e) : 4;
@@ -398,27 +414,33 @@ bool try_oneshot(hm_ctx *ctx, const GemvArgs &a, int epi, int *rc) {
     return false;
 }
 
-template <int R, int MT>
-int launch_nk(hm_ctx *ctx, const GemvArgs &a, int epi, int grid, size_t lds) {
+template <int R, int MT, bool WF32>
+int launch_nk_t(hm_ctx *ctx, const GemvArgs &a, int epi, int grid, size_t lds) {
     dim3 g(grid), b(GEMV_THREADS);
     switch (epi) {
     case GEMV_EPI_NONE:
-        hipLaunchKernelGGL((gemv_bf16_nk_kernel<R, MT, GEMV_EPI_NONE>), g, b, lds, ctx->stream, a);
+        hipLaunchKernelGGL((gemv_bf16_nk_kernel<R, MT, GEMV_EPI_NONE, WF32>), g, b, lds, ctx->stream, a);
         break;
     case GEMV_EPI_RESIDUAL:
-        hipLaunchKernelGGL((gemv_bf16_nk_kernel<R, MT, GEMV_EPI_RESIDUAL>), g, b, lds, ctx->stream, a);
+        hipLaunchKernelGGL((gemv_bf16_nk_kernel<R, MT, GEMV_EPI_RESIDUAL, WF32>), g, b, lds, ctx->stream, a);
         break;
     case GEMV_EPI_SILU_MUL_PAIRS:
-        hipLaunchKernelGGL((gemv_bf16_nk_kernel<R, MT, GEMV_EPI_SILU_MUL_PAIRS>), g, b, lds, ctx->stream, a);
+        hipLaunchKernelGGL((gemv_bf16_nk_kernel<R, MT, GEMV_EPI_SILU_MUL_PAIRS, WF32>), g, b, lds, ctx->stream, a);
         break;
     case GEMV_EPI_ARGMAX:
-        hipLaunchKernelGGL((gemv_bf16_nk_kernel<R, MT, GEMV_EPI_ARGMAX>), g, b, lds, ctx->stream, a);
+        hipLaunchKernelGGL((gemv_bf16_nk_kernel<R, MT, GEMV_EPI_ARGMAX, WF32>), g, b, lds, ctx->stream, a);
         break;
     default:
         return hm_set_error(ctx, HM_ERR_INVALID, "gemv: unknown epilogue %d", epi);
     }
     HM_LAUNCH_CHECK(ctx);
     return HM_OK;
+}
+
+template <int R, int MT>
+int launch_nk(hm_ctx *ctx, const GemvArgs &a, int epi, int grid, size_t lds) {
+    return a.w_f32 ? launch_nk_t<R, MT, true>(ctx, a, epi, grid, lds)
+                   : launch_nk_t<R, MT, false>(ctx, a, epi, grid, lds);
 }
 
 }  // namespace
@@ -432,6 +454,7 @@ int gemv_bf16_nk_grid(const hm_ctx *ctx, int N, int R) {
 
 int gemv_bf16_nk_launch(hm_ctx *ctx, GemvArgs a, int M, int epi) {
     HM_REQUIRE(ctx, a.K > 0 && a.N > 0 && a.K % 8 == 0, "gemv_bf16_nk: K=%d must be a positive multiple of 8", a.K);
+    HM_REQUIRE(ctx, a.x && a.w && a.out, "gemv_bf16_nk: NULL pointer");
     HM_REQUIRE(ctx, M >= 1 && M <= 8, "gemv_bf16_nk: M=%d outside 1..8", M);
     HM_REQUIRE(ctx, (size_t)a.K * 4 <= 64 * 1024, "gemv_bf16_nk: K=%d too large for the LDS stage", a.K);
     HM_REQUIRE(ctx, ((uintptr_t)a.w % 16) == 0 && ((uintptr_t)a.x % 16) == 0, "gemv_bf16_nk: pointers must be 16-byte aligned");
@@ -548,7 +571,32 @@ __global__ __launch_bounds__(256) void pack_kn_to_nk_kernel(const uint16_t *__re
     }
 }
 
+// f32 [K][N] -> [N][K] (LM head of the quantised plan)
+__global__ __launch_bounds__(256) void pack_f32_kn_to_nk_kernel(const float *__restrict__ src,
+                                                                float *__restrict__ dst, int K, int N) {
+    __shared__ float tile[64][65];
+    const int n0 = blockIdx.x * 64, k0 = blockIdx.y * 64;
+    const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+    for (int i = ty; i < 64; i += 4) {
+        int k = k0 + i, n = n0 + tx;
+        tile[i][tx] = (k < K && n < N) ? src[(size_t)k * N + n] : 0.f;
+    }
+    __syncthreads();
+    for (int i = ty; i < 64; i += 4) {
+        int n = n0 + i, k = k0 + tx;
+        if (n < N && k < K) dst[(size_t)n * K + k] = tile[tx][i];
+    }
+}
+
 }  // namespace
+
+int pack_f32_kn_to_nk(hm_ctx *ctx, const float *d_w_kn, float *d_dst, int K, int N) {
+    HM_REQUIRE(ctx, d_w_kn && d_dst && K > 0 && N > 0, "pack_f32_kn_to_nk: bad arguments");
+    dim3 grid((N + 63) / 64, (K + 63) / 64);
+    hipLaunchKernelGGL(pack_f32_kn_to_nk_kernel, grid, dim3(256), 0, ctx->stream, d_w_kn, d_dst, K, N);
+    HM_LAUNCH_CHECK(ctx);
+    return HM_OK;
+}
 
 int pack_bf16_kn_to_nk_strided(hm_ctx *ctx, const uint16_t *d_w_kn, uint16_t *d_dst, int K, int N,
                                int row_mult, int row_off) {

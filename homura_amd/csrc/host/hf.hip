@@ -117,8 +117,70 @@ int HfModel::set_weight(int slot, const void *h_data, size_t bytes) {
     if (finalized_) return hm_set_error(ctx_, HM_ERR_STATE, "model already finalized");
     if (!h_data) return hm_set_error(ctx_, HM_ERR_INVALID, "weight %s: NULL data", info.name.c_str());
 
+    const std::string &nm = info.name;
+    auto ends_with = [&](const char *suffix) {
+        const std::string s(suffix);
+        return nm.size() >= s.size() && nm.compare(nm.size() - s.size(), s.size(), s) == 0;
+    };
+    const int hidden = cfg_.hidden_size, inter = cfg_.intermediate_size;
+    const int qd = cfg_.q_dim(), kvd = cfg_.kv_dim();
+
+    if (dtype_is_quantized(info.dtype)) {
+        // Raw GGUF blocks [N][K/32], kept byte for byte. q|k|v and gate|up of a layer are stored
+        // back to back (rows are contiguous, so the three/two matrices form one taller matrix
+        // and one kernel launch serves them).
+        const size_t p0 = std::string("model.layers.").size();
+        const int layer = std::atoi(nm.c_str() + p0);
+        LayerPacked &lp = packed_[layer];
+        const size_t bb = dtype_block_bytes(info.dtype);
+        const size_t row_h = (size_t)(hidden / 32) * bb;  // bytes of a row with K = hidden
+        Buffer *home = nullptr;
+        size_t home_bytes = 0, offset = 0;
+        if (ends_with("q_proj.weight") || ends_with("k_proj.weight") || ends_with("v_proj.weight")) {
+            home = &lp.qkv;
+            home_bytes = (size_t)(qd + 2 * kvd) * row_h;
+            offset = ends_with("q_proj.weight") ? 0 : ends_with("k_proj.weight") ? (size_t)qd * row_h
+                                                                                  : (size_t)(qd + kvd) * row_h;
+        } else if (ends_with("gate_proj.weight") || ends_with("up_proj.weight")) {
+            home = &lp.gate_up;
+            home_bytes = (size_t)2 * inter * row_h;
+            offset = ends_with("up_proj.weight") ? (size_t)inter * row_h : 0;
+        } else if (ends_with("o_proj.weight")) {
+            home = &lp.o;
+            home_bytes = bytes;
+        } else if (ends_with("down_proj.weight")) {
+            home = &lp.down;
+            home_bytes = bytes;
+        } else {
+            return hm_set_error(ctx_, HM_ERR_INVALID, "unexpected quantised weight %s", nm.c_str());
+        }
+        if (!*home) *home = Buffer::alloc_bytes(ctx_, home_bytes, {(int64_t)home_bytes}, info.dtype);
+        if (!*home) return HM_ERR_OOM;
+        int rc = hm_upload(ctx_, (char *)home->ptr() + offset, h_data, bytes);
+        if (rc != HM_OK) return rc;
+        weight_bufs_[slot] = Buffer::view((char *)home->ptr() + offset, bytes, {(int64_t)bytes}, {1}, info.dtype);
+        weight_set_[slot] = true;
+        return HM_OK;
+    }
+
+    if (info.dtype == DType::F32 && nm == "lm_head.weight") {
+        // f32 LM head of the quantised plan: [hidden][vocab] -> [vocab][hidden] stream layout
+        Buffer staging = Buffer::alloc_bytes(ctx_, bytes, {info.dim0, info.dim1}, DType::F32);
+        lm_head_packed_ = Buffer::alloc(ctx_, {info.dim1, info.dim0}, DType::F32);
+        if (!staging || !lm_head_packed_) return HM_ERR_OOM;
+        int rc = hm_upload(ctx_, staging.ptr(), h_data, bytes);
+        if (rc == HM_OK) rc = pack_f32_kn_to_nk(ctx_, staging.as<float>(), lm_head_packed_.as<float>(),
+                                                (int)info.dim0, (int)info.dim1);
+        if (rc == HM_OK) rc = hm_sync(ctx_);
+        if (rc != HM_OK) return rc;
+        weight_bufs_[slot] = Buffer::view(lm_head_packed_.ptr(), bytes, {info.dim1, info.dim0},
+                                          {info.dim0, 1}, DType::F32);
+        weight_set_[slot] = true;
+        return HM_OK;
+    }
+
     if (info.dtype != DType::BF16) {
-        // f32 vectors / tables and raw quantised blocks are stored as they come
+        // f32 vectors and the embedding table are stored as they come
         Buffer b = Buffer::alloc_bytes(ctx_, bytes, {info.dim0, info.dim1}, info.dtype);
         if (!b) return HM_ERR_OOM;
         int rc = hm_upload(ctx_, b.ptr(), h_data, bytes);
@@ -130,8 +192,6 @@ int HfModel::set_weight(int slot, const void *h_data, size_t bytes) {
 
     // bf16 projection [K][N]: stage, then transpose into its place in the packed stream buffers
     const int K = (int)info.dim0, N = (int)info.dim1;
-    const int hidden = cfg_.hidden_size, inter = cfg_.intermediate_size;
-    const int qd = cfg_.q_dim(), kvd = cfg_.kv_dim();
     Buffer staging = Buffer::alloc_bytes(ctx_, bytes, {K, N}, DType::BF16);
     if (!staging) return HM_ERR_OOM;
     int rc = hm_upload(ctx_, staging.ptr(), h_data, bytes);
@@ -142,11 +202,6 @@ int HfModel::set_weight(int slot, const void *h_data, size_t bytes) {
     auto ensure = [&](Buffer &b, int64_t rows, int64_t cols) -> bool {
         if (!b) b = Buffer::alloc(ctx_, {rows, cols}, DType::BF16);
         return (bool)b;
-    };
-    const std::string &nm = info.name;
-    auto ends_with = [&](const char *suffix) {
-        const std::string s(suffix);
-        return nm.size() >= s.size() && nm.compare(nm.size() - s.size(), s.size(), s) == 0;
     };
     if (nm == "lm_head.weight") {
         if (!ensure(lm_head_packed_, cfg_.vocab_size, hidden)) return HM_ERR_OOM;
@@ -536,8 +591,332 @@ int HfModel::emit_transformer_plan() {
     return HM_OK;
 }
 
+// ── quantised plan ───────────────────────────────────────────────────────────
+// Step list of emit_transformer_plan_quant (reference src/hf/emitter_quant.rs:1211-1440), one
+// KernelStep per reference step: RMSNorm, QuantMM Q/K/V, PostQKV, KV concat x2, AttnBody,
+// QuantMM O, Residual+Norm, QuantMM Gate/Up, SiLU*Up, QuantMM Down, ResAdd; f32 LM head.
+// Fusions that keep the arithmetic: the Q step's launch covers K and V too (their blocks are
+// stored back to back), Gate's covers Up, and PostQKV runs in AttnBody's prologue. The
+// reference's f64 accumulations (sum of squares, sum of exps) are f32 tree sums here.
 int HfModel::emit_transformer_plan_quant() {
-    return hm_set_error(ctx_, HM_ERR_INVALID, "quantised transformer plan is not built yet");
+    const TransformerConfig c = cfg_;
+    const int64_t hidden = c.hidden_size, inter = c.intermediate_size, vocab = c.vocab_size;
+    const int64_t H = c.num_attention_heads, kvh = c.kv_heads(), hd = c.head_dim();
+    const int64_t qd = c.q_dim(), kvd = c.kv_dim();
+    const int L = c.num_hidden_layers;
+    const float eps = (float)c.rms_norm_eps;
+    const bool qkn = has_qk_norm_;
+    const DType wdt = weight_dtype_;
+    const int64_t D = DIM_DYNAMIC;
+    const double bpw = (double)dtype_block_bytes(wdt) / 32.0;  // bytes per weight
+
+    std::vector<SlotDesc> descs;
+    auto alloc = [&](std::vector<int64_t> shape, DType dt, const std::string &name) -> size_t {
+        descs.push_back(SlotDesc{std::move(shape), dt, name});
+        return descs.size() - 1;
+    };
+    std::vector<size_t> input_slots, weight_slots, past_kv, present_kv;
+    const size_t input_ids = alloc({1, D}, DType::I64, "input_ids");
+    const size_t mask = alloc({1, 1, D, D}, DType::F32, "mask");
+    const size_t cos_s = alloc({D, hd}, DType::F32, "cos");
+    const size_t sin_s = alloc({D, hd}, DType::F32, "sin");
+    input_slots = {input_ids, mask, cos_s, sin_s};
+    const size_t embed_w = alloc({vocab, hidden}, DType::F32, "embed_tokens");
+    weight_slots.push_back(embed_w);
+    const size_t embed_out = alloc({1, D, hidden}, DType::F32, "embed_out");
+
+    struct LS {
+        size_t hidden_in, input_ln, q_w, k_w, v_w, q_norm, k_norm, o_w, post_ln, gate_w, up_w, down_w;
+        size_t past_k, past_v, present_k, present_v;
+        size_t normed, q_out, k_out, v_out, q, k_bhsd, v_bhsd, attn_body, attn_out, residual, post_normed,
+            gate_out, up_out, silu, down_out, hidden_out;
+    };
+    std::vector<LS> ls(L);
+    auto qbytes = [&](int64_t K, int64_t N) { return (int64_t)dtype_bytes_for_elements(wdt, (size_t)(K * N), nullptr); };
+    for (int i = 0; i < L; i++) {
+        LS &s = ls[i];
+        const std::string p = "l" + std::to_string(i) + ".";
+        s.hidden_in = i == 0 ? embed_out : ls[i - 1].hidden_out;
+        auto w = [&](std::vector<int64_t> shape, DType dt, const std::string &n) {
+            size_t slot = alloc(std::move(shape), dt, p + n);
+            weight_slots.push_back(slot);
+            return slot;
+        };
+        // quantised weights are flat byte buffers (reference src/hf/emitter_quant.rs:213-222)
+        s.input_ln = w({hidden}, DType::F32, "input_ln");
+        s.q_w = w({qbytes(hidden, qd)}, wdt, "q_w");
+        s.k_w = w({qbytes(hidden, kvd)}, wdt, "k_w");
+        s.v_w = w({qbytes(hidden, kvd)}, wdt, "v_w");
+        s.q_norm = s.k_norm = (size_t)-1;
+        if (qkn) {
+            s.q_norm = w({hd}, DType::F32, "q_norm");
+            s.k_norm = w({hd}, DType::F32, "k_norm");
+        }
+        s.o_w = w({qbytes(qd, hidden)}, wdt, "o_w");
+        s.post_ln = w({hidden}, DType::F32, "post_ln");
+        s.gate_w = w({qbytes(hidden, inter)}, wdt, "gate_w");
+        s.up_w = w({qbytes(hidden, inter)}, wdt, "up_w");
+        s.down_w = w({qbytes(inter, hidden)}, wdt, "down_w");
+        s.past_k = alloc({1, kvh, D, hd}, DType::BF16, p + "past_k");
+        s.past_v = alloc({1, kvh, D, hd}, DType::BF16, p + "past_v");
+        past_kv.push_back(s.past_k);
+        past_kv.push_back(s.past_v);
+        input_slots.push_back(s.past_k);
+        input_slots.push_back(s.past_v);
+        s.present_k = alloc({1, kvh, D, hd}, DType::BF16, p + "present_k");
+        s.present_v = alloc({1, kvh, D, hd}, DType::BF16, p + "present_v");
+        present_kv.push_back(s.present_k);
+        present_kv.push_back(s.present_v);
+        s.normed = alloc({1, D, hidden}, DType::F32, p + "normed");
+        s.q_out = alloc({1, D, qd}, DType::F32, p + "q_proj_out");
+        s.k_out = alloc({1, D, kvd}, DType::F32, p + "k_proj_out");
+        s.v_out = alloc({1, D, kvd}, DType::F32, p + "v_proj_out");
+        s.q = alloc({1, D, H, hd}, DType::F32, p + "q");
+        s.k_bhsd = alloc({1, kvh, D, hd}, DType::F32, p + "k_bhsd");
+        s.v_bhsd = alloc({1, kvh, D, hd}, DType::F32, p + "v_bhsd");
+        s.attn_body = alloc({1, D, qd}, DType::F32, p + "attn_body_out");
+        s.attn_out = alloc({1, D, hidden}, DType::F32, p + "attn_out");
+        s.residual = alloc({1, D, hidden}, DType::F32, p + "residual");
+        s.post_normed = alloc({1, D, hidden}, DType::F32, p + "post_attn_normed");
+        s.gate_out = alloc({1, D, inter}, DType::F32, p + "gate_out");
+        s.up_out = alloc({1, D, inter}, DType::F32, p + "up_out");
+        s.silu = alloc({1, D, inter}, DType::F32, p + "silu_mul_out");
+        s.down_out = alloc({1, D, hidden}, DType::F32, p + "down_out");
+        s.hidden_out = alloc({1, D, hidden}, DType::F32, p + "hidden_out");
+    }
+    const size_t final_norm = alloc({hidden}, DType::F32, "final_norm");
+    weight_slots.push_back(final_norm);
+    const size_t lm_head = alloc({hidden, vocab}, DType::F32, "lm_head");
+    weight_slots.push_back(lm_head);
+    const size_t logits = alloc({1, D, vocab}, DType::F32, "logits");
+    std::vector<size_t> output_slots{logits};
+    output_slots.insert(output_slots.end(), present_kv.begin(), present_kv.end());
+    if (weight_slots.size() != infos_.size())
+        return hm_set_error(ctx_, HM_ERR_STATE, "plan expects %zu weights, model lists %zu",
+                            weight_slots.size(), infos_.size());
+
+    int att_chunk = 64;
+    if (const char *e = std::getenv("HOMURA_ATT_CHUNK")) att_chunk = std::atoi(e);
+    att_chunk = std::min(128, std::max(32, att_chunk / 32 * 32));
+
+    std::shared_ptr<PlanScratch> scr = scratch_;
+    std::vector<CompiledKernel> kernels;
+    std::vector<KernelStep> steps;
+    auto add_step = [&](CompiledKernel k, std::vector<size_t> in, std::vector<size_t> out) {
+        kernels.push_back(std::move(k));
+        steps.push_back(KernelStep::kernel(kernels.size() - 1, std::move(in), std::move(out)));
+    };
+    auto quant_mm = [&](const char *label, int64_t K, int64_t N, bool launches) {
+        // QuantMM step (reference emit_quant_matmul_kernel, src/hf/emitter_quant.rs:675-702):
+        // inputs [activation, weight bytes], output [1, seq, N]
+        CompiledKernel k;
+        k.ops_label = std::string("QuantMM[") + label + "]";
+        if (launches) {
+            DeviceLaunch l;
+            l.name = std::string(wdt == DType::Q8_0 ? "gemv_q8_0[" : "gemv_q4_0[") + label + "]";
+            l.bytes_fixed = (double)K * N * bpw + K * 4.0 + N * 4.0;
+            l.fn = [=](const StepContext &sc) -> int {
+                const float *x = sc.pool[sc.step.input_slots[0]]->as<float>();
+                const uint8_t *w = sc.pool[sc.step.input_slots[1]]->as<uint8_t>();
+                float *out = sc.pool[sc.step.output_slots[0]]->as<float>();
+                return wdt == DType::Q8_0 ? hm_gemv_q8_0(sc.ctx, x, w, out, 1, (int)K, (int)N)
+                                          : hm_gemv_q4_0(sc.ctx, x, w, out, 1, (int)K, (int)N);
+            };
+            k.launches.push_back(std::move(l));
+        }
+        return k;
+    };
+
+    {
+        CompiledKernel k;
+        k.ops_label = "Embed";
+        DeviceLaunch l;
+        l.name = "embed";
+        l.bytes_fixed = hidden * 4.0 * 2;
+        l.fn = [=](const StepContext &sc) -> int {
+            return embed_step_launch(sc.ctx, sc.plan->state(), sc.plan->forced_ids(),
+                                     sc.pool[sc.step.input_slots[1]]->as<float>(),
+                                     sc.pool[sc.step.output_slots[0]]->as<float>(), (int)vocab, (int)hidden);
+        };
+        k.launches.push_back(std::move(l));
+        add_step(std::move(k), {input_ids, embed_w}, {embed_out});
+    }
+    for (int i = 0; i < L; i++) {
+        const LS &s = ls[i];
+        {  // Step 1: pre-QKV RMSNorm (reference :713-791)
+            CompiledKernel k;
+            k.ops_label = "RMSNorm";
+            DeviceLaunch l;
+            l.name = "rmsnorm";
+            l.bytes_fixed = hidden * 4.0 * 3;
+            l.fn = [=](const StepContext &sc) -> int {
+                return rmsnorm_launch(sc.ctx, sc.pool[sc.step.input_slots[0]]->as<float>(), nullptr,
+                                      sc.pool[sc.step.input_slots[1]]->as<float>(),
+                                      sc.pool[sc.step.output_slots[0]]->as<float>(), nullptr, 1, (int)hidden, eps);
+            };
+            k.launches.push_back(std::move(l));
+            add_step(std::move(k), {s.hidden_in, s.input_ln}, {s.normed});
+        }
+        // Steps 2-4: QuantMM Q, K, V — one launch over the stacked q|k|v rows
+        add_step(quant_mm("qkv", hidden, qd + 2 * kvd, true), {s.normed, s.q_w}, {s.q_out});
+        add_step(quant_mm("k", hidden, kvd, false), {s.normed, s.k_w}, {s.k_out});
+        add_step(quant_mm("v", hidden, kvd, false), {s.normed, s.v_w}, {s.v_out});
+        {  // Step 5: PostQKV (reference :802-912) — runs in the attention kernel's prologue
+            CompiledKernel k;
+            k.ops_label = qkn ? "PostQKV+QKNorm+RoPE" : "PostQKV+RoPE";
+            std::vector<size_t> in{s.q_out, s.k_out, s.v_out, cos_s, sin_s};
+            if (qkn) {
+                in.push_back(s.q_norm);
+                in.push_back(s.k_norm);
+            }
+            add_step(std::move(k), in, {s.q, s.k_bhsd, s.v_bhsd});
+        }
+        for (int kv = 0; kv < 2; kv++) {  // Steps 6-7: KV concat
+            KernelStep st;
+            st.input_slots = {kv ? s.past_v : s.past_k, kv ? s.v_bhsd : s.k_bhsd};
+            st.output_slots = {kv ? s.present_v : s.present_k};
+            st.native_op = NativeOp{NativeOpKind::Concat, 2};
+            steps.push_back(st);
+        }
+        {  // Step 8: AttnBody (reference :922-975)
+            CompiledKernel k;
+            k.ops_label = "AttnBody";
+            DeviceLaunch l;
+            l.name = qkn ? "qknorm_rope_append+gqa_attn" : "rope_append+gqa_attn";
+            l.bytes_fixed = (qd + 2 * kvd) * 4.0 + qd * 4.0 + 2 * kvd * 2.0;
+            l.bytes_per_kv_row = 2.0 * kvh * hd * 2;
+            l.hip_launches = 2;
+            const size_t raw_slot = s.q_out, qn = s.q_norm, kn = s.k_norm;
+            l.fn = [=](const StepContext &sc) -> int {
+                const auto &in = sc.step.input_slots;
+                AttnArgs a;
+                a.qkv_raw = sc.pool[raw_slot]->as<float>();
+                if (qkn) {
+                    a.qw = sc.pool[qn]->as<float>();
+                    a.kw = sc.pool[kn]->as<float>();
+                }
+                a.cos_tab = sc.pool[cos_s]->as<float>();
+                a.sin_tab = sc.pool[sin_s]->as<float>();
+                a.eps = eps;
+                a.kcache = sc.pool[in[1]]->as<uint16_t>();
+                a.vcache = sc.pool[in[2]]->as<uint16_t>();
+                a.out = sc.pool[sc.step.output_slots[0]]->as<float>();
+                a.B = 1;
+                a.H = (int)H;
+                a.kvh = (int)kvh;
+                a.hd = (int)hd;
+                a.max_len = sc.plan->kv_cache()->max_len();
+                a.kv_len = 1;
+                a.scale = (float)(1.0 / std::sqrt((double)hd));
+                a.state = sc.plan->state();
+                a.fixed_chunk = att_chunk;
+                return gqa_decode_attn_launch(sc.ctx, a);
+            };
+            k.launches.push_back(std::move(l));
+            add_step(std::move(k), {s.q, s.present_k, s.present_v, mask}, {s.attn_body});
+        }
+        add_step(quant_mm("o", qd, hidden, true), {s.attn_body, s.o_w}, {s.attn_out});  // Step 9
+        {  // Step 10: Residual + RMSNorm (reference :985-1071), two outputs
+            CompiledKernel k;
+            k.ops_label = "Residual+Norm";
+            DeviceLaunch l;
+            l.name = "residual_rmsnorm";
+            l.bytes_fixed = hidden * 4.0 * 5;
+            l.fn = [=](const StepContext &sc) -> int {
+                const auto &in = sc.step.input_slots;
+                return rmsnorm_launch(sc.ctx, sc.pool[in[0]]->as<float>(), sc.pool[in[1]]->as<float>(),
+                                      sc.pool[in[2]]->as<float>(), sc.pool[sc.step.output_slots[1]]->as<float>(),
+                                      sc.pool[sc.step.output_slots[0]]->as<float>(), 1, (int)hidden, eps);
+            };
+            k.launches.push_back(std::move(l));
+            add_step(std::move(k), {s.hidden_in, s.attn_out, s.post_ln}, {s.residual, s.post_normed});
+        }
+        // Steps 11-12: QuantMM Gate, Up — one launch over the stacked gate|up rows
+        add_step(quant_mm("gate_up", hidden, 2 * inter, true), {s.post_normed, s.gate_w}, {s.gate_out});
+        add_step(quant_mm("up", hidden, inter, false), {s.post_normed, s.up_w}, {s.up_out});
+        {  // Step 13: SiLU * Up (reference :1077-1103)
+            CompiledKernel k;
+            k.ops_label = "SiLU*Up";
+            DeviceLaunch l;
+            l.name = "silu_mul";
+            l.bytes_fixed = inter * 4.0 * 3;
+            l.fn = [=](const StepContext &sc) -> int {
+                const auto &in = sc.step.input_slots;
+                return hm_silu_mul(sc.ctx, sc.pool[in[0]]->as<float>(), sc.pool[in[1]]->as<float>(),
+                                   sc.pool[sc.step.output_slots[0]]->as<float>(), (size_t)inter);
+            };
+            k.launches.push_back(std::move(l));
+            add_step(std::move(k), {s.gate_out, s.up_out}, {s.silu});
+        }
+        add_step(quant_mm("down", inter, hidden, true), {s.silu, s.down_w}, {s.down_out});  // Step 14
+        {  // Step 15: ResAdd (reference :1109-1134)
+            CompiledKernel k;
+            k.ops_label = "ResAdd";
+            DeviceLaunch l;
+            l.name = "residual_add";
+            l.bytes_fixed = hidden * 4.0 * 3;
+            l.fn = [=](const StepContext &sc) -> int {
+                const auto &in = sc.step.input_slots;
+                return hm_add(sc.ctx, sc.pool[in[0]]->as<float>(), sc.pool[in[1]]->as<float>(),
+                              sc.pool[sc.step.output_slots[0]]->as<float>(), (size_t)hidden);
+            };
+            k.launches.push_back(std::move(l));
+            add_step(std::move(k), {s.residual, s.down_out}, {s.hidden_out});
+        }
+    }
+    {  // LM head: final RMSNorm + f32 matmul (reference :1399-1440) + device-side greedy pick
+        CompiledKernel k;
+        k.ops_label = "LMHead";
+        DeviceLaunch h1;
+        h1.name = "gemv_f32[lm_head+argmax]";
+        h1.bytes_fixed = (double)hidden * vocab * 4 + hidden * 8.0 + vocab * 4.0;
+        h1.fn = [=](const StepContext &sc) -> int {
+            const auto &in = sc.step.input_slots;
+            GemvArgs g;
+            g.x = sc.pool[in[0]]->as<float>();
+            g.norm_w = sc.pool[in[1]]->as<float>();
+            g.eps = eps;
+            g.w = sc.pool[in[2]]->ptr();
+            g.w_f32 = true;
+            g.out = sc.pool[sc.step.output_slots[0]]->as<float>();
+            g.K = (int)hidden;
+            g.N = (int)vocab;
+            g.argmax_val = scr->cand_val.as<float>();
+            g.argmax_idx = scr->cand_idx.as<int>();
+            g.argmax_cap = scr->cand_cap;
+            return gemv_bf16_nk_launch(sc.ctx, g, 1, GEMV_EPI_ARGMAX);
+        };
+        k.launches.push_back(std::move(h1));
+        DeviceLaunch h2;
+        h2.name = "finish_step";
+        h2.moves_cursor = true;
+        h2.bytes_fixed = 64;
+        h2.fn = [=](const StepContext &sc) -> int {
+            const int ncand = std::min(gemv_bf16_nk_grid(sc.ctx, (int)vocab, 4), scr->cand_cap);
+            return finish_step_launch(sc.ctx, sc.plan->state(), scr->cand_val.as<float>(),
+                                      scr->cand_idx.as<int>(), ncand, sc.plan->out_tokens(),
+                                      sc.plan->out_capacity());
+        };
+        k.launches.push_back(std::move(h2));
+        add_step(std::move(k), {ls[L - 1].hidden_out, final_norm, lm_head}, {logits});
+    }
+
+    const size_t num_slots = descs.size();
+    plan_.reset(new ExecutionPlan(ctx_, std::move(kernels), std::move(steps), num_slots, input_slots,
+                                  weight_slots, output_slots, std::move(descs)));
+    KvPlanInfo info;
+    info.num_layers = L;
+    info.num_heads = (int)kvh;
+    info.head_dim = (int)hd;
+    info.past_kv_input_slots = past_kv;
+    info.present_kv_output_slots = present_kv;
+    plan_->set_kv_info(info);
+    for (int i = 0; i < L; i++) {
+        plan_->alias_slot(ls[i].k_out, ls[i].q_out, (size_t)qd * 4);
+        plan_->alias_slot(ls[i].v_out, ls[i].q_out, (size_t)(qd + kvd) * 4);
+        plan_->alias_slot(ls[i].up_out, ls[i].gate_out, (size_t)inter * 4);
+    }
+    return HM_OK;
 }
 
 // ── running ──────────────────────────────────────────────────────────────────

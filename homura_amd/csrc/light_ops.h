@@ -22,6 +22,9 @@ struct QkRopeArgs {
 };
 
 int qknorm_rope_launch(hm_ctx *ctx, const QkRopeArgs &a);
+// out = rmsnorm(x [+ res]) * w per row; resid_out (optional) receives x + res
+int rmsnorm_launch(hm_ctx *ctx, const float *d_x, const float *d_res, const float *d_w, float *d_out,
+                   float *d_resid_out, int rows, int dim, float eps);
 int embed_launch(hm_ctx *ctx, const int64_t *d_ids64, const int32_t *d_ids32, const float *d_table,
                  float *d_out, int n_ids, int vocab, int hidden);
 int argmax_candidates_launch(hm_ctx *ctx, const float *d_vals, const int *d_idxs, int n,

@@ -6,21 +6,33 @@
 
 namespace {
 
-// one workgroup per row (reference src/graph_builder/emit_linalg.rs:7-26)
+// One workgroup per row: optional residual add (reference Residual+Norm kernel,
+// src/hf/emitter_quant.rs:985-1071), then RMSNorm (src/graph_builder/emit_linalg.rs:7-26).
 __global__ __launch_bounds__(256) void rmsnorm_kernel(const float *__restrict__ x,
+                                                      const float *__restrict__ res,
                                                       const float *__restrict__ w,
-                                                      float *__restrict__ out, int dim, float eps) {
+                                                      float *__restrict__ out,
+                                                      float *__restrict__ resid_out, int dim,
+                                                      float eps) {
     __shared__ float red[4];
-    const float *xr = x + (size_t)blockIdx.x * dim;
-    float *orow = out + (size_t)blockIdx.x * dim;
+    const size_t base = (size_t)blockIdx.x * dim;
     float ss = 0.f;
-    for (int i = threadIdx.x; i < dim; i += 256) ss += xr[i] * xr[i];
+    for (int i = threadIdx.x; i < dim; i += 256) {
+        float v = x[base + i];
+        if (res) v = v + res[base + i];
+        if (resid_out) resid_out[base + i] = v;
+        ss += v * v;
+    }
     ss = wave_sum(ss);
     if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = ss;
     __syncthreads();
     const float tot = (red[0] + red[1]) + (red[2] + red[3]);
     const float inv = 1.0f / sqrtf(tot / (float)dim + eps);
-    for (int i = threadIdx.x; i < dim; i += 256) orow[i] = (xr[i] * inv) * w[i];
+    for (int i = threadIdx.x; i < dim; i += 256) {
+        float v = x[base + i];
+        if (res) v = v + res[base + i];
+        out[base + i] = (v * inv) * w[i];
+    }
 }
 
 // One wavefront per (token, head) row of q or k: optional per-head RMSNorm, then
@@ -300,6 +312,18 @@ int qknorm_rope_launch(hm_ctx *ctx, const QkRopeArgs &a) {
     return HM_OK;
 }
 
+int rmsnorm_launch(hm_ctx *ctx, const float *d_x, const float *d_res, const float *d_w, float *d_out,
+                   float *d_resid_out, int rows, int dim, float eps) {
+    HM_REQUIRE(ctx, d_x && d_w && d_out, "rmsnorm: NULL pointer");
+    HM_REQUIRE(ctx, rows >= 0 && dim > 0, "rmsnorm: bad shape");
+    HM_REQUIRE(ctx, d_out != d_x && d_out != d_res, "rmsnorm: output must not alias an input");
+    if (rows == 0) return HM_OK;
+    hipLaunchKernelGGL(rmsnorm_kernel, dim3(rows), dim3(256), 0, ctx->stream, d_x, d_res, d_w, d_out,
+                       d_resid_out, dim, eps);
+    HM_LAUNCH_CHECK(ctx);
+    return HM_OK;
+}
+
 int embed_launch(hm_ctx *ctx, const int64_t *d_ids64, const int32_t *d_ids32, const float *d_table,
                  float *d_out, int n_ids, int vocab, int hidden) {
     HM_REQUIRE(ctx, (d_ids64 || d_ids32) && d_table && d_out, "embed: NULL pointer");
@@ -324,13 +348,7 @@ extern "C" {
 int hm_rmsnorm(hm_ctx *ctx, const float *d_x, const float *d_w, float *d_out, int rows, int dim,
                float eps) {
     HM_CHECK_CTX(ctx);
-    HM_REQUIRE(ctx, d_x && d_w && d_out, "hm_rmsnorm: NULL pointer");
-    HM_REQUIRE(ctx, rows >= 0 && dim > 0, "hm_rmsnorm: bad shape");
-    if (rows == 0) return HM_OK;
-    hipLaunchKernelGGL(rmsnorm_kernel, dim3(rows), dim3(256), 0, ctx->stream, d_x, d_w, d_out, dim,
-                       eps);
-    HM_LAUNCH_CHECK(ctx);
-    return HM_OK;
+    return rmsnorm_launch(ctx, d_x, nullptr, d_w, d_out, nullptr, rows, dim, eps);
 }
 
 int hm_qknorm_rope(hm_ctx *ctx, float *d_q, float *d_k, const float *d_qw, const float *d_kw,

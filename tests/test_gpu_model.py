@@ -148,3 +148,32 @@ def test_qwen3_0p6b_decode_token_identical(ctx):
     gm.init_kv_cache(kv, fx["prefill_len"])
     assert np.array_equal(gm.generate_greedy(prompt, fx["n_new"]), want), "graph replay differs"
     gm.close()
+
+
+@pytest.mark.parametrize("wdt,name", [(2, "q8_0"), (3, "q4_0")])
+def test_quantised_plan_against_oracle(ctx, wdt, name):
+    """GGUF-quantised projections (reference emit_transformer_plan_quant): raw blocks uploaded as
+    they are, dequantised in registers; f32 LM head. Llama-style config: no QK-norm, untied head."""
+    cfg = synth_model.TINY_LLAMA
+    weights = synth_model.synth_weights(cfg, 31, wdt, has_qk_norm=False)
+    gm = synth_model.build_model(ctx, cfg, weights, 96, wdt, has_qk_norm=False)
+    om = mf.build_oracle_model(cfg, weights, 96, wdt, has_qk_norm=False)
+    kv = synth_model.synth_kv(cfg, 3, 37)
+    gm.init_kv_cache(kv, 37)
+    mf.oracle_init_kv(om, kv)
+    ids = synth.token_ids(4, 6, cfg.vocab_size)
+    got = gm.run_kv(ids)
+    want = np.concatenate([om.run_kv(ids[i:i + 1]) for i in range(6)])
+    for i in range(6):
+        assert mf.rel_err(got[i], want[i]) < 1e-2, f"{name} position {i}"
+    want_t, margins = om.generate_greedy(ids[:2], 24)
+    got_t = gm.generate_greedy(ids[:2], 24)
+    say(f"{name}: min margin {margins.min():.3e}")
+    assert np.array_equal(got_t, want_t)
+    gm.set_graph(True)
+    gm.init_kv_cache(kv, 37)
+    gm.run_kv(ids)
+    assert np.array_equal(gm.generate_greedy(ids[:2], 24), want_t)
+    names = [s[0] for s in gm.weight_slots()]
+    assert names == [n for n, _ in weights]
+    gm.close()
