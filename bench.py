@@ -46,6 +46,8 @@ def main() -> int:
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-tokens", type=int, default=96, help="tokens of the CPU-baseline sample")
     ap.add_argument("--kernel-rounds", type=int, default=20)
+    ap.add_argument("--no-kernel-configs", action="store_true",
+                    help="skip the stand-alone kernel measurements (BASELINE configurations 1, 3, 4, 5)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this build runs on one GPU only (got --gpus {args.gpus}); "
@@ -114,6 +116,10 @@ def main() -> int:
         launches = model.launches_per_step()
         device = ctx.device_name()
         model.close()
+        kernel_configs = None
+        if not args.no_kernel_configs:
+            from homura_amd import kernel_bench
+            kernel_configs = kernel_bench.run_all(ctx)
 
     cpu_baseline = None
     if not args.no_cpu_baseline:
@@ -147,6 +153,7 @@ def main() -> int:
         "cpu_baseline": cpu_baseline,
         "event_ms_per_step": round(event_ms / args.steps, 4),
         "kernels": kernels,
+        "kernel_configs": kernel_configs,
         "device": device,
         "setup_s": round(setup_s, 1),
     }

@@ -61,6 +61,10 @@ SIGNATURES = {
     "hm_event_destroy": (_I, [_P, _P]),
     "hm_event_record": (_I, [_P, _P]),
     "hm_event_elapsed_ms": (_I, [_P, _P, _P, c_f32_p]),
+    "hm_graph_begin": (_I, [_P]),
+    "hm_graph_end": (_I, [_P, c_void_pp]),
+    "hm_graph_launch": (_I, [_P, _P, _I]),
+    "hm_graph_destroy": (_I, [_P, _P]),
     "hm_gemv_bf16": (_I, [_P, _P, _P, _P, _I, _I, _I]),
     "hm_pack_bf16_kn_to_nk": (_I, [_P, _P, _P, _I, _I]),
     "hm_gemv_bf16_nk": (_I, [_P, _P, _P, _P, _I, _I, _I]),

@@ -167,6 +167,56 @@ int hm_device_name(hm_ctx *ctx, char *buf, size_t buflen) {
     return HM_OK;
 }
 
+// ── stream capture: callers with launch-bound inner loops record them once and replay ──
+
+struct hm_graph_handle {
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+};
+
+int hm_graph_begin(hm_ctx *ctx) {
+    HM_CHECK_CTX(ctx);
+    HM_HIP(ctx, hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeRelaxed));
+    return HM_OK;
+}
+
+int hm_graph_end(hm_ctx *ctx, void **graph_out) {
+    HM_CHECK_CTX(ctx);
+    HM_REQUIRE(ctx, graph_out != nullptr, "hm_graph_end: graph_out is NULL");
+    *graph_out = nullptr;
+    hipGraph_t g = nullptr;
+    HM_HIP(ctx, hipStreamEndCapture(ctx->stream, &g));
+    hm_graph_handle *h = new hm_graph_handle();
+    h->graph = g;
+    hipError_t e = hipGraphInstantiate(&h->exec, g, nullptr, nullptr, 0);
+    if (e != hipSuccess) {
+        (void)hipGraphDestroy(g);
+        delete h;
+        return hm_set_error(ctx, HM_ERR_HIP, "hipGraphInstantiate failed: %s", hipGetErrorString(e));
+    }
+    *graph_out = h;
+    return HM_OK;
+}
+
+int hm_graph_launch(hm_ctx *ctx, void *graph, int reps) {
+    HM_CHECK_CTX(ctx);
+    HM_REQUIRE(ctx, graph != nullptr && reps >= 1, "hm_graph_launch: bad arguments");
+    hm_graph_handle *h = (hm_graph_handle *)graph;
+    for (int i = 0; i < reps; i++) HM_HIP(ctx, hipGraphLaunch(h->exec, ctx->stream));
+    return HM_OK;
+}
+
+int hm_graph_destroy(hm_ctx *ctx, void *graph) {
+    HM_CHECK_CTX(ctx);
+    if (!graph) return HM_OK;
+    hm_graph_handle *h = (hm_graph_handle *)graph;
+    HM_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    if (h->exec) (void)hipGraphExecDestroy(h->exec);
+    if (h->graph) (void)hipGraphDestroy(h->graph);
+    delete h;
+    return HM_OK;
+}
+
 int hm_event_create(hm_ctx *ctx, void **ev_out) {
     HM_CHECK_CTX(ctx);
     HM_REQUIRE(ctx, ev_out != nullptr, "hm_event_create: ev_out is NULL");

@@ -495,14 +495,13 @@ constexpr int KN_COLS_PER_LANE = 4;                    // 8-byte loads
 constexpr int KN_STRIP = WAVE * KN_COLS_PER_LANE;      // 256 columns per workgroup
 
 // grid = (strips, ksplit). Each wave of the workgroup walks rows k = kbeg + wave, +4, ...
-// of the workgroup's K slice; partials are folded over the 4 waves in LDS, written to the
-// workspace, and the last workgroup to arrive for a strip folds the ksplit partials in
-// ascending order (deterministic) into out.
+// of the workgroup's K slice; partials are folded over the 4 waves in LDS and written to the
+// workspace; a second small kernel folds the ksplit partials in ascending order
+// (deterministic, and no device-scope fence is needed: the kernel boundary orders the writes).
 __global__ __launch_bounds__(GEMV_THREADS) void gemv_bf16_kn_kernel(
     const float *__restrict__ x, const uint16_t *__restrict__ w, float *__restrict__ out,
-    float *__restrict__ partial, unsigned int *__restrict__ counters, int K, int N, int kslice) {
+    float *__restrict__ partial, int K, int N, int kslice) {
     __shared__ float red[GEMV_WAVES][KN_STRIP];
-    __shared__ bool is_last;
     const int lane = threadIdx.x & (WAVE - 1);
     const int wave = threadIdx.x / WAVE;
     const int strip = blockIdx.x, ks = blockIdx.y, ksplit = gridDim.y;
@@ -512,7 +511,7 @@ __global__ __launch_bounds__(GEMV_THREADS) void gemv_bf16_kn_kernel(
 
     float acc[4] = {0.f, 0.f, 0.f, 0.f};
     if (col < N) {
-#pragma unroll 4
+#pragma unroll 8
         for (int k = kbeg + wave; k < kend; k += GEMV_WAVES) {
             const u32x2 wv = __builtin_nontemporal_load(
                 reinterpret_cast<const u32x2 *>(w + (size_t)k * N + col));
@@ -528,30 +527,21 @@ __global__ __launch_bounds__(GEMV_THREADS) void gemv_bf16_kn_kernel(
     __syncthreads();
     const int t = threadIdx.x;  // 256 threads <-> 256 columns
     const int c = strip * KN_STRIP + t;
-    float s = (red[0][t] + red[1][t]) + (red[2][t] + red[3][t]);
-    if (ksplit == 1) {
-        if (c < N) out[c] = s;
-        return;
-    }
-    if (c < N) partial[(size_t)ks * N + c] = s;
-    __threadfence();
-    __syncthreads();
-    if (t == 0) {
-        unsigned int prev = atomicAdd(&counters[strip], 1u);
-        is_last = (prev == (unsigned int)(ksplit - 1));
-    }
-    __syncthreads();
-    if (!is_last) return;
-    __threadfence();
-    if (c < N) {
-        float tot = 0.f;
-        for (int j = 0; j < ksplit; j++) tot += __builtin_nontemporal_load(&partial[(size_t)j * N + c]);
-        out[c] = tot;
-    }
-    if (t == 0) counters[strip] = 0u;  // leave the counter ready for the next call
+    const float s = (red[0][t] + red[1][t]) + (red[2][t] + red[3][t]);
+    if (c < N) (ksplit == 1 ? out : partial + (size_t)ks * N)[c] = s;
 }
 
-// [K][N] -> [N][K] through a 64x64 LDS tile (both sides coalesced).
+__global__ __launch_bounds__(256) void gemv_bf16_kn_fold_kernel(const float *__restrict__ partial,
+                                                                float *__restrict__ out, int N,
+                                                                int ksplit) {
+    const int c = blockIdx.x * 256 + threadIdx.x;
+    if (c >= N) return;
+    float tot = 0.f;
+#pragma unroll 8
+    for (int j = 0; j < ksplit; j++) tot += partial[(size_t)j * N + c];
+    out[c] = tot;
+}
+
 // Output row n lands at dst row n * row_mult + row_off (1, 0 = plain transpose; 2, 0 / 2, 1
 // interleave two matrices row by row).
 __global__ __launch_bounds__(256) void pack_kn_to_nk_kernel(const uint16_t *__restrict__ src,
@@ -632,7 +622,6 @@ int hm_gemv_bf16(hm_ctx *ctx, const float *d_x, const uint16_t *d_w_kn, float *d
     HM_REQUIRE(ctx, K > 0 && N > 0 && N % 4 == 0, "hm_gemv_bf16: need K > 0 and N %% 4 == 0 (K=%d N=%d)", K, N);
     HM_REQUIRE(ctx, ((uintptr_t)d_w_kn % 8) == 0, "hm_gemv_bf16: weight pointer must be 8-byte aligned");
     const int strips = (N + KN_STRIP - 1) / KN_STRIP;
-    HM_REQUIRE(ctx, (size_t)strips <= ctx->num_counters, "hm_gemv_bf16: N=%d too wide", N);
     // enough workgroups for ~2 per CU, but at least 16 K rows per workgroup
     int ksplit = (2 * ctx->num_cus + strips - 1) / strips;
     int max_split = (K + 15) / 16;
@@ -645,8 +634,13 @@ int hm_gemv_bf16(hm_ctx *ctx, const float *d_x, const uint16_t *d_w_kn, float *d
     for (int m = 0; m < M; m++) {
         hipLaunchKernelGGL(gemv_bf16_kn_kernel, dim3(strips, ksplit), dim3(GEMV_THREADS), 0,
                            ctx->stream, d_x + (size_t)m * K, d_w_kn, d_out + (size_t)m * N,
-                           (float *)ctx->workspace, ctx->counters, K, N, kslice);
+                           (float *)ctx->workspace, K, N, kslice);
         HM_LAUNCH_CHECK(ctx);
+        if (ksplit > 1) {
+            hipLaunchKernelGGL(gemv_bf16_kn_fold_kernel, dim3((N + 255) / 256), dim3(256), 0, ctx->stream,
+                               (const float *)ctx->workspace, d_out + (size_t)m * N, N, ksplit);
+            HM_LAUNCH_CHECK(ctx);
+        }
     }
     return HM_OK;
 }

@@ -57,9 +57,10 @@ __device__ __forceinline__ float block_dot_unsigned(const uint8_t *blk, const fl
 template <int QT>
 __global__ __launch_bounds__(QTHREADS) void gemv_quant_kernel(
     const float *__restrict__ x, const uint8_t *__restrict__ w, float *__restrict__ out, int K,
-    int N, int rows_per_wg, size_t total_bytes) {
+    int N, int rows_per_step, size_t total_bytes) {
     constexpr int BB = BlockTraits<QT>::BYTES;
     constexpr float OFFSET = QT == 0 ? 128.f : 8.f;
+    constexpr int U = 8;  // 16-byte weight loads a thread keeps in flight while staging
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     float *xs = reinterpret_cast<float *>(smem);
     uint8_t *ws = smem + (size_t)K * 4;
@@ -67,55 +68,76 @@ __global__ __launch_bounds__(QTHREADS) void gemv_quant_kernel(
     const int tid = threadIdx.x, lane = tid & (WAVE - 1), wave = tid / WAVE;
     const int nb = K / 32;
     const size_t rowbytes = (size_t)nb * BB;
-    const int r0 = blockIdx.x * rows_per_wg;
-    const int nrows = min(rows_per_wg, N - r0);
-    const size_t beg = (size_t)r0 * rowbytes;
-    const size_t end = beg + (size_t)nrows * rowbytes;
-    const size_t abeg = beg & ~(size_t)15;
-    const int shift = (int)(beg - abeg);
-    const int nchunks = (int)((end - abeg + 15) / 16);
+    const int nsteps = (N + rows_per_step - 1) / rows_per_step;
 
-    for (int i = tid; i < nchunks; i += QTHREADS) {
-        const size_t off = abeg + (size_t)i * 16;
-        if (off + 16 <= total_bytes) {
-            *reinterpret_cast<u32x4 *>(ws + (size_t)i * 16) = ld128_stream(w + off);
-        } else {  // last, partial chunk of the buffer: stay inside it
-            for (int b = 0; b < 16; b++) ws[(size_t)i * 16 + b] = off + b < total_bytes ? w[off + b] : 0;
-        }
-    }
+    // activations once per workgroup; the workgroup then walks row steps blockIdx, +grid, ...
     for (int k = tid; k < K; k += QTHREADS) xs[k] = x[k];
-    __syncthreads();
 
-    float acc[MAX_ROWS_PER_WAVE];
-#pragma unroll
-    for (int i = 0; i < MAX_ROWS_PER_WAVE; i++) acc[i] = 0.f;
+    for (int step = blockIdx.x; step < nsteps; step += gridDim.x) {
+        const int r0 = step * rows_per_step;
+        const int nrows = min(rows_per_step, N - r0);
+        const size_t beg = (size_t)r0 * rowbytes;
+        const size_t end = beg + (size_t)nrows * rowbytes;
+        const size_t abeg = beg & ~(size_t)15;
+        const int shift = (int)(beg - abeg);
+        const int nchunks = (int)((end - abeg + 15) / 16);
 
-    for (int bc = lane; bc < nb; bc += WAVE) {
-        float xv[32];
+        __syncthreads();  // previous step's readers are done with ws (and xs is complete)
+        for (int i0 = tid; i0 < nchunks; i0 += QTHREADS * U) {
+            u32x4 tmp[U];
 #pragma unroll
-        for (int j = 0; j < 8; j++) {
-            const f32x4 t = *reinterpret_cast<const f32x4 *>(xs + bc * 32 + j * 4);
-            xv[4 * j] = t.x; xv[4 * j + 1] = t.y; xv[4 * j + 2] = t.z; xv[4 * j + 3] = t.w;
+            for (int u = 0; u < U; u++) {
+                const int i = i0 + u * QTHREADS;
+                const size_t off = abeg + (size_t)i * 16;
+                tmp[u] = (i < nchunks && off + 16 <= total_bytes) ? ld128_stream(w + off)
+                                                                  : u32x4{0u, 0u, 0u, 0u};
+            }
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                const int i = i0 + u * QTHREADS;
+                if (i < nchunks) {
+                    const size_t off = abeg + (size_t)i * 16;
+                    if (off + 16 <= total_bytes) {
+                        *reinterpret_cast<u32x4 *>(ws + (size_t)i * 16) = tmp[u];
+                    } else {  // last, partial chunk of the buffer: stay inside it
+                        for (int b = 0; b < 16; b++)
+                            ws[(size_t)i * 16 + b] = off + b < total_bytes ? w[off + b] : 0;
+                    }
+                }
+            }
         }
-        float sx = 0.f;
+        __syncthreads();
+
+        float acc[MAX_ROWS_PER_WAVE];
 #pragma unroll
-        for (int j = 0; j < 32; j++) sx += xv[j];
+        for (int i = 0; i < MAX_ROWS_PER_WAVE; i++) acc[i] = 0.f;
+        for (int bc = lane; bc < nb; bc += WAVE) {
+            float xv[32];
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                const f32x4 t = *reinterpret_cast<const f32x4 *>(xs + bc * 32 + j * 4);
+                xv[4 * j] = t.x; xv[4 * j + 1] = t.y; xv[4 * j + 2] = t.z; xv[4 * j + 3] = t.w;
+            }
+            float sx = 0.f;
+#pragma unroll
+            for (int j = 0; j < 32; j++) sx += xv[j];
+#pragma unroll
+            for (int i = 0; i < MAX_ROWS_PER_WAVE; i++) {
+                const int lr = wave + QWAVES * i;
+                if (lr < nrows) {
+                    const uint8_t *blk = ws + shift + ((size_t)lr * nb + bc) * BB;
+                    const float d = f16_bits_to_f32((uint16_t)lds_u16(blk));
+                    const float s = block_dot_unsigned<QT>(blk, xv);
+                    acc[i] = fmaf(d, s - OFFSET * sx, acc[i]);
+                }
+            }
+        }
 #pragma unroll
         for (int i = 0; i < MAX_ROWS_PER_WAVE; i++) {
             const int lr = wave + QWAVES * i;
-            if (lr < nrows) {
-                const uint8_t *blk = ws + shift + ((size_t)lr * nb + bc) * BB;
-                const float d = f16_bits_to_f32((uint16_t)lds_u16(blk));
-                const float s = block_dot_unsigned<QT>(blk, xv);
-                acc[i] = fmaf(d, s - OFFSET * sx, acc[i]);
-            }
+            const float v = wave_sum(acc[i]);
+            if (lane == 0 && lr < nrows) out[r0 + lr] = v;
         }
-    }
-#pragma unroll
-    for (int i = 0; i < MAX_ROWS_PER_WAVE; i++) {
-        const int lr = wave + QWAVES * i;
-        const float v = wave_sum(acc[i]);
-        if (lane == 0 && lr < nrows) out[r0 + lr] = v;
     }
 }
 
@@ -156,14 +178,20 @@ int gemv_quant_launch(hm_ctx *ctx, const char *name, const float *d_x, const uin
     const size_t x_bytes = (size_t)K * 4;
     const size_t lds_budget = 48 * 1024;
     HM_REQUIRE(ctx, x_bytes + QWAVES * rowbytes + 32 <= 64 * 1024, "%s: K=%d too large for the LDS stage", name, K);
+    // rows staged per step: as many as fit the LDS budget (at most 8 per wavefront), but few
+    // enough that every CU gets a workgroup
     int rows = (int)((lds_budget - x_bytes) / rowbytes);
     rows = rows / QWAVES * QWAVES;
     if (rows < QWAVES) rows = QWAVES;
     if (rows > QWAVES * MAX_ROWS_PER_WAVE) rows = QWAVES * MAX_ROWS_PER_WAVE;
-    // keep at least ~4 workgroups per CU when N allows
-    while (rows > QWAVES && (N + rows - 1) / rows < 4 * ctx->num_cus) rows -= QWAVES;
+    while (rows > QWAVES && (N + rows - 1) / rows < 2 * ctx->num_cus) rows -= QWAVES;
     const size_t lds = x_bytes + (size_t)rows * rowbytes + 32;
-    const int grid = (N + rows - 1) / rows;
+    const int nsteps = (N + rows - 1) / rows;
+    // persistent workgroups: a few per CU, each stages the activations once
+    int wg_per_cu = (int)(120 * 1024 / lds);
+    if (wg_per_cu < 1) wg_per_cu = 1;
+    if (wg_per_cu > 6) wg_per_cu = 6;
+    const int grid = nsteps < ctx->num_cus * wg_per_cu ? nsteps : ctx->num_cus * wg_per_cu;
     const size_t total = (size_t)N * rowbytes;
     for (int m = 0; m < M; m++) {
         hipLaunchKernelGGL((gemv_quant_kernel<QT>), dim3(grid), dim3(QTHREADS), lds, ctx->stream,

@@ -1,0 +1,115 @@
+"""Roofline timing of the kernel-level entry points at the BASELINE shapes (configurations
+1, 3, 4, 5a, 5b). Every kernel is launched over a ring of weight copies larger than the last-
+level caches (Infinity Cache 256 MiB), all launches recorded into one HIP graph and replayed
+between two HIP events on the launch stream, so the numbers are cold-cache per-launch times.
+"""
+from __future__ import annotations
+
+import math
+
+import numpy as np
+
+from . import synth
+from .runtime import Context
+
+RING_BYTES = 400 << 20
+HBM_PEAK_GBS = 8000.0
+MFMA_BF16_PEAK_TFLOPS = 2500.0
+
+
+def _ring(ctx: Context, host: np.ndarray):
+    """Device copies of `host`, enough of them to exceed RING_BYTES."""
+    n = max(2, math.ceil(RING_BYTES / host.nbytes))
+    first = ctx.to_device(host)
+    copies = [first]
+    for _ in range(n - 1):
+        b = ctx.alloc(host.nbytes)
+        ctx._check(ctx.lib.hm_copy(ctx.h, b.ptr, first.ptr, host.nbytes))
+        copies.append(b)
+    ctx.sync()
+    return copies
+
+
+def _time(ctx: Context, launches, reps=10):
+    def record():
+        for fn in launches:
+            fn()
+    ms = ctx.time_graph_ms(record, reps=reps, warmup=2)
+    return ms * 1e3 / len(launches)  # microseconds per launch
+
+
+def _entry(name, us, nbytes=None, flops=None, note=None):
+    e = {"config": name, "avg_us": round(us, 3)}
+    if nbytes is not None:
+        gbs = nbytes / (us * 1e-6) / 1e9
+        e.update({"bytes_per_launch": int(nbytes), "GBps": round(gbs, 1),
+                  "hbm_frac": round(gbs / HBM_PEAK_GBS, 4)})
+    if flops is not None:
+        tf = flops / (us * 1e-6) / 1e12
+        e.update({"flop_per_launch": int(flops), "TFLOPs": round(tf, 1),
+                  "mfma_frac": round(tf / MFMA_BF16_PEAK_TFLOPS, 4)})
+    if note:
+        e["note"] = note
+    return e
+
+
+def run_all(ctx: Context):
+    out = []
+    # configuration 1: single bf16 GEMV x[1,896] x W[896,4864]
+    K, N = 896, 4864
+    x = ctx.to_device(synth.normal_f32(synth.SEED_CFG1, K))
+    w = synth.normal_bf16(synth.SEED_CFG1 + 1, K * N, 0.02)
+    ring = _ring(ctx, w)
+    o = ctx.empty(N)
+    nbytes = K * N * 2 + K * 4 + N * 4
+    us = _time(ctx, [lambda b=b: ctx.gemv_bf16(x, b, o, 1, K, N) for b in ring])
+    out.append(_entry("cfg1 gemv_bf16 [K,N] 896x4864", us, nbytes, note="reference weight layout"))
+    us = _time(ctx, [lambda b=b: ctx.gemv_bf16_nk(x, b, o, 1, K, N) for b in ring])
+    out.append(_entry("cfg1 gemv_bf16_nk [N,K] 4864x896", us, nbytes, note="stream layout"))
+    for b in ring:
+        b.free()
+
+    # configuration 3: Q8_0 dequant-GEMV 2048 -> 5632
+    K, N = 2048, 5632
+    x = ctx.to_device(synth.normal_f32(synth.SEED_CFG3 + 1, K))
+    ring = _ring(ctx, synth.q8_0_blocks(synth.SEED_CFG3, N * K // 32))
+    o = ctx.empty(N)
+    us = _time(ctx, [lambda b=b: ctx.gemv_q8_0(x, b, o, 1, K, N) for b in ring])
+    out.append(_entry("cfg3 gemv_q8_0 2048->5632", us, N * (K // 32) * 34 + K * 4 + N * 4))
+    for b in ring:
+        b.free()
+
+    # configuration 4: Q4_0 dequant-GEMV at LM-head shape 1536 -> 151936
+    K, N = 1536, 151936
+    x = ctx.to_device(synth.normal_f32(synth.SEED_CFG4 + 1, K))
+    ring = _ring(ctx, synth.q4_0_blocks(synth.SEED_CFG4, N * K // 32))
+    o = ctx.empty(N)
+    us = _time(ctx, [lambda b=b: ctx.gemv_q4_0(x, b, o, 1, K, N) for b in ring])
+    out.append(_entry("cfg4 gemv_q4_0 1536->151936", us, N * (K // 32) * 18 + K * 4 + N * 4))
+    for b in ring:
+        b.free()
+
+    # configuration 5a: prefill-chunk GEMM 512 x 2048 x 8192 on the matrix cores
+    M, K, N = 512, 2048, 8192
+    a = ctx.to_device(synth.normal_bf16(synth.SEED_CFG5, M * K, 1.0))
+    ring = _ring(ctx, synth.normal_bf16(synth.SEED_CFG5 + 1, K * N, 0.02))
+    c = ctx.empty(M * N)
+    us = _time(ctx, [lambda b=b: ctx.gemm_bf16(a, b, c, M, K, N) for b in ring])
+    out.append(_entry("cfg5a gemm_bf16 512x2048x8192", us, M * K * 2 + K * N * 2 + M * N * 4, 2.0 * M * K * N))
+    for b in ring:
+        b.free()
+
+    # configuration 5b: GQA decode attention, 8 sequences, 12/2 heads, hd 128, KV length 4096
+    B, H, kvh, hd, L = 8, 12, 2, 128, 4096
+    q = ctx.to_device(synth.normal_f32(synth.SEED_CFG5 + 2, B * H * hd))
+    kring = _ring(ctx, synth.normal_bf16(synth.SEED_CFG5 + 3, B * kvh * L * hd))
+    vring = _ring(ctx, synth.normal_bf16(synth.SEED_CFG5 + 4, B * kvh * L * hd))
+    o = ctx.empty(B * H * hd)
+    scale = 1.0 / math.sqrt(hd)
+    us = _time(ctx, [lambda k=k, v=v: ctx.gqa_decode_attn(q, k, v, o, B, H, kvh, hd, L, L, scale)
+                     for k, v in zip(kring, vring)])
+    out.append(_entry("cfg5b gqa_decode_attn 8x(12q/2kv)x128, kv 4096", us,
+                      2 * B * kvh * L * hd * 2 + 2 * B * H * hd * 4))
+    for b in kring + vring:
+        b.free()
+    return out

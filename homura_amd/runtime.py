@@ -124,6 +124,20 @@ class Context:
             self.lib.hm_event_destroy(self.h, e0)
             self.lib.hm_event_destroy(self.h, e1)
 
+    def time_graph_ms(self, record, reps: int = 20, warmup: int = 2) -> float:
+        """Capture the kernel launches `record()` makes into a HIP graph, replay it `reps`
+        times between two events and return the average milliseconds per replay."""
+        g = C.c_void_p()
+        self._check(self.lib.hm_graph_begin(self.h))
+        try:
+            record()
+        finally:
+            self._check(self.lib.hm_graph_end(self.h, C.byref(g)))
+        try:
+            return self.time_ms(lambda: self._check(self.lib.hm_graph_launch(self.h, g, 1)), reps, warmup)
+        finally:
+            self._check(self.lib.hm_graph_destroy(self.h, g))
+
     # kernel-level entry points (thin: pointer plumbing only)
     def gemv_bf16(self, x, w_kn, out, M, K, N):
         self._check(self.lib.hm_gemv_bf16(self.h, x.ptr, w_kn.ptr, out.ptr, M, K, N))

@@ -62,13 +62,22 @@ int hm_event_destroy(hm_ctx *ctx, void *ev);
 int hm_event_record(hm_ctx *ctx, void *ev);
 int hm_event_elapsed_ms(hm_ctx *ctx, void *ev_start, void *ev_stop, float *ms_out);
 
+/* Stream capture for launch-bound loops: every kernel-level entry point called between
+ * hm_graph_begin and hm_graph_end is recorded instead of run (no hm_alloc / hm_free / hm_upload /
+ * hm_download / hm_sync in between); hm_graph_launch replays the recording `reps` times.
+ * No counterpart in the reference (its kernels are plain host function calls). */
+int hm_graph_begin(hm_ctx *ctx);
+int hm_graph_end(hm_ctx *ctx, void **graph_out);
+int hm_graph_launch(hm_ctx *ctx, void *graph, int reps);
+int hm_graph_destroy(hm_ctx *ctx, void *graph);
+
 /* ── heavy ops ─────────────────────────────────────────────────────────────── */
 
 /* bf16-weight matmul, reference GraphBuilder::emit_matmul 3D x 2D arm with the mixed
  * f32 x bf16 region (src/graph_builder/emit_linalg.rs:1328-1339, :1928-2008, :2224-2307):
  * out[m,n] = sum_k x[m,k] * f32(W[k,n]); x f32 [M,K], W bf16 [K,N] row-major (the layout
  * the reference hands its kernels, src/hf/weights.rs:225-261), out f32 [M,N].
- * M <= 8. K % 8 == 0, N % 8 == 0. */
+ * M <= 8, N % 4 == 0. */
 int hm_gemv_bf16(hm_ctx *ctx, const float *d_x, const uint16_t *d_w_kn, float *d_out, int M,
                  int K, int N);
 
