@@ -46,6 +46,7 @@ def main() -> int:
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-tokens", type=int, default=96, help="tokens of the CPU-baseline sample")
     ap.add_argument("--kernel-rounds", type=int, default=20)
+    ap.add_argument("--kernel-reps", type=int, default=10, help="graph replays per stand-alone kernel measurement")
     ap.add_argument("--no-kernel-configs", action="store_true",
                     help="skip the stand-alone kernel measurements (BASELINE configurations 1, 3, 4, 5)")
     args = ap.parse_args()
@@ -119,6 +120,7 @@ def main() -> int:
         kernel_configs = None
         if not args.no_kernel_configs:
             from homura_amd import kernel_bench
+            kernel_bench.REPS = args.kernel_reps
             kernel_configs = kernel_bench.run_all(ctx)
 
     cpu_baseline = None

@@ -19,6 +19,10 @@ struct AttnArgs {
     const float *qw = nullptr, *kw = nullptr;
     const float *cos_tab = nullptr, *sin_tab = nullptr;  // [max_pos][hd]
     float eps = 0.f;
+    // which of the two kernels to enqueue: both (default), only the split attention, or only
+    // the fold of its partials (the decode plan lists them as separate device launches)
+    enum Phase { BOTH = 0, SPLIT_ONLY = 1, FOLD_ONLY = 2 };
+    int phase = BOTH;
 };
 
 int gqa_decode_attn_launch(hm_ctx *ctx, const AttnArgs &a);

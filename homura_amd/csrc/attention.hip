@@ -85,22 +85,22 @@ __global__ __launch_bounds__(ATT_THREADS) void gqa_decode_attn_kernel(
     const uint16_t *kbase = kcache + head_base + (size_t)n0 * HD + dl * 8;
     const uint16_t *vbase = vcache + head_base + (size_t)n0 * HD + dl * 8;
     const int nrg = chunk / (ATT_WAVES * RPI);  // row groups per wavefront (<= NRG_MAX)
-    const int row_cap = min(chunk, max_len - n0);  // rows of this chunk that exist in the cache
 
-    // ── every K and V row of the chunk is requested before anything waits ──
-    u32x4 kreg[NRG_MAX], vreg[NRG_MAX];
-#pragma unroll
-    for (int i = 0; i < NRG_MAX; i++) {
-        const int row = (i * ATT_WAVES + wave) * RPI + sub;
-        const bool ok = i < nrg && row < row_cap;
-        kreg[i] = ok ? ld128_stream(kbase + (size_t)row * HD) : u32x4{0u, 0u, 0u, 0u};
-        vreg[i] = ok ? ld128_stream(vbase + (size_t)row * HD) : u32x4{0u, 0u, 0u, 0u};
-    }
-
+    // The live length first (one scalar load): splits past it leave without touching memory.
     const int kv_len = state ? state->pos + 1 : kv_len_arg;
     const int nsplit = (kv_len + chunk - 1) / chunk;  // live splits; the grid may be larger
     if (split >= nsplit) return;
     const int cnt = min(kv_len, n0 + chunk) - n0;
+
+    // ── every live K and V row of the chunk is requested before anything waits ──
+    u32x4 kreg[NRG_MAX], vreg[NRG_MAX];
+#pragma unroll
+    for (int i = 0; i < NRG_MAX; i++) {
+        const int row = (i * ATT_WAVES + wave) * RPI + sub;
+        const bool ok = i < nrg && row < cnt;
+        kreg[i] = ok ? ld128_stream(kbase + (size_t)row * HD) : u32x4{0u, 0u, 0u, 0u};
+        vreg[i] = ok ? ld128_stream(vbase + (size_t)row * HD) : u32x4{0u, 0u, 0u, 0u};
+    }
     const bool fused = fuse.qkv_raw != nullptr;
     const int pos = kv_len - 1;
     const bool owner = fused && split == nsplit - 1;  // this chunk holds the new row
@@ -162,7 +162,7 @@ __global__ __launch_bounds__(ATT_THREADS) void gqa_decode_attn_kernel(
         if (i < nrg) {
             const int row = (i * ATT_WAVES + wave) * RPI + sub;
             const bool live = row < cnt && !(owner && row == new_row);
-            if (!live) vreg[i] = u32x4{0u, 0u, 0u, 0u};  // stale rows may hold anything
+            if (!live) vreg[i] = u32x4{0u, 0u, 0u, 0u};  // the new row's slot is not written yet
             float kf[8];
             unpack8(kreg[i], kf);
 #pragma unroll
@@ -276,55 +276,48 @@ __global__ __launch_bounds__(ATT_THREADS) void gqa_decode_attn_kernel(
     }
 }
 
-// Second half of the split attention: one workgroup per (batch, kv head) folds the partial
-// (o, max, sum) triples in ascending split order. A separate launch instead of a
-// "last workgroup to arrive" fold: the kernel boundary orders the partial writes, so no
-// device-scope fence (a full L2 write-back + invalidate on this chip) is needed.
+// Second half of the split attention: one workgroup of HD threads per (batch, query head)
+// folds that head's partial (o, max, sum) triples in ascending split order. A separate launch
+// instead of a "last workgroup to arrive" fold: the kernel boundary orders the partial writes,
+// so no device-scope fence (a full L2 write-back + invalidate on this chip) is needed.
 template <int HD, int G>
-__global__ __launch_bounds__(ATT_THREADS) void gqa_decode_fold_kernel(
+__global__ __launch_bounds__(HD) void gqa_decode_fold_kernel(
     float *__restrict__ out, const float *__restrict__ part_o, const float *__restrict__ part_ml,
     int kvh, int kv_len_arg, int chunk, const DecodeState *__restrict__ state) {
-    extern __shared__ float s_ml[];  // [nsplit][G][2]
-    const int tid = threadIdx.x;
-    const int kvhd = blockIdx.x, b = blockIdx.y;
+    extern __shared__ float s_ml[];  // [nsplit][2] of this head
+    const int d = threadIdx.x;
+    const int gi = blockIdx.x % G, kvhd = blockIdx.x / G, b = blockIdx.y;
     const int H = kvh * G;
     const int kv_len = state ? state->pos + 1 : kv_len_arg;
     const int nsplit = (kv_len + chunk - 1) / chunk;
     if (nsplit == 1) return;  // the attention kernel wrote the final result itself
     const size_t pair = (size_t)b * kvh + kvhd;
-    const float *ao = part_o + pair * nsplit * G * HD;
-    const float *aml = part_ml + pair * nsplit * G * 2;
-    for (int i = tid; i < nsplit * G * 2; i += ATT_THREADS) s_ml[i] = aml[i];
-    for (int i0 = 0; i0 < G * HD; i0 += ATT_THREADS) {
-        const int i = i0 + tid;
-        const int gi = i / HD, d = i % HD;
-        constexpr int FB = 16;  // splits fetched per batch, all loads of a batch in flight together
-        float L = 0.f, O = 0.f, M = -INFINITY;
-        bool have_m = false;
-        for (int s0 = 0; s0 < nsplit; s0 += FB) {
-            float o[FB];
+    const float *ao = part_o + (pair * nsplit * G + gi) * HD + d;
+    const float *aml = part_ml + (pair * nsplit * G + gi) * 2;
+    constexpr int FB = 16;  // splits fetched per batch, all loads of a batch in flight together
+    float o[FB];
 #pragma unroll
-            for (int u = 0; u < FB; u++)
-                o[u] = (i < G * HD && s0 + u < nsplit) ? ao[((size_t)(s0 + u) * G + gi) * HD + d] : 0.f;
-            if (!have_m) {
-                __syncthreads();  // s_ml complete (uniform across the block)
-                if (i < G * HD)
-                    for (int s = 0; s < nsplit; s++) M = fmaxf(M, s_ml[(s * G + gi) * 2]);
-                have_m = true;
-            }
-            if (i < G * HD) {
+    for (int u = 0; u < FB; u++) o[u] = u < nsplit ? ao[(size_t)u * G * HD] : 0.f;
+    for (int i = d; i < nsplit * 2; i += HD) s_ml[i] = aml[(size_t)(i >> 1) * G * 2 + (i & 1)];
+    __syncthreads();
+    float M = -INFINITY;
+    for (int s = 0; s < nsplit; s++) M = fmaxf(M, s_ml[s * 2]);
+    float L = 0.f, O = 0.f;
+    for (int s0 = 0; s0 < nsplit; s0 += FB) {
+        if (s0 > 0) {
 #pragma unroll
-                for (int u = 0; u < FB; u++) {
-                    if (s0 + u < nsplit) {
-                        const float wgt = expf(s_ml[((s0 + u) * G + gi) * 2] - M);
-                        L = fmaf(wgt, s_ml[((s0 + u) * G + gi) * 2 + 1], L);
-                        O = fmaf(wgt, o[u], O);
-                    }
-                }
+            for (int u = 0; u < FB; u++) o[u] = s0 + u < nsplit ? ao[(size_t)(s0 + u) * G * HD] : 0.f;
+        }
+#pragma unroll
+        for (int u = 0; u < FB; u++) {
+            if (s0 + u < nsplit) {
+                const float wgt = expf(s_ml[(s0 + u) * 2] - M);
+                L = fmaf(wgt, s_ml[(s0 + u) * 2 + 1], L);
+                O = fmaf(wgt, o[u], O);
             }
         }
-        if (i < G * HD) out[((size_t)b * H + kvhd * G + gi) * HD + d] = O / L;
     }
+    out[((size_t)b * H + kvhd * G + gi) * HD + d] = O / L;
 }
 
 // KvCache::append_key / append_value (reference src/runtime.rs:521-568) with the cache in
@@ -352,15 +345,18 @@ int launch_attn(hm_ctx *ctx, const AttnArgs &a, int nsplit, int chunk) {
     float *part_o = (float *)ctx->workspace;
     float *part_ml = part_o + pairs * nsplit * G * HD;
     AttnFuse f{a.qkv_raw, a.qw, a.kw, a.cos_tab, a.sin_tab, a.eps};
-    hipLaunchKernelGGL((gqa_decode_attn_kernel<HD, G>), dim3(nsplit, a.kvh, a.B), dim3(ATT_THREADS),
-                       lds, ctx->stream, a.q, const_cast<uint16_t *>(a.kcache),
-                       const_cast<uint16_t *>(a.vcache), a.out, part_o, part_ml, a.kvh, a.max_len,
-                       a.kv_len, chunk, a.scale, a.state, (int)front, f);
-    HM_LAUNCH_CHECK(ctx);
-    if (nsplit > 1) {  // nsplit is the grid's split count: 1 means no call can ever need a fold
-        const size_t fold_lds = (size_t)nsplit * G * 2 * sizeof(float);
+    if (a.phase != AttnArgs::FOLD_ONLY) {
+        hipLaunchKernelGGL((gqa_decode_attn_kernel<HD, G>), dim3(nsplit, a.kvh, a.B), dim3(ATT_THREADS),
+                           lds, ctx->stream, a.q, const_cast<uint16_t *>(a.kcache),
+                           const_cast<uint16_t *>(a.vcache), a.out, part_o, part_ml, a.kvh, a.max_len,
+                           a.kv_len, chunk, a.scale, a.state, (int)front, f);
+        HM_LAUNCH_CHECK(ctx);
+    }
+    // nsplit is the grid's split count: 1 means no call can ever need a fold
+    if (nsplit > 1 && a.phase != AttnArgs::SPLIT_ONLY) {
+        const size_t fold_lds = (size_t)nsplit * 2 * sizeof(float);
         HM_REQUIRE(ctx, fold_lds <= 64 * 1024, "gqa_decode_attn: too many splits (%d)", nsplit);
-        hipLaunchKernelGGL((gqa_decode_fold_kernel<HD, G>), dim3(a.kvh, a.B), dim3(ATT_THREADS), fold_lds,
+        hipLaunchKernelGGL((gqa_decode_fold_kernel<HD, G>), dim3(a.kvh * G, a.B), dim3(HD), fold_lds,
                            ctx->stream, a.out, part_o, part_ml, a.kvh, a.kv_len, chunk, a.state);
         HM_LAUNCH_CHECK(ctx);
     }

@@ -447,9 +447,8 @@ int HfModel::emit_transformer_plan() {
             a1.name = qkn ? "qknorm_rope_append+gqa_attn" : "rope_append+gqa_attn";
             a1.bytes_fixed = (qd + 2 * kvd) * 4.0 + qd * 4.0 + 2 * kvd * 2.0;
             a1.bytes_per_kv_row = 2.0 * kvh * hd * 2;
-            a1.hip_launches = 2;  // split attention + fold
             const size_t q_norm_slot = s.q_norm, k_norm_slot = s.k_norm;
-            a1.fn = [=](const StepContext &sc) -> int {
+            auto attn_args = [=](const StepContext &sc, int phase) {
                 const auto &in = sc.step.input_slots;
                 AttnArgs a;
                 a.qkv_raw = sc.pool[in[0]]->as<float>();  // q|k|v raw rows are adjacent
@@ -472,8 +471,21 @@ int HfModel::emit_transformer_plan() {
                 a.scale = (float)(1.0 / std::sqrt((double)hd));  // f64 -> f32 constant, emitter.rs:719
                 a.state = sc.plan->state();
                 a.fixed_chunk = att_chunk;
-                return gqa_decode_attn_launch(sc.ctx, a);
+                a.phase = phase;
+                return a;
             };
+            a1.fn = [=](const StepContext &sc) -> int {
+                return gqa_decode_attn_launch(sc.ctx, attn_args(sc, AttnArgs::SPLIT_ONLY));
+            };
+            k.launches.push_back(std::move(a1));
+            DeviceLaunch a1b;
+            a1b.name = "gqa_attn_fold";
+            a1b.bytes_fixed = qd * 4.0;
+            a1b.bytes_per_kv_row = (double)(qd + 2 * H) * 4.0 / att_chunk;  // partials: one set per chunk
+            a1b.fn = [=](const StepContext &sc) -> int {
+                return gqa_decode_attn_launch(sc.ctx, attn_args(sc, AttnArgs::FOLD_ONLY));
+            };
+            a1 = std::move(a1b);
             k.launches.push_back(std::move(a1));
             DeviceLaunch a2;
             a2.name = "gemv_bf16[o]";
@@ -785,9 +797,8 @@ int HfModel::emit_transformer_plan_quant() {
             l.name = qkn ? "qknorm_rope_append+gqa_attn" : "rope_append+gqa_attn";
             l.bytes_fixed = (qd + 2 * kvd) * 4.0 + qd * 4.0 + 2 * kvd * 2.0;
             l.bytes_per_kv_row = 2.0 * kvh * hd * 2;
-            l.hip_launches = 2;
             const size_t raw_slot = s.q_out, qn = s.q_norm, kn = s.k_norm;
-            l.fn = [=](const StepContext &sc) -> int {
+            auto attn_args = [=](const StepContext &sc, int phase) {
                 const auto &in = sc.step.input_slots;
                 AttnArgs a;
                 a.qkv_raw = sc.pool[raw_slot]->as<float>();
@@ -810,8 +821,21 @@ int HfModel::emit_transformer_plan_quant() {
                 a.scale = (float)(1.0 / std::sqrt((double)hd));
                 a.state = sc.plan->state();
                 a.fixed_chunk = att_chunk;
-                return gqa_decode_attn_launch(sc.ctx, a);
+                a.phase = phase;
+                return a;
             };
+            l.fn = [=](const StepContext &sc) -> int {
+                return gqa_decode_attn_launch(sc.ctx, attn_args(sc, AttnArgs::SPLIT_ONLY));
+            };
+            k.launches.push_back(std::move(l));
+            DeviceLaunch lf;
+            lf.name = "gqa_attn_fold";
+            lf.bytes_fixed = qd * 4.0;
+            lf.bytes_per_kv_row = (double)(qd + 2 * H) * 4.0 / att_chunk;
+            lf.fn = [=](const StepContext &sc) -> int {
+                return gqa_decode_attn_launch(sc.ctx, attn_args(sc, AttnArgs::FOLD_ONLY));
+            };
+            l = std::move(lf);
             k.launches.push_back(std::move(l));
             add_step(std::move(k), {s.q, s.present_k, s.present_v, mask}, {s.attn_body});
         }

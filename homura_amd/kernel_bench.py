@@ -30,7 +30,11 @@ def _ring(ctx: Context, host: np.ndarray):
     return copies
 
 
-def _time(ctx: Context, launches, reps=10):
+REPS = 10  # graph replays per measurement (bench.py lowers it under a profiler)
+
+
+def _time(ctx: Context, launches, reps=None):
+    reps = reps or REPS
     def record():
         for fn in launches:
             fn()
@@ -53,8 +57,20 @@ def _entry(name, us, nbytes=None, flops=None, note=None):
     return e
 
 
+def run_copy_calibration(ctx: Context):
+    """A plain transposing copy of known size (reads 32 MiB, writes 32 MiB of bf16): the yardstick
+    the FETCH_SIZE / WRITE_SIZE hardware counters of the other kernels are scaled by."""
+    K = N = 4096
+    src = ctx.to_device(synth.normal_bf16(1, K * N))
+    dst = ctx.empty(K * N, np.uint16)
+    us = _time(ctx, [lambda: ctx.pack_bf16_kn_to_nk(src, dst, K, N)] * 4)
+    src.free()
+    dst.free()
+    return _entry("calibration pack_kn_to_nk 4096x4096 bf16 (read 32 MiB + write 32 MiB)", us, 2 * K * N * 2)
+
+
 def run_all(ctx: Context):
-    out = []
+    out = [run_copy_calibration(ctx)]
     # configuration 1: single bf16 GEMV x[1,896] x W[896,4864]
     K, N = 896, 4864
     x = ctx.to_device(synth.normal_f32(synth.SEED_CFG1, K))
