@@ -111,7 +111,11 @@ def run_all(ctx: Context):
     ring = _ring(ctx, synth.normal_bf16(synth.SEED_CFG5 + 1, K * N, 0.02))
     c = ctx.empty(M * N)
     us = _time(ctx, [lambda b=b: ctx.gemm_bf16(a, b, c, M, K, N) for b in ring])
-    out.append(_entry("cfg5a gemm_bf16 512x2048x8192", us, M * K * 2 + K * N * 2 + M * N * 4, 2.0 * M * K * N))
+    out.append(_entry("cfg5a gemm_bf16 512x2048x8192", us, M * K * 2 + K * N * 2 + M * N * 4, 2.0 * M * K * N,
+                      note="B [K,N], reference weight layout"))
+    us = _time(ctx, [lambda b=b: ctx.gemm_bf16_nk(a, b, c, M, K, N) for b in ring])
+    out.append(_entry("cfg5a gemm_bf16_nk 512x2048x8192", us, M * K * 2 + K * N * 2 + M * N * 4, 2.0 * M * K * N,
+                      note="B [N,K], stream layout (same bytes; values differ from the [K,N] case)"))
     for b in ring:
         b.free()
 

@@ -163,6 +163,9 @@ class Context:
     def gemm_bf16(self, a, b, c, M, K, N):
         self._check(self.lib.hm_gemm_bf16(self.h, a.ptr, b.ptr, c.ptr, M, K, N))
 
+    def gemm_bf16_nk(self, a, b_nk, c, M, K, N):
+        self._check(self.lib.hm_gemm_bf16_nk(self.h, a.ptr, b_nk.ptr, c.ptr, M, K, N))
+
     def kv_append(self, kc, vc, k, v, B, kvh, hd, max_len, pos, n_new):
         self._check(self.lib.hm_kv_append(self.h, kc.ptr, vc.ptr, k.ptr, v.ptr, B, kvh, hd,
                                           max_len, pos, n_new))

@@ -113,6 +113,10 @@ int hm_dequant_q4_0(hm_ctx *ctx, const uint8_t *d_blocks, float *d_out, size_t n
  * C f32 [M,N], f32 accumulate. M % 128 == 0, N % 128 == 0, K % 32 == 0. */
 int hm_gemm_bf16(hm_ctx *ctx, const uint16_t *d_a_mk, const uint16_t *d_b_kn, float *d_c, int M,
                  int K, int N);
+/* Same product with B in the stream layout [N,K] (what hm_pack_bf16_kn_to_nk writes and the
+ * decode GEMVs read), so prefill and decode share one copy of a weight. Same constraints. */
+int hm_gemm_bf16_nk(hm_ctx *ctx, const uint16_t *d_a_mk, const uint16_t *d_b_nk, float *d_c, int M,
+                    int K, int N);
 
 /* ── KV cache + attention ──────────────────────────────────────────────────── */
 

@@ -125,15 +125,21 @@ def test_quant_gemv(ctx, oracle, kind, M, K, N):
 
 # ── prefill GEMM (MFMA) ───────────────────────────────────────────────────────
 
+@pytest.mark.parametrize("layout", ["kn", "nk"])
 @pytest.mark.parametrize("M,K,N", [(512, 2048, 8192),  # BASELINE config 5a
-                                   (128, 32, 128), (256, 96, 384)])
-def test_gemm_bf16_mfma(ctx, oracle, M, K, N):
-    say(f"gemm_bf16 M={M} K={K} N={N}")
+                                   (128, 32, 128), (256, 96, 384), (384, 64, 1152), (128, 160, 1024)])
+def test_gemm_bf16_mfma(ctx, oracle, M, K, N, layout):
+    say(f"gemm_bf16 M={M} K={K} N={N} B layout {layout}")
     a = synth.normal_bf16(synth.SEED_CFG5, M * K, 1.0).reshape(M, K)
     b = synth.normal_bf16(synth.SEED_CFG5 + 1, K * N, 0.02).reshape(K, N)
     want = oracle.matmul_bf16_bf16(a, b, M, K, N)
-    da, db, dc = ctx.to_device(a), ctx.to_device(b), ctx.empty(M * N)
-    ctx.gemm_bf16(da, db, dc, M, K, N)
+    da, dc = ctx.to_device(a), ctx.empty(M * N)
+    if layout == "kn":
+        db = ctx.to_device(b)
+        ctx.gemm_bf16(da, db, dc, M, K, N)
+    else:
+        db = ctx.to_device(np.ascontiguousarray(b.T))
+        ctx.gemm_bf16_nk(da, db, dc, M, K, N)
     got = dc.download(np.float32, (M, N))
     assert rel_err(got, want) < TOL
     for buf in (da, db, dc):
