@@ -3,9 +3,16 @@
 // Weights stay in HBM as the raw GGUF block bytes, rows of K/32 blocks. A workgroup takes a
 // contiguous run of rows, which is a contiguous byte range of the weight buffer, and copies
 // it into LDS with aligned 16-byte loads (blocks are 34 or 18 bytes, so block starts are only
-// 2-byte aligned; the copy is aligned on the buffer, not on the blocks). Each lane then owns
-// one block column: it keeps the 32 activations of that column in registers and walks the
-// rows, unpacking scale and quants from LDS. HBM traffic is exactly the block bytes.
+// 2-byte aligned; the copy is aligned on the buffer, not on the blocks). HBM traffic is exactly
+// the block bytes.
+//
+// The unit of work of a lane is a quarter block: 8 weights = 8 quant bytes (Q8_0) or one 32-bit
+// word of nibble pairs (Q4_0), plus the block's scale. Quarter columns are dealt to the lanes
+// round-robin (K/8 of them, so K = 1536 fills three full rounds where whole blocks would leave a
+// quarter of the wavefront idle); a lane keeps the 8 activations of each of its columns, and
+// their sum, in registers for the life of the workgroup and walks the staged rows. Quants are
+// used as stored (biased unsigned): sum_j q_j x_j - offset * sum_j x_j, four byte->float
+// conversions per 32-bit word with no shifts for the byte lanes.
 #include "hm_common.h"
 
 namespace {
@@ -13,65 +20,97 @@ namespace {
 constexpr int QTHREADS = 256;
 constexpr int QWAVES = QTHREADS / WAVE;
 constexpr int MAX_ROWS_PER_WAVE = 8;
+constexpr int MAXC = 8;  // most quarter columns a lane keeps in registers (K <= 4096); more are re-read
 
 template <int QT>
 struct BlockTraits;
 template <>
 struct BlockTraits<0> {  // Q8_0: f16 d + 32 x int8 (reference src/gguf.rs:817-831)
     static constexpr int BYTES = 34;
+    static constexpr int QUARTER = 8;  // quant bytes of 8 weights
 };
 template <>
 struct BlockTraits<1> {  // Q4_0: f16 d + 16 bytes of nibble pairs (ggml block_q4_0)
     static constexpr int BYTES = 18;
+    static constexpr int QUARTER = 4;
 };
 
 __device__ __forceinline__ uint32_t lds_u16(const uint8_t *p) {
     return *reinterpret_cast<const uint16_t *>(p);
 }
+// 32-bit word at a 2-byte aligned LDS address
+__device__ __forceinline__ uint32_t lds_u32_a2(const uint8_t *p) { return lds_u16(p) | (lds_u16(p + 2) << 16); }
 
-// sum_j q_j * x_j for one block, q taken as stored (unsigned byte / nibble); the caller
-// removes the offset (128 or 8) with the precomputed sum of the activations.
-template <int QT>
-__device__ __forceinline__ float block_dot_unsigned(const uint8_t *blk, const float *xv) {
-    float s = 0.f;
-    if (QT == 0) {
-#pragma unroll
-        for (int j = 0; j < 16; j++) {
-            uint32_t v = lds_u16(blk + 2 + 2 * j) ^ 0x8080u;  // int8 -> biased unsigned
-            s = fmaf((float)(v & 0xFFu), xv[2 * j], s);
-            s = fmaf((float)(v >> 8), xv[2 * j + 1], s);
-        }
-    } else {
-#pragma unroll
-        for (int j = 0; j < 8; j++) {
-            uint32_t v = lds_u16(blk + 2 + 2 * j);  // bytes 2j, 2j+1
-            s = fmaf((float)(v & 0xFu), xv[2 * j], s);
-            s = fmaf((float)((v >> 4) & 0xFu), xv[2 * j + 16], s);
-            s = fmaf((float)((v >> 8) & 0xFu), xv[2 * j + 1], s);
-            s = fmaf((float)(v >> 12), xv[2 * j + 17], s);
-        }
-    }
+__device__ __forceinline__ float dot4_bytes(uint32_t w, const float *xv, float s) {
+    s = fmaf((float)(w & 0xFFu), xv[0], s);
+    s = fmaf((float)((w >> 8) & 0xFFu), xv[1], s);
+    s = fmaf((float)((w >> 16) & 0xFFu), xv[2], s);
+    s = fmaf((float)(w >> 24), xv[3], s);
     return s;
 }
 
+// Activations of quarter column c (block c/4, quarter c%4) in the order the quant bytes use them.
 template <int QT>
+__device__ __forceinline__ void load_xv(const float *xs, int c, float *xv, float &sx_off) {
+    const int b = c >> 2, q = c & 3;
+    const float *p0 = xs + b * 32 + (QT == 0 ? q * 8 : q * 4);
+    const float *p1 = QT == 0 ? p0 + 4 : p0 + 16;
+    const f32x4 lo = *reinterpret_cast<const f32x4 *>(p0);
+    const f32x4 hi = *reinterpret_cast<const f32x4 *>(p1);
+    xv[0] = lo.x; xv[1] = lo.y; xv[2] = lo.z; xv[3] = lo.w;
+    xv[4] = hi.x; xv[5] = hi.y; xv[6] = hi.z; xv[7] = hi.w;
+    float sx = 0.f;
+#pragma unroll
+    for (int j = 0; j < 8; j++) sx += xv[j];
+    sx_off = sx * (QT == 0 ? 128.f : 8.f);
+}
+
+// d * (sum_j q_j x_j) for one quarter block at `blk` (start of the block in LDS).
+template <int QT>
+__device__ __forceinline__ float quarter_dot(const uint8_t *blk, int q, const float *xv, float sx_off) {
+    const float d = f16_bits_to_f32((uint16_t)lds_u16(blk));
+    float s;
+    if (QT == 0) {
+        const uint32_t w0 = lds_u32_a2(blk + 2 + q * 8) ^ 0x80808080u;  // int8 -> biased unsigned
+        const uint32_t w1 = lds_u32_a2(blk + 6 + q * 8) ^ 0x80808080u;
+        s = dot4_bytes(w1, xv + 4, dot4_bytes(w0, xv, 0.f));
+    } else {
+        // byte i of the word: low nibble = weight 4q+i, high nibble = weight 16+4q+i
+        const uint32_t w = lds_u32_a2(blk + 2 + q * 4);
+        s = dot4_bytes((w >> 4) & 0x0F0F0F0Fu, xv + 4, dot4_bytes(w & 0x0F0F0F0Fu, xv, 0.f));
+    }
+    return d * (s - sx_off);
+}
+
+// CPL = quarter columns per lane held in registers (ceil(K/8/64)); 0 = re-read them from LDS.
+template <int QT, int CPL>
 __global__ __launch_bounds__(QTHREADS) void gemv_quant_kernel(
     const float *__restrict__ x, const uint8_t *__restrict__ w, float *__restrict__ out, int K,
     int N, int rows_per_step, size_t total_bytes) {
     constexpr int BB = BlockTraits<QT>::BYTES;
-    constexpr float OFFSET = QT == 0 ? 128.f : 8.f;
     constexpr int U = 8;  // 16-byte weight loads a thread keeps in flight while staging
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     float *xs = reinterpret_cast<float *>(smem);
     uint8_t *ws = smem + (size_t)K * 4;
 
     const int tid = threadIdx.x, lane = tid & (WAVE - 1), wave = tid / WAVE;
-    const int nb = K / 32;
+    const int nb = K / 32, nq = K / 8;
+    constexpr bool resident = CPL > 0;
+    constexpr int NXV = resident ? CPL : 1;
     const size_t rowbytes = (size_t)nb * BB;
     const int nsteps = (N + rows_per_step - 1) / rows_per_step;
 
     // activations once per workgroup; the workgroup then walks row steps blockIdx, +grid, ...
-    for (int k = tid; k < K; k += QTHREADS) xs[k] = x[k];
+    for (int k = tid * 4; k < K; k += QTHREADS * 4) *reinterpret_cast<f32x4 *>(xs + k) = *reinterpret_cast<const f32x4 *>(x + k);
+    __syncthreads();
+    float xv[NXV][8], sxo[NXV];
+    if (resident) {
+#pragma unroll
+        for (int t = 0; t < NXV; t++) {
+            const int c = lane + t * WAVE;
+            if (c < nq) load_xv<QT>(xs, c, xv[t], sxo[t]);
+        }
+    }
 
     for (int step = blockIdx.x; step < nsteps; step += gridDim.x) {
         const int r0 = step * rows_per_step;
@@ -82,7 +121,7 @@ __global__ __launch_bounds__(QTHREADS) void gemv_quant_kernel(
         const int shift = (int)(beg - abeg);
         const int nchunks = (int)((end - abeg + 15) / 16);
 
-        __syncthreads();  // previous step's readers are done with ws (and xs is complete)
+        __syncthreads();  // previous step's readers are done with ws
         for (int i0 = tid; i0 < nchunks; i0 += QTHREADS * U) {
             u32x4 tmp[U];
 #pragma unroll
@@ -108,35 +147,49 @@ __global__ __launch_bounds__(QTHREADS) void gemv_quant_kernel(
         }
         __syncthreads();
 
-        float acc[MAX_ROWS_PER_WAVE];
+        if (resident) {
+            // two rows per trip: independent chains for the LDS reads and the reductions
+            for (int lr = wave; lr < nrows; lr += 2 * QWAVES) {
+                const int lr1 = lr + QWAVES;
+                const bool two = lr1 < nrows;
+                const uint8_t *row0 = ws + shift + (size_t)lr * rowbytes;
+                const uint8_t *row1 = two ? row0 + (size_t)QWAVES * rowbytes : row0;
+                float a0 = 0.f, a1 = 0.f;
 #pragma unroll
-        for (int i = 0; i < MAX_ROWS_PER_WAVE; i++) acc[i] = 0.f;
-        for (int bc = lane; bc < nb; bc += WAVE) {
-            float xv[32];
-#pragma unroll
-            for (int j = 0; j < 8; j++) {
-                const f32x4 t = *reinterpret_cast<const f32x4 *>(xs + bc * 32 + j * 4);
-                xv[4 * j] = t.x; xv[4 * j + 1] = t.y; xv[4 * j + 2] = t.z; xv[4 * j + 3] = t.w;
+                for (int t = 0; t < NXV; t++) {
+                    const int c = lane + t * WAVE;
+                    if (c < nq) {
+                        a0 += quarter_dot<QT>(row0 + (c >> 2) * BB, c & 3, xv[t], sxo[t]);
+                        a1 += quarter_dot<QT>(row1 + (c >> 2) * BB, c & 3, xv[t], sxo[t]);
+                    }
+                }
+                a0 = wave_sum(a0);
+                a1 = wave_sum(a1);
+                if (lane == 0) {
+                    out[r0 + lr] = a0;
+                    if (two) out[r0 + lr1] = a1;
+                }
             }
-            float sx = 0.f;
+        } else {  // long rows: the activations of a column are re-read from LDS
+            float acc[MAX_ROWS_PER_WAVE];
 #pragma unroll
-            for (int j = 0; j < 32; j++) sx += xv[j];
+            for (int i = 0; i < MAX_ROWS_PER_WAVE; i++) acc[i] = 0.f;
+            for (int c = lane; c < nq; c += WAVE) {
+                float xc[8], so;
+                load_xv<QT>(xs, c, xc, so);
+#pragma unroll
+                for (int i = 0; i < MAX_ROWS_PER_WAVE; i++) {
+                    const int lr = wave + QWAVES * i;
+                    if (lr < nrows)
+                        acc[i] += quarter_dot<QT>(ws + shift + (size_t)lr * rowbytes + (c >> 2) * BB, c & 3, xc, so);
+                }
+            }
 #pragma unroll
             for (int i = 0; i < MAX_ROWS_PER_WAVE; i++) {
                 const int lr = wave + QWAVES * i;
-                if (lr < nrows) {
-                    const uint8_t *blk = ws + shift + ((size_t)lr * nb + bc) * BB;
-                    const float d = f16_bits_to_f32((uint16_t)lds_u16(blk));
-                    const float s = block_dot_unsigned<QT>(blk, xv);
-                    acc[i] = fmaf(d, s - OFFSET * sx, acc[i]);
-                }
+                const float v = wave_sum(acc[i]);
+                if (lane == 0 && lr < nrows) out[r0 + lr] = v;
             }
-        }
-#pragma unroll
-        for (int i = 0; i < MAX_ROWS_PER_WAVE; i++) {
-            const int lr = wave + QWAVES * i;
-            const float v = wave_sum(acc[i]);
-            if (lane == 0 && lr < nrows) out[r0 + lr] = v;
         }
     }
 }
@@ -173,7 +226,7 @@ int gemv_quant_launch(hm_ctx *ctx, const char *name, const float *d_x, const uin
     HM_REQUIRE(ctx, d_x && d_w && d_out, "%s: NULL pointer", name);
     HM_REQUIRE(ctx, M >= 1 && M <= 8, "%s: M=%d outside 1..8", name, M);
     HM_REQUIRE(ctx, K > 0 && K % 32 == 0 && N > 0, "%s: K=%d must be a positive multiple of 32, N=%d positive", name, K, N);
-    HM_REQUIRE(ctx, ((uintptr_t)d_w % 16) == 0 && ((uintptr_t)d_x % 4) == 0, "%s: weight buffer must be 16-byte aligned", name);
+    HM_REQUIRE(ctx, ((uintptr_t)d_w % 16) == 0 && ((uintptr_t)d_x % 16) == 0, "%s: weight and activation buffers must be 16-byte aligned", name);
     const size_t rowbytes = (size_t)(K / 32) * BB;
     const size_t x_bytes = (size_t)K * 4;
     const size_t lds_budget = 48 * 1024;
@@ -193,9 +246,25 @@ int gemv_quant_launch(hm_ctx *ctx, const char *name, const float *d_x, const uin
     if (wg_per_cu > 6) wg_per_cu = 6;
     const int grid = nsteps < ctx->num_cus * wg_per_cu ? nsteps : ctx->num_cus * wg_per_cu;
     const size_t total = (size_t)N * rowbytes;
+    const int cpl = (K / 8 + WAVE - 1) / WAVE;
     for (int m = 0; m < M; m++) {
-        hipLaunchKernelGGL((gemv_quant_kernel<QT>), dim3(grid), dim3(QTHREADS), lds, ctx->stream,
-                           d_x + (size_t)m * K, d_w, d_out + (size_t)m * N, K, N, rows, total);
+        const float *xm = d_x + (size_t)m * K;
+        float *om = d_out + (size_t)m * N;
+#define HM_QUANT_CASE(C)                                                                                  \
+    hipLaunchKernelGGL((gemv_quant_kernel<QT, C>), dim3(grid), dim3(QTHREADS), lds, ctx->stream, xm, d_w, \
+                       om, K, N, rows, total)
+        switch (cpl <= MAXC ? cpl : 0) {
+            case 1: HM_QUANT_CASE(1); break;
+            case 2: HM_QUANT_CASE(2); break;
+            case 3: HM_QUANT_CASE(3); break;
+            case 4: HM_QUANT_CASE(4); break;
+            case 5: HM_QUANT_CASE(5); break;
+            case 6: HM_QUANT_CASE(6); break;
+            case 7: HM_QUANT_CASE(7); break;
+            case 8: HM_QUANT_CASE(8); break;
+            default: HM_QUANT_CASE(0); break;
+        }
+#undef HM_QUANT_CASE
         HM_LAUNCH_CHECK(ctx);
     }
     return HM_OK;

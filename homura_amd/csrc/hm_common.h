@@ -82,18 +82,35 @@ __device__ __forceinline__ float f16_bits_to_f32(uint16_t h) {
     return (float)f;
 }
 
-// Sum over the 64 lanes of a wavefront; every lane receives the total.
-// Fixed butterfly order, so the result is deterministic.
+// Wavefront reductions on the DPP path (no LDS round trips): four steps inside each row of 16
+// lanes (quad swaps, half-row and row mirrors), then lane 15 / lane 31 broadcasts carry the row
+// totals upward so that lane 63 holds the result, which is read back as a scalar. Fixed order,
+// so the result is deterministic; every lane receives the total.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_move(float v, float fill) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(fill), __float_as_int(v), CTRL, ROW_MASK,
+                                                      0xF, false));
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off, WAVE);
-    return v;
+    v += dpp_move<0xB1, 0xF>(v, 0.f);   // quad_perm [1,0,3,2]
+    v += dpp_move<0x4E, 0xF>(v, 0.f);   // quad_perm [2,3,0,1]
+    v += dpp_move<0x141, 0xF>(v, 0.f);  // row_half_mirror
+    v += dpp_move<0x140, 0xF>(v, 0.f);  // row_mirror: every lane of a row holds the row total
+    v += dpp_move<0x142, 0xA>(v, 0.f);  // row_bcast15 into rows 1 and 3
+    v += dpp_move<0x143, 0xC>(v, 0.f);  // row_bcast31 into rows 2 and 3
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
 }
 
 __device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, WAVE));
-    return v;
+    const float ninf = -__builtin_huge_valf();
+    v = fmaxf(v, dpp_move<0xB1, 0xF>(v, ninf));
+    v = fmaxf(v, dpp_move<0x4E, 0xF>(v, ninf));
+    v = fmaxf(v, dpp_move<0x141, 0xF>(v, ninf));
+    v = fmaxf(v, dpp_move<0x140, 0xF>(v, ninf));
+    v = fmaxf(v, dpp_move<0x142, 0xA>(v, ninf));
+    v = fmaxf(v, dpp_move<0x143, 0xC>(v, ninf));
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
 }
 
 // 16-byte global load as four dwords.
