@@ -65,30 +65,86 @@ __device__ __forceinline__ void load_xv(const float *xs, int c, float *xv, float
     sx_off = sx * (QT == 0 ? 128.f : 8.f);
 }
 
-// d * (sum_j q_j x_j) for one quarter block at `blk` (start of the block in LDS).
+// d * (sum_j q_j x_j - offset * sum_j x_j) for one quarter block: `dp` points at the block's scale,
+// `qp` at the quarter's quant bytes (both in LDS, 2-byte aligned).
 template <int QT>
-__device__ __forceinline__ float quarter_dot(const uint8_t *blk, int q, const float *xv, float sx_off) {
-    const float d = f16_bits_to_f32((uint16_t)lds_u16(blk));
+__device__ __forceinline__ float quarter_dot(const uint8_t *dp, const uint8_t *qp, const float *xv, float sx_off) {
+    const float d = f16_bits_to_f32((uint16_t)lds_u16(dp));
     float s;
     if (QT == 0) {
-        const uint32_t w0 = lds_u32_a2(blk + 2 + q * 8) ^ 0x80808080u;  // int8 -> biased unsigned
-        const uint32_t w1 = lds_u32_a2(blk + 6 + q * 8) ^ 0x80808080u;
+        const uint32_t w0 = lds_u32_a2(qp) ^ 0x80808080u;  // int8 -> biased unsigned
+        const uint32_t w1 = lds_u32_a2(qp + 4) ^ 0x80808080u;
         s = dot4_bytes(w1, xv + 4, dot4_bytes(w0, xv, 0.f));
     } else {
         // byte i of the word: low nibble = weight 4q+i, high nibble = weight 16+4q+i
-        const uint32_t w = lds_u32_a2(blk + 2 + q * 4);
+        const uint32_t w = lds_u32_a2(qp);
         s = dot4_bytes((w >> 4) & 0x0F0F0F0Fu, xv + 4, dot4_bytes(w & 0x0F0F0F0Fu, xv, 0.f));
     }
     return d * (s - sx_off);
+}
+
+constexpr int STAGE_U = 8;                       // 16-byte chunks a thread carries per row step
+constexpr int STAGE_BYTES = QTHREADS * STAGE_U * 16;  // most bytes one row step may span
+
+// The aligned 16-byte chunks covering rows [r0, r0+nrows): chunk i of the step starts at abeg + 16 i.
+// A chunk that holds at least one byte of the buffer lies in that byte's page, so reading whole
+// aligned chunks at both ends of the buffer cannot fault.
+struct StepRange {
+    size_t abeg;
+    int shift, nchunks, r0, nrows;
+};
+__device__ __forceinline__ StepRange step_range(int step, int rows_per_step, int N, size_t rowbytes) {
+    StepRange r;
+    r.r0 = step * rows_per_step;
+    r.nrows = min(rows_per_step, N - r.r0);
+    const size_t beg = (size_t)r.r0 * rowbytes, end = beg + (size_t)r.nrows * rowbytes;
+    r.abeg = beg & ~(size_t)15;
+    r.shift = (int)(beg - r.abeg);
+    r.nchunks = (int)((end - r.abeg + 15) / 16);
+    return r;
+}
+
+// RT rows lr, lr+QWAVES, ... of the staged step for one wavefront, activations in registers.
+// Round t of a lane is quarter column lane + 64 t: 16 blocks further along the row, a constant
+// offset from the lane's first column. Lanes past the row end read whatever follows in LDS (the
+// allocation carries slack for it) and their value is dropped by a select.
+template <int QT, int NXV, int RT>
+__device__ __forceinline__ void rows_trip(const uint8_t *base, size_t rowbytes, int lr, int lane, int nq,
+                                          const float (&xv)[NXV][8], const float (&sxo)[NXV], float *out) {
+    constexpr int BB = BlockTraits<QT>::BYTES;
+    const int doff = (lane >> 2) * BB;
+    const int qoff = doff + 2 + (lane & 3) * BlockTraits<QT>::QUARTER;
+    const uint8_t *row[RT];
+    float a[RT];
+#pragma unroll
+    for (int j = 0; j < RT; j++) {
+        row[j] = base + (size_t)(lr + j * QWAVES) * rowbytes;
+        a[j] = 0.f;
+    }
+#pragma unroll
+    for (int t = 0; t < NXV; t++) {
+        const bool live = lane + t * WAVE < nq;
+#pragma unroll
+        for (int j = 0; j < RT; j++) {
+            const float v = quarter_dot<QT>(row[j] + doff + t * 16 * BB, row[j] + qoff + t * 16 * BB, xv[t], sxo[t]);
+            a[j] += live ? v : 0.f;
+        }
+        __builtin_amdgcn_sched_barrier(0);  // keep the LDS reads of later rounds from piling up in registers
+    }
+#pragma unroll
+    for (int j = 0; j < RT; j++) {
+        a[j] = wave_sum(a[j]);
+        if (lane == 0) out[lr + j * QWAVES] = a[j];
+    }
 }
 
 // CPL = quarter columns per lane held in registers (ceil(K/8/64)); 0 = re-read them from LDS.
 template <int QT, int CPL>
 __global__ __launch_bounds__(QTHREADS) void gemv_quant_kernel(
     const float *__restrict__ x, const uint8_t *__restrict__ w, float *__restrict__ out, int K,
-    int N, int rows_per_step, size_t total_bytes) {
+    int N, int rows_per_step) {
     constexpr int BB = BlockTraits<QT>::BYTES;
-    constexpr int U = 8;  // 16-byte weight loads a thread keeps in flight while staging
+    constexpr int U = STAGE_U;
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     float *xs = reinterpret_cast<float *>(smem);
     uint8_t *ws = smem + (size_t)K * 4;
@@ -100,76 +156,70 @@ __global__ __launch_bounds__(QTHREADS) void gemv_quant_kernel(
     const size_t rowbytes = (size_t)nb * BB;
     const int nsteps = (N + rows_per_step - 1) / rows_per_step;
 
-    // activations once per workgroup; the workgroup then walks row steps blockIdx, +grid, ...
-    for (int k = tid * 4; k < K; k += QTHREADS * 4) *reinterpret_cast<f32x4 *>(xs + k) = *reinterpret_cast<const f32x4 *>(x + k);
+    // Loads return in issue order: the (small, cached) activation loads go first, the first step's
+    // weights right behind them, so staging the activations does not wait for HBM.
+    constexpr int XU = 4;  // covers K <= 4096 in one round
+    f32x4 xr[XU];
+#pragma unroll
+    for (int u = 0; u < XU; u++) {
+        const int k = (tid + u * QTHREADS) * 4;
+        xr[u] = k < K ? *reinterpret_cast<const f32x4 *>(x + k) : f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+    u32x4 tmp[U];
+    int step = blockIdx.x;
+    StepRange cur = step_range(step, rows_per_step, N, rowbytes);
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+        const int i = tid + u * QTHREADS;
+        tmp[u] = i < cur.nchunks ? ld128_stream(w + cur.abeg + (size_t)i * 16) : u32x4{0u, 0u, 0u, 0u};
+    }
+#pragma unroll
+    for (int u = 0; u < XU; u++) {
+        const int k = (tid + u * QTHREADS) * 4;
+        if (k < K) *reinterpret_cast<f32x4 *>(xs + k) = xr[u];
+    }
+    for (int k = (tid + XU * QTHREADS) * 4; k < K; k += QTHREADS * 4)  // longer rows
+        *reinterpret_cast<f32x4 *>(xs + k) = *reinterpret_cast<const f32x4 *>(x + k);
     __syncthreads();
     float xv[NXV][8], sxo[NXV];
     if (resident) {
 #pragma unroll
         for (int t = 0; t < NXV; t++) {
-            const int c = lane + t * WAVE;
-            if (c < nq) load_xv<QT>(xs, c, xv[t], sxo[t]);
+            const int c = min(lane + t * WAVE, nq - 1);  // lanes past the row end hold unused values
+            load_xv<QT>(xs, c, xv[t], sxo[t]);
         }
     }
 
-    for (int step = blockIdx.x; step < nsteps; step += gridDim.x) {
-        const int r0 = step * rows_per_step;
-        const int nrows = min(rows_per_step, N - r0);
-        const size_t beg = (size_t)r0 * rowbytes;
-        const size_t end = beg + (size_t)nrows * rowbytes;
-        const size_t abeg = beg & ~(size_t)15;
-        const int shift = (int)(beg - abeg);
-        const int nchunks = (int)((end - abeg + 15) / 16);
-
+    for (; step < nsteps; step += gridDim.x) {
         __syncthreads();  // previous step's readers are done with ws
-        for (int i0 = tid; i0 < nchunks; i0 += QTHREADS * U) {
-            u32x4 tmp[U];
 #pragma unroll
-            for (int u = 0; u < U; u++) {
-                const int i = i0 + u * QTHREADS;
-                const size_t off = abeg + (size_t)i * 16;
-                tmp[u] = (i < nchunks && off + 16 <= total_bytes) ? ld128_stream(w + off)
-                                                                  : u32x4{0u, 0u, 0u, 0u};
-            }
-#pragma unroll
-            for (int u = 0; u < U; u++) {
-                const int i = i0 + u * QTHREADS;
-                if (i < nchunks) {
-                    const size_t off = abeg + (size_t)i * 16;
-                    if (off + 16 <= total_bytes) {
-                        *reinterpret_cast<u32x4 *>(ws + (size_t)i * 16) = tmp[u];
-                    } else {  // last, partial chunk of the buffer: stay inside it
-                        for (int b = 0; b < 16; b++)
-                            ws[(size_t)i * 16 + b] = off + b < total_bytes ? w[off + b] : 0;
-                    }
-                }
-            }
+        for (int u = 0; u < U; u++) {
+            const int i = tid + u * QTHREADS;
+            if (i < cur.nchunks) *reinterpret_cast<u32x4 *>(ws + (size_t)i * 16) = tmp[u];
         }
         __syncthreads();
-
-        if (resident) {
-            // two rows per trip: independent chains for the LDS reads and the reductions
-            for (int lr = wave; lr < nrows; lr += 2 * QWAVES) {
-                const int lr1 = lr + QWAVES;
-                const bool two = lr1 < nrows;
-                const uint8_t *row0 = ws + shift + (size_t)lr * rowbytes;
-                const uint8_t *row1 = two ? row0 + (size_t)QWAVES * rowbytes : row0;
-                float a0 = 0.f, a1 = 0.f;
+        const StepRange now = cur;
+        // the next step's weights travel while this one is multiplied
+        if (step + (int)gridDim.x < nsteps) {
+            cur = step_range(step + gridDim.x, rows_per_step, N, rowbytes);
 #pragma unroll
-                for (int t = 0; t < NXV; t++) {
-                    const int c = lane + t * WAVE;
-                    if (c < nq) {
-                        a0 += quarter_dot<QT>(row0 + (c >> 2) * BB, c & 3, xv[t], sxo[t]);
-                        a1 += quarter_dot<QT>(row1 + (c >> 2) * BB, c & 3, xv[t], sxo[t]);
-                    }
-                }
-                a0 = wave_sum(a0);
-                a1 = wave_sum(a1);
-                if (lane == 0) {
-                    out[r0 + lr] = a0;
-                    if (two) out[r0 + lr1] = a1;
-                }
+            for (int u = 0; u < U; u++) {
+                const int i = tid + u * QTHREADS;
+                tmp[u] = i < cur.nchunks ? ld128_stream(w + cur.abeg + (size_t)i * 16) : u32x4{0u, 0u, 0u, 0u};
             }
+        }
+
+        const uint8_t *base = ws + now.shift;
+        if (resident) {
+            // up to four rows per trip: independent chains for the LDS reads and the reductions
+            int lr = wave;
+            for (; lr + 3 * QWAVES < now.nrows; lr += 4 * QWAVES)
+                rows_trip<QT, NXV, 4>(base, rowbytes, lr, lane, nq, xv, sxo, out + now.r0);
+            if (lr + QWAVES < now.nrows) {
+                rows_trip<QT, NXV, 2>(base, rowbytes, lr, lane, nq, xv, sxo, out + now.r0);
+                lr += 2 * QWAVES;
+            }
+            if (lr < now.nrows) rows_trip<QT, NXV, 1>(base, rowbytes, lr, lane, nq, xv, sxo, out + now.r0);
         } else {  // long rows: the activations of a column are re-read from LDS
             float acc[MAX_ROWS_PER_WAVE];
 #pragma unroll
@@ -180,15 +230,18 @@ __global__ __launch_bounds__(QTHREADS) void gemv_quant_kernel(
 #pragma unroll
                 for (int i = 0; i < MAX_ROWS_PER_WAVE; i++) {
                     const int lr = wave + QWAVES * i;
-                    if (lr < nrows)
-                        acc[i] += quarter_dot<QT>(ws + shift + (size_t)lr * rowbytes + (c >> 2) * BB, c & 3, xc, so);
+                    if (lr < now.nrows)
+                        {
+                        const uint8_t *blk = base + (size_t)lr * rowbytes + (c >> 2) * BB;
+                        acc[i] += quarter_dot<QT>(blk, blk + 2 + (c & 3) * BlockTraits<QT>::QUARTER, xc, so);
+                    }
                 }
             }
 #pragma unroll
             for (int i = 0; i < MAX_ROWS_PER_WAVE; i++) {
                 const int lr = wave + QWAVES * i;
                 const float v = wave_sum(acc[i]);
-                if (lane == 0 && lr < nrows) out[r0 + lr] = v;
+                if (lane == 0 && lr < now.nrows) out[now.r0 + lr] = v;
             }
         }
     }
@@ -230,29 +283,30 @@ int gemv_quant_launch(hm_ctx *ctx, const char *name, const float *d_x, const uin
     const size_t rowbytes = (size_t)(K / 32) * BB;
     const size_t x_bytes = (size_t)K * 4;
     const size_t lds_budget = 48 * 1024;
-    HM_REQUIRE(ctx, x_bytes + QWAVES * rowbytes + 32 <= 64 * 1024, "%s: K=%d too large for the LDS stage", name, K);
+    HM_REQUIRE(ctx, x_bytes + QWAVES * rowbytes + 32 <= 64 * 1024 && QWAVES * rowbytes + 32 <= (size_t)STAGE_BYTES,
+               "%s: K=%d too large for the LDS stage", name, K);
     // rows staged per step: as many as fit the LDS budget (at most 8 per wavefront), but few
     // enough that every CU gets a workgroup
     int rows = (int)((lds_budget - x_bytes) / rowbytes);
     rows = rows / QWAVES * QWAVES;
     if (rows < QWAVES) rows = QWAVES;
     if (rows > QWAVES * MAX_ROWS_PER_WAVE) rows = QWAVES * MAX_ROWS_PER_WAVE;
+    while (rows > QWAVES && (size_t)rows * rowbytes + 32 > (size_t)STAGE_BYTES) rows -= QWAVES;
     while (rows > QWAVES && (N + rows - 1) / rows < 2 * ctx->num_cus) rows -= QWAVES;
-    const size_t lds = x_bytes + (size_t)rows * rowbytes + 32;
+    const size_t lds = x_bytes + (size_t)rows * rowbytes + 32 + 16 * BB;  // slack: see rows_trip
     const int nsteps = (N + rows - 1) / rows;
     // persistent workgroups: a few per CU, each stages the activations once
     int wg_per_cu = (int)(120 * 1024 / lds);
     if (wg_per_cu < 1) wg_per_cu = 1;
     if (wg_per_cu > 6) wg_per_cu = 6;
     const int grid = nsteps < ctx->num_cus * wg_per_cu ? nsteps : ctx->num_cus * wg_per_cu;
-    const size_t total = (size_t)N * rowbytes;
     const int cpl = (K / 8 + WAVE - 1) / WAVE;
     for (int m = 0; m < M; m++) {
         const float *xm = d_x + (size_t)m * K;
         float *om = d_out + (size_t)m * N;
 #define HM_QUANT_CASE(C)                                                                                  \
     hipLaunchKernelGGL((gemv_quant_kernel<QT, C>), dim3(grid), dim3(QTHREADS), lds, ctx->stream, xm, d_w, \
-                       om, K, N, rows, total)
+                       om, K, N, rows)
         switch (cpl <= MAXC ? cpl : 0) {
             case 1: HM_QUANT_CASE(1); break;
             case 2: HM_QUANT_CASE(2); break;
