@@ -61,6 +61,18 @@ __device__ __forceinline__ void norm_rope_row(const float *__restrict__ src,
     o_hi = hi * c_hi + lo * s_hi;
 }
 
+// Sum over the LPR (8 or 16) adjacent lanes that share a cache row, on the DPP path; every lane of
+// the group receives the total.
+template <int LPR>
+__device__ __forceinline__ float row_group_sum(float v) {
+    static_assert(LPR == 8 || LPR == 16, "a cache row spans 8 or 16 lanes");
+    v += dpp_move<0xB1, 0xF>(v, 0.f);   // quad_perm [1,0,3,2]
+    v += dpp_move<0x4E, 0xF>(v, 0.f);   // quad_perm [2,3,0,1]
+    v += dpp_move<0x141, 0xF>(v, 0.f);  // row_half_mirror
+    if (LPR == 16) v += dpp_move<0x140, 0xF>(v, 0.f);  // row_mirror
+    return v;
+}
+
 template <int HD, int G>
 __global__ __launch_bounds__(ATT_THREADS) void gqa_decode_attn_kernel(
     const float *__restrict__ q, uint16_t *__restrict__ kcache, uint16_t *__restrict__ vcache,
@@ -71,7 +83,7 @@ __global__ __launch_bounds__(ATT_THREADS) void gqa_decode_attn_kernel(
     constexpr int RPI = WAVE / LPR;  // rows per wavefront instruction
     extern __shared__ float sm[];
     float *sc = sm;               // [G][chunk] scores, then probabilities; later the fold's (m,l)
-    float *red = sm + lds_front;  // [ATT_WAVES][G][HD]
+    float *red = sm + lds_front;  // [ATT_WAVES * RPI][G][HD]
     __shared__ float qs[G][HD];
     __shared__ float knew[HD], vnew[HD];
     __shared__ float s_m[G], s_l[G];
@@ -170,8 +182,7 @@ __global__ __launch_bounds__(ATT_THREADS) void gqa_decode_attn_kernel(
                 float p = 0.f;
 #pragma unroll
                 for (int e = 0; e < 8; e++) p = fmaf(kf[e], qv[gi][e], p);
-#pragma unroll
-                for (int off = LPR / 2; off >= 1; off >>= 1) p += __shfl_xor(p, off, WAVE);
+                p = row_group_sum<LPR>(p);
                 if (dl == 0 && live) sc[gi * chunk + row] = p * scale;
             }
         }
@@ -182,8 +193,7 @@ __global__ __launch_bounds__(ATT_THREADS) void gqa_decode_attn_kernel(
             float p = 0.f;
 #pragma unroll
             for (int e = 0; e < 8; e++) p = fmaf(knew[dl * 8 + e], qv[gi][e], p);
-#pragma unroll
-            for (int off = LPR / 2; off >= 1; off >>= 1) p += __shfl_xor(p, off, WAVE);
+            p = row_group_sum<LPR>(p);
             if (lane == 0) sc[gi * chunk + new_row] = p * scale;
         }
     }
@@ -237,21 +247,12 @@ __global__ __launch_bounds__(ATT_THREADS) void gqa_decode_attn_kernel(
             for (int e = 0; e < 8; e++) acc[gi][e] = fmaf(p, vnew[dl * 8 + e], acc[gi][e]);
         }
     }
-    // fold the RPI row-subgroups of the wavefront, then the waves of the workgroup
+    // every row-subgroup of every wavefront leaves its partial in LDS; summed below
 #pragma unroll
-    for (int gi = 0; gi < G; gi++)
-#pragma unroll
-        for (int e = 0; e < 8; e++) {
-            float v = acc[gi][e];
-#pragma unroll
-            for (int off = LPR; off < WAVE; off <<= 1) v += __shfl_xor(v, off, WAVE);
-            acc[gi][e] = v;
-        }
-    if (sub == 0) {
-#pragma unroll
-        for (int gi = 0; gi < G; gi++)
-#pragma unroll
-            for (int e = 0; e < 8; e++) red[((size_t)wave * G + gi) * HD + dl * 8 + e] = acc[gi][e];
+    for (int gi = 0; gi < G; gi++) {
+        float *dst = red + ((size_t)(wave * RPI + sub) * G + gi) * HD + dl * 8;
+        *reinterpret_cast<f32x4 *>(dst) = f32x4{acc[gi][0], acc[gi][1], acc[gi][2], acc[gi][3]};
+        *reinterpret_cast<f32x4 *>(dst + 4) = f32x4{acc[gi][4], acc[gi][5], acc[gi][6], acc[gi][7]};
     }
     __syncthreads();
 
@@ -261,7 +262,7 @@ __global__ __launch_bounds__(ATT_THREADS) void gqa_decode_attn_kernel(
     for (int i = tid; i < G * HD; i += ATT_THREADS) {
         float v = 0.f;
 #pragma unroll
-        for (int w = 0; w < ATT_WAVES; w++) v += red[(size_t)w * G * HD + i];
+        for (int w = 0; w < ATT_WAVES * RPI; w++) v += red[(size_t)w * G * HD + i];
         if (nsplit == 1) {
             const int gi = i / HD, d = i % HD;
             out[((size_t)b * H + kvhd * G + gi) * HD + d] = v / s_l[gi];
@@ -338,14 +339,21 @@ __global__ void kv_append_kernel(uint16_t *__restrict__ kc, uint16_t *__restrict
 
 template <int HD, int G>
 int launch_attn(hm_ctx *ctx, const AttnArgs &a, int nsplit, int chunk) {
-    // scores [G][chunk] + wave partials [4][G][HD]
+    // scores [G][chunk] + partials of every row-subgroup of every wavefront [4 * RPI][G][HD]
     const size_t front = (size_t)G * chunk;
-    const size_t lds = (front + (size_t)ATT_WAVES * G * HD) * sizeof(float);
+    const size_t lds = (front + (size_t)ATT_WAVES * (WAVE / (HD / 8)) * G * HD) * sizeof(float);
     const size_t pairs = (size_t)a.B * a.kvh;
     float *part_o = (float *)ctx->workspace;
     float *part_ml = part_o + pairs * nsplit * G * HD;
     AttnFuse f{a.qkv_raw, a.qw, a.kw, a.cos_tab, a.sin_tab, a.eps};
     if (a.phase != AttnArgs::FOLD_ONLY) {
+        static bool lds_limit_raised = false;  // per instantiation; large groups need more than 64 KiB
+        if (lds > 64 * 1024 && !lds_limit_raised) {
+            HM_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(&gqa_decode_attn_kernel<HD, G>),
+                                            hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024));
+            lds_limit_raised = true;
+        }
+        HM_REQUIRE(ctx, lds <= 96 * 1024, "gqa_decode_attn: LDS need %zu too large", lds);
         hipLaunchKernelGGL((gqa_decode_attn_kernel<HD, G>), dim3(nsplit, a.kvh, a.B), dim3(ATT_THREADS),
                            lds, ctx->stream, a.q, const_cast<uint16_t *>(a.kcache),
                            const_cast<uint16_t *>(a.vcache), a.out, part_o, part_ml, a.kvh, a.max_len,
