@@ -27,6 +27,7 @@ class HmTransformerConfig(C.Structure):
         ("tie_word_embeddings", C.c_int),
         ("rms_norm_eps", C.c_double),
         ("rope_theta", C.c_double),
+        ("attention_bias", C.c_int),
     ]
 
 

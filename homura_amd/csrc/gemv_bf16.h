@@ -21,6 +21,8 @@ struct GemvArgs {
     const float *norm_w = nullptr;             // [K]
     float eps = 0.f;
     float *resid_out = nullptr;                // [M][K]: receives r (written by one workgroup)
+    const float *bias = nullptr;               // [N]: out = W.x + bias (reference src/hf/emitter.rs:604-619);
+                                               // not with the paired epilogue
     const float *epilogue_residual = nullptr;  // [M][N]
     float *argmax_val = nullptr;               // [argmax_cap]
     int *argmax_idx = nullptr;                 // [argmax_cap]

@@ -208,6 +208,7 @@ __global__ __launch_bounds__(GEMV_THREADS) void gemv_bf16_nk_kernel(GemvArgs a) 
 #pragma unroll
                     for (int m = 0; m < MT; m++) {
                         float v = acc[r][m];
+                        if (a.bias) v = v + a.bias[row];
                         if (EPI == GEMV_EPI_RESIDUAL) v = a.epilogue_residual[(size_t)m * N + row] + v;
                         a.out[(size_t)m * N + row] = v;
                     }
@@ -359,6 +360,7 @@ __global__ __launch_bounds__(GEMV_THREADS) void gemv_bf16_nk_oneshot_kernel(Gemv
             const int row = row0 + r;
             if (lane == r && row < N) {
                 float v = acc[r];
+                if (a.bias) v = v + a.bias[row];
                 if (epi == GEMV_EPI_RESIDUAL) v = a.epilogue_residual[row] + v;
                 a.out[row] = v;
             }
@@ -458,8 +460,8 @@ int gemv_bf16_nk_launch(hm_ctx *ctx, GemvArgs a, int M, int epi) {
     HM_REQUIRE(ctx, M >= 1 && M <= 8, "gemv_bf16_nk: M=%d outside 1..8", M);
     HM_REQUIRE(ctx, (size_t)a.K * 4 <= 64 * 1024, "gemv_bf16_nk: K=%d too large for the LDS stage", a.K);
     HM_REQUIRE(ctx, ((uintptr_t)a.w % 16) == 0 && ((uintptr_t)a.x % 16) == 0, "gemv_bf16_nk: pointers must be 16-byte aligned");
-    if (epi == GEMV_EPI_SILU_MUL_PAIRS) HM_REQUIRE(ctx, a.N % 2 == 0, "gemv: paired epilogue needs even N");
-    if (epi == GEMV_EPI_ARGMAX) HM_REQUIRE(ctx, M == 1 && a.argmax_val && a.argmax_idx, "gemv: argmax epilogue needs M == 1 and candidate buffers");
+    if (epi == GEMV_EPI_SILU_MUL_PAIRS) HM_REQUIRE(ctx, a.N % 2 == 0 && !a.bias, "gemv: paired epilogue needs even N and no bias");
+    if (epi == GEMV_EPI_ARGMAX) HM_REQUIRE(ctx, M == 1 && a.argmax_val && a.argmax_idx && !a.bias, "gemv: argmax epilogue needs M == 1, candidate buffers and no bias");
     const int out_n = epi == GEMV_EPI_SILU_MUL_PAIRS ? a.N / 2 : a.N;
     int m0 = 0;
     while (m0 < M) {

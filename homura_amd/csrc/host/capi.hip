@@ -32,6 +32,7 @@ hm_model *hm_model_create(hm_ctx *ctx, const hm_transformer_config *cfg, int wei
     c.tie_word_embeddings = cfg->tie_word_embeddings != 0;
     c.rms_norm_eps = cfg->rms_norm_eps > 0 ? cfg->rms_norm_eps : 1e-6;
     c.rope_theta = cfg->rope_theta > 0 ? cfg->rope_theta : 10000.0;
+    c.attention_bias = cfg->attention_bias != 0;
     auto impl = HfModel::create(ctx, c, (DType)weight_dtype, has_qk_norm != 0);
     if (!impl) return nullptr;
     return new hm_model{ctx, std::move(impl)};

@@ -21,6 +21,7 @@ struct TransformerConfig {
     int max_position_embeddings = 2048;
     bool tie_word_embeddings = false;
     int head_dim_opt = 0;  // 0 => hidden_size / num_attention_heads
+    bool attention_bias = false;  // q/k/v_proj.bias present (reference src/hf/weights.rs:64-69)
 
     int kv_heads() const { return num_key_value_heads ? num_key_value_heads : num_attention_heads; }
     int head_dim() const { return head_dim_opt ? head_dim_opt : hidden_size / num_attention_heads; }
@@ -90,7 +91,7 @@ class HfModel {
     std::vector<Buffer> weight_bufs_;   // in weight_slots order, device resident
     std::vector<bool> weight_set_;
     // packed storage the bf16 weight slot buffers are views of
-    struct LayerPacked { Buffer qkv, o, gate_up, down; };
+    struct LayerPacked { Buffer qkv, o, gate_up, down, qkv_bias; };  // qkv_bias: f32 [q_dim + 2 kv_dim]
     std::vector<LayerPacked> packed_;
     Buffer lm_head_packed_;
     Buffer rope_cos_, rope_sin_;        // [max_position][head_dim] f32

@@ -57,7 +57,7 @@ std::unique_ptr<HfModel> HfModel::create(hm_ctx *ctx, const TransformerConfig &c
     m->has_qk_norm_ = has_qk_norm;
 
     // Slot order = TransformerWeights::to_slot_buffers (src/hf/weights.rs:63-116) for bf16,
-    // to_slot_buffers_quant (:136-183) for block-quantised projections; models without bias.
+    // to_slot_buffers_quant (:136-183) for block-quantised projections.
     const int64_t hidden = cfg.hidden_size, inter = cfg.intermediate_size, vocab = cfg.vocab_size;
     const int64_t qd = cfg.q_dim(), kvd = cfg.kv_dim(), hd = cfg.head_dim();
     const bool quant = dtype_is_quantized(weight_dtype);
@@ -78,8 +78,11 @@ std::unique_ptr<HfModel> HfModel::create(hm_ctx *ctx, const TransformerConfig &c
         const std::string p = "model.layers." + std::to_string(l) + ".";
         f32_vec(p + "input_layernorm.weight", hidden);
         proj(p + "self_attn.q_proj.weight", hidden, qd);
+        if (cfg.attention_bias) f32_vec(p + "self_attn.q_proj.bias", qd);
         proj(p + "self_attn.k_proj.weight", hidden, kvd);
+        if (cfg.attention_bias) f32_vec(p + "self_attn.k_proj.bias", kvd);
         proj(p + "self_attn.v_proj.weight", hidden, kvd);
+        if (cfg.attention_bias) f32_vec(p + "self_attn.v_proj.bias", kvd);
         if (has_qk_norm) {
             f32_vec(p + "self_attn.q_norm.weight", hd);
             f32_vec(p + "self_attn.k_norm.weight", hd);
@@ -175,6 +178,21 @@ int HfModel::set_weight(int slot, const void *h_data, size_t bytes) {
         if (rc != HM_OK) return rc;
         weight_bufs_[slot] = Buffer::view(lm_head_packed_.ptr(), bytes, {info.dim1, info.dim0},
                                           {info.dim0, 1}, DType::F32);
+        weight_set_[slot] = true;
+        return HM_OK;
+    }
+
+    if (ends_with("_proj.bias")) {
+        // q|k|v biases of a layer sit back to back like the rows they belong to
+        const size_t p0 = std::string("model.layers.").size();
+        LayerPacked &lp = packed_[std::atoi(nm.c_str() + p0)];
+        if (!lp.qkv_bias) lp.qkv_bias = Buffer::alloc(ctx_, {qd + 2 * kvd}, DType::F32);
+        if (!lp.qkv_bias) return HM_ERR_OOM;
+        const size_t off = ends_with("q_proj.bias") ? 0 : ends_with("k_proj.bias") ? (size_t)qd : (size_t)(qd + kvd);
+        float *dst = lp.qkv_bias.as<float>() + off;
+        int rc = hm_upload(ctx_, dst, h_data, bytes);
+        if (rc != HM_OK) return rc;
+        weight_bufs_[slot] = Buffer::view(dst, bytes, {info.dim0}, {1}, DType::F32);
         weight_set_[slot] = true;
         return HM_OK;
     }
@@ -287,7 +305,7 @@ int HfModel::finalize(int max_seq_len) {
 
 // ── bf16 plan ────────────────────────────────────────────────────────────────
 // Slot order and step list follow assign_transformer_slots / emit_transformer_plan
-// (reference src/hf/emitter.rs:74-498, :902-1014) for a model without biases.
+// (reference src/hf/emitter.rs:74-498, :902-1014).
 int HfModel::emit_transformer_plan() {
     const TransformerConfig c = cfg_;
     const int64_t hidden = c.hidden_size, inter = c.intermediate_size, vocab = c.vocab_size;
@@ -315,7 +333,7 @@ int HfModel::emit_transformer_plan() {
     const size_t embed_out = alloc({1, D, hidden}, DType::F32, "embed_out");
 
     struct LayerSlots {
-        size_t hidden_in, input_ln, q_w, k_w, v_w, q_norm, k_norm, o_w, post_ln, gate_w, up_w, down_w;
+        size_t hidden_in, input_ln, q_w, k_w, v_w, q_b, k_b, v_b, q_norm, k_norm, o_w, post_ln, gate_w, up_w, down_w;
         size_t q, k, v, past_k, past_v, present_k, present_v, attn_out, hidden_out;
     };
     std::vector<LayerSlots> ls(L);
@@ -329,9 +347,14 @@ int HfModel::emit_transformer_plan() {
             return slot;
         };
         s.input_ln = w({hidden}, DType::F32, "input_ln");
+        const bool bias = c.attention_bias;
+        s.q_b = s.k_b = s.v_b = (size_t)-1;
         s.q_w = w({hidden, qd}, DType::BF16, "q_w");
+        if (bias) s.q_b = w({qd}, DType::F32, "q_b");
         s.k_w = w({hidden, kvd}, DType::BF16, "k_w");
+        if (bias) s.k_b = w({kvd}, DType::F32, "k_b");
         s.v_w = w({hidden, kvd}, DType::BF16, "v_w");
+        if (bias) s.v_b = w({kvd}, DType::F32, "v_b");
         s.q_norm = s.k_norm = (size_t)-1;
         if (qkn) {
             s.q_norm = w({hd}, DType::F32, "q_norm");
@@ -410,11 +433,13 @@ int HfModel::emit_transformer_plan() {
             DeviceLaunch g1;
             g1.name = "gemv_bf16[qkv]";
             g1.bytes_fixed = gemv_bytes(hidden, qd + 2 * kvd, qd + 2 * kvd) + hidden * 4.0;
+            const size_t q_bias_slot = s.q_b;
             g1.fn = [=](const StepContext &sc) -> int {
                 const auto &in = sc.step.input_slots;
                 GemvArgs g;
                 g.x = sc.pool[in[0]]->as<float>();
                 g.w = sc.pool[in[2]]->as<uint16_t>();  // q|k|v rows are adjacent in the packed buffer
+                if (q_bias_slot != (size_t)-1) g.bias = sc.pool[q_bias_slot]->as<float>();  // and so are the biases
                 g.out = sc.pool[sc.step.output_slots[0]]->as<float>();  // q|k|v outputs adjacent too
                 g.K = (int)hidden;
                 g.N = (int)(qd + 2 * kvd);
@@ -424,7 +449,15 @@ int HfModel::emit_transformer_plan() {
             };
             k.launches.push_back(std::move(g1));
             kernels.push_back(std::move(k));
-            std::vector<size_t> in{s.hidden_in, s.input_ln, s.q_w, s.k_w, s.v_w, cos_s, sin_s};
+            // h, ln_w, q_w, [q_b], k_w, [k_b], v_w, [v_b], cos, sin, [q_norm_w, k_norm_w]
+            std::vector<size_t> in{s.hidden_in, s.input_ln, s.q_w};
+            if (s.q_b != (size_t)-1) in.push_back(s.q_b);
+            in.push_back(s.k_w);
+            if (s.k_b != (size_t)-1) in.push_back(s.k_b);
+            in.push_back(s.v_w);
+            if (s.v_b != (size_t)-1) in.push_back(s.v_b);
+            in.push_back(cos_s);
+            in.push_back(sin_s);
             if (qkn) {
                 in.push_back(s.q_norm);
                 in.push_back(s.k_norm);
@@ -638,7 +671,7 @@ int HfModel::emit_transformer_plan_quant() {
     const size_t embed_out = alloc({1, D, hidden}, DType::F32, "embed_out");
 
     struct LS {
-        size_t hidden_in, input_ln, q_w, k_w, v_w, q_norm, k_norm, o_w, post_ln, gate_w, up_w, down_w;
+        size_t hidden_in, input_ln, q_w, k_w, v_w, q_b, k_b, v_b, q_norm, k_norm, o_w, post_ln, gate_w, up_w, down_w;
         size_t past_k, past_v, present_k, present_v;
         size_t normed, q_out, k_out, v_out, q, k_bhsd, v_bhsd, attn_body, attn_out, residual, post_normed,
             gate_out, up_out, silu, down_out, hidden_out;
@@ -656,9 +689,14 @@ int HfModel::emit_transformer_plan_quant() {
         };
         // quantised weights are flat byte buffers (reference src/hf/emitter_quant.rs:213-222)
         s.input_ln = w({hidden}, DType::F32, "input_ln");
+        const bool bias = c.attention_bias;
+        s.q_b = s.k_b = s.v_b = (size_t)-1;
         s.q_w = w({qbytes(hidden, qd)}, wdt, "q_w");
+        if (bias) s.q_b = w({qd}, DType::F32, "q_b");
         s.k_w = w({qbytes(hidden, kvd)}, wdt, "k_w");
+        if (bias) s.k_b = w({kvd}, DType::F32, "k_b");
         s.v_w = w({qbytes(hidden, kvd)}, wdt, "v_w");
+        if (bias) s.v_b = w({kvd}, DType::F32, "v_b");
         s.q_norm = s.k_norm = (size_t)-1;
         if (qkn) {
             s.q_norm = w({hd}, DType::F32, "q_norm");
@@ -777,6 +815,22 @@ int HfModel::emit_transformer_plan_quant() {
             CompiledKernel k;
             k.ops_label = qkn ? "PostQKV+QKNorm+RoPE" : "PostQKV+RoPE";
             std::vector<size_t> in{s.q_out, s.k_out, s.v_out, cos_s, sin_s};
+            if (s.q_b != (size_t)-1) {
+                // the bias add of this reference kernel (src/hf/emitter_quant.rs:836-850): one launch
+                // over the adjacent q|k|v rows and the adjacent biases
+                in.push_back(s.q_b);
+                in.push_back(s.k_b);
+                in.push_back(s.v_b);
+                DeviceLaunch l;
+                l.name = "qkv_bias_add";
+                l.bytes_fixed = (qd + 2 * kvd) * 4.0 * 3;
+                const size_t raw = s.q_out, qb = s.q_b;
+                l.fn = [=](const StepContext &sc) -> int {
+                    float *x = sc.pool[raw]->as<float>();
+                    return hm_add(sc.ctx, x, sc.pool[qb]->as<float>(), x, (size_t)(qd + 2 * kvd));
+                };
+                k.launches.push_back(std::move(l));
+            }
             if (qkn) {
                 in.push_back(s.q_norm);
                 in.push_back(s.k_norm);

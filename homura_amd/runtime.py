@@ -209,6 +209,7 @@ class TransformerConfig:
     max_position_embeddings: int = 2048
     tie_word_embeddings: bool = False
     head_dim: int | None = None
+    attention_bias: bool = False   # q/k/v_proj.bias present (reference src/hf/weights.rs:64-69)
 
     def kv_heads(self) -> int:
         return self.num_key_value_heads or self.num_attention_heads
@@ -224,7 +225,7 @@ class TransformerConfig:
             self.hidden_size, self.intermediate_size, self.num_attention_heads,
             self.num_hidden_layers, self.num_key_value_heads or 0, self.vocab_size,
             self.head_dim or 0, self.max_position_embeddings, int(self.tie_word_embeddings),
-            self.rms_norm_eps, self.rope_theta)
+            self.rms_norm_eps, self.rope_theta, int(self.attention_bias))
 
 
 class HfModel:

@@ -23,6 +23,12 @@ TINY = TransformerConfig(
     vocab_size=1000, num_key_value_heads=2, head_dim=64, rms_norm_eps=1e-6, rope_theta=1e6,
     max_position_embeddings=512, tie_word_embeddings=True)
 
+# Qwen2.5-like: Q/K/V biases, no QK-norm, GQA 7:1 as in Qwen2.5-0.5B (14 q heads, 2 kv heads)
+TINY_QWEN2 = TransformerConfig(
+    hidden_size=448, intermediate_size=608, num_attention_heads=7, num_hidden_layers=2,
+    vocab_size=512, num_key_value_heads=1, head_dim=64, rms_norm_eps=1e-6, rope_theta=1e6,
+    max_position_embeddings=512, tie_word_embeddings=True, attention_bias=True)
+
 # TinyLlama-like proportions (MHA:GQA 4:1, no QK-norm, untied head) for the quantised plan
 TINY_LLAMA = TransformerConfig(
     hidden_size=256, intermediate_size=704, num_attention_heads=8, num_hidden_layers=2,
@@ -50,6 +56,11 @@ def synth_weights(cfg: TransformerConfig, seed: int, weight_dtype: int = DTYPE_B
         cursor[0] += n
         return (1.0 + a).astype(np.float32)
 
+    def bias_vec(n):
+        a = synth.normal_f32(seed ^ 0xB1A5, n, 0.5, first=cursor[0])
+        cursor[0] += n
+        return a.astype(np.float32)
+
     qseed = [seed * 7919 + 1]
 
     def proj(K, N):
@@ -68,8 +79,14 @@ def synth_weights(cfg: TransformerConfig, seed: int, weight_dtype: int = DTYPE_B
         p = f"model.layers.{l}."
         out.append((p + "input_layernorm.weight", norm_vec(hidden)))
         out.append((p + "self_attn.q_proj.weight", proj(hidden, qd)))
+        if cfg.attention_bias:
+            out.append((p + "self_attn.q_proj.bias", bias_vec(qd)))
         out.append((p + "self_attn.k_proj.weight", proj(hidden, kvd)))
+        if cfg.attention_bias:
+            out.append((p + "self_attn.k_proj.bias", bias_vec(kvd)))
         out.append((p + "self_attn.v_proj.weight", proj(hidden, kvd)))
+        if cfg.attention_bias:
+            out.append((p + "self_attn.v_proj.bias", bias_vec(kvd)))
         if has_qk_norm:
             out.append((p + "self_attn.q_norm.weight", norm_vec(hd)))
             out.append((p + "self_attn.k_norm.weight", norm_vec(hd)))

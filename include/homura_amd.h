@@ -183,6 +183,8 @@ typedef struct {
     int tie_word_embeddings;
     double rms_norm_eps;
     double rope_theta;
+    int attention_bias;      /* Q/K/V projections carry a bias (Qwen2-style); the reference reads this
+                                off the checkpoint (src/hf/weights.rs:64-69) */
 } hm_transformer_config;
 
 #define HM_DTYPE_F32 0

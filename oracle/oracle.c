@@ -601,7 +601,7 @@ typedef struct {
 } orc_config;
 
 /* Weight pointers in the order of TransformerWeights::to_slot_buffers
- * (src/hf/weights.rs:63-116; no-bias models): embed, per layer {input_ln, q, k, v,
+ * (src/hf/weights.rs:63-116): embed, per layer {input_ln, q, [q_bias], k, [k_bias], v, [v_bias],
  * [q_norm, k_norm], o, post_ln, gate, up, down}, final_norm, lm_head.
  * bf16 projections are [K][N] (transposed at load, src/hf/weights.rs:225-261);
  * quantised ones are raw [N][K/32] blocks (src/hf/weights.rs:136-194).
@@ -609,6 +609,7 @@ typedef struct {
 typedef struct {
     const float *input_ln, *q_norm, *k_norm, *post_ln;
     const void *q, *k, *v, *o, *gate, *up, *down;
+    const float *q_bias, *k_bias, *v_bias; /* NULL for models without Q/K/V bias */
 } orc_layer_weights;
 
 typedef struct {
@@ -660,6 +661,24 @@ ORC_API void orc_model_set_layer(orc_model *m, int l, const float *input_ln, con
     w->gate = gate;
     w->up = up;
     w->down = down;
+}
+
+/* Q/K/V projection biases (f32, Qwen2-style checkpoints): slots q,[qb],k,[kb],v,[vb] of
+ * to_slot_buffers (src/hf/weights.rs:75-86). */
+ORC_API void orc_model_set_layer_bias(orc_model *m, int l, const float *q_bias, const float *k_bias,
+                                      const float *v_bias) {
+    orc_layer_weights *w = &m->layers[l];
+    w->q_bias = q_bias;
+    w->k_bias = k_bias;
+    w->v_bias = v_bias;
+}
+
+/* q = emit_add(q, bias): the bias row broadcast over the sequence (src/hf/emitter.rs:604-619;
+ * quantised plan: emit_post_qkv_kernel, src/hf/emitter_quant.rs:802-912). */
+static void add_bias(float *x, const float *bias, int S, int n) {
+    if (!bias) return;
+    for (int s = 0; s < S; s++)
+        for (int i = 0; i < n; i++) x[(size_t)s * n + i] = x[(size_t)s * n + i] + bias[i];
 }
 
 ORC_API void orc_model_attach_kv(orc_model *m, orc_kv_cache *kv) { m->kv = kv; }
@@ -753,6 +772,9 @@ ORC_API int orc_model_run_kv(orc_model *m, const int64_t *ids, int S, float *log
         proj(m, m->normed, w->q, m->q, S, c->hidden, qd);
         proj(m, m->normed, w->k, m->k, S, c->hidden, kvd);
         proj(m, m->normed, w->v, m->v, S, c->hidden, kvd);
+        add_bias(m->q, w->q_bias, S, qd);
+        add_bias(m->k, w->k_bias, S, kvd);
+        add_bias(m->v, w->v_bias, S, kvd);
         if (c->has_qk_norm) {
             if (quant) {
                 orc_rms_norm_f64mean(m->q, w->q_norm, m->q, S * c->heads, hd, c->eps);

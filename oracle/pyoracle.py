@@ -84,6 +84,7 @@ def load() -> C.CDLL:
         "orc_model_new": (_P, [C.POINTER(OrcConfig)]),
         "orc_model_set_global": (None, [_P, _P, _P, _P, _P, _P, _I]),
         "orc_model_set_layer": (None, [_P, _I] + [_P] * 11),
+        "orc_model_set_layer_bias": (None, [_P, _I, _P, _P, _P]),
         "orc_model_attach_kv": (None, [_P, _P]),
         "orc_model_free": (None, [_P]),
         "orc_model_run_kv": (_I, [_P, _P, _I, _P]),
@@ -323,6 +324,10 @@ class Model:
                 self._hold(o), self._hold(_f32(post_ln)), self._hold(gate), self._hold(up),
                 self._hold(down)]
         self.lib.orc_model_set_layer(self.h, l, *args)
+
+    def set_layer_bias(self, l, q_bias, k_bias, v_bias):
+        self.lib.orc_model_set_layer_bias(self.h, l, self._hold(_f32(q_bias)), self._hold(_f32(k_bias)),
+                                          self._hold(_f32(v_bias)))
 
     def run_kv(self, ids):
         ids = np.ascontiguousarray(ids, np.int64).reshape(-1)

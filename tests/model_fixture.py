@@ -33,6 +33,9 @@ def build_oracle_model(cfg, weights, max_seq_len, weight_dtype=DTYPE_BF16, has_q
                     w[p + "self_attn.o_proj.weight"], w[p + "post_attention_layernorm.weight"],
                     w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"],
                     w[p + "mlp.down_proj.weight"])
+        if cfg.attention_bias:
+            m.set_layer_bias(l, w[p + "self_attn.q_proj.bias"], w[p + "self_attn.k_proj.bias"],
+                             w[p + "self_attn.v_proj.bias"])
     return m
 
 

@@ -177,3 +177,31 @@ def test_quantised_plan_against_oracle(ctx, wdt, name):
     names = [s[0] for s in gm.weight_slots()]
     assert names == [n for n, _ in weights]
     gm.close()
+
+
+@pytest.mark.parametrize("wdt,name", [(1, "bf16"), (2, "q8_0")])
+def test_qkv_bias_model_against_oracle(ctx, wdt, name):
+    """Qwen2-style checkpoint: Q/K/V biases (slots q,[qb],k,[kb],v,[vb] of the reference's
+    to_slot_buffers), no QK-norm, GQA group of 7, head_dim 64."""
+    cfg = synth_model.TINY_QWEN2
+    weights = synth_model.synth_weights(cfg, 77, wdt, has_qk_norm=False)
+    assert any(n.endswith("q_proj.bias") for n, _ in weights)
+    gm = synth_model.build_model(ctx, cfg, weights, 96, wdt, has_qk_norm=False)
+    om = mf.build_oracle_model(cfg, weights, 96, wdt, has_qk_norm=False)
+    assert [s[0] for s in gm.weight_slots()] == [n for n, _ in weights]
+    kv = synth_model.synth_kv(cfg, 8, 21)
+    gm.init_kv_cache(kv, 21)
+    mf.oracle_init_kv(om, kv)
+    ids = synth.token_ids(6, 5, cfg.vocab_size)
+    got = gm.run_kv(ids)
+    want = np.concatenate([om.run_kv(ids[i:i + 1]) for i in range(5)])
+    for i in range(5):
+        assert mf.rel_err(got[i], want[i]) < 1e-2, f"{name} position {i}"
+    want_t, margins = om.generate_greedy(ids[:2], 24)
+    say(f"bias model {name}: min margin {margins.min():.3e}")
+    assert np.array_equal(gm.generate_greedy(ids[:2], 24), want_t)
+    gm.set_graph(True)
+    gm.init_kv_cache(kv, 21)
+    gm.run_kv(ids)
+    assert np.array_equal(gm.generate_greedy(ids[:2], 24), want_t)
+    gm.close()

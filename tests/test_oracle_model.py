@@ -92,16 +92,18 @@ def test_oracle_batched_prefill_equals_token_by_token():
         a.run_kv(np.zeros(64, np.int64))  # would overflow the cache
 
 
-def test_oracle_step_against_numpy_fp64():
-    """An independent numpy/float64 forward of one decode step (textbook HF Qwen3 block) against
-    the C oracle: a dropped residual, a missing norm weight, a swapped gate/up or a wrong head
-    mapping would all show up here."""
-    cfg = synth_model.TINY
-    W = dict(synth_model.synth_weights(cfg, 99))
+@pytest.mark.parametrize("which", ["qwen3_qknorm", "qwen2_bias"])
+def test_oracle_step_against_numpy_fp64(which):
+    """An independent numpy/float64 forward of one decode step (textbook HF Qwen3 / Qwen2 block)
+    against the C oracle: a dropped residual, a missing norm weight or bias, a swapped gate/up or a
+    wrong head mapping would all show up here."""
+    qkn = which == "qwen3_qknorm"
+    cfg = synth_model.TINY if qkn else synth_model.TINY_QWEN2
+    W = dict(synth_model.synth_weights(cfg, 99, has_qk_norm=qkn))
     hd, H, kvh = cfg.get_head_dim(), cfg.num_attention_heads, cfg.kv_heads()
     past = 11
     kv = synth_model.synth_kv(cfg, 5, past)
-    om = mf.build_oracle_model(cfg, list(W.items()), 32)
+    om = mf.build_oracle_model(cfg, list(W.items()), 32, has_qk_norm=qkn)
     mf.oracle_init_kv(om, kv)
     tok = 123
     got = om.run_kv([tok])[0]
@@ -117,11 +119,13 @@ def test_oracle_step_against_numpy_fp64():
     for l in range(cfg.num_hidden_layers):
         p = f"model.layers.{l}."
         n = rms(h, f(W[p + "input_layernorm.weight"]))
-        q = (n @ f(W[p + "self_attn.q_proj.weight"])).reshape(H, hd)
-        k = (n @ f(W[p + "self_attn.k_proj.weight"])).reshape(kvh, hd)
-        v = (n @ f(W[p + "self_attn.v_proj.weight"])).reshape(kvh, hd)
-        q = rms(q, f(W[p + "self_attn.q_norm.weight"]))
-        k = rms(k, f(W[p + "self_attn.k_norm.weight"]))
+        q, k, v = (n @ f(W[p + f"self_attn.{x}_proj.weight"]) for x in "qkv")
+        if cfg.attention_bias:
+            q, k, v = (t + f(W[p + f"self_attn.{x}_proj.bias"]) for t, x in zip((q, k, v), "qkv"))
+        q, k, v = q.reshape(H, hd), k.reshape(kvh, hd), v.reshape(kvh, hd)
+        if qkn:
+            q = rms(q, f(W[p + "self_attn.q_norm.weight"]))
+            k = rms(k, f(W[p + "self_attn.k_norm.weight"]))
         q, k = q * cos + rot(q) * sin, k * cos + rot(k) * sin
         K = np.concatenate([kv[2 * l][0].astype(np.float64), bf(k)[:, None, :]], 1)   # [kvh, past+1, hd]
         V = np.concatenate([kv[2 * l + 1][0].astype(np.float64), bf(v)[:, None, :]], 1)
