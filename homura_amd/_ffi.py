@@ -75,6 +75,9 @@ SIGNATURES = {
     "hm_dequant_q4_0": (_I, [_P, _P, _P, _SZ]),
     "hm_gemm_bf16": (_I, [_P, _P, _P, _P, _I, _I, _I]),
     "hm_gemm_bf16_nk": (_I, [_P, _P, _P, _P, _I, _I, _I]),
+    "hm_ciface_bind_transformer": (_I, [_P, _P, _I]),
+    "hm_ciface_num_kernels": (_I, []),
+    "hm_ciface_unbind": (None, []),
     "hm_kv_append": (_I, [_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I]),
     "hm_gqa_decode_attn": (_I, [_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, C.c_float]),
     "hm_rmsnorm": (_I, [_P, _P, _P, _P, _I, _I, C.c_float]),

@@ -1,0 +1,280 @@
+// The reference's own kernel ABI on top of the GPU kernels: symbols
+// `_mlir__mlir_ciface_k{idx}(void **args)` that take memref descriptors, exactly what
+// CompiledGraph::load_from_handle resolves with dlsym and run_with_output_bufs calls
+// (reference src/runtime.rs:779-824, :930-1037; descriptor layout :654-698).
+//
+// With Buffers that hold device memory, the reference's ExecutionPlan can dlopen this library
+// in place of its compiled CPU kernels. hm_ciface_bind_transformer() records which fused kernel
+// each index stands for, in the order emit_transformer_plan numbers them (src/hf/emitter.rs:
+// 902-1014): k0 Embed; per layer k(3l+1) QKV(+QK-norm)+RoPE, k(3l+2) Attn, k(3l+3) MLP; then
+// LMHead. Arguments follow each emitter's input order, outputs after inputs.
+//
+// This is the compatibility path: weights are consumed in the reference's [K,N] layout, the KV
+// views are the reference's f32 cache (copied to a bf16 scratch cache per call), and every
+// reference kernel becomes several launches. The model-level API is the fast path.
+#include <cmath>
+#include <cstdio>
+#include <vector>
+
+#include "../hm_common.h"
+
+namespace {
+
+enum class Kind { Embed, Qkv, Attn, Mlp, LmHead };
+
+struct Bound {
+    hm_ctx *ctx = nullptr;
+    hm_transformer_config cfg{};
+    bool qk_norm = false;
+    int kv_heads = 0, head_dim = 0, q_dim = 0, kv_dim = 0;
+    std::vector<Kind> kinds;
+} g_bound;
+
+// One rank-N memref argument: args[i] points at a pointer to the descriptor bytes.
+struct MemRef {
+    char *data = nullptr;
+    const int64_t *sizes = nullptr, *strides = nullptr;
+    template <class T>
+    T *as() const { return reinterpret_cast<T *>(data); }
+};
+MemRef memref(void **args, int i, int rank) {
+    char *desc = *reinterpret_cast<char **>(args[i]);
+    MemRef m;
+    int64_t offset;
+    std::memcpy(&m.data, desc + 8, 8);  // aligned pointer
+    std::memcpy(&offset, desc + 16, 8);
+    (void)offset;  // always 0 (reference src/runtime.rs:689)
+    m.sizes = reinterpret_cast<const int64_t *>(desc + 24);
+    m.strides = m.sizes + rank;
+    return m;
+}
+
+// The reference's kernels return void: a failure is recorded on the context and reported here.
+void report(int idx, int rc) {
+    if (rc == HM_OK) return;
+    std::fprintf(stderr, "homura_amd: _mlir__mlir_ciface_k%d failed (%d): %s\n", idx, rc,
+                 g_bound.ctx ? hm_last_error(g_bound.ctx) : "no transformer bound");
+}
+
+#define TRY(expr)                 \
+    do {                          \
+        int _rc = (expr);         \
+        if (_rc != HM_OK) return _rc; \
+    } while (0)
+
+// Scratch carved from the context workspace, 256-byte aligned pieces. The kernels called from here
+// keep their own partials (split-K sums, attention splits, argmax segments: a few MiB at most at
+// the sizes accepted here) at the start of the workspace, so the first KERNEL_RESERVE bytes are
+// left to them.
+constexpr size_t KERNEL_RESERVE = (size_t)16 << 20;
+struct Scratch {
+    char *p;
+    size_t left;
+    explicit Scratch(hm_ctx *ctx)
+        : p((char *)ctx->workspace + KERNEL_RESERVE),
+          left(ctx->workspace_bytes > KERNEL_RESERVE ? ctx->workspace_bytes - KERNEL_RESERVE : 0) {}
+    template <class T>
+    T *take(size_t n) {
+        const size_t bytes = (n * sizeof(T) + 255) & ~(size_t)255;
+        if (bytes > left) return nullptr;
+        T *r = reinterpret_cast<T *>(p);
+        p += bytes;
+        left -= bytes;
+        return r;
+    }
+};
+
+__global__ void kv_view_to_bf16_kernel(const float *__restrict__ src, int64_t head_stride, int64_t row_stride,
+                                       uint16_t *__restrict__ dst, int rows, int hd, size_t total) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= total) return;
+    const int d = (int)(i % hd);
+    const size_t r = i / hd;
+    const int row = (int)(r % rows);
+    const size_t head = r / rows;
+    dst[i] = f32_to_bf16_rne_dev(src[head * head_stride + (size_t)row * row_stride + d]);
+}
+
+int need_single_token(hm_ctx *ctx, int64_t seq, const char *what) {
+    if (seq == 1) return HM_OK;
+    return hm_set_error(ctx, HM_ERR_INVALID, "%s: the memref entry points take one token per call (seq = %lld)",
+                        what, (long long)seq);
+}
+
+// emit_embed_kernel (src/hf/emitter.rs:506-537): ids [1,S] i64, table [V,H] f32 -> [1,S,H]
+int run_embed(void **a) {
+    const Bound &b = g_bound;
+    const MemRef ids = memref(a, 0, 2), table = memref(a, 1, 2), out = memref(a, 2, 3);
+    return hm_embed(b.ctx, ids.as<int64_t>(), table.as<float>(), out.as<float>(), (int)ids.sizes[1],
+                    b.cfg.vocab_size, b.cfg.hidden_size);
+}
+
+// emit_qkv_kernel (src/hf/emitter.rs:549-673): h, ln_w, q_w, [q_b], k_w, [k_b], v_w, [v_b], cos, sin,
+// [q_norm_w, k_norm_w] -> q [1,S,H,hd], k [1,kvh,S,hd], v [1,kvh,S,hd]
+int run_qkv(void **a) {
+    const Bound &b = g_bound;
+    hm_ctx *ctx = b.ctx;
+    const int hidden = b.cfg.hidden_size, bias = b.cfg.attention_bias ? 1 : 0;
+    int i = 0;
+    const MemRef h = memref(a, i++, 3), ln = memref(a, i++, 1), qw = memref(a, i++, 2);
+    const float *qb = bias ? memref(a, i++, 1).as<float>() : nullptr;
+    const MemRef kw = memref(a, i++, 2);
+    const float *kb = bias ? memref(a, i++, 1).as<float>() : nullptr;
+    const MemRef vw = memref(a, i++, 2);
+    const float *vb = bias ? memref(a, i++, 1).as<float>() : nullptr;
+    const MemRef cosv = memref(a, i++, 2), sinv = memref(a, i++, 2);
+    const float *qn = nullptr, *kn = nullptr;
+    if (b.qk_norm) {
+        qn = memref(a, i++, 1).as<float>();
+        kn = memref(a, i++, 1).as<float>();
+    }
+    const MemRef q = memref(a, i++, 4), k = memref(a, i++, 4), v = memref(a, i++, 4);
+    TRY(need_single_token(ctx, h.sizes[1], "QKV kernel"));
+    Scratch s(ctx);
+    float *normed = s.take<float>(hidden);
+    if (!normed) return hm_set_error(ctx, HM_ERR_OOM, "QKV kernel: workspace too small");
+    TRY(hm_rmsnorm(ctx, h.as<float>(), ln.as<float>(), normed, 1, hidden, (float)b.cfg.rms_norm_eps));
+    TRY(hm_gemv_bf16(ctx, normed, qw.as<uint16_t>(), q.as<float>(), 1, hidden, b.q_dim));
+    TRY(hm_gemv_bf16(ctx, normed, kw.as<uint16_t>(), k.as<float>(), 1, hidden, b.kv_dim));
+    TRY(hm_gemv_bf16(ctx, normed, vw.as<uint16_t>(), v.as<float>(), 1, hidden, b.kv_dim));
+    if (bias) {
+        TRY(hm_add(ctx, q.as<float>(), qb, q.as<float>(), (size_t)b.q_dim));
+        TRY(hm_add(ctx, k.as<float>(), kb, k.as<float>(), (size_t)b.kv_dim));
+        TRY(hm_add(ctx, v.as<float>(), vb, v.as<float>(), (size_t)b.kv_dim));
+    }
+    // with one token the BSHD rows and the BHSD outputs coincide
+    return hm_qknorm_rope(ctx, q.as<float>(), k.as<float>(), qn, kn, cosv.as<float>(), sinv.as<float>(), 1,
+                          b.cfg.num_attention_heads, b.kv_heads, b.head_dim, (float)b.cfg.rms_norm_eps);
+}
+
+// emit_attention_kernel (src/hf/emitter.rs:683-758): q [1,S,H,hd], k/v views [1,kvh,T,hd] f32 with the
+// cache's max-length strides (src/runtime.rs:610-615), mask [1,1,S,T], o_w [q_dim,hidden] -> [1,S,hidden]
+int run_attn(void **a) {
+    const Bound &b = g_bound;
+    hm_ctx *ctx = b.ctx;
+    const MemRef q = memref(a, 0, 4), k = memref(a, 1, 4), v = memref(a, 2, 4), ow = memref(a, 4, 2),
+                 out = memref(a, 5, 3);
+    TRY(need_single_token(ctx, q.sizes[1], "Attn kernel"));
+    const int T = (int)k.sizes[2], kvh = b.kv_heads, hd = b.head_dim;
+    if (T < 1 || k.strides[3] != 1 || v.strides[3] != 1)
+        return hm_set_error(ctx, HM_ERR_INVALID, "Attn kernel: K/V views must have >= 1 row and unit inner stride");
+    Scratch s(ctx);
+    // the attention kernel's split partials must fit the part of the workspace left to the kernels
+    if ((size_t)b.cfg.num_attention_heads * ((T + 31) / 32) * (hd + 2) * 4 > KERNEL_RESERVE)
+        return hm_set_error(ctx, HM_ERR_INVALID, "Attn kernel: %d cache rows are more than this entry point takes", T);
+    const size_t n = (size_t)kvh * T * hd;
+    uint16_t *kc = s.take<uint16_t>(n), *vc = s.take<uint16_t>(n);
+    float *flat = s.take<float>(b.q_dim);
+    if (!kc || !vc || !flat) return hm_set_error(ctx, HM_ERR_OOM, "Attn kernel: workspace too small for %d rows", T);
+    const unsigned blocks = (unsigned)((n + 255) / 256);
+    hipLaunchKernelGGL(kv_view_to_bf16_kernel, dim3(blocks), dim3(256), 0, ctx->stream, k.as<float>(), k.strides[1],
+                       k.strides[2], kc, T, hd, n);
+    hipLaunchKernelGGL(kv_view_to_bf16_kernel, dim3(blocks), dim3(256), 0, ctx->stream, v.as<float>(), v.strides[1],
+                       v.strides[2], vc, T, hd, n);
+    HM_LAUNCH_CHECK(ctx);
+    TRY(hm_gqa_decode_attn(ctx, q.as<float>(), kc, vc, flat, 1, b.cfg.num_attention_heads, kvh, hd, T, T,
+                           (float)(1.0 / std::sqrt((double)hd))));
+    return hm_gemv_bf16(ctx, flat, ow.as<uint16_t>(), out.as<float>(), 1, b.q_dim, b.cfg.hidden_size);
+}
+
+// emit_mlp_kernel (src/hf/emitter.rs:767-822): h, attn_out, ln_w, gate_w, up_w, down_w -> [1,S,hidden]
+int run_mlp(void **a) {
+    const Bound &b = g_bound;
+    hm_ctx *ctx = b.ctx;
+    const int hidden = b.cfg.hidden_size, inter = b.cfg.intermediate_size;
+    const MemRef h = memref(a, 0, 3), attn = memref(a, 1, 3), ln = memref(a, 2, 1), gw = memref(a, 3, 2),
+                 uw = memref(a, 4, 2), dw = memref(a, 5, 2), out = memref(a, 6, 3);
+    TRY(need_single_token(ctx, h.sizes[1], "MLP kernel"));
+    Scratch s(ctx);
+    float *resid = s.take<float>(hidden), *normed = s.take<float>(hidden), *gate = s.take<float>(inter),
+          *up = s.take<float>(inter), *down = s.take<float>(hidden);
+    if (!resid || !normed || !gate || !up || !down) return hm_set_error(ctx, HM_ERR_OOM, "MLP kernel: workspace too small");
+    TRY(hm_add(ctx, h.as<float>(), attn.as<float>(), resid, (size_t)hidden));
+    TRY(hm_rmsnorm(ctx, resid, ln.as<float>(), normed, 1, hidden, (float)b.cfg.rms_norm_eps));
+    TRY(hm_gemv_bf16(ctx, normed, gw.as<uint16_t>(), gate, 1, hidden, inter));
+    TRY(hm_gemv_bf16(ctx, normed, uw.as<uint16_t>(), up, 1, hidden, inter));
+    TRY(hm_silu_mul(ctx, gate, up, gate, (size_t)inter));
+    TRY(hm_gemv_bf16(ctx, gate, dw.as<uint16_t>(), down, 1, inter, hidden));
+    return hm_add(ctx, resid, down, out.as<float>(), (size_t)hidden);
+}
+
+// emit_lm_head_kernel (src/hf/emitter.rs:828-862): h, norm_w, lm_head_w [hidden,vocab] -> [1,S,vocab]
+int run_lm_head(void **a) {
+    const Bound &b = g_bound;
+    hm_ctx *ctx = b.ctx;
+    const MemRef h = memref(a, 0, 3), nw = memref(a, 1, 1), lw = memref(a, 2, 2), out = memref(a, 3, 3);
+    TRY(need_single_token(ctx, h.sizes[1], "LMHead kernel"));
+    Scratch s(ctx);
+    float *normed = s.take<float>(b.cfg.hidden_size);
+    if (!normed) return hm_set_error(ctx, HM_ERR_OOM, "LMHead kernel: workspace too small");
+    TRY(hm_rmsnorm(ctx, h.as<float>(), nw.as<float>(), normed, 1, b.cfg.hidden_size, (float)b.cfg.rms_norm_eps));
+    return hm_gemv_bf16(ctx, normed, lw.as<uint16_t>(), out.as<float>(), 1, b.cfg.hidden_size, b.cfg.vocab_size);
+}
+
+void dispatch(int idx, void **args) {
+    if (!g_bound.ctx || idx >= (int)g_bound.kinds.size()) {
+        report(idx, HM_ERR_STATE);
+        return;
+    }
+    int rc = HM_ERR_INVALID;
+    switch (g_bound.kinds[idx]) {
+    case Kind::Embed: rc = run_embed(args); break;
+    case Kind::Qkv: rc = run_qkv(args); break;
+    case Kind::Attn: rc = run_attn(args); break;
+    case Kind::Mlp: rc = run_mlp(args); break;
+    case Kind::LmHead: rc = run_lm_head(args); break;
+    }
+    report(idx, rc);
+}
+
+}  // namespace
+
+extern "C" {
+
+int hm_ciface_bind_transformer(hm_ctx *ctx, const hm_transformer_config *cfg, int has_qk_norm) {
+    HM_CHECK_CTX(ctx);
+    HM_REQUIRE(ctx, cfg, "hm_ciface_bind_transformer: NULL config");
+    const int kvh = cfg->num_key_value_heads ? cfg->num_key_value_heads : cfg->num_attention_heads;
+    HM_REQUIRE(ctx, cfg->hidden_size > 0 && cfg->num_attention_heads > 0 && cfg->num_hidden_layers > 0 &&
+                        cfg->num_attention_heads % kvh == 0,
+               "hm_ciface_bind_transformer: bad config");
+    const int n = 3 * cfg->num_hidden_layers + 2;
+    HM_REQUIRE(ctx, n <= HM_CIFACE_MAX_KERNELS, "hm_ciface_bind_transformer: %d kernels, at most %d symbols are exported",
+               n, HM_CIFACE_MAX_KERNELS);
+    Bound b;
+    b.ctx = ctx;
+    b.cfg = *cfg;
+    b.qk_norm = has_qk_norm != 0;
+    b.kv_heads = kvh;
+    b.head_dim = cfg->head_dim ? cfg->head_dim : cfg->hidden_size / cfg->num_attention_heads;
+    b.q_dim = cfg->num_attention_heads * b.head_dim;
+    b.kv_dim = kvh * b.head_dim;
+    if (b.cfg.rms_norm_eps <= 0) b.cfg.rms_norm_eps = 1e-6;
+    b.kinds.push_back(Kind::Embed);
+    for (int l = 0; l < cfg->num_hidden_layers; l++) {
+        b.kinds.push_back(Kind::Qkv);
+        b.kinds.push_back(Kind::Attn);
+        b.kinds.push_back(Kind::Mlp);
+    }
+    b.kinds.push_back(Kind::LmHead);
+    g_bound = std::move(b);
+    return HM_OK;
+}
+
+int hm_ciface_num_kernels(void) { return (int)g_bound.kinds.size(); }
+
+void hm_ciface_unbind(void) { g_bound = Bound(); }
+
+// 256 exported symbols _mlir__mlir_ciface_k0 ... _mlir__mlir_ciface_k255
+#define HM_K(i) \
+    __attribute__((visibility("default"))) void _mlir__mlir_ciface_k##i(void **args) { dispatch(i, args); }
+#define HM_K10(p) HM_K(p##0) HM_K(p##1) HM_K(p##2) HM_K(p##3) HM_K(p##4) HM_K(p##5) HM_K(p##6) HM_K(p##7) HM_K(p##8) HM_K(p##9)
+HM_K(0) HM_K(1) HM_K(2) HM_K(3) HM_K(4) HM_K(5) HM_K(6) HM_K(7) HM_K(8) HM_K(9)
+HM_K10(1) HM_K10(2) HM_K10(3) HM_K10(4) HM_K10(5) HM_K10(6) HM_K10(7) HM_K10(8) HM_K10(9)
+HM_K10(10) HM_K10(11) HM_K10(12) HM_K10(13) HM_K10(14) HM_K10(15) HM_K10(16) HM_K10(17) HM_K10(18) HM_K10(19)
+HM_K10(20) HM_K10(21) HM_K10(22) HM_K10(23) HM_K10(24)
+HM_K(250) HM_K(251) HM_K(252) HM_K(253) HM_K(254) HM_K(255)
+#undef HM_K10
+#undef HM_K
+
+}  // extern "C"

@@ -253,6 +253,24 @@ int hm_model_time_kernels(hm_model *m, int rounds, hm_kernel_profile *out, int c
 /* Number of HIP kernel launches one decode step issues. */
 int hm_model_launches_per_step(hm_model *m);
 
+/* ── the reference's kernel ABI, literally ─────────────────────────────────
+ * The library also exports HM_CIFACE_MAX_KERNELS symbols
+ *     void _mlir__mlir_ciface_k0(void **args) ... void _mlir__mlir_ciface_k255(void **args)
+ * with the signature and argument convention of the reference's compiled kernels: args[i]
+ * points at a pointer to a rank-N memref descriptor {allocated, aligned, offset, sizes[N],
+ * strides[N]} (src/runtime.rs:654-698, :930-1037), inputs first, outputs after; `aligned` holds
+ * a device pointer. CompiledGraph::load_from_handle (src/runtime.rs:803-824) resolves them with
+ * dlsym exactly as it resolves its own. hm_ciface_bind_transformer tells the library which
+ * fused kernel each index is, in emit_transformer_plan's numbering (src/hf/emitter.rs:902-1014):
+ * k0 Embed, k(3l+1) QKV(+QK-norm)+RoPE, k(3l+2) Attn, k(3l+3) MLP for layer l, then LMHead;
+ * bf16 weights [K,N], f32 K/V views with the cache's strides, one token per call. A failure
+ * cannot be returned (the ABI is void): it is recorded for hm_last_error and printed to stderr.
+ * One binding per process at a time. */
+#define HM_CIFACE_MAX_KERNELS 256
+int hm_ciface_bind_transformer(hm_ctx *ctx, const hm_transformer_config *cfg, int has_qk_norm);
+int hm_ciface_num_kernels(void);
+void hm_ciface_unbind(void);
+
 /* ── deterministic synthetic data (host side, no GPU needed) ─────────────────
  * Counter-based generator shared by tests and benchmarks: sample i of stream `seed` uses
  * outputs 3i..3i+2 of the splitmix64 sequence seeded with `seed`; a normal variate is the

@@ -1,0 +1,137 @@
+"""The reference's own kernel ABI (`_mlir__mlir_ciface_k{idx}(void **args)` with memref
+descriptors, reference src/runtime.rs:654-698, :930-1037) driven the way ExecutionPlan::run_kv
+drives it (src/runtime.rs:1580-1892): kernels in plan order, K/V appended into an f32 cache
+[1, kvh, max, hd] and handed on as strided views (src/runtime.rs:521-625)."""
+from __future__ import annotations
+
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import model_fixture as mf
+from homura_amd import _ffi, synth, synth_model
+
+pytestmark = pytest.mark.gpu
+
+
+def say(msg):
+    print(f"[ciface] {msg}", flush=True)
+
+
+class Desc:
+    """A rank-N memref descriptor plus the pointer-to-pointer the ABI wants."""
+
+    def __init__(self, ptr: int, shape, strides=None):
+        n = len(shape)
+        if strides is None:
+            strides, acc = [0] * n, 1
+            for i in reversed(range(n)):
+                strides[i] = acc
+                acc *= shape[i]
+        self.raw = (C.c_int64 * (3 + 2 * n))(ptr, ptr, 0, *shape, *strides)
+        self.p = C.c_void_p(C.addressof(self.raw))
+
+    def arg(self):
+        return C.cast(C.pointer(self.p), C.c_void_p)
+
+
+def call(lib, idx, descs):
+    args = (C.c_void_p * len(descs))(*[d.arg() for d in descs])
+    fn = getattr(lib, f"_mlir__mlir_ciface_k{idx}")
+    fn.restype, fn.argtypes = None, [C.c_void_p]
+    fn(C.cast(args, C.c_void_p))
+
+
+@pytest.mark.parametrize("which", ["qwen3_qknorm", "qwen2_bias"])
+def test_plan_through_memref_entry_points(ctx, which):
+    qkn = which == "qwen3_qknorm"
+    cfg = synth_model.TINY if qkn else synth_model.TINY_QWEN2
+    weights = synth_model.synth_weights(cfg, 314, has_qk_norm=qkn)
+    W = dict(weights)
+    L, hidden, inter, vocab = cfg.num_hidden_layers, cfg.hidden_size, cfg.intermediate_size, cfg.vocab_size
+    H, kvh, hd = cfg.num_attention_heads, cfg.kv_heads(), cfg.get_head_dim()
+    max_len, past, steps = 64, 9, 3
+    om = mf.build_oracle_model(cfg, weights, max_len, has_qk_norm=qkn)
+    kv = synth_model.synth_kv(cfg, 12, past)
+    mf.oracle_init_kv(om, kv)
+
+    lib = C.CDLL(str(_ffi.LIB_PATH))
+    ccfg = cfg.to_c()
+    ctx._check(ctx.lib.hm_ciface_bind_transformer(ctx.h, C.byref(ccfg), int(qkn)))
+    assert ctx.lib.hm_ciface_num_kernels() == 3 * L + 2
+
+    dev = {n: ctx.to_device(a) for n, a in weights}     # the reference's slot buffers, as they are
+    cos, sin = om.cos, om.sin                            # [max_pos, hd] tables (precompute_rope_cos_sin)
+    cache = []
+    for l in range(2 * L):                               # f32 caches [1, kvh, max_len, hd]
+        full = np.zeros((kvh, max_len, hd), np.float32)
+        full[:, :past] = kv[l][0]
+        cache.append(ctx.to_device(full))
+    d_h = [ctx.empty(hidden), ctx.empty(hidden)]
+    d_q, d_k, d_v = ctx.empty(H * hd), ctx.empty(kvh * hd), ctx.empty(kvh * hd)
+    d_attn, d_logits = ctx.empty(hidden), ctx.empty(vocab)
+    d_mask = ctx.empty(max_len)
+    ids = synth.token_ids(21, steps, vocab)
+    cur = past
+    for t in range(steps):
+        say(f"{which}: token {t} at position {cur}")
+        d_ids = ctx.to_device(ids[t:t + 1].astype(np.int64))
+        d_cos, d_sin = ctx.to_device(cos[cur:cur + 1]), ctx.to_device(sin[cur:cur + 1])
+        call(lib, 0, [Desc(d_ids.ptr, [1, 1]), Desc(dev["model.embed_tokens.weight"].ptr, [vocab, hidden]),
+                      Desc(d_h[0].ptr, [1, 1, hidden])])
+        for l in range(L):
+            p = f"model.layers.{l}."
+            qkv_in = [Desc(d_h[0].ptr, [1, 1, hidden]), Desc(dev[p + "input_layernorm.weight"].ptr, [hidden]),
+                      Desc(dev[p + "self_attn.q_proj.weight"].ptr, [hidden, H * hd])]
+            if cfg.attention_bias:
+                qkv_in.append(Desc(dev[p + "self_attn.q_proj.bias"].ptr, [H * hd]))
+            qkv_in.append(Desc(dev[p + "self_attn.k_proj.weight"].ptr, [hidden, kvh * hd]))
+            if cfg.attention_bias:
+                qkv_in.append(Desc(dev[p + "self_attn.k_proj.bias"].ptr, [kvh * hd]))
+            qkv_in.append(Desc(dev[p + "self_attn.v_proj.weight"].ptr, [hidden, kvh * hd]))
+            if cfg.attention_bias:
+                qkv_in.append(Desc(dev[p + "self_attn.v_proj.bias"].ptr, [kvh * hd]))
+            qkv_in += [Desc(d_cos.ptr, [1, hd]), Desc(d_sin.ptr, [1, hd])]
+            if qkn:
+                qkv_in += [Desc(dev[p + "self_attn.q_norm.weight"].ptr, [hd]),
+                           Desc(dev[p + "self_attn.k_norm.weight"].ptr, [hd])]
+            outs = [Desc(d_q.ptr, [1, 1, H, hd]), Desc(d_k.ptr, [1, kvh, 1, hd]), Desc(d_v.ptr, [1, kvh, 1, hd])]
+            call(lib, 3 * l + 1, qkv_in + outs)
+            # NativeOp::Concat on the cache: one row per kv head at row `cur`
+            for which_kv, src in ((0, d_k), (1, d_v)):
+                c = cache[2 * l + which_kv]
+                for h in range(kvh):
+                    ctx._check(ctx.lib.hm_copy(ctx.h, c.ptr + ((h * max_len + cur) * hd) * 4,
+                                               src.ptr + h * hd * 4, hd * 4))
+            view = lambda c: Desc(c.ptr, [1, kvh, cur + 1, hd], [kvh * max_len * hd, max_len * hd, hd, 1])
+            call(lib, 3 * l + 2, [Desc(d_q.ptr, [1, 1, H, hd]), view(cache[2 * l]), view(cache[2 * l + 1]),
+                                  Desc(d_mask.ptr, [1, 1, 1, cur + 1]),
+                                  Desc(dev[p + "self_attn.o_proj.weight"].ptr, [H * hd, hidden]),
+                                  Desc(d_attn.ptr, [1, 1, hidden])])
+            call(lib, 3 * l + 3, [Desc(d_h[0].ptr, [1, 1, hidden]), Desc(d_attn.ptr, [1, 1, hidden]),
+                                  Desc(dev[p + "post_attention_layernorm.weight"].ptr, [hidden]),
+                                  Desc(dev[p + "mlp.gate_proj.weight"].ptr, [hidden, inter]),
+                                  Desc(dev[p + "mlp.up_proj.weight"].ptr, [hidden, inter]),
+                                  Desc(dev[p + "mlp.down_proj.weight"].ptr, [inter, hidden]),
+                                  Desc(d_h[1].ptr, [1, 1, hidden])])
+            d_h.reverse()
+        call(lib, 3 * L + 1, [Desc(d_h[0].ptr, [1, 1, hidden]), Desc(dev["model.norm.weight"].ptr, [hidden]),
+                              Desc(dev["lm_head.weight"].ptr, [hidden, vocab]), Desc(d_logits.ptr, [1, 1, vocab])])
+        got = d_logits.download(np.float32)
+        want = om.run_kv(ids[t:t + 1])[0]
+        err = mf.rel_err(got, want)
+        say(f"{which}: token {t} logits rel err {err:.2e}")
+        assert err < 1e-2
+        assert int(len(got) - 1 - np.argmax(got[::-1])) == int(len(want) - 1 - np.argmax(want[::-1]))
+        cur += 1
+    ctx.lib.hm_ciface_unbind()
+
+
+def test_unbound_call_is_reported_not_fatal(ctx, capfd):
+    """No binding: the entry point records an error and returns (the ABI has no status)."""
+    ctx.lib.hm_ciface_unbind()
+    lib = C.CDLL(str(_ffi.LIB_PATH))
+    d = ctx.empty(4)
+    call(lib, 5, [Desc(d.ptr, [4])])
+    assert "no transformer bound" in capfd.readouterr().err
