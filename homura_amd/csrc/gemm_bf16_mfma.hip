@@ -3,9 +3,10 @@
 // stream layout the decode GEMVs use).
 //
 // The only MFMA kernel of the path (everything at batch 1 is HBM-bound). Workgroup tile 128x128,
-// four wavefronts 2x2, each owning 64x64 = 2x2 accumulator tiles of v_mfma_f32_32x32x16_bf16.
-// K advances 64 at a time. The next K tile travels global -> registers while the current one is
-// multiplied out of LDS; two LDS buffers, one barrier per tile.
+// eight wavefronts: two groups of 2x2, each wavefront owning 64x64 = 2x2 accumulator tiles of
+// v_mfma_f32_32x32x16_bf16 over half of the k steps. K advances 64 at a time. Four K tiles travel
+// global -> registers while the current one is multiplied out of LDS; two LDS buffers, one
+// barrier per tile.
 //
 // LDS holds both operands K-contiguous: row r (an m of A or an n of B) is 128 bytes = eight 16-byte
 // chunks of 8 k; chunk c of row r lives at slot c ^ (r & 7) ^ ((r >> 3) & 7). The MFMA operand read
@@ -38,73 +39,94 @@ __device__ __forceinline__ void lds_barrier() {
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }
 
-// Registers holding one K tile in flight: A always four 16-byte chunks; B four chunks as well
-// (rows of a [N][K] tile, or the 4 x 8 block of a [K][N] tile).
+constexpr int GEMM_THREADS = 512;
+
+// Registers holding a thread's share of one K tile in flight (four 16-byte chunks):
+//   B [N][K]: v[0..1] two chunks of A, v[2..3] two chunks of B;
+//   B [K][N]: threads 0..255 carry a 4(k) x 8(n) block of B as four rows, threads 256..511 four
+//             chunks of A.
 struct TileRegs {
-    u32x4 a[4], b[4];
+    u32x4 v[4];
 };
 
-// Requests one K tile. No branches: a chunk beyond K reads the last valid chunk of its row (and is
-// replaced by zeros when it is written to LDS), so the loop body stays one basic block and the
-// compiler can count exactly which loads a later LDS write has to wait for.
+// Requests one K tile. No branches on k: a chunk beyond K reads the last valid chunk of its row
+// (and is replaced by zeros when it is written to LDS), so the loop body stays one basic block and
+// the compiler can count exactly which loads a later LDS write has to wait for.
 template <bool B_NK>
 __device__ __forceinline__ void load_tile(TileRegs &t, const uint16_t *__restrict__ A,
                                           const uint16_t *__restrict__ B, int m0, int n0, int k0, int K,
                                           int N, int tid) {
+    if (B_NK) {
 #pragma unroll
-    for (int j = 0; j < 4; j++) {
-        const int id = tid + j * 256, r = id >> 3, c = id & 7;
-        const int kc = min(k0 + c * 8, K - 8);
-        t.a[j] = ld128(A + (size_t)(m0 + r) * K + kc);
-        if (B_NK) t.b[j] = ld128(B + (size_t)(n0 + r) * K + kc);
-    }
-    if (!B_NK) {
+        for (int j = 0; j < 2; j++) {
+            const int id = tid + j * GEMM_THREADS, r = id >> 3, c = id & 7;
+            const int kc = min(k0 + c * 8, K - 8);
+            t.v[j] = ld128(A + (size_t)(m0 + r) * K + kc);
+            t.v[2 + j] = ld128(B + (size_t)(n0 + r) * K + kc);
+        }
+    } else if (tid < 256) {  // wavefront-uniform
         const int ng = tid & 15, kg = tid >> 4;
 #pragma unroll
         for (int r = 0; r < 4; r++) {
             const int kc = min(k0 + kg * 4 + r, K - 1);
-            t.b[r] = ld128(B + (size_t)kc * N + n0 + ng * 8);
+            t.v[r] = ld128(B + (size_t)kc * N + n0 + ng * 8);
+        }
+    } else {
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int id = (tid - 256) + j * 256, r = id >> 3, c = id & 7;
+            const int kc = min(k0 + c * 8, K - 8);
+            t.v[j] = ld128(A + (size_t)(m0 + r) * K + kc);
         }
     }
 }
 
-// Quarter `part` (0..3) of the LDS writes of one tile; the four quarters are placed between the
-// MFMA groups of the tile being multiplied so they issue in the matrix pipe's shadow.
+// Half `part` (0, 1) of a thread's LDS writes of one tile; the halves sit next to the two MFMA
+// groups a wavefront runs per tile.
 template <bool B_NK>
 __device__ __forceinline__ void store_tile_part(const TileRegs &t, char *__restrict__ as,
                                                 char *__restrict__ bs, int tid, int part, int k0, int K) {
     const u32x4 zero = {0u, 0u, 0u, 0u};
-    {
-        const int id = tid + part * 256, r = id >> 3, c = id & 7;
+    if (B_NK) {
+        const int id = tid + part * GEMM_THREADS, r = id >> 3, c = id & 7;
         const bool ok = k0 + c * 8 < K;
-        *reinterpret_cast<u32x4 *>(as + lds_off(r, c)) = ok ? t.a[part] : zero;
-        if (B_NK) *reinterpret_cast<u32x4 *>(bs + lds_off(r, c)) = ok ? t.b[part] : zero;
-    }
-    if (!B_NK) {
+        *reinterpret_cast<u32x4 *>(as + lds_off(r, c)) = ok ? t.v[part] : zero;
+        *reinterpret_cast<u32x4 *>(bs + lds_off(r, c)) = ok ? t.v[2 + part] : zero;
+    } else if (tid < 256) {
         const int ng = tid & 15, kg = tid >> 4;
-        const int kb = k0 + kg * 4;  // K is a multiple of 32: the four rows are in or out together
-        const bool ok = kb < K;
+        const bool ok = k0 + kg * 4 < K;  // K is a multiple of 32: the four rows are in or out together
 #pragma unroll
-        for (int i = part * 2; i < part * 2 + 2; i++) {
+        for (int i = part * 4; i < part * 4 + 4; i++) {
             // column n = ng*8 + i of the block: k+0..k+3 packed low to high
             const uint32_t sel = (i & 1) ? 0x07060302u : 0x05040100u;
             u32x2 col;
-            col.x = ok ? __builtin_amdgcn_perm(t.b[1][i >> 1], t.b[0][i >> 1], sel) : 0u;
-            col.y = ok ? __builtin_amdgcn_perm(t.b[3][i >> 1], t.b[2][i >> 1], sel) : 0u;
+            col.x = ok ? __builtin_amdgcn_perm(t.v[1][i >> 1], t.v[0][i >> 1], sel) : 0u;
+            col.y = ok ? __builtin_amdgcn_perm(t.v[3][i >> 1], t.v[2][i >> 1], sel) : 0u;
             const int n = ng * 8 + i;
             *reinterpret_cast<u32x2 *>(bs + lds_off(n, kg >> 1) + (kg & 1) * 8) = col;
+        }
+    } else {
+#pragma unroll
+        for (int j = part * 2; j < part * 2 + 2; j++) {
+            const int id = (tid - 256) + j * 256, r = id >> 3, c = id & 7;
+            *reinterpret_cast<u32x4 *>(as + lds_off(r, c)) = k0 + c * 8 < K ? t.v[j] : zero;
         }
     }
 }
 
+// Eight wavefronts, two per SIMD: one wavefront alone cannot issue the LDS reads and writes, the
+// global loads and the MFMAs of a tile fast enough to keep the matrix pipe busy. Wavefronts 0-3
+// multiply k steps 0 and 1 of every K tile, wavefronts 4-7 steps 2 and 3, each group with its own
+// 2x2 arrangement of 64x64 accumulators; the two groups' sums meet in LDS at the end.
 template <bool B_NK>
-__global__ __launch_bounds__(256) void gemm_bf16_mfma_kernel(const uint16_t *__restrict__ A,
-                                                             const uint16_t *__restrict__ B,
-                                                             float *__restrict__ C, int M, int K, int N) {
+__global__ __launch_bounds__(GEMM_THREADS) void gemm_bf16_mfma_kernel(const uint16_t *__restrict__ A,
+                                                                      const uint16_t *__restrict__ B,
+                                                                      float *__restrict__ C, int M, int K,
+                                                                      int N) {
     __shared__ __attribute__((aligned(16))) char lds[2][2][TILE_BYTES];  // [buffer][A|B]
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = wave >> 1, wn = wave & 1;
+    const int kgrp = wave >> 2, wm = (wave >> 1) & 1, wn = wave & 1;
     const int l32 = lane & 31, lh = lane >> 5;
 
     // XCD-aware tile order: ids are dealt round-robin to the 8 XCDs, so XCD x runs ids x, x+8, ...;
@@ -123,7 +145,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_mfma_kernel(const uint16_t *__r
             for (int v = 0; v < 16; v++) acc[i][j][v] = 0.f;
 
     // DEPTH tiles in flight in registers: tile j is requested DEPTH iterations before its LDS
-    // writes, which sit between the MFMA groups of tile j-1. The iteration count is rounded up to
+    // writes, which sit next to the MFMA groups of tile j-1. The iteration count is rounded up to
     // a multiple of DEPTH (the extra tiles are zeros) so the register ring is indexed statically.
     constexpr int DEPTH = 4;
     const int nk = (K + TK - 1) / TK;
@@ -132,16 +154,17 @@ __global__ __launch_bounds__(256) void gemm_bf16_mfma_kernel(const uint16_t *__r
 #pragma unroll
     for (int d = 0; d < DEPTH; d++) load_tile<B_NK>(t[d], A, B, m0, n0, d * TK, K, N, tid);
 #pragma unroll
-    for (int part = 0; part < 4; part++) store_tile_part<B_NK>(t[0], lds[0][0], lds[0][1], tid, part, 0, K);
+    for (int part = 0; part < 2; part++) store_tile_part<B_NK>(t[0], lds[0][0], lds[0][1], tid, part, 0, K);
     lds_barrier();
 
-    // operand registers, two stages: the reads of step ks+1 are in flight during the MFMAs of ks
+    // operand registers, two stages: the reads of the next step are in flight during the MFMAs
     bf16x8 af[2][2], bfr[2][2];
     const int arow = wm * 64 + l32, brow = wn * 64 + l32;
+    const int chunk0 = kgrp * 4 + lh, chunk1 = chunk0 + 2;  // this group's two k steps of a tile
 #pragma unroll
     for (int i = 0; i < 2; i++) {
-        af[0][i] = *reinterpret_cast<const bf16x8 *>(lds[0][0] + lds_off(arow + i * 32, lh));
-        bfr[0][i] = *reinterpret_cast<const bf16x8 *>(lds[0][1] + lds_off(brow + i * 32, lh));
+        af[0][i] = *reinterpret_cast<const bf16x8 *>(lds[0][0] + lds_off(arow + i * 32, chunk0));
+        bfr[0][i] = *reinterpret_cast<const bf16x8 *>(lds[0][1] + lds_off(brow + i * 32, chunk0));
     }
 
     for (int kt0 = 0; kt0 < nkp; kt0 += DEPTH) {
@@ -150,44 +173,53 @@ __global__ __launch_bounds__(256) void gemm_bf16_mfma_kernel(const uint16_t *__r
             const int cur = u & 1;  // DEPTH is even: tile kt0+u sits in buffer u & 1
             // tile kt0+u left its registers during the previous iteration: refill them
             load_tile<B_NK>(t[u], A, B, m0, n0, (kt0 + u + DEPTH) * TK, K, N, tid);
+            const int k_next = (kt0 + u + 1) * TK;
+            char *an = lds[cur ^ 1][0], *bn = lds[cur ^ 1][1];
+
+            // first step: its operands are in stage 0; fetch the second step's meanwhile
 #pragma unroll
-            for (int ks = 0; ks < TK / 16; ks++) {
-                const int st = ks & 1, nx = st ^ 1;
-                if (ks < TK / 16 - 1) {
-                    const int chunk = (ks + 1) * 2 + lh;
-#pragma unroll
-                    for (int i = 0; i < 2; i++) {
-                        af[nx][i] = *reinterpret_cast<const bf16x8 *>(lds[cur][0] + lds_off(arow + i * 32, chunk));
-                        bfr[nx][i] = *reinterpret_cast<const bf16x8 *>(lds[cur][1] + lds_off(brow + i * 32, chunk));
-                    }
-                } else {
-                    // every wave has written its share of the next tile and read the last operands
-                    // of this one: switch buffers, and fetch the next tile's first operands under
-                    // the last MFMA group of this tile
-                    lds_barrier();
-#pragma unroll
-                    for (int i = 0; i < 2; i++) {
-                        af[nx][i] = *reinterpret_cast<const bf16x8 *>(lds[cur ^ 1][0] + lds_off(arow + i * 32, lh));
-                        bfr[nx][i] = *reinterpret_cast<const bf16x8 *>(lds[cur ^ 1][1] + lds_off(brow + i * 32, lh));
-                    }
-                }
-#pragma unroll
-                for (int i = 0; i < 2; i++)
-#pragma unroll
-                    for (int j = 0; j < 2; j++)
-                        acc[i][j] =
-                            __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[st][i], bfr[st][j], acc[i][j], 0, 0, 0);
-                const int k_next = (kt0 + u + 1) * TK;
-                char *an = lds[cur ^ 1][0], *bn = lds[cur ^ 1][1];
-                if (ks == 0) store_tile_part<B_NK>(t[(u + 1) % DEPTH], an, bn, tid, 0, k_next, K);
-                if (ks == 1) store_tile_part<B_NK>(t[(u + 1) % DEPTH], an, bn, tid, 1, k_next, K);
-                if (ks == 2) {
-                    store_tile_part<B_NK>(t[(u + 1) % DEPTH], an, bn, tid, 2, k_next, K);
-                    store_tile_part<B_NK>(t[(u + 1) % DEPTH], an, bn, tid, 3, k_next, K);
-                }
+            for (int i = 0; i < 2; i++) {
+                af[1][i] = *reinterpret_cast<const bf16x8 *>(lds[cur][0] + lds_off(arow + i * 32, chunk1));
+                bfr[1][i] = *reinterpret_cast<const bf16x8 *>(lds[cur][1] + lds_off(brow + i * 32, chunk1));
             }
+#pragma unroll
+            for (int i = 0; i < 2; i++)
+#pragma unroll
+                for (int j = 0; j < 2; j++)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[0][i], bfr[0][j], acc[i][j], 0, 0, 0);
+            store_tile_part<B_NK>(t[(u + 1) % DEPTH], an, bn, tid, 0, k_next, K);
+            store_tile_part<B_NK>(t[(u + 1) % DEPTH], an, bn, tid, 1, k_next, K);
+            // every wavefront has written its share of the next tile and read the last operands of
+            // this one: switch buffers, and fetch the next tile's first operands under the second
+            // MFMA group of this tile
+            lds_barrier();
+#pragma unroll
+            for (int i = 0; i < 2; i++) {
+                af[0][i] = *reinterpret_cast<const bf16x8 *>(an + lds_off(arow + i * 32, chunk0));
+                bfr[0][i] = *reinterpret_cast<const bf16x8 *>(bn + lds_off(brow + i * 32, chunk0));
+            }
+#pragma unroll
+            for (int i = 0; i < 2; i++)
+#pragma unroll
+                for (int j = 0; j < 2; j++)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[1][i], bfr[1][j], acc[i][j], 0, 0, 0);
         }
     }
+
+    // the second group hands its sums over through LDS (64 KiB = 4 wavefronts x 64 x 64 floats,
+    // lane-major so consecutive lanes touch consecutive words)
+    lds_barrier();  // nobody reads operands any more
+    float *xch = reinterpret_cast<float *>(&lds[0][0][0]) + (size_t)(wave & 3) * 64 * 64 + lane;
+    if (kgrp == 1) {
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+#pragma unroll
+            for (int j = 0; j < 2; j++)
+#pragma unroll
+                for (int v = 0; v < 16; v++) xch[((i * 2 + j) * 16 + v) * 64] = acc[i][j][v];
+    }
+    lds_barrier();
+    if (kgrp == 1) return;
 
     // accumulator element v of lane l sits at row (v/4)*8 + (l/32)*4 + v%4, column l%32
 #pragma unroll
@@ -198,7 +230,8 @@ __global__ __launch_bounds__(256) void gemm_bf16_mfma_kernel(const uint16_t *__r
             for (int v = 0; v < 16; v++) {
                 const int row = m0 + wm * 64 + i * 32 + (v >> 2) * 8 + lh * 4 + (v & 3);
                 const int col = n0 + wn * 64 + j * 32 + l32;
-                __builtin_nontemporal_store(acc[i][j][v], C + (size_t)row * N + col);
+                __builtin_nontemporal_store(acc[i][j][v] + xch[((i * 2 + j) * 16 + v) * 64],
+                                            C + (size_t)row * N + col);
             }
 }
 
@@ -213,9 +246,9 @@ int gemm_launch(hm_ctx *ctx, const char *who, const uint16_t *a, const uint16_t 
     HM_REQUIRE(ctx, (long long)(M / TM) * (N / TN) <= 0x7fffffffLL, "%s: too many tiles", who);
     const dim3 grid((M / TM) * (N / TN));
     if (b_nk)
-        hipLaunchKernelGGL(gemm_bf16_mfma_kernel<true>, grid, dim3(256), 0, ctx->stream, a, b, c, M, K, N);
+        hipLaunchKernelGGL(gemm_bf16_mfma_kernel<true>, grid, dim3(GEMM_THREADS), 0, ctx->stream, a, b, c, M, K, N);
     else
-        hipLaunchKernelGGL(gemm_bf16_mfma_kernel<false>, grid, dim3(256), 0, ctx->stream, a, b, c, M, K, N);
+        hipLaunchKernelGGL(gemm_bf16_mfma_kernel<false>, grid, dim3(GEMM_THREADS), 0, ctx->stream, a, b, c, M, K, N);
     HM_LAUNCH_CHECK(ctx);
     return HM_OK;
 }
