@@ -75,6 +75,29 @@ SIGNATURES = {
     "hm_dequant_q4_0": (_I, [_P, _P, _P, _SZ]),
     "hm_gemm_bf16": (_I, [_P, _P, _P, _P, _I, _I, _I]),
     "hm_gemm_bf16_nk": (_I, [_P, _P, _P, _P, _I, _I, _I]),
+    "hm_model_set_weight_nk": (_I, [_P, _I, _P, _SZ]),
+    "hm_model_config": (_I, [_P, _P, _P, _P]),
+    "hm_gguf_open": (_P, [C.c_char_p, C.c_char_p, _SZ]),
+    "hm_gguf_close": (None, [_P]),
+    "hm_gguf_version": (_I, [_P]),
+    "hm_gguf_num_tensors": (_I, [_P]),
+    "hm_gguf_data_offset": (_SZ, [_P]),
+    "hm_gguf_tensor_info": (_I, [_P, _I, C.c_char_p, _SZ, _P, _P, _P, _P, _P]),
+    "hm_gguf_find_tensor": (_I, [_P, C.c_char_p]),
+    "hm_gguf_tensor_data": (_P, [_P, _I]),
+    "hm_gguf_meta_str": (_I, [_P, C.c_char_p, C.c_char_p, _SZ]),
+    "hm_gguf_meta_u64": (_I, [_P, C.c_char_p, _P]),
+    "hm_gguf_meta_f32": (_I, [_P, C.c_char_p, _P]),
+    "hm_gguf_meta_array_len": (C.c_int64, [_P, C.c_char_p]),
+    "hm_gguf_transformer_config": (_I, [_P, _P, _P, C.c_char_p, _SZ]),
+    "hm_safetensors_open": (_P, [C.c_char_p, C.c_char_p, _SZ]),
+    "hm_safetensors_close": (None, [_P]),
+    "hm_safetensors_num_tensors": (_I, [_P]),
+    "hm_safetensors_tensor_info": (_I, [_P, _I, C.c_char_p, _SZ, C.c_char_p, _P, _P, _P]),
+    "hm_safetensors_tensor_data": (_P, [_P, _I]),
+    "hm_config_from_json": (_I, [C.c_char_p, _P, C.c_char_p, _SZ]),
+    "hm_model_load_gguf": (_P, [_P, C.c_char_p, _I]),
+    "hm_model_load_hf_dir": (_P, [_P, C.c_char_p, _I]),
     "hm_ciface_bind_transformer": (_I, [_P, _P, _I]),
     "hm_ciface_num_kernels": (_I, []),
     "hm_ciface_unbind": (None, []),

@@ -2,6 +2,7 @@
 #include <cstring>
 
 #include "hf.h"
+#include "loaders.h"
 
 using namespace homura;
 
@@ -63,6 +64,11 @@ int hm_model_weight_slot_info(hm_model *m, int slot, char *name_buf, size_t bufl
 int hm_model_set_weight(hm_model *m, int slot, const void *h_data, size_t bytes) {
     if (!m) return HM_ERR_INVALID;
     return m->impl->set_weight(slot, h_data, bytes);
+}
+
+int hm_model_set_weight_nk(hm_model *m, int slot, const void *h_data, size_t bytes) {
+    if (!m) return HM_ERR_INVALID;
+    return m->impl->set_weight_nk(slot, h_data, bytes);
 }
 
 int hm_model_finalize(hm_model *m, int max_seq_len) {
@@ -149,3 +155,170 @@ static int fill_profiles(const std::vector<StepProfile> &prof, hm_kernel_profile
     }
     return n;
 }
+
+// ── checkpoint containers ────────────────────────────────────────────────────
+
+struct hm_gguf {
+    std::unique_ptr<GgufFile> f;
+};
+struct hm_safetensors {
+    std::unique_ptr<SafeTensorsFile> f;
+};
+
+static void copy_err(const std::string &msg, char *err, size_t errlen) {
+    if (err && errlen) snprintf(err, errlen, "%s", msg.c_str());
+}
+
+static void fill_c_config(const TransformerConfig &c, hm_transformer_config *out) {
+    out->hidden_size = c.hidden_size;
+    out->intermediate_size = c.intermediate_size;
+    out->num_attention_heads = c.num_attention_heads;
+    out->num_hidden_layers = c.num_hidden_layers;
+    out->num_key_value_heads = c.num_key_value_heads;
+    out->vocab_size = c.vocab_size;
+    out->head_dim = c.head_dim_opt;
+    out->max_position_embeddings = c.max_position_embeddings;
+    out->tie_word_embeddings = c.tie_word_embeddings ? 1 : 0;
+    out->rms_norm_eps = c.rms_norm_eps;
+    out->rope_theta = c.rope_theta;
+    out->attention_bias = c.attention_bias ? 1 : 0;
+}
+
+extern "C" {
+
+hm_gguf *hm_gguf_open(const char *path, char *err, size_t errlen) {
+    std::string e;
+    auto f = GgufFile::load(path ? path : "", &e);
+    if (!f) {
+        copy_err(e, err, errlen);
+        return nullptr;
+    }
+    return new hm_gguf{std::move(f)};
+}
+void hm_gguf_close(hm_gguf *g) { delete g; }
+int hm_gguf_version(const hm_gguf *g) { return g ? (int)g->f->version() : HM_ERR_INVALID; }
+int hm_gguf_num_tensors(const hm_gguf *g) { return g ? (int)g->f->tensors().size() : HM_ERR_INVALID; }
+size_t hm_gguf_data_offset(const hm_gguf *g) { return g ? g->f->data_offset() : 0; }
+
+int hm_gguf_tensor_info(const hm_gguf *g, int index, char *name_buf, size_t buflen, int *n_dims, uint64_t dims[8],
+                        int *ggml_type, uint64_t *offset, size_t *nbytes) {
+    if (!g || index < 0 || index >= (int)g->f->tensors().size()) return HM_ERR_INVALID;
+    const GgufTensorInfo &t = g->f->tensors()[index];
+    if (name_buf && buflen) snprintf(name_buf, buflen, "%s", t.name.c_str());
+    if (n_dims) *n_dims = (int)t.shape.size();
+    if (dims)
+        for (size_t i = 0; i < t.shape.size() && i < 8; i++) dims[i] = t.shape[i];
+    if (ggml_type) *ggml_type = (int)t.type;
+    if (offset) *offset = t.offset;
+    if (nbytes) *nbytes = t.byte_size();
+    return HM_OK;
+}
+
+int hm_gguf_find_tensor(const hm_gguf *g, const char *name) {
+    if (!g || !name) return HM_ERR_INVALID;
+    const GgufTensorInfo *t = g->f->tensor_info(name);
+    return t ? (int)(t - g->f->tensors().data()) : -1;
+}
+
+const void *hm_gguf_tensor_data(const hm_gguf *g, int index) {
+    if (!g || index < 0 || index >= (int)g->f->tensors().size()) return nullptr;
+    return g->f->tensor_data(g->f->tensors()[index]);
+}
+
+int hm_gguf_meta_str(const hm_gguf *g, const char *key, char *buf, size_t buflen) {
+    std::string s;
+    const GgufValue *v = g && key ? g->f->meta(key) : nullptr;
+    if (!v || !v->as_str(&s)) return HM_ERR_INVALID;
+    if (buf && buflen) snprintf(buf, buflen, "%s", s.c_str());
+    return (int)s.size();
+}
+int hm_gguf_meta_u64(const hm_gguf *g, const char *key, uint64_t *out) {
+    const GgufValue *v = g && key ? g->f->meta(key) : nullptr;
+    return v && out && v->as_u64(out) ? HM_OK : HM_ERR_INVALID;
+}
+int hm_gguf_meta_f32(const hm_gguf *g, const char *key, float *out) {
+    const GgufValue *v = g && key ? g->f->meta(key) : nullptr;
+    return v && out && v->as_f32(out) ? HM_OK : HM_ERR_INVALID;
+}
+int64_t hm_gguf_meta_array_len(const hm_gguf *g, const char *key) {
+    const GgufValue *v = g && key ? g->f->meta(key) : nullptr;
+    return v && v->kind == GgufValue::Array ? (int64_t)v->arr.size() : -1;
+}
+
+int hm_gguf_transformer_config(const hm_gguf *g, hm_transformer_config *out, int *has_qk_norm, char *err,
+                               size_t errlen) {
+    if (!g || !out) return HM_ERR_INVALID;
+    TransformerConfig c;
+    std::string e;
+    if (!g->f->transformer_config(&c, &e)) {
+        copy_err(e, err, errlen);
+        return HM_ERR_INVALID;
+    }
+    fill_c_config(c, out);
+    if (has_qk_norm) *has_qk_norm = g->f->tensor_info("blk.0.attn_q_norm.weight") != nullptr;
+    return HM_OK;
+}
+
+hm_safetensors *hm_safetensors_open(const char *path, char *err, size_t errlen) {
+    std::string e;
+    auto f = SafeTensorsFile::load(path ? path : "", &e);
+    if (!f) {
+        copy_err(e, err, errlen);
+        return nullptr;
+    }
+    return new hm_safetensors{std::move(f)};
+}
+void hm_safetensors_close(hm_safetensors *s) { delete s; }
+int hm_safetensors_num_tensors(const hm_safetensors *s) { return s ? (int)s->f->tensors().size() : HM_ERR_INVALID; }
+int hm_safetensors_tensor_info(const hm_safetensors *s, int index, char *name_buf, size_t buflen, char dtype_buf[8],
+                               int *n_dims, uint64_t dims[8], size_t *nbytes) {
+    if (!s || index < 0 || index >= (int)s->f->tensors().size()) return HM_ERR_INVALID;
+    const SafeTensorInfo &t = s->f->tensors()[index];
+    if (name_buf && buflen) snprintf(name_buf, buflen, "%s", t.name.c_str());
+    if (dtype_buf) snprintf(dtype_buf, 8, "%s", t.dtype.c_str());
+    if (n_dims) *n_dims = (int)t.shape.size();
+    if (dims)
+        for (size_t i = 0; i < t.shape.size() && i < 8; i++) dims[i] = t.shape[i];
+    if (nbytes) *nbytes = t.end - t.begin;
+    return HM_OK;
+}
+const void *hm_safetensors_tensor_data(const hm_safetensors *s, int index) {
+    if (!s || index < 0 || index >= (int)s->f->tensors().size()) return nullptr;
+    return s->f->data(s->f->tensors()[index]);
+}
+
+int hm_config_from_json(const char *json_text, hm_transformer_config *out, char *err, size_t errlen) {
+    if (!json_text || !out) return HM_ERR_INVALID;
+    TransformerConfig c;
+    std::string e;
+    if (!transformer_config_from_json(json_text, &c, &e)) {
+        copy_err(e, err, errlen);
+        return HM_ERR_INVALID;
+    }
+    fill_c_config(c, out);
+    return HM_OK;
+}
+
+hm_model *hm_model_load_gguf(hm_ctx *ctx, const char *path, int max_seq_len) {
+    if (!ctx || !path) return nullptr;
+    auto impl = load_gguf_model(ctx, path, max_seq_len);
+    if (!impl) return nullptr;
+    return new hm_model{ctx, std::move(impl)};
+}
+
+hm_model *hm_model_load_hf_dir(hm_ctx *ctx, const char *dir, int max_seq_len) {
+    if (!ctx || !dir) return nullptr;
+    auto impl = load_hf_model_dir(ctx, dir, max_seq_len);
+    if (!impl) return nullptr;
+    return new hm_model{ctx, std::move(impl)};
+}
+
+int hm_model_config(hm_model *m, hm_transformer_config *out, int *has_qk_norm, int *weight_dtype) {
+    if (!m || !out) return HM_ERR_INVALID;
+    fill_c_config(m->impl->config(), out);
+    if (has_qk_norm) *has_qk_norm = m->impl->has_qk_norm() ? 1 : 0;
+    if (weight_dtype) *weight_dtype = (int)m->impl->weight_dtype();
+    return HM_OK;
+}
+
+}  // extern "C"

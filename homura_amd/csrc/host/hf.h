@@ -55,10 +55,16 @@ class HfModel {
     ~HfModel();
 
     const TransformerConfig &config() const { return cfg_; }
+    bool has_qk_norm() const { return has_qk_norm_; }
+    DType weight_dtype() const { return weight_dtype_; }
     const std::vector<WeightSlotInfo> &weight_slot_infos() const { return infos_; }
     // Upload one slot (host pointer, exact byte size). bf16 matrices arrive [K][N] and are
     // re-packed once into the K-contiguous stream layout; quantised blocks stay as they are.
-    int set_weight(int slot, const void *h_data, size_t bytes);
+    int set_weight(int slot, const void *h_data, size_t bytes) { return set_weight_impl(slot, h_data, bytes, false); }
+    // Same, but a matrix slot (bf16 projection, LM head) arrives [N][K] - one output row after the
+    // other, K contiguous: the layout of HF safetensors ([out, in]) and of GGUF tensors, and the
+    // stream layout kept in HBM, so nothing is transposed on the way in.
+    int set_weight_nk(int slot, const void *h_data, size_t bytes) { return set_weight_impl(slot, h_data, bytes, true); }
     // reference HfModel::ensure_compiled (src/hf/model.rs:148-160) + RoPE tables (:62-66)
     int finalize(int max_seq_len);
 
@@ -76,6 +82,7 @@ class HfModel {
 
   private:
     HfModel() = default;
+    int set_weight_impl(int slot, const void *h_data, size_t bytes, bool nk_layout);
     int emit_transformer_plan();        // reference src/hf/emitter.rs:867-1050
     int emit_transformer_plan_quant();  // reference src/hf/emitter_quant.rs:1142-1503
     int step_inputs(std::vector<Buffer *> &inputs);

@@ -109,7 +109,7 @@ HfModel::~HfModel() {
     if (ctx_) hm_sync(ctx_);
 }
 
-int HfModel::set_weight(int slot, const void *h_data, size_t bytes) {
+int HfModel::set_weight_impl(int slot, const void *h_data, size_t bytes, bool nk_layout) {
     if (slot < 0 || slot >= (int)infos_.size())
         return hm_set_error(ctx_, HM_ERR_INVALID, "weight slot %d out of range (have %zu)", slot, infos_.size());
     const WeightSlotInfo &info = infos_[slot];
@@ -168,13 +168,19 @@ int HfModel::set_weight(int slot, const void *h_data, size_t bytes) {
 
     if (info.dtype == DType::F32 && nm == "lm_head.weight") {
         // f32 LM head of the quantised plan: [hidden][vocab] -> [vocab][hidden] stream layout
-        Buffer staging = Buffer::alloc_bytes(ctx_, bytes, {info.dim0, info.dim1}, DType::F32);
         lm_head_packed_ = Buffer::alloc(ctx_, {info.dim1, info.dim0}, DType::F32);
-        if (!staging || !lm_head_packed_) return HM_ERR_OOM;
-        int rc = hm_upload(ctx_, staging.ptr(), h_data, bytes);
-        if (rc == HM_OK) rc = pack_f32_kn_to_nk(ctx_, staging.as<float>(), lm_head_packed_.as<float>(),
-                                                (int)info.dim0, (int)info.dim1);
-        if (rc == HM_OK) rc = hm_sync(ctx_);
+        if (!lm_head_packed_) return HM_ERR_OOM;
+        int rc;
+        if (nk_layout) {
+            rc = hm_upload(ctx_, lm_head_packed_.ptr(), h_data, bytes);
+        } else {
+            Buffer staging = Buffer::alloc_bytes(ctx_, bytes, {info.dim0, info.dim1}, DType::F32);
+            if (!staging) return HM_ERR_OOM;
+            rc = hm_upload(ctx_, staging.ptr(), h_data, bytes);
+            if (rc == HM_OK) rc = pack_f32_kn_to_nk(ctx_, staging.as<float>(), lm_head_packed_.as<float>(),
+                                                    (int)info.dim0, (int)info.dim1);
+            if (rc == HM_OK) rc = hm_sync(ctx_);
+        }
         if (rc != HM_OK) return rc;
         weight_bufs_[slot] = Buffer::view(lm_head_packed_.ptr(), bytes, {info.dim1, info.dim0},
                                           {info.dim0, 1}, DType::F32);
@@ -209,11 +215,16 @@ int HfModel::set_weight(int slot, const void *h_data, size_t bytes) {
     }
 
     // bf16 projection [K][N]: stage, then transpose into its place in the packed stream buffers
+    // ([N][K] input goes there as it is)
     const int K = (int)info.dim0, N = (int)info.dim1;
-    Buffer staging = Buffer::alloc_bytes(ctx_, bytes, {K, N}, DType::BF16);
-    if (!staging) return HM_ERR_OOM;
-    int rc = hm_upload(ctx_, staging.ptr(), h_data, bytes);
-    if (rc != HM_OK) return rc;
+    Buffer staging;
+    int rc = HM_OK;
+    if (!nk_layout) {
+        staging = Buffer::alloc_bytes(ctx_, bytes, {K, N}, DType::BF16);
+        if (!staging) return HM_ERR_OOM;
+        rc = hm_upload(ctx_, staging.ptr(), h_data, bytes);
+        if (rc != HM_OK) return rc;
+    }
 
     uint16_t *dst = nullptr;
     int row_mult = 1, row_off = 0;
@@ -249,8 +260,13 @@ int HfModel::set_weight(int slot, const void *h_data, size_t bytes) {
             return hm_set_error(ctx_, HM_ERR_INVALID, "unexpected bf16 weight %s", nm.c_str());
         }
     }
-    rc = pack_bf16_kn_to_nk_strided(ctx_, staging.as<uint16_t>(), dst, K, N, row_mult, row_off);
-    if (rc != HM_OK) return rc;
+    if (nk_layout) {
+        HM_HIP(ctx_, hipMemcpy2DAsync(dst + (size_t)row_off * K, (size_t)K * 2 * row_mult, h_data, (size_t)K * 2,
+                                      (size_t)K * 2, (size_t)N, hipMemcpyHostToDevice, ctx_->stream));
+    } else {
+        rc = pack_bf16_kn_to_nk_strided(ctx_, staging.as<uint16_t>(), dst, K, N, row_mult, row_off);
+        if (rc != HM_OK) return rc;
+    }
     if ((rc = hm_sync(ctx_)) != HM_OK) return rc;
     // the slot buffer is a view of the packed rows ([N][K], K contiguous; interleaved slots
     // have a doubled row stride)

@@ -240,6 +240,35 @@ class HfModel:
         if not self.h:
             raise HomuraError(-1, (self.lib.hm_last_error(ctx.h) or b"").decode())
 
+    @classmethod
+    def _from_handle(cls, ctx: Context, handle) -> "HfModel":
+        if not handle:
+            raise HomuraError(-1, (ctx.lib.hm_last_error(ctx.h) or b"").decode())
+        self = cls.__new__(cls)
+        self.ctx, self.lib, self.h = ctx, ctx.lib, handle
+        c, qkn, wdt = _ffi.HmTransformerConfig(), C.c_int(), C.c_int()
+        self._check(self.lib.hm_model_config(handle, C.byref(c), C.byref(qkn), C.byref(wdt)))
+        self.config = TransformerConfig(
+            hidden_size=c.hidden_size, intermediate_size=c.intermediate_size,
+            num_attention_heads=c.num_attention_heads, num_hidden_layers=c.num_hidden_layers,
+            vocab_size=c.vocab_size, num_key_value_heads=c.num_key_value_heads or None,
+            rms_norm_eps=c.rms_norm_eps, rope_theta=c.rope_theta,
+            max_position_embeddings=c.max_position_embeddings,
+            tie_word_embeddings=bool(c.tie_word_embeddings), head_dim=c.head_dim or None,
+            attention_bias=bool(c.attention_bias))
+        self.has_qk_norm, self.weight_dtype = bool(qkn.value), wdt.value
+        return self
+
+    @classmethod
+    def load_gguf(cls, ctx: Context, path, max_seq_len: int = 0) -> "HfModel":
+        """reference HfModel::load on a GGUF file (src/gguf.rs:589-708): parse, upload, finalize."""
+        return cls._from_handle(ctx, ctx.lib.hm_model_load_gguf(ctx.h, str(path).encode(), max_seq_len))
+
+    @classmethod
+    def load_hf_dir(cls, ctx: Context, model_dir, max_seq_len: int = 0) -> "HfModel":
+        """reference HfModel::load (src/hf/model.rs:75-146): config.json + safetensors."""
+        return cls._from_handle(ctx, ctx.lib.hm_model_load_hf_dir(ctx.h, str(model_dir).encode(), max_seq_len))
+
     def _check(self, rc: int):
         if rc < 0:
             raise HomuraError(rc, (self.lib.hm_last_error(self.ctx.h) or b"").decode())
@@ -265,6 +294,11 @@ class HfModel:
     def set_weight(self, slot: int, arr: np.ndarray):
         a = np.ascontiguousarray(arr)
         self._check(self.lib.hm_model_set_weight(self.h, slot, a.ctypes.data, a.nbytes))
+
+    def set_weight_nk(self, slot: int, arr: np.ndarray):
+        """Like set_weight, but a matrix slot arrives [N, K] (HF [out, in] / GGUF orientation)."""
+        arr = np.ascontiguousarray(arr)
+        self._check(self.lib.hm_model_set_weight_nk(self.h, slot, arr.ctypes.data_as(C.c_void_p), arr.nbytes))
 
     def finalize(self, max_seq_len: int):
         self._check(self.lib.hm_model_finalize(self.h, max_seq_len))

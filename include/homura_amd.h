@@ -253,6 +253,59 @@ int hm_model_time_kernels(hm_model *m, int rounds, hm_kernel_profile *out, int c
 /* Number of HIP kernel launches one decode step issues. */
 int hm_model_launches_per_step(hm_model *m);
 
+/* Same as hm_model_set_weight for every slot except matrices: a bf16 projection or an LM head
+ * arrives [N][K] (one output row after the other, K contiguous) - the layout of HF safetensors
+ * ([out, in]) and of GGUF tensors, and the layout kept in HBM, so nothing is transposed. The
+ * reference transposes these on the host (transpose_2d, src/hf/weights.rs:225-261). */
+int hm_model_set_weight_nk(hm_model *m, int slot, const void *h_data, size_t bytes);
+/* The configuration a model was created or loaded with. */
+int hm_model_config(hm_model *m, hm_transformer_config *out, int *has_qk_norm, int *weight_dtype);
+
+/* ── checkpoint containers (reference src/gguf.rs, src/hf/safetensors.rs, src/hf/config.rs) ──
+ * Host-side readers over a memory mapping; none of them needs a GPU. Open functions return NULL
+ * and write a message into err (if given). */
+typedef struct hm_gguf hm_gguf;
+/* GgufFile::load (src/gguf.rs:345-451): GGUF v2/v3 header, metadata, tensor infos. */
+hm_gguf *hm_gguf_open(const char *path, char *err, size_t errlen);
+void hm_gguf_close(hm_gguf *g);
+int hm_gguf_version(const hm_gguf *g);
+int hm_gguf_num_tensors(const hm_gguf *g);
+size_t hm_gguf_data_offset(const hm_gguf *g); /* start of the aligned tensor data region */
+/* dims come outermost first (the file stores them innermost first, src/gguf.rs:416-422);
+ * ggml_type is the GGML code (0 F32, 1 F16, 2 Q4_0, 8 Q8_0, 12 Q4_K, 14 Q6_K, 30 BF16, ...). */
+int hm_gguf_tensor_info(const hm_gguf *g, int index, char *name_buf, size_t buflen, int *n_dims,
+                        uint64_t dims[8], int *ggml_type, uint64_t *offset, size_t *nbytes);
+int hm_gguf_find_tensor(const hm_gguf *g, const char *name); /* index, -1 when absent */
+const void *hm_gguf_tensor_data(const hm_gguf *g, int index); /* raw bytes in the mapping */
+/* GgufValue::as_str / as_u64 / as_f32 (src/gguf.rs:200-233); HM_ERR_INVALID when the key is
+ * absent or of another kind. hm_gguf_meta_str returns the string length. */
+int hm_gguf_meta_str(const hm_gguf *g, const char *key, char *buf, size_t buflen);
+int hm_gguf_meta_u64(const hm_gguf *g, const char *key, uint64_t *out);
+int hm_gguf_meta_f32(const hm_gguf *g, const char *key, float *out);
+int64_t hm_gguf_meta_array_len(const hm_gguf *g, const char *key); /* -1 when not an array */
+/* GgufFile::transformer_config (src/gguf.rs:508-582). */
+int hm_gguf_transformer_config(const hm_gguf *g, hm_transformer_config *out, int *has_qk_norm, char *err,
+                               size_t errlen);
+
+typedef struct hm_safetensors hm_safetensors;
+/* the container part of load_safetensors_impl (src/hf/safetensors.rs:38-99) */
+hm_safetensors *hm_safetensors_open(const char *path, char *err, size_t errlen);
+void hm_safetensors_close(hm_safetensors *s);
+int hm_safetensors_num_tensors(const hm_safetensors *s);
+int hm_safetensors_tensor_info(const hm_safetensors *s, int index, char *name_buf, size_t buflen,
+                               char dtype_buf[8], int *n_dims, uint64_t dims[8], size_t *nbytes);
+const void *hm_safetensors_tensor_data(const hm_safetensors *s, int index);
+/* TransformerConfig::load on the text of a config.json, with its defaults (src/hf/config.rs:11-54). */
+int hm_config_from_json(const char *json_text, hm_transformer_config *out, char *err, size_t errlen);
+
+/* HfModel::load for a GGUF file (src/gguf.rs:589-708, src/hf/model.rs) and for a directory with
+ * config.json + model.safetensors (or model.safetensors.index.json and its shards)
+ * (src/hf/model.rs:75-146, src/hf/weights.rs:267-417): parse, convert, upload, finalize.
+ * max_seq_len <= 0 picks min(max_position_embeddings, 4096). NULL on failure: hm_last_error(ctx).
+ * GGUF files must be Q8_0, Q4_0 or F32/F16/BF16 throughout their projections. */
+hm_model *hm_model_load_gguf(hm_ctx *ctx, const char *path, int max_seq_len);
+hm_model *hm_model_load_hf_dir(hm_ctx *ctx, const char *dir, int max_seq_len);
+
 /* ── the reference's kernel ABI, literally ─────────────────────────────────
  * The library also exports HM_CIFACE_MAX_KERNELS symbols
  *     void _mlir__mlir_ciface_k0(void **args) ... void _mlir__mlir_ciface_k255(void **args)
