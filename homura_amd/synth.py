@@ -51,6 +51,29 @@ def q4_0_blocks(seed: int, n_blocks: int, d_scale: float = 0.01) -> np.ndarray:
     return out
 
 
+def _f16_scales(rng, n, scale):
+    return np.abs(rng.standard_normal(n) * scale).astype(np.float16).view(np.uint16)
+
+
+def q4_k_blocks(seed: int, n_blocks: int, d_scale: float = 0.001) -> np.ndarray:
+    """Random Q4_K super-blocks (144 B: f16 d, f16 dmin, 12 bytes of 6-bit scales/mins, 128 bytes of
+    nibbles; ggml block_q4_K as the reference reads it, src/gguf.rs:835-882)."""
+    rng = np.random.default_rng(seed)
+    out = rng.integers(0, 256, size=(n_blocks, 144), dtype=np.uint8)
+    out[:, 0:2] = _f16_scales(rng, n_blocks, d_scale).view(np.uint8).reshape(n_blocks, 2)
+    out[:, 2:4] = _f16_scales(rng, n_blocks, d_scale).view(np.uint8).reshape(n_blocks, 2)
+    return out.reshape(-1)
+
+
+def q6_k_blocks(seed: int, n_blocks: int, d_scale: float = 0.0005) -> np.ndarray:
+    """Random Q6_K super-blocks (210 B: 128 bytes low nibbles, 64 bytes high bit pairs, 16 int8
+    scales, f16 d; src/gguf.rs:886-917)."""
+    rng = np.random.default_rng(seed)
+    out = rng.integers(0, 256, size=(n_blocks, 210), dtype=np.uint8)
+    out[:, 208:210] = _f16_scales(rng, n_blocks, d_scale).view(np.uint8).reshape(n_blocks, 2)
+    return out.reshape(-1)
+
+
 def bf16_to_f32(bits: np.ndarray) -> np.ndarray:
     return (bits.astype(np.uint32) << 16).view(np.float32)
 

@@ -15,6 +15,14 @@
  *                           Q4_0 kernel); pinned only by the published ggml block_q4_0
  *                           layout and the formula w=(q-8)*d, cross-checked with an
  *                           independent numpy decode.
+ *   orc_dequant_q4_k / orc_dequant_q6_k .. the reference's dequant functions restated; pinned
+ *                           by hand-built blocks (d=1, sc=1, nibbles=1 => 1.0 per weight;
+ *                           Q6_K nibble 1, sc 1 => -31) and an independent numpy decode of
+ *                           the ggml block_q4_K / block_q6_K layouts
+ *   orc_gemv_q4_k / orc_gemv_q6_k ....... reference KATs emit_q4_k_correctness (128 per
+ *                           output), emit_q6_k_correctness (-7936), and agreement with
+ *                           dequant . x within the Q8_K activation rounding (the
+ *                           reference's own real-weight tests check exactly that)
  *   orc_matmul_* .......... reference exact vectors ([[19,22],[43,50]], identity cases),
  *                           fp64 brute force
  *   orc_rms_norm* ......... reference rms_norm_basic + closed form
@@ -280,6 +288,176 @@ ORC_API void orc_gemv_q4_0(const float *x, const uint8_t *w, float *out, int M, 
             }
             out[(size_t)m * N + n] = acc;
         }
+    }
+}
+
+/* ───────────────────────── K-quants (Q4_K, Q6_K) ───────────────────────── */
+
+/* get_scale_min_k4 as the reference unpacks it (src/gguf.rs:847-862): eight 6-bit scales and
+ * eight 6-bit mins out of 12 bytes. */
+static void q4k_scales(const uint8_t *raw, uint8_t *sc, uint8_t *mn) {
+    for (int i = 0; i < 4; i++) {
+        sc[i] = raw[i] & 0x3F;
+        mn[i] = raw[4 + i] & 0x3F;
+    }
+    for (int i = 0; i < 4; i++) {
+        sc[4 + i] = (uint8_t)((raw[8 + i] & 0x0F) | ((raw[i] >> 6) << 4));
+        mn[4 + i] = (uint8_t)((raw[8 + i] >> 4) | ((raw[4 + i] >> 6) << 4));
+    }
+}
+
+/* src/gguf.rs:835-882 - Q4_K: 256-weight super-blocks of 144 bytes (f16 d, f16 dmin, 12 bytes
+ * of packed scales/mins, 128 bytes of nibbles); sub-blocks come in pairs sharing 32 bytes,
+ * even = low nibbles, odd = high nibbles; w = q * (d*sc) - dmin*mn. */
+ORC_API void orc_dequant_q4_k(const uint8_t *src, size_t nblocks, float *dst) {
+    for (size_t b = 0; b < nblocks; b++) {
+        const uint8_t *blk = src + b * 144;
+        float d = orc_f16_to_f32((uint16_t)(blk[0] | (blk[1] << 8)));
+        float dmin = orc_f16_to_f32((uint16_t)(blk[2] | (blk[3] << 8)));
+        uint8_t sc[8], mn[8];
+        q4k_scales(blk + 4, sc, mn);
+        const uint8_t *qs = blk + 16;
+        for (int pair = 0; pair < 4; pair++) {
+            float scale0 = d * (float)sc[2 * pair], min0 = dmin * (float)mn[2 * pair];
+            float scale1 = d * (float)sc[2 * pair + 1], min1 = dmin * (float)mn[2 * pair + 1];
+            const uint8_t *q = qs + pair * 32;
+            float *o = dst + b * 256 + pair * 64;
+            for (int l = 0; l < 32; l++) o[l] = (float)(q[l] & 0x0F) * scale0 - min0;
+            for (int l = 0; l < 32; l++) o[32 + l] = (float)(q[l] >> 4) * scale1 - min1;
+        }
+    }
+}
+
+/* src/gguf.rs:886-917 - Q6_K: 256-weight super-blocks of 210 bytes (128 bytes low nibbles,
+ * 64 bytes high bit pairs, 16 int8 sub-block scales, f16 d); w = d * sc * (q - 32). */
+ORC_API void orc_dequant_q6_k(const uint8_t *src, size_t nblocks, float *dst) {
+    for (size_t b = 0; b < nblocks; b++) {
+        const uint8_t *blk = src + b * 210;
+        float d = orc_f16_to_f32((uint16_t)(blk[208] | (blk[209] << 8)));
+        for (int chunk = 0; chunk < 2; chunk++) {
+            const uint8_t *ql = blk + chunk * 64, *qh = blk + 128 + chunk * 32;
+            const int8_t *sc = (const int8_t *)(blk + 192 + chunk * 8);
+            float *o = dst + b * 256 + chunk * 128;
+            for (int l = 0; l < 32; l++) {
+                int is = l / 16;
+                int q1 = (int8_t)((ql[l] & 0xF) | (((qh[l] >> 0) & 3) << 4)) - 32;
+                int q2 = (int8_t)((ql[l + 32] & 0xF) | (((qh[l] >> 2) & 3) << 4)) - 32;
+                int q3 = (int8_t)((ql[l] >> 4) | (((qh[l] >> 4) & 3) << 4)) - 32;
+                int q4 = (int8_t)((ql[l + 32] >> 4) | (((qh[l] >> 6) & 3) << 4)) - 32;
+                o[l] = d * (float)sc[is] * (float)q1;
+                o[l + 32] = d * (float)sc[is + 2] * (float)q2;
+                o[l + 64] = d * (float)sc[is + 4] * (float)q3;
+                o[l + 96] = d * (float)sc[is + 6] * (float)q4;
+            }
+        }
+    }
+}
+
+/* The Q8_K quantisation of one 256-wide activation block that both K-quant kernels run first
+ * (src/graph_builder/emit_quant.rs:422-466, :625-652): amax by sequential maximumf,
+ * act_d = amax/127, iscale = 127/amax (0 for an all-zero block), q = roundeven(x*iscale)
+ * clamped to +-127; bsums = sums of 16 consecutive q. */
+ORC_API void orc_quantize_q8_k(const float *x, int8_t *q, float *act_d, int32_t *bsums) {
+    float amax = 0.0f;
+    for (int i = 0; i < 256; i++) {
+        float a = fabsf(x[i]);
+        amax = amax > a ? amax : a; /* arith.maximumf */
+    }
+    *act_d = amax / 127.0f;
+    float iscale = amax == 0.0f ? 0.0f : 127.0f / amax;
+    for (int g = 0; g < 16; g++) bsums[g] = 0;
+    for (int i = 0; i < 256; i++) {
+        float r = nearbyintf(x[i] * iscale); /* math.roundeven under the default rounding mode */
+        r = r < 127.0f ? r : 127.0f;
+        r = r > -127.0f ? r : -127.0f;
+        q[i] = (int8_t)(int32_t)r;
+        bsums[i / 16] += q[i];
+    }
+}
+
+/* src/graph_builder/emit_quant.rs:165-566 - Q4_K x Q8_K: per super-block integer dot products
+ * per sub-block, scale part d*act_d*sum(sc*isum) minus min part dmin*act_d*sum(mn[g/2]*bsums[g]),
+ * blocks accumulated in ascending order in f32. */
+ORC_API void orc_gemv_q4_k(const float *x, const uint8_t *w, float *out, int M, int K, int N) {
+    int nb = K / 256;
+    for (int m = 0; m < M; m++) {
+        int8_t *q8 = (int8_t *)malloc((size_t)K);
+        float *act_d = (float *)malloc((size_t)nb * 4);
+        int32_t *bsums = (int32_t *)malloc((size_t)nb * 16 * 4);
+        for (int kb = 0; kb < nb; kb++)
+            orc_quantize_q8_k(x + (size_t)m * K + kb * 256, q8 + kb * 256, act_d + kb, bsums + kb * 16);
+#pragma omp parallel for schedule(static)
+        for (int n = 0; n < N; n++) {
+            float acc = 0.0f;
+            for (int kb = 0; kb < nb; kb++) {
+                const uint8_t *blk = w + ((size_t)n * nb + kb) * 144;
+                float d = orc_f16_to_f32((uint16_t)(blk[0] | (blk[1] << 8)));
+                float dmin = orc_f16_to_f32((uint16_t)(blk[2] | (blk[3] << 8)));
+                uint8_t sc[8], mn[8];
+                q4k_scales(blk + 4, sc, mn);
+                const uint8_t *qs = blk + 16;
+                const int8_t *a = q8 + kb * 256;
+                int32_t scale_accum = 0;
+                for (int sb = 0; sb < 8; sb++) {
+                    const uint8_t *q = qs + (sb / 2) * 32;
+                    int32_t isum = 0;
+                    for (int l = 0; l < 32; l++) {
+                        int nib = (sb & 1) ? (q[l] >> 4) : (q[l] & 0x0F);
+                        isum += nib * (int32_t)a[sb * 32 + l];
+                    }
+                    scale_accum += (int32_t)sc[sb] * isum;
+                }
+                int32_t min_accum = 0;
+                for (int g = 0; g < 16; g++) min_accum += (int32_t)mn[g / 2] * bsums[kb * 16 + g];
+                float scale_part = (d * act_d[kb]) * (float)scale_accum;
+                float min_part = (dmin * act_d[kb]) * (float)min_accum;
+                acc = acc + (scale_part - min_part);
+            }
+            out[(size_t)m * N + n] = acc;
+        }
+        free(q8);
+        free(act_d);
+        free(bsums);
+    }
+}
+
+/* src/graph_builder/emit_quant.rs:569-816 - Q6_K x Q8_K: 16 sub-blocks of 16 weights,
+ * q = (low nibble | high pair << 4) - 32, sum(sc[sb]*isum) in i32, times d*act_d. */
+ORC_API void orc_gemv_q6_k(const float *x, const uint8_t *w, float *out, int M, int K, int N) {
+    int nb = K / 256;
+    for (int m = 0; m < M; m++) {
+        int8_t *q8 = (int8_t *)malloc((size_t)K);
+        float *act_d = (float *)malloc((size_t)nb * 4);
+        int32_t bs[16];
+        for (int kb = 0; kb < nb; kb++)
+            orc_quantize_q8_k(x + (size_t)m * K + kb * 256, q8 + kb * 256, act_d + kb, bs);
+#pragma omp parallel for schedule(static)
+        for (int n = 0; n < N; n++) {
+            float acc = 0.0f;
+            for (int kb = 0; kb < nb; kb++) {
+                const uint8_t *blk = w + ((size_t)n * nb + kb) * 210;
+                float d = orc_f16_to_f32((uint16_t)(blk[208] | (blk[209] << 8)));
+                const int8_t *sc = (const int8_t *)(blk + 192);
+                const int8_t *a = q8 + kb * 256;
+                int32_t scale_accum = 0;
+                for (int sb = 0; sb < 16; sb++) {
+                    int chunk = sb / 8, sic = sb % 8, group = sic / 2, parity = sic % 2;
+                    const uint8_t *ql = blk + chunk * 64 + (group & 1) * 32 + parity * 16;
+                    const uint8_t *qh = blk + 128 + chunk * 32 + parity * 16;
+                    int32_t isum = 0;
+                    for (int l = 0; l < 16; l++) {
+                        int lo = group >= 2 ? (ql[l] >> 4) : (ql[l] & 0x0F);
+                        int hi = (qh[l] >> (2 * group)) & 3;
+                        isum += ((lo | (hi << 4)) - 32) * (int32_t)a[sb * 16 + l];
+                    }
+                    scale_accum += (int32_t)sc[sb] * isum;
+                }
+                acc = acc + (d * act_d[kb]) * (float)scale_accum;
+            }
+            out[(size_t)m * N + n] = acc;
+        }
+        free(q8);
+        free(act_d);
     }
 }
 

@@ -49,6 +49,11 @@ def load() -> C.CDLL:
         "orc_f32_to_bf16_trunc": (C.c_uint16, [_F]),
         "orc_f32_to_bf16_rne": (C.c_uint16, [_F]),
         "orc_dequant_q8_0": (None, [_P, C.c_size_t, _P]),
+        "orc_dequant_q4_k": (None, [_P, C.c_size_t, _P]),
+        "orc_dequant_q6_k": (None, [_P, C.c_size_t, _P]),
+        "orc_quantize_q8_k": (None, [_P, _P, _P, _P]),
+        "orc_gemv_q4_k": (None, [_P, _P, _P, _I, _I, _I]),
+        "orc_gemv_q6_k": (None, [_P, _P, _P, _I, _I, _I]),
         "orc_dequant_q4_0": (None, [_P, C.c_size_t, _P]),
         "orc_matmul_f32_bf16": (None, [_P, _P, _P, _I, _I, _I]),
         "orc_matmul_f32_f32": (None, [_P, _P, _P, _I, _I, _I]),
@@ -124,6 +129,44 @@ def dequant_q8_0(blocks: np.ndarray) -> np.ndarray:
     out = np.empty(nb * 32, np.float32)
     load().orc_dequant_q8_0(_p(blocks), nb, _p(out))
     return out
+
+
+def dequant_q4_k(blocks: np.ndarray) -> np.ndarray:
+    nb = blocks.size // 144
+    out = np.empty(nb * 256, np.float32)
+    load().orc_dequant_q4_k(_p(blocks), nb, _p(out))
+    return out
+
+
+def dequant_q6_k(blocks: np.ndarray) -> np.ndarray:
+    nb = blocks.size // 210
+    out = np.empty(nb * 256, np.float32)
+    load().orc_dequant_q6_k(_p(blocks), nb, _p(out))
+    return out
+
+
+def quantize_q8_k(x: np.ndarray):
+    """(q int8[256], act_d, bsums int32[16]) of one 256-wide block."""
+    x = np.ascontiguousarray(x, np.float32)
+    q, d, bs = np.empty(256, np.int8), np.empty(1, np.float32), np.empty(16, np.int32)
+    load().orc_quantize_q8_k(_p(x), _p(q), _p(d), _p(bs))
+    return q, float(d[0]), bs
+
+
+def _gemv_k(fn, x, w, M, K, N):
+    x = np.ascontiguousarray(x, np.float32)
+    w = np.ascontiguousarray(w, np.uint8)
+    out = np.empty((M, N), np.float32)
+    fn(_p(x), _p(w), _p(out), M, K, N)
+    return out
+
+
+def gemv_q4_k(x, w, M, K, N):
+    return _gemv_k(load().orc_gemv_q4_k, x, w, M, K, N)
+
+
+def gemv_q6_k(x, w, M, K, N):
+    return _gemv_k(load().orc_gemv_q6_k, x, w, M, K, N)
 
 
 def dequant_q4_0(blocks: np.ndarray) -> np.ndarray:

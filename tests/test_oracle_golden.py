@@ -393,3 +393,144 @@ def test_config_vectors(golden):
                              num_hidden_layers=24, vocab_size=151936, num_key_value_heads=2)
     assert (cfg2.kv_heads(), cfg2.get_head_dim(), cfg2.gqa_repeat()) == (2, 64, 7)
     assert g2["expect_gqa_repeat"] == 7
+
+
+# ── K-quants: Q4_K, Q6_K (reference src/gguf.rs:835-917, src/graph_builder/emit_quant.rs:165-816) ──
+
+def _np_dequant_q4_k(raw):
+    """Independent decode of ggml block_q4_K written from the format description: 8 sub-blocks of
+    32; sub-block j of a super-block takes the low (j even) or high (j odd) nibbles of the 32 bytes
+    at qs[32*(j//2)]; 6-bit scale/min j come from the 12 packed bytes."""
+    blocks = raw.reshape(-1, 144)
+    out = np.empty((len(blocks), 256), np.float64)
+    for b, blk in enumerate(blocks):
+        d, dmin = (float(x) for x in blk[0:4].view(np.float16))
+        p = blk[4:16].astype(int)
+        for j in range(8):
+            if j < 4:
+                sc, mn = p[j] & 63, p[j + 4] & 63
+            else:
+                sc = (p[j + 4] & 15) | ((p[j - 4] >> 6) << 4)
+                mn = (p[j + 4] >> 4) | ((p[j] >> 6) << 4)
+            q = blk[16 + 32 * (j // 2): 16 + 32 * (j // 2) + 32].astype(int)
+            nib = (q >> 4) if j % 2 else (q & 15)
+            out[b, 32 * j: 32 * j + 32] = d * sc * nib - dmin * mn
+    return out.reshape(-1)
+
+
+def _np_dequant_q6_k(raw):
+    """Independent decode of ggml block_q6_K: element e of a super-block lives in half h = e // 128,
+    quarter g = (e % 128) // 32, position l = e % 32: low nibble from ql[64 h + 32 (g % 2) + l]
+    (upper nibble when g >= 2), bit pair g of qh[32 h + l], scale sc[8 h + 2 g + l // 16]."""
+    blocks = raw.reshape(-1, 210)
+    out = np.empty((len(blocks), 256), np.float64)
+    for b, blk in enumerate(blocks):
+        d = float(blk[208:210].view(np.float16)[0])
+        ql, qh, sc = blk[0:128].astype(int), blk[128:192].astype(int), blk[192:208].view(np.int8).astype(int)
+        for e in range(256):
+            h, g, l = e // 128, (e % 128) // 32, e % 32
+            lo = ql[64 * h + 32 * (g % 2) + l]
+            lo = (lo >> 4) if g >= 2 else (lo & 15)
+            hi = (qh[32 * h + l] >> (2 * g)) & 3
+            out[b, e] = d * sc[8 * h + 2 * g + l // 16] * ((lo | (hi << 4)) - 32)
+    return out.reshape(-1)
+
+
+def _q4k_kat_block():
+    """The block of the reference's emit_q4_k_correctness (src/graph_builder/emit_quant.rs:1018-1078):
+    d = 1.0, dmin = 0, scales_raw[0..3] = 1, every nibble 1."""
+    blk = np.zeros(144, np.uint8)
+    blk[0:2] = (0x00, 0x3C)
+    blk[4:8] = 1
+    blk[16:144] = 0x11
+    return blk
+
+
+def test_q4_k_reference_kat(oracle):
+    w = np.tile(_q4k_kat_block(), 4)
+    out = oracle.gemv_q4_k(np.ones(256, np.float32), w, 1, 256, 4)
+    assert np.allclose(out, 128.0, atol=1e-3)          # reference asserts |out - 128| < 1
+    deq = oracle.dequant_q4_k(w)[:256]
+    assert np.array_equal(deq[:128], np.ones(128, np.float32)) and not deq[128:].any()
+
+
+def test_q6_k_reference_kat(oracle):
+    """emit_q6_k_correctness (src/graph_builder/emit_quant.rs:1286-1360): d = 1, sc = 1, low nibbles 1,
+    high bits 0 -> every weight -31, 256 * -31 = -7936."""
+    blk = np.zeros(210, np.uint8)
+    blk[208:210] = (0x00, 0x3C)
+    blk[192:208] = 1
+    blk[0:128] = 0x11
+    w = np.tile(blk, 4)
+    out = oracle.gemv_q6_k(np.ones(256, np.float32), w, 1, 256, 4)
+    assert np.allclose(out, -7936.0, atol=1e-2)
+    assert np.array_equal(oracle.dequant_q6_k(w), np.full(1024, -31.0, np.float32))
+
+
+def test_q4_k_reference_realistic_case(oracle):
+    """emit_q4_k_correctness_realistic (src/graph_builder/emit_quant.rs:1105-1224): d = 0.5,
+    dmin = 0.25, sc = 5/10/15/20, mn = 2/4/6/8, patterned nibbles, activation all ones; the kernel
+    must equal the row sum of the dequantised weights (the reference allows 1 % or 0.1)."""
+    rows = []
+    for b in range(2):
+        blk = np.zeros(144, np.uint8)
+        blk[0:4] = (0x00, 0x38, 0x00, 0x34)
+        blk[4:12] = (5, 10, 15, 20, 2, 4, 6, 8)
+        qi = np.arange(128)
+        blk[16:144] = ((qi * 3 + b * 7) % 16) | (((qi * 5 + b * 11) % 16) << 4)
+        rows.append(blk)
+    w = np.concatenate(rows)
+    out = oracle.gemv_q4_k(np.ones(256, np.float32), w, 1, 256, 2)[0]
+    ref = _np_dequant_q4_k(w).reshape(2, 256).sum(1)
+    assert np.all(np.abs(out - ref) < np.maximum(0.01 * np.abs(ref), 0.1))
+    # with an activation of ones the Q8_K quantisation is exact (every q8 = 127): equality to rounding
+    assert np.allclose(out, ref, rtol=1e-6)
+
+
+def test_kquant_dequant_against_independent_decode(oracle):
+    from homura_amd import synth
+    w4 = synth.q4_k_blocks(11, 37)
+    assert np.allclose(oracle.dequant_q4_k(w4), _np_dequant_q4_k(w4), rtol=1e-6, atol=1e-9)
+    w6 = synth.q6_k_blocks(12, 29)
+    assert np.allclose(oracle.dequant_q6_k(w6), _np_dequant_q6_k(w6), rtol=1e-6, atol=1e-9)
+
+
+def test_q8_k_activation_quantisation(oracle):
+    """amax/127 scale, round half to even, clamp, sums of 16 (emit_quant.rs:422-466)."""
+    x = np.zeros(256, np.float32)
+    q, d, bs = oracle.quantize_q8_k(x)
+    assert d == 0.0 and not q.any() and not bs.any()          # iscale = 0 for an all-zero block
+    x[0] = 127.0                                               # iscale = 1: values map to themselves
+    x[1:6] = (0.5, 1.5, 2.5, -0.5, -3.5)
+    x[16:20] = (100.0, -127.0, 126.49, 3.0)
+    q, d, bs = oracle.quantize_q8_k(x)
+    assert d == 1.0
+    assert q[:6].tolist() == [127, 0, 2, 2, 0, -4]             # ties go to the even neighbour
+    assert q[16:20].tolist() == [100, -127, 126, 3]
+    assert bs[0] == int(q[:16].astype(int).sum()) and bs[1] == 102 and not bs[2:].any()
+    rng = np.random.default_rng(5)
+    x = rng.standard_normal(256).astype(np.float32)
+    q, d, bs = oracle.quantize_q8_k(x)
+    assert np.abs(q).max() == 127 and np.abs(q.astype(np.float64) * d - x).max() <= d / 2 + 1e-7
+    assert np.array_equal(bs, q.astype(np.int32).reshape(16, 16).sum(1))
+
+
+@pytest.mark.parametrize("kind", ["q4_k", "q6_k"])
+def test_kquant_gemv_against_dequantised_product(oracle, kind):
+    """What the reference's real-weight tests check (emit_quant.rs:1363-1500): the integer-dot kernel
+    agrees with dequantise-then-multiply up to the Q8_K rounding of the activation. A wrong sub-block
+    order, nibble half or scale index would be off by O(1), not by a fraction of a percent."""
+    from homura_amd import synth
+    K, N = 512, 24
+    w = (synth.q4_k_blocks if kind == "q4_k" else synth.q6_k_blocks)(21, N * K // 256)
+    x = np.random.default_rng(3).standard_normal((2, K)).astype(np.float32)
+    got = (oracle.gemv_q4_k if kind == "q4_k" else oracle.gemv_q6_k)(x, w, 2, K, N)
+    deq = (_np_dequant_q4_k if kind == "q4_k" else _np_dequant_q6_k)(w).reshape(N, K)
+    want = x.astype(np.float64) @ deq.T
+    err = np.abs(got - want).max() / np.abs(want).max()
+    assert err < 1e-2, err
+    # and exactly: the same integers through numpy int64 arithmetic and one float per block
+    xq = [[oracle.quantize_q8_k(x[m, kb * 256:(kb + 1) * 256]) for kb in range(K // 256)] for m in range(2)]
+    xdq = np.array([np.concatenate([q.astype(np.float64) * d for q, d, _ in row]) for row in xq])
+    exact = xdq @ deq.T
+    assert np.abs(got - exact).max() / np.abs(exact).max() < 1e-5
