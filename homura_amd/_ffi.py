@@ -73,6 +73,11 @@ SIGNATURES = {
     "hm_gemv_q4_0": (_I, [_P, _P, _P, _P, _I, _I, _I]),
     "hm_dequant_q8_0": (_I, [_P, _P, _P, _SZ]),
     "hm_dequant_q4_0": (_I, [_P, _P, _P, _SZ]),
+    "hm_gemv_q4_k": (_I, [_P, _P, _P, _P, _I, _I, _I]),
+    "hm_gemv_q6_k": (_I, [_P, _P, _P, _P, _I, _I, _I]),
+    "hm_quantize_q8_k": (_I, [_P, _P, _P, _P, _P, _I, _I]),
+    "hm_dequant_q4_k": (_I, [_P, _P, _P, _SZ]),
+    "hm_dequant_q6_k": (_I, [_P, _P, _P, _SZ]),
     "hm_gemm_bf16": (_I, [_P, _P, _P, _P, _I, _I, _I]),
     "hm_gemm_bf16_nk": (_I, [_P, _P, _P, _P, _I, _I, _I]),
     "hm_model_set_weight_nk": (_I, [_P, _I, _P, _SZ]),

@@ -1,0 +1,379 @@
+// GGUF K-quants (Q4_K, Q6_K): activation quantisation to Q8_K, integer-dot GEMV, and bit-exact
+// block dequantisation (reference src/graph_builder/emit_quant.rs:165-816, src/gguf.rs:835-917).
+//
+// The reference multiplies these weights against an activation quantised to int8 per 256-wide
+// block (Q8_K: scale amax/127, round half to even) with integer dot products per sub-block; the
+// GPU does the same arithmetic - the integer sums are identical, only the order of the f32 adds
+// differs - with v_dot4_i32_i8 doing four multiply-adds per instruction.
+//
+// Weights stay the raw GGUF super-blocks, rows of K/256 blocks. A workgroup copies a run of rows
+// into LDS with aligned 16-byte loads (the next run travels in registers meanwhile). The unit of
+// work of a lane is 16 weights: one sub-block half of Q4_K (16 bytes, low or high nibbles) or one
+// sub-block of Q6_K. Units are dealt to the lanes round-robin (K/16 per row, so K = 1024 fills the
+// wavefront exactly); a lane keeps the 16 int8 activations of each of its units, their sum and
+// the block's activation scale in registers for the life of the workgroup and walks the rows.
+#include "hm_common.h"
+
+namespace {
+
+constexpr int KTHREADS = 256;
+constexpr int KWAVES = KTHREADS / WAVE;
+constexpr int KMAX_ROWS = KWAVES * 8;
+constexpr int KSTAGE_U = 8;                            // 16-byte chunks a thread carries per row step
+constexpr int KSTAGE_BYTES = KTHREADS * KSTAGE_U * 16; // most bytes one row step may span
+constexpr int KMAXC = 8;                               // unit rounds a lane keeps in registers (K <= 8192)
+
+template <int QT>
+struct KTraits;
+template <>
+struct KTraits<0> {  // Q4_K
+    static constexpr int BYTES = 144;
+};
+template <>
+struct KTraits<1> {  // Q6_K
+    static constexpr int BYTES = 210;
+};
+
+__device__ __forceinline__ uint32_t lds16(const uint8_t *p) { return *reinterpret_cast<const uint16_t *>(p); }
+__device__ __forceinline__ uint32_t lds32_a2(const uint8_t *p) { return lds16(p) | (lds16(p + 2) << 16); }
+
+// ── Q8_K quantisation of the activation: one wavefront per 256-wide block ──
+// (emit_quant.rs:422-466) amax, act_d = amax / 127, iscale = 127 / amax (0 for a zero block),
+// q = roundeven(x * iscale) clamped to +-127, bsums = sums of 16 consecutive q.
+__global__ __launch_bounds__(WAVE) void quantize_q8_k_kernel(const float *__restrict__ x, int8_t *__restrict__ q8,
+                                                             float *__restrict__ act_d, int *__restrict__ bsums) {
+    const int lane = threadIdx.x;
+    const size_t blk = blockIdx.x;
+    const f32x4 v = *reinterpret_cast<const f32x4 *>(x + blk * 256 + lane * 4);
+    float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+    amax = wave_max(amax);
+    const float iscale = amax == 0.f ? 0.f : __fdiv_rn(127.0f, amax);
+    int q[4];
+    const float xs[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        float r = rintf(__fmul_rn(xs[i], iscale));  // round half to even
+        r = fminf(r, 127.0f);
+        r = fmaxf(r, -127.0f);
+        q[i] = (int)r;
+    }
+    const uint32_t packed = (uint32_t)(q[0] & 0xFF) | ((uint32_t)(q[1] & 0xFF) << 8) | ((uint32_t)(q[2] & 0xFF) << 16) |
+                            ((uint32_t)(q[3] & 0xFF) << 24);
+    *reinterpret_cast<uint32_t *>(q8 + blk * 256 + lane * 4) = packed;
+    // 16 consecutive values = four adjacent lanes
+    int s = q[0] + q[1] + q[2] + q[3];
+    s += __builtin_amdgcn_update_dpp(0, s, 0xB1, 0xF, 0xF, false);  // quad_perm [1,0,3,2]
+    s += __builtin_amdgcn_update_dpp(0, s, 0x4E, 0xF, 0xF, false);  // quad_perm [2,3,0,1]
+    if ((lane & 3) == 0) bsums[blk * 16 + (lane >> 2)] = s;
+    if (lane == 0) act_d[blk] = __fdiv_rn(amax, 127.0f);
+}
+
+// What a lane keeps of the activation for one of its 16-weight units.
+struct ActUnit {
+    uint32_t q[4];  // 16 int8
+    int bsum;       // their sum
+    float d;        // activation scale of the unit's 256-block
+};
+
+__device__ __forceinline__ int dot16(const uint32_t *w, const uint32_t *a) {
+    int s = 0;
+#pragma unroll
+    for (int i = 0; i < 4; i++) s = __builtin_amdgcn_sdot4((int)w[i], (int)a[i], s, false);
+    return s;
+}
+
+// One Q4_K unit: i = unit index inside the super-block (0..15) = 2 * sub-block + half.
+// Sub-blocks come in pairs sharing 32 bytes, even = low nibbles, odd = high nibbles; scale and min
+// of sub-block sb unpack from the 12 packed bytes as in get_scale_min_k4 (src/gguf.rs:847-862).
+__device__ __forceinline__ float q4k_unit(const uint8_t *blk, int i, const ActUnit &a) {
+    const int sb = i >> 1, h = i & 1, pair = sb >> 1, odd = sb & 1;
+    const uint32_t hdr = *reinterpret_cast<const uint32_t *>(blk);  // d | dmin << 16
+    const float d = f16_bits_to_f32((uint16_t)(hdr & 0xFFFFu)), dmin = f16_bits_to_f32((uint16_t)(hdr >> 16));
+    const uint8_t *raw = blk + 4;
+    int sc, mn;
+    if (sb < 4) {
+        sc = raw[sb] & 63;
+        mn = raw[sb + 4] & 63;
+    } else {
+        const int hi = raw[sb + 4];
+        sc = (hi & 15) | ((raw[sb - 4] >> 6) << 4);
+        mn = (hi >> 4) | ((raw[sb] >> 6) << 4);
+    }
+    const u32x4 w = *reinterpret_cast<const u32x4 *>(blk + 16 + pair * 32 + h * 16);
+    const int sh = odd * 4;
+    const uint32_t nib[4] = {(w.x >> sh) & 0x0F0F0F0Fu, (w.y >> sh) & 0x0F0F0F0Fu, (w.z >> sh) & 0x0F0F0F0Fu,
+                             (w.w >> sh) & 0x0F0F0F0Fu};
+    const int isum = dot16(nib, a.q);
+    // d*act_d*(sc*isum) - dmin*act_d*(mn*bsum): the unit's share of the block's scale and min parts
+    return (d * a.d) * (float)(sc * isum) - (dmin * a.d) * (float)(mn * a.bsum);
+}
+
+// One Q6_K unit: i = sub-block (0..15); chunk = i/8, group = (i%8)/2, parity = i%2:
+// low nibbles at ql[64 chunk + 32 (group&1) + 16 parity ..] (upper nibble for group >= 2), bit pair
+// `group` of qh[32 chunk + 16 parity ..], q = (lo | hi << 4) - 32 (emit_quant.rs:668-760).
+__device__ __forceinline__ float q6k_unit(const uint8_t *blk, int i, const ActUnit &a) {
+    const int chunk = i >> 3, group = (i & 7) >> 1, parity = i & 1;
+    const uint8_t *ql = blk + chunk * 64 + (group & 1) * 32 + parity * 16;
+    const uint8_t *qh = blk + 128 + chunk * 32 + parity * 16;
+    const int lo_sh = group >= 2 ? 4 : 0, hi_sh = group * 2;
+    uint32_t v[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const uint32_t l = lds32_a2(ql + 4 * j), hgh = lds32_a2(qh + 4 * j);
+        v[j] = ((l >> lo_sh) & 0x0F0F0F0Fu) | (((hgh >> hi_sh) & 0x03030303u) << 4);
+    }
+    const int isum = dot16(v, a.q) - 32 * a.bsum;
+    const int sc = (int)(int8_t)blk[192 + i];
+    const float d = f16_bits_to_f32((uint16_t)lds16(blk + 208));
+    return (d * a.d) * (float)(sc * isum);
+}
+
+struct StepRange {
+    size_t abeg;
+    int shift, nchunks, r0, nrows;
+};
+// The aligned 16-byte chunks covering rows [r0, r0+nrows). A chunk that holds at least one byte of
+// the buffer lies in that byte's page, so whole aligned chunks at the buffer's ends cannot fault.
+__device__ __forceinline__ StepRange step_range(int step, int rows_per_step, int N, size_t rowbytes) {
+    StepRange r;
+    r.r0 = step * rows_per_step;
+    r.nrows = min(rows_per_step, N - r.r0);
+    const size_t beg = (size_t)r.r0 * rowbytes, end = beg + (size_t)r.nrows * rowbytes;
+    r.abeg = beg & ~(size_t)15;
+    r.shift = (int)(beg - r.abeg);
+    r.nchunks = (int)((end - r.abeg + 15) / 16);
+    return r;
+}
+
+// RT rows lr, lr + KWAVES, ... of the staged step for one wavefront. Round t of a lane is unit
+// lane + 64 t of the row: block (lane + 64 t) / 16 = lane/16 + 4 t, unit-in-block lane % 16.
+template <int QT, int CPL, int RT>
+__device__ __forceinline__ void krows_trip(const uint8_t *base, size_t rowbytes, int lr, int lane, int nu,
+                                           const ActUnit (&act)[CPL], float *out) {
+    constexpr int BB = KTraits<QT>::BYTES;
+    const int boff = (lane >> 4) * BB, ui = lane & 15;
+    float a[RT];
+#pragma unroll
+    for (int j = 0; j < RT; j++) a[j] = 0.f;
+#pragma unroll
+    for (int t = 0; t < CPL; t++) {
+        const bool live = lane + t * WAVE < nu;
+#pragma unroll
+        for (int j = 0; j < RT; j++) {
+            // lanes past the row end read the block of unit 0..15 of the row start: valid memory, dropped below
+            const uint8_t *blk = base + (size_t)(lr + j * KWAVES) * rowbytes + (live ? boff + t * 4 * BB : 0);
+            const float v = QT == 0 ? q4k_unit(blk, ui, act[t]) : q6k_unit(blk, ui, act[t]);
+            a[j] += live ? v : 0.f;
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    }
+#pragma unroll
+    for (int j = 0; j < RT; j++) {
+        a[j] = wave_sum(a[j]);
+        if (lane == 0) out[lr + j * KWAVES] = a[j];
+    }
+}
+
+template <int QT, int CPL>
+__global__ __launch_bounds__(KTHREADS) void gemv_kquant_kernel(const int8_t *__restrict__ q8,
+                                                               const float *__restrict__ act_d,
+                                                               const int *__restrict__ bsums,
+                                                               const uint8_t *__restrict__ w, float *__restrict__ out,
+                                                               int K, int N, int rows_per_step) {
+    constexpr int BB = KTraits<QT>::BYTES;
+    constexpr int U = KSTAGE_U;
+    extern __shared__ __attribute__((aligned(16))) uint8_t ws[];
+    const int tid = threadIdx.x, lane = tid & (WAVE - 1), wave = tid / WAVE;
+    const int nb = K / 256, nu = K / 16;
+    const size_t rowbytes = (size_t)nb * BB;
+    const int nsteps = (N + rows_per_step - 1) / rows_per_step;
+
+    // the lane's share of the quantised activation first (small, cached), the first row step behind it
+    ActUnit act[CPL];
+#pragma unroll
+    for (int t = 0; t < CPL; t++) {
+        const int u = min(lane + t * WAVE, nu - 1);
+        const u32x4 q = *reinterpret_cast<const u32x4 *>(q8 + (size_t)u * 16);
+        act[t].q[0] = q.x; act[t].q[1] = q.y; act[t].q[2] = q.z; act[t].q[3] = q.w;
+        act[t].bsum = bsums[u];
+        act[t].d = act_d[u >> 4];
+    }
+    u32x4 tmp[U];
+    int step = blockIdx.x;
+    StepRange cur = step_range(step, rows_per_step, N, rowbytes);
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+        const int i = tid + u * KTHREADS;
+        tmp[u] = i < cur.nchunks ? ld128_stream(w + cur.abeg + (size_t)i * 16) : u32x4{0u, 0u, 0u, 0u};
+    }
+
+    for (; step < nsteps; step += gridDim.x) {
+        __syncthreads();  // previous step's readers are done with ws
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const int i = tid + u * KTHREADS;
+            if (i < cur.nchunks) *reinterpret_cast<u32x4 *>(ws + (size_t)i * 16) = tmp[u];
+        }
+        __syncthreads();
+        const StepRange now = cur;
+        if (step + (int)gridDim.x < nsteps) {  // the next step's weights travel while this one is multiplied
+            cur = step_range(step + gridDim.x, rows_per_step, N, rowbytes);
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                const int i = tid + u * KTHREADS;
+                tmp[u] = i < cur.nchunks ? ld128_stream(w + cur.abeg + (size_t)i * 16) : u32x4{0u, 0u, 0u, 0u};
+            }
+        }
+        const uint8_t *base = ws + now.shift;
+        float *o = out + now.r0;
+        int lr = wave;
+        for (; lr + 3 * KWAVES < now.nrows; lr += 4 * KWAVES) krows_trip<QT, CPL, 4>(base, rowbytes, lr, lane, nu, act, o);
+        if (lr + KWAVES < now.nrows) {
+            krows_trip<QT, CPL, 2>(base, rowbytes, lr, lane, nu, act, o);
+            lr += 2 * KWAVES;
+        }
+        if (lr < now.nrows) krows_trip<QT, CPL, 1>(base, rowbytes, lr, lane, nu, act, o);
+    }
+}
+
+// One thread per weight, the reference's arithmetic step by step (no contraction) so the bits match
+// the CPU: Q4_K w = q * (d * sc) - dmin * mn; Q6_K w = (d * sc) * q (src/gguf.rs:835-917).
+template <int QT>
+__global__ __launch_bounds__(256) void dequant_kquant_kernel(const uint8_t *__restrict__ blocks,
+                                                             float *__restrict__ out, size_t n_elems) {
+    constexpr int BB = KTraits<QT>::BYTES;
+    size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (; e < n_elems; e += stride) {
+        const uint8_t *blk = blocks + (e >> 8) * BB;
+        const int j = (int)(e & 255);
+        if (QT == 0) {
+            const float d = f16_bits_to_f32((uint16_t)(blk[0] | (blk[1] << 8)));
+            const float dmin = f16_bits_to_f32((uint16_t)(blk[2] | (blk[3] << 8)));
+            const uint8_t *raw = blk + 4;
+            const int sb = j >> 5, l = j & 31;
+            int sc, mn;
+            if (sb < 4) {
+                sc = raw[sb] & 63;
+                mn = raw[sb + 4] & 63;
+            } else {
+                sc = (raw[sb + 4] & 15) | ((raw[sb - 4] >> 6) << 4);
+                mn = (raw[sb + 4] >> 4) | ((raw[sb] >> 6) << 4);
+            }
+            const uint8_t byte = blk[16 + (sb >> 1) * 32 + l];
+            const int q = (sb & 1) ? (byte >> 4) : (byte & 15);
+            out[e] = __fsub_rn(__fmul_rn((float)q, __fmul_rn(d, (float)sc)), __fmul_rn(dmin, (float)mn));
+        } else {
+            const float d = f16_bits_to_f32((uint16_t)(blk[208] | (blk[209] << 8)));
+            const int h = j >> 7, g = (j & 127) >> 5, l = j & 31;
+            const uint8_t lb = blk[64 * h + 32 * (g & 1) + l];
+            const int lo = g >= 2 ? (lb >> 4) : (lb & 15);
+            const int hi = (blk[128 + 32 * h + l] >> (2 * g)) & 3;
+            const int q = (int)(int8_t)(lo | (hi << 4)) - 32;
+            const int sc = (int)(int8_t)blk[192 + 8 * h + 2 * g + (l >> 4)];
+            out[e] = __fmul_rn(__fmul_rn(d, (float)sc), (float)q);
+        }
+    }
+}
+
+int quantize_launch(hm_ctx *ctx, const float *d_x, int8_t *q8, float *act_d, int *bsums, int M, int K) {
+    hipLaunchKernelGGL(quantize_q8_k_kernel, dim3((unsigned)((size_t)M * K / 256)), dim3(WAVE), 0, ctx->stream, d_x, q8,
+                       act_d, bsums);
+    HM_LAUNCH_CHECK(ctx);
+    return HM_OK;
+}
+
+template <int QT>
+int gemv_kquant_launch(hm_ctx *ctx, const char *name, const float *d_x, const uint8_t *d_w, float *d_out, int M, int K,
+                       int N) {
+    HM_CHECK_CTX(ctx);
+    constexpr int BB = KTraits<QT>::BYTES;
+    HM_REQUIRE(ctx, d_x && d_w && d_out, "%s: NULL pointer", name);
+    HM_REQUIRE(ctx, M >= 1 && M <= 8, "%s: M=%d outside 1..8", name, M);
+    HM_REQUIRE(ctx, K > 0 && K % 256 == 0 && N > 0, "%s: K=%d must be a positive multiple of 256, N=%d positive", name, K, N);
+    HM_REQUIRE(ctx, K <= KMAXC * WAVE * 16, "%s: K=%d above %d", name, K, KMAXC * WAVE * 16);
+    HM_REQUIRE(ctx, ((uintptr_t)d_w % 16) == 0 && ((uintptr_t)d_x % 16) == 0, "%s: weight and activation buffers must be 16-byte aligned", name);
+    const size_t rowbytes = (size_t)(K / 256) * BB;
+    HM_REQUIRE(ctx, KWAVES * rowbytes + 32 <= (size_t)KSTAGE_BYTES, "%s: K=%d too large for the LDS stage", name, K);
+    // the quantised activation lives at the top of the workspace: q8 | act_d | bsums per activation row
+    const size_t per_m = ((size_t)K + (size_t)K / 256 * 4 + (size_t)K / 16 * 4 + 255) & ~(size_t)255;
+    HM_REQUIRE(ctx, per_m * M <= ctx->workspace_bytes, "%s: workspace too small", name);
+    uint8_t *wsp = (uint8_t *)ctx->workspace + ctx->workspace_bytes - per_m * M;
+
+    int rows = (int)(((size_t)40 * 1024) / rowbytes);
+    rows = rows / KWAVES * KWAVES;
+    if (rows < KWAVES) rows = KWAVES;
+    if (rows > KMAX_ROWS) rows = KMAX_ROWS;
+    while (rows > KWAVES && (size_t)rows * rowbytes + 32 > (size_t)KSTAGE_BYTES) rows -= KWAVES;
+    while (rows > KWAVES && (N + rows - 1) / rows < 2 * ctx->num_cus) rows -= KWAVES;
+    const size_t lds = (size_t)rows * rowbytes + 32 + 16;
+    const int nsteps = (N + rows - 1) / rows;
+    int wg_per_cu = (int)(120 * 1024 / lds);
+    if (wg_per_cu < 1) wg_per_cu = 1;
+    if (wg_per_cu > 6) wg_per_cu = 6;
+    const int grid = nsteps < ctx->num_cus * wg_per_cu ? nsteps : ctx->num_cus * wg_per_cu;
+    const int cpl = (K / 16 + WAVE - 1) / WAVE;
+    for (int m = 0; m < M; m++) {
+        int8_t *q8 = (int8_t *)(wsp + per_m * m);
+        float *act_d = (float *)(q8 + K);
+        int *bsums = (int *)(act_d + K / 256);
+        int rc = quantize_launch(ctx, d_x + (size_t)m * K, q8, act_d, bsums, 1, K);
+        if (rc != HM_OK) return rc;
+        float *om = d_out + (size_t)m * N;
+#define HM_KQ_CASE(C)                                                                                              \
+    hipLaunchKernelGGL((gemv_kquant_kernel<QT, C>), dim3(grid), dim3(KTHREADS), lds, ctx->stream, q8, act_d, bsums, \
+                       d_w, om, K, N, rows)
+        switch (cpl) {
+            case 1: HM_KQ_CASE(1); break;
+            case 2: HM_KQ_CASE(2); break;
+            case 3: HM_KQ_CASE(3); break;
+            case 4: HM_KQ_CASE(4); break;
+            case 5: HM_KQ_CASE(5); break;
+            case 6: HM_KQ_CASE(6); break;
+            case 7: HM_KQ_CASE(7); break;
+            default: HM_KQ_CASE(8); break;
+        }
+#undef HM_KQ_CASE
+        HM_LAUNCH_CHECK(ctx);
+    }
+    return HM_OK;
+}
+
+template <int QT>
+int dequant_kquant_launch(hm_ctx *ctx, const char *name, const uint8_t *d_blocks, float *d_out, size_t nblocks) {
+    HM_CHECK_CTX(ctx);
+    if (nblocks == 0) return HM_OK;
+    HM_REQUIRE(ctx, d_blocks && d_out, "%s: NULL pointer", name);
+    const size_t n = nblocks * 256;
+    size_t blocks = (n + 255) / 256;
+    if (blocks > 65536) blocks = 65536;
+    hipLaunchKernelGGL((dequant_kquant_kernel<QT>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, d_blocks, d_out, n);
+    HM_LAUNCH_CHECK(ctx);
+    return HM_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int hm_gemv_q4_k(hm_ctx *ctx, const float *d_x, const uint8_t *d_w_blocks, float *d_out, int M, int K, int N) {
+    return gemv_kquant_launch<0>(ctx, "hm_gemv_q4_k", d_x, d_w_blocks, d_out, M, K, N);
+}
+int hm_gemv_q6_k(hm_ctx *ctx, const float *d_x, const uint8_t *d_w_blocks, float *d_out, int M, int K, int N) {
+    return gemv_kquant_launch<1>(ctx, "hm_gemv_q6_k", d_x, d_w_blocks, d_out, M, K, N);
+}
+int hm_dequant_q4_k(hm_ctx *ctx, const uint8_t *d_blocks, float *d_out, size_t nblocks) {
+    return dequant_kquant_launch<0>(ctx, "hm_dequant_q4_k", d_blocks, d_out, nblocks);
+}
+int hm_dequant_q6_k(hm_ctx *ctx, const uint8_t *d_blocks, float *d_out, size_t nblocks) {
+    return dequant_kquant_launch<1>(ctx, "hm_dequant_q6_k", d_blocks, d_out, nblocks);
+}
+int hm_quantize_q8_k(hm_ctx *ctx, const float *d_x, int8_t *d_q8, float *d_act_d, int32_t *d_bsums, int M, int K) {
+    HM_CHECK_CTX(ctx);
+    HM_REQUIRE(ctx, d_x && d_q8 && d_act_d && d_bsums, "hm_quantize_q8_k: NULL pointer");
+    HM_REQUIRE(ctx, M >= 1 && K > 0 && K % 256 == 0, "hm_quantize_q8_k: need M >= 1 and K a positive multiple of 256");
+    HM_REQUIRE(ctx, ((uintptr_t)d_x % 16) == 0 && ((uintptr_t)d_q8 % 4) == 0, "hm_quantize_q8_k: misaligned buffer");
+    return quantize_launch(ctx, d_x, d_q8, d_act_d, d_bsums, M, K);
+}
+
+}  // extern "C"

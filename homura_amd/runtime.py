@@ -154,6 +154,21 @@ class Context:
     def gemv_q4_0(self, x, w, out, M, K, N):
         self._check(self.lib.hm_gemv_q4_0(self.h, x.ptr, w.ptr, out.ptr, M, K, N))
 
+    def gemv_q4_k(self, x, w, out, M, K, N):
+        self._check(self.lib.hm_gemv_q4_k(self.h, x.ptr, w.ptr, out.ptr, M, K, N))
+
+    def gemv_q6_k(self, x, w, out, M, K, N):
+        self._check(self.lib.hm_gemv_q6_k(self.h, x.ptr, w.ptr, out.ptr, M, K, N))
+
+    def quantize_q8_k(self, x, q8, act_d, bsums, M, K):
+        self._check(self.lib.hm_quantize_q8_k(self.h, x.ptr, q8.ptr, act_d.ptr, bsums.ptr, M, K))
+
+    def dequant_q4_k(self, blocks, out, nblocks):
+        self._check(self.lib.hm_dequant_q4_k(self.h, blocks.ptr, out.ptr, nblocks))
+
+    def dequant_q6_k(self, blocks, out, nblocks):
+        self._check(self.lib.hm_dequant_q6_k(self.h, blocks.ptr, out.ptr, nblocks))
+
     def dequant_q8_0(self, blocks, out, nblocks):
         self._check(self.lib.hm_dequant_q8_0(self.h, blocks.ptr, out.ptr, nblocks))
 

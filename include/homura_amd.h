@@ -108,6 +108,20 @@ int hm_gemv_q4_0(hm_ctx *ctx, const float *d_x, const uint8_t *d_w_blocks, float
 int hm_dequant_q8_0(hm_ctx *ctx, const uint8_t *d_blocks, float *d_out, size_t nblocks);
 int hm_dequant_q4_0(hm_ctx *ctx, const uint8_t *d_blocks, float *d_out, size_t nblocks);
 
+/* K-quants, reference emit_dequant_matmul_q4_k / _q6_k (src/graph_builder/emit_quant.rs:165-816):
+ * the f32 activation is quantised to Q8_K per 256-wide block (scale amax/127, round half to even),
+ * then integer dot products per sub-block against the raw GGUF super-blocks [N][K/256] x 144 B
+ * (Q4_K) or 210 B (Q6_K). K % 256 == 0, K <= 8192, M <= 8. The integer sums are the reference's; the
+ * f32 adds over units and blocks come in a different order. */
+int hm_gemv_q4_k(hm_ctx *ctx, const float *d_x, const uint8_t *d_w_blocks, float *d_out, int M, int K, int N);
+int hm_gemv_q6_k(hm_ctx *ctx, const float *d_x, const uint8_t *d_w_blocks, float *d_out, int M, int K, int N);
+/* The Q8_K activation quantisation on its own (emit_quant.rs:422-466): d_q8 int8 [M][K], d_act_d f32
+ * [M][K/256], d_bsums int32 [M][K/16] (sums of 16 consecutive q). Bit-exact with the CPU. */
+int hm_quantize_q8_k(hm_ctx *ctx, const float *d_x, int8_t *d_q8, float *d_act_d, int32_t *d_bsums, int M, int K);
+/* dequant_q4_k / dequant_q6_k (src/gguf.rs:835-917), 256 weights per block, bit-exact with the CPU. */
+int hm_dequant_q4_k(hm_ctx *ctx, const uint8_t *d_blocks, float *d_out, size_t nblocks);
+int hm_dequant_q6_k(hm_ctx *ctx, const uint8_t *d_blocks, float *d_out, size_t nblocks);
+
 /* Prefill-chunk GEMM on the matrix cores: the reference runs the same emit_matmul with
  * seq > 1 (docs/kv-cache.md:31-37); here A bf16 [M,K], B bf16 [K,N] (reference layout),
  * C f32 [M,N], f32 accumulate. M % 128 == 0, N % 128 == 0, K % 32 == 0. */

@@ -309,6 +309,8 @@ static void q4k_scales(const uint8_t *raw, uint8_t *sc, uint8_t *mn) {
 /* src/gguf.rs:835-882 - Q4_K: 256-weight super-blocks of 144 bytes (f16 d, f16 dmin, 12 bytes
  * of packed scales/mins, 128 bytes of nibbles); sub-blocks come in pairs sharing 32 bytes,
  * even = low nibbles, odd = high nibbles; w = q * (d*sc) - dmin*mn. */
+/* (The reference's Rust does not contract q*scale - min into an FMA; neither may this.) */
+__attribute__((optimize("fp-contract=off")))
 ORC_API void orc_dequant_q4_k(const uint8_t *src, size_t nblocks, float *dst) {
     for (size_t b = 0; b < nblocks; b++) {
         const uint8_t *blk = src + b * 144;

@@ -123,6 +123,59 @@ def test_quant_gemv(ctx, oracle, kind, M, K, N):
         b.free()
 
 
+# ── K-quants ──────────────────────────────────────────────────────────────────
+
+@pytest.mark.parametrize("kind", ["q4_k", "q6_k"])
+def test_kquant_dequant_bit_exact(ctx, oracle, kind):
+    say(f"dequant {kind}")
+    nblocks = 1031
+    raw = (synth.q4_k_blocks if kind == "q4_k" else synth.q6_k_blocks)(77, nblocks)
+    want = (oracle.dequant_q4_k if kind == "q4_k" else oracle.dequant_q6_k)(raw)
+    dw, dout = ctx.to_device(raw), ctx.empty(nblocks * 256)
+    (ctx.dequant_q4_k if kind == "q4_k" else ctx.dequant_q6_k)(dw, dout, nblocks)
+    got = dout.download(np.float32)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    dw.free(); dout.free()
+
+
+def test_quantize_q8_k_bit_exact(ctx, oracle):
+    say("quantize_q8_k")
+    M, K = 3, 1024
+    x = synth.normal_f32(31, M * K, 1.0).reshape(M, K)
+    x[0, 256:512] = 0.0                        # an all-zero block
+    x[1, :8] = (0.5, 1.5, 2.5, -0.5, -2.5, 127.0, -127.0, 63.5)
+    x[1, 8:256] = 0.0                          # amax 127 -> iscale 1: ties visible
+    dx = ctx.to_device(x)
+    dq, dd, db = ctx.alloc(M * K), ctx.empty(M * K // 256), ctx.alloc(M * K // 16 * 4)
+    ctx.quantize_q8_k(dx, dq, dd, db, M, K)
+    q, d, bs = dq.download(np.int8), dd.download(np.float32), db.download(np.int32)
+    for m in range(M):
+        for kb in range(K // 256):
+            wq, wd, wbs = oracle.quantize_q8_k(x[m, kb * 256:(kb + 1) * 256])
+            i = m * K // 256 + kb
+            assert np.array_equal(q[i * 256:(i + 1) * 256], wq) and np.float32(wd) == d[i]
+            assert np.array_equal(bs[i * 16:(i + 1) * 16], wbs)
+    assert q[K:K + 8].tolist() == [0, 2, 2, 0, -2, 127, -127, 64]
+
+
+@pytest.mark.parametrize("kind", ["q4_k", "q6_k"])
+@pytest.mark.parametrize("M,K,N", [(1, 1024, 3072), (1, 3072, 1024), (1, 1024, 151936), (2, 256, 7), (1, 2048, 515),
+                                   (1, 8192, 64)])
+def test_gemv_kquant(ctx, oracle, kind, M, K, N):
+    say(f"gemv_{kind} M={M} K={K} N={N}")
+    raw = (synth.q4_k_blocks if kind == "q4_k" else synth.q6_k_blocks)(5, N * K // 256)
+    x = synth.normal_f32(6, M * K, 1.0).reshape(M, K)
+    want = (oracle.gemv_q4_k if kind == "q4_k" else oracle.gemv_q6_k)(x, raw, M, K, N)
+    dx, dw, dout = ctx.to_device(x), ctx.to_device(raw), ctx.empty(M * N)
+    (ctx.gemv_q4_k if kind == "q4_k" else ctx.gemv_q6_k)(dx, dw, dout, M, K, N)
+    got = dout.download(np.float32, (M, N))
+    err = rel_err(got, want)
+    say(f"  rel err {err:.2e}")
+    assert err < 1e-4          # same integer sums; only the order of the f32 adds differs
+    for b in (dx, dw, dout):
+        b.free()
+
+
 # ── prefill GEMM (MFMA) ───────────────────────────────────────────────────────
 
 @pytest.mark.parametrize("layout", ["kn", "nk"])
