@@ -90,6 +90,7 @@ SIGNATURES = {
     "hm_gguf_tensor_info": (_I, [_P, _I, C.c_char_p, _SZ, _P, _P, _P, _P, _P]),
     "hm_gguf_find_tensor": (_I, [_P, C.c_char_p]),
     "hm_gguf_tensor_data": (_P, [_P, _I]),
+    "hm_gguf_tensor_f32": (_I, [_P, _I, _P, _SZ, C.c_char_p, _SZ]),
     "hm_gguf_meta_str": (_I, [_P, C.c_char_p, C.c_char_p, _SZ]),
     "hm_gguf_meta_u64": (_I, [_P, C.c_char_p, _P]),
     "hm_gguf_meta_f32": (_I, [_P, C.c_char_p, _P]),
@@ -115,6 +116,7 @@ SIGNATURES = {
     "hm_embed": (_I, [_P, _P, _P, _P, _I, _I, _I]),
     "hm_argmax": (_I, [_P, _P, _I, _P]),
     "hm_model_create": (_P, [_P, C.POINTER(HmTransformerConfig), _I, _I]),
+    "hm_model_create_mixed": (_P, [_P, C.POINTER(HmTransformerConfig), C.POINTER(_I), _I]),
     "hm_model_destroy": (None, [_P]),
     "hm_model_num_weight_slots": (_I, [_P]),
     "hm_model_weight_slot_info": (_I, [_P, _I, C.c_char_p, _SZ, C.POINTER(_I),

@@ -9,7 +9,7 @@ import numpy as np
 from . import _ffi
 from .runtime import TransformerConfig
 
-GGML_F32, GGML_F16, GGML_Q4_0, GGML_Q8_0, GGML_Q4_K, GGML_Q6_K, GGML_BF16 = 0, 1, 2, 8, 12, 14, 30
+GGML_F32, GGML_F16, GGML_Q4_0, GGML_Q8_0, GGML_Q4_K, GGML_Q5_K, GGML_Q6_K, GGML_BF16 = 0, 1, 2, 8, 12, 13, 14, 30
 
 
 def _config_from_c(c) -> TransformerConfig:
@@ -71,6 +71,18 @@ class GgufFile:
         nbytes = self.tensors()[i][4]
         ptr = self.lib.hm_gguf_tensor_data(self.h, i)
         return np.ctypeslib.as_array(C.cast(ptr, C.POINTER(C.c_uint8)), shape=(nbytes,)).copy()
+
+    def tensor_f32(self, name: str) -> np.ndarray:
+        """reference load_f32_buffer (src/gguf.rs:727-776): the tensor as f32, dequantised on the host."""
+        i = self.lib.hm_gguf_find_tensor(self.h, name.encode())
+        if i < 0:
+            raise KeyError(name)
+        shape = self.tensors()[i][1]
+        out = np.empty(shape, np.float32)
+        err = C.create_string_buffer(256)
+        if self.lib.hm_gguf_tensor_f32(self.h, i, out.ctypes.data, out.size, err, 256) != 0:
+            raise ValueError(err.value.decode())
+        return out
 
     def meta_str(self, key: str):
         buf = C.create_string_buffer(4096)

@@ -12,6 +12,7 @@
 // sub-block of Q6_K. Units are dealt to the lanes round-robin (K/16 per row, so K = 1024 fills the
 // wavefront exactly); a lane keeps the 16 int8 activations of each of its units, their sum and
 // the block's activation scale in registers for the life of the workgroup and walks the rows.
+#include "gemv_kquant.h"
 #include "hm_common.h"
 
 namespace {
@@ -285,7 +286,7 @@ int quantize_launch(hm_ctx *ctx, const float *d_x, int8_t *q8, float *act_d, int
 
 template <int QT>
 int gemv_kquant_launch(hm_ctx *ctx, const char *name, const float *d_x, const uint8_t *d_w, float *d_out, int M, int K,
-                       int N) {
+                       int N, bool reuse_activation = false) {
     HM_CHECK_CTX(ctx);
     constexpr int BB = KTraits<QT>::BYTES;
     HM_REQUIRE(ctx, d_x && d_w && d_out, "%s: NULL pointer", name);
@@ -317,8 +318,10 @@ int gemv_kquant_launch(hm_ctx *ctx, const char *name, const float *d_x, const ui
         int8_t *q8 = (int8_t *)(wsp + per_m * m);
         float *act_d = (float *)(q8 + K);
         int *bsums = (int *)(act_d + K / 256);
-        int rc = quantize_launch(ctx, d_x + (size_t)m * K, q8, act_d, bsums, 1, K);
-        if (rc != HM_OK) return rc;
+        if (!reuse_activation) {
+            int rc = quantize_launch(ctx, d_x + (size_t)m * K, q8, act_d, bsums, 1, K);
+            if (rc != HM_OK) return rc;
+        }
         float *om = d_out + (size_t)m * N;
 #define HM_KQ_CASE(C)                                                                                              \
     hipLaunchKernelGGL((gemv_kquant_kernel<QT, C>), dim3(grid), dim3(KTHREADS), lds, ctx->stream, q8, act_d, bsums, \
@@ -353,6 +356,12 @@ int dequant_kquant_launch(hm_ctx *ctx, const char *name, const uint8_t *d_blocks
 }
 
 }  // namespace
+
+int homura::gemv_kquant(hm_ctx *ctx, bool q6, const float *d_x, const uint8_t *d_w, float *d_out, int K, int N,
+                        bool reuse_activation) {
+    return q6 ? gemv_kquant_launch<1>(ctx, "gemv_kquant[q6_k]", d_x, d_w, d_out, 1, K, N, reuse_activation)
+              : gemv_kquant_launch<0>(ctx, "gemv_kquant[q4_k]", d_x, d_w, d_out, 1, K, N, reuse_activation);
+}
 
 extern "C" {
 

@@ -13,13 +13,7 @@ struct hm_model {
 
 extern "C" {
 
-hm_model *hm_model_create(hm_ctx *ctx, const hm_transformer_config *cfg, int weight_dtype,
-                          int has_qk_norm) {
-    if (!ctx) return nullptr;
-    if (!cfg) {
-        hm_set_error(ctx, HM_ERR_INVALID, "hm_model_create: NULL config");
-        return nullptr;
-    }
+static TransformerConfig config_from_c(const hm_transformer_config *cfg) {
     TransformerConfig c;
     c.hidden_size = cfg->hidden_size;
     c.intermediate_size = cfg->intermediate_size;
@@ -34,7 +28,38 @@ hm_model *hm_model_create(hm_ctx *ctx, const hm_transformer_config *cfg, int wei
     c.rms_norm_eps = cfg->rms_norm_eps > 0 ? cfg->rms_norm_eps : 1e-6;
     c.rope_theta = cfg->rope_theta > 0 ? cfg->rope_theta : 10000.0;
     c.attention_bias = cfg->attention_bias != 0;
-    auto impl = HfModel::create(ctx, c, (DType)weight_dtype, has_qk_norm != 0);
+    return c;
+}
+
+hm_model *hm_model_create(hm_ctx *ctx, const hm_transformer_config *cfg, int weight_dtype,
+                          int has_qk_norm) {
+    if (!ctx) return nullptr;
+    if (!cfg) {
+        hm_set_error(ctx, HM_ERR_INVALID, "hm_model_create: NULL config");
+        return nullptr;
+    }
+    auto impl = HfModel::create(ctx, config_from_c(cfg), (DType)weight_dtype, has_qk_norm != 0);
+    if (!impl) return nullptr;
+    return new hm_model{ctx, std::move(impl)};
+}
+
+hm_model *hm_model_create_mixed(hm_ctx *ctx, const hm_transformer_config *cfg, const int *proj_dtypes,
+                                int has_qk_norm) {
+    if (!ctx) return nullptr;
+    if (!cfg || !proj_dtypes || cfg->num_hidden_layers <= 0) {
+        hm_set_error(ctx, HM_ERR_INVALID, "hm_model_create_mixed: NULL config or dtype list");
+        return nullptr;
+    }
+    std::vector<DType> dts((size_t)cfg->num_hidden_layers * 7);
+    for (size_t i = 0; i < dts.size(); i++) {
+        if (proj_dtypes[i] < HM_DTYPE_Q8_0 || proj_dtypes[i] > HM_DTYPE_Q6_K || proj_dtypes[i] == HM_DTYPE_I64) {
+            hm_set_error(ctx, HM_ERR_INVALID, "hm_model_create_mixed: projection %zu has dtype %d, not a block-quantised one",
+                         i, proj_dtypes[i]);
+            return nullptr;
+        }
+        dts[i] = (DType)proj_dtypes[i];
+    }
+    auto impl = HfModel::create(ctx, config_from_c(cfg), dts[0], has_qk_norm != 0, &dts);
     if (!impl) return nullptr;
     return new hm_model{ctx, std::move(impl)};
 }
@@ -223,6 +248,22 @@ int hm_gguf_find_tensor(const hm_gguf *g, const char *name) {
 const void *hm_gguf_tensor_data(const hm_gguf *g, int index) {
     if (!g || index < 0 || index >= (int)g->f->tensors().size()) return nullptr;
     return g->f->tensor_data(g->f->tensors()[index]);
+}
+
+int hm_gguf_tensor_f32(const hm_gguf *g, int index, float *out, size_t n_elements, char *err, size_t errlen) {
+    auto say = [&](const std::string &m) {
+        if (err && errlen) snprintf(err, errlen, "%s", m.c_str());
+        return HM_ERR_INVALID;
+    };
+    if (!g || !out || index < 0 || index >= (int)g->f->tensors().size()) return say("bad handle, index or output");
+    const GgufTensorInfo &t = g->f->tensors()[index];
+    if (t.num_elements() != n_elements)
+        return say("tensor " + t.name + " has " + std::to_string(t.num_elements()) + " elements");
+    std::vector<float> tmp;
+    std::string e;
+    if (!ggml_to_f32(t.type, g->f->tensor_data(t), n_elements, &tmp, &e)) return say("tensor " + t.name + ": " + e);
+    std::memcpy(out, tmp.data(), n_elements * sizeof(float));
+    return HM_OK;
 }
 
 int hm_gguf_meta_str(const hm_gguf *g, const char *key, char *buf, size_t buflen) {

@@ -50,8 +50,11 @@ struct PlanScratch {
 
 class HfModel {
   public:
-    static std::unique_ptr<HfModel> create(hm_ctx *ctx, const TransformerConfig &cfg,
-                                           DType weight_dtype, bool has_qk_norm);
+    // proj_dtypes: optional, 7 per layer (q, k, v, o, gate, up, down) for a quantised model whose
+    // projections do not all share weight_dtype.
+    static std::unique_ptr<HfModel> create(hm_ctx *ctx, const TransformerConfig &cfg, DType weight_dtype,
+                                           bool has_qk_norm, const std::vector<DType> *proj_dtypes = nullptr);
+    DType proj_dtype(int layer, int which) const { return proj_dtypes_[(size_t)layer * 7 + which]; }
     ~HfModel();
 
     const TransformerConfig &config() const { return cfg_; }
@@ -94,11 +97,16 @@ class HfModel {
     bool has_qk_norm_ = false;
     bool finalized_ = false;
     int max_seq_len_ = 0;
+    std::vector<DType> proj_dtypes_;    // [layers][7]
     std::vector<WeightSlotInfo> infos_;
     std::vector<Buffer> weight_bufs_;   // in weight_slots order, device resident
     std::vector<bool> weight_set_;
     // packed storage the bf16 weight slot buffers are views of
-    struct LayerPacked { Buffer qkv, o, gate_up, down, qkv_bias; };  // qkv_bias: f32 [q_dim + 2 kv_dim]
+    // qkv_bias: f32 [q_dim + 2 kv_dim]. quant[j] (j = q k v o gate up down) is set for the first
+    // matrix of each run of same-type neighbours inside q|k|v and gate|up, and holds the whole run.
+    struct LayerPacked { Buffer qkv, o, gate_up, down, qkv_bias, quant[7]; };
+    // First member and member count of the stacked run that projection `which` of `layer` belongs to.
+    void quant_run(int layer, int which, int *first, int *count) const;
     std::vector<LayerPacked> packed_;
     Buffer lm_head_packed_;
     Buffer rope_cos_, rope_sin_;        // [max_position][head_dim] f32

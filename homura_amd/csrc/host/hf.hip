@@ -6,6 +6,7 @@
 
 #include "../attention.h"
 #include "../gemv_bf16.h"
+#include "../gemv_kquant.h"
 #include "../light_ops.h"
 
 namespace homura {
@@ -34,7 +35,8 @@ void precompute_rope_cos_sin(int head_dim, int max_seq_len, double theta, std::v
 }  // namespace
 
 std::unique_ptr<HfModel> HfModel::create(hm_ctx *ctx, const TransformerConfig &cfg,
-                                         DType weight_dtype, bool has_qk_norm) {
+                                         DType weight_dtype, bool has_qk_norm,
+                                         const std::vector<DType> *proj_dtypes) {
     auto fail = [&](const char *msg) -> std::unique_ptr<HfModel> {
         hm_set_error(ctx, HM_ERR_INVALID, "hm_model_create: %s", msg);
         return nullptr;
@@ -47,13 +49,27 @@ std::unique_ptr<HfModel> HfModel::create(hm_ctx *ctx, const TransformerConfig &c
     if (cfg.gqa_repeat() > 8) return fail("GQA group larger than 8");
     if (cfg.hidden_size % 32 || cfg.intermediate_size % 32 || cfg.q_dim() % 32)
         return fail("hidden, intermediate and q dims must be multiples of 32");
-    if (weight_dtype != DType::BF16 && weight_dtype != DType::Q8_0 && weight_dtype != DType::Q4_0)
-        return fail("projection dtype must be BF16, Q8_0 or Q4_0");
+    if (weight_dtype != DType::BF16 && !dtype_is_quantized(weight_dtype))
+        return fail("projection dtype must be BF16, Q8_0, Q4_0, Q4_K or Q6_K");
+    if (proj_dtypes) {
+        if (proj_dtypes->size() != (size_t)cfg.num_hidden_layers * 7) return fail("need 7 projection dtypes per layer");
+        for (DType t : *proj_dtypes)
+            if (!dtype_is_quantized(t)) return fail("a model with per-projection dtypes must be quantised throughout");
+        if (!dtype_is_quantized(weight_dtype)) return fail("per-projection dtypes need a quantised weight_dtype");
+    }
 
     std::unique_ptr<HfModel> m(new HfModel());
     m->ctx_ = ctx;
     m->cfg_ = cfg;
     m->weight_dtype_ = weight_dtype;
+    m->proj_dtypes_ = proj_dtypes ? *proj_dtypes : std::vector<DType>((size_t)cfg.num_hidden_layers * 7, weight_dtype);
+    if (dtype_is_quantized(weight_dtype)) {
+        const int kdim[7] = {cfg.hidden_size, cfg.hidden_size, cfg.hidden_size, cfg.q_dim(), cfg.hidden_size,
+                             cfg.hidden_size, cfg.intermediate_size};
+        for (size_t i = 0; i < m->proj_dtypes_.size(); i++)
+            if (kdim[i % 7] % (int)dtype_block_size(m->proj_dtypes_[i]) != 0)
+                return fail("a projection's input width is not a multiple of its quantisation block");
+    }
     m->has_qk_norm_ = has_qk_norm;
 
     // Slot order = TransformerWeights::to_slot_buffers (src/hf/weights.rs:63-116) for bf16,
@@ -65,11 +81,12 @@ std::unique_ptr<HfModel> HfModel::create(hm_ctx *ctx, const TransformerConfig &c
     auto f32_vec = [&](const std::string &name, int64_t n) {
         v.push_back(WeightSlotInfo{name, DType::F32, n, 1, (size_t)n * 4});
     };
+    int proj_index = 0;  // runs over (layer, q k v o gate up down) in slot order
     auto proj = [&](const std::string &name, int64_t K, int64_t N) {
-        if (quant)
-            v.push_back(WeightSlotInfo{name, weight_dtype, N, K,
-                                       dtype_bytes_for_elements(weight_dtype, (size_t)(N * K), nullptr)});
-        else
+        if (quant) {
+            const DType t = m->proj_dtypes_[proj_index++];
+            v.push_back(WeightSlotInfo{name, t, N, K, dtype_bytes_for_elements(t, (size_t)(N * K), nullptr)});
+        } else
             v.push_back(WeightSlotInfo{name, DType::BF16, K, N, (size_t)(K * N) * 2});
     };
     v.push_back(WeightSlotInfo{"model.embed_tokens.weight", DType::F32, vocab, hidden,
@@ -105,6 +122,17 @@ std::unique_ptr<HfModel> HfModel::create(hm_ctx *ctx, const TransformerConfig &c
     return m;
 }
 
+void HfModel::quant_run(int layer, int which, int *first, int *count) const {
+    int lo = which, hi = which;  // q|k|v are 0..2, gate|up are 4..5; o and down stand alone
+    const int gmin = which <= 2 ? 0 : which == 4 || which == 5 ? 4 : which;
+    const int gmax = which <= 2 ? 2 : which == 4 || which == 5 ? 5 : which;
+    const DType t = proj_dtype(layer, which);
+    while (lo > gmin && proj_dtype(layer, lo - 1) == t) lo--;
+    while (hi < gmax && proj_dtype(layer, hi + 1) == t) hi++;
+    *first = lo;
+    *count = hi - lo + 1;
+}
+
 HfModel::~HfModel() {
     if (ctx_) hm_sync(ctx_);
 }
@@ -129,34 +157,29 @@ int HfModel::set_weight_impl(int slot, const void *h_data, size_t bytes, bool nk
     const int qd = cfg_.q_dim(), kvd = cfg_.kv_dim();
 
     if (dtype_is_quantized(info.dtype)) {
-        // Raw GGUF blocks [N][K/32], kept byte for byte. q|k|v and gate|up of a layer are stored
-        // back to back (rows are contiguous, so the three/two matrices form one taller matrix
-        // and one kernel launch serves them).
+        // Raw GGUF blocks [N][K/block], kept byte for byte. Neighbours of one type inside q|k|v and
+        // gate|up of a layer are stored back to back (rows are contiguous, so the matrices form
+        // one taller matrix and one kernel launch serves them).
         const size_t p0 = std::string("model.layers.").size();
         const int layer = std::atoi(nm.c_str() + p0);
         LayerPacked &lp = packed_[layer];
-        const size_t bb = dtype_block_bytes(info.dtype);
-        const size_t row_h = (size_t)(hidden / 32) * bb;  // bytes of a row with K = hidden
-        Buffer *home = nullptr;
+        static const char *const suffix[7] = {"q_proj.weight", "k_proj.weight", "v_proj.weight", "o_proj.weight",
+                                              "gate_proj.weight", "up_proj.weight", "down_proj.weight"};
+        int which = -1;
+        for (int j = 0; j < 7; j++)
+            if (ends_with(suffix[j])) which = j;
+        if (which < 0) return hm_set_error(ctx_, HM_ERR_INVALID, "unexpected quantised weight %s", nm.c_str());
+        const int64_t kdim[7] = {hidden, hidden, hidden, qd, hidden, hidden, inter};
+        const int64_t ndim[7] = {qd, kvd, kvd, hidden, inter, inter, hidden};
+        int first, count;
+        quant_run(layer, which, &first, &count);
         size_t home_bytes = 0, offset = 0;
-        if (ends_with("q_proj.weight") || ends_with("k_proj.weight") || ends_with("v_proj.weight")) {
-            home = &lp.qkv;
-            home_bytes = (size_t)(qd + 2 * kvd) * row_h;
-            offset = ends_with("q_proj.weight") ? 0 : ends_with("k_proj.weight") ? (size_t)qd * row_h
-                                                                                  : (size_t)(qd + kvd) * row_h;
-        } else if (ends_with("gate_proj.weight") || ends_with("up_proj.weight")) {
-            home = &lp.gate_up;
-            home_bytes = (size_t)2 * inter * row_h;
-            offset = ends_with("up_proj.weight") ? (size_t)inter * row_h : 0;
-        } else if (ends_with("o_proj.weight")) {
-            home = &lp.o;
-            home_bytes = bytes;
-        } else if (ends_with("down_proj.weight")) {
-            home = &lp.down;
-            home_bytes = bytes;
-        } else {
-            return hm_set_error(ctx_, HM_ERR_INVALID, "unexpected quantised weight %s", nm.c_str());
+        for (int j = first; j < first + count; j++) {
+            const size_t b = dtype_bytes_for_elements(info.dtype, (size_t)(kdim[j] * ndim[j]), nullptr);
+            if (j < which) offset += b;
+            home_bytes += b;
         }
+        Buffer *home = &lp.quant[first];
         if (!*home) *home = Buffer::alloc_bytes(ctx_, home_bytes, {(int64_t)home_bytes}, info.dtype);
         if (!*home) return HM_ERR_OOM;
         int rc = hm_upload(ctx_, (char *)home->ptr() + offset, h_data, bytes);
@@ -667,9 +690,7 @@ int HfModel::emit_transformer_plan_quant() {
     const int L = c.num_hidden_layers;
     const float eps = (float)c.rms_norm_eps;
     const bool qkn = has_qk_norm_;
-    const DType wdt = weight_dtype_;
     const int64_t D = DIM_DYNAMIC;
-    const double bpw = (double)dtype_block_bytes(wdt) / 32.0;  // bytes per weight
 
     std::vector<SlotDesc> descs;
     auto alloc = [&](std::vector<int64_t> shape, DType dt, const std::string &name) -> size_t {
@@ -693,7 +714,9 @@ int HfModel::emit_transformer_plan_quant() {
             gate_out, up_out, silu, down_out, hidden_out;
     };
     std::vector<LS> ls(L);
-    auto qbytes = [&](int64_t K, int64_t N) { return (int64_t)dtype_bytes_for_elements(wdt, (size_t)(K * N), nullptr); };
+    auto qbytes = [&](DType t, int64_t K, int64_t N) {
+        return (int64_t)dtype_bytes_for_elements(t, (size_t)(K * N), nullptr);
+    };
     for (int i = 0; i < L; i++) {
         LS &s = ls[i];
         const std::string p = "l" + std::to_string(i) + ".";
@@ -707,22 +730,24 @@ int HfModel::emit_transformer_plan_quant() {
         s.input_ln = w({hidden}, DType::F32, "input_ln");
         const bool bias = c.attention_bias;
         s.q_b = s.k_b = s.v_b = (size_t)-1;
-        s.q_w = w({qbytes(hidden, qd)}, wdt, "q_w");
+        const DType tq = proj_dtype(i, 0), tk = proj_dtype(i, 1), tv = proj_dtype(i, 2), to = proj_dtype(i, 3),
+                    tg = proj_dtype(i, 4), tu = proj_dtype(i, 5), td = proj_dtype(i, 6);
+        s.q_w = w({qbytes(tq, hidden, qd)}, tq, "q_w");
         if (bias) s.q_b = w({qd}, DType::F32, "q_b");
-        s.k_w = w({qbytes(hidden, kvd)}, wdt, "k_w");
+        s.k_w = w({qbytes(tk, hidden, kvd)}, tk, "k_w");
         if (bias) s.k_b = w({kvd}, DType::F32, "k_b");
-        s.v_w = w({qbytes(hidden, kvd)}, wdt, "v_w");
+        s.v_w = w({qbytes(tv, hidden, kvd)}, tv, "v_w");
         if (bias) s.v_b = w({kvd}, DType::F32, "v_b");
         s.q_norm = s.k_norm = (size_t)-1;
         if (qkn) {
             s.q_norm = w({hd}, DType::F32, "q_norm");
             s.k_norm = w({hd}, DType::F32, "k_norm");
         }
-        s.o_w = w({qbytes(qd, hidden)}, wdt, "o_w");
+        s.o_w = w({qbytes(to, qd, hidden)}, to, "o_w");
         s.post_ln = w({hidden}, DType::F32, "post_ln");
-        s.gate_w = w({qbytes(hidden, inter)}, wdt, "gate_w");
-        s.up_w = w({qbytes(hidden, inter)}, wdt, "up_w");
-        s.down_w = w({qbytes(inter, hidden)}, wdt, "down_w");
+        s.gate_w = w({qbytes(tg, hidden, inter)}, tg, "gate_w");
+        s.up_w = w({qbytes(tu, hidden, inter)}, tu, "up_w");
+        s.down_w = w({qbytes(td, inter, hidden)}, td, "down_w");
         s.past_k = alloc({1, kvh, D, hd}, DType::BF16, p + "past_k");
         s.past_v = alloc({1, kvh, D, hd}, DType::BF16, p + "past_v");
         past_kv.push_back(s.past_k);
@@ -772,25 +797,56 @@ int HfModel::emit_transformer_plan_quant() {
         kernels.push_back(std::move(k));
         steps.push_back(KernelStep::kernel(kernels.size() - 1, std::move(in), std::move(out)));
     };
-    auto quant_mm = [&](const char *label, int64_t K, int64_t N, bool launches) {
-        // QuantMM step (reference emit_quant_matmul_kernel, src/hf/emitter_quant.rs:675-702):
-        // inputs [activation, weight bytes], output [1, seq, N]
+    // QuantMM step (reference emit_quant_matmul_kernel, src/hf/emitter_quant.rs:675-702): inputs
+    // [activation, weight bytes], output [1, seq, N]. The first matrix of a stacked run launches over
+    // the whole run (N rows = the run's total, its outputs are adjacent too); the others launch
+    // nothing. reuse_act: an earlier K-quant launch of the same group already quantised this
+    // activation.
+    auto quant_mm = [&](const char *label, DType wdt, int64_t K, int64_t N, bool reuse_act) {
         CompiledKernel k;
         k.ops_label = std::string("QuantMM[") + label + "]";
-        if (launches) {
+        if (N > 0) {
             DeviceLaunch l;
-            l.name = std::string(wdt == DType::Q8_0 ? "gemv_q8_0[" : "gemv_q4_0[") + label + "]";
-            l.bytes_fixed = (double)K * N * bpw + K * 4.0 + N * 4.0;
+            const char *kn = wdt == DType::Q8_0 ? "gemv_q8_0[" : wdt == DType::Q4_0 ? "gemv_q4_0["
+                             : wdt == DType::Q4_K ? "gemv_q4_k[" : "gemv_q6_k[";
+            l.name = std::string(kn) + label + "]";
+            l.bytes_fixed = (double)dtype_bytes_for_elements(wdt, (size_t)(K * N), nullptr) + K * 4.0 + N * 4.0;
             l.fn = [=](const StepContext &sc) -> int {
                 const float *x = sc.pool[sc.step.input_slots[0]]->as<float>();
                 const uint8_t *w = sc.pool[sc.step.input_slots[1]]->as<uint8_t>();
                 float *out = sc.pool[sc.step.output_slots[0]]->as<float>();
-                return wdt == DType::Q8_0 ? hm_gemv_q8_0(sc.ctx, x, w, out, 1, (int)K, (int)N)
-                                          : hm_gemv_q4_0(sc.ctx, x, w, out, 1, (int)K, (int)N);
+                switch (wdt) {
+                case DType::Q8_0: return hm_gemv_q8_0(sc.ctx, x, w, out, 1, (int)K, (int)N);
+                case DType::Q4_0: return hm_gemv_q4_0(sc.ctx, x, w, out, 1, (int)K, (int)N);
+                default: return gemv_kquant(sc.ctx, wdt == DType::Q6_K, x, w, out, (int)K, (int)N, reuse_act);
+                }
             };
             k.launches.push_back(std::move(l));
         }
         return k;
+    };
+    // The QuantMM steps of one group of matrices that share an activation (q|k|v, gate|up, or one alone)
+    struct GroupMember { const char *label; int which; int64_t N; size_t w_slot, out_slot; };
+    auto quant_group = [&](int layer, size_t act_slot, int64_t K, std::vector<GroupMember> members) {
+        bool act_quantized = false;
+        for (size_t j = 0; j < members.size(); j++) {
+            const GroupMember &gm = members[j];
+            int first, count;
+            quant_run(layer, gm.which, &first, &count);
+            const DType t = proj_dtype(layer, gm.which);
+            const bool kq = t == DType::Q4_K || t == DType::Q6_K;
+            int64_t n_run = 0;
+            std::string label = gm.label;
+            if (first == gm.which) {
+                n_run = gm.N;
+                for (int e = 1; e < count; e++) {
+                    n_run += members[j + e].N;
+                    label += members[j + e].label;
+                }
+            }
+            add_step(quant_mm(label.c_str(), t, K, n_run, kq && act_quantized), {act_slot, gm.w_slot}, {gm.out_slot});
+            if (n_run > 0 && kq) act_quantized = true;
+        }
     };
 
     {
@@ -824,9 +880,8 @@ int HfModel::emit_transformer_plan_quant() {
             add_step(std::move(k), {s.hidden_in, s.input_ln}, {s.normed});
         }
         // Steps 2-4: QuantMM Q, K, V — one launch over the stacked q|k|v rows
-        add_step(quant_mm("qkv", hidden, qd + 2 * kvd, true), {s.normed, s.q_w}, {s.q_out});
-        add_step(quant_mm("k", hidden, kvd, false), {s.normed, s.k_w}, {s.k_out});
-        add_step(quant_mm("v", hidden, kvd, false), {s.normed, s.v_w}, {s.v_out});
+        quant_group(i, s.normed, hidden, {{"q", 0, qd, s.q_w, s.q_out}, {"k", 1, kvd, s.k_w, s.k_out},
+                                          {"v", 2, kvd, s.v_w, s.v_out}});
         {  // Step 5: PostQKV (reference :802-912) — runs in the attention kernel's prologue
             CompiledKernel k;
             k.ops_label = qkn ? "PostQKV+QKNorm+RoPE" : "PostQKV+RoPE";
@@ -909,7 +964,7 @@ int HfModel::emit_transformer_plan_quant() {
             k.launches.push_back(std::move(l));
             add_step(std::move(k), {s.q, s.present_k, s.present_v, mask}, {s.attn_body});
         }
-        add_step(quant_mm("o", qd, hidden, true), {s.attn_body, s.o_w}, {s.attn_out});  // Step 9
+        quant_group(i, s.attn_body, qd, {{"o", 3, hidden, s.o_w, s.attn_out}});  // Step 9
         {  // Step 10: Residual + RMSNorm (reference :985-1071), two outputs
             CompiledKernel k;
             k.ops_label = "Residual+Norm";
@@ -926,8 +981,7 @@ int HfModel::emit_transformer_plan_quant() {
             add_step(std::move(k), {s.hidden_in, s.attn_out, s.post_ln}, {s.residual, s.post_normed});
         }
         // Steps 11-12: QuantMM Gate, Up — one launch over the stacked gate|up rows
-        add_step(quant_mm("gate_up", hidden, 2 * inter, true), {s.post_normed, s.gate_w}, {s.gate_out});
-        add_step(quant_mm("up", hidden, inter, false), {s.post_normed, s.up_w}, {s.up_out});
+        quant_group(i, s.post_normed, hidden, {{"gate", 4, inter, s.gate_w, s.gate_out}, {"up", 5, inter, s.up_w, s.up_out}});
         {  // Step 13: SiLU * Up (reference :1077-1103)
             CompiledKernel k;
             k.ops_label = "SiLU*Up";
@@ -942,7 +996,7 @@ int HfModel::emit_transformer_plan_quant() {
             k.launches.push_back(std::move(l));
             add_step(std::move(k), {s.gate_out, s.up_out}, {s.silu});
         }
-        add_step(quant_mm("down", inter, hidden, true), {s.silu, s.down_w}, {s.down_out});  // Step 14
+        quant_group(i, s.silu, inter, {{"down", 6, hidden, s.down_w, s.down_out}});  // Step 14
         {  // Step 15: ResAdd (reference :1109-1134)
             CompiledKernel k;
             k.ops_label = "ResAdd";

@@ -93,6 +93,9 @@ class GgufFile {
     std::map<std::string, size_t> by_name_;
 };
 
+// reference GgufFile::load_f32_buffer (src/gguf.rs:727-776): n elements of a GGML type as f32
+bool ggml_to_f32(GgmlType type, const uint8_t *src, size_t n, std::vector<float> *out, std::string *err);
+
 // reference load_transformer_weights + HfModel::load for a GGUF file (src/gguf.rs:589-708): projection
 // weights stay the raw blocks (Q8_0, Q4_0) or become bf16 (F32/F16/BF16 files); norms, biases and the
 // embedding become f32; the LM head is f32 in the quantised plan. Returns nullptr and sets the

@@ -117,6 +117,53 @@ void dequant_q4_0_host(const uint8_t *src, float *dst, size_t n) {
         }
     }
 }
+// Q4_K (reference dequantize_q4_k, src/gguf.rs:835-882): weight e of a 256-wide super-block sits in
+// sub-block s = e/32; sub-blocks 2p and 2p+1 share the 32 bytes at 16 + 32p (low and high nibbles);
+// the 6-bit scale and minimum of sub-block s come out of the 12 bytes at offset 4.
+// w = nibble * (d * scale) - dmin * minimum, three roundings, no fused multiply-add.
+#pragma clang fp contract(off)
+void dequant_q4_k_host(const uint8_t *src, float *dst, size_t n) {
+    for (size_t b = 0; b < n / 256; b++) {
+        const uint8_t *blk = src + b * 144, *pk = blk + 4;
+        const float d = f16_bits_to_f32_host(rd16(blk)), dmin = f16_bits_to_f32_host(rd16(blk + 2));
+        for (int s = 0; s < 8; s++) {
+            int sc, mn;
+            if (s < 4) {
+                sc = pk[s] & 63;
+                mn = pk[4 + s] & 63;
+            } else {
+                sc = (pk[4 + s] & 15) | ((pk[s - 4] >> 6) << 4);
+                mn = (pk[4 + s] >> 4) | ((pk[s] >> 6) << 4);
+            }
+            const float scale = d * (float)sc;
+            const float minimum = dmin * (float)mn;
+            const uint8_t *q = blk + 16 + 32 * (s >> 1);
+            float *o = dst + b * 256 + 32 * s;
+            for (int l = 0; l < 32; l++) {
+                const float prod = (float)((s & 1) ? (q[l] >> 4) : (q[l] & 15)) * scale;
+                o[l] = prod - minimum;
+            }
+        }
+    }
+}
+// Q6_K (reference dequantize_q6_k, src/gguf.rs:886-917): weight e = 128h + 32g + l has its low nibble in
+// byte 64h + 32(g&1) + l (upper half of the byte for g >= 2), its two high bits at bit 2g of byte
+// 128 + 32h + l, and the int8 scale 192 + 8h + 2g + l/16. w = (d * scale) * (q - 32).
+void dequant_q6_k_host(const uint8_t *src, float *dst, size_t n) {
+    for (size_t b = 0; b < n / 256; b++) {
+        const uint8_t *blk = src + b * 210;
+        const float d = f16_bits_to_f32_host(rd16(blk + 208));
+        for (int e = 0; e < 256; e++) {
+            const int h = e >> 7, g = (e & 127) >> 5, l = e & 31;
+            const uint8_t lb = blk[64 * h + 32 * (g & 1) + l];
+            const int lo = g >= 2 ? (lb >> 4) : (lb & 15);
+            const int hi = (blk[128 + 32 * h + l] >> (2 * g)) & 3;
+            const int q = (int)(int8_t)(lo | (hi << 4)) - 32;
+            const float ds = d * (float)(int8_t)blk[192 + 8 * h + 2 * g + (l >> 4)];
+            dst[b * 256 + e] = ds * (float)q;
+        }
+    }
+}
 
 }  // namespace
 
@@ -467,6 +514,8 @@ bool GgufFile::transformer_config(TransformerConfig *cfg, std::string *err) cons
 namespace {
 
 // any supported GGML type -> f32 (reference load_f32_buffer, src/gguf.rs:726-775; plus Q4_0)
+}  // namespace
+
 bool ggml_to_f32(GgmlType type, const uint8_t *src, size_t n, std::vector<float> *out, std::string *err) {
     out->resize(n);
     float *dst = out->data();
@@ -480,11 +529,24 @@ bool ggml_to_f32(GgmlType type, const uint8_t *src, size_t n, std::vector<float>
         return true;
     case GgmlType::Q8_0: dequant_q8_0_host(src, dst, n); return true;
     case GgmlType::Q4_0: dequant_q4_0_host(src, dst, n); return true;
+    case GgmlType::Q4K:
+    case GgmlType::Q6K:
+        if (n % 256 != 0) {
+            *err = std::string(ggml_type_name(type)) + " tensor whose size is not a multiple of 256";
+            return false;
+        }
+        if (type == GgmlType::Q4K)
+            dequant_q4_k_host(src, dst, n);
+        else
+            dequant_q6_k_host(src, dst, n);
+        return true;
     default:
         *err = std::string("unsupported type ") + ggml_type_name(type) + " for an f32 tensor";
         return false;
     }
 }
+
+namespace {
 
 // F32 / F16 / BF16 -> bf16 bits (F32 by truncation, as the reference's bf16 plan does)
 bool ggml_to_bf16(GgmlType type, const uint8_t *src, size_t n, std::vector<uint16_t> *out, std::string *err) {
@@ -560,23 +622,46 @@ std::unique_ptr<HfModel> load_gguf_model(hm_ctx *ctx, const std::string &path, i
         return nullptr;
     }
     const bool has_qk_norm = g->tensor_info("blk.0.attn_q_norm.weight") != nullptr;
-    const GgufTensorInfo *q0 = g->tensor_info("blk.0.attn_q.weight");
-    if (!q0) {
-        fail(ctx, path + ": missing GGUF tensor: blk.0.attn_q.weight");
+    // Every projection carries its own type (reference Buffer dtype from GgmlType::to_dtype,
+    // src/gguf.rs:593-613); a file is either block-quantised throughout (types may differ per matrix,
+    // as in Q4_K_M files) or float throughout.
+    static const char *const proj_names[7] = {"attn_q", "attn_k", "attn_v", "attn_output", "ffn_gate", "ffn_up", "ffn_down"};
+    std::vector<DType> proj_dtypes;
+    int n_float = 0;
+    for (int l = 0; l < cfg.num_hidden_layers; l++)
+        for (int j = 0; j < 7; j++) {
+            const std::string name = "blk." + std::to_string(l) + "." + proj_names[j] + ".weight";
+            const GgufTensorInfo *t = g->tensor_info(name);
+            if (!t) {
+                fail(ctx, path + ": missing GGUF tensor: " + name);
+                return nullptr;
+            }
+            switch (t->type) {
+            case GgmlType::Q8_0: proj_dtypes.push_back(DType::Q8_0); break;
+            case GgmlType::Q4_0: proj_dtypes.push_back(DType::Q4_0); break;
+            case GgmlType::Q4K: proj_dtypes.push_back(DType::Q4_K); break;
+            case GgmlType::Q6K: proj_dtypes.push_back(DType::Q6_K); break;
+            case GgmlType::F32: case GgmlType::F16: case GgmlType::BF16:
+                proj_dtypes.push_back(DType::BF16);
+                n_float++;
+                break;
+            default:
+                fail(ctx, path + ": tensor " + name + " is " + ggml_type_name(t->type) +
+                              "; this build runs Q8_0, Q4_0, Q4_K, Q6_K and F32/F16/BF16 projections");
+                return nullptr;
+            }
+        }
+    if (proj_dtypes.empty()) {
+        fail(ctx, path + ": the model has no layers");
         return nullptr;
     }
-    DType wdt;
-    switch (q0->type) {
-    case GgmlType::Q8_0: wdt = DType::Q8_0; break;
-    case GgmlType::Q4_0: wdt = DType::Q4_0; break;
-    case GgmlType::F32: case GgmlType::F16: case GgmlType::BF16: wdt = DType::BF16; break;
-    default:
-        fail(ctx, path + ": projection weights are " + ggml_type_name(q0->type) +
-                      "; this build runs Q8_0, Q4_0 and F32/F16/BF16 files");
+    if (n_float != 0 && n_float != (int)proj_dtypes.size()) {
+        fail(ctx, path + ": some projections are block-quantised and some are float (mixing the two is not supported)");
         return nullptr;
     }
-    const bool quant = dtype_is_quantized(wdt);
-    std::unique_ptr<HfModel> m = HfModel::create(ctx, cfg, wdt, has_qk_norm);
+    const bool quant = n_float == 0;
+    std::unique_ptr<HfModel> m = quant ? HfModel::create(ctx, cfg, proj_dtypes[0], has_qk_norm, &proj_dtypes)
+                                       : HfModel::create(ctx, cfg, DType::BF16, has_qk_norm);
     if (!m) return nullptr;
 
     std::vector<float> f32;
@@ -603,11 +688,6 @@ std::unique_ptr<HfModel> load_gguf_model(hm_ctx *ctx, const std::string &path, i
                 return nullptr;
             }
             if (quant) {
-                if ((wdt == DType::Q8_0 ? GgmlType::Q8_0 : GgmlType::Q4_0) != t->type) {
-                    fail(ctx, path + ": tensor " + name + " is " + ggml_type_name(t->type) + " while blk.0.attn_q.weight is " +
-                                  ggml_type_name(q0->type) + " (mixed quantisation is not supported)");
-                    return nullptr;
-                }
                 rc = m->set_weight((int)i, src, t->byte_size());
             } else {
                 if (!ggml_to_bf16(t->type, src, n, &b16, &err)) {
@@ -628,7 +708,8 @@ std::unique_ptr<HfModel> load_gguf_model(hm_ctx *ctx, const std::string &path, i
                 }
                 rc = m->set_weight_nk((int)i, f32.data(), n * 4);
             } else {
-                if (t->type == GgmlType::Q8_0 || t->type == GgmlType::Q4_0) {
+                if (t->type == GgmlType::Q8_0 || t->type == GgmlType::Q4_0 || t->type == GgmlType::Q4K ||
+                    t->type == GgmlType::Q6K) {
                     if (!ggml_to_f32(t->type, src, n, &f32, &err)) {
                         fail(ctx, path + ": tensor " + name + ": " + err);
                         return nullptr;

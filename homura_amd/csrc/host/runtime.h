@@ -15,7 +15,7 @@
 namespace homura {
 
 enum class DType : int { F32 = HM_DTYPE_F32, BF16 = HM_DTYPE_BF16, Q8_0 = HM_DTYPE_Q8_0,
-                         Q4_0 = HM_DTYPE_Q4_0, I64 = HM_DTYPE_I64 };
+                         Q4_0 = HM_DTYPE_Q4_0, I64 = HM_DTYPE_I64, Q4_K = HM_DTYPE_Q4_K, Q6_K = HM_DTYPE_Q6_K };
 
 // reference src/dtype.rs:8-92 (sizes and block maths of the supported subset)
 size_t dtype_size_bytes(DType t);       // 0 for block types

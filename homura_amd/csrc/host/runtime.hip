@@ -16,12 +16,19 @@ size_t dtype_size_bytes(DType t) {
     default: return 0;
     }
 }
-bool dtype_is_quantized(DType t) { return t == DType::Q8_0 || t == DType::Q4_0; }
-size_t dtype_block_size(DType t) { return dtype_is_quantized(t) ? 32 : 1; }
+bool dtype_is_quantized(DType t) {
+    return t == DType::Q8_0 || t == DType::Q4_0 || t == DType::Q4_K || t == DType::Q6_K;
+}
+size_t dtype_block_size(DType t) {
+    if (t == DType::Q4_K || t == DType::Q6_K) return 256;
+    return dtype_is_quantized(t) ? 32 : 1;
+}
 size_t dtype_block_bytes(DType t) {
     switch (t) {
     case DType::Q8_0: return 34;
     case DType::Q4_0: return 18;
+    case DType::Q4_K: return 144;
+    case DType::Q6_K: return 210;
     default: return dtype_size_bytes(t);
     }
 }

@@ -11,7 +11,7 @@ import numpy as np
 
 from . import _ffi
 
-DTYPE_F32, DTYPE_BF16, DTYPE_Q8_0, DTYPE_Q4_0, DTYPE_I64 = 0, 1, 2, 3, 4
+DTYPE_F32, DTYPE_BF16, DTYPE_Q8_0, DTYPE_Q4_0, DTYPE_I64, DTYPE_Q4_K, DTYPE_Q6_K = 0, 1, 2, 3, 4, 5, 6
 
 
 class HomuraError(RuntimeError):
@@ -248,10 +248,19 @@ class HfModel:
     in TransformerWeights::to_slot_buffers order, then run_kv / generate run on the GPU."""
 
     def __init__(self, ctx: Context, config: TransformerConfig, weight_dtype: int = DTYPE_BF16,
-                 has_qk_norm: bool = False):
+                 has_qk_norm: bool = False, proj_dtypes=None):
+        """proj_dtypes: optional 7 DTYPE_* codes per layer (q, k, v, o, gate, up, down) for a quantised
+        model whose projections differ in type (then weight_dtype is ignored)."""
         self.ctx, self.config, self.lib = ctx, config, ctx.lib
         cfg = config.to_c()
-        self.h = self.lib.hm_model_create(ctx.h, C.byref(cfg), weight_dtype, int(has_qk_norm))
+        if proj_dtypes is not None:
+            flat = [int(t) for t in proj_dtypes]
+            if len(flat) != 7 * config.num_hidden_layers:
+                raise ValueError(f"need {7 * config.num_hidden_layers} projection dtypes, got {len(flat)}")
+            arr = (C.c_int * len(flat))(*flat)
+            self.h = self.lib.hm_model_create_mixed(ctx.h, C.byref(cfg), arr, int(has_qk_norm))
+        else:
+            self.h = self.lib.hm_model_create(ctx.h, C.byref(cfg), weight_dtype, int(has_qk_norm))
         if not self.h:
             raise HomuraError(-1, (self.lib.hm_last_error(ctx.h) or b"").decode())
 

@@ -9,7 +9,8 @@ from __future__ import annotations
 import numpy as np
 
 from . import synth
-from .runtime import DTYPE_BF16, DTYPE_Q4_0, DTYPE_Q8_0, Context, HfModel, TransformerConfig
+from .runtime import (DTYPE_BF16, DTYPE_Q4_0, DTYPE_Q4_K, DTYPE_Q6_K, DTYPE_Q8_0, Context, HfModel,
+                      TransformerConfig)
 
 # Qwen3-0.6B shape (reference src/hf/config.rs:125-150): the decode benchmark configuration
 QWEN3_0P6B = TransformerConfig(
@@ -36,11 +37,29 @@ TINY_LLAMA = TransformerConfig(
     max_position_embeddings=512, tie_word_embeddings=False)
 
 
+# K-quant proportions (every projection input a multiple of 256) for Q4_K / Q6_K files
+TINY_K = TransformerConfig(
+    hidden_size=512, intermediate_size=768, num_attention_heads=8, num_hidden_layers=2,
+    vocab_size=640, num_key_value_heads=2, head_dim=64, rms_norm_eps=1e-5, rope_theta=1e4,
+    max_position_embeddings=512, tie_word_embeddings=False)
+
+
+def q4_k_m_mix(cfg: TransformerConfig):
+    """Per-projection types in the manner of llama.cpp's Q4_K_M files: Q4_K throughout, attn_v and
+    ffn_down in Q6_K for part of the layers (here: the even ones). 7 per layer: q k v o gate up down."""
+    out = []
+    for l in range(cfg.num_hidden_layers):
+        hi = DTYPE_Q6_K if l % 2 == 0 else DTYPE_Q4_K
+        out += [DTYPE_Q4_K, DTYPE_Q4_K, hi, DTYPE_Q4_K, DTYPE_Q4_K, DTYPE_Q4_K, hi]
+    return out
+
+
 def synth_weights(cfg: TransformerConfig, seed: int, weight_dtype: int = DTYPE_BF16,
-                  has_qk_norm: bool = True):
+                  has_qk_norm: bool = True, proj_dtypes=None):
     """[(name, array)] in slot order. Projections: bf16 bits [K, N], or raw GGUF blocks
-    [N][K/32] for Q8_0 / Q4_0 (then the LM head is f32 [hidden, vocab], as in the reference's
-    quantised plan, src/hf/weights.rs:174-180)."""
+    [N][K/block] for Q8_0 / Q4_0 / Q4_K / Q6_K (then the LM head is f32 [hidden, vocab], as in the
+    reference's quantised plan, src/hf/weights.rs:174-180). proj_dtypes: 7 types per layer
+    (q k v o gate up down) instead of one weight_dtype."""
     hidden, inter, vocab = cfg.hidden_size, cfg.intermediate_size, cfg.vocab_size
     hd = cfg.get_head_dim()
     qd, kvd = cfg.num_attention_heads * hd, cfg.kv_heads() * hd
@@ -63,12 +82,22 @@ def synth_weights(cfg: TransformerConfig, seed: int, weight_dtype: int = DTYPE_B
 
     qseed = [seed * 7919 + 1]
 
+    pidx = [0]
+
     def proj(K, N):
-        if weight_dtype == DTYPE_BF16:
+        dt = weight_dtype
+        if proj_dtypes is not None:
+            dt = proj_dtypes[pidx[0]]
+            pidx[0] += 1
+        if dt == DTYPE_BF16:
             return normal_bits(K * N, 0.02).reshape(K, N)
         qseed[0] += 1
+        if dt == DTYPE_Q4_K:    # w = d*sc*q - dmin*m with sc, m < 64 and q < 16
+            return synth.q4_k_blocks(qseed[0], N * (K // 256), 0.02 / 260.0)
+        if dt == DTYPE_Q6_K:    # w = d*sc*q with |sc| < 128 and |q| <= 32
+            return synth.q6_k_blocks(qseed[0], N * (K // 256), 0.02 / 1400.0)
         nb = N * (K // 32)
-        if weight_dtype == DTYPE_Q8_0:   # w = q * d with q in [-127,127]: d ~ 0.02 / 73
+        if dt == DTYPE_Q8_0:   # w = q * d with q in [-127,127]: d ~ 0.02 / 73
             return synth.q8_0_blocks(qseed[0], nb, 0.02 / 73.0 * 1.25)
         return synth.q4_0_blocks(qseed[0], nb, 0.02 / 4.6 * 1.25)
 
@@ -100,7 +129,7 @@ def synth_weights(cfg: TransformerConfig, seed: int, weight_dtype: int = DTYPE_B
         head_bits = np.ascontiguousarray(embed_bits.T)          # [hidden, vocab]
     else:
         head_bits = normal_bits(hidden * vocab, 0.02).reshape(hidden, vocab)
-    if weight_dtype == DTYPE_BF16:
+    if weight_dtype == DTYPE_BF16 and proj_dtypes is None:
         out.append(("lm_head.weight", head_bits))
     else:
         out.append(("lm_head.weight", synth.bf16_to_f32(head_bits)))
@@ -119,8 +148,8 @@ def synth_kv(cfg: TransformerConfig, seed: int, seq_len: int):
 
 
 def build_model(ctx: Context, cfg: TransformerConfig, weights, max_seq_len: int,
-                weight_dtype: int = DTYPE_BF16, has_qk_norm: bool = True) -> HfModel:
-    m = HfModel(ctx, cfg, weight_dtype, has_qk_norm)
+                weight_dtype: int = DTYPE_BF16, has_qk_norm: bool = True, proj_dtypes=None) -> HfModel:
+    m = HfModel(ctx, cfg, weight_dtype, has_qk_norm, proj_dtypes=proj_dtypes)
     slots = m.weight_slots()
     if len(slots) != len(weights):
         raise ValueError(f"model lists {len(slots)} weight slots, got {len(weights)} arrays")

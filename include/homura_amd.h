@@ -206,6 +206,8 @@ typedef struct {
 #define HM_DTYPE_Q8_0 2
 #define HM_DTYPE_Q4_0 3
 #define HM_DTYPE_I64 4
+#define HM_DTYPE_Q4_K 5
+#define HM_DTYPE_Q6_K 6
 
 /* HfModel::load_with_dtype / load_gguf stand-in (src/hf/model.rs:46-145) for weights that
  * are already in host memory: create, hand over every weight slot in
@@ -213,6 +215,11 @@ typedef struct {
  * `weight_dtype` is the dtype of the seven projections (BF16, Q8_0 or Q4_0). */
 hm_model *hm_model_create(hm_ctx *ctx, const hm_transformer_config *cfg, int weight_dtype,
                           int has_qk_norm);
+/* A quantised model whose projections do not all share one type (Q4_K_M files keep some in Q6_K):
+ * proj_dtypes holds 7 HM_DTYPE_* codes per layer in the order q, k, v, o, gate, up, down. The
+ * reference carries the type per weight buffer (Buffer dtype, src/hf/weights.rs:136-183). */
+hm_model *hm_model_create_mixed(hm_ctx *ctx, const hm_transformer_config *cfg, const int *proj_dtypes,
+                                int has_qk_norm);
 void hm_model_destroy(hm_model *m);
 int hm_model_num_weight_slots(hm_model *m);
 /* name is copied into buf; dtype/rows/cols describe the host buffer expected for the slot */
@@ -291,6 +298,10 @@ int hm_gguf_tensor_info(const hm_gguf *g, int index, char *name_buf, size_t bufl
                         uint64_t dims[8], int *ggml_type, uint64_t *offset, size_t *nbytes);
 int hm_gguf_find_tensor(const hm_gguf *g, const char *name); /* index, -1 when absent */
 const void *hm_gguf_tensor_data(const hm_gguf *g, int index); /* raw bytes in the mapping */
+/* GgufFile::load_f32_buffer (src/gguf.rs:727-776): the tensor as f32 in host memory, dequantised
+ * when it is F16, BF16, Q8_0, Q4_0, Q4_K or Q6_K. out holds n_elements floats; HM_ERR_INVALID for
+ * a wrong count or a type without a conversion (message in err). Host only, no GPU involved. */
+int hm_gguf_tensor_f32(const hm_gguf *g, int index, float *out, size_t n_elements, char *err, size_t errlen);
 /* GgufValue::as_str / as_u64 / as_f32 (src/gguf.rs:200-233); HM_ERR_INVALID when the key is
  * absent or of another kind. hm_gguf_meta_str returns the string length. */
 int hm_gguf_meta_str(const hm_gguf *g, const char *key, char *buf, size_t buflen);

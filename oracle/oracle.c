@@ -771,7 +771,7 @@ ORC_API int orc_kv_init_from(orc_kv_cache *c, int layer, const float *k, const f
 
 /* ───────────────────────── whole decode step ───────────────────────── */
 
-enum { ORC_W_BF16 = 1, ORC_W_Q8_0 = 2, ORC_W_Q4_0 = 3 };
+enum { ORC_W_BF16 = 1, ORC_W_Q8_0 = 2, ORC_W_Q4_0 = 3, ORC_W_Q4_K = 4, ORC_W_Q6_K = 5 };
 
 typedef struct {
     int hidden, inter, heads, kv_heads, head_dim, layers, vocab;
@@ -790,6 +790,7 @@ typedef struct {
     const float *input_ln, *q_norm, *k_norm, *post_ln;
     const void *q, *k, *v, *o, *gate, *up, *down;
     const float *q_bias, *k_bias, *v_bias; /* NULL for models without Q/K/V bias */
+    int kinds[7]; /* ORC_W_* of q k v o gate up down; 0 = the model's weight_kind */
 } orc_layer_weights;
 
 typedef struct {
@@ -853,6 +854,13 @@ ORC_API void orc_model_set_layer_bias(orc_model *m, int l, const float *q_bias, 
     w->v_bias = v_bias;
 }
 
+/* Block types per projection for files that mix them (the reference keeps the type with each
+ * weight buffer and picks the QuantMM kernel per matrix, src/hf/emitter_quant.rs:675-702):
+ * kinds = ORC_W_* of q, k, v, o, gate, up, down. */
+ORC_API void orc_model_set_layer_kinds(orc_model *m, int l, const int *kinds) {
+    memcpy(m->layers[l].kinds, kinds, sizeof(m->layers[l].kinds));
+}
+
 /* q = emit_add(q, bias): the bias row broadcast over the sequence (src/hf/emitter.rs:604-619;
  * quantised plan: emit_post_qkv_kernel, src/hf/emitter_quant.rs:802-912). */
 static void add_bias(float *x, const float *bias, int S, int n) {
@@ -902,12 +910,14 @@ static void ensure_scratch(orc_model *m, int S, int total) {
     m->scratch_total = total;
 }
 
-static void proj(const orc_model *m, const float *x, const void *w, float *out, int M, int K,
-                 int N) {
-    switch (m->cfg.weight_kind) {
+static void proj(const orc_model *m, int kind, const float *x, const void *w, float *out, int M,
+                 int K, int N) {
+    switch (kind ? kind : m->cfg.weight_kind) {
     case ORC_W_BF16: orc_matmul_f32_bf16(x, (const uint16_t *)w, out, M, K, N); break;
     case ORC_W_Q8_0: orc_gemv_q8_0(x, (const uint8_t *)w, out, M, K, N); break;
     case ORC_W_Q4_0: orc_gemv_q4_0(x, (const uint8_t *)w, out, M, K, N); break;
+    case ORC_W_Q4_K: orc_gemv_q4_k(x, (const uint8_t *)w, out, M, K, N); break;
+    case ORC_W_Q6_K: orc_gemv_q6_k(x, (const uint8_t *)w, out, M, K, N); break;
     default: abort();
     }
 }
@@ -949,9 +959,9 @@ ORC_API int orc_model_run_kv(orc_model *m, const int64_t *ids, int S, float *log
             orc_rms_norm_f64acc(m->h, w->input_ln, m->normed, S, c->hidden, c->eps);
         else
             orc_rms_norm(m->h, w->input_ln, m->normed, S, c->hidden, c->eps);
-        proj(m, m->normed, w->q, m->q, S, c->hidden, qd);
-        proj(m, m->normed, w->k, m->k, S, c->hidden, kvd);
-        proj(m, m->normed, w->v, m->v, S, c->hidden, kvd);
+        proj(m, w->kinds[0], m->normed, w->q, m->q, S, c->hidden, qd);
+        proj(m, w->kinds[1], m->normed, w->k, m->k, S, c->hidden, kvd);
+        proj(m, w->kinds[2], m->normed, w->v, m->v, S, c->hidden, kvd);
         add_bias(m->q, w->q_bias, S, qd);
         add_bias(m->k, w->k_bias, S, kvd);
         add_bias(m->v, w->v_bias, S, kvd);
@@ -977,7 +987,7 @@ ORC_API int orc_model_run_kv(orc_model *m, const int64_t *ids, int S, float *log
         orc_gqa_attention(m->q, orc_kv_key_ptr(kv, l), orc_kv_value_ptr(kv, l), m->mask,
                           m->attn_flat, S, c->heads, c->kv_heads, hd, total,
                           orc_kv_head_stride(kv), quant, m->scores);
-        proj(m, m->attn_flat, w->o, m->attn_out, S, qd, c->hidden);
+        proj(m, w->kinds[3], m->attn_flat, w->o, m->attn_out, S, qd, c->hidden);
         /* MLP kernel: src/hf/emitter.rs:767-822 (quant: Residual+Norm :985-1071, QuantMM
          * gate/up, SiLU*Up :1077-1103, QuantMM down, ResAdd :1109-1134) */
         orc_add(m->h, m->attn_out, m->resid, (size_t)S * c->hidden);
@@ -985,10 +995,10 @@ ORC_API int orc_model_run_kv(orc_model *m, const int64_t *ids, int S, float *log
             orc_rms_norm_f64acc(m->resid, w->post_ln, m->normed, S, c->hidden, c->eps);
         else
             orc_rms_norm(m->resid, w->post_ln, m->normed, S, c->hidden, c->eps);
-        proj(m, m->normed, w->gate, m->gate, S, c->hidden, c->inter);
-        proj(m, m->normed, w->up, m->up, S, c->hidden, c->inter);
+        proj(m, w->kinds[4], m->normed, w->gate, m->gate, S, c->hidden, c->inter);
+        proj(m, w->kinds[5], m->normed, w->up, m->up, S, c->hidden, c->inter);
         orc_silu_mul(m->gate, m->up, m->act, (size_t)S * c->inter);
-        proj(m, m->act, w->down, m->down, S, c->inter, c->hidden);
+        proj(m, w->kinds[6], m->act, w->down, m->down, S, c->inter, c->hidden);
         orc_add(m->resid, m->down, m->h, (size_t)S * c->hidden);
     }
     /* LM head: src/hf/emitter.rs:828-862 (bf16 weights, f32 RMSNorm); the quantised plan

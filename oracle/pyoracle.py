@@ -14,7 +14,7 @@ import numpy as np
 HERE = Path(__file__).resolve().parent
 LIB_PATH = HERE / "liboracle.so"
 
-W_BF16, W_Q8_0, W_Q4_0 = 1, 2, 3
+W_BF16, W_Q8_0, W_Q4_0, W_Q4_K, W_Q6_K = 1, 2, 3, 4, 5
 
 _P = C.c_void_p
 _I = C.c_int
@@ -90,6 +90,7 @@ def load() -> C.CDLL:
         "orc_model_set_global": (None, [_P, _P, _P, _P, _P, _P, _I]),
         "orc_model_set_layer": (None, [_P, _I] + [_P] * 11),
         "orc_model_set_layer_bias": (None, [_P, _I, _P, _P, _P]),
+        "orc_model_set_layer_kinds": (None, [_P, _I, C.POINTER(_I)]),
         "orc_model_attach_kv": (None, [_P, _P]),
         "orc_model_free": (None, [_P]),
         "orc_model_run_kv": (_I, [_P, _P, _I, _P]),
@@ -371,6 +372,11 @@ class Model:
     def set_layer_bias(self, l, q_bias, k_bias, v_bias):
         self.lib.orc_model_set_layer_bias(self.h, l, self._hold(_f32(q_bias)), self._hold(_f32(k_bias)),
                                           self._hold(_f32(v_bias)))
+
+    def set_layer_kinds(self, l, kinds):
+        """W_* of q, k, v, o, gate, up, down for a layer whose projections differ in block type."""
+        assert len(kinds) == 7
+        self.lib.orc_model_set_layer_kinds(self.h, l, (C.c_int * 7)(*[int(k) for k in kinds]))
 
     def run_kv(self, ids):
         ids = np.ascontiguousarray(ids, np.int64).reshape(-1)

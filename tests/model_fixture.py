@@ -13,12 +13,14 @@ for p in (str(ROOT), str(ROOT / "oracle")):
         sys.path.insert(0, p)
 
 from homura_amd import synth, synth_model  # noqa: E402
-from homura_amd.runtime import DTYPE_BF16, DTYPE_Q4_0, DTYPE_Q8_0  # noqa: E402
+from homura_amd.runtime import DTYPE_BF16, DTYPE_Q4_0, DTYPE_Q4_K, DTYPE_Q6_K, DTYPE_Q8_0  # noqa: E402
 
 
-def build_oracle_model(cfg, weights, max_seq_len, weight_dtype=DTYPE_BF16, has_qk_norm=True):
+def build_oracle_model(cfg, weights, max_seq_len, weight_dtype=DTYPE_BF16, has_qk_norm=True, proj_dtypes=None):
     import pyoracle
-    kind = {DTYPE_BF16: pyoracle.W_BF16, DTYPE_Q8_0: pyoracle.W_Q8_0, DTYPE_Q4_0: pyoracle.W_Q4_0}[weight_dtype]
+    kinds = {DTYPE_BF16: pyoracle.W_BF16, DTYPE_Q8_0: pyoracle.W_Q8_0, DTYPE_Q4_0: pyoracle.W_Q4_0,
+             DTYPE_Q4_K: pyoracle.W_Q4_K, DTYPE_Q6_K: pyoracle.W_Q6_K}
+    kind = kinds[proj_dtypes[0] if proj_dtypes is not None else weight_dtype]
     m = pyoracle.Model(cfg.hidden_size, cfg.intermediate_size, cfg.num_attention_heads, cfg.kv_heads(),
                        cfg.get_head_dim(), cfg.num_hidden_layers, cfg.vocab_size, cfg.rms_norm_eps,
                        weight_kind=kind, has_qk_norm=has_qk_norm, rope_theta=cfg.rope_theta,
@@ -33,6 +35,8 @@ def build_oracle_model(cfg, weights, max_seq_len, weight_dtype=DTYPE_BF16, has_q
                     w[p + "self_attn.o_proj.weight"], w[p + "post_attention_layernorm.weight"],
                     w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"],
                     w[p + "mlp.down_proj.weight"])
+        if proj_dtypes is not None:
+            m.set_layer_kinds(l, [kinds[t] for t in proj_dtypes[7 * l:7 * l + 7]])
         if cfg.attention_bias:
             m.set_layer_bias(l, w[p + "self_attn.q_proj.bias"], w[p + "self_attn.k_proj.bias"],
                              w[p + "self_attn.v_proj.bias"])

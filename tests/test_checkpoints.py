@@ -242,3 +242,32 @@ def test_config_errors_and_head_dim():
                               '"num_hidden_layers": 28, "vocab_size": 151936, "head_dim": 128, '
                               '"nested": {"a": [1, 2.5e3, -3, null, false], "s": "q\\"\\u00e9\\n"}}')
     assert cfg.get_head_dim() == 128
+
+
+def test_gguf_tensor_f32_dequantises_like_the_oracle(tmp_path):
+    """reference load_f32_buffer (src/gguf.rs:727-776): F32 as stored, F16/BF16 widened, Q8_0/Q4_0/Q4_K/
+    Q6_K dequantised. The host conversion must give the oracle's floats bit for bit (the oracle's
+    decodes are pinned by the reference's known-answer tests and independent numpy decodes)."""
+    import pyoracle
+    from homura_amd import synth
+    rng = np.random.default_rng(5)
+    f32 = rng.standard_normal(64).astype(np.float32)
+    f16 = rng.standard_normal(64).astype(np.float16)
+    b16 = synth.normal_bf16(9, 64, 1.0)
+    q8, q4 = synth.q8_0_blocks(1, 6), synth.q4_0_blocks(2, 6)
+    q4k, q6k = synth.q4_k_blocks(3, 5), synth.q6_k_blocks(4, 5)
+    tensors = [("f32", (4, 16), ck.GGML_F32, f32.tobytes()), ("f16", (64,), ck.GGML_F16, f16.tobytes()),
+               ("bf16", (64,), ck.GGML_BF16, b16.tobytes()), ("q8_0", (6, 32), ck.GGML_Q8_0, q8.tobytes()),
+               ("q4_0", (3, 64), ck.GGML_Q4_0, q4.tobytes()), ("q4_k", (5, 256), ck.GGML_Q4_K, q4k.tobytes()),
+               ("q6_k", (5, 256), ck.GGML_Q6_K, q6k.tobytes()), ("q5_k", (256,), ck.GGML_Q5_K, bytes(176))]
+    want = {"f32": f32.reshape(4, 16), "f16": f16.astype(np.float32), "bf16": synth.bf16_to_f32(b16),
+            "q8_0": pyoracle.dequant_q8_0(q8).reshape(6, 32), "q4_0": pyoracle.dequant_q4_0(q4).reshape(3, 64),
+            "q4_k": pyoracle.dequant_q4_k(q4k).reshape(5, 256), "q6_k": pyoracle.dequant_q6_k(q6k).reshape(5, 256)}
+    with ck.GgufFile(write(tmp_path, "kinds.gguf", cw.gguf_bytes([], tensors))) as g:
+        for name, w in want.items():
+            got = g.tensor_f32(name)
+            assert got.shape == w.shape and np.array_equal(got.view(np.uint32), w.view(np.uint32)), name
+        with pytest.raises(ValueError, match="q5_k"):
+            g.tensor_f32("q5_k")
+        with pytest.raises(KeyError):
+            g.tensor_f32("absent")

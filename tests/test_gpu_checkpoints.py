@@ -13,7 +13,7 @@ import ckpt_writers as cw
 import model_fixture as mf
 import pyoracle
 from homura_amd import HfModel, checkpoints as ck, synth, synth_model
-from homura_amd.runtime import DTYPE_BF16, DTYPE_Q4_0, DTYPE_Q8_0, HomuraError
+from homura_amd.runtime import DTYPE_BF16, DTYPE_Q4_0, DTYPE_Q4_K, DTYPE_Q6_K, DTYPE_Q8_0, HomuraError
 
 pytestmark = pytest.mark.gpu
 
@@ -104,6 +104,47 @@ def test_load_quantised_gguf(ctx, tmp_path, wdt, code, name):
     gm.close()
 
 
+def test_load_q4_k_m_style_gguf(ctx, tmp_path):
+    """A file quantised the way llama.cpp's Q4_K_M recipe does it: projections in Q4_K with attn_v and
+    ffn_down of some layers in Q6_K, the token embedding in Q4_K and the output matrix in Q6_K (both
+    dequantised on load, src/gguf.rs:759-764), f32 norms."""
+    cfg = synth_model.TINY_K
+    mix = synth_model.q4_k_m_mix(cfg)
+    weights = synth_model.synth_weights(cfg, 43, has_qk_norm=False, proj_dtypes=mix)
+    V, Hd = cfg.vocab_size, cfg.hidden_size
+    emb_blocks = synth.q4_k_blocks(811, V * Hd // 256, 0.02 / 260.0)
+    head_blocks = synth.q6_k_blocks(812, V * Hd // 256, 0.02 / 1400.0)
+    emb = pyoracle.dequant_q4_k(emb_blocks).reshape(V, Hd)
+    head = np.ascontiguousarray(pyoracle.dequant_q6_k(head_blocks).reshape(V, Hd).T)   # slot layout [hidden, vocab]
+    weights = [(n, emb if n == "model.embed_tokens.weight" else head if n == "lm_head.weight" else a)
+               for n, a in weights]
+    code = {DTYPE_Q4_K: ck.GGML_Q4_K, DTYPE_Q6_K: ck.GGML_Q6_K}
+    bb = {DTYPE_Q4_K: 144, DTYPE_Q6_K: 210}
+    tensors, pi = [], 0
+    for n, a in weights:
+        if n == "model.embed_tokens.weight":
+            tensors.append((gguf_name(n), (V, Hd), ck.GGML_Q4_K, emb_blocks.tobytes()))
+        elif n == "lm_head.weight":
+            tensors.append((gguf_name(n), (V, Hd), ck.GGML_Q6_K, head_blocks.tobytes()))
+        elif n.endswith("_proj.weight"):
+            K = {"q": Hd, "k": Hd, "v": Hd, "o": cfg.num_attention_heads * cfg.get_head_dim(), "gate": Hd, "up": Hd,
+                 "down": cfg.intermediate_size}[n.split(".")[-2].split("_")[0]]
+            dt = mix[pi]
+            pi += 1
+            tensors.append((gguf_name(n), (a.size // (K // 256) // bb[dt], K), code[dt], a.tobytes()))
+        else:
+            tensors.append((gguf_name(n), a.shape, ck.GGML_F32, a.tobytes()))
+    path = tmp_path / "tiny-q4_k_m.gguf"
+    path.write_bytes(cw.gguf_bytes(gguf_metadata(cfg, "llama"), tensors))
+    gm = HfModel.load_gguf(ctx, path, 96)
+    assert gm.weight_dtype == DTYPE_Q4_K and gm.has_qk_norm is False and gm.config.tie_word_embeddings is False
+    slot_types = [s[1] for s in gm.weight_slots() if s[0].endswith("_proj.weight")]
+    assert slot_types == mix
+    om = mf.build_oracle_model(cfg, weights, 96, has_qk_norm=False, proj_dtypes=mix)
+    check_against_oracle(gm, om, cfg, "gguf q4_k_m")
+    gm.close()
+
+
 def test_load_bf16_gguf_tied_qknorm(ctx, tmp_path):
     """Qwen3-style file with unquantised projections: BF16 tensors as they are, the F32 ones cut to
     their top 16 bits (reference f32_buf_to_bf16), tied head, QK-norm."""
@@ -187,11 +228,18 @@ def test_loader_errors_are_reported(ctx, tmp_path):
     cfg = synth_model.TINY_LLAMA
     with pytest.raises(HomuraError, match="No such file"):
         HfModel.load_gguf(ctx, tmp_path / "absent.gguf")
-    # a K-quant file: understood by the parser, refused by the loader with the reason
-    t = [("blk.0.attn_q.weight", (256, 256), ck.GGML_Q4_K, bytes(256 * 144))]
-    p = tmp_path / "q4k.gguf"
+    # a Q5_K projection: understood by the parser, refused by the loader with the reason
+    t = [("blk.0.attn_q.weight", (256, 256), ck.GGML_Q5_K, bytes(256 * 176))]
+    p = tmp_path / "q5k.gguf"
     p.write_bytes(cw.gguf_bytes(gguf_metadata(cfg, "llama"), t))
-    with pytest.raises(HomuraError, match="projection weights are Q4_K"):
+    with pytest.raises(HomuraError, match="blk.0.attn_q.weight is Q5_K"):
+        HfModel.load_gguf(ctx, p)
+    # float and block-quantised projections in one file
+    t = [(f"blk.{l}.{n}.weight", (32, 32), ck.GGML_Q8_0 if n == "attn_k" else ck.GGML_F32, bytes(32 * (34 if n == "attn_k" else 128)))
+         for l in range(cfg.num_hidden_layers) for n in ("attn_q", "attn_k", "attn_v", "attn_output", "ffn_gate", "ffn_up", "ffn_down")]
+    p = tmp_path / "halfquant.gguf"
+    p.write_bytes(cw.gguf_bytes(gguf_metadata(cfg, "llama"), t))
+    with pytest.raises(HomuraError, match="some projections are block-quantised and some are float"):
         HfModel.load_gguf(ctx, p)
     p = tmp_path / "empty.gguf"
     p.write_bytes(cw.gguf_bytes(gguf_metadata(cfg, "llama"), []))

@@ -205,3 +205,46 @@ def test_qkv_bias_model_against_oracle(ctx, wdt, name):
     gm.run_kv(ids)
     assert np.array_equal(gm.generate_greedy(ids[:2], 24), want_t)
     gm.close()
+
+
+@pytest.mark.parametrize("which", ["q4_k", "q6_k", "q4_k_m_mix", "q8_0_q6_k_mix"])
+def test_kquant_plan_against_oracle(ctx, which):
+    """K-quant projections, one type throughout or mixed per matrix as Q4_K_M files are (attn_v and
+    ffn_down of some layers in Q6_K): same-type neighbours share a launch, the others get their own,
+    and the activation is rounded to Q8_K once per group."""
+    cfg = synth_model.TINY_K
+    L = cfg.num_hidden_layers
+    mix = {"q4_k": [5] * 7 * L, "q6_k": [6] * 7 * L, "q4_k_m_mix": synth_model.q4_k_m_mix(cfg),
+           # q alone, k|v stacked, gate and up apart: every way a group can split
+           "q8_0_q6_k_mix": [2, 6, 6, 2, 6, 5, 2] + [6, 2, 6, 5, 5, 5, 6] * (L - 1)}[which]
+    weights = synth_model.synth_weights(cfg, 57, has_qk_norm=False, proj_dtypes=mix)
+    gm = synth_model.build_model(ctx, cfg, weights, 96, has_qk_norm=False, proj_dtypes=mix)
+    om = mf.build_oracle_model(cfg, weights, 96, has_qk_norm=False, proj_dtypes=mix)
+    assert [s[0] for s in gm.weight_slots()] == [n for n, _ in weights]
+    kv = synth_model.synth_kv(cfg, 3, 29)
+    gm.init_kv_cache(kv, 29)
+    mf.oracle_init_kv(om, kv)
+    ids = synth.token_ids(4, 5, cfg.vocab_size)
+    got = gm.run_kv(ids)
+    want = np.concatenate([om.run_kv(ids[i:i + 1]) for i in range(5)])
+    for i in range(5):
+        assert mf.rel_err(got[i], want[i]) < 1e-2, f"{which} position {i}"
+    want_t, margins = om.generate_greedy(ids[:2], 24)
+    got_t = gm.generate_greedy(ids[:2], 24)
+    say(f"{which}: min margin {margins.min():.3e}")
+    assert np.array_equal(got_t, want_t)
+    gm.set_graph(True)
+    gm.init_kv_cache(kv, 29)
+    gm.run_kv(ids)
+    assert np.array_equal(gm.generate_greedy(ids[:2], 24), want_t)
+    gm.close()
+
+
+def test_mixed_model_rejects_bad_dtype_lists(ctx):
+    cfg = synth_model.TINY_K
+    with pytest.raises(ValueError):
+        HfModel(ctx, cfg, proj_dtypes=[5] * 7)                       # 7 per layer needed
+    with pytest.raises(HomuraError):
+        HfModel(ctx, cfg, proj_dtypes=[1] * 7 * cfg.num_hidden_layers)  # bf16 is not a block type
+    with pytest.raises(HomuraError):                                 # hidden 256*k needed for K-quants
+        HfModel(ctx, synth_model.TINY_LLAMA, proj_dtypes=[2, 2, 2, 2, 2, 2, 5] * 2)  # inter 704 % 256 != 0

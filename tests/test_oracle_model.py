@@ -178,3 +178,68 @@ def test_quant_oracle_plan_runs_and_dequant_equivalence():
     logits = om.run_kv(synth.token_ids(3, 4, cfg.vocab_size))
     assert logits.shape == (4, cfg.vocab_size) and np.isfinite(logits).all()
     assert om.kv.current_len() == 4
+
+
+def test_mixed_kquant_oracle_step_against_numpy_fp64():
+    """A model whose projections mix Q4_K and Q6_K (as Q4_K_M files do): the oracle must pick the
+    decode per matrix. Independent float64 forward: every projection is (activation rounded to
+    Q8_K) @ (blocks dequantised by the matrix's own type); a type applied to the wrong matrix reads
+    blocks of the wrong size and lands far outside the tolerance."""
+    import pyoracle
+    from homura_amd.runtime import DTYPE_Q4_K, DTYPE_Q6_K
+    cfg = synth_model.TINY_K
+    mix = synth_model.q4_k_m_mix(cfg)
+    assert DTYPE_Q6_K in mix and DTYPE_Q4_K in mix and mix[2] != mix[9]  # v of layers 0 and 1 differ
+    W = dict(synth_model.synth_weights(cfg, 21, has_qk_norm=False, proj_dtypes=mix))
+    hd, H, kvh = cfg.get_head_dim(), cfg.num_attention_heads, cfg.kv_heads()
+    past = 9
+    kv = synth_model.synth_kv(cfg, 5, past)
+    om = mf.build_oracle_model(cfg, list(W.items()), 32, has_qk_norm=False, proj_dtypes=mix)
+    mf.oracle_init_kv(om, kv)
+    tok = 77
+    got = om.run_kv([tok])[0]
+
+    def act_q8k(x):
+        out = np.empty(x.size)
+        for b in range(x.size // 256):
+            q, d, _ = pyoracle.quantize_q8_k(x[256 * b:256 * b + 256].astype(np.float32))
+            out[256 * b:256 * b + 256] = q.astype(np.float64) * d
+        return out
+
+    order = ["self_attn.q_proj", "self_attn.k_proj", "self_attn.v_proj", "self_attn.o_proj", "mlp.gate_proj",
+             "mlp.up_proj", "mlp.down_proj"]
+
+    def mm(l, name, x):
+        dt = mix[7 * l + order.index(name)]
+        blocks = W[f"model.layers.{l}.{name}.weight"]
+        w = (pyoracle.dequant_q6_k if dt == DTYPE_Q6_K else pyoracle.dequant_q4_k)(blocks)
+        return w.reshape(-1, x.size).astype(np.float64) @ act_q8k(x)
+
+    f = lambda a: a.astype(np.float64)
+    rms = lambda x, w: x / np.sqrt((x * x).mean(-1, keepdims=True) + cfg.rms_norm_eps) * w
+    bf = lambda x: synth.bf16_to_f32(synth.f32_to_bf16_rne(x.astype(np.float32))).astype(np.float64)
+    h = f(W["model.embed_tokens.weight"])[tok]
+    i = np.arange(hd // 2)
+    ang = past / (cfg.rope_theta ** (2 * i / hd))
+    cos, sin = np.concatenate([np.cos(ang)] * 2), np.concatenate([np.sin(ang)] * 2)
+    rot = lambda x: np.concatenate([-x[..., hd // 2:], x[..., :hd // 2]], -1)
+    for l in range(cfg.num_hidden_layers):
+        p = f"model.layers.{l}."
+        n = rms(h, f(W[p + "input_layernorm.weight"]))
+        q, k, v = (mm(l, f"self_attn.{x}_proj", n) for x in "qkv")
+        q, k, v = q.reshape(H, hd), k.reshape(kvh, hd), v.reshape(kvh, hd)
+        q, k = q * cos + rot(q) * sin, k * cos + rot(k) * sin
+        K = np.concatenate([kv[2 * l][0].astype(np.float64), bf(k)[:, None, :]], 1)
+        V = np.concatenate([kv[2 * l + 1][0].astype(np.float64), bf(v)[:, None, :]], 1)
+        o = np.zeros((H, hd))
+        for hh in range(H):
+            s = K[hh // (H // kvh)] @ q[hh] / np.sqrt(hd)
+            pr = np.exp(s - s.max())
+            o[hh] = (pr / pr.sum()) @ V[hh // (H // kvh)]
+        r = h + mm(l, "self_attn.o_proj", o.reshape(-1))
+        n2 = rms(r, f(W[p + "post_attention_layernorm.weight"]))
+        g, u = mm(l, "mlp.gate_proj", n2), mm(l, "mlp.up_proj", n2)
+        h = r + mm(l, "mlp.down_proj", g / (1 + np.exp(-g)) * u)
+    want = rms(h, f(W["model.norm.weight"])) @ f(W["lm_head.weight"])
+    assert np.abs(want).max() > 1e-3
+    assert mf.rel_err(got, want) < 2e-3
