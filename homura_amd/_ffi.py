@@ -80,6 +80,7 @@ SIGNATURES = {
     "hm_dequant_q6_k": (_I, [_P, _P, _P, _SZ]),
     "hm_gemm_bf16": (_I, [_P, _P, _P, _P, _I, _I, _I]),
     "hm_gemm_bf16_nk": (_I, [_P, _P, _P, _P, _I, _I, _I]),
+    "hm_gemm_f32_bf16_nk": (_I, [_P, _P, _P, _P, _I, _I, _I]),
     "hm_model_set_weight_nk": (_I, [_P, _I, _P, _SZ]),
     "hm_model_config": (_I, [_P, _P, _P, _P]),
     "hm_gguf_open": (_P, [C.c_char_p, C.c_char_p, _SZ]),
@@ -109,6 +110,7 @@ SIGNATURES = {
     "hm_ciface_unbind": (None, []),
     "hm_kv_append": (_I, [_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I]),
     "hm_gqa_decode_attn": (_I, [_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, C.c_float]),
+    "hm_gqa_prefill_attn": (_I, [_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, C.c_float]),
     "hm_rmsnorm": (_I, [_P, _P, _P, _P, _I, _I, C.c_float]),
     "hm_qknorm_rope": (_I, [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, C.c_float]),
     "hm_silu_mul": (_I, [_P, _P, _P, _P, _SZ]),
@@ -129,6 +131,9 @@ SIGNATURES = {
     "hm_model_kv_cache_len": (_I, [_P]),
     "hm_model_set_graph": (_I, [_P, _I]),
     "hm_model_run_kv": (_I, [_P, C.POINTER(C.c_int64), _I, c_f32_p]),
+    "hm_model_prefill": (_I, [_P, C.POINTER(C.c_int64), _I, c_f32_p]),
+    "hm_model_set_prefill_min": (_I, [_P, _I]),
+    "hm_model_set_prefill_pieces": (_I, [_P, _I]),
     "hm_model_generate_greedy": (_I, [_P, C.POINTER(C.c_int64), _I, _I, C.POINTER(C.c_int32)]),
     "hm_model_bench_decode": (_I, [_P, C.c_int64, _I, c_f32_p, C.POINTER(C.c_int32)]),
     "hm_model_profile_step": (_I, [_P, C.c_int64, C.POINTER(HmKernelProfile), _I]),

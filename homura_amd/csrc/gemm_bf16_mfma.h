@@ -1,0 +1,19 @@
+// Internal launch interface of the MFMA GEMM used by the prefill path.
+#pragma once
+
+#include <cstdint>
+
+#include "hm_common.h"
+
+namespace homura {
+
+// C[M][N] f32 = (sum of the pieces of A)[M][K] x B[N][K]^T. d_a_split is [M][pieces * K] bf16: piece p
+// of every f32 activation in columns [p K, (p+1) K) (what the kernels of prefill.hip write). B is the
+// K-contiguous stream layout of the model weights. K % 32 == 0, pieces 1..3.
+// With parts != NULL the product may be cut along K into up to max_parts slices when M x N alone
+// leaves most of the chip idle: slice s lands in d_c + s * M * N, *parts says how many there are, and
+// the caller adds them up in index order (d_c must hold max_parts * M * N floats).
+int gemm_split_nk(hm_ctx *ctx, const uint16_t *d_a_split, int pieces, const uint16_t *d_b_nk, float *d_c, int M, int K,
+                  int N, int max_parts = 1, int *parts = nullptr);
+
+}  // namespace homura

@@ -17,6 +17,21 @@
 //
 // Workgroups that share a B column block (the M/128 row blocks) get consecutive ids on one XCD, so
 // B is fetched from HBM once and served to the others from that XCD's L2.
+//
+// M and N need not be multiples of the tile: rows past the end re-read the last row and their
+// results are not stored. Split-operand mode (prefill of f32 activations): A is [M][P Kb], P = 2 or
+// 3 bf16 pieces of every activation side by side (piece p in columns [p Kb, (p+1) Kb)); the k loop
+// runs over P Kb and B's k index wraps at Kb, so C = (sum of the pieces) x B. Three pieces carry
+// all 24 significant bits of an f32.
+//
+// Split-K: grid.y workgroups share an output tile, each multiplies a contiguous range of K tiles and
+// writes its own partial C (partial s at C + s M N); the consumer adds the partials in index order,
+// so the sum does not depend on timing. For products whose M x N alone gives too few tiles to fill
+// the chip (the O and down projections of a prompt chunk).
+#include "gemm_bf16_mfma.h"
+
+#include <algorithm>
+
 #include "hm_common.h"
 
 namespace {
@@ -40,6 +55,7 @@ __device__ __forceinline__ void lds_barrier() {
 }
 
 constexpr int GEMM_THREADS = 512;
+constexpr int GEMM_DEPTH = 4;  // K tiles in flight in registers
 
 // Registers holding a thread's share of one K tile in flight (four 16-byte chunks):
 //   B [N][K]: v[0..1] two chunks of A, v[2..3] two chunks of B;
@@ -49,34 +65,50 @@ struct TileRegs {
     u32x4 v[4];
 };
 
+// M, N: logical sizes; K: length of the k loop; lda: row stride of A; Kb: k extent of B (k wraps at Kb)
+// kt_per_split: K tiles per grid.y slice (a multiple of the register ring depth)
+struct GemmDims {
+    int M, N, K, lda, Kb, kt_per_split;
+};
+
+// k index of B for loop index kc: the loop covers at most three copies of B's k range
+__device__ __forceinline__ int wrap_k(int kc, int Kb) {
+    kc = kc >= Kb ? kc - Kb : kc;
+    return kc >= Kb ? kc - Kb : kc;
+}
+
 // Requests one K tile. No branches on k: a chunk beyond K reads the last valid chunk of its row
 // (and is replaced by zeros when it is written to LDS), so the loop body stays one basic block and
 // the compiler can count exactly which loads a later LDS write has to wait for.
 template <bool B_NK>
 __device__ __forceinline__ void load_tile(TileRegs &t, const uint16_t *__restrict__ A,
-                                          const uint16_t *__restrict__ B, int m0, int n0, int k0, int K,
-                                          int N, int tid) {
+                                          const uint16_t *__restrict__ B, int m0, int n0, int k0,
+                                          const GemmDims &g, int tid) {
+    const int K = g.K;
     if (B_NK) {
 #pragma unroll
         for (int j = 0; j < 2; j++) {
             const int id = tid + j * GEMM_THREADS, r = id >> 3, c = id & 7;
             const int kc = min(k0 + c * 8, K - 8);
-            t.v[j] = ld128(A + (size_t)(m0 + r) * K + kc);
-            t.v[2 + j] = ld128(B + (size_t)(n0 + r) * K + kc);
+            const int kb = wrap_k(kc, g.Kb);
+            t.v[j] = ld128(A + (size_t)min(m0 + r, g.M - 1) * g.lda + kc);
+            t.v[2 + j] = ld128(B + (size_t)min(n0 + r, g.N - 1) * g.Kb + kb);
         }
     } else if (tid < 256) {  // wavefront-uniform
         const int ng = tid & 15, kg = tid >> 4;
+        const int nc = min(n0 + ng * 8, g.N - 8);
 #pragma unroll
         for (int r = 0; r < 4; r++) {
             const int kc = min(k0 + kg * 4 + r, K - 1);
-            t.v[r] = ld128(B + (size_t)kc * N + n0 + ng * 8);
+            const int kb = wrap_k(kc, g.Kb);
+            t.v[r] = ld128(B + (size_t)kb * g.N + nc);
         }
     } else {
 #pragma unroll
         for (int j = 0; j < 4; j++) {
             const int id = (tid - 256) + j * 256, r = id >> 3, c = id & 7;
             const int kc = min(k0 + c * 8, K - 8);
-            t.v[j] = ld128(A + (size_t)(m0 + r) * K + kc);
+            t.v[j] = ld128(A + (size_t)min(m0 + r, g.M - 1) * g.lda + kc);
         }
     }
 }
@@ -121,8 +153,8 @@ __device__ __forceinline__ void store_tile_part(const TileRegs &t, char *__restr
 template <bool B_NK>
 __global__ __launch_bounds__(GEMM_THREADS) void gemm_bf16_mfma_kernel(const uint16_t *__restrict__ A,
                                                                       const uint16_t *__restrict__ B,
-                                                                      float *__restrict__ C, int M, int K,
-                                                                      int N) {
+                                                                      float *__restrict__ C, const GemmDims g) {
+    const int M = g.M, K = g.K, N = g.N;
     __shared__ __attribute__((aligned(16))) char lds[2][2][TILE_BYTES];  // [buffer][A|B]
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -131,7 +163,7 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_bf16_mfma_kernel(const uint
 
     // XCD-aware tile order: ids are dealt round-robin to the 8 XCDs, so XCD x runs ids x, x+8, ...;
     // give each XCD a contiguous range of the (n block major, m block minor) order.
-    const int mb = M / TM, total = gridDim.x;
+    const int mb = (M + TM - 1) / TM, total = gridDim.x;  // tiles; gridDim.y = K slices
     int lin = blockIdx.x;
     if ((total & 7) == 0) lin = (blockIdx.x & 7) * (total >> 3) + (blockIdx.x >> 3);
     const int m0 = (lin % mb) * TM, n0 = (lin / mb) * TN;
@@ -147,14 +179,19 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_bf16_mfma_kernel(const uint
     // DEPTH tiles in flight in registers: tile j is requested DEPTH iterations before its LDS
     // writes, which sit next to the MFMA groups of tile j-1. The iteration count is rounded up to
     // a multiple of DEPTH (the extra tiles are zeros) so the register ring is indexed statically.
-    constexpr int DEPTH = 4;
-    const int nk = (K + TK - 1) / TK;
+    constexpr int DEPTH = GEMM_DEPTH;
+    // this workgroup's K tiles: [kt_first, kt_first + nk). A slice that is not the last one has a
+    // multiple of DEPTH tiles, so only the last one pads (with k >= K, i.e. zeros).
+    const int kt_first = blockIdx.y * g.kt_per_split;
+    const int nk = min(g.kt_per_split, (K + TK - 1) / TK - kt_first);
     const int nkp = (nk + DEPTH - 1) / DEPTH * DEPTH;
+    const int kbase = kt_first * TK;
+    C += (size_t)blockIdx.y * M * N;
     TileRegs t[DEPTH];
 #pragma unroll
-    for (int d = 0; d < DEPTH; d++) load_tile<B_NK>(t[d], A, B, m0, n0, d * TK, K, N, tid);
+    for (int d = 0; d < DEPTH; d++) load_tile<B_NK>(t[d], A, B, m0, n0, kbase + d * TK, g, tid);
 #pragma unroll
-    for (int part = 0; part < 2; part++) store_tile_part<B_NK>(t[0], lds[0][0], lds[0][1], tid, part, 0, K);
+    for (int part = 0; part < 2; part++) store_tile_part<B_NK>(t[0], lds[0][0], lds[0][1], tid, part, kbase, K);
     lds_barrier();
 
     // operand registers, two stages: the reads of the next step are in flight during the MFMAs
@@ -172,8 +209,8 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_bf16_mfma_kernel(const uint
         for (int u = 0; u < DEPTH; u++) {
             const int cur = u & 1;  // DEPTH is even: tile kt0+u sits in buffer u & 1
             // tile kt0+u left its registers during the previous iteration: refill them
-            load_tile<B_NK>(t[u], A, B, m0, n0, (kt0 + u + DEPTH) * TK, K, N, tid);
-            const int k_next = (kt0 + u + 1) * TK;
+            load_tile<B_NK>(t[u], A, B, m0, n0, kbase + (kt0 + u + DEPTH) * TK, g, tid);
+            const int k_next = kbase + (kt0 + u + 1) * TK;
             char *an = lds[cur ^ 1][0], *bn = lds[cur ^ 1][1];
 
             // first step: its operands are in stage 0; fetch the second step's meanwhile
@@ -230,37 +267,63 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_bf16_mfma_kernel(const uint
             for (int v = 0; v < 16; v++) {
                 const int row = m0 + wm * 64 + i * 32 + (v >> 2) * 8 + lh * 4 + (v & 3);
                 const int col = n0 + wn * 64 + j * 32 + l32;
-                __builtin_nontemporal_store(acc[i][j][v] + xch[((i * 2 + j) * 16 + v) * 64],
-                                            C + (size_t)row * N + col);
+                if (row < M && col < N)
+                    __builtin_nontemporal_store(acc[i][j][v] + xch[((i * 2 + j) * 16 + v) * 64],
+                                                C + (size_t)row * N + col);
             }
 }
 
 int gemm_launch(hm_ctx *ctx, const char *who, const uint16_t *a, const uint16_t *b, float *c, int M, int K,
-                int N, bool b_nk) {
+                int N, bool b_nk, int pieces, int ksplit = 1, int *ksplit_used = nullptr) {
     HM_CHECK_CTX(ctx);
     HM_REQUIRE(ctx, a && b && c, "%s: NULL pointer", who);
-    HM_REQUIRE(ctx, M > 0 && N > 0 && K > 0 && M % TM == 0 && N % TN == 0 && K % 32 == 0,
-               "%s: need M %% 128 == 0, N %% 128 == 0, K %% 32 == 0 (M=%d K=%d N=%d)", who, M, K, N);
+    HM_REQUIRE(ctx, M > 0 && N > 0 && K > 0 && K % 32 == 0, "%s: need M, N > 0 and K %% 32 == 0 (M=%d K=%d N=%d)", who,
+               M, K, N);
+    HM_REQUIRE(ctx, b_nk || N % 8 == 0, "%s: a [K][N] operand needs N %% 8 == 0 (N=%d)", who, N);
     HM_REQUIRE(ctx, ((uintptr_t)a % 16) == 0 && ((uintptr_t)b % 16) == 0, "%s: operands must be 16-byte aligned",
                who);
-    HM_REQUIRE(ctx, (long long)(M / TM) * (N / TN) <= 0x7fffffffLL, "%s: too many tiles", who);
-    const dim3 grid((M / TM) * (N / TN));
+    const long long tiles = (long long)((M + TM - 1) / TM) * ((N + TN - 1) / TN);
+    HM_REQUIRE(ctx, tiles <= 0x7fffffffLL, "%s: too many tiles", who);
+    GemmDims g;
+    g.M = M;
+    g.N = N;
+    g.Kb = K;
+    g.K = pieces * K;
+    g.lda = g.K;
+    const int nk_total = (g.K + TK - 1) / TK;
+    if (ksplit < 1) ksplit = 1;
+    g.kt_per_split = ((nk_total + ksplit - 1) / ksplit + GEMM_DEPTH - 1) / GEMM_DEPTH * GEMM_DEPTH;
+    const int slices = (nk_total + g.kt_per_split - 1) / g.kt_per_split;
+    if (ksplit_used) *ksplit_used = slices;
+    const dim3 grid((unsigned)tiles, (unsigned)slices);
     if (b_nk)
-        hipLaunchKernelGGL(gemm_bf16_mfma_kernel<true>, grid, dim3(GEMM_THREADS), 0, ctx->stream, a, b, c, M, K, N);
+        hipLaunchKernelGGL(gemm_bf16_mfma_kernel<true>, grid, dim3(GEMM_THREADS), 0, ctx->stream, a, b, c, g);
     else
-        hipLaunchKernelGGL(gemm_bf16_mfma_kernel<false>, grid, dim3(GEMM_THREADS), 0, ctx->stream, a, b, c, M, K, N);
+        hipLaunchKernelGGL(gemm_bf16_mfma_kernel<false>, grid, dim3(GEMM_THREADS), 0, ctx->stream, a, b, c, g);
     HM_LAUNCH_CHECK(ctx);
     return HM_OK;
 }
 
 }  // namespace
 
+int homura::gemm_split_nk(hm_ctx *ctx, const uint16_t *d_a_split, int pieces, const uint16_t *d_b_nk, float *d_c,
+                          int M, int K, int N, int max_parts, int *parts) {
+    HM_REQUIRE(ctx, pieces >= 1 && pieces <= 3, "gemm_split_nk: %d pieces (1..3)", pieces);
+    // K slices until the grid has about two workgroups per compute unit, at least 4 K tiles each
+    const long long tiles = (long long)((M + TM - 1) / TM) * ((N + TN - 1) / TN);
+    const int nk_total = (pieces * K + TK - 1) / TK;
+    int want = (int)((2LL * ctx->num_cus + tiles - 1) / tiles);
+    want = std::min(std::min(want, max_parts), std::max(1, nk_total / GEMM_DEPTH));
+    if (!parts) want = 1;
+    return gemm_launch(ctx, "gemm_split_nk", d_a_split, d_b_nk, d_c, M, K, N, true, pieces, want, parts);
+}
+
 extern "C" int hm_gemm_bf16(hm_ctx *ctx, const uint16_t *d_a_mk, const uint16_t *d_b_kn, float *d_c,
                             int M, int K, int N) {
-    return gemm_launch(ctx, "hm_gemm_bf16", d_a_mk, d_b_kn, d_c, M, K, N, false);
+    return gemm_launch(ctx, "hm_gemm_bf16", d_a_mk, d_b_kn, d_c, M, K, N, false, 1);
 }
 
 extern "C" int hm_gemm_bf16_nk(hm_ctx *ctx, const uint16_t *d_a_mk, const uint16_t *d_b_nk, float *d_c,
                                int M, int K, int N) {
-    return gemm_launch(ctx, "hm_gemm_bf16_nk", d_a_mk, d_b_nk, d_c, M, K, N, true);
+    return gemm_launch(ctx, "hm_gemm_bf16_nk", d_a_mk, d_b_nk, d_c, M, K, N, true, 1);
 }

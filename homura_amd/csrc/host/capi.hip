@@ -66,6 +66,24 @@ hm_model *hm_model_create_mixed(hm_ctx *ctx, const hm_transformer_config *cfg, c
 
 void hm_model_destroy(hm_model *m) { delete m; }
 
+int hm_model_prefill(hm_model *m, const int64_t *h_ids, int n_ids, float *h_logits) {
+    if (!m) return HM_ERR_INVALID;
+    return m->impl->prefill(h_ids, n_ids, h_logits);
+}
+
+int hm_model_set_prefill_pieces(hm_model *m, int pieces) {
+    if (!m) return HM_ERR_INVALID;
+    if (pieces != 2 && pieces != 3) return hm_set_error(m->ctx, HM_ERR_INVALID, "prefill pieces must be 2 or 3");
+    m->impl->set_prefill_pieces(pieces);
+    return HM_OK;
+}
+
+int hm_model_set_prefill_min(hm_model *m, int n_tokens) {
+    if (!m || n_tokens < 0) return HM_ERR_INVALID;
+    m->impl->set_prefill_min(n_tokens);
+    return HM_OK;
+}
+
 int hm_model_num_weight_slots(hm_model *m) {
     if (!m) return HM_ERR_INVALID;
     return (int)m->impl->weight_slot_infos().size();

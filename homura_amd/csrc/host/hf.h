@@ -3,6 +3,7 @@
 // src/hf/emitter_quant.rs, src/hf/model.rs).
 #pragma once
 
+#include <map>
 #include <memory>
 #include <string>
 #include <vector>
@@ -74,6 +75,18 @@ class HfModel {
     // reference HfModel::run_kv (src/hf/model.rs:198-218); multi-token input is consumed one
     // token per plan step. h_logits: [n_ids][vocab] or NULL.
     int run_kv(const int64_t *h_ids, int n_ids, float *h_logits);
+    // The multi-token pass behind run_kv for longer inputs (reference run_kv with seq > 1,
+    // src/hf/model.rs:321-336): the chunk goes through the layers as a matrix, projections on the
+    // matrix cores, causal attention over cache + chunk; n_ids rows are appended to the KV cache.
+    // bf16 plan, head_dim 64 or 128. h_logits: [n_ids][vocab] or NULL (then the LM head is skipped).
+    int prefill(const int64_t *h_ids, int n_ids, float *h_logits);
+    bool prefill_available() const;
+    // Inputs of at least this many tokens take the prefill pass (0 = never). Default 8.
+    void set_prefill_min(int n) { prefill_min_ = n; }
+    int prefill_min() const { return prefill_min_; }
+    // bf16 pieces per f32 activation in the prefill pass: 3 (all 24 significant bits, default) or 2
+    // (16 bits, two thirds of the matrix-core work)
+    void set_prefill_pieces(int n) { prefill_pieces_ = n; }
     int init_kv_cache(const float *const *h_kv, int seq_len);
     int reset_kv_cache();
     int kv_cache_len() const;
@@ -89,6 +102,8 @@ class HfModel {
     int emit_transformer_plan();        // reference src/hf/emitter.rs:867-1050
     int emit_transformer_plan_quant();  // reference src/hf/emitter_quant.rs:1142-1503
     int step_inputs(std::vector<Buffer *> &inputs);
+    int prefill_chunk(const int32_t *h_ids, int n, float *h_logits);
+    const float *weight_f32(const std::string &name) const;
     int check_ids(const int64_t *ids, int n, std::vector<int32_t> &out);
 
     hm_ctx *ctx_ = nullptr;
@@ -112,6 +127,16 @@ class HfModel {
     Buffer rope_cos_, rope_sin_;        // [max_position][head_dim] f32
     Buffer ids_view_, mask_view_;
     std::shared_ptr<PlanScratch> scratch_;
+    // prefill pass: activations of one chunk of rows
+    struct PrefillScratch {
+        static constexpr int MAX_PARTS = 8;  // K slices a projection result may come in
+        int rows = 0;
+        Buffer ids, h, resid, split, qkv, proj_out, gate_up, logits;
+    };
+    PrefillScratch pf_;
+    int prefill_min_ = 8;
+    int prefill_pieces_ = 3;
+    std::map<std::string, int> slot_by_name_;
     std::unique_ptr<ExecutionPlan> plan_;
 };
 

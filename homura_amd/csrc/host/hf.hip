@@ -6,7 +6,9 @@
 
 #include "../attention.h"
 #include "../gemv_bf16.h"
+#include "../gemm_bf16_mfma.h"
 #include "../gemv_kquant.h"
+#include "../prefill.h"
 #include "../light_ops.h"
 
 namespace homura {
@@ -116,6 +118,7 @@ std::unique_ptr<HfModel> HfModel::create(hm_ctx *ctx, const TransformerConfig &c
     else
         v.push_back(WeightSlotInfo{"lm_head.weight", DType::BF16, hidden, vocab, (size_t)(hidden * vocab) * 2});
 
+    for (size_t i = 0; i < v.size(); i++) m->slot_by_name_[v[i].name] = (int)i;
     m->weight_bufs_.resize(v.size());
     m->weight_set_.assign(v.size(), false);
     m->packed_.resize(cfg.num_hidden_layers);
@@ -1093,6 +1096,7 @@ int HfModel::run_kv(const int64_t *h_ids, int n_ids, float *h_logits) {
     std::vector<int32_t> ids;
     int rc = check_ids(h_ids, n_ids, ids);
     if (rc != HM_OK) return rc;
+    if (prefill_min_ > 0 && n_ids >= prefill_min_ && prefill_available()) return prefill(h_ids, n_ids, h_logits);
     if (n_ids > plan_->out_capacity())
         return hm_set_error(ctx_, HM_ERR_INVALID, "run_kv: %d ids exceed the step capacity %d", n_ids, plan_->out_capacity());
     if ((rc = plan_->arm(ids.data(), n_ids)) != HM_OK) return rc;
@@ -1108,6 +1112,140 @@ int HfModel::run_kv(const int64_t *h_ids, int n_ids, float *h_logits) {
         }
     }
     return hm_sync(ctx_);
+}
+
+// ── prefill pass ─────────────────────────────────────────────────────────────
+
+bool HfModel::prefill_available() const {
+    return finalized_ && weight_dtype_ == DType::BF16 && (cfg_.head_dim() == 64 || cfg_.head_dim() == 128) &&
+           cfg_.hidden_size % 32 == 0 && cfg_.q_dim() % 32 == 0 && cfg_.intermediate_size % 32 == 0;
+}
+
+const float *HfModel::weight_f32(const std::string &name) const {
+    auto it = slot_by_name_.find(name);
+    return it == slot_by_name_.end() ? nullptr : weight_bufs_[it->second].as<float>();
+}
+
+int HfModel::prefill(const int64_t *h_ids, int n_ids, float *h_logits) {
+    if (!finalized_) return hm_set_error(ctx_, HM_ERR_STATE, "model not finalized");
+    if (!prefill_available())
+        return hm_set_error(ctx_, HM_ERR_INVALID, "prefill: needs the bf16 plan with head_dim 64 or 128 and widths that are multiples of 32");
+    if (n_ids <= 0 || !h_ids) return hm_set_error(ctx_, HM_ERR_INVALID, "prefill: no input ids");
+    if (kv_cache_len() + n_ids > max_seq_len_)
+        return hm_set_error(ctx_, HM_ERR_STATE, "KV cache full (%d + %d > %d)", kv_cache_len(), n_ids, max_seq_len_);
+    std::vector<int32_t> ids;
+    int rc = check_ids(h_ids, n_ids, ids);
+    if (rc != HM_OK) return rc;
+    constexpr int CHUNK = 512;
+    for (int at = 0; at < n_ids; at += CHUNK) {
+        const int n = std::min(CHUNK, n_ids - at);
+        rc = prefill_chunk(ids.data() + at, n, h_logits ? h_logits + (size_t)at * cfg_.vocab_size : nullptr);
+        if (rc != HM_OK) return rc;
+    }
+    return hm_sync(ctx_);
+}
+
+int HfModel::prefill_chunk(const int32_t *h_ids, int n, float *h_logits) {
+    const TransformerConfig &c = cfg_;
+    const int hidden = c.hidden_size, inter = c.intermediate_size, vocab = c.vocab_size;
+    const int H = c.num_attention_heads, kvh = c.kv_heads(), hd = c.head_dim();
+    const int qd = c.q_dim(), kvd = c.kv_dim(), nqkv = qd + 2 * kvd;
+    const float eps = (float)c.rms_norm_eps;
+    PrefillScratch &p = pf_;
+    if (p.rows < n) {
+        const int rows = std::max(n, 128);
+        const int64_t widest = std::max<int64_t>(std::max(hidden, qd), inter);
+        hm_sync(ctx_);
+        p = PrefillScratch();
+        p.ids = Buffer::alloc(ctx_, {rows}, DType::F32);  // int32 ids
+        p.h = Buffer::alloc(ctx_, {rows, hidden}, DType::F32);
+        p.resid = Buffer::alloc(ctx_, {rows, hidden}, DType::F32);
+        p.split = Buffer::alloc(ctx_, {rows, 3 * widest}, DType::BF16);
+        p.qkv = Buffer::alloc(ctx_, {PrefillScratch::MAX_PARTS, rows, nqkv}, DType::F32);
+        p.proj_out = Buffer::alloc(ctx_, {PrefillScratch::MAX_PARTS, rows, hidden}, DType::F32);
+        p.gate_up = Buffer::alloc(ctx_, {PrefillScratch::MAX_PARTS, rows, 2 * (int64_t)inter}, DType::F32);
+        if (!p.ids || !p.h || !p.resid || !p.split || !p.qkv || !p.proj_out || !p.gate_up) return HM_ERR_OOM;
+        p.rows = rows;
+    }
+    if (h_logits && !p.logits) {
+        p.logits = Buffer::alloc(ctx_, {p.rows, vocab}, DType::F32);
+        if (!p.logits) return HM_ERR_OOM;
+    }
+    KvCache *kv = plan_->kv_cache();
+    const int past = kv->current_len();
+    int rc = hm_upload(ctx_, p.ids.ptr(), h_ids, (size_t)n * 4);
+    if (rc != HM_OK) return rc;
+    float *h = p.h.as<float>(), *resid = p.resid.as<float>(), *qkv = p.qkv.as<float>();
+    float *proj_out = p.proj_out.as<float>(), *gate_up = p.gate_up.as<float>();
+    uint16_t *split = p.split.as<uint16_t>();
+    const int np = prefill_pieces_;
+    const int MP = PrefillScratch::MAX_PARTS;
+    int parts = 1;  // K slices of the latest projection
+    rc = embed_launch(ctx_, nullptr, p.ids.as<int32_t>(), weight_f32("model.embed_tokens.weight"), h, n, vocab, hidden);
+    if (rc != HM_OK) return rc;
+    for (int l = 0; l < c.num_hidden_layers; l++) {
+        const std::string pre = "model.layers." + std::to_string(l) + ".";
+        const LayerPacked &lp = packed_[l];
+        // QKV kernel (reference src/hf/emitter.rs:549-673)
+        rc = rmsnorm_split_launch(ctx_, h, nullptr, 1, weight_f32(pre + "input_layernorm.weight"), split, np, nullptr, n, hidden, eps);
+        if (rc == HM_OK) rc = gemm_split_nk(ctx_, split, np, lp.qkv.as<uint16_t>(), qkv, n, hidden, nqkv, MP, &parts);
+        if (rc != HM_OK) return rc;
+        QkvPostArgs qa;
+        qa.qkv = qkv;
+        qa.parts = parts;
+        qa.part_stride = (size_t)n * nqkv;
+        qa.bias = lp.qkv_bias ? lp.qkv_bias.as<float>() : nullptr;
+        if (has_qk_norm_) {
+            qa.qw = weight_f32(pre + "self_attn.q_norm.weight");
+            qa.kw = weight_f32(pre + "self_attn.k_norm.weight");
+        }
+        qa.cos_tab = rope_cos_.as<float>();
+        qa.sin_tab = rope_sin_.as<float>();
+        qa.kcache = kv->key_ptr(l);
+        qa.vcache = kv->value_ptr(l);
+        qa.S = n;
+        qa.H = H;
+        qa.kvh = kvh;
+        qa.hd = hd;
+        qa.max_len = kv->max_len();
+        qa.past = past;
+        qa.eps = eps;
+        if ((rc = qkv_post_launch(ctx_, qa)) != HM_OK) return rc;
+        // attention kernel (reference src/hf/emitter.rs:683-758): causal attention, then the O projection
+        PrefillAttnArgs aa;
+        aa.q = qkv;
+        aa.ldq = nqkv;
+        aa.kcache = kv->key_ptr(l);
+        aa.vcache = kv->value_ptr(l);
+        aa.out_split = split;
+        aa.S = n;
+        aa.H = H;
+        aa.kvh = kvh;
+        aa.hd = hd;
+        aa.max_len = kv->max_len();
+        aa.past = past;
+        aa.scale = (float)(1.0 / std::sqrt((double)hd));
+        aa.pieces = np;
+        if ((rc = prefill_attn_launch(ctx_, aa)) != HM_OK) return rc;
+        if ((rc = gemm_split_nk(ctx_, split, np, lp.o.as<uint16_t>(), proj_out, n, qd, hidden, MP, &parts)) != HM_OK) return rc;
+        // MLP kernel (reference src/hf/emitter.rs:767-822)
+        rc = rmsnorm_split_launch(ctx_, h, proj_out, parts, weight_f32(pre + "post_attention_layernorm.weight"), split, np,
+                                  resid, n, hidden, eps);
+        if (rc == HM_OK) rc = gemm_split_nk(ctx_, split, np, lp.gate_up.as<uint16_t>(), gate_up, n, hidden, 2 * inter, MP, &parts);
+        if (rc == HM_OK) rc = silu_mul_split_launch(ctx_, gate_up, parts, split, np, n, inter);
+        if (rc == HM_OK) rc = gemm_split_nk(ctx_, split, np, lp.down.as<uint16_t>(), proj_out, n, inter, hidden, MP, &parts);
+        if (rc == HM_OK) rc = add_parts_launch(ctx_, resid, proj_out, parts, h, (size_t)n * hidden);
+        if (rc != HM_OK) return rc;
+    }
+    if (h_logits) {  // LM head (reference src/hf/emitter.rs:828-862) for every row
+        rc = rmsnorm_split_launch(ctx_, h, nullptr, 1, weight_f32("model.norm.weight"), split, np, nullptr, n, hidden, eps);
+        if (rc == HM_OK) rc = gemm_split_nk(ctx_, split, np, lm_head_packed_.as<uint16_t>(), p.logits.as<float>(), n, hidden, vocab);
+        if (rc == HM_OK) rc = hm_download(ctx_, h_logits, p.logits.ptr(), (size_t)n * vocab * 4);
+        if (rc != HM_OK) return rc;
+    }
+    // one advance after all layers appended (reference src/runtime.rs:1875-1880)
+    kv->advance_by(n);
+    return HM_OK;
 }
 
 int HfModel::init_kv_cache(const float *const *h_kv, int seq_len) {
@@ -1127,10 +1265,19 @@ int HfModel::generate_greedy(const int64_t *h_prompt, int n_prompt, int n_new, i
     if (!finalized_) return hm_set_error(ctx_, HM_ERR_STATE, "model not finalized");
     if (n_prompt <= 0 || n_new <= 0 || !h_prompt || !h_tokens)
         return hm_set_error(ctx_, HM_ERR_INVALID, "generate_greedy: bad arguments");
-    const int steps = n_prompt + n_new - 1;
+    int steps = n_prompt + n_new - 1;
     if (kv_cache_len() + steps > max_seq_len_)  // the reference's loop stops at max_seq_len
                                                 // (src/generate.rs:188-194); here it is an error
         return hm_set_error(ctx_, HM_ERR_STATE, "KV cache full (%d + %d > %d)", kv_cache_len(), steps, max_seq_len_);
+    if (prefill_min_ > 0 && n_prompt - 1 >= prefill_min_ && prefill_available()) {
+        // reference HfGenerationContext::prefill (src/hf/model.rs:321-336): the prompt in one pass; its
+        // last token goes through the decode step, whose pick is generated token 0
+        int rc = prefill(h_prompt, n_prompt - 1, nullptr);
+        if (rc != HM_OK) return rc;
+        h_prompt += n_prompt - 1;
+        n_prompt = 1;
+        steps = n_new;
+    }
     if (steps > plan_->out_capacity())
         return hm_set_error(ctx_, HM_ERR_INVALID, "generate_greedy: %d steps exceed capacity %d", steps, plan_->out_capacity());
     std::vector<int32_t> ids;

@@ -1,0 +1,518 @@
+// Multi-token (prefill) kernels: row-wise ops that hand f32 activations to the MFMA GEMM as split
+// bf16 matrices, the tail of the QKV kernel for a block of positions, and a causal GQA attention
+// on the matrix cores.
+//
+// Attention works on the transposed problem so that softmax statistics stay inside a lane:
+//   S^T[key][q] = K[key][:] . Q[q][:]      (A operand = K rows from LDS, B operand = Q in registers)
+//   O^T[d][q]   = V^T[d][:] . P^T[:][q]    (A operand = V^T rows from LDS, B operand = P in registers)
+// With v_mfma_f32_32x32x16_bf16 a lane owns one query column of the result tile (lane % 32) and
+// 16 of its 32 rows, so the running maximum and the rescaling factor of a query are per-lane
+// scalars; only one exchange with lane ^ 32 per key tile is needed. The probabilities leave the
+// S^T accumulators and enter the second product without touching LDS: MFMA row r of a key block
+// is assigned key (r with bits 2 and 3 swapped), which makes the 8 accumulator values a lane
+// passes per k step 8 consecutive keys, matching one 16-byte chunk of a V^T row.
+// Queries and probabilities are f32 carried as two or three bf16 pieces each (see prefill.h); K and
+// V are the cache's own bf16 rows.
+#include "prefill.h"
+
+#include "gemm_bf16_mfma.h"
+
+namespace {
+
+using namespace homura;
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+// x = p[0] + p[1] + ... : each piece is the bf16 rounding (nearest-even, the hardware conversion) of
+// what the earlier ones left over; the subtraction is exact. Three pieces reproduce every finite f32
+// whose last bit is above the bf16 underflow range. Straight-line code: an infinity or NaN turns the
+// later pieces into NaN, like the product with it would be anyway.
+template <int NP>
+__device__ __forceinline__ void split_pieces(float x, uint32_t (&p)[NP]) {
+    float r = x;
+#pragma unroll
+    for (int i = 0; i < NP; i++) {
+        const __bf16 b = (__bf16)r;
+        p[i] = (uint32_t)__builtin_bit_cast(uint16_t, b);
+        r = r - (float)b;
+    }
+}
+
+// 8 floats -> NP MFMA operands
+template <int NP>
+__device__ __forceinline__ void split8(const float *f, bf16x8 (&out)[NP]) {
+    u32x4 w[NP];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        uint32_t a[NP], b[NP];
+        split_pieces<NP>(f[2 * j], a);
+        split_pieces<NP>(f[2 * j + 1], b);
+#pragma unroll
+        for (int p = 0; p < NP; p++) w[p][j] = a[p] | (b[p] << 16);
+    }
+#pragma unroll
+    for (int p = 0; p < NP; p++) out[p] = __builtin_bit_cast(bf16x8, w[p]);
+}
+
+// element c of a split row: piece p goes to column p * dim + c
+__device__ __forceinline__ void split_store(uint16_t *__restrict__ row, int dim, int c, float x, int pieces) {
+    uint32_t p[3];
+    split_pieces<3>(x, p);
+    row[c] = (uint16_t)p[0];
+    if (pieces > 1) row[dim + c] = (uint16_t)p[1];
+    if (pieces > 2) row[2 * dim + c] = (uint16_t)p[2];
+}
+
+__global__ void split_rows_kernel(const float *__restrict__ x, uint16_t *__restrict__ out, int dim, size_t n,
+                                  int pieces) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const size_t row = i / dim;
+    split_store(out + row * pieces * dim, dim, (int)(i % dim), x[i], pieces);
+}
+
+// One workgroup per row, the arithmetic of the decode path's RMSNorm kernel (reference
+// src/graph_builder/emit_linalg.rs:7-26; Residual+Norm, src/hf/emitter.rs:787-790).
+// A GEMM result that was cut along K: the slices added in index order
+__device__ __forceinline__ float sum_parts(const float *__restrict__ p, size_t i, int parts, size_t stride) {
+    float v = p[i];
+    for (int s = 1; s < parts; s++) v += p[i + s * stride];
+    return v;
+}
+
+__global__ __launch_bounds__(256) void rmsnorm_split_kernel(const float *__restrict__ x, const float *__restrict__ res,
+                                                            int res_parts, size_t res_stride,
+                                                            const float *__restrict__ w, uint16_t *__restrict__ out,
+                                                            float *__restrict__ resid_out, int dim, float eps,
+                                                            int pieces) {
+    __shared__ float red[4];
+    const size_t base = (size_t)blockIdx.x * dim;
+    float ss = 0.f;
+    float keep[4];  // dim <= 1024 keeps its row in registers; wider rows recompute below
+    int kept = 0;
+    for (int i = threadIdx.x; i < dim; i += 256) {
+        float v = x[base + i];
+        if (res) v = v + sum_parts(res, base + i, res_parts, res_stride);
+        if (resid_out) resid_out[base + i] = v;
+        if (kept < 4) keep[kept] = v;
+        kept++;
+        ss += v * v;
+    }
+    ss = wave_sum(ss);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = ss;
+    __syncthreads();
+    const float tot = (red[0] + red[1]) + (red[2] + red[3]);
+    const float inv = 1.0f / sqrtf(tot / (float)dim + eps);
+    uint16_t *o = out + (size_t)blockIdx.x * pieces * dim;
+    int at = 0;
+    for (int i = threadIdx.x; i < dim; i += 256, at++) {
+        float v;
+        if (at < 4) {
+            v = keep[at];
+        } else {
+            v = x[base + i];
+            if (res) v = v + sum_parts(res, base + i, res_parts, res_stride);
+        }
+        split_store(o, dim, i, (v * inv) * w[i], pieces);
+    }
+}
+
+// silu(gate) * up (reference src/graph_builder/emit_arithmetic.rs:101-107, src/hf/emitter.rs:797-799)
+__global__ void add_parts_kernel(const float *__restrict__ a, const float *__restrict__ b, int parts, size_t stride,
+                                 float *__restrict__ out, size_t n) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) out[i] = a[i] + sum_parts(b, i, parts, stride);
+}
+
+__global__ void silu_mul_split_kernel(const float *__restrict__ gu, int parts, size_t stride, uint16_t *__restrict__ out,
+                                      int inter, size_t n, int pieces) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const size_t row = i / inter;
+    float2 p = *reinterpret_cast<const float2 *>(gu + 2 * i);
+    for (int s = 1; s < parts; s++) {
+        const float2 q = *reinterpret_cast<const float2 *>(gu + s * stride + 2 * i);
+        p.x += q.x;
+        p.y += q.y;
+    }
+    split_store(out + row * pieces * inter, inter, (int)(i % inter), (p.x / (1.0f + expf(-p.x))) * p.y, pieces);
+}
+
+// One wavefront per (position, head) row of q, k or v.
+__global__ __launch_bounds__(256) void qkv_post_kernel(QkvPostArgs a) {
+    const int lane = threadIdx.x & 63;
+    const int per_pos = a.H + 2 * a.kvh;
+    const int r = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (r >= a.S * per_pos) return;
+    const int s = r / per_pos, j = r % per_pos;
+    const int hd = a.hd, half = hd / 2;
+    const int pos = a.past + s;
+    float *x = a.qkv + (size_t)s * per_pos * hd + (size_t)j * hd;
+    const float *b = a.bias ? a.bias + (size_t)j * hd : nullptr;
+    // element i of the row: the K slices of the projection added up, then the bias
+    auto elem = [&](int i) {
+        const float v = sum_parts(x, (size_t)i, a.parts, a.part_stride);
+        return b ? v + b[i] : v;
+    };
+
+    if (j >= a.H + a.kvh) {  // a v row: bias, then the cache append
+        uint16_t *dst = a.vcache + ((size_t)(j - a.H - a.kvh) * a.max_len + pos) * hd;
+        for (int i = lane; i < hd; i += 64) dst[i] = f32_to_bf16_rne_dev(elem(i));
+        return;
+    }
+    const bool is_q = j < a.H;
+    const float *nw = is_q ? a.qw : a.kw;
+    const float *c = a.cos_tab + (size_t)pos * hd;
+    const float *sn = a.sin_tab + (size_t)pos * hd;
+    float lo[2], hi[2];  // hd <= 256
+    float ss = 0.f;
+#pragma unroll
+    for (int t = 0; t < 2; t++) {
+        const int i = lane + 64 * t;
+        lo[t] = i < half ? elem(i) : 0.f;
+        hi[t] = i < half ? elem(i + half) : 0.f;
+        ss += lo[t] * lo[t] + hi[t] * hi[t];
+    }
+    if (nw) {
+        ss = wave_sum(ss);
+        const float inv = 1.0f / sqrtf(ss / (float)hd + a.eps);
+#pragma unroll
+        for (int t = 0; t < 2; t++) {
+            const int i = lane + 64 * t;
+            if (i < half) {
+                lo[t] = (lo[t] * inv) * nw[i];
+                hi[t] = (hi[t] * inv) * nw[i + half];
+            }
+        }
+    }
+    uint16_t *kdst = is_q ? nullptr : a.kcache + ((size_t)(j - a.H) * a.max_len + pos) * hd;
+#pragma unroll
+    for (int t = 0; t < 2; t++) {
+        const int i = lane + 64 * t;
+        if (i < half) {
+            const float o_lo = lo[t] * c[i] + (-hi[t]) * sn[i];
+            const float o_hi = hi[t] * c[i + half] + lo[t] * sn[i + half];
+            if (is_q) {
+                x[i] = o_lo;
+                x[i + half] = o_hi;
+            } else {
+                kdst[i] = f32_to_bf16_rne_dev(o_lo);
+                kdst[i + half] = f32_to_bf16_rne_dev(o_hi);
+            }
+        }
+    }
+}
+
+// ── causal attention ─────────────────────────────────────────────────────────
+
+constexpr int AT_THREADS = 256;
+constexpr int AT_QROWS = 128;  // query rows per workgroup: 4 wavefronts x 32
+constexpr int AT_KEYS = 64;    // keys per tile
+
+// V^T tile: row d holds 64 keys = 128 bytes = eight 16-byte chunks, chunk c of row r at slot
+// c ^ (r & 7) ^ ((r >> 3) & 7): conflict-free for the operand reads (32 consecutive rows, one chunk)
+// and spread for the transposing 8-byte writes.
+__device__ __forceinline__ int vt_off(int r, int chunk) {
+    return r * 128 + ((chunk ^ (r & 7) ^ ((r >> 3) & 7)) << 4);
+}
+// K tile: row = key, HD*2 bytes, same idea
+template <int HD>
+__device__ __forceinline__ int k_off(int key, int chunk) {
+    if (HD == 128) return key * 256 + ((chunk ^ (key & 15)) << 4);
+    return key * 128 + ((chunk ^ (key & 7) ^ ((key >> 3) & 7)) << 4);
+}
+
+template <int HD, int NP>
+__global__ __launch_bounds__(AT_THREADS) void prefill_attn_kernel(PrefillAttnArgs a) {
+    constexpr int CH = HD / 8;                        // 16-byte chunks per K row
+    constexpr int KLOADS = AT_KEYS * CH / AT_THREADS;  // K chunks per thread per tile
+    constexpr int KSTEPS = HD / 16;                   // k steps of K . Q
+    constexpr int DB = HD / 32;                       // 32-row blocks of O^T
+    __shared__ __attribute__((aligned(16))) char k_lds[AT_KEYS * HD * 2];
+    __shared__ __attribute__((aligned(16))) char v_lds[HD * 128];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, lh = lane >> 5;
+    const int h = blockIdx.y, kvhd = h / (a.H / a.kvh);
+    const int q0 = blockIdx.x * AT_QROWS;
+    const int kv_total = a.past + a.S;
+    const uint16_t *kc = a.kcache + (size_t)kvhd * a.max_len * HD;
+    const uint16_t *vc = a.vcache + (size_t)kvhd * a.max_len * HD;
+
+    // this lane's query (rows past the end repeat the last one and are not stored)
+    const int qrow = q0 + wave * 32 + l32;
+    const int qc = min(qrow, a.S - 1);
+    const int qabs = a.past + qc;
+    bf16x8 qp_[KSTEPS][NP];
+    {
+        const float *qp = a.q + (size_t)qc * a.ldq + (size_t)h * HD + lh * 8;
+#pragma unroll
+        for (int ks = 0; ks < KSTEPS; ks++) {
+            const f32x4 x0 = *reinterpret_cast<const f32x4 *>(qp + 16 * ks);
+            const f32x4 x1 = *reinterpret_cast<const f32x4 *>(qp + 16 * ks + 4);
+            float f[8];
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                f[i] = x0[i] * a.scale;
+                f[4 + i] = x1[i] * a.scale;
+            }
+            split8<NP>(f, qp_[ks]);
+        }
+    }
+
+    // keys [0, wg_end) are visible to some row of the workgroup, [0, wave_end) to some row of this wavefront
+    const int wg_end = a.past + min(a.S, q0 + AT_QROWS);
+    const int wave_end = q0 + wave * 32 < a.S ? a.past + min(a.S, q0 + wave * 32 + 32) : 0;
+    const int ntiles = (wg_end + AT_KEYS - 1) / AT_KEYS;
+
+    // thread's share of a tile on its way from the cache to LDS
+    u32x4 kr[KLOADS], vr[4];
+    const int v_ng = tid % CH, v_kg = tid / CH;  // V: a 4(key) x 8(d) block per thread
+    const bool v_on = v_kg < 16;
+    auto request_tile = [&](int t) {
+#pragma unroll
+        for (int j = 0; j < KLOADS; j++) {
+            const int id = tid + j * AT_THREADS, key = id / CH, c = id % CH;
+            const int row = min(t * AT_KEYS + key, kv_total - 1);
+            kr[j] = ld128(kc + (size_t)row * HD + c * 8);
+        }
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const int row = min(t * AT_KEYS + (v_on ? v_kg : 0) * 4 + r, kv_total - 1);
+            vr[r] = ld128(vc + (size_t)row * HD + v_ng * 8);
+        }
+    };
+    auto store_tile = [&]() {
+#pragma unroll
+        for (int j = 0; j < KLOADS; j++) {
+            const int id = tid + j * AT_THREADS, key = id / CH, c = id % CH;
+            *reinterpret_cast<u32x4 *>(k_lds + k_off<HD>(key, c)) = kr[j];
+        }
+        if (v_on) {
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                // column d = v_ng*8 + i of the block: keys +0..+3 packed low to high
+                const uint32_t sel = (i & 1) ? 0x07060302u : 0x05040100u;
+                u32x2 col;
+                col.x = __builtin_amdgcn_perm(vr[1][i >> 1], vr[0][i >> 1], sel);
+                col.y = __builtin_amdgcn_perm(vr[3][i >> 1], vr[2][i >> 1], sel);
+                *reinterpret_cast<u32x2 *>(v_lds + vt_off(v_ng * 8 + i, v_kg >> 1) + (v_kg & 1) * 8) = col;
+            }
+        }
+    };
+
+    f32x16 acc_o[DB];
+#pragma unroll
+    for (int db = 0; db < DB; db++)
+#pragma unroll
+        for (int v = 0; v < 16; v++) acc_o[db][v] = 0.f;
+    float m_run = -INFINITY, l_run = 0.f;
+    // MFMA row r of a key block holds key pi(r) = r with bits 2 and 3 swapped
+    const int pi = (l32 & 0x13) | ((l32 & 4) << 1) | ((l32 & 8) >> 1);
+
+    request_tile(0);
+    for (int t = 0; t < ntiles; t++) {
+        __syncthreads();  // the previous tile has been read by everybody
+        store_tile();
+        __syncthreads();
+        if (t + 1 < ntiles) request_tile(t + 1);
+        if (t * AT_KEYS >= wave_end) continue;  // wavefront-uniform: nothing visible to these 32 rows
+
+        f32x16 s[2];
+#pragma unroll
+        for (int kb = 0; kb < 2; kb++) {
+#pragma unroll
+            for (int v = 0; v < 16; v++) s[kb][v] = 0.f;
+            const int krow = 32 * kb + pi;
+#pragma unroll
+            for (int ks = 0; ks < KSTEPS; ks++) {
+                const bf16x8 kf = *reinterpret_cast<const bf16x8 *>(k_lds + k_off<HD>(krow, 2 * ks + lh));
+#pragma unroll
+                for (int p = 0; p < NP; p++)
+                    s[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qp_[ks][p], s[kb], 0, 0, 0);
+            }
+        }
+        // accumulator value v of block kb belongs to key 32 kb + 16 (v / 8) + 8 (lane / 32) + v % 8
+        float mx = -INFINITY;
+#pragma unroll
+        for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                const int key = t * AT_KEYS + 32 * kb + 16 * (v >> 3) + 8 * lh + (v & 7);
+                const float x = key > qabs ? -INFINITY : s[kb][v];
+                s[kb][v] = x;
+                mx = fmaxf(mx, x);
+            }
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        const float m_new = fmaxf(m_run, mx);  // finite: key 0 is visible to every row
+        const float alpha = expf(m_run - m_new);
+        float psum = 0.f;
+#pragma unroll
+        for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                const float p = expf(s[kb][v] - m_new);
+                s[kb][v] = p;
+                psum += p;
+            }
+        l_run = l_run * alpha + psum;  // this lane's half of the keys; the halves meet at the end
+        m_run = m_new;
+#pragma unroll
+        for (int db = 0; db < DB; db++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) acc_o[db][v] *= alpha;
+
+        bf16x8 pp[4][NP];
+#pragma unroll
+        for (int sp = 0; sp < 4; sp++) {
+            float f[8];
+#pragma unroll
+            for (int i = 0; i < 8; i++) f[i] = s[sp >> 1][8 * (sp & 1) + i];
+            split8<NP>(f, pp[sp]);
+        }
+#pragma unroll
+        for (int db = 0; db < DB; db++)
+#pragma unroll
+            for (int sp = 0; sp < 4; sp++) {
+                const bf16x8 vf = *reinterpret_cast<const bf16x8 *>(v_lds + vt_off(32 * db + l32, 2 * sp + lh));
+#pragma unroll
+                for (int p = 0; p < NP; p++)
+                    acc_o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pp[sp][p], acc_o[db], 0, 0, 0);
+            }
+    }
+
+    const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
+    if (qrow >= a.S) return;
+    const float inv = 1.0f / l_tot;
+    const int qd = a.H * HD;
+    // accumulator value v of block db is d = 32 db + 8 (v / 4) + 4 (lane / 32) + v % 4
+#pragma unroll
+    for (int db = 0; db < DB; db++)
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+            const int d0 = h * HD + 32 * db + 8 * g + 4 * lh;
+            f32x4 o;
+#pragma unroll
+            for (int i = 0; i < 4; i++) o[i] = acc_o[db][4 * g + i] * inv;
+            if (a.out_f32) *reinterpret_cast<f32x4 *>(a.out_f32 + (size_t)qrow * qd + d0) = o;
+            if (a.out_split) {
+                uint32_t pc[4][NP];
+#pragma unroll
+                for (int i = 0; i < 4; i++) split_pieces<NP>(o[i], pc[i]);
+                uint16_t *o16 = a.out_split + (size_t)qrow * NP * qd + d0;
+#pragma unroll
+                for (int p = 0; p < NP; p++) {
+                    u32x2 w;
+                    w.x = pc[0][p] | (pc[1][p] << 16);
+                    w.y = pc[2][p] | (pc[3][p] << 16);
+                    *reinterpret_cast<u32x2 *>(o16 + (size_t)p * qd) = w;
+                }
+            }
+        }
+}
+
+}  // namespace
+
+namespace homura {
+
+int rmsnorm_split_launch(hm_ctx *ctx, const float *d_x, const float *d_res, int res_parts, const float *d_w,
+                         uint16_t *d_out_split, int pieces, float *d_resid_out, int rows, int dim, float eps) {
+    HM_REQUIRE(ctx, d_x && d_w && d_out_split, "rmsnorm_split: NULL pointer");
+    HM_REQUIRE(ctx, rows > 0 && dim > 0 && pieces >= 1 && pieces <= 3 && res_parts >= 1, "rmsnorm_split: bad shape");
+    hipLaunchKernelGGL(rmsnorm_split_kernel, dim3(rows), dim3(256), 0, ctx->stream, d_x, d_res, res_parts,
+                       (size_t)rows * dim, d_w, d_out_split, d_resid_out, dim, eps, pieces);
+    HM_LAUNCH_CHECK(ctx);
+    return HM_OK;
+}
+
+int add_parts_launch(hm_ctx *ctx, const float *d_a, const float *d_b, int parts, float *d_out, size_t n) {
+    HM_REQUIRE(ctx, d_a && d_b && d_out && parts >= 1, "add_parts: bad arguments");
+    if (n == 0) return HM_OK;
+    hipLaunchKernelGGL(add_parts_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, ctx->stream, d_a, d_b, parts, n,
+                       d_out, n);
+    HM_LAUNCH_CHECK(ctx);
+    return HM_OK;
+}
+
+int silu_mul_split_launch(hm_ctx *ctx, const float *d_gu, int parts, uint16_t *d_out_split, int pieces, int rows,
+                          int inter) {
+    HM_REQUIRE(ctx, d_gu && d_out_split, "silu_mul_split: NULL pointer");
+    HM_REQUIRE(ctx, rows > 0 && inter > 0 && pieces >= 1 && pieces <= 3 && parts >= 1, "silu_mul_split: bad shape");
+    HM_REQUIRE(ctx, ((uintptr_t)d_gu % 8) == 0, "silu_mul_split: input must be 8-byte aligned");
+    const size_t n = (size_t)rows * inter;
+    hipLaunchKernelGGL(silu_mul_split_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, ctx->stream, d_gu, parts,
+                       2 * n, d_out_split, inter, n, pieces);
+    HM_LAUNCH_CHECK(ctx);
+    return HM_OK;
+}
+
+int qkv_post_launch(hm_ctx *ctx, const QkvPostArgs &a) {
+    HM_REQUIRE(ctx, a.qkv && a.cos_tab && a.sin_tab && a.kcache && a.vcache, "qkv_post: NULL pointer");
+    HM_REQUIRE(ctx, a.S > 0 && a.H > 0 && a.kvh > 0 && a.past >= 0 && a.parts >= 1, "qkv_post: bad shape");
+    HM_REQUIRE(ctx, a.hd >= 2 && a.hd <= 256 && a.hd % 2 == 0, "qkv_post: head_dim %d not supported", a.hd);
+    HM_REQUIRE(ctx, (a.qw == nullptr) == (a.kw == nullptr), "qkv_post: q and k norm weights must come together");
+    if (a.past + a.S > a.max_len)
+        return hm_set_error(ctx, HM_ERR_STATE, "KV cache full (%d + %d > %d)", a.past, a.S, a.max_len);
+    const long long rows = (long long)a.S * (a.H + 2 * a.kvh);
+    hipLaunchKernelGGL(qkv_post_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, ctx->stream, a);
+    HM_LAUNCH_CHECK(ctx);
+    return HM_OK;
+}
+
+int prefill_attn_launch(hm_ctx *ctx, const PrefillAttnArgs &a) {
+    HM_REQUIRE(ctx, a.q && a.kcache && a.vcache && (a.out_f32 || a.out_split), "prefill_attn: NULL pointer");
+    HM_REQUIRE(ctx, a.S > 0 && a.H > 0 && a.kvh > 0 && a.H % a.kvh == 0 && a.past >= 0, "prefill_attn: bad shape");
+    HM_REQUIRE(ctx, a.hd == 64 || a.hd == 128, "prefill_attn: head_dim %d not supported (64 or 128)", a.hd);
+    HM_REQUIRE(ctx, a.past + a.S <= a.max_len, "prefill_attn: %d + %d rows exceed the cache (%d)", a.past, a.S, a.max_len);
+    HM_REQUIRE(ctx, a.ldq >= a.H * a.hd && a.ldq % 4 == 0 && ((uintptr_t)a.q % 16) == 0, "prefill_attn: q rows must be 16-byte aligned");
+    HM_REQUIRE(ctx, ((uintptr_t)a.kcache % 16) == 0 && ((uintptr_t)a.vcache % 16) == 0, "prefill_attn: caches must be 16-byte aligned");
+    HM_REQUIRE(ctx, (!a.out_f32 || ((uintptr_t)a.out_f32 % 16) == 0) && (!a.out_split || ((uintptr_t)a.out_split % 8) == 0),
+               "prefill_attn: misaligned output");
+    HM_REQUIRE(ctx, a.pieces == 2 || a.pieces == 3, "prefill_attn: %d pieces (2 or 3)", a.pieces);
+    const dim3 grid((unsigned)((a.S + AT_QROWS - 1) / AT_QROWS), (unsigned)a.H);
+    if (a.hd == 128 && a.pieces == 3)
+        hipLaunchKernelGGL((prefill_attn_kernel<128, 3>), grid, dim3(AT_THREADS), 0, ctx->stream, a);
+    else if (a.hd == 128)
+        hipLaunchKernelGGL((prefill_attn_kernel<128, 2>), grid, dim3(AT_THREADS), 0, ctx->stream, a);
+    else if (a.pieces == 3)
+        hipLaunchKernelGGL((prefill_attn_kernel<64, 3>), grid, dim3(AT_THREADS), 0, ctx->stream, a);
+    else
+        hipLaunchKernelGGL((prefill_attn_kernel<64, 2>), grid, dim3(AT_THREADS), 0, ctx->stream, a);
+    HM_LAUNCH_CHECK(ctx);
+    return HM_OK;
+}
+
+}  // namespace homura
+
+extern "C" int hm_gemm_f32_bf16_nk(hm_ctx *ctx, const float *d_x_mk, const uint16_t *d_w_nk, float *d_out, int M, int K,
+                                   int N) {
+    HM_CHECK_CTX(ctx);
+    HM_REQUIRE(ctx, d_x_mk && d_w_nk && d_out, "hm_gemm_f32_bf16_nk: NULL pointer");
+    HM_REQUIRE(ctx, M > 0 && N > 0 && K > 0 && K % 32 == 0, "hm_gemm_f32_bf16_nk: need M, N > 0 and K %% 32 == 0");
+    const size_t n = (size_t)M * K;
+    HM_REQUIRE(ctx, n * 6 <= ctx->workspace_bytes, "hm_gemm_f32_bf16_nk: M * K = %zu activations exceed the workspace", n);
+    uint16_t *split = (uint16_t *)ctx->workspace;
+    hipLaunchKernelGGL(split_rows_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, ctx->stream, d_x_mk, split, K, n,
+                       3);
+    HM_LAUNCH_CHECK(ctx);
+    return homura::gemm_split_nk(ctx, split, 3, d_w_nk, d_out, M, K, N);
+}
+
+extern "C" int hm_gqa_prefill_attn(hm_ctx *ctx, const float *d_q, const uint16_t *d_kcache, const uint16_t *d_vcache,
+                                   float *d_out, int S, int H, int kvh, int hd, int max_len, int past, float scale) {
+    HM_CHECK_CTX(ctx);
+    homura::PrefillAttnArgs a;
+    a.q = d_q;
+    a.ldq = H * hd;
+    a.kcache = d_kcache;
+    a.vcache = d_vcache;
+    a.out_f32 = d_out;
+    a.S = S;
+    a.H = H;
+    a.kvh = kvh;
+    a.hd = hd;
+    a.max_len = max_len;
+    a.past = past;
+    a.scale = scale;
+    return homura::prefill_attn_launch(ctx, a);
+}

@@ -181,6 +181,13 @@ class Context:
     def gemm_bf16_nk(self, a, b_nk, c, M, K, N):
         self._check(self.lib.hm_gemm_bf16_nk(self.h, a.ptr, b_nk.ptr, c.ptr, M, K, N))
 
+    def gemm_f32_bf16_nk(self, x, w_nk, out, M, K, N):
+        self._check(self.lib.hm_gemm_f32_bf16_nk(self.h, x.ptr, w_nk.ptr, out.ptr, M, K, N))
+
+    def gqa_prefill_attn(self, q, kc, vc, out, S, H, kvh, hd, max_len, past, scale):
+        self._check(self.lib.hm_gqa_prefill_attn(self.h, q.ptr, kc.ptr, vc.ptr, out.ptr, S, H, kvh, hd,
+                                                 max_len, past, scale))
+
     def kv_append(self, kc, vc, k, v, B, kvh, hd, max_len, pos, n_new):
         self._check(self.lib.hm_kv_append(self.h, kc.ptr, vc.ptr, k.ptr, v.ptr, B, kvh, hd,
                                           max_len, pos, n_new))
@@ -349,6 +356,23 @@ class HfModel:
             self.h, ids.ctypes.data_as(C.POINTER(C.c_int64)), len(ids),
             logits.ctypes.data_as(_ffi.c_f32_p) if want_logits else None))
         return logits
+
+    def prefill(self, input_ids, want_logits: bool = True):
+        """The multi-token pass (reference HfGenerationContext::prefill, src/hf/model.rs:321-336)."""
+        ids = np.ascontiguousarray(input_ids, dtype=np.int64).reshape(-1)
+        logits = np.empty((len(ids), self.config.vocab_size), dtype=np.float32) if want_logits else None
+        self._check(self.lib.hm_model_prefill(
+            self.h, ids.ctypes.data_as(C.POINTER(C.c_int64)), len(ids),
+            logits.ctypes.data_as(_ffi.c_f32_p) if want_logits else None))
+        return logits
+
+    def set_prefill_min(self, n_tokens: int):
+        """Inputs of at least n_tokens take the prefill pass in run_kv / generate_greedy (0 = never)."""
+        self._check(self.lib.hm_model_set_prefill_min(self.h, n_tokens))
+
+    def set_prefill_pieces(self, pieces: int):
+        """bf16 numbers per f32 activation in the prefill pass: 3 (default, exact) or 2."""
+        self._check(self.lib.hm_model_set_prefill_pieces(self.h, pieces))
 
     def generate_greedy(self, prompt_ids, n_new: int) -> np.ndarray:
         ids = np.ascontiguousarray(prompt_ids, dtype=np.int64).reshape(-1)

@@ -124,13 +124,23 @@ int hm_dequant_q6_k(hm_ctx *ctx, const uint8_t *d_blocks, float *d_out, size_t n
 
 /* Prefill-chunk GEMM on the matrix cores: the reference runs the same emit_matmul with
  * seq > 1 (docs/kv-cache.md:31-37); here A bf16 [M,K], B bf16 [K,N] (reference layout),
- * C f32 [M,N], f32 accumulate. M % 128 == 0, N % 128 == 0, K % 32 == 0. */
+ * C f32 [M,N], f32 accumulate. K % 32 == 0, N % 8 == 0; any M (tiles are 128 x 128, partial
+ * tiles at the edges cost a whole one). */
 int hm_gemm_bf16(hm_ctx *ctx, const uint16_t *d_a_mk, const uint16_t *d_b_kn, float *d_c, int M,
                  int K, int N);
 /* Same product with B in the stream layout [N,K] (what hm_pack_bf16_kn_to_nk writes and the
- * decode GEMVs read), so prefill and decode share one copy of a weight. Same constraints. */
+ * decode GEMVs read), so prefill and decode share one copy of a weight. K % 32 == 0, any M and N. */
 int hm_gemm_bf16_nk(hm_ctx *ctx, const uint16_t *d_a_mk, const uint16_t *d_b_nk, float *d_c, int M,
                     int K, int N);
+
+/* The reference's mixed matmul at seq > 1 (make_mixed_matmul_region,
+ * src/graph_builder/emit_linalg.rs:2224-2307): x f32 [M,K] times W bf16 in the stream layout [N,K],
+ * out f32 [M,N]. Each activation enters the bf16 MFMA as three bf16 numbers (its bf16 rounding, the
+ * rounding of what is left, and again), which together hold all 24 significant bits, so the
+ * products are those of the f32 value. K % 32 == 0; M * K * 6 bytes must fit in the context
+ * workspace (64 MiB). */
+int hm_gemm_f32_bf16_nk(hm_ctx *ctx, const float *d_x_mk, const uint16_t *d_w_nk, float *d_out, int M, int K,
+                        int N);
 
 /* ── KV cache + attention ──────────────────────────────────────────────────── */
 
@@ -151,6 +161,16 @@ int hm_kv_append(hm_ctx *ctx, uint16_t *d_kcache, uint16_t *d_vcache, const floa
 int hm_gqa_decode_attn(hm_ctx *ctx, const float *d_q, const uint16_t *d_kcache,
                        const uint16_t *d_vcache, float *d_out, int B, int H, int kvh, int hd,
                        int max_len, int kv_len, float scale);
+
+/* Causal attention of S new query rows at positions past .. past + S - 1 over cache rows
+ * [0, past + S), batch 1: the attention part of emit_attention_kernel (src/hf/emitter.rs:709-737)
+ * under the mask of build_causal_mask (src/hf/precompute.rs:134-161: key j is visible to query i
+ * when j <= past + i). q f32 [S][H][hd], already normed and rotated; the S new K/V rows must be in
+ * the caches [kvh][max_len][hd] bf16 already (hm_kv_append); out f32 [S][H*hd]. hd = 64 or 128.
+ * QK^T and PV run on the matrix cores with q and the probabilities carried as three bf16 numbers
+ * each (all 24 significant bits). */
+int hm_gqa_prefill_attn(hm_ctx *ctx, const float *d_q, const uint16_t *d_kcache, const uint16_t *d_vcache,
+                        float *d_out, int S, int H, int kvh, int hd, int max_len, int past, float scale);
 
 /* ── light ops ─────────────────────────────────────────────────────────────── */
 
@@ -243,6 +263,18 @@ int hm_model_set_graph(hm_model *m, int on);
  * (src/runtime.rs:1580-1892): n_ids new tokens on top of the cache; h_logits receives
  * [n_ids][vocab] f32 (may be NULL to skip the download). Advances the cache by n_ids. */
 int hm_model_run_kv(hm_model *m, const int64_t *h_ids, int n_ids, float *h_logits);
+
+/* The multi-token pass that hm_model_run_kv and hm_model_generate_greedy take for inputs of at
+ * least `prefill_min` tokens (reference HfGenerationContext::prefill, src/hf/model.rs:321-336: the
+ * whole prompt in one run_kv): projections as GEMMs on the matrix cores, causal attention over
+ * cache + chunk, chunks of 512 rows. bf16 models with head_dim 64 or 128; h_logits [n_ids][vocab]
+ * or NULL (then the LM head is skipped). hm_model_set_prefill_min: 0 = always token by token
+ * (default 8). hm_model_set_prefill_pieces: bf16 numbers per f32 activation on the matrix cores,
+ * 3 (default, every bit of the f32) or 2 (16 bits, a third less MFMA work; K/V rows then round
+ * to a neighbouring bf16 now and then). */
+int hm_model_prefill(hm_model *m, const int64_t *h_ids, int n_ids, float *h_logits);
+int hm_model_set_prefill_min(hm_model *m, int n_tokens);
+int hm_model_set_prefill_pieces(hm_model *m, int pieces);
 
 /* The greedy loop of generate_streaming_core (src/generate.rs:187-270) with pure argmax:
  * the prompt is consumed as incremental prefill through run_kv, then n_new tokens are

@@ -212,6 +212,55 @@ def test_gemm_identity_exact(ctx):
     assert np.array_equal(got, synth.bf16_to_f32(b)[(np.arange(M) * 37) % K])
 
 
+@pytest.mark.parametrize("layout", ["kn", "nk"])
+@pytest.mark.parametrize("M,K,N", [(1, 64, 8), (37, 96, 200), (130, 160, 264), (512, 1024, 4096 + 64)])
+def test_gemm_bf16_ragged_edges(ctx, oracle, M, K, N, layout):
+    """M and N that are not multiples of the 128 x 128 tile: edge tiles re-read the last row and
+    must neither store outside C nor disturb the rows inside."""
+    say(f"gemm_bf16 ragged M={M} K={K} N={N} B layout {layout}")
+    a = synth.normal_bf16(11, M * K, 1.0).reshape(M, K)
+    b = synth.normal_bf16(12, K * N, 0.02).reshape(K, N)
+    want = oracle.matmul_bf16_bf16(a, b, M, K, N)
+    guard = 4096
+    host_c = np.full(M * N + guard, -77.0, np.float32)
+    da, dc = ctx.to_device(a), ctx.to_device(host_c)
+    if layout == "kn":
+        db = ctx.to_device(b)
+        ctx.gemm_bf16(da, db, dc, M, K, N)
+    else:
+        db = ctx.to_device(np.ascontiguousarray(b.T))
+        ctx.gemm_bf16_nk(da, db, dc, M, K, N)
+    got = dc.download(np.float32, (M * N + guard,))
+    assert np.all(got[M * N:] == -77.0), "wrote past the end of C"
+    assert rel_err(got[:M * N], want) < TOL
+    for buf in (da, db, dc):
+        buf.free()
+
+
+@pytest.mark.parametrize("M,K,N", [(512, 1024, 4096), (1, 1024, 1024), (77, 448, 576), (300, 3072, 1024)])
+def test_gemm_f32_activations_bf16_weights(ctx, oracle, M, K, N):
+    """The reference's mixed matmul at seq > 1: f32 activations, bf16 weights. The activation goes
+    through the bf16 matrix cores as three bf16 numbers that add up to the f32 exactly. Measured
+    against the float64 product with this file's rel_err (floor 1e-3 of the largest output): the f32
+    oracle sits between 1e-4 and 1e-3 on the outputs closest to zero and the GPU must be in the same
+    range (below 3x the oracle's own error); one bf16 rounding of the activations lands near 1."""
+    say(f"gemm_f32_bf16_nk M={M} K={K} N={N}")
+    x = synth.normal_f32(21, M * K).reshape(M, K)
+    w = synth.normal_bf16(22, K * N, 0.02).reshape(K, N)
+    want = oracle.matmul_f32_bf16(x, w, M, K, N)
+    truth = x.astype(np.float64) @ synth.bf16_to_f32(w).astype(np.float64)
+    dx, dw, dc = ctx.to_device(x), ctx.to_device(np.ascontiguousarray(w.T)), ctx.empty(M * N)
+    ctx.gemm_f32_bf16_nk(dx, dw, dc, M, K, N)
+    got = dc.download(np.float32, (M, N))
+    coarse = synth.bf16_to_f32(synth.f32_to_bf16_rne(x)).astype(np.float64) @ synth.bf16_to_f32(w).astype(np.float64)
+    e_gpu, e_orc, e_bf16 = rel_err(got, truth), rel_err(want, truth), rel_err(coarse, truth)
+    say(f"  vs float64: gpu {e_gpu:.2e}, f32 oracle {e_orc:.2e}, activations rounded to bf16 {e_bf16:.2e}")
+    assert e_gpu < 3 * e_orc and e_gpu < e_bf16 / 100
+    assert rel_err(got, want) < 2e-3
+    for buf in (dx, dw, dc):
+        buf.free()
+
+
 # ── KV cache append + decode attention ────────────────────────────────────────
 
 def test_kv_append_reference_arrays(ctx, golden):
@@ -284,6 +333,56 @@ def test_attention_uniform_keys_give_mean_of_values(ctx):
     mean = synth.bf16_to_f32(vb).astype(np.float64).mean(axis=1)
     for h in range(H):
         assert np.allclose(got[h], mean[h // 2], atol=1e-5)  # heads h0,h0,h1,h1 (floordiv map)
+
+
+@pytest.mark.parametrize("S,H,kvh,hd,max_len,past", [
+    (512, 16, 8, 128, 2048, 0),     # Qwen3-0.6B prompt chunk on an empty cache
+    (200, 16, 8, 128, 2048, 1024),  # incremental prefill on top of 1024 cached rows, ragged S
+    (1, 4, 2, 128, 64, 0),          # a single row
+    (37, 14, 2, 64, 300, 33),       # g = 7, head_dim 64, nothing aligned
+    (129, 4, 4, 64, 512, 64),       # MHA, one row into the second query block
+    (64, 12, 2, 128, 256, 191)])    # g = 6, the last key tile is a single key short of full
+def test_gqa_prefill_attn(ctx, oracle, S, H, kvh, hd, max_len, past):
+    say(f"gqa_prefill_attn S={S} H={H} kvh={kvh} hd={hd} max_len={max_len} past={past}")
+    total = past + S
+    q = synth.normal_f32(31, S * H * hd).reshape(S, H, hd)
+    kb = synth.normal_bf16(32, kvh * max_len * hd).reshape(kvh, max_len, hd)
+    vb = synth.normal_bf16(33, kvh * max_len * hd).reshape(kvh, max_len, hd)
+    # rows past the live range must never be looked at: poison them
+    kb[:, total:] = 0x7FC0
+    vb[:, total:] = 0x7FC0
+    scale = 1.0 / math.sqrt(hd)
+    dq, dk, dv, dout = ctx.to_device(q), ctx.to_device(kb), ctx.to_device(vb), ctx.empty(S * H * hd)
+    ctx.gqa_prefill_attn(dq, dk, dv, dout, S, H, kvh, hd, max_len, past, scale)
+    got = dout.download(np.float32, (S, H * hd))
+    assert np.isfinite(got).all()
+    kf, vf = synth.bf16_to_f32(kb[:, :total]), synth.bf16_to_f32(vb[:, :total])
+    want = oracle.gqa_attention(q, kf, vf, oracle.causal_mask(S, past))
+    err = rel_err(got, want)
+    say(f"  rel err {err:.2e}")
+    assert err < 5e-3   # f32 rounding noise on the outputs nearest zero is ~1e-3 in this metric
+    # the last row attends to everything: it must agree with the decode kernel on the same cache
+    d1 = ctx.empty(H * hd)
+    dq1 = ctx.to_device(q[S - 1])
+    ctx.gqa_decode_attn(dq1, dk, dv, d1, 1, H, kvh, hd, max_len, total, scale)
+    assert rel_err(got[S - 1], d1.download(np.float32, (H * hd,))) < 5e-3
+    for buf in (dq, dk, dv, dout, d1, dq1):
+        buf.free()
+
+
+def test_prefill_attn_first_row_copies_its_value_row(ctx):
+    """Position 0 on an empty cache sees one key: the output is exactly that V row for every head of
+    the group, whatever q is (softmax of a single score is 1)."""
+    S, H, kvh, hd, L = 40, 4, 2, 128, 64
+    q = synth.normal_f32(41, S * H * hd)
+    kb = synth.normal_bf16(42, kvh * L * hd).reshape(kvh, L, hd)
+    vb = synth.normal_bf16(43, kvh * L * hd).reshape(kvh, L, hd)
+    dq, dk, dv, dout = ctx.to_device(q), ctx.to_device(kb), ctx.to_device(vb), ctx.empty(S * H * hd)
+    ctx.gqa_prefill_attn(dq, dk, dv, dout, S, H, kvh, hd, L, 0, 0.1)
+    got = dout.download(np.float32, (S, H, hd))
+    v0 = synth.bf16_to_f32(vb)[:, 0]
+    for h in range(H):
+        assert np.array_equal(got[0, h], v0[h // 2])
 
 
 # ── light ops ─────────────────────────────────────────────────────────────────

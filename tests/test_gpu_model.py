@@ -140,6 +140,7 @@ def test_qwen3_0p6b_decode_token_identical(ctx):
     say(f"logits: rel err {err:.3e}, max abs diff {absd:.3e}, min fixture margin {fx['min_margin']:.3e}")
     assert err < 1e-2
     say("greedy decode on both sides")
+    gm.set_prefill_min(0)   # the prompt token by token through the batch-1 path, as the fixture defines it
     got = gm.generate_greedy(prompt[1:], fx["n_new"])
     want, margins = om.generate_greedy(prompt[1:], fx["n_new"])
     assert np.array_equal(want, np.array(fx["tokens"], np.int32)), "oracle drifted from its committed fixture"
@@ -147,6 +148,10 @@ def test_qwen3_0p6b_decode_token_identical(ctx):
     gm.set_graph(True)
     gm.init_kv_cache(kv, fx["prefill_len"])
     assert np.array_equal(gm.generate_greedy(prompt, fx["n_new"]), want), "graph replay differs"
+    say("prompt through the prefill pass (matrix cores), then decode")
+    gm.set_prefill_min(8)
+    gm.init_kv_cache(kv, fx["prefill_len"])
+    assert np.array_equal(gm.generate_greedy(prompt, fx["n_new"]), want), "prefill + decode differs"
     gm.close()
 
 
