@@ -309,10 +309,11 @@ int gemm_launch(hm_ctx *ctx, const char *who, const uint16_t *a, const uint16_t 
 int homura::gemm_split_nk(hm_ctx *ctx, const uint16_t *d_a_split, int pieces, const uint16_t *d_b_nk, float *d_c,
                           int M, int K, int N, int max_parts, int *parts) {
     HM_REQUIRE(ctx, pieces >= 1 && pieces <= 3, "gemm_split_nk: %d pieces (1..3)", pieces);
-    // K slices until the grid has about two workgroups per compute unit, at least 4 K tiles each
+    // K slices while they still add whole waves of workgroups to a grid smaller than the chip (the
+    // slices cost a write and a read of C each), at least 4 K tiles per slice
     const long long tiles = (long long)((M + TM - 1) / TM) * ((N + TN - 1) / TN);
     const int nk_total = (pieces * K + TK - 1) / TK;
-    int want = (int)((2LL * ctx->num_cus + tiles - 1) / tiles);
+    int want = (int)std::max<long long>(1, ctx->num_cus / tiles);
     want = std::min(std::min(want, max_parts), std::max(1, nk_total / GEMM_DEPTH));
     if (!parts) want = 1;
     return gemm_launch(ctx, "gemm_split_nk", d_a_split, d_b_nk, d_c, M, K, N, true, pieces, want, parts);

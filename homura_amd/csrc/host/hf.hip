@@ -1183,11 +1183,17 @@ int HfModel::prefill_chunk(const int32_t *h_ids, int n, float *h_logits) {
     int parts = 1;  // K slices of the latest projection
     rc = embed_launch(ctx_, nullptr, p.ids.as<int32_t>(), weight_f32("model.embed_tokens.weight"), h, n, vocab, hidden);
     if (rc != HM_OK) return rc;
+    // The hidden state entering a layer is x [+ res]: the embedding for the first layer, afterwards the
+    // post-attention residual plus the K slices of the previous down projection, which the next
+    // RMSNorm kernel adds on its way (the reference's ResAdd, src/hf/emitter.rs:804).
+    const float *x = h, *res = nullptr;
+    int res_parts = 1;
     for (int l = 0; l < c.num_hidden_layers; l++) {
         const std::string pre = "model.layers." + std::to_string(l) + ".";
         const LayerPacked &lp = packed_[l];
         // QKV kernel (reference src/hf/emitter.rs:549-673)
-        rc = rmsnorm_split_launch(ctx_, h, nullptr, 1, weight_f32(pre + "input_layernorm.weight"), split, np, nullptr, n, hidden, eps);
+        rc = rmsnorm_split_launch(ctx_, x, res, res_parts, weight_f32(pre + "input_layernorm.weight"), split, np,
+                                  res ? h : nullptr, n, hidden, eps);
         if (rc == HM_OK) rc = gemm_split_nk(ctx_, split, np, lp.qkv.as<uint16_t>(), qkv, n, hidden, nqkv, MP, &parts);
         if (rc != HM_OK) return rc;
         QkvPostArgs qa;
@@ -1228,17 +1234,19 @@ int HfModel::prefill_chunk(const int32_t *h_ids, int n, float *h_logits) {
         aa.pieces = np;
         if ((rc = prefill_attn_launch(ctx_, aa)) != HM_OK) return rc;
         if ((rc = gemm_split_nk(ctx_, split, np, lp.o.as<uint16_t>(), proj_out, n, qd, hidden, MP, &parts)) != HM_OK) return rc;
-        // MLP kernel (reference src/hf/emitter.rs:767-822)
+        // MLP kernel (reference src/hf/emitter.rs:767-822); h holds the layer's input by now
         rc = rmsnorm_split_launch(ctx_, h, proj_out, parts, weight_f32(pre + "post_attention_layernorm.weight"), split, np,
                                   resid, n, hidden, eps);
         if (rc == HM_OK) rc = gemm_split_nk(ctx_, split, np, lp.gate_up.as<uint16_t>(), gate_up, n, hidden, 2 * inter, MP, &parts);
         if (rc == HM_OK) rc = silu_mul_split_launch(ctx_, gate_up, parts, split, np, n, inter);
         if (rc == HM_OK) rc = gemm_split_nk(ctx_, split, np, lp.down.as<uint16_t>(), proj_out, n, inter, hidden, MP, &parts);
-        if (rc == HM_OK) rc = add_parts_launch(ctx_, resid, proj_out, parts, h, (size_t)n * hidden);
         if (rc != HM_OK) return rc;
+        x = resid;
+        res = proj_out;
+        res_parts = parts;
     }
     if (h_logits) {  // LM head (reference src/hf/emitter.rs:828-862) for every row
-        rc = rmsnorm_split_launch(ctx_, h, nullptr, 1, weight_f32("model.norm.weight"), split, np, nullptr, n, hidden, eps);
+        rc = rmsnorm_split_launch(ctx_, x, res, res_parts, weight_f32("model.norm.weight"), split, np, nullptr, n, hidden, eps);
         if (rc == HM_OK) rc = gemm_split_nk(ctx_, split, np, lm_head_packed_.as<uint16_t>(), p.logits.as<float>(), n, hidden, vocab);
         if (rc == HM_OK) rc = hm_download(ctx_, h_logits, p.logits.ptr(), (size_t)n * vocab * 4);
         if (rc != HM_OK) return rc;

@@ -25,8 +25,6 @@ namespace homura {
 int rmsnorm_split_launch(hm_ctx *ctx, const float *d_x, const float *d_res, int res_parts, const float *d_w,
                          uint16_t *d_out_split, int pieces, float *d_resid_out, int rows, int dim, float eps);
 
-// out = a + b, b in `parts` slices of n floats
-int add_parts_launch(hm_ctx *ctx, const float *d_a, const float *d_b, int parts, float *d_out, size_t n);
 
 // out_split = split(silu(gate) * up) for gate/up interleaved per row: gu [rows][2 * inter] =
 // (gate_0, up_0, gate_1, up_1, ...), the column order of the packed gate|up weight.

@@ -39,17 +39,32 @@ __device__ __forceinline__ void split_pieces(float x, uint32_t (&p)[NP]) {
     }
 }
 
+// Two neighbours at once: the packed hardware conversion yields the MFMA operand word (x0 low, x1 high)
+template <int NP>
+__device__ __forceinline__ void split_pair(float x0, float x1, uint32_t (&w)[NP]) {
+    typedef float f32x2_t __attribute__((ext_vector_type(2)));
+    typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+#pragma unroll
+    for (int i = 0; i < NP; i++) {
+        const f32x2_t r = {x0, x1};
+        w[i] = __builtin_bit_cast(uint32_t, __builtin_convertvector(r, bf16x2_t));
+        if (i + 1 < NP) {
+            x0 = x0 - __uint_as_float(w[i] << 16);
+            x1 = x1 - __uint_as_float(w[i] & 0xFFFF0000u);
+        }
+    }
+}
+
 // 8 floats -> NP MFMA operands
 template <int NP>
 __device__ __forceinline__ void split8(const float *f, bf16x8 (&out)[NP]) {
     u32x4 w[NP];
 #pragma unroll
     for (int j = 0; j < 4; j++) {
-        uint32_t a[NP], b[NP];
-        split_pieces<NP>(f[2 * j], a);
-        split_pieces<NP>(f[2 * j + 1], b);
+        uint32_t pw[NP];
+        split_pair<NP>(f[2 * j], f[2 * j + 1], pw);
 #pragma unroll
-        for (int p = 0; p < NP; p++) w[p][j] = a[p] | (b[p] << 16);
+        for (int p = 0; p < NP; p++) w[p][j] = pw[p];
     }
 #pragma unroll
     for (int p = 0; p < NP; p++) out[p] = __builtin_bit_cast(bf16x8, w[p]);
@@ -72,15 +87,34 @@ __global__ void split_rows_kernel(const float *__restrict__ x, uint16_t *__restr
     split_store(out + row * pieces * dim, dim, (int)(i % dim), x[i], pieces);
 }
 
-// One workgroup per row, the arithmetic of the decode path's RMSNorm kernel (reference
-// src/graph_builder/emit_linalg.rs:7-26; Residual+Norm, src/hf/emitter.rs:787-790).
 // A GEMM result that was cut along K: the slices added in index order
 __device__ __forceinline__ float sum_parts(const float *__restrict__ p, size_t i, int parts, size_t stride) {
     float v = p[i];
     for (int s = 1; s < parts; s++) v += p[i + s * stride];
     return v;
 }
+__device__ __forceinline__ f32x4 sum_parts4(const float *__restrict__ p, size_t i, int parts, size_t stride) {
+    f32x4 v = *reinterpret_cast<const f32x4 *>(p + i);
+    for (int s = 1; s < parts; s++) v += *reinterpret_cast<const f32x4 *>(p + i + s * stride);
+    return v;
+}
 
+// elements c .. c+3 of a split row
+__device__ __forceinline__ void split_store4(uint16_t *__restrict__ row, int dim, int c, f32x4 x, int pieces) {
+    uint32_t lo[3], hi[3];
+    split_pair<3>(x[0], x[1], lo);
+    split_pair<3>(x[2], x[3], hi);
+    for (int k = 0; k < pieces; k++) {
+        u32x2 w;
+        w.x = lo[k];
+        w.y = hi[k];
+        *reinterpret_cast<u32x2 *>(row + (size_t)k * dim + c) = w;
+    }
+}
+
+// One workgroup per row, four consecutive elements per thread and step (dim % 4 == 0); the arithmetic
+// of the decode path's RMSNorm kernel (reference src/graph_builder/emit_linalg.rs:7-26; Residual+Norm,
+// src/hf/emitter.rs:787-790).
 __global__ __launch_bounds__(256) void rmsnorm_split_kernel(const float *__restrict__ x, const float *__restrict__ res,
                                                             int res_parts, size_t res_stride,
                                                             const float *__restrict__ w, uint16_t *__restrict__ out,
@@ -88,16 +122,16 @@ __global__ __launch_bounds__(256) void rmsnorm_split_kernel(const float *__restr
                                                             int pieces) {
     __shared__ float red[4];
     const size_t base = (size_t)blockIdx.x * dim;
+    constexpr int KEEP = 2;  // rows up to 2048 wide stay in registers between the two passes
+    f32x4 keep[KEEP];
     float ss = 0.f;
-    float keep[4];  // dim <= 1024 keeps its row in registers; wider rows recompute below
-    int kept = 0;
-    for (int i = threadIdx.x; i < dim; i += 256) {
-        float v = x[base + i];
-        if (res) v = v + sum_parts(res, base + i, res_parts, res_stride);
-        if (resid_out) resid_out[base + i] = v;
-        if (kept < 4) keep[kept] = v;
-        kept++;
-        ss += v * v;
+    int at = 0;
+    for (int i = threadIdx.x * 4; i < dim; i += 1024, at++) {
+        f32x4 v = *reinterpret_cast<const f32x4 *>(x + base + i);
+        if (res) v += sum_parts4(res, base + i, res_parts, res_stride);
+        if (resid_out) *reinterpret_cast<f32x4 *>(resid_out + base + i) = v;
+        if (at < KEEP) keep[at] = v;
+        ss += (v[0] * v[0] + v[1] * v[1]) + (v[2] * v[2] + v[3] * v[3]);
     }
     ss = wave_sum(ss);
     if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = ss;
@@ -105,38 +139,36 @@ __global__ __launch_bounds__(256) void rmsnorm_split_kernel(const float *__restr
     const float tot = (red[0] + red[1]) + (red[2] + red[3]);
     const float inv = 1.0f / sqrtf(tot / (float)dim + eps);
     uint16_t *o = out + (size_t)blockIdx.x * pieces * dim;
-    int at = 0;
-    for (int i = threadIdx.x; i < dim; i += 256, at++) {
-        float v;
-        if (at < 4) {
+    at = 0;
+    for (int i = threadIdx.x * 4; i < dim; i += 1024, at++) {
+        f32x4 v;
+        if (at < KEEP) {
             v = keep[at];
         } else {
-            v = x[base + i];
-            if (res) v = v + sum_parts(res, base + i, res_parts, res_stride);
+            v = *reinterpret_cast<const f32x4 *>(x + base + i);
+            if (res) v += sum_parts4(res, base + i, res_parts, res_stride);
         }
-        split_store(o, dim, i, (v * inv) * w[i], pieces);
+        const f32x4 wv = *reinterpret_cast<const f32x4 *>(w + i);
+        f32x4 y;
+#pragma unroll
+        for (int k = 0; k < 4; k++) y[k] = (v[k] * inv) * wv[k];
+        split_store4(o, dim, i, y, pieces);
     }
 }
 
-// silu(gate) * up (reference src/graph_builder/emit_arithmetic.rs:101-107, src/hf/emitter.rs:797-799)
-__global__ void add_parts_kernel(const float *__restrict__ a, const float *__restrict__ b, int parts, size_t stride,
-                                 float *__restrict__ out, size_t n) {
-    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < n) out[i] = a[i] + sum_parts(b, i, parts, stride);
-}
-
+// silu(gate) * up (reference src/graph_builder/emit_arithmetic.rs:101-107, src/hf/emitter.rs:797-799);
+// four outputs per thread (inter % 4 == 0)
 __global__ void silu_mul_split_kernel(const float *__restrict__ gu, int parts, size_t stride, uint16_t *__restrict__ out,
                                       int inter, size_t n, int pieces) {
-    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t i = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;
     if (i >= n) return;
     const size_t row = i / inter;
-    float2 p = *reinterpret_cast<const float2 *>(gu + 2 * i);
-    for (int s = 1; s < parts; s++) {
-        const float2 q = *reinterpret_cast<const float2 *>(gu + s * stride + 2 * i);
-        p.x += q.x;
-        p.y += q.y;
-    }
-    split_store(out + row * pieces * inter, inter, (int)(i % inter), (p.x / (1.0f + expf(-p.x))) * p.y, pieces);
+    const f32x4 a = sum_parts4(gu, 2 * i, parts, stride), b = sum_parts4(gu, 2 * i + 4, parts, stride);
+    const float g[4] = {a[0], a[2], b[0], b[2]}, u[4] = {a[1], a[3], b[1], b[3]};
+    f32x4 y;
+#pragma unroll
+    for (int k = 0; k < 4; k++) y[k] = (g[k] / (1.0f + expf(-g[k]))) * u[k];
+    split_store4(out + row * pieces * inter, inter, (int)(i % inter), y, pieces);
 }
 
 // One wavefront per (position, head) row of q, k or v.
@@ -245,6 +277,7 @@ __global__ __launch_bounds__(AT_THREADS) void prefill_attn_kernel(PrefillAttnArg
     const int qabs = a.past + qc;
     bf16x8 qp_[KSTEPS][NP];
     {
+        const float qscale = a.scale * 1.44269504088896340736f;
         const float *qp = a.q + (size_t)qc * a.ldq + (size_t)h * HD + lh * 8;
 #pragma unroll
         for (int ks = 0; ks < KSTEPS; ks++) {
@@ -252,9 +285,9 @@ __global__ __launch_bounds__(AT_THREADS) void prefill_attn_kernel(PrefillAttnArg
             const f32x4 x1 = *reinterpret_cast<const f32x4 *>(qp + 16 * ks + 4);
             float f[8];
 #pragma unroll
-            for (int i = 0; i < 4; i++) {
-                f[i] = x0[i] * a.scale;
-                f[4 + i] = x1[i] * a.scale;
+            for (int i = 0; i < 4; i++) {  // scores come out in units of ln 2: the softmax uses exp2
+                f[i] = x0[i] * qscale;
+                f[4 + i] = x1[i] * qscale;
             }
             split8<NP>(f, qp_[ks]);
         }
@@ -264,6 +297,7 @@ __global__ __launch_bounds__(AT_THREADS) void prefill_attn_kernel(PrefillAttnArg
     const int wg_end = a.past + min(a.S, q0 + AT_QROWS);
     const int wave_end = q0 + wave * 32 < a.S ? a.past + min(a.S, q0 + wave * 32 + 32) : 0;
     const int ntiles = (wg_end + AT_KEYS - 1) / AT_KEYS;
+    const int wave_first = a.past + min(q0 + wave * 32, a.S - 1);  // smallest position among this wavefront's rows
 
     // thread's share of a tile on its way from the cache to LDS
     u32x4 kr[KLOADS], vr[4];
@@ -332,53 +366,63 @@ __global__ __launch_bounds__(AT_THREADS) void prefill_attn_kernel(PrefillAttnArg
                     s[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qp_[ks][p], s[kb], 0, 0, 0);
             }
         }
-        // accumulator value v of block kb belongs to key 32 kb + 16 (v / 8) + 8 (lane / 32) + v % 8
+        // accumulator value v of block kb belongs to key 32 kb + 16 (v / 8) + 8 (lane / 32) + v % 8;
+        // only tiles that reach past the first row of this wavefront need the causal mask
+        if (t * AT_KEYS + AT_KEYS - 1 > wave_first) {
+#pragma unroll
+            for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+                for (int v = 0; v < 16; v++) {
+                    const int key = t * AT_KEYS + 32 * kb + 16 * (v >> 3) + 8 * lh + (v & 7);
+                    s[kb][v] = key > qabs ? -INFINITY : s[kb][v];
+                }
+        }
         float mx = -INFINITY;
 #pragma unroll
         for (int kb = 0; kb < 2; kb++)
 #pragma unroll
-            for (int v = 0; v < 16; v++) {
-                const int key = t * AT_KEYS + 32 * kb + 16 * (v >> 3) + 8 * lh + (v & 7);
-                const float x = key > qabs ? -INFINITY : s[kb][v];
-                s[kb][v] = x;
-                mx = fmaxf(mx, x);
-            }
+            for (int v = 0; v < 16; v++) mx = fmaxf(mx, s[kb][v]);
         mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-        const float m_new = fmaxf(m_run, mx);  // finite: key 0 is visible to every row
-        const float alpha = expf(m_run - m_new);
+        // The reference point of the exponentials only has to be near the maximum, not on it (softmax is
+        // shift-invariant and l, O are f32): it moves when the maximum has grown by more than 2^8, so
+        // after the first tiles the rescaling of O is skipped for the whole wavefront. m_new is finite:
+        // key 0 is visible to every row. Both half-lanes of a query take the same decision.
+        const float m_new = mx > m_run + 8.0f ? mx : m_run;
+        const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
         float psum = 0.f;
 #pragma unroll
         for (int kb = 0; kb < 2; kb++)
 #pragma unroll
             for (int v = 0; v < 16; v++) {
-                const float p = expf(s[kb][v] - m_new);
+                const float p = __builtin_amdgcn_exp2f(s[kb][v] - m_new);
                 s[kb][v] = p;
                 psum += p;
             }
         l_run = l_run * alpha + psum;  // this lane's half of the keys; the halves meet at the end
         m_run = m_new;
+        if (__any(alpha != 1.0f)) {
 #pragma unroll
-        for (int db = 0; db < DB; db++)
+            for (int db = 0; db < DB; db++)
 #pragma unroll
-            for (int v = 0; v < 16; v++) acc_o[db][v] *= alpha;
+                for (int v = 0; v < 16; v++) acc_o[db][v] *= alpha;
+        }
 
-        bf16x8 pp[4][NP];
+        // 16 keys at a time: their probabilities become NP operands, multiplied into every block of O^T
 #pragma unroll
         for (int sp = 0; sp < 4; sp++) {
             float f[8];
 #pragma unroll
             for (int i = 0; i < 8; i++) f[i] = s[sp >> 1][8 * (sp & 1) + i];
-            split8<NP>(f, pp[sp]);
-        }
+            bf16x8 pp[NP];
+            split8<NP>(f, pp);
 #pragma unroll
-        for (int db = 0; db < DB; db++)
-#pragma unroll
-            for (int sp = 0; sp < 4; sp++) {
+            for (int db = 0; db < DB; db++) {
                 const bf16x8 vf = *reinterpret_cast<const bf16x8 *>(v_lds + vt_off(32 * db + l32, 2 * sp + lh));
 #pragma unroll
                 for (int p = 0; p < NP; p++)
-                    acc_o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pp[sp][p], acc_o[db], 0, 0, 0);
+                    acc_o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pp[p], acc_o[db], 0, 0, 0);
             }
+        }
     }
 
     const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
@@ -396,15 +440,15 @@ __global__ __launch_bounds__(AT_THREADS) void prefill_attn_kernel(PrefillAttnArg
             for (int i = 0; i < 4; i++) o[i] = acc_o[db][4 * g + i] * inv;
             if (a.out_f32) *reinterpret_cast<f32x4 *>(a.out_f32 + (size_t)qrow * qd + d0) = o;
             if (a.out_split) {
-                uint32_t pc[4][NP];
-#pragma unroll
-                for (int i = 0; i < 4; i++) split_pieces<NP>(o[i], pc[i]);
+                uint32_t lo[NP], hi[NP];
+                split_pair<NP>(o[0], o[1], lo);
+                split_pair<NP>(o[2], o[3], hi);
                 uint16_t *o16 = a.out_split + (size_t)qrow * NP * qd + d0;
 #pragma unroll
                 for (int p = 0; p < NP; p++) {
                     u32x2 w;
-                    w.x = pc[0][p] | (pc[1][p] << 16);
-                    w.y = pc[2][p] | (pc[3][p] << 16);
+                    w.x = lo[p];
+                    w.y = hi[p];
                     *reinterpret_cast<u32x2 *>(o16 + (size_t)p * qd) = w;
                 }
             }
@@ -418,18 +462,12 @@ namespace homura {
 int rmsnorm_split_launch(hm_ctx *ctx, const float *d_x, const float *d_res, int res_parts, const float *d_w,
                          uint16_t *d_out_split, int pieces, float *d_resid_out, int rows, int dim, float eps) {
     HM_REQUIRE(ctx, d_x && d_w && d_out_split, "rmsnorm_split: NULL pointer");
-    HM_REQUIRE(ctx, rows > 0 && dim > 0 && pieces >= 1 && pieces <= 3 && res_parts >= 1, "rmsnorm_split: bad shape");
+    HM_REQUIRE(ctx, rows > 0 && dim > 0 && dim % 4 == 0 && pieces >= 1 && pieces <= 3 && res_parts >= 1,
+               "rmsnorm_split: bad shape (dim %% 4 == 0 needed)");
+    HM_REQUIRE(ctx, ((uintptr_t)d_x % 16) == 0 && ((uintptr_t)d_w % 16) == 0 && ((uintptr_t)d_out_split % 8) == 0 &&
+                        ((uintptr_t)d_res % 16) == 0 && ((uintptr_t)d_resid_out % 16) == 0, "rmsnorm_split: misaligned buffer");
     hipLaunchKernelGGL(rmsnorm_split_kernel, dim3(rows), dim3(256), 0, ctx->stream, d_x, d_res, res_parts,
                        (size_t)rows * dim, d_w, d_out_split, d_resid_out, dim, eps, pieces);
-    HM_LAUNCH_CHECK(ctx);
-    return HM_OK;
-}
-
-int add_parts_launch(hm_ctx *ctx, const float *d_a, const float *d_b, int parts, float *d_out, size_t n) {
-    HM_REQUIRE(ctx, d_a && d_b && d_out && parts >= 1, "add_parts: bad arguments");
-    if (n == 0) return HM_OK;
-    hipLaunchKernelGGL(add_parts_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, ctx->stream, d_a, d_b, parts, n,
-                       d_out, n);
     HM_LAUNCH_CHECK(ctx);
     return HM_OK;
 }
@@ -437,10 +475,11 @@ int add_parts_launch(hm_ctx *ctx, const float *d_a, const float *d_b, int parts,
 int silu_mul_split_launch(hm_ctx *ctx, const float *d_gu, int parts, uint16_t *d_out_split, int pieces, int rows,
                           int inter) {
     HM_REQUIRE(ctx, d_gu && d_out_split, "silu_mul_split: NULL pointer");
-    HM_REQUIRE(ctx, rows > 0 && inter > 0 && pieces >= 1 && pieces <= 3 && parts >= 1, "silu_mul_split: bad shape");
-    HM_REQUIRE(ctx, ((uintptr_t)d_gu % 8) == 0, "silu_mul_split: input must be 8-byte aligned");
+    HM_REQUIRE(ctx, rows > 0 && inter > 0 && inter % 4 == 0 && pieces >= 1 && pieces <= 3 && parts >= 1,
+               "silu_mul_split: bad shape (intermediate size %% 4 == 0 needed)");
+    HM_REQUIRE(ctx, ((uintptr_t)d_gu % 16) == 0 && ((uintptr_t)d_out_split % 8) == 0, "silu_mul_split: misaligned buffer");
     const size_t n = (size_t)rows * inter;
-    hipLaunchKernelGGL(silu_mul_split_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, ctx->stream, d_gu, parts,
+    hipLaunchKernelGGL(silu_mul_split_kernel, dim3((unsigned)((n / 4 + 255) / 256)), dim3(256), 0, ctx->stream, d_gu, parts,
                        2 * n, d_out_split, inter, n, pieces);
     HM_LAUNCH_CHECK(ctx);
     return HM_OK;
