@@ -42,13 +42,13 @@ KERNEL_FAMILY = {
 # the factors a 32 MiB + 32 MiB copy kernel calibrates), per kernel of the table below; the
 # counter runs are separate from this program and summarised under profiles/.
 PMC_TRAFFIC_BYTES = {
-    "gemv_bf16[qkv]": 8531786,
-    "gemv_bf16[o]": 4328319,
-    "gemv_bf16[gate_up+silu]": 12768003,
-    "gemv_bf16[down+residual]": 6530325,
-    "gemv_bf16[lm_head+argmax]": 311895078,
-    "qknorm_rope_append+gqa_attn": 4619158,
-    "gqa_attn_fold": 252744,
+    "gemv_bf16[qkv]": 8532764,
+    "gemv_bf16[o]": 4332359,
+    "gemv_bf16[gate_up+silu]": 12767896,
+    "gemv_bf16[down+residual]": 6526172,
+    "gemv_bf16[lm_head+argmax]": 311888989,
+    "qknorm_rope_append+gqa_attn": 4622403,
+    "gqa_attn_fold": 269114,
 }
 
 
@@ -67,11 +67,15 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=64)
     ap.add_argument("--warmup", type=int, default=8)
-    ap.add_argument("--no-graph", action="store_true", help="launch kernel by kernel instead of graph replay")
+    ap.add_argument("--no-graph", action="store_true",
+                    help="launch kernel by kernel instead of graph replay (decode steps and stand-alone kernels)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-tokens", type=int, default=96, help="tokens of the CPU-baseline sample")
     ap.add_argument("--kernel-rounds", type=int, default=20)
     ap.add_argument("--kernel-reps", type=int, default=10, help="graph replays per stand-alone kernel measurement")
+    ap.add_argument("--kernel-max-launches", type=int, default=0,
+                    help="cap on kernel launches per stand-alone measurement graph (0 = the whole weight ring)")
+    ap.add_argument("--no-prefill", action="store_true", help="skip the prompt-pass measurement")
     ap.add_argument("--no-kernel-configs", action="store_true",
                     help="skip the stand-alone kernel measurements (BASELINE configurations 1, 3, 4, 5)")
     args = ap.parse_args()
@@ -168,6 +172,28 @@ def main() -> int:
         host_loop_s = time.perf_counter() - t0
         pcie_inclusive = {"value": round(host_steps / host_loop_s, 2), "unit": "tok/s", "steps": host_steps,
                           "what": "run_kv per token with the logits row downloaded and argmax on the host"}
+        # The prompt side of the same model: 512 tokens on an empty cache through the prefill pass
+        # (projections on the matrix cores), against the same tokens one decode step at a time.
+        prefill = None
+        if not args.no_prefill:
+            ptoks = synth.token_ids(seed + 0x300, 512, cfg.vocab_size)
+            prefill = {"tokens": 512, "unit": "tok/s"}
+            for pieces in (3, 2):
+                model.set_prefill_pieces(pieces)
+                model.reset_kv_cache()
+                model.prefill(ptoks, want_logits=False)   # warm-up (allocates the chunk's scratch)
+                best = None
+                for _ in range(5):
+                    model.reset_kv_cache()
+                    ctx.sync()
+                    t0 = time.perf_counter()
+                    model.prefill(ptoks, want_logits=False)
+                    dt = time.perf_counter() - t0
+                    best = dt if best is None or dt < best else best
+                prefill[f"bf16x{pieces}"] = {"value": round(512 / best, 1), "ms": round(best * 1e3, 3)}
+            model.set_prefill_pieces(3)
+            prefill["what"] = ("HfModel.prefill of 512 prompt tokens, empty cache, no LM head; bf16x3 = every f32 "
+                               "activation as three bf16 pieces (default, exact), bf16x2 = two pieces")
         launches = model.launches_per_step()
         device = ctx.device_name()
         model.close()
@@ -175,6 +201,8 @@ def main() -> int:
         if not args.no_kernel_configs:
             from homura_amd import kernel_bench
             kernel_bench.REPS = args.kernel_reps
+            kernel_bench.MAX_LAUNCHES = args.kernel_max_launches
+            kernel_bench.USE_GRAPH = not args.no_graph
             kernel_configs = kernel_bench.run_all(ctx)
 
     cpu_baseline = None
@@ -208,6 +236,7 @@ def main() -> int:
         "roofline": roofline,
         "cpu_baseline": cpu_baseline,
         "pcie_inclusive": pcie_inclusive,
+        "prefill": prefill,
         "event_ms_per_step": round(event_ms / args.steps, 4),
         "kernels": kernels,
         "kernel_configs": kernel_configs,

@@ -80,11 +80,38 @@ __device__ __forceinline__ int wrap_k(int kc, int Kb) {
 // Requests one K tile. No branches on k: a chunk beyond K reads the last valid chunk of its row
 // (and is replaced by zeros when it is written to LDS), so the loop body stays one basic block and
 // the compiler can count exactly which loads a later LDS write has to wait for.
-template <bool B_NK>
+// ALIGNED (the k loop length and B's k extent are multiples of the 64-wide tile): the k offsets are
+// the same for every thread, so they stay in scalar registers and a load costs one address add.
+template <bool B_NK, bool ALIGNED>
 __device__ __forceinline__ void load_tile(TileRegs &t, const uint16_t *__restrict__ A,
-                                          const uint16_t *__restrict__ B, int m0, int n0, int k0,
+                                          const uint16_t *__restrict__ B, int m0, int n0, int k0, int kb,
                                           const GemmDims &g, int tid) {
     const int K = g.K;
+    if (ALIGNED) {
+        // tiles past the end re-read the last one of A and whatever tile of B comes next (both are
+        // replaced by zeros at the LDS write)
+        const int ka = min(k0, K - TK);
+        if (B_NK) {
+#pragma unroll
+            for (int j = 0; j < 2; j++) {
+                const int id = tid + j * GEMM_THREADS, r = id >> 3, c = id & 7;
+                t.v[j] = ld128(A + ((size_t)min(m0 + r, g.M - 1) * g.lda + c * 8) + ka);
+                t.v[2 + j] = ld128(B + ((size_t)min(n0 + r, g.N - 1) * g.Kb + c * 8) + kb);
+            }
+        } else if (tid < 256) {
+            const int ng = tid & 15, kg = tid >> 4;
+            const int nc = min(n0 + ng * 8, g.N - 8);
+#pragma unroll
+            for (int r = 0; r < 4; r++) t.v[r] = ld128(B + ((size_t)(kg * 4 + r) * g.N + nc) + (size_t)kb * g.N);
+        } else {
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const int id = (tid - 256) + j * 256, r = id >> 3, c = id & 7;
+                t.v[j] = ld128(A + ((size_t)min(m0 + r, g.M - 1) * g.lda + c * 8) + ka);
+            }
+        }
+        return;
+    }
     if (B_NK) {
 #pragma unroll
         for (int j = 0; j < 2; j++) {
@@ -115,18 +142,18 @@ __device__ __forceinline__ void load_tile(TileRegs &t, const uint16_t *__restric
 
 // Half `part` (0, 1) of a thread's LDS writes of one tile; the halves sit next to the two MFMA
 // groups a wavefront runs per tile.
-template <bool B_NK>
+template <bool B_NK, bool ALIGNED>
 __device__ __forceinline__ void store_tile_part(const TileRegs &t, char *__restrict__ as,
                                                 char *__restrict__ bs, int tid, int part, int k0, int K) {
     const u32x4 zero = {0u, 0u, 0u, 0u};
     if (B_NK) {
         const int id = tid + part * GEMM_THREADS, r = id >> 3, c = id & 7;
-        const bool ok = k0 + c * 8 < K;
+        const bool ok = ALIGNED ? k0 < K : k0 + c * 8 < K;
         *reinterpret_cast<u32x4 *>(as + lds_off(r, c)) = ok ? t.v[part] : zero;
         *reinterpret_cast<u32x4 *>(bs + lds_off(r, c)) = ok ? t.v[2 + part] : zero;
     } else if (tid < 256) {
         const int ng = tid & 15, kg = tid >> 4;
-        const bool ok = k0 + kg * 4 < K;  // K is a multiple of 32: the four rows are in or out together
+        const bool ok = ALIGNED ? k0 < K : k0 + kg * 4 < K;  // K is a multiple of 32: the four rows are in or out together
 #pragma unroll
         for (int i = part * 4; i < part * 4 + 4; i++) {
             // column n = ng*8 + i of the block: k+0..k+3 packed low to high
@@ -141,7 +168,7 @@ __device__ __forceinline__ void store_tile_part(const TileRegs &t, char *__restr
 #pragma unroll
         for (int j = part * 2; j < part * 2 + 2; j++) {
             const int id = (tid - 256) + j * 256, r = id >> 3, c = id & 7;
-            *reinterpret_cast<u32x4 *>(as + lds_off(r, c)) = k0 + c * 8 < K ? t.v[j] : zero;
+            *reinterpret_cast<u32x4 *>(as + lds_off(r, c)) = (ALIGNED ? k0 < K : k0 + c * 8 < K) ? t.v[j] : zero;
         }
     }
 }
@@ -150,7 +177,7 @@ __device__ __forceinline__ void store_tile_part(const TileRegs &t, char *__restr
 // global loads and the MFMAs of a tile fast enough to keep the matrix pipe busy. Wavefronts 0-3
 // multiply k steps 0 and 1 of every K tile, wavefronts 4-7 steps 2 and 3, each group with its own
 // 2x2 arrangement of 64x64 accumulators; the two groups' sums meet in LDS at the end.
-template <bool B_NK>
+template <bool B_NK, bool ALIGNED>
 __global__ __launch_bounds__(GEMM_THREADS) void gemm_bf16_mfma_kernel(const uint16_t *__restrict__ A,
                                                                       const uint16_t *__restrict__ B,
                                                                       float *__restrict__ C, const GemmDims g) {
@@ -188,10 +215,17 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_bf16_mfma_kernel(const uint
     const int kbase = kt_first * TK;
     C += (size_t)blockIdx.y * M * N;
     TileRegs t[DEPTH];
+    // B's k offset of the next tile to request: runs along with the loop and wraps at Kb (ALIGNED only)
+    int kb_run = kbase % g.Kb;
+    auto request = [&](TileRegs &dst, int k0) {
+        load_tile<B_NK, ALIGNED>(dst, A, B, m0, n0, k0, kb_run, g, tid);
+        kb_run += TK;
+        kb_run = kb_run >= g.Kb ? kb_run - g.Kb : kb_run;
+    };
 #pragma unroll
-    for (int d = 0; d < DEPTH; d++) load_tile<B_NK>(t[d], A, B, m0, n0, kbase + d * TK, g, tid);
+    for (int d = 0; d < DEPTH; d++) request(t[d], kbase + d * TK);
 #pragma unroll
-    for (int part = 0; part < 2; part++) store_tile_part<B_NK>(t[0], lds[0][0], lds[0][1], tid, part, kbase, K);
+    for (int part = 0; part < 2; part++) store_tile_part<B_NK, ALIGNED>(t[0], lds[0][0], lds[0][1], tid, part, kbase, K);
     lds_barrier();
 
     // operand registers, two stages: the reads of the next step are in flight during the MFMAs
@@ -209,7 +243,7 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_bf16_mfma_kernel(const uint
         for (int u = 0; u < DEPTH; u++) {
             const int cur = u & 1;  // DEPTH is even: tile kt0+u sits in buffer u & 1
             // tile kt0+u left its registers during the previous iteration: refill them
-            load_tile<B_NK>(t[u], A, B, m0, n0, kbase + (kt0 + u + DEPTH) * TK, g, tid);
+            request(t[u], kbase + (kt0 + u + DEPTH) * TK);
             const int k_next = kbase + (kt0 + u + 1) * TK;
             char *an = lds[cur ^ 1][0], *bn = lds[cur ^ 1][1];
 
@@ -224,8 +258,8 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_bf16_mfma_kernel(const uint
 #pragma unroll
                 for (int j = 0; j < 2; j++)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[0][i], bfr[0][j], acc[i][j], 0, 0, 0);
-            store_tile_part<B_NK>(t[(u + 1) % DEPTH], an, bn, tid, 0, k_next, K);
-            store_tile_part<B_NK>(t[(u + 1) % DEPTH], an, bn, tid, 1, k_next, K);
+            store_tile_part<B_NK, ALIGNED>(t[(u + 1) % DEPTH], an, bn, tid, 0, k_next, K);
+            store_tile_part<B_NK, ALIGNED>(t[(u + 1) % DEPTH], an, bn, tid, 1, k_next, K);
             // every wavefront has written its share of the next tile and read the last operands of
             // this one: switch buffers, and fetch the next tile's first operands under the second
             // MFMA group of this tile
@@ -259,6 +293,7 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_bf16_mfma_kernel(const uint
     if (kgrp == 1) return;
 
     // accumulator element v of lane l sits at row (v/4)*8 + (l/32)*4 + v%4, column l%32
+    const bool interior = m0 + TM <= M && n0 + TN <= N;  // workgroup-uniform: edge tiles check every element
 #pragma unroll
     for (int i = 0; i < 2; i++)
 #pragma unroll
@@ -267,9 +302,11 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_bf16_mfma_kernel(const uint
             for (int v = 0; v < 16; v++) {
                 const int row = m0 + wm * 64 + i * 32 + (v >> 2) * 8 + lh * 4 + (v & 3);
                 const int col = n0 + wn * 64 + j * 32 + l32;
-                if (row < M && col < N)
-                    __builtin_nontemporal_store(acc[i][j][v] + xch[((i * 2 + j) * 16 + v) * 64],
-                                                C + (size_t)row * N + col);
+                const float sum = acc[i][j][v] + xch[((i * 2 + j) * 16 + v) * 64];
+                if (interior)
+                    __builtin_nontemporal_store(sum, C + (size_t)row * N + col);
+                else if (row < M && col < N)
+                    __builtin_nontemporal_store(sum, C + (size_t)row * N + col);
             }
 }
 
@@ -296,10 +333,15 @@ int gemm_launch(hm_ctx *ctx, const char *who, const uint16_t *a, const uint16_t 
     const int slices = (nk_total + g.kt_per_split - 1) / g.kt_per_split;
     if (ksplit_used) *ksplit_used = slices;
     const dim3 grid((unsigned)tiles, (unsigned)slices);
-    if (b_nk)
-        hipLaunchKernelGGL(gemm_bf16_mfma_kernel<true>, grid, dim3(GEMM_THREADS), 0, ctx->stream, a, b, c, g);
+    const bool aligned = g.K % TK == 0 && g.Kb % TK == 0;
+    if (b_nk && aligned)
+        hipLaunchKernelGGL((gemm_bf16_mfma_kernel<true, true>), grid, dim3(GEMM_THREADS), 0, ctx->stream, a, b, c, g);
+    else if (b_nk)
+        hipLaunchKernelGGL((gemm_bf16_mfma_kernel<true, false>), grid, dim3(GEMM_THREADS), 0, ctx->stream, a, b, c, g);
+    else if (aligned)
+        hipLaunchKernelGGL((gemm_bf16_mfma_kernel<false, true>), grid, dim3(GEMM_THREADS), 0, ctx->stream, a, b, c, g);
     else
-        hipLaunchKernelGGL(gemm_bf16_mfma_kernel<false>, grid, dim3(GEMM_THREADS), 0, ctx->stream, a, b, c, g);
+        hipLaunchKernelGGL((gemm_bf16_mfma_kernel<false, false>), grid, dim3(GEMM_THREADS), 0, ctx->stream, a, b, c, g);
     HM_LAUNCH_CHECK(ctx);
     return HM_OK;
 }

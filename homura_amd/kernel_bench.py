@@ -31,14 +31,21 @@ def _ring(ctx: Context, host: np.ndarray):
 
 
 REPS = 10  # graph replays per measurement (bench.py lowers it under a profiler)
+MAX_LAUNCHES = 0  # > 0: at most this many kernel launches per measurement (counter runs keep them short)
+USE_GRAPH = True  # False: launch kernel by kernel (for runs under a profiler; host launch gaps enter the time)
 
 
 def _time(ctx: Context, launches, reps=None):
     reps = reps or REPS
+    if MAX_LAUNCHES > 0:
+        launches = launches[:MAX_LAUNCHES]
     def record():
         for fn in launches:
             fn()
-    ms = ctx.time_graph_ms(record, reps=reps, warmup=2)
+    if USE_GRAPH:
+        ms = ctx.time_graph_ms(record, reps=reps, warmup=4)
+    else:
+        ms = ctx.time_ms(record, reps, 1)
     return ms * 1e3 / len(launches)  # microseconds per launch
 
 
@@ -131,5 +138,44 @@ def run_all(ctx: Context):
     out.append(_entry("cfg5b gqa_decode_attn 8x(12q/2kv)x128, kv 4096", us,
                       2 * B * kvh * L * hd * 2 + 2 * B * H * hd * 4))
     for b in kring + vring:
+        b.free()
+
+    # K-quant GEMVs at the projection shapes of a 0.6B model (Q8_K activation quantisation included)
+    for kind, bb, blocks, fn in (("q4_k", 144, synth.q4_k_blocks, ctx.gemv_q4_k), ("q6_k", 210, synth.q6_k_blocks, ctx.gemv_q6_k)):
+        for K, N in ((1024, 6144), (3072, 1024)):
+            x = ctx.to_device(synth.normal_f32(7, K))
+            ring = _ring(ctx, blocks(11, N * K // 256))
+            o = ctx.empty(N)
+            us = _time(ctx, [lambda b=b: fn(x, b, o, 1, K, N) for b in ring])
+            out.append(_entry(f"gemv_{kind} {K}->{N}", us, N * (K // 256) * bb + K * 4 + N * 4,
+                              note="two launches: activation to Q8_K, then the integer-dot GEMV"))
+            for b in ring:
+                b.free()
+            x.free()
+            o.free()
+
+    # prefill: f32 activations x bf16 weights (three bf16 pieces per activation) at config 5a's shape
+    M, K, N = 512, 2048, 8192
+    a = ctx.to_device(synth.normal_f32(synth.SEED_CFG5, M * K))
+    ring = _ring(ctx, synth.normal_bf16(synth.SEED_CFG5 + 1, K * N, 0.02))
+    c = ctx.empty(M * N)
+    us = _time(ctx, [lambda b=b: ctx.gemm_f32_bf16_nk(a, b, c, M, K, N) for b in ring])
+    out.append(_entry("gemm_f32_bf16_nk 512x2048x8192", us, M * K * 4 + K * N * 2 + M * N * 4, 3 * 2.0 * M * K * N,
+                      note="flop = the three bf16 passes the matrix cores run; includes the kernel that splits A"))
+    for b in ring + [a, c]:
+        b.free()
+
+    # prefill attention: 512 new rows on 1024 cached ones, Qwen3-0.6B heads
+    S, H, kvh, hd, L, past = 512, 16, 8, 128, 2048, 1024
+    q = ctx.to_device(synth.normal_f32(5, S * H * hd))
+    kc = ctx.to_device(synth.normal_bf16(6, kvh * L * hd))
+    vc = ctx.to_device(synth.normal_bf16(7, kvh * L * hd))
+    o = ctx.empty(S * H * hd)
+    us = _time(ctx, [lambda: ctx.gqa_prefill_attn(q, kc, vc, o, S, H, kvh, hd, L, past, 1.0 / math.sqrt(hd))] * 8)
+    visible = S * past + S * (S + 1) // 2                      # (query, key) pairs under the causal mask
+    out.append(_entry(f"gqa_prefill_attn {S} rows on {past} cached, 16q/8kv x 128", us,
+                      flops=3 * 2 * 2.0 * H * hd * visible,
+                      note="flop = QK^T and PV over the visible pairs, three bf16 passes each"))
+    for b in (q, kc, vc, o):
         b.free()
     return out
