@@ -31,6 +31,18 @@ class HmTransformerConfig(C.Structure):
     ]
 
 
+class HmSamplingConfig(C.Structure):
+    _fields_ = [
+        ("temperature", C.c_float),
+        ("top_k", C.c_int),
+        ("top_p", C.c_float),
+        ("min_p", C.c_float),
+        ("repetition_penalty", C.c_float),
+        ("frequency_penalty", C.c_float),
+        ("presence_penalty", C.c_float),
+    ]
+
+
 class HmKernelProfile(C.Structure):
     _fields_ = [
         ("label", C.c_char * 32),
@@ -132,6 +144,14 @@ SIGNATURES = {
     "hm_model_set_graph": (_I, [_P, _I]),
     "hm_model_run_kv": (_I, [_P, C.POINTER(C.c_int64), _I, c_f32_p]),
     "hm_model_prefill": (_I, [_P, C.POINTER(C.c_int64), _I, c_f32_p]),
+    "hm_model_generate": (_I, [_P, C.POINTER(C.c_int64), _I, _I, C.POINTER(HmSamplingConfig), C.c_uint64, _I,
+                               C.POINTER(C.c_int32), C.POINTER(_I)]),
+    "hm_rng_seed": (C.c_uint64, [C.c_uint64]),
+    "hm_rng_next_f32": (C.c_float, [C.POINTER(C.c_uint64)]),
+    "hm_sample_token_host": (_I, [_P, _I, C.POINTER(HmSamplingConfig), _P, _I, C.POINTER(C.c_uint64),
+                                  C.POINTER(C.c_int32)]),
+    "hm_sample_token": (_I, [_P, _P, _I, C.POINTER(HmSamplingConfig), _P, _I, C.POINTER(C.c_uint64),
+                             C.POINTER(C.c_int32)]),
     "hm_model_set_prefill_min": (_I, [_P, _I]),
     "hm_model_set_prefill_pieces": (_I, [_P, _I]),
     "hm_model_generate_greedy": (_I, [_P, C.POINTER(C.c_int64), _I, _I, C.POINTER(C.c_int32)]),

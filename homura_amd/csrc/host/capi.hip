@@ -71,6 +71,14 @@ int hm_model_prefill(hm_model *m, const int64_t *h_ids, int n_ids, float *h_logi
     return m->impl->prefill(h_ids, n_ids, h_logits);
 }
 
+int hm_model_generate(hm_model *m, const int64_t *h_prompt, int n_prompt, int max_new_tokens,
+                      const hm_sampling_config *cfg, uint64_t seed, int eos_token_id, int32_t *h_tokens_out,
+                      int *n_tokens_out) {
+    if (!m) return HM_ERR_INVALID;
+    if (!cfg) return hm_set_error(m->ctx, HM_ERR_INVALID, "hm_model_generate: NULL sampling configuration");
+    return m->impl->generate(h_prompt, n_prompt, max_new_tokens, *cfg, seed, eos_token_id, h_tokens_out, n_tokens_out);
+}
+
 int hm_model_set_prefill_pieces(hm_model *m, int pieces) {
     if (!m) return HM_ERR_INVALID;
     if (pieces != 2 && pieces != 3) return hm_set_error(m->ctx, HM_ERR_INVALID, "prefill pieces must be 2 or 3");

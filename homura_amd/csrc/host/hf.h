@@ -91,6 +91,9 @@ class HfModel {
     int reset_kv_cache();
     int kv_cache_len() const;
     int generate_greedy(const int64_t *h_prompt, int n_prompt, int n_new, int32_t *h_tokens);
+    // reference generate_streaming_core (src/generate.rs:100-315) with sample_token (:698-801)
+    int generate(const int64_t *h_prompt, int n_prompt, int max_new, const hm_sampling_config &cfg, uint64_t seed,
+                 int eos_token, int32_t *h_tokens, int *n_out);
     int bench_decode(int64_t first_id, int n_steps, float *ms_out, int32_t *h_tokens);
     int profile_step(int64_t token_id, std::vector<StepProfile> &out);
     int time_kernels(int rounds, std::vector<StepProfile> &out);
@@ -134,6 +137,7 @@ class HfModel {
         Buffer ids, h, resid, split, qkv, proj_out, gate_up, logits;
     };
     PrefillScratch pf_;
+    struct SamplerScratch { Buffer work, counts, token, list; int list_cap = 0; } sampler_;
     int prefill_min_ = 8;
     int prefill_pieces_ = 3;
     std::map<std::string, int> slot_by_name_;

@@ -1300,6 +1300,85 @@ int HfModel::generate_greedy(const int64_t *h_prompt, int n_prompt, int n_new, i
     return hm_download(ctx_, h_tokens, plan_->out_tokens() + (n_prompt - 1), (size_t)n_new * 4);
 }
 
+// sampling.hip
+int sample_check_config(hm_ctx *ctx, const hm_sampling_config *cfg, bool device);
+int sample_token_launch(hm_ctx *ctx, const float *d_logits, float *d_work, const int *d_counts, int vocab,
+                        const hm_sampling_config &cfg, float draw, int32_t *d_out, int *d_counts_update, int32_t *d_list,
+                        int list_pos);
+int zero_ints_launch(hm_ctx *ctx, int *d, size_t n);
+
+int HfModel::generate(const int64_t *h_prompt, int n_prompt, int max_new, const hm_sampling_config &cfg, uint64_t seed,
+                      int eos_token, int32_t *h_tokens, int *n_out) {
+    if (!finalized_) return hm_set_error(ctx_, HM_ERR_STATE, "model not finalized");
+    if (n_prompt <= 0 || max_new <= 0 || !h_prompt || !h_tokens || !n_out)
+        return hm_set_error(ctx_, HM_ERR_INVALID, "generate: bad arguments");
+    *n_out = 0;
+    const bool greedy = cfg.temperature <= 0.0f;
+    const bool on_device = greedy || (cfg.top_k >= 1 && cfg.top_k <= 1024);
+    int rc = sample_check_config(ctx_, &cfg, on_device);
+    if (rc != HM_OK) return rc;
+    if (kv_cache_len() + n_prompt > max_seq_len_)
+        return hm_set_error(ctx_, HM_ERR_STATE, "KV cache full (%d + %d > %d)", kv_cache_len(), n_prompt, max_seq_len_);
+    std::vector<int32_t> ids;
+    if ((rc = check_ids(h_prompt, n_prompt, ids)) != HM_OK) return rc;
+    const int vocab = cfg_.vocab_size;
+    SamplerScratch &s = sampler_;
+    if (!s.work) {
+        s.work = Buffer::alloc(ctx_, {vocab}, DType::F32);
+        s.counts = Buffer::alloc(ctx_, {vocab}, DType::F32);  // int32 counts
+        s.token = Buffer::alloc(ctx_, {64}, DType::F32);
+        if (!s.work || !s.counts || !s.token) return HM_ERR_OOM;
+    }
+    if (s.list_cap < max_new) {
+        s.list = Buffer::alloc(ctx_, {max_new}, DType::F32);  // int32 token list
+        if (!s.list) return HM_ERR_OOM;
+        s.list_cap = max_new;
+    }
+    const bool penalties = cfg.repetition_penalty != 1.0f || cfg.frequency_penalty != 0.0f || cfg.presence_penalty != 0.0f;
+    if ((rc = zero_ints_launch(ctx_, s.counts.as<int>(), (size_t)vocab)) != HM_OK) return rc;
+    // prompt: everything but its last token only has to reach the cache
+    // (reference HfGenerationContext::prefill, src/hf/model.rs:321-336)
+    if (n_prompt > 1) {
+        if ((rc = run_kv(h_prompt, n_prompt - 1, nullptr)) != HM_OK) return rc;
+    }
+    uint64_t rng = hm_rng_seed(seed);
+    std::vector<Buffer *> inputs;
+    step_inputs(inputs);
+    const size_t logits_slot = plan_->output_slots()[0];
+    std::vector<float> host_logits;
+    std::vector<uint32_t> generated;
+    int32_t current = ids[n_prompt - 1];
+    for (int step = 0; step < max_new; step++) {
+        if (kv_cache_len() >= max_seq_len_) break;  // context limit (src/generate.rs:188-194)
+        if ((rc = plan_->arm(&current, 1)) != HM_OK) return rc;
+        if ((rc = plan_->run_kv(inputs, weight_bufs_, max_seq_len_)) != HM_OK) return rc;
+        const float *d_logits = plan_->slot(logits_slot)->as<float>();
+        int32_t tok = 0;
+        if (on_device) {
+            const float draw = greedy ? 0.0f : hm_rng_next_f32(&rng);
+            rc = sample_token_launch(ctx_, d_logits, s.work.as<float>(), penalties ? s.counts.as<int>() : nullptr, vocab, cfg,
+                                     draw, s.token.as<int32_t>(), penalties ? s.counts.as<int>() : nullptr,
+                                     s.list.as<int32_t>(), step);
+            if (rc == HM_OK) rc = hm_download(ctx_, &tok, s.token.ptr(), 4);
+        } else {
+            host_logits.resize(vocab);
+            rc = hm_download(ctx_, host_logits.data(), d_logits, (size_t)vocab * 4);
+            if (rc == HM_OK)
+                rc = hm_sample_token_host(host_logits.data(), vocab, &cfg, generated.data(), (int)generated.size(), &rng, &tok);
+        }
+        if (rc != HM_OK) return rc;
+        if (tok == eos_token) {
+            // the reference leaves the loop without storing the token; on the device path it was already
+            // counted for the penalties, which no later step of this call reads
+            break;
+        }
+        generated.push_back((uint32_t)tok);
+        h_tokens[(*n_out)++] = tok;
+        current = tok;
+    }
+    return HM_OK;
+}
+
 int HfModel::bench_decode(int64_t first_id, int n_steps, float *ms_out, int32_t *h_tokens) {
     if (!finalized_) return hm_set_error(ctx_, HM_ERR_STATE, "model not finalized");
     if (n_steps <= 0 || n_steps > plan_->out_capacity())

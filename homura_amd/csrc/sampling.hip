@@ -1,0 +1,468 @@
+// Token sampling (reference sample_token, src/generate.rs:698-801, and its xorshift64 Rng, :609-642).
+//
+// Two implementations behind one configuration struct:
+//  * hm_sample_token_host: the reference's procedure statement by statement on a host logits row
+//    (libm expf, sequential f32 sums, full sort). Any top_k.
+//  * hm_sample_token: the same procedure on a logits row that stays in HBM, for 1 <= top_k <= 1024.
+//    One workgroup of 1024 threads: penalties + temperature + max, exponentials + sum, a radix select
+//    (12 + 10 + 10 bits) of the top_k-th largest exponential, the candidates gathered and sorted in LDS (probability
+//    descending, index ascending among equals), then one thread runs the reference's sequential top_p
+//    and draw loops over at most 1024 candidates. The vocabulary-wide sum is a tree sum here, so a
+//    probability may differ from the host's in the last bit; the picked token differs only when the
+//    draw sits on a cumulative boundary to within that bit.
+// The draw itself (Rng::next_f32) is taken on the host and passed in, so both consume the same stream.
+#include <algorithm>
+#include <cmath>
+#include <cstring>
+#include <vector>
+
+#include "hm_common.h"
+
+namespace {
+
+constexpr int SAMPLE_THREADS = 1024;
+constexpr int SAMPLE_MAX_K = 1024;
+
+struct SampleArgs {
+    const float *logits;
+    float *work;          // [vocab] scratch: adjusted logits, then exponentials
+    const int *counts;    // [vocab] occurrences among the generated tokens, or nullptr
+    int vocab;
+    hm_sampling_config cfg;
+    float draw;           // Rng::next_f32 of this step
+    int32_t *out;         // the picked token
+    int *counts_update;   // if set: counts_update[token]++ after the pick (the token joins generated_ids)
+    int32_t *list;        // if set: list[list_pos] = token
+    int list_pos;
+};
+
+__device__ __forceinline__ float penalised(float l, int c, const hm_sampling_config &cfg) {
+    if (c > 0) {
+        if (cfg.repetition_penalty != 1.0f)
+            for (int k = 0; k < c; k++) l = l > 0.0f ? l / cfg.repetition_penalty : l * cfg.repetition_penalty;
+        if (cfg.frequency_penalty != 0.0f || cfg.presence_penalty != 0.0f) {
+            l -= cfg.frequency_penalty * (float)c;
+            l -= cfg.presence_penalty;
+        }
+    }
+    return l;
+}
+
+// a > b in the candidate order: larger probability first, smaller index first among equals
+__device__ __forceinline__ bool cand_before(float pa, int ia, float pb, int ib) {
+    return pa > pb || (pa == pb && ia < ib);
+}
+
+__global__ __launch_bounds__(SAMPLE_THREADS) void sample_token_kernel(SampleArgs a) {
+    __shared__ float red_f[SAMPLE_THREADS / WAVE];
+    __shared__ int red_i[SAMPLE_THREADS / WAVE];
+    __shared__ unsigned hist[4096];
+    __shared__ unsigned sel_prefix, sel_need;
+    __shared__ float cand_p[SAMPLE_MAX_K];
+    __shared__ int cand_i[SAMPLE_MAX_K];
+    __shared__ unsigned n_cand, eq_taken;
+    const int tid = threadIdx.x, lane = tid & (WAVE - 1), wave = tid / WAVE;
+    const int n = a.vocab;
+    const hm_sampling_config cfg = a.cfg;
+
+    // ── pass 1: penalties, then either the greedy pick or temperature + maximum ──
+    const bool greedy = cfg.temperature <= 0.0f;
+    const float inv_temp = greedy ? 1.0f : 1.0f / cfg.temperature;
+    float mx = -INFINITY;
+    int best = -1;  // greedy: last index of the maximum (Rust max_by keeps the last of equal maxima)
+    for (int i = tid; i < n; i += SAMPLE_THREADS) {
+        float l = penalised(a.logits[i], a.counts ? a.counts[i] : 0, cfg);
+        if (greedy) {
+            if (best < 0 || l >= mx) {
+                mx = l;
+                best = i;
+            }
+        } else {
+            l *= inv_temp;
+            a.work[i] = l;
+            mx = fmaxf(mx, l);
+        }
+    }
+    if (greedy) {
+        for (int off = 32; off >= 1; off >>= 1) {
+            const float om = __shfl_xor(mx, off, WAVE);
+            const int ob = __shfl_xor(best, off, WAVE);
+            if (ob >= 0 && (best < 0 || om > mx || (om == mx && ob > best))) {
+                mx = om;
+                best = ob;
+            }
+        }
+        if (lane == 0) {
+            red_f[wave] = mx;
+            red_i[wave] = best;
+        }
+        __syncthreads();
+        if (tid == 0) {
+            for (int w = 1; w < SAMPLE_THREADS / WAVE; w++)
+                if (red_i[w] >= 0 && (best < 0 || red_f[w] > mx || (red_f[w] == mx && red_i[w] > best))) {
+                    mx = red_f[w];
+                    best = red_i[w];
+                }
+            *a.out = best < 0 ? 0 : best;
+            if (a.counts_update && best >= 0) a.counts_update[best] += 1;
+            if (a.list) a.list[a.list_pos] = best < 0 ? 0 : best;
+        }
+        return;
+    }
+    mx = wave_max(mx);
+    if (lane == 0) red_f[wave] = mx;
+    __syncthreads();
+    mx = red_f[0];
+    for (int w = 1; w < SAMPLE_THREADS / WAVE; w++) mx = fmaxf(mx, red_f[w]);
+    __syncthreads();
+
+    // ── pass 2: exponentials and their sum ──
+    float sum = 0.f;
+    for (int i = tid; i < n; i += SAMPLE_THREADS) {
+        const float e = expf(a.work[i] - mx);
+        a.work[i] = e;
+        sum += e;
+    }
+    sum = wave_sum(sum);
+    if (lane == 0) red_f[wave] = sum;
+    __syncthreads();
+    sum = 0.f;
+    for (int w = 0; w < SAMPLE_THREADS / WAVE; w++) sum += red_f[w];
+
+    // ── radix select: bit pattern of the K-th largest exponential (all are >= 0, so patterns order like
+    //    values). 12 + 10 + 10 bits: the first pass sees every element, and 4096 bins keep neighbouring
+    //    lanes off each other's LDS word; later passes only count the elements inside the chosen bin. ──
+    const unsigned K = (unsigned)min(cfg.top_k, n);
+    if (tid == 0) {
+        sel_prefix = 0;
+        sel_need = K;
+    }
+    for (int pass = 0; pass < 3; pass++) {
+        const int shift = pass == 0 ? 20 : pass == 1 ? 10 : 0;
+        const int bits = pass == 0 ? 12 : 10;
+        const int bpt = (1 << bits) / SAMPLE_THREADS;  // bins per thread: 4, 1, 1
+        for (int b = tid; b < (1 << bits); b += SAMPLE_THREADS) hist[b] = 0;
+        __syncthreads();
+        const unsigned prefix = sel_prefix, need = sel_need;
+        const unsigned mask = pass == 0 ? 0u : 0xFFFFFFFFu << (shift + bits);
+        for (int i = tid; i < n; i += SAMPLE_THREADS) {
+            const unsigned u = __float_as_uint(a.work[i]);
+            if ((u & mask) == prefix) atomicAdd(&hist[(u >> shift) & ((1u << bits) - 1u)], 1u);
+        }
+        __syncthreads();
+        // the bin that holds the need-th largest of the counted elements: thread t owns bins [t*bpt, (t+1)*bpt)
+        unsigned mine = 0;
+        for (int j = 0; j < bpt; j++) mine += hist[tid * bpt + j];
+        unsigned incl = mine;  // inclusive prefix sum over threads, low bins first
+        for (int off = 1; off < WAVE; off <<= 1) {
+            const unsigned up = __shfl_up(incl, off, WAVE);
+            if (lane >= off) incl += up;
+        }
+        if (lane == WAVE - 1) red_i[wave] = (int)incl;
+        __syncthreads();
+        unsigned before = 0, total = 0;
+        for (int w = 0; w < SAMPLE_THREADS / WAVE; w++) {
+            if (w < wave) before += (unsigned)red_i[w];
+            total += (unsigned)red_i[w];
+        }
+        const unsigned below_or_mine = before + incl;      // elements in bins up to and including mine
+        const unsigned above = total - below_or_mine;      // elements in higher bins
+        if (above < need && need <= above + mine) {        // exactly one thread
+            unsigned acc = above;
+            for (int j = bpt - 1; j >= 0; j--) {
+                const unsigned h = hist[tid * bpt + j];
+                if (acc + h >= need) {
+                    sel_prefix = prefix | ((unsigned)(tid * bpt + j) << shift);
+                    sel_need = need - acc;  // how many elements of this bin are still wanted
+                    break;
+                }
+                acc += h;
+            }
+        }
+        __syncthreads();
+    }
+    const unsigned T = sel_prefix;
+    const unsigned need_eq = sel_need;
+    if (tid == 0) {
+        n_cand = 0;
+        eq_taken = 0;
+    }
+    __syncthreads();
+    // everything above the K-th value; then the wanted number of elements equal to it, lowest indices first
+    for (int i = tid; i < n; i += SAMPLE_THREADS) {
+        const float e = a.work[i];
+        if (__float_as_uint(e) > T) {
+            const unsigned at = atomicAdd(&n_cand, 1u);
+            cand_p[at] = e;
+            cand_i[at] = i;
+        }
+    }
+    __syncthreads();
+    for (int base = 0; base < n; base += SAMPLE_THREADS) {  // index order: one block-wide ordered take per 1024
+        if (eq_taken >= need_eq) break;
+        const int i = base + tid;
+        const bool eq = i < n && __float_as_uint(a.work[i]) == T;
+        const unsigned long long m = __ballot(eq);
+        if (lane == 0) red_i[wave] = __popcll(m);
+        __syncthreads();
+        unsigned before = eq_taken;
+        for (int w = 0; w < wave; w++) before += red_i[w];
+        const unsigned rank = before + __popcll(m & ((1ull << lane) - 1ull));
+        if (eq && rank < need_eq) {
+            const unsigned at = atomicAdd(&n_cand, 1u);
+            cand_p[at] = a.work[i];
+            cand_i[at] = i;
+        }
+        __syncthreads();
+        if (tid == 0) {
+            unsigned tot = 0;
+            for (int w = 0; w < SAMPLE_THREADS / WAVE; w++) tot += red_i[w];
+            eq_taken += tot;
+        }
+        __syncthreads();
+    }
+    __syncthreads();
+    const int nc = (int)n_cand;  // == K
+    // normalise, min_p (the maximum probability is exp(0) / sum), pad to the sort size
+    const float max_prob = 1.0f / sum;
+    const float threshold = cfg.min_p * max_prob;
+    if (tid < SAMPLE_MAX_K) {
+        if (tid < nc) {
+            float p = cand_p[tid] / sum;
+            if (cfg.min_p > 0.0f && p < threshold) p = 0.0f;
+            cand_p[tid] = p;
+        } else {
+            cand_p[tid] = -1.0f;  // sorts behind every real candidate
+            cand_i[tid] = 0x7FFFFFFF;
+        }
+    }
+    __syncthreads();
+    // bitonic sort of 1024 (probability descending, index ascending among equals)
+    for (int k = 2; k <= SAMPLE_MAX_K; k <<= 1)
+        for (int j = k >> 1; j > 0; j >>= 1) {
+            const int partner = tid ^ j;
+            if (partner > tid) {
+                const float pa = cand_p[tid], pb = cand_p[partner];
+                const int ia = cand_i[tid], ib = cand_i[partner];
+                const bool up = (tid & k) == 0;  // this pair ends in candidate order
+                if (cand_before(pb, ib, pa, ia) == up) {
+                    cand_p[tid] = pb;
+                    cand_i[tid] = ib;
+                    cand_p[partner] = pa;
+                    cand_i[partner] = ia;
+                }
+            }
+            __syncthreads();
+        }
+    // the reference's sequential loops (src/generate.rs:771-800)
+    if (tid == 0) {
+        float cumulative = 0.0f;
+        int cutoff = nc;
+        for (int i = 0; i < nc; i++) {
+            cumulative += cand_p[i];
+            if (cumulative >= cfg.top_p) {
+                cutoff = i + 1;
+                break;
+            }
+        }
+        float total = 0.0f;
+        for (int i = 0; i < cutoff; i++) total += cand_p[i];
+        const float r = a.draw * total;
+        float accum = 0.0f;
+        int pick = cutoff > 0 ? cand_i[cutoff - 1] : 0;
+        for (int i = 0; i < cutoff; i++) {
+            accum += cand_p[i];
+            if (accum >= r) {
+                pick = cand_i[i];
+                break;
+            }
+        }
+        *a.out = pick;
+        if (a.counts_update) a.counts_update[pick] += 1;
+        if (a.list) a.list[a.list_pos] = pick;
+    }
+}
+
+__global__ void count_tokens_kernel(const uint32_t *__restrict__ ids, int n_ids, int *__restrict__ counts, int vocab) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n_ids && ids[i] < (uint32_t)vocab) atomicAdd(&counts[ids[i]], 1);
+}
+
+__global__ void zero_ints_kernel(int *__restrict__ p, size_t n) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = 0;
+}
+
+}  // namespace
+
+namespace homura {
+
+int sample_check_config(hm_ctx *ctx, const hm_sampling_config *cfg, bool device) {
+    HM_REQUIRE(ctx, cfg != nullptr, "sampling: NULL configuration");
+    HM_REQUIRE(ctx, cfg->top_k >= 0 && cfg->top_p > 0.0f && cfg->min_p >= 0.0f && cfg->repetition_penalty > 0.0f,
+               "sampling: need top_k >= 0, top_p > 0, min_p >= 0, repetition_penalty > 0");
+    if (device && cfg->temperature > 0.0f)
+        HM_REQUIRE(ctx, cfg->top_k >= 1 && cfg->top_k <= SAMPLE_MAX_K,
+                   "sampling on the device needs 1 <= top_k <= %d (got %d); use the host sampler", SAMPLE_MAX_K, cfg->top_k);
+    return HM_OK;
+}
+
+// counts: device [vocab] occurrences (or nullptr); work: device [vocab] floats
+int sample_token_launch(hm_ctx *ctx, const float *d_logits, float *d_work, const int *d_counts, int vocab,
+                        const hm_sampling_config &cfg, float draw, int32_t *d_out, int *d_counts_update, int32_t *d_list,
+                        int list_pos) {
+    SampleArgs a;
+    a.logits = d_logits;
+    a.work = d_work;
+    a.counts = d_counts;
+    a.vocab = vocab;
+    a.cfg = cfg;
+    a.draw = draw;
+    a.out = d_out;
+    a.counts_update = d_counts_update;
+    a.list = d_list;
+    a.list_pos = list_pos;
+    hipLaunchKernelGGL(sample_token_kernel, dim3(1), dim3(SAMPLE_THREADS), 0, ctx->stream, a);
+    HM_LAUNCH_CHECK(ctx);
+    return HM_OK;
+}
+
+int zero_ints_launch(hm_ctx *ctx, int *d, size_t n) {
+    if (n == 0) return HM_OK;
+    hipLaunchKernelGGL(zero_ints_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, ctx->stream, d, n);
+    HM_LAUNCH_CHECK(ctx);
+    return HM_OK;
+}
+
+}  // namespace homura
+
+extern "C" {
+
+uint64_t hm_rng_seed(uint64_t seed) { return seed | 1u; }
+
+float hm_rng_next_f32(uint64_t *state) {
+    uint64_t s = *state;
+    s ^= s << 13;
+    s ^= s >> 7;
+    s ^= s << 17;
+    *state = s;
+    return (float)(s >> 40) / (float)(1ull << 24);
+}
+
+int hm_sample_token_host(const float *h_logits, int vocab, const hm_sampling_config *cfg, const uint32_t *h_generated,
+                         int n_generated, uint64_t *rng_state, int32_t *token_out) {
+    if (!h_logits || vocab <= 0 || !cfg || !rng_state || !token_out || n_generated < 0 || (n_generated && !h_generated))
+        return HM_ERR_INVALID;
+    std::vector<float> logits(h_logits, h_logits + vocab);
+    if (cfg->repetition_penalty != 1.0f)
+        for (int g = 0; g < n_generated; g++) {
+            const uint32_t idx = h_generated[g];
+            if (idx < (uint32_t)vocab) {
+                if (logits[idx] > 0.0f)
+                    logits[idx] /= cfg->repetition_penalty;
+                else
+                    logits[idx] *= cfg->repetition_penalty;
+            }
+        }
+    if (cfg->frequency_penalty != 0.0f || cfg->presence_penalty != 0.0f) {
+        std::vector<int> counts(vocab, 0);
+        for (int g = 0; g < n_generated; g++)
+            if (h_generated[g] < (uint32_t)vocab) counts[h_generated[g]]++;
+        for (int i = 0; i < vocab; i++)
+            if (counts[i]) {
+                logits[i] -= cfg->frequency_penalty * (float)counts[i];
+                logits[i] -= cfg->presence_penalty;
+            }
+    }
+    if (cfg->temperature <= 0.0f) {  // greedy: the last of equal maxima (Rust max_by)
+        int best = 0;
+        for (int i = 1; i < vocab; i++)
+            if (!(logits[best] > logits[i])) best = i;
+        *token_out = best;
+        return HM_OK;
+    }
+    const float inv_temp = 1.0f / cfg->temperature;
+    float max_logit = -INFINITY;
+    for (float &l : logits) {
+        l *= inv_temp;
+        max_logit = std::fmax(max_logit, l);
+    }
+    struct Cand {
+        int idx;
+        float p;
+    };
+    std::vector<Cand> c(vocab);
+    float sum = 0.0f;
+    for (int i = 0; i < vocab; i++) {
+        c[i] = Cand{i, std::exp(logits[i] - max_logit)};
+        sum += c[i].p;
+    }
+    for (Cand &x : c) x.p /= sum;
+    if (cfg->min_p > 0.0f) {
+        float max_prob = 0.0f;
+        for (const Cand &x : c) max_prob = std::fmax(max_prob, x.p);
+        const float threshold = cfg->min_p * max_prob;
+        for (Cand &x : c)
+            if (x.p < threshold) x.p = 0.0f;
+    }
+    // probability descending; the reference's sort_unstable_by leaves equal probabilities in an
+    // unspecified order, here they keep index order
+    std::sort(c.begin(), c.end(), [](const Cand &x, const Cand &y) { return x.p > y.p || (x.p == y.p && x.idx < y.idx); });
+    size_t len = c.size();
+    if (cfg->top_k > 0 && (size_t)cfg->top_k < len) len = (size_t)cfg->top_k;
+    float cumulative = 0.0f;
+    size_t cutoff = len;
+    for (size_t i = 0; i < len; i++) {
+        cumulative += c[i].p;
+        if (cumulative >= cfg->top_p) {
+            cutoff = i + 1;
+            break;
+        }
+    }
+    float total = 0.0f;
+    for (size_t i = 0; i < cutoff; i++) total += c[i].p;
+    const float r = hm_rng_next_f32(rng_state) * total;
+    float accum = 0.0f;
+    int pick = cutoff > 0 ? c[cutoff - 1].idx : 0;
+    for (size_t i = 0; i < cutoff; i++) {
+        accum += c[i].p;
+        if (accum >= r) {
+            pick = c[i].idx;
+            break;
+        }
+    }
+    *token_out = pick;
+    return HM_OK;
+}
+
+int hm_sample_token(hm_ctx *ctx, const float *d_logits, int vocab, const hm_sampling_config *cfg,
+                    const uint32_t *h_generated, int n_generated, uint64_t *rng_state, int32_t *token_out) {
+    HM_CHECK_CTX(ctx);
+    HM_REQUIRE(ctx, d_logits && vocab > 0 && rng_state && token_out && n_generated >= 0 && (!n_generated || h_generated),
+               "hm_sample_token: bad arguments");
+    int rc = homura::sample_check_config(ctx, cfg, true);
+    if (rc != HM_OK) return rc;
+    // workspace: work [vocab] f32 | counts [vocab] i32 | token i32 | generated ids
+    const size_t need = (size_t)vocab * 8 + 256 + (size_t)n_generated * 4;
+    HM_REQUIRE(ctx, need <= ctx->workspace_bytes, "hm_sample_token: vocabulary / history too large for the workspace");
+    float *work = (float *)ctx->workspace;
+    int *counts = (int *)(work + vocab);
+    int32_t *d_tok = (int32_t *)(counts + vocab);
+    uint32_t *d_gen = (uint32_t *)((char *)d_tok + 256);
+    const bool need_counts = n_generated > 0 && (cfg->repetition_penalty != 1.0f || cfg->frequency_penalty != 0.0f ||
+                                                 cfg->presence_penalty != 0.0f);
+    if (need_counts) {
+        if ((rc = homura::zero_ints_launch(ctx, counts, (size_t)vocab)) != HM_OK) return rc;
+        if ((rc = hm_upload(ctx, d_gen, h_generated, (size_t)n_generated * 4)) != HM_OK) return rc;
+        hipLaunchKernelGGL(count_tokens_kernel, dim3((unsigned)((n_generated + 255) / 256)), dim3(256), 0, ctx->stream,
+                           d_gen, n_generated, counts, vocab);
+        HM_LAUNCH_CHECK(ctx);
+    }
+    const float draw = cfg->temperature > 0.0f ? hm_rng_next_f32(rng_state) : 0.0f;  // greedy leaves the stream alone
+    rc = homura::sample_token_launch(ctx, d_logits, work, need_counts ? counts : nullptr, vocab, *cfg, draw, d_tok, nullptr,
+                                     nullptr, 0);
+    if (rc != HM_OK) return rc;
+    return hm_download(ctx, token_out, d_tok, 4);
+}
+
+}  // extern "C"

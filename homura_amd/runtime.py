@@ -188,6 +188,14 @@ class Context:
         self._check(self.lib.hm_gqa_prefill_attn(self.h, q.ptr, kc.ptr, vc.ptr, out.ptr, S, H, kvh, hd,
                                                  max_len, past, scale))
 
+    def sample_token(self, d_logits, vocab, cfg: "SamplingConfig", generated, rng: "Rng") -> int:
+        """reference sample_token on a logits row in HBM (top_k in 1..1024 when temperature > 0)."""
+        gen = np.ascontiguousarray(generated, np.uint32).reshape(-1)
+        c, tok = cfg.to_c(), C.c_int32()
+        self._check(self.lib.hm_sample_token(self.h, d_logits.ptr, vocab, C.byref(c), gen.ctypes.data if gen.size else None,
+                                             gen.size, C.byref(rng.state), C.byref(tok)))
+        return tok.value
+
     def kv_append(self, kc, vc, k, v, B, kvh, hd, max_len, pos, n_new):
         self._check(self.lib.hm_kv_append(self.h, kc.ptr, vc.ptr, k.ptr, v.ptr, B, kvh, hd,
                                           max_len, pos, n_new))
@@ -215,6 +223,44 @@ class Context:
 
     def argmax(self, values, n, out):
         self._check(self.lib.hm_argmax(self.h, values.ptr, n, out.ptr))
+
+
+@dataclass
+class SamplingConfig:
+    """reference SamplingConfig (src/generate.rs:646-686) with its defaults; temperature <= 0 is greedy."""
+    temperature: float = 0.7
+    top_k: int = 50
+    top_p: float = 0.9
+    min_p: float = 0.0
+    repetition_penalty: float = 1.1
+    frequency_penalty: float = 0.0
+    presence_penalty: float = 0.0
+
+    def to_c(self) -> _ffi.HmSamplingConfig:
+        return _ffi.HmSamplingConfig(self.temperature, self.top_k, self.top_p, self.min_p, self.repetition_penalty,
+                                     self.frequency_penalty, self.presence_penalty)
+
+
+class Rng:
+    """reference Rng (src/generate.rs:609-642): the state lives here, the arithmetic in the library."""
+
+    def __init__(self, seed: int):
+        self.state = C.c_uint64(_ffi.load().hm_rng_seed(seed))
+
+    def next_f32(self) -> float:
+        return float(_ffi.load().hm_rng_next_f32(C.byref(self.state)))
+
+
+def sample_token_host(logits, cfg: SamplingConfig, generated, rng: Rng) -> int:
+    """reference sample_token (src/generate.rs:698-801) on a host logits row."""
+    row = np.ascontiguousarray(logits, np.float32).reshape(-1)
+    gen = np.ascontiguousarray(generated, np.uint32).reshape(-1)
+    c, tok = cfg.to_c(), C.c_int32()
+    rc = _ffi.load().hm_sample_token_host(row.ctypes.data, row.size, C.byref(c), gen.ctypes.data if gen.size else None,
+                                          gen.size, C.byref(rng.state), C.byref(tok))
+    if rc != 0:
+        raise HomuraError(rc, "hm_sample_token_host: bad arguments")
+    return tok.value
 
 
 @dataclass
@@ -369,6 +415,16 @@ class HfModel:
     def set_prefill_min(self, n_tokens: int):
         """Inputs of at least n_tokens take the prefill pass in run_kv / generate_greedy (0 = never)."""
         self._check(self.lib.hm_model_set_prefill_min(self.h, n_tokens))
+
+    def generate(self, prompt_ids, max_new_tokens: int, cfg: "SamplingConfig", seed: int = 0, eos_token_id: int = -1):
+        """reference generate_streaming_core (src/generate.rs:100-315): sampled generation; returns the new ids."""
+        ids = np.ascontiguousarray(prompt_ids, dtype=np.int64).reshape(-1)
+        out = np.empty(max_new_tokens, dtype=np.int32)
+        c, n = cfg.to_c(), C.c_int()
+        self._check(self.lib.hm_model_generate(
+            self.h, ids.ctypes.data_as(C.POINTER(C.c_int64)), len(ids), max_new_tokens, C.byref(c), seed, eos_token_id,
+            out.ctypes.data_as(C.POINTER(C.c_int32)), C.byref(n)))
+        return out[:n.value].copy()
 
     def set_prefill_pieces(self, pieces: int):
         """bf16 numbers per f32 activation in the prefill pass: 3 (default, exact) or 2."""

@@ -198,6 +198,39 @@ int hm_embed(hm_ctx *ctx, const int64_t *d_ids, const float *d_table, float *d_o
  * the LAST (Rust Iterator::max_by). Writes one int32 to d_index_out. */
 int hm_argmax(hm_ctx *ctx, const float *d_values, int n, int32_t *d_index_out);
 
+/* ── sampling ─────────────────────────────────────────────────────────────────── */
+
+/* SamplingConfig (src/generate.rs:646-686) without the stop strings and the seed; the reference's
+ * defaults are temperature 0.7, top_k 50, top_p 0.9, min_p 0, repetition_penalty 1.1, others 0. */
+typedef struct hm_sampling_config {
+    float temperature; /* <= 0: greedy */
+    int top_k;         /* 0: no cut */
+    float top_p;
+    float min_p;
+    float repetition_penalty;
+    float frequency_penalty;
+    float presence_penalty;
+} hm_sampling_config;
+
+/* Rng (src/generate.rs:609-642): xorshift64 with shifts 13, 7, 17; the state is seed | 1; next_f32 is
+ * the top 24 bits over 2^24. Host functions, no context needed. */
+uint64_t hm_rng_seed(uint64_t seed);
+float hm_rng_next_f32(uint64_t *state);
+
+/* sample_token (src/generate.rs:698-801) on a host logits row, statement by statement: repetition penalty
+ * once per occurrence in generated_ids, frequency / presence penalties, greedy when temperature <= 0
+ * (last of equal maxima, the stream is not advanced), temperature, softmax with sequential f32 sums,
+ * min_p, sort by probability (equal probabilities keep index order; the reference's unstable sort leaves
+ * that open), top_k, top_p, one draw. No GPU involved. */
+int hm_sample_token_host(const float *h_logits, int vocab, const hm_sampling_config *cfg,
+                         const uint32_t *h_generated, int n_generated, uint64_t *rng_state, int32_t *token_out);
+/* The same procedure on a logits row in HBM (the row never crosses PCIe; 4 bytes come back). Needs
+ * 1 <= top_k <= 1024 when temperature > 0. The vocabulary-wide sum of exponentials is a tree sum, so
+ * the pick can differ from the host's only when the draw sits on a cumulative boundary to within the
+ * last bit of a probability. */
+int hm_sample_token(hm_ctx *ctx, const float *d_logits, int vocab, const hm_sampling_config *cfg,
+                    const uint32_t *h_generated, int n_generated, uint64_t *rng_state, int32_t *token_out);
+
 /* ── host-side mirror of Model / ExecutionPlan / KvCache, C view ─────────────
  * The C++ classes in homura_amd/csrc/host/ keep the reference's names (HfModel,
  * ExecutionPlan, KernelStep, KvCache, Buffer); these functions are their C handles. */
@@ -282,6 +315,17 @@ int hm_model_set_prefill_pieces(hm_model *m, int pieces);
  * round trip. h_tokens_out receives n_new ids. */
 int hm_model_generate_greedy(hm_model *m, const int64_t *h_prompt, int n_prompt, int n_new,
                              int32_t *h_tokens_out);
+
+/* The generation loop of generate_streaming_core (src/generate.rs:100-315) with the reference's sampler:
+ * the prompt goes through run_kv (the prompt pass for longer prompts), the first token is sampled from
+ * the last prompt position, then one decode step + one sample per token, each new token joining
+ * generated_ids for the penalties. Stops before max_new_tokens at eos_token_id (not stored; pass -1 for
+ * none) or when the KV cache is full. Logits stay in HBM and the pick is made there when
+ * 1 <= top_k <= 1024 or temperature <= 0; otherwise each logits row is sampled on the host.
+ * h_tokens_out holds max_new_tokens ids; *n_tokens_out receives how many were produced. */
+int hm_model_generate(hm_model *m, const int64_t *h_prompt, int n_prompt, int max_new_tokens,
+                      const hm_sampling_config *cfg, uint64_t seed, int eos_token_id, int32_t *h_tokens_out,
+                      int *n_tokens_out);
 
 /* Timed decode for benchmarking: runs `n_steps` decode steps starting from token `first_id`
  * (greedy feedback on device), returns total milliseconds measured with HIP events on the

@@ -36,6 +36,11 @@
  *                           one-hot score => that V row, fp64 brute force
  *   orc_kv_* .............. reference KvCache exact arrays
  *   orc_argmax_last ....... reference greedy vector + Rust max_by tie rule
+ *   orc_rng_* ............. xorshift64 stream recomputed with Python integers; determinism test
+ *   orc_sample_token ...... reference sample_token_greedy and min_p_filters_low_prob tests; top_k = 1 is
+ *                           the argmax; a 6-way distribution reproduced from 20 000 draws; an independent
+ *                           numpy restatement on random logits. The order among EQUAL probabilities is
+ *                           PARITY UNPINNED (the reference sorts with sort_unstable_by).
  *   orc_model_run_kv ...... composition of the above following the reference's step list;
  *                           end-to-end logits of a real checkpoint are PARITY UNPINNED
  *                           (the reference's golden files for that are not shipped).
@@ -618,6 +623,136 @@ ORC_API int orc_argmax_last(const float *v, int n) {
         if (!greater) best = i;
     }
     return best;
+}
+
+/* ───────────────────────── sampling ───────────────────────── */
+
+/* src/generate.rs:609-642 — xorshift64 (13, 7, 17); seed | 1; next_f32 = top 24 bits / 2^24. */
+ORC_API uint64_t orc_rng_seed(uint64_t seed) { return seed | 1u; }
+ORC_API float orc_rng_next_f32(uint64_t *state) {
+    uint64_t s = *state;
+    s ^= s << 13;
+    s ^= s >> 7;
+    s ^= s << 17;
+    *state = s;
+    return (float)(s >> 40) / (float)(1ull << 24);
+}
+
+/* SamplingConfig without the strings (src/generate.rs:646-686) */
+typedef struct {
+    float temperature;
+    int top_k;
+    float top_p, min_p, repetition_penalty, frequency_penalty, presence_penalty;
+} orc_sampling_config;
+
+typedef struct {
+    int idx;
+    float p;
+} orc_cand;
+
+/* descending probability; equal probabilities in index order (the reference uses sort_unstable_by,
+ * whose order among equals is unspecified) */
+static int cand_cmp(const void *a, const void *b) {
+    const orc_cand *x = (const orc_cand *)a, *y = (const orc_cand *)b;
+    if (x->p > y->p) return -1;
+    if (x->p < y->p) return 1;
+    return (x->idx > y->idx) - (x->idx < y->idx);
+}
+
+/* src/generate.rs:698-801 — sample_token: repetition penalty (once per occurrence in generated_ids),
+ * frequency / presence penalties, greedy when temperature <= 0, temperature, softmax (sequential f32
+ * sum), min_p, sort descending, top_k, top_p, draw r = next_f32 * total, first cumulative >= r.
+ * margins (optional, 2 floats): the smallest relative distance of r from a cumulative boundary, and of
+ * top_p from a cumulative value; a caller comparing against another float implementation skips draws
+ * that sit on a boundary. The RNG advances only on the sampling branch, as in the reference. */
+ORC_API int orc_sample_token(const float *logits_in, int n, const orc_sampling_config *cfg,
+                             const uint32_t *generated, int n_generated, uint64_t *rng_state, float *margins) {
+    float *logits = (float *)malloc((size_t)n * 4);
+    memcpy(logits, logits_in, (size_t)n * 4);
+    if (margins) margins[0] = margins[1] = INFINITY;
+    if (cfg->repetition_penalty != 1.0f) {
+        for (int g = 0; g < n_generated; g++) {
+            uint32_t idx = generated[g];
+            if (idx < (uint32_t)n) {
+                if (logits[idx] > 0.0f)
+                    logits[idx] /= cfg->repetition_penalty;
+                else
+                    logits[idx] *= cfg->repetition_penalty;
+            }
+        }
+    }
+    if (cfg->frequency_penalty != 0.0f || cfg->presence_penalty != 0.0f) {
+        int *counts = (int *)calloc((size_t)n, sizeof(int));
+        for (int g = 0; g < n_generated; g++)
+            if (generated[g] < (uint32_t)n) counts[generated[g]]++;
+        for (int i = 0; i < n; i++)
+            if (counts[i]) {
+                logits[i] -= cfg->frequency_penalty * (float)counts[i];
+                logits[i] -= cfg->presence_penalty;
+            }
+        free(counts);
+    }
+    if (cfg->temperature <= 0.0f) {
+        int best = orc_argmax_last(logits, n);
+        free(logits);
+        return best;
+    }
+    float inv_temp = 1.0f / cfg->temperature;
+    for (int i = 0; i < n; i++) logits[i] *= inv_temp;
+    float max_logit = -INFINITY;
+    for (int i = 0; i < n; i++) max_logit = fmaxf(max_logit, logits[i]); /* f32::max ignores NaN */
+    orc_cand *c = (orc_cand *)malloc((size_t)n * sizeof(orc_cand));
+    float sum = 0.0f;
+    for (int i = 0; i < n; i++) {
+        c[i].idx = i;
+        c[i].p = expf(logits[i] - max_logit);
+        sum += c[i].p;
+    }
+    for (int i = 0; i < n; i++) c[i].p /= sum;
+    if (cfg->min_p > 0.0f) {
+        float max_prob = 0.0f;
+        for (int i = 0; i < n; i++) max_prob = fmaxf(max_prob, c[i].p);
+        float threshold = cfg->min_p * max_prob;
+        for (int i = 0; i < n; i++)
+            if (c[i].p < threshold) c[i].p = 0.0f;
+    }
+    qsort(c, (size_t)n, sizeof(orc_cand), cand_cmp);
+    int len = n;
+    if (cfg->top_k > 0 && cfg->top_k < len) len = cfg->top_k;
+    float cumulative = 0.0f;
+    int cutoff = len;
+    for (int i = 0; i < len; i++) {
+        cumulative += c[i].p;
+        if (margins) {
+            float m = fabsf(cumulative - cfg->top_p) / cfg->top_p;
+            if (m < margins[1]) margins[1] = m;
+        }
+        if (cumulative >= cfg->top_p) {
+            cutoff = i + 1;
+            break;
+        }
+    }
+    float total = 0.0f;
+    for (int i = 0; i < cutoff; i++) total += c[i].p;
+    float r = orc_rng_next_f32(rng_state) * total;
+    float accum = 0.0f;
+    int pick = cutoff > 0 ? c[cutoff - 1].idx : 0;
+    int found = 0;
+    for (int i = 0; i < cutoff; i++) {
+        accum += c[i].p;
+        if (margins) {
+            float m = fabsf(accum - r) / total;
+            if (m < margins[0]) margins[0] = m;
+        }
+        if (!found && accum >= r) {
+            pick = c[i].idx;
+            found = 1;
+            if (!margins) break;
+        }
+    }
+    free(c);
+    free(logits);
+    return pick;
 }
 
 /* ───────────────────────── attention ───────────────────────── */

@@ -21,6 +21,16 @@ _I = C.c_int
 _F = C.c_float
 
 
+class OrcSamplingConfig(C.Structure):
+    """reference SamplingConfig (src/generate.rs:646-686) without the strings; defaults as there."""
+    _fields_ = [("temperature", C.c_float), ("top_k", C.c_int), ("top_p", C.c_float), ("min_p", C.c_float),
+                ("repetition_penalty", C.c_float), ("frequency_penalty", C.c_float), ("presence_penalty", C.c_float)]
+
+    def __init__(self, temperature=0.7, top_k=50, top_p=0.9, min_p=0.0, repetition_penalty=1.1,
+                 frequency_penalty=0.0, presence_penalty=0.0):
+        super().__init__(temperature, top_k, top_p, min_p, repetition_penalty, frequency_penalty, presence_penalty)
+
+
 class OrcConfig(C.Structure):
     _fields_ = [("hidden", _I), ("inter", _I), ("heads", _I), ("kv_heads", _I),
                 ("head_dim", _I), ("layers", _I), ("vocab", _I), ("eps", _F),
@@ -96,6 +106,9 @@ def load() -> C.CDLL:
         "orc_model_run_kv": (_I, [_P, _P, _I, _P]),
         "orc_generate_greedy": (_I, [_P, _P, _I, _I, _P, _P]),
         "orc_num_threads": (_I, []),
+        "orc_rng_seed": (C.c_uint64, [C.c_uint64]),
+        "orc_rng_next_f32": (C.c_float, [C.POINTER(C.c_uint64)]),
+        "orc_sample_token": (_I, [_P, _I, C.POINTER(OrcSamplingConfig), _P, _I, C.POINTER(C.c_uint64), _P]),
     }
     for name, (res, args) in sig.items():
         fn = getattr(lib, name)
@@ -263,6 +276,27 @@ def embed(ids, table):
     out = np.empty((ids.size, table.shape[1]), np.float32)
     load().orc_embed(_p(ids), ids.size, _p(table), table.shape[1], _p(out))
     return out
+
+
+class Rng:
+    """The reference's seedable xorshift64 (src/generate.rs:609-642)."""
+
+    def __init__(self, seed: int):
+        self.state = C.c_uint64(load().orc_rng_seed(seed))
+
+    def next_f32(self) -> float:
+        return float(load().orc_rng_next_f32(C.byref(self.state)))
+
+
+def sample_token(logits, cfg: "OrcSamplingConfig", generated, rng: Rng, want_margins=False):
+    """reference sample_token (src/generate.rs:698-801). Returns the token, or (token, (draw margin,
+    top_p margin)) with want_margins."""
+    logits = _f32(logits).reshape(-1)
+    gen = np.ascontiguousarray(generated, np.uint32).reshape(-1)
+    m = np.empty(2, np.float32)
+    tok = load().orc_sample_token(_p(logits), logits.size, C.byref(cfg), _p(gen) if gen.size else None, gen.size,
+                                  C.byref(rng.state), _p(m) if want_margins else None)
+    return (tok, (float(m[0]), float(m[1]))) if want_margins else tok
 
 
 def argmax_last(v):

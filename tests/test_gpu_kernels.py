@@ -466,7 +466,15 @@ def test_bad_arguments_are_errors_not_faults(ctx):
     with pytest.raises(HomuraError):
         ctx.gemv_bf16(d, d, d, 9, 8, 8)           # M out of range
     with pytest.raises(HomuraError):
-        ctx.gemm_bf16(d, d, d, 100, 32, 128)      # M not a multiple of 128
+        ctx.gemm_bf16(d, d, d, 128, 40, 128)      # K not a multiple of 32
+    with pytest.raises(HomuraError):
+        ctx.gemm_bf16(d, d, d, 128, 32, 100)      # [K,N] operand with N not a multiple of 8
+    with pytest.raises(HomuraError):
+        ctx.gqa_prefill_attn(d, d, d, d, 4, 4, 2, 128, 16, 14, 1.0)   # past + S > max_len
+    with pytest.raises(HomuraError):
+        ctx.gqa_prefill_attn(d, d, d, d, 4, 4, 2, 96, 16, 0, 1.0)     # head_dim 96
+    with pytest.raises(HomuraError):
+        ctx.gemv_q4_k(d, d, d, 1, 128, 4)         # K not a multiple of 256
     with pytest.raises(HomuraError):
         ctx.gqa_decode_attn(d, d, d, d, 1, 6, 4, 128, 16, 4, 1.0)  # heads not divisible
     with pytest.raises(HomuraError):

@@ -1,0 +1,136 @@
+"""The reference's sampler (src/generate.rs:698-801) on logits that stay in HBM, against the oracle: the
+same token for the same xorshift64 stream. The device sums the exponentials as a tree and uses its own
+expf, so a probability can differ from the oracle's in the last bits; draws that the oracle reports within
+1e-4 (relative) of a cumulative boundary are not compared."""
+import numpy as np
+import pytest
+
+import model_fixture as mf
+import pyoracle
+from pyoracle import OrcSamplingConfig as Cfg
+from homura_amd import HomuraError, runtime, synth, synth_model
+
+pytestmark = pytest.mark.gpu
+EDGE = 1e-4
+
+
+def on_edge(margins, cfg, edge=EDGE):
+    """margins = (draw vs cumulative boundary, top_p vs cumulative value), both relative. With top_p >= 1 the
+    cut can only drop a tail whose mass is a rounding error of the total, which moves the draw by as much:
+    covered by the draw margin."""
+    return margins[0] < edge or (cfg.top_p < 1.0 and margins[1] < edge)
+
+
+def say(msg):
+    print(f"[sampling] {msg}", flush=True)
+
+
+def lib_cfg(c):
+    return runtime.SamplingConfig(c.temperature, c.top_k, c.top_p, c.min_p, c.repetition_penalty, c.frequency_penalty,
+                                  c.presence_penalty)
+
+
+CONFIGS = {
+    "reference defaults": Cfg(),
+    "greedy with penalties": Cfg(temperature=0.0, repetition_penalty=1.3, frequency_penalty=0.4, presence_penalty=0.2),
+    "top_k 1": Cfg(temperature=1.5, top_k=1, top_p=1.0, repetition_penalty=1.0),
+    "top_k 1024, top_p 1": Cfg(temperature=1.2, top_k=1024, top_p=1.0, repetition_penalty=1.0),
+    "min_p and penalties": Cfg(temperature=0.6, top_k=300, top_p=0.97, min_p=0.02, repetition_penalty=1.2,
+                               frequency_penalty=0.3, presence_penalty=0.1),
+}
+
+
+@pytest.mark.parametrize("name", list(CONFIGS))
+@pytest.mark.parametrize("vocab", [151936, 1000, 50])
+def test_device_sampler_against_oracle(ctx, name, vocab):
+    cfg = CONFIGS[name]
+    gen = np.random.default_rng(vocab + len(name))
+    compared = skipped = 0
+    for trial in range(12):
+        logits = (gen.standard_normal(vocab) * 2.5).astype(np.float32)
+        if trial % 3 == 0:                       # equal logits: equal probabilities must order by index
+            logits[gen.integers(0, vocab, 4)] = np.float32(logits.max())
+        generated = gen.integers(0, vocab, size=[0, 5, 40][trial % 3]).tolist()
+        if generated:
+            generated += generated[:2]           # repeats: the repetition penalty compounds
+        d = ctx.to_device(logits)
+        seed = 900 + trial
+        a, b = pyoracle.Rng(seed), runtime.Rng(seed)
+        for _ in range(3):
+            want, margins = pyoracle.sample_token(logits, cfg, generated, a, want_margins=True)
+            got = ctx.sample_token(d, vocab, lib_cfg(cfg), generated, b)
+            assert a.state.value == b.state.value
+            if on_edge(margins, cfg):
+                skipped += 1
+                continue
+            assert got == want, (name, vocab, trial)
+            compared += 1
+        d.free()
+    say(f"{name}, vocab {vocab}: {compared} draws identical, {skipped} on a boundary")
+    assert compared >= 24
+
+
+def test_device_sampler_reference_cases_and_errors(ctx):
+    # sample_token_greedy and min_p_filters_low_prob (src/generate.rs:891-900, :990-1008)
+    d = ctx.to_device(np.array([0.0, 1.0, 0.5, 0.2], np.float32))
+    assert ctx.sample_token(d, 4, runtime.SamplingConfig(temperature=0.0), [], runtime.Rng(1)) == 1
+    d2 = ctx.to_device(np.array([10.0, 0.0, 0.0, 0.0], np.float32))
+    cfg = runtime.SamplingConfig(temperature=1.0, min_p=0.5, top_k=4, top_p=1.0, repetition_penalty=1.0)
+    rng = runtime.Rng(42)
+    assert [ctx.sample_token(d2, 4, cfg, [], rng) for _ in range(10)] == [0] * 10
+    # last of equal maxima
+    d3 = ctx.to_device(np.array([1.0, 3.0, 3.0, 2.0], np.float32))
+    assert ctx.sample_token(d3, 4, runtime.SamplingConfig(temperature=0.0, repetition_penalty=1.0), [], runtime.Rng(1)) == 2
+    with pytest.raises(HomuraError, match="top_k"):
+        ctx.sample_token(d, 4, runtime.SamplingConfig(top_k=0), [], runtime.Rng(1))
+    with pytest.raises(HomuraError, match="top_k"):
+        ctx.sample_token(d, 4, runtime.SamplingConfig(top_k=5000), [], runtime.Rng(1))
+
+
+MODEL_CONFIGS = {
+    "reference defaults": Cfg(),
+    # min_p removes the long tail, where cumulative boundaries are closer together than the logits agree
+    "min_p and penalties": Cfg(temperature=0.8, top_k=40, top_p=0.95, min_p=0.05, repetition_penalty=1.2,
+                               frequency_penalty=0.3, presence_penalty=0.1),
+    "host path: no top_k": Cfg(temperature=0.9, top_k=0, top_p=0.9, min_p=0.6, repetition_penalty=1.15),
+}
+
+
+@pytest.mark.parametrize("name", list(MODEL_CONFIGS))
+def test_model_generate_against_oracle_loop(ctx, name):
+    """hm_model_generate against the reference's loop written with the oracle's pieces
+    (generate_streaming_core, src/generate.rs:100-315): prompt through run_kv, first token from the last
+    prompt position, then decode step + sample_token with the growing generated_ids, stop at EOS."""
+    cfg = MODEL_CONFIGS[name]
+    mcfg = synth_model.TINY
+    weights = synth_model.synth_weights(mcfg, 321)
+    gm = synth_model.build_model(ctx, mcfg, weights, 160)
+    om = mf.build_oracle_model(mcfg, weights, 160)
+    prompt = synth.token_ids(12, 20, mcfg.vocab_size)
+    agree = 0
+    for seed in (1, 2, 3):
+        gm.reset_kv_cache()
+        om.kv.reset(0)
+        rng = pyoracle.Rng(seed)
+        om.run_kv(prompt[:-1])
+        cur, want, edge_at = int(prompt[-1]), [], None
+        for step in range(40):
+            logits = om.run_kv([cur])[0]
+            tok, margins = pyoracle.sample_token(logits, cfg, want, rng, want_margins=True)
+            if edge_at is None and on_edge(margins, cfg, 3 * EDGE):   # GPU logits differ by ~3e-5 of their scale: keep clear of boundaries
+                edge_at = step
+            want.append(tok)
+            cur = tok
+        got = gm.generate(prompt, 40, lib_cfg(cfg), seed=seed)
+        upto = 40 if edge_at is None else edge_at
+        assert list(got[:upto]) == want[:upto], (name, seed, upto)
+        assert len(got) == 40 and gm.kv_cache_len() == 19 + 40
+        agree += upto
+        # EOS: declare the 6th generated token the end-of-sequence id
+        if upto > 6 and want[5] not in want[:5]:
+            gm.reset_kv_cache()
+            got_eos = gm.generate(prompt, 40, lib_cfg(cfg), seed=seed, eos_token_id=want[5])
+            assert list(got_eos) == want[:5]
+    say(f"{name}: {agree} of 120 generated tokens compared, all identical")
+    assert agree >= 30
+    gm.close()
