@@ -76,6 +76,7 @@ def main() -> int:
     ap.add_argument("--kernel-max-launches", type=int, default=0,
                     help="cap on kernel launches per stand-alone measurement graph (0 = the whole weight ring)")
     ap.add_argument("--no-prefill", action="store_true", help="skip the prompt-pass measurement")
+    ap.add_argument("--no-quantised", action="store_true", help="skip the decode measurements with quantised projections")
     ap.add_argument("--no-kernel-configs", action="store_true",
                     help="skip the stand-alone kernel measurements (BASELINE configurations 1, 3, 4, 5)")
     args = ap.parse_args()
@@ -197,6 +198,30 @@ def main() -> int:
         launches = model.launches_per_step()
         device = ctx.device_name()
         model.close()
+        # The same decode with GGUF-quantised projections (untied f32 LM head, as the reference's quantised
+        # plan keeps it): Q8_0, Q4_0 and a Q4_K_M-style mix of Q4_K and Q6_K. Reported beside `value`.
+        quantised = None
+        if not args.no_quantised:
+            import dataclasses
+            from homura_amd.runtime import DTYPE_Q4_0, DTYPE_Q8_0
+            qcfg = dataclasses.replace(cfg, tie_word_embeddings=False)
+            quantised = {"unit": "tok/s", "steps": args.steps,
+                         "what": "same shape, cache and step count; raw GGUF blocks dequantised in registers "
+                                 "(K-quants: Q8_K activations, integer dots), f32 LM head"}
+            for name, wdt, mix in (("q8_0", DTYPE_Q8_0, None), ("q4_0", DTYPE_Q4_0, None),
+                                   ("q4_k_m_mix", None, synth_model.q4_k_m_mix(qcfg))):
+                qw = synth_model.synth_weights(qcfg, seed + 7, wdt if mix is None else DTYPE_Q8_0, has_qk_norm=True,
+                                               proj_dtypes=mix)
+                qm = synth_model.build_model(ctx, qcfg, qw, 2048, wdt if mix is None else DTYPE_Q8_0, has_qk_norm=True,
+                                             proj_dtypes=mix)
+                qm.init_kv_cache(kv, PREFILL)
+                qm.set_graph(not args.no_graph)
+                qm.bench_decode(int(prompt[0]), max(args.warmup, 2))
+                q_ms, _ = qm.bench_decode(int(prompt[1]), args.steps)
+                quantised[name] = {"value": round(args.steps * 1e3 / q_ms, 1), "ms_per_step": round(q_ms / args.steps, 4),
+                                   "kernel_launches_per_step": qm.launches_per_step()}
+                qm.close()
+                del qw
         kernel_configs = None
         if not args.no_kernel_configs:
             from homura_amd import kernel_bench
@@ -237,6 +262,7 @@ def main() -> int:
         "cpu_baseline": cpu_baseline,
         "pcie_inclusive": pcie_inclusive,
         "prefill": prefill,
+        "quantised_decode": quantised,
         "event_ms_per_step": round(event_ms / args.steps, 4),
         "kernels": kernels,
         "kernel_configs": kernel_configs,

@@ -4,9 +4,17 @@
 
 #include <cstdint>
 
+#include "gemv_quant.h"
 #include "hm_common.h"
 
 namespace homura {
+
+// Fused form for the model plan: the light ops in front of the product (QuantFuse: SiLU pair, residual
+// add, RMSNorm) and the Q8_K quantisation of the resulting row all happen inside the GEMV kernel - every
+// workgroup redoes them for the one row, which is cheaper than the launches they replace - and the
+// residual add behind it rides on the way out. K <= 4096.
+int gemv_kquant_fused(hm_ctx *ctx, bool q6, const float *d_x, const uint8_t *d_w, float *d_out, int K, int N,
+                      const QuantFuse &fuse);
 
 // out[N] = W[N][K] (Q4_K when q6 is false, Q6_K when true) · x[K], x quantised to Q8_K first.
 // reuse_activation: skip the quantisation and multiply against what the previous call on this

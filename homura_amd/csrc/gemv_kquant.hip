@@ -150,7 +150,7 @@ __device__ __forceinline__ StepRange step_range(int step, int rows_per_step, int
 // lane + 64 t of the row: block (lane + 64 t) / 16 = lane/16 + 4 t, unit-in-block lane % 16.
 template <int QT, int CPL, int RT>
 __device__ __forceinline__ void krows_trip(const uint8_t *base, size_t rowbytes, int lr, int lane, int nu,
-                                           const ActUnit (&act)[CPL], float *out) {
+                                           const ActUnit (&act)[CPL], float *out, const float *add) {
     constexpr int BB = KTraits<QT>::BYTES;
     const int boff = (lane >> 4) * BB, ui = lane & 15;
     float a[RT];
@@ -171,7 +171,81 @@ __device__ __forceinline__ void krows_trip(const uint8_t *base, size_t rowbytes,
 #pragma unroll
     for (int j = 0; j < RT; j++) {
         a[j] = wave_sum(a[j]);
-        if (lane == 0) out[lr + j * KWAVES] = a[j];
+        if (lane == 0) out[lr + j * KWAVES] = add ? a[j] + add[lr + j * KWAVES] : a[j];
+    }
+}
+
+// The activation row of a fused launch, prepared by the whole workgroup into LDS: light ops (SiLU pair /
+// residual add / RMSNorm, arithmetic as in the stand-alone kernels), then the Q8_K quantisation with the
+// arithmetic of quantize_q8_k_kernel. Thread t holds elements 4 (t + 256 u) .. +3 of round u, so each
+// wavefront owns whole 256-wide blocks: amax is a wave reduction, a sum of 16 a quad reduction.
+constexpr int KXU = 4;  // rounds of 1024 elements: K <= 4096
+__device__ __forceinline__ void stage_activation(const float *__restrict__ x, const homura::QuantFuse &fuse, int K,
+                                                 int8_t *q8, float *act_d, int *bsums, float *red) {
+    const int tid = threadIdx.x, lane = tid & (WAVE - 1), wave = tid / WAVE;
+    const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
+    f32x4 xr[KXU], ar[KXU], nr[KXU];
+    const float *second = fuse.x2 ? fuse.x2 : fuse.res_in;
+#pragma unroll
+    for (int u = 0; u < KXU; u++) {
+        const int k = (tid + u * KTHREADS) * 4;
+        xr[u] = k < K ? *reinterpret_cast<const f32x4 *>(x + k) : zero4;
+        ar[u] = second && k < K ? *reinterpret_cast<const f32x4 *>(second + k) : zero4;
+        nr[u] = fuse.norm_w && k < K ? *reinterpret_cast<const f32x4 *>(fuse.norm_w + k) : zero4;
+    }
+    if (fuse.x2) {
+#pragma unroll
+        for (int u = 0; u < KXU; u++)
+#pragma unroll
+            for (int e = 0; e < 4; e++) xr[u][e] = (xr[u][e] / (1.0f + expf(-xr[u][e]))) * ar[u][e];
+    } else if (fuse.res_in) {
+#pragma unroll
+        for (int u = 0; u < KXU; u++) {
+            xr[u] += ar[u];
+            const int k = (tid + u * KTHREADS) * 4;
+            if (fuse.resid_out && blockIdx.x == 0 && k < K) *reinterpret_cast<f32x4 *>(fuse.resid_out + k) = xr[u];
+        }
+    }
+    if (fuse.norm_w) {
+        float ss = 0.f;
+#pragma unroll
+        for (int u = 0; u < KXU; u++) ss += (xr[u][0] * xr[u][0] + xr[u][1] * xr[u][1]) + (xr[u][2] * xr[u][2] + xr[u][3] * xr[u][3]);
+        ss = wave_sum(ss);
+        if (lane == 0) red[wave] = ss;
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");  // LDS only: the weight loads stay in flight
+        float tot = 0.f;
+#pragma unroll
+        for (int wv = 0; wv < KWAVES; wv++) tot += red[wv];
+        const float inv = 1.0f / sqrtf(tot / (float)K + fuse.eps);
+#pragma unroll
+        for (int u = 0; u < KXU; u++)
+#pragma unroll
+            for (int e = 0; e < 4; e++) xr[u][e] = (xr[u][e] * inv) * nr[u][e];
+    }
+#pragma unroll
+    for (int u = 0; u < KXU; u++) {
+        const int k = (tid + u * KTHREADS) * 4;  // block k / 256 = wave + 4 u belongs to this wavefront alone
+        if (u * KTHREADS * 4 >= K) break;        // uniform
+        float amax = fmaxf(fmaxf(fabsf(xr[u][0]), fabsf(xr[u][1])), fmaxf(fabsf(xr[u][2]), fabsf(xr[u][3])));
+        amax = wave_max(amax);
+        const float iscale = amax == 0.f ? 0.f : __fdiv_rn(127.0f, amax);
+        int q[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            float r = rintf(__fmul_rn(xr[u][i], iscale));  // round half to even
+            r = fminf(r, 127.0f);
+            r = fmaxf(r, -127.0f);
+            q[i] = (int)r;
+        }
+        int s = q[0] + q[1] + q[2] + q[3];
+        s += __builtin_amdgcn_update_dpp(0, s, 0xB1, 0xF, 0xF, false);  // quad_perm [1,0,3,2]
+        s += __builtin_amdgcn_update_dpp(0, s, 0x4E, 0xF, 0xF, false);  // quad_perm [2,3,0,1]
+        if (k < K) {
+            *reinterpret_cast<uint32_t *>(q8 + k) = (uint32_t)(q[0] & 0xFF) | ((uint32_t)(q[1] & 0xFF) << 8) |
+                                                    ((uint32_t)(q[2] & 0xFF) << 16) | ((uint32_t)(q[3] & 0xFF) << 24);
+            if ((lane & 3) == 0) bsums[k >> 4] = s;
+            if (lane == 0) act_d[k >> 8] = __fdiv_rn(amax, 127.0f);
+        }
     }
 }
 
@@ -180,7 +254,8 @@ __global__ __launch_bounds__(KTHREADS) void gemv_kquant_kernel(const int8_t *__r
                                                                const float *__restrict__ act_d,
                                                                const int *__restrict__ bsums,
                                                                const uint8_t *__restrict__ w, float *__restrict__ out,
-                                                               int K, int N, int rows_per_step) {
+                                                               int K, int N, int rows_per_step, const float *x_f32,
+                                                               const homura::QuantFuse fuse, int act_lds_off) {
     constexpr int BB = KTraits<QT>::BYTES;
     constexpr int U = KSTAGE_U;
     extern __shared__ __attribute__((aligned(16))) uint8_t ws[];
@@ -189,7 +264,27 @@ __global__ __launch_bounds__(KTHREADS) void gemv_kquant_kernel(const int8_t *__r
     const size_t rowbytes = (size_t)nb * BB;
     const int nsteps = (N + rows_per_step - 1) / rows_per_step;
 
-    // the lane's share of the quantised activation first (small, cached), the first row step behind it
+    // the first row step is requested before anything else waits
+    u32x4 tmp[U];
+    int step = blockIdx.x;
+    StepRange cur = step_range(step, rows_per_step, N, rowbytes);
+    if (x_f32) {  // fused launch: the f32 row is prepared and quantised here, into LDS behind the row stage
+        int8_t *lq8 = reinterpret_cast<int8_t *>(ws + act_lds_off);
+        float *ld = reinterpret_cast<float *>(lq8 + K);
+        int *lbs = reinterpret_cast<int *>(ld + nb);
+        float *red = reinterpret_cast<float *>(lbs + nu);
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const int i = tid + u * KTHREADS;
+            tmp[u] = i < cur.nchunks ? ld128_stream(w + cur.abeg + (size_t)i * 16) : u32x4{0u, 0u, 0u, 0u};
+        }
+        stage_activation(x_f32, fuse, K, lq8, ld, lbs, red);
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        q8 = lq8;
+        act_d = ld;
+        bsums = lbs;
+    }
+    // the lane's share of the quantised activation (small, cached)
     ActUnit act[CPL];
 #pragma unroll
     for (int t = 0; t < CPL; t++) {
@@ -199,13 +294,12 @@ __global__ __launch_bounds__(KTHREADS) void gemv_kquant_kernel(const int8_t *__r
         act[t].bsum = bsums[u];
         act[t].d = act_d[u >> 4];
     }
-    u32x4 tmp[U];
-    int step = blockIdx.x;
-    StepRange cur = step_range(step, rows_per_step, N, rowbytes);
+    if (!x_f32) {
 #pragma unroll
-    for (int u = 0; u < U; u++) {
-        const int i = tid + u * KTHREADS;
-        tmp[u] = i < cur.nchunks ? ld128_stream(w + cur.abeg + (size_t)i * 16) : u32x4{0u, 0u, 0u, 0u};
+        for (int u = 0; u < U; u++) {
+            const int i = tid + u * KTHREADS;
+            tmp[u] = i < cur.nchunks ? ld128_stream(w + cur.abeg + (size_t)i * 16) : u32x4{0u, 0u, 0u, 0u};
+        }
     }
 
     for (; step < nsteps; step += gridDim.x) {
@@ -227,13 +321,14 @@ __global__ __launch_bounds__(KTHREADS) void gemv_kquant_kernel(const int8_t *__r
         }
         const uint8_t *base = ws + now.shift;
         float *o = out + now.r0;
+        const float *add = fuse.res_out_add ? fuse.res_out_add + now.r0 : nullptr;
         int lr = wave;
-        for (; lr + 3 * KWAVES < now.nrows; lr += 4 * KWAVES) krows_trip<QT, CPL, 4>(base, rowbytes, lr, lane, nu, act, o);
+        for (; lr + 3 * KWAVES < now.nrows; lr += 4 * KWAVES) krows_trip<QT, CPL, 4>(base, rowbytes, lr, lane, nu, act, o, add);
         if (lr + KWAVES < now.nrows) {
-            krows_trip<QT, CPL, 2>(base, rowbytes, lr, lane, nu, act, o);
+            krows_trip<QT, CPL, 2>(base, rowbytes, lr, lane, nu, act, o, add);
             lr += 2 * KWAVES;
         }
-        if (lr < now.nrows) krows_trip<QT, CPL, 1>(base, rowbytes, lr, lane, nu, act, o);
+        if (lr < now.nrows) krows_trip<QT, CPL, 1>(base, rowbytes, lr, lane, nu, act, o, add);
     }
 }
 
@@ -286,7 +381,7 @@ int quantize_launch(hm_ctx *ctx, const float *d_x, int8_t *q8, float *act_d, int
 
 template <int QT>
 int gemv_kquant_launch(hm_ctx *ctx, const char *name, const float *d_x, const uint8_t *d_w, float *d_out, int M, int K,
-                       int N, bool reuse_activation = false) {
+                       int N, bool reuse_activation = false, const homura::QuantFuse *fuse = nullptr) {
     HM_CHECK_CTX(ctx);
     constexpr int BB = KTraits<QT>::BYTES;
     HM_REQUIRE(ctx, d_x && d_w && d_out, "%s: NULL pointer", name);
@@ -296,6 +391,12 @@ int gemv_kquant_launch(hm_ctx *ctx, const char *name, const float *d_x, const ui
     HM_REQUIRE(ctx, ((uintptr_t)d_w % 16) == 0 && ((uintptr_t)d_x % 16) == 0, "%s: weight and activation buffers must be 16-byte aligned", name);
     const size_t rowbytes = (size_t)(K / 256) * BB;
     HM_REQUIRE(ctx, KWAVES * rowbytes + 32 <= (size_t)KSTAGE_BYTES, "%s: K=%d too large for the LDS stage", name, K);
+    if (fuse) {
+        HM_REQUIRE(ctx, M == 1 && K <= KXU * KTHREADS * 4, "%s: the fused form takes one row of at most %d", name, KXU * KTHREADS * 4);
+        HM_REQUIRE(ctx, !(fuse->x2 && fuse->res_in), "%s: SiLU pair and residual input exclude each other", name);
+        HM_REQUIRE(ctx, ((uintptr_t)fuse->x2 % 16) == 0 && ((uintptr_t)fuse->res_in % 16) == 0 && ((uintptr_t)fuse->resid_out % 16) == 0 &&
+                            ((uintptr_t)fuse->norm_w % 16) == 0, "%s: fused operands must be 16-byte aligned", name);
+    }
     // the quantised activation lives at the top of the workspace: q8 | act_d | bsums per activation row
     const size_t per_m = ((size_t)K + (size_t)K / 256 * 4 + (size_t)K / 16 * 4 + 255) & ~(size_t)255;
     HM_REQUIRE(ctx, per_m * M <= ctx->workspace_bytes, "%s: workspace too small", name);
@@ -307,7 +408,9 @@ int gemv_kquant_launch(hm_ctx *ctx, const char *name, const float *d_x, const ui
     if (rows > KMAX_ROWS) rows = KMAX_ROWS;
     while (rows > KWAVES && (size_t)rows * rowbytes + 32 > (size_t)KSTAGE_BYTES) rows -= KWAVES;
     while (rows > KWAVES && (N + rows - 1) / rows < 2 * ctx->num_cus) rows -= KWAVES;
-    const size_t lds = (size_t)rows * rowbytes + 32 + 16;
+    // fused launches keep the quantised row in LDS behind the row stage: q8 | act_d | bsums | 4 floats
+    const size_t stage_bytes = ((size_t)rows * rowbytes + 32 + 16 + 15) & ~(size_t)15;
+    const size_t lds = fuse ? stage_bytes + (size_t)K + (size_t)(K / 256) * 4 + (size_t)(K / 16) * 4 + 16 : stage_bytes;
     const int nsteps = (N + rows - 1) / rows;
     int wg_per_cu = (int)(120 * 1024 / lds);
     if (wg_per_cu < 1) wg_per_cu = 1;
@@ -318,14 +421,16 @@ int gemv_kquant_launch(hm_ctx *ctx, const char *name, const float *d_x, const ui
         int8_t *q8 = (int8_t *)(wsp + per_m * m);
         float *act_d = (float *)(q8 + K);
         int *bsums = (int *)(act_d + K / 256);
-        if (!reuse_activation) {
+        if (!reuse_activation && !fuse) {
             int rc = quantize_launch(ctx, d_x + (size_t)m * K, q8, act_d, bsums, 1, K);
             if (rc != HM_OK) return rc;
         }
         float *om = d_out + (size_t)m * N;
+        const float *xf = fuse ? d_x : nullptr;
+        const homura::QuantFuse fz = fuse ? *fuse : homura::QuantFuse();
 #define HM_KQ_CASE(C)                                                                                              \
     hipLaunchKernelGGL((gemv_kquant_kernel<QT, C>), dim3(grid), dim3(KTHREADS), lds, ctx->stream, q8, act_d, bsums, \
-                       d_w, om, K, N, rows)
+                       d_w, om, K, N, rows, xf, fz, (int)stage_bytes)
         switch (cpl) {
             case 1: HM_KQ_CASE(1); break;
             case 2: HM_KQ_CASE(2); break;
@@ -356,6 +461,12 @@ int dequant_kquant_launch(hm_ctx *ctx, const char *name, const uint8_t *d_blocks
 }
 
 }  // namespace
+
+int homura::gemv_kquant_fused(hm_ctx *ctx, bool q6, const float *d_x, const uint8_t *d_w, float *d_out, int K, int N,
+                              const QuantFuse &fuse) {
+    return q6 ? gemv_kquant_launch<1>(ctx, "gemv_kquant[q6_k]", d_x, d_w, d_out, 1, K, N, false, &fuse)
+              : gemv_kquant_launch<0>(ctx, "gemv_kquant[q4_k]", d_x, d_w, d_out, 1, K, N, false, &fuse);
+}
 
 int homura::gemv_kquant(hm_ctx *ctx, bool q6, const float *d_x, const uint8_t *d_w, float *d_out, int K, int N,
                         bool reuse_activation) {

@@ -13,6 +13,7 @@
 // their sum, in registers for the life of the workgroup and walks the staged rows. Quants are
 // used as stored (biased unsigned): sum_j q_j x_j - offset * sum_j x_j, four byte->float
 // conversions per 32-bit word with no shifts for the byte lanes.
+#include "gemv_quant.h"
 #include "hm_common.h"
 
 namespace {
@@ -110,7 +111,8 @@ __device__ __forceinline__ StepRange step_range(int step, int rows_per_step, int
 // allocation carries slack for it) and their value is dropped by a select.
 template <int QT, int NXV, int RT>
 __device__ __forceinline__ void rows_trip(const uint8_t *base, size_t rowbytes, int lr, int lane, int nq,
-                                          const float (&xv)[NXV][8], const float (&sxo)[NXV], float *out) {
+                                          const float (&xv)[NXV][8], const float (&sxo)[NXV], float *out,
+                                          const float *add) {
     constexpr int BB = BlockTraits<QT>::BYTES;
     const int doff = (lane >> 2) * BB;
     const int qoff = doff + 2 + (lane & 3) * BlockTraits<QT>::QUARTER;
@@ -134,7 +136,7 @@ __device__ __forceinline__ void rows_trip(const uint8_t *base, size_t rowbytes, 
 #pragma unroll
     for (int j = 0; j < RT; j++) {
         a[j] = wave_sum(a[j]);
-        if (lane == 0) out[lr + j * QWAVES] = a[j];
+        if (lane == 0) out[lr + j * QWAVES] = add ? a[j] + add[lr + j * QWAVES] : a[j];
     }
 }
 
@@ -142,7 +144,7 @@ __device__ __forceinline__ void rows_trip(const uint8_t *base, size_t rowbytes, 
 template <int QT, int CPL>
 __global__ __launch_bounds__(QTHREADS) void gemv_quant_kernel(
     const float *__restrict__ x, const uint8_t *__restrict__ w, float *__restrict__ out, int K,
-    int N, int rows_per_step) {
+    int N, int rows_per_step, const homura::QuantFuse fuse) {
     constexpr int BB = BlockTraits<QT>::BYTES;
     constexpr int U = STAGE_U;
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -159,11 +161,15 @@ __global__ __launch_bounds__(QTHREADS) void gemv_quant_kernel(
     // Loads return in issue order: the (small, cached) activation loads go first, the first step's
     // weights right behind them, so staging the activations does not wait for HBM.
     constexpr int XU = 4;  // covers K <= 4096 in one round
-    f32x4 xr[XU];
+    const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
+    f32x4 xr[XU], ar[XU], nr[XU];  // activation; second operand (x2 or res_in); norm weight
+    const float *second = fuse.x2 ? fuse.x2 : fuse.res_in;
 #pragma unroll
     for (int u = 0; u < XU; u++) {
         const int k = (tid + u * QTHREADS) * 4;
-        xr[u] = k < K ? *reinterpret_cast<const f32x4 *>(x + k) : f32x4{0.f, 0.f, 0.f, 0.f};
+        xr[u] = k < K ? *reinterpret_cast<const f32x4 *>(x + k) : zero4;
+        ar[u] = second && k < K ? *reinterpret_cast<const f32x4 *>(second + k) : zero4;
+        nr[u] = fuse.norm_w && k < K ? *reinterpret_cast<const f32x4 *>(fuse.norm_w + k) : zero4;
     }
     u32x4 tmp[U];
     int step = blockIdx.x;
@@ -173,13 +179,56 @@ __global__ __launch_bounds__(QTHREADS) void gemv_quant_kernel(
         const int i = tid + u * QTHREADS;
         tmp[u] = i < cur.nchunks ? ld128_stream(w + cur.abeg + (size_t)i * 16) : u32x4{0u, 0u, 0u, 0u};
     }
+    // the light ops of the quantised plan that sit in front of this product (the host allows the
+    // norm only for K <= XU * 1024, where the whole row is in xr)
+    if (fuse.x2) {
+#pragma unroll
+        for (int u = 0; u < XU; u++)
+#pragma unroll
+            for (int e = 0; e < 4; e++) xr[u][e] = (xr[u][e] / (1.0f + expf(-xr[u][e]))) * ar[u][e];
+    } else if (fuse.res_in) {
+#pragma unroll
+        for (int u = 0; u < XU; u++) {
+            xr[u] += ar[u];
+            const int k = (tid + u * QTHREADS) * 4;
+            if (fuse.resid_out && blockIdx.x == 0 && k < K) *reinterpret_cast<f32x4 *>(fuse.resid_out + k) = xr[u];
+        }
+    }
+    if (fuse.norm_w) {
+        float ss = 0.f;
+#pragma unroll
+        for (int u = 0; u < XU; u++) ss += (xr[u][0] * xr[u][0] + xr[u][1] * xr[u][1]) + (xr[u][2] * xr[u][2] + xr[u][3] * xr[u][3]);
+        ss = wave_sum(ss);
+        float *red = reinterpret_cast<float *>(ws);  // the weight stage is not in use yet
+        if (lane == 0) red[wave] = ss;
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");  // LDS only: the weight loads stay in flight
+        float tot = 0.f;
+#pragma unroll
+        for (int wv = 0; wv < QWAVES; wv++) tot += red[wv];
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");  // red is read before ws is written
+        const float inv = 1.0f / sqrtf(tot / (float)K + fuse.eps);
+#pragma unroll
+        for (int u = 0; u < XU; u++)
+#pragma unroll
+            for (int e = 0; e < 4; e++) xr[u][e] = (xr[u][e] * inv) * nr[u][e];
+    }
 #pragma unroll
     for (int u = 0; u < XU; u++) {
         const int k = (tid + u * QTHREADS) * 4;
         if (k < K) *reinterpret_cast<f32x4 *>(xs + k) = xr[u];
     }
-    for (int k = (tid + XU * QTHREADS) * 4; k < K; k += QTHREADS * 4)  // longer rows
-        *reinterpret_cast<f32x4 *>(xs + k) = *reinterpret_cast<const f32x4 *>(x + k);
+    for (int k = (tid + XU * QTHREADS) * 4; k < K; k += QTHREADS * 4) {  // longer rows (no norm here)
+        f32x4 v = *reinterpret_cast<const f32x4 *>(x + k);
+        if (fuse.x2) {
+            const f32x4 o = *reinterpret_cast<const f32x4 *>(fuse.x2 + k);
+#pragma unroll
+            for (int e = 0; e < 4; e++) v[e] = (v[e] / (1.0f + expf(-v[e]))) * o[e];
+        } else if (fuse.res_in) {
+            v += *reinterpret_cast<const f32x4 *>(fuse.res_in + k);
+            if (fuse.resid_out && blockIdx.x == 0) *reinterpret_cast<f32x4 *>(fuse.resid_out + k) = v;
+        }
+        *reinterpret_cast<f32x4 *>(xs + k) = v;
+    }
     __syncthreads();
     float xv[NXV][8], sxo[NXV];
     if (resident) {
@@ -210,16 +259,17 @@ __global__ __launch_bounds__(QTHREADS) void gemv_quant_kernel(
         }
 
         const uint8_t *base = ws + now.shift;
+        const float *add = fuse.res_out_add ? fuse.res_out_add + now.r0 : nullptr;
         if (resident) {
             // up to four rows per trip: independent chains for the LDS reads and the reductions
             int lr = wave;
             for (; lr + 3 * QWAVES < now.nrows; lr += 4 * QWAVES)
-                rows_trip<QT, NXV, 4>(base, rowbytes, lr, lane, nq, xv, sxo, out + now.r0);
+                rows_trip<QT, NXV, 4>(base, rowbytes, lr, lane, nq, xv, sxo, out + now.r0, add);
             if (lr + QWAVES < now.nrows) {
-                rows_trip<QT, NXV, 2>(base, rowbytes, lr, lane, nq, xv, sxo, out + now.r0);
+                rows_trip<QT, NXV, 2>(base, rowbytes, lr, lane, nq, xv, sxo, out + now.r0, add);
                 lr += 2 * QWAVES;
             }
-            if (lr < now.nrows) rows_trip<QT, NXV, 1>(base, rowbytes, lr, lane, nq, xv, sxo, out + now.r0);
+            if (lr < now.nrows) rows_trip<QT, NXV, 1>(base, rowbytes, lr, lane, nq, xv, sxo, out + now.r0, add);
         } else {  // long rows: the activations of a column are re-read from LDS
             float acc[MAX_ROWS_PER_WAVE];
 #pragma unroll
@@ -241,7 +291,7 @@ __global__ __launch_bounds__(QTHREADS) void gemv_quant_kernel(
             for (int i = 0; i < MAX_ROWS_PER_WAVE; i++) {
                 const int lr = wave + QWAVES * i;
                 const float v = wave_sum(acc[i]);
-                if (lane == 0 && lr < now.nrows) out[now.r0 + lr] = v;
+                if (lane == 0 && lr < now.nrows) out[now.r0 + lr] = add ? v + add[lr] : v;
             }
         }
     }
@@ -273,13 +323,18 @@ __global__ __launch_bounds__(256) void dequant_kernel(const uint8_t *__restrict_
 
 template <int QT>
 int gemv_quant_launch(hm_ctx *ctx, const char *name, const float *d_x, const uint8_t *d_w,
-                      float *d_out, int M, int K, int N) {
+                      float *d_out, int M, int K, int N, const homura::QuantFuse &fuse = homura::QuantFuse()) {
     HM_CHECK_CTX(ctx);
     constexpr int BB = BlockTraits<QT>::BYTES;
     HM_REQUIRE(ctx, d_x && d_w && d_out, "%s: NULL pointer", name);
     HM_REQUIRE(ctx, M >= 1 && M <= 8, "%s: M=%d outside 1..8", name, M);
     HM_REQUIRE(ctx, K > 0 && K % 32 == 0 && N > 0, "%s: K=%d must be a positive multiple of 32, N=%d positive", name, K, N);
     HM_REQUIRE(ctx, ((uintptr_t)d_w % 16) == 0 && ((uintptr_t)d_x % 16) == 0, "%s: weight and activation buffers must be 16-byte aligned", name);
+    HM_REQUIRE(ctx, !(fuse.x2 && fuse.res_in), "%s: SiLU pair and residual input exclude each other", name);
+    HM_REQUIRE(ctx, !fuse.norm_w || K <= 4096, "%s: the fused RMSNorm holds rows up to 4096 wide (K=%d)", name, K);
+    HM_REQUIRE(ctx, ((uintptr_t)fuse.x2 % 16) == 0 && ((uintptr_t)fuse.res_in % 16) == 0 && ((uintptr_t)fuse.resid_out % 16) == 0 &&
+                        ((uintptr_t)fuse.norm_w % 16) == 0, "%s: fused operands must be 16-byte aligned", name);
+    HM_REQUIRE(ctx, M == 1 || (!fuse.x2 && !fuse.res_in && !fuse.norm_w && !fuse.res_out_add), "%s: fused light ops need M == 1", name);
     const size_t rowbytes = (size_t)(K / 32) * BB;
     const size_t x_bytes = (size_t)K * 4;
     const size_t lds_budget = 48 * 1024;
@@ -306,7 +361,7 @@ int gemv_quant_launch(hm_ctx *ctx, const char *name, const float *d_x, const uin
         float *om = d_out + (size_t)m * N;
 #define HM_QUANT_CASE(C)                                                                                  \
     hipLaunchKernelGGL((gemv_quant_kernel<QT, C>), dim3(grid), dim3(QTHREADS), lds, ctx->stream, xm, d_w, \
-                       om, K, N, rows)
+                       om, K, N, rows, fuse)
         switch (cpl <= MAXC ? cpl : 0) {
             case 1: HM_QUANT_CASE(1); break;
             case 2: HM_QUANT_CASE(2); break;
@@ -340,6 +395,12 @@ int dequant_launch(hm_ctx *ctx, const char *name, const uint8_t *d_blocks, float
 }
 
 }  // namespace
+
+int homura::gemv_quant_fused(hm_ctx *ctx, bool q4, const float *d_x, const uint8_t *d_w, float *d_out, int K, int N,
+                             const QuantFuse &fuse) {
+    return q4 ? gemv_quant_launch<1>(ctx, "gemv_quant[q4_0]", d_x, d_w, d_out, 1, K, N, fuse)
+              : gemv_quant_launch<0>(ctx, "gemv_quant[q8_0]", d_x, d_w, d_out, 1, K, N, fuse);
+}
 
 extern "C" {
 

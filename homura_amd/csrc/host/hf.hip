@@ -8,6 +8,7 @@
 #include "../gemv_bf16.h"
 #include "../gemm_bf16_mfma.h"
 #include "../gemv_kquant.h"
+#include "../gemv_quant.h"
 #include "../prefill.h"
 #include "../light_ops.h"
 
@@ -805,7 +806,13 @@ int HfModel::emit_transformer_plan_quant() {
     // the whole run (N rows = the run's total, its outputs are adjacent too); the others launch
     // nothing. reuse_act: an earlier K-quant launch of the same group already quantised this
     // activation.
-    auto quant_mm = [&](const char *label, DType wdt, int64_t K, int64_t N, bool reuse_act) {
+    // Light ops of the neighbouring steps that a Q8_0 / Q4_0 launch does on its way (slots; NO = none):
+    // x <- silu(x) * x2 | x <- x + res_in (-> resid_out) | x <- rmsnorm(x) * norm_w | out <- dot + add.
+    // x / out replace the step's own activation and output slot.
+    constexpr size_t NO = (size_t)-1;
+    struct FuseSlots { size_t x = (size_t)-1, x2 = (size_t)-1, res_in = (size_t)-1, resid_out = (size_t)-1,
+                              norm_w = (size_t)-1, add = (size_t)-1, out = (size_t)-1; };
+    auto quant_mm = [&](const char *label, DType wdt, int64_t K, int64_t N, bool reuse_act, FuseSlots fs) {
         CompiledKernel k;
         k.ops_label = std::string("QuantMM[") + label + "]";
         if (N > 0) {
@@ -813,24 +820,44 @@ int HfModel::emit_transformer_plan_quant() {
             const char *kn = wdt == DType::Q8_0 ? "gemv_q8_0[" : wdt == DType::Q4_0 ? "gemv_q4_0["
                              : wdt == DType::Q4_K ? "gemv_q4_k[" : "gemv_q6_k[";
             l.name = std::string(kn) + label + "]";
+            if (fs.norm_w != NO) l.name += fs.res_in != NO ? "+resid+norm" : "+norm";
+            if (fs.x2 != NO) l.name += "+silu";
+            if (fs.add != NO) l.name += "+resid";
             l.bytes_fixed = (double)dtype_bytes_for_elements(wdt, (size_t)(K * N), nullptr) + K * 4.0 + N * 4.0;
             l.fn = [=](const StepContext &sc) -> int {
-                const float *x = sc.pool[sc.step.input_slots[0]]->as<float>();
+                auto f32 = [&](size_t slot) { return slot == NO ? nullptr : sc.pool[slot]->as<float>(); };
+                const float *x = fs.x != NO ? f32(fs.x) : sc.pool[sc.step.input_slots[0]]->as<float>();
                 const uint8_t *w = sc.pool[sc.step.input_slots[1]]->as<uint8_t>();
-                float *out = sc.pool[sc.step.output_slots[0]]->as<float>();
-                switch (wdt) {
-                case DType::Q8_0: return hm_gemv_q8_0(sc.ctx, x, w, out, 1, (int)K, (int)N);
-                case DType::Q4_0: return hm_gemv_q4_0(sc.ctx, x, w, out, 1, (int)K, (int)N);
-                default: return gemv_kquant(sc.ctx, wdt == DType::Q6_K, x, w, out, (int)K, (int)N, reuse_act);
-                }
+                float *out = fs.out != NO ? f32(fs.out) : sc.pool[sc.step.output_slots[0]]->as<float>();
+                QuantFuse f;
+                f.x2 = f32(fs.x2);
+                f.res_in = f32(fs.res_in);
+                f.resid_out = f32(fs.resid_out);
+                f.norm_w = f32(fs.norm_w);
+                f.eps = eps;
+                f.res_out_add = f32(fs.add);
+                if (wdt == DType::Q8_0 || wdt == DType::Q4_0)
+                    return gemv_quant_fused(sc.ctx, wdt == DType::Q4_0, x, w, out, (int)K, (int)N, f);
+                if (K <= 4096)  // the row is prepared and quantised to Q8_K inside the kernel
+                    return gemv_kquant_fused(sc.ctx, wdt == DType::Q6_K, x, w, out, (int)K, (int)N, f);
+                return gemv_kquant(sc.ctx, wdt == DType::Q6_K, x, w, out, (int)K, (int)N, reuse_act);
             };
             k.launches.push_back(std::move(l));
         }
         return k;
     };
+    // Whether every launch of a group can take light ops along: Q8_0 / Q4_0 always, K-quants while the
+    // row fits the in-kernel preparation
+    auto plain_group = [&](int layer, std::initializer_list<int> which, int64_t K) {
+        for (int w : which) {
+            const DType t = proj_dtype(layer, w);
+            if ((t == DType::Q4_K || t == DType::Q6_K) && K > 4096) return false;
+        }
+        return true;
+    };
     // The QuantMM steps of one group of matrices that share an activation (q|k|v, gate|up, or one alone)
     struct GroupMember { const char *label; int which; int64_t N; size_t w_slot, out_slot; };
-    auto quant_group = [&](int layer, size_t act_slot, int64_t K, std::vector<GroupMember> members) {
+    auto quant_group = [&](int layer, size_t act_slot, int64_t K, std::vector<GroupMember> members, FuseSlots fs) {
         bool act_quantized = false;
         for (size_t j = 0; j < members.size(); j++) {
             const GroupMember &gm = members[j];
@@ -847,7 +874,7 @@ int HfModel::emit_transformer_plan_quant() {
                     label += members[j + e].label;
                 }
             }
-            add_step(quant_mm(label.c_str(), t, K, n_run, kq && act_quantized), {act_slot, gm.w_slot}, {gm.out_slot});
+            add_step(quant_mm(label.c_str(), t, K, n_run, kq && act_quantized, fs), {act_slot, gm.w_slot}, {gm.out_slot});
             if (n_run > 0 && kq) act_quantized = true;
         }
     };
@@ -868,23 +895,37 @@ int HfModel::emit_transformer_plan_quant() {
     }
     for (int i = 0; i < L; i++) {
         const LS &s = ls[i];
+        // Which light steps ride along with a Q8_0 / Q4_0 product instead of being launched (the step
+        // list keeps the reference's kernels; a step whose work moved has no launch of its own)
+        const bool fuse_in_norm = plain_group(i, {0, 1, 2}, hidden) && hidden <= 4096;
+        const bool fuse_post_norm = plain_group(i, {4, 5}, hidden) && hidden <= 4096;
+        const bool fuse_down = plain_group(i, {6}, inter);
         {  // Step 1: pre-QKV RMSNorm (reference :713-791)
             CompiledKernel k;
             k.ops_label = "RMSNorm";
-            DeviceLaunch l;
-            l.name = "rmsnorm";
-            l.bytes_fixed = hidden * 4.0 * 3;
-            l.fn = [=](const StepContext &sc) -> int {
-                return rmsnorm_launch(sc.ctx, sc.pool[sc.step.input_slots[0]]->as<float>(), nullptr,
-                                      sc.pool[sc.step.input_slots[1]]->as<float>(),
-                                      sc.pool[sc.step.output_slots[0]]->as<float>(), nullptr, 1, (int)hidden, eps);
-            };
-            k.launches.push_back(std::move(l));
+            if (!fuse_in_norm) {
+                DeviceLaunch l;
+                l.name = "rmsnorm";
+                l.bytes_fixed = hidden * 4.0 * 3;
+                l.fn = [=](const StepContext &sc) -> int {
+                    return rmsnorm_launch(sc.ctx, sc.pool[sc.step.input_slots[0]]->as<float>(), nullptr,
+                                          sc.pool[sc.step.input_slots[1]]->as<float>(),
+                                          sc.pool[sc.step.output_slots[0]]->as<float>(), nullptr, 1, (int)hidden, eps);
+                };
+                k.launches.push_back(std::move(l));
+            }
             add_step(std::move(k), {s.hidden_in, s.input_ln}, {s.normed});
         }
         // Steps 2-4: QuantMM Q, K, V — one launch over the stacked q|k|v rows
-        quant_group(i, s.normed, hidden, {{"q", 0, qd, s.q_w, s.q_out}, {"k", 1, kvd, s.k_w, s.k_out},
-                                          {"v", 2, kvd, s.v_w, s.v_out}});
+        {
+            FuseSlots fs;
+            if (fuse_in_norm) {
+                fs.x = s.hidden_in;
+                fs.norm_w = s.input_ln;
+            }
+            quant_group(i, s.normed, hidden, {{"q", 0, qd, s.q_w, s.q_out}, {"k", 1, kvd, s.k_w, s.k_out},
+                                              {"v", 2, kvd, s.v_w, s.v_out}}, fs);
+        }
         {  // Step 5: PostQKV (reference :802-912) — runs in the attention kernel's prologue
             CompiledKernel k;
             k.ops_label = qkn ? "PostQKV+QKNorm+RoPE" : "PostQKV+RoPE";
@@ -967,51 +1008,74 @@ int HfModel::emit_transformer_plan_quant() {
             k.launches.push_back(std::move(l));
             add_step(std::move(k), {s.q, s.present_k, s.present_v, mask}, {s.attn_body});
         }
-        quant_group(i, s.attn_body, qd, {{"o", 3, hidden, s.o_w, s.attn_out}});  // Step 9
+        quant_group(i, s.attn_body, qd, {{"o", 3, hidden, s.o_w, s.attn_out}}, FuseSlots());  // Step 9
         {  // Step 10: Residual + RMSNorm (reference :985-1071), two outputs
             CompiledKernel k;
             k.ops_label = "Residual+Norm";
-            DeviceLaunch l;
-            l.name = "residual_rmsnorm";
-            l.bytes_fixed = hidden * 4.0 * 5;
-            l.fn = [=](const StepContext &sc) -> int {
-                const auto &in = sc.step.input_slots;
-                return rmsnorm_launch(sc.ctx, sc.pool[in[0]]->as<float>(), sc.pool[in[1]]->as<float>(),
-                                      sc.pool[in[2]]->as<float>(), sc.pool[sc.step.output_slots[1]]->as<float>(),
-                                      sc.pool[sc.step.output_slots[0]]->as<float>(), 1, (int)hidden, eps);
-            };
-            k.launches.push_back(std::move(l));
+            if (!fuse_post_norm) {
+                DeviceLaunch l;
+                l.name = "residual_rmsnorm";
+                l.bytes_fixed = hidden * 4.0 * 5;
+                l.fn = [=](const StepContext &sc) -> int {
+                    const auto &in = sc.step.input_slots;
+                    return rmsnorm_launch(sc.ctx, sc.pool[in[0]]->as<float>(), sc.pool[in[1]]->as<float>(),
+                                          sc.pool[in[2]]->as<float>(), sc.pool[sc.step.output_slots[1]]->as<float>(),
+                                          sc.pool[sc.step.output_slots[0]]->as<float>(), 1, (int)hidden, eps);
+                };
+                k.launches.push_back(std::move(l));
+            }
             add_step(std::move(k), {s.hidden_in, s.attn_out, s.post_ln}, {s.residual, s.post_normed});
         }
-        // Steps 11-12: QuantMM Gate, Up — one launch over the stacked gate|up rows
-        quant_group(i, s.post_normed, hidden, {{"gate", 4, inter, s.gate_w, s.gate_out}, {"up", 5, inter, s.up_w, s.up_out}});
+        {  // Steps 11-12: QuantMM Gate, Up — one launch per run of equal types over the stacked rows
+            FuseSlots fs;
+            if (fuse_post_norm) {  // residual = hidden_in + attn_out, normed on the way in
+                fs.x = s.hidden_in;
+                fs.res_in = s.attn_out;
+                fs.resid_out = s.residual;
+                fs.norm_w = s.post_ln;
+            }
+            quant_group(i, s.post_normed, hidden, {{"gate", 4, inter, s.gate_w, s.gate_out}, {"up", 5, inter, s.up_w, s.up_out}}, fs);
+        }
         {  // Step 13: SiLU * Up (reference :1077-1103)
             CompiledKernel k;
             k.ops_label = "SiLU*Up";
-            DeviceLaunch l;
-            l.name = "silu_mul";
-            l.bytes_fixed = inter * 4.0 * 3;
-            l.fn = [=](const StepContext &sc) -> int {
-                const auto &in = sc.step.input_slots;
-                return hm_silu_mul(sc.ctx, sc.pool[in[0]]->as<float>(), sc.pool[in[1]]->as<float>(),
-                                   sc.pool[sc.step.output_slots[0]]->as<float>(), (size_t)inter);
-            };
-            k.launches.push_back(std::move(l));
+            if (!fuse_down) {
+                DeviceLaunch l;
+                l.name = "silu_mul";
+                l.bytes_fixed = inter * 4.0 * 3;
+                l.fn = [=](const StepContext &sc) -> int {
+                    const auto &in = sc.step.input_slots;
+                    return hm_silu_mul(sc.ctx, sc.pool[in[0]]->as<float>(), sc.pool[in[1]]->as<float>(),
+                                       sc.pool[sc.step.output_slots[0]]->as<float>(), (size_t)inter);
+                };
+                k.launches.push_back(std::move(l));
+            }
             add_step(std::move(k), {s.gate_out, s.up_out}, {s.silu});
         }
-        quant_group(i, s.silu, inter, {{"down", 6, hidden, s.down_w, s.down_out}});  // Step 14
+        {  // Step 14: QuantMM Down; with a Q8_0 / Q4_0 matrix it takes SiLU*Up on the way in and ResAdd on the way out
+            FuseSlots fs;
+            if (fuse_down) {
+                fs.x = s.gate_out;
+                fs.x2 = s.up_out;
+                fs.add = s.residual;
+                fs.out = s.hidden_out;
+            }
+            quant_group(i, s.silu, inter, {{"down", 6, hidden, s.down_w, s.down_out}}, fs);
+        }
         {  // Step 15: ResAdd (reference :1109-1134)
             CompiledKernel k;
             k.ops_label = "ResAdd";
-            DeviceLaunch l;
-            l.name = "residual_add";
-            l.bytes_fixed = hidden * 4.0 * 3;
-            l.fn = [=](const StepContext &sc) -> int {
-                const auto &in = sc.step.input_slots;
-                return hm_add(sc.ctx, sc.pool[in[0]]->as<float>(), sc.pool[in[1]]->as<float>(),
-                              sc.pool[sc.step.output_slots[0]]->as<float>(), (size_t)hidden);
-            };
-            k.launches.push_back(std::move(l));
+            if (!fuse_down) {
+                DeviceLaunch l;
+                l.name = "residual_add";
+                l.bytes_fixed = hidden * 4.0 * 3;
+                l.fn = [=](const StepContext &sc) -> int {
+                    const auto &in = sc.step.input_slots;
+                    return hm_add(sc.ctx, sc.pool[in[0]]->as<float>(), sc.pool[in[1]]->as<float>(),
+                                  sc.pool[sc.step.output_slots[0]]->as<float>(), (size_t)hidden);
+                };
+                k.launches.push_back(std::move(l));
+            }
             add_step(std::move(k), {s.residual, s.down_out}, {s.hidden_out});
         }
     }
