@@ -249,13 +249,16 @@ __device__ __forceinline__ void stage_activation(const float *__restrict__ x, co
     }
 }
 
-template <int QT, int CPL>
+template <int QT, int CPL, bool FUSED>
 __global__ __launch_bounds__(KTHREADS) void gemv_kquant_kernel(const int8_t *__restrict__ q8,
                                                                const float *__restrict__ act_d,
                                                                const int *__restrict__ bsums,
                                                                const uint8_t *__restrict__ w, float *__restrict__ out,
-                                                               int K, int N, int rows_per_step, const float *x_f32,
-                                                               const homura::QuantFuse fuse, int act_lds_off) {
+                                                               int K, int N, int rows_per_step, const float *x_f32_arg,
+                                                               const homura::QuantFuse fuse_arg, int act_lds_off) {
+    // FUSED = false is the plain product over an activation quantised by its own launch
+    const float *x_f32 = FUSED ? x_f32_arg : nullptr;
+    const homura::QuantFuse fuse = FUSED ? fuse_arg : homura::QuantFuse();
     constexpr int BB = KTraits<QT>::BYTES;
     constexpr int U = KSTAGE_U;
     extern __shared__ __attribute__((aligned(16))) uint8_t ws[];
@@ -429,8 +432,14 @@ int gemv_kquant_launch(hm_ctx *ctx, const char *name, const float *d_x, const ui
         const float *xf = fuse ? d_x : nullptr;
         const homura::QuantFuse fz = fuse ? *fuse : homura::QuantFuse();
 #define HM_KQ_CASE(C)                                                                                              \
-    hipLaunchKernelGGL((gemv_kquant_kernel<QT, C>), dim3(grid), dim3(KTHREADS), lds, ctx->stream, q8, act_d, bsums, \
-                       d_w, om, K, N, rows, xf, fz, (int)stage_bytes)
+    do {                                                                                                            \
+        if (fuse)                                                                                                   \
+            hipLaunchKernelGGL((gemv_kquant_kernel<QT, C, true>), dim3(grid), dim3(KTHREADS), lds, ctx->stream, q8, \
+                               act_d, bsums, d_w, om, K, N, rows, xf, fz, (int)stage_bytes);                        \
+        else                                                                                                        \
+            hipLaunchKernelGGL((gemv_kquant_kernel<QT, C, false>), dim3(grid), dim3(KTHREADS), lds, ctx->stream, q8, \
+                               act_d, bsums, d_w, om, K, N, rows, xf, fz, (int)stage_bytes);                        \
+    } while (0)
         switch (cpl) {
             case 1: HM_KQ_CASE(1); break;
             case 2: HM_KQ_CASE(2); break;

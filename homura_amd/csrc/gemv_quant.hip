@@ -141,10 +141,12 @@ __device__ __forceinline__ void rows_trip(const uint8_t *base, size_t rowbytes, 
 }
 
 // CPL = quarter columns per lane held in registers (ceil(K/8/64)); 0 = re-read them from LDS.
-template <int QT, int CPL>
+template <int QT, int CPL, bool FUSED>
 __global__ __launch_bounds__(QTHREADS) void gemv_quant_kernel(
     const float *__restrict__ x, const uint8_t *__restrict__ w, float *__restrict__ out, int K,
-    int N, int rows_per_step, const homura::QuantFuse fuse) {
+    int N, int rows_per_step, const homura::QuantFuse fuse_arg) {
+    // FUSED = false is the plain product: every pointer of the fusion record reads as null at compile time
+    const homura::QuantFuse fuse = FUSED ? fuse_arg : homura::QuantFuse();
     constexpr int BB = BlockTraits<QT>::BYTES;
     constexpr int U = STAGE_U;
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -356,12 +358,19 @@ int gemv_quant_launch(hm_ctx *ctx, const char *name, const float *d_x, const uin
     if (wg_per_cu > 6) wg_per_cu = 6;
     const int grid = nsteps < ctx->num_cus * wg_per_cu ? nsteps : ctx->num_cus * wg_per_cu;
     const int cpl = (K / 8 + WAVE - 1) / WAVE;
+    const bool fused = fuse.x2 || fuse.res_in || fuse.norm_w || fuse.res_out_add;
     for (int m = 0; m < M; m++) {
         const float *xm = d_x + (size_t)m * K;
         float *om = d_out + (size_t)m * N;
 #define HM_QUANT_CASE(C)                                                                                  \
-    hipLaunchKernelGGL((gemv_quant_kernel<QT, C>), dim3(grid), dim3(QTHREADS), lds, ctx->stream, xm, d_w, \
-                       om, K, N, rows, fuse)
+    do {                                                                                                  \
+        if (fused)                                                                                        \
+            hipLaunchKernelGGL((gemv_quant_kernel<QT, C, true>), dim3(grid), dim3(QTHREADS), lds, ctx->stream, xm, \
+                               d_w, om, K, N, rows, fuse);                                                \
+        else                                                                                              \
+            hipLaunchKernelGGL((gemv_quant_kernel<QT, C, false>), dim3(grid), dim3(QTHREADS), lds, ctx->stream, xm, \
+                               d_w, om, K, N, rows, fuse);                                                \
+    } while (0)
         switch (cpl <= MAXC ? cpl : 0) {
             case 1: HM_QUANT_CASE(1); break;
             case 2: HM_QUANT_CASE(2); break;
