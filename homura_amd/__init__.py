@@ -6,8 +6,8 @@ HfModel / ExecutionPlan / KvCache. There is no CPU fallback: without the built l
 or without a GPU, the calls raise.
 """
 from .runtime import (Context, DeviceBuffer, HfModel, HomuraError, TransformerConfig,  # noqa: F401
-                      DTYPE_BF16, DTYPE_F32, DTYPE_Q4_0, DTYPE_Q8_0)
+                      DTYPE_BF16, DTYPE_F32, DTYPE_Q4_0, DTYPE_Q8_0, DTYPE_Q4_K, DTYPE_Q6_K)
 from . import synth  # noqa: F401
 
 __all__ = ["Context", "DeviceBuffer", "HfModel", "HomuraError", "TransformerConfig", "synth",
-           "DTYPE_F32", "DTYPE_BF16", "DTYPE_Q8_0", "DTYPE_Q4_0"]
+           "DTYPE_F32", "DTYPE_BF16", "DTYPE_Q8_0", "DTYPE_Q4_0", "DTYPE_Q4_K", "DTYPE_Q6_K"]

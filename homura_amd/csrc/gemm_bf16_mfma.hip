@@ -67,8 +67,13 @@ struct TileRegs {
 
 // M, N: logical sizes; K: length of the k loop; lda: row stride of A; Kb: k extent of B (k wraps at Kb)
 // kt_per_split: K tiles per grid.y slice (a multiple of the register ring depth)
+// ldb, ldc: row strides of B ([N][K] layout) and C. Piece pairs (the [N][K] kernel with aligned K
+// tiles only): the k loop is `npairs` stretches of Kb; stretch p multiplies piece (apack >> 2p) & 3 of
+// A (columns [piece Kb, (piece + 1) Kb) of its rows) by piece (bpack >> 2p) & 3 of B.
 struct GemmDims {
     int M, N, K, lda, Kb, kt_per_split;
+    int ldb, ldc, npairs;
+    uint32_t apack, bpack;
 };
 
 // k index of B for loop index kc: the loop covers at most three copies of B's k range
@@ -213,7 +218,7 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_bf16_mfma_kernel(const uint
     const int nk = min(g.kt_per_split, (K + TK - 1) / TK - kt_first);
     const int nkp = (nk + DEPTH - 1) / DEPTH * DEPTH;
     const int kbase = kt_first * TK;
-    C += (size_t)blockIdx.y * M * N;
+    C += (size_t)blockIdx.y * M * g.ldc;
     TileRegs t[DEPTH];
     // B's k offset of the next tile to request: runs along with the loop and wraps at Kb (ALIGNED only)
     int kb_run = kbase % g.Kb;
@@ -304,14 +309,196 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_bf16_mfma_kernel(const uint
                 const int col = n0 + wn * 64 + j * 32 + l32;
                 const float sum = acc[i][j][v] + xch[((i * 2 + j) * 16 + v) * 64];
                 if (interior)
-                    __builtin_nontemporal_store(sum, C + (size_t)row * N + col);
+                    __builtin_nontemporal_store(sum, C + (size_t)row * g.ldc + col);
                 else if (row < M && col < N)
-                    __builtin_nontemporal_store(sum, C + (size_t)row * N + col);
+                    __builtin_nontemporal_store(sum, C + (size_t)row * g.ldc + col);
             }
 }
 
+// ---- [N][K] operand, K tiles aligned: global -> LDS loads without the trip through registers ----
+//
+// global_load_lds_dwordx4 writes lane l's 16 bytes to LDS at (wave-uniform base) + 16 l, so one
+// instruction fills eight 128-byte rows. The slot swizzle moves to the global side: the lane that
+// fills slot s of row r fetches chunk s ^ (r & 7) ^ ((r >> 3) & 7) of that row. The tiles in flight
+// live in LDS (DMA_BUFS buffers of 32 KiB), the registers of the ring above are free, and the LDS
+// write instructions are gone.
+constexpr int DMA_BUFS = 4;  // the vmcnt values in the kernel count DMA_BUFS - 1 tiles of four loads in flight
+static_assert(DMA_BUFS == 4, "adjust the wait counts of gemm_nk_dma_kernel");
+constexpr int DMA_LDS_BYTES = DMA_BUFS * 2 * TILE_BYTES;  // 128 of the CU's 160 KiB
+
+extern __shared__ __attribute__((aligned(16))) char dma_lds[];
+
+__device__ __forceinline__ void dma16(const uint16_t *src, char *dst) {
+    __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1))) *)src,
+                                     (void __attribute__((address_space(3))) *)dst, 16, 0, 0);
+}
+
+// The operand reads and their waits are written out: the compiler's own wait insertion stalls on
+// all outstanding LDS reads at the top of the loop, these wait only for the ones about to be used.
+// (LDS operations of a wavefront return in order.)
+__device__ __forceinline__ bf16x8 lds_read16(uint32_t addr) {
+    bf16x8 v;
+    asm volatile("ds_read_b128 %0, %1" : "=v"(v) : "v"(addr) : "memory");
+    return v;
+}
+
+__global__ __launch_bounds__(GEMM_THREADS) void gemm_nk_dma_kernel(const uint16_t *__restrict__ A,
+                                                                   const uint16_t *__restrict__ B,
+                                                                   float *__restrict__ C, const GemmDims g) {
+    const int M = g.M, K = g.K, N = g.N;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int kgrp = wave >> 2, wm = (wave >> 1) & 1, wn = wave & 1;
+    const int l32 = lane & 31, lh = lane >> 5;
+
+    const int mb = (M + TM - 1) / TM, total = gridDim.x;
+    int lin = blockIdx.x;
+    if ((total & 7) == 0) lin = (blockIdx.x & 7) * (total >> 3) + (blockIdx.x >> 3);
+    const int m0 = (lin % mb) * TM, n0 = (lin / mb) * TN;
+
+    f32x16 acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) acc[i][j][v] = 0.f;
+
+    const int kt_first = blockIdx.y * g.kt_per_split;
+    const int nk = min(g.kt_per_split, K / TK - kt_first);
+    C += (size_t)blockIdx.y * M * g.ldc;
+
+    // this thread's two rows of A and of B: instruction j of wavefront w fills rows 8 (2 w + j) .. + 7
+    const uint16_t *a_src[2], *b_src[2];
+    int dst_off[2];
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+        const int r = (wave * 2 + j) * 8 + (lane >> 3), s = lane & 7;
+        const int c = s ^ (r & 7) ^ ((r >> 3) & 7);
+        a_src[j] = A + (size_t)min(m0 + r, M - 1) * g.lda + c * 8;
+        b_src[j] = B + (size_t)min(n0 + r, N - 1) * g.ldb + c * 8;
+        dst_off[j] = (wave * 2 + j) * 1024;
+    }
+    // the next tile to request: stretch `pair`, k offset `koff` inside it (all scalar)
+    const int tiles_per_stretch = g.Kb / TK;
+    int pair = kt_first / tiles_per_stretch, koff = (kt_first % tiles_per_stretch) * TK;
+    // a tile past the end re-reads one of the last stretch (nobody multiplies it), so every iteration
+    // issues the same four loads and the wait counts below are exact
+    auto request = [&](int buf) {
+        char *base = dma_lds + buf * (2 * TILE_BYTES);
+        const int pr = 2 * min(pair, g.npairs - 1);
+        const int ka = (int)((g.apack >> pr) & 3u) * g.Kb + koff;
+        const int kb = (int)((g.bpack >> pr) & 3u) * g.Kb + koff;
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            dma16(a_src[j] + ka, base + dst_off[j]);
+            dma16(b_src[j] + kb, base + TILE_BYTES + dst_off[j]);
+        }
+        koff += TK;
+        if (koff == g.Kb) {
+            koff = 0;
+            pair++;
+        }
+    };
+#pragma unroll
+    for (int d = 0; d < DMA_BUFS; d++) request(d);
+
+    const int arow = wm * 64 + l32, brow = wn * 64 + l32;
+    const int chunk0 = kgrp * 4 + lh, chunk1 = chunk0 + 2;  // this group's two k steps of a tile
+    int a_off[2][2], b_off[2][2];                           // [k step][i]
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+        a_off[0][i] = lds_off(arow + i * 32, chunk0);
+        a_off[1][i] = lds_off(arow + i * 32, chunk1);
+        b_off[0][i] = TILE_BYTES + lds_off(brow + i * 32, chunk0);
+        b_off[1][i] = TILE_BYTES + lds_off(brow + i * 32, chunk1);
+    }
+
+    // operand registers, two stages: the reads of the next step are in flight during the MFMAs
+    bf16x8 af[2][2], bfr[2][2];
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char *)dma_lds;
+    // tiles 1..3 (four loads each) may still be in flight; tile 0 has landed for everyone
+    asm volatile("s_waitcnt vmcnt(12)\n\ts_barrier" ::: "memory");
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+        af[0][i] = lds_read16(lds0 + a_off[0][i]);
+        bfr[0][i] = lds_read16(lds0 + b_off[0][i]);
+    }
+
+    int u = 0;  // kt % DMA_BUFS
+    for (int kt = 0; kt < nk; kt++) {
+        const int un = u + 1 == DMA_BUFS ? 0 : u + 1;
+        const uint32_t cur = lds0 + u * (2 * TILE_BYTES);
+        const uint32_t nxt = lds0 + un * (2 * TILE_BYTES);
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            af[1][i] = lds_read16(cur + a_off[1][i]);
+            bfr[1][i] = lds_read16(cur + b_off[1][i]);
+        }
+        // the four reads above may be in flight; the four before them (stage 0) have arrived
+        asm volatile("s_waitcnt lgkmcnt(4)" : "+v"(af[0][0]), "+v"(af[0][1]), "+v"(bfr[0][0]), "+v"(bfr[0][1]));
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+#pragma unroll
+            for (int j = 0; j < 2; j++)
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[0][i], bfr[0][j], acc[i][j], 0, 0, 0);
+        // every wavefront has read its last operands of this tile, and the next tile has landed for
+        // everyone (the two after it may be in flight): this tile's buffer takes tile kt + 4
+        asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)\n\ts_barrier"
+                     : "+v"(af[1][0]), "+v"(af[1][1]), "+v"(bfr[1][0]), "+v"(bfr[1][1])
+                     :
+                     : "memory");
+        request(u);
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            af[0][i] = lds_read16(nxt + a_off[0][i]);
+            bfr[0][i] = lds_read16(nxt + b_off[0][i]);
+        }
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+#pragma unroll
+            for (int j = 0; j < 2; j++)
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[1][i], bfr[1][j], acc[i][j], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        u = un;
+    }
+
+    // drain the loads still in flight (they target LDS) before the buffers are reused for the exchange
+    asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
+    float *xch = reinterpret_cast<float *>(dma_lds) + (size_t)(wave & 3) * 64 * 64 + lane;
+    if (kgrp == 1) {
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+#pragma unroll
+            for (int j = 0; j < 2; j++)
+#pragma unroll
+                for (int v = 0; v < 16; v++) xch[((i * 2 + j) * 16 + v) * 64] = acc[i][j][v];
+    }
+    lds_barrier();
+    if (kgrp == 1) return;
+
+    const bool interior = m0 + TM <= M && n0 + TN <= N;
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                const int row = m0 + wm * 64 + i * 32 + (v >> 2) * 8 + lh * 4 + (v & 3);
+                const int col = n0 + wn * 64 + j * 32 + l32;
+                const float sum = acc[i][j][v] + xch[((i * 2 + j) * 16 + v) * 64];
+                if (interior)
+                    __builtin_nontemporal_store(sum, C + (size_t)row * g.ldc + col);
+                else if (row < M && col < N)
+                    __builtin_nontemporal_store(sum, C + (size_t)row * g.ldc + col);
+            }
+}
+
+// b_pieces == 1: C = (sum of A's `pieces` pieces) x B. b_pieces == 3 (B [N][3 K], A [M][3 K]): the six
+// products of an A piece and a B piece whose indices add up to at most 2, i.e. the product of two
+// f32 matrices up to terms below 2^-24 of it.
 int gemm_launch(hm_ctx *ctx, const char *who, const uint16_t *a, const uint16_t *b, float *c, int M, int K,
-                int N, bool b_nk, int pieces, int ksplit = 1, int *ksplit_used = nullptr) {
+                int N, bool b_nk, int pieces, int ksplit = 1, int *ksplit_used = nullptr, int b_pieces = 1,
+                int ldc = 0) {
     HM_CHECK_CTX(ctx);
     HM_REQUIRE(ctx, a && b && c, "%s: NULL pointer", who);
     HM_REQUIRE(ctx, M > 0 && N > 0 && K > 0 && K % 32 == 0, "%s: need M, N > 0 and K %% 32 == 0 (M=%d K=%d N=%d)", who,
@@ -325,8 +512,23 @@ int gemm_launch(hm_ctx *ctx, const char *who, const uint16_t *a, const uint16_t 
     g.M = M;
     g.N = N;
     g.Kb = K;
-    g.K = pieces * K;
-    g.lda = g.K;
+    g.lda = pieces * K;
+    g.ldb = b_pieces * K;
+    g.ldc = ldc > 0 ? ldc : N;
+    if (b_pieces == 1) {
+        g.npairs = pieces;
+        g.apack = 0;  // last piece first: the small terms are added while the accumulator is small
+        for (int i = 0; i < pieces; i++) g.apack |= (uint32_t)(pieces - 1 - i) << (2 * i);
+        g.bpack = 0;
+    } else {
+        HM_REQUIRE(ctx, b_nk && pieces == 3 && b_pieces == 3 && K % TK == 0,
+                   "%s: piece pairs need the [N][K] layout, three pieces a side and K %% 64 == 0", who);
+        g.npairs = 6;
+        g.apack = 0x046;  // (a, b) = (2,0) (1,1) (0,2) (1,0) (0,1) (0,0): the small terms first
+        g.bpack = 0x124;
+    }
+    g.K = g.npairs * K;
+    HM_REQUIRE(ctx, g.ldc >= N, "%s: ldc %d below N %d", who, g.ldc, N);
     const int nk_total = (g.K + TK - 1) / TK;
     if (ksplit < 1) ksplit = 1;
     g.kt_per_split = ((nk_total + ksplit - 1) / ksplit + GEMM_DEPTH - 1) / GEMM_DEPTH * GEMM_DEPTH;
@@ -334,9 +536,13 @@ int gemm_launch(hm_ctx *ctx, const char *who, const uint16_t *a, const uint16_t 
     if (ksplit_used) *ksplit_used = slices;
     const dim3 grid((unsigned)tiles, (unsigned)slices);
     const bool aligned = g.K % TK == 0 && g.Kb % TK == 0;
-    if (b_nk && aligned)
-        hipLaunchKernelGGL((gemm_bf16_mfma_kernel<true, true>), grid, dim3(GEMM_THREADS), 0, ctx->stream, a, b, c, g);
-    else if (b_nk)
+    if (b_nk && aligned) {
+        static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_nk_dma_kernel),
+                                                           hipFuncAttributeMaxDynamicSharedMemorySize, DMA_LDS_BYTES);
+        HM_REQUIRE(ctx, attr == hipSuccess, "%s: cannot reserve %d bytes of LDS: %s", who, DMA_LDS_BYTES,
+                   hipGetErrorString(attr));
+        hipLaunchKernelGGL(gemm_nk_dma_kernel, grid, dim3(GEMM_THREADS), DMA_LDS_BYTES, ctx->stream, a, b, c, g);
+    } else if (b_nk)
         hipLaunchKernelGGL((gemm_bf16_mfma_kernel<true, false>), grid, dim3(GEMM_THREADS), 0, ctx->stream, a, b, c, g);
     else if (aligned)
         hipLaunchKernelGGL((gemm_bf16_mfma_kernel<false, true>), grid, dim3(GEMM_THREADS), 0, ctx->stream, a, b, c, g);
@@ -359,6 +565,16 @@ int homura::gemm_split_nk(hm_ctx *ctx, const uint16_t *d_a_split, int pieces, co
     want = std::min(std::min(want, max_parts), std::max(1, nk_total / GEMM_DEPTH));
     if (!parts) want = 1;
     return gemm_launch(ctx, "gemm_split_nk", d_a_split, d_b_nk, d_c, M, K, N, true, pieces, want, parts);
+}
+
+int homura::gemm_split_split_nk(hm_ctx *ctx, const uint16_t *d_a_split, const uint16_t *d_b_split, float *d_c, int M,
+                                int K, int N, int max_parts, int *parts, int ldc) {
+    const long long tiles = (long long)((M + TM - 1) / TM) * ((N + TN - 1) / TN);
+    const int nk_total = 6 * K / TK;
+    int want = (int)std::max<long long>(1, ctx->num_cus / tiles);
+    want = std::min(std::min(want, max_parts), std::max(1, nk_total / GEMM_DEPTH));
+    if (!parts) want = 1;
+    return gemm_launch(ctx, "gemm_split_split_nk", d_a_split, d_b_split, d_c, M, K, N, true, 3, want, parts, 3, ldc);
 }
 
 extern "C" int hm_gemm_bf16(hm_ctx *ctx, const uint16_t *d_a_mk, const uint16_t *d_b_kn, float *d_c,

@@ -14,6 +14,7 @@
 // the block's activation scale in registers for the life of the workgroup and walks the rows.
 #include "gemv_kquant.h"
 #include "hm_common.h"
+#include "quant_formats.h"
 
 namespace {
 
@@ -340,39 +341,11 @@ __global__ __launch_bounds__(KTHREADS) void gemv_kquant_kernel(const int8_t *__r
 template <int QT>
 __global__ __launch_bounds__(256) void dequant_kquant_kernel(const uint8_t *__restrict__ blocks,
                                                              float *__restrict__ out, size_t n_elems) {
-    constexpr int BB = KTraits<QT>::BYTES;
+    constexpr int QF = QT == 0 ? homura::QF_Q4_K : homura::QF_Q6_K;
     size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     const size_t stride = (size_t)gridDim.x * blockDim.x;
-    for (; e < n_elems; e += stride) {
-        const uint8_t *blk = blocks + (e >> 8) * BB;
-        const int j = (int)(e & 255);
-        if (QT == 0) {
-            const float d = f16_bits_to_f32((uint16_t)(blk[0] | (blk[1] << 8)));
-            const float dmin = f16_bits_to_f32((uint16_t)(blk[2] | (blk[3] << 8)));
-            const uint8_t *raw = blk + 4;
-            const int sb = j >> 5, l = j & 31;
-            int sc, mn;
-            if (sb < 4) {
-                sc = raw[sb] & 63;
-                mn = raw[sb + 4] & 63;
-            } else {
-                sc = (raw[sb + 4] & 15) | ((raw[sb - 4] >> 6) << 4);
-                mn = (raw[sb + 4] >> 4) | ((raw[sb] >> 6) << 4);
-            }
-            const uint8_t byte = blk[16 + (sb >> 1) * 32 + l];
-            const int q = (sb & 1) ? (byte >> 4) : (byte & 15);
-            out[e] = __fsub_rn(__fmul_rn((float)q, __fmul_rn(d, (float)sc)), __fmul_rn(dmin, (float)mn));
-        } else {
-            const float d = f16_bits_to_f32((uint16_t)(blk[208] | (blk[209] << 8)));
-            const int h = j >> 7, g = (j & 127) >> 5, l = j & 31;
-            const uint8_t lb = blk[64 * h + 32 * (g & 1) + l];
-            const int lo = g >= 2 ? (lb >> 4) : (lb & 15);
-            const int hi = (blk[128 + 32 * h + l] >> (2 * g)) & 3;
-            const int q = (int)(int8_t)(lo | (hi << 4)) - 32;
-            const int sc = (int)(int8_t)blk[192 + 8 * h + 2 * g + (l >> 4)];
-            out[e] = __fmul_rn(__fmul_rn(d, (float)sc), (float)q);
-        }
-    }
+    for (; e < n_elems; e += stride)
+        out[e] = homura::dequant_element<QF>(blocks + (e >> 8) * KTraits<QT>::BYTES, (int)(e & 255));
 }
 
 int quantize_launch(hm_ctx *ctx, const float *d_x, int8_t *q8, float *act_d, int *bsums, int M, int K) {

@@ -14,7 +14,9 @@
 // used as stored (biased unsigned): sum_j q_j x_j - offset * sum_j x_j, four byte->float
 // conversions per 32-bit word with no shifts for the byte lanes.
 #include "gemv_quant.h"
+
 #include "hm_common.h"
+#include "quant_formats.h"
 
 namespace {
 
@@ -304,23 +306,11 @@ __global__ __launch_bounds__(QTHREADS) void gemv_quant_kernel(
 template <int QT>
 __global__ __launch_bounds__(256) void dequant_kernel(const uint8_t *__restrict__ blocks,
                                                       float *__restrict__ out, size_t n_elems) {
-    constexpr int BB = BlockTraits<QT>::BYTES;
+    constexpr int QF = QT == 0 ? homura::QF_Q8_0 : homura::QF_Q4_0;
     size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     const size_t stride = (size_t)gridDim.x * blockDim.x;
-    for (; e < n_elems; e += stride) {
-        const size_t b = e >> 5;
-        const int j = (int)(e & 31);
-        const uint8_t *blk = blocks + b * BB;
-        const float d = f16_bits_to_f32((uint16_t)(blk[0] | (blk[1] << 8)));
-        float q;
-        if (QT == 0) {
-            q = (float)(int8_t)blk[2 + j];
-        } else {
-            const uint8_t byte = blk[2 + (j & 15)];
-            q = (float)((j < 16 ? (byte & 0x0F) : (byte >> 4)) - 8);
-        }
-        out[e] = q * d;
-    }
+    for (; e < n_elems; e += stride)
+        out[e] = homura::dequant_element<QF>(blocks + (e >> 5) * BlockTraits<QT>::BYTES, (int)(e & 31));
 }
 
 template <int QT>

@@ -15,7 +15,10 @@
 // V are the cache's own bf16 rows.
 #include "prefill.h"
 
+#include <algorithm>
+
 #include "gemm_bf16_mfma.h"
+#include "quant_formats.h"
 
 namespace {
 
@@ -112,6 +115,58 @@ __device__ __forceinline__ void split_store4(uint16_t *__restrict__ row, int dim
     }
 }
 
+// The activation a K-quant product sees (reference emit_quant.rs:422-466): every 256-wide block is
+// quantised to Q8_K, q = clamp(roundeven(x * (127 / amax)), +-127) with scale amax / 127; the integer
+// dot products of the decode kernels equal a plain dot product with scale * q. A wavefront holds one
+// block, four consecutive values per lane.
+__device__ __forceinline__ f32x4 q8k_round_trip(f32x4 v) {
+    float amax = fmaxf(fmaxf(fabsf(v[0]), fabsf(v[1])), fmaxf(fabsf(v[2]), fabsf(v[3])));
+    amax = wave_max(amax);
+    const float iscale = amax == 0.f ? 0.f : __fdiv_rn(127.0f, amax);
+    const float d = __fdiv_rn(amax, 127.0f);
+    f32x4 y;
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        float r = rintf(__fmul_rn(v[k], iscale));
+        r = fmaxf(fminf(r, 127.0f), -127.0f);
+        y[k] = __fmul_rn(d, r);
+    }
+    return y;
+}
+
+// rows of f32 -> split rows, four consecutive elements per thread (dim % 4 == 0; % 256 with q8k)
+__global__ void split_rows4_kernel(const float *__restrict__ x, uint16_t *__restrict__ out, int dim, size_t n, int pieces,
+                                   int q8k) {
+    const size_t i = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;
+    if (i >= n) return;
+    f32x4 v = *reinterpret_cast<const f32x4 *>(x + i);
+    if (q8k) v = q8k_round_trip(v);
+    const size_t row = i / dim;
+    split_store4(out + row * pieces * dim, dim, (int)(i % dim), v, pieces);
+}
+
+// A quantised weight matrix, raw blocks [N][K / block], as a split matrix of its f32 values: row n goes
+// to row n * row_mult + row_off of out ([.][3 K]). Eight consecutive weights per thread.
+template <int QF>
+__global__ __launch_bounds__(256) void dequant_split_kernel(const uint8_t *__restrict__ blocks,
+                                                            uint16_t *__restrict__ out, int K, size_t n8, int row_mult,
+                                                            int row_off) {
+    constexpr int BB = QuantFormatTraits<QF>::BYTES, BE = QuantFormatTraits<QF>::ELEMS;
+    const size_t t = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= n8) return;
+    const size_t e = t * 8, row = e / K;
+    const int c = (int)(e % K);
+    const uint8_t *blk = blocks + (e / BE) * BB;  // rows are whole blocks: K % BE == 0
+    float f[8];
+#pragma unroll
+    for (int j = 0; j < 8; j++) f[j] = dequant_element<QF>(blk, (int)(e % BE) + j);
+    bf16x8 pc[3];
+    split8<3>(f, pc);
+    uint16_t *o = out + (row * row_mult + row_off) * 3 * (size_t)K + c;
+#pragma unroll
+    for (int p = 0; p < 3; p++) *reinterpret_cast<bf16x8 *>(o + (size_t)p * K) = pc[p];
+}
+
 // One workgroup per row, four consecutive elements per thread and step (dim % 4 == 0); the arithmetic
 // of the decode path's RMSNorm kernel (reference src/graph_builder/emit_linalg.rs:7-26; Residual+Norm,
 // src/hf/emitter.rs:787-790).
@@ -119,7 +174,7 @@ __global__ __launch_bounds__(256) void rmsnorm_split_kernel(const float *__restr
                                                             int res_parts, size_t res_stride,
                                                             const float *__restrict__ w, uint16_t *__restrict__ out,
                                                             float *__restrict__ resid_out, int dim, float eps,
-                                                            int pieces) {
+                                                            int pieces, int q8k) {
     __shared__ float red[4];
     const size_t base = (size_t)blockIdx.x * dim;
     constexpr int KEEP = 2;  // rows up to 2048 wide stay in registers between the two passes
@@ -152,6 +207,7 @@ __global__ __launch_bounds__(256) void rmsnorm_split_kernel(const float *__restr
         f32x4 y;
 #pragma unroll
         for (int k = 0; k < 4; k++) y[k] = (v[k] * inv) * wv[k];
+        if (q8k) y = q8k_round_trip(y);  // dim % 256 == 0: a wavefront's 256 values are one block
         split_store4(o, dim, i, y, pieces);
     }
 }
@@ -159,7 +215,7 @@ __global__ __launch_bounds__(256) void rmsnorm_split_kernel(const float *__restr
 // silu(gate) * up (reference src/graph_builder/emit_arithmetic.rs:101-107, src/hf/emitter.rs:797-799);
 // four outputs per thread (inter % 4 == 0)
 __global__ void silu_mul_split_kernel(const float *__restrict__ gu, int parts, size_t stride, uint16_t *__restrict__ out,
-                                      int inter, size_t n, int pieces) {
+                                      int inter, size_t n, int pieces, int q8k) {
     const size_t i = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;
     if (i >= n) return;
     const size_t row = i / inter;
@@ -168,6 +224,7 @@ __global__ void silu_mul_split_kernel(const float *__restrict__ gu, int parts, s
     f32x4 y;
 #pragma unroll
     for (int k = 0; k < 4; k++) y[k] = (g[k] / (1.0f + expf(-g[k]))) * u[k];
+    if (q8k) y = q8k_round_trip(y);
     split_store4(out + row * pieces * inter, inter, (int)(i % inter), y, pieces);
 }
 
@@ -460,27 +517,72 @@ __global__ __launch_bounds__(AT_THREADS) void prefill_attn_kernel(PrefillAttnArg
 namespace homura {
 
 int rmsnorm_split_launch(hm_ctx *ctx, const float *d_x, const float *d_res, int res_parts, const float *d_w,
-                         uint16_t *d_out_split, int pieces, float *d_resid_out, int rows, int dim, float eps) {
+                         uint16_t *d_out_split, int pieces, float *d_resid_out, int rows, int dim, float eps, bool q8k) {
+    HM_REQUIRE(ctx, !q8k || dim % 256 == 0, "rmsnorm_split: Q8_K activations need dim %% 256 == 0 (dim=%d)", dim);
     HM_REQUIRE(ctx, d_x && d_w && d_out_split, "rmsnorm_split: NULL pointer");
     HM_REQUIRE(ctx, rows > 0 && dim > 0 && dim % 4 == 0 && pieces >= 1 && pieces <= 3 && res_parts >= 1,
                "rmsnorm_split: bad shape (dim %% 4 == 0 needed)");
     HM_REQUIRE(ctx, ((uintptr_t)d_x % 16) == 0 && ((uintptr_t)d_w % 16) == 0 && ((uintptr_t)d_out_split % 8) == 0 &&
                         ((uintptr_t)d_res % 16) == 0 && ((uintptr_t)d_resid_out % 16) == 0, "rmsnorm_split: misaligned buffer");
     hipLaunchKernelGGL(rmsnorm_split_kernel, dim3(rows), dim3(256), 0, ctx->stream, d_x, d_res, res_parts,
-                       (size_t)rows * dim, d_w, d_out_split, d_resid_out, dim, eps, pieces);
+                       (size_t)rows * dim, d_w, d_out_split, d_resid_out, dim, eps, pieces, q8k ? 1 : 0);
     HM_LAUNCH_CHECK(ctx);
     return HM_OK;
 }
 
 int silu_mul_split_launch(hm_ctx *ctx, const float *d_gu, int parts, uint16_t *d_out_split, int pieces, int rows,
-                          int inter) {
+                          int inter, bool q8k) {
+    HM_REQUIRE(ctx, !q8k || inter % 256 == 0, "silu_mul_split: Q8_K activations need a width %% 256 == 0 (%d)", inter);
     HM_REQUIRE(ctx, d_gu && d_out_split, "silu_mul_split: NULL pointer");
     HM_REQUIRE(ctx, rows > 0 && inter > 0 && inter % 4 == 0 && pieces >= 1 && pieces <= 3 && parts >= 1,
                "silu_mul_split: bad shape (intermediate size %% 4 == 0 needed)");
     HM_REQUIRE(ctx, ((uintptr_t)d_gu % 16) == 0 && ((uintptr_t)d_out_split % 8) == 0, "silu_mul_split: misaligned buffer");
     const size_t n = (size_t)rows * inter;
     hipLaunchKernelGGL(silu_mul_split_kernel, dim3((unsigned)((n / 4 + 255) / 256)), dim3(256), 0, ctx->stream, d_gu, parts,
-                       2 * n, d_out_split, inter, n, pieces);
+                       2 * n, d_out_split, inter, n, pieces, q8k ? 1 : 0);
+    HM_LAUNCH_CHECK(ctx);
+    return HM_OK;
+}
+
+int split_rows_launch(hm_ctx *ctx, const float *d_x, uint16_t *d_out_split, int pieces, size_t rows, int dim, bool q8k) {
+    HM_REQUIRE(ctx, d_x && d_out_split, "split_rows: NULL pointer");
+    HM_REQUIRE(ctx, rows > 0 && dim > 0 && dim % 4 == 0 && pieces >= 1 && pieces <= 3, "split_rows: bad shape (dim %% 4 == 0 needed)");
+    HM_REQUIRE(ctx, !q8k || dim % 256 == 0, "split_rows: Q8_K activations need dim %% 256 == 0 (dim=%d)", dim);
+    HM_REQUIRE(ctx, ((uintptr_t)d_x % 16) == 0 && ((uintptr_t)d_out_split % 8) == 0, "split_rows: misaligned buffer");
+    const size_t n = rows * dim;
+    HM_REQUIRE(ctx, (n / 4 + 255) / 256 <= 0x7fffffffULL, "split_rows: too many elements");
+    hipLaunchKernelGGL(split_rows4_kernel, dim3((unsigned)((n / 4 + 255) / 256)), dim3(256), 0, ctx->stream, d_x, d_out_split,
+                       dim, n, pieces, q8k ? 1 : 0);
+    HM_LAUNCH_CHECK(ctx);
+    return HM_OK;
+}
+
+int dequant_split_launch(hm_ctx *ctx, int hm_dtype, const uint8_t *d_blocks, int N, int K, uint16_t *d_out_split,
+                         int row_mult, int row_off) {
+    HM_REQUIRE(ctx, d_blocks && d_out_split, "dequant_split: NULL pointer");
+    const bool kq = hm_dtype == HM_DTYPE_Q4_K || hm_dtype == HM_DTYPE_Q6_K;
+    HM_REQUIRE(ctx, N > 0 && K > 0 && K % (kq ? 256 : 32) == 0 && row_mult >= 1 && row_off >= 0 && row_off < row_mult,
+               "dequant_split: bad shape (N=%d K=%d)", N, K);
+    HM_REQUIRE(ctx, ((uintptr_t)d_out_split % 16) == 0, "dequant_split: misaligned output");
+    const size_t n8 = (size_t)N * K / 8;
+    const dim3 grid((unsigned)((n8 + 255) / 256));
+    HM_REQUIRE(ctx, (n8 + 255) / 256 <= 0x7fffffffULL, "dequant_split: matrix too large");
+    switch (hm_dtype) {
+    case HM_DTYPE_Q8_0:
+        hipLaunchKernelGGL((dequant_split_kernel<QF_Q8_0>), grid, dim3(256), 0, ctx->stream, d_blocks, d_out_split, K, n8, row_mult, row_off);
+        break;
+    case HM_DTYPE_Q4_0:
+        hipLaunchKernelGGL((dequant_split_kernel<QF_Q4_0>), grid, dim3(256), 0, ctx->stream, d_blocks, d_out_split, K, n8, row_mult, row_off);
+        break;
+    case HM_DTYPE_Q4_K:
+        hipLaunchKernelGGL((dequant_split_kernel<QF_Q4_K>), grid, dim3(256), 0, ctx->stream, d_blocks, d_out_split, K, n8, row_mult, row_off);
+        break;
+    case HM_DTYPE_Q6_K:
+        hipLaunchKernelGGL((dequant_split_kernel<QF_Q6_K>), grid, dim3(256), 0, ctx->stream, d_blocks, d_out_split, K, n8, row_mult, row_off);
+        break;
+    default:
+        return hm_set_error(ctx, HM_ERR_INVALID, "dequant_split: dtype %d is not a block format", hm_dtype);
+    }
     HM_LAUNCH_CHECK(ctx);
     return HM_OK;
 }
@@ -531,10 +633,35 @@ extern "C" int hm_gemm_f32_bf16_nk(hm_ctx *ctx, const float *d_x_mk, const uint1
     const size_t n = (size_t)M * K;
     HM_REQUIRE(ctx, n * 6 <= ctx->workspace_bytes, "hm_gemm_f32_bf16_nk: M * K = %zu activations exceed the workspace", n);
     uint16_t *split = (uint16_t *)ctx->workspace;
-    hipLaunchKernelGGL(split_rows_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, ctx->stream, d_x_mk, split, K, n,
-                       3);
-    HM_LAUNCH_CHECK(ctx);
+    const int rc = homura::split_rows_launch(ctx, d_x_mk, split, 3, (size_t)M, K);
+    if (rc != HM_OK) return rc;
     return homura::gemm_split_nk(ctx, split, 3, d_w_nk, d_out, M, K, N);
+}
+
+extern "C" int hm_gemm_f32_quant_nk(hm_ctx *ctx, const float *d_x_mk, const uint8_t *d_w_blocks, int dtype, float *d_out,
+                                    int M, int K, int N) {
+    HM_CHECK_CTX(ctx);
+    HM_REQUIRE(ctx, d_x_mk && d_w_blocks && d_out, "hm_gemm_f32_quant_nk: NULL pointer");
+    const bool kq = dtype == HM_DTYPE_Q4_K || dtype == HM_DTYPE_Q6_K;
+    HM_REQUIRE(ctx, kq || dtype == HM_DTYPE_Q8_0 || dtype == HM_DTYPE_Q4_0, "hm_gemm_f32_quant_nk: dtype %d is not a block format", dtype);
+    HM_REQUIRE(ctx, M > 0 && N > 0 && K > 0 && K % (kq ? 256 : 64) == 0,
+               "hm_gemm_f32_quant_nk: need M, N > 0 and K %% %d == 0 (K=%d)", kq ? 256 : 64, K);
+    // workspace: the split activations, then as many split weight rows as fit (a multiple of the tile)
+    const size_t a_bytes = ((size_t)M * K * 6 + 255) / 256 * 256;
+    HM_REQUIRE(ctx, a_bytes + (size_t)128 * K * 6 <= ctx->workspace_bytes,
+               "hm_gemm_f32_quant_nk: M * K = %zu activations exceed the workspace", (size_t)M * K);
+    uint16_t *a_split = (uint16_t *)ctx->workspace;
+    uint16_t *w_split = (uint16_t *)((char *)ctx->workspace + a_bytes);
+    const int slab = (int)std::min<size_t>((size_t)N, (ctx->workspace_bytes - a_bytes) / ((size_t)K * 6) / 128 * 128);
+    int rc = homura::split_rows_launch(ctx, d_x_mk, a_split, 3, (size_t)M, K, kq);
+    const size_t block_bytes = dtype == HM_DTYPE_Q8_0 ? 34 : dtype == HM_DTYPE_Q4_0 ? 18 : dtype == HM_DTYPE_Q4_K ? 144 : 210;
+    const size_t row_bytes = (size_t)K / (kq ? 256 : 32) * block_bytes;
+    for (int n0 = 0; n0 < N && rc == HM_OK; n0 += slab) {
+        const int rows = std::min(slab, N - n0);
+        rc = homura::dequant_split_launch(ctx, dtype, d_w_blocks + (size_t)n0 * row_bytes, rows, K, w_split);
+        if (rc == HM_OK) rc = homura::gemm_split_split_nk(ctx, a_split, w_split, d_out + n0, M, K, rows, 1, nullptr, N);
+    }
+    return rc;
 }
 
 extern "C" int hm_gqa_prefill_attn(hm_ctx *ctx, const float *d_q, const uint16_t *d_kcache, const uint16_t *d_vcache,

@@ -184,6 +184,10 @@ class Context:
     def gemm_f32_bf16_nk(self, x, w_nk, out, M, K, N):
         self._check(self.lib.hm_gemm_f32_bf16_nk(self.h, x.ptr, w_nk.ptr, out.ptr, M, K, N))
 
+    def gemm_f32_quant_nk(self, x, w_blocks, dtype, out, M, K, N):
+        """Prompt-pass product with a block-quantised weight matrix (dtype: DTYPE_Q8_0 / Q4_0 / Q4_K / Q6_K)."""
+        self._check(self.lib.hm_gemm_f32_quant_nk(self.h, x.ptr, w_blocks.ptr, dtype, out.ptr, M, K, N))
+
     def gqa_prefill_attn(self, q, kc, vc, out, S, H, kvh, hd, max_len, past, scale):
         self._check(self.lib.hm_gqa_prefill_attn(self.h, q.ptr, kc.ptr, vc.ptr, out.ptr, S, H, kvh, hd,
                                                  max_len, past, scale))

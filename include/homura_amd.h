@@ -142,6 +142,20 @@ int hm_gemm_bf16_nk(hm_ctx *ctx, const uint16_t *d_a_mk, const uint16_t *d_b_nk,
 int hm_gemm_f32_bf16_nk(hm_ctx *ctx, const float *d_x_mk, const uint16_t *d_w_nk, float *d_out, int M, int K,
                         int N);
 
+/* The reference's quantised matmul at seq > 1 (emit_quant_matmul_kernel,
+ * src/hf/emitter_quant.rs:675-702; src/graph_builder/emit_quant.rs): x f32 [M,K] times a block-
+ * quantised W (raw GGUF blocks [N][K / block], dtype HM_DTYPE_Q8_0 / Q4_0 / Q4_K / Q6_K), out f32
+ * [M,N], on the matrix cores. The weights are dequantised to f32 with the reference's arithmetic and,
+ * like the activations, carried as three bf16 pieces; the six piece products that matter are
+ * accumulated in f32, so the result is the f32 product up to rounding. For the K-quants every
+ * activation row first goes through the Q8_K quantisation the reference applies (per 256-wide block:
+ * scale amax / 127, round half to even, clamp +-127), and the product is taken with scale * q, which
+ * is what its integer dot products add up to. K % 64 == 0 (K % 256 for the K-quants); the split
+ * activations (M * K * 6 bytes) and at least 128 split weight rows must fit in the context
+ * workspace. */
+int hm_gemm_f32_quant_nk(hm_ctx *ctx, const float *d_x_mk, const uint8_t *d_w_blocks, int dtype, float *d_out,
+                         int M, int K, int N);
+
 /* ── KV cache + attention ──────────────────────────────────────────────────── */
 
 /* KvCache::append_key / append_value (src/runtime.rs:521-568) on an HBM cache

@@ -237,6 +237,45 @@ def test_gemm_bf16_ragged_edges(ctx, oracle, M, K, N, layout):
         buf.free()
 
 
+@pytest.mark.parametrize("kind", ["q8_0", "q4_0", "q4_k", "q6_k"])
+@pytest.mark.parametrize("M,K,N", [(200, 1024, 1000), (5, 256, 130), (64, 2048, 6000), (512, 512, 256)])
+def test_gemm_f32_quantised_weights(ctx, oracle, kind, M, K, N):
+    """The quantised matmul at seq > 1 on the matrix cores against the oracle's row-by-row product (the
+    decode formula: f32 activations for Q8_0 / Q4_0, Q8_K activations and integer sums for the
+    K-quants). Both sides add the same products in f32, in different orders. N = 6000 at K = 2048 does
+    not fit the workspace in one piece and goes through in slabs."""
+    say(f"gemm_f32_quant_nk {kind} M={M} K={K} N={N}")
+    import homura_amd
+    make = {"q8_0": synth.q8_0_blocks, "q4_0": synth.q4_0_blocks, "q4_k": synth.q4_k_blocks, "q6_k": synth.q6_k_blocks}[kind]
+    per = 32 if kind in ("q8_0", "q4_0") else 256
+    raw = make(41, N * K // per, 0.01) if per == 32 else make(41, N * K // per)
+    x = synth.normal_f32(42, M * K, 1.0).reshape(M, K)
+    want = getattr(oracle, "gemv_" + kind)(x, raw, M, K, N)
+    # float64 truth: dequantised weights times the activation the format multiplies with
+    w64 = getattr(oracle, "dequant_" + kind)(raw).reshape(N, K).astype(np.float64)
+    x64 = x.astype(np.float64)
+    if per == 256:
+        for m in range(M):
+            for kb in range(K // 256):
+                q, d, _ = oracle.quantize_q8_k(x[m, kb * 256:(kb + 1) * 256])
+                x64[m, kb * 256:(kb + 1) * 256] = np.float64(d) * q.astype(np.float64)
+    truth = x64 @ w64.T
+    dtype = {"q8_0": homura_amd.DTYPE_Q8_0, "q4_0": homura_amd.DTYPE_Q4_0, "q4_k": homura_amd.DTYPE_Q4_K,
+             "q6_k": homura_amd.DTYPE_Q6_K}[kind]
+    dx, dw, dout = ctx.to_device(x), ctx.to_device(raw), ctx.empty(M * N)
+    ctx.gemm_f32_quant_nk(dx, dw, dtype, dout, M, K, N)
+    got = dout.download(np.float32, (M, N))
+    # error in units of a typical output, sqrt(K) rms(x) rms(w): f32 accumulation leaves about 1e-6;
+    # a dropped first-order piece product would leave 1e-3, a second-order one 1e-5
+    unit = np.sqrt(K) * np.sqrt(np.mean(x64 ** 2)) * np.sqrt(np.mean(w64 ** 2))
+    e_gpu, e_orc = np.abs(got - truth).max() / unit, np.abs(want - truth).max() / unit
+    say(f"  error / typical output: gpu {e_gpu:.2e}, oracle {e_orc:.2e}; rel_err vs oracle {rel_err(got, want):.2e}")
+    assert e_gpu < 4e-6
+    assert rel_err(got, want) < 2e-3
+    for b in (dx, dw, dout):
+        b.free()
+
+
 @pytest.mark.parametrize("M,K,N", [(512, 1024, 4096), (1, 1024, 1024), (77, 448, 576), (300, 3072, 1024)])
 def test_gemm_f32_activations_bf16_weights(ctx, oracle, M, K, N):
     """The reference's mixed matmul at seq > 1: f32 activations, bf16 weights. The activation goes
