@@ -135,6 +135,7 @@ class HfModel {
         static constexpr int MAX_PARTS = 8;  // K slices a projection result may come in
         int rows = 0;
         Buffer ids, h, resid, split, qkv, proj_out, gate_up, logits;
+        Buffer wsplit;  // block formats: the matrices of one group of projections as three bf16 pieces per weight
     };
     PrefillScratch pf_;
     struct SamplerScratch { Buffer work, counts, token, list; int list_cap = 0; } sampler_;

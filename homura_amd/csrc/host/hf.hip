@@ -1181,8 +1181,20 @@ int HfModel::run_kv(const int64_t *h_ids, int n_ids, float *h_logits) {
 // ── prefill pass ─────────────────────────────────────────────────────────────
 
 bool HfModel::prefill_available() const {
-    return finalized_ && weight_dtype_ == DType::BF16 && (cfg_.head_dim() == 64 || cfg_.head_dim() == 128) &&
-           cfg_.hidden_size % 32 == 0 && cfg_.q_dim() % 32 == 0 && cfg_.intermediate_size % 32 == 0;
+    if (!finalized_ || (cfg_.head_dim() != 64 && cfg_.head_dim() != 128)) return false;
+    const int hidden = cfg_.hidden_size, qd = cfg_.q_dim(), inter = cfg_.intermediate_size;
+    if (weight_dtype_ == DType::BF16) return hidden % 32 == 0 && qd % 32 == 0 && inter % 32 == 0;
+    if (!dtype_is_quantized(weight_dtype_)) return false;
+    // Block formats: K tiles of 64; the matrices that share an activation (q|k|v, gate|up) must agree
+    // on what they multiply with, f32 rows (Q8_0, Q4_0) or Q8_K rows (the K-quants).
+    if (hidden % 64 != 0 || qd % 64 != 0 || inter % 64 != 0) return false;
+    auto kq = [&](int l, int j) { const DType t = proj_dtype(l, j); return t == DType::Q4_K || t == DType::Q6_K; };
+    for (int l = 0; l < cfg_.num_hidden_layers; l++) {
+        if (kq(l, 0) != kq(l, 1) || kq(l, 0) != kq(l, 2) || kq(l, 4) != kq(l, 5)) return false;
+        if (((kq(l, 0) || kq(l, 4)) && hidden % 256 != 0) || (kq(l, 3) && qd % 256 != 0) || (kq(l, 6) && inter % 256 != 0))
+            return false;
+    }
+    return true;
 }
 
 const float *HfModel::weight_f32(const std::string &name) const {
@@ -1193,7 +1205,7 @@ const float *HfModel::weight_f32(const std::string &name) const {
 int HfModel::prefill(const int64_t *h_ids, int n_ids, float *h_logits) {
     if (!finalized_) return hm_set_error(ctx_, HM_ERR_STATE, "model not finalized");
     if (!prefill_available())
-        return hm_set_error(ctx_, HM_ERR_INVALID, "prefill: needs the bf16 plan with head_dim 64 or 128 and widths that are multiples of 32");
+        return hm_set_error(ctx_, HM_ERR_INVALID, "prefill: needs head_dim 64 or 128 and widths that are multiples of 32 (bf16) or 64 (block formats, whose q|k|v and gate|up must each be of one kind)");
     if (n_ids <= 0 || !h_ids) return hm_set_error(ctx_, HM_ERR_INVALID, "prefill: no input ids");
     if (kv_cache_len() + n_ids > max_seq_len_)
         return hm_set_error(ctx_, HM_ERR_STATE, "KV cache full (%d + %d > %d)", kv_cache_len(), n_ids, max_seq_len_);
@@ -1216,6 +1228,7 @@ int HfModel::prefill_chunk(const int32_t *h_ids, int n, float *h_logits) {
     const int qd = c.q_dim(), kvd = c.kv_dim(), nqkv = qd + 2 * kvd;
     const float eps = (float)c.rms_norm_eps;
     PrefillScratch &p = pf_;
+    const bool quant = dtype_is_quantized(weight_dtype_);
     if (p.rows < n) {
         const int rows = std::max(n, 128);
         const int64_t widest = std::max<int64_t>(std::max(hidden, qd), inter);
@@ -1229,6 +1242,11 @@ int HfModel::prefill_chunk(const int32_t *h_ids, int n, float *h_logits) {
         p.proj_out = Buffer::alloc(ctx_, {PrefillScratch::MAX_PARTS, rows, hidden}, DType::F32);
         p.gate_up = Buffer::alloc(ctx_, {PrefillScratch::MAX_PARTS, rows, 2 * (int64_t)inter}, DType::F32);
         if (!p.ids || !p.h || !p.resid || !p.split || !p.qkv || !p.proj_out || !p.gate_up) return HM_ERR_OOM;
+        if (quant) {  // the largest group of matrices of a layer as three bf16 pieces per weight
+            const int64_t most = std::max(std::max((int64_t)nqkv * hidden, (int64_t)hidden * qd), 2 * (int64_t)inter * hidden);
+            p.wsplit = Buffer::alloc(ctx_, {3 * most}, DType::BF16);
+            if (!p.wsplit) return HM_ERR_OOM;
+        }
         p.rows = rows;
     }
     if (h_logits && !p.logits) {
@@ -1242,9 +1260,41 @@ int HfModel::prefill_chunk(const int32_t *h_ids, int n, float *h_logits) {
     float *h = p.h.as<float>(), *resid = p.resid.as<float>(), *qkv = p.qkv.as<float>();
     float *proj_out = p.proj_out.as<float>(), *gate_up = p.gate_up.as<float>();
     uint16_t *split = p.split.as<uint16_t>();
-    const int np = prefill_pieces_;
+    const int np = quant ? 3 : prefill_pieces_;
     const int MP = PrefillScratch::MAX_PARTS;
     int parts = 1;  // K slices of the latest projection
+    uint16_t *wsplit = quant ? p.wsplit.as<uint16_t>() : nullptr;
+    static const char *const proj_name[7] = {"self_attn.q_proj.weight", "self_attn.k_proj.weight", "self_attn.v_proj.weight",
+                                             "self_attn.o_proj.weight", "mlp.gate_proj.weight", "mlp.up_proj.weight",
+                                             "mlp.down_proj.weight"};
+    const int proj_n[7] = {qd, kvd, kvd, hidden, inter, inter, hidden};
+    // K-quant matrices multiply with Q8_K rows (reference emit_quant.rs:422-466), everything else with the f32 rows
+    auto q8k = [&](int l, int which) {
+        const DType t = proj_dtype(l, which);
+        return quant && (t == DType::Q4_K || t == DType::Q6_K);
+    };
+    // out[n][N] (N = the members' rows together) = split x W^T for the projections first .. first + count - 1
+    // of layer l, which share the activation in `split`. bf16: the packed stream matrix. Block formats
+    // (reference emit_quant_matmul_kernel, src/hf/emitter_quant.rs:675-702): the members are
+    // dequantised into wsplit one under the other, or row-interleaved for gate|up, which is the order
+    // the packed bf16 matrices have.
+    auto project = [&](int l, int first, int count, const Buffer &packed, int K, float *out) -> int {
+        int N = 0;
+        for (int j = first; j < first + count; j++) N += proj_n[j];
+        if (!quant) return gemm_split_nk(ctx_, split, np, packed.as<uint16_t>(), out, n, K, N, MP, &parts);
+        const bool interleave = first == 4 && count == 2;
+        int row = 0;
+        for (int j = first; j < first + count; j++) {
+            auto it = slot_by_name_.find("model.layers." + std::to_string(l) + "." + proj_name[j]);
+            if (it == slot_by_name_.end()) return hm_set_error(ctx_, HM_ERR_STATE, "prefill: weight %s missing", proj_name[j]);
+            const int rc = dequant_split_launch(ctx_, (int)proj_dtype(l, j), weight_bufs_[it->second].as<uint8_t>(), proj_n[j], K,
+                                                interleave ? wsplit : wsplit + (size_t)row * 3 * K, interleave ? 2 : 1,
+                                                interleave ? j - first : 0);
+            if (rc != HM_OK) return rc;
+            row += proj_n[j];
+        }
+        return gemm_split_split_nk(ctx_, split, wsplit, out, n, K, N, MP, &parts);
+    };
     rc = embed_launch(ctx_, nullptr, p.ids.as<int32_t>(), weight_f32("model.embed_tokens.weight"), h, n, vocab, hidden);
     if (rc != HM_OK) return rc;
     // The hidden state entering a layer is x [+ res]: the embedding for the first layer, afterwards the
@@ -1257,8 +1307,8 @@ int HfModel::prefill_chunk(const int32_t *h_ids, int n, float *h_logits) {
         const LayerPacked &lp = packed_[l];
         // QKV kernel (reference src/hf/emitter.rs:549-673)
         rc = rmsnorm_split_launch(ctx_, x, res, res_parts, weight_f32(pre + "input_layernorm.weight"), split, np,
-                                  res ? h : nullptr, n, hidden, eps);
-        if (rc == HM_OK) rc = gemm_split_nk(ctx_, split, np, lp.qkv.as<uint16_t>(), qkv, n, hidden, nqkv, MP, &parts);
+                                  res ? h : nullptr, n, hidden, eps, q8k(l, 0));
+        if (rc == HM_OK) rc = project(l, 0, 3, lp.qkv, hidden, qkv);
         if (rc != HM_OK) return rc;
         QkvPostArgs qa;
         qa.qkv = qkv;
@@ -1287,7 +1337,13 @@ int HfModel::prefill_chunk(const int32_t *h_ids, int n, float *h_logits) {
         aa.ldq = nqkv;
         aa.kcache = kv->key_ptr(l);
         aa.vcache = kv->value_ptr(l);
-        aa.out_split = split;
+        // a K-quant O projection wants whole rows for its Q8_K blocks: the heads' outputs go out as f32
+        // (into the idle gate|up scratch) and are split afterwards
+        const bool o_q8k = q8k(l, 3);
+        if (o_q8k)
+            aa.out_f32 = gate_up;
+        else
+            aa.out_split = split;
         aa.S = n;
         aa.H = H;
         aa.kvh = kvh;
@@ -1297,13 +1353,14 @@ int HfModel::prefill_chunk(const int32_t *h_ids, int n, float *h_logits) {
         aa.scale = (float)(1.0 / std::sqrt((double)hd));
         aa.pieces = np;
         if ((rc = prefill_attn_launch(ctx_, aa)) != HM_OK) return rc;
-        if ((rc = gemm_split_nk(ctx_, split, np, lp.o.as<uint16_t>(), proj_out, n, qd, hidden, MP, &parts)) != HM_OK) return rc;
+        if (o_q8k && (rc = split_rows_launch(ctx_, gate_up, split, np, (size_t)n, qd, true)) != HM_OK) return rc;
+        if ((rc = project(l, 3, 1, lp.o, qd, proj_out)) != HM_OK) return rc;
         // MLP kernel (reference src/hf/emitter.rs:767-822); h holds the layer's input by now
         rc = rmsnorm_split_launch(ctx_, h, proj_out, parts, weight_f32(pre + "post_attention_layernorm.weight"), split, np,
-                                  resid, n, hidden, eps);
-        if (rc == HM_OK) rc = gemm_split_nk(ctx_, split, np, lp.gate_up.as<uint16_t>(), gate_up, n, hidden, 2 * inter, MP, &parts);
-        if (rc == HM_OK) rc = silu_mul_split_launch(ctx_, gate_up, parts, split, np, n, inter);
-        if (rc == HM_OK) rc = gemm_split_nk(ctx_, split, np, lp.down.as<uint16_t>(), proj_out, n, inter, hidden, MP, &parts);
+                                  resid, n, hidden, eps, q8k(l, 4));
+        if (rc == HM_OK) rc = project(l, 4, 2, lp.gate_up, hidden, gate_up);
+        if (rc == HM_OK) rc = silu_mul_split_launch(ctx_, gate_up, parts, split, np, n, inter, q8k(l, 6));
+        if (rc == HM_OK) rc = project(l, 6, 1, lp.down, inter, proj_out);
         if (rc != HM_OK) return rc;
         x = resid;
         res = proj_out;
@@ -1311,7 +1368,20 @@ int HfModel::prefill_chunk(const int32_t *h_ids, int n, float *h_logits) {
     }
     if (h_logits) {  // LM head (reference src/hf/emitter.rs:828-862) for every row
         rc = rmsnorm_split_launch(ctx_, x, res, res_parts, weight_f32("model.norm.weight"), split, np, nullptr, n, hidden, eps);
-        if (rc == HM_OK) rc = gemm_split_nk(ctx_, split, np, lm_head_packed_.as<uint16_t>(), p.logits.as<float>(), n, hidden, vocab);
+        if (rc == HM_OK && !quant)
+            rc = gemm_split_nk(ctx_, split, np, lm_head_packed_.as<uint16_t>(), p.logits.as<float>(), n, hidden, vocab);
+        if (rc == HM_OK && quant) {
+            // the quantised plan's LM head is f32 [vocab][hidden] (reference src/hf/emitter_quant.rs:1390-1437):
+            // slabs of its rows become bf16 pieces in wsplit, as many as fit
+            const int slab = (int)std::min<int64_t>(vocab, (int64_t)(p.wsplit.bytes() / 2) / (3 * (int64_t)hidden) / 128 * 128);
+            if (slab <= 0) return hm_set_error(ctx_, HM_ERR_STATE, "prefill: weight scratch too small for the LM head");
+            for (int v0 = 0; v0 < vocab && rc == HM_OK; v0 += slab) {
+                const int rows = std::min(slab, vocab - v0);
+                rc = split_rows_launch(ctx_, lm_head_packed_.as<float>() + (size_t)v0 * hidden, wsplit, 3, (size_t)rows, hidden);
+                if (rc == HM_OK)
+                    rc = gemm_split_split_nk(ctx_, split, wsplit, p.logits.as<float>() + v0, n, hidden, rows, 1, nullptr, vocab);
+            }
+        }
         if (rc == HM_OK) rc = hm_download(ctx_, h_logits, p.logits.ptr(), (size_t)n * vocab * 4);
         if (rc != HM_OK) return rc;
     }

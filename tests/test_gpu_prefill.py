@@ -109,15 +109,99 @@ def test_prefill_in_chunks_and_cache_limits(ctx):
     gm.close()
 
 
-def test_prefill_needs_the_bf16_plan(ctx):
-    cfg = synth_model.TINY_LLAMA
+def _quant_case(which):
+    """(config, 7 projection types per layer) of a block-quantised model."""
+    import dataclasses
+    K = synth_model.TINY_K
+    L = K.num_hidden_layers
+    return {
+        "q8_0": (synth_model.TINY_LLAMA, [2] * 7 * synth_model.TINY_LLAMA.num_hidden_layers),
+        # 3000 rows of LM head do not fit the weight scratch at once: three slabs
+        "q4_0_wide_vocab": (dataclasses.replace(synth_model.TINY_LLAMA, vocab_size=3000),
+                            [3] * 7 * synth_model.TINY_LLAMA.num_hidden_layers),
+        "q4_k": (K, [5] * 7 * L),
+        "q6_k": (K, [6] * 7 * L),
+        "q4_k_m_mix": (K, synth_model.q4_k_m_mix(K)),
+        # f32 rows for q|k|v and down, Q8_K rows for o and gate|up
+        "q8_0_and_k_quants_by_group": (K, [2, 2, 2, 5, 6, 5, 3] * L),
+    }[which]
+
+
+@pytest.mark.parametrize("which,past,n", [("q8_0", 0, 37), ("q4_0_wide_vocab", 30, 70), ("q4_k", 0, 50), ("q6_k", 17, 33),
+                                          ("q4_k_m_mix", 40, 130), ("q8_0_and_k_quants_by_group", 0, 64)])
+def test_quantised_prefill_logits_and_following_decode(ctx, which, past, n):
+    """The prompt pass of the block-quantised plans (dequantised weights and, for the K-quants, Q8_K
+    activations as bf16 pieces on the matrix cores) against the oracle's token-by-token steps."""
+    cfg, mix = _quant_case(which)
+    weights = synth_model.synth_weights(cfg, 1717, has_qk_norm=False, proj_dtypes=mix)
+    L = past + n + 40
+    gm = synth_model.build_model(ctx, cfg, weights, L, has_qk_norm=False, proj_dtypes=mix)
+    om = mf.build_oracle_model(cfg, weights, L, has_qk_norm=False, proj_dtypes=mix)
+    if past:
+        kv = synth_model.synth_kv(cfg, 7, past)
+        gm.init_kv_cache(kv, past)
+        mf.oracle_init_kv(om, kv)
+    ids = synth.token_ids(8, n + 1, cfg.vocab_size)
+    got = gm.prefill(ids[:n])
+    want = np.concatenate([om.run_kv(ids[i:i + 1]) for i in range(n)])
+    assert gm.kv_cache_len() == past + n == om.kv.current_len()
+    errs = [logit_err(got[i], want[i]) for i in range(n)]
+    say(f"{which} past={past} n={n}: worst rel err {max(errs):.2e}")
+    big = [i for i, e in enumerate(errs) if e > 1e-4]
+    say(f"  median {np.median(errs):.2e}, first row above 1e-4: {big[0] if big else None}, rows above: {len(big)}")
+    if not any(t in (5, 6) for t in mix):
+        assert max(errs) < TOL
+    else:
+        # K-quant products see their activation through the Q8_K quantiser, a step function: a value
+        # that the two summation orders (1e-6 apart) put on either side of a rounding boundary moves by
+        # 1/127 of its block's largest, and the row it belongs to, cached as K and V, carries that into
+        # every later row. In models this small (two blocks per row) one such event shows as 1e-3..1e-2
+        # of the logit scale; a wrong operand shows as 0.1..1 in every row, a skipped quantisation as
+        # 1e-3 in every row. So: rows before the first event agree like the formats without a
+        # quantiser, typical rows stay small, and no row is far off.
+        assert min(errs) < 1e-5 and np.median(errs) < 5e-3 and max(errs) < 5e-2
+    want_t, margins = om.generate_greedy(ids[n:], 24)
+    got_t = gm.generate_greedy(ids[n:], 24)
+    say(f"  min margin {margins.min():.3e}")
+    assert np.array_equal(got_t, want_t)
+    gm.close()
+
+
+def test_quantised_generate_routes_the_prompt_through_prefill(ctx):
+    cfg, mix = _quant_case("q4_k_m_mix")
+    weights = synth_model.synth_weights(cfg, 23, has_qk_norm=False, proj_dtypes=mix)
+    gm = synth_model.build_model(ctx, cfg, weights, 256, has_qk_norm=False, proj_dtypes=mix)
+    om = mf.build_oracle_model(cfg, weights, 256, has_qk_norm=False, proj_dtypes=mix)
+    ids = synth.token_ids(3, 50, cfg.vocab_size)
+    want_t, margins = om.generate_greedy(ids, 32)
+    say(f"quantised generate: min margin {margins.min():.3e}")
+    for pmin in (8, 0):
+        gm.reset_kv_cache()
+        gm.set_prefill_min(pmin)
+        assert np.array_equal(gm.generate_greedy(ids, 32), want_t), f"prefill_min={pmin}"
+        assert gm.kv_cache_len() == 50 + 31
+    gm.close()
+
+
+def test_prefill_needs_matching_widths_and_groups(ctx):
+    """Block formats take the prompt pass when the widths are multiples of the 64-wide K tile and
+    q|k|v, gate|up each multiply with one kind of activation; otherwise run_kv steps token by token."""
+    cfg = synth_model.TINY_QWEN2                      # intermediate size 608 = 9.5 x 64
     weights = synth_model.synth_weights(cfg, 31, DTYPE_Q8_0, has_qk_norm=False)
     gm = synth_model.build_model(ctx, cfg, weights, 96, DTYPE_Q8_0, has_qk_norm=False)
     ids = synth.token_ids(4, 20, cfg.vocab_size)
-    with pytest.raises(HomuraError, match="bf16 plan"):
+    with pytest.raises(HomuraError, match="multiples of"):
         gm.prefill(ids)
     logits = gm.run_kv(ids)                      # falls back to decode steps
     assert logits.shape == (20, cfg.vocab_size) and gm.kv_cache_len() == 20
+    gm.close()
+    cfg = synth_model.TINY_K                          # q in Q8_0 next to k, v in Q6_K
+    mix = [2, 6, 6, 2, 6, 6, 2] * cfg.num_hidden_layers
+    weights = synth_model.synth_weights(cfg, 32, has_qk_norm=False, proj_dtypes=mix)
+    gm = synth_model.build_model(ctx, cfg, weights, 96, has_qk_norm=False, proj_dtypes=mix)
+    with pytest.raises(HomuraError, match="one kind"):
+        gm.prefill(ids)
+    assert gm.run_kv(ids).shape == (20, cfg.vocab_size)
     gm.close()
 
 
