@@ -314,11 +314,14 @@ int hm_model_run_kv(hm_model *m, const int64_t *h_ids, int n_ids, float *h_logit
 /* The multi-token pass that hm_model_run_kv and hm_model_generate_greedy take for inputs of at
  * least `prefill_min` tokens (reference HfGenerationContext::prefill, src/hf/model.rs:321-336: the
  * whole prompt in one run_kv): projections as GEMMs on the matrix cores, causal attention over
- * cache + chunk, chunks of 512 rows. bf16 models with head_dim 64 or 128; h_logits [n_ids][vocab]
- * or NULL (then the LM head is skipped). hm_model_set_prefill_min: 0 = always token by token
- * (default 8). hm_model_set_prefill_pieces: bf16 numbers per f32 activation on the matrix cores,
- * 3 (default, every bit of the f32) or 2 (16 bits, a third less MFMA work; K/V rows then round
- * to a neighbouring bf16 now and then). */
+ * cache + chunk, chunks of 512 rows. head_dim 64 or 128; h_logits [n_ids][vocab] or NULL (then the
+ * LM head is skipped). bf16 models need widths that are multiples of 32. Block-quantised models
+ * (the products of hm_gemm_f32_quant_nk) need multiples of 64, and q|k|v as well as gate|up must each
+ * be of one kind, Q8_0 / Q4_0 or K-quants, because the members of a group share an activation
+ * matrix; other models keep stepping token by token. hm_model_set_prefill_min: 0 = always token by
+ * token (default 8). hm_model_set_prefill_pieces (bf16 models): bf16 numbers per f32 activation on the
+ * matrix cores, 3 (default, every bit of the f32) or 2 (16 bits, a third less MFMA work; K/V rows
+ * then round to a neighbouring bf16 now and then). */
 int hm_model_prefill(hm_model *m, const int64_t *h_ids, int n_ids, float *h_logits);
 int hm_model_set_prefill_min(hm_model *m, int n_tokens);
 int hm_model_set_prefill_pieces(hm_model *m, int pieces);
@@ -417,7 +420,8 @@ int hm_config_from_json(const char *json_text, hm_transformer_config *out, char 
  * config.json + model.safetensors (or model.safetensors.index.json and its shards)
  * (src/hf/model.rs:75-146, src/hf/weights.rs:267-417): parse, convert, upload, finalize.
  * max_seq_len <= 0 picks min(max_position_embeddings, 4096). NULL on failure: hm_last_error(ctx).
- * GGUF files must be Q8_0, Q4_0 or F32/F16/BF16 throughout their projections. */
+ * The projections of a GGUF file must be all float (F32 / F16 / BF16) or all block-quantised, each
+ * tensor Q8_0, Q4_0, Q4_K or Q6_K (the Q4_K_M mixes included). */
 hm_model *hm_model_load_gguf(hm_ctx *ctx, const char *path, int max_seq_len);
 hm_model *hm_model_load_hf_dir(hm_ctx *ctx, const char *dir, int max_seq_len);
 
