@@ -96,6 +96,12 @@ SIGNATURES = {
     "hm_gemm_f32_quant_nk": (_I, [_P, _P, _P, _I, _P, _I, _I, _I]),
     "hm_model_set_weight_nk": (_I, [_P, _I, _P, _SZ]),
     "hm_model_config": (_I, [_P, _P, _P, _P]),
+    "hm_tokenizer_open": (_P, [C.c_char_p, C.c_char_p, C.c_char_p, _SZ]),
+    "hm_tokenizer_close": (None, [_P]),
+    "hm_tokenizer_vocab_size": (_I, [_P]),
+    "hm_tokenizer_encode": (C.c_longlong, [_P, C.c_char_p, _SZ, _P, _SZ]),
+    "hm_tokenizer_decode": (C.c_longlong, [_P, _P, _SZ, _P, _SZ]),
+    "hm_tokenizer_pieces": (C.c_longlong, [C.c_char_p, _SZ, _P, _SZ]),
     "hm_gguf_open": (_P, [C.c_char_p, C.c_char_p, _SZ]),
     "hm_gguf_close": (None, [_P]),
     "hm_gguf_version": (_I, [_P]),

@@ -11,6 +11,7 @@
 #include <vector>
 
 #include "hf.h"
+#include "json_map.h"
 
 namespace homura {
 

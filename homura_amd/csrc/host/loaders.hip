@@ -917,6 +917,27 @@ bool file_exists(const std::string &path) {
 
 }  // namespace
 
+bool parse_json_string_to_int_map(const char *text, size_t len, std::vector<std::pair<std::string, int64_t>> *out,
+                                  std::string *err) {
+    Json j;
+    if (!parse_json(text, len, &j, err)) return false;
+    if (j.kind != Json::Obj) {
+        *err = "JSON: expected an object of string -> integer";
+        return false;
+    }
+    out->clear();
+    out->reserve(j.obj.size());
+    for (auto &kv : j.obj) {
+        if (kv.second.kind != Json::Num || kv.second.num != std::floor(kv.second.num)) {
+            *err = "JSON: value of \"" + kv.first + "\" is not an integer";
+            return false;
+        }
+        out->emplace_back(std::move(kv.first), (int64_t)kv.second.num);
+    }
+    return true;
+}
+
+
 bool transformer_config_from_json(const std::string &text, TransformerConfig *cfg, std::string *err) {
     Json j;
     if (!parse_json(text.data(), text.size(), &j, err)) return false;

@@ -1,0 +1,384 @@
+// Byte-level BPE tokenizer (reference src/tokenizer.rs). The reference cuts the text with the regex
+//   (?i:'s|'t|'re|'ve|'m|'ll|'d) | [^\r\n\p{L}\p{N}]?\p{L}+ | \p{N}{1,3} | ' '?[^\s\p{L}\p{N}]+[\r\n]* |
+//   \s*[\r\n]+ | \s+(?!\S) | \s+
+// (src/tokenizer.rs:71-74, first alternative that matches wins, each greedy with backtracking); here the
+// seven alternatives are a hand-written scanner over code points, with the letter and number classes
+// from generated range tables.
+#include "tokenizer.h"
+
+#include <algorithm>
+#include <cstdio>
+#include <cstring>
+#include <fstream>
+#include <sstream>
+
+#include "../../../include/homura_amd.h"
+#include "json_map.h"
+#include "unicode_tables.h"
+
+namespace homura {
+
+namespace {
+
+template <size_t N>
+bool in_ranges(const uint32_t (&table)[N][2], uint32_t cp) {
+    size_t lo = 0, hi = N;
+    while (lo < hi) {
+        const size_t mid = (lo + hi) / 2;
+        if (cp < table[mid][0])
+            hi = mid;
+        else if (cp > table[mid][1])
+            lo = mid + 1;
+        else
+            return true;
+    }
+    return false;
+}
+
+bool is_letter(uint32_t cp) { return in_ranges(UNICODE_LETTER_RANGES, cp); }
+bool is_number(uint32_t cp) { return in_ranges(UNICODE_NUMBER_RANGES, cp); }
+// the White_Space property, which is what \s means in the reference's regex engine
+bool is_space(uint32_t cp) {
+    return (cp >= 9 && cp <= 13) || cp == 0x20 || cp == 0x85 || cp == 0xA0 || cp == 0x1680 || (cp >= 0x2000 && cp <= 0x200A) ||
+           cp == 0x2028 || cp == 0x2029 || cp == 0x202F || cp == 0x205F || cp == 0x3000;
+}
+bool is_newline(uint32_t cp) { return cp == '\r' || cp == '\n'; }
+
+void append_utf8(std::string *out, uint32_t cp) {
+    if (cp < 0x80) {
+        out->push_back((char)cp);
+    } else if (cp < 0x800) {
+        out->push_back((char)(0xC0 | (cp >> 6)));
+        out->push_back((char)(0x80 | (cp & 0x3F)));
+    } else if (cp < 0x10000) {
+        out->push_back((char)(0xE0 | (cp >> 12)));
+        out->push_back((char)(0x80 | ((cp >> 6) & 0x3F)));
+        out->push_back((char)(0x80 | (cp & 0x3F)));
+    } else {
+        out->push_back((char)(0xF0 | (cp >> 18)));
+        out->push_back((char)(0x80 | ((cp >> 12) & 0x3F)));
+        out->push_back((char)(0x80 | ((cp >> 6) & 0x3F)));
+        out->push_back((char)(0x80 | (cp & 0x3F)));
+    }
+}
+
+// Length of the well-formed UTF-8 sequence at s (0 if there is none) and its code point. `bad` receives
+// how many bytes form the longest prefix of a well-formed sequence (at least 1), the unit that
+// lossy decoding replaces by one U+FFFD.
+size_t utf8_at(const unsigned char *s, size_t n, uint32_t *cp, size_t *bad) {
+    const unsigned char b0 = s[0];
+    *bad = 1;
+    if (b0 < 0x80) {
+        *cp = b0;
+        return 1;
+    }
+    size_t need;
+    unsigned char lo = 0x80, hi = 0xBF;
+    uint32_t v;
+    if (b0 >= 0xC2 && b0 <= 0xDF) {
+        need = 1;
+        v = b0 & 0x1F;
+    } else if (b0 >= 0xE0 && b0 <= 0xEF) {
+        need = 2;
+        v = b0 & 0x0F;
+        if (b0 == 0xE0) lo = 0xA0;
+        if (b0 == 0xED) hi = 0x9F;
+    } else if (b0 >= 0xF0 && b0 <= 0xF4) {
+        need = 3;
+        v = b0 & 0x07;
+        if (b0 == 0xF0) lo = 0x90;
+        if (b0 == 0xF4) hi = 0x8F;
+    } else {
+        return 0;
+    }
+    for (size_t k = 1; k <= need; k++) {
+        if (k >= n || s[k] < lo || s[k] > hi) {
+            *bad = k;
+            return 0;
+        }
+        v = (v << 6) | (s[k] & 0x3F);
+        lo = 0x80;
+        hi = 0xBF;
+    }
+    *cp = v;
+    return need + 1;
+}
+
+struct CodePoints {
+    std::vector<uint32_t> cp;
+    std::vector<size_t> at;  // byte offset of each code point, plus the total length at the end
+};
+
+// A byte that is not part of well-formed UTF-8 counts as one character of no class (U+FFFD); the
+// piece still carries the original byte.
+CodePoints decode_code_points(const char *text, size_t len) {
+    CodePoints r;
+    const unsigned char *s = reinterpret_cast<const unsigned char *>(text);
+    size_t i = 0;
+    while (i < len) {
+        uint32_t cp;
+        size_t bad;
+        const size_t n = utf8_at(s + i, len - i, &cp, &bad);
+        r.at.push_back(i);
+        r.cp.push_back(n ? cp : 0xFFFD);
+        i += n ? n : 1;
+    }
+    r.at.push_back(len);
+    return r;
+}
+
+// End (exclusive, in code points) of the piece that starts at i.
+size_t match_piece(const std::vector<uint32_t> &c, size_t i) {
+    const size_t n = c.size();
+    const uint32_t c0 = c[i];
+    auto lower = [](uint32_t x) { return x >= 'A' && x <= 'Z' ? x + 32 : x; };
+    // 1. contractions, case-insensitive (U+017F, the long s, folds to s)
+    if (c0 == '\'' && i + 1 < n) {
+        const uint32_t a = c[i + 1] == 0x17F ? 's' : lower(c[i + 1]);
+        const uint32_t b = i + 2 < n ? lower(c[i + 2]) : 0;
+        if (a == 's' || a == 't') return i + 2;
+        if ((a == 'r' && b == 'e') || (a == 'v' && b == 'e')) return i + 3;
+        if (a == 'm') return i + 2;
+        if (a == 'l' && b == 'l') return i + 3;
+        if (a == 'd') return i + 2;
+    }
+    // 2. letters, with at most one leading character that is none of CR, LF, letter, number
+    {
+        size_t j = i;
+        if (!is_newline(c0) && !is_letter(c0) && !is_number(c0) && i + 1 < n && is_letter(c[i + 1])) j = i + 1;
+        if (is_letter(c[j])) {
+            while (j < n && is_letter(c[j])) j++;
+            return j;
+        }
+    }
+    // 3. one to three numbers
+    if (is_number(c0)) {
+        size_t j = i;
+        while (j < n && j < i + 3 && is_number(c[j])) j++;
+        return j;
+    }
+    // 4. punctuation and symbols, with an optional leading space and trailing newlines
+    {
+        auto symbol = [](uint32_t x) { return !is_space(x) && !is_letter(x) && !is_number(x); };
+        size_t j = i;
+        if (c0 == ' ' && i + 1 < n && symbol(c[i + 1])) j = i + 1;
+        if (symbol(c[j])) {
+            while (j < n && symbol(c[j])) j++;
+            while (j < n && is_newline(c[j])) j++;
+            return j;
+        }
+    }
+    // what is left starts a run of whitespace
+    size_t e = i;
+    while (e < n && is_space(c[e])) e++;
+    if (e == i) return i + 1;  // unreachable: every character belongs to one of the classes above
+    // 5. whitespace up to and including the last newline of the run
+    for (size_t j = e; j > i; j--)
+        if (is_newline(c[j - 1])) return j;
+    // 6. whitespace not followed by a non-space: the whole run at the end of the text, else all but its last character
+    if (e == n) return e;
+    if (e - 1 > i) return e - 1;
+    // 7. whitespace
+    return e;
+}
+
+void copy_err(const std::string &e, char *err, size_t errlen) {
+    if (err && errlen) snprintf(err, errlen, "%s", e.c_str());
+}
+
+bool read_file(const std::string &path, std::string *out, std::string *err) {
+    std::ifstream f(path, std::ios::binary);
+    if (!f) {
+        *err = "cannot open " + path;
+        return false;
+    }
+    std::ostringstream ss;
+    ss << f.rdbuf();
+    *out = ss.str();
+    return true;
+}
+
+}  // namespace
+
+std::vector<std::pair<size_t, size_t>> BpeTokenizer::pre_tokenize(const char *text, size_t len) {
+    std::vector<std::pair<size_t, size_t>> out;
+    const CodePoints c = decode_code_points(text, len);
+    for (size_t i = 0; i < c.cp.size();) {
+        const size_t j = match_piece(c.cp, i);
+        out.emplace_back(c.at[i], c.at[j]);
+        i = j;
+    }
+    return out;
+}
+
+std::unique_ptr<BpeTokenizer> BpeTokenizer::from_files(const std::string &vocab_path, const std::string &merges_path,
+                                                       std::string *err) {
+    std::string vocab_text, merges_text;
+    if (!read_file(vocab_path, &vocab_text, err) || !read_file(merges_path, &merges_text, err)) return nullptr;
+    std::vector<std::pair<std::string, int64_t>> vocab;
+    if (!parse_json_string_to_int_map(vocab_text.data(), vocab_text.size(), &vocab, err)) {
+        *err = vocab_path + ": " + *err;
+        return nullptr;
+    }
+    std::unique_ptr<BpeTokenizer> t(new BpeTokenizer());
+    for (auto &kv : vocab) {
+        if (kv.second < 0 || kv.second > 0xFFFFFFFFLL) {
+            *err = vocab_path + ": id of \"" + kv.first + "\" outside u32";
+            return nullptr;
+        }
+        t->encoder_[kv.first] = (uint32_t)kv.second;
+    }
+    for (const auto &kv : t->encoder_) t->decoder_[kv.second] = kv.first;
+    // merges.txt: "left right" per line in rank order; lines that start with '#' (the version header)
+    // and empty lines do not count (src/tokenizer.rs:54-66)
+    uint32_t rank = 0;
+    size_t pos = 0;
+    while (pos < merges_text.size()) {
+        size_t eol = merges_text.find('\n', pos);
+        if (eol == std::string::npos) eol = merges_text.size();
+        size_t end = eol;
+        if (end > pos && merges_text[end - 1] == '\r') end--;
+        if (end > pos && merges_text[pos] != '#') t->ranks_[merges_text.substr(pos, end - pos)] = rank++;
+        pos = eol + 1;
+    }
+    // GPT-2's bytes_to_unicode (src/tokenizer.rs:19-41): printable Latin-1 bytes stand for themselves,
+    // the other 68 get U+0100 onwards in byte order
+    uint32_t next = 256;
+    for (int b = 0; b < 256; b++) {
+        const bool printable = (b >= '!' && b <= '~') || (b >= 0xA1 && b <= 0xAC) || (b >= 0xAE && b <= 0xFF);
+        const uint32_t cp = printable ? (uint32_t)b : next++;
+        append_utf8(&t->byte_utf8_[b], cp);
+        t->cp_to_byte_[cp] = (uint8_t)b;
+    }
+    return t;
+}
+
+// reference bpe (src/tokenizer.rs:85-116): while some adjacent pair has a rank, merge the first
+// occurrence of the pair with the lowest rank
+std::vector<std::string> BpeTokenizer::bpe(const std::string &mapped) const {
+    std::vector<std::string> word;
+    for (size_t i = 0; i < mapped.size();) {
+        uint32_t cp;
+        size_t bad;
+        const size_t n = utf8_at(reinterpret_cast<const unsigned char *>(mapped.data()) + i, mapped.size() - i, &cp, &bad);
+        word.emplace_back(mapped, i, n ? n : 1);
+        i += n ? n : 1;
+    }
+    while (word.size() > 1) {
+        size_t best = word.size();
+        uint32_t best_rank = 0xFFFFFFFFu;
+        std::string key;
+        for (size_t i = 0; i + 1 < word.size(); i++) {
+            key.assign(word[i]);
+            key.push_back(' ');
+            key.append(word[i + 1]);
+            auto it = ranks_.find(key);
+            if (it != ranks_.end() && it->second < best_rank) {
+                best_rank = it->second;
+                best = i;
+            }
+        }
+        if (best == word.size()) break;
+        word[best] += word[best + 1];
+        word.erase(word.begin() + (long)best + 1);
+    }
+    return word;
+}
+
+std::vector<uint32_t> BpeTokenizer::encode(const char *text, size_t len) const {
+    std::vector<uint32_t> ids;
+    std::string mapped;
+    for (const auto &piece : pre_tokenize(text, len)) {
+        mapped.clear();
+        for (size_t i = piece.first; i < piece.second; i++) mapped += byte_utf8_[(unsigned char)text[i]];
+        for (const std::string &sym : bpe(mapped)) {
+            auto it = encoder_.find(sym);
+            if (it != encoder_.end()) ids.push_back(it->second);
+        }
+    }
+    return ids;
+}
+
+std::string BpeTokenizer::decode(const uint32_t *ids, size_t n) const {
+    std::string bytes;
+    for (size_t k = 0; k < n; k++) {
+        auto it = decoder_.find(ids[k]);
+        if (it == decoder_.end()) continue;
+        const std::string &tok = it->second;
+        for (size_t i = 0; i < tok.size();) {
+            uint32_t cp;
+            size_t bad;
+            const size_t m = utf8_at(reinterpret_cast<const unsigned char *>(tok.data()) + i, tok.size() - i, &cp, &bad);
+            if (m) {
+                auto b = cp_to_byte_.find(cp);
+                if (b != cp_to_byte_.end()) bytes.push_back((char)b->second);
+            }
+            i += m ? m : 1;
+        }
+    }
+    // String::from_utf8_lossy: every longest ill-formed prefix becomes one U+FFFD
+    std::string out;
+    const unsigned char *s = reinterpret_cast<const unsigned char *>(bytes.data());
+    for (size_t i = 0; i < bytes.size();) {
+        uint32_t cp;
+        size_t bad;
+        const size_t m = utf8_at(s + i, bytes.size() - i, &cp, &bad);
+        if (m) {
+            out.append(bytes, i, m);
+            i += m;
+        } else {
+            out += "\xEF\xBF\xBD";
+            i += bad;
+        }
+    }
+    return out;
+}
+
+}  // namespace homura
+
+struct hm_tokenizer {
+    std::unique_ptr<homura::BpeTokenizer> t;
+};
+
+#pragma GCC visibility push(default)
+extern "C" {
+
+hm_tokenizer *hm_tokenizer_open(const char *vocab_json_path, const char *merges_txt_path, char *err, size_t errlen) {
+    std::string e;
+    auto t = homura::BpeTokenizer::from_files(vocab_json_path ? vocab_json_path : "", merges_txt_path ? merges_txt_path : "", &e);
+    if (!t) {
+        homura::copy_err(e, err, errlen);
+        return nullptr;
+    }
+    return new hm_tokenizer{std::move(t)};
+}
+
+void hm_tokenizer_close(hm_tokenizer *t) { delete t; }
+
+int hm_tokenizer_vocab_size(const hm_tokenizer *t) { return t ? (int)t->t->vocab_size() : HM_ERR_INVALID; }
+
+long long hm_tokenizer_encode(const hm_tokenizer *t, const char *text, size_t text_len, uint32_t *ids_out, size_t capacity) {
+    if (!t || (!text && text_len) || (!ids_out && capacity)) return HM_ERR_INVALID;
+    const std::vector<uint32_t> ids = t->t->encode(text, text_len);
+    const size_t n = std::min(ids.size(), capacity);
+    if (n) memcpy(ids_out, ids.data(), n * sizeof(uint32_t));
+    return (long long)ids.size();
+}
+
+long long hm_tokenizer_decode(const hm_tokenizer *t, const uint32_t *ids, size_t n_ids, char *text_out, size_t capacity) {
+    if (!t || (!ids && n_ids) || (!text_out && capacity)) return HM_ERR_INVALID;
+    const std::string s = t->t->decode(ids, n_ids);
+    const size_t n = std::min(s.size(), capacity);
+    if (n) memcpy(text_out, s.data(), n);
+    return (long long)s.size();
+}
+
+long long hm_tokenizer_pieces(const char *text, size_t text_len, size_t *ends_out, size_t capacity) {
+    if ((!text && text_len) || (!ends_out && capacity)) return HM_ERR_INVALID;
+    const auto pieces = homura::BpeTokenizer::pre_tokenize(text, text_len);
+    for (size_t i = 0; i < pieces.size() && i < capacity; i++) ends_out[i] = pieces[i].second;
+    return (long long)pieces.size();
+}
+
+}  // extern "C"
+#pragma GCC visibility pop

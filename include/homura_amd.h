@@ -460,6 +460,25 @@ uint16_t hm_f32_to_f16_rne(float v);
 
 const char *hm_version(void);
 
+/* ── tokenizer (reference src/tokenizer.rs) ───────────────────────────────────
+ * The reference's own byte-level BPE over vocab.json + merges.txt (GPT-2 files): Tokenizer::from_files
+ * (src/tokenizer.rs:44-82), encode (:119-144), decode (:147-159). Host code, no GPU. (Its wrapper
+ * around the `tokenizers` crate for tokenizer.json files, src/hf/tokenizer.rs, has no counterpart.)
+ * hm_tokenizer_open returns NULL and writes a message into err. encode / decode return the full
+ * count of ids / bytes (negative: an HM_ERR_* code) and write at most `capacity` of them; call again
+ * with a larger buffer when the count exceeds it. The decoded text is UTF-8 without a terminator.
+ * hm_tokenizer_pieces: the end offsets (bytes) of the pieces the pre-tokeniser pattern
+ * (src/tokenizer.rs:71-74) cuts the text into. */
+typedef struct hm_tokenizer hm_tokenizer;
+hm_tokenizer *hm_tokenizer_open(const char *vocab_json_path, const char *merges_txt_path, char *err, size_t errlen);
+void hm_tokenizer_close(hm_tokenizer *t);
+int hm_tokenizer_vocab_size(const hm_tokenizer *t);
+long long hm_tokenizer_encode(const hm_tokenizer *t, const char *text, size_t text_len, uint32_t *ids_out,
+                              size_t capacity);
+long long hm_tokenizer_decode(const hm_tokenizer *t, const uint32_t *ids, size_t n_ids, char *text_out,
+                              size_t capacity);
+long long hm_tokenizer_pieces(const char *text, size_t text_len, size_t *ends_out, size_t capacity);
+
 #pragma GCC visibility pop
 
 #ifdef __cplusplus
