@@ -28,6 +28,8 @@ class HmTransformerConfig(C.Structure):
         ("rms_norm_eps", C.c_double),
         ("rope_theta", C.c_double),
         ("attention_bias", C.c_int),
+        ("eos_token_id", C.c_int),
+        ("bos_token_id", C.c_int),
     ]
 
 

@@ -20,7 +20,9 @@ def _config_from_c(c) -> TransformerConfig:
         rms_norm_eps=c.rms_norm_eps, rope_theta=c.rope_theta,
         max_position_embeddings=c.max_position_embeddings,
         tie_word_embeddings=bool(c.tie_word_embeddings), head_dim=c.head_dim or None,
-        attention_bias=bool(c.attention_bias))
+        attention_bias=bool(c.attention_bias),
+        eos_token_id=None if c.eos_token_id < 0 else c.eos_token_id,
+        bos_token_id=None if c.bos_token_id < 0 else c.bos_token_id)
 
 
 class GgufFile:

@@ -28,6 +28,8 @@ static TransformerConfig config_from_c(const hm_transformer_config *cfg) {
     c.rms_norm_eps = cfg->rms_norm_eps > 0 ? cfg->rms_norm_eps : 1e-6;
     c.rope_theta = cfg->rope_theta > 0 ? cfg->rope_theta : 10000.0;
     c.attention_bias = cfg->attention_bias != 0;
+    c.eos_token_id = cfg->eos_token_id;
+    c.bos_token_id = cfg->bos_token_id;
     return c;
 }
 
@@ -233,6 +235,8 @@ static void fill_c_config(const TransformerConfig &c, hm_transformer_config *out
     out->rms_norm_eps = c.rms_norm_eps;
     out->rope_theta = c.rope_theta;
     out->attention_bias = c.attention_bias ? 1 : 0;
+    out->eos_token_id = c.eos_token_id;
+    out->bos_token_id = c.bos_token_id;
 }
 
 extern "C" {

@@ -23,6 +23,7 @@ struct TransformerConfig {
     bool tie_word_embeddings = false;
     int head_dim_opt = 0;  // 0 => hidden_size / num_attention_heads
     bool attention_bias = false;  // q/k/v_proj.bias present (reference src/hf/weights.rs:64-69)
+    int eos_token_id = -1, bos_token_id = -1;  // -1: none (reference Option<u32>)
 
     int kv_heads() const { return num_key_value_heads ? num_key_value_heads : num_attention_heads; }
     int head_dim() const { return head_dim_opt ? head_dim_opt : hidden_size / num_attention_heads; }

@@ -505,6 +505,8 @@ bool GgufFile::transformer_config(TransformerConfig *cfg, std::string *err) cons
     c.tie_word_embeddings = tensor_info("output.weight") == nullptr;
     c.head_dim_opt = get_u64(arch + ".attention.key_length", &x) ? (int)x : 0;
     c.attention_bias = tensor_info("blk.0.attn_q.bias") != nullptr;
+    c.eos_token_id = get_u64("tokenizer.ggml.eos_token_id", &x) ? (int)x : -1;
+    c.bos_token_id = get_u64("tokenizer.ggml.bos_token_id", &x) ? (int)x : -1;
     *cfg = c;
     return true;
 }
@@ -973,6 +975,8 @@ bool transformer_config_from_json(const std::string &text, TransformerConfig *cf
     c.head_dim_opt = opt_num("head_dim", &x) ? (int)x : 0;
     const Json *tie = j.get("tie_word_embeddings");
     c.tie_word_embeddings = tie && tie->kind == Json::Bool && tie->b;
+    c.eos_token_id = opt_num("eos_token_id", &x) && x >= 0 ? (int)x : -1;
+    c.bos_token_id = opt_num("bos_token_id", &x) && x >= 0 ? (int)x : -1;
     *cfg = c;
     return true;
 }

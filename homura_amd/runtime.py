@@ -282,6 +282,8 @@ class TransformerConfig:
     tie_word_embeddings: bool = False
     head_dim: int | None = None
     attention_bias: bool = False   # q/k/v_proj.bias present (reference src/hf/weights.rs:64-69)
+    eos_token_id: int | None = None
+    bos_token_id: int | None = None
 
     def kv_heads(self) -> int:
         return self.num_key_value_heads or self.num_attention_heads
@@ -297,7 +299,9 @@ class TransformerConfig:
             self.hidden_size, self.intermediate_size, self.num_attention_heads,
             self.num_hidden_layers, self.num_key_value_heads or 0, self.vocab_size,
             self.head_dim or 0, self.max_position_embeddings, int(self.tie_word_embeddings),
-            self.rms_norm_eps, self.rope_theta, int(self.attention_bias))
+            self.rms_norm_eps, self.rope_theta, int(self.attention_bias),
+            -1 if self.eos_token_id is None else self.eos_token_id,
+            -1 if self.bos_token_id is None else self.bos_token_id)
 
 
 class HfModel:
@@ -336,7 +340,9 @@ class HfModel:
             rms_norm_eps=c.rms_norm_eps, rope_theta=c.rope_theta,
             max_position_embeddings=c.max_position_embeddings,
             tie_word_embeddings=bool(c.tie_word_embeddings), head_dim=c.head_dim or None,
-            attention_bias=bool(c.attention_bias))
+            attention_bias=bool(c.attention_bias),
+            eos_token_id=None if c.eos_token_id < 0 else c.eos_token_id,
+            bos_token_id=None if c.bos_token_id < 0 else c.bos_token_id)
         self.has_qk_norm, self.weight_dtype = bool(qkn.value), wdt.value
         return self
 

@@ -266,6 +266,8 @@ typedef struct {
     double rope_theta;
     int attention_bias;      /* Q/K/V projections carry a bias (Qwen2-style); the reference reads this
                                 off the checkpoint (src/hf/weights.rs:64-69) */
+    int eos_token_id;        /* -1 => none (the reference's Option<u32>, src/hf/config.rs:32-35; GGUF: */
+    int bos_token_id;        /*  tokenizer.ggml.eos_token_id / bos_token_id, src/gguf.rs:559-565) */
 } hm_transformer_config;
 
 #define HM_DTYPE_F32 0

@@ -110,17 +110,21 @@ def test_gguf_transformer_config(tmp_path):
         assert cfg.rope_theta == 1e6 and abs(cfg.rms_norm_eps - 1e-6) < 1e-12 and cfg.max_position_embeddings == 40960
         assert cfg.tie_word_embeddings is True        # no output.weight tensor
         assert qkn is True and cfg.attention_bias is False
+        assert cfg.eos_token_id is None and cfg.bos_token_id is None
     # defaults and fallbacks: no kv heads, no eps/theta/context, vocab from the tokenizer, untied, biased
     md = _arch_md("llama", **{"llama.attention.head_count_kv": None, "llama.vocab_size": None,
                               "llama.attention.layer_norm_rms_epsilon": None, "llama.rope.freq_base": None,
                               "llama.context_length": None, "llama.attention.key_length": None})
     md.append(("tokenizer.ggml.tokens", cw.ARRAY, (cw.STRING, [str(i) for i in range(77)])))
+    md.append(("tokenizer.ggml.eos_token_id", cw.U32, 2))          # src/gguf.rs:559-565
+    md.append(("tokenizer.ggml.bos_token_id", cw.U32, 1))
     tensors = [("output.weight", (4, 4), ck.GGML_F32, bytes(64)), ("blk.0.attn_q.bias", (4,), ck.GGML_F32, bytes(16))]
     with ck.GgufFile(write(tmp_path, "cfg2.gguf", cw.gguf_bytes(md, tensors))) as g:
         cfg, qkn = g.transformer_config()
         assert cfg.kv_heads() == 16 and cfg.vocab_size == 77 and cfg.get_head_dim() == 64
         assert cfg.rope_theta == 10000.0 and cfg.rms_norm_eps == 1e-6 and cfg.max_position_embeddings == 2048
         assert cfg.tie_word_embeddings is False and qkn is False and cfg.attention_bias is True
+        assert cfg.eos_token_id == 2 and cfg.bos_token_id == 1
     md = [m for m in _arch_md() if m[0] != "qwen3.embedding_length"]
     with ck.GgufFile(write(tmp_path, "cfg3.gguf", cw.gguf_bytes(md, []))) as g:
         with pytest.raises(ValueError, match="missing or invalid metadata: qwen3.embedding_length"):
@@ -216,6 +220,7 @@ def test_parse_qwen2_config():
     assert cfg.hidden_size == 896 and cfg.num_attention_heads == 14
     assert cfg.kv_heads() == 2 and cfg.get_head_dim() == 64 and cfg.gqa_repeat() == 7
     assert cfg.tie_word_embeddings is True and cfg.rope_theta == 1e6 and cfg.max_position_embeddings == 32768
+    assert cfg.eos_token_id == 151643 and cfg.bos_token_id == 151643
 
 
 def test_parse_llama_config_no_kv_heads():
