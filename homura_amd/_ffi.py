@@ -127,6 +127,7 @@ SIGNATURES = {
     "hm_model_load_gguf": (_P, [_P, C.c_char_p, _I]),
     "hm_model_load_hf_dir": (_P, [_P, C.c_char_p, _I]),
     "hm_ciface_bind_transformer": (_I, [_P, _P, _I]),
+    "hm_ciface_bind_transformer_quant": (_I, [_P, _P, _P, _I]),
     "hm_ciface_num_kernels": (_I, []),
     "hm_ciface_unbind": (None, []),
     "hm_kv_append": (_I, [_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I]),

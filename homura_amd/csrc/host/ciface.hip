@@ -9,9 +9,14 @@
 // 902-1014): k0 Embed; per layer k(3l+1) QKV(+QK-norm)+RoPE, k(3l+2) Attn, k(3l+3) MLP; then
 // LMHead. Arguments follow each emitter's input order, outputs after inputs.
 //
-// This is the compatibility path: weights are consumed in the reference's [K,N] layout, the KV
-// views are the reference's f32 cache (copied to a bf16 scratch cache per call), and every
-// reference kernel becomes several launches. The model-level API is the fast path.
+// hm_ciface_bind_transformer_quant() does the same for the quantised plan (src/hf/emitter_quant.rs:
+// 1170-1440): k0 Embed; per layer thirteen kernels, RMSNorm, QuantMM Q, K, V, PostQKV, AttnBody,
+// QuantMM O, Residual+Norm, QuantMM Gate, Up, SiLU*Up, QuantMM Down, ResAdd; then the f32 LMHead.
+//
+// This is the compatibility path: weights are consumed in the reference's layouts ([K,N] bf16 / f32,
+// raw GGUF blocks), the KV views are the reference's f32 cache (copied to a bf16 scratch cache per
+// call), and every reference kernel becomes one or several launches. The model-level API is the
+// fast path.
 #include <cmath>
 #include <cstdio>
 #include <vector>
@@ -20,14 +25,22 @@
 
 namespace {
 
-enum class Kind { Embed, Qkv, Attn, Mlp, LmHead };
+enum class Kind { Embed, Qkv, Attn, Mlp, LmHead,                                              // bf16 plan
+                  RmsNorm, QuantMM, PostQkv, AttnBody, ResidualNorm, SiluMul, ResAdd, LmHeadF32 };  // quantised plan
+
+struct KernelInfo {
+    Kind kind;
+    int K = 0, N = 0, dtype = 0;  // QuantMM: the matrix
+    KernelInfo(Kind k) : kind(k) {}
+    KernelInfo(int k_dim, int n_dim, int dt) : kind(Kind::QuantMM), K(k_dim), N(n_dim), dtype(dt) {}
+};
 
 struct Bound {
     hm_ctx *ctx = nullptr;
     hm_transformer_config cfg{};
     bool qk_norm = false;
     int kv_heads = 0, head_dim = 0, q_dim = 0, kv_dim = 0;
-    std::vector<Kind> kinds;
+    std::vector<KernelInfo> kinds;
 } g_bound;
 
 // One rank-N memref argument: args[i] points at a pointer to the descriptor bytes.
@@ -211,36 +224,192 @@ int run_lm_head(void **a) {
     return hm_gemv_bf16(ctx, normed, lw.as<uint16_t>(), out.as<float>(), 1, b.cfg.hidden_size, b.cfg.vocab_size);
 }
 
+// ── the quantised plan's kernels (src/hf/emitter_quant.rs) ───────────────────
+
+// out[n] = sum_k x[k] W[k][n], f32, k ascending: the LM head of the quantised plan keeps its weights
+// in f32 [hidden, vocab] (src/hf/emitter_quant.rs:1399-1440). One column per thread, coalesced rows.
+__global__ __launch_bounds__(256) void gemv_f32_kn_kernel(const float *__restrict__ x, const float *__restrict__ w,
+                                                          float *__restrict__ out, int K, int N) {
+    extern __shared__ float xs[];
+    for (int k = threadIdx.x; k < K; k += blockDim.x) xs[k] = x[k];
+    __syncthreads();
+    const int n = blockIdx.x * blockDim.x + threadIdx.x;
+    if (n >= N) return;
+    float acc = 0.f;
+    for (int k = 0; k < K; k++) acc += xs[k] * w[(size_t)k * N + n];
+    out[n] = acc;
+}
+
+// emit_rms_norm_kernel (src/hf/emitter_quant.rs:713-791): h [1,S,hidden], w [hidden] -> [1,S,hidden]
+int run_rms_norm(void **a) {
+    const Bound &b = g_bound;
+    const MemRef h = memref(a, 0, 3), w = memref(a, 1, 1), out = memref(a, 2, 3);
+    TRY(need_single_token(b.ctx, h.sizes[1], "RMSNorm kernel"));
+    return hm_rmsnorm(b.ctx, h.as<float>(), w.as<float>(), out.as<float>(), 1, b.cfg.hidden_size, (float)b.cfg.rms_norm_eps);
+}
+
+// emit_quant_matmul_kernel (src/hf/emitter_quant.rs:675-702): x [1,S,K], raw blocks (flat bytes) -> [1,S,N]
+int run_quant_mm(void **a, const KernelInfo &ki) {
+    const Bound &b = g_bound;
+    const MemRef x = memref(a, 0, 3), w = memref(a, 1, 1), out = memref(a, 2, 3);
+    TRY(need_single_token(b.ctx, x.sizes[1], "QuantMM kernel"));
+    switch (ki.dtype) {
+    case HM_DTYPE_Q8_0: return hm_gemv_q8_0(b.ctx, x.as<float>(), w.as<uint8_t>(), out.as<float>(), 1, ki.K, ki.N);
+    case HM_DTYPE_Q4_0: return hm_gemv_q4_0(b.ctx, x.as<float>(), w.as<uint8_t>(), out.as<float>(), 1, ki.K, ki.N);
+    case HM_DTYPE_Q4_K: return hm_gemv_q4_k(b.ctx, x.as<float>(), w.as<uint8_t>(), out.as<float>(), 1, ki.K, ki.N);
+    case HM_DTYPE_Q6_K: return hm_gemv_q6_k(b.ctx, x.as<float>(), w.as<uint8_t>(), out.as<float>(), 1, ki.K, ki.N);
+    }
+    return hm_set_error(b.ctx, HM_ERR_INVALID, "QuantMM kernel: dtype %d", ki.dtype);
+}
+
+// emit_post_qkv_kernel (src/hf/emitter_quant.rs:802-912): q_raw [1,S,q_dim], k_raw, v_raw [1,S,kv_dim],
+// [q_b, k_b, v_b], cos, sin, [q_norm_w, k_norm_w] -> q [1,S,H,hd], k [1,kvh,S,hd], v [1,kvh,S,hd]
+int run_post_qkv(void **a) {
+    const Bound &b = g_bound;
+    hm_ctx *ctx = b.ctx;
+    const bool bias = b.cfg.attention_bias != 0;
+    int i = 0;
+    const MemRef qr = memref(a, i++, 3), kr = memref(a, i++, 3), vr = memref(a, i++, 3);
+    const float *qb = nullptr, *kb = nullptr, *vb = nullptr;
+    if (bias) {
+        qb = memref(a, i++, 1).as<float>();
+        kb = memref(a, i++, 1).as<float>();
+        vb = memref(a, i++, 1).as<float>();
+    }
+    const MemRef cosv = memref(a, i++, 2), sinv = memref(a, i++, 2);
+    const float *qn = nullptr, *kn = nullptr;
+    if (b.qk_norm) {
+        qn = memref(a, i++, 1).as<float>();
+        kn = memref(a, i++, 1).as<float>();
+    }
+    const MemRef q = memref(a, i++, 4), k = memref(a, i++, 4), v = memref(a, i++, 4);
+    TRY(need_single_token(ctx, qr.sizes[1], "PostQKV kernel"));
+    // with one token the [1,S,dim] rows and the BSHD / BHSD outputs are the same bytes
+    if (bias) {
+        TRY(hm_add(ctx, qr.as<float>(), qb, q.as<float>(), (size_t)b.q_dim));
+        TRY(hm_add(ctx, kr.as<float>(), kb, k.as<float>(), (size_t)b.kv_dim));
+        TRY(hm_add(ctx, vr.as<float>(), vb, v.as<float>(), (size_t)b.kv_dim));
+    } else {
+        TRY(hm_copy(ctx, q.data, qr.data, (size_t)b.q_dim * 4));
+        TRY(hm_copy(ctx, k.data, kr.data, (size_t)b.kv_dim * 4));
+        TRY(hm_copy(ctx, v.data, vr.data, (size_t)b.kv_dim * 4));
+    }
+    return hm_qknorm_rope(ctx, q.as<float>(), k.as<float>(), qn, kn, cosv.as<float>(), sinv.as<float>(), 1,
+                          b.cfg.num_attention_heads, b.kv_heads, b.head_dim, (float)b.cfg.rms_norm_eps);
+}
+
+// The attention part shared by emit_attention_kernel and emit_attention_body_kernel: q [1,1,H,hd] over
+// the f32 K/V views -> out [q_dim] (device pointer)
+int attention_over_views(const MemRef &q, const MemRef &k, const MemRef &v, float *out, Scratch &s, const char *who) {
+    const Bound &b = g_bound;
+    hm_ctx *ctx = b.ctx;
+    const int T = (int)k.sizes[2], kvh = b.kv_heads, hd = b.head_dim;
+    if (T < 1 || k.strides[3] != 1 || v.strides[3] != 1)
+        return hm_set_error(ctx, HM_ERR_INVALID, "%s: K/V views must have >= 1 row and unit inner stride", who);
+    // the attention kernel's split partials must fit the part of the workspace left to the kernels
+    if ((size_t)b.cfg.num_attention_heads * ((T + 31) / 32) * (hd + 2) * 4 > KERNEL_RESERVE)
+        return hm_set_error(ctx, HM_ERR_INVALID, "%s: %d cache rows are more than this entry point takes", who, T);
+    const size_t n = (size_t)kvh * T * hd;
+    uint16_t *kc = s.take<uint16_t>(n), *vc = s.take<uint16_t>(n);
+    if (!kc || !vc) return hm_set_error(ctx, HM_ERR_OOM, "%s: workspace too small for %d rows", who, T);
+    const unsigned blocks = (unsigned)((n + 255) / 256);
+    hipLaunchKernelGGL(kv_view_to_bf16_kernel, dim3(blocks), dim3(256), 0, ctx->stream, k.as<float>(), k.strides[1],
+                       k.strides[2], kc, T, hd, n);
+    hipLaunchKernelGGL(kv_view_to_bf16_kernel, dim3(blocks), dim3(256), 0, ctx->stream, v.as<float>(), v.strides[1],
+                       v.strides[2], vc, T, hd, n);
+    HM_LAUNCH_CHECK(ctx);
+    return hm_gqa_decode_attn(ctx, q.as<float>(), kc, vc, out, 1, b.cfg.num_attention_heads, kvh, hd, T, T,
+                              (float)(1.0 / std::sqrt((double)hd)));
+}
+
+// emit_attention_body_kernel (src/hf/emitter_quant.rs:922-975): q, K view, V view, mask -> [1,S,q_dim]
+int run_attn_body(void **a) {
+    const Bound &b = g_bound;
+    const MemRef q = memref(a, 0, 4), k = memref(a, 1, 4), v = memref(a, 2, 4), out = memref(a, 4, 3);
+    TRY(need_single_token(b.ctx, q.sizes[1], "AttnBody kernel"));
+    Scratch s(b.ctx);
+    return attention_over_views(q, k, v, out.as<float>(), s, "AttnBody kernel");
+}
+
+// emit_residual_norm_kernel (src/hf/emitter_quant.rs:985-1064): h, attn_out, ln_w -> residual, normed
+int run_residual_norm(void **a) {
+    const Bound &b = g_bound;
+    const MemRef h = memref(a, 0, 3), attn = memref(a, 1, 3), w = memref(a, 2, 1), resid = memref(a, 3, 3),
+                 normed = memref(a, 4, 3);
+    TRY(need_single_token(b.ctx, h.sizes[1], "Residual+Norm kernel"));
+    TRY(hm_add(b.ctx, h.as<float>(), attn.as<float>(), resid.as<float>(), (size_t)b.cfg.hidden_size));
+    return hm_rmsnorm(b.ctx, resid.as<float>(), w.as<float>(), normed.as<float>(), 1, b.cfg.hidden_size,
+                      (float)b.cfg.rms_norm_eps);
+}
+
+// emit_silu_mul_kernel (src/hf/emitter_quant.rs:1074-1100): gate, up [1,S,inter] -> [1,S,inter]
+int run_silu_mul(void **a) {
+    const Bound &b = g_bound;
+    const MemRef g = memref(a, 0, 3), u = memref(a, 1, 3), out = memref(a, 2, 3);
+    TRY(need_single_token(b.ctx, g.sizes[1], "SiLU*Up kernel"));
+    return hm_silu_mul(b.ctx, g.as<float>(), u.as<float>(), out.as<float>(), (size_t)b.cfg.intermediate_size);
+}
+
+// emit_residual_add_kernel (src/hf/emitter_quant.rs:1110-1134): residual, down_out -> hidden_out
+int run_res_add(void **a) {
+    const Bound &b = g_bound;
+    const MemRef r = memref(a, 0, 3), d = memref(a, 1, 3), out = memref(a, 2, 3);
+    TRY(need_single_token(b.ctx, r.sizes[1], "ResAdd kernel"));
+    return hm_add(b.ctx, r.as<float>(), d.as<float>(), out.as<float>(), (size_t)b.cfg.hidden_size);
+}
+
+// LM head of the quantised plan (src/hf/emitter_quant.rs:1399-1440): h, norm_w, lm_head_w f32 [hidden,vocab]
+int run_lm_head_f32(void **a) {
+    const Bound &b = g_bound;
+    hm_ctx *ctx = b.ctx;
+    const MemRef h = memref(a, 0, 3), nw = memref(a, 1, 1), lw = memref(a, 2, 2), out = memref(a, 3, 3);
+    TRY(need_single_token(ctx, h.sizes[1], "LMHead kernel"));
+    const int hidden = b.cfg.hidden_size, vocab = b.cfg.vocab_size;
+    Scratch s(ctx);
+    float *normed = s.take<float>(hidden);
+    if (!normed) return hm_set_error(ctx, HM_ERR_OOM, "LMHead kernel: workspace too small");
+    HM_REQUIRE(ctx, (size_t)hidden * 4 <= 64 * 1024, "LMHead kernel: hidden size %d above 16384", hidden);
+    TRY(hm_rmsnorm(ctx, h.as<float>(), nw.as<float>(), normed, 1, hidden, (float)b.cfg.rms_norm_eps));
+    hipLaunchKernelGGL(gemv_f32_kn_kernel, dim3((unsigned)((vocab + 255) / 256)), dim3(256), (size_t)hidden * 4, ctx->stream,
+                       normed, lw.as<float>(), out.as<float>(), hidden, vocab);
+    HM_LAUNCH_CHECK(ctx);
+    return HM_OK;
+}
+
 void dispatch(int idx, void **args) {
     if (!g_bound.ctx || idx >= (int)g_bound.kinds.size()) {
         report(idx, HM_ERR_STATE);
         return;
     }
     int rc = HM_ERR_INVALID;
-    switch (g_bound.kinds[idx]) {
+    const KernelInfo &ki = g_bound.kinds[idx];
+    switch (ki.kind) {
     case Kind::Embed: rc = run_embed(args); break;
     case Kind::Qkv: rc = run_qkv(args); break;
     case Kind::Attn: rc = run_attn(args); break;
     case Kind::Mlp: rc = run_mlp(args); break;
     case Kind::LmHead: rc = run_lm_head(args); break;
+    case Kind::RmsNorm: rc = run_rms_norm(args); break;
+    case Kind::QuantMM: rc = run_quant_mm(args, ki); break;
+    case Kind::PostQkv: rc = run_post_qkv(args); break;
+    case Kind::AttnBody: rc = run_attn_body(args); break;
+    case Kind::ResidualNorm: rc = run_residual_norm(args); break;
+    case Kind::SiluMul: rc = run_silu_mul(args); break;
+    case Kind::ResAdd: rc = run_res_add(args); break;
+    case Kind::LmHeadF32: rc = run_lm_head_f32(args); break;
     }
     report(idx, rc);
 }
 
-}  // namespace
-
-extern "C" {
-
-int hm_ciface_bind_transformer(hm_ctx *ctx, const hm_transformer_config *cfg, int has_qk_norm) {
+int bind_common(hm_ctx *ctx, const hm_transformer_config *cfg, int has_qk_norm, int kernels, Bound *out) {
     HM_CHECK_CTX(ctx);
     HM_REQUIRE(ctx, cfg, "hm_ciface_bind_transformer: NULL config");
     const int kvh = cfg->num_key_value_heads ? cfg->num_key_value_heads : cfg->num_attention_heads;
     HM_REQUIRE(ctx, cfg->hidden_size > 0 && cfg->num_attention_heads > 0 && cfg->num_hidden_layers > 0 &&
                         cfg->num_attention_heads % kvh == 0,
                "hm_ciface_bind_transformer: bad config");
-    const int n = 3 * cfg->num_hidden_layers + 2;
-    HM_REQUIRE(ctx, n <= HM_CIFACE_MAX_KERNELS, "hm_ciface_bind_transformer: %d kernels, at most %d symbols are exported",
-               n, HM_CIFACE_MAX_KERNELS);
+    HM_REQUIRE(ctx, kernels <= HM_CIFACE_MAX_KERNELS, "hm_ciface_bind_transformer: %d kernels, at most %d symbols are exported",
+               kernels, HM_CIFACE_MAX_KERNELS);
     Bound b;
     b.ctx = ctx;
     b.cfg = *cfg;
@@ -250,6 +419,57 @@ int hm_ciface_bind_transformer(hm_ctx *ctx, const hm_transformer_config *cfg, in
     b.q_dim = cfg->num_attention_heads * b.head_dim;
     b.kv_dim = kvh * b.head_dim;
     if (b.cfg.rms_norm_eps <= 0) b.cfg.rms_norm_eps = 1e-6;
+    *out = std::move(b);
+    return HM_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int hm_ciface_bind_transformer_quant(hm_ctx *ctx, const hm_transformer_config *cfg, const int *proj_dtypes,
+                                     int has_qk_norm) {
+    Bound b;
+    const int rc = bind_common(ctx, cfg, has_qk_norm, cfg ? 13 * cfg->num_hidden_layers + 2 : 0, &b);
+    if (rc != HM_OK) return rc;
+    HM_REQUIRE(ctx, proj_dtypes, "hm_ciface_bind_transformer_quant: NULL projection types");
+    const int hidden = cfg->hidden_size, inter = cfg->intermediate_size;
+    const int kdim[7] = {hidden, hidden, hidden, b.q_dim, hidden, hidden, inter};
+    const int ndim[7] = {b.q_dim, b.kv_dim, b.kv_dim, hidden, inter, inter, hidden};
+    b.kinds.push_back(Kind::Embed);
+    for (int l = 0; l < cfg->num_hidden_layers; l++) {
+        const int *t = proj_dtypes + 7 * l;
+        for (int j = 0; j < 7; j++) {
+            const bool kq = t[j] == HM_DTYPE_Q4_K || t[j] == HM_DTYPE_Q6_K;
+            HM_REQUIRE(ctx, kq || t[j] == HM_DTYPE_Q8_0 || t[j] == HM_DTYPE_Q4_0,
+                       "hm_ciface_bind_transformer_quant: layer %d projection %d: dtype %d is not a block format", l, j, t[j]);
+            HM_REQUIRE(ctx, kdim[j] % (kq ? 256 : 32) == 0, "hm_ciface_bind_transformer_quant: layer %d projection %d: K=%d", l, j,
+                       kdim[j]);
+        }
+        auto mm = [&](int j) { return KernelInfo(kdim[j], ndim[j], t[j]); };
+        b.kinds.push_back(Kind::RmsNorm);
+        b.kinds.push_back(mm(0));
+        b.kinds.push_back(mm(1));
+        b.kinds.push_back(mm(2));
+        b.kinds.push_back(Kind::PostQkv);
+        b.kinds.push_back(Kind::AttnBody);
+        b.kinds.push_back(mm(3));
+        b.kinds.push_back(Kind::ResidualNorm);
+        b.kinds.push_back(mm(4));
+        b.kinds.push_back(mm(5));
+        b.kinds.push_back(Kind::SiluMul);
+        b.kinds.push_back(mm(6));
+        b.kinds.push_back(Kind::ResAdd);
+    }
+    b.kinds.push_back(Kind::LmHeadF32);
+    g_bound = std::move(b);
+    return HM_OK;
+}
+
+int hm_ciface_bind_transformer(hm_ctx *ctx, const hm_transformer_config *cfg, int has_qk_norm) {
+    Bound b;
+    const int rc = bind_common(ctx, cfg, has_qk_norm, cfg ? 3 * cfg->num_hidden_layers + 2 : 0, &b);
+    if (rc != HM_OK) return rc;
     b.kinds.push_back(Kind::Embed);
     for (int l = 0; l < cfg->num_hidden_layers; l++) {
         b.kinds.push_back(Kind::Qkv);
@@ -265,15 +485,17 @@ int hm_ciface_num_kernels(void) { return (int)g_bound.kinds.size(); }
 
 void hm_ciface_unbind(void) { g_bound = Bound(); }
 
-// 256 exported symbols _mlir__mlir_ciface_k0 ... _mlir__mlir_ciface_k255
+// HM_CIFACE_MAX_KERNELS exported symbols _mlir__mlir_ciface_k0 ... _mlir__mlir_ciface_k1023
 #define HM_K(i) \
     __attribute__((visibility("default"))) void _mlir__mlir_ciface_k##i(void **args) { dispatch(i, args); }
 #define HM_K10(p) HM_K(p##0) HM_K(p##1) HM_K(p##2) HM_K(p##3) HM_K(p##4) HM_K(p##5) HM_K(p##6) HM_K(p##7) HM_K(p##8) HM_K(p##9)
+#define HM_K100(p) HM_K10(p##0) HM_K10(p##1) HM_K10(p##2) HM_K10(p##3) HM_K10(p##4) HM_K10(p##5) HM_K10(p##6) HM_K10(p##7) HM_K10(p##8) HM_K10(p##9)
 HM_K(0) HM_K(1) HM_K(2) HM_K(3) HM_K(4) HM_K(5) HM_K(6) HM_K(7) HM_K(8) HM_K(9)
 HM_K10(1) HM_K10(2) HM_K10(3) HM_K10(4) HM_K10(5) HM_K10(6) HM_K10(7) HM_K10(8) HM_K10(9)
-HM_K10(10) HM_K10(11) HM_K10(12) HM_K10(13) HM_K10(14) HM_K10(15) HM_K10(16) HM_K10(17) HM_K10(18) HM_K10(19)
-HM_K10(20) HM_K10(21) HM_K10(22) HM_K10(23) HM_K10(24)
-HM_K(250) HM_K(251) HM_K(252) HM_K(253) HM_K(254) HM_K(255)
+HM_K100(1) HM_K100(2) HM_K100(3) HM_K100(4) HM_K100(5) HM_K100(6) HM_K100(7) HM_K100(8) HM_K100(9)
+HM_K10(100) HM_K10(101)
+HM_K(1020) HM_K(1021) HM_K(1022) HM_K(1023)
+#undef HM_K100
 #undef HM_K10
 #undef HM_K
 

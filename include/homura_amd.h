@@ -429,7 +429,7 @@ hm_model *hm_model_load_hf_dir(hm_ctx *ctx, const char *dir, int max_seq_len);
 
 /* ── the reference's kernel ABI, literally ─────────────────────────────────
  * The library also exports HM_CIFACE_MAX_KERNELS symbols
- *     void _mlir__mlir_ciface_k0(void **args) ... void _mlir__mlir_ciface_k255(void **args)
+ *     void _mlir__mlir_ciface_k0(void **args) ... void _mlir__mlir_ciface_k1023(void **args)
  * with the signature and argument convention of the reference's compiled kernels: args[i]
  * points at a pointer to a rank-N memref descriptor {allocated, aligned, offset, sizes[N],
  * strides[N]} (src/runtime.rs:654-698, :930-1037), inputs first, outputs after; `aligned` holds
@@ -437,11 +437,18 @@ hm_model *hm_model_load_hf_dir(hm_ctx *ctx, const char *dir, int max_seq_len);
  * dlsym exactly as it resolves its own. hm_ciface_bind_transformer tells the library which
  * fused kernel each index is, in emit_transformer_plan's numbering (src/hf/emitter.rs:902-1014):
  * k0 Embed, k(3l+1) QKV(+QK-norm)+RoPE, k(3l+2) Attn, k(3l+3) MLP for layer l, then LMHead;
- * bf16 weights [K,N], f32 K/V views with the cache's strides, one token per call. A failure
- * cannot be returned (the ABI is void): it is recorded for hm_last_error and printed to stderr.
- * One binding per process at a time. */
-#define HM_CIFACE_MAX_KERNELS 256
+ * bf16 weights [K,N], f32 K/V views with the cache's strides, one token per call.
+ * hm_ciface_bind_transformer_quant does the same for emit_transformer_plan_quant's numbering
+ * (src/hf/emitter_quant.rs:1170-1440): k0 Embed; for layer l the thirteen kernels k(13l+1) ..
+ * k(13l+13) = RMSNorm, QuantMM Q, K, V, PostQKV, AttnBody, QuantMM O, Residual+Norm, QuantMM Gate, Up,
+ * SiLU*Up, QuantMM Down, ResAdd; then the LMHead with f32 weights [hidden, vocab]. proj_dtypes: 7
+ * HM_DTYPE_* block formats per layer (q k v o gate up down); the weights are the raw GGUF blocks.
+ * A failure cannot be returned (the ABI is void): it is recorded for hm_last_error and printed to
+ * stderr. One binding per process at a time. */
+#define HM_CIFACE_MAX_KERNELS 1024
 int hm_ciface_bind_transformer(hm_ctx *ctx, const hm_transformer_config *cfg, int has_qk_norm);
+int hm_ciface_bind_transformer_quant(hm_ctx *ctx, const hm_transformer_config *cfg, const int *proj_dtypes,
+                                     int has_qk_norm);
 int hm_ciface_num_kernels(void);
 void hm_ciface_unbind(void);
 

@@ -128,6 +128,96 @@ def test_plan_through_memref_entry_points(ctx, which):
     ctx.lib.hm_ciface_unbind()
 
 
+@pytest.mark.parametrize("which", ["q8_0", "q4_k_m_mix", "q4_0_bias"])
+def test_quantised_plan_through_memref_entry_points(ctx, which):
+    """emit_transformer_plan_quant's kernels (reference src/hf/emitter_quant.rs:1170-1440) in plan
+    order: k0 Embed, thirteen kernels per layer, the f32 LMHead."""
+    import dataclasses
+    if which == "q8_0":
+        cfg, mix = synth_model.TINY_LLAMA, [2] * 7 * synth_model.TINY_LLAMA.num_hidden_layers
+    elif which == "q4_0_bias":
+        cfg = dataclasses.replace(synth_model.TINY_LLAMA, attention_bias=True)
+        mix = [3] * 7 * cfg.num_hidden_layers
+    else:
+        cfg, mix = synth_model.TINY_K, synth_model.q4_k_m_mix(synth_model.TINY_K)
+    weights = synth_model.synth_weights(cfg, 271, has_qk_norm=False, proj_dtypes=mix)
+    L, hidden, inter, vocab = cfg.num_hidden_layers, cfg.hidden_size, cfg.intermediate_size, cfg.vocab_size
+    H, kvh, hd = cfg.num_attention_heads, cfg.kv_heads(), cfg.get_head_dim()
+    qd, kvd = H * hd, kvh * hd
+    max_len, past, steps = 64, 9, 3
+    om = mf.build_oracle_model(cfg, weights, max_len, has_qk_norm=False, proj_dtypes=mix)
+    kv = synth_model.synth_kv(cfg, 12, past)
+    mf.oracle_init_kv(om, kv)
+
+    lib = C.CDLL(str(_ffi.LIB_PATH))
+    ccfg = cfg.to_c()
+    arr = (C.c_int * len(mix))(*mix)
+    ctx._check(ctx.lib.hm_ciface_bind_transformer_quant(ctx.h, C.byref(ccfg), arr, 0))
+    assert ctx.lib.hm_ciface_num_kernels() == 13 * L + 2
+
+    dev = {n: ctx.to_device(a) for n, a in weights}     # the reference's slot buffers, as they are
+    cos, sin = om.cos, om.sin
+    cache = []
+    for l in range(2 * L):                               # f32 caches [1, kvh, max_len, hd]
+        full = np.zeros((kvh, max_len, hd), np.float32)
+        full[:, :past] = kv[l][0]
+        cache.append(ctx.to_device(full))
+    f = lambda n: ctx.empty(n)
+    d_h = [f(hidden), f(hidden)]
+    d_normed, d_qr, d_kr, d_vr = f(hidden), f(qd), f(kvd), f(kvd)
+    d_q, d_k, d_v, d_body, d_attn = f(qd), f(kvd), f(kvd), f(qd), f(hidden)
+    d_resid, d_pnorm, d_gate, d_up, d_silu, d_down = f(hidden), f(hidden), f(inter), f(inter), f(inter), f(hidden)
+    d_logits, d_mask = f(vocab), f(max_len)
+    row = lambda buf, n: Desc(buf.ptr, [1, 1, n])
+    ids = synth.token_ids(21, steps, vocab)
+    cur = past
+    for t in range(steps):
+        say(f"quant {which}: token {t} at position {cur}")
+        d_ids = ctx.to_device(ids[t:t + 1].astype(np.int64))
+        d_cos, d_sin = ctx.to_device(cos[cur:cur + 1]), ctx.to_device(sin[cur:cur + 1])
+        call(lib, 0, [Desc(d_ids.ptr, [1, 1]), Desc(dev["model.embed_tokens.weight"].ptr, [vocab, hidden]), row(d_h[0], hidden)])
+        for l in range(L):
+            p, k0 = f"model.layers.{l}.", 13 * l + 1
+            w = lambda name: Desc(dev[p + name].ptr, [dev[p + name].nbytes])      # flat bytes
+            vec = lambda name, n: Desc(dev[p + name].ptr, [n])
+            call(lib, k0 + 0, [row(d_h[0], hidden), vec("input_layernorm.weight", hidden), row(d_normed, hidden)])
+            call(lib, k0 + 1, [row(d_normed, hidden), w("self_attn.q_proj.weight"), row(d_qr, qd)])
+            call(lib, k0 + 2, [row(d_normed, hidden), w("self_attn.k_proj.weight"), row(d_kr, kvd)])
+            call(lib, k0 + 3, [row(d_normed, hidden), w("self_attn.v_proj.weight"), row(d_vr, kvd)])
+            post = [row(d_qr, qd), row(d_kr, kvd), row(d_vr, kvd)]
+            if cfg.attention_bias:
+                post += [vec("self_attn.q_proj.bias", qd), vec("self_attn.k_proj.bias", kvd), vec("self_attn.v_proj.bias", kvd)]
+            post += [Desc(d_cos.ptr, [1, hd]), Desc(d_sin.ptr, [1, hd])]
+            post += [Desc(d_q.ptr, [1, 1, H, hd]), Desc(d_k.ptr, [1, kvh, 1, hd]), Desc(d_v.ptr, [1, kvh, 1, hd])]
+            call(lib, k0 + 4, post)
+            for which_kv, src in ((0, d_k), (1, d_v)):   # NativeOp::Concat on the cache
+                c = cache[2 * l + which_kv]
+                for h in range(kvh):
+                    ctx._check(ctx.lib.hm_copy(ctx.h, c.ptr + ((h * max_len + cur) * hd) * 4, src.ptr + h * hd * 4, hd * 4))
+            view = lambda c: Desc(c.ptr, [1, kvh, cur + 1, hd], [kvh * max_len * hd, max_len * hd, hd, 1])
+            call(lib, k0 + 5, [Desc(d_q.ptr, [1, 1, H, hd]), view(cache[2 * l]), view(cache[2 * l + 1]),
+                               Desc(d_mask.ptr, [1, 1, 1, cur + 1]), row(d_body, qd)])
+            call(lib, k0 + 6, [row(d_body, qd), w("self_attn.o_proj.weight"), row(d_attn, hidden)])
+            call(lib, k0 + 7, [row(d_h[0], hidden), row(d_attn, hidden), vec("post_attention_layernorm.weight", hidden),
+                               row(d_resid, hidden), row(d_pnorm, hidden)])
+            call(lib, k0 + 8, [row(d_pnorm, hidden), w("mlp.gate_proj.weight"), row(d_gate, inter)])
+            call(lib, k0 + 9, [row(d_pnorm, hidden), w("mlp.up_proj.weight"), row(d_up, inter)])
+            call(lib, k0 + 10, [row(d_gate, inter), row(d_up, inter), row(d_silu, inter)])
+            call(lib, k0 + 11, [row(d_silu, inter), w("mlp.down_proj.weight"), row(d_down, hidden)])
+            call(lib, k0 + 12, [row(d_resid, hidden), row(d_down, hidden), row(d_h[1], hidden)])
+            d_h.reverse()
+        call(lib, 13 * L + 1, [row(d_h[0], hidden), Desc(dev["model.norm.weight"].ptr, [hidden]),
+                               Desc(dev["lm_head.weight"].ptr, [hidden, vocab]), row(d_logits, vocab)])
+        got = d_logits.download(np.float32)
+        want = om.run_kv(ids[t:t + 1])[0]
+        err = mf.rel_err(got, want)
+        say(f"quant {which}: token {t} logits rel err {err:.2e}")
+        assert err < 1e-2
+        assert int(len(got) - 1 - np.argmax(got[::-1])) == int(len(want) - 1 - np.argmax(want[::-1]))
+        cur += 1
+    ctx.lib.hm_ciface_unbind()
+
+
 def test_unbound_call_is_reported_not_fatal(ctx, capfd):
     """No binding: the entry point records an error and returns (the ABI has no status)."""
     ctx.lib.hm_ciface_unbind()
