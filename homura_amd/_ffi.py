@@ -164,6 +164,7 @@ SIGNATURES = {
                              C.POINTER(C.c_int32)]),
     "hm_model_set_prefill_min": (_I, [_P, _I]),
     "hm_model_set_prefill_pieces": (_I, [_P, _I]),
+    "hm_model_set_prefill_weight_cache": (_I, [_P, _SZ]),
     "hm_model_generate_greedy": (_I, [_P, C.POINTER(C.c_int64), _I, _I, C.POINTER(C.c_int32)]),
     "hm_model_bench_decode": (_I, [_P, C.c_int64, _I, c_f32_p, C.POINTER(C.c_int32)]),
     "hm_model_profile_step": (_I, [_P, C.c_int64, C.POINTER(HmKernelProfile), _I]),

@@ -88,6 +88,12 @@ int hm_model_set_prefill_pieces(hm_model *m, int pieces) {
     return HM_OK;
 }
 
+int hm_model_set_prefill_weight_cache(hm_model *m, size_t bytes) {
+    if (!m) return HM_ERR_INVALID;
+    m->impl->set_prefill_weight_cache(bytes);
+    return HM_OK;
+}
+
 int hm_model_set_prefill_min(hm_model *m, int n_tokens) {
     if (!m || n_tokens < 0) return HM_ERR_INVALID;
     m->impl->set_prefill_min(n_tokens);

@@ -88,6 +88,10 @@ class HfModel {
     // bf16 pieces per f32 activation in the prefill pass: 3 (all 24 significant bits, default) or 2
     // (16 bits, two thirds of the matrix-core work)
     void set_prefill_pieces(int n) { prefill_pieces_ = n; }
+    // Block-quantised models: HBM the prompt pass may keep for the dequantised projections (three bf16
+    // pieces per weight, 6 bytes). When all of them fit, they are written once and stay; otherwise
+    // (or with 0) every chunk dequantises them again into one scratch matrix.
+    void set_prefill_weight_cache(size_t bytes);
     int init_kv_cache(const float *const *h_kv, int seq_len);
     int reset_kv_cache();
     int kv_cache_len() const;
@@ -137,11 +141,13 @@ class HfModel {
         int rows = 0;
         Buffer ids, h, resid, split, qkv, proj_out, gate_up, logits;
         Buffer wsplit;  // block formats: the matrices of one group of projections as three bf16 pieces per weight
+        std::vector<Buffer> wcache;  // [layer * 4 + group] resident copies of the same (q|k|v, o, gate|up, down)
     };
     PrefillScratch pf_;
     struct SamplerScratch { Buffer work, counts, token, list; int list_cap = 0; } sampler_;
     int prefill_min_ = 8;
     int prefill_pieces_ = 3;
+    size_t prefill_weight_cache_bytes_ = (size_t)32 << 30;
     std::map<std::string, int> slot_by_name_;
     std::unique_ptr<ExecutionPlan> plan_;
 };

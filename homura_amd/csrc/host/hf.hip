@@ -1197,6 +1197,12 @@ bool HfModel::prefill_available() const {
     return true;
 }
 
+void HfModel::set_prefill_weight_cache(size_t bytes) {
+    prefill_weight_cache_bytes_ = bytes;
+    if (ctx_) hm_sync(ctx_);
+    pf_.wcache.clear();
+}
+
 const float *HfModel::weight_f32(const std::string &name) const {
     auto it = slot_by_name_.find(name);
     return it == slot_by_name_.end() ? nullptr : weight_bufs_[it->second].as<float>();
@@ -1278,11 +1284,30 @@ int HfModel::prefill_chunk(const int32_t *h_ids, int n, float *h_logits) {
     // (reference emit_quant_matmul_kernel, src/hf/emitter_quant.rs:675-702): the members are
     // dequantised into wsplit one under the other, or row-interleaved for gate|up, which is the order
     // the packed bf16 matrices have.
+    // Resident pieces: when six bytes per projection weight fit the budget (and leave an eighth of the
+    // device free), each group's matrix is dequantised on first use and kept.
+    if (quant && p.wcache.empty() && prefill_weight_cache_bytes_ > 0) {
+        const size_t per_layer = ((size_t)nqkv * hidden + (size_t)hidden * qd + 3 * (size_t)inter * hidden) * 6;
+        size_t free_b = 0, total_b = 0;
+        if (hipMemGetInfo(&free_b, &total_b) != hipSuccess) free_b = total_b = 0;
+        const size_t need = per_layer * c.num_hidden_layers;
+        if (need <= prefill_weight_cache_bytes_ && need + total_b / 8 <= free_b) p.wcache.resize((size_t)c.num_hidden_layers * 4);
+    }
     auto project = [&](int l, int first, int count, const Buffer &packed, int K, float *out) -> int {
         int N = 0;
         for (int j = first; j < first + count; j++) N += proj_n[j];
         if (!quant) return gemm_split_nk(ctx_, split, np, packed.as<uint16_t>(), out, n, K, N, MP, &parts);
         const bool interleave = first == 4 && count == 2;
+        uint16_t *wsplit = p.wsplit.as<uint16_t>();
+        if (!p.wcache.empty()) {
+            Buffer &slot = p.wcache[(size_t)l * 4 + (first == 0 ? 0 : first == 3 ? 1 : first == 4 ? 2 : 3)];
+            if (slot) return gemm_split_split_nk(ctx_, split, slot.as<uint16_t>(), out, n, K, N, MP, &parts);
+            slot = Buffer::alloc(ctx_, {(int64_t)N, 3 * (int64_t)K}, DType::BF16);
+            if (slot)
+                wsplit = slot.as<uint16_t>();
+            else
+                (void)hipGetLastError();  // out of memory: this group keeps using the scratch matrix
+        }
         int row = 0;
         for (int j = first; j < first + count; j++) {
             auto it = slot_by_name_.find("model.layers." + std::to_string(l) + "." + proj_name[j]);

@@ -436,6 +436,10 @@ class HfModel:
             out.ctypes.data_as(C.POINTER(C.c_int32)), C.byref(n)))
         return out[:n.value].copy()
 
+    def set_prefill_weight_cache(self, nbytes: int):
+        """Block-quantised models: HBM the prompt pass may keep for dequantised projections (0 = none)."""
+        self._check(self.lib.hm_model_set_prefill_weight_cache(self.h, nbytes))
+
     def set_prefill_pieces(self, pieces: int):
         """bf16 numbers per f32 activation in the prefill pass: 3 (default, exact) or 2."""
         self._check(self.lib.hm_model_set_prefill_pieces(self.h, pieces))

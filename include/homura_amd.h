@@ -327,6 +327,12 @@ int hm_model_run_kv(hm_model *m, const int64_t *h_ids, int n_ids, float *h_logit
 int hm_model_prefill(hm_model *m, const int64_t *h_ids, int n_ids, float *h_logits);
 int hm_model_set_prefill_min(hm_model *m, int n_tokens);
 int hm_model_set_prefill_pieces(hm_model *m, int pieces);
+/* Block-quantised models: HBM the prompt pass may keep for the dequantised projections (three bf16
+ * pieces = 6 bytes per weight; default 32 GiB). If all projections fit, and an eighth of the device
+ * stays free, each is dequantised on first use and kept; otherwise, or with 0, every chunk
+ * dequantises them again into one scratch matrix. No counterpart in the reference (its CPU kernels
+ * dequantise in registers). */
+int hm_model_set_prefill_weight_cache(hm_model *m, size_t bytes);
 
 /* The greedy loop of generate_streaming_core (src/generate.rs:187-270) with pure argmax:
  * the prompt is consumed as incremental prefill through run_kv, then n_new tokens are

@@ -183,6 +183,24 @@ def test_quantised_generate_routes_the_prompt_through_prefill(ctx):
     gm.close()
 
 
+def test_resident_and_per_chunk_dequantisation_agree(ctx):
+    """The dequantised projections are kept in HBM when they fit the budget (default) or rebuilt for
+    every chunk (budget 0): the same bits either way, on first use and on reuse."""
+    cfg, mix = _quant_case("q8_0_and_k_quants_by_group")
+    weights = synth_model.synth_weights(cfg, 5, has_qk_norm=False, proj_dtypes=mix)
+    gm = synth_model.build_model(ctx, cfg, weights, 128, has_qk_norm=False, proj_dtypes=mix)
+    ids = synth.token_ids(6, 40, cfg.vocab_size)
+    runs = []
+    for budget in (None, None, 0, 1 << 30):
+        if budget is not None:
+            gm.set_prefill_weight_cache(budget)
+        gm.reset_kv_cache()
+        runs.append(gm.prefill(ids))
+    for r in runs[1:]:
+        assert np.array_equal(r.view(np.uint32), runs[0].view(np.uint32))
+    gm.close()
+
+
 def test_prefill_needs_matching_widths_and_groups(ctx):
     """Block formats take the prompt pass when the widths are multiples of the 64-wide K tile and
     q|k|v, gate|up each multiply with one kind of activation; otherwise run_kv steps token by token."""
