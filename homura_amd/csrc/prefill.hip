@@ -16,6 +16,7 @@
 #include "prefill.h"
 
 #include <algorithm>
+#include <cstdlib>
 
 #include "gemm_bf16_mfma.h"
 #include "quant_formats.h"
@@ -296,8 +297,13 @@ __global__ __launch_bounds__(256) void qkv_post_kernel(QkvPostArgs a) {
 // ── causal attention ─────────────────────────────────────────────────────────
 
 constexpr int AT_THREADS = 256;
-constexpr int AT_QROWS = 128;  // query rows per workgroup: 4 wavefronts x 32
-constexpr int AT_KEYS = 64;    // keys per tile
+constexpr int AT_WAVES = AT_THREADS / 64;
+constexpr int AT_KEYS = 64;  // keys per tile
+// A workgroup's four wavefronts are 4 / KS blocks of 32 query rows times KS key groups: with KS > 1
+// the wavefronts of a row block take every KS-th key tile each (KS tiles are staged per round) and
+// their partial softmax sums meet in LDS at the end. KS = 1: 128 rows per workgroup, the fewest tile
+// loads; KS = 2, 4: 64, 32 rows, for prompts whose rows x heads alone leave most of the chip idle, and
+// a KS times shorter chain of tiles per wavefront.
 
 // V^T tile: row d holds 64 keys = 128 bytes = eight 16-byte chunks, chunk c of row r at slot
 // c ^ (r & 7) ^ ((r >> 3) & 7): conflict-free for the operand reads (32 consecutive rows, one chunk)
@@ -312,16 +318,21 @@ __device__ __forceinline__ int k_off(int key, int chunk) {
     return key * 128 + ((chunk ^ (key & 7) ^ ((key >> 3) & 7)) << 4);
 }
 
-template <int HD, int NP>
+extern __shared__ __attribute__((aligned(16))) char at_lds[];
+
+template <int HD, int NP, int KS>
 __global__ __launch_bounds__(AT_THREADS) void prefill_attn_kernel(PrefillAttnArgs a) {
     constexpr int CH = HD / 8;                        // 16-byte chunks per K row
     constexpr int KLOADS = AT_KEYS * CH / AT_THREADS;  // K chunks per thread per tile
     constexpr int KSTEPS = HD / 16;                   // k steps of K . Q
     constexpr int DB = HD / 32;                       // 32-row blocks of O^T
-    __shared__ __attribute__((aligned(16))) char k_lds[AT_KEYS * HD * 2];
-    __shared__ __attribute__((aligned(16))) char v_lds[HD * 128];
+    constexpr int QW = AT_WAVES / KS;                 // 32-row query blocks per workgroup
+    constexpr int AT_QROWS = 32 * QW;
+    constexpr int K_TILE = AT_KEYS * HD * 2, V_TILE = HD * 128;  // bytes; KS of each
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, lh = lane >> 5;
+    const int qw = wave % QW, kh = wave / QW;  // row block and key group of this wavefront
+    char *k_lds = at_lds + kh * K_TILE, *v_lds = at_lds + KS * K_TILE + kh * V_TILE;
     const int h = blockIdx.y, kvhd = h / (a.H / a.kvh);
     const int q0 = blockIdx.x * AT_QROWS;
     const int kv_total = a.past + a.S;
@@ -329,7 +340,7 @@ __global__ __launch_bounds__(AT_THREADS) void prefill_attn_kernel(PrefillAttnArg
     const uint16_t *vc = a.vcache + (size_t)kvhd * a.max_len * HD;
 
     // this lane's query (rows past the end repeat the last one and are not stored)
-    const int qrow = q0 + wave * 32 + l32;
+    const int qrow = q0 + qw * 32 + l32;
     const int qc = min(qrow, a.S - 1);
     const int qabs = a.past + qc;
     bf16x8 qp_[KSTEPS][NP];
@@ -352,42 +363,51 @@ __global__ __launch_bounds__(AT_THREADS) void prefill_attn_kernel(PrefillAttnArg
 
     // keys [0, wg_end) are visible to some row of the workgroup, [0, wave_end) to some row of this wavefront
     const int wg_end = a.past + min(a.S, q0 + AT_QROWS);
-    const int wave_end = q0 + wave * 32 < a.S ? a.past + min(a.S, q0 + wave * 32 + 32) : 0;
+    const int wave_end = q0 + qw * 32 < a.S ? a.past + min(a.S, q0 + qw * 32 + 32) : 0;
     const int ntiles = (wg_end + AT_KEYS - 1) / AT_KEYS;
-    const int wave_first = a.past + min(q0 + wave * 32, a.S - 1);  // smallest position among this wavefront's rows
+    const int nrounds = (ntiles + KS - 1) / KS;  // KS tiles are staged per round, tile r KS + u in buffer u
+    const int wave_first = a.past + min(q0 + qw * 32, a.S - 1);  // smallest position among this wavefront's rows
 
-    // thread's share of a tile on its way from the cache to LDS
-    u32x4 kr[KLOADS], vr[4];
+    // thread's share of the KS tiles of a round on their way from the cache to LDS
+    u32x4 kr[KS][KLOADS], vr[KS][4];
     const int v_ng = tid % CH, v_kg = tid / CH;  // V: a 4(key) x 8(d) block per thread
     const bool v_on = v_kg < 16;
-    auto request_tile = [&](int t) {
+    auto request_round = [&](int r) {
 #pragma unroll
-        for (int j = 0; j < KLOADS; j++) {
-            const int id = tid + j * AT_THREADS, key = id / CH, c = id % CH;
-            const int row = min(t * AT_KEYS + key, kv_total - 1);
-            kr[j] = ld128(kc + (size_t)row * HD + c * 8);
-        }
+        for (int u = 0; u < KS; u++) {
+            const int t = r * KS + u;
 #pragma unroll
-        for (int r = 0; r < 4; r++) {
-            const int row = min(t * AT_KEYS + (v_on ? v_kg : 0) * 4 + r, kv_total - 1);
-            vr[r] = ld128(vc + (size_t)row * HD + v_ng * 8);
+            for (int j = 0; j < KLOADS; j++) {
+                const int id = tid + j * AT_THREADS, key = id / CH, c = id % CH;
+                const int row = min(t * AT_KEYS + key, kv_total - 1);
+                kr[u][j] = ld128(kc + (size_t)row * HD + c * 8);
+            }
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                const int row = min(t * AT_KEYS + (v_on ? v_kg : 0) * 4 + q, kv_total - 1);
+                vr[u][q] = ld128(vc + (size_t)row * HD + v_ng * 8);
+            }
         }
     };
-    auto store_tile = [&]() {
+    auto store_round = [&]() {
 #pragma unroll
-        for (int j = 0; j < KLOADS; j++) {
-            const int id = tid + j * AT_THREADS, key = id / CH, c = id % CH;
-            *reinterpret_cast<u32x4 *>(k_lds + k_off<HD>(key, c)) = kr[j];
-        }
-        if (v_on) {
+        for (int u = 0; u < KS; u++) {
+            char *kd = at_lds + u * K_TILE, *vd = at_lds + KS * K_TILE + u * V_TILE;
 #pragma unroll
-            for (int i = 0; i < 8; i++) {
-                // column d = v_ng*8 + i of the block: keys +0..+3 packed low to high
-                const uint32_t sel = (i & 1) ? 0x07060302u : 0x05040100u;
-                u32x2 col;
-                col.x = __builtin_amdgcn_perm(vr[1][i >> 1], vr[0][i >> 1], sel);
-                col.y = __builtin_amdgcn_perm(vr[3][i >> 1], vr[2][i >> 1], sel);
-                *reinterpret_cast<u32x2 *>(v_lds + vt_off(v_ng * 8 + i, v_kg >> 1) + (v_kg & 1) * 8) = col;
+            for (int j = 0; j < KLOADS; j++) {
+                const int id = tid + j * AT_THREADS, key = id / CH, c = id % CH;
+                *reinterpret_cast<u32x4 *>(kd + k_off<HD>(key, c)) = kr[u][j];
+            }
+            if (v_on) {
+#pragma unroll
+                for (int i = 0; i < 8; i++) {
+                    // column d = v_ng*8 + i of the block: keys +0..+3 packed low to high
+                    const uint32_t sel = (i & 1) ? 0x07060302u : 0x05040100u;
+                    u32x2 col;
+                    col.x = __builtin_amdgcn_perm(vr[u][1][i >> 1], vr[u][0][i >> 1], sel);
+                    col.y = __builtin_amdgcn_perm(vr[u][3][i >> 1], vr[u][2][i >> 1], sel);
+                    *reinterpret_cast<u32x2 *>(vd + vt_off(v_ng * 8 + i, v_kg >> 1) + (v_kg & 1) * 8) = col;
+                }
             }
         }
     };
@@ -401,12 +421,13 @@ __global__ __launch_bounds__(AT_THREADS) void prefill_attn_kernel(PrefillAttnArg
     // MFMA row r of a key block holds key pi(r) = r with bits 2 and 3 swapped
     const int pi = (l32 & 0x13) | ((l32 & 4) << 1) | ((l32 & 8) >> 1);
 
-    request_tile(0);
-    for (int t = 0; t < ntiles; t++) {
-        __syncthreads();  // the previous tile has been read by everybody
-        store_tile();
+    request_round(0);
+    for (int r = 0; r < nrounds; r++) {
+        __syncthreads();  // the previous tiles have been read by everybody
+        store_round();
         __syncthreads();
-        if (t + 1 < ntiles) request_tile(t + 1);
+        if (r + 1 < nrounds) request_round(r + 1);
+        const int t = r * KS + kh;               // this wavefront's tile of the round
         if (t * AT_KEYS >= wave_end) continue;  // wavefront-uniform: nothing visible to these 32 rows
 
         f32x16 s[2];
@@ -442,9 +463,11 @@ __global__ __launch_bounds__(AT_THREADS) void prefill_attn_kernel(PrefillAttnArg
         mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
         // The reference point of the exponentials only has to be near the maximum, not on it (softmax is
         // shift-invariant and l, O are f32): it moves when the maximum has grown by more than 2^8, so
-        // after the first tiles the rescaling of O is skipped for the whole wavefront. m_new is finite:
-        // key 0 is visible to every row. Both half-lanes of a query take the same decision.
-        const float m_new = mx > m_run + 8.0f ? mx : m_run;
+        // after the first tiles the rescaling of O is skipped for the whole wavefront. Both half-lanes of
+        // a query take the same decision. A row that has not seen a visible key yet (possible in key
+        // groups other than the first, whose tiles may lie wholly in a row's future) gets a finite
+        // floor as its reference point, so that every exponential below is 0 and not exp2(inf - inf).
+        const float m_new = fmaxf(mx > m_run + 8.0f ? mx : m_run, -1e30f);
         const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
         float psum = 0.f;
 #pragma unroll
@@ -482,6 +505,38 @@ __global__ __launch_bounds__(AT_THREADS) void prefill_attn_kernel(PrefillAttnArg
         }
     }
 
+    if (KS > 1) {
+        // The key groups of a row block meet: groups 1 .. KS-1 leave (O, m, l) in LDS, lane-major, and
+        // group 0 adds them in group order, rescaled to the larger reference point (a group that saw no
+        // visible key has m = -inf and weighs nothing; group 0 always sees key 0).
+        constexpr int PER_LANE = DB * 16 + 2;
+        float *xch = reinterpret_cast<float *>(at_lds);
+        __syncthreads();  // nobody reads tiles any more
+        if (kh > 0) {
+            float *mine = xch + (size_t)((kh - 1) * QW + qw) * PER_LANE * 64 + lane;
+#pragma unroll
+            for (int db = 0; db < DB; db++)
+#pragma unroll
+                for (int v = 0; v < 16; v++) mine[(db * 16 + v) * 64] = acc_o[db][v];
+            mine[(DB * 16) * 64] = m_run;
+            mine[(DB * 16 + 1) * 64] = l_run;
+        }
+        __syncthreads();
+        if (kh > 0) return;
+#pragma unroll
+        for (int g = 1; g < KS; g++) {
+            const float *other = xch + (size_t)((g - 1) * QW + qw) * PER_LANE * 64 + lane;
+            const float m_o = other[(DB * 16) * 64], l_o = other[(DB * 16 + 1) * 64];
+            const float m_new = fmaxf(m_run, m_o);
+            const float w_me = __builtin_amdgcn_exp2f(m_run - m_new), w_o = __builtin_amdgcn_exp2f(m_o - m_new);
+            l_run = l_run * w_me + l_o * w_o;
+            m_run = m_new;
+#pragma unroll
+            for (int db = 0; db < DB; db++)
+#pragma unroll
+                for (int v = 0; v < 16; v++) acc_o[db][v] = acc_o[db][v] * w_me + other[(db * 16 + v) * 64] * w_o;
+        }
+    }
     const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
     if (qrow >= a.S) return;
     const float inv = 1.0f / l_tot;
@@ -610,15 +665,42 @@ int prefill_attn_launch(hm_ctx *ctx, const PrefillAttnArgs &a) {
     HM_REQUIRE(ctx, (!a.out_f32 || ((uintptr_t)a.out_f32 % 16) == 0) && (!a.out_split || ((uintptr_t)a.out_split % 8) == 0),
                "prefill_attn: misaligned output");
     HM_REQUIRE(ctx, a.pieces == 2 || a.pieces == 3, "prefill_attn: %d pieces (2 or 3)", a.pieces);
-    const dim3 grid((unsigned)((a.S + AT_QROWS - 1) / AT_QROWS), (unsigned)a.H);
-    if (a.hd == 128 && a.pieces == 3)
-        hipLaunchKernelGGL((prefill_attn_kernel<128, 3>), grid, dim3(AT_THREADS), 0, ctx->stream, a);
-    else if (a.hd == 128)
-        hipLaunchKernelGGL((prefill_attn_kernel<128, 2>), grid, dim3(AT_THREADS), 0, ctx->stream, a);
-    else if (a.pieces == 3)
-        hipLaunchKernelGGL((prefill_attn_kernel<64, 3>), grid, dim3(AT_THREADS), 0, ctx->stream, a);
-    else
-        hipLaunchKernelGGL((prefill_attn_kernel<64, 2>), grid, dim3(AT_THREADS), 0, ctx->stream, a);
+    // the fewest key groups that still give every CU a workgroup (more groups mean more tile loads)
+    int ks = 4;
+    for (int cand = 1; cand < 4; cand *= 2)
+        if ((long long)((a.S + 128 / cand - 1) / (128 / cand)) * a.H >= ctx->num_cus) {
+            ks = cand;
+            break;
+        }
+    if (const char *e = getenv("HOMURA_PREFILL_KEY_GROUPS")) {
+        const int v = atoi(e);
+        if (v == 1 || v == 2 || v == 4) ks = v;
+    }
+    const int qrows = 128 / ks;
+    const dim3 grid((unsigned)((a.S + qrows - 1) / qrows), (unsigned)a.H);
+    const size_t lds = (size_t)ks * (AT_KEYS * a.hd * 2 + a.hd * 128);
+    auto launch = [&](auto kernel) -> int {
+        if (lds > 64 * 1024) {
+            const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+            HM_REQUIRE(ctx, e == hipSuccess, "prefill_attn: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));
+        }
+        hipLaunchKernelGGL(kernel, grid, dim3(AT_THREADS), lds, ctx->stream, a);
+        return HM_OK;
+    };
+    int rc = HM_OK;
+#define HM_AT_CASE(HDV, NPV)                                                             \
+    if (a.hd == HDV && a.pieces == NPV) {                                                \
+        if (ks == 1) rc = launch(prefill_attn_kernel<HDV, NPV, 1>);                      \
+        else if (ks == 2) rc = launch(prefill_attn_kernel<HDV, NPV, 2>);                 \
+        else rc = launch(prefill_attn_kernel<HDV, NPV, 4>);                              \
+    }
+    HM_AT_CASE(128, 3)
+    HM_AT_CASE(128, 2)
+    HM_AT_CASE(64, 3)
+    HM_AT_CASE(64, 2)
+#undef HM_AT_CASE
+    if (rc != HM_OK) return rc;
     HM_LAUNCH_CHECK(ctx);
     return HM_OK;
 }

@@ -381,8 +381,15 @@ def test_attention_uniform_keys_give_mean_of_values(ctx):
     (37, 14, 2, 64, 300, 33),       # g = 7, head_dim 64, nothing aligned
     (129, 4, 4, 64, 512, 64),       # MHA, one row into the second query block
     (64, 12, 2, 128, 256, 191)])    # g = 6, the last key tile is a single key short of full
-def test_gqa_prefill_attn(ctx, oracle, S, H, kvh, hd, max_len, past):
-    say(f"gqa_prefill_attn S={S} H={H} kvh={kvh} hd={hd} max_len={max_len} past={past}")
+@pytest.mark.parametrize("key_groups", [0, 1, 2, 4])
+def test_gqa_prefill_attn(ctx, oracle, monkeypatch, S, H, kvh, hd, max_len, past, key_groups):
+    """key_groups: how many wavefronts of a workgroup share a block of 32 query rows, each taking every
+    n-th key tile (0 = the launch's own choice by grid size; the others force a variant)."""
+    say(f"gqa_prefill_attn S={S} H={H} kvh={kvh} hd={hd} max_len={max_len} past={past} key groups {key_groups}")
+    if key_groups:
+        monkeypatch.setenv("HOMURA_PREFILL_KEY_GROUPS", str(key_groups))
+    else:
+        monkeypatch.delenv("HOMURA_PREFILL_KEY_GROUPS", raising=False)
     total = past + S
     q = synth.normal_f32(31, S * H * hd).reshape(S, H, hd)
     kb = synth.normal_bf16(32, kvh * max_len * hd).reshape(kvh, max_len, hd)
@@ -409,9 +416,11 @@ def test_gqa_prefill_attn(ctx, oracle, S, H, kvh, hd, max_len, past):
         buf.free()
 
 
-def test_prefill_attn_first_row_copies_its_value_row(ctx):
+@pytest.mark.parametrize("key_groups", [1, 2, 4])
+def test_prefill_attn_first_row_copies_its_value_row(ctx, monkeypatch, key_groups):
     """Position 0 on an empty cache sees one key: the output is exactly that V row for every head of
     the group, whatever q is (softmax of a single score is 1)."""
+    monkeypatch.setenv("HOMURA_PREFILL_KEY_GROUPS", str(key_groups))
     S, H, kvh, hd, L = 40, 4, 2, 128, 64
     q = synth.normal_f32(41, S * H * hd)
     kb = synth.normal_bf16(42, kvh * L * hd).reshape(kvh, L, hd)
