@@ -369,34 +369,38 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_nk_dma_kernel(const uint16_
 
     // this thread's two rows of A and of B: instruction j of wavefront w fills rows 8 (2 w + j) .. + 7
     const uint16_t *a_src[2], *b_src[2];
-    int dst_off[2];
 #pragma unroll
     for (int j = 0; j < 2; j++) {
         const int r = (wave * 2 + j) * 8 + (lane >> 3), s = lane & 7;
         const int c = s ^ (r & 7) ^ ((r >> 3) & 7);
         a_src[j] = A + (size_t)min(m0 + r, M - 1) * g.lda + c * 8;
         b_src[j] = B + (size_t)min(n0 + r, N - 1) * g.ldb + c * 8;
-        dst_off[j] = (wave * 2 + j) * 1024;
     }
-    // the next tile to request: stretch `pair`, k offset `koff` inside it (all scalar)
+    // where this wavefront's first instruction lands inside an operand tile (scalar: it goes to M0)
+    const int wave_dst = __builtin_amdgcn_readfirstlane(wave * 2048);
+    // The next tile to request: stretch `pair`, k offset `koff` inside it; abase / bbase are the column
+    // offsets of the stretch's pieces. All scalar and updated with a few instructions per tile: the
+    // loop is short enough for its bookkeeping to show in the run time.
     const int tiles_per_stretch = g.Kb / TK;
     int pair = kt_first / tiles_per_stretch, koff = (kt_first % tiles_per_stretch) * TK;
+    auto piece_base = [&](uint32_t pack) { return (int)((pack >> (2 * min(pair, g.npairs - 1))) & 3u) * g.Kb; };
+    int abase = piece_base(g.apack), bbase = piece_base(g.bpack);
     // a tile past the end re-reads one of the last stretch (nobody multiplies it), so every iteration
     // issues the same four loads and the wait counts below are exact
     auto request = [&](int buf) {
-        char *base = dma_lds + buf * (2 * TILE_BYTES);
-        const int pr = 2 * min(pair, g.npairs - 1);
-        const int ka = (int)((g.apack >> pr) & 3u) * g.Kb + koff;
-        const int kb = (int)((g.bpack >> pr) & 3u) * g.Kb + koff;
+        char *base = dma_lds + buf * (2 * TILE_BYTES) + wave_dst;
+        const int ka = abase + koff, kb = bbase + koff;
 #pragma unroll
         for (int j = 0; j < 2; j++) {
-            dma16(a_src[j] + ka, base + dst_off[j]);
-            dma16(b_src[j] + kb, base + TILE_BYTES + dst_off[j]);
+            dma16(a_src[j] + ka, base + j * 1024);
+            dma16(b_src[j] + kb, base + TILE_BYTES + j * 1024);
         }
         koff += TK;
-        if (koff == g.Kb) {
+        if (koff == g.Kb) {  // rare
             koff = 0;
             pair++;
+            abase = piece_base(g.apack);
+            bbase = piece_base(g.bpack);
         }
     };
 #pragma unroll
