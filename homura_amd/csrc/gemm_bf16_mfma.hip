@@ -336,9 +336,10 @@ __device__ __forceinline__ void dma16(const uint16_t *src, char *dst) {
 // The operand reads and their waits are written out: the compiler's own wait insertion stalls on
 // all outstanding LDS reads at the top of the loop, these wait only for the ones about to be used.
 // (LDS operations of a wavefront return in order.)
-__device__ __forceinline__ bf16x8 lds_read16(uint32_t addr) {
+template <int IMM>
+__device__ __forceinline__ bf16x8 lds_read16_imm(uint32_t addr) {
     bf16x8 v;
-    asm volatile("ds_read_b128 %0, %1" : "=v"(v) : "v"(addr) : "memory");
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(IMM) : "memory");
     return v;
 }
 
@@ -408,36 +409,46 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_nk_dma_kernel(const uint16_
 
     const int arow = wm * 64 + l32, brow = wn * 64 + l32;
     const int chunk0 = kgrp * 4 + lh, chunk1 = chunk0 + 2;  // this group's two k steps of a tile
-    int a_off[2][2], b_off[2][2];                           // [k step][i]
+    // LDS addresses of this lane's operands in buffer 0, [k step][i]. Buffers 1..3 are 32 KiB apart;
+    // the immediate offset of an LDS instruction has 16 bits, so buffers 2 and 3 get addresses of
+    // their own (64 KiB on) and the odd buffers the immediate 32 KiB.
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char *)dma_lds;
+    uint32_t a_lo[2][2], b_lo[2][2], a_hi[2][2], b_hi[2][2];
 #pragma unroll
     for (int i = 0; i < 2; i++) {
-        a_off[0][i] = lds_off(arow + i * 32, chunk0);
-        a_off[1][i] = lds_off(arow + i * 32, chunk1);
-        b_off[0][i] = TILE_BYTES + lds_off(brow + i * 32, chunk0);
-        b_off[1][i] = TILE_BYTES + lds_off(brow + i * 32, chunk1);
+        a_lo[0][i] = lds0 + lds_off(arow + i * 32, chunk0);
+        a_lo[1][i] = lds0 + lds_off(arow + i * 32, chunk1);
+        b_lo[0][i] = lds0 + TILE_BYTES + lds_off(brow + i * 32, chunk0);
+        b_lo[1][i] = lds0 + TILE_BYTES + lds_off(brow + i * 32, chunk1);
+#pragma unroll
+        for (int st = 0; st < 2; st++) {
+            a_hi[st][i] = a_lo[st][i] + 4 * TILE_BYTES;
+            b_hi[st][i] = b_lo[st][i] + 4 * TILE_BYTES;
+        }
     }
-
     // operand registers, two stages: the reads of the next step are in flight during the MFMAs
     bf16x8 af[2][2], bfr[2][2];
-    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char *)dma_lds;
-    // tiles 1..3 (four loads each) may still be in flight; tile 0 has landed for everyone
-    asm volatile("s_waitcnt vmcnt(12)\n\ts_barrier" ::: "memory");
-#pragma unroll
-    for (int i = 0; i < 2; i++) {
-        af[0][i] = lds_read16(lds0 + a_off[0][i]);
-        bfr[0][i] = lds_read16(lds0 + b_off[0][i]);
-    }
-
-    int u = 0;  // kt % DMA_BUFS
-    for (int kt = 0; kt < nk; kt++) {
-        const int un = u + 1 == DMA_BUFS ? 0 : u + 1;
-        const uint32_t cur = lds0 + u * (2 * TILE_BYTES);
-        const uint32_t nxt = lds0 + un * (2 * TILE_BYTES);
+    // stage `st` <- k step `st` of buffer `buf` (a compile-time constant in the main loop)
+    auto read_step = [&](int buf, int st) {
 #pragma unroll
         for (int i = 0; i < 2; i++) {
-            af[1][i] = lds_read16(cur + a_off[1][i]);
-            bfr[1][i] = lds_read16(cur + b_off[1][i]);
+            const uint32_t pa = buf < 2 ? a_lo[st][i] : a_hi[st][i], pb = buf < 2 ? b_lo[st][i] : b_hi[st][i];
+            if (buf & 1) {
+                af[st][i] = lds_read16_imm<2 * TILE_BYTES>(pa);
+                bfr[st][i] = lds_read16_imm<2 * TILE_BYTES>(pb);
+            } else {
+                af[st][i] = lds_read16_imm<0>(pa);
+                bfr[st][i] = lds_read16_imm<0>(pb);
+            }
         }
+    };
+    // tiles 1..3 (four loads each) may still be in flight; tile 0 has landed for everyone
+    asm volatile("s_waitcnt vmcnt(12)\n\ts_barrier" ::: "memory");
+    read_step(0, 0);
+
+    // one K tile out of buffer `buf`
+    auto tile = [&](int buf) {
+        read_step(buf, 1);
         // the four reads above may be in flight; the four before them (stage 0) have arrived
         asm volatile("s_waitcnt lgkmcnt(4)" : "+v"(af[0][0]), "+v"(af[0][1]), "+v"(bfr[0][0]), "+v"(bfr[0][1]));
 #pragma unroll
@@ -445,25 +456,36 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_nk_dma_kernel(const uint16_
 #pragma unroll
             for (int j = 0; j < 2; j++)
                 acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[0][i], bfr[0][j], acc[i][j], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);  // these MFMAs go out before the wait: it hides behind them
         // every wavefront has read its last operands of this tile, and the next tile has landed for
         // everyone (the two after it may be in flight): this tile's buffer takes tile kt + 4
         asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)\n\ts_barrier"
                      : "+v"(af[1][0]), "+v"(af[1][1]), "+v"(bfr[1][0]), "+v"(bfr[1][1])
                      :
                      : "memory");
-        request(u);
-#pragma unroll
-        for (int i = 0; i < 2; i++) {
-            af[0][i] = lds_read16(nxt + a_off[0][i]);
-            bfr[0][i] = lds_read16(nxt + b_off[0][i]);
-        }
+        request(buf);
+        read_step((buf + 1) % DMA_BUFS, 0);
 #pragma unroll
         for (int i = 0; i < 2; i++)
 #pragma unroll
             for (int j = 0; j < 2; j++)
                 acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[1][i], bfr[1][j], acc[i][j], 0, 0, 0);
         __builtin_amdgcn_sched_barrier(0);
-        u = un;
+    };
+    // whole rounds of four tiles: every buffer index is a constant, the body is one basic block
+    int kt = 0;
+    for (; kt + DMA_BUFS <= nk; kt += DMA_BUFS) {
+#pragma unroll
+        for (int u = 0; u < DMA_BUFS; u++) tile(u);
+    }
+    // the last zero to three tiles (buffers 0, 1, 2 in turn)
+    for (int u = 0; kt < nk; kt++, u++) {
+        if (u == 0)
+            tile(0);
+        else if (u == 1)
+            tile(1);
+        else
+            tile(2);
     }
 
     // drain the loads still in flight (they target LDS) before the buffers are reused for the exchange
