@@ -24,4 +24,9 @@ int gemm_split_nk(hm_ctx *ctx, const uint16_t *d_a_split, int pieces, const uint
 int gemm_split_split_nk(hm_ctx *ctx, const uint16_t *d_a_split, const uint16_t *d_b_split, float *d_c, int M, int K,
                         int N, int max_parts = 1, int *parts = nullptr, int ldc = 0);
 
+// The same products with every tile loaded once (gemm_pieces_mfma.hip): a_pieces x b_pieces = 2 x 1 or 3 x 1
+// (d_b_split is then the plain [N][K] bf16 matrix) or 3 x 3. K % 32 == 0. Slices and ldc as above.
+int gemm_pieces_nk(hm_ctx *ctx, const uint16_t *d_a_split, int a_pieces, const uint16_t *d_b_split, int b_pieces,
+                   float *d_c, int M, int K, int N, int max_parts = 1, int *parts = nullptr, int ldc = 0);
+
 }  // namespace homura

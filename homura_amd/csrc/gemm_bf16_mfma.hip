@@ -488,8 +488,13 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_nk_dma_kernel(const uint16_
             tile(2);
     }
 
-    // drain the loads still in flight (they target LDS) before the buffers are reused for the exchange
-    asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
+    // drain what is in flight before the buffers are reused for the exchange: the loads into LDS, and
+    // the operand reads of the tile after the last (stage 0; the wait names its registers so that they
+    // stay untouched until the data has arrived)
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier"
+                 : "+v"(af[0][0]), "+v"(af[0][1]), "+v"(bfr[0][0]), "+v"(bfr[0][1])
+                 :
+                 : "memory");
     float *xch = reinterpret_cast<float *>(dma_lds) + (size_t)(wave & 3) * 64 * 64 + lane;
     if (kgrp == 1) {
 #pragma unroll
@@ -590,17 +595,14 @@ int homura::gemm_split_nk(hm_ctx *ctx, const uint16_t *d_a_split, int pieces, co
     int want = (int)std::max<long long>(1, ctx->num_cus / tiles);
     want = std::min(std::min(want, max_parts), std::max(1, nk_total / GEMM_DEPTH));
     if (!parts) want = 1;
+    if (pieces >= 2)  // every tile once, all piece products per stage
+        return gemm_pieces_nk(ctx, d_a_split, pieces, d_b_nk, 1, d_c, M, K, N, max_parts, parts);
     return gemm_launch(ctx, "gemm_split_nk", d_a_split, d_b_nk, d_c, M, K, N, true, pieces, want, parts);
 }
 
 int homura::gemm_split_split_nk(hm_ctx *ctx, const uint16_t *d_a_split, const uint16_t *d_b_split, float *d_c, int M,
                                 int K, int N, int max_parts, int *parts, int ldc) {
-    const long long tiles = (long long)((M + TM - 1) / TM) * ((N + TN - 1) / TN);
-    const int nk_total = 6 * K / TK;
-    int want = (int)std::max<long long>(1, ctx->num_cus / tiles);
-    want = std::min(std::min(want, max_parts), std::max(1, nk_total / GEMM_DEPTH));
-    if (!parts) want = 1;
-    return gemm_launch(ctx, "gemm_split_split_nk", d_a_split, d_b_split, d_c, M, K, N, true, 3, want, parts, 3, ldc);
+    return gemm_pieces_nk(ctx, d_a_split, 3, d_b_split, 3, d_c, M, K, N, max_parts, parts, ldc);
 }
 
 extern "C" int hm_gemm_bf16(hm_ctx *ctx, const uint16_t *d_a_mk, const uint16_t *d_b_kn, float *d_c,

@@ -265,12 +265,12 @@ def test_gemm_f32_quantised_weights(ctx, oracle, kind, M, K, N):
     dx, dw, dout = ctx.to_device(x), ctx.to_device(raw), ctx.empty(M * N)
     ctx.gemm_f32_quant_nk(dx, dw, dtype, dout, M, K, N)
     got = dout.download(np.float32, (M, N))
-    # error in units of a typical output, sqrt(K) rms(x) rms(w): f32 accumulation leaves about 1e-6;
-    # a dropped first-order piece product would leave 1e-3, a second-order one 1e-5
+    # error in units of a typical output, sqrt(K) rms(x) rms(w): f32 accumulation of six products per 32 k
+    # leaves 1e-6 .. 7e-6; a dropped first-order piece product would leave 1e-3, a second-order one 3e-5
     unit = np.sqrt(K) * np.sqrt(np.mean(x64 ** 2)) * np.sqrt(np.mean(w64 ** 2))
     e_gpu, e_orc = np.abs(got - truth).max() / unit, np.abs(want - truth).max() / unit
     say(f"  error / typical output: gpu {e_gpu:.2e}, oracle {e_orc:.2e}; rel_err vs oracle {rel_err(got, want):.2e}")
-    assert e_gpu < 4e-6
+    assert e_gpu < 1.2e-5
     assert rel_err(got, want) < 2e-3
     for b in (dx, dw, dout):
         b.free()

@@ -159,7 +159,7 @@ def test_quantised_prefill_logits_and_following_decode(ctx, which, past, n):
         # of the logit scale; a wrong operand shows as 0.1..1 in every row, a skipped quantisation as
         # 1e-3 in every row. So: rows before the first event agree like the formats without a
         # quantiser, typical rows stay small, and no row is far off.
-        assert min(errs) < 1e-5 and np.median(errs) < 5e-3 and max(errs) < 5e-2
+        assert min(errs) < 1e-5 and np.median(errs) < 1.5e-2 and max(errs) < 5e-2
     want_t, margins = om.generate_greedy(ids[n:], 24)
     got_t = gm.generate_greedy(ids[n:], 24)
     say(f"  min margin {margins.min():.3e}")
