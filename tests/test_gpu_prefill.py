@@ -162,8 +162,15 @@ def test_quantised_prefill_logits_and_following_decode(ctx, which, past, n):
         assert min(errs) < 1e-5 and np.median(errs) < 1.5e-2 and max(errs) < 5e-2
     want_t, margins = om.generate_greedy(ids[n:], 24)
     got_t = gm.generate_greedy(ids[n:], 24)
-    say(f"  min margin {margins.min():.3e}")
-    assert np.array_equal(got_t, want_t)
+    # The greedy tokens that follow are the oracle's for as long as its lead of the best logit over the
+    # second exceeds what two logits may move against each other (twice the worst logit difference seen
+    # above; without a rounding event that is 1e-5 of the scale and all 24 tokens are compared).
+    thr = 2 * max(errs) * float(np.abs(want).max())
+    close = np.nonzero(margins < thr)[0]
+    n_cmp = int(close[0]) if close.size else len(want_t)
+    say(f"  min margin {margins.min():.3e}, threshold {thr:.3e}: {n_cmp} of {len(want_t)} tokens compared")
+    assert np.array_equal(got_t[:n_cmp], want_t[:n_cmp])
+    assert n_cmp == len(want_t) or any(t in (5, 6) for t in mix)   # only a quantiser event may cut it short
     gm.close()
 
 
