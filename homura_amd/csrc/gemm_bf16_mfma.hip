@@ -19,10 +19,8 @@
 // B is fetched from HBM once and served to the others from that XCD's L2.
 //
 // M and N need not be multiples of the tile: rows past the end re-read the last row and their
-// results are not stored. Split-operand mode (prefill of f32 activations): A is [M][P Kb], P = 2 or
-// 3 bf16 pieces of every activation side by side (piece p in columns [p Kb, (p+1) Kb)); the k loop
-// runs over P Kb and B's k index wraps at Kb, so C = (sum of the pieces) x B. Three pieces carry
-// all 24 significant bits of an f32.
+// results are not stored. Operands carried as several bf16 pieces (the prompt pass of f32
+// activations) go through gemm_pieces_mfma.hip.
 //
 // Split-K: grid.y workgroups share an output tile, each multiplies a contiguous range of K tiles and
 // writes its own partial C (partial s at C + s M N); the consumer adds the partials in index order,
@@ -67,13 +65,10 @@ struct TileRegs {
 
 // M, N: logical sizes; K: length of the k loop; lda: row stride of A; Kb: k extent of B (k wraps at Kb)
 // kt_per_split: K tiles per grid.y slice (a multiple of the register ring depth)
-// ldb, ldc: row strides of B ([N][K] layout) and C. Piece pairs (the [N][K] kernel with aligned K
-// tiles only): the k loop is `npairs` stretches of Kb; stretch p multiplies piece (apack >> 2p) & 3 of
-// A (columns [piece Kb, (piece + 1) Kb) of its rows) by piece (bpack >> 2p) & 3 of B.
+// ldb, ldc: row strides of B ([N][K] layout) and C
 struct GemmDims {
     int M, N, K, lda, Kb, kt_per_split;
-    int ldb, ldc, npairs;
-    uint32_t apack, bpack;
+    int ldb, ldc;
 };
 
 // k index of B for loop index kc: the loop covers at most three copies of B's k range
@@ -379,30 +374,19 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_nk_dma_kernel(const uint16_
     }
     // where this wavefront's first instruction lands inside an operand tile (scalar: it goes to M0)
     const int wave_dst = __builtin_amdgcn_readfirstlane(wave * 2048);
-    // The next tile to request: stretch `pair`, k offset `koff` inside it; abase / bbase are the column
-    // offsets of the stretch's pieces. All scalar and updated with a few instructions per tile: the
-    // loop is short enough for its bookkeeping to show in the run time.
-    const int tiles_per_stretch = g.Kb / TK;
-    int pair = kt_first / tiles_per_stretch, koff = (kt_first % tiles_per_stretch) * TK;
-    auto piece_base = [&](uint32_t pack) { return (int)((pack >> (2 * min(pair, g.npairs - 1))) & 3u) * g.Kb; };
-    int abase = piece_base(g.apack), bbase = piece_base(g.bpack);
-    // a tile past the end re-reads one of the last stretch (nobody multiplies it), so every iteration
-    // issues the same four loads and the wait counts below are exact
+    // k offset of the next tile to request (scalar; the loop is short enough for its bookkeeping to
+    // show in the run time). A tile past the end re-reads the last one (nobody multiplies it), so every
+    // iteration issues the same four loads and the wait counts below are exact.
+    int koff = kt_first * TK;
     auto request = [&](int buf) {
         char *base = dma_lds + buf * (2 * TILE_BYTES) + wave_dst;
-        const int ka = abase + koff, kb = bbase + koff;
+        const int k = min(koff, K - TK);
 #pragma unroll
         for (int j = 0; j < 2; j++) {
-            dma16(a_src[j] + ka, base + j * 1024);
-            dma16(b_src[j] + kb, base + TILE_BYTES + j * 1024);
+            dma16(a_src[j] + k, base + j * 1024);
+            dma16(b_src[j] + k, base + TILE_BYTES + j * 1024);
         }
         koff += TK;
-        if (koff == g.Kb) {  // rare
-            koff = 0;
-            pair++;
-            abase = piece_base(g.apack);
-            bbase = piece_base(g.bpack);
-        }
     };
 #pragma unroll
     for (int d = 0; d < DMA_BUFS; d++) request(d);
@@ -524,12 +508,8 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_nk_dma_kernel(const uint16_
             }
 }
 
-// b_pieces == 1: C = (sum of A's `pieces` pieces) x B. b_pieces == 3 (B [N][3 K], A [M][3 K]): the six
-// products of an A piece and a B piece whose indices add up to at most 2, i.e. the product of two
-// f32 matrices up to terms below 2^-24 of it.
 int gemm_launch(hm_ctx *ctx, const char *who, const uint16_t *a, const uint16_t *b, float *c, int M, int K,
-                int N, bool b_nk, int pieces, int ksplit = 1, int *ksplit_used = nullptr, int b_pieces = 1,
-                int ldc = 0) {
+                int N, bool b_nk, int ksplit = 1, int *ksplit_used = nullptr, int ldc = 0) {
     HM_CHECK_CTX(ctx);
     HM_REQUIRE(ctx, a && b && c, "%s: NULL pointer", who);
     HM_REQUIRE(ctx, M > 0 && N > 0 && K > 0 && K % 32 == 0, "%s: need M, N > 0 and K %% 32 == 0 (M=%d K=%d N=%d)", who,
@@ -543,22 +523,10 @@ int gemm_launch(hm_ctx *ctx, const char *who, const uint16_t *a, const uint16_t 
     g.M = M;
     g.N = N;
     g.Kb = K;
-    g.lda = pieces * K;
-    g.ldb = b_pieces * K;
+    g.K = K;
+    g.lda = K;
+    g.ldb = K;
     g.ldc = ldc > 0 ? ldc : N;
-    if (b_pieces == 1) {
-        g.npairs = pieces;
-        g.apack = 0;  // last piece first: the small terms are added while the accumulator is small
-        for (int i = 0; i < pieces; i++) g.apack |= (uint32_t)(pieces - 1 - i) << (2 * i);
-        g.bpack = 0;
-    } else {
-        HM_REQUIRE(ctx, b_nk && pieces == 3 && b_pieces == 3 && K % TK == 0,
-                   "%s: piece pairs need the [N][K] layout, three pieces a side and K %% 64 == 0", who);
-        g.npairs = 6;
-        g.apack = 0x046;  // (a, b) = (2,0) (1,1) (0,2) (1,0) (0,1) (0,0): the small terms first
-        g.bpack = 0x124;
-    }
-    g.K = g.npairs * K;
     HM_REQUIRE(ctx, g.ldc >= N, "%s: ldc %d below N %d", who, g.ldc, N);
     const int nk_total = (g.K + TK - 1) / TK;
     if (ksplit < 1) ksplit = 1;
@@ -588,16 +556,16 @@ int gemm_launch(hm_ctx *ctx, const char *who, const uint16_t *a, const uint16_t 
 int homura::gemm_split_nk(hm_ctx *ctx, const uint16_t *d_a_split, int pieces, const uint16_t *d_b_nk, float *d_c,
                           int M, int K, int N, int max_parts, int *parts) {
     HM_REQUIRE(ctx, pieces >= 1 && pieces <= 3, "gemm_split_nk: %d pieces (1..3)", pieces);
+    if (pieces >= 2)  // every tile once, all piece products per stage
+        return gemm_pieces_nk(ctx, d_a_split, pieces, d_b_nk, 1, d_c, M, K, N, max_parts, parts);
     // K slices while they still add whole waves of workgroups to a grid smaller than the chip (the
     // slices cost a write and a read of C each), at least 4 K tiles per slice
     const long long tiles = (long long)((M + TM - 1) / TM) * ((N + TN - 1) / TN);
-    const int nk_total = (pieces * K + TK - 1) / TK;
+    const int nk_total = (K + TK - 1) / TK;
     int want = (int)std::max<long long>(1, ctx->num_cus / tiles);
     want = std::min(std::min(want, max_parts), std::max(1, nk_total / GEMM_DEPTH));
     if (!parts) want = 1;
-    if (pieces >= 2)  // every tile once, all piece products per stage
-        return gemm_pieces_nk(ctx, d_a_split, pieces, d_b_nk, 1, d_c, M, K, N, max_parts, parts);
-    return gemm_launch(ctx, "gemm_split_nk", d_a_split, d_b_nk, d_c, M, K, N, true, pieces, want, parts);
+    return gemm_launch(ctx, "gemm_split_nk", d_a_split, d_b_nk, d_c, M, K, N, true, want, parts);
 }
 
 int homura::gemm_split_split_nk(hm_ctx *ctx, const uint16_t *d_a_split, const uint16_t *d_b_split, float *d_c, int M,
@@ -607,10 +575,10 @@ int homura::gemm_split_split_nk(hm_ctx *ctx, const uint16_t *d_a_split, const ui
 
 extern "C" int hm_gemm_bf16(hm_ctx *ctx, const uint16_t *d_a_mk, const uint16_t *d_b_kn, float *d_c,
                             int M, int K, int N) {
-    return gemm_launch(ctx, "hm_gemm_bf16", d_a_mk, d_b_kn, d_c, M, K, N, false, 1);
+    return gemm_launch(ctx, "hm_gemm_bf16", d_a_mk, d_b_kn, d_c, M, K, N, false);
 }
 
 extern "C" int hm_gemm_bf16_nk(hm_ctx *ctx, const uint16_t *d_a_mk, const uint16_t *d_b_nk, float *d_c,
                                int M, int K, int N) {
-    return gemm_launch(ctx, "hm_gemm_bf16_nk", d_a_mk, d_b_nk, d_c, M, K, N, true, 1);
+    return gemm_launch(ctx, "hm_gemm_bf16_nk", d_a_mk, d_b_nk, d_c, M, K, N, true);
 }
