@@ -9,6 +9,7 @@
 // (batch, kv head) in split order, so the result does not depend on timing.
 // Algorithmic HBM traffic: 2 * kv_len * HD * 2 bytes per (batch, kv head).
 #include "attention.h"
+#include "bf16_pieces.h"
 
 namespace {
 
@@ -277,6 +278,189 @@ __global__ __launch_bounds__(ATT_THREADS) void gqa_decode_attn_kernel(
     }
 }
 
+// Long caches (more rows per workgroup than fit in registers at once): the workgroup walks its
+// rows in steps of 64. The loads of step i + 1 are in flight while step i is multiplied, the
+// softmax reference point is the running maximum (sums and the output accumulators are rescaled
+// when it moves), and scores and rescale factors alternate between two LDS slots so a step needs
+// two barriers. Q.K^T runs on the matrix cores: v_mfma_f32_16x16x32_bf16 takes 16 cache rows
+// straight from memory as its A operand (lane r + 16 c holds dims 32 s + 8 c .. + 7 of row r, one
+// 16-byte load) and the G query heads, scaled and split into two bf16 pieces, as columns of B;
+// what the pieces leave out is 2^-17 of a query element. P.V stays on the vector ALUs (V would have
+// to be transposed for the matrix cores, which costs more than the multiply for so few heads).
+// Partials leave in the same (o, max, sum) form as the kernel above.
+constexpr int IT_ROWS = 64;  // rows per step: 16 per wavefront for Q.K^T
+
+template <int HD, int G>
+__global__ __launch_bounds__(ATT_THREADS) void gqa_decode_attn_stream_kernel(
+    const float *__restrict__ q, const uint16_t *__restrict__ kcache,
+    const uint16_t *__restrict__ vcache, float *__restrict__ out, float *__restrict__ part_o,
+    float *__restrict__ part_ml, int kvh, int max_len, int kv_len, int chunk, float scale,
+    int lds_front) {
+    constexpr int LPR = HD / 8, RPI = WAVE / LPR;
+    constexpr int NRG_V = IT_ROWS / (ATT_WAVES * RPI);      // V row groups per wavefront and step
+    constexpr int KS = HD / 32;                             // k steps of the score MFMA
+    constexpr int SLOTS = (G + ATT_WAVES - 1) / ATT_WAVES;  // heads whose statistics a wavefront keeps
+    static_assert(IT_ROWS == WAVE && IT_ROWS == 16 * ATT_WAVES, "one score per lane; 16 rows per wavefront");
+    static_assert(G <= 16, "heads are columns of a 16-wide MFMA tile");
+    extern __shared__ __attribute__((aligned(16))) float sm[];
+    float *sc = sm;                      // [2][G][IT_ROWS] scores, then probabilities
+    float *fac = sm + 2 * G * IT_ROWS;   // [2][G] rescale factor of the step
+    float *red = sm + lds_front;         // [ATT_WAVES * RPI][G][HD]
+    __shared__ float qs[G][HD];
+    __shared__ float s_m[G], s_l[G];
+
+    const int tid = threadIdx.x, lane = tid & (WAVE - 1), wave = tid / WAVE;
+    const int sub = lane / LPR, dl = lane % LPR;  // V: row within a group, 8-dim slice
+    const int l16 = lane & 15, kg = lane >> 4;     // K operand: row of the wavefront's 16, 8-dim slice of a k step
+    const int split = blockIdx.x, nsplit = gridDim.x, kvhd = blockIdx.y, b = blockIdx.z;
+    const int H = kvh * G;
+    const int n0 = split * chunk;
+    const size_t head_base = ((size_t)b * kvh + kvhd) * max_len * HD;
+    const uint16_t *kbase = kcache + head_base + (size_t)n0 * HD + kg * 8;
+    const uint16_t *vbase = vcache + head_base + (size_t)n0 * HD + dl * 8;
+    const int cnt = min(kv_len, n0 + chunk) - n0;  // >= 1: the grid covers kv_len exactly
+    const int iters = (cnt + IT_ROWS - 1) / IT_ROWS;
+
+    auto request = [&](u32x4(&kr)[KS], u32x4(&vr)[NRG_V], int it) {
+        const int krow = it * IT_ROWS + 16 * wave + l16;
+        const bool kok = krow < cnt;
+#pragma unroll
+        for (int s = 0; s < KS; s++)
+            kr[s] = kok ? ld128_stream(kbase + (size_t)krow * HD + 32 * s) : u32x4{0u, 0u, 0u, 0u};
+#pragma unroll
+        for (int i = 0; i < NRG_V; i++) {
+            const int row = it * IT_ROWS + (i * ATT_WAVES + wave) * RPI + sub;
+            vr[i] = row < cnt ? ld128_stream(vbase + (size_t)row * HD) : u32x4{0u, 0u, 0u, 0u};
+        }
+    };
+    u32x4 ka[KS], va[NRG_V], kb[KS], vb[NRG_V];
+    request(ka, va, 0);
+
+    for (int i = tid; i < G * HD; i += ATT_THREADS)
+        qs[i / HD][i % HD] = q[((size_t)b * H + kvhd * G) * HD + i];
+    __syncthreads();
+    // B operand: column l16 is query head l16 (columns past G are zero), scaled, as two pieces
+    bf16x8 qop[KS][2];
+#pragma unroll
+    for (int s = 0; s < KS; s++) {
+        float f[8];
+#pragma unroll
+        for (int e = 0; e < 8; e++) f[e] = l16 < G ? qs[l16 < G ? l16 : 0][32 * s + 8 * kg + e] * scale : 0.f;
+        split8<2>(f, qop[s]);
+    }
+
+    float acc[G][8];
+#pragma unroll
+    for (int gi = 0; gi < G; gi++)
+#pragma unroll
+        for (int e = 0; e < 8; e++) acc[gi][e] = 0.f;
+    float m_run[SLOTS], l_run[SLOTS];
+#pragma unroll
+    for (int s = 0; s < SLOTS; s++) {
+        m_run[s] = -INFINITY;
+        l_run[s] = 0.f;
+    }
+
+    auto step = [&](u32x4(&kr)[KS], u32x4(&vr)[NRG_V], u32x4(&nkr)[KS], u32x4(&nvr)[NRG_V], int it) {
+        if (it + 1 < iters) request(nkr, nvr, it + 1);
+        float *scp = sc + (it & 1) * G * IT_ROWS;
+        float *facp = fac + (it & 1) * G;
+        // scores of the wavefront's 16 rows against every head; the small piece first. Lane
+        // l16 + 16 c receives head l16, rows 4 c .. 4 c + 3; rows past the live range count as -inf.
+        {
+            f32x4 c = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int s = 0; s < KS; s++) {
+                const bf16x8 kop = __builtin_bit_cast(bf16x8, kr[s]);
+                c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kop, qop[s][1], c, 0, 0, 0);
+                c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kop, qop[s][0], c, 0, 0, 0);
+            }
+            const int r0 = 16 * wave + 4 * kg;
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+                if (it * IT_ROWS + r0 + i >= cnt) c[i] = -INFINITY;
+            if (l16 < G) *reinterpret_cast<f32x4 *>(scp + l16 * IT_ROWS + r0) = c;
+        }
+        __syncthreads();
+        // one wavefront per head: move the running maximum, turn scores into exp(s - max)
+#pragma unroll
+        for (int s = 0; s < SLOTS; s++) {
+            const int gi = wave + s * ATT_WAVES;
+            if (gi < G) {
+                const float x = scp[gi * IT_ROWS + lane];
+                const float m_new = fmaxf(m_run[s], wave_max(x));  // finite: row 0 of a step is live
+                const float e = expf(x - m_new);
+                scp[gi * IT_ROWS + lane] = e;
+                const float f = expf(m_run[s] - m_new);
+                l_run[s] = fmaf(l_run[s], f, wave_sum(e));
+                m_run[s] = m_new;
+                if (lane == 0) facp[gi] = f;
+            }
+        }
+        __syncthreads();
+        // o = o * factor + P.V
+#pragma unroll
+        for (int gi = 0; gi < G; gi++) {
+            const float f = facp[gi];
+            if (f != 1.f) {
+#pragma unroll
+                for (int e = 0; e < 8; e++) acc[gi][e] *= f;
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < NRG_V; i++) {
+            const int r = (i * ATT_WAVES + wave) * RPI + sub;
+            float vf[8];
+            unpack8(vr[i], vf);
+#pragma unroll
+            for (int gi = 0; gi < G; gi++) {
+                const float p = scp[gi * IT_ROWS + r];
+#pragma unroll
+                for (int e = 0; e < 8; e++) acc[gi][e] = fmaf(p, vf[e], acc[gi][e]);
+            }
+        }
+    };
+    for (int it = 0; it < iters; it += 2) {
+        step(ka, va, kb, vb, it);
+        if (it + 1 < iters) step(kb, vb, ka, va, it + 1);
+    }
+
+#pragma unroll
+    for (int s = 0; s < SLOTS; s++) {
+        const int gi = wave + s * ATT_WAVES;
+        if (gi < G && lane == 0) {
+            s_m[gi] = m_run[s];
+            s_l[gi] = l_run[s];
+        }
+    }
+#pragma unroll
+    for (int gi = 0; gi < G; gi++) {
+        float *dst = red + ((size_t)(wave * RPI + sub) * G + gi) * HD + dl * 8;
+        *reinterpret_cast<f32x4 *>(dst) = f32x4{acc[gi][0], acc[gi][1], acc[gi][2], acc[gi][3]};
+        *reinterpret_cast<f32x4 *>(dst + 4) = f32x4{acc[gi][4], acc[gi][5], acc[gi][6], acc[gi][7]};
+    }
+    __syncthreads();
+
+    const size_t pair = (size_t)b * kvh + kvhd;
+    float *po = part_o + (pair * nsplit + split) * G * HD;
+    float *pml = part_ml + (pair * nsplit + split) * G * 2;
+    for (int i = tid; i < G * HD; i += ATT_THREADS) {
+        float v = 0.f;
+#pragma unroll
+        for (int w = 0; w < ATT_WAVES * RPI; w++) v += red[(size_t)w * G * HD + i];
+        if (nsplit == 1) {
+            const int gi = i / HD, d = i % HD;
+            out[((size_t)b * H + kvhd * G + gi) * HD + d] = v / s_l[gi];
+        } else {
+            po[i] = v;
+        }
+    }
+    if (nsplit > 1 && tid < G) {
+        pml[tid * 2] = s_m[tid];
+        pml[tid * 2 + 1] = s_l[tid];
+    }
+}
+
 // Second half of the split attention: one workgroup of HD threads per (batch, query head)
 // folds that head's partial (o, max, sum) triples in ascending split order. A separate launch
 // instead of a "last workgroup to arrive" fold: the kernel boundary orders the partial writes,
@@ -371,8 +555,53 @@ int launch_attn(hm_ctx *ctx, const AttnArgs &a, int nsplit, int chunk) {
     return HM_OK;
 }
 
+// Long caches through the stepping kernel; its partials go through the same fold.
+template <int HD, int G>
+int launch_attn_stream(hm_ctx *ctx, const AttnArgs &a, int nsplit, int chunk) {
+    constexpr int RPI = WAVE / (HD / 8);
+    const size_t front = ((size_t)2 * G * IT_ROWS + 2 * G + 3) / 4 * 4;  // 16-byte rows behind it
+    const size_t lds = (front + (size_t)ATT_WAVES * RPI * G * HD) * sizeof(float);
+    const size_t pairs = (size_t)a.B * a.kvh;
+    float *part_o = (float *)ctx->workspace;
+    float *part_ml = part_o + pairs * nsplit * G * HD;
+    static bool lds_limit_raised = false;  // per instantiation
+    if (lds > 64 * 1024 && !lds_limit_raised) {
+        HM_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(&gqa_decode_attn_stream_kernel<HD, G>),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024));
+        lds_limit_raised = true;
+    }
+    HM_REQUIRE(ctx, lds <= 96 * 1024, "gqa_decode_attn: LDS need %zu too large", lds);
+    HM_REQUIRE(ctx, chunk % IT_ROWS == 0, "gqa_decode_attn: chunk %d must be a multiple of %d", chunk, IT_ROWS);
+    hipLaunchKernelGGL((gqa_decode_attn_stream_kernel<HD, G>), dim3(nsplit, a.kvh, a.B),
+                       dim3(ATT_THREADS), lds, ctx->stream, a.q, a.kcache, a.vcache, a.out, part_o,
+                       part_ml, a.kvh, a.max_len, a.kv_len, chunk, a.scale, (int)front);
+    HM_LAUNCH_CHECK(ctx);
+    if (nsplit > 1) {
+        const size_t fold_lds = (size_t)nsplit * 2 * sizeof(float);
+        HM_REQUIRE(ctx, fold_lds <= 64 * 1024, "gqa_decode_attn: too many splits (%d)", nsplit);
+        hipLaunchKernelGGL((gqa_decode_fold_kernel<HD, G>), dim3(a.kvh * G, a.B), dim3(HD), fold_lds,
+                           ctx->stream, a.out, part_o, part_ml, a.kvh, a.kv_len, chunk,
+                           (const DecodeState *)nullptr);
+        HM_LAUNCH_CHECK(ctx);
+    }
+    return HM_OK;
+}
+
 template <int HD>
-int dispatch_g(hm_ctx *ctx, const AttnArgs &a, int g, int nsplit, int chunk) {
+int dispatch_g(hm_ctx *ctx, const AttnArgs &a, int g, int nsplit, int chunk, bool stepping) {
+    if (stepping) {
+        switch (g) {
+        case 1: return launch_attn_stream<HD, 1>(ctx, a, nsplit, chunk);
+        case 2: return launch_attn_stream<HD, 2>(ctx, a, nsplit, chunk);
+        case 3: return launch_attn_stream<HD, 3>(ctx, a, nsplit, chunk);
+        case 4: return launch_attn_stream<HD, 4>(ctx, a, nsplit, chunk);
+        case 5: return launch_attn_stream<HD, 5>(ctx, a, nsplit, chunk);
+        case 6: return launch_attn_stream<HD, 6>(ctx, a, nsplit, chunk);
+        case 7: return launch_attn_stream<HD, 7>(ctx, a, nsplit, chunk);
+        case 8: return launch_attn_stream<HD, 8>(ctx, a, nsplit, chunk);
+        default: break;
+        }
+    }
     switch (g) {
     case 1: return launch_attn<HD, 1>(ctx, a, nsplit, chunk);
     case 2: return launch_attn<HD, 2>(ctx, a, nsplit, chunk);
@@ -402,10 +631,28 @@ int gqa_decode_attn_launch(hm_ctx *ctx, const AttnArgs &a) {
     const int rows_step = 32;
     const int span = a.state ? a.max_len : a.kv_len;  // rows the grid has to be able to cover
     int chunk = a.fixed_chunk;
+    bool stepping = false;
     if (chunk <= 0) {
         int want = (int)(((size_t)ctx->num_cus + pairs - 1) / pairs);
         chunk = (span + want - 1) / want;
         chunk = (chunk + rows_step - 1) / rows_step * rows_step;
+        // More rows per workgroup than its registers hold: the stepping kernel, two workgroups per
+        // CU (plain calls only; the decode plan's fused prologue lives in the other kernel).
+        if (chunk > 128 && !a.state && !a.qkv_raw) {
+            stepping = true;
+            const int it_rows = IT_ROWS;
+            want = (int)(((size_t)2 * ctx->num_cus + pairs - 1) / pairs);
+            chunk = (span + want - 1) / want;
+            chunk = (chunk + it_rows - 1) / it_rows * it_rows;
+        }
+    }
+    if (stepping) {
+        HM_REQUIRE(ctx, a.q != nullptr, "gqa_decode_attn: NULL query");
+        const int nsplit = (a.kv_len + chunk - 1) / chunk;
+        const size_t ws_need = pairs * nsplit * g * (a.hd + 2) * sizeof(float);
+        HM_REQUIRE(ctx, ws_need <= ctx->workspace_bytes, "gqa_decode_attn: workspace too small (%zu bytes needed)", ws_need);
+        if (a.hd == 128) return dispatch_g<128>(ctx, a, g, nsplit, chunk, true);
+        return dispatch_g<64>(ctx, a, g, nsplit, chunk, true);
     }
     if (chunk < rows_step) chunk = rows_step;
     if (chunk > 128) chunk = 128;
@@ -419,8 +666,8 @@ int gqa_decode_attn_launch(hm_ctx *ctx, const AttnArgs &a) {
     int nsplit = (span + chunk - 1) / chunk;
     const size_t ws_need = pairs * nsplit * g * (a.hd + 2) * sizeof(float);
     HM_REQUIRE(ctx, ws_need <= ctx->workspace_bytes, "gqa_decode_attn: workspace too small (%zu bytes needed)", ws_need);
-    if (a.hd == 128) return dispatch_g<128>(ctx, a, g, nsplit, chunk);
-    return dispatch_g<64>(ctx, a, g, nsplit, chunk);
+    if (a.hd == 128) return dispatch_g<128>(ctx, a, g, nsplit, chunk, false);
+    return dispatch_g<64>(ctx, a, g, nsplit, chunk, false);
 }
 
 extern "C" {

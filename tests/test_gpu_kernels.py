@@ -340,7 +340,13 @@ def test_kv_append_rounds_to_nearest_even(ctx, oracle):
     (1, 16, 8, 128, 1152, 1),      # first token
     (2, 14, 2, 64, 300, 33),       # Qwen2.5-0.5B heads (g = 7), ragged length
     (1, 4, 4, 128, 64, 64),        # MHA (g = 1), single split
-    (3, 32, 4, 64, 512, 511)])     # g = 8
+    (3, 32, 4, 64, 512, 511),      # g = 8
+    (8, 12, 2, 128, 4096, 3001),   # long cache, ragged: workgroups walk their rows in steps
+    (8, 8, 4, 64, 1500, 1399),     # same with 64-wide heads (g = 2)
+    (16, 32, 4, 128, 700, 650),    # same with g = 8
+    (2, 2, 1, 128, 16384, 16384),  # few (sequence, kv head) pairs, many steps per workgroup
+    (40, 4, 4, 64, 600, 577),      # same with g = 1 (MHA)
+    (24, 20, 4, 128, 1100, 1031)]) # same with g = 5
 def test_gqa_decode_attn(ctx, oracle, B, H, kvh, hd, max_len, kv_len):
     say(f"gqa_decode_attn B={B} H={H} kvh={kvh} hd={hd} max_len={max_len} kv_len={kv_len}")
     q = synth.normal_f32(synth.SEED_CFG5 + 2, B * H * hd).reshape(B, H, hd)
