@@ -107,7 +107,12 @@ def test_q8_0_reference_kat(ctx, golden):
                                         ("q4_0", 1, 1536, 151936),  # BASELINE config 4
                                         ("q8_0", 1, 2048, 2048), ("q8_0", 1, 5632, 2048),
                                         ("q8_0", 2, 4096, 77), ("q8_0", 1, 32, 5), ("q8_0", 1, 96, 1),
-                                        ("q4_0", 3, 2048, 260), ("q4_0", 1, 32, 7), ("q4_0", 1, 8960, 64)])
+                                        ("q4_0", 3, 2048, 260), ("q4_0", 1, 32, 7), ("q4_0", 1, 8960, 64),
+                                        # large Q4_0 products: short and long rows, N not a multiple
+                                        # of the rows staged per step, two rows of x
+                                        ("q4_0", 1, 256, 233100), ("q4_0", 1, 1792, 33333),
+                                        ("q4_0", 2, 2048, 29201), ("q4_0", 1, 4096, 14601),
+                                        ("q4_0", 1, 7168, 8400)])
 def test_quant_gemv(ctx, oracle, kind, M, K, N):
     say(f"gemv_{kind} M={M} K={K} N={N}")
     nb = N * (K // 32)
@@ -119,6 +124,8 @@ def test_quant_gemv(ctx, oracle, kind, M, K, N):
     (ctx.gemv_q8_0 if kind == "q8_0" else ctx.gemv_q4_0)(dx, dw, dout, M, K, N)
     got = dout.download(np.float32, (M, N))
     assert rel_err(got, want) < TOL
+    # both sides add exact products in f32, in different orders
+    assert np.abs(got - want).max() < 1e-4 * np.sqrt(np.mean(want.astype(np.float64) ** 2))
     for b in (dx, dw, dout):
         b.free()
 
