@@ -99,7 +99,12 @@ SIGNATURES = {
     "hm_model_set_weight_nk": (_I, [_P, _I, _P, _SZ]),
     "hm_model_config": (_I, [_P, _P, _P, _P]),
     "hm_tokenizer_open": (_P, [C.c_char_p, C.c_char_p, C.c_char_p, _SZ]),
+    "hm_tokenizer_open_json": (_P, [C.c_char_p, C.c_char_p, _SZ]),
     "hm_tokenizer_close": (None, [_P]),
+    "hm_tokenizer_wants_nfc": (_I, [_P]),
+    "hm_tokenizer_token_to_id": (C.c_longlong, [_P, C.c_char_p]),
+    "hm_tokenizer_encode_ex": (C.c_longlong, [_P, C.c_char_p, _SZ, _I, _P, _SZ]),
+    "hm_tokenizer_decode_ex": (C.c_longlong, [_P, _P, _SZ, _I, _P, _SZ]),
     "hm_tokenizer_vocab_size": (_I, [_P]),
     "hm_tokenizer_encode": (C.c_longlong, [_P, C.c_char_p, _SZ, _P, _SZ]),
     "hm_tokenizer_decode": (C.c_longlong, [_P, _P, _SZ, _P, _SZ]),

@@ -11,7 +11,7 @@
 #include <vector>
 
 #include "hf.h"
-#include "json_map.h"
+#include "json.h"
 
 namespace homura {
 

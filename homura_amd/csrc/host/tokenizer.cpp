@@ -13,7 +13,7 @@
 #include <sstream>
 
 #include "../../../include/homura_amd.h"
-#include "json_map.h"
+#include "json.h"
 #include "unicode_tables.h"
 
 namespace homura {
@@ -128,7 +128,7 @@ CodePoints decode_code_points(const char *text, size_t len) {
 }
 
 // End (exclusive, in code points) of the piece that starts at i.
-size_t match_piece(const std::vector<uint32_t> &c, size_t i) {
+size_t match_piece(const std::vector<uint32_t> &c, size_t i, int max_digits) {
     const size_t n = c.size();
     const uint32_t c0 = c[i];
     auto lower = [](uint32_t x) { return x >= 'A' && x <= 'Z' ? x + 32 : x; };
@@ -151,10 +151,10 @@ size_t match_piece(const std::vector<uint32_t> &c, size_t i) {
             return j;
         }
     }
-    // 3. one to three numbers
+    // 3. one to max_digits numbers
     if (is_number(c0)) {
         size_t j = i;
-        while (j < n && j < i + 3 && is_number(c[j])) j++;
+        while (j < n && j < i + (size_t)max_digits && is_number(c[j])) j++;
         return j;
     }
     // 4. punctuation and symbols, with an optional leading space and trailing newlines
@@ -200,15 +200,28 @@ bool read_file(const std::string &path, std::string *out, std::string *err) {
 
 }  // namespace
 
-std::vector<std::pair<size_t, size_t>> BpeTokenizer::pre_tokenize(const char *text, size_t len) {
+std::vector<std::pair<size_t, size_t>> BpeTokenizer::pre_tokenize(const char *text, size_t len, int max_digits) {
     std::vector<std::pair<size_t, size_t>> out;
     const CodePoints c = decode_code_points(text, len);
     for (size_t i = 0; i < c.cp.size();) {
-        const size_t j = match_piece(c.cp, i);
+        const size_t j = match_piece(c.cp, i, max_digits);
         out.emplace_back(c.at[i], c.at[j]);
         i = j;
     }
     return out;
+}
+
+// GPT-2's bytes_to_unicode (src/tokenizer.rs:19-41): printable Latin-1 bytes stand for themselves,
+// the other 68 get U+0100 onwards in byte order
+void BpeTokenizer::init_byte_alphabet() {
+    uint32_t next = 256;
+    for (int b = 0; b < 256; b++) {
+        const bool printable = (b >= '!' && b <= '~') || (b >= 0xA1 && b <= 0xAC) || (b >= 0xAE && b <= 0xFF);
+        const uint32_t cp = printable ? (uint32_t)b : next++;
+        byte_utf8_[b].clear();
+        append_utf8(&byte_utf8_[b], cp);
+        cp_to_byte_[cp] = (uint8_t)b;
+    }
 }
 
 std::unique_ptr<BpeTokenizer> BpeTokenizer::from_files(const std::string &vocab_path, const std::string &merges_path,
@@ -241,16 +254,175 @@ std::unique_ptr<BpeTokenizer> BpeTokenizer::from_files(const std::string &vocab_
         if (end > pos && merges_text[pos] != '#') t->ranks_[merges_text.substr(pos, end - pos)] = rank++;
         pos = eol + 1;
     }
-    // GPT-2's bytes_to_unicode (src/tokenizer.rs:19-41): printable Latin-1 bytes stand for themselves,
-    // the other 68 get U+0100 onwards in byte order
-    uint32_t next = 256;
-    for (int b = 0; b < 256; b++) {
-        const bool printable = (b >= '!' && b <= '~') || (b >= 0xA1 && b <= 0xAC) || (b >= 0xAE && b <= 0xFF);
-        const uint32_t cp = printable ? (uint32_t)b : next++;
-        append_utf8(&t->byte_utf8_[b], cp);
-        t->cp_to_byte_[cp] = (uint8_t)b;
+    t->init_byte_alphabet();
+    return t;
+}
+
+namespace {
+
+// The Split patterns of the byte-level BPE family this class implements; they differ in the run of numbers.
+const char *const PATTERN_QWEN2 =
+    "(?i:'s|'t|'re|'ve|'m|'ll|'d)|[^\\r\\n\\p{L}\\p{N}]?\\p{L}+|\\p{N}| ?[^\\s\\p{L}\\p{N}]+[\\r\\n]*|\\s*[\\r\\n]+|\\s+(?!\\S)|\\s+";
+const char *const PATTERN_LLAMA3 =
+    "(?i:'s|'t|'re|'ve|'m|'ll|'d)|[^\\r\\n\\p{L}\\p{N}]?\\p{L}+|\\p{N}{1,3}| ?[^\\s\\p{L}\\p{N}]+[\\r\\n]*|\\s*[\\r\\n]+|\\s+(?!\\S)|\\s+";
+
+bool json_flag(const Json &o, const char *key, bool dflt = false) {
+    const Json *v = o.get(key);
+    return v && v->kind == Json::Bool ? v->b : dflt;
+}
+
+const std::string *json_str(const Json &o, const char *key) {
+    const Json *v = o.get(key);
+    return v && v->kind == Json::Str ? &v->str : nullptr;
+}
+
+}  // namespace
+
+std::unique_ptr<BpeTokenizer> BpeTokenizer::from_tokenizer_json(const std::string &path, std::string *err) {
+    std::string text;
+    if (!read_file(path, &text, err)) return nullptr;
+    Json j;
+    if (!parse_json(text.data(), text.size(), &j, err)) {
+        *err = path + ": " + *err;
+        return nullptr;
+    }
+    auto refuse = [&](const std::string &what) {
+        *err = path + ": " + what;
+        return nullptr;
+    };
+    const Json *model = j.get("model");
+    if (!model || model->kind != Json::Obj) return refuse("no \"model\" object");
+    const std::string *mtype = json_str(*model, "type");
+    const Json *vocab = model->get("vocab"), *merges = model->get("merges");
+    if ((mtype && *mtype != "BPE") || !vocab || vocab->kind != Json::Obj || !merges || merges->kind != Json::Arr)
+        return refuse("model is not a BPE with \"vocab\" and \"merges\"");
+    for (const char *key : {"unk_token", "continuing_subword_prefix", "end_of_word_suffix", "dropout"}) {
+        const Json *v = model->get(key);
+        if (v && v->kind != Json::Null && !(v->kind == Json::Str && v->str.empty()))
+            return refuse(std::string("BPE option \"") + key + "\" is not supported");
+    }
+    if (json_flag(*model, "byte_fallback") || json_flag(*model, "fuse_unk"))
+        return refuse("BPE byte_fallback / fuse_unk are not supported");
+
+    std::unique_ptr<BpeTokenizer> t(new BpeTokenizer());
+    t->hf_decode_ = true;
+    t->ignore_merges_ = json_flag(*model, "ignore_merges");
+    for (const auto &kv : vocab->obj) {
+        if (kv.second.kind != Json::Num || kv.second.num < 0 || kv.second.num > 4294967295.0)
+            return refuse("vocabulary id of \"" + kv.first + "\" is not a u32");
+        t->encoder_[kv.first] = (uint32_t)kv.second.num;
+    }
+    for (const auto &kv : t->encoder_) t->decoder_[kv.second] = kv.first;
+    uint32_t rank = 0;
+    for (const Json &m : merges->arr) {  // "left right" strings, or [left, right] pairs
+        if (m.kind == Json::Str) {
+            t->ranks_[m.str] = rank++;
+        } else if (m.kind == Json::Arr && m.arr.size() == 2 && m.arr[0].kind == Json::Str && m.arr[1].kind == Json::Str) {
+            t->ranks_[m.arr[0].str + " " + m.arr[1].str] = rank++;
+        } else {
+            return refuse("merge " + std::to_string(rank) + " is neither a string nor a pair of strings");
+        }
+    }
+    t->init_byte_alphabet();
+
+    // normaliser: none, or NFC (left to the caller)
+    if (const Json *nz = j.get("normalizer"); nz && nz->kind == Json::Obj) {
+        const std::string *ty = json_str(*nz, "type");
+        if (!ty || *ty != "NFC") return refuse("normalizer " + (ty ? *ty : std::string("?")) + " is not supported (none or NFC)");
+        t->wants_nfc_ = true;
+    }
+    // pre-tokeniser: Sequence[Split(pattern, Isolated), ByteLevel(use_regex = false)]
+    {
+        const Json *pt = j.get("pre_tokenizer");
+        std::vector<const Json *> parts;
+        if (pt && pt->kind == Json::Obj) {
+            const std::string *ty = json_str(*pt, "type");
+            const Json *seq = pt->get("pretokenizers");
+            if (ty && *ty == "Sequence" && seq && seq->kind == Json::Arr)
+                for (const Json &e : seq->arr) parts.push_back(&e);
+            else
+                parts.push_back(pt);
+        }
+        bool have_split = false, have_bytes = false;
+        for (const Json *e : parts) {
+            const std::string *ty = e->kind == Json::Obj ? json_str(*e, "type") : nullptr;
+            if (ty && *ty == "Split") {
+                const Json *pat = e->get("pattern");
+                const std::string *re = pat && pat->kind == Json::Obj ? json_str(*pat, "Regex") : nullptr;
+                const std::string *beh = json_str(*e, "behavior");
+                if (!re || !beh || *beh != "Isolated" || json_flag(*e, "invert"))
+                    return refuse("Split pre-tokeniser must be an isolated, non-inverted regex");
+                if (*re == PATTERN_QWEN2) t->max_digits_ = 1;
+                else if (*re == PATTERN_LLAMA3) t->max_digits_ = 3;
+                else return refuse("Split pattern is not one of the two this tokenizer implements: " + *re);
+                have_split = true;
+            } else if (ty && *ty == "ByteLevel") {
+                if (json_flag(*e, "add_prefix_space", true)) return refuse("ByteLevel add_prefix_space is not supported");
+                if (json_flag(*e, "use_regex", true)) return refuse("ByteLevel with its own (GPT-2) regex is not supported");
+                have_bytes = true;
+            } else {
+                return refuse("pre-tokeniser " + (ty ? *ty : std::string("?")) + " is not supported");
+            }
+        }
+        if (!have_split || !have_bytes) return refuse("pre-tokeniser must be Split + ByteLevel");
+    }
+    if (const Json *dec = j.get("decoder"); !dec || dec->kind != Json::Obj || !json_str(*dec, "type") || *json_str(*dec, "type") != "ByteLevel")
+        return refuse("decoder must be ByteLevel");
+
+    // added tokens
+    if (const Json *added = j.get("added_tokens"); added && added->kind == Json::Arr) {
+        for (const Json &a : added->arr) {
+            const Json *id = a.kind == Json::Obj ? a.get("id") : nullptr;
+            const std::string *content = a.kind == Json::Obj ? json_str(a, "content") : nullptr;
+            if (!id || id->kind != Json::Num || !content || content->empty()) return refuse("malformed added token");
+            if (json_flag(a, "lstrip") || json_flag(a, "rstrip") || json_flag(a, "single_word"))
+                return refuse("added token \"" + *content + "\": lstrip / rstrip / single_word are not supported");
+            t->added_.push_back(Added{*content, (uint32_t)id->num, json_flag(a, "special")});
+        }
+        std::stable_sort(t->added_.begin(), t->added_.end(),
+                         [](const Added &x, const Added &y) { return x.content.size() > y.content.size(); });
+        for (size_t i = 0; i < t->added_.size(); i++) {
+            t->added_by_id_[t->added_[i].id] = i;
+            t->decoder_[t->added_[i].id] = t->added_[i].content;
+        }
+    }
+    // post-processor: ByteLevel changes no ids; TemplateProcessing wraps a single sequence in special tokens
+    if (const Json *pp = j.get("post_processor"); pp && pp->kind == Json::Obj) {
+        std::vector<const Json *> parts;
+        const std::string *ty = json_str(*pp, "type");
+        const Json *seq = pp->get("processors");
+        if (ty && *ty == "Sequence" && seq && seq->kind == Json::Arr)
+            for (const Json &e : seq->arr) parts.push_back(&e);
+        else
+            parts.push_back(pp);
+        for (const Json *e : parts) {
+            const std::string *pty = e->kind == Json::Obj ? json_str(*e, "type") : nullptr;
+            if (pty && *pty == "ByteLevel") continue;
+            if (!pty || *pty != "TemplateProcessing") return refuse("post-processor " + (pty ? *pty : std::string("?")) + " is not supported");
+            const Json *single = e->get("single");
+            if (!single || single->kind != Json::Arr) return refuse("TemplateProcessing without \"single\"");
+            bool seen_a = false;
+            for (const Json &item : single->arr) {
+                if (item.kind != Json::Obj) return refuse("malformed TemplateProcessing item");
+                if (const Json *sp = item.get("SpecialToken"); sp && sp->kind == Json::Obj) {
+                    const std::string *name = json_str(*sp, "id");
+                    const int64_t id = name ? t->token_to_id(*name) : -1;
+                    if (id < 0) return refuse("TemplateProcessing names an unknown special token");
+                    (seen_a ? t->suffix_ids_ : t->prefix_ids_).push_back((uint32_t)id);
+                } else if (item.get("Sequence")) {
+                    seen_a = true;
+                }
+            }
+        }
     }
     return t;
+}
+
+int64_t BpeTokenizer::token_to_id(const std::string &token) const {
+    for (const Added &a : added_)
+        if (a.content == token) return a.id;
+    auto it = encoder_.find(token);
+    return it == encoder_.end() ? -1 : (int64_t)it->second;
 }
 
 // reference bpe (src/tokenizer.rs:85-116): while some adjacent pair has a rank, merge the first
@@ -285,36 +457,84 @@ std::vector<std::string> BpeTokenizer::bpe(const std::string &mapped) const {
     return word;
 }
 
-std::vector<uint32_t> BpeTokenizer::encode(const char *text, size_t len) const {
-    std::vector<uint32_t> ids;
+void BpeTokenizer::encode_plain(const char *text, size_t len, std::vector<uint32_t> *ids) const {
     std::string mapped;
-    for (const auto &piece : pre_tokenize(text, len)) {
+    for (const auto &piece : pre_tokenize(text, len, max_digits_)) {
         mapped.clear();
         for (size_t i = piece.first; i < piece.second; i++) mapped += byte_utf8_[(unsigned char)text[i]];
+        if (ignore_merges_) {
+            auto whole = encoder_.find(mapped);
+            if (whole != encoder_.end()) {
+                ids->push_back(whole->second);
+                continue;
+            }
+        }
         for (const std::string &sym : bpe(mapped)) {
             auto it = encoder_.find(sym);
-            if (it != encoder_.end()) ids.push_back(it->second);
+            if (it != encoder_.end()) ids->push_back(it->second);
         }
     }
+}
+
+std::vector<uint32_t> BpeTokenizer::encode(const char *text, size_t len, bool add_special_tokens) const {
+    std::vector<uint32_t> ids;
+    if (add_special_tokens) ids = prefix_ids_;
+    if (added_.empty()) {
+        encode_plain(text, len, &ids);
+    } else {
+        // added tokens stand for themselves: the leftmost match wins, the longest at that position
+        // (added_ is sorted by length); the stretches between them are ordinary text
+        size_t plain_from = 0;
+        for (size_t i = 0; i < len;) {
+            const Added *hit = nullptr;
+            for (const Added &a : added_) {
+                if (a.content.size() <= len - i && text[i] == a.content[0] && memcmp(text + i, a.content.data(), a.content.size()) == 0) {
+                    hit = &a;
+                    break;
+                }
+            }
+            if (!hit) {
+                i++;
+                continue;
+            }
+            if (i > plain_from) encode_plain(text + plain_from, i - plain_from, &ids);
+            ids.push_back(hit->id);
+            i += hit->content.size();
+            plain_from = i;
+        }
+        if (len > plain_from) encode_plain(text + plain_from, len - plain_from, &ids);
+    }
+    if (add_special_tokens) ids.insert(ids.end(), suffix_ids_.begin(), suffix_ids_.end());
     return ids;
 }
 
-std::string BpeTokenizer::decode(const uint32_t *ids, size_t n) const {
-    std::string bytes;
+std::string BpeTokenizer::decode(const uint32_t *ids, size_t n, bool skip_special) const {
+    std::string bytes, tok_bytes;
     for (size_t k = 0; k < n; k++) {
         auto it = decoder_.find(ids[k]);
         if (it == decoder_.end()) continue;
+        if (skip_special) {
+            auto a = added_by_id_.find(ids[k]);
+            if (a != added_by_id_.end() && added_[a->second].special) continue;
+        }
         const std::string &tok = it->second;
+        tok_bytes.clear();
+        bool all_mapped = true;
         for (size_t i = 0; i < tok.size();) {
             uint32_t cp;
             size_t bad;
             const size_t m = utf8_at(reinterpret_cast<const unsigned char *>(tok.data()) + i, tok.size() - i, &cp, &bad);
             if (m) {
                 auto b = cp_to_byte_.find(cp);
-                if (b != cp_to_byte_.end()) bytes.push_back((char)b->second);
+                if (b != cp_to_byte_.end()) tok_bytes.push_back((char)b->second);
+                else all_mapped = false;
+            } else {
+                all_mapped = false;
             }
             i += m ? m : 1;
         }
+        // tokenizer.json files: a token with a character outside the byte alphabet is taken as written
+        bytes += (hf_decode_ && !all_mapped) ? tok : tok_bytes;
     }
     // String::from_utf8_lossy: every longest ill-formed prefix becomes one U+FFFD
     std::string out;
@@ -353,7 +573,42 @@ hm_tokenizer *hm_tokenizer_open(const char *vocab_json_path, const char *merges_
     return new hm_tokenizer{std::move(t)};
 }
 
+hm_tokenizer *hm_tokenizer_open_json(const char *tokenizer_json_path, char *err, size_t errlen) {
+    std::string e;
+    auto t = homura::BpeTokenizer::from_tokenizer_json(tokenizer_json_path ? tokenizer_json_path : "", &e);
+    if (!t) {
+        homura::copy_err(e, err, errlen);
+        return nullptr;
+    }
+    return new hm_tokenizer{std::move(t)};
+}
+
 void hm_tokenizer_close(hm_tokenizer *t) { delete t; }
+
+int hm_tokenizer_wants_nfc(const hm_tokenizer *t) { return t ? (t->t->wants_nfc() ? 1 : 0) : HM_ERR_INVALID; }
+
+long long hm_tokenizer_token_to_id(const hm_tokenizer *t, const char *token) {
+    if (!t || !token) return -1;
+    return (long long)t->t->token_to_id(token);
+}
+
+long long hm_tokenizer_encode_ex(const hm_tokenizer *t, const char *text, size_t text_len, int add_special_tokens,
+                                 uint32_t *ids_out, size_t capacity) {
+    if (!t || (!text && text_len) || (!ids_out && capacity)) return HM_ERR_INVALID;
+    const std::vector<uint32_t> ids = t->t->encode(text, text_len, add_special_tokens != 0);
+    const size_t n = std::min(ids.size(), capacity);
+    if (n) memcpy(ids_out, ids.data(), n * sizeof(uint32_t));
+    return (long long)ids.size();
+}
+
+long long hm_tokenizer_decode_ex(const hm_tokenizer *t, const uint32_t *ids, size_t n_ids, int skip_special_tokens,
+                                 char *text_out, size_t capacity) {
+    if (!t || (!ids && n_ids) || (!text_out && capacity)) return HM_ERR_INVALID;
+    const std::string s = t->t->decode(ids, n_ids, skip_special_tokens != 0);
+    const size_t n = std::min(s.size(), capacity);
+    if (n) memcpy(text_out, s.data(), n);
+    return (long long)s.size();
+}
 
 int hm_tokenizer_vocab_size(const hm_tokenizer *t) { return t ? (int)t->t->vocab_size() : HM_ERR_INVALID; }
 

@@ -477,16 +477,32 @@ const char *hm_version(void);
 
 /* ── tokenizer (reference src/tokenizer.rs) ───────────────────────────────────
  * The reference's own byte-level BPE over vocab.json + merges.txt (GPT-2 files): Tokenizer::from_files
- * (src/tokenizer.rs:44-82), encode (:119-144), decode (:147-159). Host code, no GPU. (Its wrapper
- * around the `tokenizers` crate for tokenizer.json files, src/hf/tokenizer.rs, has no counterpart.)
- * hm_tokenizer_open returns NULL and writes a message into err. encode / decode return the full
+ * (src/tokenizer.rs:44-82), encode (:119-144), decode (:147-159). Host code, no GPU.
+ * hm_tokenizer_open_json stands in for HfTokenizer::from_file (src/hf/tokenizer.rs:10-14), which hands a
+ * tokenizer.json to the `tokenizers` crate (0.21.4 in the reference's Cargo.lock): it reads the files of
+ * the byte-level BPE family (Qwen2/3, Llama-3: BPE model, Split on their pattern + ByteLevel, added
+ * tokens, ByteLevel or TemplateProcessing post-processor) and refuses everything else with a message.
+ * A file that asks for NFC normalisation is accepted and hm_tokenizer_wants_nfc says so: the caller
+ * normalises the text, this library does not.
+ * hm_tokenizer_open* return NULL and write a message into err. encode / decode return the full
  * count of ids / bytes (negative: an HM_ERR_* code) and write at most `capacity` of them; call again
  * with a larger buffer when the count exceeds it. The decoded text is UTF-8 without a terminator.
+ * encode_ex / decode_ex: HfTokenizer::encode (add_special_tokens = 0) and encode_with_special (1)
+ * (src/hf/tokenizer.rs:17-23, :41-47: added tokens written in the text are recognised either way, the flag
+ * puts the post-processor's template around the ids); decode (skip_special_tokens = 1) and decode_raw (0)
+ * (:25-38). hm_tokenizer_token_to_id: id of a vocabulary entry or added token, -1 when there is none.
  * hm_tokenizer_pieces: the end offsets (bytes) of the pieces the pre-tokeniser pattern
  * (src/tokenizer.rs:71-74) cuts the text into. */
 typedef struct hm_tokenizer hm_tokenizer;
 hm_tokenizer *hm_tokenizer_open(const char *vocab_json_path, const char *merges_txt_path, char *err, size_t errlen);
+hm_tokenizer *hm_tokenizer_open_json(const char *tokenizer_json_path, char *err, size_t errlen);
 void hm_tokenizer_close(hm_tokenizer *t);
+int hm_tokenizer_wants_nfc(const hm_tokenizer *t);
+long long hm_tokenizer_token_to_id(const hm_tokenizer *t, const char *token_utf8);
+long long hm_tokenizer_encode_ex(const hm_tokenizer *t, const char *text, size_t text_len, int add_special_tokens,
+                                 uint32_t *ids_out, size_t capacity);
+long long hm_tokenizer_decode_ex(const hm_tokenizer *t, const uint32_t *ids, size_t n_ids, int skip_special_tokens,
+                                 char *text_out, size_t capacity);
 int hm_tokenizer_vocab_size(const hm_tokenizer *t);
 long long hm_tokenizer_encode(const hm_tokenizer *t, const char *text, size_t text_len, uint32_t *ids_out,
                               size_t capacity);
