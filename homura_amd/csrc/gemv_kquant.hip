@@ -336,6 +336,221 @@ __global__ __launch_bounds__(KTHREADS) void gemv_kquant_kernel(const int8_t *__r
     }
 }
 
+// ── f32 activations against the dequantised weights ─────────────────────────────────────────────────
+//
+// What the reference computes when a K-quant tensor feeds an f32 kernel (its loader dequantises the
+// embedding / output matrices, src/gguf.rs:589-708, and the LM head multiplies f32 by f32): out[n] =
+// sum_k x[k] * w[n][k] with w the dequantised weight. Every w is d * sc * q (Q6_K) or q * (d * sc) - dmin * mn
+// (Q4_K) with small integers q, so a 16-weight unit is (d * sc) * (sum_j u_j x_j - off * sum_j x_j)
+// [- (dmin * mn) * sum_j x_j] in f32: one byte -> float conversion and one FMA per weight, the sums of x per
+// unit computed once. The rows are staged like in the integer kernel; optional RMSNorm of the row on the way
+// in (the LM head's final norm), optional best (value, index) per workgroup on the way out.
+struct ActF32 {
+    float x[16];
+    float sx;
+};
+
+__device__ __forceinline__ float dot16_f32(const uint32_t *w, const float *x) {
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        s = fmaf((float)(w[i] & 0xFFu), x[4 * i], s);
+        s = fmaf((float)((w[i] >> 8) & 0xFFu), x[4 * i + 1], s);
+        s = fmaf((float)((w[i] >> 16) & 0xFFu), x[4 * i + 2], s);
+        s = fmaf((float)(w[i] >> 24), x[4 * i + 3], s);
+    }
+    return s;
+}
+
+__device__ __forceinline__ float q4k_unit_f32(const uint8_t *blk, int i, const ActF32 &a) {
+    const int sb = i >> 1, h = i & 1, pair = sb >> 1, odd = sb & 1;
+    const uint32_t hdr = *reinterpret_cast<const uint32_t *>(blk);  // d | dmin << 16
+    const float d = f16_bits_to_f32((uint16_t)(hdr & 0xFFFFu)), dmin = f16_bits_to_f32((uint16_t)(hdr >> 16));
+    const uint8_t *raw = blk + 4;
+    int sc, mn;
+    if (sb < 4) {
+        sc = raw[sb] & 63;
+        mn = raw[sb + 4] & 63;
+    } else {
+        const int hi = raw[sb + 4];
+        sc = (hi & 15) | ((raw[sb - 4] >> 6) << 4);
+        mn = (hi >> 4) | ((raw[sb] >> 6) << 4);
+    }
+    const u32x4 w = *reinterpret_cast<const u32x4 *>(blk + 16 + pair * 32 + h * 16);
+    const int sh = odd * 4;
+    const uint32_t nib[4] = {(w.x >> sh) & 0x0F0F0F0Fu, (w.y >> sh) & 0x0F0F0F0Fu, (w.z >> sh) & 0x0F0F0F0Fu,
+                             (w.w >> sh) & 0x0F0F0F0Fu};
+    return (d * (float)sc) * dot16_f32(nib, a.x) - (dmin * (float)mn) * a.sx;
+}
+
+__device__ __forceinline__ float q6k_unit_f32(const uint8_t *blk, int i, const ActF32 &a) {
+    const int chunk = i >> 3, group = (i & 7) >> 1, parity = i & 1;
+    const uint8_t *ql = blk + chunk * 64 + (group & 1) * 32 + parity * 16;
+    const uint8_t *qh = blk + 128 + chunk * 32 + parity * 16;
+    const int lo_sh = group >= 2 ? 4 : 0, hi_sh = group * 2;
+    uint32_t v[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const uint32_t l = lds32_a2(ql + 4 * j), hgh = lds32_a2(qh + 4 * j);
+        v[j] = ((l >> lo_sh) & 0x0F0F0F0Fu) | (((hgh >> hi_sh) & 0x03030303u) << 4);
+    }
+    const int sc = (int)(int8_t)blk[192 + i];
+    const float d = f16_bits_to_f32((uint16_t)lds16(blk + 208));
+    return (d * (float)sc) * (dot16_f32(v, a.x) - 32.f * a.sx);
+}
+
+template <int QT, int CPL, int RT>
+__device__ __forceinline__ void krows_trip_f32(const uint8_t *base, size_t rowbytes, int lr, int lane, int nu,
+                                               const ActF32 (&act)[CPL], float *out, int row0, float &best_v, int &best_i) {
+    constexpr int BB = KTraits<QT>::BYTES;
+    const int boff = (lane >> 4) * BB, ui = lane & 15;
+    float a[RT];
+#pragma unroll
+    for (int j = 0; j < RT; j++) a[j] = 0.f;
+#pragma unroll
+    for (int t = 0; t < CPL; t++) {
+        const bool live = lane + t * WAVE < nu;
+#pragma unroll
+        for (int j = 0; j < RT; j++) {
+            const uint8_t *blk = base + (size_t)(lr + j * KWAVES) * rowbytes + (live ? boff + t * 4 * BB : 0);
+            const float v = QT == 0 ? q4k_unit_f32(blk, ui, act[t]) : q6k_unit_f32(blk, ui, act[t]);
+            a[j] += live ? v : 0.f;
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    }
+#pragma unroll
+    for (int j = 0; j < RT; j++) {
+        a[j] = wave_sum(a[j]);
+        const int r = lr + j * KWAVES;
+        if (lane == 0) out[r] = a[j];
+        // first maximum wins: rows reach a wavefront in ascending order (reference argmax, src/generate.rs:457-468)
+        if (a[j] > best_v) {
+            best_v = a[j];
+            best_i = row0 + r;
+        }
+    }
+}
+
+template <int QT, int CPL>
+__global__ __launch_bounds__(KTHREADS) void gemv_kquant_f32_kernel(const float *__restrict__ x, const float *__restrict__ norm_w,
+                                                                   float eps, const uint8_t *__restrict__ w,
+                                                                   float *__restrict__ out, int K, int N, int rows_per_step,
+                                                                   int x_lds_off, float *__restrict__ cand_v,
+                                                                   int *__restrict__ cand_i) {
+    constexpr int BB = KTraits<QT>::BYTES;
+    constexpr int U = KSTAGE_U;
+    extern __shared__ __attribute__((aligned(16))) uint8_t ws[];
+    float *xs = reinterpret_cast<float *>(ws + x_lds_off);  // [K] the (normed) row, then 8 floats of scratch
+    float *red = xs + K;
+    const int tid = threadIdx.x, lane = tid & (WAVE - 1), wave = tid / WAVE;
+    const int nb = K / 256, nu = K / 16;
+    const size_t rowbytes = (size_t)nb * BB;
+    const int nsteps = (N + rows_per_step - 1) / rows_per_step;
+
+    // the row first (loads return in issue order), the first step's weights right behind it
+    const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
+    f32x4 xr[KXU], nr[KXU];
+#pragma unroll
+    for (int u = 0; u < KXU; u++) {
+        const int k = (tid + u * KTHREADS) * 4;
+        xr[u] = k < K ? *reinterpret_cast<const f32x4 *>(x + k) : zero4;
+        nr[u] = norm_w && k < K ? *reinterpret_cast<const f32x4 *>(norm_w + k) : zero4;
+    }
+    u32x4 tmp[U];
+    int step = blockIdx.x;
+    StepRange cur = step_range(step, rows_per_step, N, rowbytes);
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+        const int i = tid + u * KTHREADS;
+        tmp[u] = i < cur.nchunks ? ld128_stream(w + cur.abeg + (size_t)i * 16) : u32x4{0u, 0u, 0u, 0u};
+    }
+    if (norm_w) {  // emit_rms_norm (src/graph_builder/emit_linalg.rs:7-26): (x * inv) * w
+        float ss = 0.f;
+#pragma unroll
+        for (int u = 0; u < KXU; u++) ss += (xr[u][0] * xr[u][0] + xr[u][1] * xr[u][1]) + (xr[u][2] * xr[u][2] + xr[u][3] * xr[u][3]);
+        ss = wave_sum(ss);
+        if (lane == 0) red[wave] = ss;
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");  // LDS only: the weight loads stay in flight
+        float tot = 0.f;
+#pragma unroll
+        for (int wv = 0; wv < KWAVES; wv++) tot += red[wv];
+        const float inv = 1.0f / sqrtf(tot / (float)K + eps);
+#pragma unroll
+        for (int u = 0; u < KXU; u++)
+#pragma unroll
+            for (int e = 0; e < 4; e++) xr[u][e] = (xr[u][e] * inv) * nr[u][e];
+    }
+#pragma unroll
+    for (int u = 0; u < KXU; u++) {
+        const int k = (tid + u * KTHREADS) * 4;
+        if (k < K) *reinterpret_cast<f32x4 *>(xs + k) = xr[u];
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    ActF32 act[CPL];
+#pragma unroll
+    for (int t = 0; t < CPL; t++) {
+        const int u = min(lane + t * WAVE, nu - 1);
+        float sx = 0.f;
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            const f32x4 v = *reinterpret_cast<const f32x4 *>(xs + (size_t)u * 16 + 4 * q);
+            act[t].x[4 * q] = v.x; act[t].x[4 * q + 1] = v.y; act[t].x[4 * q + 2] = v.z; act[t].x[4 * q + 3] = v.w;
+            sx += (v.x + v.y) + (v.z + v.w);
+        }
+        act[t].sx = sx;
+    }
+
+    float best_v = -INFINITY;
+    int best_i = 0x7FFFFFFF;
+    for (; step < nsteps; step += gridDim.x) {
+        __syncthreads();  // previous step's readers are done with the row stage
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const int i = tid + u * KTHREADS;
+            if (i < cur.nchunks) *reinterpret_cast<u32x4 *>(ws + (size_t)i * 16) = tmp[u];
+        }
+        __syncthreads();
+        const StepRange now = cur;
+        if (step + (int)gridDim.x < nsteps) {  // the next step's weights travel while this one is multiplied
+            cur = step_range(step + gridDim.x, rows_per_step, N, rowbytes);
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                const int i = tid + u * KTHREADS;
+                tmp[u] = i < cur.nchunks ? ld128_stream(w + cur.abeg + (size_t)i * 16) : u32x4{0u, 0u, 0u, 0u};
+            }
+        }
+        const uint8_t *base = ws + now.shift;
+        float *o = out + now.r0;
+        int lr = wave;
+        for (; lr + 3 * KWAVES < now.nrows; lr += 4 * KWAVES) krows_trip_f32<QT, CPL, 4>(base, rowbytes, lr, lane, nu, act, o, now.r0, best_v, best_i);
+        if (lr + KWAVES < now.nrows) {
+            krows_trip_f32<QT, CPL, 2>(base, rowbytes, lr, lane, nu, act, o, now.r0, best_v, best_i);
+            lr += 2 * KWAVES;
+        }
+        if (lr < now.nrows) krows_trip_f32<QT, CPL, 1>(base, rowbytes, lr, lane, nu, act, o, now.r0, best_v, best_i);
+    }
+    if (cand_v) {  // the workgroup's best row: largest value, lowest index among equals
+        __syncthreads();
+        int *redi = reinterpret_cast<int *>(red + KWAVES);
+        if (lane == 0) {
+            red[wave] = best_v;
+            redi[wave] = best_i;
+        }
+        __syncthreads();
+        if (tid == 0) {
+            float bv = red[0];
+            int bi = redi[0];
+            for (int wv = 1; wv < KWAVES; wv++)
+                if (red[wv] > bv || (red[wv] == bv && redi[wv] < bi)) {
+                    bv = red[wv];
+                    bi = redi[wv];
+                }
+            cand_v[blockIdx.x] = bv;
+            cand_i[blockIdx.x] = bi;
+        }
+    }
+}
+
 // One thread per weight, the reference's arithmetic step by step (no contraction) so the bits match
 // the CPU: Q4_K w = q * (d * sc) - dmin * mn; Q6_K w = (d * sc) * q (src/gguf.rs:835-917).
 template <int QT>
@@ -430,6 +645,56 @@ int gemv_kquant_launch(hm_ctx *ctx, const char *name, const float *d_x, const ui
 }
 
 template <int QT>
+int gemv_kquant_f32_launch(hm_ctx *ctx, const char *name, const float *d_x, const float *d_norm_w, float eps,
+                           const uint8_t *d_w, float *d_out, int M, int K, int N, float *cand_v, int *cand_i, int cand_cap,
+                           int *grid_out) {
+    HM_CHECK_CTX(ctx);
+    constexpr int BB = KTraits<QT>::BYTES;
+    HM_REQUIRE(ctx, d_x && d_w && d_out, "%s: NULL pointer", name);
+    HM_REQUIRE(ctx, M >= 1 && M <= 8, "%s: M=%d outside 1..8", name, M);
+    HM_REQUIRE(ctx, K > 0 && K % 256 == 0 && N > 0, "%s: K=%d must be a positive multiple of 256, N=%d positive", name, K, N);
+    HM_REQUIRE(ctx, K <= KXU * KTHREADS * 4, "%s: K=%d above %d", name, K, KXU * KTHREADS * 4);
+    HM_REQUIRE(ctx, ((uintptr_t)d_w % 16) == 0 && ((uintptr_t)d_x % 16) == 0 && ((uintptr_t)d_norm_w % 16) == 0,
+               "%s: weight, activation and norm buffers must be 16-byte aligned", name);
+    HM_REQUIRE(ctx, !cand_v || (cand_i && M == 1), "%s: argmax candidates need an index buffer and one row", name);
+    const size_t rowbytes = (size_t)(K / 256) * BB;
+    HM_REQUIRE(ctx, KWAVES * rowbytes + 32 <= (size_t)KSTAGE_BYTES, "%s: K=%d too large for the LDS stage", name, K);
+    int rows = (int)(((size_t)40 * 1024) / rowbytes);
+    rows = rows / KWAVES * KWAVES;
+    if (rows < KWAVES) rows = KWAVES;
+    if (rows > KMAX_ROWS) rows = KMAX_ROWS;
+    while (rows > KWAVES && (size_t)rows * rowbytes + 32 > (size_t)KSTAGE_BYTES) rows -= KWAVES;
+    while (rows > KWAVES && (N + rows - 1) / rows < 2 * ctx->num_cus) rows -= KWAVES;
+    const size_t stage_bytes = ((size_t)rows * rowbytes + 32 + 16 + 15) & ~(size_t)15;
+    const size_t lds = stage_bytes + (size_t)K * 4 + 64;
+    const int nsteps = (N + rows - 1) / rows;
+    int wg_per_cu = (int)(120 * 1024 / lds);
+    if (wg_per_cu < 1) wg_per_cu = 1;
+    if (wg_per_cu > 6) wg_per_cu = 6;
+    int grid = nsteps < ctx->num_cus * wg_per_cu ? nsteps : ctx->num_cus * wg_per_cu;
+    if (cand_v && grid > cand_cap) grid = cand_cap;
+    HM_REQUIRE(ctx, grid >= 1, "%s: no room for argmax candidates", name);
+    if (grid_out) *grid_out = grid;
+    const int cpl = (K / 16 + WAVE - 1) / WAVE;
+    for (int m = 0; m < M; m++) {
+        const float *xm = d_x + (size_t)m * K;
+        float *om = d_out + (size_t)m * N;
+#define HM_KF_CASE(C)                                                                                                   \
+    hipLaunchKernelGGL((gemv_kquant_f32_kernel<QT, C>), dim3(grid), dim3(KTHREADS), lds, ctx->stream, xm, d_norm_w, eps, \
+                       d_w, om, K, N, rows, (int)stage_bytes, cand_v, cand_i)
+        switch (cpl) {
+            case 1: HM_KF_CASE(1); break;
+            case 2: HM_KF_CASE(2); break;
+            case 3: HM_KF_CASE(3); break;
+            default: HM_KF_CASE(4); break;
+        }
+#undef HM_KF_CASE
+        HM_LAUNCH_CHECK(ctx);
+    }
+    return HM_OK;
+}
+
+template <int QT>
 int dequant_kquant_launch(hm_ctx *ctx, const char *name, const uint8_t *d_blocks, float *d_out, size_t nblocks) {
     HM_CHECK_CTX(ctx);
     if (nblocks == 0) return HM_OK;
@@ -463,6 +728,12 @@ int hm_gemv_q4_k(hm_ctx *ctx, const float *d_x, const uint8_t *d_w_blocks, float
 }
 int hm_gemv_q6_k(hm_ctx *ctx, const float *d_x, const uint8_t *d_w_blocks, float *d_out, int M, int K, int N) {
     return gemv_kquant_launch<1>(ctx, "hm_gemv_q6_k", d_x, d_w_blocks, d_out, M, K, N);
+}
+int hm_gemv_q4_k_f32(hm_ctx *ctx, const float *d_x, const uint8_t *d_w_blocks, float *d_out, int M, int K, int N) {
+    return gemv_kquant_f32_launch<0>(ctx, "hm_gemv_q4_k_f32", d_x, nullptr, 0.f, d_w_blocks, d_out, M, K, N, nullptr, nullptr, 0, nullptr);
+}
+int hm_gemv_q6_k_f32(hm_ctx *ctx, const float *d_x, const uint8_t *d_w_blocks, float *d_out, int M, int K, int N) {
+    return gemv_kquant_f32_launch<1>(ctx, "hm_gemv_q6_k_f32", d_x, nullptr, 0.f, d_w_blocks, d_out, M, K, N, nullptr, nullptr, 0, nullptr);
 }
 int hm_dequant_q4_k(hm_ctx *ctx, const uint8_t *d_blocks, float *d_out, size_t nblocks) {
     return dequant_kquant_launch<0>(ctx, "hm_dequant_q4_k", d_blocks, d_out, nblocks);

@@ -160,6 +160,12 @@ class Context:
     def gemv_q6_k(self, x, w, out, M, K, N):
         self._check(self.lib.hm_gemv_q6_k(self.h, x.ptr, w.ptr, out.ptr, M, K, N))
 
+    def gemv_q4_k_f32(self, x, w, out, M, K, N):
+        self._check(self.lib.hm_gemv_q4_k_f32(self.h, x.ptr, w.ptr, out.ptr, M, K, N))
+
+    def gemv_q6_k_f32(self, x, w, out, M, K, N):
+        self._check(self.lib.hm_gemv_q6_k_f32(self.h, x.ptr, w.ptr, out.ptr, M, K, N))
+
     def quantize_q8_k(self, x, q8, act_d, bsums, M, K):
         self._check(self.lib.hm_quantize_q8_k(self.h, x.ptr, q8.ptr, act_d.ptr, bsums.ptr, M, K))
 

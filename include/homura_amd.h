@@ -115,6 +115,15 @@ int hm_dequant_q4_0(hm_ctx *ctx, const uint8_t *d_blocks, float *d_out, size_t n
  * f32 adds over units and blocks come in a different order. */
 int hm_gemv_q4_k(hm_ctx *ctx, const float *d_x, const uint8_t *d_w_blocks, float *d_out, int M, int K, int N);
 int hm_gemv_q6_k(hm_ctx *ctx, const float *d_x, const uint8_t *d_w_blocks, float *d_out, int M, int K, int N);
+/* The f32 product with the dequantised weights: out[m][n] = sum_k x[m][k] * w[n][k], w = dequant_q4_k /
+ * dequant_q6_k of the blocks (src/gguf.rs:835-917). This is what the reference computes where a K-quant
+ * tensor feeds an f32 kernel: its loader dequantises the embedding and output matrices
+ * (GgufFile::load_transformer_weights, src/gguf.rs:589-708) and the LM head multiplies f32 by f32
+ * (emit_lm_head_kernel, src/hf/emitter.rs:828-862). The blocks are read as they are (144 / 210 bytes per
+ * 256 weights instead of 1024) and every weight enters as the exact dequantised value. K % 256 == 0,
+ * K <= 4096, M <= 8. */
+int hm_gemv_q4_k_f32(hm_ctx *ctx, const float *d_x, const uint8_t *d_w_blocks, float *d_out, int M, int K, int N);
+int hm_gemv_q6_k_f32(hm_ctx *ctx, const float *d_x, const uint8_t *d_w_blocks, float *d_out, int M, int K, int N);
 /* The Q8_K activation quantisation on its own (emit_quant.rs:422-466): d_q8 int8 [M][K], d_act_d f32
  * [M][K/256], d_bsums int32 [M][K/16] (sums of 16 consecutive q). Bit-exact with the CPU. */
 int hm_quantize_q8_k(hm_ctx *ctx, const float *d_x, int8_t *d_q8, float *d_act_d, int32_t *d_bsums, int M, int K);

@@ -244,6 +244,27 @@ def test_gemm_bf16_ragged_edges(ctx, oracle, M, K, N, layout):
         buf.free()
 
 
+@pytest.mark.parametrize("kind", ["q4_k", "q6_k"])
+@pytest.mark.parametrize("M,K,N", [(1, 1024, 151936),   # LM head of the Qwen3-0.6B shape
+                                   (1, 1024, 3072), (2, 256, 7), (3, 2048, 515), (1, 4096, 130), (1, 3072, 1024)])
+def test_gemv_kquant_f32_activation(ctx, oracle, kind, M, K, N):
+    """f32 row times the dequantised weights: the checker multiplies the oracle's dequantised matrix
+    (bit-exact with the reference's dequant_q4_k / dequant_q6_k) in float64."""
+    say(f"gemv_{kind}_f32 M={M} K={K} N={N}")
+    raw = (synth.q4_k_blocks if kind == "q4_k" else synth.q6_k_blocks)(15, N * K // 256)
+    x = synth.normal_f32(16, M * K, 1.0).reshape(M, K)
+    w = (oracle.dequant_q4_k if kind == "q4_k" else oracle.dequant_q6_k)(raw).reshape(N, K)
+    want = x.astype(np.float64) @ w.astype(np.float64).T
+    dx, dw, dout = ctx.to_device(x), ctx.to_device(raw), ctx.empty(M * N)
+    (ctx.gemv_q4_k_f32 if kind == "q4_k" else ctx.gemv_q6_k_f32)(dx, dw, dout, M, K, N)
+    got = dout.download(np.float32, (M, N))
+    err = np.abs(got - want).max() / np.sqrt(np.mean(want ** 2))
+    say(f"  max error / rms {err:.2e}")
+    assert err < 2e-6 * max(1.0, np.sqrt(K / 1024))   # f32 sums of exact terms
+    for b in (dx, dw, dout):
+        b.free()
+
+
 @pytest.mark.parametrize("kind", ["q8_0", "q4_0", "q4_k", "q6_k"])
 @pytest.mark.parametrize("M,K,N", [(200, 1024, 1000), (5, 256, 130), (64, 2048, 6000), (512, 512, 256)])
 def test_gemm_f32_quantised_weights(ctx, oracle, kind, M, K, N):
