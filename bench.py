@@ -207,13 +207,25 @@ def main() -> int:
             qcfg = dataclasses.replace(cfg, tie_word_embeddings=False)
             quantised = {"unit": "tok/s", "steps": args.steps,
                          "what": "same shape, cache and step count; raw GGUF blocks dequantised in registers "
-                                 "(K-quants: Q8_K activations, integer dots), f32 LM head"}
-            for name, wdt, mix in (("q8_0", DTYPE_Q8_0, None), ("q4_0", DTYPE_Q4_0, None),
-                                   ("q4_k_m_mix", None, synth_model.q4_k_m_mix(qcfg))):
+                                 "(K-quants: Q8_K activations, integer dots), f32 LM head; "
+                                 "q4_k_m_mix_q6_k_head: the head as Q6_K blocks multiplied in f32"}
+            kmix = synth_model.q4_k_m_mix(qcfg)
+            for name, wdt, mix, head_q6k in (("q8_0", DTYPE_Q8_0, None, False), ("q4_0", DTYPE_Q4_0, None, False),
+                                             ("q4_k_m_mix", None, kmix, False),
+                                             # as Q4_K_M files come: the output matrix in Q6_K, read from its blocks
+                                             ("q4_k_m_mix_q6_k_head", None, kmix, True)):
                 qw = synth_model.synth_weights(qcfg, seed + 7, wdt if mix is None else DTYPE_Q8_0, has_qk_norm=True,
                                                proj_dtypes=mix)
-                qm = synth_model.build_model(ctx, qcfg, qw, 2048, wdt if mix is None else DTYPE_Q8_0, has_qk_norm=True,
-                                             proj_dtypes=mix)
+                if head_q6k:
+                    from homura_amd.runtime import DTYPE_Q6_K, HfModel
+                    qm = HfModel(ctx, qcfg, DTYPE_Q8_0, True, proj_dtypes=mix)
+                    for i, (_n, arr) in enumerate(qw[:-1]):
+                        qm.set_weight(i, arr)
+                    qm.set_lm_head_blocks(DTYPE_Q6_K, synth.q6_k_blocks(seed + 9, qcfg.vocab_size * qcfg.hidden_size // 256))
+                    qm.finalize(2048)
+                else:
+                    qm = synth_model.build_model(ctx, qcfg, qw, 2048, wdt if mix is None else DTYPE_Q8_0, has_qk_norm=True,
+                                                 proj_dtypes=mix)
                 qm.init_kv_cache(kv, PREFILL)
                 qm.set_graph(not args.no_graph)
                 qm.bench_decode(int(prompt[0]), max(args.warmup, 2))

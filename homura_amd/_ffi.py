@@ -99,6 +99,7 @@ SIGNATURES = {
     "hm_gemm_f32_bf16_nk": (_I, [_P, _P, _P, _P, _I, _I, _I]),
     "hm_gemm_f32_quant_nk": (_I, [_P, _P, _P, _I, _P, _I, _I, _I]),
     "hm_model_set_weight_nk": (_I, [_P, _I, _P, _SZ]),
+    "hm_model_set_lm_head_blocks": (_I, [_P, _I, _P, _SZ]),
     "hm_model_config": (_I, [_P, _P, _P, _P]),
     "hm_tokenizer_open": (_P, [C.c_char_p, C.c_char_p, C.c_char_p, _SZ]),
     "hm_tokenizer_open_json": (_P, [C.c_char_p, C.c_char_p, _SZ]),

@@ -23,4 +23,12 @@ int gemv_kquant_fused(hm_ctx *ctx, bool q6, const float *d_x, const uint8_t *d_w
 int gemv_kquant(hm_ctx *ctx, bool q6, const float *d_x, const uint8_t *d_w, float *d_out, int K, int N,
                 bool reuse_activation);
 
+// LM head over K-quant blocks with f32 activations (the product with the dequantised weights): RMSNorm of
+// the row with norm_w on the way in, logits out, and the best (value, lowest index) of every workgroup in
+// cand_v / cand_i; gemv_kquant_f32_head_candidates says how many candidates that launch leaves.
+// K % 256 == 0, K <= 4096.
+int gemv_kquant_f32_head(hm_ctx *ctx, bool q6, const float *d_x, const float *d_norm_w, float eps, const uint8_t *d_w,
+                         float *d_out, int K, int N, float *cand_v, int *cand_i, int cand_cap);
+int gemv_kquant_f32_head_candidates(const hm_ctx *ctx, bool q6, int K, int N, int cand_cap);
+
 }  // namespace homura

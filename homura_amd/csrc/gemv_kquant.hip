@@ -644,6 +644,34 @@ int gemv_kquant_launch(hm_ctx *ctx, const char *name, const float *d_x, const ui
     return HM_OK;
 }
 
+// Rows per step, LDS and grid of the f32-activation kernel (the grid is also the number of argmax
+// candidates it leaves, so the plan has to be able to ask for it).
+struct F32Shape {
+    int rows, grid;
+    size_t stage_bytes, lds;
+};
+template <int QT>
+F32Shape f32_shape(const hm_ctx *ctx, int K, int N, int cand_cap) {
+    const size_t rowbytes = (size_t)(K / 256) * KTraits<QT>::BYTES;
+    int rows = (int)(((size_t)40 * 1024) / rowbytes);
+    rows = rows / KWAVES * KWAVES;
+    if (rows < KWAVES) rows = KWAVES;
+    if (rows > KMAX_ROWS) rows = KMAX_ROWS;
+    while (rows > KWAVES && (size_t)rows * rowbytes + 32 > (size_t)KSTAGE_BYTES) rows -= KWAVES;
+    while (rows > KWAVES && (N + rows - 1) / rows < 2 * ctx->num_cus) rows -= KWAVES;
+    F32Shape sh;
+    sh.rows = rows;
+    sh.stage_bytes = ((size_t)rows * rowbytes + 32 + 16 + 15) & ~(size_t)15;
+    sh.lds = sh.stage_bytes + (size_t)K * 4 + 64;
+    const int nsteps = (N + rows - 1) / rows;
+    int wg_per_cu = (int)(120 * 1024 / sh.lds);
+    if (wg_per_cu < 1) wg_per_cu = 1;
+    if (wg_per_cu > 6) wg_per_cu = 6;
+    sh.grid = nsteps < ctx->num_cus * wg_per_cu ? nsteps : ctx->num_cus * wg_per_cu;
+    if (cand_cap > 0 && sh.grid > cand_cap) sh.grid = cand_cap;
+    return sh;
+}
+
 template <int QT>
 int gemv_kquant_f32_launch(hm_ctx *ctx, const char *name, const float *d_x, const float *d_norm_w, float eps,
                            const uint8_t *d_w, float *d_out, int M, int K, int N, float *cand_v, int *cand_i, int cand_cap,
@@ -659,20 +687,9 @@ int gemv_kquant_f32_launch(hm_ctx *ctx, const char *name, const float *d_x, cons
     HM_REQUIRE(ctx, !cand_v || (cand_i && M == 1), "%s: argmax candidates need an index buffer and one row", name);
     const size_t rowbytes = (size_t)(K / 256) * BB;
     HM_REQUIRE(ctx, KWAVES * rowbytes + 32 <= (size_t)KSTAGE_BYTES, "%s: K=%d too large for the LDS stage", name, K);
-    int rows = (int)(((size_t)40 * 1024) / rowbytes);
-    rows = rows / KWAVES * KWAVES;
-    if (rows < KWAVES) rows = KWAVES;
-    if (rows > KMAX_ROWS) rows = KMAX_ROWS;
-    while (rows > KWAVES && (size_t)rows * rowbytes + 32 > (size_t)KSTAGE_BYTES) rows -= KWAVES;
-    while (rows > KWAVES && (N + rows - 1) / rows < 2 * ctx->num_cus) rows -= KWAVES;
-    const size_t stage_bytes = ((size_t)rows * rowbytes + 32 + 16 + 15) & ~(size_t)15;
-    const size_t lds = stage_bytes + (size_t)K * 4 + 64;
-    const int nsteps = (N + rows - 1) / rows;
-    int wg_per_cu = (int)(120 * 1024 / lds);
-    if (wg_per_cu < 1) wg_per_cu = 1;
-    if (wg_per_cu > 6) wg_per_cu = 6;
-    int grid = nsteps < ctx->num_cus * wg_per_cu ? nsteps : ctx->num_cus * wg_per_cu;
-    if (cand_v && grid > cand_cap) grid = cand_cap;
+    const F32Shape sh = f32_shape<QT>(ctx, K, N, cand_v ? cand_cap : 0);
+    const int rows = sh.rows, grid = sh.grid;
+    const size_t stage_bytes = sh.stage_bytes, lds = sh.lds;
     HM_REQUIRE(ctx, grid >= 1, "%s: no room for argmax candidates", name);
     if (grid_out) *grid_out = grid;
     const int cpl = (K / 16 + WAVE - 1) / WAVE;
@@ -713,6 +730,16 @@ int homura::gemv_kquant_fused(hm_ctx *ctx, bool q6, const float *d_x, const uint
                               const QuantFuse &fuse) {
     return q6 ? gemv_kquant_launch<1>(ctx, "gemv_kquant[q6_k]", d_x, d_w, d_out, 1, K, N, false, &fuse)
               : gemv_kquant_launch<0>(ctx, "gemv_kquant[q4_k]", d_x, d_w, d_out, 1, K, N, false, &fuse);
+}
+
+int homura::gemv_kquant_f32_head(hm_ctx *ctx, bool q6, const float *d_x, const float *d_norm_w, float eps,
+                                 const uint8_t *d_w, float *d_out, int K, int N, float *cand_v, int *cand_i, int cand_cap) {
+    return q6 ? gemv_kquant_f32_launch<1>(ctx, "gemv_q6_k_f32[head]", d_x, d_norm_w, eps, d_w, d_out, 1, K, N, cand_v, cand_i, cand_cap, nullptr)
+              : gemv_kquant_f32_launch<0>(ctx, "gemv_q4_k_f32[head]", d_x, d_norm_w, eps, d_w, d_out, 1, K, N, cand_v, cand_i, cand_cap, nullptr);
+}
+
+int homura::gemv_kquant_f32_head_candidates(const hm_ctx *ctx, bool q6, int K, int N, int cand_cap) {
+    return q6 ? f32_shape<1>(ctx, K, N, cand_cap).grid : f32_shape<0>(ctx, K, N, cand_cap).grid;
 }
 
 int homura::gemv_kquant(hm_ctx *ctx, bool q6, const float *d_x, const uint8_t *d_w, float *d_out, int K, int N,

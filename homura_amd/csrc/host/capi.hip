@@ -130,6 +130,13 @@ int hm_model_set_weight_nk(hm_model *m, int slot, const void *h_data, size_t byt
     return m->impl->set_weight_nk(slot, h_data, bytes);
 }
 
+int hm_model_set_lm_head_blocks(hm_model *m, int dtype, const void *h_blocks, size_t bytes) {
+    if (!m) return HM_ERR_INVALID;
+    if (dtype != HM_DTYPE_Q4_K && dtype != HM_DTYPE_Q6_K)
+        return hm_set_error(m->ctx, HM_ERR_INVALID, "hm_model_set_lm_head_blocks: dtype %d is neither Q4_K nor Q6_K", dtype);
+    return m->impl->set_lm_head_blocks((DType)dtype, h_blocks, bytes);
+}
+
 int hm_model_finalize(hm_model *m, int max_seq_len) {
     if (!m) return HM_ERR_INVALID;
     return m->impl->finalize(max_seq_len);

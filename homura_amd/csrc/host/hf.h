@@ -70,6 +70,12 @@ class HfModel {
     // other, K contiguous: the layout of HF safetensors ([out, in]) and of GGUF tensors, and the
     // stream layout kept in HBM, so nothing is transposed on the way in.
     int set_weight_nk(int slot, const void *h_data, size_t bytes) { return set_weight_impl(slot, h_data, bytes, true); }
+    // Block-quantised plans only, before finalize: the LM head as the GGUF blocks of the output matrix
+    // (Q4_K or Q6_K, [vocab][hidden / 256]) in place of the f32 slot. The head then multiplies the f32 row
+    // with the dequantised weights straight from the blocks - the numbers of the reference's f32 head over
+    // the matrix its loader dequantises (src/gguf.rs:589-708, :696-700), read at 144 / 210 bytes per 256
+    // weights instead of 1024. hidden % 256 == 0, hidden <= 4096.
+    int set_lm_head_blocks(DType dtype, const void *h_blocks, size_t bytes);
     // reference HfModel::ensure_compiled (src/hf/model.rs:148-160) + RoPE tables (:62-66)
     int finalize(int max_seq_len);
 
@@ -132,6 +138,8 @@ class HfModel {
     void quant_run(int layer, int which, int *first, int *count) const;
     std::vector<LayerPacked> packed_;
     Buffer lm_head_packed_;
+    Buffer lm_head_blocks_;             // set_lm_head_blocks: raw K-quant blocks of the output matrix
+    DType lm_head_blocks_dtype_ = DType::F32;
     Buffer rope_cos_, rope_sin_;        // [max_position][head_dim] f32
     Buffer ids_view_, mask_view_;
     std::shared_ptr<PlanScratch> scratch_;

@@ -303,6 +303,36 @@ int HfModel::set_weight_impl(int slot, const void *h_data, size_t bytes, bool nk
     return HM_OK;
 }
 
+int HfModel::set_lm_head_blocks(DType dtype, const void *h_blocks, size_t bytes) {
+    if (finalized_) return hm_set_error(ctx_, HM_ERR_STATE, "set_lm_head_blocks after finalize");
+    if (!dtype_is_quantized(weight_dtype_))
+        return hm_set_error(ctx_, HM_ERR_INVALID, "set_lm_head_blocks: only block-quantised plans keep an f32 LM head");
+    if (dtype != DType::Q4_K && dtype != DType::Q6_K)
+        return hm_set_error(ctx_, HM_ERR_INVALID, "set_lm_head_blocks: Q4_K or Q6_K blocks expected");
+    const int64_t hidden = cfg_.hidden_size, vocab = cfg_.vocab_size;
+    if (hidden % 256 != 0 || hidden > 4096)
+        return hm_set_error(ctx_, HM_ERR_INVALID, "set_lm_head_blocks: hidden_size %lld must be a multiple of 256, at most 4096", (long long)hidden);
+    size_t want = 0;
+    const size_t per = dtype_bytes_for_elements(dtype, (size_t)(hidden * vocab), nullptr);
+    want = per;
+    if (!h_blocks || bytes != want)
+        return hm_set_error(ctx_, HM_ERR_INVALID, "set_lm_head_blocks: %zu bytes given, [%lld][%lld / 256] blocks take %zu",
+                            bytes, (long long)vocab, (long long)hidden, want);
+    int slot = -1;
+    for (size_t i = 0; i < infos_.size(); i++)
+        if (infos_[i].name == "lm_head.weight") slot = (int)i;
+    if (slot < 0) return hm_set_error(ctx_, HM_ERR_STATE, "set_lm_head_blocks: the plan has no LM head slot");
+    lm_head_blocks_ = Buffer::alloc_bytes(ctx_, bytes, {(int64_t)bytes}, dtype);
+    if (!lm_head_blocks_) return HM_ERR_OOM;
+    const int rc = hm_upload(ctx_, lm_head_blocks_.ptr(), h_blocks, bytes);
+    if (rc != HM_OK) return rc;
+    lm_head_blocks_dtype_ = dtype;
+    lm_head_packed_ = Buffer();  // an f32 head uploaded earlier is no longer needed
+    weight_bufs_[slot] = Buffer::view(lm_head_blocks_.ptr(), bytes, {(int64_t)bytes}, {1}, dtype);
+    weight_set_[slot] = true;
+    return HM_OK;
+}
+
 int HfModel::finalize(int max_seq_len) {
     if (finalized_) return HM_OK;
     for (size_t i = 0; i < weight_set_.size(); i++)
@@ -1083,10 +1113,17 @@ int HfModel::emit_transformer_plan_quant() {
         CompiledKernel k;
         k.ops_label = "LMHead";
         DeviceLaunch h1;
-        h1.name = "gemv_f32[lm_head+argmax]";
-        h1.bytes_fixed = (double)hidden * vocab * 4 + hidden * 8.0 + vocab * 4.0;
+        const bool head_blocks = (bool)lm_head_blocks_;
+        const bool head_q6 = lm_head_blocks_dtype_ == DType::Q6_K;
+        h1.name = !head_blocks ? "gemv_f32[lm_head+argmax]" : head_q6 ? "gemv_q6_k_f32[lm_head+argmax]" : "gemv_q4_k_f32[lm_head+argmax]";
+        h1.bytes_fixed = (head_blocks ? (double)lm_head_blocks_.bytes() : (double)hidden * vocab * 4) + hidden * 8.0 + vocab * 4.0;
         h1.fn = [=](const StepContext &sc) -> int {
             const auto &in = sc.step.input_slots;
+            if (head_blocks)  // the f32 product with the dequantised output matrix, read from its blocks
+                return gemv_kquant_f32_head(sc.ctx, head_q6, sc.pool[in[0]]->as<float>(), sc.pool[in[1]]->as<float>(), eps,
+                                            sc.pool[in[2]]->as<uint8_t>(), sc.pool[sc.step.output_slots[0]]->as<float>(),
+                                            (int)hidden, (int)vocab, scr->cand_val.as<float>(), scr->cand_idx.as<int>(),
+                                            scr->cand_cap);
             GemvArgs g;
             g.x = sc.pool[in[0]]->as<float>();
             g.norm_w = sc.pool[in[1]]->as<float>();
@@ -1107,7 +1144,8 @@ int HfModel::emit_transformer_plan_quant() {
         h2.moves_cursor = true;
         h2.bytes_fixed = 64;
         h2.fn = [=](const StepContext &sc) -> int {
-            const int ncand = std::min(gemv_bf16_nk_grid(sc.ctx, (int)vocab, 4), scr->cand_cap);
+            const int ncand = head_blocks ? gemv_kquant_f32_head_candidates(sc.ctx, head_q6, (int)hidden, (int)vocab, scr->cand_cap)
+                                          : std::min(gemv_bf16_nk_grid(sc.ctx, (int)vocab, 4), scr->cand_cap);
             return finish_step_launch(sc.ctx, sc.plan->state(), scr->cand_val.as<float>(),
                                       scr->cand_idx.as<int>(), ncand, sc.plan->out_tokens(),
                                       sc.plan->out_capacity());
@@ -1400,9 +1438,14 @@ int HfModel::prefill_chunk(const int32_t *h_ids, int n, float *h_logits) {
             // slabs of its rows become bf16 pieces in wsplit, as many as fit
             const int slab = (int)std::min<int64_t>(vocab, (int64_t)(p.wsplit.bytes() / 2) / (3 * (int64_t)hidden) / 128 * 128);
             if (slab <= 0) return hm_set_error(ctx_, HM_ERR_STATE, "prefill: weight scratch too small for the LM head");
+            const size_t head_rowbytes = lm_head_blocks_ ? lm_head_blocks_.bytes() / (size_t)vocab : 0;
             for (int v0 = 0; v0 < vocab && rc == HM_OK; v0 += slab) {
                 const int rows = std::min(slab, vocab - v0);
-                rc = split_rows_launch(ctx_, lm_head_packed_.as<float>() + (size_t)v0 * hidden, wsplit, 3, (size_t)rows, hidden);
+                if (lm_head_blocks_)  // rows of the output matrix dequantised from its blocks (bit-exact) into the pieces
+                    rc = dequant_split_launch(ctx_, (int)lm_head_blocks_dtype_, lm_head_blocks_.as<uint8_t>() + (size_t)v0 * head_rowbytes,
+                                              rows, (int)hidden, wsplit, 1, 0);
+                else
+                    rc = split_rows_launch(ctx_, lm_head_packed_.as<float>() + (size_t)v0 * hidden, wsplit, 3, (size_t)rows, hidden);
                 if (rc == HM_OK)
                     rc = gemm_split_split_nk(ctx_, split, wsplit, p.logits.as<float>() + v0, n, hidden, rows, 1, nullptr, vocab);
             }

@@ -703,7 +703,11 @@ std::unique_ptr<HfModel> load_gguf_model(hm_ctx *ctx, const std::string &path, i
                 fail(ctx, path + ": tensor " + name + " is not [vocab, hidden]");
                 return nullptr;
             }
-            if (quant) {  // the quantised plan keeps an f32 head (src/gguf.rs:696-700)
+            if (quant && (t->type == GgmlType::Q4K || t->type == GgmlType::Q6K) && cfg.hidden_size % 256 == 0 &&
+                cfg.hidden_size <= 4096) {
+                // the f32 head of the quantised plan (src/gguf.rs:696-700), taken from the blocks as they are
+                rc = m->set_lm_head_blocks(t->type == GgmlType::Q6K ? DType::Q6_K : DType::Q4_K, src, t->byte_size());
+            } else if (quant) {  // the quantised plan keeps an f32 head (src/gguf.rs:696-700)
                 if (!ggml_to_f32(t->type, src, n, &f32, &err)) {
                     fail(ctx, path + ": tensor " + name + ": " + err);
                     return nullptr;

@@ -393,6 +393,12 @@ class HfModel:
         arr = np.ascontiguousarray(arr)
         self._check(self.lib.hm_model_set_weight_nk(self.h, slot, arr.ctypes.data_as(C.c_void_p), arr.nbytes))
 
+    def set_lm_head_blocks(self, dtype: int, blocks: np.ndarray):
+        """Block-quantised plans: the LM head as raw Q4_K / Q6_K blocks [vocab][hidden / 256] instead of the
+        f32 lm_head.weight slot (hm_model_set_lm_head_blocks)."""
+        a = np.ascontiguousarray(blocks, np.uint8).reshape(-1)
+        self._check(self.lib.hm_model_set_lm_head_blocks(self.h, int(dtype), a.ctypes.data, a.nbytes))
+
     def finalize(self, max_seq_len: int):
         self._check(self.lib.hm_model_finalize(self.h, max_seq_len))
 

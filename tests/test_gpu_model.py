@@ -253,3 +253,61 @@ def test_mixed_model_rejects_bad_dtype_lists(ctx):
         HfModel(ctx, cfg, proj_dtypes=[1] * 7 * cfg.num_hidden_layers)  # bf16 is not a block type
     with pytest.raises(HomuraError):                                 # hidden 256*k needed for K-quants
         HfModel(ctx, synth_model.TINY_LLAMA, proj_dtypes=[2, 2, 2, 2, 2, 2, 5] * 2)  # inter 704 % 256 != 0
+
+
+@pytest.mark.parametrize("kind", ["q6_k", "q4_k"])
+def test_lm_head_from_kquant_blocks(ctx, kind):
+    """The LM head of a block-quantised plan given as the raw blocks of the output matrix: the same f32
+    product as with the dequantised matrix in the f32 slot (the oracle, and a second model, get
+    oracle.dequant of the blocks), for single steps, the greedy loop, graph replay and the prompt pass."""
+    import pyoracle
+    cfg = synth_model.TINY_K
+    L = cfg.num_hidden_layers
+    mix = synth_model.q4_k_m_mix(cfg)
+    weights = synth_model.synth_weights(cfg, 91, has_qk_norm=False, proj_dtypes=mix)
+    assert weights[-1][0] == "lm_head.weight"
+    nblocks = cfg.vocab_size * cfg.hidden_size // 256
+    raw = (synth.q6_k_blocks if kind == "q6_k" else synth.q4_k_blocks)(92, nblocks)
+    dense = (pyoracle.dequant_q6_k if kind == "q6_k" else pyoracle.dequant_q4_k)(raw).reshape(cfg.vocab_size, cfg.hidden_size)
+    weights[-1] = ("lm_head.weight", np.ascontiguousarray(dense.T))   # the slot takes [hidden][vocab]
+    dense_model = synth_model.build_model(ctx, cfg, weights, 160, has_qk_norm=False, proj_dtypes=mix)
+    om = mf.build_oracle_model(cfg, weights, 160, has_qk_norm=False, proj_dtypes=mix)
+
+    gm = HfModel(ctx, cfg, has_qk_norm=False, proj_dtypes=mix)
+    for i, (name, arr) in enumerate(weights[:-1]):
+        gm.set_weight(i, arr)
+    with pytest.raises(HomuraError):
+        gm.set_lm_head_blocks(6 if kind == "q6_k" else 5, raw[:-1])       # wrong size
+    with pytest.raises(HomuraError):
+        gm.set_lm_head_blocks(2, raw)                                     # not a K-quant type
+    gm.set_lm_head_blocks(6 if kind == "q6_k" else 5, raw)
+    gm.finalize(160)
+
+    kv = synth_model.synth_kv(cfg, 3, 29)
+    ids = synth.token_ids(4, 5, cfg.vocab_size)
+    for m in (gm, dense_model):
+        m.set_prefill_min(0)
+        m.init_kv_cache(kv, 29)
+    mf.oracle_init_kv(om, kv)
+    got, dense_got = gm.run_kv(ids), dense_model.run_kv(ids)
+    want = np.concatenate([om.run_kv(ids[i:i + 1]) for i in range(5)])
+    scale = np.abs(want).max()
+    for i in range(5):
+        assert mf.rel_err(got[i], want[i]) < 1e-2, f"position {i}"
+    assert np.abs(got - dense_got).max() < 2e-5 * scale   # two f32 summation orders over the same terms
+    want_t, margins = om.generate_greedy(ids[:2], 24)
+    say(f"LM head from {kind} blocks: min margin {margins.min():.3e}, blocks vs dense {np.abs(got - dense_got).max() / scale:.1e}")
+    assert np.array_equal(gm.generate_greedy(ids[:2], 24), want_t)
+    gm.set_graph(True)
+    gm.init_kv_cache(kv, 29)
+    gm.run_kv(ids)
+    assert np.array_equal(gm.generate_greedy(ids[:2], 24), want_t)
+    # prompt pass: logits of every row through the piece GEMM over the dequantised blocks
+    long_ids = synth.token_ids(8, 40, cfg.vocab_size)
+    for m in (gm, dense_model):
+        m.set_prefill_min(8)
+        m.reset_kv_cache()
+    a, b = gm.run_kv(long_ids), dense_model.run_kv(long_ids)
+    assert np.abs(a - b).max() < 2e-5 * np.abs(b).max()
+    gm.close()
+    dense_model.close()
