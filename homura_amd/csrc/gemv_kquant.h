@@ -24,7 +24,7 @@ int gemv_kquant(hm_ctx *ctx, bool q6, const float *d_x, const uint8_t *d_w, floa
                 bool reuse_activation);
 
 // LM head over K-quant blocks with f32 activations (the product with the dequantised weights): RMSNorm of
-// the row with norm_w on the way in, logits out, and the best (value, lowest index) of every workgroup in
+// the row with norm_w on the way in, logits out, and the best (value, last index among equals; -1 without rows) of every workgroup in
 // cand_v / cand_i; gemv_kquant_f32_head_candidates says how many candidates that launch leaves.
 // K % 256 == 0, K <= 4096.
 int gemv_kquant_f32_head(hm_ctx *ctx, bool q6, const float *d_x, const float *d_norm_w, float eps, const uint8_t *d_w,

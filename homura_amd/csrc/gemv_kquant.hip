@@ -423,8 +423,9 @@ __device__ __forceinline__ void krows_trip_f32(const uint8_t *base, size_t rowby
         a[j] = wave_sum(a[j]);
         const int r = lr + j * KWAVES;
         if (lane == 0) out[r] = a[j];
-        // first maximum wins: rows reach a wavefront in ascending order (reference argmax, src/generate.rs:457-468)
-        if (a[j] > best_v) {
+        // of equal maxima the later row wins (Rust Iterator::max_by, reference src/generate.rs:457-468,
+        // :735-742); rows reach a wavefront in ascending order
+        if (best_i < 0 || a[j] >= best_v) {
             best_v = a[j];
             best_i = row0 + r;
         }
@@ -501,7 +502,7 @@ __global__ __launch_bounds__(KTHREADS) void gemv_kquant_f32_kernel(const float *
     }
 
     float best_v = -INFINITY;
-    int best_i = 0x7FFFFFFF;
+    int best_i = -1;
     for (; step < nsteps; step += gridDim.x) {
         __syncthreads();  // previous step's readers are done with the row stage
 #pragma unroll
@@ -529,7 +530,7 @@ __global__ __launch_bounds__(KTHREADS) void gemv_kquant_f32_kernel(const float *
         }
         if (lr < now.nrows) krows_trip_f32<QT, CPL, 1>(base, rowbytes, lr, lane, nu, act, o, now.r0, best_v, best_i);
     }
-    if (cand_v) {  // the workgroup's best row: largest value, lowest index among equals
+    if (cand_v) {  // the workgroup's best row: largest value, highest index among equals; -1 = no row
         __syncthreads();
         int *redi = reinterpret_cast<int *>(red + KWAVES);
         if (lane == 0) {
@@ -538,13 +539,15 @@ __global__ __launch_bounds__(KTHREADS) void gemv_kquant_f32_kernel(const float *
         }
         __syncthreads();
         if (tid == 0) {
-            float bv = red[0];
-            int bi = redi[0];
-            for (int wv = 1; wv < KWAVES; wv++)
-                if (red[wv] > bv || (red[wv] == bv && redi[wv] < bi)) {
+            float bv = -INFINITY;
+            int bi = -1;
+            for (int wv = 0; wv < KWAVES; wv++) {
+                if (redi[wv] < 0) continue;
+                if (bi < 0 || red[wv] > bv || (red[wv] == bv && redi[wv] > bi)) {
                     bv = red[wv];
                     bi = redi[wv];
                 }
+            }
             cand_v[blockIdx.x] = bv;
             cand_i[blockIdx.x] = bi;
         }

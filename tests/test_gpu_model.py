@@ -311,3 +311,21 @@ def test_lm_head_from_kquant_blocks(ctx, kind):
     assert np.abs(a - b).max() < 2e-5 * np.abs(b).max()
     gm.close()
     dense_model.close()
+
+    # equal maxima: the winning row's blocks copied to two more rows; the last of the three must win
+    # (Rust Iterator::max_by, src/generate.rs:735-742), through the candidates of every workgroup
+    rowbytes = raw.size // cfg.vocab_size
+    rows = raw.reshape(cfg.vocab_size, rowbytes).copy()
+    t = int(want_t[0])
+    twins = sorted({t, (t + 17) % cfg.vocab_size, (t + 401) % cfg.vocab_size})
+    for r in twins:
+        rows[r] = rows[t]
+    gm2 = HfModel(ctx, cfg, has_qk_norm=False, proj_dtypes=mix)
+    for i, (name, arr) in enumerate(weights[:-1]):
+        gm2.set_weight(i, arr)
+    gm2.set_lm_head_blocks(6 if kind == "q6_k" else 5, rows.reshape(-1))
+    gm2.finalize(160)
+    gm2.init_kv_cache(kv, 29)
+    gm2.run_kv(ids)
+    assert int(gm2.generate_greedy(ids[:2], 1)[0]) == twins[-1]
+    gm2.close()
