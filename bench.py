@@ -208,20 +208,22 @@ def main() -> int:
             quantised = {"unit": "tok/s", "steps": args.steps,
                          "what": "same shape, cache and step count; raw GGUF blocks dequantised in registers "
                                  "(K-quants: Q8_K activations, integer dots), f32 LM head; "
-                                 "q4_k_m_mix_q6_k_head: the head as Q6_K blocks multiplied in f32"}
+                                 "*_head: the head as Q8_0 / Q6_K blocks multiplied in f32"}
             kmix = synth_model.q4_k_m_mix(qcfg)
-            for name, wdt, mix, head_q6k in (("q8_0", DTYPE_Q8_0, None, False), ("q4_0", DTYPE_Q4_0, None, False),
-                                             ("q4_k_m_mix", None, kmix, False),
-                                             # as Q4_K_M files come: the output matrix in Q6_K, read from its blocks
-                                             ("q4_k_m_mix_q6_k_head", None, kmix, True)):
+            from homura_amd.runtime import DTYPE_Q6_K, HfModel
+            nw = qcfg.vocab_size * qcfg.hidden_size
+            for name, wdt, mix, head in (("q8_0", DTYPE_Q8_0, None, None), ("q4_0", DTYPE_Q4_0, None, None),
+                                         ("q4_k_m_mix", None, kmix, None),
+                                         # as the files come: the output matrix in blocks too, read as it is
+                                         ("q8_0_q8_0_head", DTYPE_Q8_0, None, (DTYPE_Q8_0, lambda: synth.q8_0_blocks(seed + 9, nw // 32, 0.01))),
+                                         ("q4_k_m_mix_q6_k_head", None, kmix, (DTYPE_Q6_K, lambda: synth.q6_k_blocks(seed + 9, nw // 256)))):
                 qw = synth_model.synth_weights(qcfg, seed + 7, wdt if mix is None else DTYPE_Q8_0, has_qk_norm=True,
                                                proj_dtypes=mix)
-                if head_q6k:
-                    from homura_amd.runtime import DTYPE_Q6_K, HfModel
-                    qm = HfModel(ctx, qcfg, DTYPE_Q8_0, True, proj_dtypes=mix)
+                if head is not None:
+                    qm = HfModel(ctx, qcfg, wdt if mix is None else DTYPE_Q8_0, True, proj_dtypes=mix)
                     for i, (_n, arr) in enumerate(qw[:-1]):
                         qm.set_weight(i, arr)
-                    qm.set_lm_head_blocks(DTYPE_Q6_K, synth.q6_k_blocks(seed + 9, qcfg.vocab_size * qcfg.hidden_size // 256))
+                    qm.set_lm_head_blocks(head[0], head[1]())
                     qm.finalize(2048)
                 else:
                     qm = synth_model.build_model(ctx, qcfg, qw, 2048, wdt if mix is None else DTYPE_Q8_0, has_qk_norm=True,

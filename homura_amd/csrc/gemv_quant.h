@@ -21,10 +21,17 @@ struct QuantFuse {
     float eps = 0.f;
     // result on the way out:     out[n] <- dot[n] + res_out_add[n]
     const float *res_out_add = nullptr;
+    // LM head: the best (value, last index among equals; -1 without rows) of every workgroup, one entry
+    // per workgroup of the launch (gemv_quant_workgroups of them)
+    float *cand_v = nullptr;
+    int *cand_i = nullptr;
 };
 
 // out[N] = W[N][K] (Q8_0 when q4 is false, Q4_0 when true) . f(x), one activation row
 int gemv_quant_fused(hm_ctx *ctx, bool q4, const float *d_x, const uint8_t *d_w, float *d_out, int K, int N,
                      const QuantFuse &fuse);
+
+// Workgroups gemv_quant_fused launches for this shape (= argmax candidates it leaves when asked to).
+int gemv_quant_workgroups(const hm_ctx *ctx, bool q4, int K, int N);
 
 }  // namespace homura

@@ -114,7 +114,7 @@ __device__ __forceinline__ StepRange step_range(int step, int rows_per_step, int
 template <int QT, int NXV, int RT>
 __device__ __forceinline__ void rows_trip(const uint8_t *base, size_t rowbytes, int lr, int lane, int nq,
                                           const float (&xv)[NXV][8], const float (&sxo)[NXV], float *out,
-                                          const float *add) {
+                                          const float *add, int row0, float &best_v, int &best_i) {
     constexpr int BB = BlockTraits<QT>::BYTES;
     const int doff = (lane >> 2) * BB;
     const int qoff = doff + 2 + (lane & 3) * BlockTraits<QT>::QUARTER;
@@ -138,7 +138,13 @@ __device__ __forceinline__ void rows_trip(const uint8_t *base, size_t rowbytes, 
 #pragma unroll
     for (int j = 0; j < RT; j++) {
         a[j] = wave_sum(a[j]);
-        if (lane == 0) out[lr + j * QWAVES] = add ? a[j] + add[lr + j * QWAVES] : a[j];
+        const float v = add ? a[j] + add[lr + j * QWAVES] : a[j];
+        if (lane == 0) out[lr + j * QWAVES] = v;
+        // of equal maxima the later row wins (Rust Iterator::max_by, reference src/generate.rs:735-742)
+        if (best_i < 0 || v >= best_v) {
+            best_v = v;
+            best_i = row0 + lr + j * QWAVES;
+        }
     }
 }
 
@@ -243,6 +249,8 @@ __global__ __launch_bounds__(QTHREADS) void gemv_quant_kernel(
         }
     }
 
+    float best_v = -INFINITY;
+    int best_i = -1;
     for (; step < nsteps; step += gridDim.x) {
         __syncthreads();  // previous step's readers are done with ws
 #pragma unroll
@@ -268,12 +276,12 @@ __global__ __launch_bounds__(QTHREADS) void gemv_quant_kernel(
             // up to four rows per trip: independent chains for the LDS reads and the reductions
             int lr = wave;
             for (; lr + 3 * QWAVES < now.nrows; lr += 4 * QWAVES)
-                rows_trip<QT, NXV, 4>(base, rowbytes, lr, lane, nq, xv, sxo, out + now.r0, add);
+                rows_trip<QT, NXV, 4>(base, rowbytes, lr, lane, nq, xv, sxo, out + now.r0, add, now.r0, best_v, best_i);
             if (lr + QWAVES < now.nrows) {
-                rows_trip<QT, NXV, 2>(base, rowbytes, lr, lane, nq, xv, sxo, out + now.r0, add);
+                rows_trip<QT, NXV, 2>(base, rowbytes, lr, lane, nq, xv, sxo, out + now.r0, add, now.r0, best_v, best_i);
                 lr += 2 * QWAVES;
             }
-            if (lr < now.nrows) rows_trip<QT, NXV, 1>(base, rowbytes, lr, lane, nq, xv, sxo, out + now.r0, add);
+            if (lr < now.nrows) rows_trip<QT, NXV, 1>(base, rowbytes, lr, lane, nq, xv, sxo, out + now.r0, add, now.r0, best_v, best_i);
         } else {  // long rows: the activations of a column are re-read from LDS
             float acc[MAX_ROWS_PER_WAVE];
 #pragma unroll
@@ -294,9 +302,39 @@ __global__ __launch_bounds__(QTHREADS) void gemv_quant_kernel(
 #pragma unroll
             for (int i = 0; i < MAX_ROWS_PER_WAVE; i++) {
                 const int lr = wave + QWAVES * i;
-                const float v = wave_sum(acc[i]);
-                if (lane == 0 && lr < now.nrows) out[now.r0 + lr] = add ? v + add[lr] : v;
+                const float dot = wave_sum(acc[i]);
+                if (lr < now.nrows) {
+                    const float v = add ? dot + add[lr] : dot;
+                    if (lane == 0) out[now.r0 + lr] = v;
+                    if (best_i < 0 || v >= best_v) {
+                        best_v = v;
+                        best_i = now.r0 + lr;
+                    }
+                }
             }
+        }
+    }
+    if (fuse.cand_v) {  // the workgroup's best row: largest value, highest index among equals; -1 = no row
+        __syncthreads();
+        float *cv = reinterpret_cast<float *>(ws);
+        int *ci = reinterpret_cast<int *>(ws) + QWAVES;
+        if (lane == 0) {
+            cv[wave] = best_v;
+            ci[wave] = best_i;
+        }
+        __syncthreads();
+        if (tid == 0) {
+            float bv = -INFINITY;
+            int bi = -1;
+            for (int wv = 0; wv < QWAVES; wv++) {
+                if (ci[wv] < 0) continue;
+                if (bi < 0 || cv[wv] > bv || (cv[wv] == bv && ci[wv] > bi)) {
+                    bv = cv[wv];
+                    bi = ci[wv];
+                }
+            }
+            fuse.cand_v[blockIdx.x] = bv;
+            fuse.cand_i[blockIdx.x] = bi;
         }
     }
 }
@@ -311,6 +349,35 @@ __global__ __launch_bounds__(256) void dequant_kernel(const uint8_t *__restrict_
     const size_t stride = (size_t)gridDim.x * blockDim.x;
     for (; e < n_elems; e += stride)
         out[e] = homura::dequant_element<QF>(blocks + (e >> 5) * BlockTraits<QT>::BYTES, (int)(e & 31));
+}
+
+// Rows staged per step, LDS and grid of gemv_quant_kernel for a shape.
+struct QuantShape {
+    int rows, grid;
+    size_t lds;
+};
+template <int QT>
+QuantShape quant_shape(const hm_ctx *ctx, int K, int N) {
+    constexpr int BB = BlockTraits<QT>::BYTES;
+    const size_t rowbytes = (size_t)(K / 32) * BB, x_bytes = (size_t)K * 4, lds_budget = 48 * 1024;
+    // rows staged per step: as many as fit the LDS budget (at most 8 per wavefront), but few
+    // enough that every CU gets a workgroup
+    int rows = (int)((lds_budget - x_bytes) / rowbytes);
+    rows = rows / QWAVES * QWAVES;
+    if (rows < QWAVES) rows = QWAVES;
+    if (rows > QWAVES * MAX_ROWS_PER_WAVE) rows = QWAVES * MAX_ROWS_PER_WAVE;
+    while (rows > QWAVES && (size_t)rows * rowbytes + 32 > (size_t)STAGE_BYTES) rows -= QWAVES;
+    while (rows > QWAVES && (N + rows - 1) / rows < 2 * ctx->num_cus) rows -= QWAVES;
+    QuantShape sh;
+    sh.rows = rows;
+    sh.lds = x_bytes + (size_t)rows * rowbytes + 32 + 16 * BB;  // slack: see rows_trip
+    const int nsteps = (N + rows - 1) / rows;
+    // persistent workgroups: a few per CU, each stages the activations once
+    int wg_per_cu = (int)(120 * 1024 / sh.lds);
+    if (wg_per_cu < 1) wg_per_cu = 1;
+    if (wg_per_cu > 6) wg_per_cu = 6;
+    sh.grid = nsteps < ctx->num_cus * wg_per_cu ? nsteps : ctx->num_cus * wg_per_cu;
+    return sh;
 }
 
 template <int QT>
@@ -329,26 +396,14 @@ int gemv_quant_launch(hm_ctx *ctx, const char *name, const float *d_x, const uin
     HM_REQUIRE(ctx, M == 1 || (!fuse.x2 && !fuse.res_in && !fuse.norm_w && !fuse.res_out_add), "%s: fused light ops need M == 1", name);
     const size_t rowbytes = (size_t)(K / 32) * BB;
     const size_t x_bytes = (size_t)K * 4;
-    const size_t lds_budget = 48 * 1024;
     HM_REQUIRE(ctx, x_bytes + QWAVES * rowbytes + 32 <= 64 * 1024 && QWAVES * rowbytes + 32 <= (size_t)STAGE_BYTES,
                "%s: K=%d too large for the LDS stage", name, K);
-    // rows staged per step: as many as fit the LDS budget (at most 8 per wavefront), but few
-    // enough that every CU gets a workgroup
-    int rows = (int)((lds_budget - x_bytes) / rowbytes);
-    rows = rows / QWAVES * QWAVES;
-    if (rows < QWAVES) rows = QWAVES;
-    if (rows > QWAVES * MAX_ROWS_PER_WAVE) rows = QWAVES * MAX_ROWS_PER_WAVE;
-    while (rows > QWAVES && (size_t)rows * rowbytes + 32 > (size_t)STAGE_BYTES) rows -= QWAVES;
-    while (rows > QWAVES && (N + rows - 1) / rows < 2 * ctx->num_cus) rows -= QWAVES;
-    const size_t lds = x_bytes + (size_t)rows * rowbytes + 32 + 16 * BB;  // slack: see rows_trip
-    const int nsteps = (N + rows - 1) / rows;
-    // persistent workgroups: a few per CU, each stages the activations once
-    int wg_per_cu = (int)(120 * 1024 / lds);
-    if (wg_per_cu < 1) wg_per_cu = 1;
-    if (wg_per_cu > 6) wg_per_cu = 6;
-    const int grid = nsteps < ctx->num_cus * wg_per_cu ? nsteps : ctx->num_cus * wg_per_cu;
+    const QuantShape sh = quant_shape<QT>(ctx, K, N);
+    const int rows = sh.rows, grid = sh.grid;
+    const size_t lds = sh.lds;
+    HM_REQUIRE(ctx, !fuse.cand_v || fuse.cand_i, "%s: argmax candidates need an index buffer", name);
     const int cpl = (K / 8 + WAVE - 1) / WAVE;
-    const bool fused = fuse.x2 || fuse.res_in || fuse.norm_w || fuse.res_out_add;
+    const bool fused = fuse.x2 || fuse.res_in || fuse.norm_w || fuse.res_out_add || fuse.cand_v;
     for (int m = 0; m < M; m++) {
         const float *xm = d_x + (size_t)m * K;
         float *om = d_out + (size_t)m * N;
@@ -394,6 +449,10 @@ int dequant_launch(hm_ctx *ctx, const char *name, const uint8_t *d_blocks, float
 }
 
 }  // namespace
+
+int homura::gemv_quant_workgroups(const hm_ctx *ctx, bool q4, int K, int N) {
+    return q4 ? quant_shape<1>(ctx, K, N).grid : quant_shape<0>(ctx, K, N).grid;
+}
 
 int homura::gemv_quant_fused(hm_ctx *ctx, bool q4, const float *d_x, const uint8_t *d_w, float *d_out, int K, int N,
                              const QuantFuse &fuse) {

@@ -132,8 +132,8 @@ int hm_model_set_weight_nk(hm_model *m, int slot, const void *h_data, size_t byt
 
 int hm_model_set_lm_head_blocks(hm_model *m, int dtype, const void *h_blocks, size_t bytes) {
     if (!m) return HM_ERR_INVALID;
-    if (dtype != HM_DTYPE_Q4_K && dtype != HM_DTYPE_Q6_K)
-        return hm_set_error(m->ctx, HM_ERR_INVALID, "hm_model_set_lm_head_blocks: dtype %d is neither Q4_K nor Q6_K", dtype);
+    if (dtype != HM_DTYPE_Q8_0 && dtype != HM_DTYPE_Q4_0 && dtype != HM_DTYPE_Q4_K && dtype != HM_DTYPE_Q6_K)
+        return hm_set_error(m->ctx, HM_ERR_INVALID, "hm_model_set_lm_head_blocks: dtype %d is not a block type", dtype);
     return m->impl->set_lm_head_blocks((DType)dtype, h_blocks, bytes);
 }
 

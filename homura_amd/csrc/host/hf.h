@@ -71,10 +71,10 @@ class HfModel {
     // stream layout kept in HBM, so nothing is transposed on the way in.
     int set_weight_nk(int slot, const void *h_data, size_t bytes) { return set_weight_impl(slot, h_data, bytes, true); }
     // Block-quantised plans only, before finalize: the LM head as the GGUF blocks of the output matrix
-    // (Q4_K or Q6_K, [vocab][hidden / 256]) in place of the f32 slot. The head then multiplies the f32 row
-    // with the dequantised weights straight from the blocks - the numbers of the reference's f32 head over
-    // the matrix its loader dequantises (src/gguf.rs:589-708, :696-700), read at 144 / 210 bytes per 256
-    // weights instead of 1024. hidden % 256 == 0, hidden <= 4096.
+    // (Q8_0, Q4_0, Q4_K or Q6_K, rows of hidden / 32 or hidden / 256 blocks) in place of the f32 slot. The head
+    // then multiplies the f32 row with the dequantised weights straight from the blocks - the numbers of the
+    // reference's f32 head over the matrix its loader dequantises (src/gguf.rs:589-708, :696-700), read at a
+    // sixth to a quarter of the bytes. hidden a multiple of the block length, at most 4096.
     int set_lm_head_blocks(DType dtype, const void *h_blocks, size_t bytes);
     // reference HfModel::ensure_compiled (src/hf/model.rs:148-160) + RoPE tables (:62-66)
     int finalize(int max_seq_len);

@@ -307,17 +307,19 @@ int HfModel::set_lm_head_blocks(DType dtype, const void *h_blocks, size_t bytes)
     if (finalized_) return hm_set_error(ctx_, HM_ERR_STATE, "set_lm_head_blocks after finalize");
     if (!dtype_is_quantized(weight_dtype_))
         return hm_set_error(ctx_, HM_ERR_INVALID, "set_lm_head_blocks: only block-quantised plans keep an f32 LM head");
-    if (dtype != DType::Q4_K && dtype != DType::Q6_K)
-        return hm_set_error(ctx_, HM_ERR_INVALID, "set_lm_head_blocks: Q4_K or Q6_K blocks expected");
+    if (!dtype_is_quantized(dtype))
+        return hm_set_error(ctx_, HM_ERR_INVALID, "set_lm_head_blocks: Q8_0, Q4_0, Q4_K or Q6_K blocks expected");
     const int64_t hidden = cfg_.hidden_size, vocab = cfg_.vocab_size;
-    if (hidden % 256 != 0 || hidden > 4096)
-        return hm_set_error(ctx_, HM_ERR_INVALID, "set_lm_head_blocks: hidden_size %lld must be a multiple of 256, at most 4096", (long long)hidden);
+    const int64_t per_block = (dtype == DType::Q4_K || dtype == DType::Q6_K) ? 256 : 32;
+    if (hidden % per_block != 0 || hidden > 4096)
+        return hm_set_error(ctx_, HM_ERR_INVALID, "set_lm_head_blocks: hidden_size %lld must be a multiple of %lld, at most 4096",
+                            (long long)hidden, (long long)per_block);
     size_t want = 0;
     const size_t per = dtype_bytes_for_elements(dtype, (size_t)(hidden * vocab), nullptr);
     want = per;
     if (!h_blocks || bytes != want)
-        return hm_set_error(ctx_, HM_ERR_INVALID, "set_lm_head_blocks: %zu bytes given, [%lld][%lld / 256] blocks take %zu",
-                            bytes, (long long)vocab, (long long)hidden, want);
+        return hm_set_error(ctx_, HM_ERR_INVALID, "set_lm_head_blocks: %zu bytes given, [%lld][%lld / %lld] blocks take %zu",
+                            bytes, (long long)vocab, (long long)hidden, (long long)per_block, want);
     int slot = -1;
     for (size_t i = 0; i < infos_.size(); i++)
         if (infos_[i].name == "lm_head.weight") slot = (int)i;
@@ -1114,11 +1116,25 @@ int HfModel::emit_transformer_plan_quant() {
         k.ops_label = "LMHead";
         DeviceLaunch h1;
         const bool head_blocks = (bool)lm_head_blocks_;
-        const bool head_q6 = lm_head_blocks_dtype_ == DType::Q6_K;
-        h1.name = !head_blocks ? "gemv_f32[lm_head+argmax]" : head_q6 ? "gemv_q6_k_f32[lm_head+argmax]" : "gemv_q4_k_f32[lm_head+argmax]";
+        const DType head_dt = lm_head_blocks_dtype_;
+        const bool head_q6 = head_dt == DType::Q6_K;
+        const bool head_k = head_dt == DType::Q4_K || head_dt == DType::Q6_K;  // else Q8_0 / Q4_0
+        h1.name = !head_blocks ? "gemv_f32[lm_head+argmax]"
+                  : head_q6    ? "gemv_q6_k_f32[lm_head+argmax]"
+                  : head_k     ? "gemv_q4_k_f32[lm_head+argmax]"
+                  : head_dt == DType::Q8_0 ? "gemv_q8_0[lm_head+argmax]" : "gemv_q4_0[lm_head+argmax]";
         h1.bytes_fixed = (head_blocks ? (double)lm_head_blocks_.bytes() : (double)hidden * vocab * 4) + hidden * 8.0 + vocab * 4.0;
         h1.fn = [=](const StepContext &sc) -> int {
             const auto &in = sc.step.input_slots;
+            if (head_blocks && !head_k) {  // Q8_0 / Q4_0: the dequant-GEMV of the projections, norm in, candidates out
+                QuantFuse f;
+                f.norm_w = sc.pool[in[1]]->as<float>();
+                f.eps = eps;
+                f.cand_v = scr->cand_val.as<float>();
+                f.cand_i = scr->cand_idx.as<int>();
+                return gemv_quant_fused(sc.ctx, head_dt == DType::Q4_0, sc.pool[in[0]]->as<float>(), sc.pool[in[2]]->as<uint8_t>(),
+                                        sc.pool[sc.step.output_slots[0]]->as<float>(), (int)hidden, (int)vocab, f);
+            }
             if (head_blocks)  // the f32 product with the dequantised output matrix, read from its blocks
                 return gemv_kquant_f32_head(sc.ctx, head_q6, sc.pool[in[0]]->as<float>(), sc.pool[in[1]]->as<float>(), eps,
                                             sc.pool[in[2]]->as<uint8_t>(), sc.pool[sc.step.output_slots[0]]->as<float>(),
@@ -1144,8 +1160,9 @@ int HfModel::emit_transformer_plan_quant() {
         h2.moves_cursor = true;
         h2.bytes_fixed = 64;
         h2.fn = [=](const StepContext &sc) -> int {
-            const int ncand = head_blocks ? gemv_kquant_f32_head_candidates(sc.ctx, head_q6, (int)hidden, (int)vocab, scr->cand_cap)
-                                          : std::min(gemv_bf16_nk_grid(sc.ctx, (int)vocab, 4), scr->cand_cap);
+            const int ncand = !head_blocks ? std::min(gemv_bf16_nk_grid(sc.ctx, (int)vocab, 4), scr->cand_cap)
+                              : head_k ? gemv_kquant_f32_head_candidates(sc.ctx, head_q6, (int)hidden, (int)vocab, scr->cand_cap)
+                                       : gemv_quant_workgroups(sc.ctx, head_dt == DType::Q4_0, (int)hidden, (int)vocab);
             return finish_step_launch(sc.ctx, sc.plan->state(), scr->cand_val.as<float>(),
                                       scr->cand_idx.as<int>(), ncand, sc.plan->out_tokens(),
                                       sc.plan->out_capacity());

@@ -703,10 +703,13 @@ std::unique_ptr<HfModel> load_gguf_model(hm_ctx *ctx, const std::string &path, i
                 fail(ctx, path + ": tensor " + name + " is not [vocab, hidden]");
                 return nullptr;
             }
-            if (quant && (t->type == GgmlType::Q4K || t->type == GgmlType::Q6K) && cfg.hidden_size % 256 == 0 &&
-                cfg.hidden_size <= 4096) {
+            const bool k_head = t->type == GgmlType::Q4K || t->type == GgmlType::Q6K;
+            const bool b32_head = t->type == GgmlType::Q8_0 || t->type == GgmlType::Q4_0;
+            if (quant && (k_head || b32_head) && cfg.hidden_size % (k_head ? 256 : 32) == 0 && cfg.hidden_size <= 4096) {
                 // the f32 head of the quantised plan (src/gguf.rs:696-700), taken from the blocks as they are
-                rc = m->set_lm_head_blocks(t->type == GgmlType::Q6K ? DType::Q6_K : DType::Q4_K, src, t->byte_size());
+                const DType hd = t->type == GgmlType::Q6K ? DType::Q6_K : t->type == GgmlType::Q4K ? DType::Q4_K
+                                 : t->type == GgmlType::Q8_0 ? DType::Q8_0 : DType::Q4_0;
+                rc = m->set_lm_head_blocks(hd, src, t->byte_size());
             } else if (quant) {  // the quantised plan keeps an f32 head (src/gguf.rs:696-700)
                 if (!ggml_to_f32(t->type, src, n, &f32, &err)) {
                     fail(ctx, path + ": tensor " + name + ": " + err);

@@ -392,14 +392,15 @@ int hm_model_launches_per_step(hm_model *m);
  * ([out, in]) and of GGUF tensors, and the layout kept in HBM, so nothing is transposed. The
  * reference transposes these on the host (transpose_2d, src/hf/weights.rs:225-261). */
 int hm_model_set_weight_nk(hm_model *m, int slot, const void *h_data, size_t bytes);
-/* Block-quantised models, before hm_model_finalize: the LM head as the raw Q4_K / Q6_K blocks of the
- * output matrix, [vocab][hidden / 256] x 144 / 210 bytes, in place of the f32 lm_head.weight slot (which
+/* Block-quantised models, before hm_model_finalize: the LM head as the raw blocks of the output matrix
+ * (Q4_K / Q6_K: [vocab][hidden / 256] x 144 / 210 bytes; Q8_0 / Q4_0: [vocab][hidden / 32] x 34 / 18 bytes),
+ * in place of the f32 lm_head.weight slot (which
  * need not be set then). The reference's quantised plan keeps an f32 head over the matrix its loader
  * dequantises (src/gguf.rs:696-700, emit_lm_head_kernel src/hf/emitter.rs:828-862); here the same product
  * is taken with every weight dequantised in registers, so a token reads 125 or 87 MB of head instead of
- * 622 MB at the Qwen3-0.6B width. hidden_size % 256 == 0 and <= 4096. hm_model_load_gguf does this by
- * itself when the file's output matrix (or, for tied models, its embedding) is Q4_K or Q6_K. No
- * counterpart call in the reference. */
+ * 622 MB at the Qwen3-0.6B width. hidden_size a multiple of the block length and <= 4096.
+ * hm_model_load_gguf does this by itself when the file's output matrix (or, for tied models, its
+ * embedding) has one of these types. No counterpart call in the reference. */
 int hm_model_set_lm_head_blocks(hm_model *m, int dtype, const void *h_blocks, size_t bytes);
 /* The configuration a model was created or loaded with. */
 int hm_model_config(hm_model *m, hm_transformer_config *out, int *has_qk_norm, int *weight_dtype);

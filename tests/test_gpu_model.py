@@ -255,7 +255,7 @@ def test_mixed_model_rejects_bad_dtype_lists(ctx):
         HfModel(ctx, synth_model.TINY_LLAMA, proj_dtypes=[2, 2, 2, 2, 2, 2, 5] * 2)  # inter 704 % 256 != 0
 
 
-@pytest.mark.parametrize("kind", ["q6_k", "q4_k"])
+@pytest.mark.parametrize("kind", ["q6_k", "q4_k", "q8_0", "q4_0"])
 def test_lm_head_from_kquant_blocks(ctx, kind):
     """The LM head of a block-quantised plan given as the raw blocks of the output matrix: the same f32
     product as with the dequantised matrix in the f32 slot (the oracle, and a second model, get
@@ -266,9 +266,14 @@ def test_lm_head_from_kquant_blocks(ctx, kind):
     mix = synth_model.q4_k_m_mix(cfg)
     weights = synth_model.synth_weights(cfg, 91, has_qk_norm=False, proj_dtypes=mix)
     assert weights[-1][0] == "lm_head.weight"
-    nblocks = cfg.vocab_size * cfg.hidden_size // 256
-    raw = (synth.q6_k_blocks if kind == "q6_k" else synth.q4_k_blocks)(92, nblocks)
-    dense = (pyoracle.dequant_q6_k if kind == "q6_k" else pyoracle.dequant_q4_k)(raw).reshape(cfg.vocab_size, cfg.hidden_size)
+    code = {"q8_0": 2, "q4_0": 3, "q4_k": 5, "q6_k": 6}[kind]
+    if kind in ("q6_k", "q4_k"):
+        raw = (synth.q6_k_blocks if kind == "q6_k" else synth.q4_k_blocks)(92, cfg.vocab_size * cfg.hidden_size // 256)
+    else:
+        raw = (synth.q8_0_blocks if kind == "q8_0" else synth.q4_0_blocks)(92, cfg.vocab_size * cfg.hidden_size // 32, 0.01)
+    dequant = {"q8_0": pyoracle.dequant_q8_0, "q4_0": pyoracle.dequant_q4_0, "q4_k": pyoracle.dequant_q4_k,
+               "q6_k": pyoracle.dequant_q6_k}[kind]
+    dense = dequant(raw).reshape(cfg.vocab_size, cfg.hidden_size)
     weights[-1] = ("lm_head.weight", np.ascontiguousarray(dense.T))   # the slot takes [hidden][vocab]
     dense_model = synth_model.build_model(ctx, cfg, weights, 160, has_qk_norm=False, proj_dtypes=mix)
     om = mf.build_oracle_model(cfg, weights, 160, has_qk_norm=False, proj_dtypes=mix)
@@ -277,10 +282,10 @@ def test_lm_head_from_kquant_blocks(ctx, kind):
     for i, (name, arr) in enumerate(weights[:-1]):
         gm.set_weight(i, arr)
     with pytest.raises(HomuraError):
-        gm.set_lm_head_blocks(6 if kind == "q6_k" else 5, raw[:-1])       # wrong size
+        gm.set_lm_head_blocks(code, raw[:-1])       # wrong size
     with pytest.raises(HomuraError):
-        gm.set_lm_head_blocks(2, raw)                                     # not a K-quant type
-    gm.set_lm_head_blocks(6 if kind == "q6_k" else 5, raw)
+        gm.set_lm_head_blocks(1, raw)               # bf16 is not a block type
+    gm.set_lm_head_blocks(code, raw)
     gm.finalize(160)
 
     kv = synth_model.synth_kv(cfg, 3, 29)
@@ -323,7 +328,7 @@ def test_lm_head_from_kquant_blocks(ctx, kind):
     gm2 = HfModel(ctx, cfg, has_qk_norm=False, proj_dtypes=mix)
     for i, (name, arr) in enumerate(weights[:-1]):
         gm2.set_weight(i, arr)
-    gm2.set_lm_head_blocks(6 if kind == "q6_k" else 5, rows.reshape(-1))
+    gm2.set_lm_head_blocks(code, rows.reshape(-1))
     gm2.finalize(160)
     gm2.init_kv_cache(kv, 29)
     gm2.run_kv(ids)
