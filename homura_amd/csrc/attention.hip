@@ -321,16 +321,17 @@ __global__ __launch_bounds__(ATT_THREADS) void gqa_decode_attn_stream_kernel(
     const int cnt = min(kv_len, n0 + chunk) - n0;  // >= 1: the grid covers kv_len exactly
     const int iters = (cnt + IT_ROWS - 1) / IT_ROWS;
 
+    // Rows past the live range are clamped to the last live row instead of masked: every request issues
+    // the same number of loads, so the waits can leave the next step's loads in flight. Their scores become
+    // -inf below, hence their probabilities zero, and the clamped V rows are finite.
     auto request = [&](u32x4(&kr)[KS], u32x4(&vr)[NRG_V], int it) {
-        const int krow = it * IT_ROWS + 16 * wave + l16;
-        const bool kok = krow < cnt;
+        const int krow = min(it * IT_ROWS + 16 * wave + l16, cnt - 1);
 #pragma unroll
-        for (int s = 0; s < KS; s++)
-            kr[s] = kok ? ld128_stream(kbase + (size_t)krow * HD + 32 * s) : u32x4{0u, 0u, 0u, 0u};
+        for (int s = 0; s < KS; s++) kr[s] = ld128_stream(kbase + (size_t)krow * HD + 32 * s);
 #pragma unroll
         for (int i = 0; i < NRG_V; i++) {
-            const int row = it * IT_ROWS + (i * ATT_WAVES + wave) * RPI + sub;
-            vr[i] = row < cnt ? ld128_stream(vbase + (size_t)row * HD) : u32x4{0u, 0u, 0u, 0u};
+            const int row = min(it * IT_ROWS + (i * ATT_WAVES + wave) * RPI + sub, cnt - 1);
+            vr[i] = ld128_stream(vbase + (size_t)row * HD);
         }
     };
     u32x4 ka[KS], va[NRG_V], kb[KS], vb[NRG_V];
@@ -362,7 +363,7 @@ __global__ __launch_bounds__(ATT_THREADS) void gqa_decode_attn_stream_kernel(
     }
 
     auto step = [&](u32x4(&kr)[KS], u32x4(&vr)[NRG_V], u32x4(&nkr)[KS], u32x4(&nvr)[NRG_V], int it) {
-        if (it + 1 < iters) request(nkr, nvr, it + 1);
+        request(nkr, nvr, min(it + 1, iters - 1));  // the last step re-reads itself: a fixed number of loads in flight
         float *scp = sc + (it & 1) * G * IT_ROWS;
         float *facp = fac + (it & 1) * G;
         // scores of the wavefront's 16 rows against every head; the small piece first. Lane
