@@ -42,13 +42,13 @@ KERNEL_FAMILY = {
 # the factors a 32 MiB + 32 MiB copy kernel calibrates), per kernel of the table below; the
 # counter runs are separate from this program and summarised under profiles/.
 PMC_TRAFFIC_BYTES = {
-    "gemv_bf16[qkv]": 8532785,
-    "gemv_bf16[o]": 4332370,
-    "gemv_bf16[gate_up+silu]": 12767925,
-    "gemv_bf16[down+residual]": 6526183,
-    "gemv_bf16[lm_head+argmax]": 311889780,
-    "qknorm_rope_append+gqa_attn": 4607833,
-    "gqa_attn_fold": 266045,
+    "gemv_bf16[qkv]": 8532745,
+    "gemv_bf16[o]": 4332353,
+    "gemv_bf16[gate_up+silu]": 12767903,
+    "gemv_bf16[down+residual]": 6526161,
+    "gemv_bf16[lm_head+argmax]": 311888819,
+    "qknorm_rope_append+gqa_attn": 4607523,
+    "gqa_attn_fold": 260929,
 }
 
 
