@@ -16,6 +16,12 @@ namespace homura {
 int gemv_kquant_fused(hm_ctx *ctx, bool q6, const float *d_x, const uint8_t *d_w, float *d_out, int K, int N,
                       const QuantFuse &fuse);
 
+// The fused form over two matrices of the two different K-quant types that share the row (q|k in Q4_K with v in
+// Q6_K, as Q4_K_M files have them): one launch, the row prepared once per workgroup. Residual and norm
+// prologue only. K <= 4096.
+int gemv_kquant_fused_pair(hm_ctx *ctx, bool first_q6, const float *d_x, const uint8_t *d_w, float *d_out, int N,
+                           const uint8_t *d_w2, float *d_out2, int N2, int K, const QuantFuse &fuse);
+
 // out[N] = W[N][K] (Q4_K when q6 is false, Q6_K when true) · x[K], x quantised to Q8_K first.
 // reuse_activation: skip the quantisation and multiply against what the previous call on this
 // context's stream left at the top of the workspace (same x, same K). Q4_K and Q6_K share the

@@ -250,13 +250,20 @@ __device__ __forceinline__ void stage_activation(const float *__restrict__ x, co
     }
 }
 
-template <int QT, int CPL, bool FUSED>
+// QT2 >= 0: a second matrix of the other K-quant type (w2, N2 rows, results to out2) shares the launch and
+// the prepared activation row - q|k in Q4_K with v in Q6_K, as Q4_K_M files have them. Its row steps follow
+// the first matrix's; a step never straddles the two.
+template <int QT, int CPL, bool FUSED, int QT2 = -1>
 __global__ __launch_bounds__(KTHREADS) void gemv_kquant_kernel(const int8_t *__restrict__ q8,
                                                                const float *__restrict__ act_d,
                                                                const int *__restrict__ bsums,
                                                                const uint8_t *__restrict__ w, float *__restrict__ out,
                                                                int K, int N, int rows_per_step, const float *x_f32_arg,
-                                                               const homura::QuantFuse fuse_arg, int act_lds_off) {
+                                                               const homura::QuantFuse fuse_arg, int act_lds_off,
+                                                               const uint8_t *__restrict__ w2 = nullptr,
+                                                               float *__restrict__ out2 = nullptr, int N2 = 0) {
+    constexpr bool TWO = QT2 >= 0;
+    constexpr int BB2 = KTraits<TWO ? QT2 : QT>::BYTES;
     // FUSED = false is the plain product over an activation quantised by its own launch
     const float *x_f32 = FUSED ? x_f32_arg : nullptr;
     const homura::QuantFuse fuse = FUSED ? fuse_arg : homura::QuantFuse();
@@ -265,13 +272,20 @@ __global__ __launch_bounds__(KTHREADS) void gemv_kquant_kernel(const int8_t *__r
     extern __shared__ __attribute__((aligned(16))) uint8_t ws[];
     const int tid = threadIdx.x, lane = tid & (WAVE - 1), wave = tid / WAVE;
     const int nb = K / 256, nu = K / 16;
-    const size_t rowbytes = (size_t)nb * BB;
-    const int nsteps = (N + rows_per_step - 1) / rows_per_step;
+    const size_t rowbytes = (size_t)nb * BB, rowbytes2 = (size_t)nb * BB2;
+    const int nsteps1 = (N + rows_per_step - 1) / rows_per_step;
+    const int nsteps = nsteps1 + (TWO ? (N2 + rows_per_step - 1) / rows_per_step : 0);
+    auto range_of = [&](int st) {
+        return TWO && st >= nsteps1 ? step_range(st - nsteps1, rows_per_step, N2, rowbytes2)
+                                    : step_range(st, rows_per_step, N, rowbytes);
+    };
+    auto src_of = [&](int st) { return TWO && st >= nsteps1 ? w2 : w; };
 
     // the first row step is requested before anything else waits
     u32x4 tmp[U];
     int step = blockIdx.x;
-    StepRange cur = step_range(step, rows_per_step, N, rowbytes);
+    StepRange cur = range_of(step);
+    const uint8_t *src = src_of(step);
     if (x_f32) {  // fused launch: the f32 row is prepared and quantised here, into LDS behind the row stage
         int8_t *lq8 = reinterpret_cast<int8_t *>(ws + act_lds_off);
         float *ld = reinterpret_cast<float *>(lq8 + K);
@@ -280,7 +294,7 @@ __global__ __launch_bounds__(KTHREADS) void gemv_kquant_kernel(const int8_t *__r
 #pragma unroll
         for (int u = 0; u < U; u++) {
             const int i = tid + u * KTHREADS;
-            tmp[u] = i < cur.nchunks ? ld128_stream(w + cur.abeg + (size_t)i * 16) : u32x4{0u, 0u, 0u, 0u};
+            tmp[u] = i < cur.nchunks ? ld128_stream(src + cur.abeg + (size_t)i * 16) : u32x4{0u, 0u, 0u, 0u};
         }
         stage_activation(x_f32, fuse, K, lq8, ld, lbs, red);
         asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
@@ -302,7 +316,7 @@ __global__ __launch_bounds__(KTHREADS) void gemv_kquant_kernel(const int8_t *__r
 #pragma unroll
         for (int u = 0; u < U; u++) {
             const int i = tid + u * KTHREADS;
-            tmp[u] = i < cur.nchunks ? ld128_stream(w + cur.abeg + (size_t)i * 16) : u32x4{0u, 0u, 0u, 0u};
+            tmp[u] = i < cur.nchunks ? ld128_stream(src + cur.abeg + (size_t)i * 16) : u32x4{0u, 0u, 0u, 0u};
         }
     }
 
@@ -315,18 +329,31 @@ __global__ __launch_bounds__(KTHREADS) void gemv_kquant_kernel(const int8_t *__r
         }
         __syncthreads();
         const StepRange now = cur;
+        const bool second = TWO && step >= nsteps1;
         if (step + (int)gridDim.x < nsteps) {  // the next step's weights travel while this one is multiplied
-            cur = step_range(step + gridDim.x, rows_per_step, N, rowbytes);
+            cur = range_of(step + gridDim.x);
+            src = src_of(step + gridDim.x);
 #pragma unroll
             for (int u = 0; u < U; u++) {
                 const int i = tid + u * KTHREADS;
-                tmp[u] = i < cur.nchunks ? ld128_stream(w + cur.abeg + (size_t)i * 16) : u32x4{0u, 0u, 0u, 0u};
+                tmp[u] = i < cur.nchunks ? ld128_stream(src + cur.abeg + (size_t)i * 16) : u32x4{0u, 0u, 0u, 0u};
             }
         }
         const uint8_t *base = ws + now.shift;
+        int lr = wave;
+        if (second) {
+            constexpr int Q2 = TWO ? QT2 : QT;
+            float *o = out2 + now.r0;
+            for (; lr + 3 * KWAVES < now.nrows; lr += 4 * KWAVES) krows_trip<Q2, CPL, 4>(base, rowbytes2, lr, lane, nu, act, o, nullptr);
+            if (lr + KWAVES < now.nrows) {
+                krows_trip<Q2, CPL, 2>(base, rowbytes2, lr, lane, nu, act, o, nullptr);
+                lr += 2 * KWAVES;
+            }
+            if (lr < now.nrows) krows_trip<Q2, CPL, 1>(base, rowbytes2, lr, lane, nu, act, o, nullptr);
+            continue;
+        }
         float *o = out + now.r0;
         const float *add = fuse.res_out_add ? fuse.res_out_add + now.r0 : nullptr;
-        int lr = wave;
         for (; lr + 3 * KWAVES < now.nrows; lr += 4 * KWAVES) krows_trip<QT, CPL, 4>(base, rowbytes, lr, lane, nu, act, o, add);
         if (lr + KWAVES < now.nrows) {
             krows_trip<QT, CPL, 2>(base, rowbytes, lr, lane, nu, act, o, add);
@@ -647,6 +674,53 @@ int gemv_kquant_launch(hm_ctx *ctx, const char *name, const float *d_x, const ui
     return HM_OK;
 }
 
+// One fused launch over two matrices of different K-quant types that share the activation row: the first
+// (type QT, N rows, results to d_out) and the second (the other type, N2 rows, results to d_out2).
+template <int QT>
+int gemv_kquant_pair_launch(hm_ctx *ctx, const char *name, const float *d_x, const uint8_t *d_w, float *d_out, int N,
+                            const uint8_t *d_w2, float *d_out2, int N2, int K, const homura::QuantFuse &fuse) {
+    HM_CHECK_CTX(ctx);
+    constexpr int QT2 = 1 - QT;
+    constexpr int BBMAX = KTraits<1>::BYTES;  // Q6_K rows are the longer ones
+    HM_REQUIRE(ctx, d_x && d_w && d_out && d_w2 && d_out2, "%s: NULL pointer", name);
+    HM_REQUIRE(ctx, K > 0 && K % 256 == 0 && N > 0 && N2 > 0, "%s: K=%d must be a positive multiple of 256, N=%d and N2=%d positive", name, K, N, N2);
+    HM_REQUIRE(ctx, K <= KXU * KTHREADS * 4, "%s: the fused form takes one row of at most %d", name, KXU * KTHREADS * 4);
+    HM_REQUIRE(ctx, ((uintptr_t)d_w % 16) == 0 && ((uintptr_t)d_w2 % 16) == 0 && ((uintptr_t)d_x % 16) == 0,
+               "%s: weight and activation buffers must be 16-byte aligned", name);
+    HM_REQUIRE(ctx, !fuse.x2 && !fuse.res_out_add, "%s: a pair takes the residual and norm prologue only", name);
+    HM_REQUIRE(ctx, ((uintptr_t)fuse.res_in % 16) == 0 && ((uintptr_t)fuse.resid_out % 16) == 0 && ((uintptr_t)fuse.norm_w % 16) == 0,
+               "%s: fused operands must be 16-byte aligned", name);
+    const size_t rowbytes = (size_t)(K / 256) * BBMAX;
+    HM_REQUIRE(ctx, KWAVES * rowbytes + 32 <= (size_t)KSTAGE_BYTES, "%s: K=%d too large for the LDS stage", name, K);
+    int rows = (int)(((size_t)40 * 1024) / rowbytes);
+    rows = rows / KWAVES * KWAVES;
+    if (rows < KWAVES) rows = KWAVES;
+    if (rows > KMAX_ROWS) rows = KMAX_ROWS;
+    while (rows > KWAVES && (size_t)rows * rowbytes + 32 > (size_t)KSTAGE_BYTES) rows -= KWAVES;
+    while (rows > KWAVES && (N + N2 + rows - 1) / rows < 2 * ctx->num_cus) rows -= KWAVES;
+    const size_t stage_bytes = ((size_t)rows * rowbytes + 32 + 16 + 15) & ~(size_t)15;
+    const size_t lds = stage_bytes + (size_t)K + (size_t)(K / 256) * 4 + (size_t)(K / 16) * 4 + 16;
+    const int nsteps = (N + rows - 1) / rows + (N2 + rows - 1) / rows;
+    int wg_per_cu = (int)(120 * 1024 / lds);
+    if (wg_per_cu < 1) wg_per_cu = 1;
+    if (wg_per_cu > 6) wg_per_cu = 6;
+    const int grid = nsteps < ctx->num_cus * wg_per_cu ? nsteps : ctx->num_cus * wg_per_cu;
+    const int cpl = (K / 16 + WAVE - 1) / WAVE;
+#define HM_KP_CASE(C)                                                                                                   \
+    hipLaunchKernelGGL((gemv_kquant_kernel<QT, C, true, QT2>), dim3(grid), dim3(KTHREADS), lds, ctx->stream,             \
+                       (const int8_t *)nullptr, (const float *)nullptr, (const int *)nullptr, d_w, d_out, K, N, rows, d_x, \
+                       fuse, (int)stage_bytes, d_w2, d_out2, N2)
+    switch (cpl) {
+        case 1: HM_KP_CASE(1); break;
+        case 2: HM_KP_CASE(2); break;
+        case 3: HM_KP_CASE(3); break;
+        default: HM_KP_CASE(4); break;
+    }
+#undef HM_KP_CASE
+    HM_LAUNCH_CHECK(ctx);
+    return HM_OK;
+}
+
 // Rows per step, LDS and grid of the f32-activation kernel (the grid is also the number of argmax
 // candidates it leaves, so the plan has to be able to ask for it).
 struct F32Shape {
@@ -743,6 +817,12 @@ int homura::gemv_kquant_f32_head(hm_ctx *ctx, bool q6, const float *d_x, const f
 
 int homura::gemv_kquant_f32_head_candidates(const hm_ctx *ctx, bool q6, int K, int N, int cand_cap) {
     return q6 ? f32_shape<1>(ctx, K, N, cand_cap).grid : f32_shape<0>(ctx, K, N, cand_cap).grid;
+}
+
+int homura::gemv_kquant_fused_pair(hm_ctx *ctx, bool first_q6, const float *d_x, const uint8_t *d_w, float *d_out, int N,
+                                   const uint8_t *d_w2, float *d_out2, int N2, int K, const QuantFuse &fuse) {
+    return first_q6 ? gemv_kquant_pair_launch<1>(ctx, "gemv_kquant[q6_k+q4_k]", d_x, d_w, d_out, N, d_w2, d_out2, N2, K, fuse)
+                    : gemv_kquant_pair_launch<0>(ctx, "gemv_kquant[q4_k+q6_k]", d_x, d_w, d_out, N, d_w2, d_out2, N2, K, fuse);
 }
 
 int homura::gemv_kquant(hm_ctx *ctx, bool q6, const float *d_x, const uint8_t *d_w, float *d_out, int K, int N,

@@ -844,10 +844,33 @@ int HfModel::emit_transformer_plan_quant() {
     constexpr size_t NO = (size_t)-1;
     struct FuseSlots { size_t x = (size_t)-1, x2 = (size_t)-1, res_in = (size_t)-1, resid_out = (size_t)-1,
                               norm_w = (size_t)-1, add = (size_t)-1, out = (size_t)-1; };
-    auto quant_mm = [&](const char *label, DType wdt, int64_t K, int64_t N, bool reuse_act, FuseSlots fs) {
+    // A second run of the group that rides in the first run's launch (the two K-quant types side by side)
+    struct PairedRun { size_t w_slot = (size_t)-1, out_slot = (size_t)-1; int64_t N = 0; DType dtype = DType::F32; std::string label; };
+    auto quant_mm = [&](const char *label, DType wdt, int64_t K, int64_t N, bool reuse_act, FuseSlots fs,
+                        PairedRun pair = PairedRun()) {
         CompiledKernel k;
         k.ops_label = std::string("QuantMM[") + label + "]";
-        if (N > 0) {
+        if (N > 0 && pair.N > 0) {
+            DeviceLaunch l;
+            l.name = std::string(wdt == DType::Q4_K ? "gemv_q4_k+q6_k[" : "gemv_q6_k+q4_k[") + label + "|" + pair.label + "]";
+            if (fs.norm_w != NO) l.name += fs.res_in != NO ? "+resid+norm" : "+norm";
+            l.bytes_fixed = (double)dtype_bytes_for_elements(wdt, (size_t)(K * N), nullptr) +
+                            (double)dtype_bytes_for_elements(pair.dtype, (size_t)(K * pair.N), nullptr) + K * 4.0 + (N + pair.N) * 4.0;
+            l.fn = [=](const StepContext &sc) -> int {
+                auto f32 = [&](size_t slot) { return slot == NO ? nullptr : sc.pool[slot]->as<float>(); };
+                const float *x = fs.x != NO ? f32(fs.x) : sc.pool[sc.step.input_slots[0]]->as<float>();
+                float *out = fs.out != NO ? f32(fs.out) : sc.pool[sc.step.output_slots[0]]->as<float>();
+                QuantFuse f;
+                f.res_in = f32(fs.res_in);
+                f.resid_out = f32(fs.resid_out);
+                f.norm_w = f32(fs.norm_w);
+                f.eps = eps;
+                return gemv_kquant_fused_pair(sc.ctx, wdt == DType::Q6_K, x, sc.pool[sc.step.input_slots[1]]->as<uint8_t>(), out, (int)N,
+                                              sc.pool[pair.w_slot]->as<uint8_t>(), sc.pool[pair.out_slot]->as<float>(), (int)pair.N,
+                                              (int)K, f);
+            };
+            k.launches.push_back(std::move(l));
+        } else if (N > 0) {
             DeviceLaunch l;
             const char *kn = wdt == DType::Q8_0 ? "gemv_q8_0[" : wdt == DType::Q4_0 ? "gemv_q4_0["
                              : wdt == DType::Q4_K ? "gemv_q4_k[" : "gemv_q6_k[";
@@ -890,23 +913,46 @@ int HfModel::emit_transformer_plan_quant() {
     // The QuantMM steps of one group of matrices that share an activation (q|k|v, gate|up, or one alone)
     struct GroupMember { const char *label; int which; int64_t N; size_t w_slot, out_slot; };
     auto quant_group = [&](int layer, size_t act_slot, int64_t K, std::vector<GroupMember> members, FuseSlots fs) {
+        // the runs of same-type neighbours: (first member, count, rows, label)
+        struct Run { size_t j; int count; int64_t n; std::string label; DType t; };
+        std::vector<Run> runs;
+        for (size_t j = 0; j < members.size(); j++) {
+            int first, count;
+            quant_run(layer, members[j].which, &first, &count);
+            if (first != members[j].which) continue;
+            Run r{j, count, 0, "", proj_dtype(layer, members[j].which)};
+            for (int e = 0; e < count; e++) {
+                r.n += members[j + e].N;
+                r.label += members[j + e].label;
+            }
+            runs.push_back(std::move(r));
+        }
+        auto is_k = [](DType t) { return t == DType::Q4_K || t == DType::Q6_K; };
+        // two runs, one of each K-quant type, prepared in the kernel: one launch for both
+        const bool paired = runs.size() == 2 && is_k(runs[0].t) && is_k(runs[1].t) && runs[0].t != runs[1].t && K <= 4096 &&
+                            fs.x2 == NO && fs.add == NO && fs.out == NO;
         bool act_quantized = false;
         for (size_t j = 0; j < members.size(); j++) {
             const GroupMember &gm = members[j];
-            int first, count;
-            quant_run(layer, gm.which, &first, &count);
             const DType t = proj_dtype(layer, gm.which);
-            const bool kq = t == DType::Q4_K || t == DType::Q6_K;
-            int64_t n_run = 0;
-            std::string label = gm.label;
-            if (first == gm.which) {
-                n_run = gm.N;
-                for (int e = 1; e < count; e++) {
-                    n_run += members[j + e].N;
-                    label += members[j + e].label;
-                }
+            const bool kq = is_k(t);
+            const Run *run = nullptr;
+            for (const Run &r : runs)
+                if (r.j == j) run = &r;
+            int64_t n_run = run ? run->n : 0;
+            const std::string label = run ? run->label : std::string(gm.label);
+            PairedRun pair;
+            if (paired && run == &runs[0]) {
+                const GroupMember &second = members[runs[1].j];
+                pair.w_slot = second.w_slot;
+                pair.out_slot = second.out_slot;
+                pair.N = runs[1].n;
+                pair.dtype = runs[1].t;
+                pair.label = runs[1].label;
+            } else if (paired && run == &runs[1]) {
+                n_run = 0;  // rides in the first run's launch
             }
-            add_step(quant_mm(label.c_str(), t, K, n_run, kq && act_quantized, fs), {act_slot, gm.w_slot}, {gm.out_slot});
+            add_step(quant_mm(label.c_str(), t, K, n_run, kq && act_quantized, fs, pair), {act_slot, gm.w_slot}, {gm.out_slot});
             if (n_run > 0 && kq) act_quantized = true;
         }
     };
