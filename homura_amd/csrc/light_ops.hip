@@ -250,17 +250,23 @@ __global__ __launch_bounds__(256) void finish_step_kernel(DecodeState *__restric
     __shared__ float s_v[4];
     __shared__ int s_i[4];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    // the cursor is requested together with the candidates (volatile: the loads stay up here), not after the fold
+    const volatile DecodeState *cursor = state;
+    int step = 0, pos = 0;
+    if (threadIdx.x == 0) {
+        step = cursor->step;
+        pos = cursor->pos;
+    }
     float bv = -INFINITY;
     int bi = -1;
     for (int i = threadIdx.x; i < n; i += 256) arg_merge(bv, bi, vals[i], idxs[i]);
-    for (int off = 32; off >= 1; off >>= 1) {
-        const float ov = __shfl_xor(bv, off, 64);
-        const int oi = __shfl_xor(bi, off, 64);
-        arg_merge(bv, bi, ov, oi);
-    }
+    // wave fold on the DPP path: the maximum, then the highest index that holds it (indices are below 2^24,
+    // exact as floats; -1 marks a lane without a candidate)
+    const float m = wave_max(bi >= 0 ? bv : -INFINITY);
+    const float sel = wave_max(bi >= 0 && bv == m ? (float)bi : -1.f);
     if (lane == 0) {
-        s_v[wave] = bv;
-        s_i[wave] = bi;
+        s_v[wave] = m;
+        s_i[wave] = (int)sel;
     }
     __syncthreads();
     if (threadIdx.x == 0) {
@@ -268,11 +274,10 @@ __global__ __launch_bounds__(256) void finish_step_kernel(DecodeState *__restric
         bi = -1;
         for (int w = 0; w < 4; w++) arg_merge(bv, bi, s_v[w], s_i[w]);
         const int tok = bi < 0 ? 0 : bi;
-        const int step = state->step;
         if (step < out_cap) out_tokens[step] = tok;
         state->token = tok;
         state->step = step + 1;
-        state->pos = state->pos + 1;
+        state->pos = pos + 1;
     }
 }
 
