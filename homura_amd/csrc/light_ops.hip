@@ -236,10 +236,17 @@ __global__ void embed_step_kernel(const DecodeState *__restrict__ state,
                                   const int32_t *__restrict__ forced,
                                   const float *__restrict__ table, float *__restrict__ out,
                                   int hidden, int vocab) {
-    int id = state->step < state->n_forced ? forced[state->step] : state->token;
+    const int step = state->step, n_forced = state->n_forced, token = state->token;  // one round trip
+    int id = step < n_forced ? forced[step] : token;
     if (id < 0 || id >= vocab) id = 0;
     const float *src = table + (size_t)id * hidden;
-    for (int k = threadIdx.x; k < hidden; k += blockDim.x) out[k] = src[k];
+    if ((hidden & 3) == 0 && ((uintptr_t)table & 15) == 0 && ((uintptr_t)out & 15) == 0) {
+        // 16 bytes per thread: a row of 1024 is one load per thread, not four in a row
+        for (int k = threadIdx.x * 4; k < hidden; k += blockDim.x * 4)
+            *reinterpret_cast<f32x4 *>(out + k) = *reinterpret_cast<const f32x4 *>(src + k);
+    } else {
+        for (int k = threadIdx.x; k < hidden; k += blockDim.x) out[k] = src[k];
+    }
 }
 
 __global__ __launch_bounds__(256) void finish_step_kernel(DecodeState *__restrict__ state,
@@ -259,7 +266,19 @@ __global__ __launch_bounds__(256) void finish_step_kernel(DecodeState *__restric
     }
     float bv = -INFINITY;
     int bi = -1;
-    for (int i = threadIdx.x; i < n; i += 256) arg_merge(bv, bi, vals[i], idxs[i]);
+    // the first 4096 candidates in one round trip (all loads issued before the first merge), the rest in a loop
+    constexpr int FU = 16;
+    float cv[FU];
+    int ci[FU];
+#pragma unroll
+    for (int u = 0; u < FU; u++) {
+        const int i = threadIdx.x + u * 256;
+        cv[u] = i < n ? vals[i] : -INFINITY;
+        ci[u] = i < n ? idxs[i] : -1;
+    }
+#pragma unroll
+    for (int u = 0; u < FU; u++) arg_merge(bv, bi, cv[u], ci[u]);
+    for (int i = threadIdx.x + FU * 256; i < n; i += 256) arg_merge(bv, bi, vals[i], idxs[i]);
     // wave fold on the DPP path: the maximum, then the highest index that holds it (indices are below 2^24,
     // exact as floats; -1 marks a lane without a candidate)
     const float m = wave_max(bi >= 0 ? bv : -INFINITY);
