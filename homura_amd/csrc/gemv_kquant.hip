@@ -113,16 +113,28 @@ __device__ __forceinline__ float q4k_unit(const uint8_t *blk, int i, const ActUn
 // One Q6_K unit: i = sub-block (0..15); chunk = i/8, group = (i%8)/2, parity = i%2:
 // low nibbles at ql[64 chunk + 32 (group&1) + 16 parity ..] (upper nibble for group >= 2), bit pair
 // `group` of qh[32 chunk + 16 parity ..], q = (lo | hi << 4) - 32 (emit_quant.rs:668-760).
-__device__ __forceinline__ float q6k_unit(const uint8_t *blk, int i, const ActUnit &a) {
+// stage = start of the LDS row stage (16-byte aligned), off = byte offset of the block in it (even): the
+// 16-byte pieces sit two bytes into a dword for every other block, so each is read as five aligned dwords
+// and shifted into place (five LDS reads and four funnel shifts instead of eight 16-bit reads and four merges).
+__device__ __forceinline__ float q6k_unit(const uint8_t *stage, int off, int i, const ActUnit &a) {
+    const uint8_t *blk = stage + off;
     const int chunk = i >> 3, group = (i & 7) >> 1, parity = i & 1;
-    const uint8_t *ql = blk + chunk * 64 + (group & 1) * 32 + parity * 16;
-    const uint8_t *qh = blk + 128 + chunk * 32 + parity * 16;
+    const int qlo = off + chunk * 64 + (group & 1) * 32 + parity * 16, qho = off + 128 + chunk * 32 + parity * 16;
+    const uint32_t sh = (uint32_t)(off & 2) * 8;
+    const uint32_t *pl = reinterpret_cast<const uint32_t *>(stage + (qlo & ~3));
+    const uint32_t *ph = reinterpret_cast<const uint32_t *>(stage + (qho & ~3));
+    uint32_t l[5], hg[5];
+#pragma unroll
+    for (int j = 0; j < 5; j++) {
+        l[j] = pl[j];
+        hg[j] = ph[j];
+    }
     const int lo_sh = group >= 2 ? 4 : 0, hi_sh = group * 2;
     uint32_t v[4];
 #pragma unroll
     for (int j = 0; j < 4; j++) {
-        const uint32_t l = lds32_a2(ql + 4 * j), hgh = lds32_a2(qh + 4 * j);
-        v[j] = ((l >> lo_sh) & 0x0F0F0F0Fu) | (((hgh >> hi_sh) & 0x03030303u) << 4);
+        const uint32_t lw = __builtin_amdgcn_alignbit(l[j + 1], l[j], sh), hw = __builtin_amdgcn_alignbit(hg[j + 1], hg[j], sh);
+        v[j] = ((lw >> lo_sh) & 0x0F0F0F0Fu) | (((hw >> hi_sh) & 0x03030303u) << 4);
     }
     const int isum = dot16(v, a.q) - 32 * a.bsum;
     const int sc = (int)(int8_t)blk[192 + i];
@@ -150,7 +162,7 @@ __device__ __forceinline__ StepRange step_range(int step, int rows_per_step, int
 // RT rows lr, lr + KWAVES, ... of the staged step for one wavefront. Round t of a lane is unit
 // lane + 64 t of the row: block (lane + 64 t) / 16 = lane/16 + 4 t, unit-in-block lane % 16.
 template <int QT, int CPL, int RT>
-__device__ __forceinline__ void krows_trip(const uint8_t *base, size_t rowbytes, int lr, int lane, int nu,
+__device__ __forceinline__ void krows_trip(const uint8_t *stage, int shift, size_t rowbytes, int lr, int lane, int nu,
                                            const ActUnit (&act)[CPL], float *out, const float *add) {
     constexpr int BB = KTraits<QT>::BYTES;
     const int boff = (lane >> 4) * BB, ui = lane & 15;
@@ -163,8 +175,8 @@ __device__ __forceinline__ void krows_trip(const uint8_t *base, size_t rowbytes,
 #pragma unroll
         for (int j = 0; j < RT; j++) {
             // lanes past the row end read the block of unit 0..15 of the row start: valid memory, dropped below
-            const uint8_t *blk = base + (size_t)(lr + j * KWAVES) * rowbytes + (live ? boff + t * 4 * BB : 0);
-            const float v = QT == 0 ? q4k_unit(blk, ui, act[t]) : q6k_unit(blk, ui, act[t]);
+            const int off = shift + (lr + j * KWAVES) * (int)rowbytes + (live ? boff + t * 4 * BB : 0);
+            const float v = QT == 0 ? q4k_unit(stage + off, ui, act[t]) : q6k_unit(stage, off, ui, act[t]);
             a[j] += live ? v : 0.f;
         }
         __builtin_amdgcn_sched_barrier(0);
@@ -339,27 +351,26 @@ __global__ __launch_bounds__(KTHREADS) void gemv_kquant_kernel(const int8_t *__r
                 tmp[u] = i < cur.nchunks ? ld128_stream(src + cur.abeg + (size_t)i * 16) : u32x4{0u, 0u, 0u, 0u};
             }
         }
-        const uint8_t *base = ws + now.shift;
         int lr = wave;
         if (second) {
             constexpr int Q2 = TWO ? QT2 : QT;
             float *o = out2 + now.r0;
-            for (; lr + 3 * KWAVES < now.nrows; lr += 4 * KWAVES) krows_trip<Q2, CPL, 4>(base, rowbytes2, lr, lane, nu, act, o, nullptr);
+            for (; lr + 3 * KWAVES < now.nrows; lr += 4 * KWAVES) krows_trip<Q2, CPL, 4>(ws, now.shift, rowbytes2, lr, lane, nu, act, o, nullptr);
             if (lr + KWAVES < now.nrows) {
-                krows_trip<Q2, CPL, 2>(base, rowbytes2, lr, lane, nu, act, o, nullptr);
+                krows_trip<Q2, CPL, 2>(ws, now.shift, rowbytes2, lr, lane, nu, act, o, nullptr);
                 lr += 2 * KWAVES;
             }
-            if (lr < now.nrows) krows_trip<Q2, CPL, 1>(base, rowbytes2, lr, lane, nu, act, o, nullptr);
+            if (lr < now.nrows) krows_trip<Q2, CPL, 1>(ws, now.shift, rowbytes2, lr, lane, nu, act, o, nullptr);
             continue;
         }
         float *o = out + now.r0;
         const float *add = fuse.res_out_add ? fuse.res_out_add + now.r0 : nullptr;
-        for (; lr + 3 * KWAVES < now.nrows; lr += 4 * KWAVES) krows_trip<QT, CPL, 4>(base, rowbytes, lr, lane, nu, act, o, add);
+        for (; lr + 3 * KWAVES < now.nrows; lr += 4 * KWAVES) krows_trip<QT, CPL, 4>(ws, now.shift, rowbytes, lr, lane, nu, act, o, add);
         if (lr + KWAVES < now.nrows) {
-            krows_trip<QT, CPL, 2>(base, rowbytes, lr, lane, nu, act, o, add);
+            krows_trip<QT, CPL, 2>(ws, now.shift, rowbytes, lr, lane, nu, act, o, add);
             lr += 2 * KWAVES;
         }
-        if (lr < now.nrows) krows_trip<QT, CPL, 1>(base, rowbytes, lr, lane, nu, act, o, add);
+        if (lr < now.nrows) krows_trip<QT, CPL, 1>(ws, now.shift, rowbytes, lr, lane, nu, act, o, add);
     }
 }
 
@@ -410,16 +421,26 @@ __device__ __forceinline__ float q4k_unit_f32(const uint8_t *blk, int i, const A
     return (d * (float)sc) * dot16_f32(nib, a.x) - (dmin * (float)mn) * a.sx;
 }
 
-__device__ __forceinline__ float q6k_unit_f32(const uint8_t *blk, int i, const ActF32 &a) {
+// same reads as q6k_unit: aligned dwords and funnel shifts
+__device__ __forceinline__ float q6k_unit_f32(const uint8_t *stage, int off, int i, const ActF32 &a) {
+    const uint8_t *blk = stage + off;
     const int chunk = i >> 3, group = (i & 7) >> 1, parity = i & 1;
-    const uint8_t *ql = blk + chunk * 64 + (group & 1) * 32 + parity * 16;
-    const uint8_t *qh = blk + 128 + chunk * 32 + parity * 16;
+    const int qlo = off + chunk * 64 + (group & 1) * 32 + parity * 16, qho = off + 128 + chunk * 32 + parity * 16;
+    const uint32_t sh = (uint32_t)(off & 2) * 8;
+    const uint32_t *pl = reinterpret_cast<const uint32_t *>(stage + (qlo & ~3));
+    const uint32_t *ph = reinterpret_cast<const uint32_t *>(stage + (qho & ~3));
+    uint32_t l[5], hg[5];
+#pragma unroll
+    for (int j = 0; j < 5; j++) {
+        l[j] = pl[j];
+        hg[j] = ph[j];
+    }
     const int lo_sh = group >= 2 ? 4 : 0, hi_sh = group * 2;
     uint32_t v[4];
 #pragma unroll
     for (int j = 0; j < 4; j++) {
-        const uint32_t l = lds32_a2(ql + 4 * j), hgh = lds32_a2(qh + 4 * j);
-        v[j] = ((l >> lo_sh) & 0x0F0F0F0Fu) | (((hgh >> hi_sh) & 0x03030303u) << 4);
+        const uint32_t lw = __builtin_amdgcn_alignbit(l[j + 1], l[j], sh), hw = __builtin_amdgcn_alignbit(hg[j + 1], hg[j], sh);
+        v[j] = ((lw >> lo_sh) & 0x0F0F0F0Fu) | (((hw >> hi_sh) & 0x03030303u) << 4);
     }
     const int sc = (int)(int8_t)blk[192 + i];
     const float d = f16_bits_to_f32((uint16_t)lds16(blk + 208));
@@ -427,7 +448,7 @@ __device__ __forceinline__ float q6k_unit_f32(const uint8_t *blk, int i, const A
 }
 
 template <int QT, int CPL, int RT>
-__device__ __forceinline__ void krows_trip_f32(const uint8_t *base, size_t rowbytes, int lr, int lane, int nu,
+__device__ __forceinline__ void krows_trip_f32(const uint8_t *stage, int shift, size_t rowbytes, int lr, int lane, int nu,
                                                const ActF32 (&act)[CPL], float *out, int row0, float &best_v, int &best_i) {
     constexpr int BB = KTraits<QT>::BYTES;
     const int boff = (lane >> 4) * BB, ui = lane & 15;
@@ -439,8 +460,8 @@ __device__ __forceinline__ void krows_trip_f32(const uint8_t *base, size_t rowby
         const bool live = lane + t * WAVE < nu;
 #pragma unroll
         for (int j = 0; j < RT; j++) {
-            const uint8_t *blk = base + (size_t)(lr + j * KWAVES) * rowbytes + (live ? boff + t * 4 * BB : 0);
-            const float v = QT == 0 ? q4k_unit_f32(blk, ui, act[t]) : q6k_unit_f32(blk, ui, act[t]);
+            const int off = shift + (lr + j * KWAVES) * (int)rowbytes + (live ? boff + t * 4 * BB : 0);
+            const float v = QT == 0 ? q4k_unit_f32(stage + off, ui, act[t]) : q6k_unit_f32(stage, off, ui, act[t]);
             a[j] += live ? v : 0.f;
         }
         __builtin_amdgcn_sched_barrier(0);
@@ -547,15 +568,14 @@ __global__ __launch_bounds__(KTHREADS) void gemv_kquant_f32_kernel(const float *
                 tmp[u] = i < cur.nchunks ? ld128_stream(w + cur.abeg + (size_t)i * 16) : u32x4{0u, 0u, 0u, 0u};
             }
         }
-        const uint8_t *base = ws + now.shift;
         float *o = out + now.r0;
         int lr = wave;
-        for (; lr + 3 * KWAVES < now.nrows; lr += 4 * KWAVES) krows_trip_f32<QT, CPL, 4>(base, rowbytes, lr, lane, nu, act, o, now.r0, best_v, best_i);
+        for (; lr + 3 * KWAVES < now.nrows; lr += 4 * KWAVES) krows_trip_f32<QT, CPL, 4>(ws, now.shift, rowbytes, lr, lane, nu, act, o, now.r0, best_v, best_i);
         if (lr + KWAVES < now.nrows) {
-            krows_trip_f32<QT, CPL, 2>(base, rowbytes, lr, lane, nu, act, o, now.r0, best_v, best_i);
+            krows_trip_f32<QT, CPL, 2>(ws, now.shift, rowbytes, lr, lane, nu, act, o, now.r0, best_v, best_i);
             lr += 2 * KWAVES;
         }
-        if (lr < now.nrows) krows_trip_f32<QT, CPL, 1>(base, rowbytes, lr, lane, nu, act, o, now.r0, best_v, best_i);
+        if (lr < now.nrows) krows_trip_f32<QT, CPL, 1>(ws, now.shift, rowbytes, lr, lane, nu, act, o, now.r0, best_v, best_i);
     }
     if (cand_v) {  // the workgroup's best row: largest value, highest index among equals; -1 = no row
         __syncthreads();
