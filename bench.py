@@ -42,13 +42,13 @@ KERNEL_FAMILY = {
 # the factors a 32 MiB + 32 MiB copy kernel calibrates), per kernel of the table below; the
 # counter runs are separate from this program and summarised under profiles/.
 PMC_TRAFFIC_BYTES = {
-    "gemv_bf16[qkv]": 8532729,
-    "gemv_bf16[o]": 4332348,
-    "gemv_bf16[gate_up+silu]": 12767883,
-    "gemv_bf16[down+residual]": 6526157,
-    "gemv_bf16[lm_head+argmax]": 311888402,
-    "qknorm_rope_append+gqa_attn": 4607535,
-    "gqa_attn_fold": 260935,
+    "gemv_bf16[qkv]": 8532770,
+    "gemv_bf16[o]": 4332364,
+    "gemv_bf16[gate_up+silu]": 12767935,
+    "gemv_bf16[down+residual]": 6526184,
+    "gemv_bf16[lm_head+argmax]": 311889597,
+    "qknorm_rope_append+gqa_attn": 4607533,
+    "gqa_attn_fold": 260930,
 }
 
 
