@@ -160,6 +160,10 @@ SIGNATURES = {
     "hm_model_reset_kv_cache": (_I, [_P]),
     "hm_model_kv_cache_len": (_I, [_P]),
     "hm_model_set_graph": (_I, [_P, _I]),
+    "hm_model_set_whole_step": (_I, [_P, _I]),
+    "hm_model_whole_step": (_I, [_P]),
+    "hm_model_whole_step_available": (_I, [_P]),
+    "hm_model_whole_step_status": (_I, [_P]),
     "hm_model_run_kv": (_I, [_P, C.POINTER(C.c_int64), _I, c_f32_p]),
     "hm_model_prefill": (_I, [_P, C.POINTER(C.c_int64), _I, c_f32_p]),
     "hm_model_generate": (_I, [_P, C.POINTER(C.c_int64), _I, _I, C.POINTER(HmSamplingConfig), C.c_uint64, _I,

@@ -1,0 +1,44 @@
+// Internal launch interface of the whole-step decode kernel (one launch for the embedding row
+// and every decoder layer of a bf16 model), shared with the decode plan.
+#pragma once
+#include "hm_common.h"
+
+// Per-layer device pointers. Matrices are in the K-contiguous stream layout the plan keeps:
+// wqkv [q_dim + 2 kv_dim][hidden], wo [hidden][q_dim], wgu [2 inter][hidden] with gate and up rows
+// interleaved (g0, u0, g1, u1, ...), wd [hidden][inter].
+struct FusedLayerPtrs {
+    const uint16_t *wqkv, *wo, *wgu, *wd;
+    const float *in_ln, *post_ln;
+    const float *q_norm, *k_norm;  // [head_dim] or nullptr (both)
+    const float *qkv_bias;         // [q_dim + 2 kv_dim] or nullptr
+    uint16_t *kcache, *vcache;     // [kv_heads][max_len][head_dim] bf16
+};
+
+struct FusedShape {
+    int hidden, heads, kv_heads, head_dim, inter;
+};
+
+struct FusedDecodeArgs {
+    const FusedLayerPtrs *layers;  // device array [n_layers]
+    int n_layers;
+    const float *embed;  // [vocab][hidden] f32
+    int vocab;
+    const DecodeState *state;
+    const int32_t *forced;
+    float *hidden_out;  // [hidden]: the last layer's output (input of the LM head)
+    const float *cos_tab, *sin_tab;  // [max_pos][head_dim]
+    float eps, scale;
+    int max_len;         // rows per KV head in the caches
+    unsigned char *xch;  // exchange area, decode_fused_xch_bytes() bytes, zeroed once
+    uint32_t *ctl;       // [0] launches so far (tag base), [1] sticky status (0 = ok), zeroed once
+};
+
+// Whether a kernel instance exists for this shape on this device; max_seq_len rows must fit the
+// attention phase's register-resident splits. `why` receives a short reason when not.
+bool decode_fused_supported(const hm_ctx *ctx, const FusedShape &s, int n_layers, int max_seq_len, const char **why);
+size_t decode_fused_xch_bytes(const FusedShape &s);
+// Largest cache length the attention phase serves for this shape (0 if unsupported)
+int decode_fused_max_kv(const FusedShape &s);
+int decode_fused_launch(hm_ctx *ctx, const FusedShape &s, const FusedDecodeArgs &a);
+// Reads the sticky status word (synchronises the stream). HM_OK or HM_ERR_HIP with a message.
+int decode_fused_check(hm_ctx *ctx, const uint32_t *d_ctl);

@@ -164,6 +164,26 @@ int hm_model_set_graph(hm_model *m, int on) {
     return m->impl->plan()->enable_graph(on != 0);
 }
 
+int hm_model_set_whole_step(hm_model *m, int on) {
+    if (!m) return HM_ERR_INVALID;
+    return m->impl->set_whole_step(on != 0);
+}
+
+int hm_model_whole_step(hm_model *m) {
+    if (!m) return HM_ERR_INVALID;
+    return m->impl->whole_step() ? 1 : 0;
+}
+
+int hm_model_whole_step_available(hm_model *m) {
+    if (!m) return HM_ERR_INVALID;
+    return m->impl->whole_step_available() ? 1 : 0;
+}
+
+int hm_model_whole_step_status(hm_model *m) {
+    if (!m) return HM_ERR_INVALID;
+    return m->impl->whole_step_status();
+}
+
 int hm_model_run_kv(hm_model *m, const int64_t *h_ids, int n_ids, float *h_logits) {
     if (!m) return HM_ERR_INVALID;
     return m->impl->run_kv(h_ids, n_ids, h_logits);

@@ -46,6 +46,9 @@ struct WeightSlotInfo {
 // O projection, the MLP's residual and activation) plus the LM-head argmax candidates.
 struct PlanScratch {
     Buffer attn_flat, resid, act, cand_val, cand_idx;
+    // whole-step decode launch (bf16 plans of a served shape): device layer table, exchange area,
+    // control words {launch count, status}
+    Buffer fused_layers, fused_xch, fused_ctl;
     Buffer normed, gate, up, down, q_raw, k_raw, v_raw;  // quantised plan only
     int cand_cap = 0;
 };
@@ -107,6 +110,13 @@ class HfModel {
                  int eos_token, int32_t *h_tokens, int *n_out);
     int bench_decode(int64_t first_id, int n_steps, float *ms_out, int32_t *h_tokens);
     int profile_step(int64_t token_id, std::vector<StepProfile> &out);
+    // The whole-step decode launch (one kernel for the embedding row and all layers) instead of one
+    // launch per projection. Available for bf16 models of a served shape; on by default then.
+    bool whole_step_available() const { return fused_available_; }
+    int set_whole_step(bool on);
+    bool whole_step() const { return plan_ && plan_->whole_step(); }
+    // HM_OK, or the error a whole-step launch left behind (an exchange that timed out)
+    int whole_step_status();
     int time_kernels(int rounds, std::vector<StepProfile> &out);
     ExecutionPlan *plan() { return plan_.get(); }
 
@@ -116,6 +126,8 @@ class HfModel {
     int emit_transformer_plan();        // reference src/hf/emitter.rs:867-1050
     int emit_transformer_plan_quant();  // reference src/hf/emitter_quant.rs:1142-1503
     int step_inputs(std::vector<Buffer *> &inputs);
+    int refresh_fused_table();
+    int finish_sync();
     int prefill_chunk(const int32_t *h_ids, int n, float *h_logits);
     const float *weight_f32(const std::string &name) const;
     int check_ids(const int64_t *ids, int n, std::vector<int32_t> &out);
@@ -125,6 +137,9 @@ class HfModel {
     DType weight_dtype_ = DType::BF16;
     bool has_qk_norm_ = false;
     bool finalized_ = false;
+    bool fused_available_ = false;
+    const void *fused_table_kv_ = nullptr;  // key_ptr(0) the device layer table was built for
+    int fused_table_max_len_ = 0;
     int max_seq_len_ = 0;
     std::vector<DType> proj_dtypes_;    // [layers][7]
     std::vector<WeightSlotInfo> infos_;

@@ -5,6 +5,7 @@
 #include <cstdlib>
 
 #include "../attention.h"
+#include "../decode_fused.h"
 #include "../gemv_bf16.h"
 #include "../gemm_bf16_mfma.h"
 #include "../gemv_kquant.h"
@@ -364,12 +365,35 @@ int HfModel::finalize(int max_seq_len) {
     s.cand_idx = Buffer::alloc(ctx_, {s.cand_cap}, DType::F32);
     if (!s.attn_flat || !s.resid || !s.act || !s.cand_val || !s.cand_idx) return HM_ERR_OOM;
 
+    // The whole-step decode launch serves bf16 models of a shape it has an instance for.
+    fused_available_ = false;
+    if (weight_dtype_ == DType::BF16) {
+        const FusedShape fs{cfg_.hidden_size, cfg_.num_attention_heads, cfg_.kv_heads(), cfg_.head_dim(),
+                            cfg_.intermediate_size};
+        if (decode_fused_supported(ctx_, fs, cfg_.num_hidden_layers, max_seq_len, nullptr)) {
+            s.fused_layers = Buffer::alloc_bytes(ctx_, sizeof(FusedLayerPtrs) * (size_t)cfg_.num_hidden_layers,
+                                                 {cfg_.num_hidden_layers}, DType::I64);
+            const size_t xb = decode_fused_xch_bytes(fs);
+            s.fused_xch = Buffer::alloc_bytes(ctx_, xb, {(int64_t)xb}, DType::I64);
+            s.fused_ctl = Buffer::alloc_bytes(ctx_, 64, {16}, DType::I64);
+            if (!s.fused_layers || !s.fused_xch || !s.fused_ctl) return HM_ERR_OOM;
+            HM_HIP(ctx_, hipMemsetAsync(s.fused_xch.ptr(), 0, xb, ctx_->stream));
+            HM_HIP(ctx_, hipMemsetAsync(s.fused_ctl.ptr(), 0, 64, ctx_->stream));
+            fused_available_ = true;
+        }
+    }
+
     rc = dtype_is_quantized(weight_dtype_) ? emit_transformer_plan_quant() : emit_transformer_plan();
     if (rc != HM_OK) return rc;
     rc = plan_->prepare(std::max(max_seq_len, 16));
     if (rc != HM_OK) return rc;
     rc = plan_->ensure_kv_cache(max_seq_len_);
     if (rc != HM_OK) return rc;
+    if (fused_available_) {
+        plan_->set_pre_run([this]() { return refresh_fused_table(); });
+        const char *e = std::getenv("HOMURA_WHOLE_STEP");  // 0: keep one launch per projection
+        if (!(e && std::atoi(e) == 0) && (rc = plan_->set_whole_step(true)) != HM_OK) return rc;
+    }
     ids_view_ = Buffer::view(plan_->forced_ids(), (size_t)plan_->out_capacity() * 4, {1, DIM_DYNAMIC},
                              {1, 1}, DType::I64);
     mask_view_ = Buffer::view(plan_->state(), sizeof(DecodeState), {1, 1, 1, DIM_DYNAMIC}, {1, 1, 1, 1},
@@ -491,7 +515,40 @@ int HfModel::emit_transformer_plan() {
             return embed_step_launch(sc.ctx, sc.plan->state(), sc.plan->forced_ids(), table->as<float>(),
                                      out->as<float>(), (int)vocab, (int)hidden);
         };
+        if (fused_available_) l.mode = DeviceLaunch::Mode::PerKernel;
         k.launches.push_back(std::move(l));
+        if (fused_available_) {
+            // One launch for the embedding row and every layer (decode_fused.hip); the layer kernels below
+            // then enqueue nothing, and the last hidden state lands in the last layer's output slot.
+            DeviceLaunch f;
+            f.name = "decode_whole_step[embed+layers]";
+            f.mode = DeviceLaunch::Mode::WholeStep;
+            const double layer_w = (double)hidden * (qd + 2 * kvd) * 2 + (double)qd * hidden * 2 +
+                                   (double)hidden * 2 * inter * 2 + (double)inter * hidden * 2;
+            f.bytes_fixed = L * (layer_w + 2 * hidden * 4.0 + 2 * kvd * 2.0) + hidden * 4.0 * 2;
+            f.bytes_per_kv_row = L * 2.0 * kvh * hd * 2;
+            const FusedShape fs{(int)hidden, (int)H, (int)kvh, (int)hd, (int)inter};
+            const size_t hidden_out_slot = ls[L - 1].hidden_out;
+            f.fn = [=](const StepContext &sc) -> int {
+                FusedDecodeArgs fa{};
+                fa.layers = reinterpret_cast<const FusedLayerPtrs *>(scr->fused_layers.ptr());
+                fa.n_layers = L;
+                fa.embed = sc.pool[sc.step.input_slots[1]]->as<float>();
+                fa.vocab = (int)vocab;
+                fa.state = sc.plan->state();
+                fa.forced = sc.plan->forced_ids();
+                fa.hidden_out = sc.pool[hidden_out_slot]->as<float>();
+                fa.cos_tab = sc.pool[cos_s]->as<float>();
+                fa.sin_tab = sc.pool[sin_s]->as<float>();
+                fa.eps = eps;
+                fa.scale = (float)(1.0 / std::sqrt((double)hd));  // f64 -> f32 constant, emitter.rs:719
+                fa.max_len = sc.plan->kv_cache()->max_len();
+                fa.xch = scr->fused_xch.as<unsigned char>();
+                fa.ctl = scr->fused_ctl.as<uint32_t>();
+                return decode_fused_launch(sc.ctx, fs, fa);
+            };
+            k.launches.push_back(std::move(f));
+        }
         kernels.push_back(std::move(k));
         steps.push_back(KernelStep::kernel(kernels.size() - 1, {input_ids, embed_w}, {embed_out}));
     }
@@ -522,6 +579,7 @@ int HfModel::emit_transformer_plan() {
                 g.eps = eps;
                 return gemv_bf16_nk_launch(sc.ctx, g, 1, GEMV_EPI_NONE);
             };
+            if (fused_available_) g1.mode = DeviceLaunch::Mode::PerKernel;
             k.launches.push_back(std::move(g1));
             kernels.push_back(std::move(k));
             // h, ln_w, q_w, [q_b], k_w, [k_b], v_w, [v_b], cos, sin, [q_norm_w, k_norm_w]
@@ -585,6 +643,7 @@ int HfModel::emit_transformer_plan() {
             a1.fn = [=](const StepContext &sc) -> int {
                 return gqa_decode_attn_launch(sc.ctx, attn_args(sc, AttnArgs::SPLIT_ONLY));
             };
+            if (fused_available_) a1.mode = DeviceLaunch::Mode::PerKernel;
             k.launches.push_back(std::move(a1));
             DeviceLaunch a1b;
             a1b.name = "gqa_attn_fold";
@@ -594,6 +653,7 @@ int HfModel::emit_transformer_plan() {
                 return gqa_decode_attn_launch(sc.ctx, attn_args(sc, AttnArgs::FOLD_ONLY));
             };
             a1 = std::move(a1b);
+            if (fused_available_) a1.mode = DeviceLaunch::Mode::PerKernel;
             k.launches.push_back(std::move(a1));
             DeviceLaunch a2;
             a2.name = "gemv_bf16[o]";
@@ -607,6 +667,7 @@ int HfModel::emit_transformer_plan() {
                 g.N = (int)hidden;
                 return gemv_bf16_nk_launch(sc.ctx, g, 1, GEMV_EPI_NONE);
             };
+            if (fused_available_) a2.mode = DeviceLaunch::Mode::PerKernel;
             k.launches.push_back(std::move(a2));
             kernels.push_back(std::move(k));
             steps.push_back(KernelStep::kernel(kernels.size() - 1,
@@ -633,6 +694,7 @@ int HfModel::emit_transformer_plan() {
                 g.N = (int)(2 * inter);
                 return gemv_bf16_nk_launch(sc.ctx, g, 1, GEMV_EPI_SILU_MUL_PAIRS);
             };
+            if (fused_available_) m1.mode = DeviceLaunch::Mode::PerKernel;
             k.launches.push_back(std::move(m1));
             DeviceLaunch m2;
             m2.name = "gemv_bf16[down+residual]";
@@ -647,6 +709,7 @@ int HfModel::emit_transformer_plan() {
                 d.epilogue_residual = scr->resid.as<float>();
                 return gemv_bf16_nk_launch(sc.ctx, d, 1, GEMV_EPI_RESIDUAL);
             };
+            if (fused_available_) m2.mode = DeviceLaunch::Mode::PerKernel;
             k.launches.push_back(std::move(m2));
             kernels.push_back(std::move(k));
             steps.push_back(KernelStep::kernel(
@@ -1242,6 +1305,58 @@ int HfModel::step_inputs(std::vector<Buffer *> &inputs) {
     return HM_OK;
 }
 
+// The device table of per-layer pointers the whole-step launch reads. It holds the KV cache's
+// addresses, so it is rebuilt when the cache has been re-created.
+int HfModel::refresh_fused_table() {
+    if (!fused_available_ || !plan_ || !plan_->kv_cache()) return HM_OK;
+    KvCache *kv = plan_->kv_cache();
+    if (fused_table_kv_ == kv->key_ptr(0) && fused_table_max_len_ == kv->max_len()) return HM_OK;
+    const int L = cfg_.num_hidden_layers;
+    std::vector<FusedLayerPtrs> t((size_t)L);
+    for (int l = 0; l < L; l++) {
+        const std::string p = "model.layers." + std::to_string(l) + ".";
+        FusedLayerPtrs &f = t[l];
+        f.wqkv = packed_[l].qkv.as<uint16_t>();
+        f.wo = packed_[l].o.as<uint16_t>();
+        f.wgu = packed_[l].gate_up.as<uint16_t>();
+        f.wd = packed_[l].down.as<uint16_t>();
+        f.in_ln = weight_f32(p + "input_layernorm.weight");
+        f.post_ln = weight_f32(p + "post_attention_layernorm.weight");
+        f.q_norm = has_qk_norm_ ? weight_f32(p + "self_attn.q_norm.weight") : nullptr;
+        f.k_norm = has_qk_norm_ ? weight_f32(p + "self_attn.k_norm.weight") : nullptr;
+        f.qkv_bias = cfg_.attention_bias ? packed_[l].qkv_bias.as<float>() : nullptr;
+        f.kcache = kv->key_ptr(l);
+        f.vcache = kv->value_ptr(l);
+        if (!f.wqkv || !f.wo || !f.wgu || !f.wd || !f.in_ln || !f.post_ln || !f.kcache || !f.vcache)
+            return hm_set_error(ctx_, HM_ERR_STATE, "whole-step decode: layer %d has an unset pointer", l);
+    }
+    int rc = hm_sync(ctx_);  // no launch may still be reading the old table
+    if (rc == HM_OK) rc = hm_upload(ctx_, scratch_->fused_layers.ptr(), t.data(), t.size() * sizeof(FusedLayerPtrs));
+    if (rc != HM_OK) return rc;
+    fused_table_kv_ = kv->key_ptr(0);
+    fused_table_max_len_ = kv->max_len();
+    return HM_OK;
+}
+
+// Stream sync plus, when steps went through the whole-step launch, its status word.
+int HfModel::finish_sync() {
+    int rc = hm_sync(ctx_);
+    if (rc == HM_OK && plan_ && plan_->whole_step()) rc = whole_step_status();
+    return rc;
+}
+
+int HfModel::set_whole_step(bool on) {
+    if (!finalized_) return hm_set_error(ctx_, HM_ERR_STATE, "model not finalized");
+    if (on && !fused_available_)
+        return hm_set_error(ctx_, HM_ERR_INVALID, "whole-step decode is not available for this model (bf16 weights and a served shape are needed)");
+    return plan_->set_whole_step(on);
+}
+
+int HfModel::whole_step_status() {
+    if (!fused_available_) return HM_OK;
+    return decode_fused_check(ctx_, scratch_->fused_ctl.as<uint32_t>());
+}
+
 int HfModel::check_ids(const int64_t *ids, int n, std::vector<int32_t> &out) {
     out.resize(n);
     for (int i = 0; i < n; i++) {
@@ -1276,7 +1391,7 @@ int HfModel::run_kv(const int64_t *h_ids, int n_ids, float *h_logits) {
             if (rc != HM_OK) return rc;
         }
     }
-    return hm_sync(ctx_);
+    return finish_sync();
 }
 
 // ── prefill pass ─────────────────────────────────────────────────────────────
@@ -1562,7 +1677,8 @@ int HfModel::generate_greedy(const int64_t *h_prompt, int n_prompt, int n_new, i
     for (int i = 0; i < steps; i++)
         if ((rc = plan_->run_kv(inputs, weight_bufs_, max_seq_len_)) != HM_OK) return rc;
     // the pick after prompt token n_prompt-1 is generated token 0
-    return hm_download(ctx_, h_tokens, plan_->out_tokens() + (n_prompt - 1), (size_t)n_new * 4);
+    rc = hm_download(ctx_, h_tokens, plan_->out_tokens() + (n_prompt - 1), (size_t)n_new * 4);
+    return rc == HM_OK ? finish_sync() : rc;
 }
 
 // sampling.hip
@@ -1671,7 +1787,7 @@ int HfModel::bench_decode(int64_t first_id, int n_steps, float *ms_out, int32_t 
     (void)hipEventDestroy(e1);
     if (rc != HM_OK) return rc;
     if (h_tokens) rc = hm_download(ctx_, h_tokens, plan_->out_tokens(), (size_t)n_steps * 4);
-    return rc;
+    return rc == HM_OK ? finish_sync() : rc;
 }
 
 int HfModel::time_kernels(int rounds, std::vector<StepProfile> &out) {

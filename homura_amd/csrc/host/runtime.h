@@ -154,13 +154,18 @@ struct DeviceLaunch {
     double bytes_per_kv_row = 0;      // plus this much per cached row (attention)
     bool moves_cursor = false;        // advances the DecodeState (must run exactly once per step)
     int hip_launches = 1;             // HIP kernels this entry enqueues
+    // A plan may carry two ways through the layers: one launch per projection, or one launch for the
+    // whole step. Entries of the way that is switched off are skipped.
+    enum class Mode { Always, PerKernel, WholeStep };
+    Mode mode = Mode::Always;
     std::function<int(const StepContext &)> fn;
 };
 struct CompiledKernel {
     std::string ops_label;  // "Embed", "QKV+QKNorm+RoPE", "Attn", "MLP", "LMHead", "QuantMM[q]", ...
     std::vector<DeviceLaunch> launches;
-    int launch(const StepContext &sc) const {
+    int launch(const StepContext &sc, bool whole_step) const {
         for (const auto &l : launches) {
+            if (l.mode == (whole_step ? DeviceLaunch::Mode::PerKernel : DeviceLaunch::Mode::WholeStep)) continue;
             int rc = l.fn(sc);
             if (rc != HM_OK) return rc;
         }
@@ -219,6 +224,15 @@ class ExecutionPlan {
     // Graph replay of the step (captured lazily on first use; arguments never change).
     int enable_graph(bool on);
     bool graph_enabled() const { return use_graph_; }
+    // Take the whole-step launch (when the plan has one) instead of the per-projection launches.
+    int set_whole_step(bool on);
+    bool whole_step() const { return whole_step_; }
+    bool skips(const DeviceLaunch &l) const {
+        return l.mode == (whole_step_ ? DeviceLaunch::Mode::PerKernel : DeviceLaunch::Mode::WholeStep);
+    }
+    // Called before a step is enqueued or captured, with the KV cache in place (device tables that
+    // depend on the cache's addresses are refreshed here, outside any capture).
+    void set_pre_run(std::function<int()> fn) { pre_run_ = std::move(fn); }
 
     // Per-kernel timing of one step (HOMURA_PROFILE analogue, reference src/runtime.rs:1849-1873):
     // HIP events around every device launch of a real decode step.
@@ -264,6 +278,8 @@ class ExecutionPlan {
     int out_cap_ = 0;
     bool prepared_ = false;
     bool use_graph_ = false;
+    bool whole_step_ = false;
+    std::function<int()> pre_run_;
     hipGraph_t graph_ = nullptr;
     hipGraphExec_t graph_exec_ = nullptr;
 };

@@ -292,6 +292,10 @@ int ExecutionPlan::init_kv_cache(const float *const *h_kv, int seq_len, int max_
             (void)hipGraphExecDestroy(graph_exec_);
             graph_exec_ = nullptr;
         }
+        if (graph_) {
+            (void)hipGraphDestroy(graph_);
+            graph_ = nullptr;
+        }
     }
     int rc = ensure_kv_cache(max_seq_len);
     if (rc != HM_OK) return rc;
@@ -337,7 +341,8 @@ int ExecutionPlan::launches_per_step() const {
     int n = 0;
     for (const auto &st : steps_)
         if (st.native_op.kind == NativeOpKind::None)
-            for (const auto &l : kernels_[st.kernel_idx].launches) n += l.hip_launches;
+            for (const auto &l : kernels_[st.kernel_idx].launches)
+                if (!skips(l)) n += l.hip_launches;
     return n;
 }
 
@@ -366,11 +371,12 @@ int ExecutionPlan::run_steps(std::vector<StepProfile> *profile) {
         const CompiledKernel &k = kernels_[step.kernel_idx];
         StepContext sc{ctx_, this, pool_, step};
         if (!profile) {
-            int rc = k.launch(sc);
+            int rc = k.launch(sc, whole_step_);
             if (rc != HM_OK) return rc;
             continue;
         }
         for (const DeviceLaunch &l : k.launches) {
+            if (skips(l)) continue;
             HM_HIP(ctx_, hipEventRecord(e0, ctx_->stream));
             int rc = l.fn(sc);
             if (rc != HM_OK) return rc;
@@ -406,12 +412,13 @@ int ExecutionPlan::time_kernels(const std::vector<Buffer *> &inputs, std::vector
     if (kv_cache_->current_len() + 1 > kv_cache_->max_len())
         return hm_set_error(ctx_, HM_ERR_STATE, "KV cache full (%d + 1 > %d)", kv_cache_->current_len(), kv_cache_->max_len());
     if ((rc = bind(inputs, weights)) != HM_OK) return rc;
+    if (pre_run_ && (rc = pre_run_()) != HM_OK) return rc;
     const int kv_rows = kv_cache_->current_len() + 1;
     std::vector<std::string> names;
     for (const auto &st : steps_) {
         if (st.native_op.kind != NativeOpKind::None) continue;
         for (const auto &l : kernels_[st.kernel_idx].launches)
-            if (!l.moves_cursor && std::find(names.begin(), names.end(), l.name) == names.end())
+            if (!l.moves_cursor && !skips(l) && std::find(names.begin(), names.end(), l.name) == names.end())
                 names.push_back(l.name);
     }
     hipEvent_t e0, e1;
@@ -425,7 +432,7 @@ int ExecutionPlan::time_kernels(const std::vector<Buffer *> &inputs, std::vector
                 if (st.native_op.kind != NativeOpKind::None) continue;
                 StepContext sc{ctx_, this, pool_, st};
                 for (const auto &l : kernels_[st.kernel_idx].launches) {
-                    if (l.name != name) continue;
+                    if (l.name != name || skips(l)) continue;
                     if ((rc = l.fn(sc)) != HM_OK) return rc;
                     if (r >= 0) {
                         p.launches++;
@@ -449,6 +456,21 @@ int ExecutionPlan::enable_graph(bool on) {
     return HM_OK;
 }
 
+int ExecutionPlan::set_whole_step(bool on) {
+    if (on == whole_step_) return HM_OK;
+    whole_step_ = on;
+    if (graph_exec_) {  // the captured step took the other way through the layers
+        HM_HIP(ctx_, hipStreamSynchronize(ctx_->stream));
+        (void)hipGraphExecDestroy(graph_exec_);
+        graph_exec_ = nullptr;
+    }
+    if (graph_) {
+        (void)hipGraphDestroy(graph_);
+        graph_ = nullptr;
+    }
+    return HM_OK;
+}
+
 int ExecutionPlan::run_kv(const std::vector<Buffer *> &inputs, std::vector<Buffer> &weights,
                           int max_seq_len) {
     if (!prepared_) return hm_set_error(ctx_, HM_ERR_STATE, "plan not prepared");
@@ -456,8 +478,13 @@ int ExecutionPlan::run_kv(const std::vector<Buffer *> &inputs, std::vector<Buffe
     if (rc != HM_OK) return rc;
     if ((rc = kv_cache_->note_appended(1)) != HM_OK) return rc;  // "KV cache full"
     if ((rc = bind(inputs, weights)) != HM_OK) return rc;
+    if (pre_run_ && (rc = pre_run_()) != HM_OK) return rc;
     if (use_graph_) {
         if (!graph_exec_) {
+            if (graph_) {
+                (void)hipGraphDestroy(graph_);
+                graph_ = nullptr;
+            }
             HM_HIP(ctx_, hipStreamBeginCapture(ctx_->stream, hipStreamCaptureModeRelaxed));
             rc = run_steps(nullptr);
             hipGraph_t g = nullptr;
@@ -487,6 +514,7 @@ int ExecutionPlan::profile_step(const std::vector<Buffer *> &inputs, std::vector
     if (rc != HM_OK) return rc;
     if ((rc = kv_cache_->note_appended(1)) != HM_OK) return rc;
     if ((rc = bind(inputs, weights)) != HM_OK) return rc;
+    if (pre_run_ && (rc = pre_run_()) != HM_OK) return rc;
     rc = run_steps(&out);
     if (rc != HM_OK) return rc;
     kv_cache_->advance_by(kv_cache_->new_tokens());

@@ -411,6 +411,21 @@ class HfModel:
         """Replay each decode step from a captured HIP graph instead of launching kernel by kernel."""
         self._check(self.lib.hm_model_set_graph(self.h, int(on)))
 
+    def set_whole_step(self, on: bool):
+        """One launch for the embedding row and all layers of a decode step (bf16 models of a served
+        shape) instead of one launch per projection."""
+        self._check(self.lib.hm_model_set_whole_step(self.h, int(on)))
+
+    def whole_step(self) -> bool:
+        return bool(self._check(self.lib.hm_model_whole_step(self.h)))
+
+    def whole_step_available(self) -> bool:
+        return bool(self._check(self.lib.hm_model_whole_step_available(self.h)))
+
+    def whole_step_status(self):
+        """Raises if a whole-step launch left an error behind (an exchange that timed out)."""
+        self._check(self.lib.hm_model_whole_step_status(self.h))
+
     def reset_kv_cache(self):
         self._check(self.lib.hm_model_reset_kv_cache(self.h))
 

@@ -320,6 +320,18 @@ int hm_model_kv_cache_len(hm_model *m);    /* src/runtime.rs:1948-1950 */
  * No counterpart in the reference (its plan is a host loop over dlsym'ed functions). */
 int hm_model_set_graph(hm_model *m, int on);
 
+/* One launch for a whole decode step's embedding row and decoder layers (on != 0) instead of one
+ * launch per projection; the reference dispatches 1 + 3 * layers + 1 kernels per step
+ * (src/hf/emitter.rs:1016-1021). Served for bf16 models whose shape has a kernel instance
+ * (hm_model_whole_step_available) and whose cache fits it; on by default then. Results agree with the
+ * per-projection path to f32 summation order. hm_model_whole_step_status returns HM_OK, or the error
+ * left behind by a step whose workgroups stopped waiting for one another (bounded waits; the
+ * outputs of such a step are not valid). */
+int hm_model_set_whole_step(hm_model *m, int on);
+int hm_model_whole_step(hm_model *m);
+int hm_model_whole_step_available(hm_model *m);
+int hm_model_whole_step_status(hm_model *m);
+
 /* HfModel::run_kv (src/hf/model.rs:198-218) -> ExecutionPlan::run_kv
  * (src/runtime.rs:1580-1892): n_ids new tokens on top of the cache; h_logits receives
  * [n_ids][vocab] f32 (may be NULL to skip the download). Advances the cache by n_ids. */
