@@ -55,9 +55,19 @@ struct Geo {
     static constexpr int FPW = QD / NWG;                       // folded attention outputs per workgroup
     static constexpr int PART = G * HD + 2 * G;                // one split's partial: o[G][HD], (m, l)[G]
     static constexpr int NJ = HIDDEN / CT;                     // hidden elements per communicating thread
-    // exchange area of one layer parity, in 8-byte slots
-    static constexpr int XH = 0, XO = HIDDEN, XQ = 2 * HIDDEN, XA = XQ + NQKV, XC = XA + QD, XP = XC + INTER;
-    static constexpr int PAR_SLOTS = (XP + KVH * SPH * PART + 31) / 32 * 32;
+    static constexpr int NXCD = 8, NPX = NWG / NXCD;           // accelerator dies (one L2 each), workgroups per die
+    static constexpr int GROWS = (G + 2) * HD;                 // q|k|v rows of one KV head
+    // A KV head's workgroups are wg % KVH == head; with workgroups dealt round-robin to the dies they all
+    // share one L2 when KVH is a multiple of the die count.
+    static constexpr bool GROUP_ON_XCD = KVH % NXCD == 0;
+    // Exchange area of one layer parity, in 8-byte slots: the vectors every workgroup reads (hidden
+    // increments XH / XO, folded attention XA, SiLU*up XC), one relay copy of those per die, and per KV
+    // head the raw q|k|v rows (LQ) and the attention partials of its splits (LP).
+    static constexpr int XH = 0, XO = HIDDEN, XA = 2 * HIDDEN, XC = XA + QD, GLOB_SLOTS = XC + INTER;
+    static constexpr int RELAY0 = GLOB_SLOTS, LQ0 = RELAY0 + NXCD * GLOB_SLOTS, LP0 = LQ0 + KVH * GROWS;
+    static constexpr int PAR_SLOTS = (LP0 + KVH * SPH * PART + 31) / 32 * 32;
+    static constexpr int CHK0 = 2 * PAR_SLOTS;                 // placement check: one slot per workgroup
+    static constexpr int ALL_SLOTS = CHK0 + NWG;
     static constexpr int PUB = (PART > RQ ? PART : RQ) > RG ? (PART > RQ ? PART : RQ) : RG;
     static_assert(HIDDEN % 512 == 0 && QD % 512 == 0 && INTER % 512 == 0, "rows are cut into 512-wide chunks");
     static_assert(NQKV % (NWG * NCW) == 0 && HIDDEN % (NWG * NCW) == 0 && (2 * INTER) % (NWG * NCW) == 0,
@@ -67,6 +77,15 @@ struct Geo {
     static_assert(HD == 64 || HD == 128, "head_dim 64 or 128");
     static_assert(QD % NWG == 0 && FPW % 2 == 0 && HD % FPW == 0, "a workgroup folds a run inside one head");
     static_assert(RQ <= CT && RO <= CT && APW <= CT, "one publishing thread per value");
+    static_assert(GROWS % SPH == 0 && GROWS / SPH == RQ && HD % RQW == 0, "a wavefront's q|k|v rows lie in one of q, k, v");
+    static_assert(NWG % NXCD == 0 && (HIDDEN / 2) % NPX == 0 && (QD / 2) % NPX == 0 && (INTER / 2) % NPX == 0 &&
+                      INTER / 2 / NPX <= WAVE && QD / 2 / NPX <= WAVE && HIDDEN / 2 / NPX <= WAVE,
+                  "one wavefront relays a die's share of a vector");
+    static_assert(NWG % 2 == 0 && NWG / 2 <= 2 * WAVE, "two placement-check units per lane");
+    // row of the stacked q|k|v matrix for local row lr of KV head kh
+    __device__ static int qkv_row(int kh, int lr) {
+        return lr < G * HD ? kh * G * HD + lr : (lr < (G + 1) * HD ? QD + kh * HD + (lr - G * HD) : QD + KVD + kh * HD + (lr - (G + 1) * HD));
+    }
 };
 
 template <class GE>
@@ -83,7 +102,6 @@ struct Lds {
     float pub[GE::PUB];                   // results of the phase, read by the publishing threads
     float red[4];
     float bias[GE::RQ];
-    int arrive;
     FusedLayerPtrs lp[MAX_LAYERS];        // the layer table (compute wavefronts must not wait on global loads)
 };
 
@@ -102,18 +120,32 @@ __device__ __forceinline__ void wg_barrier() {
     asm volatile("" ::: "memory");
 }
 
-__device__ __forceinline__ void st_slot(unsigned char *area, int slot, float v, uint32_t tag) {
-    __hip_atomic_store(reinterpret_cast<uint64_t *>(area) + slot, ((uint64_t)tag << 32) | __float_as_uint(v),
-                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+// Exchange primitives. Every poll is a device-scope load: it never reads the CU's L1, and it sees what its
+// die's L2 holds. "Far" stores cross dies: device scope, written through to memory. "Near" stores are
+// plain stores, which stop in the die's L2 (0.27 us from store to a poll on the same die, against 0.6 us
+// through memory); they are only used between workgroups that the placement check found on one die, and
+// never on memory that far stores touch. (Non-temporal loads also skip the L1 most of the time, but a
+// line they left there can be served again later: a poll built on them can spin on a stale copy.)
+__device__ __forceinline__ void st_slot(unsigned char *area, int slot, float v, uint32_t tag, bool near) {
+    unsigned char *p = area + (size_t)slot * 8;
+    const uint64_t w = ((uint64_t)tag << 32) | __float_as_uint(v);
+    // compiler-issued stores: a store written in inline asm is invisible to the hazard recognizer (a store
+    // of more than 8 bytes must not be followed at once by a write to its data registers)
+    if (near)
+        *reinterpret_cast<uint64_t *>(p) = w;
+    else
+        __hip_atomic_store(reinterpret_cast<uint64_t *>(p), w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    asm volatile("" ::: "memory");
 }
 
 struct PollState {
     uint32_t *ctl;
     bool failed;
+    uint32_t where;  // what is being waited for: phase | layer << 4 | workgroup << 12, stored on a timeout
 };
 
-// Device-scope 16-byte loads of `NU` units {v0, tag, v1, tag}, all issued before one wait, repeated
-// until every wanted unit carries `tag` in both halves. Units with on[u] false are not waited for.
+// 16-byte loads of `NU` units {v0, tag, v1, tag}, all issued before one wait, repeated until every
+// wanted unit carries `tag` in both halves. Units with on[u] false are not waited for.
 template <int NU>
 __device__ __forceinline__ void poll_units(PollState &ps, const unsigned char *area, const int (&unit)[NU],
                                            const bool (&on)[NU], uint32_t tag, u32x4 (&w)[NU]) {
@@ -139,7 +171,7 @@ __device__ __forceinline__ void poll_units(PollState &ps, const unsigned char *a
         for (int u = 0; u < NU; u++) ok = ok && (!on[u] || (w[u].y == tag && w[u].w == tag));
         if (ok) return;
         if (++spins > SPIN_MAX) {
-            __hip_atomic_store(ps.ctl + 1, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            atomicCAS(ps.ctl + 1, 0u, 0x80000000u | ps.where);  // the first timeout is the one reported
             ps.failed = true;
             return;
         }
@@ -188,25 +220,122 @@ __device__ __forceinline__ float row_sum(float v) {
 
 // One wavefront: optional RMSNorm over hd, then x*cos + rotate_half(x)*sin (the arithmetic of
 // attention.hip's fused prologue; reference src/hf/emitter.rs:629-644). Lane i < hd/2 owns the pair
-// (i, i + hd/2).
+// (i, i + hd/2); the lane's table entries and norm weights are handed in (loaded before the wait for
+// the row, so no global load sits between the row's arrival and the result).
+struct RopeLane {
+    float c_lo, c_hi, s_lo, s_hi;
+};
 template <int HD>
-__device__ __forceinline__ void norm_rope(const float *src, const float *__restrict__ nwp,
-                                          const float *__restrict__ c, const float *__restrict__ sn, float eps,
-                                          int lane, float &o_lo, float &o_hi) {
+__device__ __forceinline__ void norm_rope(const float *src, bool normed, float w_lo, float w_hi, const RopeLane &t,
+                                          float eps, int lane, float &o_lo, float &o_hi) {
     constexpr int HALF = HD / 2;
     const bool on = lane < HALF;
     float lo = on ? src[lane] : 0.f, hi = on ? src[lane + HALF] : 0.f;
-    const float c_lo = on ? c[lane] : 0.f, c_hi = on ? c[lane + HALF] : 0.f;
-    const float s_lo = on ? sn[lane] : 0.f, s_hi = on ? sn[lane + HALF] : 0.f;
-    const float w_lo = (on && nwp) ? ldf_global(nwp + lane) : 1.f, w_hi = (on && nwp) ? ldf_global(nwp + lane + HALF) : 1.f;
-    if (nwp) {
+    if (normed) {
         const float ss = wave_sum(lo * lo + hi * hi);
         const float inv = 1.0f / sqrtf(ss / (float)HD + eps);
         lo = (lo * inv) * w_lo;
         hi = (hi * inv) * w_hi;
     }
-    o_lo = lo * c_lo + (-hi) * s_lo;
-    o_hi = hi * c_hi + lo * s_hi;
+    o_lo = lo * t.c_lo + (-hi) * t.s_lo;
+    o_hi = hi * t.c_hi + lo * t.s_hi;
+}
+
+// Dot products of R rows x C chunks kept as R * C independent chains (one wavefront per SIMD: the
+// chains are what hides the latency of a dependent multiply-add), the k loop outermost.
+template <int R, int C>
+__device__ __forceinline__ void dots_from(const u32x4 (&w)[R][C], const float (&xv)[C][8], float (&acc)[R][C]) {
+#pragma unroll
+    for (int r = 0; r < R; r++)
+#pragma unroll
+        for (int c = 0; c < C; c++) acc[r][c] = 0.f;
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+#pragma unroll
+        for (int r = 0; r < R; r++)
+#pragma unroll
+            for (int c = 0; c < C; c++) {
+                const uint32_t d = e == 0 ? w[r][c].x : (e == 1 ? w[r][c].y : (e == 2 ? w[r][c].z : w[r][c].w));
+                acc[r][c] = fmaf(bf16_lo(d), xv[c][2 * e], acc[r][c]);
+            }
+#pragma unroll
+        for (int r = 0; r < R; r++)
+#pragma unroll
+            for (int c = 0; c < C; c++) {
+                const uint32_t d = e == 0 ? w[r][c].x : (e == 1 ? w[r][c].y : (e == 2 ? w[r][c].z : w[r][c].w));
+                acc[r][c] = fmaf(bf16_hi(d), xv[c][2 * e + 1], acc[r][c]);
+            }
+    }
+}
+
+// rows against (h * inv) * norm_w read from LDS (RMSNorm: reference src/graph_builder/emit_linalg.rs:7-26)
+template <int R, int C>
+__device__ __forceinline__ void normed_dots(const u32x4 (&w)[R][C], const float *hx, const float *nw, float inv,
+                                            int lane, float (&acc)[R][C]) {
+    float xv[C][8];
+#pragma unroll
+    for (int c = 0; c < C; c++) {
+        float hv[8], wv[8];
+        lds_x8(hx, (c * WAVE + lane) * 8, hv);
+        lds_x8(nw, (c * WAVE + lane) * 8, wv);
+#pragma unroll
+        for (int e = 0; e < 8; e++) xv[c][e] = (hv[e] * inv) * wv[e];
+    }
+    dots_from<R, C>(w, xv, acc);
+}
+
+template <int R, int C>
+__device__ __forceinline__ void plain_dots(const u32x4 (&w)[R][C], const float *x, int lane, float (&acc)[R][C]) {
+    float xv[C][8];
+#pragma unroll
+    for (int c = 0; c < C; c++) lds_x8(x, (c * WAVE + lane) * 8, xv[c]);
+    dots_from<R, C>(w, xv, acc);
+}
+
+template <int C>
+__device__ __forceinline__ float chunk_total(const float (&a)[C]) {
+    float t = a[0];
+#pragma unroll
+    for (int c = 1; c < C; c++) t += a[c];
+    return t;
+}
+
+// wave_sum / wave_max of N values with the N chains stepping side by side; every lane gets the totals
+template <int N>
+__device__ __forceinline__ void wave_sum_n(float (&v)[N]) {
+#pragma unroll
+    for (int i = 0; i < N; i++) v[i] += dpp_move<0xB1, 0xF>(v[i], 0.f);
+#pragma unroll
+    for (int i = 0; i < N; i++) v[i] += dpp_move<0x4E, 0xF>(v[i], 0.f);
+#pragma unroll
+    for (int i = 0; i < N; i++) v[i] += dpp_move<0x141, 0xF>(v[i], 0.f);
+#pragma unroll
+    for (int i = 0; i < N; i++) v[i] += dpp_move<0x140, 0xF>(v[i], 0.f);
+#pragma unroll
+    for (int i = 0; i < N; i++) v[i] += dpp_move<0x142, 0xA>(v[i], 0.f);
+#pragma unroll
+    for (int i = 0; i < N; i++) v[i] += dpp_move<0x143, 0xC>(v[i], 0.f);
+#pragma unroll
+    for (int i = 0; i < N; i++) v[i] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v[i]), 63));
+}
+
+template <int N>
+__device__ __forceinline__ void wave_max_n(float (&v)[N]) {
+    const float ninf = -__builtin_huge_valf();
+#pragma unroll
+    for (int i = 0; i < N; i++) v[i] = fmaxf(v[i], dpp_move<0xB1, 0xF>(v[i], ninf));
+#pragma unroll
+    for (int i = 0; i < N; i++) v[i] = fmaxf(v[i], dpp_move<0x4E, 0xF>(v[i], ninf));
+#pragma unroll
+    for (int i = 0; i < N; i++) v[i] = fmaxf(v[i], dpp_move<0x141, 0xF>(v[i], ninf));
+#pragma unroll
+    for (int i = 0; i < N; i++) v[i] = fmaxf(v[i], dpp_move<0x140, 0xF>(v[i], ninf));
+#pragma unroll
+    for (int i = 0; i < N; i++) v[i] = fmaxf(v[i], dpp_move<0x142, 0xA>(v[i], ninf));
+#pragma unroll
+    for (int i = 0; i < N; i++) v[i] = fmaxf(v[i], dpp_move<0x143, 0xC>(v[i], ninf));
+#pragma unroll
+    for (int i = 0; i < N; i++) v[i] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v[i]), 63));
 }
 
 // The attention split of a workgroup for a cache of kv_len rows (the new row included).
@@ -218,8 +347,8 @@ struct Split {
         const int kv_len = pos + 1;
         const int chunk = (kv_len + GE::SPH - 1) / GE::SPH;
         nsl = (kv_len + chunk - 1) / chunk;
-        kh = wg / GE::SPH;
-        split = wg % GE::SPH;
+        kh = wg % GE::KVH;
+        split = wg / GE::KVH;
         n0 = split * chunk;
         cnt = min(kv_len, n0 + chunk) - n0;
         if (cnt < 0) cnt = 0;
@@ -248,16 +377,21 @@ __device__ __forceinline__ void compute_role(const FusedDecodeArgs &a, Lds<GE> &
     const int L = a.n_layers;
     Slice<GE> s;
 
-    auto load_wq = [&](const FusedLayerPtrs &lp) {
+    // Requests are spread over the step in small batches (rows [r0, r1) of a slice at a time): a batch that
+    // overfills the CU's memory pipeline blocks the wavefront that issues it, and a burst from all
+    // CUs at once delays the polls of the communication wavefronts behind it.
+    auto load_wq = [&](const FusedLayerPtrs &lp, int r0, int r1) {
 #pragma unroll
         for (int r = 0; r < GE::RQW; r++)
 #pragma unroll
             for (int c = 0; c < GE::CH; c++)
-                s.wq[r][c] = ld128_global_stream(lp.wqkv + (size_t)(wg * GE::RQ + cw * GE::RQW + r) * GE::HIDDEN + (c * WAVE + lane) * 8);
+                if (r >= r0 && r < r1)
+                    s.wq[r][c] = ld128_global_stream(lp.wqkv + (size_t)GE::qkv_row(sp.kh, sp.split * GE::RQ + cw * GE::RQW + r) * GE::HIDDEN + (c * WAVE + lane) * 8);
     };
-    auto load_kv = [&](const FusedLayerPtrs &lp) {
+    auto load_kv = [&](const FusedLayerPtrs &lp, int i0, int i1) {
 #pragma unroll
         for (int i = 0; i < NR; i++) {
+            if (i < i0 || i >= i1) continue;
             const int rl = (i * NCW + cw) * RPI + sub;
             const int row = rl < sp.cached ? sp.n0 + rl : 0;  // rows outside the split re-read a valid row
             const size_t off = ((size_t)sp.kh * a.max_len + row) * HD + dl * 8;
@@ -272,12 +406,13 @@ __device__ __forceinline__ void compute_role(const FusedDecodeArgs &a, Lds<GE> &
             for (int c = 0; c < GE::CO; c++)
                 s.wo[r][c] = ld128_global_stream(lp.wo + (size_t)(wg * GE::RO + cw * GE::ROW + r) * GE::QD + (c * WAVE + lane) * 8);
     };
-    auto load_wg = [&](const FusedLayerPtrs &lp) {
+    auto load_wg = [&](const FusedLayerPtrs &lp, int r0, int r1) {
 #pragma unroll
         for (int r = 0; r < GE::RGW; r++)
 #pragma unroll
             for (int c = 0; c < GE::CH; c++)
-                s.wg[r][c] = ld128_global_stream(lp.wgu + (size_t)(wg * GE::RG + cw * GE::RGW + r) * GE::HIDDEN + (c * WAVE + lane) * 8);
+                if (r >= r0 && r < r1)
+                    s.wg[r][c] = ld128_global_stream(lp.wgu + (size_t)(wg * GE::RG + cw * GE::RGW + r) * GE::HIDDEN + (c * WAVE + lane) * 8);
     };
     auto load_wd = [&](const FusedLayerPtrs &lp) {
 #pragma unroll
@@ -287,252 +422,214 @@ __device__ __forceinline__ void compute_role(const FusedDecodeArgs &a, Lds<GE> &
                 s.wd[r][c] = ld128_global_stream(lp.wd + (size_t)(wg * GE::RO + cw * GE::ROW + r) * GE::INTER + (c * WAVE + lane) * 8);
     };
 
+    constexpr int KV_CUT = NR / 2, WG_CUT = 2 * GE::RGW / 3;
     {
+        // the first layer's slice, in the order the loop re-requests it (the rest follows inside the loop)
         const FusedLayerPtrs lp = sm.lp[0];
-        load_wq(lp);
-        load_kv(lp);
+        load_wq(lp, 0, GE::RQW);
+        load_kv(lp, 0, NR);
         load_wo(lp);
-        load_wg(lp);
-        load_wd(lp);
+        load_wg(lp, 0, WG_CUT);
     }
 
     for (int l = 0; l < L; l++) {
-        // The slice of the next layer replaces each phase's registers as soon as the phase is over. After
-        // the last layer the first layer's slice is requested again and never used: the request keeps the
+        // The slice of the next layer replaces each phase's registers once the phase is over. After the
+        // last layer the first layer's slice is requested again and never used: the requests keep the
         // number of loads in flight the same in every iteration, which the wait counts rely on.
         const FusedLayerPtrs nx = sm.lp[l + 1 < L ? l + 1 : 0];
         const bool has_bias = sm.lp[l].qkv_bias != nullptr;
 
         // ── Q|K|V rows (RMSNorm applied on the way in; reference src/hf/emitter.rs:560-619) ──
         wg_barrier();
+        // Requests go out at the start of a phase, never right before the communicating wavefronts poll:
+        // the CU's vector memory pipeline returns data in order, so a poll issued behind a weight request
+        // waits for HBM. Here: this layer's down rows and last gate|up rows (registers last read one layer ago).
+        load_wd(sm.lp[l]);
+        load_wg(sm.lp[l], WG_CUT, GE::RGW);
         {
             const float tot = ((sm.red[0] + sm.red[1]) + sm.red[2]) + sm.red[3];
             const float inv = 1.0f / sqrtf(tot / (float)GE::HIDDEN + a.eps);
-            float acc[GE::RQW];
+            float acc[GE::RQW][GE::CH];
+            normed_dots<GE::RQW, GE::CH>(s.wq, sm.hx, sm.nw, inv, lane, acc);
+            float v[GE::RQW];
 #pragma unroll
-            for (int r = 0; r < GE::RQW; r++) acc[r] = 0.f;
+            for (int r = 0; r < GE::RQW; r++) v[r] = chunk_total<GE::CH>(acc[r]);
+            wave_sum_n<GE::RQW>(v);
+            if (has_bias) {
 #pragma unroll
-            for (int c = 0; c < GE::CH; c++) {
-                const int k = (c * WAVE + lane) * 8;
-                float hv[8], wv[8], xv[8];
-                lds_x8(sm.hx, k, hv);
-                lds_x8(sm.nw, k, wv);
-#pragma unroll
-                for (int e = 0; e < 8; e++) xv[e] = (hv[e] * inv) * wv[e];
-#pragma unroll
-                for (int r = 0; r < GE::RQW; r++) acc[r] = dot8f(s.wq[r][c], xv, acc[r]);
+                for (int r = 0; r < GE::RQW; r++) v[r] = v[r] + sm.bias[cw * GE::RQW + r];
             }
+            float mine = 0.f;
 #pragma unroll
-            for (int r = 0; r < GE::RQW; r++) {
-                float v = wave_sum(acc[r]);
-                if (has_bias) v = v + sm.bias[cw * GE::RQW + r];
-                if (lane == 0) sm.pub[cw * GE::RQW + r] = v;
-            }
-            load_wq(nx);
+            for (int r = 0; r < GE::RQW; r++) mine = lane == r ? v[r] : mine;
+            if (lane < GE::RQW) sm.pub[cw * GE::RQW + lane] = mine;
         }
         wg_barrier();
 
-        // ── attention over this workgroup's split of the cache (reference src/hf/emitter.rs:709-731) ──
+        // ── attention over this workgroup's split of the cache (reference src/hf/emitter.rs:709-731).
+        //    Every wavefront leaves the (max, sum, P.V) of its own rows in LDS; the publishing threads
+        //    merge the four. ──
         wg_barrier();
+        load_wq(nx, 0, GE::RQW);
         if (sp.split < sp.nsl) {
             float qv[G][8];
 #pragma unroll
             for (int g = 0; g < G; g++) lds_x8(sm.qs[g], dl * 8, qv[g]);
-            float sc[G][NR];
-            bool live[NR];
+            const bool with_new = sp.owner && cw == 0;  // the new row rides with wavefront 0 of the last split
+            float kf[NR + 1][8];
 #pragma unroll
-            for (int i = 0; i < NR; i++) {
-                const int rl = (i * NCW + cw) * RPI + sub;
-                live[i] = rl < sp.cached;
-                float kf[8];
-                unpack8f(s.kr[i], kf);
+            for (int i = 0; i < NR; i++) unpack8f(s.kr[i], kf[i]);
+            lds_x8(sm.knew, dl * 8, kf[NR]);
+            float sc[G][NR + 1];
+#pragma unroll
+            for (int g = 0; g < G; g++)
+#pragma unroll
+                for (int i = 0; i <= NR; i++) sc[g][i] = 0.f;
+#pragma unroll
+            for (int e = 0; e < 8; e++)
+#pragma unroll
+                for (int g = 0; g < G; g++)
+#pragma unroll
+                    for (int i = 0; i <= NR; i++) sc[g][i] = fmaf(kf[i][e], qv[g][e], sc[g][i]);
+            // sums over the lanes of a row, all (head, row) chains side by side
+#pragma unroll
+            for (int g = 0; g < G; g++)
+#pragma unroll
+                for (int i = 0; i <= NR; i++) sc[g][i] += dpp_move<0xB1, 0xF>(sc[g][i], 0.f);
+#pragma unroll
+            for (int g = 0; g < G; g++)
+#pragma unroll
+                for (int i = 0; i <= NR; i++) sc[g][i] += dpp_move<0x4E, 0xF>(sc[g][i], 0.f);
+#pragma unroll
+            for (int g = 0; g < G; g++)
+#pragma unroll
+                for (int i = 0; i <= NR; i++) sc[g][i] += dpp_move<0x141, 0xF>(sc[g][i], 0.f);
+            if (LPR == 16) {
+#pragma unroll
+                for (int g = 0; g < G; g++)
+#pragma unroll
+                    for (int i = 0; i <= NR; i++) sc[g][i] += dpp_move<0x140, 0xF>(sc[g][i], 0.f);
+            }
+            bool live[NR + 1];
+#pragma unroll
+            for (int i = 0; i < NR; i++) live[i] = (i * NCW + cw) * RPI + sub < sp.cached;
+            live[NR] = with_new;
+            float m[G];
+#pragma unroll
+            for (int g = 0; g < G; g++) {
+                m[g] = -INFINITY;
+#pragma unroll
+                for (int i = 0; i <= NR; i++) {
+                    sc[g][i] = live[i] ? sc[g][i] * a.scale : -INFINITY;
+                    m[g] = fmaxf(m[g], sc[g][i]);
+                }
+            }
+            wave_max_n<G>(m);
+            // softmax terms against the wavefront's own maximum (max, exp, sum:
+            // reference emit_softmax, src/graph_builder/emit_linalg.rs:509-528)
+            float pr[G][NR + 1], lsum[G];
+#pragma unroll
+            for (int g = 0; g < G; g++) {
+                lsum[g] = 0.f;
+#pragma unroll
+                for (int i = 0; i <= NR; i++) {
+                    pr[g][i] = live[i] ? __expf(sc[g][i] - m[g]) : 0.f;
+                    // a cache row is counted by the first of its lanes, the new row by lane 0
+                    if (i < NR ? dl == 0 : lane == 0) lsum[g] += pr[g][i];
+                }
+            }
+            wave_sum_n<G>(lsum);
+            if (lane < G) {
+                float mm = 0.f, ll = 0.f;
 #pragma unroll
                 for (int g = 0; g < G; g++) {
-                    float p = 0.f;
-#pragma unroll
-                    for (int e = 0; e < 8; e++) p = fmaf(kf[e], qv[g][e], p);
-                    p = row_sum<LPR>(p);
-                    sc[g][i] = live[i] ? p * a.scale : -INFINITY;
+                    mm = lane == g ? m[g] : mm;
+                    ll = lane == g ? lsum[g] : ll;
                 }
+                sm.wstat[cw][lane][0] = mm;
+                sm.wstat[cw][lane][1] = ll;
             }
-            const bool with_new = sp.owner && cw == 0;  // the new row rides with wavefront 0 of the last split
-            float sc_new[G];
+            float vf[NR + 1][8];
 #pragma unroll
-            for (int g = 0; g < G; g++) {
-                float kn[8];
-                lds_x8(sm.knew, dl * 8, kn);
-                float p = 0.f;
-#pragma unroll
-                for (int e = 0; e < 8; e++) p = fmaf(kn[e], qv[g][e], p);
-                p = row_sum<LPR>(p);
-                sc_new[g] = with_new ? p * a.scale : -INFINITY;
-            }
+            for (int i = 0; i < NR; i++) unpack8f(s.vr[i], vf[i]);
+            lds_x8(sm.vnew, dl * 8, vf[NR]);
             float acc[G][8];
 #pragma unroll
-            for (int g = 0; g < G; g++) {
-                float m = sc_new[g];
-#pragma unroll
-                for (int i = 0; i < NR; i++) m = fmaxf(m, sc[g][i]);
-                m = wave_max(m);
-                // softmax terms against the wavefront's own maximum (max, exp, sum:
-                // reference emit_softmax, src/graph_builder/emit_linalg.rs:509-528)
-                float lsum = 0.f;
-                float pr[NR];
-#pragma unroll
-                for (int i = 0; i < NR; i++) {
-                    pr[i] = live[i] ? expf(sc[g][i] - m) : 0.f;
-                    if (dl == 0) lsum += pr[i];
-                }
-                const float pn = with_new ? expf(sc_new[g] - m) : 0.f;
-                if (lane == 0) lsum += pn;
-                lsum = wave_sum(lsum);
-                if (lane == 0) {
-                    sm.wstat[cw][g][0] = m;
-                    sm.wstat[cw][g][1] = lsum;
-                }
+            for (int g = 0; g < G; g++)
 #pragma unroll
                 for (int e = 0; e < 8; e++) acc[g][e] = 0.f;
 #pragma unroll
-                for (int i = 0; i < NR; i++) {
-                    float vf[8];
-                    unpack8f(s.vr[i], vf);
+            for (int i = 0; i <= NR; i++) {
 #pragma unroll
-                    for (int e = 0; e < 8; e++) acc[g][e] = fmaf(pr[i], vf[e], acc[g][e]);
-                }
-                if (with_new && sub == 0) {
-                    float vn[8];
-                    lds_x8(sm.vnew, dl * 8, vn);
+                for (int g = 0; g < G; g++) {
+                    const float p = (i < NR || sub == 0) ? pr[g][i] : 0.f;  // the new row: one row group only
 #pragma unroll
-                    for (int e = 0; e < 8; e++) acc[g][e] = fmaf(pn, vn[e], acc[g][e]);
+                    for (int e = 0; e < 8; e++) acc[g][e] = fmaf(p, vf[i][e], acc[g][e]);
                 }
+            }
+#pragma unroll
+            for (int g = 0; g < G; g++) {
                 float *dst = &sm.part[cw * RPI + sub][g][dl * 8];
                 *reinterpret_cast<f32x4 *>(dst) = f32x4{acc[g][0], acc[g][1], acc[g][2], acc[g][3]};
                 *reinterpret_cast<f32x4 *>(dst + 4) = f32x4{acc[g][4], acc[g][5], acc[g][6], acc[g][7]};
             }
-            // the last of the four wavefronts to get here merges their partials (LDS operations of a CU
-            // execute in order: a later arrival sees what the earlier ones wrote before they counted in)
-            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-            int arrived = 0;
-            if (lane == 0) arrived = atomicAdd(&sm.arrive, 1);
-            arrived = __builtin_amdgcn_readfirstlane(arrived);
-            if (arrived == NCW - 1) {
-                if (lane == 0) sm.arrive = 0;
-                float f[G][NCW], mx[G], ls[G];
-#pragma unroll
-                for (int g = 0; g < G; g++) {
-                    float m = -INFINITY;
-#pragma unroll
-                    for (int w = 0; w < NCW; w++) m = fmaxf(m, sm.wstat[w][g][0]);
-                    float lt = 0.f;
-#pragma unroll
-                    for (int w = 0; w < NCW; w++) {
-                        const float mw = sm.wstat[w][g][0];
-                        f[g][w] = mw == -INFINITY ? 0.f : expf(mw - m);
-                        lt += f[g][w] * sm.wstat[w][g][1];
-                    }
-                    mx[g] = m;
-                    ls[g] = lt;
-                }
-                constexpr int QUADS = G * HD / 4;
-#pragma unroll
-                for (int q0 = 0; q0 < QUADS; q0 += WAVE) {
-                    const int q = q0 + lane;
-                    if (q < QUADS) {
-                        const int g = q / (HD / 4), d = (q % (HD / 4)) * 4;
-                        f32x4 o = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                        for (int w = 0; w < NCW; w++) {
-                            f32x4 t = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                            for (int sb = 0; sb < RPI; sb++) t += *reinterpret_cast<const f32x4 *>(&sm.part[w * RPI + sb][g][d]);
-                            float fw = 0.f;
-#pragma unroll
-                            for (int gg = 0; gg < G; gg++) fw = gg == g ? f[gg][w] : fw;
-                            o += fw * t;
-                        }
-                        *reinterpret_cast<f32x4 *>(&sm.pub[g * HD + d]) = o;
-                    }
-                }
-#pragma unroll
-                for (int g = 0; g < G; g++)
-                    if (lane == g) {
-                        sm.pub[G * HD + 2 * g] = mx[g];
-                        sm.pub[G * HD + 2 * g + 1] = ls[g];
-                    }
-            }
         }
-        load_kv(nx);
         wg_barrier();
 
         // ── O projection rows (reference src/hf/emitter.rs:738-745) ──
         wg_barrier();
+        load_kv(nx, 0, KV_CUT);
         {
-            float acc[GE::ROW];
+            float acc[GE::ROW][GE::CO];
+            plain_dots<GE::ROW, GE::CO>(s.wo, sm.attn, lane, acc);
+            float v[GE::ROW];
 #pragma unroll
-            for (int r = 0; r < GE::ROW; r++) acc[r] = 0.f;
+            for (int r = 0; r < GE::ROW; r++) v[r] = chunk_total<GE::CO>(acc[r]);
+            wave_sum_n<GE::ROW>(v);
+            float mine = 0.f;
 #pragma unroll
-            for (int c = 0; c < GE::CO; c++) {
-                float xv[8];
-                lds_x8(sm.attn, (c * WAVE + lane) * 8, xv);
-#pragma unroll
-                for (int r = 0; r < GE::ROW; r++) acc[r] = dot8f(s.wo[r][c], xv, acc[r]);
-            }
-#pragma unroll
-            for (int r = 0; r < GE::ROW; r++) {
-                const float v = wave_sum(acc[r]);
-                if (lane == 0) sm.pub[cw * GE::ROW + r] = v;
-            }
-            load_wo(nx);
+            for (int r = 0; r < GE::ROW; r++) mine = lane == r ? v[r] : mine;
+            if (lane < GE::ROW) sm.pub[cw * GE::ROW + lane] = mine;
         }
         wg_barrier();
 
         // ── gate|up rows, SiLU(gate) * up (reference src/hf/emitter.rs:787-799) ──
         wg_barrier();
+        load_kv(nx, KV_CUT, NR);
+        load_wo(nx);
         {
             const float tot = ((sm.red[0] + sm.red[1]) + sm.red[2]) + sm.red[3];
             const float inv = 1.0f / sqrtf(tot / (float)GE::HIDDEN + a.eps);
-            float acc[GE::RGW];
+            float acc[GE::RGW][GE::CH];
+            normed_dots<GE::RGW, GE::CH>(s.wg, sm.hx, sm.nw, inv, lane, acc);
+            float v[GE::RGW];
 #pragma unroll
-            for (int r = 0; r < GE::RGW; r++) acc[r] = 0.f;
-#pragma unroll
-            for (int c = 0; c < GE::CH; c++) {
-                const int k = (c * WAVE + lane) * 8;
-                float hv[8], wv[8], xv[8];
-                lds_x8(sm.hx, k, hv);
-                lds_x8(sm.nw, k, wv);
-#pragma unroll
-                for (int e = 0; e < 8; e++) xv[e] = (hv[e] * inv) * wv[e];
-#pragma unroll
-                for (int r = 0; r < GE::RGW; r++) acc[r] = dot8f(s.wg[r][c], xv, acc[r]);
-            }
+            for (int r = 0; r < GE::RGW; r++) v[r] = chunk_total<GE::CH>(acc[r]);
+            wave_sum_n<GE::RGW>(v);
+            float gte = 0.f, up = 0.f;
 #pragma unroll
             for (int r = 0; r < GE::RGW; r += 2) {
-                const float gte = wave_sum(acc[r]), up = wave_sum(acc[r + 1]);
-                if (lane == 0) sm.pub[cw * (GE::RGW / 2) + r / 2] = (gte / (1.0f + expf(-gte))) * up;
+                gte = lane == r / 2 ? v[r] : gte;
+                up = lane == r / 2 ? v[r + 1] : up;
             }
-            load_wg(nx);
+            if (lane < GE::RGW / 2) sm.pub[cw * (GE::RGW / 2) + lane] = (gte / (1.0f + expf(-gte))) * up;
         }
         wg_barrier();
 
         // ── down rows (reference src/hf/emitter.rs:801-804; the residual is added by the readers) ──
         wg_barrier();
+        load_wg(nx, 0, WG_CUT);
         {
-            float acc[GE::ROW];
+            float acc[GE::ROW][GE::CD];
+            plain_dots<GE::ROW, GE::CD>(s.wd, sm.act, lane, acc);
+            float v[GE::ROW];
 #pragma unroll
-            for (int r = 0; r < GE::ROW; r++) acc[r] = 0.f;
+            for (int r = 0; r < GE::ROW; r++) v[r] = chunk_total<GE::CD>(acc[r]);
+            wave_sum_n<GE::ROW>(v);
+            float mine = 0.f;
 #pragma unroll
-            for (int c = 0; c < GE::CD; c++) {
-                float xv[8];
-                lds_x8(sm.act, (c * WAVE + lane) * 8, xv);
-#pragma unroll
-                for (int r = 0; r < GE::ROW; r++) acc[r] = dot8f(s.wd[r][c], xv, acc[r]);
-            }
-#pragma unroll
-            for (int r = 0; r < GE::ROW; r++) {
-                const float v = wave_sum(acc[r]);
-                if (lane == 0) sm.pub[cw * GE::ROW + r] = v;
-            }
-            load_wd(nx);
+            for (int r = 0; r < GE::ROW; r++) mine = lane == r ? v[r] : mine;
+            if (lane < GE::ROW) sm.pub[cw * GE::ROW + lane] = mine;
         }
         wg_barrier();
     }
@@ -546,15 +643,22 @@ __device__ __forceinline__ int hidden_slot(int k) {
     return 2 * ((j / 2) * CT + c) + (j & 1);
 }
 
+__device__ __forceinline__ unsigned xcc_id() { return __builtin_amdgcn_s_getreg((3 << 11) | (0 << 6) | 20) & 0xF; }
+
 template <class GE>
 __device__ __forceinline__ void comm_role(const FusedDecodeArgs &a, Lds<GE> &sm, const int wg, const int cwv,
-                                          const int lane, const int pos, const uint32_t base) {
+                                          const int lane, const int pos, const uint32_t launches) {
     constexpr int G = GE::G, HD = GE::HD, NJ = GE::NJ;
     const Split<GE> sp(wg, pos);
     const int ct = cwv * WAVE + lane;
     const int L = a.n_layers;
-    PollState ps{a.ctl, false};
+    const uint32_t base = launches * (uint32_t)L;
+    PollState ps{a.ctl, false, 0u};
     const size_t par_bytes = (size_t)GE::PAR_SLOTS * 8;
+    unsigned long long *trace = (wg == 0 && ct == 0) ? a.trace : nullptr;
+    auto mark = [&]() {
+        if (trace) *trace++ = wall_clock64();
+    };
 
     // the token of this step (reference embed kernel, src/hf/emitter.rs:506-537)
     const int step = a.state->step, n_forced = a.state->n_forced;
@@ -564,13 +668,74 @@ __device__ __forceinline__ void comm_role(const FusedDecodeArgs &a, Lds<GE> &sm,
 #pragma unroll
     for (int j = 0; j < NJ; j++) h[j] = a.embed[(size_t)id * GE::HIDDEN + ct + CT * j];
 
-    // hidden <- hidden + (the vector published in `area` at slot offset `off`), then stage hidden, the
-    // norm weights and this wavefront's share of the sum of squares
-    auto stage_hidden = [&](const unsigned char *area, int off, uint32_t tag, bool add, const float *norm_w) {
+    // this position's RoPE table entries (the same for every layer)
+    RopeLane rope{0.f, 0.f, 0.f, 0.f};
+    if (lane < HD / 2) {
+        const float *c = a.cos_tab + (size_t)pos * HD, *sn = a.sin_tab + (size_t)pos * HD;
+        rope = RopeLane{c[lane], c[lane + HD / 2], sn[lane], sn[lane + HD / 2]};
+    }
+
+    // ── placement check: workgroups are dealt to the dies round-robin, starting wherever the previous
+    //    launch stopped, so wg % 8 names a die up to a rotation. Every workgroup reports the die it runs
+    //    on, every communicating wavefront reads all reports and reaches the same verdict: die-local
+    //    traffic is used only if all workgroups with the same wg % 8 sit on one die. ──
+    const int xcd = wg % GE::NXCD, rank = wg / GE::NXCD;
+    bool die_ok;
+    {
+        unsigned char *chk = a.xch + (size_t)GE::CHK0 * 8;
+        if (ct == 0) st_slot(chk, wg, (float)xcc_id(), launches + 1u, false);
+        int unit[2] = {lane, lane + WAVE};
+        bool on[2] = {lane < GE::NWG / 2, lane + WAVE < GE::NWG / 2};
+        u32x4 w[2];
+        poll_units<2>(ps, chk, unit, on, launches + 1u, w);
+        float ref[GE::NXCD];  // the dies of workgroups 0..7
+#pragma unroll
+        for (int j = 0; j < GE::NXCD; j++)
+            ref[j] = __shfl(__uint_as_float((j & 1) ? w[0].z : w[0].x), j / 2);
+        bool mine = true;
+#pragma unroll
+        for (int u = 0; u < 2; u++) {
+            const int j0 = (2 * unit[u]) % GE::NXCD;  // even, so the unit's two reports are j0 and j0 + 1
+            float r0 = 0.f, r1 = 0.f;
+#pragma unroll
+            for (int j = 0; j < GE::NXCD; j += 2) {
+                r0 = j == j0 ? ref[j] : r0;
+                r1 = j == j0 ? ref[j + 1] : r1;
+            }
+            if (on[u]) mine = mine && __uint_as_float(w[u].x) == r0 && __uint_as_float(w[u].z) == r1;
+        }
+        die_ok = __all(mine) && !__any(ps.failed);
+        if (!die_ok && wg == 0 && ct == 0) atomicAdd(a.ctl + 2, 1u);  // steps that ran without die-local traffic
+    }
+    const bool near_g = die_ok && GE::GROUP_ON_XCD;  // a KV head's workgroups talk through their die's L2
+
+    // A vector that every workgroup reads is fetched from memory once per die: one wavefront of each of the
+    // die's workgroups waits for its share of the units and copies them to the die's relay area, which all
+    // of them then read through the L2. Without die-local placement everyone reads the far copy.
+    auto relay = [&](unsigned char *par, int off, int n_units, uint32_t tag) -> const unsigned char * {
+        if (!die_ok) return par;
+        unsigned char *rel = par + (size_t)(GE::RELAY0 + xcd * GE::GLOB_SLOTS) * 8;
+        if (cwv == 3) {  // wavefront 0 may still be folding
+            const int per = n_units / GE::NPX;
+            int unit[1] = {off / 2 + rank * per + lane};
+            bool on[1] = {lane < per};
+            u32x4 w[1];
+            poll_units<1>(ps, par, unit, on, tag, w);
+            if (on[0]) {
+                *reinterpret_cast<u32x4 *>(rel + (size_t)unit[0] * 16) = w[0];  // plain store: stays in the die's L2
+                asm volatile("" ::: "memory");
+            }
+        }
+        return rel;
+    };
+    // hidden <- hidden + (the vector at slot offset `off`), then stage hidden, the norm weights and this
+    // wavefront's share of the sum of squares
+    auto stage_hidden = [&](unsigned char *par, int off, uint32_t tag, bool add, const float *norm_w) {
         float nwv[NJ];
 #pragma unroll
         for (int j = 0; j < NJ; j++) nwv[j] = ldf_global(norm_w + ct + CT * j);
         if (add) {
+            const unsigned char *src = relay(par, off, GE::HIDDEN / 2, tag);
             int unit[NJ / 2];
             bool on[NJ / 2];
             u32x4 w[NJ / 2];
@@ -579,7 +744,7 @@ __device__ __forceinline__ void comm_role(const FusedDecodeArgs &a, Lds<GE> &sm,
                 unit[u] = off / 2 + u * CT + ct;
                 on[u] = true;
             }
-            poll_units<NJ / 2>(ps, area, unit, on, tag, w);
+            poll_units<NJ / 2>(ps, src, unit, on, tag, w);
 #pragma unroll
             for (int u = 0; u < NJ / 2; u++) {
                 h[2 * u] = h[2 * u] + __uint_as_float(w[u].x);
@@ -597,9 +762,10 @@ __device__ __forceinline__ void comm_role(const FusedDecodeArgs &a, Lds<GE> &sm,
             sm.nw[ct + CT * j] = nwv[j];
         }
     };
-    // copy a published vector of n values (plain slot order) into LDS
-    auto stage_vector = [&](const unsigned char *area, int off, uint32_t tag, float *dst, auto nu_tag) {
+    // copy a published vector (plain slot order) into LDS
+    auto stage_vector = [&](unsigned char *par, int off, uint32_t tag, float *dst, auto nu_tag) {
         constexpr int NU = decltype(nu_tag)::value;
+        const unsigned char *src = relay(par, off, NU * CT, tag);
         int unit[NU];
         bool on[NU];
         u32x4 w[NU];
@@ -608,7 +774,7 @@ __device__ __forceinline__ void comm_role(const FusedDecodeArgs &a, Lds<GE> &sm,
             unit[u] = off / 2 + u * CT + ct;
             on[u] = true;
         }
-        poll_units<NU>(ps, area, unit, on, tag, w);
+        poll_units<NU>(ps, src, unit, on, tag, w);
 #pragma unroll
         for (int u = 0; u < NU; u++) {
             dst[2 * (u * CT + ct)] = __uint_as_float(w[u].x);
@@ -618,30 +784,42 @@ __device__ __forceinline__ void comm_role(const FusedDecodeArgs &a, Lds<GE> &sm,
 
     for (int l = 0; l < L; l++) {
         const FusedLayerPtrs cur = sm.lp[l];
+        const bool qk_normed = cur.q_norm != nullptr;
+        float qn_lo = 1.f, qn_hi = 1.f, kn_lo = 1.f, kn_hi = 1.f;  // requested now, used in the attention phase
+        if (qk_normed && lane < HD / 2) {
+            qn_lo = ldf_global(cur.q_norm + lane);
+            qn_hi = ldf_global(cur.q_norm + lane + HD / 2);
+            kn_lo = ldf_global(cur.k_norm + lane);
+            kn_hi = ldf_global(cur.k_norm + lane + HD / 2);
+        }
         const uint32_t gl = base + (uint32_t)l;  // layers run since the exchange area was zeroed
         const uint32_t tag = gl + 1u;
         unsigned char *xc = a.xch + (size_t)(gl & 1u) * par_bytes;
-        const unsigned char *xprev = a.xch + (size_t)((gl & 1u) ^ 1u) * par_bytes;
+        unsigned char *xprev = a.xch + (size_t)((gl & 1u) ^ 1u) * par_bytes;
+        unsigned char *lq = xc + (size_t)(GE::LQ0 + sp.kh * GE::GROWS) * 8;             // this KV head's raw rows
+        unsigned char *lp = xc + (size_t)(GE::LP0 + sp.kh * GE::SPH * GE::PART) * 8;    // and its splits' partials
 
         // ── into the Q|K|V phase: hidden += down rows of the previous layer ──
+        ps.where = 1u | (uint32_t)l << 4 | (uint32_t)wg << 12;
         stage_hidden(xprev, GE::XH, tag - 1u, l > 0, cur.in_ln);
-        if (cur.qkv_bias && ct < GE::RQ) sm.bias[ct] = ldf_global(cur.qkv_bias + wg * GE::RQ + ct);
+        if (cur.qkv_bias && ct < GE::RQ)
+            sm.bias[ct] = ldf_global(cur.qkv_bias + GE::qkv_row(sp.kh, sp.split * GE::RQ + ct));
         wg_barrier();
+        mark();
         wg_barrier();
-        if (ct < GE::RQ) st_slot(xc, GE::XQ + wg * GE::RQ + ct, sm.pub[ct], tag);
+        mark();
+        if (ct < GE::RQ) st_slot(lq, sp.split * GE::RQ + ct, sm.pub[ct], tag, near_g);
 
         // ── into attention: this KV head's raw q rows (and k, v for the split that holds the new row),
         //    QK-norm + RoPE, cache append (reference src/hf/emitter.rs:629-649, src/runtime.rs:521-568) ──
+        ps.where = 2u | (uint32_t)l << 4 | (uint32_t)wg << 12;
         if (sp.split < sp.nsl) {
-            const float *c = a.cos_tab + (size_t)pos * HD;
-            const float *sn = a.sin_tab + (size_t)pos * HD;
             for (int t = cwv; t < G + 2; t += 4) {
                 if (t >= G && !sp.owner) continue;
-                const int first = t < G ? (sp.kh * G + t) * HD : (t == G ? GE::QD : GE::QD + GE::KVD) + sp.kh * HD;
-                int unit[1] = {(GE::XQ + first) / 2 + lane};
+                int unit[1] = {t * HD / 2 + lane};
                 bool on[1] = {lane < HD / 2};
                 u32x4 w[1];
-                poll_units<1>(ps, xc, unit, on, tag, w);
+                poll_units<1>(ps, lq, unit, on, tag, w);
                 if (on[0]) {
                     sm.rowbuf[t][2 * lane] = __uint_as_float(w[0].x);
                     sm.rowbuf[t][2 * lane + 1] = __uint_as_float(w[0].z);
@@ -651,14 +829,14 @@ __device__ __forceinline__ void comm_role(const FusedDecodeArgs &a, Lds<GE> &sm,
                 const size_t row_off = ((size_t)sp.kh * a.max_len + pos) * HD;
                 if (t < G) {
                     float lo, hi;
-                    norm_rope<HD>(sm.rowbuf[t], cur.q_norm, c, sn, a.eps, lane, lo, hi);
+                    norm_rope<HD>(sm.rowbuf[t], qk_normed, qn_lo, qn_hi, rope, a.eps, lane, lo, hi);
                     if (lane < HALF) {
                         sm.qs[t][lane] = lo;
                         sm.qs[t][lane + HALF] = hi;
                     }
                 } else if (t == G) {
                     float lo, hi;
-                    norm_rope<HD>(sm.rowbuf[t], cur.k_norm, c, sn, a.eps, lane, lo, hi);
+                    norm_rope<HD>(sm.rowbuf[t], qk_normed, kn_lo, kn_hi, rope, a.eps, lane, lo, hi);
                     if (lane < HALF) {  // rounded to bf16 once; cache and this step use the same values
                         uint16_t *dst = cur.kcache + row_off;
                         const uint16_t r_lo = f32_to_bf16_rne_dev(lo), r_hi = f32_to_bf16_rne_dev(hi);
@@ -678,61 +856,102 @@ __device__ __forceinline__ void comm_role(const FusedDecodeArgs &a, Lds<GE> &sm,
             }
         }
         wg_barrier();
+        mark();
         wg_barrier();
-        if (sp.split < sp.nsl)
-            for (int i = ct; i < GE::PART; i += CT)
-                st_slot(xc, GE::XP + (sp.kh * GE::SPH + sp.split) * GE::PART + i, sm.pub[i], tag);
+        mark();
+        if (sp.split < sp.nsl) {
+            // merge the compute wavefronts' partials (one output per thread) and publish the split's
+            // (o, max, sum): o = sum_w exp(m_w - M) * (sum over w's row groups), in wavefront order
+            for (int i = ct; i < GE::PART; i += CT) {
+                const int g = i < G * HD ? i / HD : (i - G * HD) / 2;
+                float mw[NCW], M = -INFINITY;
+#pragma unroll
+                for (int w = 0; w < NCW; w++) {
+                    mw[w] = sm.wstat[w][g][0];
+                    M = fmaxf(M, mw[w]);
+                }
+                float v = 0.f;
+#pragma unroll
+                for (int w = 0; w < NCW; w++) {
+                    const float f = mw[w] == -INFINITY ? 0.f : __expf(mw[w] - M);
+                    float t;
+                    if (i < G * HD) {
+                        t = 0.f;
+#pragma unroll
+                        for (int sb = 0; sb < GE::RPI; sb++) t += sm.part[w * GE::RPI + sb][g][i % HD];
+                    } else {
+                        t = sm.wstat[w][g][1];
+                    }
+                    v += f * t;
+                }
+                if (i >= G * HD && ((i - G * HD) & 1) == 0) v = M;
+                st_slot(lp, sp.split * GE::PART + i, v, tag, near_g);
+            }
+        }
 
-        // ── fold the splits of one head for this workgroup's FPW outputs (one wavefront) ──
+        // ── fold the splits of this KV head for FPW of its outputs (one wavefront) ──
+        ps.where = 3u | (uint32_t)l << 4 | (uint32_t)wg << 12;
         if (cwv == 0) {
             constexpr int FU = GE::FPW / 2;
-            const int hh = (wg * GE::FPW) / HD, d0 = (wg * GE::FPW) % HD;
-            const int kh2 = hh / G, gg = hh % G;
-            const int pbase = GE::XP + (kh2 * GE::SPH + lane) * GE::PART;
+            const int o0 = sp.split * GE::FPW;  // first output, counted inside the KV head's G * HD
+            const int t = o0 / HD, d0 = o0 % HD;
+            const int pbase = lane * GE::PART;
             int unit[FU + 1];
             bool on[FU + 1];
             u32x4 w[FU + 1];
 #pragma unroll
             for (int u = 0; u < FU; u++) {
-                unit[u] = (pbase + gg * HD + d0) / 2 + u;
+                unit[u] = (pbase + t * HD + d0) / 2 + u;
                 on[u] = lane < sp.nsl;
             }
-            unit[FU] = (pbase + G * HD + 2 * gg) / 2;
+            unit[FU] = (pbase + G * HD + 2 * t) / 2;
             on[FU] = lane < sp.nsl;
-            poll_units<FU + 1>(ps, xc, unit, on, tag, w);
+            poll_units<FU + 1>(ps, lp, unit, on, tag, w);
             const float m_s = on[FU] ? __uint_as_float(w[FU].x) : -INFINITY;
             const float l_s = on[FU] ? __uint_as_float(w[FU].z) : 0.f;
             const float m = wave_max(m_s);
-            const float f = on[FU] ? expf(m_s - m) : 0.f;
-            const float lt = wave_sum(f * l_s);
-            float mine = 0.f;
+            const float f = on[FU] ? __expf(m_s - m) : 0.f;
+            float red[2 * FU + 1];  // the sum of the splits' sums, then the FPW weighted outputs
+            red[0] = f * l_s;
 #pragma unroll
             for (int u = 0; u < FU; u++) {
-                const float o0 = wave_sum(f * __uint_as_float(w[u].x)) / lt;
-                const float o1 = wave_sum(f * __uint_as_float(w[u].z)) / lt;
-                if (lane == 2 * u) mine = o0;
-                if (lane == 2 * u + 1) mine = o1;
+                red[1 + 2 * u] = f * __uint_as_float(w[u].x);
+                red[2 + 2 * u] = f * __uint_as_float(w[u].z);
             }
-            if (lane < GE::FPW) st_slot(xc, GE::XA + wg * GE::FPW + lane, mine, tag);
+            wave_sum_n<2 * FU + 1>(red);
+            float mine = 0.f;
+#pragma unroll
+            for (int e = 0; e < GE::FPW; e++) mine = lane == e ? red[1 + e] / red[0] : mine;
+            if (lane < GE::FPW) st_slot(xc, GE::XA + sp.kh * G * HD + o0 + lane, mine, tag, false);
         }
+        mark();
 
         // ── into the O phase ──
+        ps.where = 4u | (uint32_t)l << 4 | (uint32_t)wg << 12;
         stage_vector(xc, GE::XA, tag, sm.attn, std::integral_constant<int, GE::QD / 2 / CT>());
         wg_barrier();
+        mark();
         wg_barrier();
-        if (ct < GE::RO) st_slot(xc, GE::XO + hidden_slot(wg * GE::RO + ct), sm.pub[ct], tag);
+        mark();
+        if (ct < GE::RO) st_slot(xc, GE::XO + hidden_slot(wg * GE::RO + ct), sm.pub[ct], tag, false);
 
         // ── into the gate|up phase: hidden += O rows (reference src/hf/emitter.rs:787) ──
+        ps.where = 5u | (uint32_t)l << 4 | (uint32_t)wg << 12;
         stage_hidden(xc, GE::XO, tag, true, cur.post_ln);
         wg_barrier();
+        mark();
         wg_barrier();
-        if (ct < GE::APW) st_slot(xc, GE::XC + wg * GE::APW + ct, sm.pub[ct], tag);
+        mark();
+        if (ct < GE::APW) st_slot(xc, GE::XC + wg * GE::APW + ct, sm.pub[ct], tag, false);
 
         // ── into the down phase ──
+        ps.where = 6u | (uint32_t)l << 4 | (uint32_t)wg << 12;
         stage_vector(xc, GE::XC, tag, sm.act, std::integral_constant<int, GE::INTER / 2 / CT>());
         wg_barrier();
+        mark();
         wg_barrier();
-        if (ct < GE::RO) st_slot(xc, GE::XH + hidden_slot(wg * GE::RO + ct), sm.pub[ct], tag);
+        mark();
+        if (ct < GE::RO) st_slot(xc, GE::XH + hidden_slot(wg * GE::RO + ct), sm.pub[ct], tag, false);
     }
 
     // hidden += down rows of the last layer: the LM head's input
@@ -755,8 +974,10 @@ __device__ __forceinline__ void comm_role(const FusedDecodeArgs &a, Lds<GE> &sm,
         }
         // Every workgroup read the launch count before its first exchange, and this point is only reached
         // after all of them have published their last rows.
-        if (ct == 0)
-            __hip_atomic_store(a.ctl, base / (uint32_t)L + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (ct == 0) __hip_atomic_store(a.ctl, launches + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        mark();
+        if (trace) *trace++ = die_ok ? 1ull : 0ull;
+
     }
 }
 
@@ -773,14 +994,13 @@ __global__ __launch_bounds__(FT) void decode_fused_kernel(FusedDecodeArgs a) {
         uint64_t *dst = reinterpret_cast<uint64_t *>(sm.lp);
         const int words = a.n_layers * (int)(sizeof(FusedLayerPtrs) / 8);
         for (int i = threadIdx.x; i < words; i += FT) dst[i] = src[i];
-        if (threadIdx.x == 0) sm.arrive = 0;
         __syncthreads();
     }
     if (wave < NCW) {
         compute_role<GE>(a, sm, wg, wave, lane, pos);
     } else {
         const uint32_t launches = __hip_atomic_load(a.ctl, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        comm_role<GE>(a, sm, wg, wave - NCW, lane, pos, launches * (uint32_t)a.n_layers);
+        comm_role<GE>(a, sm, wg, wave - NCW, lane, pos, launches);
     }
 }
 
@@ -818,8 +1038,8 @@ int decode_fused_max_kv(const FusedShape &s) {
 }
 
 size_t decode_fused_xch_bytes(const FusedShape &s) {
-    if (shape_is<GeoQwen3_0p6b>(s)) return (size_t)GeoQwen3_0p6b::PAR_SLOTS * 8 * 2;
-    if (shape_is<GeoSmall>(s)) return (size_t)GeoSmall::PAR_SLOTS * 8 * 2;
+    if (shape_is<GeoQwen3_0p6b>(s)) return (size_t)GeoQwen3_0p6b::ALL_SLOTS * 8;
+    if (shape_is<GeoSmall>(s)) return (size_t)GeoSmall::ALL_SLOTS * 8;
     return 0;
 }
 
@@ -861,10 +1081,13 @@ int decode_fused_launch(hm_ctx *ctx, const FusedShape &s, const FusedDecodeArgs 
 }
 
 int decode_fused_check(hm_ctx *ctx, const uint32_t *d_ctl) {
-    uint32_t h[2] = {0, 0};
+    uint32_t h[16] = {0};
     int rc = hm_download(ctx, h, d_ctl, sizeof(h));
     if (rc != HM_OK) return rc;
     if (h[1] != 0)
-        return hm_set_error(ctx, HM_ERR_HIP, "decode_fused: an exchange timed out (status %u after %u launches)", h[1], h[0]);
+        return hm_set_error(ctx, HM_ERR_HIP,
+                            "decode_fused: workgroup %u stopped waiting in phase %u of layer %u (launch %u)",
+                            (h[1] >> 12) & 0xFFFFu, h[1] & 15u, (h[1] >> 4) & 255u, h[0]);
+    
     return HM_OK;
 }

@@ -2,6 +2,7 @@
 #include <cstring>
 
 #include "hf.h"
+#include "../../../include/homura_amd_bench.h"
 #include "loaders.h"
 
 using namespace homura;
@@ -177,6 +178,11 @@ int hm_model_whole_step(hm_model *m) {
 int hm_model_whole_step_available(hm_model *m) {
     if (!m) return HM_ERR_INVALID;
     return m->impl->whole_step_available() ? 1 : 0;
+}
+
+int hm_model_whole_step_trace(hm_model *m, unsigned long long *h_out, int cap, int *n_out) {
+    if (!m || !n_out) return HM_ERR_INVALID;
+    return m->impl->whole_step_trace(h_out, cap, n_out);
 }
 
 int hm_model_whole_step_status(hm_model *m) {

@@ -48,7 +48,7 @@ struct PlanScratch {
     Buffer attn_flat, resid, act, cand_val, cand_idx;
     // whole-step decode launch (bf16 plans of a served shape): device layer table, exchange area,
     // control words {launch count, status}
-    Buffer fused_layers, fused_xch, fused_ctl;
+    Buffer fused_layers, fused_xch, fused_ctl, fused_trace;
     Buffer normed, gate, up, down, q_raw, k_raw, v_raw;  // quantised plan only
     int cand_cap = 0;
 };
@@ -117,6 +117,10 @@ class HfModel {
     bool whole_step() const { return plan_ && plan_->whole_step(); }
     // HM_OK, or the error a whole-step launch left behind (an exchange that timed out)
     int whole_step_status();
+    // Phase trace of the latest whole-step launch (device clock ticks at 100 MHz; 11 entries per layer
+    // and a final one, see decode_fused.h). Recording starts with the first call, which returns 0
+    // entries; later calls return the trace of the step that ran last.
+    int whole_step_trace(unsigned long long *h_out, int cap, int *n_out);
     int time_kernels(int rounds, std::vector<StepProfile> &out);
     ExecutionPlan *plan() { return plan_.get(); }
 

@@ -545,6 +545,7 @@ int HfModel::emit_transformer_plan() {
                 fa.max_len = sc.plan->kv_cache()->max_len();
                 fa.xch = scr->fused_xch.as<unsigned char>();
                 fa.ctl = scr->fused_ctl.as<uint32_t>();
+                fa.trace = scr->fused_trace ? scr->fused_trace.as<unsigned long long>() : nullptr;
                 return decode_fused_launch(sc.ctx, fs, fa);
             };
             k.launches.push_back(std::move(f));
@@ -1336,6 +1337,27 @@ int HfModel::refresh_fused_table() {
     fused_table_kv_ = kv->key_ptr(0);
     fused_table_max_len_ = kv->max_len();
     return HM_OK;
+}
+
+int HfModel::whole_step_trace(unsigned long long *h_out, int cap, int *n_out) {
+    if (!fused_available_) return hm_set_error(ctx_, HM_ERR_STATE, "whole-step decode is not available for this model");
+    const int n = cfg_.num_hidden_layers * FUSED_TRACE_PER_LAYER + 2;
+    *n_out = 0;
+    int rc = hm_sync(ctx_);
+    if (rc != HM_OK) return rc;
+    if (!scratch_->fused_trace) {
+        scratch_->fused_trace = Buffer::alloc_bytes(ctx_, (size_t)n * 8, {n}, DType::I64);
+        if (!scratch_->fused_trace) return HM_ERR_OOM;
+        HM_HIP(ctx_, hipMemsetAsync(scratch_->fused_trace.ptr(), 0, (size_t)n * 8, ctx_->stream));
+        // a captured step does not know the trace buffer yet
+        const bool was = plan_->whole_step();
+        if ((rc = plan_->set_whole_step(!was)) != HM_OK || (rc = plan_->set_whole_step(was)) != HM_OK) return rc;
+        return hm_sync(ctx_);
+    }
+    if (cap < n) return hm_set_error(ctx_, HM_ERR_INVALID, "whole_step_trace: room for %d entries, %d needed", cap, n);
+    rc = hm_download(ctx_, h_out, scratch_->fused_trace.ptr(), (size_t)n * 8);
+    if (rc == HM_OK) *n_out = n;
+    return rc;
 }
 
 // Stream sync plus, when steps went through the whole-step launch, its status word.

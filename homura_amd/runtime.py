@@ -426,6 +426,16 @@ class HfModel:
         """Raises if a whole-step launch left an error behind (an exchange that timed out)."""
         self._check(self.lib.hm_model_whole_step_status(self.h))
 
+    def whole_step_trace(self) -> np.ndarray:
+        """Device-clock ticks (100 MHz) of the latest whole-step launch: 11 per layer (both barriers of the
+        Q|K|V, attention, O, gate|up and down phases; the fold's end comes after attention's) and a final
+        one. The first call only switches recording on and returns an empty array."""
+        cap = 64 * 11 + 2
+        out = np.zeros(cap, dtype=np.uint64)
+        n = C.c_int(0)
+        self._check(self.lib.hm_model_whole_step_trace(self.h, out.ctypes.data, cap, C.byref(n)))
+        return out[:n.value]
+
     def reset_kv_cache(self):
         self._check(self.lib.hm_model_reset_kv_cache(self.h))
 

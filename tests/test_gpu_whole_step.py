@@ -1,0 +1,193 @@
+"""The whole-step decode launch (one resident kernel for the embedding row and every layer, phases
+exchanging tagged values through device memory) against the CPU oracle and against the plan's
+one-launch-per-projection path, through the C boundary. Logits within 1e-2 max relative error,
+|gpu - ref| / max(|ref|, 1e-2 * max|ref|); greedy tokens identical."""
+import dataclasses
+
+import numpy as np
+import pytest
+
+import model_fixture as mf
+from homura_amd import HomuraError, synth, synth_model
+
+pytestmark = pytest.mark.gpu
+
+
+def say(msg):
+    print(msg, flush=True)
+
+
+@pytest.fixture(scope="module")
+def small(ctx):
+    cfg = synth_model.SMALL_WS
+    weights = synth_model.synth_weights(cfg, 5151)
+    gm = synth_model.build_model(ctx, cfg, weights, 2048)
+    om = mf.build_oracle_model(cfg, weights, 2048)
+    yield cfg, weights, gm, om
+    gm.close()
+
+
+def test_small_shape_is_served_and_on_by_default(small):
+    _cfg, _w, gm, _om = small
+    assert gm.whole_step_available() and gm.whole_step()
+
+
+@pytest.mark.parametrize("cache_rows", [0, 2, 31, 50, 333])
+def test_logits_and_tokens_against_oracle(small, cache_rows):
+    """Caches that leave most attention splits empty (0, 2 rows), that straddle a split boundary while
+    tokens are appended (31 -> 36), and ordinary ones. (With so few rows one cache row that lands on the
+    other side of a bf16 rounding boundary moves the logits by 1e-4..4e-4 of their scale; both GPU paths
+    show it against the oracle, e.g. from a one-row cache, and the 1% floor of rel_err absorbs it here.)"""
+    cfg, _w, gm, om = small
+    kv = synth_model.synth_kv(cfg, 7 + cache_rows, max(cache_rows, 1))
+    gm.set_whole_step(True)
+    gm.init_kv_cache(kv, cache_rows)
+    mf.oracle_init_kv(om, kv)
+    om.kv.reset(cache_rows)
+    ids = synth.token_ids(8 + cache_rows, 5, cfg.vocab_size)
+    gm.set_prefill_min(0)
+    got = gm.run_kv(ids)
+    gm.whole_step_status()
+    want = np.concatenate([om.run_kv(ids[i:i + 1]) for i in range(5)])
+    for i in range(5):
+        assert mf.rel_err(got[i], want[i]) < 1e-2, f"cache {cache_rows}, position {i}"
+    want_t, margins = om.generate_greedy(ids[:2], 24)
+    got_t = gm.generate_greedy(ids[:2], 24)
+    say(f"cache {cache_rows}: min margin {margins.min():.3e}")
+    assert np.array_equal(got_t, want_t)
+    assert gm.kv_cache_len() == cache_rows + 5 + 2 + 23
+
+
+def test_whole_step_against_per_projection_path(small):
+    """Same arithmetic as the per-projection kernels up to the order of f32 sums in attention."""
+    cfg, _w, gm, _om = small
+    kv = synth_model.synth_kv(cfg, 21, 200)
+    ids = synth.token_ids(22, 6, cfg.vocab_size)
+    gm.set_prefill_min(0)
+    gm.set_whole_step(False)
+    gm.init_kv_cache(kv, 200)
+    ref = gm.run_kv(ids)
+    ref_t = gm.generate_greedy(ids[:1], 30)
+    gm.set_whole_step(True)
+    gm.init_kv_cache(kv, 200)
+    got = gm.run_kv(ids)
+    got_t = gm.generate_greedy(ids[:1], 30)
+    gm.whole_step_status()
+    assert mf.rel_err(got, ref) < 1e-3
+    assert np.array_equal(got_t, ref_t)
+
+
+def test_graph_replay_and_cache_rebuild(small):
+    """Replays interleaved with eager work; re-creating the KV cache (other max length would move its
+    addresses) refreshes the device layer table."""
+    cfg, _w, gm, _om = small
+    kv = synth_model.synth_kv(cfg, 17, 30)
+    ids = synth.token_ids(18, 4, cfg.vocab_size)
+    gm.set_whole_step(True)
+    gm.set_prefill_min(0)
+    gm.init_kv_cache(kv, 30)
+    eager_tokens = gm.generate_greedy(ids, 24)
+    gm.init_kv_cache(kv, 30)
+    eager_logits = gm.run_kv(ids[:1])
+    gm.set_graph(True)
+    try:
+        for rep in range(3):
+            gm.init_kv_cache(kv, 30)
+            assert np.array_equal(gm.generate_greedy(ids, 24), eager_tokens), f"replay round {rep}"
+            gm.init_kv_cache(kv, 30)
+            assert np.array_equal(gm.run_kv(ids[:1]), eager_logits)
+    finally:
+        gm.set_graph(False)
+    gm.whole_step_status()
+
+
+def test_long_cache_up_to_the_served_maximum(small):
+    """2048 rows is what the attention phase of this instance keeps in registers (32 splits x 64 rows)."""
+    cfg, _w, gm, om = small
+    rows = 2040
+    kv = synth_model.synth_kv(cfg, 99, rows)
+    gm.set_whole_step(True)
+    gm.set_prefill_min(0)
+    gm.init_kv_cache(kv, rows)
+    mf.oracle_init_kv(om, kv)
+    ids = synth.token_ids(98, 8, cfg.vocab_size)
+    got = gm.run_kv(ids)
+    gm.whole_step_status()
+    want = np.concatenate([om.run_kv(ids[i:i + 1]) for i in range(8)])
+    assert gm.kv_cache_len() == 2048
+    for i in range(8):
+        assert mf.rel_err(got[i], want[i]) < 1e-2, f"position {i}"
+    with pytest.raises(HomuraError) as e:
+        gm.run_kv(ids[:1])
+    assert "KV cache full" in str(e.value)
+
+
+def test_bias_and_no_qk_norm_variant(ctx):
+    """Q/K/V biases ride in the Q|K|V phase; without QK-norm the rows go straight to RoPE."""
+    cfg = dataclasses.replace(synth_model.SMALL_WS, attention_bias=True)
+    weights = synth_model.synth_weights(cfg, 77, has_qk_norm=False)
+    assert any(n.endswith("q_proj.bias") for n, _ in weights)
+    gm = synth_model.build_model(ctx, cfg, weights, 128, has_qk_norm=False)
+    om = mf.build_oracle_model(cfg, weights, 128, has_qk_norm=False)
+    assert gm.whole_step()
+    kv = synth_model.synth_kv(cfg, 8, 21)
+    gm.init_kv_cache(kv, 21)
+    mf.oracle_init_kv(om, kv)
+    ids = synth.token_ids(6, 5, cfg.vocab_size)
+    gm.set_prefill_min(0)
+    got = gm.run_kv(ids)
+    want = np.concatenate([om.run_kv(ids[i:i + 1]) for i in range(5)])
+    for i in range(5):
+        assert mf.rel_err(got[i], want[i]) < 1e-2, f"position {i}"
+    want_t, _ = om.generate_greedy(ids[:2], 20)
+    assert np.array_equal(gm.generate_greedy(ids[:2], 20), want_t)
+    gm.whole_step_status()
+    gm.close()
+
+
+def test_qwen3_0p6b_shape_against_per_projection_path(ctx):
+    """The benchmark shape: same tokens and close logits from both ways through the layers (the 64-token
+    oracle identity of this shape runs in test_gpu_model.py with the whole-step launch on)."""
+    cfg = synth_model.QWEN3_0P6B
+    weights = synth_model.synth_weights(cfg, 0xC0FFEE02)
+    gm = synth_model.build_model(ctx, cfg, weights, 1120)
+    assert gm.whole_step_available() and gm.whole_step()
+    kv = synth_model.synth_kv(cfg, 5, 1024)
+    ids = synth.token_ids(6, 3, cfg.vocab_size)
+    gm.set_prefill_min(0)
+    gm.set_graph(True)
+    gm.init_kv_cache(kv, 1024)
+    got = gm.run_kv(ids)
+    got_t = gm.generate_greedy(ids[:1], 32)
+    gm.whole_step_status()
+    trace = gm.whole_step_trace()      # switches recording on
+    assert len(trace) == 0
+    gm.generate_greedy(ids[:1], 2)
+    trace = gm.whole_step_trace().astype(np.int64)
+    assert len(trace) == cfg.num_hidden_layers * 11 + 2
+    assert np.all(np.diff(trace[:-1]) >= 0) and trace[-1] in (0, 1)
+    say(f"whole-step kernel {(trace[-2] - trace[0]) / 100.0:.1f} us from first to last mark, die-local exchanges: {trace[-1]}")
+    gm.set_whole_step(False)
+    gm.init_kv_cache(kv, 1024)
+    ref = gm.run_kv(ids)
+    ref_t = gm.generate_greedy(ids[:1], 32)
+    assert mf.rel_err(got, ref) < 1e-3
+    assert np.array_equal(got_t, ref_t)
+    gm.close()
+
+
+def test_unserved_shapes_keep_the_per_projection_path(ctx):
+    cfg = synth_model.TINY
+    weights = synth_model.synth_weights(cfg, 4242)
+    gm = synth_model.build_model(ctx, cfg, weights, 64)
+    assert not gm.whole_step_available() and not gm.whole_step()
+    with pytest.raises(HomuraError):
+        gm.set_whole_step(True)
+    gm.whole_step_status()
+    gm.close()
+    # a served shape whose cache is longer than the attention phase keeps in registers
+    cfg2 = dataclasses.replace(synth_model.SMALL_WS, max_position_embeddings=4096)
+    w2 = synth_model.synth_weights(cfg2, 1)
+    gm2 = synth_model.build_model(ctx, cfg2, w2, 4096)
+    assert not gm2.whole_step_available()
+    gm2.close()
