@@ -11,7 +11,7 @@
 #include <thread>
 #include <vector>
 
-#include "../../include/homura_amd.h"
+#include "../../include/homura_amd_bench.h"
 
 namespace {
 

@@ -376,26 +376,6 @@ int hm_model_generate(hm_model *m, const int64_t *h_prompt, int n_prompt, int ma
                       const hm_sampling_config *cfg, uint64_t seed, int eos_token_id, int32_t *h_tokens_out,
                       int *n_tokens_out);
 
-/* Timed decode for benchmarking: runs `n_steps` decode steps starting from token `first_id`
- * (greedy feedback on device), returns total milliseconds measured with HIP events on the
- * context stream. */
-int hm_model_bench_decode(hm_model *m, int64_t first_id, int n_steps, float *ms_out,
-                          int32_t *h_tokens_out);
-
-/* Per-kernel profile of one decode step (HOMURA_PROFILE analogue, reference
- * src/runtime.rs:1849-1873): HIP events around every device launch; one record per device
- * kernel name. Fills up to `cap` records; returns the number written. */
-typedef struct {
-    char label[32]; /* "gemv_bf16[qkv]", "gqa_decode_attn", "gemv_bf16[lm_head+argmax]", ... */
-    float ms;       /* summed over the launches */
-    int launches;
-    double bytes;   /* algorithmic bytes moved by these launches */
-} hm_kernel_profile;
-int hm_model_profile_step(hm_model *m, int64_t token_id, hm_kernel_profile *out, int cap);
-/* Roofline timing: per device kernel name, all of the step's launches of that kernel (one per
- * layer, different weights each) back to back, `rounds` times, between two HIP events.
- * Disturbs activations and the current cache row: call after the decode. */
-int hm_model_time_kernels(hm_model *m, int rounds, hm_kernel_profile *out, int cap);
 /* Number of HIP kernel launches one decode step issues. */
 int hm_model_launches_per_step(hm_model *m);
 
@@ -492,18 +472,6 @@ int hm_ciface_bind_transformer_quant(hm_ctx *ctx, const hm_transformer_config *c
 int hm_ciface_num_kernels(void);
 void hm_ciface_unbind(void);
 
-/* ── deterministic synthetic data (host side, no GPU needed) ─────────────────
- * Counter-based generator shared by tests and benchmarks: sample i of stream `seed` uses
- * outputs 3i..3i+2 of the splitmix64 sequence seeded with `seed`; a normal variate is the
- * centred sum of the twelve 16-bit fields of those outputs (Irwin-Hall, unit variance),
- * computed in integers so that every platform produces the same bits. */
-void hm_synth_normal_f32(uint64_t seed, uint64_t first, size_t n, float scale, float *out);
-void hm_synth_normal_bf16(uint64_t seed, uint64_t first, size_t n, float scale, uint16_t *out);
-void hm_synth_token_ids(uint64_t seed, size_t n, int vocab, int64_t *out);
-/* n_blocks Q8_0 blocks: q uniform in [-127,127], d = f16(|N(0,1)| * d_scale) */
-void hm_synth_q8_0(uint64_t seed, size_t n_blocks, float d_scale, uint8_t *out);
-/* n_blocks Q4_0 blocks: nibbles uniform in [0,15], d = f16(|N(0,1)| * d_scale) */
-void hm_synth_q4_0(uint64_t seed, size_t n_blocks, float d_scale, uint8_t *out);
 uint16_t hm_f32_to_bf16_rne(float v);
 uint16_t hm_f32_to_f16_rne(float v);
 
