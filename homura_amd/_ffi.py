@@ -140,6 +140,8 @@ SIGNATURES = {
     "hm_ciface_unbind": (None, []),
     "hm_kv_append": (_I, [_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I]),
     "hm_gqa_decode_attn": (_I, [_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, C.c_float]),
+    "hm_gqa_decode_attn_noalloc": (_I, [_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, C.c_float]),
+    "hm_gqa_decode_attn_noalloc_limit": (_SZ, []),
     "hm_gqa_prefill_attn": (_I, [_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, C.c_float]),
     "hm_rmsnorm": (_I, [_P, _P, _P, _P, _I, _I, C.c_float]),
     "hm_qknorm_rope": (_I, [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, C.c_float]),

@@ -23,6 +23,13 @@ struct AttnArgs {
     // the fold of its partials (the decode plan lists them as separate device launches)
     enum Phase { BOTH = 0, SPLIT_ONLY = 1, FOLD_ONLY = 2 };
     int phase = BOTH;
+    // Where the splits' partial (o, max, sum) go: the context's workspace when null.
+    float *partials = nullptr;
+    size_t partials_bytes = 0;
 };
+
+// Resolves the device address of the library's fixed partials array on the context's device
+// (called once per context by hm_init, with that device current).
+int gqa_attn_fixed_scratch_setup(hm_ctx *ctx);
 
 int gqa_decode_attn_launch(hm_ctx *ctx, const AttnArgs &a);

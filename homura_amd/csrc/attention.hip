@@ -528,7 +528,7 @@ int launch_attn(hm_ctx *ctx, const AttnArgs &a, int nsplit, int chunk) {
     const size_t front = (size_t)G * chunk;
     const size_t lds = (front + (size_t)ATT_WAVES * (WAVE / (HD / 8)) * G * HD) * sizeof(float);
     const size_t pairs = (size_t)a.B * a.kvh;
-    float *part_o = (float *)ctx->workspace;
+    float *part_o = a.partials ? a.partials : (float *)ctx->workspace;
     float *part_ml = part_o + pairs * nsplit * G * HD;
     AttnFuse f{a.qkv_raw, a.qw, a.kw, a.cos_tab, a.sin_tab, a.eps};
     if (a.phase != AttnArgs::FOLD_ONLY) {
@@ -563,7 +563,7 @@ int launch_attn_stream(hm_ctx *ctx, const AttnArgs &a, int nsplit, int chunk) {
     const size_t front = ((size_t)2 * G * IT_ROWS + 2 * G + 3) / 4 * 4;  // 16-byte rows behind it
     const size_t lds = (front + (size_t)ATT_WAVES * RPI * G * HD) * sizeof(float);
     const size_t pairs = (size_t)a.B * a.kvh;
-    float *part_o = (float *)ctx->workspace;
+    float *part_o = a.partials ? a.partials : (float *)ctx->workspace;
     float *part_ml = part_o + pairs * nsplit * G * HD;
     static bool lds_limit_raised = false;  // per instantiation
     if (lds > 64 * 1024 && !lds_limit_raised) {
@@ -617,7 +617,21 @@ int dispatch_g(hm_ctx *ctx, const AttnArgs &a, int g, int nsplit, int chunk, boo
     }
 }
 
+// Partial results of hm_gqa_decode_attn_noalloc. In host code this name is only a handle for
+// hipGetSymbolAddress; kernels get the address that call returns. Every GPU the library runs on
+// holds its own copy until the process ends.
+constexpr size_t FIXED_SCRATCH_BYTES = (size_t)4 << 20;
+static __device__ __align__(256) unsigned char fixed_scratch[FIXED_SCRATCH_BYTES];
+
 }  // namespace
+
+int gqa_attn_fixed_scratch_setup(hm_ctx *ctx) {
+    void *p = nullptr;
+    HM_HIP(ctx, hipGetSymbolAddress(&p, HIP_SYMBOL(fixed_scratch)));
+    HM_REQUIRE(ctx, p != nullptr, "gqa_decode_attn: the fixed partials array has no device address");
+    ctx->attn_fixed_scratch = p;
+    return HM_OK;
+}
 
 int gqa_decode_attn_launch(hm_ctx *ctx, const AttnArgs &a) {
     HM_REQUIRE(ctx, a.kcache && a.vcache && a.out, "gqa_decode_attn: NULL pointer");
@@ -627,6 +641,7 @@ int gqa_decode_attn_launch(hm_ctx *ctx, const AttnArgs &a) {
     HM_REQUIRE(ctx, ((uintptr_t)a.kcache % 16) == 0 && ((uintptr_t)a.vcache % 16) == 0, "gqa_decode_attn: caches must be 16-byte aligned");
     const int g = a.H / a.kvh;
     const size_t pairs = (size_t)a.B * a.kvh;
+    const size_t ws_have = a.partials ? a.partials_bytes : ctx->workspace_bytes;
     // A workgroup keeps its whole chunk in registers: 32..128 rows. Aim at about one workgroup
     // per CU over the rows that can be live.
     const int rows_step = 32;
@@ -651,7 +666,7 @@ int gqa_decode_attn_launch(hm_ctx *ctx, const AttnArgs &a) {
         HM_REQUIRE(ctx, a.q != nullptr, "gqa_decode_attn: NULL query");
         const int nsplit = (a.kv_len + chunk - 1) / chunk;
         const size_t ws_need = pairs * nsplit * g * (a.hd + 2) * sizeof(float);
-        HM_REQUIRE(ctx, ws_need <= ctx->workspace_bytes, "gqa_decode_attn: workspace too small (%zu bytes needed)", ws_need);
+        HM_REQUIRE(ctx, ws_need <= ws_have, "gqa_decode_attn: %zu bytes of partial results exceed the %zu available", ws_need, ws_have);
         if (a.hd == 128) return dispatch_g<128>(ctx, a, g, nsplit, chunk, true);
         return dispatch_g<64>(ctx, a, g, nsplit, chunk, true);
     }
@@ -666,7 +681,7 @@ int gqa_decode_attn_launch(hm_ctx *ctx, const AttnArgs &a) {
     }
     int nsplit = (span + chunk - 1) / chunk;
     const size_t ws_need = pairs * nsplit * g * (a.hd + 2) * sizeof(float);
-    HM_REQUIRE(ctx, ws_need <= ctx->workspace_bytes, "gqa_decode_attn: workspace too small (%zu bytes needed)", ws_need);
+    HM_REQUIRE(ctx, ws_need <= ws_have, "gqa_decode_attn: %zu bytes of partial results exceed the %zu available", ws_need, ws_have);
     if (a.hd == 128) return dispatch_g<128>(ctx, a, g, nsplit, chunk, false);
     return dispatch_g<64>(ctx, a, g, nsplit, chunk, false);
 }
@@ -691,6 +706,30 @@ int hm_gqa_decode_attn(hm_ctx *ctx, const float *d_q, const uint16_t *d_kcache,
     a.scale = scale;
     return gqa_decode_attn_launch(ctx, a);
 }
+
+int hm_gqa_decode_attn_noalloc(hm_ctx *ctx, const float *d_q, const uint16_t *d_kcache,
+                               const uint16_t *d_vcache, float *d_out, int B, int H, int kvh, int hd,
+                               int max_len, int kv_len, float scale) {
+    HM_CHECK_CTX(ctx);
+    HM_REQUIRE(ctx, ctx->attn_fixed_scratch != nullptr, "hm_gqa_decode_attn_noalloc: the fixed partials array was not set up");
+    AttnArgs a;
+    a.q = d_q;
+    a.kcache = d_kcache;
+    a.vcache = d_vcache;
+    a.out = d_out;
+    a.B = B;
+    a.H = H;
+    a.kvh = kvh;
+    a.hd = hd;
+    a.max_len = max_len;
+    a.kv_len = kv_len;
+    a.scale = scale;
+    a.partials = (float *)ctx->attn_fixed_scratch;
+    a.partials_bytes = FIXED_SCRATCH_BYTES;
+    return gqa_decode_attn_launch(ctx, a);
+}
+
+size_t hm_gqa_decode_attn_noalloc_limit(void) { return FIXED_SCRATCH_BYTES; }
 
 int hm_kv_append(hm_ctx *ctx, uint16_t *d_kcache, uint16_t *d_vcache, const float *d_k,
                  const float *d_v, int B, int kvh, int hd, int max_len, int pos, int n_new) {

@@ -1,5 +1,6 @@
 // Context, device memory and stream plumbing behind the C boundary.
 #include "hm_common.h"
+#include "attention.h"
 
 #include <mutex>
 
@@ -66,6 +67,11 @@ hm_ctx *hm_init(int device) {
     }
     (void)hipMemsetAsync(ctx->counters, 0, ctx->num_counters * sizeof(unsigned int), ctx->stream);
     (void)hipStreamSynchronize(ctx->stream);
+    if (gqa_attn_fixed_scratch_setup(ctx) != HM_OK) {
+        hm_set_error(nullptr, HM_ERR_HIP, "%s", ctx->last_error.c_str());
+        hm_destroy(ctx);
+        return nullptr;
+    }
     return ctx;
 }
 

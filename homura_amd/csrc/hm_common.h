@@ -21,6 +21,8 @@ struct hm_ctx {
     // 4-byte counters used by "last workgroup finishes" reductions; always left at zero.
     unsigned int *counters = nullptr;
     size_t num_counters = 0;
+    // Device address, on this context's device, of the fixed array behind hm_gqa_decode_attn_noalloc.
+    void *attn_fixed_scratch = nullptr;
     std::string last_error;
     char device_name[128] = {0};
 };

@@ -214,6 +214,11 @@ class Context:
         self._check(self.lib.hm_gqa_decode_attn(self.h, q.ptr, kc.ptr, vc.ptr, out.ptr, B, H, kvh,
                                                 hd, max_len, kv_len, scale))
 
+    def gqa_decode_attn_noalloc(self, q, kc, vc, out, B, H, kvh, hd, max_len, kv_len, scale):
+        """hm_gqa_decode_attn with the partial sums in the library's fixed array (allocates nothing)."""
+        self._check(self.lib.hm_gqa_decode_attn_noalloc(self.h, q.ptr, kc.ptr, vc.ptr, out.ptr, B, H,
+                                                        kvh, hd, max_len, kv_len, scale))
+
     def rmsnorm(self, x, w, out, rows, dim, eps):
         self._check(self.lib.hm_rmsnorm(self.h, x.ptr, w.ptr, out.ptr, rows, dim, eps))
 

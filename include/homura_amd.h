@@ -188,6 +188,19 @@ int hm_gqa_decode_attn(hm_ctx *ctx, const float *d_q, const uint16_t *d_kcache,
                        const uint16_t *d_vcache, float *d_out, int B, int H, int kvh, int hd,
                        int max_len, int kv_len, float scale);
 
+/* hm_gqa_decode_attn for callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid it). It has no counterpart in the reference. Same
+ * arguments, kernels and results; the splits' partial sums go to a fixed array inside the library
+ * (hm_gqa_decode_attn_noalloc_limit() bytes, 4 MiB, held by each GPU the library runs on until the
+ * process ends) whose device address hm_init resolves once per context. The call allocates nothing
+ * and fails with HM_ERR_INVALID when B * kv_heads * splits * (H / kv_heads) * (hd + 2) * 4 bytes exceed
+ * the limit. Nothing in the array has to start at zero (every partial is written before it is read),
+ * but all calls on one GPU share it: calls that overlap on one GPU (two streams, two contexts) race. */
+int hm_gqa_decode_attn_noalloc(hm_ctx *ctx, const float *d_q, const uint16_t *d_kcache,
+                               const uint16_t *d_vcache, float *d_out, int B, int H, int kvh, int hd,
+                               int max_len, int kv_len, float scale);
+size_t hm_gqa_decode_attn_noalloc_limit(void);
+
 /* Causal attention of S new query rows at positions past .. past + S - 1 over cache rows
  * [0, past + S), batch 1: the attention part of emit_attention_kernel (src/hf/emitter.rs:709-737)
  * under the mask of build_causal_mask (src/hf/precompute.rs:134-161: key j is visible to query i
