@@ -167,6 +167,8 @@ SIGNATURES = {
     "hm_model_whole_step_available": (_I, [_P]),
     "hm_model_whole_step_status": (_I, [_P]),
     "hm_model_whole_step_trace": (_I, [_P, _P, _I, C.POINTER(C.c_int)]),
+    "hm_model_prefill_capture_q8k_inputs": (_I, [_P, _I]),
+    "hm_model_prefill_captured_q8k_inputs": (_I, [_P, _P, _SZ]),
     "hm_model_run_kv": (_I, [_P, C.POINTER(C.c_int64), _I, c_f32_p]),
     "hm_model_prefill": (_I, [_P, C.POINTER(C.c_int64), _I, c_f32_p]),
     "hm_model_generate": (_I, [_P, C.POINTER(C.c_int64), _I, _I, C.POINTER(HmSamplingConfig), C.c_uint64, _I,

@@ -31,13 +31,15 @@ struct FusedDecodeArgs {
     int max_len;         // rows per KV head in the caches
     unsigned char *xch;  // exchange area, decode_fused_xch_bytes() bytes, zeroed once
     uint32_t *ctl;       // [0] launches so far (tag base), [1] sticky status (0 = ok), zeroed once
-    // Optional phase trace (nullptr = off): workgroup 0 stores the 100 MHz device clock at 11 points per
+    // Optional phase trace (nullptr = off; room for FUSED_TRACE_WGS workgroups x (11 n_layers + 2) entries):
+    // every workgroup stores, in its own row, the 100 MHz device clock at 11 points per
     // layer - both barriers of the Q|K|V, attention, O, gate|up and down phases, and the end of the fold
     // after attention's second barrier - followed by one entry at the end of the kernel and a last word that
     // is 1 when the step's exchanges went through the dies' L2s.
     unsigned long long *trace;
 };
 constexpr int FUSED_TRACE_PER_LAYER = 11;
+constexpr int FUSED_TRACE_WGS = 256;  // rows of the trace buffer (the largest grid of any instance)
 
 // Whether a kernel instance exists for this shape on this device; max_seq_len rows must fit the
 // attention phase's register-resident splits. `why` receives a short reason when not.

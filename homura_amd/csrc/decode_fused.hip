@@ -655,7 +655,7 @@ __device__ __forceinline__ void comm_role(const FusedDecodeArgs &a, Lds<GE> &sm,
     const uint32_t base = launches * (uint32_t)L;
     PollState ps{a.ctl, false, 0u};
     const size_t par_bytes = (size_t)GE::PAR_SLOTS * 8;
-    unsigned long long *trace = (wg == 0 && ct == 0) ? a.trace : nullptr;
+    unsigned long long *trace = (a.trace && ct == 0) ? a.trace + (size_t)wg * (L * FUSED_TRACE_PER_LAYER + 2) : nullptr;
     auto mark = [&]() {
         if (trace) *trace++ = wall_clock64();
     };
@@ -730,10 +730,7 @@ __device__ __forceinline__ void comm_role(const FusedDecodeArgs &a, Lds<GE> &sm,
     };
     // hidden <- hidden + (the vector at slot offset `off`), then stage hidden, the norm weights and this
     // wavefront's share of the sum of squares
-    auto stage_hidden = [&](unsigned char *par, int off, uint32_t tag, bool add, const float *norm_w) {
-        float nwv[NJ];
-#pragma unroll
-        for (int j = 0; j < NJ; j++) nwv[j] = ldf_global(norm_w + ct + CT * j);
+    auto stage_hidden = [&](unsigned char *par, int off, uint32_t tag, bool add, const float (&nwv)[NJ]) {
         if (add) {
             const unsigned char *src = relay(par, off, GE::HIDDEN / 2, tag);
             int unit[NJ / 2];
@@ -782,16 +779,36 @@ __device__ __forceinline__ void comm_role(const FusedDecodeArgs &a, Lds<GE> &sm,
         }
     };
 
+    // The small per-layer parameters (norm weights, bias) are requested one layer before their use, right
+    // after the barrier that ends the use of the previous layer's: a load that misses the die's L2 would
+    // otherwise sit in front of the polls of the exchange that follows it (loads return in issue order).
+    float nw_in[NJ], nw_post[NJ], bias_v = 0.f;
+    float qn_lo = 1.f, qn_hi = 1.f, kn_lo = 1.f, kn_hi = 1.f;
+    auto load_in_ln = [&](const FusedLayerPtrs &p) {
+#pragma unroll
+        for (int j = 0; j < NJ; j++) nw_in[j] = ldf_global(p.in_ln + ct + CT * j);
+        if (p.qkv_bias && ct < GE::RQ) bias_v = ldf_global(p.qkv_bias + GE::qkv_row(sp.kh, sp.split * GE::RQ + ct));
+    };
+    auto load_post_ln = [&](const FusedLayerPtrs &p) {
+#pragma unroll
+        for (int j = 0; j < NJ; j++) nw_post[j] = ldf_global(p.post_ln + ct + CT * j);
+    };
+    auto load_qk_norm = [&](const FusedLayerPtrs &p) {
+        if (p.q_norm != nullptr && lane < HD / 2) {
+            qn_lo = ldf_global(p.q_norm + lane);
+            qn_hi = ldf_global(p.q_norm + lane + HD / 2);
+            kn_lo = ldf_global(p.k_norm + lane);
+            kn_hi = ldf_global(p.k_norm + lane + HD / 2);
+        }
+    };
+    load_in_ln(sm.lp[0]);
+    load_post_ln(sm.lp[0]);
+    load_qk_norm(sm.lp[0]);
+
     for (int l = 0; l < L; l++) {
         const FusedLayerPtrs cur = sm.lp[l];
+        const FusedLayerPtrs nxt = sm.lp[l + 1 < L ? l + 1 : l];
         const bool qk_normed = cur.q_norm != nullptr;
-        float qn_lo = 1.f, qn_hi = 1.f, kn_lo = 1.f, kn_hi = 1.f;  // requested now, used in the attention phase
-        if (qk_normed && lane < HD / 2) {
-            qn_lo = ldf_global(cur.q_norm + lane);
-            qn_hi = ldf_global(cur.q_norm + lane + HD / 2);
-            kn_lo = ldf_global(cur.k_norm + lane);
-            kn_hi = ldf_global(cur.k_norm + lane + HD / 2);
-        }
         const uint32_t gl = base + (uint32_t)l;  // layers run since the exchange area was zeroed
         const uint32_t tag = gl + 1u;
         unsigned char *xc = a.xch + (size_t)(gl & 1u) * par_bytes;
@@ -801,10 +818,10 @@ __device__ __forceinline__ void comm_role(const FusedDecodeArgs &a, Lds<GE> &sm,
 
         // ── into the Q|K|V phase: hidden += down rows of the previous layer ──
         ps.where = 1u | (uint32_t)l << 4 | (uint32_t)wg << 12;
-        stage_hidden(xprev, GE::XH, tag - 1u, l > 0, cur.in_ln);
-        if (cur.qkv_bias && ct < GE::RQ)
-            sm.bias[ct] = ldf_global(cur.qkv_bias + GE::qkv_row(sp.kh, sp.split * GE::RQ + ct));
+        stage_hidden(xprev, GE::XH, tag - 1u, l > 0, nw_in);
+        if (cur.qkv_bias && ct < GE::RQ) sm.bias[ct] = bias_v;
         wg_barrier();
+        load_in_ln(nxt);
         mark();
         wg_barrier();
         mark();
@@ -856,6 +873,7 @@ __device__ __forceinline__ void comm_role(const FusedDecodeArgs &a, Lds<GE> &sm,
             }
         }
         wg_barrier();
+        load_qk_norm(nxt);
         mark();
         wg_barrier();
         mark();
@@ -937,8 +955,9 @@ __device__ __forceinline__ void comm_role(const FusedDecodeArgs &a, Lds<GE> &sm,
 
         // ── into the gate|up phase: hidden += O rows (reference src/hf/emitter.rs:787) ──
         ps.where = 5u | (uint32_t)l << 4 | (uint32_t)wg << 12;
-        stage_hidden(xc, GE::XO, tag, true, cur.post_ln);
+        stage_hidden(xc, GE::XO, tag, true, nw_post);
         wg_barrier();
+        load_post_ln(nxt);
         mark();
         wg_barrier();
         mark();
@@ -975,10 +994,9 @@ __device__ __forceinline__ void comm_role(const FusedDecodeArgs &a, Lds<GE> &sm,
         // Every workgroup read the launch count before its first exchange, and this point is only reached
         // after all of them have published their last rows.
         if (ct == 0) __hip_atomic_store(a.ctl, launches + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        mark();
-        if (trace) *trace++ = die_ok ? 1ull : 0ull;
-
     }
+    mark();
+    if (trace) *trace++ = die_ok ? 1ull : 0ull;
 }
 
 template <class GE>

@@ -180,6 +180,16 @@ int hm_model_whole_step_available(hm_model *m) {
     return m->impl->whole_step_available() ? 1 : 0;
 }
 
+int hm_model_prefill_capture_q8k_inputs(hm_model *m, int rows) {
+    if (!m) return HM_ERR_INVALID;
+    return m->impl->prefill_capture_q8k_inputs(rows);
+}
+
+int hm_model_prefill_captured_q8k_inputs(hm_model *m, float *h_out, size_t n_floats) {
+    if (!m || !h_out) return HM_ERR_INVALID;
+    return m->impl->prefill_captured_q8k_inputs(h_out, n_floats);
+}
+
 int hm_model_whole_step_trace(hm_model *m, unsigned long long *h_out, int cap, int *n_out) {
     if (!m || !n_out) return HM_ERR_INVALID;
     return m->impl->whole_step_trace(h_out, cap, n_out);

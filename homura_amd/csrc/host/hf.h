@@ -121,6 +121,10 @@ class HfModel {
     // and a final one, see decode_fused.h). Recording starts with the first call, which returns 0
     // entries; later calls return the trace of the step that ran last.
     int whole_step_trace(unsigned long long *h_out, int cap, int *n_out);
+    // Test support: keep the activation rows that the prompt pass hands to the Q8_K quantiser for the next
+    // `rows` cache positions (0 = stop and free), and copy them out (layout at PrefillScratch::capture).
+    int prefill_capture_q8k_inputs(int rows);
+    int prefill_captured_q8k_inputs(float *h_out, size_t n_floats);
     int time_kernels(int rounds, std::vector<StepProfile> &out);
     ExecutionPlan *plan() { return plan_.get(); }
 
@@ -169,6 +173,11 @@ class HfModel {
         Buffer ids, h, resid, split, qkv, proj_out, gate_up, logits;
         Buffer wsplit;  // block formats: the matrices of one group of projections as three bf16 pieces per weight
         std::vector<Buffer> wcache;  // [layer * 4 + group] resident copies of the same (q|k|v, o, gate|up, down)
+        // Tests: the f32 rows entering the Q8_K quantisation of the K-quant products, for cache positions
+        // [capture_base, capture_base + capture_rows); per layer [rows][hidden] (q|k|v), [rows][q_dim] (o),
+        // [rows][hidden] (gate|up), [rows][inter] (down).
+        Buffer capture;
+        int capture_rows = 0, capture_base = 0;
     };
     PrefillScratch pf_;
     struct SamplerScratch { Buffer work, counts, token, list; int list_cap = 0; } sampler_;

@@ -1339,22 +1339,53 @@ int HfModel::refresh_fused_table() {
     return HM_OK;
 }
 
+int HfModel::prefill_capture_q8k_inputs(int rows) {
+    PrefillScratch &p = pf_;
+    int rc = hm_sync(ctx_);
+    if (rc != HM_OK) return rc;
+    p.capture = Buffer();
+    p.capture_rows = 0;
+    if (rows <= 0) return HM_OK;
+    const TransformerConfig &c = cfg_;
+    const size_t per_row = 2 * (size_t)c.hidden_size + (size_t)c.q_dim() + c.intermediate_size;
+    const size_t n = (size_t)c.num_hidden_layers * rows * per_row;
+    p.capture = Buffer::alloc(ctx_, {(int64_t)n}, DType::F32);
+    if (!p.capture) return HM_ERR_OOM;
+    HM_HIP(ctx_, hipMemsetAsync(p.capture.ptr(), 0, n * 4, ctx_->stream));
+    p.capture_rows = rows;
+    p.capture_base = plan_->kv_cache() ? plan_->kv_cache()->current_len() : 0;
+    return hm_sync(ctx_);
+}
+
+int HfModel::prefill_captured_q8k_inputs(float *h_out, size_t n_floats) {
+    PrefillScratch &p = pf_;
+    if (!p.capture) return hm_set_error(ctx_, HM_ERR_STATE, "no activation rows were captured");
+    if (n_floats * 4 != p.capture.bytes())
+        return hm_set_error(ctx_, HM_ERR_INVALID, "captured rows: %zu floats kept, %zu asked for", p.capture.bytes() / 4, n_floats);
+    int rc = hm_sync(ctx_);
+    if (rc != HM_OK) return rc;
+    return hm_download(ctx_, h_out, p.capture.ptr(), n_floats * 4);
+}
+
 int HfModel::whole_step_trace(unsigned long long *h_out, int cap, int *n_out) {
     if (!fused_available_) return hm_set_error(ctx_, HM_ERR_STATE, "whole-step decode is not available for this model");
-    const int n = cfg_.num_hidden_layers * FUSED_TRACE_PER_LAYER + 2;
+    const int per_wg = cfg_.num_hidden_layers * FUSED_TRACE_PER_LAYER + 2;
+    const int all = per_wg * FUSED_TRACE_WGS;
     *n_out = 0;
     int rc = hm_sync(ctx_);
     if (rc != HM_OK) return rc;
     if (!scratch_->fused_trace) {
-        scratch_->fused_trace = Buffer::alloc_bytes(ctx_, (size_t)n * 8, {n}, DType::I64);
+        scratch_->fused_trace = Buffer::alloc_bytes(ctx_, (size_t)all * 8, {all}, DType::I64);
         if (!scratch_->fused_trace) return HM_ERR_OOM;
-        HM_HIP(ctx_, hipMemsetAsync(scratch_->fused_trace.ptr(), 0, (size_t)n * 8, ctx_->stream));
+        HM_HIP(ctx_, hipMemsetAsync(scratch_->fused_trace.ptr(), 0, (size_t)all * 8, ctx_->stream));
         // a captured step does not know the trace buffer yet
         const bool was = plan_->whole_step();
         if ((rc = plan_->set_whole_step(!was)) != HM_OK || (rc = plan_->set_whole_step(was)) != HM_OK) return rc;
         return hm_sync(ctx_);
     }
-    if (cap < n) return hm_set_error(ctx_, HM_ERR_INVALID, "whole_step_trace: room for %d entries, %d needed", cap, n);
+    if (cap < per_wg) return hm_set_error(ctx_, HM_ERR_INVALID, "whole_step_trace: room for %d entries, %d needed", cap, per_wg);
+    // workgroup 0's row, or every workgroup's rows when there is room for them
+    const int n = cap >= all ? all : per_wg;
     rc = hm_download(ctx_, h_out, scratch_->fused_trace.ptr(), (size_t)n * 8);
     if (rc == HM_OK) *n_out = n;
     return rc;
@@ -1477,7 +1508,13 @@ int HfModel::prefill_chunk(const int32_t *h_ids, int n, float *h_logits) {
         const int rows = std::max(n, 128);
         const int64_t widest = std::max<int64_t>(std::max(hidden, qd), inter);
         hm_sync(ctx_);
-        p = PrefillScratch();
+        {
+            PrefillScratch grown;  // a capture that a test switched on outlives the regrowth
+            grown.capture = std::move(p.capture);
+            grown.capture_rows = p.capture_rows;
+            grown.capture_base = p.capture_base;
+            p = std::move(grown);
+        }
         p.ids = Buffer::alloc(ctx_, {rows}, DType::F32);  // int32 ids
         p.h = Buffer::alloc(ctx_, {rows, hidden}, DType::F32);
         p.resid = Buffer::alloc(ctx_, {rows, hidden}, DType::F32);
@@ -1560,6 +1597,16 @@ int HfModel::prefill_chunk(const int32_t *h_ids, int n, float *h_logits) {
     };
     rc = embed_launch(ctx_, nullptr, p.ids.as<int32_t>(), weight_f32("model.embed_tokens.weight"), h, n, vocab, hidden);
     if (rc != HM_OK) return rc;
+    // where (layer, group)'s rows of this chunk go in the capture buffer, or nullptr
+    auto capture_at = [&](int l, int group) -> float * {
+        if (!p.capture) return nullptr;
+        const int r0 = past - p.capture_base;
+        if (r0 < 0 || r0 + n > p.capture_rows) return nullptr;
+        const size_t R = (size_t)p.capture_rows;
+        const size_t goff[4] = {0, R * hidden, R * (hidden + qd), R * (2 * (size_t)hidden + qd)};
+        const size_t gdim[4] = {(size_t)hidden, (size_t)qd, (size_t)hidden, (size_t)inter};
+        return p.capture.as<float>() + (size_t)l * R * (2 * (size_t)hidden + qd + inter) + goff[group] + (size_t)r0 * gdim[group];
+    };
     // The hidden state entering a layer is x [+ res]: the embedding for the first layer, afterwards the
     // post-attention residual plus the K slices of the previous down projection, which the next
     // RMSNorm kernel adds on its way (the reference's ResAdd, src/hf/emitter.rs:804).
@@ -1570,7 +1617,7 @@ int HfModel::prefill_chunk(const int32_t *h_ids, int n, float *h_logits) {
         const LayerPacked &lp = packed_[l];
         // QKV kernel (reference src/hf/emitter.rs:549-673)
         rc = rmsnorm_split_launch(ctx_, x, res, res_parts, weight_f32(pre + "input_layernorm.weight"), split, np,
-                                  res ? h : nullptr, n, hidden, eps, q8k(l, 0));
+                                  res ? h : nullptr, n, hidden, eps, q8k(l, 0), q8k(l, 0) ? capture_at(l, 0) : nullptr);
         if (rc == HM_OK) rc = project(l, 0, 3, lp.qkv, hidden, qkv);
         if (rc != HM_OK) return rc;
         QkvPostArgs qa;
@@ -1617,12 +1664,14 @@ int HfModel::prefill_chunk(const int32_t *h_ids, int n, float *h_logits) {
         aa.pieces = np;
         if ((rc = prefill_attn_launch(ctx_, aa)) != HM_OK) return rc;
         if (o_q8k && (rc = split_rows_launch(ctx_, gate_up, split, np, (size_t)n, qd, true)) != HM_OK) return rc;
+        if (o_q8k && capture_at(l, 1))
+            HM_HIP(ctx_, hipMemcpyAsync(capture_at(l, 1), gate_up, (size_t)n * qd * 4, hipMemcpyDeviceToDevice, ctx_->stream));
         if ((rc = project(l, 3, 1, lp.o, qd, proj_out)) != HM_OK) return rc;
         // MLP kernel (reference src/hf/emitter.rs:767-822); h holds the layer's input by now
         rc = rmsnorm_split_launch(ctx_, h, proj_out, parts, weight_f32(pre + "post_attention_layernorm.weight"), split, np,
-                                  resid, n, hidden, eps, q8k(l, 4));
+                                  resid, n, hidden, eps, q8k(l, 4), q8k(l, 4) ? capture_at(l, 2) : nullptr);
         if (rc == HM_OK) rc = project(l, 4, 2, lp.gate_up, hidden, gate_up);
-        if (rc == HM_OK) rc = silu_mul_split_launch(ctx_, gate_up, parts, split, np, n, inter, q8k(l, 6));
+        if (rc == HM_OK) rc = silu_mul_split_launch(ctx_, gate_up, parts, split, np, n, inter, q8k(l, 6), q8k(l, 6) ? capture_at(l, 3) : nullptr);
         if (rc == HM_OK) rc = project(l, 6, 1, lp.down, inter, proj_out);
         if (rc != HM_OK) return rc;
         x = resid;

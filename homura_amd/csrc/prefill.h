@@ -24,9 +24,10 @@ namespace homura {
 // x: [rows][dim] f32; res: [res_parts][rows][dim] or NULL.
 // q8k: the values go through the Q8_K quantisation of a K-quant product's activation first (per
 // 256-wide block of the row, dim % 256 == 0), so the split matrix holds scale * q.
+// d_pre_q8k (optional, [rows][dim] f32; tests): receives the values as they enter that quantisation.
 int rmsnorm_split_launch(hm_ctx *ctx, const float *d_x, const float *d_res, int res_parts, const float *d_w,
                          uint16_t *d_out_split, int pieces, float *d_resid_out, int rows, int dim, float eps,
-                         bool q8k = false);
+                         bool q8k = false, float *d_pre_q8k = nullptr);
 
 // out_split = split(x) (through Q8_K first with q8k); x: [rows][dim] f32, dim % 4 == 0
 int split_rows_launch(hm_ctx *ctx, const float *d_x, uint16_t *d_out_split, int pieces, size_t rows, int dim,
@@ -42,7 +43,7 @@ int dequant_split_launch(hm_ctx *ctx, int hm_dtype, const uint8_t *d_blocks, int
 // out_split = split(silu(gate) * up) for gate/up interleaved per row: gu [rows][2 * inter] =
 // (gate_0, up_0, gate_1, up_1, ...), the column order of the packed gate|up weight.
 int silu_mul_split_launch(hm_ctx *ctx, const float *d_gu, int parts, uint16_t *d_out_split, int pieces, int rows,
-                          int inter, bool q8k = false);
+                          int inter, bool q8k = false, float *d_pre_q8k = nullptr);
 
 // The tail of the reference's QKV kernel for S rows at positions past .. past + S - 1
 // (src/hf/emitter.rs:604-649): bias add, per-head QK-norm, RoPE on q and k in place, and the

@@ -129,7 +129,7 @@ __global__ __launch_bounds__(256) void rmsnorm_split_kernel(const float *__restr
                                                             int res_parts, size_t res_stride,
                                                             const float *__restrict__ w, uint16_t *__restrict__ out,
                                                             float *__restrict__ resid_out, int dim, float eps,
-                                                            int pieces, int q8k) {
+                                                            int pieces, int q8k, float *__restrict__ pre_q8k) {
     __shared__ float red[4];
     const size_t base = (size_t)blockIdx.x * dim;
     constexpr int KEEP = 2;  // rows up to 2048 wide stay in registers between the two passes
@@ -162,6 +162,7 @@ __global__ __launch_bounds__(256) void rmsnorm_split_kernel(const float *__restr
         f32x4 y;
 #pragma unroll
         for (int k = 0; k < 4; k++) y[k] = (v[k] * inv) * wv[k];
+        if (pre_q8k) *reinterpret_cast<f32x4 *>(pre_q8k + base + i) = y;
         if (q8k) y = q8k_round_trip(y);  // dim % 256 == 0: a wavefront's 256 values are one block
         split_store4(o, dim, i, y, pieces);
     }
@@ -170,7 +171,7 @@ __global__ __launch_bounds__(256) void rmsnorm_split_kernel(const float *__restr
 // silu(gate) * up (reference src/graph_builder/emit_arithmetic.rs:101-107, src/hf/emitter.rs:797-799);
 // four outputs per thread (inter % 4 == 0)
 __global__ void silu_mul_split_kernel(const float *__restrict__ gu, int parts, size_t stride, uint16_t *__restrict__ out,
-                                      int inter, size_t n, int pieces, int q8k) {
+                                      int inter, size_t n, int pieces, int q8k, float *__restrict__ pre_q8k) {
     const size_t i = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;
     if (i >= n) return;
     const size_t row = i / inter;
@@ -179,6 +180,7 @@ __global__ void silu_mul_split_kernel(const float *__restrict__ gu, int parts, s
     f32x4 y;
 #pragma unroll
     for (int k = 0; k < 4; k++) y[k] = (g[k] / (1.0f + expf(-g[k]))) * u[k];
+    if (pre_q8k) *reinterpret_cast<f32x4 *>(pre_q8k + i) = y;
     if (q8k) y = q8k_round_trip(y);
     split_store4(out + row * pieces * inter, inter, (int)(i % inter), y, pieces);
 }
@@ -526,7 +528,8 @@ __global__ __launch_bounds__(AT_THREADS) void prefill_attn_kernel(PrefillAttnArg
 namespace homura {
 
 int rmsnorm_split_launch(hm_ctx *ctx, const float *d_x, const float *d_res, int res_parts, const float *d_w,
-                         uint16_t *d_out_split, int pieces, float *d_resid_out, int rows, int dim, float eps, bool q8k) {
+                         uint16_t *d_out_split, int pieces, float *d_resid_out, int rows, int dim, float eps, bool q8k,
+                         float *d_pre_q8k) {
     HM_REQUIRE(ctx, !q8k || dim % 256 == 0, "rmsnorm_split: Q8_K activations need dim %% 256 == 0 (dim=%d)", dim);
     HM_REQUIRE(ctx, d_x && d_w && d_out_split, "rmsnorm_split: NULL pointer");
     HM_REQUIRE(ctx, rows > 0 && dim > 0 && dim % 4 == 0 && pieces >= 1 && pieces <= 3 && res_parts >= 1,
@@ -534,13 +537,13 @@ int rmsnorm_split_launch(hm_ctx *ctx, const float *d_x, const float *d_res, int 
     HM_REQUIRE(ctx, ((uintptr_t)d_x % 16) == 0 && ((uintptr_t)d_w % 16) == 0 && ((uintptr_t)d_out_split % 8) == 0 &&
                         ((uintptr_t)d_res % 16) == 0 && ((uintptr_t)d_resid_out % 16) == 0, "rmsnorm_split: misaligned buffer");
     hipLaunchKernelGGL(rmsnorm_split_kernel, dim3(rows), dim3(256), 0, ctx->stream, d_x, d_res, res_parts,
-                       (size_t)rows * dim, d_w, d_out_split, d_resid_out, dim, eps, pieces, q8k ? 1 : 0);
+                       (size_t)rows * dim, d_w, d_out_split, d_resid_out, dim, eps, pieces, q8k ? 1 : 0, d_pre_q8k);
     HM_LAUNCH_CHECK(ctx);
     return HM_OK;
 }
 
 int silu_mul_split_launch(hm_ctx *ctx, const float *d_gu, int parts, uint16_t *d_out_split, int pieces, int rows,
-                          int inter, bool q8k) {
+                          int inter, bool q8k, float *d_pre_q8k) {
     HM_REQUIRE(ctx, !q8k || inter % 256 == 0, "silu_mul_split: Q8_K activations need a width %% 256 == 0 (%d)", inter);
     HM_REQUIRE(ctx, d_gu && d_out_split, "silu_mul_split: NULL pointer");
     HM_REQUIRE(ctx, rows > 0 && inter > 0 && inter % 4 == 0 && pieces >= 1 && pieces <= 3 && parts >= 1,
@@ -548,7 +551,7 @@ int silu_mul_split_launch(hm_ctx *ctx, const float *d_gu, int parts, uint16_t *d
     HM_REQUIRE(ctx, ((uintptr_t)d_gu % 16) == 0 && ((uintptr_t)d_out_split % 8) == 0, "silu_mul_split: misaligned buffer");
     const size_t n = (size_t)rows * inter;
     hipLaunchKernelGGL(silu_mul_split_kernel, dim3((unsigned)((n / 4 + 255) / 256)), dim3(256), 0, ctx->stream, d_gu, parts,
-                       2 * n, d_out_split, inter, n, pieces, q8k ? 1 : 0);
+                       2 * n, d_out_split, inter, n, pieces, q8k ? 1 : 0, d_pre_q8k);
     HM_LAUNCH_CHECK(ctx);
     return HM_OK;
 }

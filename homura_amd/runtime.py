@@ -431,15 +431,31 @@ class HfModel:
         """Raises if a whole-step launch left an error behind (an exchange that timed out)."""
         self._check(self.lib.hm_model_whole_step_status(self.h))
 
-    def whole_step_trace(self) -> np.ndarray:
+    def whole_step_trace(self, all_workgroups: bool = False) -> np.ndarray:
         """Device-clock ticks (100 MHz) of the latest whole-step launch: 11 per layer (both barriers of the
         Q|K|V, attention, O, gate|up and down phases; the fold's end comes after attention's) and a final
-        one. The first call only switches recording on and returns an empty array."""
-        cap = 64 * 11 + 2
+        one. The first call only switches recording on and returns an empty array. With all_workgroups
+        the rows of all 256 workgroup slots come back (rows of workgroups the grid does not have stay 0)."""
+        cap = (64 * 11 + 2) * (256 if all_workgroups else 1)
         out = np.zeros(cap, dtype=np.uint64)
         n = C.c_int(0)
         self._check(self.lib.hm_model_whole_step_trace(self.h, out.ctypes.data, cap, C.byref(n)))
         return out[:n.value]
+
+    def prefill_capture_q8k_inputs(self, rows: int):
+        """Test support: keep the rows the prompt pass hands to the Q8_K quantiser for the next `rows`
+        cache positions (0 = stop)."""
+        self._check(self.lib.hm_model_prefill_capture_q8k_inputs(self.h, rows))
+        self._capture_rows = rows
+
+    def prefill_captured_q8k_inputs(self) -> np.ndarray:
+        """Those rows: per layer [rows][hidden], [rows][q_dim], [rows][hidden], [rows][inter], flat f32."""
+        c = self.config
+        n = c.num_hidden_layers * self._capture_rows * (
+            2 * c.hidden_size + c.num_attention_heads * c.get_head_dim() + c.intermediate_size)
+        out = np.zeros(n, np.float32)
+        self._check(self.lib.hm_model_prefill_captured_q8k_inputs(self.h, out.ctypes.data, n))
+        return out
 
     def reset_kv_cache(self):
         self._check(self.lib.hm_model_reset_kv_cache(self.h))

@@ -49,8 +49,19 @@ void hm_synth_q4_0(uint64_t seed, size_t n_blocks, float d_scale, uint8_t *out);
  * phases; the end of the fold follows attention's second barrier) and one at the end of the kernel, then
  * a word that is 1 when the step found its workgroups dealt round-robin to the dies and used die-local
  * exchanges. The first call switches recording on and stores 0 in *n_out; later calls copy
- * layers * 11 + 2 entries of the step that ran last. */
+ * layers * 11 + 2 entries of the step that ran last (workgroup 0's), or, when cap has room for 256
+ * times as many, one such row per workgroup (256 rows; those of workgroups the grid lacks stay 0). */
 int hm_model_whole_step_trace(hm_model *m, unsigned long long *h_out, int cap, int *n_out);
+
+/* Test support for block-quantised models with K-quant projections: keep the f32 activation rows that the
+ * prompt pass hands to the Q8_K quantiser (reference emit_quant.rs:422-466) for the next `rows` cache
+ * positions (0 = stop, free the buffer), and copy them to the host afterwards. Per layer: [rows][hidden]
+ * (input of q|k|v), [rows][heads * head_dim] (o), [rows][hidden] (gate|up), [rows][intermediate] (down);
+ * rows of groups whose matrices are not K-quants stay zero. A checker can then quantise the very values
+ * the GPU quantised, so that a rounding decision taken differently on the two sides is counted instead of
+ * being seen as an error. */
+int hm_model_prefill_capture_q8k_inputs(hm_model *m, int rows);
+int hm_model_prefill_captured_q8k_inputs(hm_model *m, float *h_out, size_t n_floats);
 
 #pragma GCC visibility pop
 #ifdef __cplusplus

@@ -941,6 +941,13 @@ typedef struct {
     float *h, *normed, *q, *k, *v, *attn_flat, *attn_out, *resid, *gate, *up, *act, *down,
         *scores, *mask;
     int scratch_seq, scratch_total;
+    /* Test device (no counterpart in the reference): activation rows handed in from outside that the
+     * K-quant products quantise instead of the model's own rows, see orc_model_set_q8k_inputs. */
+    const float *sub;
+    float *sub_capture; /* when set, the model's own rows are written here instead (same layout) */
+    int sub_rows, sub_base_pos;
+    long long sub_blocks, sub_flips;
+    float sub_maxdiff;
 } orc_model;
 
 ORC_API orc_model *orc_model_new(const orc_config *cfg) {
@@ -996,6 +1003,38 @@ ORC_API void orc_model_set_layer_kinds(orc_model *m, int l, const int *kinds) {
     memcpy(m->layers[l].kinds, kinds, sizeof(m->layers[l].kinds));
 }
 
+/* Test device for comparing against an implementation whose activations differ from this model's in the
+ * last bits. Q8_K is a step function: where the two sides round an activation to different integers the
+ * outputs differ by 1/127 of the block's largest value although both are right. With rows handed in here
+ * the K-quant products (kinds Q4_K / Q6_K) of cache positions [base_pos, base_pos + rows) quantise the
+ * OTHER side's activations, so both sides multiply the same integers, and the model keeps count of
+ * what that hid: blocks seen, quantised values that its own activations would have rounded differently
+ * (flips) and the largest |own - given| / amax of a block. Layout, f32, per layer: [rows][hidden] input of
+ * q|k|v, [rows][heads * head_dim] input of o, [rows][hidden] input of gate|up, [rows][inter] input of
+ * down. sub = NULL switches it off. */
+ORC_API void orc_model_set_q8k_inputs(orc_model *m, const float *sub, int rows, int base_pos) {
+    m->sub = sub;
+    m->sub_capture = NULL;
+    m->sub_rows = rows;
+    m->sub_base_pos = base_pos;
+    m->sub_blocks = m->sub_flips = 0;
+    m->sub_maxdiff = 0.0f;
+}
+
+/* The reverse: the model writes the rows its K-quant products quantise into dst (same layout), so a
+ * test can hand a model its own activations back and must then see identical results and no flips. */
+ORC_API void orc_model_capture_q8k_inputs(orc_model *m, float *dst, int rows, int base_pos) {
+    orc_model_set_q8k_inputs(m, dst, rows, base_pos);
+    m->sub_capture = dst;
+}
+
+ORC_API void orc_model_q8k_input_stats(const orc_model *m, long long *blocks, long long *flips,
+                                       float *maxdiff) {
+    *blocks = m->sub_blocks;
+    *flips = m->sub_flips;
+    *maxdiff = m->sub_maxdiff;
+}
+
 /* q = emit_add(q, bias): the bias row broadcast over the sequence (src/hf/emitter.rs:604-619;
  * quantised plan: emit_post_qkv_kernel, src/hf/emitter_quant.rs:802-912). */
 static void add_bias(float *x, const float *bias, int S, int n) {
@@ -1043,6 +1082,59 @@ static void ensure_scratch(orc_model *m, int S, int total) {
     m->mask = (float *)malloc(s * total * 4);
     m->scratch_seq = S;
     m->scratch_total = total;
+}
+
+static void proj(const orc_model *m, int kind, const float *x, const void *w, float *out, int M,
+                 int K, int N);
+
+/* proj for projection `group` (0 q|k|v, 1 o, 2 gate|up, 3 down) of layer l at cache positions
+ * past .. past + M - 1, with the handed-in activation rows where there are any */
+static void proj_at(orc_model *m, int l, int group, int past, int count_stats, int kind, const float *x,
+                    const void *w, float *out, int M, int K, int N) {
+    int kk = kind ? kind : m->cfg.weight_kind;
+    if (!m->sub || (kk != ORC_W_Q4_K && kk != ORC_W_Q6_K)) {
+        proj(m, kind, x, w, out, M, K, N);
+        return;
+    }
+    const orc_config *c = &m->cfg;
+    int qd = c->heads * c->head_dim;
+    size_t per_layer = (size_t)m->sub_rows * (2 * (size_t)c->hidden + qd + c->inter);
+    size_t goff[4] = {0, (size_t)m->sub_rows * c->hidden, (size_t)m->sub_rows * (c->hidden + qd),
+                      (size_t)m->sub_rows * (2 * (size_t)c->hidden + qd)};
+    const float *base = m->sub + (size_t)l * per_layer + goff[group];
+    float *xs = (float *)malloc((size_t)M * K * 4);
+    memcpy(xs, x, (size_t)M * K * 4);
+    for (int r = 0; r < M; r++) {
+        int idx = past + r - m->sub_base_pos;
+        if (idx < 0 || idx >= m->sub_rows) continue;
+        const float *given = base + (size_t)idx * K;
+        if (m->sub_capture) {
+            memcpy(m->sub_capture + (given - m->sub), x + (size_t)r * K, (size_t)K * 4);
+            continue;
+        }
+        if (count_stats) {
+            for (int kb = 0; kb < K / 256; kb++) {
+                int8_t qa[256], qb[256];
+                float da, db;
+                int32_t bs[16];
+                orc_quantize_q8_k(x + (size_t)r * K + kb * 256, qa, &da, bs);
+                orc_quantize_q8_k(given + kb * 256, qb, &db, bs);
+                float amax = da * 127.0f, worst = 0.0f;
+                for (int i = 0; i < 256; i++) {
+                    if (qa[i] != qb[i]) m->sub_flips++;
+                    float d = fabsf(x[(size_t)r * K + kb * 256 + i] - given[kb * 256 + i]);
+                    worst = worst > d ? worst : d;
+                }
+                if (amax > 0.0f) worst /= amax;
+                /* a NaN must not pass as "no difference" */
+                if (!(worst <= m->sub_maxdiff)) m->sub_maxdiff = worst;
+                m->sub_blocks++;
+            }
+        }
+        memcpy(xs + (size_t)r * K, given, (size_t)K * 4);
+    }
+    proj(m, kind, xs, w, out, M, K, N);
+    free(xs);
 }
 
 static void proj(const orc_model *m, int kind, const float *x, const void *w, float *out, int M,
@@ -1094,9 +1186,9 @@ ORC_API int orc_model_run_kv(orc_model *m, const int64_t *ids, int S, float *log
             orc_rms_norm_f64acc(m->h, w->input_ln, m->normed, S, c->hidden, c->eps);
         else
             orc_rms_norm(m->h, w->input_ln, m->normed, S, c->hidden, c->eps);
-        proj(m, w->kinds[0], m->normed, w->q, m->q, S, c->hidden, qd);
-        proj(m, w->kinds[1], m->normed, w->k, m->k, S, c->hidden, kvd);
-        proj(m, w->kinds[2], m->normed, w->v, m->v, S, c->hidden, kvd);
+        proj_at(m, l, 0, past, 1, w->kinds[0], m->normed, w->q, m->q, S, c->hidden, qd);
+        proj_at(m, l, 0, past, 0, w->kinds[1], m->normed, w->k, m->k, S, c->hidden, kvd);
+        proj_at(m, l, 0, past, 0, w->kinds[2], m->normed, w->v, m->v, S, c->hidden, kvd);
         add_bias(m->q, w->q_bias, S, qd);
         add_bias(m->k, w->k_bias, S, kvd);
         add_bias(m->v, w->v_bias, S, kvd);
@@ -1122,7 +1214,7 @@ ORC_API int orc_model_run_kv(orc_model *m, const int64_t *ids, int S, float *log
         orc_gqa_attention(m->q, orc_kv_key_ptr(kv, l), orc_kv_value_ptr(kv, l), m->mask,
                           m->attn_flat, S, c->heads, c->kv_heads, hd, total,
                           orc_kv_head_stride(kv), quant, m->scores);
-        proj(m, w->kinds[3], m->attn_flat, w->o, m->attn_out, S, qd, c->hidden);
+        proj_at(m, l, 1, past, 1, w->kinds[3], m->attn_flat, w->o, m->attn_out, S, qd, c->hidden);
         /* MLP kernel: src/hf/emitter.rs:767-822 (quant: Residual+Norm :985-1071, QuantMM
          * gate/up, SiLU*Up :1077-1103, QuantMM down, ResAdd :1109-1134) */
         orc_add(m->h, m->attn_out, m->resid, (size_t)S * c->hidden);
@@ -1130,10 +1222,10 @@ ORC_API int orc_model_run_kv(orc_model *m, const int64_t *ids, int S, float *log
             orc_rms_norm_f64acc(m->resid, w->post_ln, m->normed, S, c->hidden, c->eps);
         else
             orc_rms_norm(m->resid, w->post_ln, m->normed, S, c->hidden, c->eps);
-        proj(m, w->kinds[4], m->normed, w->gate, m->gate, S, c->hidden, c->inter);
-        proj(m, w->kinds[5], m->normed, w->up, m->up, S, c->hidden, c->inter);
+        proj_at(m, l, 2, past, 1, w->kinds[4], m->normed, w->gate, m->gate, S, c->hidden, c->inter);
+        proj_at(m, l, 2, past, 0, w->kinds[5], m->normed, w->up, m->up, S, c->hidden, c->inter);
         orc_silu_mul(m->gate, m->up, m->act, (size_t)S * c->inter);
-        proj(m, w->kinds[6], m->act, w->down, m->down, S, c->inter, c->hidden);
+        proj_at(m, l, 3, past, 1, w->kinds[6], m->act, w->down, m->down, S, c->inter, c->hidden);
         orc_add(m->resid, m->down, m->h, (size_t)S * c->hidden);
     }
     /* LM head: src/hf/emitter.rs:828-862 (bf16 weights, f32 RMSNorm); the quantised plan

@@ -104,6 +104,9 @@ def load() -> C.CDLL:
         "orc_model_attach_kv": (None, [_P, _P]),
         "orc_model_free": (None, [_P]),
         "orc_model_run_kv": (_I, [_P, _P, _I, _P]),
+        "orc_model_set_q8k_inputs": (None, [_P, _P, _I, _I]),
+        "orc_model_capture_q8k_inputs": (None, [_P, _P, _I, _I]),
+        "orc_model_q8k_input_stats": (None, [_P, C.POINTER(C.c_longlong), C.POINTER(C.c_longlong), C.POINTER(C.c_float)]),
         "orc_generate_greedy": (_I, [_P, _P, _I, _I, _P, _P]),
         "orc_num_threads": (_I, []),
         "orc_rng_seed": (C.c_uint64, [C.c_uint64]),
@@ -411,6 +414,37 @@ class Model:
         """W_* of q, k, v, o, gate, up, down for a layer whose projections differ in block type."""
         assert len(kinds) == 7
         self.lib.orc_model_set_layer_kinds(self.h, l, (C.c_int * 7)(*[int(k) for k in kinds]))
+
+    def q8k_inputs_size(self, rows):
+        """Floats of the activation rows that the K-quant products of `rows` cache positions quantise
+        (per layer: q|k|v input, o input, gate|up input, down input)."""
+        c = self.cfg
+        return c.layers * rows * (2 * c.hidden + c.heads * c.head_dim + c.inter)
+
+    def set_q8k_inputs(self, rows_f32, rows, base_pos):
+        """K-quant products of cache positions [base_pos, base_pos + rows) quantise these rows instead of
+        the model's own (None switches it off). See orc_model_set_q8k_inputs."""
+        if rows_f32 is None:
+            self.lib.orc_model_set_q8k_inputs(self.h, None, 0, 0)
+            return
+        a = np.ascontiguousarray(rows_f32, np.float32).reshape(-1)
+        assert a.size == self.q8k_inputs_size(rows)
+        self._q8k_rows = a
+        self.lib.orc_model_set_q8k_inputs(self.h, _p(a), rows, base_pos)
+
+    def capture_q8k_inputs(self, rows, base_pos):
+        """The model's own rows of those positions are written to the returned array as it runs."""
+        a = np.zeros(self.q8k_inputs_size(rows), np.float32)
+        self._q8k_rows = a
+        self.lib.orc_model_capture_q8k_inputs(self.h, _p(a), rows, base_pos)
+        return a
+
+    def q8k_input_stats(self):
+        """(blocks quantised from handed-in rows, values the model's own rows would have rounded
+        differently, largest |own - given| / amax of a block)"""
+        b, f, d = C.c_longlong(0), C.c_longlong(0), C.c_float(0)
+        self.lib.orc_model_q8k_input_stats(self.h, C.byref(b), C.byref(f), C.byref(d))
+        return b.value, f.value, d.value
 
     def run_kv(self, ids):
         ids = np.ascontiguousarray(ids, np.int64).reshape(-1)

@@ -184,6 +184,46 @@ def test_quantised_plan_against_oracle(ctx, wdt, name):
     gm.close()
 
 
+@pytest.mark.parametrize("name", ["q8_0", "q4_0", "q4_k_m_mix"])
+def test_qwen3_0p6b_shape_quantised_decode_against_oracle(ctx, name):
+    """The quantised decode plans at the shape bench.py times them on (Qwen3-0.6B widths, 28 layers, untied
+    f32 LM head, cache pre-filled to 1024 rows): first-step logits and 16 greedy tokens against the oracle.
+    Q8_0 / Q4_0 have no step function besides the bf16 cache rounding: tokens identical. The Q4_K_M-style
+    mix quantises its activations to Q8_K on both sides independently; tokens are compared while the
+    oracle's lead of the best logit exceeds what rounding decisions taken differently move two logits by at
+    this width (measured worst row 2e-4 of the logit scale; allowed 1e-3 each)."""
+    import dataclasses
+    from homura_amd.runtime import DTYPE_Q4_0, DTYPE_Q8_0
+    cfg = dataclasses.replace(synth_model.QWEN3_0P6B, tie_word_embeddings=False)
+    mix = synth_model.q4_k_m_mix(cfg) if name == "q4_k_m_mix" else None
+    wdt = {"q8_0": DTYPE_Q8_0, "q4_0": DTYPE_Q4_0, "q4_k_m_mix": DTYPE_Q8_0}[name]
+    say(f"{name}: synthesising weights")
+    weights = synth_model.synth_weights(cfg, synth.SEED_CFG2 + 7, wdt, has_qk_norm=True, proj_dtypes=mix)
+    kv = synth_model.synth_kv(cfg, synth.SEED_CFG2 + 0x100, 1024)
+    gm = synth_model.build_model(ctx, cfg, weights, 1200, wdt, has_qk_norm=True, proj_dtypes=mix)
+    om = mf.build_oracle_model(cfg, weights, 1200, wdt, has_qk_norm=True, proj_dtypes=mix)
+    gm.init_kv_cache(kv, 1024)
+    mf.oracle_init_kv(om, kv)
+    gm.set_graph(True)
+    gm.set_prefill_min(0)
+    ids = synth.token_ids(synth.SEED_CFG2 + 0x200, 3, cfg.vocab_size)
+    got = gm.run_kv(ids[:1])
+    want = om.run_kv(ids[:1])
+    err = mf.rel_err(got, want)
+    say(f"{name}: first-step logits rel err {err:.2e}")
+    assert err < 1e-2
+    want_t, margins = om.generate_greedy(ids[1:], 16)
+    got_t = gm.generate_greedy(ids[1:], 16)
+    scale = float(np.abs(want).max())
+    thr = 2 * 1e-3 * scale if mix is not None else 0.0
+    close = np.nonzero(margins < thr)[0]
+    n_cmp = int(close[0]) if close.size else len(want_t)
+    say(f"{name}: min margin {margins.min():.3e} (logit scale {scale:.3e}), {n_cmp} of 16 tokens compared")
+    assert n_cmp >= 8
+    assert np.array_equal(got_t[:n_cmp], want_t[:n_cmp])
+    gm.close()
+
+
 @pytest.mark.parametrize("wdt,name", [(1, "bf16"), (2, "q8_0")])
 def test_qkv_bias_model_against_oracle(ctx, wdt, name):
     """Qwen2-style checkpoint: Q/K/V biases (slots q,[qb],k,[kb],v,[vb] of the reference's

@@ -245,3 +245,68 @@ def test_mixed_kquant_oracle_step_against_numpy_fp64():
     want = rms(h, f(W["model.norm.weight"])) @ f(W["lm_head.weight"])
     assert np.abs(want).max() > 1e-3
     assert mf.rel_err(got, want) < 2e-3
+
+
+def test_q8k_activation_hand_in_is_pinned():
+    """The oracle's test device for K-quant comparisons (orc_model_set_q8k_inputs): K-quant products
+    quantise activation rows handed in from outside. Pinned here by what it must do on the oracle's own
+    rows: handing a model its own activations back changes nothing and reports no flip; one value pushed
+    across a Q8_K rounding boundary is counted as exactly one flip per product group that sees it and
+    moves the logits; a value moved by less than the distance to its boundary is no flip but shows in
+    the largest difference; rows outside the handed-in range keep the model's own activations."""
+    import pyoracle
+    cfg = synth_model.TINY_K
+    mix = synth_model.q4_k_m_mix(cfg)
+    W = synth_model.synth_weights(cfg, 33, has_qk_norm=False, proj_dtypes=mix)
+    ids = synth.token_ids(5, 6, cfg.vocab_size)
+
+    def fresh():
+        return mf.build_oracle_model(cfg, W, 32, has_qk_norm=False, proj_dtypes=mix)
+
+    a = fresh()
+    rows = a.capture_q8k_inputs(4, 1)           # positions 1..4 of 0..5
+    want = np.concatenate([a.run_kv(ids[i:i + 1]) for i in range(6)])
+    rows = rows.copy()
+    assert np.abs(rows).max() > 0
+    plain = fresh()
+    assert np.array_equal(np.concatenate([plain.run_kv(ids[i:i + 1]) for i in range(6)]), want)  # capture changes nothing
+
+    b = fresh()
+    b.set_q8k_inputs(rows, 4, 1)
+    got = np.concatenate([b.run_kv(ids[i:i + 1]) for i in range(6)])
+    blocks, flips, maxdiff = b.q8k_input_stats()
+    c = cfg
+    per_row = (2 * c.hidden_size + c.num_attention_heads * c.get_head_dim() + c.intermediate_size) // 256
+    assert blocks == c.num_hidden_layers * 4 * per_row and flips == 0 and maxdiff == 0.0
+    assert np.array_equal(got, want)
+
+    # layer 0, q|k|v input, handed-in row 2 (position 3): push one value across its rounding boundary
+    hidden = c.hidden_size
+    blk = rows[2 * hidden:2 * hidden + 256].copy()
+    q, d, _ = pyoracle.quantize_q8_k(blk)
+    j = int(np.argsort(np.abs(blk))[128])        # a mid-sized value, not the block maximum
+    moved = rows.copy()
+    moved[2 * hidden + j] = np.float32((int(q[j]) + (0.75 if q[j] >= 0 else -0.75)) * d)
+    q2, d2, _ = pyoracle.quantize_q8_k(moved[2 * hidden:2 * hidden + 256])
+    assert d2 == d and (q2 != q).sum() == 1 and abs(int(q2[j]) - int(q[j])) == 1
+    m = fresh()
+    m.set_q8k_inputs(moved, 4, 1)
+    got2 = np.concatenate([m.run_kv(ids[i:i + 1]) for i in range(6)])
+    blocks2, flips2, maxdiff2 = m.q8k_input_stats()
+    # The moved value is counted, and so is what it does to the model's own later activations of that
+    # position (the handed-in rows come from a run without the move): the difference is reported.
+    assert flips2 >= 1 and maxdiff2 > 0.2 / 127
+    # Every projection of positions 1..4 multiplies the handed-in rows, so their logits are those of the
+    # captured run; the moved value lives on in K and V of position 3 and reaches position 5, which
+    # attends to it and has no hand-in.
+    assert np.array_equal(got2[:5], want[:5])
+    assert not np.array_equal(got2[5], want[5])
+
+    # a nudge far smaller than the distance to the boundary: no flip, but visible in the difference
+    nudged = rows.copy()
+    nudged[2 * hidden + j] = np.float32(blk[j] * (1 + 3e-7))
+    n = fresh()
+    n.set_q8k_inputs(nudged, 4, 1)
+    np.concatenate([n.run_kv(ids[i:i + 1]) for i in range(6)])
+    _, flips3, maxdiff3 = n.q8k_input_stats()
+    assert flips3 == 0 and 0 < maxdiff3 < 1e-6
