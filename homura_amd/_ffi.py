@@ -138,6 +138,8 @@ SIGNATURES = {
     "hm_ciface_bind_transformer_quant": (_I, [_P, _P, _P, _I]),
     "hm_ciface_num_kernels": (_I, []),
     "hm_ciface_unbind": (None, []),
+    "hm_ciface_last_status": (_I, [C.POINTER(C.c_int)]),
+    "hm_ciface_clear_status": (None, []),
     "hm_kv_append": (_I, [_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I]),
     "hm_gqa_decode_attn": (_I, [_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, C.c_float]),
     "hm_gqa_decode_attn_noalloc": (_I, [_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, C.c_float]),

@@ -17,6 +17,15 @@
 // raw GGUF blocks), the KV views are the reference's f32 cache (copied to a bf16 scratch cache per
 // call), and every reference kernel becomes one or several launches. The model-level API is the
 // fast path.
+//
+// A call may carry any number of tokens (the reference's prefill hands the whole prompt to the same
+// kernels, src/hf/model.rs:321-336): matrix products go through the GEMVs in blocks of up to eight rows,
+// attention with more than one query row through the causal prompt kernel, which applies the mask of
+// build_causal_mask (src/hf/precompute.rs:134-161) by position instead of reading the mask operand.
+//
+// The ABI returns void. A failing call prints a line, fills every output operand with NaN (all-ones
+// bytes), and leaves its code in a sticky status word that hm_ciface_last_status() reads and
+// hm_ciface_clear_status() resets.
 #include <cmath>
 #include <cstdio>
 #include <vector>
@@ -62,9 +71,16 @@ MemRef memref(void **args, int i, int rank) {
     return m;
 }
 
+int g_status = HM_OK;       // first failure since the last hm_ciface_clear_status
+int g_status_kernel = -1;
+
 // The reference's kernels return void: a failure is recorded on the context and reported here.
 void report(int idx, int rc) {
     if (rc == HM_OK) return;
+    if (g_status == HM_OK) {
+        g_status = rc;
+        g_status_kernel = idx;
+    }
     std::fprintf(stderr, "homura_amd: _mlir__mlir_ciface_k%d failed (%d): %s\n", idx, rc,
                  g_bound.ctx ? hm_last_error(g_bound.ctx) : "no transformer bound");
 }
@@ -108,10 +124,48 @@ __global__ void kv_view_to_bf16_kernel(const float *__restrict__ src, int64_t he
     dst[i] = f32_to_bf16_rne_dev(src[head * head_stride + (size_t)row * row_stride + d]);
 }
 
-int need_single_token(hm_ctx *ctx, int64_t seq, const char *what) {
-    if (seq == 1) return HM_OK;
-    return hm_set_error(ctx, HM_ERR_INVALID, "%s: the memref entry points take one token per call (seq = %lld)",
-                        what, (long long)seq);
+__global__ void add_bias_rows_kernel(float *__restrict__ x, const float *__restrict__ bias, int n, size_t total) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < total) x[i] = x[i] + bias[i % n];
+}
+
+// [S][heads][hd] -> [heads][S][hd] (the BSHD -> BHSD transposes of src/hf/emitter.rs:648-649)
+__global__ void bshd_to_bhsd_kernel(const float *__restrict__ src, float *__restrict__ dst, int S, int heads, int hd,
+                                    size_t total) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= total) return;
+    const int d = (int)(i % hd);
+    const size_t r = i / hd;
+    const int h = (int)(r % heads);
+    const size_t sq = r / heads;
+    dst[((size_t)h * S + sq) * hd + d] = src[i];
+}
+
+int seq_ok(hm_ctx *ctx, int64_t seq, const char *what) {
+    if (seq >= 1 && seq <= (1 << 20)) return HM_OK;
+    return hm_set_error(ctx, HM_ERR_INVALID, "%s: %lld tokens in one call", what, (long long)seq);
+}
+
+int add_bias_rows(hm_ctx *ctx, float *x, const float *bias, int rows, int n) {
+    const size_t total = (size_t)rows * n;
+    hipLaunchKernelGGL(add_bias_rows_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, ctx->stream, x, bias, n, total);
+    HM_LAUNCH_CHECK(ctx);
+    return HM_OK;
+}
+
+int bshd_to_bhsd(hm_ctx *ctx, const float *src, float *dst, int S, int heads, int hd) {
+    const size_t total = (size_t)S * heads * hd;
+    hipLaunchKernelGGL(bshd_to_bhsd_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, ctx->stream, src, dst, S, heads,
+                       hd, total);
+    HM_LAUNCH_CHECK(ctx);
+    return HM_OK;
+}
+
+// out [S][N] = x [S][K] times a [K,N] bf16 matrix: the batch-1 kernel takes up to eight rows a launch
+int rows_gemv_bf16(hm_ctx *ctx, const float *x, const uint16_t *w, float *out, int S, int K, int N) {
+    for (int r = 0; r < S; r += 8)
+        TRY(hm_gemv_bf16(ctx, x + (size_t)r * K, w, out + (size_t)r * N, S - r < 8 ? S - r : 8, K, N));
+    return HM_OK;
 }
 
 // emit_embed_kernel (src/hf/emitter.rs:506-537): ids [1,S] i64, table [V,H] f32 -> [1,S,H]
@@ -142,52 +196,46 @@ int run_qkv(void **a) {
         kn = memref(a, i++, 1).as<float>();
     }
     const MemRef q = memref(a, i++, 4), k = memref(a, i++, 4), v = memref(a, i++, 4);
-    TRY(need_single_token(ctx, h.sizes[1], "QKV kernel"));
+    const int S = (int)h.sizes[1], H = b.cfg.num_attention_heads;
+    TRY(seq_ok(ctx, h.sizes[1], "QKV kernel"));
     Scratch s(ctx);
-    float *normed = s.take<float>(hidden);
-    if (!normed) return hm_set_error(ctx, HM_ERR_OOM, "QKV kernel: workspace too small");
-    TRY(hm_rmsnorm(ctx, h.as<float>(), ln.as<float>(), normed, 1, hidden, (float)b.cfg.rms_norm_eps));
-    TRY(hm_gemv_bf16(ctx, normed, qw.as<uint16_t>(), q.as<float>(), 1, hidden, b.q_dim));
-    TRY(hm_gemv_bf16(ctx, normed, kw.as<uint16_t>(), k.as<float>(), 1, hidden, b.kv_dim));
-    TRY(hm_gemv_bf16(ctx, normed, vw.as<uint16_t>(), v.as<float>(), 1, hidden, b.kv_dim));
+    float *normed = s.take<float>((size_t)S * hidden);
+    // more than one token: k and v are projected as [S][kvh][hd] rows and transposed into the outputs
+    float *krows = S > 1 ? s.take<float>((size_t)S * b.kv_dim) : k.as<float>();
+    float *vrows = S > 1 ? s.take<float>((size_t)S * b.kv_dim) : v.as<float>();
+    if (!normed || !krows || !vrows) return hm_set_error(ctx, HM_ERR_OOM, "QKV kernel: workspace too small for %d tokens", S);
+    TRY(hm_rmsnorm(ctx, h.as<float>(), ln.as<float>(), normed, S, hidden, (float)b.cfg.rms_norm_eps));
+    TRY(rows_gemv_bf16(ctx, normed, qw.as<uint16_t>(), q.as<float>(), S, hidden, b.q_dim));
+    TRY(rows_gemv_bf16(ctx, normed, kw.as<uint16_t>(), krows, S, hidden, b.kv_dim));
+    TRY(rows_gemv_bf16(ctx, normed, vw.as<uint16_t>(), vrows, S, hidden, b.kv_dim));
     if (bias) {
-        TRY(hm_add(ctx, q.as<float>(), qb, q.as<float>(), (size_t)b.q_dim));
-        TRY(hm_add(ctx, k.as<float>(), kb, k.as<float>(), (size_t)b.kv_dim));
-        TRY(hm_add(ctx, v.as<float>(), vb, v.as<float>(), (size_t)b.kv_dim));
+        TRY(add_bias_rows(ctx, q.as<float>(), qb, S, b.q_dim));
+        TRY(add_bias_rows(ctx, krows, kb, S, b.kv_dim));
+        TRY(add_bias_rows(ctx, vrows, vb, S, b.kv_dim));
     }
-    // with one token the BSHD rows and the BHSD outputs coincide
-    return hm_qknorm_rope(ctx, q.as<float>(), k.as<float>(), qn, kn, cosv.as<float>(), sinv.as<float>(), 1,
-                          b.cfg.num_attention_heads, b.kv_heads, b.head_dim, (float)b.cfg.rms_norm_eps);
+    TRY(hm_qknorm_rope(ctx, q.as<float>(), krows, qn, kn, cosv.as<float>(), sinv.as<float>(), S, H, b.kv_heads, b.head_dim,
+                       (float)b.cfg.rms_norm_eps));
+    if (S == 1) return HM_OK;  // with one token the BSHD rows and the BHSD outputs coincide
+    TRY(bshd_to_bhsd(ctx, krows, k.as<float>(), S, b.kv_heads, b.head_dim));
+    return bshd_to_bhsd(ctx, vrows, v.as<float>(), S, b.kv_heads, b.head_dim);
 }
 
 // emit_attention_kernel (src/hf/emitter.rs:683-758): q [1,S,H,hd], k/v views [1,kvh,T,hd] f32 with the
 // cache's max-length strides (src/runtime.rs:610-615), mask [1,1,S,T], o_w [q_dim,hidden] -> [1,S,hidden]
+int attention_over_views(const MemRef &q, const MemRef &k, const MemRef &v, float *out, Scratch &s, const char *who);
+
 int run_attn(void **a) {
     const Bound &b = g_bound;
     hm_ctx *ctx = b.ctx;
     const MemRef q = memref(a, 0, 4), k = memref(a, 1, 4), v = memref(a, 2, 4), ow = memref(a, 4, 2),
                  out = memref(a, 5, 3);
-    TRY(need_single_token(ctx, q.sizes[1], "Attn kernel"));
-    const int T = (int)k.sizes[2], kvh = b.kv_heads, hd = b.head_dim;
-    if (T < 1 || k.strides[3] != 1 || v.strides[3] != 1)
-        return hm_set_error(ctx, HM_ERR_INVALID, "Attn kernel: K/V views must have >= 1 row and unit inner stride");
+    TRY(seq_ok(ctx, q.sizes[1], "Attn kernel"));
+    const int S = (int)q.sizes[1];
     Scratch s(ctx);
-    // the attention kernel's split partials must fit the part of the workspace left to the kernels
-    if ((size_t)b.cfg.num_attention_heads * ((T + 31) / 32) * (hd + 2) * 4 > KERNEL_RESERVE)
-        return hm_set_error(ctx, HM_ERR_INVALID, "Attn kernel: %d cache rows are more than this entry point takes", T);
-    const size_t n = (size_t)kvh * T * hd;
-    uint16_t *kc = s.take<uint16_t>(n), *vc = s.take<uint16_t>(n);
-    float *flat = s.take<float>(b.q_dim);
-    if (!kc || !vc || !flat) return hm_set_error(ctx, HM_ERR_OOM, "Attn kernel: workspace too small for %d rows", T);
-    const unsigned blocks = (unsigned)((n + 255) / 256);
-    hipLaunchKernelGGL(kv_view_to_bf16_kernel, dim3(blocks), dim3(256), 0, ctx->stream, k.as<float>(), k.strides[1],
-                       k.strides[2], kc, T, hd, n);
-    hipLaunchKernelGGL(kv_view_to_bf16_kernel, dim3(blocks), dim3(256), 0, ctx->stream, v.as<float>(), v.strides[1],
-                       v.strides[2], vc, T, hd, n);
-    HM_LAUNCH_CHECK(ctx);
-    TRY(hm_gqa_decode_attn(ctx, q.as<float>(), kc, vc, flat, 1, b.cfg.num_attention_heads, kvh, hd, T, T,
-                           (float)(1.0 / std::sqrt((double)hd))));
-    return hm_gemv_bf16(ctx, flat, ow.as<uint16_t>(), out.as<float>(), 1, b.q_dim, b.cfg.hidden_size);
+    float *flat = s.take<float>((size_t)S * b.q_dim);
+    if (!flat) return hm_set_error(ctx, HM_ERR_OOM, "Attn kernel: workspace too small for %d tokens", S);
+    TRY(attention_over_views(q, k, v, flat, s, "Attn kernel"));
+    return rows_gemv_bf16(ctx, flat, ow.as<uint16_t>(), out.as<float>(), S, b.q_dim, b.cfg.hidden_size);
 }
 
 // emit_mlp_kernel (src/hf/emitter.rs:767-822): h, attn_out, ln_w, gate_w, up_w, down_w -> [1,S,hidden]
@@ -197,18 +245,20 @@ int run_mlp(void **a) {
     const int hidden = b.cfg.hidden_size, inter = b.cfg.intermediate_size;
     const MemRef h = memref(a, 0, 3), attn = memref(a, 1, 3), ln = memref(a, 2, 1), gw = memref(a, 3, 2),
                  uw = memref(a, 4, 2), dw = memref(a, 5, 2), out = memref(a, 6, 3);
-    TRY(need_single_token(ctx, h.sizes[1], "MLP kernel"));
+    TRY(seq_ok(ctx, h.sizes[1], "MLP kernel"));
+    const size_t S = (size_t)h.sizes[1];
     Scratch s(ctx);
-    float *resid = s.take<float>(hidden), *normed = s.take<float>(hidden), *gate = s.take<float>(inter),
-          *up = s.take<float>(inter), *down = s.take<float>(hidden);
-    if (!resid || !normed || !gate || !up || !down) return hm_set_error(ctx, HM_ERR_OOM, "MLP kernel: workspace too small");
-    TRY(hm_add(ctx, h.as<float>(), attn.as<float>(), resid, (size_t)hidden));
-    TRY(hm_rmsnorm(ctx, resid, ln.as<float>(), normed, 1, hidden, (float)b.cfg.rms_norm_eps));
-    TRY(hm_gemv_bf16(ctx, normed, gw.as<uint16_t>(), gate, 1, hidden, inter));
-    TRY(hm_gemv_bf16(ctx, normed, uw.as<uint16_t>(), up, 1, hidden, inter));
-    TRY(hm_silu_mul(ctx, gate, up, gate, (size_t)inter));
-    TRY(hm_gemv_bf16(ctx, gate, dw.as<uint16_t>(), down, 1, inter, hidden));
-    return hm_add(ctx, resid, down, out.as<float>(), (size_t)hidden);
+    float *resid = s.take<float>(S * hidden), *normed = s.take<float>(S * hidden), *gate = s.take<float>(S * inter),
+          *up = s.take<float>(S * inter), *down = s.take<float>(S * hidden);
+    if (!resid || !normed || !gate || !up || !down)
+        return hm_set_error(ctx, HM_ERR_OOM, "MLP kernel: workspace too small for %d tokens", (int)S);
+    TRY(hm_add(ctx, h.as<float>(), attn.as<float>(), resid, S * hidden));
+    TRY(hm_rmsnorm(ctx, resid, ln.as<float>(), normed, (int)S, hidden, (float)b.cfg.rms_norm_eps));
+    TRY(rows_gemv_bf16(ctx, normed, gw.as<uint16_t>(), gate, (int)S, hidden, inter));
+    TRY(rows_gemv_bf16(ctx, normed, uw.as<uint16_t>(), up, (int)S, hidden, inter));
+    TRY(hm_silu_mul(ctx, gate, up, gate, S * inter));
+    TRY(rows_gemv_bf16(ctx, gate, dw.as<uint16_t>(), down, (int)S, inter, hidden));
+    return hm_add(ctx, resid, down, out.as<float>(), S * hidden);
 }
 
 // emit_lm_head_kernel (src/hf/emitter.rs:828-862): h, norm_w, lm_head_w [hidden,vocab] -> [1,S,vocab]
@@ -216,12 +266,13 @@ int run_lm_head(void **a) {
     const Bound &b = g_bound;
     hm_ctx *ctx = b.ctx;
     const MemRef h = memref(a, 0, 3), nw = memref(a, 1, 1), lw = memref(a, 2, 2), out = memref(a, 3, 3);
-    TRY(need_single_token(ctx, h.sizes[1], "LMHead kernel"));
+    TRY(seq_ok(ctx, h.sizes[1], "LMHead kernel"));
+    const int S = (int)h.sizes[1];
     Scratch s(ctx);
-    float *normed = s.take<float>(b.cfg.hidden_size);
-    if (!normed) return hm_set_error(ctx, HM_ERR_OOM, "LMHead kernel: workspace too small");
-    TRY(hm_rmsnorm(ctx, h.as<float>(), nw.as<float>(), normed, 1, b.cfg.hidden_size, (float)b.cfg.rms_norm_eps));
-    return hm_gemv_bf16(ctx, normed, lw.as<uint16_t>(), out.as<float>(), 1, b.cfg.hidden_size, b.cfg.vocab_size);
+    float *normed = s.take<float>((size_t)S * b.cfg.hidden_size);
+    if (!normed) return hm_set_error(ctx, HM_ERR_OOM, "LMHead kernel: workspace too small for %d tokens", S);
+    TRY(hm_rmsnorm(ctx, h.as<float>(), nw.as<float>(), normed, S, b.cfg.hidden_size, (float)b.cfg.rms_norm_eps));
+    return rows_gemv_bf16(ctx, normed, lw.as<uint16_t>(), out.as<float>(), S, b.cfg.hidden_size, b.cfg.vocab_size);
 }
 
 // ── the quantised plan's kernels (src/hf/emitter_quant.rs) ───────────────────
@@ -244,22 +295,30 @@ __global__ __launch_bounds__(256) void gemv_f32_kn_kernel(const float *__restric
 int run_rms_norm(void **a) {
     const Bound &b = g_bound;
     const MemRef h = memref(a, 0, 3), w = memref(a, 1, 1), out = memref(a, 2, 3);
-    TRY(need_single_token(b.ctx, h.sizes[1], "RMSNorm kernel"));
-    return hm_rmsnorm(b.ctx, h.as<float>(), w.as<float>(), out.as<float>(), 1, b.cfg.hidden_size, (float)b.cfg.rms_norm_eps);
+    TRY(seq_ok(b.ctx, h.sizes[1], "RMSNorm kernel"));
+    return hm_rmsnorm(b.ctx, h.as<float>(), w.as<float>(), out.as<float>(), (int)h.sizes[1], b.cfg.hidden_size,
+                      (float)b.cfg.rms_norm_eps);
 }
 
 // emit_quant_matmul_kernel (src/hf/emitter_quant.rs:675-702): x [1,S,K], raw blocks (flat bytes) -> [1,S,N]
 int run_quant_mm(void **a, const KernelInfo &ki) {
     const Bound &b = g_bound;
     const MemRef x = memref(a, 0, 3), w = memref(a, 1, 1), out = memref(a, 2, 3);
-    TRY(need_single_token(b.ctx, x.sizes[1], "QuantMM kernel"));
-    switch (ki.dtype) {
-    case HM_DTYPE_Q8_0: return hm_gemv_q8_0(b.ctx, x.as<float>(), w.as<uint8_t>(), out.as<float>(), 1, ki.K, ki.N);
-    case HM_DTYPE_Q4_0: return hm_gemv_q4_0(b.ctx, x.as<float>(), w.as<uint8_t>(), out.as<float>(), 1, ki.K, ki.N);
-    case HM_DTYPE_Q4_K: return hm_gemv_q4_k(b.ctx, x.as<float>(), w.as<uint8_t>(), out.as<float>(), 1, ki.K, ki.N);
-    case HM_DTYPE_Q6_K: return hm_gemv_q6_k(b.ctx, x.as<float>(), w.as<uint8_t>(), out.as<float>(), 1, ki.K, ki.N);
+    TRY(seq_ok(b.ctx, x.sizes[1], "QuantMM kernel"));
+    const int S = (int)x.sizes[1];
+    for (int r = 0; r < S; r += 8) {
+        const float *xr = x.as<float>() + (size_t)r * ki.K;
+        float *outr = out.as<float>() + (size_t)r * ki.N;
+        const int m = S - r < 8 ? S - r : 8;
+        switch (ki.dtype) {
+        case HM_DTYPE_Q8_0: TRY(hm_gemv_q8_0(b.ctx, xr, w.as<uint8_t>(), outr, m, ki.K, ki.N)); break;
+        case HM_DTYPE_Q4_0: TRY(hm_gemv_q4_0(b.ctx, xr, w.as<uint8_t>(), outr, m, ki.K, ki.N)); break;
+        case HM_DTYPE_Q4_K: TRY(hm_gemv_q4_k(b.ctx, xr, w.as<uint8_t>(), outr, m, ki.K, ki.N)); break;
+        case HM_DTYPE_Q6_K: TRY(hm_gemv_q6_k(b.ctx, xr, w.as<uint8_t>(), outr, m, ki.K, ki.N)); break;
+        default: return hm_set_error(b.ctx, HM_ERR_INVALID, "QuantMM kernel: dtype %d", ki.dtype);
+        }
     }
-    return hm_set_error(b.ctx, HM_ERR_INVALID, "QuantMM kernel: dtype %d", ki.dtype);
+    return HM_OK;
 }
 
 // emit_post_qkv_kernel (src/hf/emitter_quant.rs:802-912): q_raw [1,S,q_dim], k_raw, v_raw [1,S,kv_dim],
@@ -283,29 +342,39 @@ int run_post_qkv(void **a) {
         kn = memref(a, i++, 1).as<float>();
     }
     const MemRef q = memref(a, i++, 4), k = memref(a, i++, 4), v = memref(a, i++, 4);
-    TRY(need_single_token(ctx, qr.sizes[1], "PostQKV kernel"));
-    // with one token the [1,S,dim] rows and the BSHD / BHSD outputs are the same bytes
+    TRY(seq_ok(ctx, qr.sizes[1], "PostQKV kernel"));
+    const int S = (int)qr.sizes[1];
+    Scratch s(ctx);
+    // q [1,S,H,hd] is the raw row layout; k and v leave as [1,kvh,S,hd], so with more than one token they
+    // are finished as rows in scratch and transposed on the way out
+    float *krows = S > 1 ? s.take<float>((size_t)S * b.kv_dim) : k.as<float>();
+    float *vrows = S > 1 ? s.take<float>((size_t)S * b.kv_dim) : v.as<float>();
+    if (!krows || !vrows) return hm_set_error(ctx, HM_ERR_OOM, "PostQKV kernel: workspace too small for %d tokens", S);
+    TRY(hm_copy(ctx, q.data, qr.data, (size_t)S * b.q_dim * 4));
+    TRY(hm_copy(ctx, krows, kr.data, (size_t)S * b.kv_dim * 4));
+    TRY(hm_copy(ctx, vrows, vr.data, (size_t)S * b.kv_dim * 4));
     if (bias) {
-        TRY(hm_add(ctx, qr.as<float>(), qb, q.as<float>(), (size_t)b.q_dim));
-        TRY(hm_add(ctx, kr.as<float>(), kb, k.as<float>(), (size_t)b.kv_dim));
-        TRY(hm_add(ctx, vr.as<float>(), vb, v.as<float>(), (size_t)b.kv_dim));
-    } else {
-        TRY(hm_copy(ctx, q.data, qr.data, (size_t)b.q_dim * 4));
-        TRY(hm_copy(ctx, k.data, kr.data, (size_t)b.kv_dim * 4));
-        TRY(hm_copy(ctx, v.data, vr.data, (size_t)b.kv_dim * 4));
+        TRY(add_bias_rows(ctx, q.as<float>(), qb, S, b.q_dim));
+        TRY(add_bias_rows(ctx, krows, kb, S, b.kv_dim));
+        TRY(add_bias_rows(ctx, vrows, vb, S, b.kv_dim));
     }
-    return hm_qknorm_rope(ctx, q.as<float>(), k.as<float>(), qn, kn, cosv.as<float>(), sinv.as<float>(), 1,
-                          b.cfg.num_attention_heads, b.kv_heads, b.head_dim, (float)b.cfg.rms_norm_eps);
+    TRY(hm_qknorm_rope(ctx, q.as<float>(), krows, qn, kn, cosv.as<float>(), sinv.as<float>(), S, b.cfg.num_attention_heads,
+                       b.kv_heads, b.head_dim, (float)b.cfg.rms_norm_eps));
+    if (S == 1) return HM_OK;
+    TRY(bshd_to_bhsd(ctx, krows, k.as<float>(), S, b.kv_heads, b.head_dim));
+    return bshd_to_bhsd(ctx, vrows, v.as<float>(), S, b.kv_heads, b.head_dim);
 }
 
-// The attention part shared by emit_attention_kernel and emit_attention_body_kernel: q [1,1,H,hd] over
-// the f32 K/V views -> out [q_dim] (device pointer)
+// The attention part shared by emit_attention_kernel and emit_attention_body_kernel: q [1,S,H,hd] over the
+// f32 K/V views [1,kvh,T,hd], whose last S rows are the new tokens' -> out [S][q_dim] (device pointer).
+// One query row attends to all T rows (the decode mask is all zero, src/hf/precompute.rs:49-64); S rows
+// attend causally, row i to keys 0 .. T - S + i.
 int attention_over_views(const MemRef &q, const MemRef &k, const MemRef &v, float *out, Scratch &s, const char *who) {
     const Bound &b = g_bound;
     hm_ctx *ctx = b.ctx;
-    const int T = (int)k.sizes[2], kvh = b.kv_heads, hd = b.head_dim;
-    if (T < 1 || k.strides[3] != 1 || v.strides[3] != 1)
-        return hm_set_error(ctx, HM_ERR_INVALID, "%s: K/V views must have >= 1 row and unit inner stride", who);
+    const int S = (int)q.sizes[1], T = (int)k.sizes[2], kvh = b.kv_heads, hd = b.head_dim;
+    if (T < S || k.strides[3] != 1 || v.strides[3] != 1 || v.sizes[2] != k.sizes[2])
+        return hm_set_error(ctx, HM_ERR_INVALID, "%s: K/V views must hold the %d new rows and have unit inner stride", who, S);
     // the attention kernel's split partials must fit the part of the workspace left to the kernels
     if ((size_t)b.cfg.num_attention_heads * ((T + 31) / 32) * (hd + 2) * 4 > KERNEL_RESERVE)
         return hm_set_error(ctx, HM_ERR_INVALID, "%s: %d cache rows are more than this entry point takes", who, T);
@@ -318,15 +387,16 @@ int attention_over_views(const MemRef &q, const MemRef &k, const MemRef &v, floa
     hipLaunchKernelGGL(kv_view_to_bf16_kernel, dim3(blocks), dim3(256), 0, ctx->stream, v.as<float>(), v.strides[1],
                        v.strides[2], vc, T, hd, n);
     HM_LAUNCH_CHECK(ctx);
-    return hm_gqa_decode_attn(ctx, q.as<float>(), kc, vc, out, 1, b.cfg.num_attention_heads, kvh, hd, T, T,
-                              (float)(1.0 / std::sqrt((double)hd)));
+    const float scale = (float)(1.0 / std::sqrt((double)hd));
+    if (S == 1) return hm_gqa_decode_attn(ctx, q.as<float>(), kc, vc, out, 1, b.cfg.num_attention_heads, kvh, hd, T, T, scale);
+    return hm_gqa_prefill_attn(ctx, q.as<float>(), kc, vc, out, S, b.cfg.num_attention_heads, kvh, hd, T, T - S, scale);
 }
 
 // emit_attention_body_kernel (src/hf/emitter_quant.rs:922-975): q, K view, V view, mask -> [1,S,q_dim]
 int run_attn_body(void **a) {
     const Bound &b = g_bound;
     const MemRef q = memref(a, 0, 4), k = memref(a, 1, 4), v = memref(a, 2, 4), out = memref(a, 4, 3);
-    TRY(need_single_token(b.ctx, q.sizes[1], "AttnBody kernel"));
+    TRY(seq_ok(b.ctx, q.sizes[1], "AttnBody kernel"));
     Scratch s(b.ctx);
     return attention_over_views(q, k, v, out.as<float>(), s, "AttnBody kernel");
 }
@@ -336,9 +406,10 @@ int run_residual_norm(void **a) {
     const Bound &b = g_bound;
     const MemRef h = memref(a, 0, 3), attn = memref(a, 1, 3), w = memref(a, 2, 1), resid = memref(a, 3, 3),
                  normed = memref(a, 4, 3);
-    TRY(need_single_token(b.ctx, h.sizes[1], "Residual+Norm kernel"));
-    TRY(hm_add(b.ctx, h.as<float>(), attn.as<float>(), resid.as<float>(), (size_t)b.cfg.hidden_size));
-    return hm_rmsnorm(b.ctx, resid.as<float>(), w.as<float>(), normed.as<float>(), 1, b.cfg.hidden_size,
+    TRY(seq_ok(b.ctx, h.sizes[1], "Residual+Norm kernel"));
+    const int S = (int)h.sizes[1];
+    TRY(hm_add(b.ctx, h.as<float>(), attn.as<float>(), resid.as<float>(), (size_t)S * b.cfg.hidden_size));
+    return hm_rmsnorm(b.ctx, resid.as<float>(), w.as<float>(), normed.as<float>(), S, b.cfg.hidden_size,
                       (float)b.cfg.rms_norm_eps);
 }
 
@@ -346,16 +417,16 @@ int run_residual_norm(void **a) {
 int run_silu_mul(void **a) {
     const Bound &b = g_bound;
     const MemRef g = memref(a, 0, 3), u = memref(a, 1, 3), out = memref(a, 2, 3);
-    TRY(need_single_token(b.ctx, g.sizes[1], "SiLU*Up kernel"));
-    return hm_silu_mul(b.ctx, g.as<float>(), u.as<float>(), out.as<float>(), (size_t)b.cfg.intermediate_size);
+    TRY(seq_ok(b.ctx, g.sizes[1], "SiLU*Up kernel"));
+    return hm_silu_mul(b.ctx, g.as<float>(), u.as<float>(), out.as<float>(), (size_t)g.sizes[1] * b.cfg.intermediate_size);
 }
 
 // emit_residual_add_kernel (src/hf/emitter_quant.rs:1110-1134): residual, down_out -> hidden_out
 int run_res_add(void **a) {
     const Bound &b = g_bound;
     const MemRef r = memref(a, 0, 3), d = memref(a, 1, 3), out = memref(a, 2, 3);
-    TRY(need_single_token(b.ctx, r.sizes[1], "ResAdd kernel"));
-    return hm_add(b.ctx, r.as<float>(), d.as<float>(), out.as<float>(), (size_t)b.cfg.hidden_size);
+    TRY(seq_ok(b.ctx, r.sizes[1], "ResAdd kernel"));
+    return hm_add(b.ctx, r.as<float>(), d.as<float>(), out.as<float>(), (size_t)r.sizes[1] * b.cfg.hidden_size);
 }
 
 // LM head of the quantised plan (src/hf/emitter_quant.rs:1399-1440): h, norm_w, lm_head_w f32 [hidden,vocab]
@@ -363,17 +434,54 @@ int run_lm_head_f32(void **a) {
     const Bound &b = g_bound;
     hm_ctx *ctx = b.ctx;
     const MemRef h = memref(a, 0, 3), nw = memref(a, 1, 1), lw = memref(a, 2, 2), out = memref(a, 3, 3);
-    TRY(need_single_token(ctx, h.sizes[1], "LMHead kernel"));
+    TRY(seq_ok(ctx, h.sizes[1], "LMHead kernel"));
+    const int S = (int)h.sizes[1];
     const int hidden = b.cfg.hidden_size, vocab = b.cfg.vocab_size;
     Scratch s(ctx);
-    float *normed = s.take<float>(hidden);
-    if (!normed) return hm_set_error(ctx, HM_ERR_OOM, "LMHead kernel: workspace too small");
+    float *normed = s.take<float>((size_t)S * hidden);
+    if (!normed) return hm_set_error(ctx, HM_ERR_OOM, "LMHead kernel: workspace too small for %d tokens", S);
     HM_REQUIRE(ctx, (size_t)hidden * 4 <= 64 * 1024, "LMHead kernel: hidden size %d above 16384", hidden);
-    TRY(hm_rmsnorm(ctx, h.as<float>(), nw.as<float>(), normed, 1, hidden, (float)b.cfg.rms_norm_eps));
-    hipLaunchKernelGGL(gemv_f32_kn_kernel, dim3((unsigned)((vocab + 255) / 256)), dim3(256), (size_t)hidden * 4, ctx->stream,
-                       normed, lw.as<float>(), out.as<float>(), hidden, vocab);
-    HM_LAUNCH_CHECK(ctx);
+    TRY(hm_rmsnorm(ctx, h.as<float>(), nw.as<float>(), normed, S, hidden, (float)b.cfg.rms_norm_eps));
+    for (int r = 0; r < S; r++) {
+        hipLaunchKernelGGL(gemv_f32_kn_kernel, dim3((unsigned)((vocab + 255) / 256)), dim3(256), (size_t)hidden * 4, ctx->stream,
+                           normed + (size_t)r * hidden, lw.as<float>(), out.as<float>() + (size_t)r * vocab, hidden, vocab);
+        HM_LAUNCH_CHECK(ctx);
+    }
     return HM_OK;
+}
+
+// The operands a kernel writes: (first output operand, count, rank) by kind, in each emitter's order.
+void outputs_of(const KernelInfo &ki, int *first, int *count, int *rank) {
+    const Bound &b = g_bound;
+    const int bias = b.cfg.attention_bias ? 1 : 0, qkn = b.qk_norm ? 2 : 0;
+    *count = 1;
+    *rank = 3;
+    switch (ki.kind) {
+    case Kind::Embed: *first = 2; break;
+    case Kind::Qkv: *first = 7 + 3 * bias + qkn; *count = 3; *rank = 4; break;
+    case Kind::Attn: *first = 5; break;
+    case Kind::Mlp: *first = 6; break;
+    case Kind::LmHead: case Kind::LmHeadF32: *first = 3; break;
+    case Kind::RmsNorm: case Kind::QuantMM: case Kind::SiluMul: case Kind::ResAdd: *first = 2; break;
+    case Kind::PostQkv: *first = 5 + 3 * bias + qkn; *count = 3; *rank = 4; break;
+    case Kind::AttnBody: *first = 4; break;
+    case Kind::ResidualNorm: *first = 3; *count = 2; break;
+    }
+}
+
+// After a failure no caller may mistake stale bytes for results: every output operand becomes NaN.
+void poison_outputs(const KernelInfo &ki, void **args) {
+    hm_ctx *ctx = g_bound.ctx;
+    int first, count, rank;
+    outputs_of(ki, &first, &count, &rank);
+    for (int j = 0; j < count; j++) {
+        const MemRef m = memref(args, first + j, rank);
+        size_t n = 1;
+        for (int d = 0; d < rank; d++) n *= (size_t)(m.sizes[d] > 0 ? m.sizes[d] : 0);
+        if (m.data && n && n < ((size_t)1 << 34)) (void)hipMemsetAsync(m.data, 0xFF, n * 4, ctx->stream);
+    }
+    (void)hipStreamSynchronize(ctx->stream);
+    (void)hipGetLastError();
 }
 
 void dispatch(int idx, void **args) {
@@ -398,6 +506,7 @@ void dispatch(int idx, void **args) {
     case Kind::ResAdd: rc = run_res_add(args); break;
     case Kind::LmHeadF32: rc = run_lm_head_f32(args); break;
     }
+    if (rc != HM_OK) poison_outputs(ki, args);
     report(idx, rc);
 }
 
@@ -484,6 +593,16 @@ int hm_ciface_bind_transformer(hm_ctx *ctx, const hm_transformer_config *cfg, in
 int hm_ciface_num_kernels(void) { return (int)g_bound.kinds.size(); }
 
 void hm_ciface_unbind(void) { g_bound = Bound(); }
+
+int hm_ciface_last_status(int *kernel_index) {
+    if (kernel_index) *kernel_index = g_status_kernel;
+    return g_status;
+}
+
+void hm_ciface_clear_status(void) {
+    g_status = HM_OK;
+    g_status_kernel = -1;
+}
 
 // HM_CIFACE_MAX_KERNELS exported symbols _mlir__mlir_ciface_k0 ... _mlir__mlir_ciface_k1023
 #define HM_K(i) \

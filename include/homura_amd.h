@@ -470,20 +470,28 @@ hm_model *hm_model_load_hf_dir(hm_ctx *ctx, const char *dir, int max_seq_len);
  * dlsym exactly as it resolves its own. hm_ciface_bind_transformer tells the library which
  * fused kernel each index is, in emit_transformer_plan's numbering (src/hf/emitter.rs:902-1014):
  * k0 Embed, k(3l+1) QKV(+QK-norm)+RoPE, k(3l+2) Attn, k(3l+3) MLP for layer l, then LMHead;
- * bf16 weights [K,N], f32 K/V views with the cache's strides, one token per call.
+ * bf16 weights [K,N], f32 K/V views with the cache's strides; a call carries any number of tokens
+ * (the reference's prefill feeds whole prompts to the same kernels, src/hf/model.rs:321-336): with more
+ * than one query row attention is causal by position (build_causal_mask, src/hf/precompute.rs:134-161;
+ * the mask operand itself is not read), the last S rows of the K/V views being the new tokens'.
  * hm_ciface_bind_transformer_quant does the same for emit_transformer_plan_quant's numbering
  * (src/hf/emitter_quant.rs:1170-1440): k0 Embed; for layer l the thirteen kernels k(13l+1) ..
  * k(13l+13) = RMSNorm, QuantMM Q, K, V, PostQKV, AttnBody, QuantMM O, Residual+Norm, QuantMM Gate, Up,
  * SiLU*Up, QuantMM Down, ResAdd; then the LMHead with f32 weights [hidden, vocab]. proj_dtypes: 7
  * HM_DTYPE_* block formats per layer (q k v o gate up down); the weights are the raw GGUF blocks.
  * A failure cannot be returned (the ABI is void): it is recorded for hm_last_error and printed to
- * stderr. One binding per process at a time. */
+ * stderr, every output operand of the failing call is filled with NaN, and the first failure's code stays
+ * in a status word until it is cleared: hm_ciface_last_status returns it (HM_OK when every call since the
+ * last clear went through) and stores the failing kernel's index in *kernel_index (may be NULL).
+ * One binding per process at a time. */
 #define HM_CIFACE_MAX_KERNELS 1024
 int hm_ciface_bind_transformer(hm_ctx *ctx, const hm_transformer_config *cfg, int has_qk_norm);
 int hm_ciface_bind_transformer_quant(hm_ctx *ctx, const hm_transformer_config *cfg, const int *proj_dtypes,
                                      int has_qk_norm);
 int hm_ciface_num_kernels(void);
 void hm_ciface_unbind(void);
+int hm_ciface_last_status(int *kernel_index);
+void hm_ciface_clear_status(void);
 
 uint16_t hm_f32_to_bf16_rne(float v);
 uint16_t hm_f32_to_f16_rne(float v);
