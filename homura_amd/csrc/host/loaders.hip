@@ -871,6 +871,10 @@ std::unique_ptr<SafeTensorsFile> SafeTensorsFile::load(const std::string &path, 
             }
             t.shape.push_back((uint64_t)d.num);
         }
+        if (t.shape.size() > 8) {  // as the GGUF reader: the C boundary reports at most eight dimensions
+            *err = "safetensors: tensor '" + kv.first + "' has " + std::to_string(t.shape.size()) + " dimensions";
+            return nullptr;
+        }
         t.begin = (size_t)off->arr[0].num;
         t.end = (size_t)off->arr[1].num;
         if (t.begin > t.end || t.end > data_size) {

@@ -196,6 +196,9 @@ def test_safetensors_metadata_and_errors(tmp_path):
         ck.SafeTensorsFile(write(tmp_path, "o.safetensors", struct.pack("<Q", len(bad)) + bad + bytes(8)))
     with pytest.raises(ValueError, match="JSON"):
         ck.SafeTensorsFile(write(tmp_path, "j.safetensors", struct.pack("<Q", 5) + b"{oops"))
+    deep = b'{"x":{"dtype":"F32","shape":[1,1,1,1,1,1,1,1,2],"data_offsets":[0,8]}}'   # nine dimensions
+    with pytest.raises(ValueError, match="9 dimensions"):
+        ck.SafeTensorsFile(write(tmp_path, "d.safetensors", struct.pack("<Q", len(deep)) + deep + bytes(8)))
 
 
 # ── config.json: the reference's fixtures ────────────────────────────────────
