@@ -408,14 +408,14 @@ class HfModel:
         self._check(self.lib.hm_model_finalize(self.h, max_seq_len))
 
     def init_kv_cache(self, kv_buffers: list[np.ndarray], seq_len: int):
-        """kv_buffers: key and value of every layer in turn, each kv_heads * seq_len * head_dim floats
+        """kv_buffers: key and value of every layer in turn, each at least kv_heads * seq_len * head_dim floats
         ([1, kv_heads, seq_len, head_dim]); the C side reads exactly that many from every pointer."""
         c = self.config
         want = c.kv_heads() * seq_len * c.get_head_dim()
         if len(kv_buffers) != 2 * c.num_hidden_layers:
             raise ValueError(f"init_kv_cache: {len(kv_buffers)} buffers for {c.num_hidden_layers} layers (2 per layer needed)")
         for i, b in enumerate(kv_buffers):
-            if np.asarray(b).size != want:
+            if np.asarray(b).size < want:
                 raise ValueError(f"init_kv_cache: buffer {i} holds {np.asarray(b).size} values, {want} needed")
         arrs = [np.ascontiguousarray(b, dtype=np.float32) for b in kv_buffers]
         ptrs = (_ffi.c_f32_p * len(arrs))(*[a.ctypes.data_as(_ffi.c_f32_p) for a in arrs])
