@@ -85,6 +85,12 @@ SIGNATURES = {
     "hm_gemv_bf16_nk": (_I, [_P, _P, _P, _P, _I, _I, _I]),
     "hm_gemv_q8_0": (_I, [_P, _P, _P, _P, _I, _I, _I]),
     "hm_gemv_q4_0": (_I, [_P, _P, _P, _P, _I, _I, _I]),
+    "hm_quant_planes_bytes": (_SZ, [_I, _I, _I]),
+    "hm_pack_quant_planes": (_I, [_P, _I, _P, _P, _I, _I]),
+    "hm_unpack_quant_planes": (_I, [_P, _I, _P, _P, _I, _I]),
+    "hm_gemv_q8_0_planes": (_I, [_P, _P, _P, _P, _I, _I, _I]),
+    "hm_gemv_q4_0_planes": (_I, [_P, _P, _P, _P, _I, _I, _I]),
+    "hm_dequant_quant_planes": (_I, [_P, _I, _P, _P, _I, _I]),
     "hm_dequant_q8_0": (_I, [_P, _P, _P, _SZ]),
     "hm_dequant_q4_0": (_I, [_P, _P, _P, _SZ]),
     "hm_gemv_q4_k": (_I, [_P, _P, _P, _P, _I, _I, _I]),

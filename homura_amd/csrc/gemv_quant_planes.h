@@ -1,0 +1,27 @@
+// Launch interface of the Q8_0 / Q4_0 GEMV over re-packed weights ("planes": all quant bytes row after
+// row, then all f16 scales row after row; the same bytes as the GGUF blocks), shared with the model.
+#pragma once
+
+#include <cstddef>
+#include <cstdint>
+
+#include "gemv_quant.h"
+#include "hm_common.h"
+
+namespace homura {
+
+// Bytes of the planes of an [N][K] matrix, and where the scale plane starts (256-byte aligned).
+size_t quant_planes_bytes(bool q4, int N, int K);
+size_t quant_planes_scale_offset(bool q4, int N, int K);
+
+// raw blocks [N][K / 32] -> planes (one launch, at upload)
+int pack_quant_planes(hm_ctx *ctx, bool q4, const uint8_t *d_blocks, uint8_t *d_planes, int N, int K);
+
+// out[N] = W[N][K] . f(x) with the light ops of QuantFuse, W as planes; K <= 4096
+int gemv_planes_fused(hm_ctx *ctx, bool q4, const float *d_x, const uint8_t *d_planes, float *d_out, int K, int N,
+                      const QuantFuse &fuse);
+
+// Workgroups gemv_planes_fused launches for this shape (= argmax candidates it leaves when asked to).
+int gemv_planes_workgroups(const hm_ctx *ctx, bool q4, int K, int N);
+
+}  // namespace homura

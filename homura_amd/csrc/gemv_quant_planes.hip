@@ -1,0 +1,519 @@
+// Q8_0 / Q4_0 dequant-GEMV over weights re-packed once, at upload, into two planes: the quant bytes
+// of all blocks, row after row (Q8_0: K bytes a row; Q4_0: K / 2, each block's 16 bytes of nibble
+// pairs as they are in the file), then the f16 scales of all blocks, row after row. Same bytes as the
+// GGUF blocks (reference src/hf/weights.rs:136-194 keeps them raw; src/graph_builder/emit_quant.rs:17-21
+// layout), but every quant word sits at its natural alignment, so a lane loads its words straight
+// from global memory into registers: no LDS stage, no two-byte LDS reads, no funnel shifts.
+//
+// A lane's unit of work is a quarter block (8 weights = 8 quant bytes for Q8_0, one 32-bit word of
+// nibble pairs for Q4_0) plus the block's scale; quarter columns are dealt to the lanes round-robin as
+// in gemv_quant.hip, and the arithmetic is that kernel's: d * (sum_j q_j x_j - offset * sum_j x_j) with
+// the quants used as stored. A wavefront walks the rows in trips of RB rows, the loads of the next
+// trip in flight while this one is multiplied.
+#include "gemv_quant_planes.h"
+
+#include "hm_common.h"
+#include "quant_formats.h"
+
+namespace {
+
+using homura::QuantFuse;
+
+constexpr int PTHREADS = 256;
+constexpr int PWAVES = PTHREADS / WAVE;
+
+template <int QT>
+struct PlaneTraits;
+template <>
+struct PlaneTraits<0> {  // Q8_0
+    static constexpr int QBYTES = 8;  // quant bytes of a quarter block
+    static constexpr int BLOCK = 34;
+};
+template <>
+struct PlaneTraits<1> {  // Q4_0
+    static constexpr int QBYTES = 4;
+    static constexpr int BLOCK = 18;
+};
+
+// The four bytes of w as floats against xv. The empty asm keeps the compiler from folding the mask that
+// produced w into one bit-field extract per byte: on a masked dword the four conversions select their
+// byte themselves (v_cvt_f32_ubyte0..3), one instruction a weight instead of two.
+__device__ __forceinline__ float dot4_bytes(uint32_t w, const float *xv, float s) {
+    asm("" : "+v"(w));
+    s = fmaf((float)(w & 0xFFu), xv[0], s);
+    s = fmaf((float)((w >> 8) & 0xFFu), xv[1], s);
+    s = fmaf((float)((w >> 16) & 0xFFu), xv[2], s);
+    s = fmaf((float)(w >> 24), xv[3], s);
+    return s;
+}
+
+// Activations of quarter column c (block c / 4, quarter c % 4) in the order the quant bytes use them,
+// and offset * their sum.
+template <int QT>
+__device__ __forceinline__ void load_xv(const float *xs, int c, float *xv, float &sx_off) {
+    const int b = c >> 2, q = c & 3;
+    const float *p0 = xs + b * 32 + (QT == 0 ? q * 8 : q * 4);
+    const float *p1 = QT == 0 ? p0 + 4 : p0 + 16;
+    const f32x4 lo = *reinterpret_cast<const f32x4 *>(p0);
+    const f32x4 hi = *reinterpret_cast<const f32x4 *>(p1);
+    xv[0] = lo.x; xv[1] = lo.y; xv[2] = lo.z; xv[3] = lo.w;
+    xv[4] = hi.x; xv[5] = hi.y; xv[6] = hi.z; xv[7] = hi.w;
+    float sx = 0.f;
+#pragma unroll
+    for (int j = 0; j < 8; j++) sx += xv[j];
+    sx_off = sx * (QT == 0 ? 128.f : 8.f);
+}
+
+// The quant words of one quarter: Q8_0 two dwords, Q4_0 one.
+template <int QT>
+struct QWords {
+    uint32_t w0, w1;
+};
+
+typedef const uint32_t __attribute__((address_space(1))) *global_u32_ptr;
+typedef const u32x2 __attribute__((address_space(1))) *global_u32x2_ptr;
+typedef const uint16_t __attribute__((address_space(1))) *global_u16_ptr;
+
+template <int QT>
+__device__ __forceinline__ QWords<QT> load_quarter(const uint8_t *q) {
+    QWords<QT> r;
+    if (QT == 0) {
+        const u32x2 v = __builtin_nontemporal_load((global_u32x2_ptr)q);
+        r.w0 = v.x;
+        r.w1 = v.y;
+    } else {
+        r.w0 = __builtin_nontemporal_load((global_u32_ptr)q);
+        r.w1 = 0u;
+    }
+    return r;
+}
+
+template <int QT>
+__device__ __forceinline__ float quarter_value(const QWords<QT> &w, uint32_t scale_bits, const float *xv, float sx_off) {
+    const float d = f16_bits_to_f32((uint16_t)scale_bits);
+    float s;
+    if (QT == 0) {
+        s = dot4_bytes(w.w1 ^ 0x80808080u, xv + 4, dot4_bytes(w.w0 ^ 0x80808080u, xv, 0.f));  // int8 -> biased unsigned
+    } else {
+        // byte i of the word: low nibble = weight 4q + i, high nibble = weight 16 + 4q + i
+        s = dot4_bytes((w.w0 >> 4) & 0x0F0F0F0Fu, xv + 4, dot4_bytes(w.w0 & 0x0F0F0F0Fu, xv, 0.f));
+    }
+    return d * (s - sx_off);
+}
+
+// CPL = quarter columns per lane (ceil(K / 8 / 64)); RB = rows per trip of a wavefront.
+template <int QT, int CPL, int RB, bool FUSED>
+__global__ __launch_bounds__(PTHREADS) void gemv_planes_kernel(const float *__restrict__ x, const uint8_t *__restrict__ quants,
+                                                               const uint16_t *__restrict__ scales, float *__restrict__ out,
+                                                               int K, int N, const QuantFuse fuse_arg) {
+    const QuantFuse fuse = FUSED ? fuse_arg : QuantFuse();
+    constexpr int QB = PlaneTraits<QT>::QBYTES;
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    float *xs = reinterpret_cast<float *>(smem);
+    float *red = xs + K;  // [PWAVES] sums of squares, later the wavefronts' argmax candidates
+    const int tid = threadIdx.x, lane = tid & (WAVE - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(tid / WAVE);  // uniform: row addresses stay in scalar registers
+    const int nb = K / 32, nq = K / 8;
+    const size_t qrow = (size_t)nq * QB;
+
+    // this wavefront's trips: rows (trip * total waves + global wave) * RB ...
+    const int gw = blockIdx.x * PWAVES + wave, nwaves = gridDim.x * PWAVES;
+    const int ntrips = (N + RB - 1) / RB;
+    QWords<QT> qn[RB][CPL];
+    uint32_t sn[RB][CPL];
+    int col[CPL];
+    bool live[CPL];
+#pragma unroll
+    for (int t = 0; t < CPL; t++) {
+        live[t] = lane + t * WAVE < nq;
+        col[t] = live[t] ? lane + t * WAVE : nq - 1;  // lanes past the row end re-read its last column
+    }
+    auto request = [&](int trip) {
+#pragma unroll
+        for (int r = 0; r < RB; r++) {
+            const int row = min(trip * RB + r, N - 1);  // rows past the end re-read the last one
+            const uint8_t *qr = quants + (size_t)row * qrow;
+            const uint16_t *sr = scales + (size_t)row * nb;
+#pragma unroll
+            for (int t = 0; t < CPL; t++) {
+                qn[r][t] = load_quarter<QT>(qr + (size_t)col[t] * QB);
+                sn[r][t] = __builtin_nontemporal_load((global_u16_ptr)(sr + (col[t] >> 2)));
+            }
+        }
+    };
+
+    // Loads return in issue order: the (small, cached) activation loads go first, the first trip's
+    // weights right behind them, so staging the activations does not wait for HBM.
+    constexpr int XU = 4;  // covers K <= 4096 in one round
+    const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
+    f32x4 xr[XU], ar[XU], nr[XU];  // activation; second operand (x2 or res_in); norm weight
+    const float *second = fuse.x2 ? fuse.x2 : fuse.res_in;
+#pragma unroll
+    for (int u = 0; u < XU; u++) {
+        const int k = (tid + u * PTHREADS) * 4;
+        xr[u] = k < K ? *reinterpret_cast<const f32x4 *>(x + k) : zero4;
+        ar[u] = second && k < K ? *reinterpret_cast<const f32x4 *>(second + k) : zero4;
+        nr[u] = fuse.norm_w && k < K ? *reinterpret_cast<const f32x4 *>(fuse.norm_w + k) : zero4;
+    }
+    int trip = gw;
+    if (trip < ntrips) request(trip);
+    // the light ops of the quantised plan that sit in front of this product (reference
+    // src/hf/emitter_quant.rs:713-791, :985-1071, :1077-1103); the host allows the norm only for
+    // K <= XU * 1024, where the whole row is in xr
+    if (fuse.x2) {
+#pragma unroll
+        for (int u = 0; u < XU; u++)
+#pragma unroll
+            for (int e = 0; e < 4; e++) xr[u][e] = (xr[u][e] / (1.0f + expf(-xr[u][e]))) * ar[u][e];
+    } else if (fuse.res_in) {
+#pragma unroll
+        for (int u = 0; u < XU; u++) {
+            xr[u] += ar[u];
+            const int k = (tid + u * PTHREADS) * 4;
+            if (fuse.resid_out && blockIdx.x == 0 && k < K) *reinterpret_cast<f32x4 *>(fuse.resid_out + k) = xr[u];
+        }
+    }
+    if (fuse.norm_w) {
+        float ss = 0.f;
+#pragma unroll
+        for (int u = 0; u < XU; u++) ss += (xr[u][0] * xr[u][0] + xr[u][1] * xr[u][1]) + (xr[u][2] * xr[u][2] + xr[u][3] * xr[u][3]);
+        ss = wave_sum(ss);
+        if (lane == 0) red[wave] = ss;
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");  // LDS only: the weight loads stay in flight
+        float tot = 0.f;
+#pragma unroll
+        for (int wv = 0; wv < PWAVES; wv++) tot += red[wv];
+        const float inv = 1.0f / sqrtf(tot / (float)K + fuse.eps);
+#pragma unroll
+        for (int u = 0; u < XU; u++)
+#pragma unroll
+            for (int e = 0; e < 4; e++) xr[u][e] = (xr[u][e] * inv) * nr[u][e];
+    }
+#pragma unroll
+    for (int u = 0; u < XU; u++) {
+        const int k = (tid + u * PTHREADS) * 4;
+        if (k < K) *reinterpret_cast<f32x4 *>(xs + k) = xr[u];
+    }
+    for (int k = (tid + XU * PTHREADS) * 4; k < K; k += PTHREADS * 4) {  // longer rows (no norm here)
+        f32x4 v = *reinterpret_cast<const f32x4 *>(x + k);
+        if (fuse.x2) {
+            const f32x4 o = *reinterpret_cast<const f32x4 *>(fuse.x2 + k);
+#pragma unroll
+            for (int e = 0; e < 4; e++) v[e] = (v[e] / (1.0f + expf(-v[e]))) * o[e];
+        } else if (fuse.res_in) {
+            v += *reinterpret_cast<const f32x4 *>(fuse.res_in + k);
+            if (fuse.resid_out && blockIdx.x == 0) *reinterpret_cast<f32x4 *>(fuse.resid_out + k) = v;
+        }
+        *reinterpret_cast<f32x4 *>(xs + k) = v;
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    float xv[CPL][8], sxo[CPL];
+#pragma unroll
+    for (int t = 0; t < CPL; t++) load_xv<QT>(xs, col[t], xv[t], sxo[t]);
+
+    float best_v = -INFINITY;
+    int best_i = -1;
+    for (; trip < ntrips; trip += nwaves) {
+        QWords<QT> qc[RB][CPL];
+        uint32_t sc[RB][CPL];
+#pragma unroll
+        for (int r = 0; r < RB; r++)
+#pragma unroll
+            for (int t = 0; t < CPL; t++) {
+                qc[r][t] = qn[r][t];
+                sc[r][t] = sn[r][t];
+            }
+        if (trip + nwaves < ntrips) request(trip + nwaves);  // the next trip travels while this one is multiplied
+        float a[RB];
+#pragma unroll
+        for (int r = 0; r < RB; r++) a[r] = 0.f;
+#pragma unroll
+        for (int t = 0; t < CPL; t++)
+#pragma unroll
+            for (int r = 0; r < RB; r++) {
+                const float v = quarter_value<QT>(qc[r][t], sc[r][t], xv[t], sxo[t]);
+                a[r] += live[t] ? v : 0.f;
+            }
+        // wave sums of the RB rows, the chains stepping side by side
+#pragma unroll
+        for (int r = 0; r < RB; r++) a[r] += dpp_move<0xB1, 0xF>(a[r], 0.f);
+#pragma unroll
+        for (int r = 0; r < RB; r++) a[r] += dpp_move<0x4E, 0xF>(a[r], 0.f);
+#pragma unroll
+        for (int r = 0; r < RB; r++) a[r] += dpp_move<0x141, 0xF>(a[r], 0.f);
+#pragma unroll
+        for (int r = 0; r < RB; r++) a[r] += dpp_move<0x140, 0xF>(a[r], 0.f);
+#pragma unroll
+        for (int r = 0; r < RB; r++) a[r] += dpp_move<0x142, 0xA>(a[r], 0.f);
+#pragma unroll
+        for (int r = 0; r < RB; r++) a[r] += dpp_move<0x143, 0xC>(a[r], 0.f);
+#pragma unroll
+        for (int r = 0; r < RB; r++) {
+            const int row = trip * RB + r;
+            float v = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(a[r]), 63));
+            if (row < N) {
+                if (fuse.res_out_add) v = v + fuse.res_out_add[row];
+                if (lane == 0) out[row] = v;
+                // of equal maxima the later row wins (Rust Iterator::max_by, reference src/generate.rs:735-742)
+                if (best_i < 0 || v > best_v || (v == best_v && row > best_i)) {
+                    best_v = v;
+                    best_i = row;
+                }
+            }
+        }
+    }
+    if (fuse.cand_v) {  // the workgroup's best row: largest value, highest index among equals; -1 = no row
+        __syncthreads();
+        float *cv = red;
+        int *ci = reinterpret_cast<int *>(red) + PWAVES;
+        if (lane == 0) {
+            cv[wave] = best_v;
+            ci[wave] = best_i;
+        }
+        __syncthreads();
+        if (tid == 0) {
+            float bv = -INFINITY;
+            int bi = -1;
+            for (int wv = 0; wv < PWAVES; wv++) {
+                if (ci[wv] < 0) continue;
+                if (bi < 0 || cv[wv] > bv || (cv[wv] == bv && ci[wv] > bi)) {
+                    bv = cv[wv];
+                    bi = ci[wv];
+                }
+            }
+            fuse.cand_v[blockIdx.x] = bv;
+            fuse.cand_i[blockIdx.x] = bi;
+        }
+    }
+}
+
+// raw GGUF blocks [N][K / 32] -> planes; one thread per quarter block
+template <int QT>
+__global__ __launch_bounds__(256) void pack_planes_kernel(const uint8_t *__restrict__ blocks, uint8_t *__restrict__ quants,
+                                                          uint16_t *__restrict__ scales, size_t n_quarters) {
+    constexpr int QB = PlaneTraits<QT>::QBYTES, BB = PlaneTraits<QT>::BLOCK;
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n_quarters) return;
+    const size_t b = i >> 2;
+    const int q = (int)(i & 3);
+    const uint8_t *blk = blocks + b * BB;
+    if (q == 0) scales[b] = (uint16_t)(blk[0] | (blk[1] << 8));
+#pragma unroll
+    for (int j = 0; j < QB; j++) quants[i * QB + j] = blk[2 + q * QB + j];
+}
+
+// planes -> raw blocks (the inverse, for checks)
+template <int QT>
+__global__ __launch_bounds__(256) void unpack_planes_kernel(const uint8_t *__restrict__ quants, const uint16_t *__restrict__ scales,
+                                                            uint8_t *__restrict__ blocks, size_t n_quarters) {
+    constexpr int QB = PlaneTraits<QT>::QBYTES, BB = PlaneTraits<QT>::BLOCK;
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n_quarters) return;
+    const size_t b = i >> 2;
+    const int q = (int)(i & 3);
+    uint8_t *blk = blocks + b * BB;
+    if (q == 0) {
+        blk[0] = (uint8_t)(scales[b] & 0xFF);
+        blk[1] = (uint8_t)(scales[b] >> 8);
+    }
+#pragma unroll
+    for (int j = 0; j < QB; j++) blk[2 + q * QB + j] = quants[i * QB + j];
+}
+
+// One thread per element, the reference's one multiply (src/gguf.rs:825-829), read from the planes.
+template <int QT>
+__global__ __launch_bounds__(256) void dequant_planes_kernel(const uint8_t *__restrict__ quants, const uint16_t *__restrict__ scales,
+                                                             float *__restrict__ out, size_t n_elems) {
+    size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (; e < n_elems; e += stride) {
+        const size_t b = e >> 5;
+        const int j = (int)(e & 31);
+        const float d = f16_bits_to_f32(scales[b]);
+        float q;
+        if (QT == 0) {
+            q = (float)(int8_t)quants[e];
+        } else {
+            const uint8_t byte = quants[b * 16 + (j & 15)];
+            q = (float)((j < 16 ? (byte & 0x0F) : (byte >> 4)) - 8);
+        }
+        out[e] = __fmul_rn(q, d);
+    }
+}
+
+// Rows per trip for C quarter columns per lane: two trips live in registers (this one and the next), and
+// four workgroups should fit a CU, so the longer the rows the fewer of them; a power of two up to 8.
+template <int QT, int C>
+struct TripRows {
+    static constexpr int CAP = 12 / C;
+    static constexpr int MOST = CAP >= 8 ? 8 : (CAP >= 4 ? 4 : (CAP >= 2 ? 2 : 1));
+};
+
+constexpr int planes_cpl_instance(int cpl) {  // the kernel instance that serves cpl quarter columns per lane
+    return cpl <= 4 ? cpl : (cpl <= 6 ? 6 : 8);
+}
+
+struct PlanesShape {
+    int rb, grid;
+    size_t lds;
+};
+
+PlanesShape planes_shape(const hm_ctx *ctx, bool q4, int K, int N) {
+    PlanesShape s;
+    const int c = planes_cpl_instance((K / 8 + WAVE - 1) / WAVE);
+    const int cap = 12 / c;
+    const int most = cap >= 8 ? 8 : (cap >= 4 ? 4 : (cap >= 2 ? 2 : 1));
+    // long trips where there are rows enough to give every CU two workgroups of them, else single rows
+    (void)q4;
+    s.rb = (N + most - 1) / most >= 2 * PWAVES * ctx->num_cus ? most : 1;
+    const int ntrips = (N + s.rb - 1) / s.rb;
+    const int want = (ntrips + PWAVES - 1) / PWAVES;
+    const int persistent = 4 * ctx->num_cus;  // four workgroups a CU: measured better than two with trips twice as long
+    s.grid = want < persistent ? want : persistent;
+    if (s.grid < 1) s.grid = 1;
+    s.lds = (size_t)K * 4 + 2 * PWAVES * 4 + 16;
+    return s;
+}
+
+template <int QT>
+int planes_launch(hm_ctx *ctx, const char *name, const float *d_x, const uint8_t *d_planes, float *d_out, int M, int K, int N,
+                  const QuantFuse &fuse) {
+    HM_CHECK_CTX(ctx);
+    HM_REQUIRE(ctx, d_x && d_planes && d_out, "%s: NULL pointer", name);
+    HM_REQUIRE(ctx, M >= 1 && M <= 8, "%s: M=%d outside 1..8", name, M);
+    HM_REQUIRE(ctx, K > 0 && K % 32 == 0 && K <= 4096 && N > 0, "%s: K=%d must be a multiple of 32 up to 4096, N=%d positive", name, K, N);
+    HM_REQUIRE(ctx, ((uintptr_t)d_planes % 16) == 0 && ((uintptr_t)d_x % 16) == 0, "%s: weight and activation buffers must be 16-byte aligned", name);
+    HM_REQUIRE(ctx, !(fuse.x2 && fuse.res_in), "%s: SiLU pair and residual input exclude each other", name);
+    HM_REQUIRE(ctx, !fuse.norm_w || K <= 4096, "%s: the fused RMSNorm holds rows up to 4096 wide (K=%d)", name, K);
+    HM_REQUIRE(ctx, ((uintptr_t)fuse.x2 % 16) == 0 && ((uintptr_t)fuse.res_in % 16) == 0 && ((uintptr_t)fuse.resid_out % 16) == 0 &&
+                        ((uintptr_t)fuse.norm_w % 16) == 0, "%s: fused operands must be 16-byte aligned", name);
+    HM_REQUIRE(ctx, M == 1 || (!fuse.x2 && !fuse.res_in && !fuse.norm_w && !fuse.res_out_add), "%s: fused light ops need M == 1", name);
+    HM_REQUIRE(ctx, !fuse.cand_v || fuse.cand_i, "%s: argmax candidates need an index buffer", name);
+    const bool q4 = QT == 1;
+    const PlanesShape sh = planes_shape(ctx, q4, K, N);
+    const uint8_t *quants = d_planes;
+    const uint16_t *scales = reinterpret_cast<const uint16_t *>(d_planes + homura::quant_planes_scale_offset(q4, N, K));
+    const int cpl = (K / 8 + WAVE - 1) / WAVE;
+    const bool fused = fuse.x2 || fuse.res_in || fuse.norm_w || fuse.res_out_add || fuse.cand_v;
+    for (int m = 0; m < M; m++) {
+        const float *xm = d_x + (size_t)m * K;
+        float *om = d_out + (size_t)m * N;
+#define HM_PL(C, R)                                                                                                        \
+    do {                                                                                                                   \
+        if (fused)                                                                                                         \
+            hipLaunchKernelGGL((gemv_planes_kernel<QT, C, R, true>), dim3(sh.grid), dim3(PTHREADS), sh.lds, ctx->stream, xm, \
+                               quants, scales, om, K, N, fuse);                                                            \
+        else                                                                                                               \
+            hipLaunchKernelGGL((gemv_planes_kernel<QT, C, R, false>), dim3(sh.grid), dim3(PTHREADS), sh.lds, ctx->stream, xm, \
+                               quants, scales, om, K, N, fuse);                                                            \
+    } while (0)
+#define HM_PL_RB(C)                                      \
+    do {                                                 \
+        if (sh.rb == 1)                                  \
+            HM_PL(C, 1);                                 \
+        else                                             \
+            HM_PL(C, (TripRows<QT, C>::MOST));           \
+    } while (0)
+        switch (planes_cpl_instance(cpl)) {
+        case 1: HM_PL_RB(1); break;
+        case 2: HM_PL_RB(2); break;
+        case 3: HM_PL_RB(3); break;
+        case 4: HM_PL_RB(4); break;
+        case 6: HM_PL_RB(6); break;
+        default: HM_PL_RB(8); break;
+        }
+#undef HM_PL_RB
+#undef HM_PL
+        HM_LAUNCH_CHECK(ctx);
+    }
+    return HM_OK;
+}
+
+template <int QT>
+int pack_launch(hm_ctx *ctx, const char *name, const uint8_t *d_blocks, uint8_t *d_planes, int N, int K, bool unpack) {
+    HM_CHECK_CTX(ctx);
+    HM_REQUIRE(ctx, d_blocks && d_planes, "%s: NULL pointer", name);
+    HM_REQUIRE(ctx, N > 0 && K > 0 && K % 32 == 0, "%s: K=%d must be a positive multiple of 32, N=%d positive", name, K, N);
+    HM_REQUIRE(ctx, ((uintptr_t)d_planes % 16) == 0, "%s: the planes must be 16-byte aligned", name);
+    const size_t nq = (size_t)N * (K / 8);
+    uint16_t *scales = reinterpret_cast<uint16_t *>(d_planes + homura::quant_planes_scale_offset(QT == 1, N, K));
+    const unsigned grid = (unsigned)((nq + 255) / 256);
+    if (unpack)
+        hipLaunchKernelGGL((unpack_planes_kernel<QT>), dim3(grid), dim3(256), 0, ctx->stream, d_planes, scales,
+                           const_cast<uint8_t *>(d_blocks), nq);
+    else
+        hipLaunchKernelGGL((pack_planes_kernel<QT>), dim3(grid), dim3(256), 0, ctx->stream, d_blocks, d_planes, scales, nq);
+    HM_LAUNCH_CHECK(ctx);
+    return HM_OK;
+}
+
+}  // namespace
+
+size_t homura::quant_planes_scale_offset(bool q4, int N, int K) {
+    const size_t qbytes = (size_t)N * (q4 ? K / 2 : K);
+    return (qbytes + 255) & ~(size_t)255;
+}
+
+size_t homura::quant_planes_bytes(bool q4, int N, int K) {
+    return quant_planes_scale_offset(q4, N, K) + (size_t)N * (K / 32) * 2;
+}
+
+int homura::gemv_planes_workgroups(const hm_ctx *ctx, bool q4, int K, int N) { return planes_shape(ctx, q4, K, N).grid; }
+
+int homura::gemv_planes_fused(hm_ctx *ctx, bool q4, const float *d_x, const uint8_t *d_planes, float *d_out, int K, int N,
+                              const QuantFuse &fuse) {
+    return q4 ? planes_launch<1>(ctx, "gemv_planes[q4_0]", d_x, d_planes, d_out, 1, K, N, fuse)
+              : planes_launch<0>(ctx, "gemv_planes[q8_0]", d_x, d_planes, d_out, 1, K, N, fuse);
+}
+
+int homura::pack_quant_planes(hm_ctx *ctx, bool q4, const uint8_t *d_blocks, uint8_t *d_planes, int N, int K) {
+    return q4 ? pack_launch<1>(ctx, "pack_quant_planes[q4_0]", d_blocks, d_planes, N, K, false)
+              : pack_launch<0>(ctx, "pack_quant_planes[q8_0]", d_blocks, d_planes, N, K, false);
+}
+
+extern "C" {
+
+size_t hm_quant_planes_bytes(int hm_dtype, int N, int K) {
+    if ((hm_dtype != HM_DTYPE_Q8_0 && hm_dtype != HM_DTYPE_Q4_0) || N <= 0 || K <= 0 || K % 32 != 0) return 0;
+    return homura::quant_planes_bytes(hm_dtype == HM_DTYPE_Q4_0, N, K);
+}
+
+int hm_pack_quant_planes(hm_ctx *ctx, int hm_dtype, const uint8_t *d_blocks, uint8_t *d_planes, int N, int K) {
+    HM_CHECK_CTX(ctx);
+    HM_REQUIRE(ctx, hm_dtype == HM_DTYPE_Q8_0 || hm_dtype == HM_DTYPE_Q4_0, "hm_pack_quant_planes: dtype %d is not Q8_0 or Q4_0", hm_dtype);
+    return homura::pack_quant_planes(ctx, hm_dtype == HM_DTYPE_Q4_0, d_blocks, d_planes, N, K);
+}
+
+int hm_unpack_quant_planes(hm_ctx *ctx, int hm_dtype, const uint8_t *d_planes, uint8_t *d_blocks, int N, int K) {
+    HM_CHECK_CTX(ctx);
+    HM_REQUIRE(ctx, hm_dtype == HM_DTYPE_Q8_0 || hm_dtype == HM_DTYPE_Q4_0, "hm_unpack_quant_planes: dtype %d is not Q8_0 or Q4_0", hm_dtype);
+    return hm_dtype == HM_DTYPE_Q4_0 ? pack_launch<1>(ctx, "hm_unpack_quant_planes", d_blocks, const_cast<uint8_t *>(d_planes), N, K, true)
+                                     : pack_launch<0>(ctx, "hm_unpack_quant_planes", d_blocks, const_cast<uint8_t *>(d_planes), N, K, true);
+}
+
+int hm_gemv_q8_0_planes(hm_ctx *ctx, const float *d_x, const uint8_t *d_planes, float *d_out, int M, int K, int N) {
+    return planes_launch<0>(ctx, "hm_gemv_q8_0_planes", d_x, d_planes, d_out, M, K, N, QuantFuse());
+}
+
+int hm_gemv_q4_0_planes(hm_ctx *ctx, const float *d_x, const uint8_t *d_planes, float *d_out, int M, int K, int N) {
+    return planes_launch<1>(ctx, "hm_gemv_q4_0_planes", d_x, d_planes, d_out, M, K, N, QuantFuse());
+}
+
+int hm_dequant_quant_planes(hm_ctx *ctx, int hm_dtype, const uint8_t *d_planes, float *d_out, int N, int K) {
+    HM_CHECK_CTX(ctx);
+    HM_REQUIRE(ctx, hm_dtype == HM_DTYPE_Q8_0 || hm_dtype == HM_DTYPE_Q4_0, "hm_dequant_quant_planes: dtype %d is not Q8_0 or Q4_0", hm_dtype);
+    HM_REQUIRE(ctx, d_planes && d_out && N > 0 && K > 0 && K % 32 == 0, "hm_dequant_quant_planes: bad arguments");
+    const bool q4 = hm_dtype == HM_DTYPE_Q4_0;
+    const size_t n = (size_t)N * K;
+    size_t blocks = (n + 255) / 256;
+    if (blocks > 65536) blocks = 65536;
+    const uint16_t *scales = reinterpret_cast<const uint16_t *>(d_planes + homura::quant_planes_scale_offset(q4, N, K));
+    if (q4)
+        hipLaunchKernelGGL((dequant_planes_kernel<1>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, d_planes, scales, d_out, n);
+    else
+        hipLaunchKernelGGL((dequant_planes_kernel<0>), dim3((unsigned)blocks), dim3(256), 0, ctx->stream, d_planes, scales, d_out, n);
+    HM_LAUNCH_CHECK(ctx);
+    return HM_OK;
+}
+
+}  // extern "C"

@@ -156,12 +156,16 @@ class HfModel {
     // packed storage the bf16 weight slot buffers are views of
     // qkv_bias: f32 [q_dim + 2 kv_dim]. quant[j] (j = q k v o gate up down) is set for the first
     // matrix of each run of same-type neighbours inside q|k|v and gate|up, and holds the whole run.
-    struct LayerPacked { Buffer qkv, o, gate_up, down, qkv_bias, quant[7]; };
+    // quant[first]: the raw blocks of a stacked run; planes[first]: the same run re-packed for the decode
+    // GEMVs (Q8_0 / Q4_0 with K <= 4096; empty otherwise)
+    struct LayerPacked { Buffer qkv, o, gate_up, down, qkv_bias, quant[7], planes[7]; };
+    int build_quant_planes();
     // First member and member count of the stacked run that projection `which` of `layer` belongs to.
     void quant_run(int layer, int which, int *first, int *count) const;
     std::vector<LayerPacked> packed_;
     Buffer lm_head_packed_;
-    Buffer lm_head_blocks_;             // set_lm_head_blocks: raw K-quant blocks of the output matrix
+    Buffer lm_head_blocks_;             // set_lm_head_blocks: raw blocks of the output matrix
+    Buffer lm_head_planes_;             // Q8_0 / Q4_0 output matrix re-packed for the decode GEMV
     DType lm_head_blocks_dtype_ = DType::F32;
     Buffer rope_cos_, rope_sin_;        // [max_position][head_dim] f32
     Buffer ids_view_, mask_view_;

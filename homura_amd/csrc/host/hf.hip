@@ -10,6 +10,7 @@
 #include "../gemm_bf16_mfma.h"
 #include "../gemv_kquant.h"
 #include "../gemv_quant.h"
+#include "../gemv_quant_planes.h"
 #include "../prefill.h"
 #include "../light_ops.h"
 
@@ -136,6 +137,41 @@ void HfModel::quant_run(int layer, int which, int *first, int *count) const {
     while (hi < gmax && proj_dtype(layer, hi + 1) == t) hi++;
     *first = lo;
     *count = hi - lo + 1;
+}
+
+// The decode GEMVs of Q8_0 / Q4_0 runs read a re-packed copy of the blocks (quant bytes and scales in
+// planes of their own: same bytes, naturally aligned words); the raw blocks stay for the prompt pass and
+// the weight listing. HOMURA_QUANT_PLANES=0 keeps the decode on the raw blocks.
+int HfModel::build_quant_planes() {
+    if (const char *e = std::getenv("HOMURA_QUANT_PLANES"))
+        if (std::atoi(e) == 0) return HM_OK;
+    const int hidden = cfg_.hidden_size, inter = cfg_.intermediate_size, qd = cfg_.q_dim(), kvd = cfg_.kv_dim();
+    const int kdim[7] = {hidden, hidden, hidden, qd, hidden, hidden, inter};
+    const int ndim[7] = {qd, kvd, kvd, hidden, inter, inter, hidden};
+    for (int l = 0; l < cfg_.num_hidden_layers; l++)
+        for (int j = 0; j < 7; j++) {
+            int first, count;
+            quant_run(l, j, &first, &count);
+            const DType t = proj_dtype(l, j);
+            if (first != j || (t != DType::Q8_0 && t != DType::Q4_0) || kdim[j] > 4096 || !packed_[l].quant[j]) continue;
+            int n = 0;
+            for (int e = j; e < j + count; e++) n += ndim[e];
+            const size_t bytes = quant_planes_bytes(t == DType::Q4_0, n, kdim[j]);
+            packed_[l].planes[j] = Buffer::alloc_bytes(ctx_, bytes, {(int64_t)bytes}, t);
+            if (!packed_[l].planes[j]) return HM_ERR_OOM;
+            const int rc = pack_quant_planes(ctx_, t == DType::Q4_0, packed_[l].quant[j].as<uint8_t>(),
+                                             packed_[l].planes[j].as<uint8_t>(), n, kdim[j]);
+            if (rc != HM_OK) return rc;
+        }
+    if (lm_head_blocks_ && (lm_head_blocks_dtype_ == DType::Q8_0 || lm_head_blocks_dtype_ == DType::Q4_0) && hidden <= 4096) {
+        const bool q4 = lm_head_blocks_dtype_ == DType::Q4_0;
+        const size_t bytes = quant_planes_bytes(q4, cfg_.vocab_size, hidden);
+        lm_head_planes_ = Buffer::alloc_bytes(ctx_, bytes, {(int64_t)bytes}, lm_head_blocks_dtype_);
+        if (!lm_head_planes_) return HM_ERR_OOM;
+        const int rc = pack_quant_planes(ctx_, q4, lm_head_blocks_.as<uint8_t>(), lm_head_planes_.as<uint8_t>(), cfg_.vocab_size, hidden);
+        if (rc != HM_OK) return rc;
+    }
+    return hm_sync(ctx_);
 }
 
 HfModel::~HfModel() {
@@ -383,6 +419,7 @@ int HfModel::finalize(int max_seq_len) {
         }
     }
 
+    if (dtype_is_quantized(weight_dtype_) && (rc = build_quant_planes()) != HM_OK) return rc;
     rc = dtype_is_quantized(weight_dtype_) ? emit_transformer_plan_quant() : emit_transformer_plan();
     if (rc != HM_OK) return rc;
     rc = plan_->prepare(std::max(max_seq_len, 16));
@@ -911,7 +948,7 @@ int HfModel::emit_transformer_plan_quant() {
     // A second run of the group that rides in the first run's launch (the two K-quant types side by side)
     struct PairedRun { size_t w_slot = (size_t)-1, out_slot = (size_t)-1; int64_t N = 0; DType dtype = DType::F32; std::string label; };
     auto quant_mm = [&](const char *label, DType wdt, int64_t K, int64_t N, bool reuse_act, FuseSlots fs,
-                        PairedRun pair = PairedRun()) {
+                        PairedRun pair = PairedRun(), const uint8_t *planes = nullptr) {
         CompiledKernel k;
         k.ops_label = std::string("QuantMM[") + label + "]";
         if (N > 0 && pair.N > 0) {
@@ -955,6 +992,8 @@ int HfModel::emit_transformer_plan_quant() {
                 f.norm_w = f32(fs.norm_w);
                 f.eps = eps;
                 f.res_out_add = f32(fs.add);
+                if (planes)  // the run re-packed at finalize
+                    return gemv_planes_fused(sc.ctx, wdt == DType::Q4_0, x, planes, out, (int)K, (int)N, f);
                 if (wdt == DType::Q8_0 || wdt == DType::Q4_0)
                     return gemv_quant_fused(sc.ctx, wdt == DType::Q4_0, x, w, out, (int)K, (int)N, f);
                 if (K <= 4096)  // the row is prepared and quantised to Q8_K inside the kernel
@@ -1016,7 +1055,9 @@ int HfModel::emit_transformer_plan_quant() {
             } else if (paired && run == &runs[1]) {
                 n_run = 0;  // rides in the first run's launch
             }
-            add_step(quant_mm(label.c_str(), t, K, n_run, kq && act_quantized, fs, pair), {act_slot, gm.w_slot}, {gm.out_slot});
+            const Buffer &pl = packed_[layer].planes[gm.which];  // set for the first member of a re-packed run
+            add_step(quant_mm(label.c_str(), t, K, n_run, kq && act_quantized, fs, pair, n_run > 0 && pl ? pl.as<uint8_t>() : nullptr),
+                     {act_slot, gm.w_slot}, {gm.out_slot});
             if (n_run > 0 && kq) act_quantized = true;
         }
     };
@@ -1229,6 +1270,7 @@ int HfModel::emit_transformer_plan_quant() {
         const DType head_dt = lm_head_blocks_dtype_;
         const bool head_q6 = head_dt == DType::Q6_K;
         const bool head_k = head_dt == DType::Q4_K || head_dt == DType::Q6_K;  // else Q8_0 / Q4_0
+        const uint8_t *head_planes = lm_head_planes_ ? lm_head_planes_.as<uint8_t>() : nullptr;
         h1.name = !head_blocks ? "gemv_f32[lm_head+argmax]"
                   : head_q6    ? "gemv_q6_k_f32[lm_head+argmax]"
                   : head_k     ? "gemv_q4_k_f32[lm_head+argmax]"
@@ -1242,6 +1284,9 @@ int HfModel::emit_transformer_plan_quant() {
                 f.eps = eps;
                 f.cand_v = scr->cand_val.as<float>();
                 f.cand_i = scr->cand_idx.as<int>();
+                if (head_planes)
+                    return gemv_planes_fused(sc.ctx, head_dt == DType::Q4_0, sc.pool[in[0]]->as<float>(), head_planes,
+                                             sc.pool[sc.step.output_slots[0]]->as<float>(), (int)hidden, (int)vocab, f);
                 return gemv_quant_fused(sc.ctx, head_dt == DType::Q4_0, sc.pool[in[0]]->as<float>(), sc.pool[in[2]]->as<uint8_t>(),
                                         sc.pool[sc.step.output_slots[0]]->as<float>(), (int)hidden, (int)vocab, f);
             }
@@ -1272,6 +1317,7 @@ int HfModel::emit_transformer_plan_quant() {
         h2.fn = [=](const StepContext &sc) -> int {
             const int ncand = !head_blocks ? std::min(gemv_bf16_nk_grid(sc.ctx, (int)vocab, 4), scr->cand_cap)
                               : head_k ? gemv_kquant_f32_head_candidates(sc.ctx, head_q6, (int)hidden, (int)vocab, scr->cand_cap)
+                              : head_planes ? gemv_planes_workgroups(sc.ctx, head_dt == DType::Q4_0, (int)hidden, (int)vocab)
                                        : gemv_quant_workgroups(sc.ctx, head_dt == DType::Q4_0, (int)hidden, (int)vocab);
             return finish_step_launch(sc.ctx, sc.plan->state(), scr->cand_val.as<float>(),
                                       scr->cand_idx.as<int>(), ncand, sc.plan->out_tokens(),

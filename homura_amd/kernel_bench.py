@@ -76,6 +76,30 @@ def run_copy_calibration(ctx: Context):
     return _entry("calibration pack_kn_to_nk 4096x4096 bf16 (read 32 MiB + write 32 MiB)", us, 2 * K * N * 2)
 
 
+def run_quant_cases(ctx: Context):
+    """Configurations 3 and 4, each on the raw GGUF blocks (what a drop-in caller hands over) and on the
+    same weights re-packed into planes at upload (what the model keeps)."""
+    from .runtime import DTYPE_Q4_0, DTYPE_Q8_0
+    out = []
+    for name, dt, bb, blocks, seed, K, N, raw_fn, planes_fn in (
+            ("cfg3 gemv_q8_0 2048->5632", DTYPE_Q8_0, 34, synth.q8_0_blocks, synth.SEED_CFG3, 2048, 5632, ctx.gemv_q8_0, ctx.gemv_q8_0_planes),
+            ("cfg4 gemv_q4_0 1536->151936", DTYPE_Q4_0, 18, synth.q4_0_blocks, synth.SEED_CFG4, 1536, 151936, ctx.gemv_q4_0, ctx.gemv_q4_0_planes)):
+        x = ctx.to_device(synth.normal_f32(seed + 1, K))
+        ring = _ring(ctx, blocks(seed, N * K // 32))
+        o = ctx.empty(N)
+        nbytes = N * (K // 32) * bb + K * 4 + N * 4
+        us = _time(ctx, [lambda b=b: raw_fn(x, b, o, 1, K, N) for b in ring])
+        out.append(_entry(name, us, nbytes, note="raw GGUF blocks"))
+        planes = [ctx.pack_quant_planes(dt, b, N, K) for b in ring]
+        for b in ring:
+            b.free()
+        us = _time(ctx, [lambda p=p: planes_fn(x, p, o, 1, K, N) for p in planes])
+        out.append(_entry(name.replace(" gemv", " planes gemv"), us, nbytes, note="the same blocks re-packed into planes at upload"))
+        for b in planes + [x, o]:
+            b.free()
+    return out
+
+
 def run_all(ctx: Context):
     out = [run_copy_calibration(ctx)]
     # configuration 1: single bf16 GEMV x[1,896] x W[896,4864]
@@ -92,25 +116,7 @@ def run_all(ctx: Context):
     for b in ring:
         b.free()
 
-    # configuration 3: Q8_0 dequant-GEMV 2048 -> 5632
-    K, N = 2048, 5632
-    x = ctx.to_device(synth.normal_f32(synth.SEED_CFG3 + 1, K))
-    ring = _ring(ctx, synth.q8_0_blocks(synth.SEED_CFG3, N * K // 32))
-    o = ctx.empty(N)
-    us = _time(ctx, [lambda b=b: ctx.gemv_q8_0(x, b, o, 1, K, N) for b in ring])
-    out.append(_entry("cfg3 gemv_q8_0 2048->5632", us, N * (K // 32) * 34 + K * 4 + N * 4))
-    for b in ring:
-        b.free()
-
-    # configuration 4: Q4_0 dequant-GEMV at LM-head shape 1536 -> 151936
-    K, N = 1536, 151936
-    x = ctx.to_device(synth.normal_f32(synth.SEED_CFG4 + 1, K))
-    ring = _ring(ctx, synth.q4_0_blocks(synth.SEED_CFG4, N * K // 32))
-    o = ctx.empty(N)
-    us = _time(ctx, [lambda b=b: ctx.gemv_q4_0(x, b, o, 1, K, N) for b in ring])
-    out.append(_entry("cfg4 gemv_q4_0 1536->151936", us, N * (K // 32) * 18 + K * 4 + N * 4))
-    for b in ring:
-        b.free()
+    out += run_quant_cases(ctx)
 
     # configuration 5a: prefill-chunk GEMM 512 x 2048 x 8192 on the matrix cores
     M, K, N = 512, 2048, 8192

@@ -154,6 +154,24 @@ class Context:
     def gemv_q4_0(self, x, w, out, M, K, N):
         self._check(self.lib.hm_gemv_q4_0(self.h, x.ptr, w.ptr, out.ptr, M, K, N))
 
+    def pack_quant_planes(self, dtype, blocks, N, K):
+        """Raw Q8_0 / Q4_0 blocks [N][K/32] (device buffer) -> a new device buffer holding their planes."""
+        planes = self.alloc(self.lib.hm_quant_planes_bytes(dtype, N, K))
+        self._check(self.lib.hm_pack_quant_planes(self.h, dtype, blocks.ptr, planes.ptr, N, K))
+        return planes
+
+    def unpack_quant_planes(self, dtype, planes, blocks_out, N, K):
+        self._check(self.lib.hm_unpack_quant_planes(self.h, dtype, planes.ptr, blocks_out.ptr, N, K))
+
+    def gemv_q8_0_planes(self, x, planes, out, M, K, N):
+        self._check(self.lib.hm_gemv_q8_0_planes(self.h, x.ptr, planes.ptr, out.ptr, M, K, N))
+
+    def gemv_q4_0_planes(self, x, planes, out, M, K, N):
+        self._check(self.lib.hm_gemv_q4_0_planes(self.h, x.ptr, planes.ptr, out.ptr, M, K, N))
+
+    def dequant_quant_planes(self, dtype, planes, out, N, K):
+        self._check(self.lib.hm_dequant_quant_planes(self.h, dtype, planes.ptr, out.ptr, N, K))
+
     def gemv_q4_k(self, x, w, out, M, K, N):
         self._check(self.lib.hm_gemv_q4_k(self.h, x.ptr, w.ptr, out.ptr, M, K, N))
 

@@ -103,6 +103,22 @@ int hm_gemv_q8_0(hm_ctx *ctx, const float *d_x, const uint8_t *d_w_blocks, float
 int hm_gemv_q4_0(hm_ctx *ctx, const float *d_x, const uint8_t *d_w_blocks, float *d_out, int M,
                  int K, int N);
 
+/* The same two products over weights re-packed once into "planes": the quant bytes of all blocks row after
+ * row (Q8_0: K bytes a row; Q4_0: K / 2, each block's 16 bytes as in the file), then, from the next
+ * multiple of 256 bytes, the f16 scales of all blocks row after row. The bytes are those of the GGUF blocks
+ * (src/graph_builder/emit_quant.rs:17-21 layout) in another order: quant words sit at their natural
+ * alignment and are loaded straight into registers. hm_quant_planes_bytes gives the size of the planes
+ * of an [N][K] matrix (0 for a type other than HM_DTYPE_Q8_0 / Q4_0 or a bad shape), hm_pack_quant_planes
+ * fills them from raw blocks [N][K/32] in one launch, hm_unpack_quant_planes is its inverse.
+ * Results equal hm_gemv_q8_0 / hm_gemv_q4_0 up to the order of the f32 additions. M <= 8, K % 32 == 0,
+ * K <= 4096. hm_dequant_quant_planes writes the N * K dequantised weights, bit-exact with the CPU. */
+size_t hm_quant_planes_bytes(int hm_dtype, int N, int K);
+int hm_pack_quant_planes(hm_ctx *ctx, int hm_dtype, const uint8_t *d_blocks, uint8_t *d_planes, int N, int K);
+int hm_unpack_quant_planes(hm_ctx *ctx, int hm_dtype, const uint8_t *d_planes, uint8_t *d_blocks, int N, int K);
+int hm_gemv_q8_0_planes(hm_ctx *ctx, const float *d_x, const uint8_t *d_planes, float *d_out, int M, int K, int N);
+int hm_gemv_q4_0_planes(hm_ctx *ctx, const float *d_x, const uint8_t *d_planes, float *d_out, int M, int K, int N);
+int hm_dequant_quant_planes(hm_ctx *ctx, int hm_dtype, const uint8_t *d_planes, float *d_out, int N, int K);
+
 /* Block dequantisation to f32, reference dequant_q8_0 (src/gguf.rs:817-831): one f32
  * multiply per element, bit-exact with the CPU. hm_dequant_q4_0 is its Q4_0 analogue. */
 int hm_dequant_q8_0(hm_ctx *ctx, const uint8_t *d_blocks, float *d_out, size_t nblocks);

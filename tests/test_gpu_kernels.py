@@ -130,6 +130,88 @@ def test_quant_gemv(ctx, oracle, kind, M, K, N):
         b.free()
 
 
+# ── Q8_0 / Q4_0 re-packed into planes ─────────────────────────────────────────
+
+@pytest.mark.parametrize("kind", ["q8_0", "q4_0"])
+def test_quant_planes_hold_the_blocks_bit_for_bit(ctx, oracle, kind):
+    """The re-packed form is the same bytes in another order: packing and unpacking returns the blocks,
+    the planes are where the declaration says (quants row after row, scales from the next multiple of 256
+    bytes), and dequantising from the planes gives the oracle's bits, special scales included."""
+    from homura_amd.runtime import DTYPE_Q4_0, DTYPE_Q8_0
+    dt, bb, qpb = (DTYPE_Q8_0, 34, 32) if kind == "q8_0" else (DTYPE_Q4_0, 18, 16)
+    N, K = 203, 96
+    nb = N * (K // 32)
+    raw = (synth.q8_0_blocks if kind == "q8_0" else synth.q4_0_blocks)(91, nb)
+    blk = raw.reshape(nb, bb)
+    for i, bits in enumerate([0x0001, 0x03FF, 0x0000, 0x8000, 0x7BFF, 0x7C00, 0xFC00, 0x7E00, 0x0400]):
+        blk[i, 0], blk[i, 1] = bits & 0xFF, bits >> 8
+    d_raw = ctx.to_device(raw)
+    planes = ctx.pack_quant_planes(dt, d_raw, N, K)
+    size = ctx.lib.hm_quant_planes_bytes(dt, N, K)
+    qbytes = nb * qpb
+    soff = (qbytes + 255) // 256 * 256
+    assert size == soff + nb * 2
+    host = planes.download(np.uint8)[:size]
+    assert np.array_equal(host[:qbytes].reshape(nb, qpb), blk[:, 2:])
+    assert np.array_equal(host[soff:soff + 2 * nb].reshape(nb, 2), blk[:, :2])
+    back = ctx.empty(raw.size, np.uint8)
+    ctx.unpack_quant_planes(dt, planes, back, N, K)
+    assert np.array_equal(back.download(np.uint8), raw.reshape(-1))
+    want = (oracle.dequant_q8_0 if kind == "q8_0" else oracle.dequant_q4_0)(raw)
+    d_out = ctx.empty(N * K)
+    ctx.dequant_quant_planes(dt, planes, d_out, N, K)
+    got = d_out.download(np.float32)
+    nan = np.isnan(want)
+    assert np.array_equal(np.isnan(got), nan)
+    assert np.array_equal(got[~nan].view(np.uint32), want[~nan].view(np.uint32))
+    for b in (d_raw, planes, back, d_out):
+        b.free()
+
+
+@pytest.mark.parametrize("kind,M,K,N", [("q8_0", 1, 2048, 5632),    # BASELINE config 3
+                                        ("q4_0", 1, 1536, 151936),  # BASELINE config 4
+                                        ("q8_0", 1, 1024, 151936),  # an LM head read from Q8_0 blocks
+                                        ("q8_0", 1, 2048, 2048), ("q8_0", 1, 3072, 1024), ("q8_0", 2, 4096, 77),
+                                        ("q8_0", 1, 32, 5), ("q8_0", 1, 96, 1), ("q8_0", 1, 1024, 6144),
+                                        ("q4_0", 3, 2048, 260), ("q4_0", 1, 32, 7), ("q4_0", 1, 3072, 1024),
+                                        ("q4_0", 1, 256, 233100), ("q4_0", 1, 1792, 33333),
+                                        ("q4_0", 2, 2048, 29201), ("q4_0", 1, 4096, 14601), ("q4_0", 1, 2528, 4099)])
+def test_quant_planes_gemv(ctx, oracle, kind, M, K, N):
+    """The dequant-GEMV over the re-packed weights against the oracle on the raw blocks."""
+    from homura_amd.runtime import DTYPE_Q4_0, DTYPE_Q8_0
+    say(f"gemv_{kind}_planes M={M} K={K} N={N}")
+    nb = N * (K // 32)
+    seed = synth.SEED_CFG3 if kind == "q8_0" else synth.SEED_CFG4
+    raw = (synth.q8_0_blocks if kind == "q8_0" else synth.q4_0_blocks)(seed, nb, 0.01)
+    x = synth.normal_f32(seed + 1, M * K).reshape(M, K)
+    want = (oracle.gemv_q8_0 if kind == "q8_0" else oracle.gemv_q4_0)(x, raw, M, K, N)
+    dx, dw, dout = ctx.to_device(x), ctx.to_device(raw), ctx.empty(M * N)
+    planes = ctx.pack_quant_planes(DTYPE_Q8_0 if kind == "q8_0" else DTYPE_Q4_0, dw, N, K)
+    (ctx.gemv_q8_0_planes if kind == "q8_0" else ctx.gemv_q4_0_planes)(dx, planes, dout, M, K, N)
+    got = dout.download(np.float32, (M, N))
+    assert rel_err(got, want) < TOL
+    # both sides add exact products in f32, in different orders
+    assert np.abs(got - want).max() < 1e-4 * np.sqrt(np.mean(want.astype(np.float64) ** 2))
+    for b in (dx, dw, dout, planes):
+        b.free()
+
+
+def test_quant_planes_reference_kat_and_limits(ctx, golden):
+    from homura_amd.runtime import DTYPE_Q8_0
+    g = golden["emit_q8_0_correctness"]     # reference src/graph_builder/emit_quant.rs:893-958: every output 528
+    N, K = g["N"], g["K"]
+    raw = np.zeros((N, 34), np.uint8)
+    raw[:, 0], raw[:, 1] = g["scale_bits"] & 0xFF, g["scale_bits"] >> 8
+    raw[:, 2:] = np.arange(1, 33, dtype=np.uint8)
+    dx, dw, dout = ctx.to_device(np.ones(K, np.float32)), ctx.to_device(raw), ctx.empty(N)
+    planes = ctx.pack_quant_planes(DTYPE_Q8_0, dw, N, K)
+    ctx.gemv_q8_0_planes(dx, planes, dout, 1, K, N)
+    assert np.all(dout.download(np.float32) == g["expected_each"])
+    assert ctx.lib.hm_quant_planes_bytes(1, 8, 32) == 0 and ctx.lib.hm_quant_planes_bytes(DTYPE_Q8_0, 8, 48) == 0
+    with pytest.raises(HomuraError, match="up to 4096"):
+        ctx.gemv_q8_0_planes(dx, planes, dout, 1, 8192, 1)
+
+
 # ── K-quants ──────────────────────────────────────────────────────────────────
 
 @pytest.mark.parametrize("kind", ["q4_k", "q6_k"])
