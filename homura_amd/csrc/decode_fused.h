@@ -3,11 +3,17 @@
 #pragma once
 #include "hm_common.h"
 
-// Per-layer device pointers. Matrices are in the K-contiguous stream layout the plan keeps:
+// Weight formats the kernel has instances for.
+enum : int { FUSED_WF_BF16 = 0, FUSED_WF_Q8_0 = 1, FUSED_WF_Q4_0 = 2 };
+
+// Per-layer device pointers. bf16: matrices in the K-contiguous stream layout the plan keeps:
 // wqkv [q_dim + 2 kv_dim][hidden], wo [hidden][q_dim], wgu [2 inter][hidden] with gate and up rows
-// interleaved (g0, u0, g1, u1, ...), wd [hidden][inter].
+// interleaved (g0, u0, g1, u1, ...), wd [hidden][inter]; the s* pointers are unused. Q8_0 / Q4_0: w* are the
+// quant planes and s* the scale planes of the same matrices re-packed as gemv_quant_planes.hip describes,
+// q|k|v stacked in that order, wgu all gate rows and then all up rows.
 struct FusedLayerPtrs {
-    const uint16_t *wqkv, *wo, *wgu, *wd;
+    const void *wqkv, *wo, *wgu, *wd;
+    const uint16_t *sqkv, *so, *sgu, *sd;
     const float *in_ln, *post_ln;
     const float *q_norm, *k_norm;  // [head_dim] or nullptr (both)
     const float *qkv_bias;         // [q_dim + 2 kv_dim] or nullptr
@@ -16,6 +22,7 @@ struct FusedLayerPtrs {
 
 struct FusedShape {
     int hidden, heads, kv_heads, head_dim, inter;
+    int wf = FUSED_WF_BF16;  // FUSED_WF_*
 };
 
 struct FusedDecodeArgs {

@@ -338,6 +338,147 @@ __device__ __forceinline__ void wave_max_n(float (&v)[N]) {
     for (int i = 0; i < N; i++) v[i] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v[i]), 63));
 }
 
+// ── the rows of one matrix that a compute wavefront keeps in registers, by weight format ──
+//
+// bf16 (stream layout [N][K]): a lane holds 8 consecutive weights of each 512-wide chunk of a row, and the
+// products are those of gemv_bf16.hip bit for bit. Q8_0 / Q4_0 (planes, gemv_quant_planes.hip: quant
+// bytes [N][K] or [N][K / 2], f16 scales [N][K / 32]): a lane holds half a block, 16 weights, of each
+// 1024-wide chunk plus the block's scale, and a row is sum over half blocks of d * (sum_j q_j x_j -
+// offset * sum_j x_j) with the quants used as stored, as in gemv_quant.hip.
+typedef const uint16_t __attribute__((address_space(1))) *global_u16_ptr;
+typedef const u32x2 __attribute__((address_space(1))) *global_u32x2_ptr;
+
+template <int WF, int R, int K>
+struct Rows;
+
+template <int R, int K>
+struct Rows<FUSED_WF_BF16, R, K> {
+    static constexpr int C = K / 512;
+    static_assert(K % 512 == 0, "bf16 rows are cut into 512-wide chunks");
+    u32x4 w[R][C];
+    template <class RowOf>
+    __device__ __forceinline__ void load(const void *quants, const uint16_t *, RowOf row_of, int r0, int r1, int lane) {
+        const uint16_t *base = reinterpret_cast<const uint16_t *>(quants);
+#pragma unroll
+        for (int r = 0; r < R; r++)
+#pragma unroll
+            for (int c = 0; c < C; c++)
+                if (r >= r0 && r < r1) w[r][c] = ld128_global_stream(base + (size_t)row_of(r) * K + (c * WAVE + lane) * 8);
+    }
+    __device__ __forceinline__ void dots_normed(const float *hx, const float *nw, float inv, int lane, float (&v)[R]) const {
+        float acc[R][C];
+        normed_dots<R, C>(w, hx, nw, inv, lane, acc);
+#pragma unroll
+        for (int r = 0; r < R; r++) v[r] = chunk_total<C>(acc[r]);
+    }
+    __device__ __forceinline__ void dots_plain(const float *x, int lane, float (&v)[R]) const {
+        float acc[R][C];
+        plain_dots<R, C>(w, x, lane, acc);
+#pragma unroll
+        for (int r = 0; r < R; r++) v[r] = chunk_total<C>(acc[r]);
+    }
+};
+
+// The four bytes of w as floats against xv (the empty asm keeps the compiler from folding the mask that made
+// w into one bit-field extract per byte: the conversions select their byte themselves).
+__device__ __forceinline__ float dot4_bytes(uint32_t w, const float *xv, float s) {
+    asm("" : "+v"(w));
+    s = fmaf((float)(w & 0xFFu), xv[0], s);
+    s = fmaf((float)((w >> 8) & 0xFFu), xv[1], s);
+    s = fmaf((float)((w >> 16) & 0xFFu), xv[2], s);
+    s = fmaf((float)(w >> 24), xv[3], s);
+    return s;
+}
+
+template <int WF, int R, int K>
+struct Rows {
+    static constexpr bool Q4 = WF == FUSED_WF_Q4_0;
+    static constexpr int C = K / 1024;
+    static_assert(K % 1024 == 0, "quantised rows are cut into 1024-wide chunks (16 weights a lane)");
+    uint32_t q[R][C][Q4 ? 2 : 4];  // the lane's half block: 8 bytes of nibble pairs or 16 int8
+    uint32_t d[R][C];              // f16 bits of its block's scale
+    template <class RowOf>
+    __device__ __forceinline__ void load(const void *quants, const uint16_t *scales, RowOf row_of, int r0, int r1, int lane) {
+        const unsigned char *base = reinterpret_cast<const unsigned char *>(quants);
+#pragma unroll
+        for (int r = 0; r < R; r++)
+#pragma unroll
+            for (int c = 0; c < C; c++)
+                if (r >= r0 && r < r1) {
+                    const size_t row = (size_t)row_of(r);
+                    const int hb = c * WAVE + lane;  // half block of the row
+                    if constexpr (Q4) {
+                        const u32x2 t = __builtin_nontemporal_load((global_u32x2_ptr)(base + row * (K / 2) + (size_t)hb * 8));
+                        q[r][c][0] = t.x;
+                        q[r][c][1] = t.y;
+                    } else {
+                        const u32x4 t = ld128_global_stream(base + row * K + (size_t)hb * 16);
+                        q[r][c][0] = t.x;
+                        q[r][c][1] = t.y;
+                        q[r][c][2] = t.z;
+                        q[r][c][3] = t.w;
+                    }
+                    d[r][c] = __builtin_nontemporal_load((global_u16_ptr)(scales + row * (K / 32) + (hb >> 1)));
+                }
+    }
+    // the lane's 16 activations of chunk c in the order its quant bytes use them: Q8_0 16 in a row; Q4_0 the
+    // low nibbles' eight (8 h + j of the block), then the high nibbles' (16 + 8 h + j)
+    __device__ __forceinline__ static int x_index(int c, int lane, int part) {
+        const int hb = c * WAVE + lane;
+        return Q4 ? (hb >> 1) * 32 + (hb & 1) * 8 + part * 16 : hb * 16 + part * 8;
+    }
+    __device__ __forceinline__ void finish(const float (&xv)[C][16], float (&v)[R]) const {
+        float off[C];
+#pragma unroll
+        for (int c = 0; c < C; c++) {
+            float sx = 0.f;
+#pragma unroll
+            for (int j = 0; j < 16; j++) sx += xv[c][j];
+            off[c] = sx * (Q4 ? 8.f : 128.f);
+        }
+#pragma unroll
+        for (int r = 0; r < R; r++) v[r] = 0.f;
+#pragma unroll
+        for (int c = 0; c < C; c++)
+#pragma unroll
+            for (int r = 0; r < R; r++) {
+                float sum;
+                if constexpr (Q4) {
+                    const uint32_t w0 = q[r][c][0], w1 = q[r][c][1];
+                    sum = dot4_bytes(w1 & 0x0F0F0F0Fu, xv[c] + 4, dot4_bytes(w0 & 0x0F0F0F0Fu, xv[c], 0.f));
+                    sum = dot4_bytes((w1 >> 4) & 0x0F0F0F0Fu, xv[c] + 12, dot4_bytes((w0 >> 4) & 0x0F0F0F0Fu, xv[c] + 8, sum));
+                } else {
+                    sum = 0.f;
+#pragma unroll
+                    for (int e = 0; e < 4; e++) sum = dot4_bytes(q[r][c][e] ^ 0x80808080u, xv[c] + 4 * e, sum);  // int8 -> biased unsigned
+                }
+                v[r] += f16_bits_to_f32((uint16_t)d[r][c]) * (sum - off[c]);
+            }
+    }
+    __device__ __forceinline__ void dots_normed(const float *hx, const float *nw, float inv, int lane, float (&v)[R]) const {
+        float xv[C][16];
+#pragma unroll
+        for (int c = 0; c < C; c++)
+#pragma unroll
+            for (int part = 0; part < 2; part++) {
+                float hv[8], wv[8];
+                lds_x8(hx, x_index(c, lane, part), hv);
+                lds_x8(nw, x_index(c, lane, part), wv);
+#pragma unroll
+                for (int e = 0; e < 8; e++) xv[c][part * 8 + e] = (hv[e] * inv) * wv[e];
+            }
+        finish(xv, v);
+    }
+    __device__ __forceinline__ void dots_plain(const float *x, int lane, float (&v)[R]) const {
+        float xv[C][16];
+#pragma unroll
+        for (int c = 0; c < C; c++)
+#pragma unroll
+            for (int part = 0; part < 2; part++) lds_x8(x, x_index(c, lane, part), xv[c] + part * 8);
+        finish(xv, v);
+    }
+};
+
 // The attention split of a workgroup for a cache of kv_len rows (the new row included).
 template <class GE>
 struct Split {
@@ -359,34 +500,29 @@ struct Split {
 };
 
 // Registers of one compute wavefront that hold its slice of a layer.
-template <class GE>
+template <class GE, int WF>
 struct Slice {
-    u32x4 wq[GE::RQW][GE::CH];
+    Rows<WF, GE::RQW, GE::HIDDEN> wq;
     u32x4 kr[GE::NR], vr[GE::NR];
-    u32x4 wo[GE::ROW][GE::CO];
-    u32x4 wg[GE::RGW][GE::CH];
-    u32x4 wd[GE::ROW][GE::CD];
+    Rows<WF, GE::ROW, GE::QD> wo;
+    Rows<WF, GE::RGW, GE::HIDDEN> wg;
+    Rows<WF, GE::ROW, GE::INTER> wd;
 };
 
-template <class GE>
+template <class GE, int WF>
 __device__ __forceinline__ void compute_role(const FusedDecodeArgs &a, Lds<GE> &sm, const int wg, const int cw,
                                              const int lane, const int pos) {
     const Split<GE> sp(wg, pos);
     constexpr int LPR = GE::LPR, RPI = GE::RPI, G = GE::G, HD = GE::HD, NR = GE::NR;
     const int sub = lane / LPR, dl = lane % LPR;
     const int L = a.n_layers;
-    Slice<GE> s;
+    Slice<GE, WF> s;
 
     // Requests are spread over the step in small batches (rows [r0, r1) of a slice at a time): a batch that
     // overfills the CU's memory pipeline blocks the wavefront that issues it, and a burst from all
     // CUs at once delays the polls of the communication wavefronts behind it.
     auto load_wq = [&](const FusedLayerPtrs &lp, int r0, int r1) {
-#pragma unroll
-        for (int r = 0; r < GE::RQW; r++)
-#pragma unroll
-            for (int c = 0; c < GE::CH; c++)
-                if (r >= r0 && r < r1)
-                    s.wq[r][c] = ld128_global_stream(lp.wqkv + (size_t)GE::qkv_row(sp.kh, sp.split * GE::RQ + cw * GE::RQW + r) * GE::HIDDEN + (c * WAVE + lane) * 8);
+        s.wq.load(lp.wqkv, lp.sqkv, [&](int r) { return GE::qkv_row(sp.kh, sp.split * GE::RQ + cw * GE::RQW + r); }, r0, r1, lane);
     };
     auto load_kv = [&](const FusedLayerPtrs &lp, int i0, int i1) {
 #pragma unroll
@@ -400,26 +536,18 @@ __device__ __forceinline__ void compute_role(const FusedDecodeArgs &a, Lds<GE> &
         }
     };
     auto load_wo = [&](const FusedLayerPtrs &lp) {
-#pragma unroll
-        for (int r = 0; r < GE::ROW; r++)
-#pragma unroll
-            for (int c = 0; c < GE::CO; c++)
-                s.wo[r][c] = ld128_global_stream(lp.wo + (size_t)(wg * GE::RO + cw * GE::ROW + r) * GE::QD + (c * WAVE + lane) * 8);
+        s.wo.load(lp.wo, lp.so, [&](int r) { return wg * GE::RO + cw * GE::ROW + r; }, 0, GE::ROW, lane);
     };
+    // bf16 keeps gate and up rows interleaved (g0, u0, g1, u1, ...); the quantised formats keep the run as
+    // uploaded, all gate rows and then all up rows, so local row r = 2 p + (0 gate | 1 up) of pair p
     auto load_wg = [&](const FusedLayerPtrs &lp, int r0, int r1) {
-#pragma unroll
-        for (int r = 0; r < GE::RGW; r++)
-#pragma unroll
-            for (int c = 0; c < GE::CH; c++)
-                if (r >= r0 && r < r1)
-                    s.wg[r][c] = ld128_global_stream(lp.wgu + (size_t)(wg * GE::RG + cw * GE::RGW + r) * GE::HIDDEN + (c * WAVE + lane) * 8);
+        s.wg.load(lp.wgu, lp.sgu, [&](int r) {
+            const int lr = cw * GE::RGW + r;
+            return WF == FUSED_WF_BF16 ? wg * GE::RG + lr : (lr & 1) * GE::INTER + wg * GE::APW + (lr >> 1);
+        }, r0, r1, lane);
     };
     auto load_wd = [&](const FusedLayerPtrs &lp) {
-#pragma unroll
-        for (int r = 0; r < GE::ROW; r++)
-#pragma unroll
-            for (int c = 0; c < GE::CD; c++)
-                s.wd[r][c] = ld128_global_stream(lp.wd + (size_t)(wg * GE::RO + cw * GE::ROW + r) * GE::INTER + (c * WAVE + lane) * 8);
+        s.wd.load(lp.wd, lp.sd, [&](int r) { return wg * GE::RO + cw * GE::ROW + r; }, 0, GE::ROW, lane);
     };
 
     constexpr int KV_CUT = NR / 2, WG_CUT = 2 * GE::RGW / 3;
@@ -449,11 +577,8 @@ __device__ __forceinline__ void compute_role(const FusedDecodeArgs &a, Lds<GE> &
         {
             const float tot = ((sm.red[0] + sm.red[1]) + sm.red[2]) + sm.red[3];
             const float inv = 1.0f / sqrtf(tot / (float)GE::HIDDEN + a.eps);
-            float acc[GE::RQW][GE::CH];
-            normed_dots<GE::RQW, GE::CH>(s.wq, sm.hx, sm.nw, inv, lane, acc);
             float v[GE::RQW];
-#pragma unroll
-            for (int r = 0; r < GE::RQW; r++) v[r] = chunk_total<GE::CH>(acc[r]);
+            s.wq.dots_normed(sm.hx, sm.nw, inv, lane, v);
             wave_sum_n<GE::RQW>(v);
             if (has_bias) {
 #pragma unroll
@@ -580,11 +705,8 @@ __device__ __forceinline__ void compute_role(const FusedDecodeArgs &a, Lds<GE> &
         wg_barrier();
         load_kv(nx, 0, KV_CUT);
         {
-            float acc[GE::ROW][GE::CO];
-            plain_dots<GE::ROW, GE::CO>(s.wo, sm.attn, lane, acc);
             float v[GE::ROW];
-#pragma unroll
-            for (int r = 0; r < GE::ROW; r++) v[r] = chunk_total<GE::CO>(acc[r]);
+            s.wo.dots_plain(sm.attn, lane, v);
             wave_sum_n<GE::ROW>(v);
             float mine = 0.f;
 #pragma unroll
@@ -600,11 +722,8 @@ __device__ __forceinline__ void compute_role(const FusedDecodeArgs &a, Lds<GE> &
         {
             const float tot = ((sm.red[0] + sm.red[1]) + sm.red[2]) + sm.red[3];
             const float inv = 1.0f / sqrtf(tot / (float)GE::HIDDEN + a.eps);
-            float acc[GE::RGW][GE::CH];
-            normed_dots<GE::RGW, GE::CH>(s.wg, sm.hx, sm.nw, inv, lane, acc);
             float v[GE::RGW];
-#pragma unroll
-            for (int r = 0; r < GE::RGW; r++) v[r] = chunk_total<GE::CH>(acc[r]);
+            s.wg.dots_normed(sm.hx, sm.nw, inv, lane, v);
             wave_sum_n<GE::RGW>(v);
             float gte = 0.f, up = 0.f;
 #pragma unroll
@@ -620,11 +739,8 @@ __device__ __forceinline__ void compute_role(const FusedDecodeArgs &a, Lds<GE> &
         wg_barrier();
         load_wg(nx, 0, WG_CUT);
         {
-            float acc[GE::ROW][GE::CD];
-            plain_dots<GE::ROW, GE::CD>(s.wd, sm.act, lane, acc);
             float v[GE::ROW];
-#pragma unroll
-            for (int r = 0; r < GE::ROW; r++) v[r] = chunk_total<GE::CD>(acc[r]);
+            s.wd.dots_plain(sm.act, lane, v);
             wave_sum_n<GE::ROW>(v);
             float mine = 0.f;
 #pragma unroll
@@ -999,7 +1115,7 @@ __device__ __forceinline__ void comm_role(const FusedDecodeArgs &a, Lds<GE> &sm,
     if (trace) *trace++ = die_ok ? 1ull : 0ull;
 }
 
-template <class GE>
+template <class GE, int WF>
 __global__ __launch_bounds__(FT) void decode_fused_kernel(FusedDecodeArgs a) {
     __shared__ Lds<GE> sm;
     const int lane = threadIdx.x & (WAVE - 1);
@@ -1015,16 +1131,18 @@ __global__ __launch_bounds__(FT) void decode_fused_kernel(FusedDecodeArgs a) {
         __syncthreads();
     }
     if (wave < NCW) {
-        compute_role<GE>(a, sm, wg, wave, lane, pos);
+        compute_role<GE, WF>(a, sm, wg, wave, lane, pos);
     } else {
         const uint32_t launches = __hip_atomic_load(a.ctl, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         comm_role<GE>(a, sm, wg, wave - NCW, lane, pos, launches);
     }
 }
 
-// Qwen3-0.6B and a small shape of the same family for tests
+// Kernel instances: Qwen3-0.6B in the three weight formats, a small shape of the same family for tests
+// (bf16), and a small shape whose widths are multiples of 1024 for the quantised formats.
 using GeoQwen3_0p6b = Geo<1024, 16, 8, 128, 3072, 256>;
 using GeoSmall = Geo<512, 4, 2, 128, 1024, 64>;
+using GeoSmallQ = Geo<1024, 8, 4, 128, 1024, 64>;
 
 template <class GE>
 bool shape_is(const FusedShape &s) {
@@ -1032,33 +1150,39 @@ bool shape_is(const FusedShape &s) {
            s.inter == GE::INTER;
 }
 
-template <class GE>
-bool fits_device(const hm_ctx *ctx, const char **why) {
-    if (ctx->num_cus < GE::NWG) {
-        *why = "fewer compute units than resident workgroups";
-        return false;
-    }
-    int per_cu = 0;
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, decode_fused_kernel<GE>, FT, 0) != hipSuccess || per_cu < 1) {
-        (void)hipGetLastError();
-        *why = "the kernel does not fit a compute unit";
-        return false;
-    }
-    return true;
+struct Instance {
+    bool (*matches)(const FusedShape &);
+    int wf, max_kv, nwg;
+    size_t xch_bytes;
+    const void *kernel;
+};
+
+template <class GE, int WF>
+Instance instance() {
+    return Instance{&shape_is<GE>, WF, GE::MAX_KV, GE::NWG, (size_t)GE::ALL_SLOTS * 8,
+                    reinterpret_cast<const void *>(&decode_fused_kernel<GE, WF>)};
+}
+
+const Instance *find_instance(const FusedShape &s) {
+    static const Instance table[] = {
+        instance<GeoQwen3_0p6b, FUSED_WF_BF16>(), instance<GeoQwen3_0p6b, FUSED_WF_Q8_0>(), instance<GeoQwen3_0p6b, FUSED_WF_Q4_0>(),
+        instance<GeoSmall, FUSED_WF_BF16>(),      instance<GeoSmallQ, FUSED_WF_Q8_0>(),     instance<GeoSmallQ, FUSED_WF_Q4_0>(),
+    };
+    for (const Instance &i : table)
+        if (i.wf == s.wf && i.matches(s)) return &i;
+    return nullptr;
 }
 
 }  // namespace
 
 int decode_fused_max_kv(const FusedShape &s) {
-    if (shape_is<GeoQwen3_0p6b>(s)) return GeoQwen3_0p6b::MAX_KV;
-    if (shape_is<GeoSmall>(s)) return GeoSmall::MAX_KV;
-    return 0;
+    const Instance *i = find_instance(s);
+    return i ? i->max_kv : 0;
 }
 
 size_t decode_fused_xch_bytes(const FusedShape &s) {
-    if (shape_is<GeoQwen3_0p6b>(s)) return (size_t)GeoQwen3_0p6b::ALL_SLOTS * 8;
-    if (shape_is<GeoSmall>(s)) return (size_t)GeoSmall::ALL_SLOTS * 8;
-    return 0;
+    const Instance *i = find_instance(s);
+    return i ? i->xch_bytes : 0;
 }
 
 bool decode_fused_supported(const hm_ctx *ctx, const FusedShape &s, int n_layers, int max_seq_len, const char **why) {
@@ -1070,31 +1194,38 @@ bool decode_fused_supported(const hm_ctx *ctx, const FusedShape &s, int n_layers
         *why = "layer count outside 1..64";
         return false;
     }
-    const int max_kv = decode_fused_max_kv(s);
-    if (!max_kv) {
-        *why = "no kernel instance for this shape";
+    const Instance *i = find_instance(s);
+    if (!i) {
+        *why = "no kernel instance for this shape and weight format";
         return false;
     }
-    if (max_seq_len > max_kv) {
+    if (max_seq_len > i->max_kv) {
         *why = "cache longer than the attention phase keeps in registers";
         return false;
     }
-    if (shape_is<GeoQwen3_0p6b>(s)) return fits_device<GeoQwen3_0p6b>(ctx, why);
-    return fits_device<GeoSmall>(ctx, why);
+    if (ctx->num_cus < i->nwg) {
+        *why = "fewer compute units than resident workgroups";
+        return false;
+    }
+    int per_cu = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, i->kernel, FT, 0) != hipSuccess || per_cu < 1) {
+        (void)hipGetLastError();
+        *why = "the kernel does not fit a compute unit";
+        return false;
+    }
+    return true;
 }
 
 int decode_fused_launch(hm_ctx *ctx, const FusedShape &s, const FusedDecodeArgs &a) {
     HM_REQUIRE(ctx, a.layers && a.embed && a.state && a.forced && a.hidden_out && a.cos_tab && a.sin_tab && a.xch && a.ctl,
                "decode_fused: NULL pointer");
-    HM_REQUIRE(ctx, a.n_layers >= 1 && a.n_layers <= MAX_LAYERS && a.max_len >= 1 && a.max_len <= decode_fused_max_kv(s),
+    const Instance *i = find_instance(s);
+    if (!i) return hm_set_error(ctx, HM_ERR_INVALID, "decode_fused: no kernel instance for this shape and weight format");
+    HM_REQUIRE(ctx, a.n_layers >= 1 && a.n_layers <= MAX_LAYERS && a.max_len >= 1 && a.max_len <= i->max_kv,
                "decode_fused: %d layers / %d cache rows not served for this shape", a.n_layers, a.max_len);
-    if (shape_is<GeoQwen3_0p6b>(s))
-        hipLaunchKernelGGL(decode_fused_kernel<GeoQwen3_0p6b>, dim3(GeoQwen3_0p6b::NWG), dim3(FT), 0, ctx->stream, a);
-    else if (shape_is<GeoSmall>(s))
-        hipLaunchKernelGGL(decode_fused_kernel<GeoSmall>, dim3(GeoSmall::NWG), dim3(FT), 0, ctx->stream, a);
-    else
-        return hm_set_error(ctx, HM_ERR_INVALID, "decode_fused: no kernel instance for this shape");
-    HM_LAUNCH_CHECK(ctx);
+    FusedDecodeArgs args = a;
+    void *params[] = {&args};
+    HM_HIP(ctx, hipLaunchKernel(i->kernel, dim3(i->nwg), dim3(FT), params, 0, ctx->stream));
     return HM_OK;
 }
 

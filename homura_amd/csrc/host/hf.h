@@ -146,6 +146,7 @@ class HfModel {
     bool has_qk_norm_ = false;
     bool finalized_ = false;
     bool fused_available_ = false;
+    int fused_wf_ = 0;  // FUSED_WF_* of the whole-step kernel instance
     const void *fused_table_kv_ = nullptr;  // key_ptr(0) the device layer table was built for
     int fused_table_max_len_ = 0;
     int max_seq_len_ = 0;

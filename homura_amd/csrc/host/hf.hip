@@ -401,11 +401,25 @@ int HfModel::finalize(int max_seq_len) {
     s.cand_idx = Buffer::alloc(ctx_, {s.cand_cap}, DType::F32);
     if (!s.attn_flat || !s.resid || !s.act || !s.cand_val || !s.cand_idx) return HM_ERR_OOM;
 
-    // The whole-step decode launch serves bf16 models of a shape it has an instance for.
+    if (dtype_is_quantized(weight_dtype_) && (rc = build_quant_planes()) != HM_OK) return rc;
+
+    // The whole-step decode launch serves bf16 models, and models whose projections are all Q8_0 or all
+    // Q4_0 (re-packed into planes), of a shape it has an instance for.
     fused_available_ = false;
-    if (weight_dtype_ == DType::BF16) {
+    fused_wf_ = FUSED_WF_BF16;
+    bool fused_format = weight_dtype_ == DType::BF16;
+    if (dtype_is_quantized(weight_dtype_)) {
+        const DType t = proj_dtype(0, 0);
+        fused_format = t == DType::Q8_0 || t == DType::Q4_0;
+        for (int l = 0; l < cfg_.num_hidden_layers && fused_format; l++) {
+            for (int j = 0; j < 7; j++) fused_format = fused_format && proj_dtype(l, j) == t;
+            fused_format = fused_format && packed_[l].planes[0] && packed_[l].planes[3] && packed_[l].planes[4] && packed_[l].planes[6];
+        }
+        fused_wf_ = t == DType::Q4_0 ? FUSED_WF_Q4_0 : FUSED_WF_Q8_0;
+    }
+    if (fused_format) {
         const FusedShape fs{cfg_.hidden_size, cfg_.num_attention_heads, cfg_.kv_heads(), cfg_.head_dim(),
-                            cfg_.intermediate_size};
+                            cfg_.intermediate_size, fused_wf_};
         if (decode_fused_supported(ctx_, fs, cfg_.num_hidden_layers, max_seq_len, nullptr)) {
             s.fused_layers = Buffer::alloc_bytes(ctx_, sizeof(FusedLayerPtrs) * (size_t)cfg_.num_hidden_layers,
                                                  {cfg_.num_hidden_layers}, DType::I64);
@@ -419,7 +433,6 @@ int HfModel::finalize(int max_seq_len) {
         }
     }
 
-    if (dtype_is_quantized(weight_dtype_) && (rc = build_quant_planes()) != HM_OK) return rc;
     rc = dtype_is_quantized(weight_dtype_) ? emit_transformer_plan_quant() : emit_transformer_plan();
     if (rc != HM_OK) return rc;
     rc = plan_->prepare(std::max(max_seq_len, 16));
@@ -1073,9 +1086,50 @@ int HfModel::emit_transformer_plan_quant() {
                                      sc.pool[sc.step.input_slots[1]]->as<float>(),
                                      sc.pool[sc.step.output_slots[0]]->as<float>(), (int)vocab, (int)hidden);
         };
+        if (fused_available_) l.mode = DeviceLaunch::Mode::PerKernel;
         k.launches.push_back(std::move(l));
+        if (fused_available_) {
+            // One launch for the embedding row and every layer (decode_fused.hip, reading the re-packed
+            // planes); the layer kernels below then enqueue nothing, and the last hidden state lands in the
+            // last layer's output slot.
+            DeviceLaunch f;
+            f.name = "decode_whole_step[embed+layers]";
+            f.mode = DeviceLaunch::Mode::WholeStep;
+            double layer_w = 0;
+            {
+                const int64_t kd[7] = {hidden, hidden, hidden, qd, hidden, hidden, inter};
+                const int64_t nd[7] = {qd, kvd, kvd, hidden, inter, inter, hidden};
+                for (int j = 0; j < 7; j++) layer_w += (double)dtype_bytes_for_elements(proj_dtype(0, j), (size_t)(kd[j] * nd[j]), nullptr);
+            }
+            f.bytes_fixed = L * (layer_w + 2 * hidden * 4.0 + 2 * kvd * 2.0) + hidden * 4.0 * 2;
+            f.bytes_per_kv_row = L * 2.0 * kvh * hd * 2;
+            const FusedShape fshape{(int)hidden, (int)H, (int)kvh, (int)hd, (int)inter, fused_wf_};
+            const size_t hidden_out_slot = ls[L - 1].hidden_out;
+            const size_t cos_slot = cos_s, sin_slot = sin_s;
+            f.fn = [=](const StepContext &sc) -> int {
+                FusedDecodeArgs fa{};
+                fa.layers = reinterpret_cast<const FusedLayerPtrs *>(scr->fused_layers.ptr());
+                fa.n_layers = (int)L;
+                fa.embed = sc.pool[sc.step.input_slots[1]]->as<float>();
+                fa.vocab = (int)vocab;
+                fa.state = sc.plan->state();
+                fa.forced = sc.plan->forced_ids();
+                fa.hidden_out = sc.pool[hidden_out_slot]->as<float>();
+                fa.cos_tab = sc.pool[cos_slot]->as<float>();
+                fa.sin_tab = sc.pool[sin_slot]->as<float>();
+                fa.eps = eps;
+                fa.scale = (float)(1.0 / std::sqrt((double)hd));
+                fa.max_len = sc.plan->kv_cache()->max_len();
+                fa.xch = scr->fused_xch.as<unsigned char>();
+                fa.ctl = scr->fused_ctl.as<uint32_t>();
+                fa.trace = scr->fused_trace ? scr->fused_trace.as<unsigned long long>() : nullptr;
+                return decode_fused_launch(sc.ctx, fshape, fa);
+            };
+            k.launches.push_back(std::move(f));
+        }
         add_step(std::move(k), {input_ids, embed_w}, {embed_out});
     }
+    const size_t first_layer_kernel = kernels.size();
     for (int i = 0; i < L; i++) {
         const LS &s = ls[i];
         // Which light steps ride along with a Q8_0 / Q4_0 product instead of being launched (the step
@@ -1262,6 +1316,9 @@ int HfModel::emit_transformer_plan_quant() {
             add_step(std::move(k), {s.residual, s.down_out}, {s.hidden_out});
         }
     }
+    if (fused_available_)  // in whole-step mode the layers' own launches stay out
+        for (size_t ki = first_layer_kernel; ki < kernels.size(); ki++)
+            for (DeviceLaunch &dl : kernels[ki].launches) dl.mode = DeviceLaunch::Mode::PerKernel;
     {  // LM head: final RMSNorm + f32 matmul (reference :1399-1440) + device-side greedy pick
         CompiledKernel k;
         k.ops_label = "LMHead";
@@ -1363,10 +1420,28 @@ int HfModel::refresh_fused_table() {
     for (int l = 0; l < L; l++) {
         const std::string p = "model.layers." + std::to_string(l) + ".";
         FusedLayerPtrs &f = t[l];
-        f.wqkv = packed_[l].qkv.as<uint16_t>();
-        f.wo = packed_[l].o.as<uint16_t>();
-        f.wgu = packed_[l].gate_up.as<uint16_t>();
-        f.wd = packed_[l].down.as<uint16_t>();
+        if (fused_wf_ == FUSED_WF_BF16) {
+            f.wqkv = packed_[l].qkv.ptr();
+            f.wo = packed_[l].o.ptr();
+            f.wgu = packed_[l].gate_up.ptr();
+            f.wd = packed_[l].down.ptr();
+            f.sqkv = f.so = f.sgu = f.sd = nullptr;
+        } else {  // quant planes of the four runs, scales behind the quants
+            const bool q4 = fused_wf_ == FUSED_WF_Q4_0;
+            const int hidden = cfg_.hidden_size, inter = cfg_.intermediate_size, qd = cfg_.q_dim(), kvd = cfg_.kv_dim();
+            auto scales = [&](const Buffer &b, int n, int k) {
+                return reinterpret_cast<const uint16_t *>(b.as<uint8_t>() + quant_planes_scale_offset(q4, n, k));
+            };
+            const LayerPacked &lp = packed_[l];
+            f.wqkv = lp.planes[0].ptr();
+            f.sqkv = scales(lp.planes[0], qd + 2 * kvd, hidden);
+            f.wo = lp.planes[3].ptr();
+            f.so = scales(lp.planes[3], hidden, qd);
+            f.wgu = lp.planes[4].ptr();
+            f.sgu = scales(lp.planes[4], 2 * inter, hidden);
+            f.wd = lp.planes[6].ptr();
+            f.sd = scales(lp.planes[6], hidden, inter);
+        }
         f.in_ln = weight_f32(p + "input_layernorm.weight");
         f.post_ln = weight_f32(p + "post_attention_layernorm.weight");
         f.q_norm = has_qk_norm_ ? weight_f32(p + "self_attn.q_norm.weight") : nullptr;

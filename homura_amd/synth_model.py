@@ -30,6 +30,12 @@ SMALL_WS = TransformerConfig(
     vocab_size=1000, num_key_value_heads=2, head_dim=128, rms_norm_eps=1e-6, rope_theta=1e6,
     max_position_embeddings=2048, tie_word_embeddings=True)
 
+# the small shape the whole-step decode launch serves in Q8_0 / Q4_0 (widths that are multiples of 1024)
+SMALL_WS_Q = TransformerConfig(
+    hidden_size=1024, intermediate_size=1024, num_attention_heads=8, num_hidden_layers=3,
+    vocab_size=1000, num_key_value_heads=4, head_dim=128, rms_norm_eps=1e-6, rope_theta=1e6,
+    max_position_embeddings=1024, tie_word_embeddings=False)
+
 # Qwen2.5-like: Q/K/V biases, no QK-norm, GQA 7:1 as in Qwen2.5-0.5B (14 q heads, 2 kv heads)
 TINY_QWEN2 = TransformerConfig(
     hidden_size=448, intermediate_size=608, num_attention_heads=7, num_hidden_layers=2,
