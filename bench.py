@@ -9,7 +9,8 @@ A "step" is one decode token: embed -> 28 x (QKV+QK-norm+RoPE+append, attention+
     python bench.py --gpus 1 --steps 64 --warmup 8
 
 Prints one JSON line. `roofline` describes the device kernel with the largest share of a step
-(its per-layer launches are timed back to back with HIP events on the launch stream);
+(timed with HIP events on the launch stream; `traffic` comes from the committed rocprofv3 --pmc table
+under profiles/, flagged `traffic_stale` when the kernel sources have changed since);
 `cpu_baseline` is the CPU oracle (a port of the reference's CPU kernels) timed on this host.
 """
 from __future__ import annotations
@@ -38,18 +39,34 @@ KERNEL_FAMILY = {
     "gqa_attn_fold": "gqa_decode_fold_kernel",
 }
 
-# HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE x 1.9985 + WRITE_SIZE x 1.0,
-# the factors a 32 MiB + 32 MiB copy kernel calibrates), per kernel of the table below; the
-# counter runs are separate from this program and summarised under profiles/.
-PMC_TRAFFIC_BYTES = {
-    "gemv_bf16[qkv]": 8532770,
-    "gemv_bf16[o]": 4332364,
-    "gemv_bf16[gate_up+silu]": 12767935,
-    "gemv_bf16[down+residual]": 6526184,
-    "gemv_bf16[lm_head+argmax]": 311889597,
-    "qknorm_rope_append+gqa_attn": 4607533,
-    "gqa_attn_fold": 260930,
-}
+TRAFFIC_TABLE = ROOT / "profiles" / "hbm_traffic_decode_and_kernel_cases_pmc.md"
+
+
+def kernel_sources_hash() -> str:
+    """sha256/16 over the kernel sources (names and contents), the stamp the traffic table carries."""
+    import hashlib
+    h = hashlib.sha256()
+    csrc = ROOT / "homura_amd" / "csrc"
+    for f in sorted(list(csrc.glob("*.hip")) + list(csrc.glob("*.h")), key=lambda p: str(p)):
+        h.update(f.name.encode())
+        h.update(f.read_bytes())
+    return h.hexdigest()[:16]
+
+
+def measured_traffic():
+    """HBM bytes per launch by bench.py kernel label, from the committed rocprofv3 --pmc summary
+    (FETCH_SIZE and WRITE_SIZE scaled by a copy kernel of known size; the counter runs are separate from
+    this program). Returns (table, stale): stale when the kernel sources changed since the table was made."""
+    table, stamp = {}, None
+    if not TRAFFIC_TABLE.exists():
+        return table, True
+    for line in TRAFFIC_TABLE.read_text().splitlines():
+        if line.startswith("kernel sources sha256/16:"):
+            stamp = line.split(":", 1)[1].strip()
+        cells = [c.strip() for c in line.split("|")]
+        if len(cells) > 9 and cells[2].startswith("`") and cells[8].isdigit():
+            table[cells[2].strip("`")] = int(cells[8])
+    return table, stamp != kernel_sources_hash()
 
 
 def algorithmic_bytes_per_token(cfg, kv_rows: float) -> float:
@@ -135,6 +152,7 @@ def main() -> int:
                 "GBps": round(per_launch_bytes / (us * 1e-6) / 1e9, 1),
                 "step_share_us": round(us * (r["launches"] // args.kernel_rounds), 2),
             })
+        PMC_TRAFFIC_BYTES, traffic_stale = measured_traffic()
         fams = {}
         for k in kernels:
             f = fams.setdefault(KERNEL_FAMILY.get(k["kernel"], k["kernel"]),
@@ -155,6 +173,7 @@ def main() -> int:
             "bytes_per_launch": int(dom["bytes"] / dom["launches"]),
             "launches_per_step": dom["launches"], "step_share_us": round(dom["us"], 1),
             "traffic": None if dom["traffic"] is None else int(dom["traffic"] / dom["launches"]),
+            "traffic_stale": traffic_stale,
             "whole_step": {"bytes_per_token": int(bytes_tok), "achieved": round(step_gbs, 1),
                            "frac": round(step_gbs / HBM_PEAK_GBS, 4)},
         }
