@@ -47,8 +47,23 @@ __device__ __forceinline__ float dot4_bytes(uint32_t w, const float *xv, float s
     return s;
 }
 
+// A masked dword of nibbles (each byte 0..15) as four floats, two conversions instead of four: read as
+// OCP FP8 E4M3 a byte 0000nnnn is n * 2^-9 whether n falls in the subnormal range (n < 8: 2^-6 * n / 8) or in
+// the first binade (n >= 8: 2^-6 * (1 + (n - 8) / 8)), and v_cvt_pk_f32_fp8 converts two bytes at a time,
+// exactly. The activations carry the factor 2^9 (exact as well), so the products are those of n.
+constexpr float NIBBLE_FP8_UNIT = 512.0f;
+__device__ __forceinline__ float dot4_nibbles(uint32_t w, const float *xs512, float s) {
+    const auto lo = __builtin_amdgcn_cvt_pk_f32_fp8((int)w, false);
+    const auto hi = __builtin_amdgcn_cvt_pk_f32_fp8((int)w, true);
+    s = fmaf(lo[0], xs512[0], s);
+    s = fmaf(lo[1], xs512[1], s);
+    s = fmaf(hi[0], xs512[2], s);
+    s = fmaf(hi[1], xs512[3], s);
+    return s;
+}
+
 // Activations of quarter column c (block c / 4, quarter c % 4) in the order the quant bytes use them,
-// and offset * their sum.
+// and offset * their sum. Q4_0: the activations come back multiplied by 2^9 for dot4_nibbles.
 template <int QT>
 __device__ __forceinline__ void load_xv(const float *xs, int c, float *xv, float &sx_off) {
     const int b = c >> 2, q = c & 3;
@@ -62,6 +77,10 @@ __device__ __forceinline__ void load_xv(const float *xs, int c, float *xv, float
 #pragma unroll
     for (int j = 0; j < 8; j++) sx += xv[j];
     sx_off = sx * (QT == 0 ? 128.f : 8.f);
+    if (QT == 1) {
+#pragma unroll
+        for (int j = 0; j < 8; j++) xv[j] *= NIBBLE_FP8_UNIT;
+    }
 }
 
 // The quant words of one quarter: Q8_0 two dwords, Q4_0 one.
@@ -96,7 +115,7 @@ __device__ __forceinline__ float quarter_value(const QWords<QT> &w, uint32_t sca
         s = dot4_bytes(w.w1 ^ 0x80808080u, xv + 4, dot4_bytes(w.w0 ^ 0x80808080u, xv, 0.f));  // int8 -> biased unsigned
     } else {
         // byte i of the word: low nibble = weight 4q + i, high nibble = weight 16 + 4q + i
-        s = dot4_bytes((w.w0 >> 4) & 0x0F0F0F0Fu, xv + 4, dot4_bytes(w.w0 & 0x0F0F0F0Fu, xv, 0.f));
+        s = dot4_nibbles((w.w0 >> 4) & 0x0F0F0F0Fu, xv + 4, dot4_nibbles(w.w0 & 0x0F0F0F0Fu, xv, 0.f));
     }
     return d * (s - sx_off);
 }
@@ -121,12 +140,15 @@ __global__ __launch_bounds__(PTHREADS) void gemv_planes_kernel(const float *__re
     const int ntrips = (N + RB - 1) / RB;
     QWords<QT> qn[RB][CPL];
     uint32_t sn[RB][CPL];
+    uint32_t qoff[CPL], soff[CPL];  // byte offsets of the lane's quarters / element offsets of their scales in a row
     int col[CPL];
     bool live[CPL];
 #pragma unroll
     for (int t = 0; t < CPL; t++) {
         live[t] = lane + t * WAVE < nq;
-        col[t] = live[t] ? lane + t * WAVE : nq - 1;  // lanes past the row end re-read its last column
+        col[t] = live[t] ? lane + t * WAVE : nq - 1;  // lanes past the row end re-read its last column ...
+        qoff[t] = (uint32_t)col[t] * QB;
+        soff[t] = (uint32_t)col[t] >> 2;
     }
     auto request = [&](int trip) {
 #pragma unroll
@@ -136,8 +158,8 @@ __global__ __launch_bounds__(PTHREADS) void gemv_planes_kernel(const float *__re
             const uint16_t *sr = scales + (size_t)row * nb;
 #pragma unroll
             for (int t = 0; t < CPL; t++) {
-                qn[r][t] = load_quarter<QT>(qr + (size_t)col[t] * QB);
-                sn[r][t] = __builtin_nontemporal_load((global_u16_ptr)(sr + (col[t] >> 2)));
+                qn[r][t] = load_quarter<QT>(qr + qoff[t]);
+                sn[r][t] = __builtin_nontemporal_load((global_u16_ptr)(sr + soff[t]));
             }
         }
     };
@@ -209,7 +231,14 @@ __global__ __launch_bounds__(PTHREADS) void gemv_planes_kernel(const float *__re
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
     float xv[CPL][8], sxo[CPL];
 #pragma unroll
-    for (int t = 0; t < CPL; t++) load_xv<QT>(xs, col[t], xv[t], sxo[t]);
+    for (int t = 0; t < CPL; t++) {
+        load_xv<QT>(xs, col[t], xv[t], sxo[t]);
+        if (!live[t]) {  // ... against activations of zero, so they add nothing
+#pragma unroll
+            for (int j = 0; j < 8; j++) xv[t][j] = 0.f;
+            sxo[t] = 0.f;
+        }
+    }
 
     float best_v = -INFINITY;
     int best_i = -1;
@@ -231,8 +260,7 @@ __global__ __launch_bounds__(PTHREADS) void gemv_planes_kernel(const float *__re
         for (int t = 0; t < CPL; t++)
 #pragma unroll
             for (int r = 0; r < RB; r++) {
-                const float v = quarter_value<QT>(qc[r][t], sc[r][t], xv[t], sxo[t]);
-                a[r] += live[t] ? v : 0.f;
+                a[r] += quarter_value<QT>(qc[r][t], sc[r][t], xv[t], sxo[t]);
             }
         // wave sums of the RB rows, the chains stepping side by side
 #pragma unroll
