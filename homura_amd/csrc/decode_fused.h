@@ -38,6 +38,17 @@ struct FusedDecodeArgs {
     int max_len;         // rows per KV head in the caches
     unsigned char *xch;  // exchange area, decode_fused_xch_bytes() bytes, zeroed once
     uint32_t *ctl;       // [0] launches so far (tag base), [1] sticky status (0 = ok), zeroed once
+    // Optional LM head and greedy pick inside the same launch (head_w == nullptr: the launch ends with
+    // hidden_out, as the layers' last output). head_w: bf16 [vocab][hidden] in the stream layout; head_norm: the
+    // final RMSNorm weights; logits: [vocab] f32. With advance set, workgroup 0 finishes the step as
+    // finish_step does: out_tokens[step] = pick (while step < out_cap), state->token = pick, step and pos + 1.
+    const uint16_t *head_w;
+    const float *head_norm;
+    float *logits;
+    DecodeState *state_rw;
+    int32_t *out_tokens;
+    int out_cap;
+    int advance;
     // Optional phase trace (nullptr = off; room for FUSED_TRACE_WGS workgroups x (11 n_layers + 2) entries):
     // every workgroup stores, in its own row, the 100 MHz device clock at 11 points per
     // layer - both barriers of the Q|K|V, attention, O, gate|up and down phases, and the end of the fold

@@ -67,7 +67,9 @@ struct Geo {
     static constexpr int RELAY0 = GLOB_SLOTS, LQ0 = RELAY0 + NXCD * GLOB_SLOTS, LP0 = LQ0 + KVH * GROWS;
     static constexpr int PAR_SLOTS = (LP0 + KVH * SPH * PART + 31) / 32 * 32;
     static constexpr int CHK0 = 2 * PAR_SLOTS;                 // placement check: one slot per workgroup
-    static constexpr int ALL_SLOTS = CHK0 + NWG;
+    static constexpr int CAND0 = CHK0 + NWG;                   // LM head: one {value, index} unit per workgroup
+    static constexpr int ALL_SLOTS = CAND0 + 2 * NWG;
+    static constexpr int HR = 8;                               // LM-head rows a wavefront multiplies per batch
     static constexpr int PUB = (PART > RQ ? PART : RQ) > RG ? (PART > RQ ? PART : RQ) : RG;
     static_assert(HIDDEN % 512 == 0 && QD % 512 == 0 && INTER % 512 == 0, "rows are cut into 512-wide chunks");
     static_assert(NQKV % (NWG * NCW) == 0 && HIDDEN % (NWG * NCW) == 0 && (2 * INTER) % (NWG * NCW) == 0,
@@ -82,6 +84,7 @@ struct Geo {
                       INTER / 2 / NPX <= WAVE && QD / 2 / NPX <= WAVE && HIDDEN / 2 / NPX <= WAVE,
                   "one wavefront relays a die's share of a vector");
     static_assert(NWG % 2 == 0 && NWG / 2 <= 2 * WAVE, "two placement-check units per lane");
+    static_assert(NWG % WAVE == 0 && NWG / WAVE <= 8, "workgroup 0 gathers the LM-head candidates with one wavefront");
     // row of the stacked q|k|v matrix for local row lr of KV head kh
     __device__ static int qkv_row(int kh, int lr) {
         return lr < G * HD ? kh * G * HD + lr : (lr < (G + 1) * HD ? QD + kh * HD + (lr - G * HD) : QD + KVD + kh * HD + (lr - (G + 1) * HD));
@@ -101,6 +104,8 @@ struct Lds {
     float wstat[NCW][GE::G][2];
     float pub[GE::PUB];                   // results of the phase, read by the publishing threads
     float red[4];
+    float head_v[NCW + 4];                // LM head: every wavefront's best row
+    int head_i[NCW + 4];
     float bias[GE::RQ];
     FusedLayerPtrs lp[MAX_LAYERS];        // the layer table (compute wavefronts must not wait on global loads)
 };
@@ -499,6 +504,74 @@ struct Split {
     }
 };
 
+// LM head (reference src/hf/emitter.rs:828-862) and the wavefront's best row. The workgroup owns a contiguous
+// run of the vocabulary; all eight wavefronts (the communicating ones have nothing else left to do) take
+// batches of HR rows in turn, the next batch's rows in flight while this one is multiplied. EARLY: the
+// caller has not yet passed the barrier behind which the last hidden state is staged, and the first batch is
+// requested before it. Ends behind the barrier after which head_v / head_i hold every wavefront's best row.
+constexpr int HEAD_WORKERS = NCW + 4;
+template <class GE, bool EARLY>
+__device__ __forceinline__ void head_rows(const FusedDecodeArgs &a, Lds<GE> &sm, const int wg, const int worker, const int lane) {
+    constexpr int HR = GE::HR, HC = GE::HIDDEN / 512;
+    const int per_wg = (a.vocab + GE::NWG - 1) / GE::NWG;
+    const int row0 = wg * per_wg, row1 = min(a.vocab, row0 + per_wg);
+    const int nbatch = (max(row1 - row0, 0) + HEAD_WORKERS * HR - 1) / (HEAD_WORKERS * HR);  // batches of this wavefront
+    u32x4 wn[HR][HC];
+    auto request = [&](int b) {
+#pragma unroll
+        for (int r = 0; r < HR; r++) {
+            const int row = min(row0 + (b * HEAD_WORKERS + worker) * HR + r, a.vocab - 1);  // rows past the end re-read the last one
+#pragma unroll
+            for (int c = 0; c < HC; c++) wn[r][c] = ld128_global_stream(a.head_w + (size_t)row * GE::HIDDEN + (c * WAVE + lane) * 8);
+        }
+    };
+    if (nbatch > 0) request(0);
+    if (EARLY) wg_barrier();
+    const float tot = ((sm.red[0] + sm.red[1]) + sm.red[2]) + sm.red[3];
+    const float inv = 1.0f / sqrtf(tot / (float)GE::HIDDEN + a.eps);
+    float xv[HC][8];
+#pragma unroll
+    for (int c = 0; c < HC; c++) {
+        float hv[8], wv[8];
+        lds_x8(sm.hx, (c * WAVE + lane) * 8, hv);
+        lds_x8(sm.nw, (c * WAVE + lane) * 8, wv);
+#pragma unroll
+        for (int e = 0; e < 8; e++) xv[c][e] = (hv[e] * inv) * wv[e];
+    }
+    float best_v = -INFINITY;
+    int best_i = -1;
+    for (int b = 0; b < nbatch; b++) {
+        u32x4 wc[HR][HC];
+#pragma unroll
+        for (int r = 0; r < HR; r++)
+#pragma unroll
+            for (int c = 0; c < HC; c++) wc[r][c] = wn[r][c];
+        if (b + 1 < nbatch) request(b + 1);
+        float acc[HR][HC], v[HR];
+        dots_from<HR, HC>(wc, xv, acc);
+#pragma unroll
+        for (int r = 0; r < HR; r++) v[r] = chunk_total<HC>(acc[r]);
+        wave_sum_n<HR>(v);
+        const int first = row0 + (b * HEAD_WORKERS + worker) * HR;
+        float mine = 0.f;
+#pragma unroll
+        for (int r = 0; r < HR; r++) {
+            mine = lane == r ? v[r] : mine;
+            // of equal maxima the later row wins (Rust Iterator::max_by, reference src/generate.rs:735-742)
+            if (first + r < row1 && (best_i < 0 || v[r] >= best_v)) {
+                best_v = v[r];
+                best_i = first + r;
+            }
+        }
+        if (lane < HR && first + lane < row1) a.logits[first + lane] = mine;
+    }
+    if (lane == 0) {
+        sm.head_v[worker] = best_v;
+        sm.head_i[worker] = best_i;
+    }
+    wg_barrier();
+}
+
 // Registers of one compute wavefront that hold its slice of a layer.
 template <class GE, int WF>
 struct Slice {
@@ -749,6 +822,8 @@ __device__ __forceinline__ void compute_role(const FusedDecodeArgs &a, Lds<GE> &
         }
         wg_barrier();
     }
+
+    if (a.head_w) head_rows<GE, true>(a, sm, wg, cw, lane);
 }
 
 // Slot of hidden element k in the XH / XO areas: the communicating thread c = k % 256 owns elements
@@ -920,6 +995,9 @@ __device__ __forceinline__ void comm_role(const FusedDecodeArgs &a, Lds<GE> &sm,
     load_in_ln(sm.lp[0]);
     load_post_ln(sm.lp[0]);
     load_qk_norm(sm.lp[0]);
+    float nw_head[NJ];  // the final norm's weights, for the LM head
+#pragma unroll
+    for (int j = 0; j < NJ; j++) nw_head[j] = a.head_w ? ldf_global(a.head_norm + ct + CT * j) : 0.f;
 
     for (int l = 0; l < L; l++) {
         const FusedLayerPtrs cur = sm.lp[l];
@@ -1089,8 +1167,72 @@ __device__ __forceinline__ void comm_role(const FusedDecodeArgs &a, Lds<GE> &sm,
         if (ct < GE::RO) st_slot(xc, GE::XH + hidden_slot(wg * GE::RO + ct), sm.pub[ct], tag, false);
     }
 
-    // hidden += down rows of the last layer: the LM head's input
-    if (wg == 0) {
+    if (a.head_w) {
+        // ── into the LM head: hidden += down rows of the last layer, under the final RMSNorm ──
+        const uint32_t gl = base + (uint32_t)(L - 1);
+        unsigned char *xl = a.xch + (size_t)(gl & 1u) * par_bytes;
+        ps.where = 7u | (uint32_t)(L - 1) << 4 | (uint32_t)wg << 12;
+        stage_hidden(xl, GE::XH, gl + 1u, true, nw_head);
+        if (wg == 0) {
+#pragma unroll
+            for (int j = 0; j < NJ; j++) a.hidden_out[ct + CT * j] = h[j];
+        }
+        wg_barrier();
+        head_rows<GE, false>(a, sm, wg, NCW + cwv, lane);
+        // this workgroup's best row, then (workgroup 0) the best of all and the end of the step
+        // (greedy pick of reference src/generate.rs:735-742 taken on the device)
+        unsigned char *cand = a.xch + (size_t)GE::CAND0 * 8;
+        const uint32_t ctag = launches + 1u;
+        if (cwv == 0) {
+            float bv = -INFINITY;
+            int bi = -1;
+            if (lane < HEAD_WORKERS) {
+                bv = sm.head_v[lane];
+                bi = sm.head_i[lane];
+            }
+            const float m = wave_max(bi >= 0 ? bv : -INFINITY);
+            const float sel = wave_max(bi >= 0 && bv == m ? (float)bi : -1.f);  // indices are below 2^24: exact as floats
+            if (lane == 0) {
+                st_slot(cand, 2 * wg, m, ctag, false);
+                st_slot(cand, 2 * wg + 1, __int_as_float((int)sel), ctag, false);
+            }
+            if (wg == 0) {
+                constexpr int NU = GE::NWG / WAVE;
+                int unit[NU];
+                bool on[NU];
+                u32x4 w[NU];
+#pragma unroll
+                for (int u = 0; u < NU; u++) {
+                    unit[u] = u * WAVE + lane;
+                    on[u] = true;
+                }
+                poll_units<NU>(ps, cand, unit, on, ctag, w);
+                float gv = -INFINITY;
+                int gi = -1;
+#pragma unroll
+                for (int u = 0; u < NU; u++) {
+                    const float v = __uint_as_float(w[u].x);
+                    const int i = (int)w[u].z;
+                    if (i >= 0 && (gi < 0 || v > gv || (v == gv && i > gi))) {
+                        gv = v;
+                        gi = i;
+                    }
+                }
+                const float gm = wave_max(gi >= 0 ? gv : -INFINITY);
+                const float gs = wave_max(gi >= 0 && gv == gm ? (float)gi : -1.f);
+                if (lane == 0 && a.advance && !ps.failed) {
+                    const int tok = gs < 0.f ? 0 : (int)gs;
+                    if (step < a.out_cap) a.out_tokens[step] = tok;
+                    a.state_rw->token = tok;
+                    a.state_rw->step = step + 1;
+                    a.state_rw->pos = pos + 1;
+                }
+                // every workgroup read the launch count before its first exchange
+                if (lane == 0) __hip_atomic_store(a.ctl, launches + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+        }
+    } else if (wg == 0) {
+        // hidden += down rows of the last layer: the LM head's input
         const uint32_t gl = base + (uint32_t)(L - 1);
         const unsigned char *xl = a.xch + (size_t)(gl & 1u) * par_bytes;
         int unit[NJ / 2];
@@ -1221,6 +1363,8 @@ int decode_fused_launch(hm_ctx *ctx, const FusedShape &s, const FusedDecodeArgs 
                "decode_fused: NULL pointer");
     const Instance *i = find_instance(s);
     if (!i) return hm_set_error(ctx, HM_ERR_INVALID, "decode_fused: no kernel instance for this shape and weight format");
+    HM_REQUIRE(ctx, !a.head_w || (a.head_norm && a.logits && a.state_rw && a.out_tokens && i->wf == FUSED_WF_BF16),
+               "decode_fused: the LM head needs its norm weights, a logits row, the cursor and the token list (bf16 instances only)");
     HM_REQUIRE(ctx, a.n_layers >= 1 && a.n_layers <= MAX_LAYERS && a.max_len >= 1 && a.max_len <= i->max_kv,
                "decode_fused: %d layers / %d cache rows not served for this shape", a.n_layers, a.max_len);
     FusedDecodeArgs args = a;

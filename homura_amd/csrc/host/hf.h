@@ -147,6 +147,7 @@ class HfModel {
     bool finalized_ = false;
     bool fused_available_ = false;
     int fused_wf_ = 0;  // FUSED_WF_* of the whole-step kernel instance
+    bool fused_head_ = false;  // the whole-step launch also runs the LM head and the greedy pick (bf16 plan)
     const void *fused_table_kv_ = nullptr;  // key_ptr(0) the device layer table was built for
     int fused_table_max_len_ = 0;
     int max_seq_len_ = 0;

@@ -571,11 +571,16 @@ int HfModel::emit_transformer_plan() {
             // One launch for the embedding row and every layer (decode_fused.hip); the layer kernels below
             // then enqueue nothing, and the last hidden state lands in the last layer's output slot.
             DeviceLaunch f;
-            f.name = "decode_whole_step[embed+layers]";
+            // ... and, unless HOMURA_WHOLE_STEP_HEAD=0, the LM head and the greedy pick as well: the step is one launch
+            bool with_head = true;
+            if (const char *e = std::getenv("HOMURA_WHOLE_STEP_HEAD")) with_head = std::atoi(e) != 0;
+            fused_head_ = with_head;
+            f.name = with_head ? "decode_whole_step[+head+pick]" : "decode_whole_step[embed+layers]";
             f.mode = DeviceLaunch::Mode::WholeStep;
             const double layer_w = (double)hidden * (qd + 2 * kvd) * 2 + (double)qd * hidden * 2 +
                                    (double)hidden * 2 * inter * 2 + (double)inter * hidden * 2;
             f.bytes_fixed = L * (layer_w + 2 * hidden * 4.0 + 2 * kvd * 2.0) + hidden * 4.0 * 2;
+            if (with_head) f.bytes_fixed += gemv_bytes(hidden, vocab, vocab) + hidden * 4.0;
             f.bytes_per_kv_row = L * 2.0 * kvh * hd * 2;
             const FusedShape fs{(int)hidden, (int)H, (int)kvh, (int)hd, (int)inter};
             const size_t hidden_out_slot = ls[L - 1].hidden_out;
@@ -596,6 +601,15 @@ int HfModel::emit_transformer_plan() {
                 fa.xch = scr->fused_xch.as<unsigned char>();
                 fa.ctl = scr->fused_ctl.as<uint32_t>();
                 fa.trace = scr->fused_trace ? scr->fused_trace.as<unsigned long long>() : nullptr;
+                if (with_head) {
+                    fa.head_w = sc.pool[lm_head]->as<uint16_t>();
+                    fa.head_norm = sc.pool[final_norm]->as<float>();
+                    fa.logits = sc.pool[logits]->as<float>();
+                    fa.state_rw = sc.plan->state();
+                    fa.out_tokens = sc.plan->out_tokens();
+                    fa.out_cap = sc.plan->out_capacity();
+                    fa.advance = sc.timing ? 0 : 1;
+                }
                 return decode_fused_launch(sc.ctx, fs, fa);
             };
             k.launches.push_back(std::move(f));
@@ -791,11 +805,13 @@ int HfModel::emit_transformer_plan() {
             g.argmax_cap = scr->cand_cap;
             return gemv_bf16_nk_launch(sc.ctx, g, 1, GEMV_EPI_ARGMAX);
         };
+        if (fused_available_ && fused_head_) h1.mode = DeviceLaunch::Mode::PerKernel;
         k.launches.push_back(std::move(h1));
         DeviceLaunch h2;
         h2.name = "finish_step";
         h2.moves_cursor = true;
         h2.bytes_fixed = 64;
+        if (fused_available_ && fused_head_) h2.mode = DeviceLaunch::Mode::PerKernel;
         h2.fn = [=](const StepContext &sc) -> int {
             const int ncand = std::min(gemv_bf16_nk_grid(sc.ctx, (int)vocab, 4), scr->cand_cap);
             return finish_step_launch(sc.ctx, sc.plan->state(), scr->cand_val.as<float>(),

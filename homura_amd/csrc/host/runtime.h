@@ -145,6 +145,7 @@ struct StepContext {
     ExecutionPlan *plan;
     const std::vector<Buffer *> &pool;  // slot -> buffer (inputs, weights, intermediates)
     const KernelStep &step;
+    bool timing = false;  // launched over and over to be timed: a launch that would end the step must not move the cursor
 };
 // One HIP kernel launch inside a compiled kernel, named so that timings and byte counts can be
 // reported per device kernel.

@@ -430,7 +430,7 @@ int ExecutionPlan::time_kernels(const std::vector<Buffer *> &inputs, std::vector
             if (r == 0) HM_HIP(ctx_, hipEventRecord(e0, ctx_->stream));
             for (const auto &st : steps_) {
                 if (st.native_op.kind != NativeOpKind::None) continue;
-                StepContext sc{ctx_, this, pool_, st};
+                StepContext sc{ctx_, this, pool_, st, true};
                 for (const auto &l : kernels_[st.kernel_idx].launches) {
                     if (l.name != name || skips(l)) continue;
                     if ((rc = l.fn(sc)) != HM_OK) return rc;

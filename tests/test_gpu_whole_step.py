@@ -30,6 +30,7 @@ def small(ctx):
 def test_small_shape_is_served_and_on_by_default(small):
     _cfg, _w, gm, _om = small
     assert gm.whole_step_available() and gm.whole_step()
+    assert gm.launches_per_step() == 1   # embedding row, layers, LM head and greedy pick in one launch
 
 
 @pytest.mark.parametrize("cache_rows", [0, 2, 31, 50, 333])
