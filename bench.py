@@ -192,6 +192,22 @@ def main() -> int:
         host_loop_s = time.perf_counter() - t0
         pcie_inclusive = {"value": round(host_steps / host_loop_s, 2), "unit": "tok/s", "steps": host_steps,
                           "what": "run_kv per token with the logits row downloaded and argmax on the host"}
+        # Sampled decoding through hm_model_generate (reference generate_streaming_core with its default
+        # SamplingConfig, src/generate.rs:646-686): the sampler kernel runs behind every step on the GPU and
+        # the host reads tokens back once per 16 steps.
+        sampled = None
+        room = 2046 - model.kv_cache_len()
+        if room >= 72:
+            from homura_amd.runtime import SamplingConfig
+            scfg = SamplingConfig(0.7, 50, 0.9, 0.0, 1.1, 0.0, 0.0)
+            model.generate([tok], 8, scfg, seed=1)
+            ctx.sync()
+            t0 = time.perf_counter()
+            got = model.generate([tok], 64, scfg, seed=2)
+            dt = time.perf_counter() - t0
+            sampled = {"value": round(len(got) / dt, 2), "unit": "tok/s", "steps": int(len(got)),
+                       "what": "hm_model_generate, temperature 0.7, top_k 50, top_p 0.9, repetition penalty 1.1; "
+                               "wall clock around the call"}
         # The prompt side of the same model: 512 tokens on an empty cache through the prefill pass
         # (projections on the matrix cores), against the same tokens one decode step at a time.
         prefill = None
@@ -308,6 +324,7 @@ def main() -> int:
         "roofline": roofline,
         "cpu_baseline": cpu_baseline,
         "pcie_inclusive": pcie_inclusive,
+        "sampled_decode": sampled,
         "prefill": prefill,
         "quantised_decode": quantised,
         "event_ms_per_step": round(event_ms / args.steps, 4),

@@ -186,7 +186,7 @@ class HfModel {
         int capture_rows = 0, capture_base = 0;
     };
     PrefillScratch pf_;
-    struct SamplerScratch { Buffer work, counts, token, list; int list_cap = 0; } sampler_;
+    struct SamplerScratch { Buffer work, counts, token, list, draws; int list_cap = 0, draws_cap = 0; } sampler_;
     int prefill_min_ = 8;
     int prefill_pieces_ = 3;
     size_t prefill_weight_cache_bytes_ = (size_t)32 << 30;

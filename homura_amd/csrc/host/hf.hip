@@ -1894,6 +1894,9 @@ int sample_check_config(hm_ctx *ctx, const hm_sampling_config *cfg, bool device)
 int sample_token_launch(hm_ctx *ctx, const float *d_logits, float *d_work, const int *d_counts, int vocab,
                         const hm_sampling_config &cfg, float draw, int32_t *d_out, int *d_counts_update, int32_t *d_list,
                         int list_pos);
+int sample_step_launch(hm_ctx *ctx, const float *d_logits, float *d_work, int *d_counts, int vocab,
+                       const hm_sampling_config &cfg, DecodeState *d_cursor, const float *d_draws, int32_t *d_list,
+                       int eos, int *d_stop, int32_t *d_out);
 int zero_ints_launch(hm_ctx *ctx, int *d, size_t n);
 
 int HfModel::generate(const int64_t *h_prompt, int n_prompt, int max_new, const hm_sampling_config &cfg, uint64_t seed,
@@ -1937,30 +1940,73 @@ int HfModel::generate(const int64_t *h_prompt, int n_prompt, int max_new, const 
     std::vector<float> host_logits;
     std::vector<uint32_t> generated;
     int32_t current = ids[n_prompt - 1];
+    if (on_device) {
+        // Device-resident loop: steps are enqueued in chunks with nothing read back in between. The step's
+        // own pick (greedy, no penalties) or the sampler launched behind it (its draw taken from a list made
+        // up front, its pick written over the cursor's next input) feeds the next step on the GPU; the host
+        // reads a chunk's tokens once, and on an end-of-sequence token takes the cache back to the row of the
+        // step that produced it (the reference stops there: src/generate.rs:231-246).
+        const bool own_pick = greedy && !penalties;
+        if (!greedy) {
+            std::vector<float> draws((size_t)max_new);
+            for (auto &d : draws) d = hm_rng_next_f32(&rng);
+            if (s.draws_cap < max_new) {
+                s.draws = Buffer::alloc(ctx_, {max_new}, DType::F32);
+                if (!s.draws) return HM_ERR_OOM;
+                s.draws_cap = max_new;
+            }
+            if ((rc = hm_upload(ctx_, s.draws.ptr(), draws.data(), draws.size() * 4)) != HM_OK) return rc;
+        }
+        const int chunk_cap = std::min(plan_->out_capacity(), 16);
+        std::vector<int32_t> got((size_t)chunk_cap);
+        int done = 0;
+        while (done < max_new) {
+            const int len0 = kv_cache_len();
+            const int n = std::min({chunk_cap, max_new - done, max_seq_len_ - len0});
+            if (n <= 0) break;  // context limit (src/generate.rs:188-194)
+            if ((rc = plan_->arm(&current, 1)) != HM_OK) return rc;
+            int32_t *d_stop = s.token.as<int32_t>() + 1;
+            const int32_t minus_one = -1;
+            if (!own_pick && (rc = hm_upload(ctx_, d_stop, &minus_one, 4)) != HM_OK) return rc;
+            for (int i = 0; i < n; i++) {
+                if ((rc = plan_->run_kv(inputs, weight_bufs_, max_seq_len_)) != HM_OK) return rc;
+                if (own_pick) continue;
+                rc = sample_step_launch(ctx_, plan_->slot(logits_slot)->as<float>(), s.work.as<float>(),
+                                        penalties ? s.counts.as<int>() : nullptr, vocab, cfg, plan_->state(),
+                                        greedy ? nullptr : s.draws.as<float>() + done, s.list.as<int32_t>() + done, eos_token,
+                                        d_stop, s.token.as<int32_t>());
+                if (rc != HM_OK) return rc;
+            }
+            rc = hm_download(ctx_, got.data(), own_pick ? plan_->out_tokens() : s.list.as<int32_t>() + done, (size_t)n * 4);
+            if (rc != HM_OK) return rc;
+            int taken = n;
+            for (int i = 0; i < n; i++)
+                if (got[i] == eos_token) {
+                    taken = i;
+                    break;
+                }
+            for (int i = 0; i < taken; i++) h_tokens[(*n_out)++] = got[i];
+            if (taken < n) {
+                plan_->kv_cache()->reset(len0 + taken + 1);  // rows of the steps behind the stop are dropped
+                break;
+            }
+            current = got[n - 1];
+            done += n;
+        }
+        return finish_sync();
+    }
     for (int step = 0; step < max_new; step++) {
         if (kv_cache_len() >= max_seq_len_) break;  // context limit (src/generate.rs:188-194)
         if ((rc = plan_->arm(&current, 1)) != HM_OK) return rc;
         if ((rc = plan_->run_kv(inputs, weight_bufs_, max_seq_len_)) != HM_OK) return rc;
         const float *d_logits = plan_->slot(logits_slot)->as<float>();
         int32_t tok = 0;
-        if (on_device) {
-            const float draw = greedy ? 0.0f : hm_rng_next_f32(&rng);
-            rc = sample_token_launch(ctx_, d_logits, s.work.as<float>(), penalties ? s.counts.as<int>() : nullptr, vocab, cfg,
-                                     draw, s.token.as<int32_t>(), penalties ? s.counts.as<int>() : nullptr,
-                                     s.list.as<int32_t>(), step);
-            if (rc == HM_OK) rc = hm_download(ctx_, &tok, s.token.ptr(), 4);
-        } else {
-            host_logits.resize(vocab);
-            rc = hm_download(ctx_, host_logits.data(), d_logits, (size_t)vocab * 4);
-            if (rc == HM_OK)
-                rc = hm_sample_token_host(host_logits.data(), vocab, &cfg, generated.data(), (int)generated.size(), &rng, &tok);
-        }
+        host_logits.resize(vocab);
+        rc = hm_download(ctx_, host_logits.data(), d_logits, (size_t)vocab * 4);
+        if (rc == HM_OK)
+            rc = hm_sample_token_host(host_logits.data(), vocab, &cfg, generated.data(), (int)generated.size(), &rng, &tok);
         if (rc != HM_OK) return rc;
-        if (tok == eos_token) {
-            // the reference leaves the loop without storing the token; on the device path it was already
-            // counted for the penalties, which no later step of this call reads
-            break;
-        }
+        if (tok == eos_token) break;  // the reference leaves the loop without storing the token
         generated.push_back((uint32_t)tok);
         h_tokens[(*n_out)++] = tok;
         current = tok;

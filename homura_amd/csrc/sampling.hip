@@ -34,7 +34,28 @@ struct SampleArgs {
     int *counts_update;   // if set: counts_update[token]++ after the pick (the token joins generated_ids)
     int32_t *list;        // if set: list[list_pos] = token
     int list_pos;
+    // Device-resident loop: the step that was just taken is cursor->step - 1; its draw is draws[that], the pick
+    // goes to list[that] and replaces the step's own greedy pick as the next input (cursor->token), and the
+    // first step whose pick is `eos` is noted in stop[0] (-1 until then).
+    DecodeState *cursor;
+    const float *draws;
+    int eos;
+    int *stop;
 };
+
+// Where the pick goes (and which draw it uses) when the cursor says which step this is.
+__device__ __forceinline__ void deliver_pick(const SampleArgs &a, int pick) {
+    *a.out = pick;
+    if (a.counts_update) a.counts_update[pick] += 1;
+    if (a.cursor) {
+        const int idx = a.cursor->step - 1;
+        if (a.list) a.list[idx] = pick;
+        a.cursor->token = pick;
+        if (a.stop && pick == a.eos && *a.stop < 0) *a.stop = idx;
+    } else if (a.list) {
+        a.list[a.list_pos] = pick;
+    }
+}
 
 __device__ __forceinline__ float penalised(float l, int c, const hm_sampling_config &cfg) {
     if (c > 0) {
@@ -53,6 +74,32 @@ __device__ __forceinline__ bool cand_before(float pa, int ia, float pb, int ib) 
     return pa > pb || (pa == pb && ia < ib);
 }
 
+// One pass of the workgroup over [0, n): thread t visits t, t + 1024, ... in ascending order, eight elements'
+// loads in flight before the first is used (a plain strided loop waits for every load in turn, and with one
+// workgroup on the whole chip the passes are pure latency).
+template <class Load, class Use>
+__device__ __forceinline__ void sweep(int n, int tid, Load load, Use use) {
+    constexpr int UN = 8;
+    for (int base = tid; base < n; base += UN * SAMPLE_THREADS) {
+        decltype(load(0)) v[UN];
+#pragma unroll
+        for (int u = 0; u < UN; u++) {
+            const int i = base + u * SAMPLE_THREADS;
+            if (i < n) v[u] = load(i);
+        }
+#pragma unroll
+        for (int u = 0; u < UN; u++) {
+            const int i = base + u * SAMPLE_THREADS;
+            if (i < n) use(i, v[u]);
+        }
+    }
+}
+
+struct LogitAndCount {
+    float l;
+    int c;
+};
+
 __global__ __launch_bounds__(SAMPLE_THREADS) void sample_token_kernel(SampleArgs a) {
     __shared__ float red_f[SAMPLE_THREADS / WAVE];
     __shared__ int red_i[SAMPLE_THREADS / WAVE];
@@ -60,7 +107,8 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_token_kernel(SampleArgs
     __shared__ unsigned sel_prefix, sel_need;
     __shared__ float cand_p[SAMPLE_MAX_K];
     __shared__ int cand_i[SAMPLE_MAX_K];
-    __shared__ unsigned n_cand, eq_taken;
+    __shared__ unsigned n_cand, eq_taken, n_eq;
+    __shared__ int eq_idx[SAMPLE_MAX_K];
     const int tid = threadIdx.x, lane = tid & (WAVE - 1), wave = tid / WAVE;
     const int n = a.vocab;
     const hm_sampling_config cfg = a.cfg;
@@ -70,19 +118,20 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_token_kernel(SampleArgs
     const float inv_temp = greedy ? 1.0f : 1.0f / cfg.temperature;
     float mx = -INFINITY;
     int best = -1;  // greedy: last index of the maximum (Rust max_by keeps the last of equal maxima)
-    for (int i = tid; i < n; i += SAMPLE_THREADS) {
-        float l = penalised(a.logits[i], a.counts ? a.counts[i] : 0, cfg);
-        if (greedy) {
-            if (best < 0 || l >= mx) {
-                mx = l;
-                best = i;
-            }
-        } else {
-            l *= inv_temp;
-            a.work[i] = l;
-            mx = fmaxf(mx, l);
-        }
-    }
+    sweep(n, tid, [&](int i) { return LogitAndCount{a.logits[i], a.counts ? a.counts[i] : 0}; },
+          [&](int i, const LogitAndCount &lc) {
+              float l = penalised(lc.l, lc.c, cfg);
+              if (greedy) {
+                  if (best < 0 || l >= mx) {
+                      mx = l;
+                      best = i;
+                  }
+              } else {
+                  l *= inv_temp;
+                  a.work[i] = l;
+                  mx = fmaxf(mx, l);
+              }
+          });
     if (greedy) {
         for (int off = 32; off >= 1; off >>= 1) {
             const float om = __shfl_xor(mx, off, WAVE);
@@ -103,9 +152,7 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_token_kernel(SampleArgs
                     mx = red_f[w];
                     best = red_i[w];
                 }
-            *a.out = best < 0 ? 0 : best;
-            if (a.counts_update && best >= 0) a.counts_update[best] += 1;
-            if (a.list) a.list[a.list_pos] = best < 0 ? 0 : best;
+            deliver_pick(a, best < 0 ? 0 : best);
         }
         return;
     }
@@ -118,11 +165,11 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_token_kernel(SampleArgs
 
     // ── pass 2: exponentials and their sum ──
     float sum = 0.f;
-    for (int i = tid; i < n; i += SAMPLE_THREADS) {
-        const float e = expf(a.work[i] - mx);
+    sweep(n, tid, [&](int i) { return a.work[i]; }, [&](int i, float l) {
+        const float e = expf(l - mx);
         a.work[i] = e;
         sum += e;
-    }
+    });
     sum = wave_sum(sum);
     if (lane == 0) red_f[wave] = sum;
     __syncthreads();
@@ -145,10 +192,10 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_token_kernel(SampleArgs
         __syncthreads();
         const unsigned prefix = sel_prefix, need = sel_need;
         const unsigned mask = pass == 0 ? 0u : 0xFFFFFFFFu << (shift + bits);
-        for (int i = tid; i < n; i += SAMPLE_THREADS) {
-            const unsigned u = __float_as_uint(a.work[i]);
+        sweep(n, tid, [&](int i) { return a.work[i]; }, [&](int, float e) {
+            const unsigned u = __float_as_uint(e);
             if ((u & mask) == prefix) atomicAdd(&hist[(u >> shift) & ((1u << bits) - 1u)], 1u);
-        }
+        });
         __syncthreads();
         // the bin that holds the need-th largest of the counted elements: thread t owns bins [t*bpt, (t+1)*bpt)
         unsigned mine = 0;
@@ -186,20 +233,36 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_token_kernel(SampleArgs
     if (tid == 0) {
         n_cand = 0;
         eq_taken = 0;
+        n_eq = 0;
     }
     __syncthreads();
     // everything above the K-th value; then the wanted number of elements equal to it, lowest indices first
-    for (int i = tid; i < n; i += SAMPLE_THREADS) {
-        const float e = a.work[i];
+    sweep(n, tid, [&](int i) { return a.work[i]; }, [&](int i, float e) {
         if (__float_as_uint(e) > T) {
             const unsigned at = atomicAdd(&n_cand, 1u);
             cand_p[at] = e;
             cand_i[at] = i;
+        } else if (__float_as_uint(e) == T) {
+            const unsigned at = atomicAdd(&n_eq, 1u);
+            if (at < (unsigned)SAMPLE_MAX_K) eq_idx[at] = i;
+        }
+    });
+    __syncthreads();
+    // Few elements equal the K-th value (nearly always exactly one): they were noted on the way, and each takes
+    // its rank among them by index. Otherwise (a flat tail, underflowed exponentials) one ordered walk.
+    const bool eq_listed = n_eq <= (unsigned)SAMPLE_MAX_K;
+    if (eq_listed && tid < (int)n_eq) {
+        const int mine = eq_idx[tid];
+        unsigned rank = 0;
+        for (unsigned j = 0; j < n_eq; j++) rank += eq_idx[j] < mine ? 1u : 0u;
+        if (rank < need_eq) {
+            const unsigned at = atomicAdd(&n_cand, 1u);
+            cand_p[at] = __uint_as_float(T);
+            cand_i[at] = mine;
         }
     }
-    __syncthreads();
     for (int base = 0; base < n; base += SAMPLE_THREADS) {  // index order: one block-wide ordered take per 1024
-        if (eq_taken >= need_eq) break;
+        if (eq_listed || eq_taken >= need_eq) break;
         const int i = base + tid;
         const bool eq = i < n && __float_as_uint(a.work[i]) == T;
         const unsigned long long m = __ballot(eq);
@@ -267,7 +330,7 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_token_kernel(SampleArgs
         }
         float total = 0.0f;
         for (int i = 0; i < cutoff; i++) total += cand_p[i];
-        const float r = a.draw * total;
+        const float r = (a.cursor ? a.draws[a.cursor->step - 1] : a.draw) * total;
         float accum = 0.0f;
         int pick = cutoff > 0 ? cand_i[cutoff - 1] : 0;
         for (int i = 0; i < cutoff; i++) {
@@ -277,9 +340,7 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_token_kernel(SampleArgs
                 break;
             }
         }
-        *a.out = pick;
-        if (a.counts_update) a.counts_update[pick] += 1;
-        if (a.list) a.list[a.list_pos] = pick;
+        deliver_pick(a, pick);
     }
 }
 
@@ -322,6 +383,35 @@ int sample_token_launch(hm_ctx *ctx, const float *d_logits, float *d_work, const
     a.counts_update = d_counts_update;
     a.list = d_list;
     a.list_pos = list_pos;
+    a.cursor = nullptr;
+    a.draws = nullptr;
+    a.eos = -1;
+    a.stop = nullptr;
+    hipLaunchKernelGGL(sample_token_kernel, dim3(1), dim3(SAMPLE_THREADS), 0, ctx->stream, a);
+    HM_LAUNCH_CHECK(ctx);
+    return HM_OK;
+}
+
+// The sampler behind a decode step whose cursor has already moved on: no argument depends on the step, so the
+// host can enqueue step after step without reading anything back.
+int sample_step_launch(hm_ctx *ctx, const float *d_logits, float *d_work, int *d_counts, int vocab,
+                       const hm_sampling_config &cfg, DecodeState *d_cursor, const float *d_draws, int32_t *d_list,
+                       int eos, int *d_stop, int32_t *d_out) {
+    SampleArgs a;
+    a.logits = d_logits;
+    a.work = d_work;
+    a.counts = d_counts;
+    a.vocab = vocab;
+    a.cfg = cfg;
+    a.draw = 0.0f;
+    a.out = d_out;
+    a.counts_update = d_counts;
+    a.list = d_list;
+    a.list_pos = 0;
+    a.cursor = d_cursor;
+    a.draws = d_draws;
+    a.eos = eos;
+    a.stop = d_stop;
     hipLaunchKernelGGL(sample_token_kernel, dim3(1), dim3(SAMPLE_THREADS), 0, ctx->stream, a);
     HM_LAUNCH_CHECK(ctx);
     return HM_OK;

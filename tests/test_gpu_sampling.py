@@ -131,8 +131,54 @@ def test_model_generate_against_oracle_loop(ctx, name):
             gm.reset_kv_cache()
             got_eos = gm.generate(prompt, 40, lib_cfg(cfg), seed=seed, eos_token_id=want[5])
             assert list(got_eos) == want[:5]
+            # the cache ends behind the step that produced the end token, although more steps were enqueued
+            assert gm.kv_cache_len() == 19 + 6
     say(f"{name}: {agree} of 120 generated tokens compared, all identical")
     assert agree >= 30
+    gm.close()
+
+
+@pytest.mark.parametrize("model", ["tiny", "whole_step"])
+def test_generate_stops_on_device_and_resumes(ctx, model):
+    """The device-resident loop enqueues steps in chunks and reads the tokens back once per chunk: an
+    end-of-sequence token in the middle of a chunk must cut the output there, take the cache back to the row of
+    the step that produced it, and a continuation from that token must land where the uninterrupted run went
+    (the rows of the dropped steps are written again). Greedy, and sampled with a fixed seed, against the
+    same model's uninterrupted run; the greedy run also against hm_model_generate_greedy."""
+    mcfg = synth_model.TINY if model == "tiny" else synth_model.SMALL_WS
+    weights = synth_model.synth_weights(mcfg, 99)
+    gm = synth_model.build_model(ctx, mcfg, weights, 256)
+    prompt = synth.token_ids(5, 11, mcfg.vocab_size)
+    greedy = runtime.SamplingConfig(0.0, 0, 1.0, 0.0, 1.0, 0.0, 0.0)
+    whole = gm.generate(prompt, 45, greedy)
+    assert len(whole) == 45 and gm.kv_cache_len() == 10 + 45
+    gm.reset_kv_cache()
+    assert list(gm.generate_greedy(prompt, 45)) == list(whole)
+
+    def stop_index(seq):
+        """last position that holds an id for the first time, away from the chunk borders when there is one"""
+        firsts = [i for i in range(len(seq)) if seq[i] not in seq[:i]]
+        inner = [i for i in firsts if 17 <= i <= 29]   # steps behind it in the same chunk of 16 have been enqueued
+        return (inner or firsts)[-1]
+
+    notes = []
+    # greedy (the step's own pick), greedy with a repetition penalty (the sampler kernel behind every step, and a
+    # varied sequence), sampled (draws made up front, one per step): the uninterrupted run is the yardstick
+    for name, cfg, seed in (("greedy", greedy, 0),
+                            ("penalised greedy", runtime.SamplingConfig(0.0, 0, 1.0, 0.0, 1.5, 0.2, 0.1), 0),
+                            ("sampled", runtime.SamplingConfig(0.8, 40, 0.95, 0.0, 1.1, 0.0, 0.0), 7)):
+        gm.reset_kv_cache()
+        full = gm.generate(prompt, 45, cfg, seed=seed)
+        assert len(full) == 45
+        j = stop_index(list(full))
+        gm.reset_kv_cache()
+        cut = gm.generate(prompt, 45, cfg, seed=seed, eos_token_id=int(full[j]))
+        assert list(cut) == list(full[:j]) and gm.kv_cache_len() == 10 + j + 1, name
+        if name == "greedy" and j < 44:
+            rest = gm.generate([int(full[j])], 45 - j - 1, cfg)
+            assert list(rest) == list(full[j + 1:])
+        notes.append(f"{name}: stop at step {j} ({len(set(full.tolist()))} distinct ids)")
+    say(f"{model}: " + "; ".join(notes))
     gm.close()
 
 
