@@ -208,6 +208,11 @@ def main() -> int:
             sampled = {"value": round(len(got) / dt, 2), "unit": "tok/s", "steps": int(len(got)),
                        "what": "hm_model_generate, temperature 0.7, top_k 50, top_p 0.9, repetition penalty 1.1; "
                                "wall clock around the call"}
+        # What a step of one launch per projection could reach at best: the per-projection plan's 171 launches
+        # as empty kernels in one graph, and the same with a 4-byte dependency from each to the next.
+        launch_floor = {"kernels": 171, "unit": "us per replay",
+                        "empty": round(ctx.launch_floor(171, False), 1),
+                        "chained_4_byte_load": round(ctx.launch_floor(171, True), 1)}
         # The prompt side of the same model: 512 tokens on an empty cache through the prefill pass
         # (projections on the matrix cores), against the same tokens one decode step at a time.
         prefill = None
@@ -325,6 +330,7 @@ def main() -> int:
         "cpu_baseline": cpu_baseline,
         "pcie_inclusive": pcie_inclusive,
         "sampled_decode": sampled,
+        "launch_floor": launch_floor,
         "prefill": prefill,
         "quantised_decode": quantised,
         "event_ms_per_step": round(event_ms / args.steps, 4),

@@ -195,6 +195,7 @@ SIGNATURES = {
     "hm_model_profile_step": (_I, [_P, C.c_int64, C.POINTER(HmKernelProfile), _I]),
     "hm_model_time_kernels": (_I, [_P, _I, C.POINTER(HmKernelProfile), _I]),
     "hm_model_launches_per_step": (_I, [_P]),
+    "hm_bench_launch_floor": (_I, [_P, _I, _I, _I, c_f32_p]),
     "hm_synth_normal_f32": (None, [C.c_uint64, C.c_uint64, _SZ, C.c_float, _P]),
     "hm_synth_normal_bf16": (None, [C.c_uint64, C.c_uint64, _SZ, C.c_float, _P]),
     "hm_synth_token_ids": (None, [C.c_uint64, _SZ, _I, _P]),

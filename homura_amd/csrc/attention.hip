@@ -334,8 +334,11 @@ __global__ __launch_bounds__(ATT_THREADS) void gqa_decode_attn_stream_kernel(
             vr[i] = ld128_stream(vbase + (size_t)row * HD);
         }
     };
+    // Two steps are in flight from the start (a short walk has its whole range requested at once; the second
+    // request of a one-step walk re-reads the first, so the number of loads outstanding is the same for all).
     u32x4 ka[KS], va[NRG_V], kb[KS], vb[NRG_V];
     request(ka, va, 0);
+    request(kb, vb, min(1, iters - 1));
 
     for (int i = tid; i < G * HD; i += ATT_THREADS)
         qs[i / HD][i % HD] = q[((size_t)b * H + kvhd * G) * HD + i];
@@ -362,8 +365,7 @@ __global__ __launch_bounds__(ATT_THREADS) void gqa_decode_attn_stream_kernel(
         l_run[s] = 0.f;
     }
 
-    auto step = [&](u32x4(&kr)[KS], u32x4(&vr)[NRG_V], u32x4(&nkr)[KS], u32x4(&nvr)[NRG_V], int it) {
-        request(nkr, nvr, min(it + 1, iters - 1));  // the last step re-reads itself: a fixed number of loads in flight
+    auto step = [&](u32x4(&kr)[KS], u32x4(&vr)[NRG_V], int it) {
         float *scp = sc + (it & 1) * G * IT_ROWS;
         float *facp = fac + (it & 1) * G;
         // scores of the wavefront's 16 rows against every head; the small piece first. Lane
@@ -421,10 +423,20 @@ __global__ __launch_bounds__(ATT_THREADS) void gqa_decode_attn_stream_kernel(
             }
         }
     };
-    for (int it = 0; it < iters; it += 2) {
-        step(ka, va, kb, vb, it);
-        if (it + 1 < iters) step(kb, vb, ka, va, it + 1);
+    // A step's registers are asked for again (two steps on) as soon as it has been multiplied; the last steps,
+    // with nothing left to ask for, are written out so that every wait knows how many loads are behind it.
+    int it = 0;
+    for (; it + 3 < iters; it += 2) {
+        step(ka, va, it);
+        request(ka, va, it + 2);
+        step(kb, vb, it + 1);
+        request(kb, vb, it + 3);
     }
+    const int left = iters - it;  // 1..3
+    step(ka, va, it);
+    if (left == 3) request(ka, va, it + 2);
+    if (left >= 2) step(kb, vb, it + 1);
+    if (left == 3) step(ka, va, it + 2);
 
 #pragma unroll
     for (int s = 0; s < SLOTS; s++) {

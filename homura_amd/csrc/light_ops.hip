@@ -3,6 +3,7 @@
 // weight streams; they exist as separate entry points because the reference's quantised plan
 // runs them as separate kernels (src/hf/emitter_quant.rs:713-1134).
 #include "light_ops.h"
+#include "../../include/homura_amd_bench.h"
 
 namespace {
 
@@ -367,7 +368,60 @@ int argmax_candidates_launch(hm_ctx *ctx, const float *d_vals, const int *d_idxs
     return HM_OK;
 }
 
+// A kernel that does nothing, and one that waits for a 4-byte load that depends on its predecessor's store:
+// the two floors of a step built from dependent launches.
+__global__ void floor_empty_kernel() {}
+__global__ void floor_chain_kernel(const int *__restrict__ in, int *__restrict__ out) {
+    if (threadIdx.x == 0) *out = *in + 1;
+}
+
 extern "C" {
+
+int hm_bench_launch_floor(hm_ctx *ctx, int n_kernels, int chained, int replays, float *us_per_replay) {
+    HM_CHECK_CTX(ctx);
+    HM_REQUIRE(ctx, n_kernels > 0 && n_kernels <= 4096 && replays > 0 && us_per_replay, "hm_bench_launch_floor: bad arguments");
+    int *cells = nullptr;
+    HM_HIP(ctx, hipMalloc(&cells, 2 * sizeof(int)));
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    int rc = HM_OK;
+    auto step = [&](hipError_t e) {
+        if (rc == HM_OK && e != hipSuccess) rc = hm_set_error(ctx, HM_ERR_HIP, "launch floor: %s", hipGetErrorString(e));
+    };
+    floor_chain_kernel<<<1, 64, 0, ctx->stream>>>(cells, cells + 1);  // first use outside the capture; cells need no start value
+    step(hipGetLastError());
+    step(hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeRelaxed));
+    if (rc == HM_OK) {
+        for (int i = 0; i < n_kernels; i++) {
+            if (chained)
+                floor_chain_kernel<<<1, 64, 0, ctx->stream>>>(cells + (i & 1), cells + ((i + 1) & 1));
+            else
+                floor_empty_kernel<<<1, 64, 0, ctx->stream>>>();
+        }
+        step(hipStreamEndCapture(ctx->stream, &graph));
+    }
+    if (rc == HM_OK) step(hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0));
+    if (rc == HM_OK) step(hipEventCreate(&e0));
+    if (rc == HM_OK) step(hipEventCreate(&e1));
+    if (rc == HM_OK) {
+        for (int i = 0; i < 3; i++) step(hipGraphLaunch(exec, ctx->stream));
+        step(hipEventRecord(e0, ctx->stream));
+        for (int i = 0; i < replays; i++) step(hipGraphLaunch(exec, ctx->stream));
+        step(hipEventRecord(e1, ctx->stream));
+        step(hipEventSynchronize(e1));
+        float ms = 0.f;
+        step(hipEventElapsedTime(&ms, e0, e1));
+        *us_per_replay = ms * 1000.0f / (float)replays;
+    }
+    if (e0) (void)hipEventDestroy(e0);
+    if (e1) (void)hipEventDestroy(e1);
+    if (exec) (void)hipGraphExecDestroy(exec);
+    if (graph) (void)hipGraphDestroy(graph);
+    (void)hipStreamSynchronize(ctx->stream);
+    (void)hipFree(cells);
+    return rc;
+}
 
 int hm_rmsnorm(hm_ctx *ctx, const float *d_x, const float *d_w, float *d_out, int rows, int dim,
                float eps) {

@@ -1,7 +1,8 @@
 """Roofline timing of the kernel-level entry points at the BASELINE shapes (configurations
 1, 3, 4, 5a, 5b). Every kernel is launched over a ring of weight copies larger than the last-
 level caches (Infinity Cache 256 MiB), all launches recorded into one HIP graph and replayed
-between two HIP events on the launch stream, so the numbers are cold-cache per-launch times.
+between two HIP events on the launch stream, so the numbers are cold-cache per-launch times;
+configurations 1 and 3 also carry `hot_us`, the same launch repeated on one weight buffer.
 """
 from __future__ import annotations
 
@@ -49,8 +50,16 @@ def _time(ctx: Context, launches, reps=None):
     return ms * 1e3 / len(launches)  # microseconds per launch
 
 
-def _entry(name, us, nbytes=None, flops=None, note=None):
+def _hot(ctx: Context, fn, launches=32):
+    """The same launch over and over on one set of buffers: weights that fit the caches stay in them
+    (the per-die L2s hold 32 MiB together, the Infinity Cache 256 MiB)."""
+    return _time(ctx, [fn] * launches)
+
+
+def _entry(name, us, nbytes=None, flops=None, note=None, hot_us=None):
     e = {"config": name, "avg_us": round(us, 3)}
+    if hot_us is not None:
+        e["hot_us"] = round(hot_us, 3)
     if nbytes is not None:
         gbs = nbytes / (us * 1e-6) / 1e9
         e.update({"bytes_per_launch": int(nbytes), "GBps": round(gbs, 1),
@@ -89,12 +98,15 @@ def run_quant_cases(ctx: Context):
         o = ctx.empty(N)
         nbytes = N * (K // 32) * bb + K * 4 + N * 4
         us = _time(ctx, [lambda b=b: raw_fn(x, b, o, 1, K, N) for b in ring])
-        out.append(_entry(name, us, nbytes, note="raw GGUF blocks"))
+        hot = _hot(ctx, lambda: raw_fn(x, ring[0], o, 1, K, N)) if nbytes < (64 << 20) else None
+        out.append(_entry(name, us, nbytes, note="raw GGUF blocks", hot_us=hot))
         planes = [ctx.pack_quant_planes(dt, b, N, K) for b in ring]
         for b in ring:
             b.free()
         us = _time(ctx, [lambda p=p: planes_fn(x, p, o, 1, K, N) for p in planes])
-        out.append(_entry(name.replace(" gemv", " planes gemv"), us, nbytes, note="the same blocks re-packed into planes at upload"))
+        hot = _hot(ctx, lambda: planes_fn(x, planes[0], o, 1, K, N)) if nbytes < (64 << 20) else None
+        out.append(_entry(name.replace(" gemv", " planes gemv"), us, nbytes, note="the same blocks re-packed into planes at upload",
+                          hot_us=hot))
         for b in planes + [x, o]:
             b.free()
     return out
@@ -110,9 +122,11 @@ def run_all(ctx: Context):
     o = ctx.empty(N)
     nbytes = K * N * 2 + K * 4 + N * 4
     us = _time(ctx, [lambda b=b: ctx.gemv_bf16(x, b, o, 1, K, N) for b in ring])
-    out.append(_entry("cfg1 gemv_bf16 [K,N] 896x4864", us, nbytes, note="reference weight layout"))
+    out.append(_entry("cfg1 gemv_bf16 [K,N] 896x4864", us, nbytes, note="reference weight layout",
+                      hot_us=_hot(ctx, lambda: ctx.gemv_bf16(x, ring[0], o, 1, K, N))))
     us = _time(ctx, [lambda b=b: ctx.gemv_bf16_nk(x, b, o, 1, K, N) for b in ring])
-    out.append(_entry("cfg1 gemv_bf16_nk [N,K] 4864x896", us, nbytes, note="stream layout"))
+    out.append(_entry("cfg1 gemv_bf16_nk [N,K] 4864x896", us, nbytes, note="stream layout",
+                      hot_us=_hot(ctx, lambda: ctx.gemv_bf16_nk(x, ring[0], o, 1, K, N))))
     for b in ring:
         b.free()
 

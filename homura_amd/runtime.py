@@ -99,6 +99,13 @@ class Context:
     def sync(self):
         self._check(self.lib.hm_sync(self.h))
 
+    def launch_floor(self, n_kernels: int, chained: bool, replays: int = 20) -> float:
+        """Microseconds per replay of a graph of n_kernels dependent one-wavefront kernels (empty, or each
+        reading 4 bytes its predecessor wrote)."""
+        us = C.c_float()
+        self._check(self.lib.hm_bench_launch_floor(self.h, n_kernels, int(chained), replays, C.byref(us)))
+        return us.value
+
     def device_name(self) -> str:
         buf = C.create_string_buffer(128)
         self._check(self.lib.hm_device_name(self.h, buf, 128))

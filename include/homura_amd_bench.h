@@ -44,6 +44,11 @@ void hm_synth_q8_0(uint64_t seed, size_t n_blocks, float d_scale, uint8_t *out);
 /* n_blocks Q4_0 blocks: nibbles uniform in [0,15], d = f16(|N(0,1)| * d_scale) */
 void hm_synth_q4_0(uint64_t seed, size_t n_blocks, float d_scale, uint8_t *out);
 
+/* Floor of a step made of dependent launches: a HIP graph of `n_kernels` one-wavefront kernels that do
+ * nothing (chained = 0) or that each read 4 bytes their predecessor wrote and write 4 bytes (chained = 1),
+ * replayed `replays` times between two events; microseconds per replay. */
+int hm_bench_launch_floor(hm_ctx *ctx, int n_kernels, int chained, int replays, float *us_per_replay);
+
 /* Phase trace of the latest whole-step decode launch: device-clock ticks (100 MHz) taken by workgroup
  * 0 at 11 points per layer (both workgroup barriers of the Q|K|V, attention, O, gate|up and down
  * phases; the end of the fold follows attention's second barrier) and one at the end of the kernel, then
