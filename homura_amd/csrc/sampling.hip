@@ -100,86 +100,39 @@ struct LogitAndCount {
     int c;
 };
 
-__global__ __launch_bounds__(SAMPLE_THREADS) void sample_token_kernel(SampleArgs a) {
-    __shared__ float red_f[SAMPLE_THREADS / WAVE];
-    __shared__ int red_i[SAMPLE_THREADS / WAVE];
-    __shared__ unsigned hist[4096];
-    __shared__ unsigned sel_prefix, sel_need;
-    __shared__ float cand_p[SAMPLE_MAX_K];
-    __shared__ int cand_i[SAMPLE_MAX_K];
-    __shared__ unsigned n_cand, eq_taken, n_eq;
-    __shared__ int eq_idx[SAMPLE_MAX_K];
+// Shared memory of the selection below.
+struct SelectShared {
+    float red_f[SAMPLE_THREADS / WAVE];
+    int red_i[SAMPLE_THREADS / WAVE];
+    unsigned hist[4096];
+    unsigned sel_prefix, sel_need;
+    float cand_p[SAMPLE_MAX_K];
+    int cand_i[SAMPLE_MAX_K];
+    unsigned n_cand, eq_taken, n_eq;
+    int eq_idx[SAMPLE_MAX_K];
+};
+
+// The second half of the procedure over n items: key_at(j) is item j's 32-bit key (larger key = larger
+// exponential; items with equal keys must appear in ascending token order), idx_at(j) its token,
+// weight_of(key) its exponential; `sum` is the sum of all n_all exponentials of the vocabulary. Selects the
+// top_k items, normalises, applies min_p, sorts and runs the reference's sequential top_p and draw loops.
+template <class KeyAt, class IdxAt, class WeightOf>
+__device__ __forceinline__ void select_sort_draw(SelectShared &sh, const SampleArgs &a, int n, int n_all, float sum, KeyAt key_at,
+                                                 IdxAt idx_at, WeightOf weight_of) {
+    float (&red_f)[SAMPLE_THREADS / WAVE] = sh.red_f;
+    int (&red_i)[SAMPLE_THREADS / WAVE] = sh.red_i;
+    unsigned (&hist)[4096] = sh.hist;
+    unsigned &sel_prefix = sh.sel_prefix, &sel_need = sh.sel_need;
+    float (&cand_p)[SAMPLE_MAX_K] = sh.cand_p;
+    int (&cand_i)[SAMPLE_MAX_K] = sh.cand_i;
+    unsigned &n_cand = sh.n_cand, &eq_taken = sh.eq_taken, &n_eq = sh.n_eq;
+    int (&eq_idx)[SAMPLE_MAX_K] = sh.eq_idx;
+    (void)red_f;
     const int tid = threadIdx.x, lane = tid & (WAVE - 1), wave = tid / WAVE;
-    const int n = a.vocab;
     const hm_sampling_config cfg = a.cfg;
-
-    // ── pass 1: penalties, then either the greedy pick or temperature + maximum ──
-    const bool greedy = cfg.temperature <= 0.0f;
-    const float inv_temp = greedy ? 1.0f : 1.0f / cfg.temperature;
-    float mx = -INFINITY;
-    int best = -1;  // greedy: last index of the maximum (Rust max_by keeps the last of equal maxima)
-    sweep(n, tid, [&](int i) { return LogitAndCount{a.logits[i], a.counts ? a.counts[i] : 0}; },
-          [&](int i, const LogitAndCount &lc) {
-              float l = penalised(lc.l, lc.c, cfg);
-              if (greedy) {
-                  if (best < 0 || l >= mx) {
-                      mx = l;
-                      best = i;
-                  }
-              } else {
-                  l *= inv_temp;
-                  a.work[i] = l;
-                  mx = fmaxf(mx, l);
-              }
-          });
-    if (greedy) {
-        for (int off = 32; off >= 1; off >>= 1) {
-            const float om = __shfl_xor(mx, off, WAVE);
-            const int ob = __shfl_xor(best, off, WAVE);
-            if (ob >= 0 && (best < 0 || om > mx || (om == mx && ob > best))) {
-                mx = om;
-                best = ob;
-            }
-        }
-        if (lane == 0) {
-            red_f[wave] = mx;
-            red_i[wave] = best;
-        }
-        __syncthreads();
-        if (tid == 0) {
-            for (int w = 1; w < SAMPLE_THREADS / WAVE; w++)
-                if (red_i[w] >= 0 && (best < 0 || red_f[w] > mx || (red_f[w] == mx && red_i[w] > best))) {
-                    mx = red_f[w];
-                    best = red_i[w];
-                }
-            deliver_pick(a, best < 0 ? 0 : best);
-        }
-        return;
-    }
-    mx = wave_max(mx);
-    if (lane == 0) red_f[wave] = mx;
-    __syncthreads();
-    mx = red_f[0];
-    for (int w = 1; w < SAMPLE_THREADS / WAVE; w++) mx = fmaxf(mx, red_f[w]);
-    __syncthreads();
-
-    // ── pass 2: exponentials and their sum ──
-    float sum = 0.f;
-    sweep(n, tid, [&](int i) { return a.work[i]; }, [&](int i, float l) {
-        const float e = expf(l - mx);
-        a.work[i] = e;
-        sum += e;
-    });
-    sum = wave_sum(sum);
-    if (lane == 0) red_f[wave] = sum;
-    __syncthreads();
-    sum = 0.f;
-    for (int w = 0; w < SAMPLE_THREADS / WAVE; w++) sum += red_f[w];
-
-    // ── radix select: bit pattern of the K-th largest exponential (all are >= 0, so patterns order like
-    //    values). 12 + 10 + 10 bits: the first pass sees every element, and 4096 bins keep neighbouring
+    // ── radix select: key of the K-th largest item (keys order like the exponentials). 12 + 10 + 10 bits: the first pass sees every element, and 4096 bins keep neighbouring
     //    lanes off each other's LDS word; later passes only count the elements inside the chosen bin. ──
-    const unsigned K = (unsigned)min(cfg.top_k, n);
+    const unsigned K = (unsigned)min(cfg.top_k, n_all);
     if (tid == 0) {
         sel_prefix = 0;
         sel_need = K;
@@ -192,8 +145,7 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_token_kernel(SampleArgs
         __syncthreads();
         const unsigned prefix = sel_prefix, need = sel_need;
         const unsigned mask = pass == 0 ? 0u : 0xFFFFFFFFu << (shift + bits);
-        sweep(n, tid, [&](int i) { return a.work[i]; }, [&](int, float e) {
-            const unsigned u = __float_as_uint(e);
+        sweep(n, tid, key_at, [&](int, unsigned u) {
             if ((u & mask) == prefix) atomicAdd(&hist[(u >> shift) & ((1u << bits) - 1u)], 1u);
         });
         __syncthreads();
@@ -237,14 +189,14 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_token_kernel(SampleArgs
     }
     __syncthreads();
     // everything above the K-th value; then the wanted number of elements equal to it, lowest indices first
-    sweep(n, tid, [&](int i) { return a.work[i]; }, [&](int i, float e) {
-        if (__float_as_uint(e) > T) {
+    sweep(n, tid, key_at, [&](int i, unsigned u) {
+        if (u > T) {
             const unsigned at = atomicAdd(&n_cand, 1u);
-            cand_p[at] = e;
-            cand_i[at] = i;
-        } else if (__float_as_uint(e) == T) {
+            cand_p[at] = weight_of(u);
+            cand_i[at] = idx_at(i);
+        } else if (u == T) {
             const unsigned at = atomicAdd(&n_eq, 1u);
-            if (at < (unsigned)SAMPLE_MAX_K) eq_idx[at] = i;
+            if (at < (unsigned)SAMPLE_MAX_K) eq_idx[at] = idx_at(i);
         }
     });
     __syncthreads();
@@ -257,14 +209,14 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_token_kernel(SampleArgs
         for (unsigned j = 0; j < n_eq; j++) rank += eq_idx[j] < mine ? 1u : 0u;
         if (rank < need_eq) {
             const unsigned at = atomicAdd(&n_cand, 1u);
-            cand_p[at] = __uint_as_float(T);
+            cand_p[at] = weight_of(T);
             cand_i[at] = mine;
         }
     }
     for (int base = 0; base < n; base += SAMPLE_THREADS) {  // index order: one block-wide ordered take per 1024
         if (eq_listed || eq_taken >= need_eq) break;
         const int i = base + tid;
-        const bool eq = i < n && __float_as_uint(a.work[i]) == T;
+        const bool eq = i < n && key_at(i) == T;
         const unsigned long long m = __ballot(eq);
         if (lane == 0) red_i[wave] = __popcll(m);
         __syncthreads();
@@ -273,8 +225,8 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_token_kernel(SampleArgs
         const unsigned rank = before + __popcll(m & ((1ull << lane) - 1ull));
         if (eq && rank < need_eq) {
             const unsigned at = atomicAdd(&n_cand, 1u);
-            cand_p[at] = a.work[i];
-            cand_i[at] = i;
+            cand_p[at] = weight_of(T);
+            cand_i[at] = idx_at(i);
         }
         __syncthreads();
         if (tid == 0) {
@@ -344,6 +296,196 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_token_kernel(SampleArgs
     }
 }
 
+__global__ __launch_bounds__(SAMPLE_THREADS) void sample_token_kernel(SampleArgs a) {
+    __shared__ SelectShared sh;
+    float (&red_f)[SAMPLE_THREADS / WAVE] = sh.red_f;
+    int (&red_i)[SAMPLE_THREADS / WAVE] = sh.red_i;
+    const int tid = threadIdx.x, lane = tid & (WAVE - 1), wave = tid / WAVE;
+    const int n = a.vocab;
+    const hm_sampling_config cfg = a.cfg;
+
+    // ── pass 1: penalties, then either the greedy pick or temperature + maximum ──
+    const bool greedy = cfg.temperature <= 0.0f;
+    const float inv_temp = greedy ? 1.0f : 1.0f / cfg.temperature;
+    float mx = -INFINITY;
+    int best = -1;  // greedy: last index of the maximum (Rust max_by keeps the last of equal maxima)
+    sweep(n, tid, [&](int i) { return LogitAndCount{a.logits[i], a.counts ? a.counts[i] : 0}; },
+          [&](int i, const LogitAndCount &lc) {
+              float l = penalised(lc.l, lc.c, cfg);
+              if (greedy) {
+                  if (best < 0 || l >= mx) {
+                      mx = l;
+                      best = i;
+                  }
+              } else {
+                  l *= inv_temp;
+                  a.work[i] = l;
+                  mx = fmaxf(mx, l);
+              }
+          });
+    if (greedy) {
+        for (int off = 32; off >= 1; off >>= 1) {
+            const float om = __shfl_xor(mx, off, WAVE);
+            const int ob = __shfl_xor(best, off, WAVE);
+            if (ob >= 0 && (best < 0 || om > mx || (om == mx && ob > best))) {
+                mx = om;
+                best = ob;
+            }
+        }
+        if (lane == 0) {
+            red_f[wave] = mx;
+            red_i[wave] = best;
+        }
+        __syncthreads();
+        if (tid == 0) {
+            for (int w = 1; w < SAMPLE_THREADS / WAVE; w++)
+                if (red_i[w] >= 0 && (best < 0 || red_f[w] > mx || (red_f[w] == mx && red_i[w] > best))) {
+                    mx = red_f[w];
+                    best = red_i[w];
+                }
+            deliver_pick(a, best < 0 ? 0 : best);
+        }
+        return;
+    }
+    mx = wave_max(mx);
+    if (lane == 0) red_f[wave] = mx;
+    __syncthreads();
+    mx = red_f[0];
+    for (int w = 1; w < SAMPLE_THREADS / WAVE; w++) mx = fmaxf(mx, red_f[w]);
+    __syncthreads();
+
+    // ── pass 2: exponentials and their sum ──
+    float sum = 0.f;
+    sweep(n, tid, [&](int i) { return a.work[i]; }, [&](int i, float l) {
+        const float e = expf(l - mx);
+        a.work[i] = e;
+        sum += e;
+    });
+    sum = wave_sum(sum);
+    if (lane == 0) red_f[wave] = sum;
+    __syncthreads();
+    sum = 0.f;
+    for (int w = 0; w < SAMPLE_THREADS / WAVE; w++) sum += red_f[w];
+    __syncthreads();
+    // exponentials are >= 0, so their bit patterns order like their values
+    select_sort_draw(sh, a, n, n, sum, [&](int i) { return __float_as_uint(a.work[i]); }, [&](int i) { return i; },
+                     [&](unsigned key) { return __uint_as_float(key); });
+}
+
+// ── Small top_k (<= 64) over a large vocabulary: two launches instead of one workgroup's eight passes ──
+// Front: a workgroup per 1024 tokens applies penalties and temperature, takes its maximum and the sum of
+// exponentials relative to it, sorts its tokens (logit descending, token ascending) and keeps the first 64:
+// the vocabulary's top_k are among them. Back: one workgroup combines the maxima and sums (sum over the
+// vocabulary = sum_b sum_b * exp(max_b - max), equal to the single pass's up to rounding) and runs the shared
+// selection over the kept tokens; it selects by logit, which orders tokens like their exponentials except
+// where two different logits round to one exponential.
+constexpr int FRONT_KEEP = 64;
+
+// larger float <-> larger key (-inf the smallest key of all finite and infinite values)
+__device__ __forceinline__ unsigned order_key(float x) {
+    const unsigned u = __float_as_uint(x);
+    return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+__device__ __forceinline__ float key_value(unsigned k) {
+    return __uint_as_float((k & 0x80000000u) ? (k & 0x7FFFFFFFu) : ~k);
+}
+
+struct FrontOut {
+    unsigned *key;  // [blocks][FRONT_KEEP]
+    int *idx;       // [blocks][FRONT_KEEP]
+    float *stat;    // [blocks][2]: maximum, sum of exponentials relative to it
+};
+__host__ __device__ inline FrontOut front_out(float *work, int blocks) {
+    FrontOut f;
+    f.key = reinterpret_cast<unsigned *>(work);
+    f.idx = reinterpret_cast<int *>(work) + (size_t)blocks * FRONT_KEEP;
+    f.stat = work + (size_t)blocks * FRONT_KEEP * 2;
+    return f;
+}
+
+__global__ __launch_bounds__(SAMPLE_THREADS) void sample_front_kernel(SampleArgs a) {
+    __shared__ float sx[SAMPLE_THREADS];
+    __shared__ int si[SAMPLE_THREADS];
+    __shared__ float red[SAMPLE_THREADS / WAVE];
+    const int tid = threadIdx.x, lane = tid & (WAVE - 1), wave = tid / WAVE;
+    const int i = blockIdx.x * SAMPLE_THREADS + tid;
+    const bool on = i < a.vocab;
+    const float inv_temp = 1.0f / a.cfg.temperature;
+    const float x = on ? penalised(a.logits[i], a.counts ? a.counts[i] : 0, a.cfg) * inv_temp : -INFINITY;
+    float m = wave_max(x);
+    if (lane == 0) red[wave] = m;
+    __syncthreads();
+    m = red[0];
+    for (int w = 1; w < SAMPLE_THREADS / WAVE; w++) m = fmaxf(m, red[w]);
+    __syncthreads();
+    const float e = (on && x > -INFINITY) ? expf(x - m) : 0.f;
+    const float ws = wave_sum(e);
+    if (lane == 0) red[wave] = ws;
+    sx[tid] = x;
+    si[tid] = on ? i : 0x7FFFFFFF;
+    __syncthreads();
+    // bitonic sort: logit descending, token ascending among equals
+    for (int k = 2; k <= SAMPLE_THREADS; k <<= 1)
+        for (int j = k >> 1; j > 0; j >>= 1) {
+            const int partner = tid ^ j;
+            if (partner > tid) {
+                const float xa = sx[tid], xb = sx[partner];
+                const int ia = si[tid], ib = si[partner];
+                const bool up = (tid & k) == 0;
+                if (cand_before(xb, ib, xa, ia) == up) {
+                    sx[tid] = xb;
+                    si[tid] = ib;
+                    sx[partner] = xa;
+                    si[partner] = ia;
+                }
+            }
+            __syncthreads();
+        }
+    const FrontOut f = front_out(a.work, gridDim.x);
+    if (tid < FRONT_KEEP) {
+        f.key[(size_t)blockIdx.x * FRONT_KEEP + tid] = order_key(sx[tid]);
+        f.idx[(size_t)blockIdx.x * FRONT_KEEP + tid] = si[tid];
+    }
+    if (tid == 0) {
+        float sum = 0.f;
+        for (int w = 0; w < SAMPLE_THREADS / WAVE; w++) sum += red[w];
+        f.stat[blockIdx.x * 2] = m;
+        f.stat[blockIdx.x * 2 + 1] = sum;
+    }
+}
+
+__global__ __launch_bounds__(SAMPLE_THREADS) void sample_back_kernel(SampleArgs a, int blocks) {
+    __shared__ SelectShared sh;
+    const int tid = threadIdx.x, lane = tid & (WAVE - 1), wave = tid / WAVE;
+    const FrontOut f = front_out(a.work, blocks);
+    float m = -INFINITY;
+    for (int b = tid; b < blocks; b += SAMPLE_THREADS) m = fmaxf(m, f.stat[b * 2]);
+    m = wave_max(m);
+    if (lane == 0) sh.red_f[wave] = m;
+    __syncthreads();
+    m = sh.red_f[0];
+    for (int w = 1; w < SAMPLE_THREADS / WAVE; w++) m = fmaxf(m, sh.red_f[w]);
+    __syncthreads();
+    float sum = 0.f;
+    for (int b = tid; b < blocks; b += SAMPLE_THREADS) {
+        const float bm = f.stat[b * 2];
+        if (bm > -INFINITY) sum += f.stat[b * 2 + 1] * expf(bm - m);
+    }
+    sum = wave_sum(sum);
+    if (lane == 0) sh.red_f[wave] = sum;
+    __syncthreads();
+    sum = 0.f;
+    for (int w = 0; w < SAMPLE_THREADS / WAVE; w++) sum += sh.red_f[w];
+    __syncthreads();
+    // padding entries (tokens past the vocabulary) carry the key of -inf and the largest token number: they sort
+    // behind every real token and are never among the vocabulary's top_k
+    select_sort_draw(sh, a, blocks * FRONT_KEEP, a.vocab, sum, [&](int j) { return f.key[j]; }, [&](int j) { return f.idx[j]; },
+                     [&](unsigned key) {
+                         const float x = key_value(key);
+                         return x > -INFINITY ? expf(x - m) : 0.f;
+                     });
+}
+
 __global__ void count_tokens_kernel(const uint32_t *__restrict__ ids, int n_ids, int *__restrict__ counts, int vocab) {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i < n_ids && ids[i] < (uint32_t)vocab) atomicAdd(&counts[ids[i]], 1);
@@ -368,6 +510,22 @@ int sample_check_config(hm_ctx *ctx, const hm_sampling_config *cfg, bool device)
     return HM_OK;
 }
 
+// One workgroup for everything, or the front / back pair when top_k is small and the vocabulary large (the pair
+// keeps its 130 words per 1024 tokens in `work`, which has a word per token).
+static int sample_enqueue(hm_ctx *ctx, const SampleArgs &a) {
+    const bool pair = a.cfg.temperature > 0.0f && a.cfg.top_k >= 1 && a.cfg.top_k <= FRONT_KEEP && a.vocab >= 4096;
+    if (pair) {
+        const int blocks = (a.vocab + SAMPLE_THREADS - 1) / SAMPLE_THREADS;
+        hipLaunchKernelGGL(sample_front_kernel, dim3(blocks), dim3(SAMPLE_THREADS), 0, ctx->stream, a);
+        HM_LAUNCH_CHECK(ctx);
+        hipLaunchKernelGGL(sample_back_kernel, dim3(1), dim3(SAMPLE_THREADS), 0, ctx->stream, a, blocks);
+    } else {
+        hipLaunchKernelGGL(sample_token_kernel, dim3(1), dim3(SAMPLE_THREADS), 0, ctx->stream, a);
+    }
+    HM_LAUNCH_CHECK(ctx);
+    return HM_OK;
+}
+
 // counts: device [vocab] occurrences (or nullptr); work: device [vocab] floats
 int sample_token_launch(hm_ctx *ctx, const float *d_logits, float *d_work, const int *d_counts, int vocab,
                         const hm_sampling_config &cfg, float draw, int32_t *d_out, int *d_counts_update, int32_t *d_list,
@@ -387,9 +545,7 @@ int sample_token_launch(hm_ctx *ctx, const float *d_logits, float *d_work, const
     a.draws = nullptr;
     a.eos = -1;
     a.stop = nullptr;
-    hipLaunchKernelGGL(sample_token_kernel, dim3(1), dim3(SAMPLE_THREADS), 0, ctx->stream, a);
-    HM_LAUNCH_CHECK(ctx);
-    return HM_OK;
+    return sample_enqueue(ctx, a);
 }
 
 // The sampler behind a decode step whose cursor has already moved on: no argument depends on the step, so the
@@ -412,9 +568,7 @@ int sample_step_launch(hm_ctx *ctx, const float *d_logits, float *d_work, int *d
     a.draws = d_draws;
     a.eos = eos;
     a.stop = d_stop;
-    hipLaunchKernelGGL(sample_token_kernel, dim3(1), dim3(SAMPLE_THREADS), 0, ctx->stream, a);
-    HM_LAUNCH_CHECK(ctx);
-    return HM_OK;
+    return sample_enqueue(ctx, a);
 }
 
 int zero_ints_launch(hm_ctx *ctx, int *d, size_t n) {
