@@ -303,6 +303,7 @@ def main() -> int:
         sys.path.insert(0, str(ROOT / "tests"))
         import model_fixture as mf  # the CPU oracle: checker / baseline only
         import pyoracle
+        pyoracle.use_isa(pyoracle.best_isa())  # the AVX-512 build of the same source where the host has it
         om = mf.build_oracle_model(cfg, weights, 2048)
         mf.oracle_init_kv(om, kv)
         om.generate_greedy(prompt[:1], 4)  # warm-up
@@ -313,7 +314,7 @@ def main() -> int:
             "value": round(args.cpu_tokens / cpu_s, 2), "unit": "tok/s",
             "cores": pyoracle.num_threads(), "kind": "port",
             "sample": f"{args.cpu_tokens} greedy tokens of the same model from the same 1024-row cache "
-                      f"(C oracle, OpenMP, f32 KV values rounded to bf16)",
+                      f"(C oracle built for {pyoracle.isa()}, OpenMP, f32 KV values rounded to bf16)",
         }
 
     out = {

@@ -38,20 +38,47 @@ class OrcConfig(C.Structure):
 
 
 def build():
-    """Compile the oracle with gcc (a few seconds)."""
-    subprocess.run(["make", "-s", "-C", str(HERE), "liboracle.so"], check=True)
+    """Compile the oracle with gcc (a few seconds): the x86-64-v3 build the tests use and the AVX-512 one."""
+    subprocess.run(["make", "-s", "-C", str(HERE), "all"], check=True)
 
 
 _lib = None
+_isa = "x86-64-v3"
+
+
+def best_isa() -> str:
+    """'x86-64-v4' where this host lists the AVX-512 sets that level needs, else 'x86-64-v3'."""
+    try:
+        flags = next(l for l in open("/proc/cpuinfo") if l.startswith("flags")).split()
+    except (OSError, StopIteration):
+        return "x86-64-v3"
+    need = {"avx512f", "avx512bw", "avx512cd", "avx512dq", "avx512vl"}
+    return "x86-64-v4" if need <= set(flags) else "x86-64-v3"
+
+
+def use_isa(isa: str):
+    """Pick the build before the first load(): the timed CPU baseline asks for best_isa(), everything else
+    keeps the default."""
+    global _isa
+    if _lib is not None and isa != _isa:
+        raise RuntimeError("the oracle library is already loaded")
+    if isa not in ("x86-64-v3", "x86-64-v4"):
+        raise ValueError(isa)
+    _isa = isa
+
+
+def isa() -> str:
+    return _isa
 
 
 def load() -> C.CDLL:
     global _lib
     if _lib is not None:
         return _lib
-    if not LIB_PATH.exists():
+    path = LIB_PATH if _isa == "x86-64-v3" else HERE / "liboracle_v4.so"
+    if not path.exists():
         build()
-    lib = C.CDLL(str(LIB_PATH))
+    lib = C.CDLL(str(path))
     sig = {
         "orc_f16_to_f32": (_F, [C.c_uint16]),
         "orc_f16_to_f32_array": (None, [_P, C.c_size_t, _P]),

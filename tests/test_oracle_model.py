@@ -310,3 +310,32 @@ def test_q8k_activation_hand_in_is_pinned():
     np.concatenate([n.run_kv(ids[i:i + 1]) for i in range(6)])
     _, flips3, maxdiff3 = n.q8k_input_stats()
     assert flips3 == 0 and 0 < maxdiff3 < 1e-6
+
+
+def test_avx512_build_of_the_oracle_gives_the_same_bits():
+    """bench.py times the x86-64-v4 build of oracle.c where the host has AVX-512; the tests check against the
+    x86-64-v3 build. Same source, no value-changing compiler options: a prompt pass and a few greedy steps of a
+    small model must agree bit for bit (run in a child process, the library choice is per process)."""
+    import subprocess
+    import sys
+    import pyoracle
+    if pyoracle.best_isa() != "x86-64-v4":
+        pytest.skip("this host has no AVX-512")
+    code = r"""
+import sys
+sys.path[:0] = [%r, %r, %r]
+import numpy as np
+import pyoracle
+pyoracle.use_isa(sys.argv[1])
+import model_fixture as mf
+from homura_amd import synth, synth_model
+cfg = synth_model.TINY
+om = mf.build_oracle_model(cfg, synth_model.synth_weights(cfg, 5), 64)
+logits = om.run_kv(synth.token_ids(9, 7, cfg.vocab_size))
+toks = om.generate_greedy([3], 6)
+sys.stdout.buffer.write(np.asarray(logits, np.float32).tobytes() + np.asarray(toks, np.int32).tobytes())
+""" % (str(Path(__file__).resolve().parent), str(Path(__file__).resolve().parents[1] / "oracle"),
+       str(Path(__file__).resolve().parents[1]))
+    outs = [subprocess.run([sys.executable, "-c", code, isa], check=True, capture_output=True).stdout
+            for isa in ("x86-64-v3", "x86-64-v4")]
+    assert len(outs[0]) > 7 * 1000 * 4 and outs[0] == outs[1]
