@@ -278,72 +278,91 @@ __global__ __launch_bounds__(ATT_THREADS) void gqa_decode_attn_kernel(
     }
 }
 
-// Long caches (more rows per workgroup than fit in registers at once): the workgroup walks its
-// rows in steps of 64. The loads of step i + 1 are in flight while step i is multiplied, the
-// softmax reference point is the running maximum (sums and the output accumulators are rescaled
-// when it moves), and scores and rescale factors alternate between two LDS slots so a step needs
-// two barriers. Q.K^T runs on the matrix cores: v_mfma_f32_16x16x32_bf16 takes 16 cache rows
-// straight from memory as its A operand (lane r + 16 c holds dims 32 s + 8 c .. + 7 of row r, one
-// 16-byte load) and the G query heads, scaled and split into two bf16 pieces, as columns of B;
-// what the pieces leave out is 2^-17 of a query element. P.V stays on the vector ALUs (V would have
-// to be transposed for the matrix cores, which costs more than the multiply for so few heads).
-// Partials leave in the same (o, max, sum) form as the kernel above.
-constexpr int IT_ROWS = 64;  // rows per step: 16 per wavefront for Q.K^T
+// Long caches (more rows per workgroup than fit in registers at once): the workgroup walks its rows in
+// steps of 128, a wavefront owning 32 rows of a step from the scores to P.V with its own softmax reference
+// point (nothing inside a step waits for another wavefront; the four wavefronts' results are brought to a
+// common maximum once, at the end). Both products run on the matrix cores (v_mfma_f32_16x16x32_bf16):
+//  * Q.K^T, contraction over the head dimension: 16 cache rows straight from memory are the A operand (lane
+//    r + 16 c holds dims 32 s + 8 c .. + 7 of row r, one 16-byte load), the G query heads, scaled and split
+//    into two bf16 pieces (2^-17 of an element left out), are columns of B. Lane h + 16 c receives head h,
+//    rows 4 c .. 4 c + 3 of the tile.
+//  * P.V, contraction over the 32 rows: contraction slot 4 t + i of lane group c stands for row 16 t + 4 c + i,
+//    which is exactly where the scores of the two 16-row tiles t already sit, so the probabilities (two bf16
+//    pieces) are the A operand without leaving their lanes. V needs rows along the contraction: lane d + 16 c
+//    loads dims 8 d .. 8 d + 7 of its group's eight rows (eight 16-byte loads, 256 contiguous bytes per row and
+//    instruction) and transposes the 8 x 8 block in its registers with byte permutes; matrix e of the eight
+//    takes dim 8 d + e as column d. The output lane d + 16 c holds heads 4 c .. 4 c + 3 at dim 8 d + e.
+// The reference point of a head only moves when a score exceeds it by more than LAZY (the exponentials stay
+// below e^LAZY), so the accumulators are rarely rescaled. Partials leave in the same (o, max, sum) form as the
+// kernel above, the "max" being the reference point.
+constexpr int IT_ROWS = 128;  // rows per step: 32 per wavefront
+constexpr float LAZY = 8.0f;
 
 template <int HD, int G>
 __global__ __launch_bounds__(ATT_THREADS) void gqa_decode_attn_stream_kernel(
     const float *__restrict__ q, const uint16_t *__restrict__ kcache,
     const uint16_t *__restrict__ vcache, float *__restrict__ out, float *__restrict__ part_o,
-    float *__restrict__ part_ml, int kvh, int max_len, int kv_len, int chunk, float scale,
-    int lds_front) {
-    constexpr int LPR = HD / 8, RPI = WAVE / LPR;
-    constexpr int NRG_V = IT_ROWS / (ATT_WAVES * RPI);      // V row groups per wavefront and step
-    constexpr int KS = HD / 32;                             // k steps of the score MFMA
-    constexpr int SLOTS = (G + ATT_WAVES - 1) / ATT_WAVES;  // heads whose statistics a wavefront keeps
-    static_assert(IT_ROWS == WAVE && IT_ROWS == 16 * ATT_WAVES, "one score per lane; 16 rows per wavefront");
-    static_assert(G <= 16, "heads are columns of a 16-wide MFMA tile");
-    extern __shared__ __attribute__((aligned(16))) float sm[];
-    float *sc = sm;                      // [2][G][IT_ROWS] scores, then probabilities
-    float *fac = sm + 2 * G * IT_ROWS;   // [2][G] rescale factor of the step
-    float *red = sm + lds_front;         // [ATT_WAVES * RPI][G][HD]
+    float *__restrict__ part_ml, int kvh, int max_len, int kv_len, int chunk, float scale) {
+    constexpr int KS = HD / 32;  // k steps of the score MFMA
+    constexpr int DS = HD / 8;   // 8-dim slices of a row
+    static_assert(IT_ROWS == 32 * ATT_WAVES, "32 rows per wavefront and step");
+    static_assert(G <= 8, "heads 4 c + i of lane group c < 2");
+    __shared__ __attribute__((aligned(16))) float red[ATT_WAVES][G][HD];
     __shared__ float qs[G][HD];
     __shared__ float s_m[G], s_l[G];
+    __shared__ float s_mw[ATT_WAVES][G], s_lw[ATT_WAVES][G];
 
     const int tid = threadIdx.x, lane = tid & (WAVE - 1), wave = tid / WAVE;
-    const int sub = lane / LPR, dl = lane % LPR;  // V: row within a group, 8-dim slice
-    const int l16 = lane & 15, kg = lane >> 4;     // K operand: row of the wavefront's 16, 8-dim slice of a k step
+    const int l16 = lane & 15, kg = lane >> 4;
     const int split = blockIdx.x, nsplit = gridDim.x, kvhd = blockIdx.y, b = blockIdx.z;
     const int H = kvh * G;
     const int n0 = split * chunk;
     const size_t head_base = ((size_t)b * kvh + kvhd) * max_len * HD;
     const uint16_t *kbase = kcache + head_base + (size_t)n0 * HD + kg * 8;
-    const uint16_t *vbase = vcache + head_base + (size_t)n0 * HD + dl * 8;
+    const uint16_t *vbase = vcache + head_base + (size_t)n0 * HD + (l16 < DS ? l16 : 0) * 8;
     const int cnt = min(kv_len, n0 + chunk) - n0;  // >= 1: the grid covers kv_len exactly
     const int iters = (cnt + IT_ROWS - 1) / IT_ROWS;
 
     // Rows past the live range are clamped to the last live row instead of masked: every request issues
     // the same number of loads, so the waits can leave the next step's loads in flight. Their scores become
     // -inf below, hence their probabilities zero, and the clamped V rows are finite.
-    auto request = [&](u32x4(&kr)[KS], u32x4(&vr)[NRG_V], int it) {
-        const int krow = min(it * IT_ROWS + 16 * wave + l16, cnt - 1);
+    // One set of row registers: the next step's K rows are asked for as soon as this step's scores are out of
+    // the matrix cores, its V rows as soon as this step's P.V is. (A second set with two steps in flight was
+    // slower, alone on a CU or not.)
+    u32x4 kr0[2][KS], vr0[8];
+    auto request_k = [&](u32x4(&kr)[2][KS], int it) {
+        const int base = it * IT_ROWS + 32 * wave;
 #pragma unroll
-        for (int s = 0; s < KS; s++) kr[s] = ld128_stream(kbase + (size_t)krow * HD + 32 * s);
+        for (int t = 0; t < 2; t++) {
+            const int krow = min(base + 16 * t + l16, cnt - 1);
 #pragma unroll
-        for (int i = 0; i < NRG_V; i++) {
-            const int row = min(it * IT_ROWS + (i * ATT_WAVES + wave) * RPI + sub, cnt - 1);
-            vr[i] = ld128_stream(vbase + (size_t)row * HD);
+            for (int s = 0; s < KS; s++) kr[t][s] = ld128_stream(kbase + (size_t)krow * HD + 32 * s);
         }
     };
-    // Two steps are in flight from the start (a short walk has its whole range requested at once; the second
-    // request of a one-step walk re-reads the first, so the number of loads outstanding is the same for all).
-    u32x4 ka[KS], va[NRG_V], kb[KS], vb[NRG_V];
-    request(ka, va, 0);
-    request(kb, vb, min(1, iters - 1));
-
-    for (int i = tid; i < G * HD; i += ATT_THREADS)
-        qs[i / HD][i % HD] = q[((size_t)b * H + kvhd * G) * HD + i];
+    auto request_v = [&](u32x4(&vr)[8], int it) {
+        const int base = it * IT_ROWS + 32 * wave;
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const int row = min(base + 16 * (j / 4) + 4 * kg + (j % 4), cnt - 1);
+            vr[j] = ld128_stream(vbase + (size_t)row * HD);
+        }
+    };
+    // the queries are asked for first: loads return in order, and the operand below is built while the rows arrive
+    float qv[(G * HD + ATT_THREADS - 1) / ATT_THREADS];
+#pragma unroll
+    for (int u = 0; u < (G * HD + ATT_THREADS - 1) / ATT_THREADS; u++) {
+        const int i = tid + u * ATT_THREADS;
+        qv[u] = i < G * HD ? q[((size_t)b * H + kvhd * G) * HD + i] : 0.f;
+    }
+    request_k(kr0, 0);
+    request_v(vr0, 0);
+#pragma unroll
+    for (int u = 0; u < (G * HD + ATT_THREADS - 1) / ATT_THREADS; u++) {
+        const int i = tid + u * ATT_THREADS;
+        if (i < G * HD) qs[i / HD][i % HD] = qv[u];
+    }
     __syncthreads();
-    // B operand: column l16 is query head l16 (columns past G are zero), scaled, as two pieces
+    // B operand of the scores: column l16 is query head l16 (columns past G are zero), scaled, as two pieces
     bf16x8 qop[KS][2];
 #pragma unroll
     for (int s = 0; s < KS; s++) {
@@ -353,104 +372,121 @@ __global__ __launch_bounds__(ATT_THREADS) void gqa_decode_attn_stream_kernel(
         split8<2>(f, qop[s]);
     }
 
-    float acc[G][8];
+    f32x4 acc[8];  // matrix e: heads 4 kg .. 4 kg + 3 at dim 8 l16 + e
 #pragma unroll
-    for (int gi = 0; gi < G; gi++)
-#pragma unroll
-        for (int e = 0; e < 8; e++) acc[gi][e] = 0.f;
-    float m_run[SLOTS], l_run[SLOTS];
-#pragma unroll
-    for (int s = 0; s < SLOTS; s++) {
-        m_run[s] = -INFINITY;
-        l_run[s] = 0.f;
-    }
+    for (int e = 0; e < 8; e++) acc[e] = f32x4{0.f, 0.f, 0.f, 0.f};
+    // Softmax state of head l16 over this wavefront's rows so far (the four lanes that share an l16 agree;
+    // lanes with l16 >= G carry nothing).
+    float m_run = -INFINITY, l_run = 0.f;
 
-    auto step = [&](u32x4(&kr)[KS], u32x4(&vr)[NRG_V], int it) {
-        float *scp = sc + (it & 1) * G * IT_ROWS;
-        float *facp = fac + (it & 1) * G;
-        // scores of the wavefront's 16 rows against every head; the small piece first. Lane
-        // l16 + 16 c receives head l16, rows 4 c .. 4 c + 3; rows past the live range count as -inf.
-        {
-            f32x4 c = {0.f, 0.f, 0.f, 0.f};
+    bf16x8 pop[2];  // this step's probabilities as the A operand of P.V, two pieces
+    auto scores = [&](u32x4(&kr)[2][KS], int it) {
+        f32x4 c[2];
+#pragma unroll
+        for (int t = 0; t < 2; t++) {
+            c[t] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int s = 0; s < KS; s++) {
-                const bf16x8 kop = __builtin_bit_cast(bf16x8, kr[s]);
-                c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kop, qop[s][1], c, 0, 0, 0);
-                c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kop, qop[s][0], c, 0, 0, 0);
-            }
-            const int r0 = 16 * wave + 4 * kg;
-#pragma unroll
-            for (int i = 0; i < 4; i++)
-                if (it * IT_ROWS + r0 + i >= cnt) c[i] = -INFINITY;
-            if (l16 < G) *reinterpret_cast<f32x4 *>(scp + l16 * IT_ROWS + r0) = c;
-        }
-        __syncthreads();
-        // one wavefront per head: move the running maximum, turn scores into exp(s - max)
-#pragma unroll
-        for (int s = 0; s < SLOTS; s++) {
-            const int gi = wave + s * ATT_WAVES;
-            if (gi < G) {
-                const float x = scp[gi * IT_ROWS + lane];
-                const float m_new = fmaxf(m_run[s], wave_max(x));  // finite: row 0 of a step is live
-                const float e = expf(x - m_new);
-                scp[gi * IT_ROWS + lane] = e;
-                const float f = expf(m_run[s] - m_new);
-                l_run[s] = fmaf(l_run[s], f, wave_sum(e));
-                m_run[s] = m_new;
-                if (lane == 0) facp[gi] = f;
+                const bf16x8 kop = __builtin_bit_cast(bf16x8, kr[t][s]);
+                c[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kop, qop[s][1], c[t], 0, 0, 0);  // the small piece first
+                c[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kop, qop[s][0], c[t], 0, 0, 0);
             }
         }
-        __syncthreads();
-        // o = o * factor + P.V
+        const int r0 = it * IT_ROWS + 32 * wave + 4 * kg;
+        float mx = -INFINITY;
 #pragma unroll
-        for (int gi = 0; gi < G; gi++) {
-            const float f = facp[gi];
-            if (f != 1.f) {
+        for (int t = 0; t < 2; t++)
 #pragma unroll
-                for (int e = 0; e < 8; e++) acc[gi][e] *= f;
+            for (int i = 0; i < 4; i++) {
+                if (r0 + 16 * t + i >= cnt) c[t][i] = -INFINITY;
+                mx = fmaxf(mx, c[t][i]);
+            }
+        // the head's maximum over the 32 rows: eight in this lane, the rest in the lanes 16, 32, 48 on
+        mx = fmaxf(mx, __shfl_xor(mx, 16, WAVE));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
+        // move the reference point only when it has to move (first live row, or a score LAZY above it)
+        const bool move = mx > m_run + LAZY || (m_run == -INFINITY && mx > -INFINITY);
+        if (__any(move && l16 < G)) {
+            const float m_new = move ? mx : m_run;
+            const float f = m_run == -INFINITY ? 0.f : expf(m_run - m_new);  // 1 where the point stays
+            l_run *= f;
+            m_run = m_new;
+            float fh[8];  // factor of head j: held by the lanes with l16 == j
+#pragma unroll
+            for (int j = 0; j < 8; j++) fh[j] = j < G ? __int_as_float(__builtin_amdgcn_readlane(__float_as_int(f), j)) : 1.f;
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const float fi = kg == 0 ? fh[i] : fh[4 + i];
+#pragma unroll
+                for (int e = 0; e < 8; e++) acc[e][i] *= fi;
             }
         }
+        const float m_ref = m_run == -INFINITY ? 0.f : m_run;  // no live row yet: everything below becomes 0
+        float p[8];
+        float psum = 0.f;
 #pragma unroll
-        for (int i = 0; i < NRG_V; i++) {
-            const int r = (i * ATT_WAVES + wave) * RPI + sub;
-            float vf[8];
-            unpack8(vr[i], vf);
+        for (int t = 0; t < 2; t++)
 #pragma unroll
-            for (int gi = 0; gi < G; gi++) {
-                const float p = scp[gi * IT_ROWS + r];
-#pragma unroll
-                for (int e = 0; e < 8; e++) acc[gi][e] = fmaf(p, vf[e], acc[gi][e]);
+            for (int i = 0; i < 4; i++) {
+                p[4 * t + i] = expf(c[t][i] - m_ref);
+                psum += p[4 * t + i];
             }
+        psum += __shfl_xor(psum, 16, WAVE);
+        psum += __shfl_xor(psum, 32, WAVE);
+        l_run += psum;
+        split8<2>(p, pop);
+    };
+    auto multiply_v = [&](u32x4(&vr)[8]) {
+        // V^T: the 8 (rows) x 8 (dims) block of this lane, transposed in registers
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            u32x4 tv;
+#pragma unroll
+            for (int qd = 0; qd < 4; qd++)
+                tv[qd] = __builtin_amdgcn_perm(vr[2 * qd + 1][e / 2], vr[2 * qd][e / 2], (e & 1) ? 0x07060302u : 0x05040100u);
+            if (l16 >= DS) tv = u32x4{0u, 0u, 0u, 0u};
+            const bf16x8 vop = __builtin_bit_cast(bf16x8, tv);
+            acc[e] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pop[1], vop, acc[e], 0, 0, 0);
+            acc[e] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pop[0], vop, acc[e], 0, 0, 0);
         }
     };
-    // A step's registers are asked for again (two steps on) as soon as it has been multiplied; the last steps,
-    // with nothing left to ask for, are written out so that every wait knows how many loads are behind it.
     int it = 0;
-    for (; it + 3 < iters; it += 2) {
-        step(ka, va, it);
-        request(ka, va, it + 2);
-        step(kb, vb, it + 1);
-        request(kb, vb, it + 3);
+    for (; it + 1 < iters; it++) {
+        scores(kr0, it);
+        request_k(kr0, it + 1);
+        multiply_v(vr0);
+        request_v(vr0, it + 1);
     }
-    const int left = iters - it;  // 1..3
-    step(ka, va, it);
-    if (left == 3) request(ka, va, it + 2);
-    if (left >= 2) step(kb, vb, it + 1);
-    if (left == 3) step(ka, va, it + 2);
+    scores(kr0, it);
+    multiply_v(vr0);
 
-#pragma unroll
-    for (int s = 0; s < SLOTS; s++) {
-        const int gi = wave + s * ATT_WAVES;
-        if (gi < G && lane == 0) {
-            s_m[gi] = m_run[s];
-            s_l[gi] = l_run[s];
-        }
+    // the four wavefronts' results to a common reference point per head
+    if (kg == 0 && l16 < G) {
+        s_mw[wave][l16] = m_run;
+        s_lw[wave][l16] = l_run;
     }
+    __syncthreads();
+    if (tid < G) {
+        float M = s_mw[0][tid];
+        for (int w = 1; w < ATT_WAVES; w++) M = fmaxf(M, s_mw[w][tid]);  // finite: row 0 of the split is live
+        float L = 0.f;
+        for (int w = 0; w < ATT_WAVES; w++) L = fmaf(s_lw[w][tid], expf(s_mw[w][tid] - M), L);
+        s_m[tid] = M;
+        s_l[tid] = L;
+    }
+    if (kg < 2) {
 #pragma unroll
-    for (int gi = 0; gi < G; gi++) {
-        float *dst = red + ((size_t)(wave * RPI + sub) * G + gi) * HD + dl * 8;
-        *reinterpret_cast<f32x4 *>(dst) = f32x4{acc[gi][0], acc[gi][1], acc[gi][2], acc[gi][3]};
-        *reinterpret_cast<f32x4 *>(dst + 4) = f32x4{acc[gi][4], acc[gi][5], acc[gi][6], acc[gi][7]};
+        for (int i = 0; i < 4; i++) {
+            const int gi = 4 * kg + i;
+            if (gi < G && l16 < DS) {
+                float M = s_mw[0][gi];
+                for (int w = 1; w < ATT_WAVES; w++) M = fmaxf(M, s_mw[w][gi]);
+                const float sc_w = expf(s_mw[wave][gi] - M);
+                float *dst = &red[wave][gi][8 * l16];
+                *reinterpret_cast<f32x4 *>(dst) = f32x4{acc[0][i] * sc_w, acc[1][i] * sc_w, acc[2][i] * sc_w, acc[3][i] * sc_w};
+                *reinterpret_cast<f32x4 *>(dst + 4) = f32x4{acc[4][i] * sc_w, acc[5][i] * sc_w, acc[6][i] * sc_w, acc[7][i] * sc_w};
+            }
+        }
     }
     __syncthreads();
 
@@ -460,7 +496,7 @@ __global__ __launch_bounds__(ATT_THREADS) void gqa_decode_attn_stream_kernel(
     for (int i = tid; i < G * HD; i += ATT_THREADS) {
         float v = 0.f;
 #pragma unroll
-        for (int w = 0; w < ATT_WAVES * RPI; w++) v += red[(size_t)w * G * HD + i];
+        for (int w = 0; w < ATT_WAVES; w++) v += (&red[w][0][0])[i];
         if (nsplit == 1) {
             const int gi = i / HD, d = i % HD;
             out[((size_t)b * H + kvhd * G + gi) * HD + d] = v / s_l[gi];
@@ -492,7 +528,7 @@ __global__ __launch_bounds__(HD) void gqa_decode_fold_kernel(
     const size_t pair = (size_t)b * kvh + kvhd;
     const float *ao = part_o + (pair * nsplit * G + gi) * HD + d;
     const float *aml = part_ml + (pair * nsplit * G + gi) * 2;
-    constexpr int FB = 16;  // splits fetched per batch, all loads of a batch in flight together
+    constexpr int FB = 32;  // splits fetched per batch, all loads of a batch in flight together
     float o[FB];
 #pragma unroll
     for (int u = 0; u < FB; u++) o[u] = u < nsplit ? ao[(size_t)u * G * HD] : 0.f;
@@ -571,23 +607,13 @@ int launch_attn(hm_ctx *ctx, const AttnArgs &a, int nsplit, int chunk) {
 // Long caches through the stepping kernel; its partials go through the same fold.
 template <int HD, int G>
 int launch_attn_stream(hm_ctx *ctx, const AttnArgs &a, int nsplit, int chunk) {
-    constexpr int RPI = WAVE / (HD / 8);
-    const size_t front = ((size_t)2 * G * IT_ROWS + 2 * G + 3) / 4 * 4;  // 16-byte rows behind it
-    const size_t lds = (front + (size_t)ATT_WAVES * RPI * G * HD) * sizeof(float);
     const size_t pairs = (size_t)a.B * a.kvh;
     float *part_o = a.partials ? a.partials : (float *)ctx->workspace;
     float *part_ml = part_o + pairs * nsplit * G * HD;
-    static bool lds_limit_raised = false;  // per instantiation
-    if (lds > 64 * 1024 && !lds_limit_raised) {
-        HM_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(&gqa_decode_attn_stream_kernel<HD, G>),
-                                        hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024));
-        lds_limit_raised = true;
-    }
-    HM_REQUIRE(ctx, lds <= 96 * 1024, "gqa_decode_attn: LDS need %zu too large", lds);
     HM_REQUIRE(ctx, chunk % IT_ROWS == 0, "gqa_decode_attn: chunk %d must be a multiple of %d", chunk, IT_ROWS);
     hipLaunchKernelGGL((gqa_decode_attn_stream_kernel<HD, G>), dim3(nsplit, a.kvh, a.B),
-                       dim3(ATT_THREADS), lds, ctx->stream, a.q, a.kcache, a.vcache, a.out, part_o,
-                       part_ml, a.kvh, a.max_len, a.kv_len, chunk, a.scale, (int)front);
+                       dim3(ATT_THREADS), 0, ctx->stream, a.q, a.kcache, a.vcache, a.out, part_o,
+                       part_ml, a.kvh, a.max_len, a.kv_len, chunk, a.scale);
     HM_LAUNCH_CHECK(ctx);
     if (nsplit > 1) {
         const size_t fold_lds = (size_t)nsplit * 2 * sizeof(float);
@@ -664,14 +690,18 @@ int gqa_decode_attn_launch(hm_ctx *ctx, const AttnArgs &a) {
         int want = (int)(((size_t)ctx->num_cus + pairs - 1) / pairs);
         chunk = (span + want - 1) / want;
         chunk = (chunk + rows_step - 1) / rows_step * rows_step;
-        // More rows per workgroup than its registers hold: the stepping kernel, two workgroups per
-        // CU (plain calls only; the decode plan's fused prologue lives in the other kernel).
+        // More rows per workgroup than its registers hold: the stepping kernel (plain calls only; the decode
+        // plan's fused prologue lives in the other kernel). One workgroup a CU while that keeps a workgroup's
+        // walk at four steps or fewer (fewer partial results, a shorter fold), else two.
         if (chunk > 128 && !a.state && !a.qkv_raw) {
-            stepping = true;
             const int it_rows = IT_ROWS;
-            want = (int)(((size_t)2 * ctx->num_cus + pairs - 1) / pairs);
-            chunk = (span + want - 1) / want;
             chunk = (chunk + it_rows - 1) / it_rows * it_rows;
+            stepping = true;
+            if (chunk > 4 * it_rows) {
+                want = (int)(((size_t)2 * ctx->num_cus + pairs - 1) / pairs);
+                chunk = (span + want - 1) / want;
+                chunk = (chunk + it_rows - 1) / it_rows * it_rows;
+            }
         }
     }
     if (stepping) {
@@ -679,8 +709,8 @@ int gqa_decode_attn_launch(hm_ctx *ctx, const AttnArgs &a) {
         const int nsplit = (a.kv_len + chunk - 1) / chunk;
         const size_t ws_need = pairs * nsplit * g * (a.hd + 2) * sizeof(float);
         HM_REQUIRE(ctx, ws_need <= ws_have, "gqa_decode_attn: %zu bytes of partial results exceed the %zu available", ws_need, ws_have);
-        if (a.hd == 128) return dispatch_g<128>(ctx, a, g, nsplit, chunk, true);
-        return dispatch_g<64>(ctx, a, g, nsplit, chunk, true);
+        if (a.hd == 128) return dispatch_g<128>(ctx, a, g, nsplit, chunk, stepping);
+        return dispatch_g<64>(ctx, a, g, nsplit, chunk, stepping);
     }
     if (chunk < rows_step) chunk = rows_step;
     if (chunk > 128) chunk = 128;

@@ -198,8 +198,8 @@ int hm_kv_append(hm_ctx *ctx, uint16_t *d_kcache, uint16_t *d_vcache, const floa
  * attended (the all-zero decode mask of src/hf/precompute.rs:49-64); kv head = h / (H/kvh);
  * scores * scale, softmax in f32, out f32 [B][H*hd]. hd == 128 or 64. The cache rows are split over
  * workgroups and a second launch folds the partial sums in row order; with more than 128 rows per
- * workgroup (long caches, many sequences) the workgroups walk their rows in steps and take Q.K^T on the
- * matrix cores with q as two bf16 pieces (2^-17 of an element left out). */
+ * workgroup (long caches, many sequences) the workgroups walk their rows in steps and take both products
+ * on the matrix cores, q and the probabilities as two bf16 pieces each (2^-17 of an element left out). */
 int hm_gqa_decode_attn(hm_ctx *ctx, const float *d_q, const uint16_t *d_kcache,
                        const uint16_t *d_vcache, float *d_out, int B, int H, int kvh, int hd,
                        int max_len, int kv_len, float scale);
