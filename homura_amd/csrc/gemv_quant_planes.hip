@@ -330,6 +330,139 @@ __global__ __launch_bounds__(256) void pack_planes_kernel(const uint8_t *__restr
     for (int j = 0; j < QB; j++) quants[i * QB + j] = blk[2 + q * QB + j];
 }
 
+// Q4_0, tall matrices (the LM-head shape), no fused light ops: a lane's unit is half a block. A trip is two
+// rows; their 4 * K / 32 half blocks lie one after the other in the quant plane, so lane l takes halves l,
+// l + 64, ... of the trip with one 8-byte and one 2-byte load each: half the load instructions of the
+// quarter-block kernel above, one scale conversion per 16 weights instead of 8, and the half's 16 activations
+// (times 2^9) stay in registers for every trip. A row's halves are spread over the lanes (and over a lane's
+// units), so the two row sums are masked wave sums. Needs K / 32 a multiple of 16 (the trip then is UPL * 64
+// halves) and UPL <= 4. (Whole blocks per lane, four rows a trip: 144 registers, three workgroups a CU, slower.)
+template <int UPL>
+__global__ __launch_bounds__(PTHREADS) void gemv_q4_0_halves_kernel(const float *__restrict__ x, const uint8_t *__restrict__ quants,
+                                                                    const uint16_t *__restrict__ scales, float *__restrict__ out,
+                                                                    int K, int N) {
+    constexpr int RB = 2;
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    float *xs = reinterpret_cast<float *>(smem);
+    const int tid = threadIdx.x, lane = tid & (WAVE - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(tid / WAVE);
+    const int nb = K / 32;  // == UPL * 16
+    const int gw = blockIdx.x * PWAVES + wave, nwaves = gridDim.x * PWAVES;
+    const int ntrips = (N + RB - 1) / RB;
+    // this lane's units: row (within the trip), block (within the row) and half (within the block) of unit u
+    int urow[UPL], ublk[UPL], uhalf[UPL];
+#pragma unroll
+    for (int u = 0; u < UPL; u++) {
+        const int f = u * WAVE + lane;
+        urow[u] = f / (2 * nb);
+        ublk[u] = (f % (2 * nb)) >> 1;
+        uhalf[u] = f & 1;
+    }
+    // D trips of a wavefront are in flight at a time (1.7 KB each at K = 1536): with one, the sixteen wavefronts
+    // of a CU have 27 KB outstanding (30.8 us at the 1536 -> 151936 shape), with four 29.2 us; six cost a
+    // workgroup of occupancy and bring nothing.
+    constexpr int D = 4;
+    u32x2 qn[D][UPL];
+    uint32_t sn[D][UPL];
+    auto request = [&](u32x2(&q)[UPL], uint32_t(&sc)[UPL], int trip) {
+#pragma unroll
+        for (int u = 0; u < UPL; u++) {
+            const int row = min(trip * RB + urow[u], N - 1);  // rows past the end re-read the last one
+            const size_t blk = (size_t)row * nb + ublk[u];
+            q[u] = __builtin_nontemporal_load((global_u32x2_ptr)(quants + blk * 16 + uhalf[u] * 8));
+            sc[u] = __builtin_nontemporal_load((global_u16_ptr)(scales + blk));
+        }
+    };
+    // activations first (loads return in issue order), the first trip's weights right behind them
+    f32x4 xr[4];
+#pragma unroll
+    for (int u = 0; u < 4; u++) {
+        const int k = (tid + u * PTHREADS) * 4;
+        xr[u] = k < K ? *reinterpret_cast<const f32x4 *>(x + k) : f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+    int trip = gw;  // the trip in buffer 0; buffer d holds trip + d * nwaves
+#pragma unroll
+    for (int d = 0; d < D; d++)
+        if (trip + d * nwaves < ntrips) request(qn[d], sn[d], trip + d * nwaves);
+#pragma unroll
+    for (int u = 0; u < 4; u++) {
+        const int k = (tid + u * PTHREADS) * 4;
+        if (k < K) *reinterpret_cast<f32x4 *>(xs + k) = xr[u];
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");  // LDS only: the weight loads stay in flight
+    // byte j of a block holds weight j (low nibble) and weight 16 + j (high nibble); this half has bytes 8 h .. 8 h + 7
+    float xlo[UPL][8], xhi[UPL][8], sx8[UPL];
+#pragma unroll
+    for (int u = 0; u < UPL; u++) {
+        float sx = 0.f;
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            const f32x4 a = *reinterpret_cast<const f32x4 *>(xs + ublk[u] * 32 + uhalf[u] * 8 + 4 * j);
+            const f32x4 b = *reinterpret_cast<const f32x4 *>(xs + ublk[u] * 32 + 16 + uhalf[u] * 8 + 4 * j);
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                sx += a[e] + b[e];
+                xlo[u][4 * j + e] = a[e] * NIBBLE_FP8_UNIT;
+                xhi[u][4 * j + e] = b[e] * NIBBLE_FP8_UNIT;
+            }
+        }
+        sx8[u] = sx * 8.f;
+    }
+    auto consume = [&](const u32x2(&qc)[UPL], const uint32_t(&sc)[UPL], int t) {
+        float a[RB] = {0.f, 0.f};
+#pragma unroll
+        for (int u = 0; u < UPL; u++) {
+            float s0 = 0.f, s1 = 0.f;  // two chains
+#pragma unroll
+            for (int j = 0; j < 2; j++) {
+                s0 = dot4_nibbles(qc[u][j] & 0x0F0F0F0Fu, &xlo[u][4 * j], s0);
+                s1 = dot4_nibbles((qc[u][j] >> 4) & 0x0F0F0F0Fu, &xhi[u][4 * j], s1);
+            }
+            const float v = f16_bits_to_f32((uint16_t)sc[u]) * ((s0 + s1) - sx8[u]);
+#pragma unroll
+            for (int r = 0; r < RB; r++) a[r] += urow[u] == r ? v : 0.f;
+        }
+        // wave sums of the two rows, the chains stepping side by side
+#pragma unroll
+        for (int r = 0; r < RB; r++) a[r] += dpp_move<0xB1, 0xF>(a[r], 0.f);
+#pragma unroll
+        for (int r = 0; r < RB; r++) a[r] += dpp_move<0x4E, 0xF>(a[r], 0.f);
+#pragma unroll
+        for (int r = 0; r < RB; r++) a[r] += dpp_move<0x141, 0xF>(a[r], 0.f);
+#pragma unroll
+        for (int r = 0; r < RB; r++) a[r] += dpp_move<0x140, 0xF>(a[r], 0.f);
+#pragma unroll
+        for (int r = 0; r < RB; r++) a[r] += dpp_move<0x142, 0xA>(a[r], 0.f);
+#pragma unroll
+        for (int r = 0; r < RB; r++) a[r] += dpp_move<0x143, 0xC>(a[r], 0.f);
+        // lane 63 holds the totals; it stores the rows
+#pragma unroll
+        for (int r = 0; r < RB; r++)
+            if (lane == WAVE - 1 && t * RB + r < N) out[(size_t)t * RB + r] = a[r];
+    };
+    // steady state: every buffer is multiplied and asked for again, D trips on, with no condition in the way
+    // (every wait then knows how many loads are behind the ones it needs)
+    while (trip + (2 * D - 1) * nwaves < ntrips) {
+#pragma unroll
+        for (int d = 0; d < D; d++) {
+            consume(qn[d], sn[d], trip + d * nwaves);
+            request(qn[d], sn[d], trip + (D + d) * nwaves);
+        }
+        trip += D * nwaves;
+    }
+    // what the buffers still hold, then at most D - 1 trips behind them
+#pragma unroll
+    for (int d = 0; d < D; d++)
+        if (trip + d * nwaves < ntrips) consume(qn[d], sn[d], trip + d * nwaves);
+    trip += D * nwaves;
+#pragma unroll
+    for (int d = 0; d < D; d++)
+        if (trip + d * nwaves < ntrips) request(qn[d], sn[d], trip + d * nwaves);
+#pragma unroll
+    for (int d = 0; d < D; d++)
+        if (trip + d * nwaves < ntrips) consume(qn[d], sn[d], trip + d * nwaves);
+}
+
 // planes -> raw blocks (the inverse, for checks)
 template <int QT>
 __global__ __launch_bounds__(256) void unpack_planes_kernel(const uint8_t *__restrict__ quants, const uint16_t *__restrict__ scales,
@@ -423,6 +556,26 @@ int planes_launch(hm_ctx *ctx, const char *name, const float *d_x, const uint8_t
     const uint16_t *scales = reinterpret_cast<const uint16_t *>(d_planes + homura::quant_planes_scale_offset(q4, N, K));
     const int cpl = (K / 8 + WAVE - 1) / WAVE;
     const bool fused = fuse.x2 || fuse.res_in || fuse.norm_w || fuse.res_out_add || fuse.cand_v;
+    // Q4_0 at the LM-head shape: the half-block-per-lane kernel
+    const int nblk = K / 32;
+    if (q4 && !fused && nblk % 16 == 0 && nblk / 16 <= 4 && N >= 8 * PWAVES * ctx->num_cus) {
+        const int ntrips = (N + 1) / 2;
+        const int want = (ntrips + PWAVES - 1) / PWAVES;
+        const int grid = std::min(want, 4 * ctx->num_cus);  // four workgroups a CU (five fit: slower)
+        const size_t lds = (size_t)K * 4 + 16;
+        for (int m = 0; m < M; m++) {
+            const float *xm = d_x + (size_t)m * K;
+            float *om = d_out + (size_t)m * N;
+            switch (nblk / 16) {
+            case 1: hipLaunchKernelGGL((gemv_q4_0_halves_kernel<1>), dim3(grid), dim3(PTHREADS), lds, ctx->stream, xm, quants, scales, om, K, N); break;
+            case 2: hipLaunchKernelGGL((gemv_q4_0_halves_kernel<2>), dim3(grid), dim3(PTHREADS), lds, ctx->stream, xm, quants, scales, om, K, N); break;
+            case 3: hipLaunchKernelGGL((gemv_q4_0_halves_kernel<3>), dim3(grid), dim3(PTHREADS), lds, ctx->stream, xm, quants, scales, om, K, N); break;
+            default: hipLaunchKernelGGL((gemv_q4_0_halves_kernel<4>), dim3(grid), dim3(PTHREADS), lds, ctx->stream, xm, quants, scales, om, K, N); break;
+            }
+            HM_LAUNCH_CHECK(ctx);
+        }
+        return HM_OK;
+    }
     for (int m = 0; m < M; m++) {
         const float *xm = d_x + (size_t)m * K;
         float *om = d_out + (size_t)m * N;
