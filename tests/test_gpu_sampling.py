@@ -70,6 +70,35 @@ def test_device_sampler_against_oracle(ctx, name, vocab):
     assert compared >= 24
 
 
+@pytest.mark.parametrize("vocab,top_k", [(5000, 64), (4096, 33), (151936, 7)])
+def test_two_launch_sampler_with_ties_and_masked_logits(ctx, vocab, top_k):
+    """The front / back pair (top_k <= 64, vocabulary >= 4096) where its selection is hardest: logits on a
+    coarse grid, so that the top_k-th value is shared by many tokens spread over the front workgroups (the
+    lowest token numbers must win, as in the oracle's stable order), a run of -inf logits, a last block that
+    is not full, and top_k at the limit."""
+    gen = np.random.default_rng(vocab * 131 + top_k)
+    cfg = Cfg(temperature=0.9, top_k=top_k, top_p=0.98, min_p=0.0, repetition_penalty=1.0)
+    compared = skipped = 0
+    for trial in range(8):
+        logits = (np.round(gen.standard_normal(vocab) * 4.0) * 0.5).astype(np.float32)   # steps of 0.5: heavy ties
+        logits[gen.integers(0, vocab, vocab // 10)] = -np.inf
+        if trial % 2:
+            logits[-3:] = logits.max()            # ties at the very end of the partial block
+        d = ctx.to_device(logits)
+        a, b = pyoracle.Rng(50 + trial), runtime.Rng(50 + trial)
+        for _ in range(4):
+            want, margins = pyoracle.sample_token(logits, cfg, [], a, want_margins=True)
+            got = ctx.sample_token(d, vocab, lib_cfg(cfg), [], b)
+            if on_edge(margins, cfg):
+                skipped += 1
+                continue
+            assert got == want, (vocab, top_k, trial)
+            compared += 1
+        d.free()
+    say(f"ties, vocab {vocab}, top_k {top_k}: {compared} draws identical, {skipped} on a boundary")
+    assert compared >= 16
+
+
 def test_device_sampler_reference_cases_and_errors(ctx):
     # sample_token_greedy and min_p_filters_low_prob (src/generate.rs:891-900, :990-1008)
     d = ctx.to_device(np.array([0.0, 1.0, 0.5, 0.2], np.float32))
