@@ -477,6 +477,42 @@ def test_gqa_decode_attn(ctx, oracle, B, H, kvh, hd, max_len, kv_len):
         buf.free()
 
 
+@pytest.mark.parametrize("rising", [True, False])
+def test_long_cache_attention_with_scores_that_keep_moving_the_maximum(ctx, oracle, rising):
+    """The stepping kernel moves a wavefront's softmax reference point only when a score exceeds it by a
+    margin, and rescales its sums and accumulators then. Random keys never do that after the first step; here
+    the scores climb (or fall) by tens over every workgroup's rows, several margins from one step to the next, so the rescaling, the
+    exponentials far below the reference point and the merge of wavefronts with very different reference
+    points all carry weight in the result."""
+    B, H, kvh, hd, L = 8, 12, 2, 128, 4096   # 16 (sequence, kv head) pairs x 4096 rows: 256 rows a workgroup, two steps
+    q = synth.normal_f32(71, B * H * hd).reshape(B, H, hd)
+    kf = synth.bf16_to_f32(synth.normal_bf16(72, B * kvh * L * hd)).reshape(B, kvh, L, hd) * 0.05
+    ramp = (np.arange(L) % 256).astype(np.float32) / 256.0   # a sawtooth: the climb repeats inside every workgroup's rows
+    if not rising:
+        ramp = 1.0 - ramp
+    for b in range(B):
+        for k in range(kvh):
+            direction = q[b, k * (H // kvh)] / np.linalg.norm(q[b, k * (H // kvh)])   # the first head of the group
+            kf[b, k] += np.outer(ramp * 60.0, direction)
+    kb = synth.f32_to_bf16_rne(kf.reshape(-1)).reshape(B, kvh, L, hd)
+    vb = synth.normal_bf16(73, B * kvh * L * hd).reshape(B, kvh, L, hd)
+    scale = 1.0 / math.sqrt(hd)
+    dq, dk, dv, dout = ctx.to_device(q), ctx.to_device(kb), ctx.to_device(vb), ctx.empty(B * H * hd)
+    ctx.gqa_decode_attn(dq, dk, dv, dout, B, H, kvh, hd, L, L, scale)
+    got = dout.download(np.float32, (B, H * hd))
+    mask = np.zeros((1, L), np.float32)
+    spread = 0.0
+    for b in range(B):
+        want = oracle.gqa_attention(q[b:b + 1], synth.bf16_to_f32(kb[b]), synth.bf16_to_f32(vb[b]), mask)
+        assert rel_err(got[b], want) < TOL, f"sequence {b}"
+        s = (synth.bf16_to_f32(kb[b, 0]) @ q[b, 0]) * scale
+        spread = max(spread, float(s.max() - s.min()))
+    say(f"long-cache attention, scores {'rising' if rising else 'falling'} over a range of {spread:.0f}: within tolerance")
+    assert spread > 30
+    for buf in (dq, dk, dv, dout):
+        buf.free()
+
+
 def test_attention_uniform_keys_give_mean_of_values(ctx):
     B, H, kvh, hd, L = 1, 4, 2, 128, 200
     q = synth.normal_f32(1, H * hd)
