@@ -59,11 +59,12 @@ struct FusedDecodeArgs {
 constexpr int FUSED_TRACE_PER_LAYER = 11;
 constexpr int FUSED_TRACE_WGS = 256;  // rows of the trace buffer (the largest grid of any instance)
 
-// Whether a kernel instance exists for this shape on this device; max_seq_len rows must fit the
-// attention phase's register-resident splits. `why` receives a short reason when not.
+// Whether a kernel instance exists for this shape on this device (the cache may be of any length; a step is
+// served while its live rows, the new one included, are at most decode_fused_max_kv). `why` receives a short
+// reason when not.
 bool decode_fused_supported(const hm_ctx *ctx, const FusedShape &s, int n_layers, int max_seq_len, const char **why);
 size_t decode_fused_xch_bytes(const FusedShape &s);
-// Largest cache length the attention phase serves for this shape (0 if unsupported)
+// Most live cache rows (the new one included) the attention phase serves for this shape (0 if unsupported)
 int decode_fused_max_kv(const FusedShape &s);
 int decode_fused_launch(hm_ctx *ctx, const FusedShape &s, const FusedDecodeArgs &a);
 // Reads the sticky status word (synchronises the stream). HM_OK or HM_ERR_HIP with a message.

@@ -1264,6 +1264,13 @@ __global__ __launch_bounds__(FT) void decode_fused_kernel(FusedDecodeArgs a) {
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);
     const int wg = blockIdx.x;
     const int pos = a.state->pos;
+    // The attention phase keeps a split's rows in registers: more live rows than MAX_KV are not served. The
+    // host takes the other path through the layers from there on; should a launch get here all the same,
+    // every workgroup leaves at once (they all read the same position) and the status word says why.
+    if (pos + 1 > GE::MAX_KV || pos + 1 > a.max_len) {
+        if (wg == 0 && threadIdx.x == 0) atomicCAS(a.ctl + 1, 0u, 0x80000000u | 0xFu);
+        return;
+    }
     {
         static_assert(sizeof(FusedLayerPtrs) % 8 == 0, "the table is copied in 8-byte words");
         const uint64_t *src = reinterpret_cast<const uint64_t *>(a.layers);
@@ -1341,10 +1348,7 @@ bool decode_fused_supported(const hm_ctx *ctx, const FusedShape &s, int n_layers
         *why = "no kernel instance for this shape and weight format";
         return false;
     }
-    if (max_seq_len > i->max_kv) {
-        *why = "cache longer than the attention phase keeps in registers";
-        return false;
-    }
+    (void)max_seq_len;  // any cache length: what is limited is the number of live rows (decode_fused_max_kv)
     if (ctx->num_cus < i->nwg) {
         *why = "fewer compute units than resident workgroups";
         return false;
@@ -1365,7 +1369,7 @@ int decode_fused_launch(hm_ctx *ctx, const FusedShape &s, const FusedDecodeArgs 
     if (!i) return hm_set_error(ctx, HM_ERR_INVALID, "decode_fused: no kernel instance for this shape and weight format");
     HM_REQUIRE(ctx, !a.head_w || (a.head_norm && a.logits && a.state_rw && a.out_tokens && i->wf == FUSED_WF_BF16),
                "decode_fused: the LM head needs its norm weights, a logits row, the cursor and the token list (bf16 instances only)");
-    HM_REQUIRE(ctx, a.n_layers >= 1 && a.n_layers <= MAX_LAYERS && a.max_len >= 1 && a.max_len <= i->max_kv,
+    HM_REQUIRE(ctx, a.n_layers >= 1 && a.n_layers <= MAX_LAYERS && a.max_len >= 1,
                "decode_fused: %d layers / %d cache rows not served for this shape", a.n_layers, a.max_len);
     FusedDecodeArgs args = a;
     void *params[] = {&args};
@@ -1377,6 +1381,8 @@ int decode_fused_check(hm_ctx *ctx, const uint32_t *d_ctl) {
     uint32_t h[16] = {0};
     int rc = hm_download(ctx, h, d_ctl, sizeof(h));
     if (rc != HM_OK) return rc;
+    if (h[1] != 0 && (h[1] & 15u) == 15u)
+        return hm_set_error(ctx, HM_ERR_HIP, "decode_fused: launched with more live cache rows than the kernel serves (launch %u)", h[0]);
     if (h[1] != 0)
         return hm_set_error(ctx, HM_ERR_HIP,
                             "decode_fused: workgroup %u stopped waiting in phase %u of layer %u (launch %u)",

@@ -146,6 +146,8 @@ class HfModel {
     bool has_qk_norm_ = false;
     bool finalized_ = false;
     bool fused_available_ = false;
+    int fused_max_kv_ = 0;            // live cache rows (the new one included) a whole-step launch serves
+    bool whole_step_wanted_ = false;  // the caller's choice; the plan follows it while the cache is short enough
     int fused_wf_ = 0;  // FUSED_WF_* of the whole-step kernel instance
     bool fused_head_ = false;  // the whole-step launch also runs the LM head and the greedy pick (bf16 plan)
     const void *fused_table_kv_ = nullptr;  // key_ptr(0) the device layer table was built for

@@ -440,9 +440,19 @@ int HfModel::finalize(int max_seq_len) {
     rc = plan_->ensure_kv_cache(max_seq_len_);
     if (rc != HM_OK) return rc;
     if (fused_available_) {
-        plan_->set_pre_run([this]() { return refresh_fused_table(); });
+        const FusedShape fs{cfg_.hidden_size, cfg_.num_attention_heads, cfg_.kv_heads(), cfg_.head_dim(),
+                            cfg_.intermediate_size, fused_wf_};
+        fused_max_kv_ = decode_fused_max_kv(fs);
         const char *e = std::getenv("HOMURA_WHOLE_STEP");  // 0: keep one launch per projection
-        if (!(e && std::atoi(e) == 0) && (rc = plan_->set_whole_step(true)) != HM_OK) return rc;
+        whole_step_wanted_ = !(e && std::atoi(e) == 0);
+        // Before every step: the whole-step launch while the step's live rows (the cache and the new row) are
+        // within what its attention phase holds, one launch per projection beyond (a longer conversation
+        // changes over once; a cache reset changes back).
+        plan_->set_pre_run([this]() {
+            const int rc = plan_->set_whole_step(whole_step_wanted_ && plan_->kv_cache_len() + 1 <= fused_max_kv_);
+            return rc != HM_OK ? rc : refresh_fused_table();
+        });
+        if (whole_step_wanted_ && (rc = plan_->set_whole_step(true)) != HM_OK) return rc;
     }
     ids_view_ = Buffer::view(plan_->forced_ids(), (size_t)plan_->out_capacity() * 4, {1, DIM_DYNAMIC},
                              {1, 1}, DType::I64);
@@ -1539,7 +1549,8 @@ int HfModel::set_whole_step(bool on) {
     if (!finalized_) return hm_set_error(ctx_, HM_ERR_STATE, "model not finalized");
     if (on && !fused_available_)
         return hm_set_error(ctx_, HM_ERR_INVALID, "whole-step decode is not available for this model (bf16 weights and a served shape are needed)");
-    return plan_->set_whole_step(on);
+    whole_step_wanted_ = on;
+    return plan_->set_whole_step(on && plan_->kv_cache_len() + 1 <= fused_max_kv_);
 }
 
 int HfModel::whole_step_status() {

@@ -229,9 +229,46 @@ def test_unserved_shapes_keep_the_per_projection_path(ctx):
         gm.set_whole_step(True)
     gm.whole_step_status()
     gm.close()
-    # a served shape whose cache is longer than the attention phase keeps in registers
-    cfg2 = dataclasses.replace(synth_model.SMALL_WS, max_position_embeddings=4096)
-    w2 = synth_model.synth_weights(cfg2, 1)
-    gm2 = synth_model.build_model(ctx, cfg2, w2, 4096)
-    assert not gm2.whole_step_available()
-    gm2.close()
+
+
+def test_cache_longer_than_the_kernel_serves_changes_over_and_back(ctx):
+    """The whole-step launch holds a split's cache rows in registers: 2048 live rows for this shape. A model
+    with a longer cache starts on it, takes one launch per projection once a step's live rows exceed that,
+    and comes back after a cache reset; the steps on either side of the change give the oracle's logits and
+    the per-projection path's tokens."""
+    cfg = dataclasses.replace(synth_model.SMALL_WS, max_position_embeddings=4096)
+    weights = synth_model.synth_weights(cfg, 31)
+    gm = synth_model.build_model(ctx, cfg, weights, 2400)
+    plain = synth_model.build_model(ctx, cfg, weights, 2400)
+    plain.set_whole_step(False)
+    om = mf.build_oracle_model(cfg, weights, 2400)
+    assert gm.whole_step_available() and gm.whole_step() and gm.launches_per_step() == 1
+    rows = 2040
+    kv = synth_model.synth_kv(cfg, 32, rows)
+    for m in (gm, plain):
+        m.set_prefill_min(0)
+        m.init_kv_cache(kv, rows)
+    mf.oracle_init_kv(om, kv)
+    ids = synth.token_ids(33, 14, cfg.vocab_size)
+    got = gm.run_kv(ids)                      # positions 2040 .. 2053: the change comes after position 2047
+    gm.whole_step_status()
+    want = np.concatenate([om.run_kv(ids[i:i + 1]) for i in range(14)])
+    for i in range(14):
+        assert mf.rel_err(got[i], want[i]) < 1e-2, f"position {rows + i}"
+    assert gm.kv_cache_len() == rows + 14 and not gm.whole_step() and gm.launches_per_step() > 3
+    plain.run_kv(ids)
+    a, b = gm.generate_greedy(ids[:1], 12), plain.generate_greedy(ids[:1], 12)
+    assert np.array_equal(a, b)
+    # a device-resident run across the border: 2030 cached rows, 40 steps
+    for m in (gm, plain):
+        m.init_kv_cache(synth_model.synth_kv(cfg, 34, 2030), 2030)
+    a, b = gm.generate_greedy(ids[:1], 2), plain.generate_greedy(ids[:1], 2)   # the path is chosen step by step
+    assert np.array_equal(a, b) and gm.whole_step()
+    a, b = gm.generate_greedy(ids[:3], 40), plain.generate_greedy(ids[:3], 40)
+    gm.whole_step_status()
+    assert np.array_equal(a, b) and not gm.whole_step()
+    gm.reset_kv_cache()
+    gm.run_kv(ids[:2])
+    assert gm.whole_step()
+    gm.close()
+    plain.close()
