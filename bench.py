@@ -1,6 +1,6 @@
 #!/usr/bin/env python3
 """Decode benchmark: tokens/s of batch-1 greedy decode on the Qwen3-0.6B-shaped model
-(BASELINE configuration 2: 28 layers, hidden 1024, 16/8 heads, head_dim 128, SwiGLU 3072,
+(benchmark configuration 2: 28 layers, hidden 1024, 16/8 heads, head_dim 128, SwiGLU 3072,
 vocab 151936, tied bf16 LM head; KV cache pre-filled to 1024 rows; synthetic seeded weights).
 
 A "step" is one decode token: embed -> 28 x (QKV+QK-norm+RoPE+append, attention+O, MLP) -> LM head
@@ -95,7 +95,7 @@ def main() -> int:
     ap.add_argument("--no-prefill", action="store_true", help="skip the prompt-pass measurement")
     ap.add_argument("--no-quantised", action="store_true", help="skip the decode measurements with quantised projections")
     ap.add_argument("--no-kernel-configs", action="store_true",
-                    help="skip the stand-alone kernel measurements (BASELINE configurations 1, 3, 4, 5)")
+                    help="skip the stand-alone kernel measurements (benchmark configurations 1, 3, 4, 5)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this build runs on one GPU only (got --gpus {args.gpus}); "

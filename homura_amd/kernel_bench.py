@@ -1,4 +1,4 @@
-"""Roofline timing of the kernel-level entry points at the BASELINE shapes (configurations
+"""Roofline timing of the kernel-level entry points at the benchmark shapes (configurations
 1, 3, 4, 5a, 5b). Every kernel is launched over a ring of weight copies larger than the last-
 level caches (Infinity Cache 256 MiB), all launches recorded into one HIP graph and replayed
 between two HIP events on the launch stream, so the numbers are cold-cache per-launch times;

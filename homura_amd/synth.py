@@ -1,7 +1,7 @@
 """Deterministic synthetic tensors (numpy views of the library's host-side generator).
 
 Same bits on every platform: the generator is integer arithmetic (see csrc/synth.cpp).
-Seeds used by the BASELINE configurations live here so tests and bench agree.
+Seeds used by the benchmark configurations live here so tests and bench agree.
 """
 from __future__ import annotations
 

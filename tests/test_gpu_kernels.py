@@ -28,7 +28,7 @@ def say(msg):
 
 # ── bf16 GEMV (reference emit_matmul with bf16 weights) ───────────────────────
 
-@pytest.mark.parametrize("M,K,N", [(1, 896, 4864),   # BASELINE config 1
+@pytest.mark.parametrize("M,K,N", [(1, 896, 4864),   # benchmark configuration 1
                                    (1, 1024, 4096), (1, 3072, 1024), (1, 2048, 1024),
                                    (3, 896, 4864), (5, 1024, 1024), (8, 256, 136),
                                    (1, 40, 12), (2, 8, 8)])
@@ -103,8 +103,8 @@ def test_q8_0_reference_kat(ctx, golden):
     assert np.all(dout.download(np.float32) == g["expected_each"])
 
 
-@pytest.mark.parametrize("kind,M,K,N", [("q8_0", 1, 2048, 5632),    # BASELINE config 3
-                                        ("q4_0", 1, 1536, 151936),  # BASELINE config 4
+@pytest.mark.parametrize("kind,M,K,N", [("q8_0", 1, 2048, 5632),    # benchmark configuration 3
+                                        ("q4_0", 1, 1536, 151936),  # benchmark configuration 4
                                         ("q8_0", 1, 2048, 2048), ("q8_0", 1, 5632, 2048),
                                         ("q8_0", 2, 4096, 77), ("q8_0", 1, 32, 5), ("q8_0", 1, 96, 1),
                                         ("q4_0", 3, 2048, 260), ("q4_0", 1, 32, 7), ("q4_0", 1, 8960, 64),
@@ -168,8 +168,8 @@ def test_quant_planes_hold_the_blocks_bit_for_bit(ctx, oracle, kind):
         b.free()
 
 
-@pytest.mark.parametrize("kind,M,K,N", [("q8_0", 1, 2048, 5632),    # BASELINE config 3
-                                        ("q4_0", 1, 1536, 151936),  # BASELINE config 4
+@pytest.mark.parametrize("kind,M,K,N", [("q8_0", 1, 2048, 5632),    # benchmark configuration 3
+                                        ("q4_0", 1, 1536, 151936),  # benchmark configuration 4
                                         ("q8_0", 1, 1024, 151936),  # an LM head read from Q8_0 blocks
                                         ("q8_0", 1, 2048, 2048), ("q8_0", 1, 3072, 1024), ("q8_0", 2, 4096, 77),
                                         ("q8_0", 1, 32, 5), ("q8_0", 1, 96, 1), ("q8_0", 1, 1024, 6144),
@@ -268,7 +268,7 @@ def test_gemv_kquant(ctx, oracle, kind, M, K, N):
 # ── prefill GEMM (MFMA) ───────────────────────────────────────────────────────
 
 @pytest.mark.parametrize("layout", ["kn", "nk"])
-@pytest.mark.parametrize("M,K,N", [(512, 2048, 8192),  # BASELINE config 5a
+@pytest.mark.parametrize("M,K,N", [(512, 2048, 8192),  # benchmark configuration 5a
                                    (128, 32, 128), (256, 96, 384), (384, 64, 1152), (128, 160, 1024)])
 def test_gemm_bf16_mfma(ctx, oracle, M, K, N, layout):
     say(f"gemm_bf16 M={M} K={K} N={N} B layout {layout}")
@@ -445,7 +445,7 @@ def test_kv_append_rounds_to_nearest_even(ctx, oracle):
 
 
 @pytest.mark.parametrize("B,H,kvh,hd,max_len,kv_len", [
-    (8, 12, 2, 128, 4096, 4096),   # BASELINE config 5b
+    (8, 12, 2, 128, 4096, 4096),   # benchmark configuration 5b
     (1, 16, 8, 128, 2048, 1025),   # Qwen3-0.6B decode shape
     (1, 16, 8, 128, 1152, 1),      # first token
     (2, 14, 2, 64, 300, 33),       # Qwen2.5-0.5B heads (g = 7), ragged length

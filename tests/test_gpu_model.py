@@ -118,7 +118,7 @@ def test_weight_slot_listing_matches_reference_order(tiny):
 
 
 def test_qwen3_0p6b_decode_token_identical(ctx):
-    """BASELINE configuration 2: 28-layer Qwen3-0.6B shape, cache pre-filled to 1024 rows,
+    """benchmark configuration 2: 28-layer Qwen3-0.6B shape, cache pre-filled to 1024 rows,
     32 prompt ids, 64 greedy tokens: GPU tokens == oracle tokens == committed fixture."""
     fx = json.loads((GOLDEN / "qwen3_0p6b_decode.json").read_text())
     cfg = synth_model.QWEN3_0P6B
