@@ -66,6 +66,12 @@ bool decode_fused_supported(const hm_ctx *ctx, const FusedShape &s, int n_layers
 size_t decode_fused_xch_bytes(const FusedShape &s);
 // Most live cache rows (the new one included) the attention phase serves for this shape (0 if unsupported)
 int decode_fused_max_kv(const FusedShape &s);
-int decode_fused_launch(hm_ctx *ctx, const FusedShape &s, const FusedDecodeArgs &a);
+// The instances of a shape differ in how many live rows they hold (the ones that hold fewer are faster): the
+// capacity of the instance that a step with `live_rows` live rows takes, 0 if none serves it. A recorded
+// launch stays good while this value does not change.
+int decode_fused_tier(const FusedShape &s, int live_rows);
+// live_rows: the cache rows of the step, the new one included (the host's count; the kernel reads the position
+// from the cursor and leaves with a status code if it does not fit the instance).
+int decode_fused_launch(hm_ctx *ctx, const FusedShape &s, const FusedDecodeArgs &a, int live_rows);
 // Reads the sticky status word (synchronises the stream). HM_OK or HM_ERR_HIP with a message.
 int decode_fused_check(hm_ctx *ctx, const uint32_t *d_ctl);

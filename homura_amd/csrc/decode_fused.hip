@@ -39,7 +39,7 @@ constexpr int CT = 256;     // communicating threads
 constexpr int SPIN_MAX = 1 << 20;
 constexpr int MAX_LAYERS = 64;
 
-template <int HIDDEN_, int H_, int KVH_, int HD_, int INTER_, int NWG_>
+template <int HIDDEN_, int H_, int KVH_, int HD_, int INTER_, int NWG_, int NR_ = 4>
 struct Geo {
     static constexpr int HIDDEN = HIDDEN_, H = H_, KVH = KVH_, HD = HD_, INTER = INTER_, NWG = NWG_;
     static constexpr int G = H / KVH, QD = H * HD, KVD = KVH * HD, NQKV = QD + 2 * KVD;
@@ -49,7 +49,7 @@ struct Geo {
     static constexpr int RG = 2 * INTER / NWG, RGW = RG / NCW; // gate|up rows (interleaved pairs)
     static constexpr int APW = INTER / NWG;                    // SiLU*up values per workgroup
     static constexpr int SPH = NWG / KVH;                      // cache splits per KV head
-    static constexpr int NR = 4;                               // row rounds a wavefront keeps in registers
+    static constexpr int NR = NR_;                             // row rounds a wavefront keeps in registers
     static constexpr int LPR = HD / 8, RPI = WAVE / LPR;       // lanes per cache row, rows per load
     static constexpr int MAX_KV = SPH * NR * NCW * RPI;
     static constexpr int FPW = QD / NWG;                       // folded attention outputs per workgroup
@@ -1292,6 +1292,11 @@ __global__ __launch_bounds__(FT) void decode_fused_kernel(FusedDecodeArgs a) {
 using GeoQwen3_0p6b = Geo<1024, 16, 8, 128, 3072, 256>;
 using GeoSmall = Geo<512, 4, 2, 128, 1024, 64>;
 using GeoSmallQ = Geo<1024, 8, 4, 128, 1024, 64>;
+// The same shapes with eight row rounds: twice the live cache rows (4096) for 32 more registers a lane and an
+// attention phase twice as long; taken only by steps that the four-round instances do not serve.
+using GeoQwen3_0p6bLong = Geo<1024, 16, 8, 128, 3072, 256, 8>;
+using GeoSmallLong = Geo<512, 4, 2, 128, 1024, 64, 8>;
+using GeoSmallQLong = Geo<1024, 8, 4, 128, 1024, 64, 8>;
 
 template <class GE>
 bool shape_is(const FusedShape &s) {
@@ -1312,20 +1317,33 @@ Instance instance() {
                     reinterpret_cast<const void *>(&decode_fused_kernel<GE, WF>)};
 }
 
-const Instance *find_instance(const FusedShape &s) {
+// The first instance of the shape and format that holds `live_rows` cache rows (the short ones come first); with
+// live_rows = 0, the one that holds the most.
+const Instance *find_instance(const FusedShape &s, int live_rows = 1) {
     static const Instance table[] = {
         instance<GeoQwen3_0p6b, FUSED_WF_BF16>(), instance<GeoQwen3_0p6b, FUSED_WF_Q8_0>(), instance<GeoQwen3_0p6b, FUSED_WF_Q4_0>(),
         instance<GeoSmall, FUSED_WF_BF16>(),      instance<GeoSmallQ, FUSED_WF_Q8_0>(),     instance<GeoSmallQ, FUSED_WF_Q4_0>(),
+        instance<GeoQwen3_0p6bLong, FUSED_WF_BF16>(), instance<GeoQwen3_0p6bLong, FUSED_WF_Q8_0>(), instance<GeoQwen3_0p6bLong, FUSED_WF_Q4_0>(),
+        instance<GeoSmallLong, FUSED_WF_BF16>(),      instance<GeoSmallQLong, FUSED_WF_Q8_0>(),     instance<GeoSmallQLong, FUSED_WF_Q4_0>(),
     };
-    for (const Instance &i : table)
-        if (i.wf == s.wf && i.matches(s)) return &i;
-    return nullptr;
+    const Instance *most = nullptr;
+    for (const Instance &i : table) {
+        if (i.wf != s.wf || !i.matches(s)) continue;
+        if (live_rows > 0 && i.max_kv >= live_rows) return &i;
+        if (!most || i.max_kv > most->max_kv) most = &i;
+    }
+    return live_rows > 0 ? nullptr : most;
 }
 
 }  // namespace
 
 int decode_fused_max_kv(const FusedShape &s) {
-    const Instance *i = find_instance(s);
+    const Instance *i = find_instance(s, 0);
+    return i ? i->max_kv : 0;
+}
+
+int decode_fused_tier(const FusedShape &s, int live_rows) {
+    const Instance *i = find_instance(s, live_rows);
     return i ? i->max_kv : 0;
 }
 
@@ -1362,11 +1380,11 @@ bool decode_fused_supported(const hm_ctx *ctx, const FusedShape &s, int n_layers
     return true;
 }
 
-int decode_fused_launch(hm_ctx *ctx, const FusedShape &s, const FusedDecodeArgs &a) {
+int decode_fused_launch(hm_ctx *ctx, const FusedShape &s, const FusedDecodeArgs &a, int live_rows) {
     HM_REQUIRE(ctx, a.layers && a.embed && a.state && a.forced && a.hidden_out && a.cos_tab && a.sin_tab && a.xch && a.ctl,
                "decode_fused: NULL pointer");
-    const Instance *i = find_instance(s);
-    if (!i) return hm_set_error(ctx, HM_ERR_INVALID, "decode_fused: no kernel instance for this shape and weight format");
+    const Instance *i = find_instance(s, live_rows < 1 ? 1 : live_rows);
+    if (!i) return hm_set_error(ctx, HM_ERR_INVALID, "decode_fused: no kernel instance for this shape, weight format and %d live cache rows", live_rows);
     HM_REQUIRE(ctx, !a.head_w || (a.head_norm && a.logits && a.state_rw && a.out_tokens && i->wf == FUSED_WF_BF16),
                "decode_fused: the LM head needs its norm weights, a logits row, the cursor and the token list (bf16 instances only)");
     HM_REQUIRE(ctx, a.n_layers >= 1 && a.n_layers <= MAX_LAYERS && a.max_len >= 1,

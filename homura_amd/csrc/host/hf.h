@@ -147,6 +147,7 @@ class HfModel {
     bool finalized_ = false;
     bool fused_available_ = false;
     int fused_max_kv_ = 0;            // live cache rows (the new one included) a whole-step launch serves
+    int fused_tier_ = 0;              // capacity of the kernel instance the recorded step launches
     bool whole_step_wanted_ = false;  // the caller's choice; the plan follows it while the cache is short enough
     int fused_wf_ = 0;  // FUSED_WF_* of the whole-step kernel instance
     bool fused_head_ = false;  // the whole-step launch also runs the LM head and the greedy pick (bf16 plan)

@@ -448,8 +448,14 @@ int HfModel::finalize(int max_seq_len) {
         // Before every step: the whole-step launch while the step's live rows (the cache and the new row) are
         // within what its attention phase holds, one launch per projection beyond (a longer conversation
         // changes over once; a cache reset changes back).
-        plan_->set_pre_run([this]() {
-            const int rc = plan_->set_whole_step(whole_step_wanted_ && plan_->kv_cache_len() + 1 <= fused_max_kv_);
+        plan_->set_pre_run([this, fs]() {
+            const int live = plan_->kv_cache_len() + 1;
+            const int tier = decode_fused_tier(fs, live);  // 0: no instance holds that many rows
+            int rc = plan_->set_whole_step(whole_step_wanted_ && tier > 0);
+            if (rc == HM_OK && plan_->whole_step() && tier != fused_tier_) {
+                rc = plan_->invalidate_graph();  // the recorded launch is another instance's
+                fused_tier_ = tier;
+            }
             return rc != HM_OK ? rc : refresh_fused_table();
         });
         if (whole_step_wanted_ && (rc = plan_->set_whole_step(true)) != HM_OK) return rc;
@@ -620,7 +626,7 @@ int HfModel::emit_transformer_plan() {
                     fa.out_cap = sc.plan->out_capacity();
                     fa.advance = sc.timing ? 0 : 1;
                 }
-                return decode_fused_launch(sc.ctx, fs, fa);
+                return decode_fused_launch(sc.ctx, fs, fa, sc.plan->kv_cache_len() + 1);
             };
             k.launches.push_back(std::move(f));
         }
@@ -1149,7 +1155,7 @@ int HfModel::emit_transformer_plan_quant() {
                 fa.xch = scr->fused_xch.as<unsigned char>();
                 fa.ctl = scr->fused_ctl.as<uint32_t>();
                 fa.trace = scr->fused_trace ? scr->fused_trace.as<unsigned long long>() : nullptr;
-                return decode_fused_launch(sc.ctx, fshape, fa);
+                return decode_fused_launch(sc.ctx, fshape, fa, sc.plan->kv_cache_len() + 1);
             };
             k.launches.push_back(std::move(f));
         }

@@ -228,6 +228,8 @@ class ExecutionPlan {
     // Take the whole-step launch (when the plan has one) instead of the per-projection launches.
     int set_whole_step(bool on);
     bool whole_step() const { return whole_step_; }
+    // Forget the recorded step (its launches' arguments or kernels are about to change); the next run records anew.
+    int invalidate_graph();
     bool skips(const DeviceLaunch &l) const {
         return l.mode == (whole_step_ ? DeviceLaunch::Mode::PerKernel : DeviceLaunch::Mode::WholeStep);
     }

@@ -459,7 +459,11 @@ int ExecutionPlan::enable_graph(bool on) {
 int ExecutionPlan::set_whole_step(bool on) {
     if (on == whole_step_) return HM_OK;
     whole_step_ = on;
-    if (graph_exec_) {  // the captured step took the other way through the layers
+    return invalidate_graph();  // the captured step took the other way through the layers
+}
+
+int ExecutionPlan::invalidate_graph() {
+    if (graph_exec_) {
         HM_HIP(ctx_, hipStreamSynchronize(ctx_->stream));
         (void)hipGraphExecDestroy(graph_exec_);
         graph_exec_ = nullptr;

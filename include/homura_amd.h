@@ -353,8 +353,9 @@ int hm_model_set_graph(hm_model *m, int on);
  * launch per projection; the reference dispatches 1 + 3 * layers + 1 kernels per step
  * (src/hf/emitter.rs:1016-1021). Served for bf16, all-Q8_0 and all-Q4_0 models whose shape has a kernel
  * instance (hm_model_whole_step_available); on by default then, and for bf16 models the same launch runs the
- * LM head and the greedy pick. The cache may be of any length: a step whose live rows exceed what the launch
- * holds (2048) takes the per-projection path, chosen step by step. Results agree with the per-projection
+ * LM head and the greedy pick. The cache may be of any length: up to 2048 live rows a step takes the fastest
+ * instance of the kernel, up to 4096 one that holds twice the rows, beyond that the per-projection path,
+ * chosen step by step. Results agree with the per-projection
  * path to f32 summation order. hm_model_whole_step_status returns HM_OK, or the error
  * left behind by a step whose workgroups stopped waiting for one another (bounded waits; the
  * outputs of such a step are not valid). */

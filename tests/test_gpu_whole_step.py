@@ -232,41 +232,44 @@ def test_unserved_shapes_keep_the_per_projection_path(ctx):
 
 
 def test_cache_longer_than_the_kernel_serves_changes_over_and_back(ctx):
-    """The whole-step launch holds a split's cache rows in registers: 2048 live rows for this shape. A model
-    with a longer cache starts on it, takes one launch per projection once a step's live rows exceed that,
-    and comes back after a cache reset; the steps on either side of the change give the oracle's logits and
-    the per-projection path's tokens."""
-    cfg = dataclasses.replace(synth_model.SMALL_WS, max_position_embeddings=4096)
+    """The whole-step launch holds a split's cache rows in registers: an instance with four row rounds serves
+    2048 live rows of this shape, one with eight 4096. A model with a longer cache starts on the first, takes
+    the second from the step whose live rows exceed 2048, one launch per projection beyond 4096, and comes
+    back after a cache reset; the steps on either side of each change give the oracle's logits and the
+    per-projection path's tokens."""
+    cfg = dataclasses.replace(synth_model.SMALL_WS, max_position_embeddings=8192)
     weights = synth_model.synth_weights(cfg, 31)
-    gm = synth_model.build_model(ctx, cfg, weights, 2400)
-    plain = synth_model.build_model(ctx, cfg, weights, 2400)
+    L = 4200
+    gm = synth_model.build_model(ctx, cfg, weights, L)
+    plain = synth_model.build_model(ctx, cfg, weights, L)
     plain.set_whole_step(False)
-    om = mf.build_oracle_model(cfg, weights, 2400)
+    om = mf.build_oracle_model(cfg, weights, L)
     assert gm.whole_step_available() and gm.whole_step() and gm.launches_per_step() == 1
-    rows = 2040
-    kv = synth_model.synth_kv(cfg, 32, rows)
-    for m in (gm, plain):
-        m.set_prefill_min(0)
-        m.init_kv_cache(kv, rows)
-    mf.oracle_init_kv(om, kv)
     ids = synth.token_ids(33, 14, cfg.vocab_size)
-    got = gm.run_kv(ids)                      # positions 2040 .. 2053: the change comes after position 2047
-    gm.whole_step_status()
-    want = np.concatenate([om.run_kv(ids[i:i + 1]) for i in range(14)])
-    for i in range(14):
-        assert mf.rel_err(got[i], want[i]) < 1e-2, f"position {rows + i}"
-    assert gm.kv_cache_len() == rows + 14 and not gm.whole_step() and gm.launches_per_step() > 3
-    plain.run_kv(ids)
-    a, b = gm.generate_greedy(ids[:1], 12), plain.generate_greedy(ids[:1], 12)
-    assert np.array_equal(a, b)
-    # a device-resident run across the border: 2030 cached rows, 40 steps
-    for m in (gm, plain):
-        m.init_kv_cache(synth_model.synth_kv(cfg, 34, 2030), 2030)
-    a, b = gm.generate_greedy(ids[:1], 2), plain.generate_greedy(ids[:1], 2)   # the path is chosen step by step
-    assert np.array_equal(a, b) and gm.whole_step()
-    a, b = gm.generate_greedy(ids[:3], 40), plain.generate_greedy(ids[:3], 40)
-    gm.whole_step_status()
-    assert np.array_equal(a, b) and not gm.whole_step()
+    for rows, still_whole in ((2040, True), (4088, False)):
+        kv = synth_model.synth_kv(cfg, 32 + rows, rows)
+        for m in (gm, plain):
+            m.set_prefill_min(0)
+            m.init_kv_cache(kv, rows)
+        mf.oracle_init_kv(om, kv)
+        got = gm.run_kv(ids)                      # 14 positions across the border
+        gm.whole_step_status()
+        want = np.concatenate([om.run_kv(ids[i:i + 1]) for i in range(14)])
+        for i in range(14):
+            assert mf.rel_err(got[i], want[i]) < 1e-2, f"position {rows + i}"
+        assert gm.kv_cache_len() == rows + 14 and gm.whole_step() == still_whole
+        assert (gm.launches_per_step() == 1) == still_whole
+        plain.run_kv(ids)
+        a, b = gm.generate_greedy(ids[:1], 12), plain.generate_greedy(ids[:1], 12)
+        assert np.array_equal(a, b)
+        # a device-resident run across the same border
+        for m in (gm, plain):
+            m.init_kv_cache(synth_model.synth_kv(cfg, 34, rows - 10), rows - 10)
+        a, b = gm.generate_greedy(ids[:1], 2), plain.generate_greedy(ids[:1], 2)   # the path is chosen step by step
+        assert np.array_equal(a, b) and gm.whole_step()
+        a, b = gm.generate_greedy(ids[:3], 40), plain.generate_greedy(ids[:3], 40)
+        gm.whole_step_status()
+        assert np.array_equal(a, b) and gm.whole_step() == still_whole
     gm.reset_kv_cache()
     gm.run_kv(ids[:2])
     assert gm.whole_step()
