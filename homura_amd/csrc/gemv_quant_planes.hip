@@ -655,19 +655,22 @@ int homura::pack_quant_planes(hm_ctx *ctx, bool q4, const uint8_t *d_blocks, uin
 extern "C" {
 
 size_t hm_quant_planes_bytes(int hm_dtype, int N, int K) {
+    if (hm_dtype == HM_DTYPE_Q6_K) return N > 0 && K > 0 && K % 256 == 0 ? homura::q6k_planes_bytes(N, K) : 0;
     if ((hm_dtype != HM_DTYPE_Q8_0 && hm_dtype != HM_DTYPE_Q4_0) || N <= 0 || K <= 0 || K % 32 != 0) return 0;
     return homura::quant_planes_bytes(hm_dtype == HM_DTYPE_Q4_0, N, K);
 }
 
 int hm_pack_quant_planes(hm_ctx *ctx, int hm_dtype, const uint8_t *d_blocks, uint8_t *d_planes, int N, int K) {
     HM_CHECK_CTX(ctx);
-    HM_REQUIRE(ctx, hm_dtype == HM_DTYPE_Q8_0 || hm_dtype == HM_DTYPE_Q4_0, "hm_pack_quant_planes: dtype %d is not Q8_0 or Q4_0", hm_dtype);
+    if (hm_dtype == HM_DTYPE_Q6_K) return homura::pack_q6k_planes(ctx, d_blocks, d_planes, N, K, false);
+    HM_REQUIRE(ctx, hm_dtype == HM_DTYPE_Q8_0 || hm_dtype == HM_DTYPE_Q4_0, "hm_pack_quant_planes: dtype %d is not Q8_0, Q4_0 or Q6_K", hm_dtype);
     return homura::pack_quant_planes(ctx, hm_dtype == HM_DTYPE_Q4_0, d_blocks, d_planes, N, K);
 }
 
 int hm_unpack_quant_planes(hm_ctx *ctx, int hm_dtype, const uint8_t *d_planes, uint8_t *d_blocks, int N, int K) {
     HM_CHECK_CTX(ctx);
-    HM_REQUIRE(ctx, hm_dtype == HM_DTYPE_Q8_0 || hm_dtype == HM_DTYPE_Q4_0, "hm_unpack_quant_planes: dtype %d is not Q8_0 or Q4_0", hm_dtype);
+    if (hm_dtype == HM_DTYPE_Q6_K) return homura::pack_q6k_planes(ctx, d_blocks, const_cast<uint8_t *>(d_planes), N, K, true);
+    HM_REQUIRE(ctx, hm_dtype == HM_DTYPE_Q8_0 || hm_dtype == HM_DTYPE_Q4_0, "hm_unpack_quant_planes: dtype %d is not Q8_0, Q4_0 or Q6_K", hm_dtype);
     return hm_dtype == HM_DTYPE_Q4_0 ? pack_launch<1>(ctx, "hm_unpack_quant_planes", d_blocks, const_cast<uint8_t *>(d_planes), N, K, true)
                                      : pack_launch<0>(ctx, "hm_unpack_quant_planes", d_blocks, const_cast<uint8_t *>(d_planes), N, K, true);
 }
@@ -680,9 +683,14 @@ int hm_gemv_q4_0_planes(hm_ctx *ctx, const float *d_x, const uint8_t *d_planes, 
     return planes_launch<1>(ctx, "hm_gemv_q4_0_planes", d_x, d_planes, d_out, M, K, N, QuantFuse());
 }
 
+int hm_gemv_q6_k_f32_planes(hm_ctx *ctx, const float *d_x, const uint8_t *d_planes, float *d_out, int M, int K, int N) {
+    return homura::gemv_q6k_planes_f32(ctx, "hm_gemv_q6_k_f32_planes", d_x, nullptr, 0.f, d_planes, d_out, M, K, N, nullptr, nullptr, 0);
+}
+
 int hm_dequant_quant_planes(hm_ctx *ctx, int hm_dtype, const uint8_t *d_planes, float *d_out, int N, int K) {
     HM_CHECK_CTX(ctx);
-    HM_REQUIRE(ctx, hm_dtype == HM_DTYPE_Q8_0 || hm_dtype == HM_DTYPE_Q4_0, "hm_dequant_quant_planes: dtype %d is not Q8_0 or Q4_0", hm_dtype);
+    if (hm_dtype == HM_DTYPE_Q6_K) return homura::dequant_q6k_planes(ctx, d_planes, d_out, N, K);
+    HM_REQUIRE(ctx, hm_dtype == HM_DTYPE_Q8_0 || hm_dtype == HM_DTYPE_Q4_0, "hm_dequant_quant_planes: dtype %d is not Q8_0, Q4_0 or Q6_K", hm_dtype);
     HM_REQUIRE(ctx, d_planes && d_out && N > 0 && K > 0 && K % 32 == 0, "hm_dequant_quant_planes: bad arguments");
     const bool q4 = hm_dtype == HM_DTYPE_Q4_0;
     const size_t n = (size_t)N * K;

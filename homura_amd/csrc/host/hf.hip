@@ -171,6 +171,13 @@ int HfModel::build_quant_planes() {
         const int rc = pack_quant_planes(ctx_, q4, lm_head_blocks_.as<uint8_t>(), lm_head_planes_.as<uint8_t>(), cfg_.vocab_size, hidden);
         if (rc != HM_OK) return rc;
     }
+    if (lm_head_blocks_ && lm_head_blocks_dtype_ == DType::Q6_K && q6k_planes_shape_ok(cfg_.vocab_size, hidden)) {
+        const size_t bytes = q6k_planes_bytes(cfg_.vocab_size, hidden);
+        lm_head_planes_ = Buffer::alloc_bytes(ctx_, bytes, {(int64_t)bytes}, lm_head_blocks_dtype_);
+        if (!lm_head_planes_) return HM_ERR_OOM;
+        const int rc = pack_q6k_planes(ctx_, lm_head_blocks_.as<uint8_t>(), lm_head_planes_.as<uint8_t>(), cfg_.vocab_size, hidden, false);
+        if (rc != HM_OK) return rc;
+    }
     return hm_sync(ctx_);
 }
 
@@ -1379,6 +1386,10 @@ int HfModel::emit_transformer_plan_quant() {
                 return gemv_quant_fused(sc.ctx, head_dt == DType::Q4_0, sc.pool[in[0]]->as<float>(), sc.pool[in[2]]->as<uint8_t>(),
                                         sc.pool[sc.step.output_slots[0]]->as<float>(), (int)hidden, (int)vocab, f);
             }
+            if (head_q6 && head_planes)  // the same product over the re-packed output matrix
+                return gemv_q6k_planes_f32(sc.ctx, "gemv_q6_k_f32_planes[head]", sc.pool[in[0]]->as<float>(), sc.pool[in[1]]->as<float>(), eps,
+                                           head_planes, sc.pool[sc.step.output_slots[0]]->as<float>(), 1, (int)hidden, (int)vocab,
+                                           scr->cand_val.as<float>(), scr->cand_idx.as<int>(), scr->cand_cap);
             if (head_blocks)  // the f32 product with the dequantised output matrix, read from its blocks
                 return gemv_kquant_f32_head(sc.ctx, head_q6, sc.pool[in[0]]->as<float>(), sc.pool[in[1]]->as<float>(), eps,
                                             sc.pool[in[2]]->as<uint8_t>(), sc.pool[sc.step.output_slots[0]]->as<float>(),
@@ -1405,6 +1416,7 @@ int HfModel::emit_transformer_plan_quant() {
         h2.bytes_fixed = 64;
         h2.fn = [=](const StepContext &sc) -> int {
             const int ncand = !head_blocks ? std::min(gemv_bf16_nk_grid(sc.ctx, (int)vocab, 4), scr->cand_cap)
+                              : head_q6 && head_planes ? q6k_planes_workgroups(sc.ctx, (int)hidden, (int)vocab, scr->cand_cap)
                               : head_k ? gemv_kquant_f32_head_candidates(sc.ctx, head_q6, (int)hidden, (int)vocab, scr->cand_cap)
                               : head_planes ? gemv_planes_workgroups(sc.ctx, head_dt == DType::Q4_0, (int)hidden, (int)vocab)
                                        : gemv_quant_workgroups(sc.ctx, head_dt == DType::Q4_0, (int)hidden, (int)vocab);

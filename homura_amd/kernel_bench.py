@@ -109,6 +109,29 @@ def run_quant_cases(ctx: Context):
                           hot_us=hot))
         for b in planes + [x, o]:
             b.free()
+    out += run_q6_k_head_case(ctx)
+    return out
+
+
+def run_q6_k_head_case(ctx: Context):
+    """The f32 product of a Q6_K output matrix at the Qwen3-0.6B shape (the LM head of a Q4_K_M file),
+    on the raw blocks and on the planes the model keeps."""
+    from .runtime import DTYPE_Q6_K
+    K, N = 1024, 151936
+    x = ctx.to_device(synth.normal_f32(31, K))
+    ring = _ring(ctx, synth.q6_k_blocks(30, N * K // 256))
+    o = ctx.empty(N)
+    nbytes = N * (K // 256) * 210 + K * 4 + N * 4
+    name = "LM head gemv_q6_k_f32 1024->151936"
+    us = _time(ctx, [lambda b=b: ctx.gemv_q6_k_f32(x, b, o, 1, K, N) for b in ring])
+    out = [_entry(name, us, nbytes, note="raw GGUF blocks")]
+    planes = [ctx.pack_quant_planes(DTYPE_Q6_K, b, N, K) for b in ring]
+    for b in ring:
+        b.free()
+    us = _time(ctx, [lambda p=p: ctx.gemv_q6_k_f32_planes(x, p, o, 1, K, N) for p in planes])
+    out.append(_entry(name.replace(" gemv", " planes gemv"), us, nbytes, note="the same blocks re-packed into planes at upload"))
+    for b in planes + [x, o]:
+        b.free()
     return out
 
 

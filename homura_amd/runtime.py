@@ -176,6 +176,9 @@ class Context:
     def gemv_q4_0_planes(self, x, planes, out, M, K, N):
         self._check(self.lib.hm_gemv_q4_0_planes(self.h, x.ptr, planes.ptr, out.ptr, M, K, N))
 
+    def gemv_q6_k_f32_planes(self, x, planes, out, M, K, N):
+        self._check(self.lib.hm_gemv_q6_k_f32_planes(self.h, x.ptr, planes.ptr, out.ptr, M, K, N))
+
     def dequant_quant_planes(self, dtype, planes, out, N, K):
         self._check(self.lib.hm_dequant_quant_planes(self.h, dtype, planes.ptr, out.ptr, N, K))
 

@@ -108,7 +108,7 @@ int hm_gemv_q4_0(hm_ctx *ctx, const float *d_x, const uint8_t *d_w_blocks, float
  * multiple of 256 bytes, the f16 scales of all blocks row after row. The bytes are those of the GGUF blocks
  * (src/graph_builder/emit_quant.rs:17-21 layout) in another order: quant words sit at their natural
  * alignment and are loaded straight into registers. hm_quant_planes_bytes gives the size of the planes
- * of an [N][K] matrix (0 for a type other than HM_DTYPE_Q8_0 / Q4_0 or a bad shape), hm_pack_quant_planes
+ * of an [N][K] matrix (0 for a type other than HM_DTYPE_Q8_0 / Q4_0 / Q6_K or a bad shape), hm_pack_quant_planes
  * fills them from raw blocks [N][K/32] in one launch, hm_unpack_quant_planes is its inverse.
  * Results equal hm_gemv_q8_0 / hm_gemv_q4_0 up to the order of the f32 additions. M <= 8, K % 32 == 0,
  * K <= 4096. hm_dequant_quant_planes writes the N * K dequantised weights, bit-exact with the CPU. */
@@ -118,6 +118,16 @@ int hm_unpack_quant_planes(hm_ctx *ctx, int hm_dtype, const uint8_t *d_planes, u
 int hm_gemv_q8_0_planes(hm_ctx *ctx, const float *d_x, const uint8_t *d_planes, float *d_out, int M, int K, int N);
 int hm_gemv_q4_0_planes(hm_ctx *ctx, const float *d_x, const uint8_t *d_planes, float *d_out, int M, int K, int N);
 int hm_dequant_quant_planes(hm_ctx *ctx, int hm_dtype, const uint8_t *d_planes, float *d_out, int N, int K);
+
+/* Q6_K planes (the same four functions with HM_DTYPE_Q6_K; K % 256 == 0). A 210-byte block (src/gguf.rs:880-917)
+ * interleaves four 16-weight groups in every byte run; the unit that shares bytes is 64 weights (groups g, g + 2,
+ * g + 4, g + 6 of one 128-weight half, l in 0..15 or 16..31). The planes hold, for all units of all rows in
+ * order: [units][32] low nibbles (ql[64h + 16p + j], then ql[64h + 32 + 16p + j], j = 0..15), from the next
+ * multiple of 256 bytes [units][16] top bits (qh[32h + 16p + j]), then [units][4] int8 scales (sc[8h + p + 2g]),
+ * then [blocks] f16 d; unit 2h + p of a block. hm_gemv_q6_k_f32_planes is hm_gemv_q6_k_f32 over them
+ * (f32 row x dequantised weights, the product of a Q6_K LM head; results equal up to the order of the f32
+ * additions) for K = 256, 512, 1024, 2048 or 4096 and M <= 8. */
+int hm_gemv_q6_k_f32_planes(hm_ctx *ctx, const float *d_x, const uint8_t *d_planes, float *d_out, int M, int K, int N);
 
 /* Block dequantisation to f32, reference dequant_q8_0 (src/gguf.rs:817-831): one f32
  * multiply per element, bit-exact with the CPU. hm_dequant_q4_0 is its Q4_0 analogue. */

@@ -212,6 +212,76 @@ def test_quant_planes_reference_kat_and_limits(ctx, golden):
         ctx.gemv_q8_0_planes(dx, planes, dout, 1, 8192, 1)
 
 
+def test_q6_k_planes_hold_the_blocks_bit_for_bit(ctx, oracle):
+    """Q6_K re-packed into four planes: every byte of a block sits where the declaration says (a numpy
+    restatement of the unit order), unpacking returns the blocks, and dequantising from the planes gives the
+    oracle's bits, special block scales included."""
+    from homura_amd.runtime import DTYPE_Q6_K
+    N, K = 37, 768
+    nb = N * (K // 256)
+    raw = synth.q6_k_blocks(93, nb)
+    blk = raw.reshape(nb, 210)
+    for i, bits in enumerate([0x0001, 0x03FF, 0x0000, 0x8000, 0x7BFF, 0x7C00, 0xFC00, 0x7E00, 0x0400]):
+        blk[i, 208], blk[i, 209] = bits & 0xFF, bits >> 8
+    d_raw = ctx.to_device(raw)
+    planes = ctx.pack_quant_planes(DTYPE_Q6_K, d_raw, N, K)
+    size = ctx.lib.hm_quant_planes_bytes(DTYPE_Q6_K, N, K)
+    units = nb * 4
+    up = lambda v: (v + 255) // 256 * 256
+    top_off = up(units * 32)
+    sc_off = up(top_off + units * 16)
+    d_off = up(sc_off + units * 4)
+    assert size == d_off + nb * 2
+    host = planes.download(np.uint8)[:size]
+    nib = host[:units * 32].reshape(nb, 2, 2, 2, 16)          # block, h, p, run, j
+    ql = blk[:, :128].reshape(nb, 2, 2, 2, 16)                 # block, h, run (l / 32), p, j
+    assert np.array_equal(nib, ql.transpose(0, 1, 3, 2, 4))
+    top = host[top_off:top_off + units * 16].reshape(nb, 2, 2, 16)
+    assert np.array_equal(top, blk[:, 128:192].reshape(nb, 2, 2, 16))
+    sc = host[sc_off:sc_off + units * 4].reshape(nb, 2, 2, 4)  # block, h, p, g
+    assert np.array_equal(sc, blk[:, 192:208].reshape(nb, 2, 4, 2).transpose(0, 1, 3, 2))
+    assert np.array_equal(host[d_off:d_off + 2 * nb].reshape(nb, 2), blk[:, 208:])
+    back = ctx.empty(raw.size, np.uint8)
+    ctx.unpack_quant_planes(DTYPE_Q6_K, planes, back, N, K)
+    assert np.array_equal(back.download(np.uint8), raw.reshape(-1))
+    want = oracle.dequant_q6_k(raw)
+    d_out = ctx.empty(N * K)
+    ctx.dequant_quant_planes(DTYPE_Q6_K, planes, d_out, N, K)
+    got = d_out.download(np.float32)
+    nan = np.isnan(want)
+    assert np.array_equal(np.isnan(got), nan)
+    assert np.array_equal(got[~nan].view(np.uint32), want[~nan].view(np.uint32))
+    assert ctx.lib.hm_quant_planes_bytes(DTYPE_Q6_K, 8, 128) == 0
+    for b in (d_raw, planes, back, d_out):
+        b.free()
+
+
+@pytest.mark.parametrize("M,K,N", [(1, 1024, 151936),   # LM head of the Qwen3-0.6B shape
+                                   (1, 1024, 3073), (2, 256, 7), (3, 2048, 515), (1, 4096, 130), (1, 512, 1001),
+                                   (1, 2048, 1), (1, 1024, 2)])
+def test_q6_k_planes_f32_product(ctx, oracle, M, K, N):
+    """f32 row times the dequantised Q6_K weights, read from the planes: the checker multiplies the oracle's
+    dequantised matrix (bit-exact with the reference's dequant_q6_k) in float64; widths the unit kernel has
+    no instance for are refused."""
+    from homura_amd.runtime import DTYPE_Q6_K
+    say(f"gemv_q6_k_f32_planes M={M} K={K} N={N}")
+    raw = synth.q6_k_blocks(15, N * K // 256)
+    x = synth.normal_f32(16, M * K, 1.0).reshape(M, K)
+    w = oracle.dequant_q6_k(raw).reshape(N, K)
+    want = x.astype(np.float64) @ w.astype(np.float64).T
+    dx, dw, dout = ctx.to_device(x), ctx.to_device(raw), ctx.empty(M * N)
+    planes = ctx.pack_quant_planes(DTYPE_Q6_K, dw, N, K)
+    ctx.gemv_q6_k_f32_planes(dx, planes, dout, M, K, N)
+    got = dout.download(np.float32, (M, N))
+    err = np.abs(got - want).max() / np.sqrt(np.mean(want ** 2))
+    say(f"  max error / rms {err:.2e}")
+    assert err < 2e-6 * max(1.0, np.sqrt(K / 1024))   # f32 sums of exact terms
+    with pytest.raises(HomuraError, match="must be 256, 512, 1024, 2048 or 4096"):
+        ctx.gemv_q6_k_f32_planes(dx, planes, dout, 1, 768, 1)
+    for b in (dx, dw, dout, planes):
+        b.free()
+
+
 # ── K-quants ──────────────────────────────────────────────────────────────────
 
 @pytest.mark.parametrize("kind", ["q4_k", "q6_k"])
