@@ -45,10 +45,14 @@ struct Geo {
     static constexpr int G = H / KVH, QD = H * HD, KVD = KVH * HD, NQKV = QD + 2 * KVD;
     static constexpr int CH = HIDDEN / 512, CO = QD / 512, CD = INTER / 512;  // 512-wide chunks of a row
     static constexpr int RQ = NQKV / NWG, RQW = RQ / NCW;      // Q|K|V rows per workgroup / wavefront
-    static constexpr int RO = HIDDEN / NWG, ROW = RO / NCW;    // O and down rows
+    static constexpr int SPH = NWG / KVH;                      // workgroups (= cache splits) per KV head
+    // O and down: the workgroups of a KV head multiply a K slice (the head group's own attention outputs,
+    // its own SiLU*up values) for every output row, RPG rows a workgroup; the KVH partial vectors are
+    // added up on the way into the next phase.
+    static constexpr int RPG = HIDDEN / SPH, RPW = RPG / NCW;  // partial rows per workgroup / wavefront
+    static constexpr int KSO = G * HD, KSD = INTER / KVH;      // K slice of the O / down projection
     static constexpr int RG = 2 * INTER / NWG, RGW = RG / NCW; // gate|up rows (interleaved pairs)
     static constexpr int APW = INTER / NWG;                    // SiLU*up values per workgroup
-    static constexpr int SPH = NWG / KVH;                      // cache splits per KV head
     static constexpr int NR = NR_;                             // row rounds a wavefront keeps in registers
     static constexpr int LPR = HD / 8, RPI = WAVE / LPR;       // lanes per cache row, rows per load
     static constexpr int MAX_KV = SPH * NR * NCW * RPI;
@@ -60,28 +64,33 @@ struct Geo {
     // A KV head's workgroups are wg % KVH == head; with workgroups dealt round-robin to the dies they all
     // share one L2 when KVH is a multiple of the die count.
     static constexpr bool GROUP_ON_XCD = KVH % NXCD == 0;
-    // Exchange area of one layer parity, in 8-byte slots: the vectors every workgroup reads (hidden
-    // increments XH / XO, folded attention XA, SiLU*up XC), one relay copy of those per die, and per KV
-    // head the raw q|k|v rows (LQ) and the attention partials of its splits (LP).
-    static constexpr int XH = 0, XO = HIDDEN, XA = 2 * HIDDEN, XC = XA + QD, GLOB_SLOTS = XC + INTER;
-    static constexpr int RELAY0 = GLOB_SLOTS, LQ0 = RELAY0 + NXCD * GLOB_SLOTS, LP0 = LQ0 + KVH * GROWS;
-    static constexpr int PAR_SLOTS = (LP0 + KVH * SPH * PART + 31) / 32 * 32;
+    // Exchange area of one layer parity, in 8-byte slots: the partial hidden increments of every KV-head
+    // group (down rows XH, O rows XO: KVH vectors each), per die one relay copy of their sums, and per KV
+    // head the raw q|k|v rows (LQ), the attention partials of its splits (LP), its folded attention
+    // outputs (LA) and its SiLU*up values (LC).
+    static constexpr int XH = 0, XO = KVH * HIDDEN, GLOB_SLOTS = 2 * KVH * HIDDEN;
+    static constexpr int RELAY0 = GLOB_SLOTS, RELAY_SLOTS = 2 * HIDDEN;
+    static constexpr int LQ0 = RELAY0 + NXCD * RELAY_SLOTS, LP0 = LQ0 + KVH * GROWS, LA0 = LP0 + KVH * SPH * PART;
+    static constexpr int LC0 = LA0 + KVH * KSO;
+    static constexpr int PAR_SLOTS = (LC0 + KVH * KSD + 31) / 32 * 32;
     static constexpr int CHK0 = 2 * PAR_SLOTS;                 // placement check: one slot per workgroup
     static constexpr int CAND0 = CHK0 + NWG;                   // LM head: one {value, index} unit per workgroup
     static constexpr int ALL_SLOTS = CAND0 + 2 * NWG;
     static constexpr int HR = 8;                               // LM-head rows a wavefront multiplies per batch
-    static constexpr int PUB = (PART > RQ ? PART : RQ) > RG ? (PART > RQ ? PART : RQ) : RG;
+    static constexpr int PUB0 = (PART > RQ ? PART : RQ) > RG ? (PART > RQ ? PART : RQ) : RG;
+    static constexpr int PUB = PUB0 > RPG ? PUB0 : RPG;
     static_assert(HIDDEN % 512 == 0 && QD % 512 == 0 && INTER % 512 == 0, "rows are cut into 512-wide chunks");
-    static_assert(NQKV % (NWG * NCW) == 0 && HIDDEN % (NWG * NCW) == 0 && (2 * INTER) % (NWG * NCW) == 0,
+    static_assert(NQKV % (NWG * NCW) == 0 && HIDDEN % (SPH * NCW) == 0 && (2 * INTER) % (NWG * NCW) == 0,
                   "every wavefront owns whole rows");
+    static_assert(KSO % 128 == 0 && KSD % 128 == 0 && INTER % KVH == 0, "K slices are cut into 128-wide parts");
     static_assert(RGW % 2 == 0, "a wavefront owns whole gate|up pairs");
     static_assert(NWG % KVH == 0 && SPH <= WAVE, "one fold lane per cache split");
     static_assert(HD == 64 || HD == 128, "head_dim 64 or 128");
     static_assert(QD % NWG == 0 && FPW % 2 == 0 && HD % FPW == 0, "a workgroup folds a run inside one head");
-    static_assert(RQ <= CT && RO <= CT && APW <= CT, "one publishing thread per value");
+    static_assert(RQ <= CT && RPG <= CT && APW <= CT, "one publishing thread per value");
+    static_assert(KSO / 2 <= CT && KSD / 2 <= CT, "one staging thread per 16-byte unit of a K slice");
     static_assert(GROWS % SPH == 0 && GROWS / SPH == RQ && HD % RQW == 0, "a wavefront's q|k|v rows lie in one of q, k, v");
-    static_assert(NWG % NXCD == 0 && (HIDDEN / 2) % NPX == 0 && (QD / 2) % NPX == 0 && (INTER / 2) % NPX == 0 &&
-                      INTER / 2 / NPX <= WAVE && QD / 2 / NPX <= WAVE && HIDDEN / 2 / NPX <= WAVE,
+    static_assert(NWG % NXCD == 0 && (HIDDEN / 2) % NPX == 0 && HIDDEN / 2 / NPX <= WAVE,
                   "one wavefront relays a die's share of a vector");
     static_assert(NWG % 2 == 0 && NWG / 2 <= 2 * WAVE, "two placement-check units per lane");
     static_assert(NWG % WAVE == 0 && NWG / WAVE <= 8, "workgroup 0 gathers the LM-head candidates with one wavefront");
@@ -95,8 +104,8 @@ template <class GE>
 struct Lds {
     float hx[GE::HIDDEN];                 // hidden state entering the phase's RMSNorm
     float nw[GE::HIDDEN];                 // that norm's weights
-    float attn[GE::QD];                   // folded attention output
-    float act[GE::INTER];                 // SiLU(gate) * up
+    float attn[GE::KSO];                  // folded attention output of this workgroup's KV head
+    float act[GE::KSD];                   // SiLU(gate) * up of this workgroup's KV-head group
     float rowbuf[GE::G + 2][GE::HD];      // raw q heads, k, v of this workgroup's KV head
     float qs[GE::G][GE::HD];              // after QK-norm and RoPE
     float knew[GE::HD], vnew[GE::HD];     // the new cache row, as rounded to bf16
@@ -484,6 +493,122 @@ struct Rows {
     }
 };
 
+// ── rows of one matrix restricted to a K slice, as a compute wavefront keeps them for the O and down phases ──
+//
+// R rows x KS columns [k0, k0 + KS) of an [N][KTOT] matrix. bf16: a register holds four rows of one 128-wide
+// part of the slice (lane = 16 * row + position, 8 weights a lane), so a row's sum is the sum of its parts'
+// registers followed by a reduction inside a DPP row of 16 lanes. Q8_0 / Q4_0 planes: a lane holds half a
+// block (16 weights), a register set eight rows of one part, and a row's sum ends inside 8 lanes. dots()
+// leaves in v[q], in every lane of row q * ROWS_PER_SET + lane / LANES_PER_ROW, that row's sum.
+template <int WF, int R, int KS, int KTOT>
+struct SliceRows;
+
+template <int R, int KS, int KTOT>
+struct SliceRows<FUSED_WF_BF16, R, KS, KTOT> {
+    static constexpr int P = KS / 128, LANES_PER_ROW = 16, ROWS_PER_SET = 4, Q = R / ROWS_PER_SET;
+    static_assert(KS % 128 == 0 && R % ROWS_PER_SET == 0 && Q >= 1, "four rows and a 128-wide part per register");
+    u32x4 w[Q][P];
+    __device__ __forceinline__ void load(const void *quants, const uint16_t *, int row0, int k0, int lane) {
+        const uint16_t *base = reinterpret_cast<const uint16_t *>(quants);
+#pragma unroll
+        for (int q = 0; q < Q; q++)
+#pragma unroll
+            for (int p = 0; p < P; p++)
+                w[q][p] = ld128_global_stream(base + (size_t)(row0 + q * ROWS_PER_SET + lane / LANES_PER_ROW) * KTOT + k0 + p * 128 +
+                                              (lane % LANES_PER_ROW) * 8);
+    }
+    __device__ __forceinline__ void dots(const float *x, int lane, float (&v)[Q]) const {
+        float xv[P][8], acc[Q][P];
+#pragma unroll
+        for (int p = 0; p < P; p++) lds_x8(x, p * 128 + (lane % LANES_PER_ROW) * 8, xv[p]);
+        dots_from<Q, P>(w, xv, acc);
+#pragma unroll
+        for (int q = 0; q < Q; q++) v[q] = chunk_total<P>(acc[q]);
+#pragma unroll
+        for (int q = 0; q < Q; q++) v[q] += dpp_move<0xB1, 0xF>(v[q], 0.f);
+#pragma unroll
+        for (int q = 0; q < Q; q++) v[q] += dpp_move<0x4E, 0xF>(v[q], 0.f);
+#pragma unroll
+        for (int q = 0; q < Q; q++) v[q] += dpp_move<0x141, 0xF>(v[q], 0.f);
+#pragma unroll
+        for (int q = 0; q < Q; q++) v[q] += dpp_move<0x140, 0xF>(v[q], 0.f);
+    }
+};
+
+// sum_j q_j x_j of half a block with the quants used as stored (Q8_0: biased to unsigned), xv in the order
+// of Rows::x_index
+template <bool Q4>
+__device__ __forceinline__ float half_block_dot(const uint32_t *qw, const float *xv) {
+    float sum;
+    if constexpr (Q4) {
+        const uint32_t w0 = qw[0], w1 = qw[1];
+        sum = dot4_bytes(w1 & 0x0F0F0F0Fu, xv + 4, dot4_bytes(w0 & 0x0F0F0F0Fu, xv, 0.f));
+        sum = dot4_bytes((w1 >> 4) & 0x0F0F0F0Fu, xv + 12, dot4_bytes((w0 >> 4) & 0x0F0F0F0Fu, xv + 8, sum));
+    } else {
+        sum = 0.f;
+#pragma unroll
+        for (int e = 0; e < 4; e++) sum = dot4_bytes(qw[e] ^ 0x80808080u, xv + 4 * e, sum);  // int8 -> biased unsigned
+    }
+    return sum;
+}
+
+template <int WF, int R, int KS, int KTOT>
+struct SliceRows {
+    static constexpr bool Q4 = WF == FUSED_WF_Q4_0;
+    static constexpr int P = KS / 128, LANES_PER_ROW = 8, ROWS_PER_SET = 8, Q = R / ROWS_PER_SET;
+    static_assert(KS % 128 == 0 && R % ROWS_PER_SET == 0 && Q >= 1 && KTOT % 32 == 0, "eight rows and a 128-wide part per register set");
+    uint32_t q[Q][P][Q4 ? 2 : 4];  // the lane's half block: 8 bytes of nibble pairs or 16 int8
+    uint32_t d[Q][P];              // f16 bits of its block's scale
+    __device__ __forceinline__ void load(const void *quants, const uint16_t *scales, int row0, int k0, int lane) {
+        const unsigned char *base = reinterpret_cast<const unsigned char *>(quants);
+#pragma unroll
+        for (int s = 0; s < Q; s++)
+#pragma unroll
+            for (int p = 0; p < P; p++) {
+                const size_t row = (size_t)(row0 + s * ROWS_PER_SET + lane / LANES_PER_ROW);
+                const int hb = (k0 + p * 128) / 16 + lane % LANES_PER_ROW;  // half block of the row
+                if constexpr (Q4) {
+                    const u32x2 t = __builtin_nontemporal_load((global_u32x2_ptr)(base + row * (KTOT / 2) + (size_t)hb * 8));
+                    q[s][p][0] = t.x;
+                    q[s][p][1] = t.y;
+                } else {
+                    const u32x4 t = ld128_global_stream(base + row * KTOT + (size_t)hb * 16);
+                    q[s][p][0] = t.x;
+                    q[s][p][1] = t.y;
+                    q[s][p][2] = t.z;
+                    q[s][p][3] = t.w;
+                }
+                d[s][p] = __builtin_nontemporal_load((global_u16_ptr)(scales + row * (KTOT / 32) + (hb >> 1)));
+            }
+    }
+    __device__ __forceinline__ void dots(const float *x, int lane, float (&v)[Q]) const {
+        float xv[P][16], off[P];
+#pragma unroll
+        for (int p = 0; p < P; p++) {
+            const int hb = p * 8 + lane % LANES_PER_ROW;  // half block inside the slice (slices start on a block)
+#pragma unroll
+            for (int part = 0; part < 2; part++)
+                lds_x8(x, Q4 ? (hb >> 1) * 32 + (hb & 1) * 8 + part * 16 : hb * 16 + part * 8, xv[p] + part * 8);
+            float sx = 0.f;
+#pragma unroll
+            for (int j = 0; j < 16; j++) sx += xv[p][j];
+            off[p] = sx * (Q4 ? 8.f : 128.f);
+        }
+#pragma unroll
+        for (int s = 0; s < Q; s++) v[s] = 0.f;
+#pragma unroll
+        for (int p = 0; p < P; p++)
+#pragma unroll
+            for (int s = 0; s < Q; s++) v[s] += f16_bits_to_f32((uint16_t)d[s][p]) * (half_block_dot<Q4>(q[s][p], xv[p]) - off[p]);
+#pragma unroll
+        for (int s = 0; s < Q; s++) v[s] += dpp_move<0xB1, 0xF>(v[s], 0.f);
+#pragma unroll
+        for (int s = 0; s < Q; s++) v[s] += dpp_move<0x4E, 0xF>(v[s], 0.f);
+#pragma unroll
+        for (int s = 0; s < Q; s++) v[s] += dpp_move<0x141, 0xF>(v[s], 0.f);
+    }
+};
+
 // The attention split of a workgroup for a cache of kv_len rows (the new row included).
 template <class GE>
 struct Split {
@@ -577,9 +702,9 @@ template <class GE, int WF>
 struct Slice {
     Rows<WF, GE::RQW, GE::HIDDEN> wq;
     u32x4 kr[GE::NR], vr[GE::NR];
-    Rows<WF, GE::ROW, GE::QD> wo;
+    SliceRows<WF, GE::RPW, GE::KSO, GE::QD> wo;
     Rows<WF, GE::RGW, GE::HIDDEN> wg;
-    Rows<WF, GE::ROW, GE::INTER> wd;
+    SliceRows<WF, GE::RPW, GE::KSD, GE::INTER> wd;
 };
 
 template <class GE, int WF>
@@ -609,18 +734,20 @@ __device__ __forceinline__ void compute_role(const FusedDecodeArgs &a, Lds<GE> &
         }
     };
     auto load_wo = [&](const FusedLayerPtrs &lp) {
-        s.wo.load(lp.wo, lp.so, [&](int r) { return wg * GE::RO + cw * GE::ROW + r; }, 0, GE::ROW, lane);
+        s.wo.load(lp.wo, lp.so, sp.split * GE::RPG + cw * GE::RPW, sp.kh * GE::KSO, lane);
     };
     // bf16 keeps gate and up rows interleaved (g0, u0, g1, u1, ...); the quantised formats keep the run as
-    // uploaded, all gate rows and then all up rows, so local row r = 2 p + (0 gate | 1 up) of pair p
+    // uploaded, all gate rows and then all up rows, so local row r = 2 p + (0 gate | 1 up) of pair p.
+    // Pairs are dealt by KV-head group first (wgp), so a group's SiLU*up values are one K slice of down.
+    const int wgp = sp.kh * GE::SPH + sp.split;
     auto load_wg = [&](const FusedLayerPtrs &lp, int r0, int r1) {
         s.wg.load(lp.wgu, lp.sgu, [&](int r) {
             const int lr = cw * GE::RGW + r;
-            return WF == FUSED_WF_BF16 ? wg * GE::RG + lr : (lr & 1) * GE::INTER + wg * GE::APW + (lr >> 1);
+            return WF == FUSED_WF_BF16 ? wgp * GE::RG + lr : (lr & 1) * GE::INTER + wgp * GE::APW + (lr >> 1);
         }, r0, r1, lane);
     };
     auto load_wd = [&](const FusedLayerPtrs &lp) {
-        s.wd.load(lp.wd, lp.sd, [&](int r) { return wg * GE::RO + cw * GE::ROW + r; }, 0, GE::ROW, lane);
+        s.wd.load(lp.wd, lp.sd, sp.split * GE::RPG + cw * GE::RPW, sp.kh * GE::KSD, lane);
     };
 
     constexpr int KV_CUT = NR / 2, WG_CUT = 2 * GE::RGW / 3;
@@ -778,13 +905,13 @@ __device__ __forceinline__ void compute_role(const FusedDecodeArgs &a, Lds<GE> &
         wg_barrier();
         load_kv(nx, 0, KV_CUT);
         {
-            float v[GE::ROW];
-            s.wo.dots_plain(sm.attn, lane, v);
-            wave_sum_n<GE::ROW>(v);
-            float mine = 0.f;
+            using S = decltype(s.wo);
+            float v[S::Q];
+            s.wo.dots(sm.attn, lane, v);
+            if (lane % S::LANES_PER_ROW == 0) {
 #pragma unroll
-            for (int r = 0; r < GE::ROW; r++) mine = lane == r ? v[r] : mine;
-            if (lane < GE::ROW) sm.pub[cw * GE::ROW + lane] = mine;
+                for (int q = 0; q < S::Q; q++) sm.pub[cw * GE::RPW + q * S::ROWS_PER_SET + lane / S::LANES_PER_ROW] = v[q];
+            }
         }
         wg_barrier();
 
@@ -812,13 +939,13 @@ __device__ __forceinline__ void compute_role(const FusedDecodeArgs &a, Lds<GE> &
         wg_barrier();
         load_wg(nx, 0, WG_CUT);
         {
-            float v[GE::ROW];
-            s.wd.dots_plain(sm.act, lane, v);
-            wave_sum_n<GE::ROW>(v);
-            float mine = 0.f;
+            using S = decltype(s.wd);
+            float v[S::Q];
+            s.wd.dots(sm.act, lane, v);
+            if (lane % S::LANES_PER_ROW == 0) {
 #pragma unroll
-            for (int r = 0; r < GE::ROW; r++) mine = lane == r ? v[r] : mine;
-            if (lane < GE::ROW) sm.pub[cw * GE::ROW + lane] = mine;
+                for (int q = 0; q < S::Q; q++) sm.pub[cw * GE::RPW + q * S::ROWS_PER_SET + lane / S::LANES_PER_ROW] = v[q];
+            }
         }
         wg_barrier();
     }
@@ -900,36 +1027,48 @@ __device__ __forceinline__ void comm_role(const FusedDecodeArgs &a, Lds<GE> &sm,
     }
     const bool near_g = die_ok && GE::GROUP_ON_XCD;  // a KV head's workgroups talk through their die's L2
 
-    // A vector that every workgroup reads is fetched from memory once per die: one wavefront of each of the
-    // die's workgroups waits for its share of the units and copies them to the die's relay area, which all
-    // of them then read through the L2. Without die-local placement everyone reads the far copy.
-    auto relay = [&](unsigned char *par, int off, int n_units, uint32_t tag) -> const unsigned char * {
-        if (!die_ok) return par;
-        unsigned char *rel = par + (size_t)(GE::RELAY0 + xcd * GE::GLOB_SLOTS) * 8;
+    // The hidden increments reach the exchange area as KVH partial vectors (one per KV-head group, each a K
+    // slice of the O or down projection). They are fetched from memory once per die: one wavefront of each
+    // of the die's workgroups waits for its share of the units of all KVH vectors, adds them in group order
+    // and writes the sums to the die's relay area, which all of the die's workgroups then read through
+    // the L2. Without die-local placement the relay's stores go through to memory.
+    auto relay_sum = [&](unsigned char *par, int off, uint32_t tag) -> const unsigned char * {
+        unsigned char *rel = par + (size_t)(GE::RELAY0 + xcd * GE::RELAY_SLOTS + (off == GE::XH ? 0 : GE::HIDDEN)) * 8;
         if (cwv == 3) {  // wavefront 0 may still be folding
-            const int per = n_units / GE::NPX;
-            int unit[1] = {off / 2 + rank * per + lane};
-            bool on[1] = {lane < per};
-            u32x4 w[1];
-            poll_units<1>(ps, par, unit, on, tag, w);
-            if (on[0]) {
-                *reinterpret_cast<u32x4 *>(rel + (size_t)unit[0] * 16) = w[0];  // plain store: stays in the die's L2
-                asm volatile("" ::: "memory");
+            constexpr int per = GE::HIDDEN / 2 / GE::NPX;
+            int unit[GE::KVH];
+            bool on[GE::KVH];
+            u32x4 w[GE::KVH];
+#pragma unroll
+            for (int d = 0; d < GE::KVH; d++) {
+                unit[d] = (off + d * GE::HIDDEN) / 2 + rank * per + lane;
+                on[d] = lane < per;
+            }
+            poll_units<GE::KVH>(ps, par, unit, on, tag, w);
+            if (lane < per) {
+                float v0 = __uint_as_float(w[0].x), v1 = __uint_as_float(w[0].z);
+#pragma unroll
+                for (int d = 1; d < GE::KVH; d++) {
+                    v0 += __uint_as_float(w[d].x);
+                    v1 += __uint_as_float(w[d].z);
+                }
+                st_slot(rel, 2 * (rank * per + lane), v0, tag, die_ok);
+                st_slot(rel, 2 * (rank * per + lane) + 1, v1, tag, die_ok);
             }
         }
         return rel;
     };
-    // hidden <- hidden + (the vector at slot offset `off`), then stage hidden, the norm weights and this
-    // wavefront's share of the sum of squares
+    // hidden <- hidden + (the sum of the partial vectors at slot offset `off`), then stage hidden, the norm
+    // weights and this wavefront's share of the sum of squares
     auto stage_hidden = [&](unsigned char *par, int off, uint32_t tag, bool add, const float (&nwv)[NJ]) {
         if (add) {
-            const unsigned char *src = relay(par, off, GE::HIDDEN / 2, tag);
+            const unsigned char *src = relay_sum(par, off, tag);
             int unit[NJ / 2];
             bool on[NJ / 2];
             u32x4 w[NJ / 2];
 #pragma unroll
             for (int u = 0; u < NJ / 2; u++) {
-                unit[u] = off / 2 + u * CT + ct;
+                unit[u] = u * CT + ct;
                 on[u] = true;
             }
             poll_units<NJ / 2>(ps, src, unit, on, tag, w);
@@ -950,23 +1089,15 @@ __device__ __forceinline__ void comm_role(const FusedDecodeArgs &a, Lds<GE> &sm,
             sm.nw[ct + CT * j] = nwv[j];
         }
     };
-    // copy a published vector (plain slot order) into LDS
-    auto stage_vector = [&](unsigned char *par, int off, uint32_t tag, float *dst, auto nu_tag) {
-        constexpr int NU = decltype(nu_tag)::value;
-        const unsigned char *src = relay(par, off, NU * CT, tag);
-        int unit[NU];
-        bool on[NU];
-        u32x4 w[NU];
-#pragma unroll
-        for (int u = 0; u < NU; u++) {
-            unit[u] = off / 2 + u * CT + ct;
-            on[u] = true;
-        }
-        poll_units<NU>(ps, src, unit, on, tag, w);
-#pragma unroll
-        for (int u = 0; u < NU; u++) {
-            dst[2 * (u * CT + ct)] = __uint_as_float(w[u].x);
-            dst[2 * (u * CT + ct) + 1] = __uint_as_float(w[u].z);
+    // copy a vector of this KV head's group (n_units 16-byte units in plain slot order) into LDS
+    auto stage_group = [&](const unsigned char *src, int n_units, uint32_t tag, float *dst) {
+        int unit[1] = {ct};
+        bool on[1] = {ct < n_units};
+        u32x4 w[1];
+        poll_units<1>(ps, src, unit, on, tag, w);
+        if (on[0]) {
+            dst[2 * ct] = __uint_as_float(w[0].x);
+            dst[2 * ct + 1] = __uint_as_float(w[0].z);
         }
     };
 
@@ -1008,7 +1139,9 @@ __device__ __forceinline__ void comm_role(const FusedDecodeArgs &a, Lds<GE> &sm,
         unsigned char *xc = a.xch + (size_t)(gl & 1u) * par_bytes;
         unsigned char *xprev = a.xch + (size_t)((gl & 1u) ^ 1u) * par_bytes;
         unsigned char *lq = xc + (size_t)(GE::LQ0 + sp.kh * GE::GROWS) * 8;             // this KV head's raw rows
-        unsigned char *lp = xc + (size_t)(GE::LP0 + sp.kh * GE::SPH * GE::PART) * 8;    // and its splits' partials
+        unsigned char *lp = xc + (size_t)(GE::LP0 + sp.kh * GE::SPH * GE::PART) * 8;    // its splits' partials,
+        unsigned char *la = xc + (size_t)(GE::LA0 + sp.kh * GE::KSO) * 8;               // its folded attention outputs
+        unsigned char *lc = xc + (size_t)(GE::LC0 + sp.kh * GE::KSD) * 8;               // and its group's SiLU*up values
 
         // ── into the Q|K|V phase: hidden += down rows of the previous layer ──
         ps.where = 1u | (uint32_t)l << 4 | (uint32_t)wg << 12;
@@ -1134,18 +1267,18 @@ __device__ __forceinline__ void comm_role(const FusedDecodeArgs &a, Lds<GE> &sm,
             float mine = 0.f;
 #pragma unroll
             for (int e = 0; e < GE::FPW; e++) mine = lane == e ? red[1 + e] / red[0] : mine;
-            if (lane < GE::FPW) st_slot(xc, GE::XA + sp.kh * G * HD + o0 + lane, mine, tag, false);
+            if (lane < GE::FPW) st_slot(la, o0 + lane, mine, tag, near_g);
         }
         mark();
 
         // ── into the O phase ──
         ps.where = 4u | (uint32_t)l << 4 | (uint32_t)wg << 12;
-        stage_vector(xc, GE::XA, tag, sm.attn, std::integral_constant<int, GE::QD / 2 / CT>());
+        stage_group(la, GE::KSO / 2, tag, sm.attn);
         wg_barrier();
         mark();
         wg_barrier();
         mark();
-        if (ct < GE::RO) st_slot(xc, GE::XO + hidden_slot(wg * GE::RO + ct), sm.pub[ct], tag, false);
+        if (ct < GE::RPG) st_slot(xc, GE::XO + sp.kh * GE::HIDDEN + hidden_slot(sp.split * GE::RPG + ct), sm.pub[ct], tag, false);
 
         // ── into the gate|up phase: hidden += O rows (reference src/hf/emitter.rs:787) ──
         ps.where = 5u | (uint32_t)l << 4 | (uint32_t)wg << 12;
@@ -1155,16 +1288,16 @@ __device__ __forceinline__ void comm_role(const FusedDecodeArgs &a, Lds<GE> &sm,
         mark();
         wg_barrier();
         mark();
-        if (ct < GE::APW) st_slot(xc, GE::XC + wg * GE::APW + ct, sm.pub[ct], tag, false);
+        if (ct < GE::APW) st_slot(lc, sp.split * GE::APW + ct, sm.pub[ct], tag, near_g);
 
         // ── into the down phase ──
         ps.where = 6u | (uint32_t)l << 4 | (uint32_t)wg << 12;
-        stage_vector(xc, GE::XC, tag, sm.act, std::integral_constant<int, GE::INTER / 2 / CT>());
+        stage_group(lc, GE::KSD / 2, tag, sm.act);
         wg_barrier();
         mark();
         wg_barrier();
         mark();
-        if (ct < GE::RO) st_slot(xc, GE::XH + hidden_slot(wg * GE::RO + ct), sm.pub[ct], tag, false);
+        if (ct < GE::RPG) st_slot(xc, GE::XH + sp.kh * GE::HIDDEN + hidden_slot(sp.split * GE::RPG + ct), sm.pub[ct], tag, false);
     }
 
     if (a.head_w) {
@@ -1232,23 +1365,31 @@ __device__ __forceinline__ void comm_role(const FusedDecodeArgs &a, Lds<GE> &sm,
             }
         }
     } else if (wg == 0) {
-        // hidden += down rows of the last layer: the LM head's input
+        // hidden += down rows of the last layer (the groups' partial vectors, added in group order as the
+        // relays do): the LM head's input
         const uint32_t gl = base + (uint32_t)(L - 1);
         const unsigned char *xl = a.xch + (size_t)(gl & 1u) * par_bytes;
-        int unit[NJ / 2];
-        bool on[NJ / 2];
-        u32x4 w[NJ / 2];
+        float inc[NJ];
 #pragma unroll
-        for (int u = 0; u < NJ / 2; u++) {
-            unit[u] = GE::XH / 2 + u * CT + ct;
-            on[u] = true;
-        }
-        poll_units<NJ / 2>(ps, xl, unit, on, gl + 1u, w);
+        for (int j = 0; j < NJ; j++) inc[j] = 0.f;
+        for (int d = 0; d < GE::KVH; d++) {
+            int unit[NJ / 2];
+            bool on[NJ / 2];
+            u32x4 w[NJ / 2];
 #pragma unroll
-        for (int u = 0; u < NJ / 2; u++) {
-            a.hidden_out[ct + CT * (2 * u)] = h[2 * u] + __uint_as_float(w[u].x);
-            a.hidden_out[ct + CT * (2 * u + 1)] = h[2 * u + 1] + __uint_as_float(w[u].z);
+            for (int u = 0; u < NJ / 2; u++) {
+                unit[u] = (GE::XH + d * GE::HIDDEN) / 2 + u * CT + ct;
+                on[u] = true;
+            }
+            poll_units<NJ / 2>(ps, xl, unit, on, gl + 1u, w);
+#pragma unroll
+            for (int u = 0; u < NJ / 2; u++) {
+                inc[2 * u] = d == 0 ? __uint_as_float(w[u].x) : inc[2 * u] + __uint_as_float(w[u].x);
+                inc[2 * u + 1] = d == 0 ? __uint_as_float(w[u].z) : inc[2 * u + 1] + __uint_as_float(w[u].z);
+            }
         }
+#pragma unroll
+        for (int j = 0; j < NJ; j++) a.hidden_out[ct + CT * j] = h[j] + inc[j];
         // Every workgroup read the launch count before its first exchange, and this point is only reached
         // after all of them have published their last rows.
         if (ct == 0) __hip_atomic_store(a.ctl, launches + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
