@@ -51,6 +51,10 @@ struct Geo {
     // added up on the way into the next phase.
     static constexpr int RPG = HIDDEN / SPH, RPW = RPG / NCW;  // partial rows per workgroup / wavefront
     static constexpr int KSO = G * HD, KSD = INTER / KVH;      // K slice of the O / down projection
+    // A workgroup's partial rows are two runs of RPG / 2 rows, 256 rows apart: hidden elements k and k + 256
+    // share a 16-byte exchange unit (hidden_slot), which one workgroup then writes whole.
+    static constexpr int RUN = RPG / 2, WPP = 256 / RUN;
+    __device__ static int partial_row(int split, int i) { return (split % WPP) * RUN + i % RUN + 256 * (2 * (split / WPP) + i / RUN); }
     static constexpr int RG = 2 * INTER / NWG, RGW = RG / NCW; // gate|up rows (interleaved pairs)
     static constexpr int APW = INTER / NWG;                    // SiLU*up values per workgroup
     static constexpr int NR = NR_;                             // row rounds a wavefront keeps in registers
@@ -83,6 +87,7 @@ struct Geo {
     static_assert(NQKV % (NWG * NCW) == 0 && HIDDEN % (SPH * NCW) == 0 && (2 * INTER) % (NWG * NCW) == 0,
                   "every wavefront owns whole rows");
     static_assert(KSO % 128 == 0 && KSD % 128 == 0 && INTER % KVH == 0, "K slices are cut into 128-wide parts");
+    static_assert(RUN % RPW == 0 && 256 % RUN == 0 && SPH % WPP == 0, "a wavefront's partial rows lie in one run");
     static_assert(RGW % 2 == 0, "a wavefront owns whole gate|up pairs");
     static_assert(NWG % KVH == 0 && SPH <= WAVE, "one fold lane per cache split");
     static_assert(HD == 64 || HD == 128, "head_dim 64 or 128");
@@ -734,7 +739,7 @@ __device__ __forceinline__ void compute_role(const FusedDecodeArgs &a, Lds<GE> &
         }
     };
     auto load_wo = [&](const FusedLayerPtrs &lp) {
-        s.wo.load(lp.wo, lp.so, sp.split * GE::RPG + cw * GE::RPW, sp.kh * GE::KSO, lane);
+        s.wo.load(lp.wo, lp.so, GE::partial_row(sp.split, cw * GE::RPW), sp.kh * GE::KSO, lane);
     };
     // bf16 keeps gate and up rows interleaved (g0, u0, g1, u1, ...); the quantised formats keep the run as
     // uploaded, all gate rows and then all up rows, so local row r = 2 p + (0 gate | 1 up) of pair p.
@@ -747,7 +752,7 @@ __device__ __forceinline__ void compute_role(const FusedDecodeArgs &a, Lds<GE> &
         }, r0, r1, lane);
     };
     auto load_wd = [&](const FusedLayerPtrs &lp) {
-        s.wd.load(lp.wd, lp.sd, sp.split * GE::RPG + cw * GE::RPW, sp.kh * GE::KSD, lane);
+        s.wd.load(lp.wd, lp.sd, GE::partial_row(sp.split, cw * GE::RPW), sp.kh * GE::KSD, lane);
     };
 
     constexpr int KV_CUT = NR / 2, WG_CUT = 2 * GE::RGW / 3;
@@ -1278,7 +1283,7 @@ __device__ __forceinline__ void comm_role(const FusedDecodeArgs &a, Lds<GE> &sm,
         mark();
         wg_barrier();
         mark();
-        if (ct < GE::RPG) st_slot(xc, GE::XO + sp.kh * GE::HIDDEN + hidden_slot(sp.split * GE::RPG + ct), sm.pub[ct], tag, false);
+        if (ct < GE::RPG) st_slot(xc, GE::XO + sp.kh * GE::HIDDEN + hidden_slot(GE::partial_row(sp.split, ct)), sm.pub[ct], tag, false);
 
         // ── into the gate|up phase: hidden += O rows (reference src/hf/emitter.rs:787) ──
         ps.where = 5u | (uint32_t)l << 4 | (uint32_t)wg << 12;
@@ -1297,7 +1302,7 @@ __device__ __forceinline__ void comm_role(const FusedDecodeArgs &a, Lds<GE> &sm,
         mark();
         wg_barrier();
         mark();
-        if (ct < GE::RPG) st_slot(xc, GE::XH + sp.kh * GE::HIDDEN + hidden_slot(sp.split * GE::RPG + ct), sm.pub[ct], tag, false);
+        if (ct < GE::RPG) st_slot(xc, GE::XH + sp.kh * GE::HIDDEN + hidden_slot(GE::partial_row(sp.split, ct)), sm.pub[ct], tag, false);
     }
 
     if (a.head_w) {
