@@ -49,6 +49,9 @@ struct FusedDecodeArgs {
     int32_t *out_tokens;
     int out_cap;
     int advance;
+    // 1: take every exchange through memory, as a step does whose workgroups the placement check does not
+    // find dealt to the dies round-robin (for tests of that path; the host sets it from HOMURA_WHOLE_STEP_FAR)
+    int far_only;
     // Optional phase trace (nullptr = off; room for FUSED_TRACE_WGS workgroups x (11 n_layers + 2) entries):
     // every workgroup stores, in its own row, the 100 MHz device clock at 11 points per
     // layer - both barriers of the Q|K|V, attention, O, gate|up and down phases, and the end of the fold

@@ -19,11 +19,18 @@
 //  * The four communication wavefronts of a workgroup do all the polling and publishing (loads return
 //    to a wavefront in issue order, so a poll issued behind a weight prefetch would wait for HBM), stage
 //    the phase input in LDS, and meet the compute wavefronts at two workgroup barriers per phase.
+//  * The workgroups of a KV head (one die when there are as many KV heads as dies) form a group, and the
+//    groups split the layer like tensor-parallel ranks: Q|K|V and gate|up by rows (a group computes its
+//    own heads' rows and a contiguous share of the SiLU*up values), O and down by K (a group multiplies
+//    the K slice it produced itself for every output row). What a group's phases hand to each other
+//    stays in the group; only the partial hidden increments cross groups, and they are added up on the
+//    way into the next phase.
 //
 // Six exchanges per layer: hidden -> (Q|K|V rows) -> (attention partials per cache split) ->
-// (folded heads) -> (O rows) -> (SiLU*up) -> (down rows). The arithmetic and its order are those of
-// gemv_bf16.hip and attention.hip (the GEMV phases bit for bit; attention splits the cache into
-// NWG / kv_heads pieces instead of 64-row chunks).
+// (folded heads) -> (partial O rows, summed over the groups) -> (SiLU*up) -> (partial down rows, summed).
+// The arithmetic is that of gemv_bf16.hip and attention.hip: Q|K|V and gate|up rows bit for bit, O and
+// down rows as sums of per-group partial dot products, attention with the cache split into
+// NWG / kv_heads pieces instead of 64-row chunks.
 //
 // Every wait is a bounded spin: on a timeout the workgroup records a status word, stops waiting,
 // and still walks through the remaining barriers, so the grid always drains.
@@ -1027,7 +1034,7 @@ __device__ __forceinline__ void comm_role(const FusedDecodeArgs &a, Lds<GE> &sm,
             }
             if (on[u]) mine = mine && __uint_as_float(w[u].x) == r0 && __uint_as_float(w[u].z) == r1;
         }
-        die_ok = __all(mine) && !__any(ps.failed);
+        die_ok = __all(mine) && !__any(ps.failed) && !a.far_only;
         if (!die_ok && wg == 0 && ct == 0) atomicAdd(a.ctl + 2, 1u);  // steps that ran without die-local traffic
     }
     const bool near_g = die_ok && GE::GROUP_ON_XCD;  // a KV head's workgroups talk through their die's L2

@@ -37,6 +37,13 @@ void precompute_rope_cos_sin(int head_dim, int max_seq_len, double theta, std::v
         }
 }
 
+// HOMURA_WHOLE_STEP_FAR=1 (read when the plan is built): the whole-step kernel takes every exchange through
+// memory, as it does when it does not find its workgroups dealt to the dies round-robin.
+int whole_step_far_only() {
+    const char *e = std::getenv("HOMURA_WHOLE_STEP_FAR");
+    return e && std::atoi(e) != 0 ? 1 : 0;
+}
+
 }  // namespace
 
 std::unique_ptr<HfModel> HfModel::create(hm_ctx *ctx, const TransformerConfig &cfg,
@@ -607,6 +614,7 @@ int HfModel::emit_transformer_plan() {
             f.bytes_per_kv_row = L * 2.0 * kvh * hd * 2;
             const FusedShape fs{(int)hidden, (int)H, (int)kvh, (int)hd, (int)inter};
             const size_t hidden_out_slot = ls[L - 1].hidden_out;
+            const int far_only = whole_step_far_only();
             f.fn = [=](const StepContext &sc) -> int {
                 FusedDecodeArgs fa{};
                 fa.layers = reinterpret_cast<const FusedLayerPtrs *>(scr->fused_layers.ptr());
@@ -624,6 +632,7 @@ int HfModel::emit_transformer_plan() {
                 fa.xch = scr->fused_xch.as<unsigned char>();
                 fa.ctl = scr->fused_ctl.as<uint32_t>();
                 fa.trace = scr->fused_trace ? scr->fused_trace.as<unsigned long long>() : nullptr;
+                fa.far_only = far_only;
                 if (with_head) {
                     fa.head_w = sc.pool[lm_head]->as<uint16_t>();
                     fa.head_norm = sc.pool[final_norm]->as<float>();
@@ -1145,6 +1154,7 @@ int HfModel::emit_transformer_plan_quant() {
             const FusedShape fshape{(int)hidden, (int)H, (int)kvh, (int)hd, (int)inter, fused_wf_};
             const size_t hidden_out_slot = ls[L - 1].hidden_out;
             const size_t cos_slot = cos_s, sin_slot = sin_s;
+            const int far_only = whole_step_far_only();
             f.fn = [=](const StepContext &sc) -> int {
                 FusedDecodeArgs fa{};
                 fa.layers = reinterpret_cast<const FusedLayerPtrs *>(scr->fused_layers.ptr());
@@ -1162,6 +1172,7 @@ int HfModel::emit_transformer_plan_quant() {
                 fa.xch = scr->fused_xch.as<unsigned char>();
                 fa.ctl = scr->fused_ctl.as<uint32_t>();
                 fa.trace = scr->fused_trace ? scr->fused_trace.as<unsigned long long>() : nullptr;
+                fa.far_only = far_only;
                 return decode_fused_launch(sc.ctx, fshape, fa, sc.plan->kv_cache_len() + 1);
             };
             k.launches.push_back(std::move(f));

@@ -220,6 +220,36 @@ def test_qwen3_0p6b_shape_against_per_projection_path(ctx):
     gm.close()
 
 
+@pytest.mark.parametrize("shape", ["small", "qwen3_0p6b"])
+def test_exchanges_through_memory_when_placement_is_not_die_local(ctx, monkeypatch, shape):
+    """The path a step takes when the kernel does not find its workgroups dealt to the dies round-robin (no
+    die-local stores, the relays publish their sums through memory), forced from the host: same logits and
+    tokens as with die-local exchanges, and the trace's last word says which path ran."""
+    cfg = synth_model.SMALL_WS if shape == "small" else synth_model.QWEN3_0P6B
+    rows = 150 if shape == "small" else 700
+    weights = synth_model.synth_weights(cfg, 777)
+    kv = synth_model.synth_kv(cfg, 8, rows)
+    ids = synth.token_ids(9, 4, cfg.vocab_size)
+    out = {}
+    for far in ("1", "0"):
+        monkeypatch.setenv("HOMURA_WHOLE_STEP_FAR", far)
+        gm = synth_model.build_model(ctx, cfg, weights, rows + 64)
+        assert gm.whole_step_available() and gm.whole_step()
+        gm.set_prefill_min(0)
+        gm.init_kv_cache(kv, rows)
+        gm.whole_step_trace()          # switches recording on
+        logits = gm.run_kv(ids)
+        tokens = gm.generate_greedy(ids[:1], 24)
+        gm.whole_step_status()
+        trace = gm.whole_step_trace()
+        out[far] = (logits, tokens, int(trace[-1]))
+        gm.close()
+    assert out["1"][2] == 0
+    say(f"{shape}: die-local exchanges in the unforced run: {out['0'][2]}")
+    assert mf.rel_err(out["1"][0], out["0"][0]) < 1e-5   # the same sums in the same order
+    assert np.array_equal(out["1"][1], out["0"][1])
+
+
 def test_unserved_shapes_keep_the_per_projection_path(ctx):
     cfg = synth_model.TINY
     weights = synth_model.synth_weights(cfg, 4242)
