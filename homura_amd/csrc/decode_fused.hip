@@ -416,6 +416,23 @@ __device__ __forceinline__ float dot4_bytes(uint32_t w, const float *xv, float s
     return s;
 }
 
+// sum_j q_j x_j of half a block with the quants used as stored (Q8_0: biased to unsigned); xv holds the half's
+// 16 activations in the order its quant bytes use them (Rows::x_index)
+template <bool Q4>
+__device__ __forceinline__ float half_block_dot(const uint32_t *qw, const float *xv) {
+    float sum;
+    if constexpr (Q4) {
+        const uint32_t w0 = qw[0], w1 = qw[1];
+        sum = dot4_bytes(w1 & 0x0F0F0F0Fu, xv + 4, dot4_bytes(w0 & 0x0F0F0F0Fu, xv, 0.f));
+        sum = dot4_bytes((w1 >> 4) & 0x0F0F0F0Fu, xv + 12, dot4_bytes((w0 >> 4) & 0x0F0F0F0Fu, xv + 8, sum));
+    } else {
+        sum = 0.f;
+#pragma unroll
+        for (int e = 0; e < 4; e++) sum = dot4_bytes(qw[e] ^ 0x80808080u, xv + 4 * e, sum);  // int8 -> biased unsigned
+    }
+    return sum;
+}
+
 template <int WF, int R, int K>
 struct Rows {
     static constexpr bool Q4 = WF == FUSED_WF_Q4_0;
@@ -468,17 +485,7 @@ struct Rows {
         for (int c = 0; c < C; c++)
 #pragma unroll
             for (int r = 0; r < R; r++) {
-                float sum;
-                if constexpr (Q4) {
-                    const uint32_t w0 = q[r][c][0], w1 = q[r][c][1];
-                    sum = dot4_bytes(w1 & 0x0F0F0F0Fu, xv[c] + 4, dot4_bytes(w0 & 0x0F0F0F0Fu, xv[c], 0.f));
-                    sum = dot4_bytes((w1 >> 4) & 0x0F0F0F0Fu, xv[c] + 12, dot4_bytes((w0 >> 4) & 0x0F0F0F0Fu, xv[c] + 8, sum));
-                } else {
-                    sum = 0.f;
-#pragma unroll
-                    for (int e = 0; e < 4; e++) sum = dot4_bytes(q[r][c][e] ^ 0x80808080u, xv[c] + 4 * e, sum);  // int8 -> biased unsigned
-                }
-                v[r] += f16_bits_to_f32((uint16_t)d[r][c]) * (sum - off[c]);
+                v[r] += f16_bits_to_f32((uint16_t)d[r][c]) * (half_block_dot<Q4>(q[r][c], xv[c]) - off[c]);
             }
     }
     __device__ __forceinline__ void dots_normed(const float *hx, const float *nw, float inv, int lane, float (&v)[R]) const {
@@ -546,23 +553,6 @@ struct SliceRows<FUSED_WF_BF16, R, KS, KTOT> {
         for (int q = 0; q < Q; q++) v[q] += dpp_move<0x140, 0xF>(v[q], 0.f);
     }
 };
-
-// sum_j q_j x_j of half a block with the quants used as stored (Q8_0: biased to unsigned), xv in the order
-// of Rows::x_index
-template <bool Q4>
-__device__ __forceinline__ float half_block_dot(const uint32_t *qw, const float *xv) {
-    float sum;
-    if constexpr (Q4) {
-        const uint32_t w0 = qw[0], w1 = qw[1];
-        sum = dot4_bytes(w1 & 0x0F0F0F0Fu, xv + 4, dot4_bytes(w0 & 0x0F0F0F0Fu, xv, 0.f));
-        sum = dot4_bytes((w1 >> 4) & 0x0F0F0F0Fu, xv + 12, dot4_bytes((w0 >> 4) & 0x0F0F0F0Fu, xv + 8, sum));
-    } else {
-        sum = 0.f;
-#pragma unroll
-        for (int e = 0; e < 4; e++) sum = dot4_bytes(qw[e] ^ 0x80808080u, xv + 4 * e, sum);  // int8 -> biased unsigned
-    }
-    return sum;
-}
 
 template <int WF, int R, int KS, int KTOT>
 struct SliceRows {

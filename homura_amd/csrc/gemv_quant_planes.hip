@@ -12,6 +12,8 @@
 // trip in flight while this one is multiplied.
 #include "gemv_quant_planes.h"
 
+#include <algorithm>
+
 #include "hm_common.h"
 #include "quant_formats.h"
 
@@ -463,6 +465,138 @@ __global__ __launch_bounds__(PTHREADS) void gemv_q4_0_halves_kernel(const float 
         if (trip + d * nwaves < ntrips) consume(qn[d], sn[d], trip + d * nwaves);
 }
 
+// Q4_0, tall matrices, no fused light ops: a lane's unit is a whole block (one 16-byte and one 2-byte load for
+// 32 weights). A trip is two runs of UPL * 64 consecutive blocks = 2 * RB whole rows; a lane takes the same block
+// position in both runs, so the block's activations, which stay in LDS (times 2^9, a block's 32 floats 36
+// apart so that the sixteen lanes of a 16-byte LDS read hit sixteen different bank groups), are read once
+// for two blocks of weights. The registers hold only the trips in flight.
+template <int UPL, int RB>
+__global__ __launch_bounds__(PTHREADS) void gemv_q4_0_blocks_kernel(const float *__restrict__ x, const uint8_t *__restrict__ quants,
+                                                                    const uint16_t *__restrict__ scales, float *__restrict__ out,
+                                                                    int K, int N) {
+    constexpr int XPAD = 36, TR = 2 * RB;  // rows of a trip
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    float *xs = reinterpret_cast<float *>(smem);  // [nb][XPAD]: 32 activations * 2^9, then 8 * their sum
+    const int tid = threadIdx.x, lane = tid & (WAVE - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(tid / WAVE);
+    const int nb = K / 32;  // == UPL * 64 / RB
+    const int gw = blockIdx.x * PWAVES + wave, nwaves = gridDim.x * PWAVES;
+    const int ntrips = (N + TR - 1) / TR;
+    int urow[UPL], ublk[UPL];
+#pragma unroll
+    for (int u = 0; u < UPL; u++) {
+        const int f = u * WAVE + lane;
+        urow[u] = f / nb;
+        ublk[u] = f % nb;
+    }
+    constexpr int D = 2;  // trips of a wavefront in flight
+    u32x4 qn[D][2][UPL];
+    uint32_t sn[D][2][UPL];
+    auto request = [&](u32x4(&q)[2][UPL], uint32_t(&sc)[2][UPL], int trip) {
+#pragma unroll
+        for (int h = 0; h < 2; h++)
+#pragma unroll
+            for (int u = 0; u < UPL; u++) {
+                const int row = min(trip * TR + h * RB + urow[u], N - 1);  // rows past the end re-read the last one
+                const size_t blk = (size_t)row * nb + ublk[u];
+                q[h][u] = ld128_stream(quants + blk * 16);
+                sc[h][u] = __builtin_nontemporal_load((global_u16_ptr)(scales + blk));
+            }
+    };
+    // activations first (loads return in issue order), the first trips' weights right behind them
+    f32x4 xr[4];
+#pragma unroll
+    for (int u = 0; u < 4; u++) {
+        const int k = (tid + u * PTHREADS) * 4;
+        xr[u] = k < K ? *reinterpret_cast<const f32x4 *>(x + k) : f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+    int trip = gw;  // the trip in buffer 0; buffer d holds trip + d * nwaves
+#pragma unroll
+    for (int d = 0; d < D; d++)
+        if (trip + d * nwaves < ntrips) request(qn[d], sn[d], trip + d * nwaves);
+#pragma unroll
+    for (int u = 0; u < 4; u++) {
+        const int k = (tid + u * PTHREADS) * 4;
+        if (k < K) *reinterpret_cast<f32x4 *>(xs + (k >> 5) * XPAD + (k & 31)) = xr[u] * NIBBLE_FP8_UNIT;
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");  // LDS only: the weight loads stay in flight
+    for (int b = tid; b < nb; b += PTHREADS) {
+        float sx = 0.f;
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const f32x4 v = *reinterpret_cast<const f32x4 *>(xs + b * XPAD + 4 * j);
+            sx += (v.x + v.y) + (v.z + v.w);
+        }
+        xs[b * XPAD + 32] = sx * (8.f / NIBBLE_FP8_UNIT);
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    auto consume = [&](const u32x4(&qc)[2][UPL], const uint32_t(&sc)[2][UPL], int t) {
+        float a[TR];
+#pragma unroll
+        for (int r = 0; r < TR; r++) a[r] = 0.f;
+#pragma unroll
+        for (int u = 0; u < UPL; u++) {
+            int xoff = ublk[u] * XPAD;
+            asm volatile("" : "+v"(xoff));  // read again in every trip: hoisted out of the loop the activations would fill the registers
+            const float *xb = xs + xoff;
+            float s[2][2] = {{0.f, 0.f}, {0.f, 0.f}};  // two chains a block
+#pragma unroll
+            for (int j = 0; j < 4; j++) {  // byte i of word j: low nibble = weight 4 j + i, high nibble = weight 16 + 4 j + i
+                const f32x4 lo = *reinterpret_cast<const f32x4 *>(xb + 4 * j);
+                const f32x4 hi = *reinterpret_cast<const f32x4 *>(xb + 16 + 4 * j);
+                const float xl[4] = {lo.x, lo.y, lo.z, lo.w}, xh[4] = {hi.x, hi.y, hi.z, hi.w};
+#pragma unroll
+                for (int h = 0; h < 2; h++) {
+                    s[h][0] = dot4_nibbles(qc[h][u][j] & 0x0F0F0F0Fu, xl, s[h][0]);
+                    s[h][1] = dot4_nibbles((qc[h][u][j] >> 4) & 0x0F0F0F0Fu, xh, s[h][1]);
+                }
+            }
+            const float sx8 = xb[32];
+#pragma unroll
+            for (int h = 0; h < 2; h++) {
+                const float v = f16_bits_to_f32((uint16_t)sc[h][u]) * ((s[h][0] + s[h][1]) - sx8);
+#pragma unroll
+                for (int r = 0; r < RB; r++) a[h * RB + r] += (RB == 1 || urow[u] == r) ? v : 0.f;
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < TR; r++) a[r] += dpp_move<0xB1, 0xF>(a[r], 0.f);
+#pragma unroll
+        for (int r = 0; r < TR; r++) a[r] += dpp_move<0x4E, 0xF>(a[r], 0.f);
+#pragma unroll
+        for (int r = 0; r < TR; r++) a[r] += dpp_move<0x141, 0xF>(a[r], 0.f);
+#pragma unroll
+        for (int r = 0; r < TR; r++) a[r] += dpp_move<0x140, 0xF>(a[r], 0.f);
+#pragma unroll
+        for (int r = 0; r < TR; r++) a[r] += dpp_move<0x142, 0xA>(a[r], 0.f);
+#pragma unroll
+        for (int r = 0; r < TR; r++) a[r] += dpp_move<0x143, 0xC>(a[r], 0.f);
+        // lane 63 holds the totals; it stores the rows
+#pragma unroll
+        for (int r = 0; r < TR; r++)
+            if (lane == WAVE - 1 && t * TR + r < N) out[(size_t)t * TR + r] = a[r];
+    };
+    // steady state: every buffer is multiplied and asked for again, D trips on, with no condition in the way
+    while (trip + (2 * D - 1) * nwaves < ntrips) {
+#pragma unroll
+        for (int d = 0; d < D; d++) {
+            consume(qn[d], sn[d], trip + d * nwaves);
+            request(qn[d], sn[d], trip + (D + d) * nwaves);
+        }
+        trip += D * nwaves;
+    }
+#pragma unroll
+    for (int d = 0; d < D; d++)
+        if (trip + d * nwaves < ntrips) consume(qn[d], sn[d], trip + d * nwaves);
+    trip += D * nwaves;
+#pragma unroll
+    for (int d = 0; d < D; d++)
+        if (trip + d * nwaves < ntrips) request(qn[d], sn[d], trip + d * nwaves);
+#pragma unroll
+    for (int d = 0; d < D; d++)
+        if (trip + d * nwaves < ntrips) consume(qn[d], sn[d], trip + d * nwaves);
+}
+
 // planes -> raw blocks (the inverse, for checks)
 template <int QT>
 __global__ __launch_bounds__(256) void unpack_planes_kernel(const uint8_t *__restrict__ quants, const uint16_t *__restrict__ scales,
@@ -558,6 +692,28 @@ int planes_launch(hm_ctx *ctx, const char *name, const float *d_x, const uint8_t
     const bool fused = fuse.x2 || fuse.res_in || fuse.norm_w || fuse.res_out_add || fuse.cand_v;
     // Q4_0 at the LM-head shape: the half-block-per-lane kernel
     const int nblk = K / 32;
+    // Q4_0, tall matrices with rows of 2048, 3072 or 4096: the whole-block-per-lane kernel (35.6 us against 39.5 of
+    // the half-block kernel at 2048 -> 151936; 25 against 31 us and 30 against 44 us of the quarter-block kernel at
+    // 3072 and 4096 -> 65536); narrower rows are no faster that way (29-30 us at 1536 -> 151936 either way)
+    if (q4 && !fused && N >= 8 * PWAVES * ctx->num_cus && (nblk == 64 || nblk == 96 || nblk == 128)) {
+        const int rb = nblk == 96 ? 2 : 1;
+        const int ntrips = (N + 2 * rb - 1) / (2 * rb);
+        const int want = (ntrips + PWAVES - 1) / PWAVES;
+        const int grid = std::min(want, 8 * ctx->num_cus);
+        const size_t lds = (size_t)nblk * 36 * 4 + 16;
+        for (int m = 0; m < M; m++) {
+            const float *xm = d_x + (size_t)m * K;
+            float *om = d_out + (size_t)m * N;
+            if (nblk == 64)
+                hipLaunchKernelGGL((gemv_q4_0_blocks_kernel<1, 1>), dim3(grid), dim3(PTHREADS), lds, ctx->stream, xm, quants, scales, om, K, N);
+            else if (nblk == 96)
+                hipLaunchKernelGGL((gemv_q4_0_blocks_kernel<3, 2>), dim3(grid), dim3(PTHREADS), lds, ctx->stream, xm, quants, scales, om, K, N);
+            else
+                hipLaunchKernelGGL((gemv_q4_0_blocks_kernel<2, 1>), dim3(grid), dim3(PTHREADS), lds, ctx->stream, xm, quants, scales, om, K, N);
+            HM_LAUNCH_CHECK(ctx);
+        }
+        return HM_OK;
+    }
     if (q4 && !fused && nblk % 16 == 0 && nblk / 16 <= 4 && N >= 8 * PWAVES * ctx->num_cus) {
         const int ntrips = (N + 1) / 2;
         const int want = (ntrips + PWAVES - 1) / PWAVES;

@@ -175,7 +175,8 @@ def test_quant_planes_hold_the_blocks_bit_for_bit(ctx, oracle, kind):
                                         ("q8_0", 1, 32, 5), ("q8_0", 1, 96, 1), ("q8_0", 1, 1024, 6144),
                                         ("q4_0", 3, 2048, 260), ("q4_0", 1, 32, 7), ("q4_0", 1, 3072, 1024),
                                         ("q4_0", 1, 256, 233100), ("q4_0", 1, 1792, 33333),
-                                        ("q4_0", 2, 2048, 29201), ("q4_0", 1, 4096, 14601), ("q4_0", 1, 2528, 4099)])
+                                        ("q4_0", 2, 2048, 29201), ("q4_0", 1, 4096, 14601), ("q4_0", 1, 2528, 4099),
+                                        ("q4_0", 1, 3072, 9001), ("q4_0", 1, 2048, 8193)])
 def test_quant_planes_gemv(ctx, oracle, kind, M, K, N):
     """The dequant-GEMV over the re-packed weights against the oracle on the raw blocks."""
     from homura_amd.runtime import DTYPE_Q4_0, DTYPE_Q8_0
