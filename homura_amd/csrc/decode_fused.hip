@@ -1435,6 +1435,10 @@ __global__ __launch_bounds__(FT) void decode_fused_kernel(FusedDecodeArgs a) {
 using GeoQwen3_0p6b = Geo<1024, 16, 8, 128, 3072, 256>;
 using GeoSmall = Geo<512, 4, 2, 128, 1024, 64>;
 using GeoSmallQ = Geo<1024, 8, 4, 128, 1024, 64>;
+// The same shapes with three row rounds: caches up to 1536 live rows, with an attention phase a fifth shorter.
+using GeoQwen3_0p6bShort = Geo<1024, 16, 8, 128, 3072, 256, 3>;
+using GeoSmallShort = Geo<512, 4, 2, 128, 1024, 64, 3>;
+using GeoSmallQShort = Geo<1024, 8, 4, 128, 1024, 64, 3>;
 // The same shapes with eight row rounds: twice the live cache rows (4096) for 32 more registers a lane and an
 // attention phase twice as long; taken only by steps that the four-round instances do not serve.
 using GeoQwen3_0p6bLong = Geo<1024, 16, 8, 128, 3072, 256, 8>;
@@ -1464,6 +1468,8 @@ Instance instance() {
 // live_rows = 0, the one that holds the most.
 const Instance *find_instance(const FusedShape &s, int live_rows = 1) {
     static const Instance table[] = {
+        instance<GeoQwen3_0p6bShort, FUSED_WF_BF16>(), instance<GeoQwen3_0p6bShort, FUSED_WF_Q8_0>(), instance<GeoQwen3_0p6bShort, FUSED_WF_Q4_0>(),
+        instance<GeoSmallShort, FUSED_WF_BF16>(),      instance<GeoSmallQShort, FUSED_WF_Q8_0>(),     instance<GeoSmallQShort, FUSED_WF_Q4_0>(),
         instance<GeoQwen3_0p6b, FUSED_WF_BF16>(), instance<GeoQwen3_0p6b, FUSED_WF_Q8_0>(), instance<GeoQwen3_0p6b, FUSED_WF_Q4_0>(),
         instance<GeoSmall, FUSED_WF_BF16>(),      instance<GeoSmallQ, FUSED_WF_Q8_0>(),     instance<GeoSmallQ, FUSED_WF_Q4_0>(),
         instance<GeoQwen3_0p6bLong, FUSED_WF_BF16>(), instance<GeoQwen3_0p6bLong, FUSED_WF_Q8_0>(), instance<GeoQwen3_0p6bLong, FUSED_WF_Q4_0>(),

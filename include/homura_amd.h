@@ -363,8 +363,8 @@ int hm_model_set_graph(hm_model *m, int on);
  * launch per projection; the reference dispatches 1 + 3 * layers + 1 kernels per step
  * (src/hf/emitter.rs:1016-1021). Served for bf16, all-Q8_0 and all-Q4_0 models whose shape has a kernel
  * instance (hm_model_whole_step_available); on by default then, and for bf16 models the same launch runs the
- * LM head and the greedy pick. The cache may be of any length: up to 2048 live rows a step takes the fastest
- * instance of the kernel, up to 4096 one that holds twice the rows, beyond that the per-projection path,
+ * LM head and the greedy pick. The cache may be of any length: a step takes the instance of the kernel that
+ * holds its live rows (1536, 2048 or 4096 of them; the smaller the faster), beyond 4096 the per-projection path,
  * chosen step by step. Results agree with the per-projection
  * path to f32 summation order. hm_model_whole_step_status returns HM_OK, or the error
  * left behind by a step whose workgroups stopped waiting for one another (bounded waits; the

@@ -262,11 +262,11 @@ def test_unserved_shapes_keep_the_per_projection_path(ctx):
 
 
 def test_cache_longer_than_the_kernel_serves_changes_over_and_back(ctx):
-    """The whole-step launch holds a split's cache rows in registers: an instance with four row rounds serves
-    2048 live rows of this shape, one with eight 4096. A model with a longer cache starts on the first, takes
-    the second from the step whose live rows exceed 2048, one launch per projection beyond 4096, and comes
-    back after a cache reset; the steps on either side of each change give the oracle's logits and the
-    per-projection path's tokens."""
+    """The whole-step launch holds a split's cache rows in registers: an instance with three row rounds serves
+    1536 live rows of this shape, one with four 2048, one with eight 4096. A model with a longer cache starts
+    on the first, takes the next from the step whose live rows exceed it, one launch per projection beyond
+    4096, and comes back after a cache reset; the steps on either side of each change give the oracle's
+    logits and the per-projection path's tokens."""
     cfg = dataclasses.replace(synth_model.SMALL_WS, max_position_embeddings=8192)
     weights = synth_model.synth_weights(cfg, 31)
     L = 4200
@@ -276,7 +276,7 @@ def test_cache_longer_than_the_kernel_serves_changes_over_and_back(ctx):
     om = mf.build_oracle_model(cfg, weights, L)
     assert gm.whole_step_available() and gm.whole_step() and gm.launches_per_step() == 1
     ids = synth.token_ids(33, 14, cfg.vocab_size)
-    for rows, still_whole in ((2040, True), (4088, False)):
+    for rows, still_whole in ((1528, True), (2040, True), (4088, False)):
         kv = synth_model.synth_kv(cfg, 32 + rows, rows)
         for m in (gm, plain):
             m.set_prefill_min(0)
