@@ -92,6 +92,7 @@ SIGNATURES = {
     "hm_gemv_q4_0_planes": (_I, [_P, _P, _P, _P, _I, _I, _I]),
     "hm_dequant_quant_planes": (_I, [_P, _I, _P, _P, _I, _I]),
     "hm_gemv_q6_k_f32_planes": (_I, [_P, _P, _P, _P, _I, _I, _I]),
+    "hm_test_fill_lds": (_I, [_P, C.c_uint32]),
     "hm_dequant_q8_0": (_I, [_P, _P, _P, _SZ]),
     "hm_dequant_q4_0": (_I, [_P, _P, _P, _SZ]),
     "hm_gemv_q4_k": (_I, [_P, _P, _P, _P, _I, _I, _I]),

@@ -2,6 +2,7 @@
 #include "hm_common.h"
 #include "attention.h"
 
+#include <cstdlib>
 #include <mutex>
 
 static std::mutex g_err_mutex;
@@ -100,6 +101,13 @@ int hm_alloc(hm_ctx *ctx, size_t bytes, void **d_out) {
     if (e != hipSuccess)
         return hm_set_error(ctx, HM_ERR_OOM, "hipMalloc(%zu) failed: %s", bytes,
                             hipGetErrorString(e));
+    // HOMURA_ALLOC_FILL=<byte>: every new allocation starts filled with that byte (0xFF makes every float a
+    // NaN), so that a kernel which reads memory nobody wrote shows in the results. For tests.
+    static const int fill = [] {
+        const char *v = std::getenv("HOMURA_ALLOC_FILL");
+        return v ? (int)(std::strtol(v, nullptr, 0) & 0xFF) : -1;
+    }();
+    if (fill >= 0) HM_HIP(ctx, hipMemsetAsync(*d_out, fill, bytes, ctx->stream));
     return HM_OK;
 }
 

@@ -1420,6 +1420,12 @@ __global__ __launch_bounds__(FT) void decode_fused_kernel(FusedDecodeArgs a) {
         uint64_t *dst = reinterpret_cast<uint64_t *>(sm.lp);
         const int words = a.n_layers * (int)(sizeof(FusedLayerPtrs) / 8);
         for (int i = threadIdx.x; i < words; i += FT) dst[i] = src[i];
+        // Only the workgroup that holds the new cache row stages it; the others multiply these by a weight of
+        // zero, so they must not hold whatever an earlier kernel left in LDS (0 * NaN is NaN).
+        for (int i = threadIdx.x; i < GE::HD; i += FT) {
+            sm.knew[i] = 0.f;
+            sm.vnew[i] = 0.f;
+        }
         __syncthreads();
     }
     if (wave < NCW) {

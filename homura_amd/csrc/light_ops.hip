@@ -375,7 +375,32 @@ __global__ void floor_chain_kernel(const int *__restrict__ in, int *__restrict__
     if (threadIdx.x == 0) *out = *in + 1;
 }
 
+// Fills the LDS of the CU it runs on with a word and stays for a moment, so that the grid spreads over all CUs.
+__global__ __launch_bounds__(256) void fill_lds_kernel(uint32_t word, int words) {
+    extern __shared__ uint32_t lds_words[];
+    for (int i = threadIdx.x; i < words; i += 256) lds_words[i] = word;
+    __syncthreads();
+    uint32_t x = lds_words[(threadIdx.x * 61) % words];
+    for (int i = 0; i < 200; i++) x = x * 1664525u + 1013904223u;  // a few microseconds of residence
+    if (x == 0x12345678u && words < 0) lds_words[0] = x;            // keeps the loop
+}
+
 extern "C" {
+
+int hm_test_fill_lds(hm_ctx *ctx, uint32_t word) {
+    HM_CHECK_CTX(ctx);
+    hipDeviceProp_t prop;
+    HM_HIP(ctx, hipGetDeviceProperties(&prop, ctx->device));
+    size_t bytes = prop.maxSharedMemoryPerMultiProcessor;  // the whole LDS of a CU: one workgroup a CU at a time
+    if (bytes == 0 || bytes > (size_t)160 << 10) bytes = (size_t)64 << 10;
+    if (hipFuncSetAttribute(reinterpret_cast<const void *>(fill_lds_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes) != hipSuccess) {
+        (void)hipGetLastError();
+        bytes = (size_t)64 << 10;
+    }
+    hipLaunchKernelGGL(fill_lds_kernel, dim3(8 * ctx->num_cus), dim3(256), bytes, ctx->stream, word, (int)(bytes / 4));
+    HM_LAUNCH_CHECK(ctx);
+    return HM_OK;
+}
 
 int hm_bench_launch_floor(hm_ctx *ctx, int n_kernels, int chained, int replays, float *us_per_replay) {
     HM_CHECK_CTX(ctx);

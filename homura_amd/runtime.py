@@ -99,6 +99,10 @@ class Context:
     def sync(self):
         self._check(self.lib.hm_sync(self.h))
 
+    def fill_lds(self, word: int = 0xFFFFFFFF):
+        """Test support: overwrite the LDS of every CU with `word` (default: a NaN pattern)."""
+        self._check(self.lib.hm_test_fill_lds(self.h, word))
+
     def launch_floor(self, n_kernels: int, chained: bool, replays: int = 20) -> float:
         """Microseconds per replay of a graph of n_kernels dependent one-wavefront kernels (empty, or each
         reading 4 bytes its predecessor wrote)."""

@@ -49,6 +49,13 @@ void hm_synth_q4_0(uint64_t seed, size_t n_blocks, float d_scale, uint8_t *out);
  * replayed `replays` times between two events; microseconds per replay. */
 int hm_bench_launch_floor(hm_ctx *ctx, int n_kernels, int chained, int replays, float *us_per_replay);
 
+/* Test support: writes `word` over the whole LDS of every CU (a grid of workgroups that each take a CU's LDS).
+ * LDS keeps its contents from one kernel to the next, and from one process to the next: a kernel that reads
+ * LDS it did not write works or fails by what ran before it. Filled with 0xFFFFFFFF (a NaN), any such read
+ * that reaches a result shows. Device allocations can be pre-filled the same way with the environment
+ * variable HOMURA_ALLOC_FILL=<byte>, read when the first buffer is allocated. */
+int hm_test_fill_lds(hm_ctx *ctx, uint32_t word);
+
 /* Phase trace of the latest whole-step decode launch: device-clock ticks (100 MHz) taken by workgroup
  * 0 at 11 points per layer (both workgroup barriers of the Q|K|V, attention, O, gate|up and down
  * phases; the end of the fold follows attention's second barrier) and one at the end of the kernel, then

@@ -224,6 +224,56 @@ def test_qwen3_0p6b_shape_quantised_decode_against_oracle(ctx, name):
     gm.close()
 
 
+@pytest.mark.parametrize("kind", ["q6_k", "q8_0"])
+def test_qwen3_0p6b_shape_lm_head_from_blocks_against_oracle(ctx, kind):
+    """The configurations bench.py times with the output matrix read from its blocks (re-packed into planes at
+    finalize): the Q4_K_M-style mix with a Q6_K head and the Q8_0 plan with a Q8_0 head, at Qwen3-0.6B widths
+    with a 1024-row cache. The oracle multiplies the dequantised matrix in its f32 slot: first-step logits,
+    and greedy tokens while the oracle's margin exceeds what differently taken Q8_K rounding decisions move
+    two logits by (mix only)."""
+    import dataclasses
+    import pyoracle
+    from homura_amd.runtime import DTYPE_Q8_0
+    cfg = dataclasses.replace(synth_model.QWEN3_0P6B, tie_word_embeddings=False)
+    mix = synth_model.q4_k_m_mix(cfg) if kind == "q6_k" else None
+    say(f"head from {kind} blocks: synthesising weights")
+    weights = synth_model.synth_weights(cfg, synth.SEED_CFG2 + 9, DTYPE_Q8_0, has_qk_norm=True, proj_dtypes=mix)
+    assert weights[-1][0] == "lm_head.weight"
+    if kind == "q6_k":
+        raw, code = synth.q6_k_blocks(93, cfg.vocab_size * cfg.hidden_size // 256), 6
+        dense = pyoracle.dequant_q6_k(raw)
+    else:
+        raw, code = synth.q8_0_blocks(93, cfg.vocab_size * cfg.hidden_size // 32, 0.01), 2
+        dense = pyoracle.dequant_q8_0(raw)
+    weights[-1] = ("lm_head.weight", np.ascontiguousarray(dense.reshape(cfg.vocab_size, cfg.hidden_size).T))
+    om = mf.build_oracle_model(cfg, weights, 1200, DTYPE_Q8_0, has_qk_norm=True, proj_dtypes=mix)
+    gm = HfModel(ctx, cfg, weight_dtype=DTYPE_Q8_0, has_qk_norm=True, proj_dtypes=mix)
+    for i, (_name, arr) in enumerate(weights[:-1]):
+        gm.set_weight(i, arr)
+    gm.set_lm_head_blocks(code, raw)
+    gm.finalize(1200)
+    kv = synth_model.synth_kv(cfg, synth.SEED_CFG2 + 0x101, 1024)
+    gm.init_kv_cache(kv, 1024)
+    mf.oracle_init_kv(om, kv)
+    gm.set_graph(True)
+    gm.set_prefill_min(0)
+    ids = synth.token_ids(synth.SEED_CFG2 + 0x201, 3, cfg.vocab_size)
+    got, want = gm.run_kv(ids[:1]), om.run_kv(ids[:1])
+    err = mf.rel_err(got, want)
+    say(f"head from {kind} blocks: first-step logits rel err {err:.2e}")
+    assert err < 1e-2
+    want_t, margins = om.generate_greedy(ids[1:], 12)
+    got_t = gm.generate_greedy(ids[1:], 12)
+    scale = float(np.abs(want).max())
+    thr = 2 * 1e-3 * scale if mix is not None else 0.0
+    close = np.nonzero(margins < thr)[0]
+    n_cmp = int(close[0]) if close.size else len(want_t)
+    say(f"head from {kind} blocks: min margin {margins.min():.3e} (logit scale {scale:.3e}), {n_cmp} of 12 tokens compared")
+    assert n_cmp >= 6
+    assert np.array_equal(got_t[:n_cmp], want_t[:n_cmp])
+    gm.close()
+
+
 @pytest.mark.parametrize("wdt,name", [(1, "bf16"), (2, "q8_0")])
 def test_qkv_bias_model_against_oracle(ctx, wdt, name):
     """Qwen2-style checkpoint: Q/K/V biases (slots q,[qb],k,[kb],v,[vb] of the reference's
