@@ -62,15 +62,18 @@ def rel_err(a, b, floor_frac=1e-2):
 
 
 def smoke_decode():
-    """One small decode through the HIP path on GPU 0, checked against the oracle."""
+    """One small decode through the HIP path on GPU 0 (a shape the whole-step kernel serves, on LDS that has
+    been overwritten with NaNs first), checked against the oracle."""
     import homura_amd
-    cfg = synth_model.TINY
+    cfg = synth_model.SMALL_WS
     weights = synth_model.synth_weights(cfg, 1234)
     kv = synth_model.synth_kv(cfg, 99, 40)
     prompt = synth.token_ids(5, 4, cfg.vocab_size)
     with homura_amd.Context(0) as ctx:
         print("smoke: device", ctx.device_name(), flush=True)
+        ctx.fill_lds()
         gm = synth_model.build_model(ctx, cfg, weights, 128)
+        assert gm.whole_step(), "smoke: the whole-step kernel does not serve the smoke shape"
         gm.init_kv_cache(kv, 40)
         om = build_oracle_model(cfg, weights, 128)
         oracle_init_kv(om, kv)
