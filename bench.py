@@ -119,6 +119,13 @@ def main() -> int:
         model = synth_model.build_model(ctx, cfg, weights, 2048)
         model.init_kv_cache(kv, PREFILL)
         model.set_graph(not args.no_graph)
+        # untimed: the first tokens of the same greedy run that the CPU baseline leg makes below, kept to be
+        # compared with its tokens (the cache is set up again afterwards)
+        gpu_check_tokens = None
+        if not args.no_cpu_baseline:
+            model.generate_greedy(prompt[:1], 4)  # the baseline leg's warm-up, which moves its cache on
+            gpu_check_tokens = [int(t) for t in model.generate_greedy(prompt[1:2], min(16, args.cpu_tokens))]
+            model.init_kv_cache(kv, PREFILL)
         setup_s = time.perf_counter() - t_setup
 
         if args.warmup:
@@ -308,13 +315,18 @@ def main() -> int:
         mf.oracle_init_kv(om, kv)
         om.generate_greedy(prompt[:1], 4)  # warm-up
         t0 = time.perf_counter()
-        om.generate_greedy(prompt[1:2], args.cpu_tokens)
+        cpu_tokens, _margins = om.generate_greedy(prompt[1:2], args.cpu_tokens)
         cpu_s = time.perf_counter() - t0
+        n_chk = len(gpu_check_tokens)
+        same = 0
+        while same < n_chk and int(cpu_tokens[same]) == gpu_check_tokens[same]:
+            same += 1
         cpu_baseline = {
             "value": round(args.cpu_tokens / cpu_s, 2), "unit": "tok/s",
             "cores": pyoracle.num_threads(), "kind": "port",
             "sample": f"{args.cpu_tokens} greedy tokens of the same model from the same 1024-row cache "
                       f"(C oracle built for {pyoracle.isa()}, OpenMP, f32 KV values rounded to bf16)",
+            "gpu_tokens_identical": f"{same} of the first {n_chk} tokens of that run, taken on the GPU before the timed region",
         }
 
     out = {
