@@ -241,7 +241,9 @@ __device__ __forceinline__ void select_sort_draw(SelectShared &sh, const SampleA
     // normalise, min_p (the maximum probability is exp(0) / sum), pad to the sort size
     const float max_prob = 1.0f / sum;
     const float threshold = cfg.min_p * max_prob;
-    if (tid < SAMPLE_MAX_K) {
+    int sort_n = 2;  // the power of two that holds the candidates: 64 for the default top_k of 50, not 1024
+    while (sort_n < nc) sort_n <<= 1;
+    if (tid < sort_n) {
         if (tid < nc) {
             float p = cand_p[tid] / sum;
             if (cfg.min_p > 0.0f && p < threshold) p = 0.0f;
@@ -252,11 +254,11 @@ __device__ __forceinline__ void select_sort_draw(SelectShared &sh, const SampleA
         }
     }
     __syncthreads();
-    // bitonic sort of 1024 (probability descending, index ascending among equals)
-    for (int k = 2; k <= SAMPLE_MAX_K; k <<= 1)
+    // bitonic sort of sort_n (probability descending, index ascending among equals)
+    for (int k = 2; k <= sort_n; k <<= 1)
         for (int j = k >> 1; j > 0; j >>= 1) {
             const int partner = tid ^ j;
-            if (partner > tid) {
+            if (partner > tid && tid < sort_n) {
                 const float pa = cand_p[tid], pb = cand_p[partner];
                 const int ia = cand_i[tid], ib = cand_i[partner];
                 const bool up = (tid & k) == 0;  // this pair ends in candidate order
