@@ -1208,10 +1208,11 @@ __device__ __forceinline__ void comm_role(const FusedDecodeArgs &a, Lds<GE> &sm,
         mark();
         if (sp.split < sp.nsl) {
             // merge the compute wavefronts' partials (one output per thread) and publish the split's
-            // (o, max, sum): o = sum_w exp(m_w - M) * (sum over w's row groups), in wavefront order
-            for (int i = ct; i < GE::PART; i += CT) {
-                const int g = i < G * HD ? i / HD : (i - G * HD) / 2;
-                float mw[NCW], M = -INFINITY;
+            // (o, max, sum): o = sum_w exp(m_w - M) * (sum over w's row groups), in wavefront order. The
+            // threads of a head's first two outputs also publish the head's (max, sum): same weights.
+            for (int i = ct; i < G * HD; i += CT) {
+                const int g = i / HD, d = i % HD;
+                float mw[NCW], f[NCW], M = -INFINITY;
 #pragma unroll
                 for (int w = 0; w < NCW; w++) {
                     mw[w] = sm.wstat[w][g][0];
@@ -1220,19 +1221,22 @@ __device__ __forceinline__ void comm_role(const FusedDecodeArgs &a, Lds<GE> &sm,
                 float v = 0.f;
 #pragma unroll
                 for (int w = 0; w < NCW; w++) {
-                    const float f = mw[w] == -INFINITY ? 0.f : __expf(mw[w] - M);
-                    float t;
-                    if (i < G * HD) {
-                        t = 0.f;
+                    f[w] = mw[w] == -INFINITY ? 0.f : __expf(mw[w] - M);
+                    float t = 0.f;
 #pragma unroll
-                        for (int sb = 0; sb < GE::RPI; sb++) t += sm.part[w * GE::RPI + sb][g][i % HD];
-                    } else {
-                        t = sm.wstat[w][g][1];
-                    }
-                    v += f * t;
+                    for (int sb = 0; sb < GE::RPI; sb++) t += sm.part[w * GE::RPI + sb][g][d];
+                    v += f[w] * t;
                 }
-                if (i >= G * HD && ((i - G * HD) & 1) == 0) v = M;
                 st_slot(lp, sp.split * GE::PART + i, v, tag, near_g);
+                if (d < 2) {
+                    float st = M;
+                    if (d == 1) {
+                        st = 0.f;
+#pragma unroll
+                        for (int w = 0; w < NCW; w++) st += f[w] * sm.wstat[w][g][1];
+                    }
+                    st_slot(lp, sp.split * GE::PART + G * HD + 2 * g + d, st, tag, near_g);
+                }
             }
         }
 
@@ -1268,8 +1272,8 @@ __device__ __forceinline__ void comm_role(const FusedDecodeArgs &a, Lds<GE> &sm,
             wave_sum_n<2 * FU + 1>(red);
             float mine = 0.f;
 #pragma unroll
-            for (int e = 0; e < GE::FPW; e++) mine = lane == e ? red[1 + e] / red[0] : mine;
-            if (lane < GE::FPW) st_slot(la, o0 + lane, mine, tag, near_g);
+            for (int e = 0; e < GE::FPW; e++) mine = lane == e ? red[1 + e] : mine;
+            if (lane < GE::FPW) st_slot(la, o0 + lane, mine / red[0], tag, near_g);
         }
         mark();
 
