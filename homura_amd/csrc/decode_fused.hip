@@ -1242,7 +1242,63 @@ __device__ __forceinline__ void comm_role(const FusedDecodeArgs &a, Lds<GE> &sm,
 
         // ── fold the splits of this KV head for FPW of its outputs (one wavefront) ──
         ps.where = 3u | (uint32_t)l << 4 | (uint32_t)wg << 12;
-        if (cwv == 0) {
+        constexpr bool FOLD_HALVES = GE::SPH <= 32 && (GE::FPW / 2) % 2 == 0;
+        if (cwv == 0 && FOLD_HALVES) {
+            // lanes 0-31 fold the first half of the workgroup's outputs over the (at most 32) splits, lanes 32-63
+            // the second half: half the loads and half the sums a lane, and a sum ends inside 32 lanes
+            constexpr int HU = GE::FPW / 4;  // 16-byte units of outputs per lane
+            const int o0 = sp.split * GE::FPW;
+            const int t = o0 / HD, d0 = o0 % HD;
+            const int half = lane >> 5, sl = lane & 31;
+            const int pbase = sl * GE::PART;
+            int unit[HU + 1];
+            bool on[HU + 1];
+            u32x4 w[HU + 1];
+#pragma unroll
+            for (int u = 0; u < HU; u++) {
+                unit[u] = (pbase + t * HD + d0) / 2 + half * HU + u;
+                on[u] = sl < sp.nsl;
+            }
+            unit[HU] = (pbase + G * HD + 2 * t) / 2;
+            on[HU] = sl < sp.nsl;
+            poll_units<HU + 1>(ps, lp, unit, on, tag, w);
+            const float m_s = on[HU] ? __uint_as_float(w[HU].x) : -INFINITY;
+            const float l_s = on[HU] ? __uint_as_float(w[HU].z) : 0.f;
+            const float m = wave_max(m_s);  // both halves hold the same maxima
+            const float f = on[HU] ? __expf(m_s - m) : 0.f;
+            float red[2 * HU + 1];  // the sum of the splits' sums, then this half's weighted outputs
+            red[0] = f * l_s;
+#pragma unroll
+            for (int u = 0; u < HU; u++) {
+                red[1 + 2 * u] = f * __uint_as_float(w[u].x);
+                red[2 + 2 * u] = f * __uint_as_float(w[u].z);
+            }
+#pragma unroll
+            for (int i = 0; i < 2 * HU + 1; i++) red[i] += dpp_move<0xB1, 0xF>(red[i], 0.f);
+#pragma unroll
+            for (int i = 0; i < 2 * HU + 1; i++) red[i] += dpp_move<0x4E, 0xF>(red[i], 0.f);
+#pragma unroll
+            for (int i = 0; i < 2 * HU + 1; i++) red[i] += dpp_move<0x141, 0xF>(red[i], 0.f);
+#pragma unroll
+            for (int i = 0; i < 2 * HU + 1; i++) red[i] += dpp_move<0x140, 0xF>(red[i], 0.f);
+#pragma unroll
+            for (int i = 0; i < 2 * HU + 1; i++) red[i] += dpp_move<0x142, 0xA>(red[i], 0.f);  // lanes 31 and 63: the halves' totals
+            const int e = lane % (2 * HU);  // lane l < FPW publishes output l: half l / (2 HU), element l % (2 HU)
+            float num = 0.f, den = 0.f;
+#pragma unroll
+            for (int hh = 0; hh < 2; hh++) {
+                const float d0v = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(red[0]), 31 + 32 * hh));
+#pragma unroll
+                for (int k = 0; k < 2 * HU; k++) {
+                    const float nv = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(red[1 + k]), 31 + 32 * hh));
+                    if (lane / (2 * HU) == hh && e == k) {
+                        num = nv;
+                        den = d0v;
+                    }
+                }
+            }
+            if (lane < GE::FPW) st_slot(la, o0 + lane, num / den, tag, near_g);
+        } else if (cwv == 0) {
             constexpr int FU = GE::FPW / 2;
             const int o0 = sp.split * GE::FPW;  // first output, counted inside the KV head's G * HD
             const int t = o0 / HD, d0 = o0 % HD;
