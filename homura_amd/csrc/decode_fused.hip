@@ -1036,7 +1036,12 @@ __device__ __forceinline__ void comm_role(const FusedDecodeArgs &a, Lds<GE> &sm,
     // the L2. Without die-local placement the relay's stores go through to memory.
     auto relay_sum = [&](unsigned char *par, int off, uint32_t tag) -> const unsigned char * {
         unsigned char *rel = par + (size_t)(GE::RELAY0 + xcd * GE::RELAY_SLOTS + (off == GE::XH ? 0 : GE::HIDDEN)) * 8;
-        if (cwv == 3) {  // wavefront 0 may still be folding
+        {
+            // All four wavefronts poll for the same share, a quarter of a round trip apart (whichever sees it
+            // complete first publishes the sums; the others publish the same values again): a share is noticed sooner.
+            if (cwv == 1) __builtin_amdgcn_s_sleep(4);
+            if (cwv == 2) __builtin_amdgcn_s_sleep(8);
+            if (cwv == 3) __builtin_amdgcn_s_sleep(12);
             constexpr int per = GE::HIDDEN / 2 / GE::NPX;
             int unit[GE::KVH];
             bool on[GE::KVH];
