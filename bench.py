@@ -4,7 +4,8 @@
 vocab 151936, tied bf16 LM head; KV cache pre-filled to 1024 rows; synthetic seeded weights).
 
 A "step" is one decode token: embed -> 28 x (QKV+QK-norm+RoPE+append, attention+O, MLP) -> LM head
--> greedy pick, all on the GPU, replayed from one HIP graph, the pick fed back on the device.
+-> greedy pick, all on the GPU, the pick fed back on the device. A step of many launches is replayed from one
+HIP graph; the whole-step kernel makes a step one launch, and the library then launches it directly.
 
     python bench.py --gpus 1 --steps 64 --warmup 8
 
@@ -337,7 +338,7 @@ def main() -> int:
         "dtype": "bf16 weights / f32 accumulate", "data": "synthetic",
         "config": {"workload": "Qwen3-0.6B-shape decode: 28 layers, hidden 1024, 16q/8kv heads x 128, "
                                "SwiGLU 3072, vocab 151936 tied head, KV cache 1024+ rows, batch 1, greedy",
-                   "kv_rows_start": pos0, "graph_replay": not args.no_graph,
+                   "kv_rows_start": pos0, "graph_replay": (not args.no_graph) and launches > 2,
                    "kernel_launches_per_step": launches},
         "roofline": roofline,
         "cpu_baseline": cpu_baseline,

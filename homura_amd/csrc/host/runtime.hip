@@ -483,7 +483,9 @@ int ExecutionPlan::run_kv(const std::vector<Buffer *> &inputs, std::vector<Buffe
     if ((rc = kv_cache_->note_appended(1)) != HM_OK) return rc;  // "KV cache full"
     if ((rc = bind(inputs, weights)) != HM_OK) return rc;
     if (pre_run_ && (rc = pre_run_()) != HM_OK) return rc;
-    if (use_graph_) {
+    // A graph pays when a step is many launches. A step of one or two is quicker launched directly: the replay
+    // of a one-node graph costs more on the GPU's queue than the kernel's own dispatch packet.
+    if (use_graph_ && launches_per_step() > 2) {
         if (!graph_exec_) {
             if (graph_) {
                 (void)hipGraphDestroy(graph_);

@@ -355,8 +355,9 @@ int hm_model_init_kv_cache(hm_model *m, const float *const *h_kv, int seq_len);
 int hm_model_reset_kv_cache(hm_model *m);  /* src/runtime.rs:1941-1945 */
 int hm_model_kv_cache_len(hm_model *m);    /* src/runtime.rs:1948-1950 */
 
-/* Replay every decode step from one captured HIP graph (on != 0) or launch kernel by kernel.
- * No counterpart in the reference (its plan is a host loop over dlsym'ed functions). */
+/* Replay every decode step from one captured HIP graph (on != 0) or launch kernel by kernel. A step of
+ * one or two launches (the whole-step kernel) is launched directly either way: that is quicker than replaying
+ * a graph of one node. No counterpart in the reference (its plan is a host loop over dlsym'ed functions). */
 int hm_model_set_graph(hm_model *m, int on);
 
 /* One launch for a whole decode step's embedding row and decoder layers (on != 0) instead of one
