@@ -197,14 +197,14 @@ __global__ __launch_bounds__(QTHREADS) void gemv_q6k_units_kernel(const float *_
         }
         trip += D * nwaves;
     }
-    // what the buffers still hold, then at most D - 1 trips behind them
+    // what the buffers still hold, each asked for again at once where a trip is left for it (at most D - 1 are)
 #pragma unroll
     for (int d = 0; d < D; d++)
-        if (trip + d * nwaves < ntrips) consume(un[d], trip + d * nwaves);
+        if (trip + d * nwaves < ntrips) {
+            consume(un[d], trip + d * nwaves);
+            if (trip + (D + d) * nwaves < ntrips) request(un[d], trip + (D + d) * nwaves);
+        }
     trip += D * nwaves;
-#pragma unroll
-    for (int d = 0; d < D; d++)
-        if (trip + d * nwaves < ntrips) request(un[d], trip + d * nwaves);
 #pragma unroll
     for (int d = 0; d < D; d++)
         if (trip + d * nwaves < ntrips) consume(un[d], trip + d * nwaves);

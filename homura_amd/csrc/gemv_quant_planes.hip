@@ -452,14 +452,14 @@ __global__ __launch_bounds__(PTHREADS) void gemv_q4_0_halves_kernel(const float 
         }
         trip += D * nwaves;
     }
-    // what the buffers still hold, then at most D - 1 trips behind them
+    // what the buffers still hold, each asked for again at once where a trip is left for it (at most D - 1 are)
 #pragma unroll
     for (int d = 0; d < D; d++)
-        if (trip + d * nwaves < ntrips) consume(qn[d], sn[d], trip + d * nwaves);
+        if (trip + d * nwaves < ntrips) {
+            consume(qn[d], sn[d], trip + d * nwaves);
+            if (trip + (D + d) * nwaves < ntrips) request(qn[d], sn[d], trip + (D + d) * nwaves);
+        }
     trip += D * nwaves;
-#pragma unroll
-    for (int d = 0; d < D; d++)
-        if (trip + d * nwaves < ntrips) request(qn[d], sn[d], trip + d * nwaves);
 #pragma unroll
     for (int d = 0; d < D; d++)
         if (trip + d * nwaves < ntrips) consume(qn[d], sn[d], trip + d * nwaves);
@@ -587,11 +587,11 @@ __global__ __launch_bounds__(PTHREADS) void gemv_q4_0_blocks_kernel(const float 
     }
 #pragma unroll
     for (int d = 0; d < D; d++)
-        if (trip + d * nwaves < ntrips) consume(qn[d], sn[d], trip + d * nwaves);
+        if (trip + d * nwaves < ntrips) {
+            consume(qn[d], sn[d], trip + d * nwaves);
+            if (trip + (D + d) * nwaves < ntrips) request(qn[d], sn[d], trip + (D + d) * nwaves);
+        }
     trip += D * nwaves;
-#pragma unroll
-    for (int d = 0; d < D; d++)
-        if (trip + d * nwaves < ntrips) request(qn[d], sn[d], trip + d * nwaves);
 #pragma unroll
     for (int d = 0; d < D; d++)
         if (trip + d * nwaves < ntrips) consume(qn[d], sn[d], trip + d * nwaves);
