@@ -27,6 +27,21 @@ def test_library_exports_every_declared_symbol():
     assert b"gfx950" in lib.hm_version()
 
 
+def test_what_the_gpu_runs_load_travels_with_the_tree():
+    """The list of paths that stay behind when the tree is sent to a GPU machine names nothing that the GPU
+    tests, the smoke run or bench.py read there: the package and its built library, the oracle, the tests with
+    their fixtures, the headers and the HBM traffic table under profiles/."""
+    import bench
+    ignored = [l.strip() for l in (ROOT / ".gpurunignore").read_text().splitlines() if l.strip()]
+    needed = [bench.TRAFFIC_TABLE, _ffi.LIB_PATH, ROOT / "oracle" / "pyoracle.py", ROOT / "tests" / "golden" / "reference_vectors.json",
+              ROOT / "include" / "homura_amd.h", ROOT / "__graft_entry__.py", ROOT / "bench.py"]
+    for path in needed:
+        rel = "./" + str(Path(path).resolve().relative_to(ROOT))
+        for pat in ignored:
+            assert not (rel == pat or rel.startswith(pat.rstrip("/") + "/")), (rel, pat)
+            assert not (pat.startswith("*") and rel.endswith(pat[1:])), (rel, pat)
+
+
 def test_library_exports_the_reference_kernel_symbols():
     """The reference's loader resolves `_mlir__mlir_ciface_k{idx}` by dlsym
     (reference src/runtime.rs:803-824): all 1024 must be there (the quantised plan of a 28-layer
