@@ -176,6 +176,7 @@ SIGNATURES = {
     "hm_model_whole_step": (_I, [_P]),
     "hm_model_whole_step_available": (_I, [_P]),
     "hm_model_whole_step_status": (_I, [_P]),
+    "hm_model_whole_step_inject_timeout": (_I, [_P, _I, _I]),
     "hm_model_whole_step_trace": (_I, [_P, _P, _I, C.POINTER(C.c_int)]),
     "hm_model_prefill_capture_q8k_inputs": (_I, [_P, _I]),
     "hm_model_prefill_captured_q8k_inputs": (_I, [_P, _P, _SZ]),

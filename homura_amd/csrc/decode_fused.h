@@ -52,12 +52,23 @@ struct FusedDecodeArgs {
     // 1: take every exchange through memory, as a step does whose workgroups the placement check does not
     // find dealt to the dies round-robin (for tests of that path; the host sets it from HOMURA_WHOLE_STEP_FAR)
     int far_only;
+    // Test support. spin_limit > 0: a wait gives up after that many polls instead of 2^20. withhold_wg >= 0: that
+    // workgroup does not publish its Q|K|V rows of layer 0, so every wait for them runs into its bound, all
+    // workgroups walk on without waiting, and the launch ends normally with the status word set.
+    int spin_limit;
+    int withhold_wg;
     // Optional phase trace (nullptr = off; room for FUSED_TRACE_WGS workgroups x (11 n_layers + 2) entries):
     // every workgroup stores, in its own row, the 100 MHz device clock at 11 points per
     // layer - both barriers of the Q|K|V, attention, O, gate|up and down phases, and the end of the fold
     // after attention's second barrier - followed by one entry at the end of the kernel and a last word that
     // is 1 when the step's exchanges went through the dies' L2s.
     unsigned long long *trace;
+};
+// ctl words: [0] launches so far, [1] first wait that gave up (0 = none), [2] steps that ran without die-local
+// traffic, [3] warnings (FUSED_WARN_*)
+enum : uint32_t {
+    FUSED_WARN_TOKEN_RANGE = 1u,      // a fed-back token id lay outside the vocabulary and was replaced by 0
+    FUSED_WARN_NO_FINITE_LOGIT = 2u,  // the greedy pick found no finite logit and took token 0
 };
 constexpr int FUSED_TRACE_PER_LAYER = 11;
 constexpr int FUSED_TRACE_WGS = 256;  // rows of the trace buffer (the largest grid of any instance)
@@ -76,5 +87,6 @@ int decode_fused_tier(const FusedShape &s, int live_rows);
 // live_rows: the cache rows of the step, the new one included (the host's count; the kernel reads the position
 // from the cursor and leaves with a status code if it does not fit the instance).
 int decode_fused_launch(hm_ctx *ctx, const FusedShape &s, const FusedDecodeArgs &a, int live_rows);
-// Reads the sticky status word (synchronises the stream). HM_OK or HM_ERR_HIP with a message.
-int decode_fused_check(hm_ctx *ctx, const uint32_t *d_ctl);
+// Reads the sticky status words (synchronises the stream). HM_OK, or HM_ERR_HIP with a message; *gave_up (when
+// given) tells a wait that ran into its bound, which the caller can recover from, from the other failures.
+int decode_fused_check(hm_ctx *ctx, const uint32_t *d_ctl, bool *gave_up = nullptr);

@@ -36,6 +36,7 @@
 // and still walks through the remaining barriers, so the grid always drains.
 #include "decode_fused.h"
 
+#include <cstdlib>
 #include <type_traits>
 
 namespace {
@@ -158,7 +159,7 @@ __device__ __forceinline__ void st_slot(unsigned char *area, int slot, float v, 
     // compiler-issued stores: a store written in inline asm is invisible to the hazard recognizer (a store
     // of more than 8 bytes must not be followed at once by a write to its data registers)
     if (near)
-        *reinterpret_cast<uint64_t *>(p) = w;
+        __hip_atomic_store(reinterpret_cast<uint64_t *>(p), w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WAVEFRONT);
     else
         __hip_atomic_store(reinterpret_cast<uint64_t *>(p), w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     asm volatile("" ::: "memory");
@@ -168,6 +169,7 @@ struct PollState {
     uint32_t *ctl;
     bool failed;
     uint32_t where;  // what is being waited for: phase | layer << 4 | workgroup << 12, stored on a timeout
+    int spin_max;    // polls before a wait gives up
 };
 
 // 16-byte loads of `NU` units {v0, tag, v1, tag}, all issued before one wait, repeated until every
@@ -196,7 +198,7 @@ __device__ __forceinline__ void poll_units(PollState &ps, const unsigned char *a
 #pragma unroll
         for (int u = 0; u < NU; u++) ok = ok && (!on[u] || (w[u].y == tag && w[u].w == tag));
         if (ok) return;
-        if (++spins > SPIN_MAX) {
+        if (++spins > ps.spin_max) {
             atomicCAS(ps.ctl + 1, 0u, 0x80000000u | ps.where);  // the first timeout is the one reported
             ps.failed = true;
             return;
@@ -259,7 +261,7 @@ __device__ __forceinline__ void norm_rope(const float *src, bool normed, float w
     float lo = on ? src[lane] : 0.f, hi = on ? src[lane + HALF] : 0.f;
     if (normed) {
         const float ss = wave_sum(lo * lo + hi * hi);
-        const float inv = 1.0f / sqrtf(ss / (float)HD + eps);
+        const float inv = __builtin_amdgcn_rsqf(ss / (float)HD + eps);
         lo = (lo * inv) * w_lo;
         hi = (hi * inv) * w_hi;
     }
@@ -655,7 +657,7 @@ __device__ __forceinline__ void head_rows(const FusedDecodeArgs &a, Lds<GE> &sm,
     if (nbatch > 0) request(0);
     if (EARLY) wg_barrier();
     const float tot = ((sm.red[0] + sm.red[1]) + sm.red[2]) + sm.red[3];
-    const float inv = 1.0f / sqrtf(tot / (float)GE::HIDDEN + a.eps);
+    const float inv = __builtin_amdgcn_rsqf(tot / (float)GE::HIDDEN + a.eps);
     float xv[HC][8];
 #pragma unroll
     for (int c = 0; c < HC; c++) {
@@ -778,7 +780,7 @@ __device__ __forceinline__ void compute_role(const FusedDecodeArgs &a, Lds<GE> &
         load_wg(sm.lp[l], WG_CUT, GE::RGW);
         {
             const float tot = ((sm.red[0] + sm.red[1]) + sm.red[2]) + sm.red[3];
-            const float inv = 1.0f / sqrtf(tot / (float)GE::HIDDEN + a.eps);
+            const float inv = __builtin_amdgcn_rsqf(tot / (float)GE::HIDDEN + a.eps);
             float v[GE::RQW];
             s.wq.dots_normed(sm.hx, sm.nw, inv, lane, v);
             wave_sum_n<GE::RQW>(v);
@@ -923,7 +925,7 @@ __device__ __forceinline__ void compute_role(const FusedDecodeArgs &a, Lds<GE> &
         load_wo(nx);
         {
             const float tot = ((sm.red[0] + sm.red[1]) + sm.red[2]) + sm.red[3];
-            const float inv = 1.0f / sqrtf(tot / (float)GE::HIDDEN + a.eps);
+            const float inv = __builtin_amdgcn_rsqf(tot / (float)GE::HIDDEN + a.eps);
             float v[GE::RGW];
             s.wg.dots_normed(sm.hx, sm.nw, inv, lane, v);
             wave_sum_n<GE::RGW>(v);
@@ -933,7 +935,7 @@ __device__ __forceinline__ void compute_role(const FusedDecodeArgs &a, Lds<GE> &
                 gte = lane == r / 2 ? v[r] : gte;
                 up = lane == r / 2 ? v[r + 1] : up;
             }
-            if (lane < GE::RGW / 2) sm.pub[cw * (GE::RGW / 2) + lane] = (gte / (1.0f + expf(-gte))) * up;
+            if (lane < GE::RGW / 2) sm.pub[cw * (GE::RGW / 2) + lane] = (gte * __builtin_amdgcn_rcpf(1.0f + __expf(-gte))) * up;
         }
         wg_barrier();
 
@@ -973,7 +975,7 @@ __device__ __forceinline__ void comm_role(const FusedDecodeArgs &a, Lds<GE> &sm,
     const int ct = cwv * WAVE + lane;
     const int L = a.n_layers;
     const uint32_t base = launches * (uint32_t)L;
-    PollState ps{a.ctl, false, 0u};
+    PollState ps{a.ctl, false, 0u, a.spin_limit > 0 ? a.spin_limit : SPIN_MAX};
     const size_t par_bytes = (size_t)GE::PAR_SLOTS * 8;
     unsigned long long *trace = (a.trace && ct == 0) ? a.trace + (size_t)wg * (L * FUSED_TRACE_PER_LAYER + 2) : nullptr;
     auto mark = [&]() {
@@ -983,7 +985,10 @@ __device__ __forceinline__ void comm_role(const FusedDecodeArgs &a, Lds<GE> &sm,
     // the token of this step (reference embed kernel, src/hf/emitter.rs:506-537)
     const int step = a.state->step, n_forced = a.state->n_forced;
     int id = step < n_forced ? a.forced[step] : a.state->token;
-    if (id < 0 || id >= a.vocab) id = 0;
+    if (id < 0 || id >= a.vocab) {  // decoding goes on with id 0; the host reports it
+        if (wg == 0 && ct == 0) atomicOr(a.ctl + 3, FUSED_WARN_TOKEN_RANGE);
+        id = 0;
+    }
     float h[NJ];
 #pragma unroll
     for (int j = 0; j < NJ; j++) h[j] = a.embed[(size_t)id * GE::HIDDEN + ct + CT * j];
@@ -1159,7 +1164,8 @@ __device__ __forceinline__ void comm_role(const FusedDecodeArgs &a, Lds<GE> &sm,
         mark();
         wg_barrier();
         mark();
-        if (ct < GE::RQ) st_slot(lq, sp.split * GE::RQ + ct, sm.pub[ct], tag, near_g);
+        // (a.withhold_wg: a test's way to make every wait for this workgroup's rows run into its bound)
+        if (ct < GE::RQ && !(l == 0 && wg == a.withhold_wg)) st_slot(lq, sp.split * GE::RQ + ct, sm.pub[ct], tag, near_g);
 
         // ── into attention: this KV head's raw q rows (and k, v for the split that holds the new row),
         //    QK-norm + RoPE, cache append (reference src/hf/emitter.rs:629-649, src/runtime.rs:521-568) ──
@@ -1302,7 +1308,7 @@ __device__ __forceinline__ void comm_role(const FusedDecodeArgs &a, Lds<GE> &sm,
                     }
                 }
             }
-            if (lane < GE::FPW) st_slot(la, o0 + lane, num / den, tag, near_g);
+            if (lane < GE::FPW) st_slot(la, o0 + lane, num * __builtin_amdgcn_rcpf(den), tag, near_g);
         } else if (cwv == 0) {
             constexpr int FU = GE::FPW / 2;
             const int o0 = sp.split * GE::FPW;  // first output, counted inside the KV head's G * HD
@@ -1334,7 +1340,7 @@ __device__ __forceinline__ void comm_role(const FusedDecodeArgs &a, Lds<GE> &sm,
             float mine = 0.f;
 #pragma unroll
             for (int e = 0; e < GE::FPW; e++) mine = lane == e ? red[1 + e] : mine;
-            if (lane < GE::FPW) st_slot(la, o0 + lane, mine / red[0], tag, near_g);
+            if (lane < GE::FPW) st_slot(la, o0 + lane, mine * __builtin_amdgcn_rcpf(red[0]), tag, near_g);
         }
         mark();
 
@@ -1420,7 +1426,9 @@ __device__ __forceinline__ void comm_role(const FusedDecodeArgs &a, Lds<GE> &sm,
                 }
                 const float gm = wave_max(gi >= 0 ? gv : -INFINITY);
                 const float gs = wave_max(gi >= 0 && gv == gm ? (float)gi : -1.f);
-                if (lane == 0 && a.advance && !ps.failed) {
+                if (lane == 0 && gs < 0.f) atomicOr(a.ctl + 3, FUSED_WARN_NO_FINITE_LOGIT);
+                const bool gave_up = ps.failed || __hip_atomic_load(a.ctl + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u;
+                if (lane == 0 && a.advance && !gave_up) {
                     const int tok = gs < 0.f ? 0 : (int)gs;
                     if (step < a.out_cap) a.out_tokens[step] = tok;
                     a.state_rw->token = tok;
@@ -1591,11 +1599,17 @@ bool decode_fused_supported(const hm_ctx *ctx, const FusedShape &s, int n_layers
         *why = "fewer compute units than resident workgroups";
         return false;
     }
-    int per_cu = 0;
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, i->kernel, FT, 0) != hipSuccess || per_cu < 1) {
-        (void)hipGetLastError();
-        *why = "the kernel does not fit a compute unit";
-        return false;
+    // every instance a step of this shape and format may take must fit a compute unit
+    for (int rows = 1; rows > 0;) {
+        const Instance *j = find_instance(s, rows);
+        if (!j) break;
+        int per_cu = 0;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, j->kernel, FT, 0) != hipSuccess || per_cu < 1) {
+            (void)hipGetLastError();
+            *why = "the kernel does not fit a compute unit";
+            return false;
+        }
+        rows = j->max_kv + 1;
     }
     return true;
 }
@@ -1611,20 +1625,36 @@ int decode_fused_launch(hm_ctx *ctx, const FusedShape &s, const FusedDecodeArgs 
                "decode_fused: %d layers / %d cache rows not served for this shape", a.n_layers, a.max_len);
     FusedDecodeArgs args = a;
     void *params[] = {&args};
-    HM_HIP(ctx, hipLaunchKernel(i->kernel, dim3(i->nwg), dim3(FT), params, 0, ctx->stream));
+    // HOMURA_WHOLE_STEP_COOP=1: a cooperative launch, which the runtime refuses when the grid cannot be resident
+    // as a whole (it does not reserve the compute units against other streams either)
+    static const bool coop = [] {
+        const char *e = std::getenv("HOMURA_WHOLE_STEP_COOP");
+        return e && std::atoi(e) != 0;
+    }();
+    if (coop)
+        HM_HIP(ctx, hipLaunchCooperativeKernel(i->kernel, dim3(i->nwg), dim3(FT), params, 0, ctx->stream));
+    else
+        HM_HIP(ctx, hipLaunchKernel(i->kernel, dim3(i->nwg), dim3(FT), params, 0, ctx->stream));
     return HM_OK;
 }
 
-int decode_fused_check(hm_ctx *ctx, const uint32_t *d_ctl) {
+int decode_fused_check(hm_ctx *ctx, const uint32_t *d_ctl, bool *gave_up) {
     uint32_t h[16] = {0};
+    if (gave_up) *gave_up = false;
     int rc = hm_download(ctx, h, d_ctl, sizeof(h));
     if (rc != HM_OK) return rc;
     if (h[1] != 0 && (h[1] & 15u) == 15u)
         return hm_set_error(ctx, HM_ERR_HIP, "decode_fused: launched with more live cache rows than the kernel serves (launch %u)", h[0]);
-    if (h[1] != 0)
+    if (h[1] != 0) {
+        if (gave_up) *gave_up = true;
         return hm_set_error(ctx, HM_ERR_HIP,
-                            "decode_fused: workgroup %u stopped waiting in phase %u of layer %u (launch %u)",
+                            "decode_fused: workgroup %u stopped waiting in phase %u of layer %u (launch %u): the grid's "
+                            "workgroups were not all resident at once, or another whole-step model ran on this GPU",
                             (h[1] >> 12) & 0xFFFFu, h[1] & 15u, (h[1] >> 4) & 255u, h[0]);
-    
+    }
+    if (h[3] & FUSED_WARN_TOKEN_RANGE)
+        return hm_set_error(ctx, HM_ERR_HIP, "decode_fused: a fed-back token id lay outside the vocabulary (decoded as id 0; launch %u)", h[0]);
+    if (h[3] & FUSED_WARN_NO_FINITE_LOGIT)
+        return hm_set_error(ctx, HM_ERR_HIP, "decode_fused: a step's logits held no finite value (token 0 taken; launch %u)", h[0]);
     return HM_OK;
 }

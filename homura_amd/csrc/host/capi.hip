@@ -195,6 +195,11 @@ int hm_model_whole_step_trace(hm_model *m, unsigned long long *h_out, int cap, i
     return m->impl->whole_step_trace(h_out, cap, n_out);
 }
 
+int hm_model_whole_step_inject_timeout(hm_model *m, int workgroup, int spin_limit) {
+    if (!m || !m->impl) return HM_ERR_INVALID;
+    return m->impl->whole_step_inject_timeout(workgroup, spin_limit);
+}
+
 int hm_model_whole_step_status(hm_model *m) {
     if (!m) return HM_ERR_INVALID;
     return m->impl->whole_step_status();

@@ -476,9 +476,33 @@ void poison_outputs(const KernelInfo &ki, void **args) {
     outputs_of(ki, &first, &count, &rank);
     for (int j = 0; j < count; j++) {
         const MemRef m = memref(args, first + j, rank);
+        if (!m.data || rank < 1) continue;
         size_t n = 1;
-        for (int d = 0; d < rank; d++) n *= (size_t)(m.sizes[d] > 0 ? m.sizes[d] : 0);
-        if (m.data && n && n < ((size_t)1 << 34)) (void)hipMemsetAsync(m.data, 0xFF, n * 4, ctx->stream);
+        bool dense = true;  // row-major without gaps: one fill covers the operand
+        for (int d = rank - 1; d >= 0; d--) {
+            const size_t sz = (size_t)(m.sizes[d] > 0 ? m.sizes[d] : 0);
+            if (sz > 1 && m.strides[d] != (int64_t)n) dense = false;
+            n *= sz;
+        }
+        if (n == 0 || n >= ((size_t)1 << 34)) continue;
+        if (dense) {
+            (void)hipMemsetAsync(m.data, 0xFF, n * 4, ctx->stream);
+            continue;
+        }
+        // A strided view (say, rows of one head inside a longer cache): fill run by run along the innermost
+        // dimension, and only where that dimension is contiguous, so that no byte outside the operand changes.
+        const size_t inner = (size_t)m.sizes[rank - 1];
+        if (m.strides[rank - 1] != 1 || n / inner > ((size_t)1 << 20)) continue;
+        std::vector<int64_t> idx((size_t)rank, 0);
+        for (size_t run = 0; run < n / inner; run++) {
+            int64_t off = 0;
+            for (int d = 0; d < rank - 1; d++) off += idx[(size_t)d] * m.strides[d];
+            (void)hipMemsetAsync(m.data + off * 4, 0xFF, inner * 4, ctx->stream);
+            for (int d = rank - 2; d >= 0; d--) {
+                if (++idx[(size_t)d] < m.sizes[d]) break;
+                idx[(size_t)d] = 0;
+            }
+        }
     }
     (void)hipStreamSynchronize(ctx->stream);
     (void)hipGetLastError();

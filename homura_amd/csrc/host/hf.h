@@ -49,6 +49,8 @@ struct PlanScratch {
     // whole-step decode launch (bf16 plans of a served shape): device layer table, exchange area,
     // control words {launch count, status}
     Buffer fused_layers, fused_xch, fused_ctl, fused_trace;
+    // test support (hm_model_whole_step_inject_timeout): handed to the next whole-step launches
+    int inject_spin_limit = 0, inject_withhold_wg = -1;
     Buffer normed, gate, up, down, q_raw, k_raw, v_raw;  // quantised plan only
     int cand_cap = 0;
 };
@@ -115,8 +117,13 @@ class HfModel {
     bool whole_step_available() const { return fused_available_; }
     int set_whole_step(bool on);
     bool whole_step() const { return plan_ && plan_->whole_step(); }
-    // HM_OK, or the error a whole-step launch left behind (an exchange that timed out)
+    // HM_OK, or the error a whole-step launch left behind. A wait that ran into its bound is recovered from by
+    // the call that met it (the steps of that call run again, one launch per projection, and so do later
+    // calls); it stays reported here until reset_kv_cache or set_whole_step(true) re-arms the launch.
     int whole_step_status();
+    // Test support: the next whole-step launches give up a wait after `spin_limit` polls, and workgroup
+    // `workgroup` withholds its first publish, so that every workgroup runs into that bound and leaves normally.
+    int whole_step_inject_timeout(int workgroup, int spin_limit);
     // Phase trace of the latest whole-step launch (device clock ticks at 100 MHz; 11 entries per layer
     // and a final one, see decode_fused.h). Recording starts with the first call, which returns 0
     // entries; later calls return the trace of the step that ran last.
@@ -136,6 +143,15 @@ class HfModel {
     int step_inputs(std::vector<Buffer *> &inputs);
     int refresh_fused_table();
     int finish_sync();
+    int recover_whole_step();
+    // the bodies of the calls of the same name, which run them again after a recovered whole-step timeout
+    int run_kv_once(const int64_t *h_ids, int n_ids, float *h_logits);
+    int generate_greedy_once(const int64_t *h_prompt, int n_prompt, int n_new, int32_t *h_tokens);
+    int generate_once(const int64_t *h_prompt, int n_prompt, int max_new, const hm_sampling_config &cfg, uint64_t seed,
+                      int eos_token, int32_t *h_tokens, int *n_out);
+    int bench_decode_once(int64_t first_id, int n_steps, float *ms_out, int32_t *h_tokens);
+    template <class Body>
+    int with_whole_step_retry(Body body);
     int prefill_chunk(const int32_t *h_ids, int n, float *h_logits);
     const float *weight_f32(const std::string &name) const;
     int check_ids(const int64_t *ids, int n, std::vector<int32_t> &out);
@@ -149,6 +165,9 @@ class HfModel {
     int fused_max_kv_ = 0;            // live cache rows (the new one included) a whole-step launch serves
     int fused_tier_ = 0;              // capacity of the kernel instance the recorded step launches
     bool whole_step_wanted_ = false;  // the caller's choice; the plan follows it while the cache is short enough
+    bool fused_dirty_ = false;        // whole-step launches were enqueued since the status words were last read
+    bool fused_gave_up_ = false;      // a launch ran into a wait's bound: one launch per projection until re-armed
+    std::string fused_gave_up_msg_;
     int fused_wf_ = 0;  // FUSED_WF_* of the whole-step kernel instance
     bool fused_head_ = false;  // the whole-step launch also runs the LM head and the greedy pick (bf16 plan)
     const void *fused_table_kv_ = nullptr;  // key_ptr(0) the device layer table was built for

@@ -465,7 +465,8 @@ int HfModel::finalize(int max_seq_len) {
         plan_->set_pre_run([this, fs]() {
             const int live = plan_->kv_cache_len() + 1;
             const int tier = decode_fused_tier(fs, live);  // 0: no instance holds that many rows
-            int rc = plan_->set_whole_step(whole_step_wanted_ && tier > 0);
+            int rc = plan_->set_whole_step(whole_step_wanted_ && !fused_gave_up_ && tier > 0);
+            fused_dirty_ = fused_dirty_ || plan_->whole_step();
             if (rc == HM_OK && plan_->whole_step() && tier != fused_tier_) {
                 rc = plan_->invalidate_graph();  // the recorded launch is another instance's
                 fused_tier_ = tier;
@@ -633,6 +634,8 @@ int HfModel::emit_transformer_plan() {
                 fa.ctl = scr->fused_ctl.as<uint32_t>();
                 fa.trace = scr->fused_trace ? scr->fused_trace.as<unsigned long long>() : nullptr;
                 fa.far_only = far_only;
+                fa.spin_limit = scr->inject_spin_limit;
+                fa.withhold_wg = scr->inject_withhold_wg;
                 if (with_head) {
                     fa.head_w = sc.pool[lm_head]->as<uint16_t>();
                     fa.head_norm = sc.pool[final_norm]->as<float>();
@@ -1173,6 +1176,8 @@ int HfModel::emit_transformer_plan_quant() {
                 fa.ctl = scr->fused_ctl.as<uint32_t>();
                 fa.trace = scr->fused_trace ? scr->fused_trace.as<unsigned long long>() : nullptr;
                 fa.far_only = far_only;
+                fa.spin_limit = scr->inject_spin_limit;
+                fa.withhold_wg = scr->inject_withhold_wg;
                 return decode_fused_launch(sc.ctx, fshape, fa, sc.plan->kv_cache_len() + 1);
             };
             k.launches.push_back(std::move(f));
@@ -1567,11 +1572,52 @@ int HfModel::whole_step_trace(unsigned long long *h_out, int cap, int *n_out) {
     return rc;
 }
 
-// Stream sync plus, when steps went through the whole-step launch, its status word.
+// Internal return code of finish_sync: a whole-step launch ran into a wait's bound and the model has been
+// switched to one launch per projection; the caller runs its steps again.
+constexpr int HM_RETRY_STEPS = -1000;
+
+// Stream sync plus, when steps went through the whole-step launch since the last look, its status words.
 int HfModel::finish_sync() {
     int rc = hm_sync(ctx_);
-    if (rc == HM_OK && plan_ && plan_->whole_step()) rc = whole_step_status();
+    if (rc != HM_OK || !fused_available_ || !fused_dirty_) return rc;
+    fused_dirty_ = false;
+    bool gave_up = false;
+    rc = decode_fused_check(ctx_, scratch_->fused_ctl.as<uint32_t>(), &gave_up);
+    if (rc == HM_OK) return rc;
+    if (gave_up) return recover_whole_step();
+    // a warning (token id out of range, no finite logit): reported once
+    (void)hipMemsetAsync(scratch_->fused_ctl.as<uint32_t>() + 3, 0, 4, ctx_->stream);
+    (void)hm_sync(ctx_);
     return rc;
+}
+
+// After a wait that gave up: keep what the launch reported, clear the exchange area and the control words (the
+// launch count with them: tags start over on a zeroed area), and leave the whole-step launch out until the
+// caller re-arms it. The grid has drained - every wait is bounded - so nothing is in flight.
+int HfModel::recover_whole_step() {
+    fused_gave_up_msg_ = ctx_->last_error;
+    fused_gave_up_ = true;
+    scratch_->inject_spin_limit = 0;
+    scratch_->inject_withhold_wg = -1;
+    HM_HIP(ctx_, hipMemsetAsync(scratch_->fused_xch.ptr(), 0, scratch_->fused_xch.bytes(), ctx_->stream));
+    HM_HIP(ctx_, hipMemsetAsync(scratch_->fused_ctl.ptr(), 0, 64, ctx_->stream));
+    int rc = hm_sync(ctx_);
+    if (rc == HM_OK) rc = plan_->set_whole_step(false);
+    if (rc == HM_OK) rc = plan_->invalidate_graph();
+    return rc == HM_OK ? HM_RETRY_STEPS : rc;
+}
+
+// Runs `body`; when a whole-step launch inside it gave up a wait, takes the cache back to where the call
+// found it and runs the body again, which now takes one launch per projection (rows the failed steps
+// appended are written again).
+template <class Body>
+int HfModel::with_whole_step_retry(Body body) {
+    const int len0 = kv_cache_len();
+    int rc = body();
+    if (rc != HM_RETRY_STEPS) return rc;
+    plan_->kv_cache()->reset(len0);
+    rc = body();
+    return rc == HM_RETRY_STEPS ? hm_set_error(ctx_, HM_ERR_HIP, "whole-step decode gave up twice: %s", fused_gave_up_msg_.c_str()) : rc;
 }
 
 int HfModel::set_whole_step(bool on) {
@@ -1579,12 +1625,32 @@ int HfModel::set_whole_step(bool on) {
     if (on && !fused_available_)
         return hm_set_error(ctx_, HM_ERR_INVALID, "whole-step decode is not available for this model (bf16 weights and a served shape are needed)");
     whole_step_wanted_ = on;
+    if (on) fused_gave_up_ = false;  // an explicit request re-arms the launch after a recovered timeout
     return plan_->set_whole_step(on && plan_->kv_cache_len() + 1 <= fused_max_kv_);
 }
 
 int HfModel::whole_step_status() {
     if (!fused_available_) return HM_OK;
-    return decode_fused_check(ctx_, scratch_->fused_ctl.as<uint32_t>());
+    if (fused_gave_up_)
+        return hm_set_error(ctx_, HM_ERR_HIP, "%s; steps take one launch per projection until reset_kv_cache or set_whole_step(true)",
+                            fused_gave_up_msg_.c_str());
+    int rc = hm_sync(ctx_);
+    if (rc != HM_OK) return rc;
+    fused_dirty_ = false;
+    bool gave_up = false;
+    rc = decode_fused_check(ctx_, scratch_->fused_ctl.as<uint32_t>(), &gave_up);
+    if (gave_up && recover_whole_step() == HM_RETRY_STEPS)
+        return hm_set_error(ctx_, HM_ERR_HIP, "%s; steps take one launch per projection until reset_kv_cache or set_whole_step(true)",
+                            fused_gave_up_msg_.c_str());
+    return rc;
+}
+
+int HfModel::whole_step_inject_timeout(int workgroup, int spin_limit) {
+    if (!fused_available_) return hm_set_error(ctx_, HM_ERR_STATE, "whole-step decode is not available for this model");
+    if (workgroup < 0 || spin_limit < 1) return hm_set_error(ctx_, HM_ERR_INVALID, "inject_timeout: workgroup >= 0 and spin_limit >= 1 needed");
+    scratch_->inject_spin_limit = spin_limit;
+    scratch_->inject_withhold_wg = workgroup;
+    return plan_->invalidate_graph();  // a recorded launch carries the old arguments
 }
 
 int HfModel::check_ids(const int64_t *ids, int n, std::vector<int32_t> &out) {
@@ -1599,6 +1665,11 @@ int HfModel::check_ids(const int64_t *ids, int n, std::vector<int32_t> &out) {
 }
 
 int HfModel::run_kv(const int64_t *h_ids, int n_ids, float *h_logits) {
+    if (!finalized_) return hm_set_error(ctx_, HM_ERR_STATE, "model not finalized");
+    return with_whole_step_retry([&] { return run_kv_once(h_ids, n_ids, h_logits); });
+}
+
+int HfModel::run_kv_once(const int64_t *h_ids, int n_ids, float *h_logits) {
     if (!finalized_) return hm_set_error(ctx_, HM_ERR_STATE, "model not finalized");
     if (n_ids <= 0 || !h_ids) return hm_set_error(ctx_, HM_ERR_INVALID, "run_kv: no input ids");
     if (kv_cache_len() + n_ids > max_seq_len_)
@@ -1892,12 +1963,18 @@ int HfModel::init_kv_cache(const float *const *h_kv, int seq_len) {
 int HfModel::reset_kv_cache() {
     if (!finalized_) return hm_set_error(ctx_, HM_ERR_STATE, "model not finalized");
     plan_->reset_kv_cache();
+    fused_gave_up_ = false;  // a new conversation re-arms the whole-step launch after a recovered timeout
     return HM_OK;
 }
 
 int HfModel::kv_cache_len() const { return plan_ ? plan_->kv_cache_len() : 0; }
 
 int HfModel::generate_greedy(const int64_t *h_prompt, int n_prompt, int n_new, int32_t *h_tokens) {
+    if (!finalized_) return hm_set_error(ctx_, HM_ERR_STATE, "model not finalized");
+    return with_whole_step_retry([&] { return generate_greedy_once(h_prompt, n_prompt, n_new, h_tokens); });
+}
+
+int HfModel::generate_greedy_once(const int64_t *h_prompt, int n_prompt, int n_new, int32_t *h_tokens) {
     if (!finalized_) return hm_set_error(ctx_, HM_ERR_STATE, "model not finalized");
     if (n_prompt <= 0 || n_new <= 0 || !h_prompt || !h_tokens)
         return hm_set_error(ctx_, HM_ERR_INVALID, "generate_greedy: bad arguments");
@@ -1942,6 +2019,12 @@ int zero_ints_launch(hm_ctx *ctx, int *d, size_t n);
 int HfModel::generate(const int64_t *h_prompt, int n_prompt, int max_new, const hm_sampling_config &cfg, uint64_t seed,
                       int eos_token, int32_t *h_tokens, int *n_out) {
     if (!finalized_) return hm_set_error(ctx_, HM_ERR_STATE, "model not finalized");
+    return with_whole_step_retry([&] { return generate_once(h_prompt, n_prompt, max_new, cfg, seed, eos_token, h_tokens, n_out); });
+}
+
+int HfModel::generate_once(const int64_t *h_prompt, int n_prompt, int max_new, const hm_sampling_config &cfg, uint64_t seed,
+                           int eos_token, int32_t *h_tokens, int *n_out) {
+    if (!finalized_) return hm_set_error(ctx_, HM_ERR_STATE, "model not finalized");
     if (n_prompt <= 0 || max_new <= 0 || !h_prompt || !h_tokens || !n_out)
         return hm_set_error(ctx_, HM_ERR_INVALID, "generate: bad arguments");
     *n_out = 0;
@@ -1971,7 +2054,7 @@ int HfModel::generate(const int64_t *h_prompt, int n_prompt, int max_new, const 
     // prompt: everything but its last token only has to reach the cache
     // (reference HfGenerationContext::prefill, src/hf/model.rs:321-336)
     if (n_prompt > 1) {
-        if ((rc = run_kv(h_prompt, n_prompt - 1, nullptr)) != HM_OK) return rc;
+        if ((rc = run_kv_once(h_prompt, n_prompt - 1, nullptr)) != HM_OK) return rc;
     }
     uint64_t rng = hm_rng_seed(seed);
     std::vector<Buffer *> inputs;
@@ -2051,10 +2134,15 @@ int HfModel::generate(const int64_t *h_prompt, int n_prompt, int max_new, const 
         h_tokens[(*n_out)++] = tok;
         current = tok;
     }
-    return HM_OK;
+    return finish_sync();
 }
 
 int HfModel::bench_decode(int64_t first_id, int n_steps, float *ms_out, int32_t *h_tokens) {
+    if (!finalized_) return hm_set_error(ctx_, HM_ERR_STATE, "model not finalized");
+    return with_whole_step_retry([&] { return bench_decode_once(first_id, n_steps, ms_out, h_tokens); });
+}
+
+int HfModel::bench_decode_once(int64_t first_id, int n_steps, float *ms_out, int32_t *h_tokens) {
     if (!finalized_) return hm_set_error(ctx_, HM_ERR_STATE, "model not finalized");
     if (n_steps <= 0 || n_steps > plan_->out_capacity())
         return hm_set_error(ctx_, HM_ERR_INVALID, "bench_decode: bad step count %d", n_steps);

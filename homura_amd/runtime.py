@@ -472,6 +472,11 @@ class HfModel:
         """Raises if a whole-step launch left an error behind (an exchange that timed out)."""
         self._check(self.lib.hm_model_whole_step_status(self.h))
 
+    def whole_step_inject_timeout(self, workgroup: int, spin_limit: int):
+        """Test support: the next whole-step launches give up a wait after `spin_limit` polls and workgroup
+        `workgroup` withholds its first publish, so the launch ends normally with its status set."""
+        self._check(self.lib.hm_model_whole_step_inject_timeout(self.h, workgroup, spin_limit))
+
     def whole_step_trace(self, all_workgroups: bool = False) -> np.ndarray:
         """Device-clock ticks (100 MHz) of the latest whole-step launch: 11 per layer (both barriers of the
         Q|K|V, attention, O, gate|up and down phases; the fold's end comes after attention's) and a final

@@ -367,13 +367,28 @@ int hm_model_set_graph(hm_model *m, int on);
  * LM head and the greedy pick. The cache may be of any length: a step takes the instance of the kernel that
  * holds its live rows (1536, 2048 or 4096 of them; the smaller the faster), beyond 4096 the per-projection path,
  * chosen step by step. Results agree with the per-projection
- * path to f32 summation order. hm_model_whole_step_status returns HM_OK, or the error
- * left behind by a step whose workgroups stopped waiting for one another (bounded waits; the
- * outputs of such a step are not valid). */
+ * path to f32 summation order.
+ *
+ * The launch needs all its workgroups (one per compute unit) resident at once, since they wait for one
+ * another: one whole-step model per GPU at a time, and nothing else that holds compute units while it
+ * steps. Every wait is bounded. When one runs into its bound (the grid was not resident as a whole), the
+ * launch ends normally without moving the cursor, and the call that finds the status - hm_model_run_kv,
+ * hm_model_generate_greedy, hm_model_generate, hm_model_bench_decode - clears the exchange state, takes
+ * the cache back to where it found it, and runs its steps again with one launch per projection, as do the
+ * calls after it; it returns what that second run returns. hm_model_whole_step_status then keeps returning
+ * the error the launch left behind (phase, layer and workgroup of the first wait that gave up) until
+ * hm_model_reset_kv_cache or hm_model_set_whole_step(m, 1) re-arms the launch. It also reports, once, a
+ * fed-back token id outside the vocabulary or a step whose logits held no finite value (both decoded as
+ * token 0). */
 int hm_model_set_whole_step(hm_model *m, int on);
 int hm_model_whole_step(hm_model *m);
 int hm_model_whole_step_available(hm_model *m);
 int hm_model_whole_step_status(hm_model *m);
+/* Test support, no counterpart in the reference: the next whole-step launches give up a wait after
+ * `spin_limit` polls (instead of 2^20), and workgroup `workgroup` withholds its first publish, so that every
+ * workgroup runs into that bound and the launch ends normally with its status set. Cleared by the recovery
+ * described above. */
+int hm_model_whole_step_inject_timeout(hm_model *m, int workgroup, int spin_limit);
 
 /* HfModel::run_kv (src/hf/model.rs:198-218) -> ExecutionPlan::run_kv
  * (src/runtime.rs:1580-1892): n_ids new tokens on top of the cache; h_logits receives

@@ -305,3 +305,63 @@ def test_cache_longer_than_the_kernel_serves_changes_over_and_back(ctx):
     assert gm.whole_step()
     gm.close()
     plain.close()
+
+
+def test_a_wait_that_gives_up_is_reported_and_the_call_runs_again_per_projection(small):
+    """Forced from the host: a small spin bound and one workgroup that withholds its first publish, so every
+    workgroup gives up its wait and the launch ends normally with the status word set. The call that meets
+    the status clears the exchange state, takes the cache back and runs its steps again with one launch per
+    projection; the status stays readable until the launch is re-armed."""
+    cfg, _w, gm, _om = small
+    kv = synth_model.synth_kv(cfg, 41, 100)
+    ids = synth.token_ids(42, 4, cfg.vocab_size)
+    gm.set_prefill_min(0)
+    gm.set_whole_step(True)
+    try:
+        gm.init_kv_cache(kv, 100)
+        healthy = gm.run_kv(ids)
+        gm.whole_step_status()
+        assert gm.whole_step()
+        gm.set_whole_step(False)
+        gm.init_kv_cache(kv, 100)
+        per_projection = gm.run_kv(ids)
+        per_projection_tokens = gm.generate_greedy(ids[:1], 6)
+        gm.set_whole_step(True)
+
+        gm.init_kv_cache(kv, 100)
+        gm.whole_step_inject_timeout(workgroup=5, spin_limit=3000)
+        got = gm.run_kv(ids)
+        assert gm.kv_cache_len() == 104          # the failed launch moved nothing; the second run appended 4 rows
+        assert not gm.whole_step()               # one launch per projection from here on
+        assert np.array_equal(got, per_projection)
+        with pytest.raises(HomuraError) as e:
+            gm.whole_step_status()
+        msg = str(e.value)
+        say(msg)
+        assert "stopped waiting in phase 2 of layer 0" in msg and "workgroup" in msg
+        # later calls stay on the per-projection path, and the status stays readable
+        assert np.array_equal(gm.generate_greedy(ids[:1], 6), per_projection_tokens)
+        assert not gm.whole_step()
+        with pytest.raises(HomuraError):
+            gm.whole_step_status()
+        # a new conversation re-arms the launch, and it works as before
+        gm.reset_kv_cache()
+        gm.whole_step_status()
+        gm.init_kv_cache(kv, 100)
+        again = gm.run_kv(ids)
+        gm.whole_step_status()
+        assert gm.whole_step()
+        assert np.array_equal(again, healthy)
+        # the device-resident greedy loop recovers the same way
+        gm.set_whole_step(False)
+        gm.init_kv_cache(kv, 100)
+        want_tokens = gm.generate_greedy(ids, 6)
+        gm.set_whole_step(True)
+        gm.init_kv_cache(kv, 100)
+        gm.whole_step_inject_timeout(workgroup=0, spin_limit=3000)
+        assert np.array_equal(gm.generate_greedy(ids, 6), want_tokens)
+        assert not gm.whole_step()
+    finally:
+        gm.reset_kv_cache()
+        gm.set_whole_step(True)
+
