@@ -16,6 +16,10 @@ namespace homura {
 int gemm_split_nk(hm_ctx *ctx, const uint16_t *d_a_split, int pieces, const uint16_t *d_b_nk, float *d_c, int M, int K,
                   int N, int max_parts = 1, int *parts = nullptr);
 
+// The same sum of piece products against B in the reference's layout [K][N] (N contiguous; N % 8 == 0, K % 32 == 0).
+int gemm_split_kn(hm_ctx *ctx, const uint16_t *d_a_split, int pieces, const uint16_t *d_b_kn, float *d_c, int M, int K,
+                  int N);
+
 // C = A x B^T for two f32 matrices, each given as three bf16 pieces per element: d_a_split [M][3 K],
 // d_b_split [N][3 K] (piece p in columns [p K, (p+1) K)). The six products of an A piece and a B piece
 // whose indices add up to at most 2 are accumulated; what is left out is below 2^-24 of the result.

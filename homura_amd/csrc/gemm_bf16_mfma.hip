@@ -508,8 +508,10 @@ __global__ __launch_bounds__(GEMM_THREADS) void gemm_nk_dma_kernel(const uint16_
             }
 }
 
+// a_pieces > 1: A is a split matrix [M][a_pieces * K] and the k loop runs over all its pieces against the same B
+// (B's k index wraps at K), so C is the sum of the pieces' products.
 int gemm_launch(hm_ctx *ctx, const char *who, const uint16_t *a, const uint16_t *b, float *c, int M, int K,
-                int N, bool b_nk, int ksplit = 1, int *ksplit_used = nullptr, int ldc = 0) {
+                int N, bool b_nk, int ksplit = 1, int *ksplit_used = nullptr, int ldc = 0, int a_pieces = 1) {
     HM_CHECK_CTX(ctx);
     HM_REQUIRE(ctx, a && b && c, "%s: NULL pointer", who);
     HM_REQUIRE(ctx, M > 0 && N > 0 && K > 0 && K % 32 == 0, "%s: need M, N > 0 and K %% 32 == 0 (M=%d K=%d N=%d)", who,
@@ -523,8 +525,8 @@ int gemm_launch(hm_ctx *ctx, const char *who, const uint16_t *a, const uint16_t 
     g.M = M;
     g.N = N;
     g.Kb = K;
-    g.K = K;
-    g.lda = K;
+    g.K = a_pieces * K;
+    g.lda = a_pieces * K;
     g.ldb = K;
     g.ldc = ldc > 0 ? ldc : N;
     HM_REQUIRE(ctx, g.ldc >= N, "%s: ldc %d below N %d", who, g.ldc, N);
@@ -571,6 +573,12 @@ int homura::gemm_split_nk(hm_ctx *ctx, const uint16_t *d_a_split, int pieces, co
 int homura::gemm_split_split_nk(hm_ctx *ctx, const uint16_t *d_a_split, const uint16_t *d_b_split, float *d_c, int M,
                                 int K, int N, int max_parts, int *parts, int ldc) {
     return gemm_pieces_nk(ctx, d_a_split, 3, d_b_split, 3, d_c, M, K, N, max_parts, parts, ldc);
+}
+
+int homura::gemm_split_kn(hm_ctx *ctx, const uint16_t *d_a_split, int pieces, const uint16_t *d_b_kn, float *d_c, int M,
+                          int K, int N) {
+    HM_REQUIRE(ctx, pieces >= 1 && pieces <= 3, "gemm_split_kn: %d pieces (1..3)", pieces);
+    return gemm_launch(ctx, "gemm_split_kn", d_a_split, d_b_kn, d_c, M, K, N, false, 1, nullptr, 0, pieces);
 }
 
 extern "C" int hm_gemm_bf16(hm_ctx *ctx, const uint16_t *d_a_mk, const uint16_t *d_b_kn, float *d_c,

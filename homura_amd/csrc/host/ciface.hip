@@ -19,8 +19,9 @@
 // fast path.
 //
 // A call may carry any number of tokens (the reference's prefill hands the whole prompt to the same
-// kernels, src/hf/model.rs:321-336): matrix products go through the GEMVs in blocks of up to eight rows,
-// attention with more than one query row through the causal prompt kernel, which applies the mask of
+// kernels, src/hf/model.rs:321-336): matrix products of fewer than 16 rows go through the GEMVs in blocks of
+// up to eight rows, longer ones through the matrix-core GEMMs (f32 rows as three bf16 pieces; Q8_0 / Q4_0
+// matrices dequantised to pieces first), attention with more than one query row through the causal prompt kernel, which applies the mask of
 // build_causal_mask (src/hf/precompute.rs:134-161) by position instead of reading the mask operand.
 //
 // The ABI returns void. A failing call prints a line, fills every output operand with NaN (all-ones
@@ -30,7 +31,9 @@
 #include <cstdio>
 #include <vector>
 
+#include "../gemm_bf16_mfma.h"
 #include "../hm_common.h"
+#include "../prefill.h"
 
 namespace {
 
@@ -161,8 +164,21 @@ int bshd_to_bhsd(hm_ctx *ctx, const float *src, float *dst, int S, int heads, in
     return HM_OK;
 }
 
-// out [S][N] = x [S][K] times a [K,N] bf16 matrix: the batch-1 kernel takes up to eight rows a launch
-int rows_gemv_bf16(hm_ctx *ctx, const float *x, const uint16_t *w, float *out, int S, int K, int N) {
+// Calls of at least this many tokens take their matrix products to the matrix cores.
+constexpr int GEMM_MIN_ROWS = 16;
+
+// out [S][N] = x [S][K] times a [K,N] bf16 matrix. A few rows: the batch-1 kernel, up to eight rows a launch.
+// A prompt (the reference's prefill hands all its tokens to the same kernels, src/hf/model.rs:321-336): the
+// f32 rows as three bf16 pieces each (all 24 significant bits) against the matrix on the matrix cores.
+int rows_matmul_bf16(hm_ctx *ctx, Scratch &s, const float *x, const uint16_t *w, float *out, int S, int K, int N) {
+    if (S >= GEMM_MIN_ROWS && K % 32 == 0 && N % 8 == 0 && ((uintptr_t)w % 16) == 0) {
+        Scratch local = s;  // the pieces are dead once the product is enqueued: later calls may reuse the space
+        uint16_t *split = local.take<uint16_t>((size_t)S * 3 * K);
+        if (split) {
+            TRY(homura::split_rows_launch(ctx, x, split, 3, (size_t)S, K));
+            return homura::gemm_split_kn(ctx, split, 3, w, out, S, K, N);
+        }
+    }
     for (int r = 0; r < S; r += 8)
         TRY(hm_gemv_bf16(ctx, x + (size_t)r * K, w, out + (size_t)r * N, S - r < 8 ? S - r : 8, K, N));
     return HM_OK;
@@ -205,9 +221,9 @@ int run_qkv(void **a) {
     float *vrows = S > 1 ? s.take<float>((size_t)S * b.kv_dim) : v.as<float>();
     if (!normed || !krows || !vrows) return hm_set_error(ctx, HM_ERR_OOM, "QKV kernel: workspace too small for %d tokens", S);
     TRY(hm_rmsnorm(ctx, h.as<float>(), ln.as<float>(), normed, S, hidden, (float)b.cfg.rms_norm_eps));
-    TRY(rows_gemv_bf16(ctx, normed, qw.as<uint16_t>(), q.as<float>(), S, hidden, b.q_dim));
-    TRY(rows_gemv_bf16(ctx, normed, kw.as<uint16_t>(), krows, S, hidden, b.kv_dim));
-    TRY(rows_gemv_bf16(ctx, normed, vw.as<uint16_t>(), vrows, S, hidden, b.kv_dim));
+    TRY(rows_matmul_bf16(ctx, s, normed, qw.as<uint16_t>(), q.as<float>(), S, hidden, b.q_dim));
+    TRY(rows_matmul_bf16(ctx, s, normed, kw.as<uint16_t>(), krows, S, hidden, b.kv_dim));
+    TRY(rows_matmul_bf16(ctx, s, normed, vw.as<uint16_t>(), vrows, S, hidden, b.kv_dim));
     if (bias) {
         TRY(add_bias_rows(ctx, q.as<float>(), qb, S, b.q_dim));
         TRY(add_bias_rows(ctx, krows, kb, S, b.kv_dim));
@@ -235,7 +251,7 @@ int run_attn(void **a) {
     float *flat = s.take<float>((size_t)S * b.q_dim);
     if (!flat) return hm_set_error(ctx, HM_ERR_OOM, "Attn kernel: workspace too small for %d tokens", S);
     TRY(attention_over_views(q, k, v, flat, s, "Attn kernel"));
-    return rows_gemv_bf16(ctx, flat, ow.as<uint16_t>(), out.as<float>(), S, b.q_dim, b.cfg.hidden_size);
+    return rows_matmul_bf16(ctx, s, flat, ow.as<uint16_t>(), out.as<float>(), S, b.q_dim, b.cfg.hidden_size);
 }
 
 // emit_mlp_kernel (src/hf/emitter.rs:767-822): h, attn_out, ln_w, gate_w, up_w, down_w -> [1,S,hidden]
@@ -254,10 +270,10 @@ int run_mlp(void **a) {
         return hm_set_error(ctx, HM_ERR_OOM, "MLP kernel: workspace too small for %d tokens", (int)S);
     TRY(hm_add(ctx, h.as<float>(), attn.as<float>(), resid, S * hidden));
     TRY(hm_rmsnorm(ctx, resid, ln.as<float>(), normed, (int)S, hidden, (float)b.cfg.rms_norm_eps));
-    TRY(rows_gemv_bf16(ctx, normed, gw.as<uint16_t>(), gate, (int)S, hidden, inter));
-    TRY(rows_gemv_bf16(ctx, normed, uw.as<uint16_t>(), up, (int)S, hidden, inter));
+    TRY(rows_matmul_bf16(ctx, s, normed, gw.as<uint16_t>(), gate, (int)S, hidden, inter));
+    TRY(rows_matmul_bf16(ctx, s, normed, uw.as<uint16_t>(), up, (int)S, hidden, inter));
     TRY(hm_silu_mul(ctx, gate, up, gate, S * inter));
-    TRY(rows_gemv_bf16(ctx, gate, dw.as<uint16_t>(), down, (int)S, inter, hidden));
+    TRY(rows_matmul_bf16(ctx, s, gate, dw.as<uint16_t>(), down, (int)S, inter, hidden));
     return hm_add(ctx, resid, down, out.as<float>(), S * hidden);
 }
 
@@ -272,7 +288,7 @@ int run_lm_head(void **a) {
     float *normed = s.take<float>((size_t)S * b.cfg.hidden_size);
     if (!normed) return hm_set_error(ctx, HM_ERR_OOM, "LMHead kernel: workspace too small for %d tokens", S);
     TRY(hm_rmsnorm(ctx, h.as<float>(), nw.as<float>(), normed, S, b.cfg.hidden_size, (float)b.cfg.rms_norm_eps));
-    return rows_gemv_bf16(ctx, normed, lw.as<uint16_t>(), out.as<float>(), S, b.cfg.hidden_size, b.cfg.vocab_size);
+    return rows_matmul_bf16(ctx, s, normed, lw.as<uint16_t>(), out.as<float>(), S, b.cfg.hidden_size, b.cfg.vocab_size);
 }
 
 // ── the quantised plan's kernels (src/hf/emitter_quant.rs) ───────────────────
@@ -306,6 +322,19 @@ int run_quant_mm(void **a, const KernelInfo &ki) {
     const MemRef x = memref(a, 0, 3), w = memref(a, 1, 1), out = memref(a, 2, 3);
     TRY(seq_ok(b.ctx, x.sizes[1], "QuantMM kernel"));
     const int S = (int)x.sizes[1];
+    const bool kq = ki.dtype == HM_DTYPE_Q4_K || ki.dtype == HM_DTYPE_Q6_K;
+    if (S >= GEMM_MIN_ROWS && ki.K % 64 == 0 && (!kq || ki.K % 256 == 0)) {
+        // A prompt: the rows (through the Q8_K quantisation first where the reference's kernel quantises its
+        // activations, src/graph_builder/emit_quant.rs:422-466) and the dequantised matrix as three bf16 pieces
+        // each, multiplied on the matrix cores. Falls through to the row blocks when the workspace is too small.
+        Scratch s(b.ctx);
+        uint16_t *xs = s.take<uint16_t>((size_t)S * 3 * ki.K), *ws = s.take<uint16_t>((size_t)ki.N * 3 * ki.K);
+        if (xs && ws) {
+            TRY(homura::split_rows_launch(b.ctx, x.as<float>(), xs, 3, (size_t)S, ki.K, kq));
+            TRY(homura::dequant_split_launch(b.ctx, ki.dtype, w.as<uint8_t>(), ki.N, ki.K, ws));
+            return homura::gemm_split_split_nk(b.ctx, xs, ws, out.as<float>(), S, ki.K, ki.N);
+        }
+    }
     for (int r = 0; r < S; r += 8) {
         const float *xr = x.as<float>() + (size_t)r * ki.K;
         float *outr = out.as<float>() + (size_t)r * ki.N;

@@ -2,14 +2,13 @@
 
 `python -m homura_amd.phase_trace [--out FILE.md] [--dump FILE.npy]` runs a few decode steps with
 `hm_model_whole_step_trace` recording, and prints, as Markdown, what a layer spends between each pair of
-the kernel's 11 per-layer marks: mean and spread over workgroups and over layers 1..L-2 (the first and last
-layer carry the start and the LM head's prefetch). Which kernel form ran (streamed through LDS, or slices in
-registers with communicating wavefronts: HOMURA_WHOLE_STEP_STREAMED=0) decides what the marks mean.
+the kernel's 11 per-layer marks (both barriers of the Q|K|V, attention, O, gate|up and down phases, and the end
+of the fold): mean and spread over workgroups and over layers 1..L-2 (the first and last layer carry the
+start and the LM head's prefetch).
 """
 from __future__ import annotations
 
 import argparse
-import os
 
 import numpy as np
 
@@ -17,20 +16,7 @@ from . import synth, synth_model
 from .runtime import Context
 
 # what lies between mark i and mark i + 1 (the last entry: from mark 10 to mark 0 of the next layer)
-STREAMED = [
-    ("Q|K|V: normalised hidden state seen -> rows published", "compute"),
-    ("raw q rows arrive, QK-norm + RoPE", "exchange (die)"),
-    ("attention over the wavefront's cache rows, partial published", "compute"),
-    ("fold of the KV head's sub-splits, folded outputs published", "exchange (die) + fold"),
-    ("folded attention arrives", "exchange (die)"),
-    ("O rows of the K slice, partial rows published", "compute"),
-    ("partial O rows summed by the relays, hidden staged", "exchange (memory + die)"),
-    ("gate|up rows, SiLU*up published", "compute"),
-    ("SiLU*up of the group arrives", "exchange (die)"),
-    ("down rows of the K slice, partial rows published", "compute"),
-    ("partial down rows summed by the relays, hidden staged (next layer)", "exchange (memory + die)"),
-]
-RESIDENT = [
+INTERVALS = [
     ("Q|K|V rows (between the phase's barriers)", "compute"),
     ("rows published, raw q rows arrive, QK-norm + RoPE, cache append", "exchange (die)"),
     ("attention over the workgroup's cache split", "compute"),
@@ -66,16 +52,15 @@ def collect(steps: int = 4):
     return marks, total, bool(t[:, -1].min())
 
 
-def summary(marks: np.ndarray, total: float, die_local: bool, streamed: bool) -> str:
+def summary(marks: np.ndarray, total: float, die_local: bool) -> str:
     L = marks.shape[1]
-    names = STREAMED if streamed else RESIDENT
+    names = INTERVALS
     # interval i of layer l, per workgroup: mark i+1 - mark i (the last one reaches into the next layer)
     nxt = np.concatenate([marks[:, :, 1:], np.concatenate([marks[:, 1:, :1], marks[:, -1:, :1]], axis=1)], axis=2)
     d = (nxt - marks)[:, 1:L - 1, :]                 # [wg][layer][11]
     per_layer = marks[:, 2:L, 0].mean(axis=0) - marks[:, 1:L - 1, 0].mean(axis=0)
     out = []
-    out.append(f"kernel form: {'streamed through LDS (decode_streamed.hip)' if streamed else 'slices in registers (decode_fused.hip)'}; "
-               f"die-local exchanges: {die_local}")
+    out.append(f"decode_fused_kernel, Qwen3-0.6B shape, 1024 cached rows; die-local exchanges: {die_local}")
     out.append(f"launch, first mark to last: {total:.1f} us; one layer (layers 1..{L - 2}): mean {per_layer.mean():.2f} us, "
                f"min {per_layer.min():.2f}, max {per_layer.max():.2f}")
     out.append("")
@@ -100,9 +85,8 @@ def main():
     ap.add_argument("--dump")
     ap.add_argument("--steps", type=int, default=4)
     args = ap.parse_args()
-    streamed = os.environ.get("HOMURA_WHOLE_STEP_STREAMED", "1") != "0"
     marks, total, die_local = collect(args.steps)
-    text = summary(marks, total, die_local, streamed)
+    text = summary(marks, total, die_local)
     print(text, flush=True)
     if args.out:
         with open(args.out, "w") as f:

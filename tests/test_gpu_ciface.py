@@ -44,8 +44,9 @@ def call(lib, idx, descs):
 
 
 # Tokens per call: the reference's prefill hands the whole prompt to the kernels (src/hf/model.rs:321-336),
-# its decode one token; eleven rows take the matrix products through more than one block of eight rows.
-CHUNKS = [5, 1, 11]
+# its decode one token; eleven rows take the matrix products through more than one block of eight rows, and
+# sixty-four through the matrix-core GEMMs.
+CHUNKS = [5, 1, 11, 64]
 
 
 def check_rows(which, got, want, tol=1e-2):
@@ -65,7 +66,7 @@ def test_plan_through_memref_entry_points(ctx, which):
     W = dict(weights)
     L, hidden, inter, vocab = cfg.num_hidden_layers, cfg.hidden_size, cfg.intermediate_size, cfg.vocab_size
     H, kvh, hd = cfg.num_attention_heads, cfg.kv_heads(), cfg.get_head_dim()
-    max_len, past, chunks = 64, 9, CHUNKS
+    max_len, past, chunks = 128, 9, CHUNKS
     SM = max(chunks)
     om = mf.build_oracle_model(cfg, weights, max_len, has_qk_norm=qkn)
     kv = synth_model.synth_kv(cfg, 12, past)
@@ -157,7 +158,7 @@ def test_quantised_plan_through_memref_entry_points(ctx, which):
     L, hidden, inter, vocab = cfg.num_hidden_layers, cfg.hidden_size, cfg.intermediate_size, cfg.vocab_size
     H, kvh, hd = cfg.num_attention_heads, cfg.kv_heads(), cfg.get_head_dim()
     qd, kvd = H * hd, kvh * hd
-    max_len, past, chunks = 64, 9, CHUNKS
+    max_len, past, chunks = 128, 9, CHUNKS
     SM = max(chunks)
     om = mf.build_oracle_model(cfg, weights, max_len, has_qk_norm=False, proj_dtypes=mix)
     kv = synth_model.synth_kv(cfg, 12, past)
