@@ -90,3 +90,5 @@ int decode_fused_launch(hm_ctx *ctx, const FusedShape &s, const FusedDecodeArgs 
 // Reads the sticky status words (synchronises the stream). HM_OK, or HM_ERR_HIP with a message; *gave_up (when
 // given) tells a wait that ran into its bound, which the caller can recover from, from the other failures.
 int decode_fused_check(hm_ctx *ctx, const uint32_t *d_ctl, bool *gave_up = nullptr);
+// The same verdict from a host copy of the 16 control words.
+int decode_fused_check_words(hm_ctx *ctx, const uint32_t *h_ctl, bool *gave_up);

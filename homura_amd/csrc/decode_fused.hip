@@ -1643,6 +1643,11 @@ int decode_fused_check(hm_ctx *ctx, const uint32_t *d_ctl, bool *gave_up) {
     if (gave_up) *gave_up = false;
     int rc = hm_download(ctx, h, d_ctl, sizeof(h));
     if (rc != HM_OK) return rc;
+    return decode_fused_check_words(ctx, h, gave_up);
+}
+
+int decode_fused_check_words(hm_ctx *ctx, const uint32_t *h, bool *gave_up) {
+    if (gave_up) *gave_up = false;
     if (h[1] != 0 && (h[1] & 15u) == 15u)
         return hm_set_error(ctx, HM_ERR_HIP, "decode_fused: launched with more live cache rows than the kernel serves (launch %u)", h[0]);
     if (h[1] != 0) {

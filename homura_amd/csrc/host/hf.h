@@ -168,6 +168,10 @@ class HfModel {
     bool fused_dirty_ = false;        // whole-step launches were enqueued since the status words were last read
     bool fused_gave_up_ = false;      // a launch ran into a wait's bound: one launch per projection until re-armed
     std::string fused_gave_up_msg_;
+    // pinned host staging of run_kv: a logits row and the whole-step status words arrive with one synchronisation
+    void *h_stage_ = nullptr;
+    size_t h_stage_bytes_ = 0;
+    int check_fused_words(const uint32_t *h_ctl);
     int fused_wf_ = 0;  // FUSED_WF_* of the whole-step kernel instance
     bool fused_head_ = false;  // the whole-step launch also runs the LM head and the greedy pick (bf16 plan)
     const void *fused_table_kv_ = nullptr;  // key_ptr(0) the device layer table was built for

@@ -190,6 +190,7 @@ int HfModel::build_quant_planes() {
 
 HfModel::~HfModel() {
     if (ctx_) hm_sync(ctx_);
+    if (h_stage_) (void)hipHostFree(h_stage_);
 }
 
 int HfModel::set_weight_impl(int slot, const void *h_data, size_t bytes, bool nk_layout) {
@@ -1581,11 +1582,18 @@ int HfModel::finish_sync() {
     int rc = hm_sync(ctx_);
     if (rc != HM_OK || !fused_available_ || !fused_dirty_) return rc;
     fused_dirty_ = false;
+    uint32_t h[16] = {0};
+    rc = hm_download(ctx_, h, scratch_->fused_ctl.ptr(), sizeof(h));
+    return rc == HM_OK ? check_fused_words(h) : rc;
+}
+
+// What a host copy of the whole-step control words says: HM_OK, HM_RETRY_STEPS after the recovery from a wait
+// that gave up, or the error of a warning, which is reported once.
+int HfModel::check_fused_words(const uint32_t *h_ctl) {
     bool gave_up = false;
-    rc = decode_fused_check(ctx_, scratch_->fused_ctl.as<uint32_t>(), &gave_up);
+    const int rc = decode_fused_check_words(ctx_, h_ctl, &gave_up);
     if (rc == HM_OK) return rc;
     if (gave_up) return recover_whole_step();
-    // a warning (token id out of range, no finite logit): reported once
     (void)hipMemsetAsync(scratch_->fused_ctl.as<uint32_t>() + 3, 0, 4, ctx_->stream);
     (void)hm_sync(ctx_);
     return rc;
@@ -1684,12 +1692,29 @@ int HfModel::run_kv_once(const int64_t *h_ids, int n_ids, float *h_logits) {
     std::vector<Buffer *> inputs;
     step_inputs(inputs);
     const size_t logits_slot = plan_->output_slots()[0];
+    // The reference's decode loop reads a logits row per token (HfGenerationContext::decode_step,
+    // src/hf/model.rs:340-371). The row and the whole-step status words are copied into pinned host memory
+    // behind the step, so a token costs one stream synchronisation.
+    const size_t row_bytes = (size_t)cfg_.vocab_size * 4;
+    if (h_logits && h_stage_bytes_ < row_bytes + 64) {
+        if (h_stage_) (void)hipHostFree(h_stage_);
+        h_stage_ = nullptr;
+        h_stage_bytes_ = 0;
+        HM_HIP(ctx_, hipHostMalloc(&h_stage_, row_bytes + 64, hipHostMallocDefault));
+        h_stage_bytes_ = row_bytes + 64;
+    }
     for (int i = 0; i < n_ids; i++) {
         if ((rc = plan_->run_kv(inputs, weight_bufs_, max_seq_len_)) != HM_OK) return rc;
-        if (h_logits) {
-            rc = hm_download(ctx_, h_logits + (size_t)i * cfg_.vocab_size, plan_->slot(logits_slot)->ptr(),
-                             (size_t)cfg_.vocab_size * 4);
-            if (rc != HM_OK) return rc;
+        if (!h_logits) continue;
+        char *stage = static_cast<char *>(h_stage_);
+        HM_HIP(ctx_, hipMemcpyAsync(stage, plan_->slot(logits_slot)->ptr(), row_bytes, hipMemcpyDeviceToHost, ctx_->stream));
+        const bool look = fused_available_ && fused_dirty_;
+        if (look) HM_HIP(ctx_, hipMemcpyAsync(stage + row_bytes, scratch_->fused_ctl.ptr(), 64, hipMemcpyDeviceToHost, ctx_->stream));
+        HM_HIP(ctx_, hipStreamSynchronize(ctx_->stream));
+        std::memcpy(h_logits + (size_t)i * cfg_.vocab_size, stage, row_bytes);
+        if (look) {
+            fused_dirty_ = false;
+            if ((rc = check_fused_words(reinterpret_cast<const uint32_t *>(stage + row_bytes))) != HM_OK) return rc;
         }
     }
     return finish_sync();

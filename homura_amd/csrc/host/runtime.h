@@ -278,6 +278,10 @@ class ExecutionPlan {
     std::vector<Buffer> kv_views_;  // per-step views of the cache bound to present_kv slots
     std::vector<Buffer *> pool_;
     Buffer state_, forced_, out_tokens_;
+    // arm(): the cursor and the forced ids go out from pinned host memory with asynchronous copies (no stream
+    // synchronisation per call); the event tells when that memory may be written again
+    void *arm_pinned_ = nullptr;
+    hipEvent_t arm_done_ = nullptr;
     int out_cap_ = 0;
     bool prepared_ = false;
     bool use_graph_ = false;

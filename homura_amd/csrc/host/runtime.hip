@@ -201,6 +201,11 @@ ExecutionPlan::ExecutionPlan(hm_ctx *ctx, std::vector<CompiledKernel> kernels,
 }
 
 ExecutionPlan::~ExecutionPlan() {
+    if (arm_done_) {
+        (void)hipEventSynchronize(arm_done_);
+        (void)hipEventDestroy(arm_done_);
+    }
+    if (arm_pinned_) (void)hipHostFree(arm_pinned_);
     if (graph_exec_) (void)hipGraphExecDestroy(graph_exec_);
     if (graph_) (void)hipGraphDestroy(graph_);
 }
@@ -314,10 +319,21 @@ void ExecutionPlan::reset_kv_cache() {
 int ExecutionPlan::arm(const int32_t *h_forced, int n_forced) {
     if (!prepared_) return hm_set_error(ctx_, HM_ERR_STATE, "plan not prepared");
     if (n_forced > out_cap_) return hm_set_error(ctx_, HM_ERR_INVALID, "%d forced ids exceed the plan's capacity %d", n_forced, out_cap_);
-    DecodeState st{kv_cache_len(), 0, 0, n_forced};
-    int rc = hm_upload(ctx_, state_.ptr(), &st, sizeof(st));
-    if (rc == HM_OK && n_forced > 0) rc = hm_upload(ctx_, forced_.ptr(), h_forced, (size_t)n_forced * 4);
-    return rc;
+    const DecodeState st{kv_cache_len(), 0, 0, n_forced};
+    if (!arm_pinned_) {
+        HM_HIP(ctx_, hipHostMalloc(&arm_pinned_, sizeof(DecodeState) + (size_t)out_cap_ * 4, hipHostMallocDefault));
+        HM_HIP(ctx_, hipEventCreateWithFlags(&arm_done_, hipEventDisableTiming));
+    } else {
+        HM_HIP(ctx_, hipEventSynchronize(arm_done_));  // the previous call's copies have read the staging memory
+    }
+    char *stage = static_cast<char *>(arm_pinned_);
+    std::memcpy(stage, &st, sizeof(st));
+    if (n_forced > 0) std::memcpy(stage + sizeof(st), h_forced, (size_t)n_forced * 4);
+    HM_HIP(ctx_, hipMemcpyAsync(state_.ptr(), stage, sizeof(st), hipMemcpyHostToDevice, ctx_->stream));
+    if (n_forced > 0)
+        HM_HIP(ctx_, hipMemcpyAsync(forced_.ptr(), stage + sizeof(st), (size_t)n_forced * 4, hipMemcpyHostToDevice, ctx_->stream));
+    HM_HIP(ctx_, hipEventRecord(arm_done_, ctx_->stream));
+    return HM_OK;
 }
 
 int ExecutionPlan::bind(const std::vector<Buffer *> &inputs, std::vector<Buffer> &weights) {
