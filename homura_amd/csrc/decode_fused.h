@@ -4,13 +4,17 @@
 #include "hm_common.h"
 
 // Weight formats the kernel has instances for.
-enum : int { FUSED_WF_BF16 = 0, FUSED_WF_Q8_0 = 1, FUSED_WF_Q4_0 = 2 };
+// FUSED_WF_K8: Q4_K / Q6_K matrices (any mix) re-packed by kquant_planes8.hip: every weight as one signed byte,
+// a scale and a minimum factor per 16 weights, the super-block's f16 d and dmin; multiplied as the reference
+// multiplies K-quants, against the Q8_K quantisation of the activations in integer dot products.
+enum : int { FUSED_WF_BF16 = 0, FUSED_WF_Q8_0 = 1, FUSED_WF_Q4_0 = 2, FUSED_WF_K8 = 3 };
 
 // Per-layer device pointers. bf16: matrices in the K-contiguous stream layout the plan keeps:
 // wqkv [q_dim + 2 kv_dim][hidden], wo [hidden][q_dim], wgu [2 inter][hidden] with gate and up rows
 // interleaved (g0, u0, g1, u1, ...), wd [hidden][inter]; the s* pointers are unused. Q8_0 / Q4_0: w* are the
 // quant planes and s* the scale planes of the same matrices re-packed as gemv_quant_planes.hip describes,
-// q|k|v stacked in that order, wgu all gate rows and then all up rows.
+// q|k|v stacked in that order, wgu all gate rows and then all up rows. K8: w* the byte planes [N][K], s* the
+// per-row scale records (kquant_planes8.h), same row order.
 struct FusedLayerPtrs {
     const void *wqkv, *wo, *wgu, *wd;
     const uint16_t *sqkv, *so, *sgu, *sd;

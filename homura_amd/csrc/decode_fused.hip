@@ -84,7 +84,11 @@ struct Geo {
     static constexpr int RELAY0 = GLOB_SLOTS, RELAY_SLOTS = 2 * HIDDEN;
     static constexpr int LQ0 = RELAY0 + NXCD * RELAY_SLOTS, LP0 = LQ0 + KVH * GROWS, LA0 = LP0 + KVH * SPH * PART;
     static constexpr int LC0 = LA0 + KVH * KSO;
-    static constexpr int PAR_SLOTS = (LC0 + KVH * KSD + 31) / 32 * 32;
+    // K8 format, when a group's K slice of down does not start and end on 256-wide blocks: per workgroup the
+    // largest |SiLU*up| among its values in the block that the slice shares with the group before (first slot)
+    // and with the group after (second slot)
+    static constexpr int LM0 = LC0 + KVH * KSD;
+    static constexpr int PAR_SLOTS = (LM0 + 2 * NWG + 31) / 32 * 32;
     static constexpr int CHK0 = 2 * PAR_SLOTS;                 // placement check: one slot per workgroup
     static constexpr int CAND0 = CHK0 + NWG;                   // LM head: one {value, index} unit per workgroup
     static constexpr int ALL_SLOTS = CAND0 + 2 * NWG;
@@ -126,6 +130,7 @@ struct Lds {
     float wstat[NCW][GE::G][2];
     float pub[GE::PUB];                   // results of the phase, read by the publishing threads
     float red[4];
+    float nbmax[2];                       // K8: the neighbouring groups' maxima of the two shared blocks
     float head_v[NCW + 4];                // LM head: every wavefront's best row
     int head_i[NCW + 4];
     float bias[GE::RQ];
@@ -237,6 +242,29 @@ __device__ __forceinline__ void lds_x8(const float *v, int k, float *xv) {
     xv[4] = b.x; xv[5] = b.y; xv[6] = b.z; xv[7] = b.w;
 }
 
+// Vectors that the compute wavefronts read out of LDS (the staged hidden state and its norm weights, the folded
+// attention outputs, the SiLU*up values) are stored permuted, by weight format: a lane reads GRP consecutive
+// elements (8 with bf16 weights, 16 with the byte formats) as 16-byte pieces, and piece j of every group lies
+// in quarter j of the vector, so that the lanes of one read touch consecutive addresses (no bank conflicts;
+// stored in index order a read strides by 32 or 64 bytes a lane). Q4_0 reads two runs of 8 a lane and keeps
+// the index order.
+template <int WF>
+struct XLay {
+    static constexpr int GRP = (WF == FUSED_WF_Q8_0 || WF == FUSED_WF_K8) ? 16 : (WF == FUSED_WF_BF16 ? 8 : 0);
+    __device__ __forceinline__ static int pos(int k, int n) {
+        if (GRP == 0) return k;
+        return ((k % GRP) / 4) * (n / (GRP / 4)) + (k / GRP) * 4 + (k % 4);
+    }
+};
+// elements k .. k + 7 (k a multiple of 8) of a vector of n elements stored as XLay<WF> lays it out
+template <int WF>
+__device__ __forceinline__ void lds_v8(const float *v, int n, int k, float *xv) {
+    const f32x4 a = *reinterpret_cast<const f32x4 *>(v + XLay<WF>::pos(k, n));
+    const f32x4 b = *reinterpret_cast<const f32x4 *>(v + XLay<WF>::pos(k + 4, n));
+    xv[0] = a.x; xv[1] = a.y; xv[2] = a.z; xv[3] = a.w;
+    xv[4] = b.x; xv[5] = b.y; xv[6] = b.z; xv[7] = b.w;
+}
+
 template <int LPR>
 __device__ __forceinline__ float row_sum(float v) {
     v += dpp_move<0xB1, 0xF>(v, 0.f);
@@ -304,8 +332,8 @@ __device__ __forceinline__ void normed_dots(const u32x4 (&w)[R][C], const float 
 #pragma unroll
     for (int c = 0; c < C; c++) {
         float hv[8], wv[8];
-        lds_x8(hx, (c * WAVE + lane) * 8, hv);
-        lds_x8(nw, (c * WAVE + lane) * 8, wv);
+        lds_v8<FUSED_WF_BF16>(hx, C * 512, (c * WAVE + lane) * 8, hv);
+        lds_v8<FUSED_WF_BF16>(nw, C * 512, (c * WAVE + lane) * 8, wv);
 #pragma unroll
         for (int e = 0; e < 8; e++) xv[c][e] = (hv[e] * inv) * wv[e];
     }
@@ -316,7 +344,7 @@ template <int R, int C>
 __device__ __forceinline__ void plain_dots(const u32x4 (&w)[R][C], const float *x, int lane, float (&acc)[R][C]) {
     float xv[C][8];
 #pragma unroll
-    for (int c = 0; c < C; c++) lds_x8(x, (c * WAVE + lane) * 8, xv[c]);
+    for (int c = 0; c < C; c++) lds_v8<FUSED_WF_BF16>(x, C * 512, (c * WAVE + lane) * 8, xv[c]);
     dots_from<R, C>(w, xv, acc);
 }
 
@@ -497,8 +525,8 @@ struct Rows {
 #pragma unroll
             for (int part = 0; part < 2; part++) {
                 float hv[8], wv[8];
-                lds_x8(hx, x_index(c, lane, part), hv);
-                lds_x8(nw, x_index(c, lane, part), wv);
+                lds_v8<WF>(hx, K, x_index(c, lane, part), hv);
+                lds_v8<WF>(nw, K, x_index(c, lane, part), wv);
 #pragma unroll
                 for (int e = 0; e < 8; e++) xv[c][part * 8 + e] = (hv[e] * inv) * wv[e];
             }
@@ -509,7 +537,7 @@ struct Rows {
 #pragma unroll
         for (int c = 0; c < C; c++)
 #pragma unroll
-            for (int part = 0; part < 2; part++) lds_x8(x, x_index(c, lane, part), xv[c] + part * 8);
+            for (int part = 0; part < 2; part++) lds_v8<WF>(x, K, x_index(c, lane, part), xv[c] + part * 8);
         finish(xv, v);
     }
 };
@@ -541,7 +569,7 @@ struct SliceRows<FUSED_WF_BF16, R, KS, KTOT> {
     __device__ __forceinline__ void dots(const float *x, int lane, float (&v)[Q]) const {
         float xv[P][8], acc[Q][P];
 #pragma unroll
-        for (int p = 0; p < P; p++) lds_x8(x, p * 128 + (lane % LANES_PER_ROW) * 8, xv[p]);
+        for (int p = 0; p < P; p++) lds_v8<FUSED_WF_BF16>(x, KS, p * 128 + (lane % LANES_PER_ROW) * 8, xv[p]);
         dots_from<Q, P>(w, xv, acc);
 #pragma unroll
         for (int q = 0; q < Q; q++) v[q] = chunk_total<P>(acc[q]);
@@ -592,7 +620,7 @@ struct SliceRows {
             const int hb = p * 8 + lane % LANES_PER_ROW;  // half block inside the slice (slices start on a block)
 #pragma unroll
             for (int part = 0; part < 2; part++)
-                lds_x8(x, Q4 ? (hb >> 1) * 32 + (hb & 1) * 8 + part * 16 : hb * 16 + part * 8, xv[p] + part * 8);
+                lds_v8<WF>(x, KS, Q4 ? (hb >> 1) * 32 + (hb & 1) * 8 + part * 16 : hb * 16 + part * 8, xv[p] + part * 8);
             float sx = 0.f;
 #pragma unroll
             for (int j = 0; j < 16; j++) sx += xv[p][j];
@@ -610,6 +638,208 @@ struct SliceRows {
         for (int s = 0; s < Q; s++) v[s] += dpp_move<0x4E, 0xF>(v[s], 0.f);
 #pragma unroll
         for (int s = 0; s < Q; s++) v[s] += dpp_move<0x141, 0xF>(v[s], 0.f);
+    }
+};
+
+
+// ── K8: Q4_K / Q6_K matrices as byte planes (kquant_planes8.h) ──
+//
+// A lane holds one 16-weight sub-block of each 1024-wide chunk of a row: its 16 signed bytes, its scale and
+// minimum factor, and the f16 d | dmin of its 256-wide super-block, which is exactly one DPP row of 16 lanes.
+// The activations go through the reference's Q8_K quantisation (src/graph_builder/emit_quant.rs:422-466:
+// amax over the block, d = amax / 127, q = roundeven(x * 127 / amax) clamped to +-127) in every wavefront, the
+// products are integer dot products, and a block contributes (d * act_d) * float(sum sc * isum) -
+// (dmin * act_d) * float(sum mn * bsum) with both sums exact in i32 (emit_quant.rs:165-816); blocks are added
+// in ascending order, as the reference adds them.
+__device__ __forceinline__ int dpp_row_isum(int v) {
+    v += __builtin_amdgcn_update_dpp(0, v, 0xB1, 0xF, 0xF, false);
+    v += __builtin_amdgcn_update_dpp(0, v, 0x4E, 0xF, 0xF, false);
+    v += __builtin_amdgcn_update_dpp(0, v, 0x141, 0xF, 0xF, false);
+    v += __builtin_amdgcn_update_dpp(0, v, 0x140, 0xF, 0xF, false);
+    return v;
+}
+__device__ __forceinline__ float dpp_row_fmax(float v) {
+    v = fmaxf(v, dpp_move<0xB1, 0xF>(v, 0.f));
+    v = fmaxf(v, dpp_move<0x4E, 0xF>(v, 0.f));
+    v = fmaxf(v, dpp_move<0x141, 0xF>(v, 0.f));
+    v = fmaxf(v, dpp_move<0x140, 0xF>(v, 0.f));
+    return v;
+}
+
+// The Q8_K form of a lane's 16 activations of a block whose largest magnitude is amax: four words of four
+// bytes, their sum, and the block's act_d.
+struct Q8kLane {
+    uint32_t q[4];
+    int bsum;
+    float act_d;
+};
+__device__ __forceinline__ Q8kLane q8k_lane(const float (&x)[16], float amax) {
+    Q8kLane r;
+    r.act_d = amax / 127.0f;
+    const float iscale = amax == 0.0f ? 0.0f : 127.0f / amax;
+    r.bsum = 0;
+#pragma unroll
+    for (int w = 0; w < 4; w++) {
+        int qi[4];
+#pragma unroll
+        for (int e = 0; e < 4; e++)  // round half to even, clamp to +-127 (one median instruction)
+            qi[e] = (int)__builtin_amdgcn_fmed3f(rintf(__fmul_rn(x[4 * w + e], iscale)), -127.0f, 127.0f);
+        // the low bytes of the four integers side by side
+        const uint32_t lo = __builtin_amdgcn_perm((uint32_t)qi[1], (uint32_t)qi[0], 0x0c0c0400u);
+        const uint32_t hi = __builtin_amdgcn_perm((uint32_t)qi[3], (uint32_t)qi[2], 0x0c0c0400u);
+        r.q[w] = __builtin_amdgcn_perm(hi, lo, 0x05040100u);
+        r.bsum = __builtin_amdgcn_sdot4((int)r.q[w], 0x01010101, r.bsum, false);
+    }
+    return r;
+}
+__device__ __forceinline__ float abs_max16(const float (&x)[16]) {
+    float m = 0.f;
+#pragma unroll
+    for (int j = 0; j < 16; j++) m = fmaxf(m, fabsf(x[j]));
+    return m;
+}
+// One block's share of a row from the lane's sub-block: every lane of the block's DPP row gets it.
+__device__ __forceinline__ float k8_block(const u32x4 w, uint32_t sub, uint32_t dd, const Q8kLane &a) {
+    int isum = __builtin_amdgcn_sdot4((int)w.x, (int)a.q[0], 0, false);
+    isum = __builtin_amdgcn_sdot4((int)w.y, (int)a.q[1], isum, false);
+    isum = __builtin_amdgcn_sdot4((int)w.z, (int)a.q[2], isum, false);
+    isum = __builtin_amdgcn_sdot4((int)w.w, (int)a.q[3], isum, false);
+    const int sc = (int)(int8_t)(sub & 0xFFu), mn = (int)((sub >> 8) & 0xFFu);
+    const int s_tot = dpp_row_isum(sc * isum), m_tot = dpp_row_isum(mn * a.bsum);
+    const float d = f16_bits_to_f32((uint16_t)(dd & 0xFFFFu)), dmin = f16_bits_to_f32((uint16_t)(dd >> 16));
+    const float scale_part = __fmul_rn(__fmul_rn(d, a.act_d), (float)s_tot);
+    const float min_part = __fmul_rn(__fmul_rn(dmin, a.act_d), (float)m_tot);
+    return __fsub_rn(scale_part, min_part);
+}
+
+typedef const uint32_t __attribute__((address_space(1))) *global_u32_ptr;
+
+template <int R, int K>
+struct Rows<FUSED_WF_K8, R, K> {
+    static constexpr int C = K / 1024;
+    static constexpr int RS = K / 8 + K / 64;  // bytes of a row's scale record: (sc, mn) per 16 weights, then (d, dmin) per 256
+    static_assert(K % 1024 == 0, "K8 rows are cut into 1024-wide chunks (16 weights a lane)");
+    u32x4 q[R][C];
+    uint32_t sub[R][C], dd[R][C];
+    template <class RowOf>
+    __device__ __forceinline__ void load(const void *quants, const uint16_t *scales, RowOf row_of, int r0, int r1, int lane) {
+        const unsigned char *base = reinterpret_cast<const unsigned char *>(quants);
+        const unsigned char *rec = reinterpret_cast<const unsigned char *>(scales);
+#pragma unroll
+        for (int r = 0; r < R; r++)
+#pragma unroll
+            for (int c = 0; c < C; c++)
+                if (r >= r0 && r < r1) {
+                    const size_t row = (size_t)row_of(r);
+                    const int s16 = c * WAVE + lane;  // sub-block of the row
+                    q[r][c] = ld128_global_stream(base + row * K + (size_t)s16 * 16);
+                    sub[r][c] = __builtin_nontemporal_load((global_u16_ptr)(rec + row * RS + (size_t)s16 * 2));
+                    dd[r][c] = __builtin_nontemporal_load((global_u32_ptr)(rec + row * RS + K / 8 + (size_t)(s16 / 16) * 4));
+                }
+    }
+    // v[r]: the row's value in lane 0, zero in the others (the caller's sum over the wavefront keeps it exact)
+    __device__ __forceinline__ void finish(const float (&xv)[C][16], int lane, float (&v)[R]) const {
+        Q8kLane a[C];
+#pragma unroll
+        for (int c = 0; c < C; c++) a[c] = q8k_lane(xv[c], dpp_row_fmax(abs_max16(xv[c])));
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            float acc = 0.f;
+#pragma unroll
+            for (int c = 0; c < C; c++) {
+                const float p = k8_block(q[r][c], sub[r][c], dd[r][c], a[c]);
+#pragma unroll
+                for (int b = 0; b < 4; b++)  // the chunk's four blocks, ascending
+                    acc = __fadd_rn(acc, __int_as_float(__builtin_amdgcn_readlane(__float_as_int(p), 16 * b)));
+            }
+            v[r] = lane == 0 ? acc : 0.f;
+        }
+    }
+    __device__ __forceinline__ void dots_normed(const float *hx, const float *nw, float inv, int lane, float (&v)[R]) const {
+        float xv[C][16];
+#pragma unroll
+        for (int c = 0; c < C; c++)
+#pragma unroll
+            for (int part = 0; part < 2; part++) {
+                float hv[8], wv[8];
+                lds_v8<FUSED_WF_K8>(hx, K, (c * WAVE + lane) * 16 + part * 8, hv);
+                lds_v8<FUSED_WF_K8>(nw, K, (c * WAVE + lane) * 16 + part * 8, wv);
+#pragma unroll
+                for (int e = 0; e < 8; e++) xv[c][part * 8 + e] = (hv[e] * inv) * wv[e];
+            }
+        finish(xv, lane, v);
+    }
+    __device__ __forceinline__ void dots_plain(const float *x, int lane, float (&v)[R]) const {
+        float xv[C][16];
+#pragma unroll
+        for (int c = 0; c < C; c++)
+#pragma unroll
+            for (int part = 0; part < 2; part++) lds_v8<FUSED_WF_K8>(x, K, (c * WAVE + lane) * 16 + part * 8, xv[c] + part * 8);
+        finish(xv, lane, v);
+    }
+};
+
+// R rows x the K slice [k0, k0 + KS) of a K8 matrix with KTOT columns. A register set holds four rows of one
+// 256-wide block that the slice touches (lane = 16 * row + sub-block of the block); lanes whose sub-block lies
+// outside the slice carry zeros. A block that the slice shares with a neighbouring slice takes its Q8_K
+// maximum from both sides: `shared_max[0]` is the other side's maximum of the block the slice starts in,
+// `shared_max[1]` that of the block it ends in.
+template <int R, int KS, int KTOT>
+struct SliceRows<FUSED_WF_K8, R, KS, KTOT> {
+    static constexpr int LANES_PER_ROW = 16, ROWS_PER_SET = 4, Q = R / ROWS_PER_SET;
+    static constexpr int P = (KS + 255) / 256;  // blocks a slice touches (slices start on a block or end on one)
+    static constexpr int RS = KTOT / 8 + KTOT / 64;
+    static_assert(R % ROWS_PER_SET == 0 && Q >= 1 && KTOT % 256 == 0 && KS % 16 == 0, "four rows and one block per register set");
+    static_assert(KS % 256 == 0 || (KS % 128 == 0 && P == KS / 256 + 1), "slices are whole blocks, or whole blocks and a half");
+    u32x4 q[Q][P];
+    uint32_t sub[Q][P], dd[Q][P];
+    // global column of the lane's sub-block in part p, and whether it lies inside the slice
+    __device__ __forceinline__ static int col(int k0, int p, int lane) { return (k0 / 256 + p) * 256 + (lane % LANES_PER_ROW) * 16; }
+    __device__ __forceinline__ static bool inside(int k0, int p, int lane) {
+        const int k = col(k0, p, lane);
+        return k >= k0 && k < k0 + KS;
+    }
+    __device__ __forceinline__ void load(const void *quants, const uint16_t *scales, int row0, int k0, int lane, int s0 = 0, int s1 = Q) {
+        const unsigned char *base = reinterpret_cast<const unsigned char *>(quants);
+        const unsigned char *rec = reinterpret_cast<const unsigned char *>(scales);
+#pragma unroll
+        for (int s = 0; s < Q; s++)
+#pragma unroll
+            for (int p = 0; p < P; p++) {
+                if (s < s0 || s >= s1) continue;
+                const size_t row = (size_t)(row0 + s * ROWS_PER_SET + lane / LANES_PER_ROW);
+                const bool in = inside(k0, p, lane);
+                const int k = in ? col(k0, p, lane) : k0;  // lanes outside re-read the slice's first sub-block
+                q[s][p] = ld128_global_stream(base + row * KTOT + k);
+                sub[s][p] = __builtin_nontemporal_load((global_u16_ptr)(rec + row * RS + (size_t)(k / 16) * 2));
+                dd[s][p] = __builtin_nontemporal_load((global_u32_ptr)(rec + row * RS + KTOT / 8 + (size_t)(k0 / 256 + p) * 4));
+                if (!in) q[s][p] = u32x4{0u, 0u, 0u, 0u};
+            }
+    }
+    __device__ __forceinline__ void dots(const float *x, int lane, int k0, const float *shared_max, float (&v)[Q]) const {
+        Q8kLane a[P];
+#pragma unroll
+        for (int p = 0; p < P; p++) {
+            float xv[16];
+            const bool in = inside(k0, p, lane);
+            const int local = in ? col(k0, p, lane) - k0 : 0;
+            lds_v8<FUSED_WF_K8>(x, KS, local, xv);
+            lds_v8<FUSED_WF_K8>(x, KS, local + 8, xv + 8);
+#pragma unroll
+            for (int j = 0; j < 16; j++) xv[j] = in ? xv[j] : 0.f;
+            float amax = dpp_row_fmax(abs_max16(xv));
+            const int b_lo = (k0 / 256 + p) * 256;  // the block's first column
+            if (b_lo < k0) amax = fmaxf(amax, shared_max[0]);
+            if (b_lo + 256 > k0 + KS) amax = fmaxf(amax, shared_max[1]);
+            a[p] = q8k_lane(xv, amax);
+        }
+#pragma unroll
+        for (int s = 0; s < Q; s++) {
+            float acc = 0.f;
+#pragma unroll
+            for (int p = 0; p < P; p++) acc = __fadd_rn(acc, k8_block(q[s][p], sub[s][p], dd[s][p], a[p]));
+            v[s] = acc;
+        }
     }
 };
 
@@ -639,7 +869,7 @@ struct Split {
 // caller has not yet passed the barrier behind which the last hidden state is staged, and the first batch is
 // requested before it. Ends behind the barrier after which head_v / head_i hold every wavefront's best row.
 constexpr int HEAD_WORKERS = NCW + 4;
-template <class GE, bool EARLY>
+template <class GE, int WF, bool EARLY>
 __device__ __forceinline__ void head_rows(const FusedDecodeArgs &a, Lds<GE> &sm, const int wg, const int worker, const int lane) {
     constexpr int HR = GE::HR, HC = GE::HIDDEN / 512;
     const int per_wg = (a.vocab + GE::NWG - 1) / GE::NWG;
@@ -662,8 +892,8 @@ __device__ __forceinline__ void head_rows(const FusedDecodeArgs &a, Lds<GE> &sm,
 #pragma unroll
     for (int c = 0; c < HC; c++) {
         float hv[8], wv[8];
-        lds_x8(sm.hx, (c * WAVE + lane) * 8, hv);
-        lds_x8(sm.nw, (c * WAVE + lane) * 8, wv);
+        lds_v8<WF>(sm.hx, GE::HIDDEN, (c * WAVE + lane) * 8, hv);
+        lds_v8<WF>(sm.nw, GE::HIDDEN, (c * WAVE + lane) * 8, wv);
 #pragma unroll
         for (int e = 0; e < 8; e++) xv[c][e] = (hv[e] * inv) * wv[e];
     }
@@ -911,7 +1141,8 @@ __device__ __forceinline__ void compute_role(const FusedDecodeArgs &a, Lds<GE> &
         {
             using S = decltype(s.wo);
             float v[S::Q];
-            s.wo.dots(sm.attn, lane, v);
+            if constexpr (WF == FUSED_WF_K8) s.wo.dots(sm.attn, lane, sp.kh * GE::KSO, sm.nbmax, v);  // whole blocks: nbmax is not read
+            else s.wo.dots(sm.attn, lane, v);
             if (lane % S::LANES_PER_ROW == 0) {
 #pragma unroll
                 for (int q = 0; q < S::Q; q++) sm.pub[cw * GE::RPW + q * S::ROWS_PER_SET + lane / S::LANES_PER_ROW] = v[q];
@@ -945,7 +1176,8 @@ __device__ __forceinline__ void compute_role(const FusedDecodeArgs &a, Lds<GE> &
         {
             using S = decltype(s.wd);
             float v[S::Q];
-            s.wd.dots(sm.act, lane, v);
+            if constexpr (WF == FUSED_WF_K8) s.wd.dots(sm.act, lane, sp.kh * GE::KSD, sm.nbmax, v);
+            else s.wd.dots(sm.act, lane, v);
             if (lane % S::LANES_PER_ROW == 0) {
 #pragma unroll
                 for (int q = 0; q < S::Q; q++) sm.pub[cw * GE::RPW + q * S::ROWS_PER_SET + lane / S::LANES_PER_ROW] = v[q];
@@ -954,7 +1186,7 @@ __device__ __forceinline__ void compute_role(const FusedDecodeArgs &a, Lds<GE> &
         wg_barrier();
     }
 
-    if (a.head_w) head_rows<GE, true>(a, sm, wg, cw, lane);
+    if (a.head_w) head_rows<GE, WF, true>(a, sm, wg, cw, lane);
 }
 
 // Slot of hidden element k in the XH / XO areas: the communicating thread c = k % 256 owns elements
@@ -967,7 +1199,7 @@ __device__ __forceinline__ int hidden_slot(int k) {
 
 __device__ __forceinline__ unsigned xcc_id() { return __builtin_amdgcn_s_getreg((3 << 11) | (0 << 6) | 20) & 0xF; }
 
-template <class GE>
+template <class GE, int WF>
 __device__ __forceinline__ void comm_role(const FusedDecodeArgs &a, Lds<GE> &sm, const int wg, const int cwv,
                                           const int lane, const int pos, const uint32_t launches) {
     constexpr int G = GE::G, HD = GE::HD, NJ = GE::NJ;
@@ -1097,8 +1329,8 @@ __device__ __forceinline__ void comm_role(const FusedDecodeArgs &a, Lds<GE> &sm,
         if (lane == 0) sm.red[cwv] = ss;
 #pragma unroll
         for (int j = 0; j < NJ; j++) {
-            sm.hx[ct + CT * j] = h[j];
-            sm.nw[ct + CT * j] = nwv[j];
+            sm.hx[XLay<WF>::pos(ct + CT * j, GE::HIDDEN)] = h[j];
+            sm.nw[XLay<WF>::pos(ct + CT * j, GE::HIDDEN)] = nwv[j];
         }
     };
     // copy a vector of this KV head's group (n_units 16-byte units in plain slot order) into LDS
@@ -1108,8 +1340,8 @@ __device__ __forceinline__ void comm_role(const FusedDecodeArgs &a, Lds<GE> &sm,
         u32x4 w[1];
         poll_units<1>(ps, src, unit, on, tag, w);
         if (on[0]) {
-            dst[2 * ct] = __uint_as_float(w[0].x);
-            dst[2 * ct + 1] = __uint_as_float(w[0].z);
+            dst[XLay<WF>::pos(2 * ct, 2 * n_units)] = __uint_as_float(w[0].x);
+            dst[XLay<WF>::pos(2 * ct + 1, 2 * n_units)] = __uint_as_float(w[0].z);
         }
     };
 
@@ -1362,10 +1594,47 @@ __device__ __forceinline__ void comm_role(const FusedDecodeArgs &a, Lds<GE> &sm,
         wg_barrier();
         mark();
         if (ct < GE::APW) st_slot(lc, sp.split * GE::APW + ct, sm.pub[ct], tag, near_g);
+        // K8 with K slices of down that share a 256-wide block with the neighbouring group: the Q8_K scale of such
+        // a block needs the largest magnitude on both sides. Every workgroup writes the maxima of its own values
+        // in the block its group's slice starts in and in the block it ends in through to memory ...
+        constexpr bool SHARED_BLOCKS = WF == FUSED_WF_K8 && GE::KSD % 256 != 0;
+        unsigned char *lm = xc + (size_t)GE::LM0 * 8;
+        if (SHARED_BLOCKS && cwv == 1) {  // (wavefront 0 is busy publishing the values themselves)
+            static_assert(GE::APW <= WAVE, "one wavefront holds a workgroup's SiLU*up values");
+            const int k0 = sp.kh * GE::KSD, k = k0 + sp.split * GE::APW + lane;  // column of this lane's value
+            const float mag = lane < GE::APW ? fabsf(sm.pub[lane]) : 0.f;
+            const bool first = lane < GE::APW && k / 256 * 256 < k0, last = lane < GE::APW && k / 256 * 256 + 256 > k0 + GE::KSD;
+            const float m_first = wave_max(first ? mag : 0.f), m_last = wave_max(last ? mag : 0.f);
+            if (lane == 0) {
+                st_slot(lm, 2 * wg, m_first, tag, false);
+                st_slot(lm, 2 * wg + 1, m_last, tag, false);
+            }
+        }
 
         // ── into the down phase ──
         ps.where = 6u | (uint32_t)l << 4 | (uint32_t)wg << 12;
         stage_group(lc, GE::KSD / 2, tag, sm.act);
+        // (behind the staging, not beside it: a CU returns its loads in issue order, and a poll of this CU's L2
+        // issued behind a poll that goes to memory would wait for it)
+        if (SHARED_BLOCKS && cwv == 0) {
+            // ... and reads the group before's maxima of its last block (lanes 0-31) and the group after's of its
+            // first block (lanes 32-63): the workgroups of KV head kh are wg = kh + KVH * split
+            static_assert(GE::SPH <= 32, "a neighbouring group's workgroups fit half a wavefront");
+            const int k0 = sp.kh * GE::KSD;
+            const bool after = lane >= 32;
+            const int nb = sp.kh + (after ? 1 : -1), i = lane & 31;
+            const bool want = i < GE::SPH && (after ? (k0 + GE::KSD) % 256 != 0 && nb < GE::KVH : k0 % 256 != 0 && nb >= 0);
+            int unit[1] = {want ? nb + GE::KVH * i : 0};
+            bool on[1] = {want};
+            u32x4 w[1];
+            poll_units<1>(ps, lm, unit, on, tag, w);
+            const float m = want ? __uint_as_float(after ? w[0].x : w[0].z) : 0.f;
+            const float m_before = wave_max(after ? 0.f : m), m_after = wave_max(after ? m : 0.f);
+            if (lane == 0) {
+                sm.nbmax[0] = m_before;
+                sm.nbmax[1] = m_after;
+            }
+        }
         wg_barrier();
         mark();
         wg_barrier();
@@ -1384,7 +1653,7 @@ __device__ __forceinline__ void comm_role(const FusedDecodeArgs &a, Lds<GE> &sm,
             for (int j = 0; j < NJ; j++) a.hidden_out[ct + CT * j] = h[j];
         }
         wg_barrier();
-        head_rows<GE, false>(a, sm, wg, NCW + cwv, lane);
+        head_rows<GE, WF, false>(a, sm, wg, NCW + cwv, lane);
         // this workgroup's best row, then (workgroup 0) the best of all and the end of the step
         // (greedy pick of reference src/generate.rs:735-742 taken on the device)
         unsigned char *cand = a.xch + (size_t)GE::CAND0 * 8;
@@ -1505,7 +1774,7 @@ __global__ __launch_bounds__(FT) void decode_fused_kernel(FusedDecodeArgs a) {
         compute_role<GE, WF>(a, sm, wg, wave, lane, pos);
     } else {
         const uint32_t launches = __hip_atomic_load(a.ctl, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        comm_role<GE>(a, sm, wg, wave - NCW, lane, pos, launches);
+        comm_role<GE, WF>(a, sm, wg, wave - NCW, lane, pos, launches);
     }
 }
 
@@ -1547,6 +1816,9 @@ Instance instance() {
 // live_rows = 0, the one that holds the most.
 const Instance *find_instance(const FusedShape &s, int live_rows = 1) {
     static const Instance table[] = {
+        instance<GeoQwen3_0p6bShort, FUSED_WF_K8>(), instance<GeoSmallQShort, FUSED_WF_K8>(),
+        instance<GeoQwen3_0p6b, FUSED_WF_K8>(), instance<GeoSmallQ, FUSED_WF_K8>(),
+        instance<GeoQwen3_0p6bLong, FUSED_WF_K8>(), instance<GeoSmallQLong, FUSED_WF_K8>(),
         instance<GeoQwen3_0p6bShort, FUSED_WF_BF16>(), instance<GeoQwen3_0p6bShort, FUSED_WF_Q8_0>(), instance<GeoQwen3_0p6bShort, FUSED_WF_Q4_0>(),
         instance<GeoSmallShort, FUSED_WF_BF16>(),      instance<GeoSmallQShort, FUSED_WF_Q8_0>(),     instance<GeoSmallQShort, FUSED_WF_Q4_0>(),
         instance<GeoQwen3_0p6b, FUSED_WF_BF16>(), instance<GeoQwen3_0p6b, FUSED_WF_Q8_0>(), instance<GeoQwen3_0p6b, FUSED_WF_Q4_0>(),

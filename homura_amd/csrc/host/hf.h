@@ -186,8 +186,11 @@ class HfModel {
     // matrix of each run of same-type neighbours inside q|k|v and gate|up, and holds the whole run.
     // quant[first]: the raw blocks of a stacked run; planes[first]: the same run re-packed for the decode
     // GEMVs (Q8_0 / Q4_0 with K <= 4096; empty otherwise)
-    struct LayerPacked { Buffer qkv, o, gate_up, down, qkv_bias, quant[7], planes[7]; };
+    // k8[g] (g = q|k|v, o, gate|up, down): a K-quant model's matrices re-packed for the whole-step launch
+    // (kquant_planes8.h): the byte plane of the stacked rows, then their scale records
+    struct LayerPacked { Buffer qkv, o, gate_up, down, qkv_bias, quant[7], planes[7], k8[4]; };
     int build_quant_planes();
+    int build_k8_planes();
     // First member and member count of the stacked run that projection `which` of `layer` belongs to.
     void quant_run(int layer, int which, int *first, int *count) const;
     std::vector<LayerPacked> packed_;

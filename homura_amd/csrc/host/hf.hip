@@ -6,6 +6,7 @@
 
 #include "../attention.h"
 #include "../decode_fused.h"
+#include "../kquant_planes8.h"
 #include "../gemv_bf16.h"
 #include "../gemm_bf16_mfma.h"
 #include "../gemv_kquant.h"
@@ -185,6 +186,43 @@ int HfModel::build_quant_planes() {
         const int rc = pack_q6k_planes(ctx_, lm_head_blocks_.as<uint8_t>(), lm_head_planes_.as<uint8_t>(), cfg_.vocab_size, hidden, false);
         if (rc != HM_OK) return rc;
     }
+    return hm_sync(ctx_);
+}
+
+// A model whose projections are all Q4_K or Q6_K (the Q4_K_M-style mixes): every group of matrices that share an
+// activation (q|k|v, o, gate|up, down) once more as byte planes with per-row scale records, which the whole-step
+// launch reads (the raw blocks stay for the prompt pass, the per-projection path and the weight listing).
+int HfModel::build_k8_planes() {
+    const int hidden = cfg_.hidden_size, inter = cfg_.intermediate_size, qd = cfg_.q_dim(), kvd = cfg_.kv_dim();
+    const int kdim[7] = {hidden, hidden, hidden, qd, hidden, hidden, inter};
+    const int ndim[7] = {qd, kvd, kvd, hidden, inter, inter, hidden};
+    const int group_first[4] = {0, 3, 4, 6}, group_count[4] = {3, 1, 2, 1};
+    for (int l = 0; l < cfg_.num_hidden_layers; l++)
+        for (int g = 0; g < 4; g++) {
+            const int K = kdim[group_first[g]];
+            int n = 0;
+            for (int e = 0; e < group_count[g]; e++) n += ndim[group_first[g] + e];
+            const size_t bytes = k8_plane_bytes(n, K) + k8_record_bytes(n, K);
+            Buffer &dst = packed_[l].k8[g];
+            dst = Buffer::alloc_bytes(ctx_, bytes, {(int64_t)bytes}, DType::Q4_K);
+            if (!dst) return HM_ERR_OOM;
+            int row0 = 0;
+            for (int e = 0; e < group_count[g]; e++) {
+                const int j = group_first[g] + e;
+                const DType t = proj_dtype(l, j);
+                // projection j's raw blocks sit in the run of same-typed neighbours that starts at `first`
+                int first, count;
+                quant_run(l, j, &first, &count);
+                if (!packed_[l].quant[first]) return hm_set_error(ctx_, HM_ERR_STATE, "layer %d projection %d has no blocks", l, j);
+                size_t skip = 0;
+                for (int b = first; b < j; b++) skip += dtype_bytes_for_elements(t, (size_t)ndim[b] * K, nullptr);
+                const int rc = pack_k8_rows(ctx_, t == DType::Q6_K ? HM_DTYPE_Q6_K : HM_DTYPE_Q4_K,
+                                            packed_[l].quant[first].as<uint8_t>() + skip, ndim[j], K, dst.as<uint8_t>(),
+                                            dst.as<uint8_t>() + k8_plane_bytes(n, K), row0);
+                if (rc != HM_OK) return rc;
+                row0 += ndim[j];
+            }
+        }
     return hm_sync(ctx_);
 }
 
@@ -426,16 +464,25 @@ int HfModel::finalize(int max_seq_len) {
     if (dtype_is_quantized(weight_dtype_)) {
         const DType t = proj_dtype(0, 0);
         fused_format = t == DType::Q8_0 || t == DType::Q4_0;
+        bool all_kquant = true;  // any mix of Q4_K and Q6_K
+        for (int l = 0; l < cfg_.num_hidden_layers; l++)
+            for (int j = 0; j < 7; j++) all_kquant = all_kquant && (proj_dtype(l, j) == DType::Q4_K || proj_dtype(l, j) == DType::Q6_K);
         for (int l = 0; l < cfg_.num_hidden_layers && fused_format; l++) {
             for (int j = 0; j < 7; j++) fused_format = fused_format && proj_dtype(l, j) == t;
             fused_format = fused_format && packed_[l].planes[0] && packed_[l].planes[3] && packed_[l].planes[4] && packed_[l].planes[6];
         }
         fused_wf_ = t == DType::Q4_0 ? FUSED_WF_Q4_0 : FUSED_WF_Q8_0;
+        if (all_kquant) {
+            fused_format = true;
+            fused_wf_ = FUSED_WF_K8;
+        }
     }
     if (fused_format) {
         const FusedShape fs{cfg_.hidden_size, cfg_.num_attention_heads, cfg_.kv_heads(), cfg_.head_dim(),
                             cfg_.intermediate_size, fused_wf_};
-        if (decode_fused_supported(ctx_, fs, cfg_.num_hidden_layers, max_seq_len, nullptr)) {
+        bool served = decode_fused_supported(ctx_, fs, cfg_.num_hidden_layers, max_seq_len, nullptr);
+        if (served && fused_wf_ == FUSED_WF_K8 && (rc = build_k8_planes()) != HM_OK) return rc;
+        if (served) {
             s.fused_layers = Buffer::alloc_bytes(ctx_, sizeof(FusedLayerPtrs) * (size_t)cfg_.num_hidden_layers,
                                                  {cfg_.num_hidden_layers}, DType::I64);
             const size_t xb = decode_fused_xch_bytes(fs);
@@ -1487,6 +1534,20 @@ int HfModel::refresh_fused_table() {
             f.wgu = packed_[l].gate_up.ptr();
             f.wd = packed_[l].down.ptr();
             f.sqkv = f.so = f.sgu = f.sd = nullptr;
+        } else if (fused_wf_ == FUSED_WF_K8) {  // byte planes of the four groups, scale records behind them
+            const int hidden = cfg_.hidden_size, inter = cfg_.intermediate_size, qd = cfg_.q_dim(), kvd = cfg_.kv_dim();
+            auto records = [&](const Buffer &b, int n, int k) {
+                return reinterpret_cast<const uint16_t *>(b.as<uint8_t>() + k8_plane_bytes(n, k));
+            };
+            const LayerPacked &lp = packed_[l];
+            f.wqkv = lp.k8[0].ptr();
+            f.sqkv = records(lp.k8[0], qd + 2 * kvd, hidden);
+            f.wo = lp.k8[1].ptr();
+            f.so = records(lp.k8[1], hidden, qd);
+            f.wgu = lp.k8[2].ptr();
+            f.sgu = records(lp.k8[2], 2 * inter, hidden);
+            f.wd = lp.k8[3].ptr();
+            f.sd = records(lp.k8[3], hidden, inter);
         } else {  // quant planes of the four runs, scales behind the quants
             const bool q4 = fused_wf_ == FUSED_WF_Q4_0;
             const int hidden = cfg_.hidden_size, inter = cfg_.intermediate_size, qd = cfg_.q_dim(), kvd = cfg_.kv_dim();

@@ -365,3 +365,42 @@ def test_a_wait_that_gives_up_is_reported_and_the_call_runs_again_per_projection
         gm.reset_kv_cache()
         gm.set_whole_step(True)
 
+
+
+def test_kquant_mix_whole_step_against_oracle_and_per_projection_path(ctx):
+    """Q4_K / Q6_K projections (a Q4_K_M-style mix, re-packed into byte planes at finalize) through the
+    whole-step launch: the same Q8_K activation quantisation and integer dot products as the per-projection
+    kernels and the oracle (reference src/graph_builder/emit_quant.rs:165-816). Where the two GPU paths or the
+    oracle round an activation to different Q8_K integers the logits move by ~1e-3 of their scale; tokens are
+    compared where the oracle's margin is clear."""
+    from homura_amd.runtime import DTYPE_Q8_0
+    cfg = synth_model.SMALL_WS_Q
+    mix = synth_model.q4_k_m_mix(cfg)
+    weights = synth_model.synth_weights(cfg, 911, DTYPE_Q8_0, has_qk_norm=True, proj_dtypes=mix)
+    gm = synth_model.build_model(ctx, cfg, weights, 1024, DTYPE_Q8_0, has_qk_norm=True, proj_dtypes=mix)
+    om = mf.build_oracle_model(cfg, weights, 1024, DTYPE_Q8_0, has_qk_norm=True, proj_dtypes=mix)
+    assert gm.whole_step_available() and gm.whole_step()
+    kv = synth_model.synth_kv(cfg, 31, 61)
+    ids = synth.token_ids(32, 7, cfg.vocab_size)
+    gm.set_prefill_min(0)
+    gm.init_kv_cache(kv, 61)
+    mf.oracle_init_kv(om, kv)
+    got = gm.run_kv(ids)
+    got_t = gm.generate_greedy(ids[:1], 20)
+    gm.whole_step_status()
+    assert gm.launches_per_step() == 3
+    want = np.concatenate([om.run_kv(ids[i:i + 1]) for i in range(7)])
+    for i in range(7):
+        err = mf.rel_err(got[i], want[i])
+        say(f"k-quant mix: position {i} rel err {err:.2e}")
+        assert err < 1e-2
+    gm.set_whole_step(False)
+    gm.init_kv_cache(kv, 61)
+    ref = gm.run_kv(ids)
+    ref_t = gm.generate_greedy(ids[:1], 20)
+    assert gm.launches_per_step() > 3
+    assert mf.rel_err(got, ref) < 1e-2
+    same = int(np.sum(got_t == ref_t))
+    say(f"k-quant mix: {same} of {len(ref_t)} greedy tokens equal on the two GPU paths")
+    assert np.array_equal(got_t[:4], ref_t[:4])
+    gm.close()
