@@ -985,6 +985,11 @@ __device__ __forceinline__ void compute_role(const FusedDecodeArgs &a, Lds<GE> &
     };
 
     constexpr int KV_CUT = NR / 2, WG_CUT = 2 * GE::RGW / 3;
+    // With more than four row rounds in registers a layer's slices and the next layer's cache rows do not
+    // all fit at once (a spilled value would come back through the memory pipeline, behind every outstanding
+    // weight request): those instances request the down rows, the second half of the cache rows and the
+    // Q|K|V rows one phase later, when the registers they land in have just been read for the last time.
+    constexpr bool LATE = NR > 4;
     {
         // the first layer's slice, in the order the loop re-requests it (the rest follows inside the loop)
         const FusedLayerPtrs lp = sm.lp[0];
@@ -1006,7 +1011,7 @@ __device__ __forceinline__ void compute_role(const FusedDecodeArgs &a, Lds<GE> &
         // Requests go out at the start of a phase, never right before the communicating wavefronts poll:
         // the CU's vector memory pipeline returns data in order, so a poll issued behind a weight request
         // waits for HBM. Here: this layer's down rows and last gate|up rows (registers last read one layer ago).
-        load_wd(sm.lp[l]);
+        if (!LATE) load_wd(sm.lp[l]);
         load_wg(sm.lp[l], WG_CUT, GE::RGW);
         {
             const float tot = ((sm.red[0] + sm.red[1]) + sm.red[2]) + sm.red[3];
@@ -1029,101 +1034,136 @@ __device__ __forceinline__ void compute_role(const FusedDecodeArgs &a, Lds<GE> &
         //    Every wavefront leaves the (max, sum, P.V) of its own rows in LDS; the publishing threads
         //    merge the four. ──
         wg_barrier();
-        load_wq(nx, 0, GE::RQW);
+        if (!LATE) load_wq(nx, 0, GE::RQW);
         if (sp.split < sp.nsl) {
             float qv[G][8];
 #pragma unroll
             for (int g = 0; g < G; g++) lds_x8(sm.qs[g], dl * 8, qv[g]);
             const bool with_new = sp.owner && cw == 0;  // the new row rides with wavefront 0 of the last split
-            float kf[NR + 1][8];
+            // The rounds held in registers are taken PR at a time (their float forms would not fit beside the
+            // weight slices otherwise, and a spilled register is reloaded through the same in-order memory
+            // pipeline the weight requests wait in); passes after the first rescale what the earlier ones left.
+            // The new row rides with the last pass.
+            constexpr int PR = NR > 4 ? 2 : NR, NPASS = NR / PR;
+            static_assert(NR % PR == 0, "row rounds are taken in equal passes");
+            float m[G], lsum[G], acc[G][8];
 #pragma unroll
-            for (int i = 0; i < NR; i++) unpack8f(s.kr[i], kf[i]);
-            lds_x8(sm.knew, dl * 8, kf[NR]);
-            float sc[G][NR + 1];
+            for (int ps = 0; ps < NPASS; ps++) {
+                const int i0 = ps * PR;
+                const bool last = ps == NPASS - 1;
+                // slot PR is the new row (last pass only; elsewhere it is dead and multiplies zeros)
+                float kf[PR + 1][8];
 #pragma unroll
-            for (int g = 0; g < G; g++)
+                for (int i = 0; i < PR; i++) unpack8f(s.kr[i0 + i], kf[i]);
+                if (last) lds_x8(sm.knew, dl * 8, kf[PR]);
+                else {
 #pragma unroll
-                for (int i = 0; i <= NR; i++) sc[g][i] = 0.f;
-#pragma unroll
-            for (int e = 0; e < 8; e++)
+                    for (int e = 0; e < 8; e++) kf[PR][e] = 0.f;
+                }
+                float sc[G][PR + 1];
 #pragma unroll
                 for (int g = 0; g < G; g++)
 #pragma unroll
-                    for (int i = 0; i <= NR; i++) sc[g][i] = fmaf(kf[i][e], qv[g][e], sc[g][i]);
-            // sums over the lanes of a row, all (head, row) chains side by side
+                    for (int i = 0; i <= PR; i++) sc[g][i] = 0.f;
 #pragma unroll
-            for (int g = 0; g < G; g++)
+                for (int e = 0; e < 8; e++)
 #pragma unroll
-                for (int i = 0; i <= NR; i++) sc[g][i] += dpp_move<0xB1, 0xF>(sc[g][i], 0.f);
+                    for (int g = 0; g < G; g++)
 #pragma unroll
-            for (int g = 0; g < G; g++)
-#pragma unroll
-                for (int i = 0; i <= NR; i++) sc[g][i] += dpp_move<0x4E, 0xF>(sc[g][i], 0.f);
-#pragma unroll
-            for (int g = 0; g < G; g++)
-#pragma unroll
-                for (int i = 0; i <= NR; i++) sc[g][i] += dpp_move<0x141, 0xF>(sc[g][i], 0.f);
-            if (LPR == 16) {
+                        for (int i = 0; i <= PR; i++) sc[g][i] = fmaf(kf[i][e], qv[g][e], sc[g][i]);
+                // sums over the lanes of a row, all (head, row) chains side by side
 #pragma unroll
                 for (int g = 0; g < G; g++)
 #pragma unroll
-                    for (int i = 0; i <= NR; i++) sc[g][i] += dpp_move<0x140, 0xF>(sc[g][i], 0.f);
-            }
-            bool live[NR + 1];
+                    for (int i = 0; i <= PR; i++) sc[g][i] += dpp_move<0xB1, 0xF>(sc[g][i], 0.f);
 #pragma unroll
-            for (int i = 0; i < NR; i++) live[i] = (i * NCW + cw) * RPI + sub < sp.cached;
-            live[NR] = with_new;
-            float m[G];
+                for (int g = 0; g < G; g++)
 #pragma unroll
-            for (int g = 0; g < G; g++) {
-                m[g] = -INFINITY;
+                    for (int i = 0; i <= PR; i++) sc[g][i] += dpp_move<0x4E, 0xF>(sc[g][i], 0.f);
 #pragma unroll
-                for (int i = 0; i <= NR; i++) {
-                    sc[g][i] = live[i] ? sc[g][i] * a.scale : -INFINITY;
-                    m[g] = fmaxf(m[g], sc[g][i]);
+                for (int g = 0; g < G; g++)
+#pragma unroll
+                    for (int i = 0; i <= PR; i++) sc[g][i] += dpp_move<0x141, 0xF>(sc[g][i], 0.f);
+                if (LPR == 16) {
+#pragma unroll
+                    for (int g = 0; g < G; g++)
+#pragma unroll
+                        for (int i = 0; i <= PR; i++) sc[g][i] += dpp_move<0x140, 0xF>(sc[g][i], 0.f);
                 }
-            }
-            wave_max_n<G>(m);
-            // softmax terms against the wavefront's own maximum (max, exp, sum:
-            // reference emit_softmax, src/graph_builder/emit_linalg.rs:509-528)
-            float pr[G][NR + 1], lsum[G];
+                bool live[PR + 1];
 #pragma unroll
-            for (int g = 0; g < G; g++) {
-                lsum[g] = 0.f;
-#pragma unroll
-                for (int i = 0; i <= NR; i++) {
-                    pr[g][i] = live[i] ? __expf(sc[g][i] - m[g]) : 0.f;
-                    // a cache row is counted by the first of its lanes, the new row by lane 0
-                    if (i < NR ? dl == 0 : lane == 0) lsum[g] += pr[g][i];
-                }
-            }
-            wave_sum_n<G>(lsum);
-            if (lane < G) {
-                float mm = 0.f, ll = 0.f;
+                for (int i = 0; i < PR; i++) live[i] = ((i0 + i) * NCW + cw) * RPI + sub < sp.cached;
+                live[PR] = last && with_new;
+                float mp[G];
 #pragma unroll
                 for (int g = 0; g < G; g++) {
-                    mm = lane == g ? m[g] : mm;
-                    ll = lane == g ? lsum[g] : ll;
+                    mp[g] = -INFINITY;
+#pragma unroll
+                    for (int i = 0; i <= PR; i++) {
+                        sc[g][i] = live[i] ? sc[g][i] * a.scale : -INFINITY;
+                        mp[g] = fmaxf(mp[g], sc[g][i]);
+                    }
                 }
-                sm.wstat[cw][lane][0] = mm;
-                sm.wstat[cw][lane][1] = ll;
-            }
-            float vf[NR + 1][8];
-#pragma unroll
-            for (int i = 0; i < NR; i++) unpack8f(s.vr[i], vf[i]);
-            lds_x8(sm.vnew, dl * 8, vf[NR]);
-            float acc[G][8];
-#pragma unroll
-            for (int g = 0; g < G; g++)
-#pragma unroll
-                for (int e = 0; e < 8; e++) acc[g][e] = 0.f;
-#pragma unroll
-            for (int i = 0; i <= NR; i++) {
+                wave_max_n<G>(mp);
+                // softmax terms against the wavefront's own maximum (max, exp, sum:
+                // reference emit_softmax, src/graph_builder/emit_linalg.rs:509-528)
+                float alpha[G];
 #pragma unroll
                 for (int g = 0; g < G; g++) {
-                    const float p = (i < NR || sub == 0) ? pr[g][i] : 0.f;  // the new row: one row group only
+                    if (ps == 0) {
+                        m[g] = mp[g];
+                        alpha[g] = 0.f;
+                        lsum[g] = 0.f;
+                    } else {
+                        const float mn = fmaxf(m[g], mp[g]);
+                        alpha[g] = m[g] == -INFINITY ? 0.f : __expf(m[g] - mn);  // nothing live so far: nothing to keep
+                        m[g] = mn;
+                        lsum[g] *= alpha[g];
+                    }
+                }
+                float pr[G][PR + 1];
 #pragma unroll
-                    for (int e = 0; e < 8; e++) acc[g][e] = fmaf(p, vf[i][e], acc[g][e]);
+                for (int g = 0; g < G; g++) {
+#pragma unroll
+                    for (int i = 0; i <= PR; i++) {
+                        pr[g][i] = live[i] ? __expf(sc[g][i] - m[g]) : 0.f;
+                        // a cache row is counted by the first of its lanes, the new row by lane 0
+                        if (i < PR ? dl == 0 : lane == 0) lsum[g] += pr[g][i];
+                    }
+                }
+                if (last) {
+                    wave_sum_n<G>(lsum);
+                    if (lane < G) {
+                        float mm = 0.f, ll = 0.f;
+#pragma unroll
+                        for (int g = 0; g < G; g++) {
+                            mm = lane == g ? m[g] : mm;
+                            ll = lane == g ? lsum[g] : ll;
+                        }
+                        sm.wstat[cw][lane][0] = mm;
+                        sm.wstat[cw][lane][1] = ll;
+                    }
+                }
+                float vf[PR + 1][8];
+#pragma unroll
+                for (int i = 0; i < PR; i++) unpack8f(s.vr[i0 + i], vf[i]);
+                if (last) lds_x8(sm.vnew, dl * 8, vf[PR]);
+                else {
+#pragma unroll
+                    for (int e = 0; e < 8; e++) vf[PR][e] = 0.f;
+                }
+#pragma unroll
+                for (int g = 0; g < G; g++)
+#pragma unroll
+                    for (int e = 0; e < 8; e++) acc[g][e] = ps == 0 ? 0.f : acc[g][e] * alpha[g];
+#pragma unroll
+                for (int i = 0; i <= PR; i++) {
+#pragma unroll
+                    for (int g = 0; g < G; g++) {
+                        const float p = (i < PR || sub == 0) ? pr[g][i] : 0.f;  // the new row: one row group only
+#pragma unroll
+                        for (int e = 0; e < 8; e++) acc[g][e] = fmaf(p, vf[i][e], acc[g][e]);
+                    }
                 }
             }
 #pragma unroll
@@ -1133,11 +1173,13 @@ __device__ __forceinline__ void compute_role(const FusedDecodeArgs &a, Lds<GE> &
                 *reinterpret_cast<f32x4 *>(dst + 4) = f32x4{acc[g][4], acc[g][5], acc[g][6], acc[g][7]};
             }
         }
+        if (LATE) load_wq(nx, 0, GE::RQW);  // behind the arithmetic that needed the registers
         wg_barrier();
 
         // ── O projection rows (reference src/hf/emitter.rs:738-745) ──
         wg_barrier();
         load_kv(nx, 0, KV_CUT);
+        if (LATE) load_wd(sm.lp[l]);
         {
             using S = decltype(s.wo);
             float v[S::Q];
@@ -1152,7 +1194,7 @@ __device__ __forceinline__ void compute_role(const FusedDecodeArgs &a, Lds<GE> &
 
         // ── gate|up rows, SiLU(gate) * up (reference src/hf/emitter.rs:787-799) ──
         wg_barrier();
-        load_kv(nx, KV_CUT, NR);
+        if (!LATE) load_kv(nx, KV_CUT, NR);
         load_wo(nx);
         {
             const float tot = ((sm.red[0] + sm.red[1]) + sm.red[2]) + sm.red[3];
@@ -1173,6 +1215,7 @@ __device__ __forceinline__ void compute_role(const FusedDecodeArgs &a, Lds<GE> &
         // ── down rows (reference src/hf/emitter.rs:801-804; the residual is added by the readers) ──
         wg_barrier();
         load_wg(nx, 0, WG_CUT);
+        if (LATE) load_kv(nx, KV_CUT, NR);
         {
             using S = decltype(s.wd);
             float v[S::Q];
