@@ -362,8 +362,8 @@ int hm_model_set_graph(hm_model *m, int on);
 
 /* One launch for a whole decode step's embedding row and decoder layers (on != 0) instead of one
  * launch per projection; the reference dispatches 1 + 3 * layers + 1 kernels per step
- * (src/hf/emitter.rs:1016-1021). Served for bf16, all-Q8_0 and all-Q4_0 models whose shape has a kernel
- * instance (hm_model_whole_step_available); on by default then, and for bf16 models the same launch runs the
+ * (src/hf/emitter.rs:1016-1021). Served for bf16, all-Q8_0, all-Q4_0 and Q4_K / Q6_K (in any mix per
+ * projection) models whose shape has a kernel instance (hm_model_whole_step_available); on by default then, and for bf16 models the same launch runs the
  * LM head and the greedy pick. The cache may be of any length: a step takes the instance of the kernel that
  * holds its live rows (1536, 2048 or 4096 of them; the smaller the faster), beyond 4096 the per-projection path,
  * chosen step by step. Results agree with the per-projection
