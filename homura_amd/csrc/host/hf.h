@@ -208,6 +208,11 @@ class HfModel {
         Buffer ids, h, resid, split, qkv, proj_out, gate_up, logits;
         Buffer wsplit;  // block formats: the matrices of one group of projections as three bf16 pieces per weight
         std::vector<Buffer> wcache;  // [layer * 4 + group] resident copies of the same (q|k|v, o, gate|up, down)
+        // K-quant groups on the integer matrix cores: the chunk's Q8_K rows (int8 values, one f32 scale per
+        // 256) and, per [layer * 4 + group], the group's int8 digit planes followed by its block scales
+        Buffer q8, q8s;
+        std::vector<Buffer> icache;
+        bool icache_off = false;  // the planes did not fit: K-quant groups keep the bf16 pieces
         // Tests: the f32 rows entering the Q8_K quantisation of the K-quant products, for cache positions
         // [capture_base, capture_base + capture_rows); per layer [rows][hidden] (q|k|v), [rows][q_dim] (o),
         // [rows][hidden] (gate|up), [rows][inter] (down).

@@ -7,6 +7,7 @@
 #include "../attention.h"
 #include "../decode_fused.h"
 #include "../kquant_planes8.h"
+#include "../gemm_kquant_i8.h"
 #include "../gemv_bf16.h"
 #include "../gemm_bf16_mfma.h"
 #include "../gemv_kquant.h"
@@ -1847,6 +1848,8 @@ int HfModel::prefill_chunk(const int32_t *h_ids, int n, float *h_logits) {
             grown.capture = std::move(p.capture);
             grown.capture_rows = p.capture_rows;
             grown.capture_base = p.capture_base;
+            grown.icache = std::move(p.icache);  // weights, not rows: they do not depend on the chunk size
+            grown.icache_off = p.icache_off;
             p = std::move(grown);
         }
         p.ids = Buffer::alloc(ctx_, {rows}, DType::F32);  // int32 ids
@@ -1857,6 +1860,11 @@ int HfModel::prefill_chunk(const int32_t *h_ids, int n, float *h_logits) {
         p.proj_out = Buffer::alloc(ctx_, {PrefillScratch::MAX_PARTS, rows, hidden}, DType::F32);
         p.gate_up = Buffer::alloc(ctx_, {PrefillScratch::MAX_PARTS, rows, 2 * (int64_t)inter}, DType::F32);
         if (!p.ids || !p.h || !p.resid || !p.split || !p.qkv || !p.proj_out || !p.gate_up) return HM_ERR_OOM;
+        if (quant && widest % 256 == 0) {  // Q8_K rows for K-quant groups (a float holds four of the int8 values)
+            p.q8 = Buffer::alloc(ctx_, {rows, widest / 4}, DType::F32);
+            p.q8s = Buffer::alloc(ctx_, {rows, widest / 256}, DType::F32);
+            if (!p.q8 || !p.q8s) return HM_ERR_OOM;
+        }
         if (quant) {  // the largest group of matrices of a layer as three bf16 pieces per weight
             const int64_t most = std::max(std::max((int64_t)nqkv * hidden, (int64_t)hidden * qd), 2 * (int64_t)inter * hidden);
             p.wsplit = Buffer::alloc(ctx_, {3 * most}, DType::BF16);
@@ -1902,10 +1910,68 @@ int HfModel::prefill_chunk(const int32_t *h_ids, int n, float *h_logits) {
         const size_t need = per_layer * c.num_hidden_layers;
         if (need <= prefill_weight_cache_bytes_ && need + total_b / 8 <= free_b) p.wcache.resize((size_t)c.num_hidden_layers * 4);
     }
+    // K-quant groups multiply on the integer matrix cores (gemm_kquant_i8.h) when their digit planes
+    // (3 bytes a weight) fit the same budget: packed on first use, resident afterwards.
+    if (quant && p.icache.empty() && !p.icache_off && p.q8 && prefill_weight_cache_bytes_ > 0) {
+        size_t need = 0;
+        const int gK[4] = {hidden, qd, hidden, inter}, gN[4] = {nqkv, hidden, 2 * inter, hidden}, gfirst[4] = {0, 3, 4, 6};
+        for (int l = 0; l < c.num_hidden_layers; l++)
+            for (int gq = 0; gq < 4; gq++)
+                if (q8k(l, gfirst[gq]) && gK[gq] % 256 == 0 && gK[gq] / 256 <= 16 * MP)
+                    need += kq_i8_plane_bytes(gN[gq], gK[gq]) + kq_i8_scale_bytes(gN[gq], gK[gq]) + 256;
+        size_t free_b = 0, total_b = 0;
+        if (hipMemGetInfo(&free_b, &total_b) != hipSuccess) free_b = total_b = 0;
+        if (need > 0 && need <= prefill_weight_cache_bytes_ && need + total_b / 8 <= free_b)
+            p.icache.resize((size_t)c.num_hidden_layers * 4);
+        else
+            p.icache_off = true;
+    }
+    // the planes of group g (0 q|k|v, 1 o, 2 gate|up, 3 down) of layer l, packed now if this is their first use;
+    // nullptr: the group goes through the bf16 pieces
+    auto i8_planes = [&](int l, int g, int first, int count, int K) -> const Buffer * {
+        if (p.icache.empty() || !q8k(l, first) || K % 256 != 0 || K / 256 > 16 * MP) return nullptr;
+        Buffer &slot = p.icache[(size_t)l * 4 + g];
+        if (slot) return &slot;
+        int N = 0;
+        for (int j = first; j < first + count; j++) N += proj_n[j];
+        const size_t pb = (kq_i8_plane_bytes(N, K) + 255) / 256 * 256, sb = kq_i8_scale_bytes(N, K);
+        slot = Buffer::alloc(ctx_, {(int64_t)((pb + sb + 3) / 4)}, DType::F32);
+        if (!slot) {
+            (void)hipGetLastError();
+            return nullptr;
+        }
+        const bool interleave = first == 4 && count == 2;
+        int8_t *planes = slot.as<int8_t>();
+        float *scales = reinterpret_cast<float *>(slot.as<char>() + pb);
+        int row = 0;
+        for (int j = first; j < first + count; j++) {
+            auto it = slot_by_name_.find("model.layers." + std::to_string(l) + "." + proj_name[j]);
+            int rc2 = it == slot_by_name_.end() ? HM_ERR_STATE : HM_OK;
+            if (rc2 == HM_OK)
+                rc2 = kq_i8_pack(ctx_, (int)proj_dtype(l, j), weight_bufs_[it->second].as<uint8_t>(), proj_n[j], K,
+                                 interleave ? planes : planes + (size_t)row * K,
+                                 interleave ? scales : scales + (size_t)row * (K / 256) * 2, N, interleave ? 2 : 1,
+                                 interleave ? j - first : 0);
+            if (rc2 != HM_OK) {
+                slot = Buffer();
+                return nullptr;
+            }
+            row += proj_n[j];
+        }
+        return &slot;
+    };
+    const Buffer *i8 = nullptr;  // the planes of the group about to be multiplied, if it takes that path
+    int8_t *q8 = p.q8 ? p.q8.as<int8_t>() : nullptr;
+    float *q8s = p.q8s ? p.q8s.as<float>() : nullptr;
     auto project = [&](int l, int first, int count, const Buffer &packed, int K, float *out) -> int {
         int N = 0;
         for (int j = first; j < first + count; j++) N += proj_n[j];
         if (!quant) return gemm_split_nk(ctx_, split, np, packed.as<uint16_t>(), out, n, K, N, MP, &parts);
+        if (i8) {
+            const size_t pb = (kq_i8_plane_bytes(N, K) + 255) / 256 * 256;
+            return gemm_q8k_kquant_nk(ctx_, q8, q8s, i8->as<int8_t>(), reinterpret_cast<const float *>(i8->as<char>() + pb), out, n,
+                                      K, N, MP, &parts);
+        }
         const bool interleave = first == 4 && count == 2;
         uint16_t *wsplit = p.wsplit.as<uint16_t>();
         if (!p.wcache.empty()) {
@@ -1950,8 +2016,10 @@ int HfModel::prefill_chunk(const int32_t *h_ids, int n, float *h_logits) {
         const std::string pre = "model.layers." + std::to_string(l) + ".";
         const LayerPacked &lp = packed_[l];
         // QKV kernel (reference src/hf/emitter.rs:549-673)
+        i8 = i8_planes(l, 0, 0, 3, hidden);
         rc = rmsnorm_split_launch(ctx_, x, res, res_parts, weight_f32(pre + "input_layernorm.weight"), split, np,
-                                  res ? h : nullptr, n, hidden, eps, q8k(l, 0), q8k(l, 0) ? capture_at(l, 0) : nullptr);
+                                  res ? h : nullptr, n, hidden, eps, q8k(l, 0), q8k(l, 0) ? capture_at(l, 0) : nullptr,
+                                  i8 ? q8 : nullptr, i8 ? q8s : nullptr);
         if (rc == HM_OK) rc = project(l, 0, 3, lp.qkv, hidden, qkv);
         if (rc != HM_OK) return rc;
         QkvPostArgs qa;
@@ -1997,16 +2065,23 @@ int HfModel::prefill_chunk(const int32_t *h_ids, int n, float *h_logits) {
         aa.scale = (float)(1.0 / std::sqrt((double)hd));
         aa.pieces = np;
         if ((rc = prefill_attn_launch(ctx_, aa)) != HM_OK) return rc;
-        if (o_q8k && (rc = split_rows_launch(ctx_, gate_up, split, np, (size_t)n, qd, true)) != HM_OK) return rc;
+        i8 = i8_planes(l, 1, 3, 1, qd);
+        if (o_q8k && i8 && (rc = quantize_q8k_rows_launch(ctx_, gate_up, q8, q8s, (size_t)n, qd)) != HM_OK) return rc;
+        if (o_q8k && !i8 && (rc = split_rows_launch(ctx_, gate_up, split, np, (size_t)n, qd, true)) != HM_OK) return rc;
         if (o_q8k && capture_at(l, 1))
             HM_HIP(ctx_, hipMemcpyAsync(capture_at(l, 1), gate_up, (size_t)n * qd * 4, hipMemcpyDeviceToDevice, ctx_->stream));
         if ((rc = project(l, 3, 1, lp.o, qd, proj_out)) != HM_OK) return rc;
         // MLP kernel (reference src/hf/emitter.rs:767-822); h holds the layer's input by now
+        i8 = i8_planes(l, 2, 4, 2, hidden);
         rc = rmsnorm_split_launch(ctx_, h, proj_out, parts, weight_f32(pre + "post_attention_layernorm.weight"), split, np,
-                                  resid, n, hidden, eps, q8k(l, 4), q8k(l, 4) ? capture_at(l, 2) : nullptr);
+                                  resid, n, hidden, eps, q8k(l, 4), q8k(l, 4) ? capture_at(l, 2) : nullptr,
+                                  i8 ? q8 : nullptr, i8 ? q8s : nullptr);
         if (rc == HM_OK) rc = project(l, 4, 2, lp.gate_up, hidden, gate_up);
-        if (rc == HM_OK) rc = silu_mul_split_launch(ctx_, gate_up, parts, split, np, n, inter, q8k(l, 6), q8k(l, 6) ? capture_at(l, 3) : nullptr);
+        i8 = i8_planes(l, 3, 6, 1, inter);
+        if (rc == HM_OK) rc = silu_mul_split_launch(ctx_, gate_up, parts, split, np, n, inter, q8k(l, 6), q8k(l, 6) ? capture_at(l, 3) : nullptr,
+                                                    i8 ? q8 : nullptr, i8 ? q8s : nullptr);
         if (rc == HM_OK) rc = project(l, 6, 1, lp.down, inter, proj_out);
+        i8 = nullptr;
         if (rc != HM_OK) return rc;
         x = resid;
         res = proj_out;

@@ -25,9 +25,11 @@ namespace homura {
 // q8k: the values go through the Q8_K quantisation of a K-quant product's activation first (per
 // 256-wide block of the row, dim % 256 == 0), so the split matrix holds scale * q.
 // d_pre_q8k (optional, [rows][dim] f32; tests): receives the values as they enter that quantisation.
+// d_q8 / d_q8_scale (optional, with q8k): the Q8_K rows themselves, [rows][dim] int8 and [rows][dim / 256] f32,
+// for the integer matrix cores (gemm_kquant_i8.h); no split matrix is written then.
 int rmsnorm_split_launch(hm_ctx *ctx, const float *d_x, const float *d_res, int res_parts, const float *d_w,
                          uint16_t *d_out_split, int pieces, float *d_resid_out, int rows, int dim, float eps,
-                         bool q8k = false, float *d_pre_q8k = nullptr);
+                         bool q8k = false, float *d_pre_q8k = nullptr, int8_t *d_q8 = nullptr, float *d_q8_scale = nullptr);
 
 // out_split = split(x) (through Q8_K first with q8k); x: [rows][dim] f32, dim % 4 == 0
 int split_rows_launch(hm_ctx *ctx, const float *d_x, uint16_t *d_out_split, int pieces, size_t rows, int dim,
@@ -43,7 +45,8 @@ int dequant_split_launch(hm_ctx *ctx, int hm_dtype, const uint8_t *d_blocks, int
 // out_split = split(silu(gate) * up) for gate/up interleaved per row: gu [rows][2 * inter] =
 // (gate_0, up_0, gate_1, up_1, ...), the column order of the packed gate|up weight.
 int silu_mul_split_launch(hm_ctx *ctx, const float *d_gu, int parts, uint16_t *d_out_split, int pieces, int rows,
-                          int inter, bool q8k = false, float *d_pre_q8k = nullptr);
+                          int inter, bool q8k = false, float *d_pre_q8k = nullptr, int8_t *d_q8 = nullptr,
+                          float *d_q8_scale = nullptr);
 
 // The tail of the reference's QKV kernel for S rows at positions past .. past + S - 1
 // (src/hf/emitter.rs:604-649): bias add, per-head QK-norm, RoPE on q and k in place, and the

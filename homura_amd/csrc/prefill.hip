@@ -20,6 +20,7 @@
 #include <cstdlib>
 
 #include "gemm_bf16_mfma.h"
+#include "gemm_kquant_i8.h"
 #include "quant_formats.h"
 
 namespace {
@@ -129,7 +130,8 @@ __global__ __launch_bounds__(256) void rmsnorm_split_kernel(const float *__restr
                                                             int res_parts, size_t res_stride,
                                                             const float *__restrict__ w, uint16_t *__restrict__ out,
                                                             float *__restrict__ resid_out, int dim, float eps,
-                                                            int pieces, int q8k, float *__restrict__ pre_q8k) {
+                                                            int pieces, int q8k, float *__restrict__ pre_q8k,
+                                                            int8_t *__restrict__ q8, float *__restrict__ q8_scale) {
     __shared__ float red[4];
     const size_t base = (size_t)blockIdx.x * dim;
     constexpr int KEEP = 2;  // rows up to 2048 wide stay in registers between the two passes
@@ -163,7 +165,13 @@ __global__ __launch_bounds__(256) void rmsnorm_split_kernel(const float *__restr
 #pragma unroll
         for (int k = 0; k < 4; k++) y[k] = (v[k] * inv) * wv[k];
         if (pre_q8k) *reinterpret_cast<f32x4 *>(pre_q8k + base + i) = y;
-        if (q8k) y = q8k_round_trip(y);  // dim % 256 == 0: a wavefront's 256 values are one block
+        if (q8) {  // the Q8_K row itself, for the integer matrix cores (dim % 256 == 0: a wavefront's 256 values are one block)
+            float d;
+            *reinterpret_cast<uint32_t *>(q8 + base + i) = q8k_quantize4(y, d);
+            if ((threadIdx.x & 63) == 0) q8_scale[(base + i) / 256] = d;
+            continue;
+        }
+        if (q8k) y = q8k_round_trip(y);
         split_store4(o, dim, i, y, pieces);
     }
 }
@@ -171,7 +179,8 @@ __global__ __launch_bounds__(256) void rmsnorm_split_kernel(const float *__restr
 // silu(gate) * up (reference src/graph_builder/emit_arithmetic.rs:101-107, src/hf/emitter.rs:797-799);
 // four outputs per thread (inter % 4 == 0)
 __global__ void silu_mul_split_kernel(const float *__restrict__ gu, int parts, size_t stride, uint16_t *__restrict__ out,
-                                      int inter, size_t n, int pieces, int q8k, float *__restrict__ pre_q8k) {
+                                      int inter, size_t n, int pieces, int q8k, float *__restrict__ pre_q8k,
+                                      int8_t *__restrict__ q8, float *__restrict__ q8_scale) {
     const size_t i = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;
     if (i >= n) return;
     const size_t row = i / inter;
@@ -181,6 +190,12 @@ __global__ void silu_mul_split_kernel(const float *__restrict__ gu, int parts, s
 #pragma unroll
     for (int k = 0; k < 4; k++) y[k] = (g[k] / (1.0f + expf(-g[k]))) * u[k];
     if (pre_q8k) *reinterpret_cast<f32x4 *>(pre_q8k + i) = y;
+    if (q8) {
+        float d;
+        *reinterpret_cast<uint32_t *>(q8 + i) = q8k_quantize4(y, d);
+        if ((threadIdx.x & 63) == 0) q8_scale[i / 256] = d;
+        return;
+    }
     if (q8k) y = q8k_round_trip(y);
     split_store4(out + row * pieces * inter, inter, (int)(i % inter), y, pieces);
 }
@@ -529,29 +544,32 @@ namespace homura {
 
 int rmsnorm_split_launch(hm_ctx *ctx, const float *d_x, const float *d_res, int res_parts, const float *d_w,
                          uint16_t *d_out_split, int pieces, float *d_resid_out, int rows, int dim, float eps, bool q8k,
-                         float *d_pre_q8k) {
+                         float *d_pre_q8k, int8_t *d_q8, float *d_q8_scale) {
     HM_REQUIRE(ctx, !q8k || dim % 256 == 0, "rmsnorm_split: Q8_K activations need dim %% 256 == 0 (dim=%d)", dim);
-    HM_REQUIRE(ctx, d_x && d_w && d_out_split, "rmsnorm_split: NULL pointer");
+    HM_REQUIRE(ctx, d_x && d_w && (d_out_split || d_q8), "rmsnorm_split: NULL pointer");
+    HM_REQUIRE(ctx, !d_q8 || (q8k && d_q8_scale && ((uintptr_t)d_q8 % 4) == 0), "rmsnorm_split: Q8_K rows need q8k, a scale buffer and 4-byte alignment");
     HM_REQUIRE(ctx, rows > 0 && dim > 0 && dim % 4 == 0 && pieces >= 1 && pieces <= 3 && res_parts >= 1,
                "rmsnorm_split: bad shape (dim %% 4 == 0 needed)");
     HM_REQUIRE(ctx, ((uintptr_t)d_x % 16) == 0 && ((uintptr_t)d_w % 16) == 0 && ((uintptr_t)d_out_split % 8) == 0 &&
                         ((uintptr_t)d_res % 16) == 0 && ((uintptr_t)d_resid_out % 16) == 0, "rmsnorm_split: misaligned buffer");
     hipLaunchKernelGGL(rmsnorm_split_kernel, dim3(rows), dim3(256), 0, ctx->stream, d_x, d_res, res_parts,
-                       (size_t)rows * dim, d_w, d_out_split, d_resid_out, dim, eps, pieces, q8k ? 1 : 0, d_pre_q8k);
+                       (size_t)rows * dim, d_w, d_out_split, d_resid_out, dim, eps, pieces, q8k ? 1 : 0, d_pre_q8k, d_q8,
+                       d_q8_scale);
     HM_LAUNCH_CHECK(ctx);
     return HM_OK;
 }
 
 int silu_mul_split_launch(hm_ctx *ctx, const float *d_gu, int parts, uint16_t *d_out_split, int pieces, int rows,
-                          int inter, bool q8k, float *d_pre_q8k) {
+                          int inter, bool q8k, float *d_pre_q8k, int8_t *d_q8, float *d_q8_scale) {
     HM_REQUIRE(ctx, !q8k || inter % 256 == 0, "silu_mul_split: Q8_K activations need a width %% 256 == 0 (%d)", inter);
-    HM_REQUIRE(ctx, d_gu && d_out_split, "silu_mul_split: NULL pointer");
+    HM_REQUIRE(ctx, d_gu && (d_out_split || d_q8), "silu_mul_split: NULL pointer");
+    HM_REQUIRE(ctx, !d_q8 || (q8k && d_q8_scale && ((uintptr_t)d_q8 % 4) == 0), "silu_mul_split: Q8_K rows need q8k, a scale buffer and 4-byte alignment");
     HM_REQUIRE(ctx, rows > 0 && inter > 0 && inter % 4 == 0 && pieces >= 1 && pieces <= 3 && parts >= 1,
                "silu_mul_split: bad shape (intermediate size %% 4 == 0 needed)");
     HM_REQUIRE(ctx, ((uintptr_t)d_gu % 16) == 0 && ((uintptr_t)d_out_split % 8) == 0, "silu_mul_split: misaligned buffer");
     const size_t n = (size_t)rows * inter;
     hipLaunchKernelGGL(silu_mul_split_kernel, dim3((unsigned)((n / 4 + 255) / 256)), dim3(256), 0, ctx->stream, d_gu, parts,
-                       2 * n, d_out_split, inter, n, pieces, q8k ? 1 : 0, d_pre_q8k);
+                       2 * n, d_out_split, inter, n, pieces, q8k ? 1 : 0, d_pre_q8k, d_q8, d_q8_scale);
     HM_LAUNCH_CHECK(ctx);
     return HM_OK;
 }
@@ -685,6 +703,28 @@ extern "C" int hm_gemm_f32_quant_nk(hm_ctx *ctx, const float *d_x_mk, const uint
     HM_REQUIRE(ctx, kq || dtype == HM_DTYPE_Q8_0 || dtype == HM_DTYPE_Q4_0, "hm_gemm_f32_quant_nk: dtype %d is not a block format", dtype);
     HM_REQUIRE(ctx, M > 0 && N > 0 && K > 0 && K % (kq ? 256 : 64) == 0,
                "hm_gemm_f32_quant_nk: need M, N > 0 and K %% %d == 0 (K=%d)", kq ? 256 : 64, K);
+    if (kq && K / 256 <= 16) {  // (wider rows would need K slices: they keep the bf16 pieces below)
+        // K-quants: Q8_K rows x the matrix's int8 digit planes on the integer matrix cores. Workspace: the
+        // quantised rows and their scales, then the planes and block scales of as many weight rows as fit.
+        const size_t q_bytes = ((size_t)M * K + 255) / 256 * 256, s_bytes = ((size_t)M * (K / 256) * 4 + 255) / 256 * 256;
+        const size_t per_row = (size_t)3 * K + (size_t)(K / 256) * 8;
+        HM_REQUIRE(ctx, q_bytes + s_bytes + 128 * per_row + 256 <= ctx->workspace_bytes,
+                   "hm_gemm_f32_quant_nk: M * K = %zu activations exceed the workspace", (size_t)M * K);
+        int8_t *aq = (int8_t *)ctx->workspace;
+        float *asc = (float *)((char *)ctx->workspace + q_bytes);
+        char *wbase = (char *)ctx->workspace + q_bytes + s_bytes;
+        const int slab = (int)std::min<size_t>((size_t)N, (ctx->workspace_bytes - q_bytes - s_bytes - 256) / per_row / 128 * 128);
+        int rc = homura::quantize_q8k_rows_launch(ctx, d_x_mk, aq, asc, (size_t)M, K);
+        const size_t row_bytes = (size_t)K / 256 * (dtype == HM_DTYPE_Q4_K ? 144 : 210);
+        for (int n0 = 0; n0 < N && rc == HM_OK; n0 += slab) {
+            const int rows = std::min(slab, N - n0);
+            int8_t *planes = (int8_t *)wbase;
+            float *wsc = (float *)(wbase + ((size_t)3 * rows * K + 255) / 256 * 256);
+            rc = homura::kq_i8_pack(ctx, dtype, d_w_blocks + (size_t)n0 * row_bytes, rows, K, planes, wsc, rows, 1, 0);
+            if (rc == HM_OK) rc = homura::gemm_q8k_kquant_nk(ctx, aq, asc, planes, wsc, d_out + n0, M, K, rows, 1, nullptr, N);
+        }
+        return rc;
+    }
     // workspace: the split activations, then as many split weight rows as fit (a multiple of the tile)
     const size_t a_bytes = ((size_t)M * K * 6 + 255) / 256 * 256;
     HM_REQUIRE(ctx, a_bytes + (size_t)128 * K * 6 <= ctx->workspace_bytes,

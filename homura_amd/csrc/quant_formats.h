@@ -69,4 +69,27 @@ __device__ __forceinline__ float dequant_element(const uint8_t *__restrict__ blk
     }
 }
 
+// Four consecutive values of a 256-wide block held by one wavefront (four per lane) through the Q8_K
+// quantiser (reference quantize_row_q8_k, src/graph_builder/emit_quant.rs:422-466): q = clamp(roundeven(x *
+// (127 / amax)), +-127), scale d = amax / 127. Returns the four int8 values packed low to high.
+__device__ __forceinline__ uint32_t q8k_quantize4(f32x4 v, float &d, float r_out[4]) {
+    float amax = fmaxf(fmaxf(fabsf(v[0]), fabsf(v[1])), fmaxf(fabsf(v[2]), fabsf(v[3])));
+    amax = wave_max(amax);
+    const float iscale = amax == 0.f ? 0.f : __fdiv_rn(127.0f, amax);
+    d = __fdiv_rn(amax, 127.0f);
+    uint32_t packed = 0;
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        float r = rintf(__fmul_rn(v[k], iscale));
+        r = fmaxf(fminf(r, 127.0f), -127.0f);
+        r_out[k] = r;
+        packed |= ((uint32_t)(int)r & 0xFFu) << (8 * k);
+    }
+    return packed;
+}
+__device__ __forceinline__ uint32_t q8k_quantize4(f32x4 v, float &d) {
+    float r[4];
+    return q8k_quantize4(v, d, r);
+}
+
 }  // namespace homura
