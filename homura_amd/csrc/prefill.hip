@@ -76,17 +76,11 @@ __device__ __forceinline__ void split_store4(uint16_t *__restrict__ row, int dim
 // dot products of the decode kernels equal a plain dot product with scale * q. A wavefront holds one
 // block, four consecutive values per lane.
 __device__ __forceinline__ f32x4 q8k_round_trip(f32x4 v) {
-    float amax = fmaxf(fmaxf(fabsf(v[0]), fabsf(v[1])), fmaxf(fabsf(v[2]), fabsf(v[3])));
-    amax = wave_max(amax);
-    const float iscale = amax == 0.f ? 0.f : __fdiv_rn(127.0f, amax);
-    const float d = __fdiv_rn(amax, 127.0f);
+    float d, r[4];
+    (void)q8k_quantize4(v, d, r);
     f32x4 y;
 #pragma unroll
-    for (int k = 0; k < 4; k++) {
-        float r = rintf(__fmul_rn(v[k], iscale));
-        r = fmaxf(fminf(r, 127.0f), -127.0f);
-        y[k] = __fmul_rn(d, r);
-    }
+    for (int k = 0; k < 4; k++) y[k] = __fmul_rn(d, r[k]);
     return y;
 }
 

@@ -419,12 +419,14 @@ def test_gemv_kquant_f32_activation(ctx, oracle, kind, M, K, N):
 
 
 @pytest.mark.parametrize("kind", ["q8_0", "q4_0", "q4_k", "q6_k"])
-@pytest.mark.parametrize("M,K,N", [(200, 1024, 1000), (5, 256, 130), (64, 2048, 6000), (512, 512, 256)])
+@pytest.mark.parametrize("M,K,N", [(200, 1024, 1000), (5, 256, 130), (64, 2048, 6000), (512, 512, 256), (3, 4352, 200)])
 def test_gemm_f32_quantised_weights(ctx, oracle, kind, M, K, N):
     """The quantised matmul at seq > 1 on the matrix cores against the oracle's row-by-row product (the
     decode formula: f32 activations for Q8_0 / Q4_0, Q8_K activations and integer sums for the
     K-quants). Both sides add the same products in f32, in different orders. N = 6000 at K = 2048 does
-    not fit the workspace in one piece and goes through in slabs."""
+    not fit the workspace in one piece and goes through in slabs. K-quants up to 4096 wide multiply on the
+    integer matrix cores with the decode kernels' block arithmetic (the oracle's, up to how the host compiler
+    contracts it); K = 4352 takes the bf16 pieces."""
     say(f"gemm_f32_quant_nk {kind} M={M} K={K} N={N}")
     import homura_amd
     make = {"q8_0": synth.q8_0_blocks, "q4_0": synth.q4_0_blocks, "q4_k": synth.q4_k_blocks, "q6_k": synth.q6_k_blocks}[kind]
@@ -452,7 +454,7 @@ def test_gemm_f32_quantised_weights(ctx, oracle, kind, M, K, N):
     e_gpu, e_orc = np.abs(got - truth).max() / unit, np.abs(want - truth).max() / unit
     say(f"  error / typical output: gpu {e_gpu:.2e}, oracle {e_orc:.2e}; rel_err vs oracle {rel_err(got, want):.2e}")
     assert e_gpu < 1.2e-5
-    assert rel_err(got, want) < 2e-3
+    assert rel_err(got, want) < (1e-4 if per == 256 and K <= 4096 else 2e-3)
     for b in (dx, dw, dout):
         b.free()
 
