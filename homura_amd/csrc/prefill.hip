@@ -4,13 +4,12 @@
 //
 // Attention works on the transposed problem so that softmax statistics stay inside a lane:
 //   S^T[key][q] = K[key][:] . Q[q][:]      (A operand = K rows from LDS, B operand = Q in registers)
-//   O^T[d][q]   = V^T[d][:] . P^T[:][q]    (A operand = V^T rows from LDS, B operand = P in registers)
-// With v_mfma_f32_32x32x16_bf16 a lane owns one query column of the result tile (lane % 32) and
-// 16 of its 32 rows, so the running maximum and the rescaling factor of a query are per-lane
-// scalars; only one exchange with lane ^ 32 per key tile is needed. The probabilities leave the
-// S^T accumulators and enter the second product without touching LDS: MFMA row r of a key block
-// is assigned key (r with bits 2 and 3 swapped), which makes the 8 accumulator values a lane
-// passes per k step 8 consecutive keys, matching one 16-byte chunk of a V^T row.
+//   O^T[d][q]   = V^T[d][:] . P^T[:][q]    (A operand = V^T from LDS, B operand = P in registers)
+// With v_mfma_f32_16x16x32_bf16 a lane owns one query column of the result tile (lane % 16) and four of
+// its 16 rows, so the running maximum and the rescaling factor of a query are per-lane scalars; the four
+// lanes of a query exchange one maximum per key tile. The probabilities leave the S^T accumulators and
+// enter the second product without touching LDS (the contraction slots of the second product are numbered
+// the way the scores arrive; see the kernel).
 // Queries and probabilities are f32 carried as two or three bf16 pieces each (see prefill.h); K and
 // V are the cache's own bf16 rows.
 #include "prefill.h"
@@ -261,22 +260,8 @@ __global__ __launch_bounds__(256) void qkv_post_kernel(QkvPostArgs a) {
 
 // ── causal attention ─────────────────────────────────────────────────────────
 
-constexpr int AT_THREADS = 256;
-constexpr int AT_WAVES = AT_THREADS / 64;
-constexpr int AT_KEYS = 64;  // keys per tile
-// A workgroup's four wavefronts are 4 / KS blocks of 32 query rows times KS key groups: with KS > 1
-// the wavefronts of a row block take every KS-th key tile each (KS tiles are staged per round) and
-// their partial softmax sums meet in LDS at the end. KS = 1: 128 rows per workgroup, the fewest tile
-// loads; KS = 2, 4: 64, 32 rows, for prompts whose rows x heads alone leave most of the chip idle, and
-// a KS times shorter chain of tiles per wavefront.
-
-// V^T tile: row d holds 64 keys = 128 bytes = eight 16-byte chunks, chunk c of row r at slot
-// c ^ (r & 7) ^ ((r >> 3) & 7): conflict-free for the operand reads (32 consecutive rows, one chunk)
-// and spread for the transposing 8-byte writes.
-__device__ __forceinline__ int vt_off(int r, int chunk) {
-    return r * 128 + ((chunk ^ (r & 7) ^ ((r >> 3) & 7)) << 4);
-}
-// K tile: row = key, HD*2 bytes, same idea
+// K / V tile in LDS: row = key, HD * 2 bytes, 16-byte chunk c of row r at slot c ^ (swizzle of r): conflict-free
+// for the operand reads (16 consecutive rows, one chunk)
 template <int HD>
 __device__ __forceinline__ int k_off(int key, int chunk) {
     if (HD == 128) return key * 256 + ((chunk ^ (key & 15)) << 4);
@@ -285,213 +270,236 @@ __device__ __forceinline__ int k_off(int key, int chunk) {
 
 extern __shared__ __attribute__((aligned(16))) char at_lds[];
 
-template <int HD, int NP, int KS>
-__global__ __launch_bounds__(AT_THREADS) void prefill_attn_kernel(PrefillAttnArgs a) {
-    constexpr int CH = HD / 8;                        // 16-byte chunks per K row
-    constexpr int KLOADS = AT_KEYS * CH / AT_THREADS;  // K chunks per thread per tile
-    constexpr int KSTEPS = HD / 16;                   // k steps of K . Q
-    constexpr int DB = HD / 32;                       // 32-row blocks of O^T
-    constexpr int QW = AT_WAVES / KS;                 // 32-row query blocks per workgroup
-    constexpr int AT_QROWS = 32 * QW;
-    constexpr int K_TILE = AT_KEYS * HD * 2, V_TILE = HD * 128;  // bytes; KS of each
+// 16 query rows per wavefront (v_mfma_f32_16x16x32_bf16) and eight wavefronts a workgroup: 8 / KS blocks of 16
+// rows times KS key groups (with KS > 1 the wavefronts of a row block take every KS-th key tile each and their
+// partial softmax sums meet in LDS at the end; KS = 1: 128 rows per workgroup, the fewest tile loads; KS = 2, 4:
+// 64, 32 rows, for prompts whose rows x heads alone leave most of the chip idle). A wavefront needs ~150
+// registers, so two or three share a SIMD and one's matrix instructions run under the others' softmax arithmetic.
+// K and V tiles (32 keys) go global -> LDS directly (global_load_lds_dwordx4, no staging registers, no LDS
+// write instructions), row-major and XOR-swizzled on the global side; two sets of KS tile pairs alternate, the
+// next round's tiles arrive while this round is multiplied.
+//   S^T block: A = 16 keys x 32 dims from the K tile, B = the queries' pieces; lane q + 16 c receives keys
+//   4 c .. 4 c + 3 of the block for query q.
+//   O^T block: A = 16 dims x 32 keys, B = the probabilities' pieces. Contraction slot 8 c + i (i < 4) stands
+//   for key 4 c + i of the tile, slot 8 c + 4 + i for key 16 + 4 c + i: exactly the eight scores lane q + 16 c
+//   holds from the tile's two key blocks, so the probabilities never leave their lanes. V^T comes out of the
+//   row-major V tile through the transposing LDS read (ds_read_b64_tr_b16: lane l of a group of 16 receives
+//   element l % 4 of the 8 bytes that lanes l / 4, 4 + l / 4, 8 + l / 4, 12 + l / 4 point at): lane i points at
+//   dims 16 db + 4 (i % 4) .. + 3 of key 4 c + i / 4, and receives dim 16 db + i of keys 4 c .. 4 c + 3.
+constexpr int A8_THREADS = 512;
+constexpr int A8_WAVES = A8_THREADS / 64;
+constexpr int A8_KEYS = 32;  // keys per tile
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, lh = lane >> 5;
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ void dma16_lds(const uint16_t *src, char *dst) {
+    __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1))) *)src,
+                                     (void __attribute__((address_space(3))) *)dst, 16, 0, 0);
+}
+
+// max / sum over the four lanes l16 + 16 c of a wavefront, every lane receives it: the row swaps of gfx950
+// (odd rows of one operand against even rows of the other, then the upper half against the lower) instead of
+// two trips through the LDS crossbar
+__device__ __forceinline__ float quad_rows_max(float x) {
+    const auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    const float m = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+    const auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(m), __float_as_uint(m), false, false);
+    return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+}
+__device__ __forceinline__ float quad_rows_sum(float x) {
+    const auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    const float m = __uint_as_float(a[0]) + __uint_as_float(a[1]);
+    const auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(m), __float_as_uint(m), false, false);
+    return __uint_as_float(b[0]) + __uint_as_float(b[1]);
+}
+
+template <int HD, int NP, int KS>
+__global__ __launch_bounds__(A8_THREADS) void prefill_attn16_kernel(PrefillAttnArgs a) {
+    constexpr int CH = HD / 8;                         // 16-byte chunks per row
+    constexpr int KSTEPS = HD / 32;                    // k steps of K . Q
+    constexpr int DB = HD / 16;                        // 16-row blocks of O^T
+    constexpr int QW = A8_WAVES / KS;                  // 16-row query blocks per workgroup
+    constexpr int AT_QROWS = 16 * QW;
+    constexpr int TILE = A8_KEYS * HD * 2;             // bytes of a K or V tile
+    constexpr int SET = KS * 2 * TILE;                 // the KS tile pairs of a round
+    constexpr int ROWS_PER_DMA = 1024 / (HD * 2);      // rows one wavefront-wide 16-byte-per-lane load fills
+    constexpr int DMA_WAVES = A8_KEYS / ROWS_PER_DMA;  // wavefronts that fill a tile (8 or 4)
+    static_assert(DMA_WAVES <= A8_WAVES, "head_dim 64 or 128");
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l16 = lane & 15, c4 = lane >> 4;
     const int qw = wave % QW, kh = wave / QW;  // row block and key group of this wavefront
-    char *k_lds = at_lds + kh * K_TILE, *v_lds = at_lds + KS * K_TILE + kh * V_TILE;
-    const int h = blockIdx.y, kvhd = h / (a.H / a.kvh);
-    const int q0 = blockIdx.x * AT_QROWS;
+    // Workgroups are dealt to the eight dies round-robin by their linear index. With a multiple of eight heads
+    // every die gets H / 8 neighbouring heads and all their row blocks, so the K and V rows of a KV head are
+    // fetched into one die's L2 (or as few as the head grouping allows) instead of all eight.
+    int hx = blockIdx.y, bx = blockIdx.x;
+    if (a.H % 8 == 0) {
+        const int lin = blockIdx.y * gridDim.x + blockIdx.x, per = a.H / 8;
+        hx = (lin & 7) * per + (lin >> 3) % per;
+        bx = (lin >> 3) / per;
+    }
+    const int h = hx, kvhd = h / (a.H / a.kvh);
+    const int q0 = bx * AT_QROWS;
     const int kv_total = a.past + a.S;
     const uint16_t *kc = a.kcache + (size_t)kvhd * a.max_len * HD;
     const uint16_t *vc = a.vcache + (size_t)kvhd * a.max_len * HD;
 
-    // this lane's query (rows past the end repeat the last one and are not stored)
-    const int qrow = q0 + qw * 32 + l32;
+    const int wg_end = a.past + min(a.S, q0 + AT_QROWS);
+    const int wave_end = q0 + qw * 16 < a.S ? a.past + min(a.S, q0 + qw * 16 + 16) : 0;
+    const int ntiles = (wg_end + A8_KEYS - 1) / A8_KEYS;
+    const int nrounds = (ntiles + KS - 1) / KS;
+    const int wave_first = a.past + min(q0 + qw * 16, a.S - 1);
+
+    // This lane's part of a tile load: row dma_row of the tile, the chunk that belongs in slot dma_slot.
+    const int dma_row = wave * ROWS_PER_DMA + lane / CH, dma_slot = lane % CH;
+    const int dma_chunk = (k_off<HD>(dma_row, dma_slot) - dma_row * HD * 2) >> 4;  // the swizzle is an involution
+    const int wave_dst = __builtin_amdgcn_readfirstlane(wave * 1024);
+    auto request_round = [&](int r) {
+        if (wave >= DMA_WAVES) return;
+        char *base = at_lds + (r & 1) * SET + wave_dst;
+#pragma unroll
+        for (int u = 0; u < KS; u++) {
+            const int row = min((r * KS + u) * A8_KEYS + dma_row, kv_total - 1);
+            dma16_lds(kc + (size_t)row * HD + dma_chunk * 8, base + u * 2 * TILE);
+            dma16_lds(vc + (size_t)row * HD + dma_chunk * 8, base + u * 2 * TILE + TILE);
+        }
+    };
+    // this lane's query (rows past the end repeat the last one and are not stored): dims 32 ks + 8 c4 .. + 7.
+    // Asked for ahead of the first tiles (loads return in order): it is split into pieces while they arrive.
+    const int qrow = q0 + qw * 16 + l16;
     const int qc = min(qrow, a.S - 1);
     const int qabs = a.past + qc;
     bf16x8 qp_[KSTEPS][NP];
     {
-        const float qscale = a.scale * 1.44269504088896340736f;
-        const float *qp = a.q + (size_t)qc * a.ldq + (size_t)h * HD + lh * 8;
+        const float qscale = a.scale * 1.44269504088896340736f;  // scores in units of ln 2: the softmax uses exp2
+        const float *qp = a.q + (size_t)qc * a.ldq + (size_t)h * HD + c4 * 8;
+        f32x4 x0[KSTEPS], x1[KSTEPS];
 #pragma unroll
         for (int ks = 0; ks < KSTEPS; ks++) {
-            const f32x4 x0 = *reinterpret_cast<const f32x4 *>(qp + 16 * ks);
-            const f32x4 x1 = *reinterpret_cast<const f32x4 *>(qp + 16 * ks + 4);
+            x0[ks] = *reinterpret_cast<const f32x4 *>(qp + 32 * ks);
+            x1[ks] = *reinterpret_cast<const f32x4 *>(qp + 32 * ks + 4);
+        }
+        request_round(0);
+#pragma unroll
+        for (int ks = 0; ks < KSTEPS; ks++) {
             float f[8];
 #pragma unroll
-            for (int i = 0; i < 4; i++) {  // scores come out in units of ln 2: the softmax uses exp2
-                f[i] = x0[i] * qscale;
-                f[4 + i] = x1[i] * qscale;
+            for (int i = 0; i < 4; i++) {
+                f[i] = x0[ks][i] * qscale;
+                f[4 + i] = x1[ks][i] * qscale;
             }
             split8<NP>(f, qp_[ks]);
         }
     }
 
-    // keys [0, wg_end) are visible to some row of the workgroup, [0, wave_end) to some row of this wavefront
-    const int wg_end = a.past + min(a.S, q0 + AT_QROWS);
-    const int wave_end = q0 + qw * 32 < a.S ? a.past + min(a.S, q0 + qw * 32 + 32) : 0;
-    const int ntiles = (wg_end + AT_KEYS - 1) / AT_KEYS;
-    const int nrounds = (ntiles + KS - 1) / KS;  // KS tiles are staged per round, tile r KS + u in buffer u
-    const int wave_first = a.past + min(q0 + qw * 32, a.S - 1);  // smallest position among this wavefront's rows
-
-    // thread's share of the KS tiles of a round on their way from the cache to LDS
-    u32x4 kr[KS][KLOADS], vr[KS][4];
-    const int v_ng = tid % CH, v_kg = tid / CH;  // V: a 4(key) x 8(d) block per thread
-    const bool v_on = v_kg < 16;
-    auto request_round = [&](int r) {
+    f32x4 acc_o[DB];
 #pragma unroll
-        for (int u = 0; u < KS; u++) {
-            const int t = r * KS + u;
-#pragma unroll
-            for (int j = 0; j < KLOADS; j++) {
-                const int id = tid + j * AT_THREADS, key = id / CH, c = id % CH;
-                const int row = min(t * AT_KEYS + key, kv_total - 1);
-                kr[u][j] = ld128(kc + (size_t)row * HD + c * 8);
-            }
-#pragma unroll
-            for (int q = 0; q < 4; q++) {
-                const int row = min(t * AT_KEYS + (v_on ? v_kg : 0) * 4 + q, kv_total - 1);
-                vr[u][q] = ld128(vc + (size_t)row * HD + v_ng * 8);
-            }
-        }
-    };
-    auto store_round = [&]() {
-#pragma unroll
-        for (int u = 0; u < KS; u++) {
-            char *kd = at_lds + u * K_TILE, *vd = at_lds + KS * K_TILE + u * V_TILE;
-#pragma unroll
-            for (int j = 0; j < KLOADS; j++) {
-                const int id = tid + j * AT_THREADS, key = id / CH, c = id % CH;
-                *reinterpret_cast<u32x4 *>(kd + k_off<HD>(key, c)) = kr[u][j];
-            }
-            if (v_on) {
-#pragma unroll
-                for (int i = 0; i < 8; i++) {
-                    // column d = v_ng*8 + i of the block: keys +0..+3 packed low to high
-                    const uint32_t sel = (i & 1) ? 0x07060302u : 0x05040100u;
-                    u32x2 col;
-                    col.x = __builtin_amdgcn_perm(vr[u][1][i >> 1], vr[u][0][i >> 1], sel);
-                    col.y = __builtin_amdgcn_perm(vr[u][3][i >> 1], vr[u][2][i >> 1], sel);
-                    *reinterpret_cast<u32x2 *>(vd + vt_off(v_ng * 8 + i, v_kg >> 1) + (v_kg & 1) * 8) = col;
-                }
-            }
-        }
-    };
-
-    f32x16 acc_o[DB];
-#pragma unroll
-    for (int db = 0; db < DB; db++)
-#pragma unroll
-        for (int v = 0; v < 16; v++) acc_o[db][v] = 0.f;
+    for (int db = 0; db < DB; db++) acc_o[db] = f32x4{0.f, 0.f, 0.f, 0.f};
     float m_run = -INFINITY, l_run = 0.f;
-    // MFMA row r of a key block holds key pi(r) = r with bits 2 and 3 swapped
-    const int pi = (l32 & 0x13) | ((l32 & 4) << 1) | ((l32 & 8) >> 1);
+    // transposing V reads: lane i of a group points at dims 4 (i % 4) .. + 3 of a 16-dim block, key 4 c4 + i / 4
+    const int v_key = 4 * c4 + (l16 >> 2), v_sub = l16 & 3;
 
-    request_round(0);
     for (int r = 0; r < nrounds; r++) {
-        __syncthreads();  // the previous tiles have been read by everybody
-        store_round();
+        // this round's tiles have landed for this wavefront (nothing else is in flight), then for everybody,
+        // and everybody is done with the other set
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
         if (r + 1 < nrounds) request_round(r + 1);
         const int t = r * KS + kh;               // this wavefront's tile of the round
-        if (t * AT_KEYS >= wave_end) continue;  // wavefront-uniform: nothing visible to these 32 rows
+        if (t * A8_KEYS >= wave_end) continue;  // wavefront-uniform: nothing visible to these 16 rows
+        const char *k_lds = at_lds + (r & 1) * SET + kh * 2 * TILE, *v_lds = k_lds + TILE;
 
-        f32x16 s[2];
+        f32x4 s[2];  // key blocks of 16
+        s[0] = s[1] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int kb = 0; kb < 2; kb++) {
+        for (int ks = 0; ks < KSTEPS; ks++) {
+            bf16x8 kf[2];
 #pragma unroll
-            for (int v = 0; v < 16; v++) s[kb][v] = 0.f;
-            const int krow = 32 * kb + pi;
+            for (int kb = 0; kb < 2; kb++)
+                kf[kb] = *reinterpret_cast<const bf16x8 *>(k_lds + k_off<HD>(16 * kb + l16, 4 * ks + c4));
 #pragma unroll
-            for (int ks = 0; ks < KSTEPS; ks++) {
-                const bf16x8 kf = *reinterpret_cast<const bf16x8 *>(k_lds + k_off<HD>(krow, 2 * ks + lh));
+            for (int p = NP - 1; p >= 0; p--)
 #pragma unroll
-                for (int p = 0; p < NP; p++)
-                    s[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qp_[ks][p], s[kb], 0, 0, 0);
-            }
+                for (int kb = 0; kb < 2; kb++)
+                    s[kb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[kb], qp_[ks][p], s[kb], 0, 0, 0);
         }
-        // accumulator value v of block kb belongs to key 32 kb + 16 (v / 8) + 8 (lane / 32) + v % 8;
-        // only tiles that reach past the first row of this wavefront need the causal mask
-        if (t * AT_KEYS + AT_KEYS - 1 > wave_first) {
+        // value i of block kb belongs to key 16 kb + 4 c4 + i; only tiles that reach past the first row of
+        // this wavefront need the causal mask
+        if (t * A8_KEYS + A8_KEYS - 1 > wave_first) {
 #pragma unroll
             for (int kb = 0; kb < 2; kb++)
 #pragma unroll
-                for (int v = 0; v < 16; v++) {
-                    const int key = t * AT_KEYS + 32 * kb + 16 * (v >> 3) + 8 * lh + (v & 7);
-                    s[kb][v] = key > qabs ? -INFINITY : s[kb][v];
+                for (int i = 0; i < 4; i++) {
+                    const int key = t * A8_KEYS + 16 * kb + 4 * c4 + i;
+                    s[kb][i] = key > qabs ? -INFINITY : s[kb][i];
                 }
         }
         float mx = -INFINITY;
 #pragma unroll
         for (int kb = 0; kb < 2; kb++)
 #pragma unroll
-            for (int v = 0; v < 16; v++) mx = fmaxf(mx, s[kb][v]);
-        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+            for (int i = 0; i < 4; i++) mx = fmaxf(mx, s[kb][i]);
+        mx = quad_rows_max(mx);
         // The reference point of the exponentials only has to be near the maximum, not on it (softmax is
-        // shift-invariant and l, O are f32): it moves when the maximum has grown by more than 2^8, so
-        // after the first tiles the rescaling of O is skipped for the whole wavefront. Both half-lanes of
-        // a query take the same decision. A row that has not seen a visible key yet (possible in key
-        // groups other than the first, whose tiles may lie wholly in a row's future) gets a finite
-        // floor as its reference point, so that every exponential below is 0 and not exp2(inf - inf).
+        // shift-invariant and l, O are f32): it moves when the maximum has grown by more than 2^8, so after the
+        // first tiles the rescaling of O is skipped for the whole wavefront. The four lanes of a query decide
+        // alike. A row that has not seen a visible key yet (possible in key groups other than the first, whose
+        // tiles may lie wholly in a row's future) gets a finite floor as its reference point, so that every
+        // exponential below is 0 and not exp2(inf - inf).
         const float m_new = fmaxf(mx > m_run + 8.0f ? mx : m_run, -1e30f);
         const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
-        float psum = 0.f;
+        float f[8], psum = 0.f;
 #pragma unroll
         for (int kb = 0; kb < 2; kb++)
 #pragma unroll
-            for (int v = 0; v < 16; v++) {
-                const float p = __builtin_amdgcn_exp2f(s[kb][v] - m_new);
-                s[kb][v] = p;
-                psum += p;
+            for (int i = 0; i < 4; i++) {
+                f[4 * kb + i] = __builtin_amdgcn_exp2f(s[kb][i] - m_new);
+                psum += f[4 * kb + i];
             }
-        l_run = l_run * alpha + psum;  // this lane's half of the keys; the halves meet at the end
+        l_run = l_run * alpha + psum;  // this lane's quarter of the keys; the quarters meet at the end
         m_run = m_new;
         if (__any(alpha != 1.0f)) {
 #pragma unroll
-            for (int db = 0; db < DB; db++)
-#pragma unroll
-                for (int v = 0; v < 16; v++) acc_o[db][v] *= alpha;
+            for (int db = 0; db < DB; db++) acc_o[db] *= alpha;
         }
-
-        // 16 keys at a time: their probabilities become NP operands, multiplied into every block of O^T
+        bf16x8 pp[NP];
+        split8<NP>(f, pp);
 #pragma unroll
-        for (int sp = 0; sp < 4; sp++) {
-            float f[8];
+        for (int db = 0; db < DB; db++) {
+            const int chunk = 2 * db + (v_sub >> 1), within = (v_sub & 1) * 8;
+            const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                (s16x4 __attribute__((address_space(3))) *)(v_lds + k_off<HD>(v_key, chunk) + within));
+            const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                (s16x4 __attribute__((address_space(3))) *)(v_lds + k_off<HD>(16 + v_key, chunk) + within));
+            struct Pair { s16x4 lo, hi; } pr{lo, hi};
+            const bf16x8 vf = __builtin_bit_cast(bf16x8, pr);
 #pragma unroll
-            for (int i = 0; i < 8; i++) f[i] = s[sp >> 1][8 * (sp & 1) + i];
-            bf16x8 pp[NP];
-            split8<NP>(f, pp);
-#pragma unroll
-            for (int db = 0; db < DB; db++) {
-                const bf16x8 vf = *reinterpret_cast<const bf16x8 *>(v_lds + vt_off(32 * db + l32, 2 * sp + lh));
-#pragma unroll
-                for (int p = 0; p < NP; p++)
-                    acc_o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pp[p], acc_o[db], 0, 0, 0);
-            }
+            for (int p = NP - 1; p >= 0; p--)
+                acc_o[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pp[p], acc_o[db], 0, 0, 0);
         }
     }
 
     if (KS > 1) {
-        // The key groups of a row block meet: groups 1 .. KS-1 leave (O, m, l) in LDS, lane-major, and
-        // group 0 adds them in group order, rescaled to the larger reference point (a group that saw no
-        // visible key has m = -inf and weighs nothing; group 0 always sees key 0).
-        constexpr int PER_LANE = DB * 16 + 2;
+        // The key groups of a row block meet: groups 1 .. KS-1 leave (O, m, l) in LDS, lane-major, and group 0
+        // adds them in group order, rescaled to the larger reference point (a group that saw no visible key has
+        // m = -inf and weighs nothing; group 0 always sees key 0).
+        constexpr int PER_LANE = DB * 4 + 2;
         float *xch = reinterpret_cast<float *>(at_lds);
-        __syncthreads();  // nobody reads tiles any more
+        __syncthreads();  // nobody reads tiles any more (and no tile load is in flight: the last round requested none)
         if (kh > 0) {
             float *mine = xch + (size_t)((kh - 1) * QW + qw) * PER_LANE * 64 + lane;
 #pragma unroll
             for (int db = 0; db < DB; db++)
 #pragma unroll
-                for (int v = 0; v < 16; v++) mine[(db * 16 + v) * 64] = acc_o[db][v];
-            mine[(DB * 16) * 64] = m_run;
-            mine[(DB * 16 + 1) * 64] = l_run;
+                for (int v = 0; v < 4; v++) mine[(db * 4 + v) * 64] = acc_o[db][v];
+            mine[(DB * 4) * 64] = m_run;
+            mine[(DB * 4 + 1) * 64] = l_run;
         }
         __syncthreads();
         if (kh > 0) return;
 #pragma unroll
         for (int g = 1; g < KS; g++) {
             const float *other = xch + (size_t)((g - 1) * QW + qw) * PER_LANE * 64 + lane;
-            const float m_o = other[(DB * 16) * 64], l_o = other[(DB * 16 + 1) * 64];
+            const float m_o = other[(DB * 4) * 64], l_o = other[(DB * 4 + 1) * 64];
             const float m_new = fmaxf(m_run, m_o);
             const float w_me = __builtin_amdgcn_exp2f(m_run - m_new), w_o = __builtin_amdgcn_exp2f(m_o - m_new);
             l_run = l_run * w_me + l_o * w_o;
@@ -499,37 +507,33 @@ __global__ __launch_bounds__(AT_THREADS) void prefill_attn_kernel(PrefillAttnArg
 #pragma unroll
             for (int db = 0; db < DB; db++)
 #pragma unroll
-                for (int v = 0; v < 16; v++) acc_o[db][v] = acc_o[db][v] * w_me + other[(db * 16 + v) * 64] * w_o;
+                for (int v = 0; v < 4; v++) acc_o[db][v] = acc_o[db][v] * w_me + other[(db * 4 + v) * 64] * w_o;
         }
     }
-    const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
+    const float l_tot = quad_rows_sum(l_run);
     if (qrow >= a.S) return;
     const float inv = 1.0f / l_tot;
     const int qd = a.H * HD;
-    // accumulator value v of block db is d = 32 db + 8 (v / 4) + 4 (lane / 32) + v % 4
+    // value v of block db is d = 16 db + 4 c4 + v
 #pragma unroll
-    for (int db = 0; db < DB; db++)
+    for (int db = 0; db < DB; db++) {
+        const int d0 = h * HD + 16 * db + 4 * c4;
+        f32x4 o = acc_o[db] * inv;
+        if (a.out_f32) *reinterpret_cast<f32x4 *>(a.out_f32 + (size_t)qrow * qd + d0) = o;
+        if (a.out_split) {
+            uint32_t lo[NP], hi[NP];
+            split_pair<NP>(o[0], o[1], lo);
+            split_pair<NP>(o[2], o[3], hi);
+            uint16_t *o16 = a.out_split + (size_t)qrow * NP * qd + d0;
 #pragma unroll
-        for (int g = 0; g < 4; g++) {
-            const int d0 = h * HD + 32 * db + 8 * g + 4 * lh;
-            f32x4 o;
-#pragma unroll
-            for (int i = 0; i < 4; i++) o[i] = acc_o[db][4 * g + i] * inv;
-            if (a.out_f32) *reinterpret_cast<f32x4 *>(a.out_f32 + (size_t)qrow * qd + d0) = o;
-            if (a.out_split) {
-                uint32_t lo[NP], hi[NP];
-                split_pair<NP>(o[0], o[1], lo);
-                split_pair<NP>(o[2], o[3], hi);
-                uint16_t *o16 = a.out_split + (size_t)qrow * NP * qd + d0;
-#pragma unroll
-                for (int p = 0; p < NP; p++) {
-                    u32x2 w;
-                    w.x = lo[p];
-                    w.y = hi[p];
-                    *reinterpret_cast<u32x2 *>(o16 + (size_t)p * qd) = w;
-                }
+            for (int p = 0; p < NP; p++) {
+                u32x2 w;
+                w.x = lo[p];
+                w.y = hi[p];
+                *reinterpret_cast<u32x2 *>(o16 + (size_t)p * qd) = w;
             }
         }
+    }
 }
 
 }  // namespace
@@ -647,22 +651,24 @@ int prefill_attn_launch(hm_ctx *ctx, const PrefillAttnArgs &a) {
     }
     const int qrows = 128 / ks;
     const dim3 grid((unsigned)((a.S + qrows - 1) / qrows), (unsigned)a.H);
-    const size_t lds = (size_t)ks * (AT_KEYS * a.hd * 2 + a.hd * 128);
+    // two sets of ks pairs of 32-key tiles; the final exchange of the key groups wants
+    // (ks - 1) * (128 / ks / 16) sets of (hd / 4 + 2) * 256 bytes
+    const size_t lds = std::max<size_t>((size_t)2 * ks * 2 * A8_KEYS * a.hd * 2, (size_t)(ks - 1) * (8 / ks) * (a.hd / 4 + 2) * 256);
     auto launch = [&](auto kernel) -> int {
         if (lds > 64 * 1024) {
             const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
             HM_REQUIRE(ctx, e == hipSuccess, "prefill_attn: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));
         }
-        hipLaunchKernelGGL(kernel, grid, dim3(AT_THREADS), lds, ctx->stream, a);
+        hipLaunchKernelGGL(kernel, grid, dim3(A8_THREADS), lds, ctx->stream, a);
         return HM_OK;
     };
     int rc = HM_OK;
 #define HM_AT_CASE(HDV, NPV)                                                             \
     if (a.hd == HDV && a.pieces == NPV) {                                                \
-        if (ks == 1) rc = launch(prefill_attn_kernel<HDV, NPV, 1>);                      \
-        else if (ks == 2) rc = launch(prefill_attn_kernel<HDV, NPV, 2>);                 \
-        else rc = launch(prefill_attn_kernel<HDV, NPV, 4>);                              \
+        if (ks == 1) rc = launch(prefill_attn16_kernel<HDV, NPV, 1>);                    \
+        else if (ks == 2) rc = launch(prefill_attn16_kernel<HDV, NPV, 2>);               \
+        else rc = launch(prefill_attn16_kernel<HDV, NPV, 4>);                            \
     }
     HM_AT_CASE(128, 3)
     HM_AT_CASE(128, 2)

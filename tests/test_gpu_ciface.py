@@ -50,11 +50,19 @@ CHUNKS = [5, 1, 11, 64]
 
 
 def check_rows(which, got, want, tol=1e-2):
-    """Logits of one call against the oracle's batched run_kv over the same tokens."""
+    """Logits of one call against the oracle's batched run_kv over the same tokens. Calls of 16 tokens or more
+    run on the matrix cores like the prompt pass and are held to the prompt-pass tests' bound: 2e-3 of the
+    logit scale (K/V elements that land on the other side of a bf16 rounding boundary move small logits by
+    ~1e-4 of the scale, which the element-wise metric of the shorter calls counts as 1e-2)."""
     for r in range(len(want)):
-        err = mf.rel_err(got[r], want[r])
-        say(f"{which}: row {r} of {len(want)} logits rel err {err:.2e}")
-        assert err < tol
+        if len(want) >= 16:
+            err = float(np.abs(np.asarray(got[r], np.float64) - want[r]).max() / np.abs(want[r]).max())
+            say(f"{which}: row {r} of {len(want)} logits err / logit scale {err:.2e}")
+            assert err < 2e-3
+        else:
+            err = mf.rel_err(got[r], want[r])
+            say(f"{which}: row {r} of {len(want)} logits rel err {err:.2e}")
+            assert err < tol
         assert int(len(got[r]) - 1 - np.argmax(got[r][::-1])) == int(len(want[r]) - 1 - np.argmax(want[r][::-1]))
 
 
