@@ -33,4 +33,12 @@ int gemm_split_split_nk(hm_ctx *ctx, const uint16_t *d_a_split, const uint16_t *
 int gemm_pieces_nk(hm_ctx *ctx, const uint16_t *d_a_split, int a_pieces, const uint16_t *d_b_split, int b_pieces,
                    float *d_c, int M, int K, int N, int max_parts = 1, int *parts = nullptr, int ldc = 0);
 
+// 3 x 1 pieces against a block-scaled integer matrix: d_b_ints [N][K] bf16 holds the integers of a Q8_0 / Q4_0
+// matrix (exact), d_scales [K / 32][npad] f32 the scale of every 32-wide block of every row (npad >= N rounded
+// up to 128). C = sum over blocks of scale * (A x ints^T over the block). Slices and ldc as above.
+int gemm_pieces_scaled_nk(hm_ctx *ctx, const uint16_t *d_a_split, const uint16_t *d_b_ints, const float *d_scales, int npad,
+                          float *d_c, int M, int K, int N, int max_parts = 1, int *parts = nullptr, int ldc = 0);
+int gemm_pieces_any(hm_ctx *ctx, const uint16_t *d_a_split, int a_pieces, const uint16_t *d_b_split, int b_pieces,
+                    const float *d_scales, int npad, float *d_c, int M, int K, int N, int max_parts, int *parts, int ldc);
+
 }  // namespace homura

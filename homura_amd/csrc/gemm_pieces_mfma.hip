@@ -15,6 +15,12 @@
 // fills slot s of row r fetches chunk s ^ ((r >> 2) & 3), which makes the operand reads conflict
 // free). NB stages rotate through LDS (128 to 144 KiB), one barrier per stage. M, N ragged as in the
 // other kernel; K slices (grid.y) write partial sums the consumer adds in index order.
+//
+// SC (block-scaled B): B holds the integers of a Q8_0 / Q4_0 matrix as bf16 (exact) and every 32-wide block
+// of a row has an f32 scale, scales[k / 32][n] (row stride npad, a multiple of 128). A stage is exactly one
+// block: its AP products are summed on their own and join the result times the block's scale, d * sum(x q),
+// the decode kernels' form of the reference's sum(x (d q)) (src/hf/emitter_quant.rs:675-702). The 128 scales
+// of a stage travel with its tiles (64 bytes per wavefront).
 #include <algorithm>
 #include <type_traits>
 
@@ -34,6 +40,8 @@ constexpr int THREADS = 512;
 struct PieceDims {
     int M, N, Kb, lda, ldb, ldc;
     int stages_per_split;  // stages of 32 k per grid.y slice
+    const float *scales;   // SC: [Kb / 32][npad]
+    int npad;
 };
 
 __device__ __forceinline__ int lds_off(int r, int chunk) { return r * ROW_BYTES + ((chunk ^ ((r >> 2) & 3)) << 4); }
@@ -50,23 +58,30 @@ __device__ __forceinline__ bf16x8 lds_read16(uint32_t addr) {
     asm volatile("ds_read_b128 %0, %1" : "=v"(v) : "v"(addr) : "memory");
     return v;
 }
+__device__ __forceinline__ float lds_read4(uint32_t addr) {
+    float v;
+    asm volatile("ds_read_b32 %0, %1" : "=v"(v) : "v"(addr) : "memory");
+    return v;
+}
 
 extern __shared__ __attribute__((aligned(16))) char stage_lds[];
 
-template <int AP, int BP>
+template <int AP, int BP, bool SC = false>
 struct Shape {
-    static constexpr int T = AP + BP;                       // tiles (and loads per wavefront) per stage
-    static constexpr int STAGE = T * PIECE_TILE;            // bytes
-    static constexpr int NB = STAGE <= 32 * 1024 ? 4 : 3;   // stages in LDS
+    static constexpr int TILES = AP + BP;                   // operand tiles per stage
+    static constexpr int T = TILES + (SC ? 1 : 0);          // loads per wavefront and stage
+    static constexpr int STAGE = TILES * PIECE_TILE + (SC ? TN * 4 : 0);  // bytes
+    static constexpr int NB = TILES * PIECE_TILE <= 32 * 1024 ? 4 : 3;    // stages in LDS
     static constexpr int LDS = NB * STAGE > 64 * 1024 ? NB * STAGE : 64 * 1024;  // the final exchange wants 64 KiB
 };
 
-template <int AP, int BP>
+template <int AP, int BP, bool SC = false>
 __global__ __launch_bounds__(THREADS) void gemm_pieces_kernel(const uint16_t *__restrict__ A,
                                                               const uint16_t *__restrict__ B, float *__restrict__ C,
                                                               const PieceDims g) {
-    using S = Shape<AP, BP>;
+    using S = Shape<AP, BP, SC>;
     constexpr int T = S::T, NB = S::NB, STAGE = S::STAGE;
+    static_assert(!SC || BP == 1, "block scales go with a single B operand");
     const int M = g.M, N = g.N;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int kgrp = wave >> 2, wm = (wave >> 1) & 1, wn = wave & 1;
@@ -99,6 +114,8 @@ __global__ __launch_bounds__(THREADS) void gemm_pieces_kernel(const uint16_t *__
         b_src = B + (size_t)min(n0 + r, N - 1) * g.ldb + c * 8;
     }
     const int wave_dst = __builtin_amdgcn_readfirstlane(wave * 1024);
+    const int wave_dst64 = __builtin_amdgcn_readfirstlane(wave * 64);
+    const float *s_src = SC ? g.scales + n0 + wave * 16 + (lane & 3) * 4 : nullptr;  // (n0 + 127 < npad)
     int k_req = s_first * TK;  // k of the next stage to request
     // a stage past the end re-reads the last one (nobody multiplies it): the wait counts stay exact
     auto request = [&](int buf) {
@@ -108,6 +125,9 @@ __global__ __launch_bounds__(THREADS) void gemm_pieces_kernel(const uint16_t *__
         for (int p = 0; p < AP; p++) dma16(a_src + p * g.Kb + k, base + p * PIECE_TILE);
 #pragma unroll
         for (int p = 0; p < BP; p++) dma16(b_src + p * g.Kb + k, base + (AP + p) * PIECE_TILE);
+        if (SC && lane < 4)  // this wavefront's 16 of the stage's 128 block scales
+            dma16(reinterpret_cast<const uint16_t *>(s_src + (size_t)(k / TK) * g.npad),
+                  stage_lds + buf * STAGE + S::TILES * PIECE_TILE + wave_dst64);
         k_req += TK;
     };
 #pragma unroll
@@ -124,8 +144,14 @@ __global__ __launch_bounds__(THREADS) void gemm_pieces_kernel(const uint16_t *__
     }
     // operand registers, two sets: the reads of the next stage are in flight during the MFMAs
     bf16x8 fa[2][AP][2], fb[2][BP][2];
+    float fs[2][2];  // SC: the block scales of this lane's two columns
+    const uint32_t s_off = lds0 + S::TILES * PIECE_TILE + (wn * 64 + l32) * 4;
     auto read_stage = [&](int set, int buf) {
         const uint32_t off = (uint32_t)(buf * STAGE);
+        if (SC) {
+#pragma unroll
+            for (int j = 0; j < 2; j++) fs[set][j] = lds_read4(s_off + off + j * 128);
+        }
 #pragma unroll
         for (int p = 0; p < AP; p++)
 #pragma unroll
@@ -140,7 +166,14 @@ __global__ __launch_bounds__(THREADS) void gemm_pieces_kernel(const uint16_t *__
     // youngest (NB - 2) T (DRAIN: for all of them), then meet the other wavefronts.
 #define HM_PIECES_WAIT(CNT, SET)                                                                                    \
     do {                                                                                                            \
-        if constexpr (AP == 3 && BP == 3)                                                                           \
+        if constexpr (SC)                                                                                           \
+            asm volatile("s_waitcnt vmcnt(" #CNT ") lgkmcnt(0)\n\ts_barrier"                                        \
+                         : "+v"(fa[SET][0][0]), "+v"(fa[SET][0][1]), "+v"(fa[SET][1][0]), "+v"(fa[SET][1][1]),      \
+                           "+v"(fa[SET][2][0]), "+v"(fa[SET][2][1]), "+v"(fb[SET][0][0]), "+v"(fb[SET][0][1]),      \
+                           "+v"(fs[SET][0]), "+v"(fs[SET][1])                                                       \
+                         :                                                                                          \
+                         : "memory");                                                                               \
+        else if constexpr (AP == 3 && BP == 3)                                                                      \
             asm volatile("s_waitcnt vmcnt(" #CNT ") lgkmcnt(0)\n\ts_barrier"                                        \
                          : "+v"(fa[SET][0][0]), "+v"(fa[SET][0][1]), "+v"(fa[SET][1][0]), "+v"(fa[SET][1][1]),      \
                            "+v"(fa[SET][2][0]), "+v"(fa[SET][2][1]), "+v"(fb[SET][0][0]), "+v"(fb[SET][0][1]),      \
@@ -161,17 +194,35 @@ __global__ __launch_bounds__(THREADS) void gemm_pieces_kernel(const uint16_t *__
                          : "memory");                                                                               \
     } while (0)
     // (NB - 2) T: 3 x 1 pieces 8, 2 x 1 pieces 6, 3 x 3 pieces 6
-    static_assert((AP == 3 && BP == 1 && (NB - 2) * T == 8) || (AP != 3 || BP != 1), "wait count");
-    static_assert(((AP == 2 || BP == 3) && (NB - 2) * T == 6) || (AP == 3 && BP == 1), "wait count");
+    static_assert(!SC || (AP == 3 && (NB - 2) * T == 10), "wait count");
+    static_assert(SC || (AP == 3 && BP == 1 && (NB - 2) * T == 8) || (AP != 3 || BP != 1), "wait count");
+    static_assert(SC || ((AP == 2 || BP == 3) && (NB - 2) * T == 6) || (AP == 3 && BP == 1), "wait count");
     auto wait_and_meet = [&](int set) {
         if (set == 0) {
-            if constexpr (AP == 3 && BP == 1) HM_PIECES_WAIT(8, 0); else HM_PIECES_WAIT(6, 0);
+            if constexpr (SC) HM_PIECES_WAIT(10, 0); else if constexpr (AP == 3 && BP == 1) HM_PIECES_WAIT(8, 0); else HM_PIECES_WAIT(6, 0);
         } else {
-            if constexpr (AP == 3 && BP == 1) HM_PIECES_WAIT(8, 1); else HM_PIECES_WAIT(6, 1);
+            if constexpr (SC) HM_PIECES_WAIT(10, 1); else if constexpr (AP == 3 && BP == 1) HM_PIECES_WAIT(8, 1); else HM_PIECES_WAIT(6, 1);
         }
     };
     // the products of one stage: smallest pieces first
     auto multiply = [&](int set) {
+        if constexpr (SC) {
+            // the block's sum on its own (smallest pieces first), then times the block's scale
+#pragma unroll
+            for (int i = 0; i < 2; i++)
+#pragma unroll
+                for (int j = 0; j < 2; j++) {
+                    f32x16 t;
+#pragma unroll
+                    for (int v = 0; v < 16; v++) t[v] = 0.f;
+#pragma unroll
+                    for (int pa = AP - 1; pa >= 0; pa--)
+                        t = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[set][pa][i], fb[set][0][j], t, 0, 0, 0);
+#pragma unroll
+                    for (int v = 0; v < 16; v++) acc[i][j][v] = fmaf(t[v], fs[set][j], acc[i][j][v]);
+                }
+            return;
+        }
 #pragma unroll
         for (int order = AP + BP - 2; order >= 0; order--)
 #pragma unroll
@@ -244,23 +295,37 @@ __global__ __launch_bounds__(THREADS) void gemm_pieces_kernel(const uint16_t *__
             }
 }
 
-template <int AP, int BP>
+template <int AP, int BP, bool SC = false>
 int launch(hm_ctx *ctx, const char *who, const uint16_t *a, const uint16_t *b, float *c, const PieceDims &g,
            unsigned tiles, unsigned slices) {
-    using S = Shape<AP, BP>;
-    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_pieces_kernel<AP, BP>),
+    using S = Shape<AP, BP, SC>;
+    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_pieces_kernel<AP, BP, SC>),
                                                        hipFuncAttributeMaxDynamicSharedMemorySize, S::LDS);
     HM_REQUIRE(ctx, attr == hipSuccess, "%s: cannot reserve %d bytes of LDS: %s", who, S::LDS, hipGetErrorString(attr));
-    hipLaunchKernelGGL((gemm_pieces_kernel<AP, BP>), dim3(tiles, slices), dim3(THREADS), S::LDS, ctx->stream, a, b, c, g);
+    hipLaunchKernelGGL((gemm_pieces_kernel<AP, BP, SC>), dim3(tiles, slices), dim3(THREADS), S::LDS, ctx->stream, a, b, c, g);
     HM_LAUNCH_CHECK(ctx);
     return HM_OK;
 }
 
 }  // namespace
 
+int homura::gemm_pieces_scaled_nk(hm_ctx *ctx, const uint16_t *d_a_split, const uint16_t *d_b_ints, const float *d_scales,
+                                  int npad, float *d_c, int M, int K, int N, int max_parts, int *parts, int ldc) {
+    HM_CHECK_CTX(ctx);
+    HM_REQUIRE(ctx, d_scales && npad >= (N + TN - 1) / TN * TN && npad % 4 == 0 && ((uintptr_t)d_scales % 16) == 0,
+               "gemm_pieces_scaled_nk: the scales need a row stride of whole tiles (N=%d, stride %d)", N, npad);
+    return gemm_pieces_any(ctx, d_a_split, 3, d_b_ints, 1, d_scales, npad, d_c, M, K, N, max_parts, parts, ldc);
+}
+
 int homura::gemm_pieces_nk(hm_ctx *ctx, const uint16_t *d_a_split, int a_pieces, const uint16_t *d_b_split, int b_pieces,
                            float *d_c, int M, int K, int N, int max_parts, int *parts, int ldc) {
-    const char *who = "gemm_pieces_nk";
+    return gemm_pieces_any(ctx, d_a_split, a_pieces, d_b_split, b_pieces, nullptr, 0, d_c, M, K, N, max_parts, parts, ldc);
+}
+
+int homura::gemm_pieces_any(hm_ctx *ctx, const uint16_t *d_a_split, int a_pieces, const uint16_t *d_b_split, int b_pieces,
+                            const float *d_scales, int npad, float *d_c, int M, int K, int N, int max_parts, int *parts,
+                            int ldc) {
+    const char *who = d_scales ? "gemm_pieces_scaled_nk" : "gemm_pieces_nk";
     HM_CHECK_CTX(ctx);
     HM_REQUIRE(ctx, d_a_split && d_b_split && d_c, "%s: NULL pointer", who);
     HM_REQUIRE(ctx, M > 0 && N > 0 && K > 0 && K % TK == 0, "%s: need M, N > 0 and K %% 32 == 0 (M=%d K=%d N=%d)", who, M, K, N);
@@ -276,6 +341,8 @@ int homura::gemm_pieces_nk(hm_ctx *ctx, const uint16_t *d_a_split, int a_pieces,
     g.lda = a_pieces * K;
     g.ldb = b_pieces * K;
     g.ldc = ldc > 0 ? ldc : N;
+    g.scales = d_scales;
+    g.npad = npad;
     HM_REQUIRE(ctx, g.ldc >= N, "%s: ldc %d below N %d", who, g.ldc, N);
     // K slices while they still add whole waves of workgroups to a grid smaller than the chip, at least
     // eight stages (256 k) per slice
@@ -286,6 +353,7 @@ int homura::gemm_pieces_nk(hm_ctx *ctx, const uint16_t *d_a_split, int a_pieces,
     g.stages_per_split = ((ns_total + want - 1) / want + 1) / 2 * 2;  // even: stages run in pairs
     const int slices = (ns_total + g.stages_per_split - 1) / g.stages_per_split;
     if (parts) *parts = slices;
+    if (d_scales) return launch<3, 1, true>(ctx, who, d_a_split, d_b_split, d_c, g, (unsigned)tiles, (unsigned)slices);
     if (b_pieces == 3) return launch<3, 3>(ctx, who, d_a_split, d_b_split, d_c, g, (unsigned)tiles, (unsigned)slices);
     if (a_pieces == 3) return launch<3, 1>(ctx, who, d_a_split, d_b_split, d_c, g, (unsigned)tiles, (unsigned)slices);
     return launch<2, 1>(ctx, who, d_a_split, d_b_split, d_c, g, (unsigned)tiles, (unsigned)slices);

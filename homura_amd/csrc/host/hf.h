@@ -213,6 +213,10 @@ class HfModel {
         Buffer q8, q8s;
         std::vector<Buffer> icache;
         bool icache_off = false;  // the planes did not fit: K-quant groups keep the bf16 pieces
+        // Q8_0 / Q4_0 groups: per [layer * 4 + group] the group's integers as bf16 followed by its block
+        // scales [K / 32][N rounded up to 128] (gemm_pieces_scaled_nk)
+        std::vector<Buffer> scache;
+        bool scache_off = false;
         // Tests: the f32 rows entering the Q8_K quantisation of the K-quant products, for cache positions
         // [capture_base, capture_base + capture_rows); per layer [rows][hidden] (q|k|v), [rows][q_dim] (o),
         // [rows][hidden] (gate|up), [rows][inter] (down).

@@ -1850,6 +1850,8 @@ int HfModel::prefill_chunk(const int32_t *h_ids, int n, float *h_logits) {
             grown.capture_base = p.capture_base;
             grown.icache = std::move(p.icache);  // weights, not rows: they do not depend on the chunk size
             grown.icache_off = p.icache_off;
+            grown.scache = std::move(p.scache);
+            grown.scache_off = p.scache_off;
             p = std::move(grown);
         }
         p.ids = Buffer::alloc(ctx_, {rows}, DType::F32);  // int32 ids
@@ -1960,6 +1962,61 @@ int HfModel::prefill_chunk(const int32_t *h_ids, int n, float *h_logits) {
         }
         return &slot;
     };
+    // Q8_0 / Q4_0 groups multiply their integers (bf16, exact) and apply the block scales in the GEMM
+    // (2 bytes a weight + the scales), under the same budget; otherwise the dequantised weights as bf16 pieces.
+    auto plain_block = [&](int l, int which) {
+        const DType t = proj_dtype(l, which);
+        return quant && (t == DType::Q8_0 || t == DType::Q4_0);
+    };
+    if (quant && p.scache.empty() && !p.scache_off && prefill_weight_cache_bytes_ > 0) {
+        size_t need = 0;
+        const int gK[4] = {hidden, qd, hidden, inter}, gN[4] = {nqkv, hidden, 2 * inter, hidden}, gfirst[4] = {0, 3, 4, 6};
+        for (int l = 0; l < c.num_hidden_layers; l++)
+            for (int gq = 0; gq < 4; gq++)
+                if (plain_block(l, gfirst[gq]))
+                    need += (size_t)gN[gq] * gK[gq] * 2 + (size_t)(gK[gq] / 32) * (gN[gq] + 127) * 4 + 512;
+        size_t free_b = 0, total_b = 0;
+        if (hipMemGetInfo(&free_b, &total_b) != hipSuccess) free_b = total_b = 0;
+        if (need > 0 && need <= prefill_weight_cache_bytes_ && need + total_b / 8 <= free_b)
+            p.scache.resize((size_t)c.num_hidden_layers * 4);
+        else
+            p.scache_off = true;
+    }
+    auto scaled_ints = [&](int l, int g, int first, int count, int K, int *npad_out) -> const Buffer * {
+        if (p.scache.empty()) return nullptr;
+        for (int j = first; j < first + count; j++)
+            if (!plain_block(l, j)) return nullptr;
+        int N = 0;
+        for (int j = first; j < first + count; j++) N += proj_n[j];
+        const int npad = (N + 127) / 128 * 128;
+        *npad_out = npad;
+        Buffer &slot = p.scache[(size_t)l * 4 + g];
+        if (slot) return &slot;
+        const size_t ib = ((size_t)N * K * 2 + 255) / 256 * 256, sb = (size_t)(K / 32) * npad * 4;
+        slot = Buffer::alloc(ctx_, {(int64_t)((ib + sb + 3) / 4)}, DType::F32);
+        if (!slot) {
+            (void)hipGetLastError();
+            return nullptr;
+        }
+        const bool interleave = first == 4 && count == 2;
+        uint16_t *ints = slot.as<uint16_t>();
+        float *scales = reinterpret_cast<float *>(slot.as<char>() + ib);
+        int row = 0;
+        for (int j = first; j < first + count; j++) {
+            auto it = slot_by_name_.find("model.layers." + std::to_string(l) + "." + proj_name[j]);
+            int rc2 = it == slot_by_name_.end() ? HM_ERR_STATE : HM_OK;
+            if (rc2 == HM_OK)
+                rc2 = quant_ints_launch(ctx_, (int)proj_dtype(l, j), weight_bufs_[it->second].as<uint8_t>(), proj_n[j], K,
+                                        interleave ? ints : ints + (size_t)row * K, interleave ? scales : scales + row, npad,
+                                        interleave ? 2 : 1, interleave ? j - first : 0);
+            if (rc2 != HM_OK) {
+                slot = Buffer();
+                return nullptr;
+            }
+            row += proj_n[j];
+        }
+        return &slot;
+    };
     const Buffer *i8 = nullptr;  // the planes of the group about to be multiplied, if it takes that path
     int8_t *q8 = p.q8 ? p.q8.as<int8_t>() : nullptr;
     float *q8s = p.q8s ? p.q8s.as<float>() : nullptr;
@@ -1971,6 +2028,15 @@ int HfModel::prefill_chunk(const int32_t *h_ids, int n, float *h_logits) {
             const size_t pb = (kq_i8_plane_bytes(N, K) + 255) / 256 * 256;
             return gemm_q8k_kquant_nk(ctx_, q8, q8s, i8->as<int8_t>(), reinterpret_cast<const float *>(i8->as<char>() + pb), out, n,
                                       K, N, MP, &parts);
+        }
+        {
+            int npad = 0;
+            const int g = first == 0 ? 0 : first == 3 ? 1 : first == 4 ? 2 : 3;
+            if (const Buffer *sc = scaled_ints(l, g, first, count, K, &npad)) {
+                const size_t ib = ((size_t)N * K * 2 + 255) / 256 * 256;
+                return gemm_pieces_scaled_nk(ctx_, split, sc->as<uint16_t>(), reinterpret_cast<const float *>(sc->as<char>() + ib),
+                                             npad, out, n, K, N, MP, &parts);
+            }
         }
         const bool interleave = first == 4 && count == 2;
         uint16_t *wsplit = p.wsplit.as<uint16_t>();

@@ -42,6 +42,12 @@ int dequant_split_launch(hm_ctx *ctx, int hm_dtype, const uint8_t *d_blocks, int
                          int row_mult = 1, int row_off = 0);
 
 
+// A Q8_0 / Q4_0 matrix (raw GGUF blocks [N][K / 32]) as the operands of gemm_pieces_scaled_nk: its integers as
+// bf16 (exact), row n in row n * row_mult + row_off of d_ints ([.][K]), and its block scales, d_scales
+// [K / 32][npad] f32 (column = output row).
+int quant_ints_launch(hm_ctx *ctx, int hm_dtype, const uint8_t *d_blocks, int N, int K, uint16_t *d_ints, float *d_scales,
+                      int npad, int row_mult = 1, int row_off = 0);
+
 // out_split = split(silu(gate) * up) for gate/up interleaved per row: gu [rows][2 * inter] =
 // (gate_0, up_0, gate_1, up_1, ...), the column order of the packed gate|up weight.
 int silu_mul_split_launch(hm_ctx *ctx, const float *d_gu, int parts, uint16_t *d_out_split, int pieces, int rows,

@@ -116,6 +116,36 @@ __global__ __launch_bounds__(256) void dequant_split_kernel(const uint8_t *__res
     for (int p = 0; p < 3; p++) *reinterpret_cast<bf16x8 *>(o + (size_t)p * K) = pc[p];
 }
 
+// A Q8_0 / Q4_0 matrix as its integers (bf16, exact) and its block scales: row n goes to row n * row_mult +
+// row_off of ints ([.][K]) and to that column of scales ([K / 32][npad] f32). Eight consecutive weights per
+// thread. The weight is scale * integer (reference src/gguf.rs:825-833; Q4_0: nibble - 8).
+template <int QF>
+__global__ __launch_bounds__(256) void quant_ints_kernel(const uint8_t *__restrict__ blocks, uint16_t *__restrict__ ints,
+                                                         float *__restrict__ scales, int K, size_t n8, int npad,
+                                                         int row_mult, int row_off) {
+    constexpr int BB = QuantFormatTraits<QF>::BYTES;
+    static_assert(QF == QF_Q8_0 || QF == QF_Q4_0, "32-wide blocks with one scale");
+    const size_t t = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= n8) return;
+    const size_t e = t * 8, row = e / K, orow = row * row_mult + row_off;
+    const int c = (int)(e % K), j0 = c % 32;
+    const uint8_t *blk = blocks + (e / 32) * BB;
+    float f[8];
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+        if (QF == QF_Q8_0) {
+            f[j] = (float)(int8_t)blk[2 + j0 + j];
+        } else {
+            const uint8_t byte = blk[2 + (j0 + j) % 16];
+            f[j] = (float)((j0 + j < 16 ? (byte & 0x0F) : (byte >> 4)) - 8);
+        }
+    }
+    bf16x8 pc[1];
+    split8<1>(f, pc);  // integers of at most 8 bits: the bf16 is exact
+    *reinterpret_cast<bf16x8 *>(ints + orow * (size_t)K + c) = pc[0];
+    if (j0 == 0) scales[(size_t)(c / 32) * npad + orow] = f16_at(blk);
+}
+
 // One workgroup per row, four consecutive elements per thread and step (dim % 4 == 0); the arithmetic
 // of the decode path's RMSNorm kernel (reference src/graph_builder/emit_linalg.rs:7-26; Residual+Norm,
 // src/hf/emitter.rs:787-790).
@@ -615,6 +645,25 @@ int dequant_split_launch(hm_ctx *ctx, int hm_dtype, const uint8_t *d_blocks, int
     return HM_OK;
 }
 
+int quant_ints_launch(hm_ctx *ctx, int hm_dtype, const uint8_t *d_blocks, int N, int K, uint16_t *d_ints, float *d_scales,
+                      int npad, int row_mult, int row_off) {
+    HM_REQUIRE(ctx, d_blocks && d_ints && d_scales, "quant_ints: NULL pointer");
+    HM_REQUIRE(ctx, hm_dtype == HM_DTYPE_Q8_0 || hm_dtype == HM_DTYPE_Q4_0, "quant_ints: dtype %d is not Q8_0 / Q4_0", hm_dtype);
+    HM_REQUIRE(ctx, N > 0 && K > 0 && K % 32 == 0 && row_mult >= 1 && row_off >= 0 && row_off < row_mult &&
+                        (size_t)(N - 1) * row_mult + row_off < (size_t)npad,
+               "quant_ints: bad shape (N=%d K=%d stride %d)", N, K, npad);
+    HM_REQUIRE(ctx, ((uintptr_t)d_ints % 16) == 0, "quant_ints: misaligned output");
+    const size_t n8 = (size_t)N * K / 8;
+    HM_REQUIRE(ctx, (n8 + 255) / 256 <= 0x7fffffffULL, "quant_ints: matrix too large");
+    const dim3 grid((unsigned)((n8 + 255) / 256));
+    if (hm_dtype == HM_DTYPE_Q8_0)
+        hipLaunchKernelGGL((quant_ints_kernel<QF_Q8_0>), grid, dim3(256), 0, ctx->stream, d_blocks, d_ints, d_scales, K, n8, npad, row_mult, row_off);
+    else
+        hipLaunchKernelGGL((quant_ints_kernel<QF_Q4_0>), grid, dim3(256), 0, ctx->stream, d_blocks, d_ints, d_scales, K, n8, npad, row_mult, row_off);
+    HM_LAUNCH_CHECK(ctx);
+    return HM_OK;
+}
+
 int qkv_post_launch(hm_ctx *ctx, const QkvPostArgs &a) {
     HM_REQUIRE(ctx, a.qkv && a.cos_tab && a.sin_tab && a.kcache && a.vcache, "qkv_post: NULL pointer");
     HM_REQUIRE(ctx, a.S > 0 && a.H > 0 && a.kvh > 0 && a.past >= 0 && a.parts >= 1, "qkv_post: bad shape");
@@ -725,6 +774,28 @@ extern "C" int hm_gemm_f32_quant_nk(hm_ctx *ctx, const float *d_x_mk, const uint
         }
         return rc;
     }
+    if (!kq) {
+        // Q8_0 / Q4_0: three-piece rows x the matrix's integers, every 32-wide block's sum times its scale.
+        // Workspace: the split activations, then the integers (bf16) and scales of as many weight rows as fit.
+        const size_t a_bytes = ((size_t)M * K * 6 + 255) / 256 * 256;
+        const size_t per_row = (size_t)K * 2 + (size_t)(K / 32) * 4;
+        HM_REQUIRE(ctx, a_bytes + 128 * per_row + 256 <= ctx->workspace_bytes,
+                   "hm_gemm_f32_quant_nk: M * K = %zu activations exceed the workspace", (size_t)M * K);
+        uint16_t *a_split = (uint16_t *)ctx->workspace;
+        char *wbase = (char *)ctx->workspace + a_bytes;
+        const int slab = (int)std::min<size_t>((size_t)(N + 127) / 128 * 128, (ctx->workspace_bytes - a_bytes - 256) / per_row / 128 * 128);
+        int rc = homura::split_rows_launch(ctx, d_x_mk, a_split, 3, (size_t)M, K, false);
+        const size_t row_bytes = (size_t)K / 32 * (dtype == HM_DTYPE_Q8_0 ? 34 : 18);
+        for (int n0 = 0; n0 < N && rc == HM_OK; n0 += slab) {
+            const int rows = std::min(slab, N - n0), npad = (rows + 127) / 128 * 128;
+            uint16_t *ints = (uint16_t *)wbase;
+            float *wsc = (float *)(wbase + ((size_t)rows * K * 2 + 255) / 256 * 256);
+            rc = homura::quant_ints_launch(ctx, dtype, d_w_blocks + (size_t)n0 * row_bytes, rows, K, ints, wsc, npad);
+            if (rc == HM_OK) rc = homura::gemm_pieces_scaled_nk(ctx, a_split, ints, wsc, npad, d_out + n0, M, K, rows, 1, nullptr, N);
+        }
+        return rc;
+    }
+    // (K-quant rows wider than the int8 path takes)
     // workspace: the split activations, then as many split weight rows as fit (a multiple of the tile)
     const size_t a_bytes = ((size_t)M * K * 6 + 255) / 256 * 256;
     HM_REQUIRE(ctx, a_bytes + (size_t)128 * K * 6 <= ctx->workspace_bytes,
