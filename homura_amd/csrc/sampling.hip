@@ -43,15 +43,30 @@ struct SampleArgs {
     int *stop;
 };
 
-// Where the pick goes (and which draw it uses) when the cursor says which step this is.
-__device__ __forceinline__ void deliver_pick(const SampleArgs &a, int pick) {
+// What a sampler kernel needs to know about its step, read once at its start: the loads are two dependent trips
+// to memory (the cursor, then the draw it points at) that would otherwise sit at the very end of a kernel that
+// runs as a single workgroup.
+struct StepInfo {
+    int idx;     // the step that was just taken (cursor->step - 1), or -1 without a cursor
+    float draw;  // Rng::next_f32 of this step
+    int stop;    // *stop (-1: no end-of-sequence pick so far), 0 without a stop cell
+};
+__device__ __forceinline__ StepInfo load_step(const SampleArgs &a) {
+    StepInfo s;
+    s.idx = a.cursor ? a.cursor->step - 1 : -1;
+    s.draw = (a.cursor && a.draws) ? a.draws[s.idx] : a.draw;  // (a greedy pick with penalties has no draws)
+    s.stop = a.stop ? *a.stop : 0;
+    return s;
+}
+
+// Where the pick goes when the cursor says which step this is.
+__device__ __forceinline__ void deliver_pick(const SampleArgs &a, const StepInfo &st, int pick) {
     *a.out = pick;
     if (a.counts_update) a.counts_update[pick] += 1;
     if (a.cursor) {
-        const int idx = a.cursor->step - 1;
-        if (a.list) a.list[idx] = pick;
+        if (a.list) a.list[st.idx] = pick;
         a.cursor->token = pick;
-        if (a.stop && pick == a.eos && *a.stop < 0) *a.stop = idx;
+        if (a.stop && pick == a.eos && st.stop < 0) *a.stop = st.idx;
     } else if (a.list) {
         a.list[a.list_pos] = pick;
     }
@@ -117,8 +132,8 @@ struct SelectShared {
 // weight_of(key) its exponential; `sum` is the sum of all n_all exponentials of the vocabulary. Selects the
 // top_k items, normalises, applies min_p, sorts and runs the reference's sequential top_p and draw loops.
 template <class KeyAt, class IdxAt, class WeightOf>
-__device__ __forceinline__ void select_sort_draw(SelectShared &sh, const SampleArgs &a, int n, int n_all, float sum, KeyAt key_at,
-                                                 IdxAt idx_at, WeightOf weight_of) {
+__device__ __forceinline__ void select_sort_draw(SelectShared &sh, const SampleArgs &a, const StepInfo &st, int n, int n_all,
+                                                 float sum, KeyAt key_at, IdxAt idx_at, WeightOf weight_of) {
     float (&red_f)[SAMPLE_THREADS / WAVE] = sh.red_f;
     int (&red_i)[SAMPLE_THREADS / WAVE] = sh.red_i;
     unsigned (&hist)[4096] = sh.hist;
@@ -271,7 +286,39 @@ __device__ __forceinline__ void select_sort_draw(SelectShared &sh, const SampleA
             }
             __syncthreads();
         }
-    // the reference's sequential loops (src/generate.rs:771-800)
+    // the reference's sequential loops (src/generate.rs:771-800). Up to a wavefront's worth of candidates (the
+    // default top_k of 50) sit in the registers of wavefront 0 and the loops read them lane by lane: the same
+    // additions in the same order, without an LDS round trip per step.
+    if (nc <= WAVE) {
+        if (wave != 0) return;
+        const float p = lane < nc ? cand_p[lane] : 0.0f;
+        const int ci = lane < nc ? cand_i[lane] : 0;
+        auto p_at = [&](int i) { return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(p), i)); };
+        float cumulative = 0.0f;
+        int cutoff = nc;
+        for (int i = 0; i < nc; i++) {
+            cumulative += p_at(i);
+            if (cumulative >= cfg.top_p) {
+                cutoff = i + 1;
+                break;
+            }
+        }
+        float total = 0.0f;
+        for (int i = 0; i < cutoff; i++) total += p_at(i);
+        const float r = st.draw * total;
+        float accum = 0.0f;
+        int at = cutoff > 0 ? cutoff - 1 : -1;
+        for (int i = 0; i < cutoff; i++) {
+            accum += p_at(i);
+            if (accum >= r) {
+                at = i;
+                break;
+            }
+        }
+        const int pick = at >= 0 ? __builtin_amdgcn_readlane(ci, at) : 0;
+        if (lane == 0) deliver_pick(a, st, pick);
+        return;
+    }
     if (tid == 0) {
         float cumulative = 0.0f;
         int cutoff = nc;
@@ -284,7 +331,7 @@ __device__ __forceinline__ void select_sort_draw(SelectShared &sh, const SampleA
         }
         float total = 0.0f;
         for (int i = 0; i < cutoff; i++) total += cand_p[i];
-        const float r = (a.cursor ? a.draws[a.cursor->step - 1] : a.draw) * total;
+        const float r = st.draw * total;
         float accum = 0.0f;
         int pick = cutoff > 0 ? cand_i[cutoff - 1] : 0;
         for (int i = 0; i < cutoff; i++) {
@@ -294,7 +341,7 @@ __device__ __forceinline__ void select_sort_draw(SelectShared &sh, const SampleA
                 break;
             }
         }
-        deliver_pick(a, pick);
+        deliver_pick(a, st, pick);
     }
 }
 
@@ -305,6 +352,7 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_token_kernel(SampleArgs
     const int tid = threadIdx.x, lane = tid & (WAVE - 1), wave = tid / WAVE;
     const int n = a.vocab;
     const hm_sampling_config cfg = a.cfg;
+    const StepInfo st = load_step(a);
 
     // ── pass 1: penalties, then either the greedy pick or temperature + maximum ──
     const bool greedy = cfg.temperature <= 0.0f;
@@ -345,7 +393,7 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_token_kernel(SampleArgs
                     mx = red_f[w];
                     best = red_i[w];
                 }
-            deliver_pick(a, best < 0 ? 0 : best);
+            deliver_pick(a, st, best < 0 ? 0 : best);
         }
         return;
     }
@@ -370,14 +418,14 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_token_kernel(SampleArgs
     for (int w = 0; w < SAMPLE_THREADS / WAVE; w++) sum += red_f[w];
     __syncthreads();
     // exponentials are >= 0, so their bit patterns order like their values
-    select_sort_draw(sh, a, n, n, sum, [&](int i) { return __float_as_uint(a.work[i]); }, [&](int i) { return i; },
+    select_sort_draw(sh, a, st, n, n, sum, [&](int i) { return __float_as_uint(a.work[i]); }, [&](int i) { return i; },
                      [&](unsigned key) { return __uint_as_float(key); });
 }
 
 // ── Small top_k (<= 64) over a large vocabulary: two launches instead of one workgroup's eight passes ──
 // Front: a workgroup per 1024 tokens applies penalties and temperature, takes its maximum and the sum of
-// exponentials relative to it, sorts its tokens (logit descending, token ascending) and keeps the first 64:
-// the vocabulary's top_k are among them. Back: one workgroup combines the maxima and sums (sum over the
+// exponentials relative to it, and keeps the 64 of its tokens that come first by (logit descending, token
+// ascending), in token order: the vocabulary's top_k are among them. Back: one workgroup combines the maxima and sums (sum over the
 // vocabulary = sum_b sum_b * exp(max_b - max), equal to the single pass's up to rounding) and runs the shared
 // selection over the kept tokens; it selects by logit, which orders tokens like their exponentials except
 // where two different logits round to one exponential.
@@ -406,9 +454,10 @@ __host__ __device__ inline FrontOut front_out(float *work, int blocks) {
 }
 
 __global__ __launch_bounds__(SAMPLE_THREADS) void sample_front_kernel(SampleArgs a) {
-    __shared__ float sx[SAMPLE_THREADS];
-    __shared__ int si[SAMPLE_THREADS];
-    __shared__ float red[SAMPLE_THREADS / WAVE];
+    __shared__ unsigned hist[4096];
+    __shared__ float red[SAMPLE_THREADS / WAVE], red_s[SAMPLE_THREADS / WAVE];
+    __shared__ int red_i[SAMPLE_THREADS / WAVE];
+    __shared__ unsigned sel_prefix, sel_need;
     const int tid = threadIdx.x, lane = tid & (WAVE - 1), wave = tid / WAVE;
     const int i = blockIdx.x * SAMPLE_THREADS + tid;
     const bool on = i < a.vocab;
@@ -416,41 +465,83 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_front_kernel(SampleArgs
     const float x = on ? penalised(a.logits[i], a.counts ? a.counts[i] : 0, a.cfg) * inv_temp : -INFINITY;
     float m = wave_max(x);
     if (lane == 0) red[wave] = m;
+    if (tid == 0) {
+        sel_prefix = 0;
+        sel_need = FRONT_KEEP;
+    }
     __syncthreads();
     m = red[0];
     for (int w = 1; w < SAMPLE_THREADS / WAVE; w++) m = fmaxf(m, red[w]);
-    __syncthreads();
     const float e = (on && x > -INFINITY) ? expf(x - m) : 0.f;
     const float ws = wave_sum(e);
-    if (lane == 0) red[wave] = ws;
-    sx[tid] = x;
-    si[tid] = on ? i : 0x7FFFFFFF;
-    __syncthreads();
-    // bitonic sort: logit descending, token ascending among equals
-    for (int k = 2; k <= SAMPLE_THREADS; k <<= 1)
-        for (int j = k >> 1; j > 0; j >>= 1) {
-            const int partner = tid ^ j;
-            if (partner > tid) {
-                const float xa = sx[tid], xb = sx[partner];
-                const int ia = si[tid], ib = si[partner];
-                const bool up = (tid & k) == 0;
-                if (cand_before(xb, ib, xa, ia) == up) {
-                    sx[tid] = xb;
-                    si[tid] = ib;
-                    sx[partner] = xa;
-                    si[partner] = ia;
-                }
-            }
-            __syncthreads();
+    if (lane == 0) red_s[wave] = ws;
+    // The 64 tokens that come first by (logit descending, token ascending), kept in token order: the key of the
+    // 64th by a radix select over the 1024 keys (12 + 10 + 10 bits, one element per thread), then everything
+    // above it and the lowest-numbered of the tokens equal to it. Tokens past the vocabulary carry the key of
+    // -inf and come last among equals.
+    const unsigned key = order_key(x);
+    for (int pass = 0; pass < 3; pass++) {
+        const int shift = pass == 0 ? 20 : pass == 1 ? 10 : 0;
+        const int bits = pass == 0 ? 12 : 10;
+        const int bpt = (1 << bits) / SAMPLE_THREADS;  // bins per thread: 4, 1, 1
+        for (int b = tid; b < (1 << bits); b += SAMPLE_THREADS) hist[b] = 0;
+        __syncthreads();
+        const unsigned prefix = sel_prefix, need = sel_need;
+        const unsigned mask = pass == 0 ? 0u : 0xFFFFFFFFu << (shift + bits);
+        if ((key & mask) == prefix) atomicAdd(&hist[(key >> shift) & ((1u << bits) - 1u)], 1u);
+        __syncthreads();
+        unsigned mine = 0;
+        for (int j = 0; j < bpt; j++) mine += hist[tid * bpt + j];
+        unsigned incl = mine;  // inclusive prefix sum over threads, low bins first
+        for (int off = 1; off < WAVE; off <<= 1) {
+            const unsigned up = __shfl_up(incl, off, WAVE);
+            if (lane >= off) incl += up;
         }
+        if (lane == WAVE - 1) red_i[wave] = (int)incl;
+        __syncthreads();
+        unsigned before = 0, total = 0;
+        for (int w = 0; w < SAMPLE_THREADS / WAVE; w++) {
+            if (w < wave) before += (unsigned)red_i[w];
+            total += (unsigned)red_i[w];
+        }
+        const unsigned above = total - (before + incl);  // elements in higher bins
+        if (above < need && need <= above + mine) {      // exactly one thread
+            unsigned acc = above;
+            for (int j = bpt - 1; j >= 0; j--) {
+                const unsigned h = hist[tid * bpt + j];
+                if (acc + h >= need) {
+                    sel_prefix = prefix | ((unsigned)(tid * bpt + j) << shift);
+                    sel_need = need - acc;
+                    break;
+                }
+                acc += h;
+            }
+        }
+        __syncthreads();
+    }
+    const unsigned T = sel_prefix, need_eq = sel_need;
+    // rank of this thread among the threads whose key equals T (thread order = token order)
+    const bool eq = key == T;
+    const unsigned long long em = __ballot(eq);
+    if (lane == 0) red_i[wave] = __popcll(em);
+    __syncthreads();
+    unsigned eq_rank = __popcll(em & ((1ull << lane) - 1ull));
+    for (int w = 0; w < wave; w++) eq_rank += (unsigned)red_i[w];
+    __syncthreads();
+    const bool keep = key > T || (eq && eq_rank < need_eq);
+    const unsigned long long km = __ballot(keep);
+    if (lane == 0) red_i[wave] = __popcll(km);
+    __syncthreads();
+    unsigned pos = __popcll(km & ((1ull << lane) - 1ull));
+    for (int w = 0; w < wave; w++) pos += (unsigned)red_i[w];
     const FrontOut f = front_out(a.work, gridDim.x);
-    if (tid < FRONT_KEEP) {
-        f.key[(size_t)blockIdx.x * FRONT_KEEP + tid] = order_key(sx[tid]);
-        f.idx[(size_t)blockIdx.x * FRONT_KEEP + tid] = si[tid];
+    if (keep) {  // exactly FRONT_KEEP threads
+        f.key[(size_t)blockIdx.x * FRONT_KEEP + pos] = key;
+        f.idx[(size_t)blockIdx.x * FRONT_KEEP + pos] = on ? i : 0x7FFFFFFF;
     }
     if (tid == 0) {
         float sum = 0.f;
-        for (int w = 0; w < SAMPLE_THREADS / WAVE; w++) sum += red[w];
+        for (int w = 0; w < SAMPLE_THREADS / WAVE; w++) sum += red_s[w];
         f.stat[blockIdx.x * 2] = m;
         f.stat[blockIdx.x * 2 + 1] = sum;
     }
@@ -459,7 +550,23 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_front_kernel(SampleArgs
 __global__ __launch_bounds__(SAMPLE_THREADS) void sample_back_kernel(SampleArgs a, int blocks) {
     __shared__ SelectShared sh;
     const int tid = threadIdx.x, lane = tid & (WAVE - 1), wave = tid / WAVE;
+    const StepInfo st = load_step(a);
     const FrontOut f = front_out(a.work, blocks);
+    // This kernel is one workgroup, and every dependent trip to memory costs it a couple of microseconds: the kept
+    // tokens (up to PRE per thread) are asked for before anything waits on the blocks' statistics.
+    constexpr int PRE = 16;
+    const int n_kept = blocks * FRONT_KEEP;
+    const bool preloaded = n_kept <= PRE * SAMPLE_THREADS;
+    unsigned pk[PRE];
+    int pi[PRE];
+    if (preloaded) {
+#pragma unroll
+        for (int u = 0; u < PRE; u++) {
+            const int j = tid + u * SAMPLE_THREADS;
+            pk[u] = j < n_kept ? f.key[j] : 0u;
+            pi[u] = j < n_kept ? f.idx[j] : 0;
+        }
+    }
     float m = -INFINITY;
     for (int b = tid; b < blocks; b += SAMPLE_THREADS) m = fmaxf(m, f.stat[b * 2]);
     m = wave_max(m);
@@ -479,13 +586,112 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_back_kernel(SampleArgs 
     sum = 0.f;
     for (int w = 0; w < SAMPLE_THREADS / WAVE; w++) sum += sh.red_f[w];
     __syncthreads();
+    auto weight = [&](unsigned key) {
+        const float x = key_value(key);
+        return x > -INFINITY ? expf(x - m) : 0.f;
+    };
+    // The K-th largest of the blocks' maxima is a floor for the K-th largest logit of the vocabulary (K tokens reach
+    // it), so only kept tokens at or above it can be among the top K: usually a hundred or so of the blocks * 64.
+    // With at most 1024 of them the selection is done by rank: every survivor counts the survivors ahead of it in
+    // (logit descending, token ascending), the first K take their rank as their place, and after normalisation and
+    // min_p the same count over (probability descending, token ascending) gives the order the reference's
+    // sequential loops walk. A flat distribution (more survivors) takes the general selection over the full list.
+    // a survivor as one 64-bit number that orders like (logit descending, token ascending): key, then the
+    // token counted down from the largest
+    __shared__ unsigned bkey[SAMPLE_THREADS], tau, fcount;
+    __shared__ unsigned long long fcomp[SAMPLE_MAX_K];
+    const unsigned K = (unsigned)min(a.cfg.top_k, a.vocab);
+    if (preloaded && blocks <= SAMPLE_THREADS && (unsigned)blocks >= K && K >= 1 && K <= (unsigned)WAVE) {
+        bkey[tid] = tid < blocks ? order_key(f.stat[tid * 2]) : 0u;
+        if (tid == 0) fcount = 0;
+        __syncthreads();
+        if (tid < blocks) {
+            const unsigned mine = bkey[tid];
+            unsigned rank = 0;
+#pragma unroll 16
+            for (int c = 0; c < blocks; c++) {  // (unrolled: sixteen LDS reads in flight, not one)
+                const unsigned o = bkey[c];
+                rank += ((o > mine) | ((o == mine) & (c < tid))) ? 1u : 0u;
+            }
+            if (rank == K - 1) tau = mine;
+        }
+        __syncthreads();
+        const unsigned floor_key = tau;
+#pragma unroll
+        for (int u = 0; u < PRE; u++) {
+            const int j = tid + u * SAMPLE_THREADS;
+            if (j < n_kept && pk[u] >= floor_key) {
+                const unsigned at = atomicAdd(&fcount, 1u);
+                if (at < (unsigned)SAMPLE_MAX_K) fcomp[at] = ((unsigned long long)pk[u] << 32) | (unsigned)(0x7FFFFFFF - pi[u]);
+            }
+        }
+        __syncthreads();
+        const int nf = (int)fcount;
+        if (nf <= SAMPLE_MAX_K) {
+            float (&cand_p)[SAMPLE_MAX_K] = sh.cand_p;
+            int (&cand_i)[SAMPLE_MAX_K] = sh.cand_i;
+            if (tid < nf) {
+                const unsigned long long mine = fcomp[tid];
+                const int mi = 0x7FFFFFFF - (int)(unsigned)(mine & 0xFFFFFFFFull);
+                unsigned rank = 0;
+#pragma unroll 16
+                for (int c = 0; c < nf; c++) rank += fcomp[c] > mine ? 1u : 0u;  // (straight-line: sixteen LDS reads in flight)
+                if (rank < K) {  // normalise, min_p (the maximum probability is exp(0) / sum)
+                    float p = weight((unsigned)(mine >> 32)) / sum;
+                    if (a.cfg.min_p > 0.0f && p < a.cfg.min_p * (1.0f / sum)) p = 0.0f;
+                    cand_p[rank] = p;
+                    cand_i[rank] = mi;
+                }
+            }
+            __syncthreads();
+            if (wave != 0) return;
+            // K <= 64 candidates, one per lane: place by (probability descending, token ascending), then the
+            // reference's sequential loops (src/generate.rs:771-800) over the lanes
+            const int nc = (int)K;
+            const float p0 = lane < nc ? cand_p[lane] : -1.0f;
+            const int i0 = lane < nc ? cand_i[lane] : 0x7FFFFFFF;
+            // (lanes past nc hold (-1, largest token): behind every candidate. Constant lane numbers: the
+            // loops below are straight-line code.)
+            int place = 0;
+#pragma unroll
+            for (int c = 0; c < WAVE; c++) {
+                const float pc = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(p0), c));
+                const int ic = __builtin_amdgcn_readlane(i0, c);
+                place += cand_before(pc, ic, p0, i0) ? 1 : 0;
+            }
+            // lane l wants the candidate whose place is l: scatter through LDS (wavefront 0 only; no other
+            // wavefront touches cand_p / cand_i any more)
+            cand_p[SAMPLE_MAX_K / 2 + place] = p0;  // (the candidates' places are 0 .. nc - 1; every other lane writes slot nc)
+            cand_i[SAMPLE_MAX_K / 2 + place] = i0;
+            __builtin_amdgcn_wave_barrier();  // (LDS operations of a wavefront execute in order)
+            const float p = lane < nc ? cand_p[SAMPLE_MAX_K / 2 + lane] : 0.0f;
+            const int ci = cand_i[SAMPLE_MAX_K / 2 + lane];
+            // The reference's three loops add the same probabilities in the same order from zero: cumulative until
+            // top_p is reached, the total of the kept candidates (= that cumulative sum), and the running sum
+            // the draw is compared with. One chain of additions gives all three; lane i keeps the sum after
+            // candidate i. (Lanes past nc add 0.)
+            float chain = 0.0f, upto = 0.0f;
+#pragma unroll
+            for (int i = 0; i < WAVE; i++) {
+                chain += __int_as_float(__builtin_amdgcn_readlane(__float_as_int(p), i));
+                upto = lane == i ? chain : upto;
+            }
+            const unsigned long long live = nc >= WAVE ? ~0ull : ((1ull << nc) - 1ull);
+            const unsigned long long reached = __ballot(upto >= a.cfg.top_p) & live;
+            const int cutoff = reached ? __ffsll((long long)reached) : nc;  // index of the first + 1
+            const float total = cutoff > 0 ? __int_as_float(__builtin_amdgcn_readlane(__float_as_int(upto), cutoff - 1)) : 0.0f;
+            const float r = st.draw * total;
+            const unsigned long long kept = cutoff >= WAVE ? ~0ull : ((1ull << cutoff) - 1ull);
+            const unsigned long long hit = __ballot(upto >= r) & kept;
+            const int at = hit ? __ffsll((long long)hit) - 1 : cutoff - 1;
+            const int pick = at >= 0 ? __builtin_amdgcn_readlane(ci, at) : 0;
+            if (lane == 0) deliver_pick(a, st, pick);
+            return;
+        }
+    }
     // padding entries (tokens past the vocabulary) carry the key of -inf and the largest token number: they sort
     // behind every real token and are never among the vocabulary's top_k
-    select_sort_draw(sh, a, blocks * FRONT_KEEP, a.vocab, sum, [&](int j) { return f.key[j]; }, [&](int j) { return f.idx[j]; },
-                     [&](unsigned key) {
-                         const float x = key_value(key);
-                         return x > -INFINITY ? expf(x - m) : 0.f;
-                     });
+    select_sort_draw(sh, a, st, n_kept, a.vocab, sum, [&](int j) { return f.key[j]; }, [&](int j) { return f.idx[j]; }, weight);
 }
 
 __global__ void count_tokens_kernel(const uint32_t *__restrict__ ids, int n_ids, int *__restrict__ counts, int vocab) {

@@ -75,7 +75,7 @@ def test_two_launch_sampler_with_ties_and_masked_logits(ctx, vocab, top_k):
     """The front / back pair (top_k <= 64, vocabulary >= 4096) where its selection is hardest: logits on a
     coarse grid, so that the top_k-th value is shared by many tokens spread over the front workgroups (the
     lowest token numbers must win, as in the oracle's stable order), a run of -inf logits, a last block that
-    is not full, and top_k at the limit."""
+    is not full, top_k at the limit, and a plateau of equal maxima wider than the back launch's short list."""
     gen = np.random.default_rng(vocab * 131 + top_k)
     cfg = Cfg(temperature=0.9, top_k=top_k, top_p=0.98, min_p=0.0, repetition_penalty=1.0)
     compared = skipped = 0
@@ -84,6 +84,10 @@ def test_two_launch_sampler_with_ties_and_masked_logits(ctx, vocab, top_k):
         logits[gen.integers(0, vocab, vocab // 10)] = -np.inf
         if trial % 2:
             logits[-3:] = logits.max()            # ties at the very end of the partial block
+        if trial in (2, 5):
+            # a plateau: a third of the vocabulary shares the maximum, so more tokens reach the back launch's
+            # floor than its short list holds and the selection walks the full list in token order
+            logits[gen.integers(0, vocab, vocab // 3)] = logits.max()
         d = ctx.to_device(logits)
         a, b = pyoracle.Rng(50 + trial), runtime.Rng(50 + trial)
         for _ in range(4):
