@@ -298,6 +298,15 @@ __device__ __forceinline__ int k_off(int key, int chunk) {
     return key * 128 + ((chunk ^ (key & 7) ^ ((key >> 3) & 7)) << 4);
 }
 
+// V tile: the transposing reads of a group of 16 lanes take 32 contiguous bytes (two chunks) from each of four
+// neighbouring rows, and a pass of the LDS serves two such groups: the swizzle moves chunk PAIRS, by the row's
+// low three bits, so that eight neighbouring rows land on eight different bank groups.
+template <int HD>
+__device__ __forceinline__ int v_off(int key, int chunk) {
+    if (HD == 128) return key * 256 + (((((chunk >> 1) ^ (key & 7)) << 1) | (chunk & 1)) << 4);
+    return k_off<HD>(key, chunk);
+}
+
 extern __shared__ __attribute__((aligned(16))) char at_lds[];
 
 // 16 query rows per wavefront (v_mfma_f32_16x16x32_bf16) and eight wavefronts a workgroup: 8 / KS blocks of 16
@@ -381,7 +390,8 @@ __global__ __launch_bounds__(A8_THREADS) void prefill_attn16_kernel(PrefillAttnA
 
     // This lane's part of a tile load: row dma_row of the tile, the chunk that belongs in slot dma_slot.
     const int dma_row = wave * ROWS_PER_DMA + lane / CH, dma_slot = lane % CH;
-    const int dma_chunk = (k_off<HD>(dma_row, dma_slot) - dma_row * HD * 2) >> 4;  // the swizzle is an involution
+    const int dma_chunk = (k_off<HD>(dma_row, dma_slot) - dma_row * HD * 2) >> 4;  // the swizzles are involutions
+    const int dma_chunk_v = (v_off<HD>(dma_row, dma_slot) - dma_row * HD * 2) >> 4;
     const int wave_dst = __builtin_amdgcn_readfirstlane(wave * 1024);
     auto request_round = [&](int r) {
         if (wave >= DMA_WAVES) return;
@@ -390,7 +400,7 @@ __global__ __launch_bounds__(A8_THREADS) void prefill_attn16_kernel(PrefillAttnA
         for (int u = 0; u < KS; u++) {
             const int row = min((r * KS + u) * A8_KEYS + dma_row, kv_total - 1);
             dma16_lds(kc + (size_t)row * HD + dma_chunk * 8, base + u * 2 * TILE);
-            dma16_lds(vc + (size_t)row * HD + dma_chunk * 8, base + u * 2 * TILE + TILE);
+            dma16_lds(vc + (size_t)row * HD + dma_chunk_v * 8, base + u * 2 * TILE + TILE);
         }
     };
     // this lane's query (rows past the end repeat the last one and are not stored): dims 32 ks + 8 c4 .. + 7.
@@ -497,9 +507,9 @@ __global__ __launch_bounds__(A8_THREADS) void prefill_attn16_kernel(PrefillAttnA
         for (int db = 0; db < DB; db++) {
             const int chunk = 2 * db + (v_sub >> 1), within = (v_sub & 1) * 8;
             const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                (s16x4 __attribute__((address_space(3))) *)(v_lds + k_off<HD>(v_key, chunk) + within));
+                (s16x4 __attribute__((address_space(3))) *)(v_lds + v_off<HD>(v_key, chunk) + within));
             const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                (s16x4 __attribute__((address_space(3))) *)(v_lds + k_off<HD>(16 + v_key, chunk) + within));
+                (s16x4 __attribute__((address_space(3))) *)(v_lds + v_off<HD>(16 + v_key, chunk) + within));
             struct Pair { s16x4 lo, hi; } pr{lo, hi};
             const bf16x8 vf = __builtin_bit_cast(bf16x8, pr);
 #pragma unroll
