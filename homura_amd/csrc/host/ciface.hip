@@ -323,18 +323,12 @@ int run_quant_mm(void **a, const KernelInfo &ki) {
     TRY(seq_ok(b.ctx, x.sizes[1], "QuantMM kernel"));
     const int S = (int)x.sizes[1];
     const bool kq = ki.dtype == HM_DTYPE_Q4_K || ki.dtype == HM_DTYPE_Q6_K;
-    if (S >= GEMM_MIN_ROWS && ki.K % 64 == 0 && (!kq || ki.K % 256 == 0)) {
-        // A prompt: the rows (through the Q8_K quantisation first where the reference's kernel quantises its
-        // activations, src/graph_builder/emit_quant.rs:422-466) and the dequantised matrix as three bf16 pieces
-        // each, multiplied on the matrix cores. Falls through to the row blocks when the workspace is too small.
-        Scratch s(b.ctx);
-        uint16_t *xs = s.take<uint16_t>((size_t)S * 3 * ki.K), *ws = s.take<uint16_t>((size_t)ki.N * 3 * ki.K);
-        if (xs && ws) {
-            TRY(homura::split_rows_launch(b.ctx, x.as<float>(), xs, 3, (size_t)S, ki.K, kq));
-            TRY(homura::dequant_split_launch(b.ctx, ki.dtype, w.as<uint8_t>(), ki.N, ki.K, ws));
-            return homura::gemm_split_split_nk(b.ctx, xs, ws, out.as<float>(), S, ki.K, ki.N);
-        }
-    }
+    // A prompt goes to the matrix cores (hm_gemm_f32_quant_nk: Q8_K rows x int8 digit planes for the K-quants,
+    // whose kernel quantises its activations, src/graph_builder/emit_quant.rs:422-466; three-piece rows x block
+    // integers with block scales for Q8_0 / Q4_0), when the rows fit the workspace beside a slab of the matrix.
+    if (S >= GEMM_MIN_ROWS && ki.K % 64 == 0 && (!kq || ki.K % 256 == 0) &&
+        ((size_t)S + 160) * ki.K * 8 <= b.ctx->workspace_bytes)
+        return hm_gemm_f32_quant_nk(b.ctx, x.as<float>(), w.as<uint8_t>(), ki.dtype, out.as<float>(), S, ki.K, ki.N);
     for (int r = 0; r < S; r += 8) {
         const float *xr = x.as<float>() + (size_t)r * ki.K;
         float *outr = out.as<float>() + (size_t)r * ki.N;
