@@ -47,7 +47,7 @@ constexpr int CT = 256;     // communicating threads
 constexpr int SPIN_MAX = 1 << 20;
 constexpr int MAX_LAYERS = 64;
 
-template <int HIDDEN_, int H_, int KVH_, int HD_, int INTER_, int NWG_, int NR_ = 4>
+template <int HIDDEN_, int H_, int KVH_, int HD_, int INTER_, int NWG_, int NR_ = 4, int XR_ = 0>
 struct Geo {
     static constexpr int HIDDEN = HIDDEN_, H = H_, KVH = KVH_, HD = HD_, INTER = INTER_, NWG = NWG_;
     static constexpr int G = H / KVH, QD = H * HD, KVD = KVH * HD, NQKV = QD + 2 * KVD;
@@ -67,7 +67,8 @@ struct Geo {
     static constexpr int APW = INTER / NWG;                    // SiLU*up values per workgroup
     static constexpr int NR = NR_;                             // row rounds a wavefront keeps in registers
     static constexpr int LPR = HD / 8, RPI = WAVE / LPR;       // lanes per cache row, rows per load
-    static constexpr int MAX_KV = SPH * NR * NCW * RPI;
+    static constexpr int XR = XR_;                             // further rounds, streamed inside the attention phase
+    static constexpr int MAX_KV = SPH * (NR + XR) * NCW * RPI;
     static constexpr int FPW = QD / NWG;                       // folded attention outputs per workgroup
     static constexpr int PART = G * HD + 2 * G;                // one split's partial: o[G][HD], (m, l)[G]
     static constexpr int NJ = HIDDEN / CT;                     // hidden elements per communicating thread
@@ -956,19 +957,35 @@ __device__ __forceinline__ void compute_role(const FusedDecodeArgs &a, Lds<GE> &
     auto load_wq = [&](const FusedLayerPtrs &lp, int r0, int r1) {
         s.wq.load(lp.wqkv, lp.sqkv, [&](int r) { return GE::qkv_row(sp.kh, sp.split * GE::RQ + cw * GE::RQW + r); }, r0, r1, lane);
     };
+    // Element offset of this lane's part of round `round` of the split. With streamed rounds (XR > 0) the
+    // lane's row is made opaque at every use: the offsets of all rounds, kept across the layer loop as loop
+    // invariants, would take the registers the slices need (and a spilled one comes back behind every
+    // outstanding weight request).
+    auto kv_off = [&](int round) -> size_t {
+        int r0 = cw * RPI + sub;
+        if constexpr (GE::XR > 0) asm volatile("" : "+v"(r0));
+        const int rl = round * NCW * RPI + r0;
+        const int row = rl < sp.cached ? sp.n0 + rl : 0;  // rows outside the split re-read a valid row
+        if constexpr (GE::XR > 0) return (size_t)(((uint32_t)sp.kh * (uint32_t)a.max_len + (uint32_t)row) * HD + dl * 8);  // < 2^32: checked by the host
+        else return ((size_t)sp.kh * a.max_len + row) * HD + dl * 8;
+    };
     auto load_kv = [&](const FusedLayerPtrs &lp, int i0, int i1) {
 #pragma unroll
         for (int i = 0; i < NR; i++) {
             if (i < i0 || i >= i1) continue;
-            const int rl = (i * NCW + cw) * RPI + sub;
-            const int row = rl < sp.cached ? sp.n0 + rl : 0;  // rows outside the split re-read a valid row
-            const size_t off = ((size_t)sp.kh * a.max_len + row) * HD + dl * 8;
+            const size_t off = kv_off(i);
             s.kr[i] = ld128_global_stream(lp.kcache + off);
             s.vr[i] = ld128_global_stream(lp.vcache + off);
         }
     };
+    // (the lane index is made opaque for the same reason as in kv_off: per-lane row offsets are recomputed, not held)
+    auto opaque_lane = [&]() {
+        int ln = lane;
+        if constexpr (GE::XR > 0) asm volatile("" : "+v"(ln));
+        return ln;
+    };
     auto load_wo = [&](const FusedLayerPtrs &lp) {
-        s.wo.load(lp.wo, lp.so, GE::partial_row(sp.split, cw * GE::RPW), sp.kh * GE::KSO, lane);
+        s.wo.load(lp.wo, lp.so, GE::partial_row(sp.split, cw * GE::RPW), sp.kh * GE::KSO, opaque_lane());
     };
     // bf16 keeps gate and up rows interleaved (g0, u0, g1, u1, ...); the quantised formats keep the run as
     // uploaded, all gate rows and then all up rows, so local row r = 2 p + (0 gate | 1 up) of pair p.
@@ -981,7 +998,7 @@ __device__ __forceinline__ void compute_role(const FusedDecodeArgs &a, Lds<GE> &
         }, r0, r1, lane);
     };
     auto load_wd = [&](const FusedLayerPtrs &lp) {
-        s.wd.load(lp.wd, lp.sd, GE::partial_row(sp.split, cw * GE::RPW), sp.kh * GE::KSD, lane);
+        s.wd.load(lp.wd, lp.sd, GE::partial_row(sp.split, cw * GE::RPW), sp.kh * GE::KSD, opaque_lane());
     };
 
     constexpr int KV_CUT = NR / 2, WG_CUT = 2 * GE::RGW / 3;
@@ -1047,14 +1064,13 @@ __device__ __forceinline__ void compute_role(const FusedDecodeArgs &a, Lds<GE> &
             constexpr int PR = NR > 4 ? 2 : NR, NPASS = NR / PR;
             static_assert(NR % PR == 0, "row rounds are taken in equal passes");
             float m[G], lsum[G], acc[G][8];
-#pragma unroll
-            for (int ps = 0; ps < NPASS; ps++) {
-                const int i0 = ps * PR;
-                const bool last = ps == NPASS - 1;
+            // One pass: rounds i0 .. i0 + PR - 1 of the split, their rows handed over by kk(i) / vv(i).
+            auto attn_pass = [&](auto first_tag, auto kk, auto vv, const int i0, const bool last) __attribute__((always_inline)) {
+                constexpr bool FIRST = decltype(first_tag)::value;
                 // slot PR is the new row (last pass only; elsewhere it is dead and multiplies zeros)
                 float kf[PR + 1][8];
 #pragma unroll
-                for (int i = 0; i < PR; i++) unpack8f(s.kr[i0 + i], kf[i]);
+                for (int i = 0; i < PR; i++) unpack8f(kk(i), kf[i]);
                 if (last) lds_x8(sm.knew, dl * 8, kf[PR]);
                 else {
 #pragma unroll
@@ -1110,7 +1126,7 @@ __device__ __forceinline__ void compute_role(const FusedDecodeArgs &a, Lds<GE> &
                 float alpha[G];
 #pragma unroll
                 for (int g = 0; g < G; g++) {
-                    if (ps == 0) {
+                    if (FIRST) {
                         m[g] = mp[g];
                         alpha[g] = 0.f;
                         lsum[g] = 0.f;
@@ -1146,7 +1162,7 @@ __device__ __forceinline__ void compute_role(const FusedDecodeArgs &a, Lds<GE> &
                 }
                 float vf[PR + 1][8];
 #pragma unroll
-                for (int i = 0; i < PR; i++) unpack8f(s.vr[i0 + i], vf[i]);
+                for (int i = 0; i < PR; i++) unpack8f(vv(i), vf[i]);
                 if (last) lds_x8(sm.vnew, dl * 8, vf[PR]);
                 else {
 #pragma unroll
@@ -1155,7 +1171,7 @@ __device__ __forceinline__ void compute_role(const FusedDecodeArgs &a, Lds<GE> &
 #pragma unroll
                 for (int g = 0; g < G; g++)
 #pragma unroll
-                    for (int e = 0; e < 8; e++) acc[g][e] = ps == 0 ? 0.f : acc[g][e] * alpha[g];
+                    for (int e = 0; e < 8; e++) acc[g][e] = FIRST ? 0.f : acc[g][e] * alpha[g];
 #pragma unroll
                 for (int i = 0; i <= PR; i++) {
 #pragma unroll
@@ -1163,6 +1179,46 @@ __device__ __forceinline__ void compute_role(const FusedDecodeArgs &a, Lds<GE> &
                         const float p = (i < PR || sub == 0) ? pr[g][i] : 0.f;  // the new row: one row group only
 #pragma unroll
                         for (int e = 0; e < 8; e++) acc[g][e] = fmaf(p, vf[i][e], acc[g][e]);
+                    }
+                }
+            };
+            // Rounds past the held ones (XR > 0: caches longer than the registers hold) are streamed inside
+            // the phase, two sets of PR rounds in turn: one is multiplied while the other is in flight.
+            int npx = 0;
+            if constexpr (GE::XR > 0) {
+                const int over = sp.cached - NR * NCW * RPI;
+                npx = over > 0 ? (over + PR * NCW * RPI - 1) / (PR * NCW * RPI) : 0;
+            }
+            u32x4 kxa[PR], vxa[PR], kxb[PR], vxb[PR];
+            auto load_x = [&](u32x4 (&kx)[PR], u32x4 (&vx)[PR], const int r0) __attribute__((always_inline)) {
+                const uint16_t *kc = sm.lp[l].kcache, *vc = sm.lp[l].vcache;
+#pragma unroll
+                for (int i = 0; i < PR; i++) {
+                    const size_t off = kv_off(r0 + i);
+                    kx[i] = ld128_global_stream(kc + off);
+                    vx[i] = ld128_global_stream(vc + off);
+                }
+            };
+#pragma unroll
+            for (int ps = 0; ps < NPASS; ps++) {
+                const int i0 = ps * PR;
+                auto kk = [&](int i) { return s.kr[i0 + i]; };
+                auto vv = [&](int i) { return s.vr[i0 + i]; };
+                const bool last = ps == NPASS - 1 && npx == 0;
+                // the first streamed set goes out ahead of the last held pass, into registers of earlier rounds
+                if constexpr (GE::XR > 0) {
+                    if (ps == NPASS - 1 && npx > 0) load_x(kxa, vxa, NR);
+                }
+                if (ps == 0) attn_pass(std::true_type{}, kk, vv, i0, last);
+                else attn_pass(std::false_type{}, kk, vv, i0, last);
+            }
+            if constexpr (GE::XR > 0) {
+                for (int x = 0; x < npx; x += 2) {
+                    if (x + 1 < npx) load_x(kxb, vxb, NR + (x + 1) * PR);
+                    attn_pass(std::false_type{}, [&](int i) { return kxa[i]; }, [&](int i) { return vxa[i]; }, NR + x * PR, x == npx - 1);
+                    if (x + 1 < npx) {
+                        if (x + 2 < npx) load_x(kxa, vxa, NR + (x + 2) * PR);
+                        attn_pass(std::false_type{}, [&](int i) { return kxb[i]; }, [&](int i) { return vxb[i]; }, NR + (x + 1) * PR, x + 1 == npx - 1);
                     }
                 }
             }
@@ -1835,6 +1891,12 @@ using GeoSmallQShort = Geo<1024, 8, 4, 128, 1024, 64, 3>;
 using GeoQwen3_0p6bLong = Geo<1024, 16, 8, 128, 3072, 256, 8>;
 using GeoSmallLong = Geo<512, 4, 2, 128, 1024, 64, 8>;
 using GeoSmallQLong = Geo<1024, 8, 4, 128, 1024, 64, 8>;
+// Eight row rounds held and up to 56 more streamed inside the attention phase: 32768 live rows. Every further
+// 1000 rows cost the Qwen3-0.6B shape about 26 us a token; below 4096 rows these instances are 1-2 % slower than
+// the ones above (per-lane offsets are recomputed in every layer instead of held), so they come last.
+using GeoQwen3_0p6bStream = Geo<1024, 16, 8, 128, 3072, 256, 8, 56>;
+using GeoSmallStream = Geo<512, 4, 2, 128, 1024, 64, 8, 56>;
+using GeoSmallQStream = Geo<1024, 8, 4, 128, 1024, 64, 8, 56>;
 
 template <class GE>
 bool shape_is(const FusedShape &s) {
@@ -1862,12 +1924,15 @@ const Instance *find_instance(const FusedShape &s, int live_rows = 1) {
         instance<GeoQwen3_0p6bShort, FUSED_WF_K8>(), instance<GeoSmallQShort, FUSED_WF_K8>(),
         instance<GeoQwen3_0p6b, FUSED_WF_K8>(), instance<GeoSmallQ, FUSED_WF_K8>(),
         instance<GeoQwen3_0p6bLong, FUSED_WF_K8>(), instance<GeoSmallQLong, FUSED_WF_K8>(),
+        instance<GeoQwen3_0p6bStream, FUSED_WF_K8>(), instance<GeoSmallQStream, FUSED_WF_K8>(),
         instance<GeoQwen3_0p6bShort, FUSED_WF_BF16>(), instance<GeoQwen3_0p6bShort, FUSED_WF_Q8_0>(), instance<GeoQwen3_0p6bShort, FUSED_WF_Q4_0>(),
         instance<GeoSmallShort, FUSED_WF_BF16>(),      instance<GeoSmallQShort, FUSED_WF_Q8_0>(),     instance<GeoSmallQShort, FUSED_WF_Q4_0>(),
         instance<GeoQwen3_0p6b, FUSED_WF_BF16>(), instance<GeoQwen3_0p6b, FUSED_WF_Q8_0>(), instance<GeoQwen3_0p6b, FUSED_WF_Q4_0>(),
         instance<GeoSmall, FUSED_WF_BF16>(),      instance<GeoSmallQ, FUSED_WF_Q8_0>(),     instance<GeoSmallQ, FUSED_WF_Q4_0>(),
         instance<GeoQwen3_0p6bLong, FUSED_WF_BF16>(), instance<GeoQwen3_0p6bLong, FUSED_WF_Q8_0>(), instance<GeoQwen3_0p6bLong, FUSED_WF_Q4_0>(),
         instance<GeoSmallLong, FUSED_WF_BF16>(),      instance<GeoSmallQLong, FUSED_WF_Q8_0>(),     instance<GeoSmallQLong, FUSED_WF_Q4_0>(),
+        instance<GeoQwen3_0p6bStream, FUSED_WF_BF16>(), instance<GeoQwen3_0p6bStream, FUSED_WF_Q8_0>(), instance<GeoQwen3_0p6bStream, FUSED_WF_Q4_0>(),
+        instance<GeoSmallStream, FUSED_WF_BF16>(),      instance<GeoSmallQStream, FUSED_WF_Q8_0>(),     instance<GeoSmallQStream, FUSED_WF_Q4_0>(),
     };
     const Instance *most = nullptr;
     for (const Instance &i : table) {
@@ -1909,7 +1974,12 @@ bool decode_fused_supported(const hm_ctx *ctx, const FusedShape &s, int n_layers
         *why = "no kernel instance for this shape and weight format";
         return false;
     }
-    (void)max_seq_len;  // any cache length: what is limited is the number of live rows (decode_fused_max_kv)
+    // any cache length: what is limited is the number of live rows (decode_fused_max_kv); the instances that
+    // stream cache rows address a layer's cache with 32-bit element offsets
+    if ((uint64_t)s.kv_heads * (uint64_t)(max_seq_len < 0 ? 0 : max_seq_len) * s.head_dim >= (1ull << 32)) {
+        *why = "a layer's KV cache holds 2^32 elements or more";
+        return false;
+    }
     if (ctx->num_cus < i->nwg) {
         *why = "fewer compute units than resident workgroups";
         return false;

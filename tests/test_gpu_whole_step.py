@@ -261,22 +261,67 @@ def test_unserved_shapes_keep_the_per_projection_path(ctx):
     gm.close()
 
 
+@pytest.fixture(scope="module")
+def long_small(ctx):
+    cfg = dataclasses.replace(synth_model.SMALL_WS, max_position_embeddings=32768)
+    weights = synth_model.synth_weights(cfg, 4141)
+    L = 32768
+    gm = synth_model.build_model(ctx, cfg, weights, L)
+    plain = synth_model.build_model(ctx, cfg, weights, L)
+    plain.set_whole_step(False)
+    om = mf.build_oracle_model(cfg, weights, L)
+    yield cfg, gm, plain, om
+    gm.close()
+    plain.close()
+
+
+@pytest.mark.parametrize("rows", [4094, 4600, 5000, 6200, 9000, 12287, 20000, 32754])
+def test_rows_streamed_inside_the_attention_phase(long_small, rows):
+    """More than 4096 live rows: a split's rows beyond the eight rounds held in registers are loaded inside
+    the attention phase, two rounds at a time in two alternating register sets. The lengths give a split one
+    streamed row (4097 live rows: 129 a split), a partly filled round, an odd and an even number of
+    passes, a split boundary that moves while tokens are appended, and the last round the instance
+    serves (32768 rows). Logits against the oracle, tokens against the per-projection path."""
+    cfg, gm, plain, om = long_small
+    kv = synth_model.synth_kv(cfg, 900 + rows, rows)
+    n = 10
+    ids = synth.token_ids(901 + rows, n, cfg.vocab_size)
+    for m in (gm, plain):
+        m.set_prefill_min(0)
+        m.init_kv_cache(kv, rows)
+    gm.set_whole_step(True)
+    mf.oracle_init_kv(om, kv)
+    say(f"streamed rounds: {rows} cached rows")
+    got = gm.run_kv(ids)
+    gm.whole_step_status()
+    assert gm.whole_step() and gm.launches_per_step() == 1
+    want = np.concatenate([om.run_kv(ids[i:i + 1]) for i in range(n)])
+    for i in range(n):
+        assert mf.rel_err(got[i], want[i]) < 1e-2, f"position {rows + i}"
+    ref = plain.run_kv(ids)
+    assert mf.rel_err(got, ref) < 1e-2
+    a, b = gm.generate_greedy(ids[:1], 4), plain.generate_greedy(ids[:1], 4)   # 32754: up to the last row of the cache
+    assert np.array_equal(a, b)
+    gm.whole_step_status()
+    assert gm.kv_cache_len() == rows + n + 4
+
+
 def test_cache_longer_than_the_kernel_serves_changes_over_and_back(ctx):
     """The whole-step launch holds a split's cache rows in registers: an instance with three row rounds serves
-    1536 live rows of this shape, one with four 2048, one with eight 4096. A model with a longer cache starts
-    on the first, takes the next from the step whose live rows exceed it, one launch per projection beyond
-    4096, and comes back after a cache reset; the steps on either side of each change give the oracle's
-    logits and the per-projection path's tokens."""
-    cfg = dataclasses.replace(synth_model.SMALL_WS, max_position_embeddings=8192)
+    1536 live rows of this shape, one with four 2048, one with eight 4096 and, streaming further rounds inside
+    its attention phase, 32768. A model with a longer cache starts on the first, takes the next from the step
+    whose live rows exceed it, one launch per projection beyond 32768, and comes back after a cache reset; the
+    steps on either side of each change give the oracle's logits and the per-projection path's tokens."""
+    cfg = dataclasses.replace(synth_model.SMALL_WS, max_position_embeddings=65536)
     weights = synth_model.synth_weights(cfg, 31)
-    L = 4200
+    L = 32900
     gm = synth_model.build_model(ctx, cfg, weights, L)
     plain = synth_model.build_model(ctx, cfg, weights, L)
     plain.set_whole_step(False)
     om = mf.build_oracle_model(cfg, weights, L)
     assert gm.whole_step_available() and gm.whole_step() and gm.launches_per_step() == 1
     ids = synth.token_ids(33, 14, cfg.vocab_size)
-    for rows, still_whole in ((1528, True), (2040, True), (4088, False)):
+    for rows, still_whole in ((1528, True), (2040, True), (4088, True), (32760, False)):
         kv = synth_model.synth_kv(cfg, 32 + rows, rows)
         for m in (gm, plain):
             m.set_prefill_min(0)
