@@ -957,13 +957,14 @@ __device__ __forceinline__ void compute_role(const FusedDecodeArgs &a, Lds<GE> &
     auto load_wq = [&](const FusedLayerPtrs &lp, int r0, int r1) {
         s.wq.load(lp.wqkv, lp.sqkv, [&](int r) { return GE::qkv_row(sp.kh, sp.split * GE::RQ + cw * GE::RQW + r); }, r0, r1, lane);
     };
+    constexpr bool RECOMPUTE = GE::XR > 0 || (WF == FUSED_WF_K8 && NR > 4);
     // Element offset of this lane's part of round `round` of the split. With streamed rounds (XR > 0) the
     // lane's row is made opaque at every use: the offsets of all rounds, kept across the layer loop as loop
     // invariants, would take the registers the slices need (and a spilled one comes back behind every
     // outstanding weight request).
     auto kv_off = [&](int round) -> size_t {
         int r0 = cw * RPI + sub;
-        if constexpr (GE::XR > 0) asm volatile("" : "+v"(r0));
+        if constexpr (RECOMPUTE) asm volatile("" : "+v"(r0));
         const int rl = round * NCW * RPI + r0;
         const int row = rl < sp.cached ? sp.n0 + rl : 0;  // rows outside the split re-read a valid row
         if constexpr (GE::XR > 0) return (size_t)(((uint32_t)sp.kh * (uint32_t)a.max_len + (uint32_t)row) * HD + dl * 8);  // < 2^32: checked by the host
@@ -981,7 +982,7 @@ __device__ __forceinline__ void compute_role(const FusedDecodeArgs &a, Lds<GE> &
     // (the lane index is made opaque for the same reason as in kv_off: per-lane row offsets are recomputed, not held)
     auto opaque_lane = [&]() {
         int ln = lane;
-        if constexpr (GE::XR > 0) asm volatile("" : "+v"(ln));
+        if constexpr (RECOMPUTE) asm volatile("" : "+v"(ln));
         return ln;
     };
     auto load_wo = [&](const FusedLayerPtrs &lp) {
