@@ -416,6 +416,157 @@ bool try_oneshot(hm_ctx *ctx, const GemvArgs &a, int epi, int *rc) {
     return false;
 }
 
+// Rows cut across the wavefronts of a workgroup. With whole rows per wavefront a matrix of a few thousand rows
+// gives a few hundred wavefronts, each walking its rows with a handful of loads in flight (the down projection
+// of a 1.5B model, 8960 -> 1536: 22 us); and a matrix that one wave of loads covers still leaves every
+// wavefront's requests queued behind one another. Here a workgroup owns R rows and its four wavefronts take K
+// in interleaved 512-wide chunks, NC a wavefront, everything requested at once (the activation pieces first:
+// loads return in issue order); the four partial sums of a row meet in LDS and are added in wavefront order.
+// PRO: residual add and RMSNorm of the activation row (reference src/hf/emitter.rs:787,
+// src/graph_builder/emit_linalg.rs:7-26) on the pieces in registers - the wavefronts' chunks cover the row
+// exactly once, so their sums of squares add up to the row's. Nothing is staged in LDS.
+template <int R, int NC, bool PRO>
+__global__ __launch_bounds__(GEMV_THREADS) void gemv_bf16_nk_splitk_kernel(GemvArgs a, int epi) {
+    __shared__ float part[GEMV_WAVES][R];
+    __shared__ float red[GEMV_WAVES];
+    const int K = a.K, N = a.N;
+    const int lane = threadIdx.x & (WAVE - 1);
+    const int wave = threadIdx.x / WAVE;
+    const int row0 = blockIdx.x * R;
+    const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
+    f32x4 x0[NC], x1[NC], p0[PRO ? NC : 1], p1[PRO ? NC : 1], n0[PRO ? NC : 1], n1[PRO ? NC : 1];
+    u32x4 wv[NC][R];
+#pragma unroll
+    for (int c = 0; c < NC; c++) {
+        const int k = ((c * GEMV_WAVES + wave) * WAVE + lane) * 8;
+        const bool ok = k < K;
+        x0[c] = ok ? *reinterpret_cast<const f32x4 *>(a.x + k) : zero;
+        x1[c] = ok ? *reinterpret_cast<const f32x4 *>(a.x + k + 4) : zero;
+        if constexpr (PRO) {
+            p0[c] = (ok && a.prologue_residual) ? *reinterpret_cast<const f32x4 *>(a.prologue_residual + k) : zero;
+            p1[c] = (ok && a.prologue_residual) ? *reinterpret_cast<const f32x4 *>(a.prologue_residual + k + 4) : zero;
+            n0[c] = (ok && a.norm_w) ? *reinterpret_cast<const f32x4 *>(a.norm_w + k) : zero;
+            n1[c] = (ok && a.norm_w) ? *reinterpret_cast<const f32x4 *>(a.norm_w + k + 4) : zero;
+        }
+    }
+#pragma unroll
+    for (int c = 0; c < NC; c++) {
+        const int k = ((c * GEMV_WAVES + wave) * WAVE + lane) * 8;
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            const int row = row0 + r < N ? row0 + r : N - 1;  // clamp: stays inside the matrix
+            wv[c][r] = k < K ? ld128_stream(static_cast<const uint16_t *>(a.w) + (size_t)row * K + k)
+                             : u32x4{0u, 0u, 0u, 0u};
+        }
+    }
+    if constexpr (PRO) {
+        float ss = 0.f;
+#pragma unroll
+        for (int c = 0; c < NC; c++) {
+            if (a.prologue_residual) {
+                x0[c] = x0[c] + p0[c];
+                x1[c] = x1[c] + p1[c];
+            }
+            ss += x0[c].x * x0[c].x + x0[c].y * x0[c].y + x0[c].z * x0[c].z + x0[c].w * x0[c].w;
+            ss += x1[c].x * x1[c].x + x1[c].y * x1[c].y + x1[c].z * x1[c].z + x1[c].w * x1[c].w;
+            const int k = ((c * GEMV_WAVES + wave) * WAVE + lane) * 8;
+            if (blockIdx.x == 0 && a.resid_out && k < K) {
+                *reinterpret_cast<f32x4 *>(a.resid_out + k) = x0[c];
+                *reinterpret_cast<f32x4 *>(a.resid_out + k + 4) = x1[c];
+            }
+        }
+        if (a.norm_w) {
+            ss = wave_sum(ss);
+            if (lane == 0) red[wave] = ss;
+            __syncthreads();
+            float tot = 0.f;
+#pragma unroll
+            for (int w = 0; w < GEMV_WAVES; w++) tot += red[w];
+            const float inv = 1.0f / sqrtf(tot / (float)K + a.eps);
+#pragma unroll
+            for (int c = 0; c < NC; c++) {
+                x0[c] = (x0[c] * inv) * n0[c];
+                x1[c] = (x1[c] * inv) * n1[c];
+            }
+        }
+    }
+    float acc[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) acc[r] = 0.f;
+#pragma unroll
+    for (int c = 0; c < NC; c++) {
+        const float xv[8] = {x0[c].x, x0[c].y, x0[c].z, x0[c].w, x1[c].x, x1[c].y, x1[c].z, x1[c].w};
+#pragma unroll
+        for (int r = 0; r < R; r++) acc[r] = dot8(wv[c][r], xv, acc[r]);
+    }
+#pragma unroll
+    for (int r = 0; r < R; r++) acc[r] = wave_sum(acc[r]);
+    if (lane == 0) {
+#pragma unroll
+        for (int r = 0; r < R; r++) part[wave][r] = acc[r];
+    }
+    __syncthreads();
+    const int t = threadIdx.x;
+    auto row_sum = [&](int r) {
+        float v = part[0][r];
+#pragma unroll
+        for (int w = 1; w < GEMV_WAVES; w++) v += part[w][r];
+        return v;
+    };
+    if (epi == GEMV_EPI_SILU_MUL_PAIRS) {
+        // rows come in (gate_i, up_i) pairs; output index = row / 2 (reference src/hf/emitter.rs:794-799)
+        if (R % 2 == 0 && t < R / 2 && row0 + 2 * t < N) {
+            const float gte = row_sum(2 * t), up = row_sum(2 * t + 1);
+            a.out[(row0 + 2 * t) / 2] = (gte / (1.0f + expf(-gte))) * up;
+        }
+    } else if (t < R && row0 + t < N) {
+        float v = row_sum(t);
+        const int row = row0 + t;
+        if (a.bias) v = v + a.bias[row];
+        if (epi == GEMV_EPI_RESIDUAL) v = a.epilogue_residual[row] + v;
+        a.out[row] = v;
+    }
+}
+
+template <int R, int NC>
+int launch_splitk(hm_ctx *ctx, const GemvArgs &a, int epi, bool pro) {
+    const int grid = (a.N + R - 1) / R;
+    if (pro) {
+        if constexpr (NC <= 4)
+            hipLaunchKernelGGL((gemv_bf16_nk_splitk_kernel<R, NC, true>), dim3(grid), dim3(GEMV_THREADS), 0, ctx->stream, a, epi);
+    } else {
+        hipLaunchKernelGGL((gemv_bf16_nk_splitk_kernel<R, NC, false>), dim3(grid), dim3(GEMV_THREADS), 0, ctx->stream, a, epi);
+    }
+    HM_LAUNCH_CHECK(ctx);
+    return HM_OK;
+}
+
+// One activation row, bf16 weights, rows of 512 .. 16384 elements (with a prologue: up to 8192), fewer than
+// 65536 of them (the LM heads keep the persistent kernel and its candidates).
+bool try_splitk(hm_ctx *ctx, const GemvArgs &a, int epi, int *rc) {
+    static const bool enabled = [] {  // HOMURA_GEMV_SPLITK=0: rows are never cut (for comparisons)
+        const char *e = getenv("HOMURA_GEMV_SPLITK");
+        return !e || atoi(e) != 0;
+    }();
+    if (!enabled || a.w_f32 || epi == GEMV_EPI_ARGMAX) return false;
+    const bool pro = a.norm_w || a.prologue_residual || a.resid_out;
+    const int per_wg = WAVE * 8 * GEMV_WAVES;  // k covered by one chunk of each wavefront
+    const int nc = (a.K + per_wg - 1) / per_wg;
+    if (a.K < 512 || nc > (pro ? 4 : 8) || a.N >= 65536) return false;
+    // rows a workgroup: measured best of 1, 2, 4 over 25 shapes (the choices lie within 5 % of each other
+    // except for one row a workgroup on short rows and many of them)
+    const size_t bytes = (size_t)2 * a.K * a.N;
+    int r = (a.K >= 4096 && a.N >= 2048) ? 4 : ((a.N <= 1536 && bytes < ((size_t)17 << 19)) ? 1 : 2);
+    if (epi == GEMV_EPI_SILU_MUL_PAIRS && r == 1) r = 2;
+#define HM_SPLITK(RR, CC) \
+    if (r == RR && nc == CC) { *rc = launch_splitk<RR, CC>(ctx, a, epi, pro); return true; }
+    HM_SPLITK(1, 1) HM_SPLITK(1, 2) HM_SPLITK(1, 3) HM_SPLITK(1, 4) HM_SPLITK(1, 5) HM_SPLITK(1, 6) HM_SPLITK(1, 7) HM_SPLITK(1, 8)
+    HM_SPLITK(2, 1) HM_SPLITK(2, 2) HM_SPLITK(2, 3) HM_SPLITK(2, 4) HM_SPLITK(2, 5) HM_SPLITK(2, 6) HM_SPLITK(2, 7) HM_SPLITK(2, 8)
+    HM_SPLITK(4, 1) HM_SPLITK(4, 2) HM_SPLITK(4, 3) HM_SPLITK(4, 4) HM_SPLITK(4, 5) HM_SPLITK(4, 6) HM_SPLITK(4, 7) HM_SPLITK(4, 8)
+#undef HM_SPLITK
+    return false;
+}
+
 template <int R, int MT, bool WF32>
 int launch_nk_t(hm_ctx *ctx, const GemvArgs &a, int epi, int grid, size_t lds) {
     dim3 g(grid), b(GEMV_THREADS);
@@ -477,7 +628,7 @@ int gemv_bf16_nk_launch(hm_ctx *ctx, GemvArgs a, int M, int epi) {
             rc = launch_nk<2, 4>(ctx, b, epi, grid, (size_t)4 * a.K * 4);
             m0 += 4;
         } else {
-            if (!try_oneshot(ctx, b, epi, &rc)) {
+            if (!try_splitk(ctx, b, epi, &rc) && !try_oneshot(ctx, b, epi, &rc)) {
                 int grid = gemv_bf16_nk_grid(ctx, a.N, 4);
                 if (epi == GEMV_EPI_ARGMAX && grid > a.argmax_cap) grid = a.argmax_cap;
                 rc = launch_nk<4, 1>(ctx, b, epi, grid, (size_t)a.K * 4);
