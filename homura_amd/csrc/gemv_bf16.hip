@@ -553,16 +553,20 @@ bool try_splitk(hm_ctx *ctx, const GemvArgs &a, int epi, int *rc) {
     const int per_wg = WAVE * 8 * GEMV_WAVES;  // k covered by one chunk of each wavefront
     const int nc = (a.K + per_wg - 1) / per_wg;
     if (a.K < 512 || nc > (pro ? 4 : 8) || a.N >= 65536) return false;
-    // rows a workgroup: measured best of 1, 2, 4 over 25 shapes (the choices lie within 5 % of each other
-    // except for one row a workgroup on short rows and many of them)
+    // Rows a workgroup, the best of 1 .. 16 measured over 25 shapes. Every workgroup reads the activation
+    // pieces itself (4 bytes per k, 12 with residual and norm weights, against 2 R of weights), so a prologue
+    // wants more rows; few short rows want one.
     const size_t bytes = (size_t)2 * a.K * a.N;
-    int r = (a.K >= 4096 && a.N >= 2048) ? 4 : ((a.N <= 1536 && bytes < ((size_t)17 << 19)) ? 1 : 2);
+    int r;
+    if (pro) r = (a.K >= 4096 && a.N >= 8192) ? 8 : 4;
+    else r = (a.K >= 4096 && a.N >= 2048) ? 4 : ((a.N <= 1536 && bytes < ((size_t)17 << 19)) ? 1 : 2);
     if (epi == GEMV_EPI_SILU_MUL_PAIRS && r == 1) r = 2;
 #define HM_SPLITK(RR, CC) \
     if (r == RR && nc == CC) { *rc = launch_splitk<RR, CC>(ctx, a, epi, pro); return true; }
     HM_SPLITK(1, 1) HM_SPLITK(1, 2) HM_SPLITK(1, 3) HM_SPLITK(1, 4) HM_SPLITK(1, 5) HM_SPLITK(1, 6) HM_SPLITK(1, 7) HM_SPLITK(1, 8)
     HM_SPLITK(2, 1) HM_SPLITK(2, 2) HM_SPLITK(2, 3) HM_SPLITK(2, 4) HM_SPLITK(2, 5) HM_SPLITK(2, 6) HM_SPLITK(2, 7) HM_SPLITK(2, 8)
     HM_SPLITK(4, 1) HM_SPLITK(4, 2) HM_SPLITK(4, 3) HM_SPLITK(4, 4) HM_SPLITK(4, 5) HM_SPLITK(4, 6) HM_SPLITK(4, 7) HM_SPLITK(4, 8)
+    HM_SPLITK(8, 1) HM_SPLITK(8, 2) HM_SPLITK(8, 3) HM_SPLITK(8, 4)
 #undef HM_SPLITK
     return false;
 }
