@@ -24,6 +24,11 @@ constexpr int KMAX_ROWS = KWAVES * 8;
 constexpr int KSTAGE_U = 8;                            // 16-byte chunks a thread carries per row step
 constexpr int KSTAGE_BYTES = KTHREADS * KSTAGE_U * 16; // most bytes one row step may span
 constexpr int KMAXC = 8;                               // unit rounds a lane keeps in registers (K <= 8192)
+// Rows of 8193 .. 16384 (the down projection of models with wide MLPs): twice the rounds, a deeper row stage,
+// no light ops inside the launch.
+constexpr int KMAXC_LONG = 16;
+constexpr int KSTAGE_U_LONG = 14;
+constexpr int KSTAGE_BYTES_LONG = KTHREADS * KSTAGE_U_LONG * 16;
 
 template <int QT>
 struct KTraits;
@@ -265,7 +270,7 @@ __device__ __forceinline__ void stage_activation(const float *__restrict__ x, co
 // QT2 >= 0: a second matrix of the other K-quant type (w2, N2 rows, results to out2) shares the launch and
 // the prepared activation row - q|k in Q4_K with v in Q6_K, as Q4_K_M files have them. Its row steps follow
 // the first matrix's; a step never straddles the two.
-template <int QT, int CPL, bool FUSED, int QT2 = -1>
+template <int QT, int CPL, bool FUSED, int QT2 = -1, int U_ = KSTAGE_U>
 __global__ __launch_bounds__(KTHREADS) void gemv_kquant_kernel(const int8_t *__restrict__ q8,
                                                                const float *__restrict__ act_d,
                                                                const int *__restrict__ bsums,
@@ -280,7 +285,7 @@ __global__ __launch_bounds__(KTHREADS) void gemv_kquant_kernel(const int8_t *__r
     const float *x_f32 = FUSED ? x_f32_arg : nullptr;
     const homura::QuantFuse fuse = FUSED ? fuse_arg : homura::QuantFuse();
     constexpr int BB = KTraits<QT>::BYTES;
-    constexpr int U = KSTAGE_U;
+    constexpr int U = U_;
     extern __shared__ __attribute__((aligned(16))) uint8_t ws[];
     const int tid = threadIdx.x, lane = tid & (WAVE - 1), wave = tid / WAVE;
     const int nb = K / 256, nu = K / 16;
@@ -365,12 +370,16 @@ __global__ __launch_bounds__(KTHREADS) void gemv_kquant_kernel(const int8_t *__r
         }
         float *o = out + now.r0;
         const float *add = fuse.res_out_add ? fuse.res_out_add + now.r0 : nullptr;
-        for (; lr + 3 * KWAVES < now.nrows; lr += 4 * KWAVES) krows_trip<QT, CPL, 4>(ws, now.shift, rowbytes, lr, lane, nu, act, o, add);
-        if (lr + KWAVES < now.nrows) {
-            krows_trip<QT, CPL, 2>(ws, now.shift, rowbytes, lr, lane, nu, act, o, add);
-            lr += 2 * KWAVES;
+        if constexpr (CPL <= KMAXC) {
+            for (; lr + 3 * KWAVES < now.nrows; lr += 4 * KWAVES) krows_trip<QT, CPL, 4>(ws, now.shift, rowbytes, lr, lane, nu, act, o, add);
+            if (lr + KWAVES < now.nrows) {
+                krows_trip<QT, CPL, 2>(ws, now.shift, rowbytes, lr, lane, nu, act, o, add);
+                lr += 2 * KWAVES;
+            }
+            if (lr < now.nrows) krows_trip<QT, CPL, 1>(ws, now.shift, rowbytes, lr, lane, nu, act, o, add);
+        } else {  // long rows: the lane's share of the activation takes the registers of the side-by-side chains
+            for (; lr < now.nrows; lr += KWAVES) krows_trip<QT, CPL, 1>(ws, now.shift, rowbytes, lr, lane, nu, act, o, add);
         }
-        if (lr < now.nrows) krows_trip<QT, CPL, 1>(ws, now.shift, rowbytes, lr, lane, nu, act, o, add);
     }
 }
 
@@ -628,10 +637,13 @@ int gemv_kquant_launch(hm_ctx *ctx, const char *name, const float *d_x, const ui
     HM_REQUIRE(ctx, d_x && d_w && d_out, "%s: NULL pointer", name);
     HM_REQUIRE(ctx, M >= 1 && M <= 8, "%s: M=%d outside 1..8", name, M);
     HM_REQUIRE(ctx, K > 0 && K % 256 == 0 && N > 0, "%s: K=%d must be a positive multiple of 256, N=%d positive", name, K, N);
-    HM_REQUIRE(ctx, K <= KMAXC * WAVE * 16, "%s: K=%d above %d", name, K, KMAXC * WAVE * 16);
+    HM_REQUIRE(ctx, K <= KMAXC_LONG * WAVE * 16, "%s: K=%d above %d", name, K, KMAXC_LONG * WAVE * 16);
     HM_REQUIRE(ctx, ((uintptr_t)d_w % 16) == 0 && ((uintptr_t)d_x % 16) == 0, "%s: weight and activation buffers must be 16-byte aligned", name);
     const size_t rowbytes = (size_t)(K / 256) * BB;
-    HM_REQUIRE(ctx, KWAVES * rowbytes + 32 <= (size_t)KSTAGE_BYTES, "%s: K=%d too large for the LDS stage", name, K);
+    const bool long_rows = K > KMAXC * WAVE * 16 || KWAVES * rowbytes + 32 > (size_t)KSTAGE_BYTES;
+    const size_t stage_cap = long_rows ? (size_t)KSTAGE_BYTES_LONG : (size_t)KSTAGE_BYTES;
+    HM_REQUIRE(ctx, KWAVES * rowbytes + 32 <= stage_cap, "%s: K=%d too large for the LDS stage", name, K);
+    HM_REQUIRE(ctx, !(fuse && long_rows), "%s: the fused form takes rows up to %d", name, KMAXC * WAVE * 16);
     if (fuse) {
         HM_REQUIRE(ctx, M == 1 && K <= KXU * KTHREADS * 4, "%s: the fused form takes one row of at most %d", name, KXU * KTHREADS * 4);
         HM_REQUIRE(ctx, !(fuse->x2 && fuse->res_in), "%s: SiLU pair and residual input exclude each other", name);
@@ -647,7 +659,7 @@ int gemv_kquant_launch(hm_ctx *ctx, const char *name, const float *d_x, const ui
     rows = rows / KWAVES * KWAVES;
     if (rows < KWAVES) rows = KWAVES;
     if (rows > KMAX_ROWS) rows = KMAX_ROWS;
-    while (rows > KWAVES && (size_t)rows * rowbytes + 32 > (size_t)KSTAGE_BYTES) rows -= KWAVES;
+    while (rows > KWAVES && (size_t)rows * rowbytes + 32 > stage_cap) rows -= KWAVES;
     while (rows > KWAVES && (N + rows - 1) / rows < 2 * ctx->num_cus) rows -= KWAVES;
     // fused launches keep the quantised row in LDS behind the row stage: q8 | act_d | bsums | 4 floats
     const size_t stage_bytes = ((size_t)rows * rowbytes + 32 + 16 + 15) & ~(size_t)15;
@@ -678,6 +690,14 @@ int gemv_kquant_launch(hm_ctx *ctx, const char *name, const float *d_x, const ui
             hipLaunchKernelGGL((gemv_kquant_kernel<QT, C, false>), dim3(grid), dim3(KTHREADS), lds, ctx->stream, q8, \
                                act_d, bsums, d_w, om, K, N, rows, xf, fz, (int)stage_bytes);                        \
     } while (0)
+#define HM_KQ_LONG(C)                                                                                                     \
+    hipLaunchKernelGGL((gemv_kquant_kernel<QT, C, false, -1, KSTAGE_U_LONG>), dim3(grid), dim3(KTHREADS), lds, ctx->stream, \
+                       q8, act_d, bsums, d_w, om, K, N, rows, xf, fz, (int)stage_bytes)
+        if (long_rows) {
+            if (cpl <= 10) HM_KQ_LONG(10);
+            else if (cpl <= 12) HM_KQ_LONG(12);
+            else HM_KQ_LONG(16);
+        } else
         switch (cpl) {
             case 1: HM_KQ_CASE(1); break;
             case 2: HM_KQ_CASE(2); break;
@@ -688,6 +708,7 @@ int gemv_kquant_launch(hm_ctx *ctx, const char *name, const float *d_x, const ui
             case 7: HM_KQ_CASE(7); break;
             default: HM_KQ_CASE(8); break;
         }
+#undef HM_KQ_LONG
 #undef HM_KQ_CASE
         HM_LAUNCH_CHECK(ctx);
     }

@@ -94,6 +94,7 @@ struct QWords {
 typedef const uint32_t __attribute__((address_space(1))) *global_u32_ptr;
 typedef const u32x2 __attribute__((address_space(1))) *global_u32x2_ptr;
 typedef const uint16_t __attribute__((address_space(1))) *global_u16_ptr;
+typedef const u32x4 __attribute__((address_space(1))) *global_u32x4_ptr;
 
 template <int QT>
 __device__ __forceinline__ QWords<QT> load_quarter(const uint8_t *q) {
@@ -314,6 +315,124 @@ __global__ __launch_bounds__(PTHREADS) void gemv_planes_kernel(const float *__re
             fuse.cand_v[blockIdx.x] = bv;
             fuse.cand_i[blockIdx.x] = bi;
         }
+    }
+}
+
+// Rows cut across the wavefronts of a workgroup, for rows longer than gemv_planes_kernel keeps in registers
+// (K > 4096: the down projection of models with wide MLPs) and for matrices of few rows. A workgroup owns R
+// rows; a lane's unit is 16 bytes of a row's quant plane (Q8_0: half a block, Q4_0: a whole block) and its
+// scale, a wavefront's chunk 64 units, the four wavefronts take a row's chunks in turn, NC each. Every load is
+// requested before anything waits, the activation pieces first; the light ops in front of the product
+// (SiLU pair, residual add) are applied to the pieces in registers; the four partial sums of a row meet in
+// LDS and are added in wavefront order. No RMSNorm here (rows that long are normalised by their own launch).
+template <int QT, int R, int NC, bool FUSED>
+__global__ __launch_bounds__(PTHREADS) void gemv_planes_splitk_kernel(const float *__restrict__ x, const uint8_t *__restrict__ quants,
+                                                                      const uint16_t *__restrict__ scales, float *__restrict__ out,
+                                                                      int K, int N, const QuantFuse fuse_arg) {
+    const QuantFuse fuse = FUSED ? fuse_arg : QuantFuse();
+    constexpr int KPL = QT == 0 ? 16 : 32, XV = KPL / 4;  // weights and f32x4 activation pieces of a unit
+    __shared__ float part[PWAVES][R];
+    const int lane = threadIdx.x & (WAVE - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);
+    const int row0 = blockIdx.x * R;
+    const size_t qrow = QT == 0 ? (size_t)K : (size_t)K / 2;
+    const int nb = K / 32;
+    const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
+    f32x4 xr[NC][XV], ar[FUSED ? NC : 1][FUSED ? XV : 1];
+    u32x4 qw[NC][R];
+    uint32_t sc[NC][R];
+    const float *second = fuse.x2 ? fuse.x2 : fuse.res_in;
+#pragma unroll
+    for (int c = 0; c < NC; c++) {
+        const int k = ((c * PWAVES + wave) * WAVE + lane) * KPL;
+#pragma unroll
+        for (int j = 0; j < XV; j++) {
+            xr[c][j] = k < K ? *reinterpret_cast<const f32x4 *>(x + k + 4 * j) : zero4;
+            if constexpr (FUSED) ar[c][j] = (second && k < K) ? *reinterpret_cast<const f32x4 *>(second + k + 4 * j) : zero4;
+        }
+    }
+#pragma unroll
+    for (int c = 0; c < NC; c++) {
+        const int k = ((c * PWAVES + wave) * WAVE + lane) * KPL;
+        const int kc = k < K ? k : 0;  // units past the row end re-read its first one against activations of zero
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            const int row = min(row0 + r, N - 1);  // rows past the end re-read the last one
+            qw[c][r] = __builtin_nontemporal_load((global_u32x4_ptr)(quants + (size_t)row * qrow + (QT == 0 ? kc : kc / 2)));
+            sc[c][r] = __builtin_nontemporal_load((global_u16_ptr)(scales + (size_t)row * nb + kc / 32));
+        }
+    }
+    // the light ops of the quantised plan in front of this product (reference src/hf/emitter_quant.rs:985-1103)
+    if constexpr (FUSED) {
+        if (fuse.x2) {
+#pragma unroll
+            for (int c = 0; c < NC; c++)
+#pragma unroll
+                for (int j = 0; j < XV; j++)
+#pragma unroll
+                    for (int e = 0; e < 4; e++) xr[c][j][e] = (xr[c][j][e] / (1.0f + expf(-xr[c][j][e]))) * ar[c][j][e];
+        } else if (fuse.res_in) {
+#pragma unroll
+            for (int c = 0; c < NC; c++) {
+                const int k = ((c * PWAVES + wave) * WAVE + lane) * KPL;
+#pragma unroll
+                for (int j = 0; j < XV; j++) {
+                    xr[c][j] += ar[c][j];
+                    if (fuse.resid_out && blockIdx.x == 0 && k < K) *reinterpret_cast<f32x4 *>(fuse.resid_out + k + 4 * j) = xr[c][j];
+                }
+            }
+        }
+    }
+    float a[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) a[r] = 0.f;
+#pragma unroll
+    for (int c = 0; c < NC; c++) {
+        float xv[KPL], sx = 0.f;
+#pragma unroll
+        for (int j = 0; j < XV; j++)
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                xv[4 * j + e] = xr[c][j][e];
+                sx += xr[c][j][e];
+            }
+        const float sx_off = sx * (QT == 0 ? 128.f : 8.f);
+        if (QT == 1) {
+#pragma unroll
+            for (int j = 0; j < KPL; j++) xv[j] *= NIBBLE_FP8_UNIT;
+        }
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            const float d = f16_bits_to_f32((uint16_t)sc[c][r]);
+            const uint32_t w[4] = {qw[c][r].x, qw[c][r].y, qw[c][r].z, qw[c][r].w};
+            float t = 0.f;
+            if (QT == 0) {
+#pragma unroll
+                for (int i = 0; i < 4; i++) t = dot4_bytes(w[i] ^ 0x80808080u, xv + 4 * i, t);  // int8 -> biased unsigned
+            } else {
+                // byte i of the block's 16: low nibble = weight i, high nibble = weight 16 + i
+#pragma unroll
+                for (int i = 0; i < 4; i++) t = dot4_nibbles(w[i] & 0x0F0F0F0Fu, xv + 4 * i, t);
+#pragma unroll
+                for (int i = 0; i < 4; i++) t = dot4_nibbles((w[i] >> 4) & 0x0F0F0F0Fu, xv + 16 + 4 * i, t);
+            }
+            a[r] += d * (t - sx_off);
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < R; r++) a[r] = wave_sum(a[r]);
+    if (lane == 0) {
+#pragma unroll
+        for (int r = 0; r < R; r++) part[wave][r] = a[r];
+    }
+    __syncthreads();
+    const int t = threadIdx.x;
+    if (t < R && row0 + t < N) {
+        float v = part[0][t];
+#pragma unroll
+        for (int w = 1; w < PWAVES; w++) v += part[w][t];
+        if (fuse.res_out_add) v = v + fuse.res_out_add[row0 + t];
+        out[row0 + t] = v;
     }
 }
 
@@ -676,7 +795,7 @@ int planes_launch(hm_ctx *ctx, const char *name, const float *d_x, const uint8_t
     HM_CHECK_CTX(ctx);
     HM_REQUIRE(ctx, d_x && d_planes && d_out, "%s: NULL pointer", name);
     HM_REQUIRE(ctx, M >= 1 && M <= 8, "%s: M=%d outside 1..8", name, M);
-    HM_REQUIRE(ctx, K > 0 && K % 32 == 0 && K <= 4096 && N > 0, "%s: K=%d must be a multiple of 32 up to 4096, N=%d positive", name, K, N);
+    HM_REQUIRE(ctx, K > 0 && K % 32 == 0 && K <= 16384 && N > 0, "%s: K=%d must be a multiple of 32 up to 16384, N=%d positive", name, K, N);
     HM_REQUIRE(ctx, ((uintptr_t)d_planes % 16) == 0 && ((uintptr_t)d_x % 16) == 0, "%s: weight and activation buffers must be 16-byte aligned", name);
     HM_REQUIRE(ctx, !(fuse.x2 && fuse.res_in), "%s: SiLU pair and residual input exclude each other", name);
     HM_REQUIRE(ctx, !fuse.norm_w || K <= 4096, "%s: the fused RMSNorm holds rows up to 4096 wide (K=%d)", name, K);
@@ -685,11 +804,47 @@ int planes_launch(hm_ctx *ctx, const char *name, const float *d_x, const uint8_t
     HM_REQUIRE(ctx, M == 1 || (!fuse.x2 && !fuse.res_in && !fuse.norm_w && !fuse.res_out_add), "%s: fused light ops need M == 1", name);
     HM_REQUIRE(ctx, !fuse.cand_v || fuse.cand_i, "%s: argmax candidates need an index buffer", name);
     const bool q4 = QT == 1;
-    const PlanesShape sh = planes_shape(ctx, q4, K, N);
     const uint8_t *quants = d_planes;
     const uint16_t *scales = reinterpret_cast<const uint16_t *>(d_planes + homura::quant_planes_scale_offset(q4, N, K));
     const int cpl = (K / 8 + WAVE - 1) / WAVE;
     const bool fused = fuse.x2 || fuse.res_in || fuse.norm_w || fuse.res_out_add || fuse.cand_v;
+    // rows longer than the kernels below hold: cut across the wavefronts of a workgroup
+    static const bool force_cut = [] {
+        const char *e = getenv("HOMURA_PLANES_SPLITK");
+        return e && atoi(e) != 0;
+    }();
+    if ((K > 4096 || force_cut) && !fuse.norm_w && !fuse.cand_v) {
+        const int round_k = PWAVES * WAVE * (q4 ? 32 : 16);
+        const int nc = (K + round_k - 1) / round_k;
+        for (int m = 0; m < M; m++) {
+            const float *xm = d_x + (size_t)m * K;
+            float *om = d_out + (size_t)m * N;
+#define HM_CUT(RR, CC)                                                                                                      \
+    do {                                                                                                                    \
+        const int grid = (N + RR - 1) / RR;                                                                                 \
+        if (fused)                                                                                                          \
+            hipLaunchKernelGGL((gemv_planes_splitk_kernel<QT, RR, CC, true>), dim3(grid), dim3(PTHREADS), 0, ctx->stream, xm, \
+                               quants, scales, om, K, N, fuse);                                                             \
+        else                                                                                                                \
+            hipLaunchKernelGGL((gemv_planes_splitk_kernel<QT, RR, CC, false>), dim3(grid), dim3(PTHREADS), 0, ctx->stream, xm, \
+                               quants, scales, om, K, N, fuse);                                                             \
+    } while (0)
+            if (!q4) {
+                if (nc == 1) HM_CUT(8, 1);
+                else if (nc == 2) HM_CUT(8, 2);
+                else if (nc == 3) { if (fused) HM_CUT(4, 3); else HM_CUT(8, 3); }
+                else HM_CUT(4, 4);
+            } else {
+                if (nc == 1) { if (fused) HM_CUT(8, 1); else HM_CUT(16, 1); }
+                else { if (fused) HM_CUT(4, 2); else HM_CUT(8, 2); }
+            }
+#undef HM_CUT
+            HM_LAUNCH_CHECK(ctx);
+        }
+        return HM_OK;
+    }
+    HM_REQUIRE(ctx, K <= 4096, "%s: K=%d above 4096 with a fused RMSNorm or argmax candidates", name, K);
+    const PlanesShape sh = planes_shape(ctx, q4, K, N);
     // Q4_0 at the LM-head shape: the half-block-per-lane kernel
     const int nblk = K / 32;
     // Q4_0, tall matrices with rows of 2048, 3072 or 4096: the whole-block-per-lane kernel (35.6 us against 39.5 of

@@ -162,7 +162,7 @@ int HfModel::build_quant_planes() {
             int first, count;
             quant_run(l, j, &first, &count);
             const DType t = proj_dtype(l, j);
-            if (first != j || (t != DType::Q8_0 && t != DType::Q4_0) || kdim[j] > 4096 || !packed_[l].quant[j]) continue;
+            if (first != j || (t != DType::Q8_0 && t != DType::Q4_0) || kdim[j] > 16384 || !packed_[l].quant[j]) continue;
             int n = 0;
             for (int e = j; e < j + count; e++) n += ndim[e];
             const size_t bytes = quant_planes_bytes(t == DType::Q4_0, n, kdim[j]);

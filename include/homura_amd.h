@@ -111,7 +111,7 @@ int hm_gemv_q4_0(hm_ctx *ctx, const float *d_x, const uint8_t *d_w_blocks, float
  * of an [N][K] matrix (0 for a type other than HM_DTYPE_Q8_0 / Q4_0 / Q6_K or a bad shape), hm_pack_quant_planes
  * fills them from raw blocks [N][K/32] in one launch, hm_unpack_quant_planes is its inverse.
  * Results equal hm_gemv_q8_0 / hm_gemv_q4_0 up to the order of the f32 additions. M <= 8, K % 32 == 0,
- * K <= 4096. hm_dequant_quant_planes writes the N * K dequantised weights, bit-exact with the CPU. */
+ * K <= 16384 (rows above 4096 are cut across the wavefronts of a workgroup). hm_dequant_quant_planes writes the N * K dequantised weights, bit-exact with the CPU. */
 size_t hm_quant_planes_bytes(int hm_dtype, int N, int K);
 int hm_pack_quant_planes(hm_ctx *ctx, int hm_dtype, const uint8_t *d_blocks, uint8_t *d_planes, int N, int K);
 int hm_unpack_quant_planes(hm_ctx *ctx, int hm_dtype, const uint8_t *d_planes, uint8_t *d_blocks, int N, int K);
@@ -137,7 +137,7 @@ int hm_dequant_q4_0(hm_ctx *ctx, const uint8_t *d_blocks, float *d_out, size_t n
 /* K-quants, reference emit_dequant_matmul_q4_k / _q6_k (src/graph_builder/emit_quant.rs:165-816):
  * the f32 activation is quantised to Q8_K per 256-wide block (scale amax/127, round half to even),
  * then integer dot products per sub-block against the raw GGUF super-blocks [N][K/256] x 144 B
- * (Q4_K) or 210 B (Q6_K). K % 256 == 0, K <= 8192, M <= 8. The integer sums are the reference's; the
+ * (Q4_K) or 210 B (Q6_K). K % 256 == 0, K <= 16384, M <= 8. The integer sums are the reference's; the
  * f32 adds over units and blocks come in a different order. */
 int hm_gemv_q4_k(hm_ctx *ctx, const float *d_x, const uint8_t *d_w_blocks, float *d_out, int M, int K, int N);
 int hm_gemv_q6_k(hm_ctx *ctx, const float *d_x, const uint8_t *d_w_blocks, float *d_out, int M, int K, int N);

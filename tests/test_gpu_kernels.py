@@ -176,7 +176,14 @@ def test_quant_planes_hold_the_blocks_bit_for_bit(ctx, oracle, kind):
                                         ("q4_0", 3, 2048, 260), ("q4_0", 1, 32, 7), ("q4_0", 1, 3072, 1024),
                                         ("q4_0", 1, 256, 233100), ("q4_0", 1, 1792, 33333),
                                         ("q4_0", 2, 2048, 29201), ("q4_0", 1, 4096, 14601), ("q4_0", 1, 2528, 4099),
-                                        ("q4_0", 1, 3072, 9001), ("q4_0", 1, 2048, 8193)])
+                                        ("q4_0", 1, 3072, 9001), ("q4_0", 1, 2048, 8193),
+                                        # rows cut across a workgroup's wavefronts (K > 4096): the down projections of
+                                        # Qwen2.5-1.5B, TinyLlama, SmolLM2, Llama-2-7B; ragged ends; the widest served
+                                        ("q8_0", 1, 8960, 1536), ("q4_0", 1, 8960, 1536), ("q8_0", 1, 5632, 2048),
+                                        ("q4_0", 1, 5632, 2048), ("q8_0", 2, 8192, 2047), ("q4_0", 1, 8192, 2049),
+                                        ("q8_0", 1, 11008, 515), ("q4_0", 3, 11008, 77), ("q8_0", 1, 4128, 9),
+                                        ("q4_0", 1, 4128, 3), ("q8_0", 1, 16384, 130), ("q4_0", 1, 16384, 130),
+                                        ("q8_0", 1, 12320, 21), ("q4_0", 1, 8224, 17)])
 def test_quant_planes_gemv(ctx, oracle, kind, M, K, N):
     """The dequant-GEMV over the re-packed weights against the oracle on the raw blocks."""
     from homura_amd.runtime import DTYPE_Q4_0, DTYPE_Q8_0
@@ -209,8 +216,8 @@ def test_quant_planes_reference_kat_and_limits(ctx, golden):
     ctx.gemv_q8_0_planes(dx, planes, dout, 1, K, N)
     assert np.all(dout.download(np.float32) == g["expected_each"])
     assert ctx.lib.hm_quant_planes_bytes(1, 8, 32) == 0 and ctx.lib.hm_quant_planes_bytes(DTYPE_Q8_0, 8, 48) == 0
-    with pytest.raises(HomuraError, match="up to 4096"):
-        ctx.gemv_q8_0_planes(dx, planes, dout, 1, 8192, 1)
+    with pytest.raises(HomuraError, match="up to 16384"):
+        ctx.gemv_q8_0_planes(dx, planes, dout, 1, 16416, 1)
 
 
 def test_q6_k_planes_hold_the_blocks_bit_for_bit(ctx, oracle):
@@ -320,7 +327,10 @@ def test_quantize_q8_k_bit_exact(ctx, oracle):
 
 @pytest.mark.parametrize("kind", ["q4_k", "q6_k"])
 @pytest.mark.parametrize("M,K,N", [(1, 1024, 3072), (1, 3072, 1024), (1, 1024, 151936), (2, 256, 7), (1, 2048, 515),
-                                   (1, 8192, 64)])
+                                   (1, 8192, 64),
+                                   # rows above 8192: twice the rounds a lane, a deeper row stage (Qwen2.5-1.5B's and
+                                   # Llama-2-7B's down projections, the widest row served)
+                                   (1, 8960, 1536), (2, 11008, 130), (1, 16384, 33), (1, 8448, 5)])
 def test_gemv_kquant(ctx, oracle, kind, M, K, N):
     say(f"gemv_{kind} M={M} K={K} N={N}")
     raw = (synth.q4_k_blocks if kind == "q4_k" else synth.q6_k_blocks)(5, N * K // 256)
@@ -331,7 +341,8 @@ def test_gemv_kquant(ctx, oracle, kind, M, K, N):
     got = dout.download(np.float32, (M, N))
     err = rel_err(got, want)
     say(f"  rel err {err:.2e}")
-    assert err < 1e-4          # same integer sums; only the order of the f32 adds differs
+    # same integer sums; only the order of the f32 adds differs (35-64 block sums a row above 8192)
+    assert err < (1e-4 if K <= 8192 else 3e-4)
     for b in (dx, dw, dout):
         b.free()
 
