@@ -49,6 +49,31 @@ TINY_LLAMA = TransformerConfig(
     max_position_embeddings=512, tie_word_embeddings=False)
 
 
+# The widths of the other models the reference lists with decode figures (README "Performance"): these run
+# one launch per projection. `layers` cuts the depth for tests; vocabularies as the checkpoints have them.
+def listed_shape(name: str, layers: int | None = None, vocab: int | None = None) -> TransformerConfig:
+    shapes = {
+        "qwen2.5-0.5b": dict(hidden_size=896, intermediate_size=4864, num_attention_heads=14, num_hidden_layers=24,
+                             vocab_size=151936, num_key_value_heads=2, head_dim=64, rms_norm_eps=1e-6, rope_theta=1e6,
+                             tie_word_embeddings=True, attention_bias=True),
+        "tinyllama-1.1b": dict(hidden_size=2048, intermediate_size=5632, num_attention_heads=32, num_hidden_layers=22,
+                               vocab_size=32000, num_key_value_heads=4, head_dim=64, rms_norm_eps=1e-5, rope_theta=1e4,
+                               tie_word_embeddings=False),
+        "qwen2.5-1.5b": dict(hidden_size=1536, intermediate_size=8960, num_attention_heads=12, num_hidden_layers=28,
+                             vocab_size=151936, num_key_value_heads=2, head_dim=128, rms_norm_eps=1e-6, rope_theta=1e6,
+                             tie_word_embeddings=True, attention_bias=True),
+        "smollm2-1.7b": dict(hidden_size=2048, intermediate_size=8192, num_attention_heads=32, num_hidden_layers=24,
+                             vocab_size=49152, num_key_value_heads=32, head_dim=64, rms_norm_eps=1e-5, rope_theta=1.3e5,
+                             tie_word_embeddings=True),
+    }
+    d = dict(shapes[name], max_position_embeddings=2048)
+    if layers is not None:
+        d["num_hidden_layers"] = layers
+    if vocab is not None:
+        d["vocab_size"] = vocab
+    return TransformerConfig(**d)
+
+
 # K-quant proportions (every projection input a multiple of 256) for Q4_K / Q6_K files
 TINY_K = TransformerConfig(
     hidden_size=512, intermediate_size=768, num_attention_heads=8, num_hidden_layers=2,
