@@ -95,6 +95,7 @@ def main() -> int:
                     help="cap on kernel launches per stand-alone measurement graph (0 = the whole weight ring)")
     ap.add_argument("--no-prefill", action="store_true", help="skip the prompt-pass measurement")
     ap.add_argument("--no-quantised", action="store_true", help="skip the decode measurements with quantised projections")
+    ap.add_argument("--no-other-shapes", action="store_true", help="skip the decode measurements at the other listed models' shapes")
     ap.add_argument("--no-kernel-configs", action="store_true",
                     help="skip the stand-alone kernel measurements (benchmark configurations 1, 3, 4, 5)")
     args = ap.parse_args()
@@ -301,6 +302,36 @@ def main() -> int:
                     quantised[name]["prefill_512"] = {"value": round(512 / best, 1), "unit": "tok/s", "ms": round(best * 1e3, 3)}
                 qm.close()
                 del qw
+        # The other models the reference lists with decode figures, at their full depth and vocabulary: no
+        # whole-step instance, one launch per projection replayed from a graph. Reported beside `value`.
+        other_shapes = None
+        if not args.no_other_shapes:
+            import dataclasses
+            from homura_amd.runtime import DTYPE_Q8_0 as _Q8
+            other_shapes = {"unit": "tok/s", "steps": args.steps,
+                            "what": "greedy decode from a 1024-row cache, one launch per projection (graph replay); "
+                                    "bf16 weights, and a Q4_K_M-style mix of Q4_K / Q6_K with an f32 LM head; "
+                                    "reference_cpu_tok_s: the reference's README figure (bf16, Ryzen 9 7900X3D)"}
+            for name, ref_tok_s in (("qwen2.5-0.5b", 36), ("tinyllama-1.1b", 20), ("qwen2.5-1.5b", 13), ("smollm2-1.7b", 11)):
+                ocfg = synth_model.listed_shape(name)
+                entry = {"reference_cpu_tok_s": ref_tok_s}
+                for fmt in ("bf16", "q4_k_m_mix"):
+                    if fmt != "bf16" and ocfg.hidden_size % 256 != 0:
+                        continue   # K-quant blocks are 256 wide
+                    fcfg = ocfg if fmt == "bf16" else dataclasses.replace(ocfg, tie_word_embeddings=False)
+                    mix = None if fmt == "bf16" else synth_model.q4_k_m_mix(fcfg)
+                    wdt = 1 if fmt == "bf16" else _Q8
+                    ow = synth_model.synth_weights(fcfg, seed + 21, wdt, has_qk_norm=False, proj_dtypes=mix)
+                    omdl = synth_model.build_model(ctx, fcfg, ow, 2048, wdt, has_qk_norm=False, proj_dtypes=mix)
+                    del ow
+                    omdl.init_kv_cache(synth_model.synth_kv(fcfg, seed + 22, PREFILL), PREFILL)
+                    omdl.set_graph(not args.no_graph)
+                    omdl.bench_decode(int(prompt[0]) % fcfg.vocab_size, max(args.warmup, 2))
+                    o_ms, _ = omdl.bench_decode(int(prompt[1]) % fcfg.vocab_size, args.steps)
+                    entry[fmt] = {"value": round(args.steps * 1e3 / o_ms, 1), "ms_per_step": round(o_ms / args.steps, 4),
+                                  "kernel_launches_per_step": omdl.launches_per_step()}
+                    omdl.close()
+                other_shapes[name] = entry
         kernel_configs = None
         if not args.no_kernel_configs:
             from homura_amd import kernel_bench
@@ -350,6 +381,7 @@ def main() -> int:
         "launch_floor": launch_floor,
         "prefill": prefill,
         "quantised_decode": quantised,
+        "other_shapes": other_shapes,
         "event_ms_per_step": round(event_ms / args.steps, 4),
         "kernels": kernels,
         "kernel_configs": kernel_configs,
