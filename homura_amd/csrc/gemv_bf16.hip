@@ -459,6 +459,7 @@ __global__ __launch_bounds__(GEMV_THREADS) void gemv_bf16_nk_splitk_kernel(GemvA
                              : u32x4{0u, 0u, 0u, 0u};
         }
     }
+    __builtin_amdgcn_sched_barrier(0);  // every request above goes out before any arithmetic below
     if constexpr (PRO) {
         float ss = 0.f;
 #pragma unroll

@@ -362,6 +362,7 @@ __global__ __launch_bounds__(PTHREADS) void gemv_planes_splitk_kernel(const floa
             sc[c][r] = __builtin_nontemporal_load((global_u16_ptr)(scales + (size_t)row * nb + kc / 32));
         }
     }
+    __builtin_amdgcn_sched_barrier(0);  // every request above goes out before any arithmetic below
     // the light ops of the quantised plan in front of this product (reference src/hf/emitter_quant.rs:985-1103)
     if constexpr (FUSED) {
         if (fuse.x2) {

@@ -1,6 +1,7 @@
 // HfModel and the bf16 plan emitter on the GPU runtime (see hf.h).
 #include "hf.h"
 
+#include <algorithm>
 #include <cmath>
 #include <cstdlib>
 
@@ -10,6 +11,7 @@
 #include "../gemm_kquant_i8.h"
 #include "../gemv_bf16.h"
 #include "../gemm_bf16_mfma.h"
+#include "../gemv_k8.h"
 #include "../gemv_kquant.h"
 #include "../gemv_quant.h"
 #include "../gemv_quant_planes.h"
@@ -476,13 +478,17 @@ int HfModel::finalize(int max_seq_len) {
         if (all_kquant) {
             fused_format = true;
             fused_wf_ = FUSED_WF_K8;
+            // the K8 form serves the whole-step launch and the per-projection decode GEMVs alike
+            if (cfg_.hidden_size % 256 == 0 && cfg_.q_dim() % 256 == 0 && cfg_.intermediate_size % 256 == 0 &&
+                std::max({cfg_.hidden_size, cfg_.q_dim(), cfg_.intermediate_size}) <= 16384 && (rc = build_k8_planes()) != HM_OK)
+                return rc;
         }
     }
     if (fused_format) {
         const FusedShape fs{cfg_.hidden_size, cfg_.num_attention_heads, cfg_.kv_heads(), cfg_.head_dim(),
                             cfg_.intermediate_size, fused_wf_};
         bool served = decode_fused_supported(ctx_, fs, cfg_.num_hidden_layers, max_seq_len, nullptr);
-        if (served && fused_wf_ == FUSED_WF_K8 && (rc = build_k8_planes()) != HM_OK) return rc;
+        served = served && (fused_wf_ != FUSED_WF_K8 || (bool)packed_[0].k8[0]);
         if (served) {
             s.fused_layers = Buffer::alloc_bytes(ctx_, sizeof(FusedLayerPtrs) * (size_t)cfg_.num_hidden_layers,
                                                  {cfg_.num_hidden_layers}, DType::I64);
@@ -1120,6 +1126,7 @@ int HfModel::emit_transformer_plan_quant() {
     // Whether every launch of a group can take light ops along: Q8_0 / Q4_0 always, K-quants while the
     // row fits the in-kernel preparation
     auto plain_group = [&](int layer, std::initializer_list<int> which, int64_t K) {
+        if (packed_[layer].k8[0]) return true;  // the K8 launch prepares rows of any width it serves
         for (int w : which) {
             const DType t = proj_dtype(layer, w);
             if ((t == DType::Q4_K || t == DType::Q6_K) && K > 4096) return false;
@@ -1129,6 +1136,50 @@ int HfModel::emit_transformer_plan_quant() {
     // The QuantMM steps of one group of matrices that share an activation (q|k|v, gate|up, or one alone)
     struct GroupMember { const char *label; int which; int64_t N; size_t w_slot, out_slot; };
     auto quant_group = [&](int layer, size_t act_slot, int64_t K, std::vector<GroupMember> members, FuseSlots fs) {
+        // A model whose K-quant matrices were re-packed into the K8 form: one launch for the whole group, whatever
+        // mix of Q4_K and Q6_K its members are (their outputs are adjacent); the row is prepared and quantised to
+        // Q8_K inside the launch. The step list keeps the reference's kernels; the other members launch nothing.
+        const int group_of[7] = {0, 0, 0, 1, 2, 2, 3};
+        const Buffer &k8 = packed_[layer].k8[group_of[members[0].which]];
+        if (k8 && (fs.norm_w == NO || K <= 8192)) {
+            int64_t n_all = 0;
+            std::string label;
+            for (const GroupMember &gm : members) {
+                n_all += gm.N;
+                label += gm.label;
+            }
+            const uint8_t *plane = k8.as<uint8_t>();
+            const uint8_t *records = plane + k8_plane_bytes((int)n_all, (int)K);
+            for (size_t j = 0; j < members.size(); j++) {
+                CompiledKernel k;
+                k.ops_label = std::string("QuantMM[") + members[j].label + "]";
+                if (j == 0) {
+                    DeviceLaunch l;
+                    l.name = "gemv_k8[" + label + "]";
+                    if (fs.norm_w != NO) l.name += fs.res_in != NO ? "+resid+norm" : "+norm";
+                    if (fs.x2 != NO) l.name += "+silu";
+                    if (fs.add != NO) l.name += "+resid";
+                    l.bytes_fixed = (double)k8.bytes() + K * 4.0 + n_all * 4.0;
+                    const int64_t Kc = K, Nc = n_all;
+                    l.fn = [=](const StepContext &sc) -> int {
+                        auto f32 = [&](size_t slot) { return slot == NO ? nullptr : sc.pool[slot]->as<float>(); };
+                        const float *x = fs.x != NO ? f32(fs.x) : sc.pool[sc.step.input_slots[0]]->as<float>();
+                        float *out = fs.out != NO ? f32(fs.out) : sc.pool[sc.step.output_slots[0]]->as<float>();
+                        QuantFuse f;
+                        f.x2 = f32(fs.x2);
+                        f.res_in = f32(fs.res_in);
+                        f.resid_out = f32(fs.resid_out);
+                        f.norm_w = f32(fs.norm_w);
+                        f.eps = eps;
+                        f.res_out_add = f32(fs.add);
+                        return gemv_k8_fused(sc.ctx, x, plane, records, out, (int)Kc, (int)Nc, f);
+                    };
+                    k.launches.push_back(std::move(l));
+                }
+                add_step(std::move(k), {act_slot, members[j].w_slot}, {members[j].out_slot});
+            }
+            return;
+        }
         // the runs of same-type neighbours: (first member, count, rows, label)
         struct Run { size_t j; int count; int64_t n; std::string label; DType t; };
         std::vector<Run> runs;
