@@ -38,30 +38,6 @@ struct AttnFuse {
     float eps;
 };
 
-// One wavefront: optional RMSNorm over hd, then x*cos + rotate_half(x)*sin; lane i < hd/2 owns
-// the rotation pair (i, i + hd/2) and gets its two results back in (o_lo, o_hi).
-template <int HD>
-__device__ __forceinline__ void norm_rope_row(const float *__restrict__ src,
-                                              const float *__restrict__ nw,
-                                              const float *__restrict__ c,
-                                              const float *__restrict__ sn, float eps, int lane,
-                                              float &o_lo, float &o_hi) {
-    constexpr int HALF = HD / 2;
-    const bool on = lane < HALF;
-    float lo = on ? src[lane] : 0.f, hi = on ? src[lane + HALF] : 0.f;
-    const float c_lo = on ? c[lane] : 0.f, c_hi = on ? c[lane + HALF] : 0.f;
-    const float s_lo = on ? sn[lane] : 0.f, s_hi = on ? sn[lane + HALF] : 0.f;
-    const float w_lo = (on && nw) ? nw[lane] : 1.f, w_hi = (on && nw) ? nw[lane + HALF] : 1.f;
-    if (nw) {
-        const float ss = wave_sum(lo * lo + hi * hi);
-        const float inv = 1.0f / sqrtf(ss / (float)HD + eps);
-        lo = (lo * inv) * w_lo;
-        hi = (hi * inv) * w_hi;
-    }
-    o_lo = lo * c_lo + (-hi) * s_lo;
-    o_hi = hi * c_hi + lo * s_hi;
-}
-
 // Sum over the LPR (8 or 16) adjacent lanes that share a cache row, on the DPP path; every lane of
 // the group receives the total.
 template <int LPR>
@@ -121,24 +97,55 @@ __global__ __launch_bounds__(ATT_THREADS) void gqa_decode_attn_kernel(
 
     // ── queries (and, for the owner, the new K/V row) into LDS ──
     if (fused) {
+        // A wavefront prepares rows t = wave, wave + 4, ... of (G query heads, new K row, new V row). Every load
+        // of all its rows goes out before the first is used: with more than four rows (G > 2) a loop over the rows
+        // would pay one trip to memory per turn.
         const float *c = fuse.cos_tab + (size_t)pos * HD;
         const float *sn = fuse.sin_tab + (size_t)pos * HD;
-        constexpr int HALF = HD / 2;
-        for (int t = wave; t < G + 2; t += ATT_WAVES) {
+        constexpr int HALF = HD / 2, TMAX = (G + 2 + ATT_WAVES - 1) / ATT_WAVES;
+        const bool on = lane < HALF;
+        float rlo[TMAX], rhi[TMAX];
+#pragma unroll
+        for (int j = 0; j < TMAX; j++) {
+            const int t = wave + j * ATT_WAVES;
+            const float *src = nullptr;
+            if (t < G) src = fuse.qkv_raw + (size_t)(kvhd * G + t) * HD;
+            else if (owner && t == G) src = fuse.qkv_raw + (size_t)H * HD + (size_t)kvhd * HD;
+            else if (owner && t == G + 1) src = fuse.qkv_raw + (size_t)(H + kvh) * HD + (size_t)kvhd * HD;
+            rlo[j] = (src && on) ? src[lane] : 0.f;
+            rhi[j] = (src && on) ? src[lane + HALF] : 0.f;
+        }
+        const float c_lo = on ? c[lane] : 0.f, c_hi = on ? c[lane + HALF] : 0.f;
+        const float s_lo = on ? sn[lane] : 0.f, s_hi = on ? sn[lane + HALF] : 0.f;
+        const float qw_lo = (on && fuse.qw) ? fuse.qw[lane] : 1.f, qw_hi = (on && fuse.qw) ? fuse.qw[lane + HALF] : 1.f;
+        const float kw_lo = (on && fuse.kw) ? fuse.kw[lane] : 1.f, kw_hi = (on && fuse.kw) ? fuse.kw[lane + HALF] : 1.f;
+        // one row: optional RMSNorm over hd, then x*cos + rotate_half(x)*sin; lane i < hd/2 owns the rotation pair
+        // (i, i + hd/2)
+        auto norm_rope = [&](float lo, float hi, bool norm, float w_lo, float w_hi, float &o_lo, float &o_hi) {
+            if (norm) {
+                const float ss = wave_sum(lo * lo + hi * hi);
+                const float inv = 1.0f / sqrtf(ss / (float)HD + fuse.eps);
+                lo = (lo * inv) * w_lo;
+                hi = (hi * inv) * w_hi;
+            }
+            o_lo = lo * c_lo + (-hi) * s_lo;
+            o_hi = hi * c_hi + lo * s_hi;
+        };
+#pragma unroll
+        for (int j = 0; j < TMAX; j++) {
+            const int t = wave + j * ATT_WAVES;
             if (t < G) {
                 float lo, hi;
-                norm_rope_row<HD>(fuse.qkv_raw + (size_t)(kvhd * G + t) * HD, fuse.qw, c, sn, fuse.eps,
-                                  lane, lo, hi);
-                if (lane < HALF) {
+                norm_rope(rlo[j], rhi[j], fuse.qw != nullptr, qw_lo, qw_hi, lo, hi);
+                if (on) {
                     qs[t][lane] = lo;
                     qs[t][lane + HALF] = hi;
                 }
             } else if (owner && t == G) {
                 float lo, hi;
-                norm_rope_row<HD>(fuse.qkv_raw + (size_t)H * HD + (size_t)kvhd * HD, fuse.kw, c, sn,
-                                  fuse.eps, lane, lo, hi);
+                norm_rope(rlo[j], rhi[j], fuse.kw != nullptr, kw_lo, kw_hi, lo, hi);
                 // round to bf16 exactly once; cache and this kernel use the same rounded values
-                if (lane < HALF) {
+                if (on) {
                     uint16_t *dst = kcache + head_base + (size_t)pos * HD;
                     const uint16_t r_lo = f32_to_bf16_rne_dev(lo), r_hi = f32_to_bf16_rne_dev(hi);
                     dst[lane] = r_lo;
@@ -147,12 +154,13 @@ __global__ __launch_bounds__(ATT_THREADS) void gqa_decode_attn_kernel(
                     knew[lane + HALF] = __uint_as_float((uint32_t)r_hi << 16);
                 }
             } else if (owner && t == G + 1) {
-                const float *src = fuse.qkv_raw + (size_t)(H + kvh) * HD + (size_t)kvhd * HD;
-                uint16_t *dst = vcache + head_base + (size_t)pos * HD;
-                for (int i = lane; i < HD; i += WAVE) {
-                    const uint16_t r = f32_to_bf16_rne_dev(src[i]);
-                    dst[i] = r;
-                    vnew[i] = __uint_as_float((uint32_t)r << 16);
+                if (on) {
+                    uint16_t *dst = vcache + head_base + (size_t)pos * HD;
+                    const uint16_t r_lo = f32_to_bf16_rne_dev(rlo[j]), r_hi = f32_to_bf16_rne_dev(rhi[j]);
+                    dst[lane] = r_lo;
+                    dst[lane + HALF] = r_hi;
+                    vnew[lane] = __uint_as_float((uint32_t)r_lo << 16);
+                    vnew[lane + HALF] = __uint_as_float((uint32_t)r_hi << 16);
                 }
             }
         }
