@@ -14,6 +14,7 @@
 // used as stored (biased unsigned): sum_j q_j x_j - offset * sum_j x_j, four byte->float
 // conversions per 32-bit word with no shifts for the byte lanes.
 #include "gemv_quant.h"
+#include "gemv_quant_planes.h"
 
 #include "hm_common.h"
 #include "quant_formats.h"
@@ -425,8 +426,20 @@ int gemv_quant_launch(hm_ctx *ctx, const char *name, const float *d_x, const uin
     HM_REQUIRE(ctx, M == 1 || (!fuse.x2 && !fuse.res_in && !fuse.norm_w && !fuse.res_out_add), "%s: fused light ops need M == 1", name);
     const size_t rowbytes = (size_t)(K / 32) * BB;
     const size_t x_bytes = (size_t)K * 4;
-    HM_REQUIRE(ctx, x_bytes + QWAVES * rowbytes + 32 <= 64 * 1024 && QWAVES * rowbytes + 32 <= (size_t)STAGE_BYTES,
-               "%s: K=%d too large for the LDS stage", name, K);
+    if (!(x_bytes + QWAVES * rowbytes + 32 <= 64 * 1024 && QWAVES * rowbytes + 32 <= (size_t)STAGE_BYTES)) {
+        // Rows too long for the LDS stage (above about 7700 for Q8_0, 14500 for Q4_0): the blocks are re-packed
+        // into planes in the workspace and multiplied by the cut-row kernel, two launches a call. (A caller that
+        // keeps its weights on the device packs them once and calls the planes entry points.)
+        const size_t need = homura::quant_planes_bytes(QT == 1, N, K);
+        HM_REQUIRE(ctx, K <= 16384 && need <= ctx->workspace_bytes && !fuse.norm_w && !fuse.cand_v,
+                   "%s: K=%d too large for the LDS stage (and %zu bytes of planes do not fit the workspace, or a norm / "
+                   "argmax rides along)", name, K, need);
+        uint8_t *planes = static_cast<uint8_t *>(ctx->workspace);
+        int rc = homura::pack_quant_planes(ctx, QT == 1, d_w, planes, N, K);
+        for (int m = 0; m < M && rc == HM_OK; m++)
+            rc = homura::gemv_planes_fused(ctx, QT == 1, d_x + (size_t)m * K, planes, d_out + (size_t)m * N, K, N, fuse);
+        return rc;
+    }
     const QuantShape sh = quant_shape<QT>(ctx, K, N);
     const int rows = sh.rows, grid = sh.grid;
     const size_t lds = sh.lds;

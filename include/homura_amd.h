@@ -92,7 +92,10 @@ int hm_gemv_bf16_nk(hm_ctx *ctx, const float *d_x, const uint16_t *d_w_nk, float
 
 /* Q8_0 dequant-matmul, reference emit_dequant_matmul_q8_0
  * (src/graph_builder/emit_quant.rs:30-142): weight = raw GGUF blocks [N][K/32] x 34 bytes
- * (LE f16 d + 32 int8), out[m,n] = sum_k x[m,k] * (q * d). M <= 8, K % 32 == 0. */
+ * (LE f16 d + 32 int8), out[m,n] = sum_k x[m,k] * (q * d). M <= 8, K % 32 == 0, K <= 16384. Rows above
+ * about 7700 (Q4_0: 14500) do not fit the kernel's LDS stage: such a call re-packs the blocks into planes in the
+ * context's workspace first (the planes must fit it: 64 MiB) and multiplies those - a caller that owns its
+ * device copies packs once (hm_pack_quant_planes) and calls hm_gemv_q8_0_planes. */
 int hm_gemv_q8_0(hm_ctx *ctx, const float *d_x, const uint8_t *d_w_blocks, float *d_out, int M,
                  int K, int N);
 

@@ -112,7 +112,9 @@ def test_q8_0_reference_kat(ctx, golden):
                                         # of the rows staged per step, two rows of x
                                         ("q4_0", 1, 256, 233100), ("q4_0", 1, 1792, 33333),
                                         ("q4_0", 2, 2048, 29201), ("q4_0", 1, 4096, 14601),
-                                        ("q4_0", 1, 7168, 8400)])
+                                        ("q4_0", 1, 7168, 8400),
+                                        # rows too long for the LDS stage: re-packed into planes in the workspace
+                                        ("q8_0", 1, 8960, 1536), ("q8_0", 2, 8192, 300), ("q4_0", 1, 16384, 130)])
 def test_quant_gemv(ctx, oracle, kind, M, K, N):
     say(f"gemv_{kind} M={M} K={K} N={N}")
     nb = N * (K // 32)
