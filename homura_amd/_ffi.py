@@ -97,6 +97,9 @@ SIGNATURES = {
     "hm_dequant_q4_0": (_I, [_P, _P, _P, _SZ]),
     "hm_gemv_q4_k": (_I, [_P, _P, _P, _P, _I, _I, _I]),
     "hm_gemv_q6_k": (_I, [_P, _P, _P, _P, _I, _I, _I]),
+    "hm_k8_bytes": (_SZ, [_I, _I]),
+    "hm_pack_k8": (_I, [_P, _I, _P, _I, _P, _I, _I, _I]),
+    "hm_gemv_k8": (_I, [_P, _P, _P, _P, _I, _I, _I]),
     "hm_gemv_q4_k_f32": (_I, [_P, _P, _P, _P, _I, _I, _I]),
     "hm_gemv_q6_k_f32": (_I, [_P, _P, _P, _P, _I, _I, _I]),
     "hm_quantize_q8_k": (_I, [_P, _P, _P, _P, _P, _I, _I]),

@@ -145,12 +145,25 @@ __global__ __launch_bounds__(GTHREADS) void gemv_k8_kernel(const float *__restri
     }
     __syncthreads();
     const int t = threadIdx.x;
-    if (t < SETS * R) {
+    auto row_total = [&](int ts, int tr) {
+        float v = part[ts * WPS][tr];
+#pragma unroll
+        for (int w = 1; w < WPS; w++) v += part[ts * WPS + w][tr];
+        return v;
+    };
+    if (fuse_arg.silu_pairs) {
+        // rows come in (gate_i, up_i) pairs (reference src/hf/emitter_quant.rs:1077-1103: silu(gate) * up)
+        if (t < SETS * (R / 2)) {
+            const int ts = t / (R / 2), tp = t % (R / 2), row = (blockIdx.x * SETS + ts) * R + 2 * tp;
+            if (row + 1 < N) {
+                const float gte = row_total(ts, 2 * tp), up = row_total(ts, 2 * tp + 1);
+                out[row / 2] = (gte / (1.0f + expf(-gte))) * up;
+            }
+        }
+    } else if (t < SETS * R) {
         const int ts = t / R, tr = t % R, row = (blockIdx.x * SETS + ts) * R + tr;
         if (row < N) {
-            float v = part[ts * WPS][tr];
-#pragma unroll
-            for (int w = 1; w < WPS; w++) v += part[ts * WPS + w][tr];
+            float v = row_total(ts, tr);
             if (res_out_add) v = v + res_out_add[row];
             out[row] = v;
         }
@@ -175,6 +188,7 @@ int homura::gemv_k8_fused(hm_ctx *ctx, const float *d_x, const uint8_t *d_plane,
     HM_REQUIRE(ctx, !(fuse.x2 && fuse.res_in) && !(fuse.x2 && fuse.norm_w), "gemv_k8: the SiLU pair excludes a residual input and a norm");
     HM_REQUIRE(ctx, !fuse.norm_w || K <= 8192, "gemv_k8: the fused RMSNorm holds rows up to 8192 wide (K=%d)", K);
     HM_REQUIRE(ctx, !fuse.cand_v, "gemv_k8: no argmax candidates here");
+    HM_REQUIRE(ctx, !fuse.silu_pairs || (N % 2 == 0 && !fuse.res_out_add), "gemv_k8: the paired epilogue needs an even N and no residual");
     HM_REQUIRE(ctx, ((uintptr_t)d_x % 16) == 0 && ((uintptr_t)d_plane % 16) == 0 && ((uintptr_t)d_records % 4) == 0 &&
                         ((uintptr_t)fuse.x2 % 16) == 0 && ((uintptr_t)fuse.res_in % 16) == 0 && ((uintptr_t)fuse.resid_out % 16) == 0 &&
                         ((uintptr_t)fuse.norm_w % 16) == 0, "gemv_k8: operands must be 16-byte aligned");
@@ -219,3 +233,33 @@ int homura::gemv_k8_fused(hm_ctx *ctx, const float *d_x, const uint8_t *d_plane,
 #undef HM_K8_R
 #undef HM_K8
 }
+
+extern "C" {
+
+size_t hm_k8_bytes(int N, int K) {
+    if (N <= 0 || K <= 0 || K % 256 != 0) return 0;
+    return k8_plane_bytes(N, K) + k8_record_bytes(N, K);
+}
+
+int hm_pack_k8(hm_ctx *ctx, int hm_dtype, const uint8_t *d_blocks, int rows, uint8_t *d_k8, int N, int K, int row0) {
+    HM_CHECK_CTX(ctx);
+    HM_REQUIRE(ctx, d_blocks && d_k8, "hm_pack_k8: NULL pointer");
+    HM_REQUIRE(ctx, hm_dtype == HM_DTYPE_Q4_K || hm_dtype == HM_DTYPE_Q6_K, "hm_pack_k8: dtype %d is not Q4_K or Q6_K", hm_dtype);
+    HM_REQUIRE(ctx, N > 0 && K > 0 && K % 256 == 0 && rows > 0 && row0 >= 0 && row0 + rows <= N,
+               "hm_pack_k8: rows [%d, %d) of %d, K=%d (a multiple of 256)", row0, row0 + rows, N, K);
+    return pack_k8_rows(ctx, hm_dtype, d_blocks, rows, K, d_k8, d_k8 + k8_plane_bytes(N, K), row0);
+}
+
+int hm_gemv_k8(hm_ctx *ctx, const float *d_x, const uint8_t *d_k8, float *d_out, int M, int K, int N) {
+    HM_CHECK_CTX(ctx);
+    HM_REQUIRE(ctx, d_x && d_k8 && d_out, "hm_gemv_k8: NULL pointer");
+    HM_REQUIRE(ctx, M >= 1 && M <= 8 && N > 0 && K > 0 && K % 256 == 0, "hm_gemv_k8: M=%d outside 1..8 or bad shape K=%d N=%d", M, K, N);
+    for (int m = 0; m < M; m++) {
+        const int rc = homura::gemv_k8_fused(ctx, d_x + (size_t)m * K, d_k8, d_k8 + k8_plane_bytes(N, K), d_out + (size_t)m * N, K, N,
+                                             homura::QuantFuse());
+        if (rc != HM_OK) return rc;
+    }
+    return HM_OK;
+}
+
+}  // extern "C"

@@ -21,6 +21,8 @@ struct QuantFuse {
     float eps = 0.f;
     // result on the way out:     out[n] <- dot[n] + res_out_add[n]
     const float *res_out_add = nullptr;
+    // (K8 product only) rows come in (gate_i, up_i) pairs: out[i] <- silu(dot[2 i]) * dot[2 i + 1], N / 2 results
+    bool silu_pairs = false;
     // LM head: the best (value, last index among equals; -1 without rows) of every workgroup, one entry
     // per workgroup of the launch (gemv_quant_workgroups of them)
     float *cand_v = nullptr;

@@ -191,6 +191,10 @@ class HfModel {
     struct LayerPacked { Buffer qkv, o, gate_up, down, qkv_bias, quant[7], planes[7], k8[4]; };
     int build_quant_planes();
     int build_k8_planes();
+    // gate and up rows of the K8 form interleaved (g0, u0, g1, u1, ...): SiLU * up is then the epilogue of the
+    // gate|up launch. Set for K-quant models that the whole-step launch does not serve (its instances read the
+    // rows stacked).
+    bool k8_pairs_ = false;
     // First member and member count of the stacked run that projection `which` of `layer` belongs to.
     void quant_run(int layer, int which, int *first, int *count) const;
     std::vector<LayerPacked> packed_;

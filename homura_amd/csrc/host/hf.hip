@@ -219,9 +219,10 @@ int HfModel::build_k8_planes() {
                 if (!packed_[l].quant[first]) return hm_set_error(ctx_, HM_ERR_STATE, "layer %d projection %d has no blocks", l, j);
                 size_t skip = 0;
                 for (int b = first; b < j; b++) skip += dtype_bytes_for_elements(t, (size_t)ndim[b] * K, nullptr);
+                const bool pairs = k8_pairs_ && g == 2;  // gate row r -> 2 r, up row r -> 2 r + 1
                 const int rc = pack_k8_rows(ctx_, t == DType::Q6_K ? HM_DTYPE_Q6_K : HM_DTYPE_Q4_K,
                                             packed_[l].quant[first].as<uint8_t>() + skip, ndim[j], K, dst.as<uint8_t>(),
-                                            dst.as<uint8_t>() + k8_plane_bytes(n, K), row0);
+                                            dst.as<uint8_t>() + k8_plane_bytes(n, K), pairs ? e : row0, pairs ? 2 : 1);
                 if (rc != HM_OK) return rc;
                 row0 += ndim[j];
             }
@@ -480,8 +481,12 @@ int HfModel::finalize(int max_seq_len) {
             fused_wf_ = FUSED_WF_K8;
             // the K8 form serves the whole-step launch and the per-projection decode GEMVs alike
             if (cfg_.hidden_size % 256 == 0 && cfg_.q_dim() % 256 == 0 && cfg_.intermediate_size % 256 == 0 &&
-                std::max({cfg_.hidden_size, cfg_.q_dim(), cfg_.intermediate_size}) <= 16384 && (rc = build_k8_planes()) != HM_OK)
-                return rc;
+                std::max({cfg_.hidden_size, cfg_.q_dim(), cfg_.intermediate_size}) <= 16384) {
+                const FusedShape fs8{cfg_.hidden_size, cfg_.num_attention_heads, cfg_.kv_heads(), cfg_.head_dim(),
+                                     cfg_.intermediate_size, FUSED_WF_K8};
+                k8_pairs_ = !decode_fused_supported(ctx_, fs8, cfg_.num_hidden_layers, max_seq_len, nullptr);
+                if ((rc = build_k8_planes()) != HM_OK) return rc;
+            }
         }
     }
     if (fused_format) {
@@ -1063,7 +1068,8 @@ int HfModel::emit_transformer_plan_quant() {
     // x / out replace the step's own activation and output slot.
     constexpr size_t NO = (size_t)-1;
     struct FuseSlots { size_t x = (size_t)-1, x2 = (size_t)-1, res_in = (size_t)-1, resid_out = (size_t)-1,
-                              norm_w = (size_t)-1, add = (size_t)-1, out = (size_t)-1; };
+                              norm_w = (size_t)-1, add = (size_t)-1, out = (size_t)-1;
+                       bool silu_pairs = false; };
     // A second run of the group that rides in the first run's launch (the two K-quant types side by side)
     struct PairedRun { size_t w_slot = (size_t)-1, out_slot = (size_t)-1; int64_t N = 0; DType dtype = DType::F32; std::string label; };
     auto quant_mm = [&](const char *label, DType wdt, int64_t K, int64_t N, bool reuse_act, FuseSlots fs,
@@ -1158,6 +1164,7 @@ int HfModel::emit_transformer_plan_quant() {
                     l.name = "gemv_k8[" + label + "]";
                     if (fs.norm_w != NO) l.name += fs.res_in != NO ? "+resid+norm" : "+norm";
                     if (fs.x2 != NO) l.name += "+silu";
+                    if (fs.silu_pairs) l.name += "+silu*up";
                     if (fs.add != NO) l.name += "+resid";
                     l.bytes_fixed = (double)k8.bytes() + K * 4.0 + n_all * 4.0;
                     const int64_t Kc = K, Nc = n_all;
@@ -1172,6 +1179,7 @@ int HfModel::emit_transformer_plan_quant() {
                         f.norm_w = f32(fs.norm_w);
                         f.eps = eps;
                         f.res_out_add = f32(fs.add);
+                        f.silu_pairs = fs.silu_pairs;
                         return gemv_k8_fused(sc.ctx, x, plane, records, out, (int)Kc, (int)Nc, f);
                     };
                     k.launches.push_back(std::move(l));
@@ -1426,6 +1434,10 @@ int HfModel::emit_transformer_plan_quant() {
                 fs.resid_out = s.residual;
                 fs.norm_w = s.post_ln;
             }
+            if (k8_pairs_ && packed_[i].k8[2]) {  // interleaved rows: SiLU * up leaves this launch (Step 13's work)
+                fs.silu_pairs = true;
+                fs.out = s.silu;
+            }
             quant_group(i, s.post_normed, hidden, {{"gate", 4, inter, s.gate_w, s.gate_out}, {"up", 5, inter, s.up_w, s.up_out}}, fs);
         }
         {  // Step 13: SiLU * Up (reference :1077-1103)
@@ -1447,8 +1459,10 @@ int HfModel::emit_transformer_plan_quant() {
         {  // Step 14: QuantMM Down; with a Q8_0 / Q4_0 matrix it takes SiLU*Up on the way in and ResAdd on the way out
             FuseSlots fs;
             if (fuse_down) {
-                fs.x = s.gate_out;
-                fs.x2 = s.up_out;
+                if (!(k8_pairs_ && packed_[i].k8[2])) {  // else SiLU * up already sits in the step's own input
+                    fs.x = s.gate_out;
+                    fs.x2 = s.up_out;
+                }
                 fs.add = s.residual;
                 fs.out = s.hidden_out;
             }

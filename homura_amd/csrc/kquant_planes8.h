@@ -13,6 +13,6 @@
 inline size_t k8_plane_bytes(int N, int K) { return (size_t)N * K; }
 inline size_t k8_record_bytes(int N, int K) { return (size_t)N * (K / 8 + K / 64); }
 // Re-packs `rows` rows of raw blocks (hm_dtype HM_DTYPE_Q4_K or HM_DTYPE_Q6_K, K % 256 == 0) into rows
-// [row0, row0 + rows) of the byte plane d_plane and of the records d_records.
+// row0, row0 + row_mult, row0 + 2 row_mult, ... of the byte plane d_plane and of the records d_records.
 int pack_k8_rows(hm_ctx *ctx, int hm_dtype, const uint8_t *d_blocks, int rows, int K, uint8_t *d_plane, uint8_t *d_records,
-                 int row0);
+                 int row0, int row_mult = 1);

@@ -15,15 +15,17 @@ __device__ __forceinline__ void q4k_scale_min(const uint8_t *raw, int j, int &sc
 
 // one thread per (row, 16-weight sub-block)
 __global__ __launch_bounds__(256) void pack_k8_kernel(const uint8_t *__restrict__ blocks, int q6, int rows, int K,
-                                                      uint8_t *__restrict__ plane, uint8_t *__restrict__ records, int row0) {
+                                                      uint8_t *__restrict__ plane, uint8_t *__restrict__ records, int row0,
+                                                      int row_mult) {
     const int per_row = K / 16;
     const size_t id = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (id >= (size_t)rows * per_row) return;
     const int r = (int)(id / per_row), s = (int)(id % per_row), b = s / 16, t = s % 16;
     const uint8_t *blk = blocks + ((size_t)r * (K / 256) + b) * (q6 ? 210 : 144);
     const size_t RS = (size_t)(K / 8 + K / 64);
-    uint8_t *out = plane + ((size_t)(row0 + r) * K) + (size_t)s * 16;
-    uint8_t *rec = records + (size_t)(row0 + r) * RS;
+    const size_t dst_row = (size_t)row0 + (size_t)r * row_mult;
+    uint8_t *out = plane + dst_row * K + (size_t)s * 16;
+    uint8_t *rec = records + dst_row * RS;
     int sc, mn;
     if (q6) {
         // reference dequant_q6_k (src/gguf.rs:886-917): weight w = 128 chunk + 32 grp + l
@@ -67,14 +69,14 @@ __global__ __launch_bounds__(256) void pack_k8_kernel(const uint8_t *__restrict_
 }  // namespace
 
 int pack_k8_rows(hm_ctx *ctx, int hm_dtype, const uint8_t *d_blocks, int rows, int K, uint8_t *d_plane, uint8_t *d_records,
-                 int row0) {
+                 int row0, int row_mult) {
     HM_CHECK_CTX(ctx);
     HM_REQUIRE(ctx, hm_dtype == HM_DTYPE_Q4_K || hm_dtype == HM_DTYPE_Q6_K, "pack_k8_rows: dtype %d is not a K-quant", hm_dtype);
-    HM_REQUIRE(ctx, d_blocks && d_plane && d_records && rows > 0 && K > 0 && K % 256 == 0 && row0 >= 0,
+    HM_REQUIRE(ctx, d_blocks && d_plane && d_records && rows > 0 && K > 0 && K % 256 == 0 && row0 >= 0 && row_mult >= 1,
                "pack_k8_rows: bad arguments (rows=%d K=%d)", rows, K);
     const size_t total = (size_t)rows * (K / 16);
     hipLaunchKernelGGL(pack_k8_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, ctx->stream, d_blocks,
-                       hm_dtype == HM_DTYPE_Q6_K ? 1 : 0, rows, K, d_plane, d_records, row0);
+                       hm_dtype == HM_DTYPE_Q6_K ? 1 : 0, rows, K, d_plane, d_records, row0, row_mult);
     HM_LAUNCH_CHECK(ctx);
     return HM_OK;
 }

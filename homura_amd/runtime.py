@@ -192,6 +192,15 @@ class Context:
     def gemv_q6_k(self, x, w, out, M, K, N):
         self._check(self.lib.hm_gemv_q6_k(self.h, x.ptr, w.ptr, out.ptr, M, K, N))
 
+    def pack_k8(self, dtype, blocks, N, K):
+        """Raw Q4_K / Q6_K blocks [N][K/256] (device buffer) -> a new device buffer holding their K8 form."""
+        k8 = self.alloc(self.lib.hm_k8_bytes(N, K))
+        self._check(self.lib.hm_pack_k8(self.h, dtype, blocks.ptr, N, k8.ptr, N, K, 0))
+        return k8
+
+    def gemv_k8(self, x, k8, out, M, K, N):
+        self._check(self.lib.hm_gemv_k8(self.h, x.ptr, k8.ptr, out.ptr, M, K, N))
+
     def gemv_q4_k_f32(self, x, w, out, M, K, N):
         self._check(self.lib.hm_gemv_q4_k_f32(self.h, x.ptr, w.ptr, out.ptr, M, K, N))
 

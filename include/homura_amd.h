@@ -144,6 +144,17 @@ int hm_dequant_q4_0(hm_ctx *ctx, const uint8_t *d_blocks, float *d_out, size_t n
  * f32 adds over units and blocks come in a different order. */
 int hm_gemv_q4_k(hm_ctx *ctx, const float *d_x, const uint8_t *d_w_blocks, float *d_out, int M, int K, int N);
 int hm_gemv_q6_k(hm_ctx *ctx, const float *d_x, const uint8_t *d_w_blocks, float *d_out, int M, int K, int N);
+/* The same product over the "K8" form of a Q4_K / Q6_K matrix, for a caller that keeps its weights on the device:
+ * every weight as one signed byte in a plane [N][K] (Q4_K: the nibble; Q6_K: the 6-bit value - 32), then, from byte
+ * N * K on, a record of K / 8 + K / 64 bytes per row: (scale, minimum factor) per 16 weights, then the f16 (d, dmin)
+ * per 256 - the same integers as the blocks at 1.14 bytes a weight, both types alike, so matrices of either type can be
+ * stacked by rows and multiplied in one call. hm_k8_bytes gives the size (0 for a bad shape), hm_pack_k8 fills rows
+ * [row0, row0 + rows) of a K8 matrix of N rows from `rows` rows of raw blocks of one type. hm_gemv_k8: the
+ * activation row is quantised to Q8_K inside the launch (no pass through memory), integer sums as the reference's
+ * (emit_quant.rs:165-816, :422-466). K % 256 == 0, K <= 16384, M <= 8. This is what the model's decode reads. */
+size_t hm_k8_bytes(int N, int K);
+int hm_pack_k8(hm_ctx *ctx, int hm_dtype, const uint8_t *d_blocks, int rows, uint8_t *d_k8, int N, int K, int row0);
+int hm_gemv_k8(hm_ctx *ctx, const float *d_x, const uint8_t *d_k8, float *d_out, int M, int K, int N);
 /* The f32 product with the dequantised weights: out[m][n] = sum_k x[m][k] * w[n][k], w = dequant_q4_k /
  * dequant_q6_k of the blocks (src/gguf.rs:835-917). This is what the reference computes where a K-quant
  * tensor feeds an f32 kernel: its loader dequantises the embedding and output matrices

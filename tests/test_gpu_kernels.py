@@ -349,6 +349,46 @@ def test_gemv_kquant(ctx, oracle, kind, M, K, N):
         b.free()
 
 
+@pytest.mark.parametrize("kind", ["q4_k", "q6_k", "mixed"])
+@pytest.mark.parametrize("M,K,N", [(1, 1024, 3072), (1, 1536, 2048), (1, 2048, 515), (2, 256, 7), (1, 3072, 1024),
+                                   (1, 4096, 130), (1, 5632, 2048), (1, 8960, 1536), (1, 16384, 33), (1, 768, 9)])
+def test_gemv_k8(ctx, oracle, kind, M, K, N):
+    """The K-quant product over the K8 form (rows cut across a workgroup's wavefronts, the activation row quantised
+    to Q8_K on the pieces in registers) against the oracle's product on the raw blocks: same integer sums, the f32
+    adds in another order. "mixed": the upper rows Q4_K, the lower ones Q6_K, stacked in one K8 matrix and
+    multiplied in one launch."""
+    from homura_amd.runtime import DTYPE_Q4_K, DTYPE_Q6_K
+    say(f"gemv_k8 {kind} M={M} K={K} N={N}")
+    x = synth.normal_f32(16, M * K, 1.0).reshape(M, K)
+    n4 = N if kind == "q4_k" else (0 if kind == "q6_k" else N // 2)
+    n6 = N - n4
+    dx, dout = ctx.to_device(x), ctx.empty(M * N)
+    k8 = ctx.alloc(ctx.lib.hm_k8_bytes(N, K))
+    want = np.zeros((M, N), np.float32)
+    held = []
+    if n4:
+        raw = synth.q4_k_blocks(15, n4 * K // 256)
+        want[:, :n4] = oracle.gemv_q4_k(x, raw, M, K, n4)
+        d = ctx.to_device(raw)
+        held.append(d)
+        ctx._check(ctx.lib.hm_pack_k8(ctx.h, DTYPE_Q4_K, d.ptr, n4, k8.ptr, N, K, 0))
+    if n6:
+        raw = synth.q6_k_blocks(17, n6 * K // 256)
+        want[:, n4:] = oracle.gemv_q6_k(x, raw, M, K, n6)
+        d = ctx.to_device(raw)
+        held.append(d)
+        ctx._check(ctx.lib.hm_pack_k8(ctx.h, DTYPE_Q6_K, d.ptr, n6, k8.ptr, N, K, n4))
+    ctx.gemv_k8(dx, k8, dout, M, K, N)
+    got = dout.download(np.float32, (M, N))
+    err = rel_err(got, want)
+    say(f"  rel err {err:.2e}")
+    assert err < (1e-4 if K <= 8192 else 3e-4)
+    with pytest.raises(HomuraError):
+        ctx.gemv_k8(dx, k8, dout, 1, 128, N)     # K not a multiple of 256
+    for b in held + [dx, dout, k8]:
+        b.free()
+
+
 # ── prefill GEMM (MFMA) ───────────────────────────────────────────────────────
 
 @pytest.mark.parametrize("layout", ["kn", "nk"])
