@@ -1317,11 +1317,20 @@ int HfModel::emit_transformer_plan_quant() {
             add_step(std::move(k), {s.hidden_in, s.input_ln}, {s.normed});
         }
         // Steps 2-4: QuantMM Q, K, V — one launch over the stacked q|k|v rows
+        // Where q|k|v multiply in one launch, the bias add of the next reference kernel rides out with it (the
+        // biases are adjacent like the rows): out = dot + bias, the same single addition.
+        bool bias_folded = false;
         {
             FuseSlots fs;
             if (fuse_in_norm) {
                 fs.x = s.hidden_in;
                 fs.norm_w = s.input_ln;
+            }
+            int first_run, count_run;
+            quant_run(i, 0, &first_run, &count_run);
+            if (s.q_b != (size_t)-1 && (packed_[i].k8[0] || count_run == 3)) {
+                fs.add = s.q_b;
+                bias_folded = true;
             }
             quant_group(i, s.normed, hidden, {{"q", 0, qd, s.q_w, s.q_out}, {"k", 1, kvd, s.k_w, s.k_out},
                                               {"v", 2, kvd, s.v_w, s.v_out}}, fs);
@@ -1331,11 +1340,13 @@ int HfModel::emit_transformer_plan_quant() {
             k.ops_label = qkn ? "PostQKV+QKNorm+RoPE" : "PostQKV+RoPE";
             std::vector<size_t> in{s.q_out, s.k_out, s.v_out, cos_s, sin_s};
             if (s.q_b != (size_t)-1) {
-                // the bias add of this reference kernel (src/hf/emitter_quant.rs:836-850): one launch
-                // over the adjacent q|k|v rows and the adjacent biases
                 in.push_back(s.q_b);
                 in.push_back(s.k_b);
                 in.push_back(s.v_b);
+            }
+            if (s.q_b != (size_t)-1 && !bias_folded) {
+                // the bias add of this reference kernel (src/hf/emitter_quant.rs:836-850): one launch
+                // over the adjacent q|k|v rows and the adjacent biases
                 DeviceLaunch l;
                 l.name = "qkv_bias_add";
                 l.bytes_fixed = (qd + 2 * kvd) * 4.0 * 3;
