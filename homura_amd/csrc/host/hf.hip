@@ -1300,6 +1300,10 @@ int HfModel::emit_transformer_plan_quant() {
         const bool fuse_in_norm = plain_group(i, {0, 1, 2}, hidden) && hidden <= 4096;
         const bool fuse_post_norm = plain_group(i, {4, 5}, hidden) && hidden <= 4096;
         const bool fuse_down = plain_group(i, {6}, inter);
+        // Long Q8_0 / Q4_0 rows go through the cut-row kernel, where every workgroup would redo SiLU * up over
+        // the whole row (8960 -> 1536: 12.6 us against 7.3 + a 2.5 us launch of its own; no gain below 8192)
+        const bool silu_apart = fuse_down && !packed_[i].k8[3] && inter >= 8192 &&
+                                (proj_dtype(i, 6) == DType::Q8_0 || proj_dtype(i, 6) == DType::Q4_0);
         {  // Step 1: pre-QKV RMSNorm (reference :713-791)
             CompiledKernel k;
             k.ops_label = "RMSNorm";
@@ -1454,7 +1458,7 @@ int HfModel::emit_transformer_plan_quant() {
         {  // Step 13: SiLU * Up (reference :1077-1103)
             CompiledKernel k;
             k.ops_label = "SiLU*Up";
-            if (!fuse_down) {
+            if (!fuse_down || silu_apart) {
                 DeviceLaunch l;
                 l.name = "silu_mul";
                 l.bytes_fixed = inter * 4.0 * 3;
@@ -1470,7 +1474,7 @@ int HfModel::emit_transformer_plan_quant() {
         {  // Step 14: QuantMM Down; with a Q8_0 / Q4_0 matrix it takes SiLU*Up on the way in and ResAdd on the way out
             FuseSlots fs;
             if (fuse_down) {
-                if (!(k8_pairs_ && packed_[i].k8[2])) {  // else SiLU * up already sits in the step's own input
+                if (!(k8_pairs_ && packed_[i].k8[2]) && !silu_apart) {  // else SiLU * up already sits in the step's own input
                     fs.x = s.gate_out;
                     fs.x2 = s.up_out;
                 }
