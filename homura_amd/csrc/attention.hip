@@ -55,7 +55,7 @@ __global__ __launch_bounds__(ATT_THREADS) void gqa_decode_attn_kernel(
     const float *__restrict__ q, uint16_t *__restrict__ kcache, uint16_t *__restrict__ vcache,
     float *__restrict__ out, float *__restrict__ part_o, float *__restrict__ part_ml, int kvh,
     int max_len, int kv_len_arg, int chunk, float scale, const DecodeState *__restrict__ state,
-    int lds_front, AttnFuse fuse) {
+    int lds_front, AttnFuse fuse, int g_total) {
     constexpr int LPR = HD / 8;      // lanes per row
     constexpr int RPI = WAVE / LPR;  // rows per wavefront instruction
     extern __shared__ float sm[];
@@ -67,8 +67,12 @@ __global__ __launch_bounds__(ATT_THREADS) void gqa_decode_attn_kernel(
 
     const int tid = threadIdx.x, lane = tid & (WAVE - 1), wave = tid / WAVE;
     const int sub = lane / LPR, dl = lane % LPR;
-    const int split = blockIdx.x, kvhd = blockIdx.y, b = blockIdx.z;
-    const int H = kvh * G;
+    // A workgroup serves G of the g_total query heads that share a KV head (all of them when g_total <= G):
+    // blockIdx.y = kv head * groups + group. Heads past g_total in the last group multiply zeros and write nothing.
+    const int ngroups = (g_total + G - 1) / G;
+    const int split = blockIdx.x, kvhd = blockIdx.y / ngroups, hg = blockIdx.y % ngroups, b = blockIdx.z;
+    const int g0 = hg * G, g_here = min(G, g_total - g0);
+    const int H = kvh * g_total;
     const int n0 = split * chunk;
     const size_t head_base = ((size_t)b * kvh + kvhd) * max_len * HD;
     const uint16_t *kbase = kcache + head_base + (size_t)n0 * HD + dl * 8;
@@ -109,7 +113,7 @@ __global__ __launch_bounds__(ATT_THREADS) void gqa_decode_attn_kernel(
         for (int j = 0; j < TMAX; j++) {
             const int t = wave + j * ATT_WAVES;
             const float *src = nullptr;
-            if (t < G) src = fuse.qkv_raw + (size_t)(kvhd * G + t) * HD;
+            if (t < g_here) src = fuse.qkv_raw + (size_t)(kvhd * g_total + g0 + t) * HD;
             else if (owner && t == G) src = fuse.qkv_raw + (size_t)H * HD + (size_t)kvhd * HD;
             else if (owner && t == G + 1) src = fuse.qkv_raw + (size_t)(H + kvh) * HD + (size_t)kvhd * HD;
             rlo[j] = (src && on) ? src[lane] : 0.f;
@@ -148,8 +152,10 @@ __global__ __launch_bounds__(ATT_THREADS) void gqa_decode_attn_kernel(
                 if (on) {
                     uint16_t *dst = kcache + head_base + (size_t)pos * HD;
                     const uint16_t r_lo = f32_to_bf16_rne_dev(lo), r_hi = f32_to_bf16_rne_dev(hi);
-                    dst[lane] = r_lo;
-                    dst[lane + HALF] = r_hi;
+                    if (hg == 0) {  // every group rounds the row for itself, the first one appends it
+                        dst[lane] = r_lo;
+                        dst[lane + HALF] = r_hi;
+                    }
                     knew[lane] = __uint_as_float((uint32_t)r_lo << 16);
                     knew[lane + HALF] = __uint_as_float((uint32_t)r_hi << 16);
                 }
@@ -157,8 +163,10 @@ __global__ __launch_bounds__(ATT_THREADS) void gqa_decode_attn_kernel(
                 if (on) {
                     uint16_t *dst = vcache + head_base + (size_t)pos * HD;
                     const uint16_t r_lo = f32_to_bf16_rne_dev(rlo[j]), r_hi = f32_to_bf16_rne_dev(rhi[j]);
-                    dst[lane] = r_lo;
-                    dst[lane + HALF] = r_hi;
+                    if (hg == 0) {
+                        dst[lane] = r_lo;
+                        dst[lane + HALF] = r_hi;
+                    }
                     vnew[lane] = __uint_as_float((uint32_t)r_lo << 16);
                     vnew[lane + HALF] = __uint_as_float((uint32_t)r_hi << 16);
                 }
@@ -166,7 +174,7 @@ __global__ __launch_bounds__(ATT_THREADS) void gqa_decode_attn_kernel(
         }
     } else {
         for (int i = tid; i < G * HD; i += ATT_THREADS)
-            qs[i / HD][i % HD] = q[((size_t)b * H + kvhd * G) * HD + i];
+            qs[i / HD][i % HD] = i < g_here * HD ? q[((size_t)b * H + kvhd * g_total + g0) * HD + i] : 0.f;
     }
     __syncthreads();
 
@@ -266,21 +274,21 @@ __global__ __launch_bounds__(ATT_THREADS) void gqa_decode_attn_kernel(
     __syncthreads();
 
     const size_t pair = (size_t)b * kvh + kvhd;
-    float *po = part_o + (pair * nsplit + split) * G * HD;
-    float *pml = part_ml + (pair * nsplit + split) * G * 2;
-    for (int i = tid; i < G * HD; i += ATT_THREADS) {
+    float *po = part_o + ((pair * nsplit + split) * g_total + g0) * HD;
+    float *pml = part_ml + ((pair * nsplit + split) * g_total + g0) * 2;
+    for (int i = tid; i < g_here * HD; i += ATT_THREADS) {
         float v = 0.f;
 #pragma unroll
         for (int w = 0; w < ATT_WAVES * RPI; w++) v += red[(size_t)w * G * HD + i];
         if (nsplit == 1) {
             const int gi = i / HD, d = i % HD;
-            out[((size_t)b * H + kvhd * G + gi) * HD + d] = v / s_l[gi];
+            out[((size_t)b * H + kvhd * g_total + g0 + gi) * HD + d] = v / s_l[gi];
         } else {
             po[i] = v;
         }
     }
     if (nsplit == 1) return;
-    if (tid < G) {
+    if (tid < g_here) {
         pml[tid * 2] = s_m[tid];
         pml[tid * 2 + 1] = s_l[tid];
     }
@@ -578,11 +586,16 @@ __global__ void kv_append_kernel(uint16_t *__restrict__ kc, uint16_t *__restrict
     vc[dst] = f32_to_bf16_rne_dev(v[i]);
 }
 
+// G = the query heads that share a KV head. A workgroup of the split kernel serves GB of them: all when there are
+// at most four, else two (the kernel's length grows with the heads it serves, and with two KV heads a 1024-row
+// cache gives only 32 workgroups of all heads; groups of three or four measured slower than two at G = 6 .. 8,
+// single heads slower again).
 template <int HD, int G>
 int launch_attn(hm_ctx *ctx, const AttnArgs &a, int nsplit, int chunk) {
-    // scores [G][chunk] + partials of every row-subgroup of every wavefront [4 * RPI][G][HD]
-    const size_t front = (size_t)G * chunk;
-    const size_t lds = (front + (size_t)ATT_WAVES * (WAVE / (HD / 8)) * G * HD) * sizeof(float);
+    constexpr int GB = G <= 4 ? G : 2, NG = (G + GB - 1) / GB;
+    // scores [GB][chunk] + partials of every row-subgroup of every wavefront [4 * RPI][GB][HD]
+    const size_t front = (size_t)GB * chunk;
+    const size_t lds = (front + (size_t)ATT_WAVES * (WAVE / (HD / 8)) * GB * HD) * sizeof(float);
     const size_t pairs = (size_t)a.B * a.kvh;
     float *part_o = a.partials ? a.partials : (float *)ctx->workspace;
     float *part_ml = part_o + pairs * nsplit * G * HD;
@@ -590,15 +603,15 @@ int launch_attn(hm_ctx *ctx, const AttnArgs &a, int nsplit, int chunk) {
     if (a.phase != AttnArgs::FOLD_ONLY) {
         static bool lds_limit_raised = false;  // per instantiation; large groups need more than 64 KiB
         if (lds > 64 * 1024 && !lds_limit_raised) {
-            HM_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(&gqa_decode_attn_kernel<HD, G>),
+            HM_HIP(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(&gqa_decode_attn_kernel<HD, GB>),
                                             hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024));
             lds_limit_raised = true;
         }
         HM_REQUIRE(ctx, lds <= 96 * 1024, "gqa_decode_attn: LDS need %zu too large", lds);
-        hipLaunchKernelGGL((gqa_decode_attn_kernel<HD, G>), dim3(nsplit, a.kvh, a.B), dim3(ATT_THREADS),
+        hipLaunchKernelGGL((gqa_decode_attn_kernel<HD, GB>), dim3(nsplit, a.kvh * NG, a.B), dim3(ATT_THREADS),
                            lds, ctx->stream, a.q, const_cast<uint16_t *>(a.kcache),
                            const_cast<uint16_t *>(a.vcache), a.out, part_o, part_ml, a.kvh, a.max_len,
-                           a.kv_len, chunk, a.scale, a.state, (int)front, f);
+                           a.kv_len, chunk, a.scale, a.state, (int)front, f, G);
         HM_LAUNCH_CHECK(ctx);
     }
     // nsplit is the grid's split count: 1 means no call can ever need a fold
