@@ -325,7 +325,7 @@ __global__ __launch_bounds__(PTHREADS) void gemv_planes_kernel(const float *__re
 // requested before anything waits, the activation pieces first; the light ops in front of the product
 // (SiLU pair, residual add) are applied to the pieces in registers; the four partial sums of a row meet in
 // LDS and are added in wavefront order. No RMSNorm here (rows that long are normalised by their own launch).
-template <int QT, int R, int NC, bool FUSED>
+template <int QT, int R, int NC, bool FUSED, int WPS>
 __global__ __launch_bounds__(PTHREADS) void gemv_planes_splitk_kernel(const float *__restrict__ x, const uint8_t *__restrict__ quants,
                                                                       const uint16_t *__restrict__ scales, float *__restrict__ out,
                                                                       int K, int N, const QuantFuse fuse_arg) {
@@ -334,7 +334,11 @@ __global__ __launch_bounds__(PTHREADS) void gemv_planes_splitk_kernel(const floa
     __shared__ float part[PWAVES][R];
     const int lane = threadIdx.x & (WAVE - 1);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);
-    const int row0 = blockIdx.x * R;
+    // WPS wavefronts (as many as a row has chunks, so that none idles) share a set of R rows; a workgroup works
+    // on PWAVES / WPS sets
+    constexpr int SETS = PWAVES / WPS;
+    const int set = wave / WPS, wis = wave % WPS;
+    const int row0 = (blockIdx.x * SETS + set) * R;
     const size_t qrow = QT == 0 ? (size_t)K : (size_t)K / 2;
     const int nb = K / 32;
     const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
@@ -344,7 +348,7 @@ __global__ __launch_bounds__(PTHREADS) void gemv_planes_splitk_kernel(const floa
     const float *second = fuse.x2 ? fuse.x2 : fuse.res_in;
 #pragma unroll
     for (int c = 0; c < NC; c++) {
-        const int k = ((c * PWAVES + wave) * WAVE + lane) * KPL;
+        const int k = ((c * WPS + wis) * WAVE + lane) * KPL;
 #pragma unroll
         for (int j = 0; j < XV; j++) {
             xr[c][j] = k < K ? *reinterpret_cast<const f32x4 *>(x + k + 4 * j) : zero4;
@@ -353,7 +357,7 @@ __global__ __launch_bounds__(PTHREADS) void gemv_planes_splitk_kernel(const floa
     }
 #pragma unroll
     for (int c = 0; c < NC; c++) {
-        const int k = ((c * PWAVES + wave) * WAVE + lane) * KPL;
+        const int k = ((c * WPS + wis) * WAVE + lane) * KPL;
         const int kc = k < K ? k : 0;  // units past the row end re-read its first one against activations of zero
 #pragma unroll
         for (int r = 0; r < R; r++) {
@@ -375,11 +379,11 @@ __global__ __launch_bounds__(PTHREADS) void gemv_planes_splitk_kernel(const floa
         } else if (fuse.res_in) {
 #pragma unroll
             for (int c = 0; c < NC; c++) {
-                const int k = ((c * PWAVES + wave) * WAVE + lane) * KPL;
+                const int k = ((c * WPS + wis) * WAVE + lane) * KPL;
 #pragma unroll
                 for (int j = 0; j < XV; j++) {
                     xr[c][j] += ar[c][j];
-                    if (fuse.resid_out && blockIdx.x == 0 && k < K) *reinterpret_cast<f32x4 *>(fuse.resid_out + k + 4 * j) = xr[c][j];
+                    if (fuse.resid_out && blockIdx.x == 0 && set == 0 && k < K) *reinterpret_cast<f32x4 *>(fuse.resid_out + k + 4 * j) = xr[c][j];
                 }
             }
         }
@@ -428,12 +432,15 @@ __global__ __launch_bounds__(PTHREADS) void gemv_planes_splitk_kernel(const floa
     }
     __syncthreads();
     const int t = threadIdx.x;
-    if (t < R && row0 + t < N) {
-        float v = part[0][t];
+    if (t < SETS * R) {
+        const int ts = t / R, tr = t % R, row = (blockIdx.x * SETS + ts) * R + tr;
+        if (row < N) {
+            float v = part[ts * WPS][tr];
 #pragma unroll
-        for (int w = 1; w < PWAVES; w++) v += part[w][t];
-        if (fuse.res_out_add) v = v + fuse.res_out_add[row0 + t];
-        out[row0 + t] = v;
+            for (int w = 1; w < WPS; w++) v += part[ts * WPS + w][tr];
+            if (fuse.res_out_add) v = v + fuse.res_out_add[row];
+            out[row] = v;
+        }
     }
 }
 
@@ -814,30 +821,43 @@ int planes_launch(hm_ctx *ctx, const char *name, const float *d_x, const uint8_t
         const char *e = getenv("HOMURA_PLANES_SPLITK");
         return e && atoi(e) != 0;
     }();
-    if ((K > 4096 || force_cut) && !fuse.norm_w && !fuse.cand_v) {
-        const int round_k = PWAVES * WAVE * (q4 ? 32 : 16);
-        const int nc = (K + round_k - 1) / round_k;
+    // ... and Q8_0 matrices of fewer than 32768 rows at any width (2048 -> 5632: 4.6 us against 5.3; Q4_0 rows up to
+    // 4096 and the LM heads measured no faster that way)
+    if ((K > 4096 || force_cut || (!q4 && N < 32768)) && !fuse.norm_w && !fuse.cand_v) {
+        const int chunk_k = WAVE * (q4 ? 32 : 16);
+        const int wps = K <= chunk_k ? 1 : (K <= 2 * chunk_k ? 2 : 4);
+        const int nc = (K + wps * chunk_k - 1) / (wps * chunk_k);
         for (int m = 0; m < M; m++) {
             const float *xm = d_x + (size_t)m * K;
             float *om = d_out + (size_t)m * N;
-#define HM_CUT(RR, CC)                                                                                                      \
+#define HM_CUT(RR, CC, WW)                                                                                                  \
     do {                                                                                                                    \
-        const int grid = (N + RR - 1) / RR;                                                                                 \
+        const int rows_wg = RR * (PWAVES / WW), grid = (N + rows_wg - 1) / rows_wg;                                         \
         if (fused)                                                                                                          \
-            hipLaunchKernelGGL((gemv_planes_splitk_kernel<QT, RR, CC, true>), dim3(grid), dim3(PTHREADS), 0, ctx->stream, xm, \
-                               quants, scales, om, K, N, fuse);                                                             \
+            hipLaunchKernelGGL((gemv_planes_splitk_kernel<QT, RR, CC, true, WW>), dim3(grid), dim3(PTHREADS), 0, ctx->stream, \
+                               xm, quants, scales, om, K, N, fuse);                                                         \
         else                                                                                                                \
-            hipLaunchKernelGGL((gemv_planes_splitk_kernel<QT, RR, CC, false>), dim3(grid), dim3(PTHREADS), 0, ctx->stream, xm, \
-                               quants, scales, om, K, N, fuse);                                                             \
+            hipLaunchKernelGGL((gemv_planes_splitk_kernel<QT, RR, CC, false, WW>), dim3(grid), dim3(PTHREADS), 0, ctx->stream, \
+                               xm, quants, scales, om, K, N, fuse);                                                         \
     } while (0)
-            if (!q4) {
-                if (nc == 1) HM_CUT(8, 1);
-                else if (nc == 2) HM_CUT(8, 2);
-                else if (nc == 3) { if (fused) HM_CUT(4, 3); else HM_CUT(8, 3); }
-                else HM_CUT(4, 4);
+            if (wps <= 2) {
+                // rows a set: as many as leave a thousand workgroups or so (every set re-reads the activation pieces)
+                const int sets = PWAVES / wps;
+                int r = N / (16 * sets) >= 1024 ? 16 : (N / (8 * sets) >= 512 ? 8 : 4);
+                if (fused && r > 8) r = 8;
+                if (wps == 1) {
+                    if (r == 16) HM_CUT(16, 1, 1); else if (r == 8) HM_CUT(8, 1, 1); else HM_CUT(4, 1, 1);
+                } else {
+                    if (r == 16) HM_CUT(16, 1, 2); else if (r == 8) HM_CUT(8, 1, 2); else HM_CUT(4, 1, 2);
+                }
+            } else if (!q4) {
+                if (nc == 1) HM_CUT(8, 1, 4);
+                else if (nc == 2) HM_CUT(8, 2, 4);
+                else if (nc == 3) { if (fused) HM_CUT(4, 3, 4); else HM_CUT(8, 3, 4); }
+                else HM_CUT(4, 4, 4);
             } else {
-                if (nc == 1) { if (fused) HM_CUT(8, 1); else HM_CUT(16, 1); }
-                else { if (fused) HM_CUT(4, 2); else HM_CUT(8, 2); }
+                if (nc == 1) { if (fused) HM_CUT(8, 1, 4); else HM_CUT(16, 1, 4); }
+                else { if (fused) HM_CUT(4, 2, 4); else HM_CUT(8, 2, 4); }
             }
 #undef HM_CUT
             HM_LAUNCH_CHECK(ctx);
