@@ -325,13 +325,16 @@ __global__ __launch_bounds__(PTHREADS) void gemv_planes_kernel(const float *__re
 // requested before anything waits, the activation pieces first; the light ops in front of the product
 // (SiLU pair, residual add) are applied to the pieces in registers; the four partial sums of a row meet in
 // LDS and are added in wavefront order. No RMSNorm here (rows that long are normalised by their own launch).
-template <int QT, int R, int NC, bool FUSED, int WPS>
+// MODE 0: plain row. 1: a second operand (x2 or res_in). 2: RMSNorm, with or without res_in.
+template <int QT, int R, int NC, int MODE, int WPS>
 __global__ __launch_bounds__(PTHREADS) void gemv_planes_splitk_kernel(const float *__restrict__ x, const uint8_t *__restrict__ quants,
                                                                       const uint16_t *__restrict__ scales, float *__restrict__ out,
                                                                       int K, int N, const QuantFuse fuse_arg) {
+    constexpr bool FUSED = MODE >= 1;
     const QuantFuse fuse = FUSED ? fuse_arg : QuantFuse();
     constexpr int KPL = QT == 0 ? 16 : 32, XV = KPL / 4;  // weights and f32x4 activation pieces of a unit
     __shared__ float part[PWAVES][R];
+    __shared__ float red[PWAVES];
     const int lane = threadIdx.x & (WAVE - 1);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);
     // WPS wavefronts (as many as a row has chunks, so that none idles) share a set of R rows; a workgroup works
@@ -342,7 +345,7 @@ __global__ __launch_bounds__(PTHREADS) void gemv_planes_splitk_kernel(const floa
     const size_t qrow = QT == 0 ? (size_t)K : (size_t)K / 2;
     const int nb = K / 32;
     const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
-    f32x4 xr[NC][XV], ar[FUSED ? NC : 1][FUSED ? XV : 1];
+    f32x4 xr[NC][XV], ar[FUSED ? NC : 1][FUSED ? XV : 1], nr[MODE == 2 ? NC : 1][MODE == 2 ? XV : 1];
     u32x4 qw[NC][R];
     uint32_t sc[NC][R];
     const float *second = fuse.x2 ? fuse.x2 : fuse.res_in;
@@ -353,6 +356,7 @@ __global__ __launch_bounds__(PTHREADS) void gemv_planes_splitk_kernel(const floa
         for (int j = 0; j < XV; j++) {
             xr[c][j] = k < K ? *reinterpret_cast<const f32x4 *>(x + k + 4 * j) : zero4;
             if constexpr (FUSED) ar[c][j] = (second && k < K) ? *reinterpret_cast<const f32x4 *>(second + k + 4 * j) : zero4;
+            if constexpr (MODE == 2) nr[c][j] = (fuse.norm_w && k < K) ? *reinterpret_cast<const f32x4 *>(fuse.norm_w + k + 4 * j) : zero4;
         }
     }
 #pragma unroll
@@ -386,6 +390,30 @@ __global__ __launch_bounds__(PTHREADS) void gemv_planes_splitk_kernel(const floa
                     if (fuse.resid_out && blockIdx.x == 0 && set == 0 && k < K) *reinterpret_cast<f32x4 *>(fuse.resid_out + k + 4 * j) = xr[c][j];
                 }
             }
+        }
+    }
+    if constexpr (MODE == 2) {
+        // RMSNorm on the pieces: the set's wavefronts cover the row exactly once, their sums of squares meet in LDS
+        if (fuse.norm_w) {
+            float ss = 0.f;
+#pragma unroll
+            for (int c = 0; c < NC; c++)
+#pragma unroll
+                for (int j = 0; j < XV; j++)
+                    ss += (xr[c][j][0] * xr[c][j][0] + xr[c][j][1] * xr[c][j][1]) + (xr[c][j][2] * xr[c][j][2] + xr[c][j][3] * xr[c][j][3]);
+            ss = wave_sum(ss);
+            if (lane == 0) red[wave] = ss;
+            __syncthreads();
+            float tot = 0.f;
+#pragma unroll
+            for (int w = 0; w < WPS; w++) tot += red[set * WPS + w];
+            const float inv = 1.0f / sqrtf(tot / (float)K + fuse.eps);
+#pragma unroll
+            for (int c = 0; c < NC; c++)
+#pragma unroll
+                for (int j = 0; j < XV; j++)
+#pragma unroll
+                    for (int e = 0; e < 4; e++) xr[c][j][e] = (xr[c][j][e] * inv) * nr[c][j][e];
         }
     }
     float a[R];
@@ -822,8 +850,10 @@ int planes_launch(hm_ctx *ctx, const char *name, const float *d_x, const uint8_t
         return e && atoi(e) != 0;
     }();
     // ... and Q8_0 matrices of fewer than 32768 rows at any width (2048 -> 5632: 4.6 us against 5.3; Q4_0 rows up to
-    // 4096 and the LM heads measured no faster that way)
-    if ((K > 4096 || force_cut || (!q4 && N < 32768)) && !fuse.norm_w && !fuse.cand_v) {
+    // 4096 and the LM heads measured no faster that way), with an RMSNorm riding in up to 16 M weights (beyond,
+    // the trips of gemv_planes_kernel, which prepares the row once per workgroup, are faster)
+    if ((K > 4096 || force_cut || (!q4 && N < 32768)) && !(fuse.norm_w && (K > 4096 || q4 || (size_t)N * K > ((size_t)16 << 20))) && !fuse.cand_v) {
+        const int mode = fuse.norm_w ? 2 : ((fuse.x2 || fuse.res_in) ? 1 : 0);
         const int chunk_k = WAVE * (q4 ? 32 : 16);
         const int wps = K <= chunk_k ? 1 : (K <= 2 * chunk_k ? 2 : 4);
         const int nc = (K + wps * chunk_k - 1) / (wps * chunk_k);
@@ -833,11 +863,15 @@ int planes_launch(hm_ctx *ctx, const char *name, const float *d_x, const uint8_t
 #define HM_CUT(RR, CC, WW)                                                                                                  \
     do {                                                                                                                    \
         const int rows_wg = RR * (PWAVES / WW), grid = (N + rows_wg - 1) / rows_wg;                                         \
-        if (fused)                                                                                                          \
-            hipLaunchKernelGGL((gemv_planes_splitk_kernel<QT, RR, CC, true, WW>), dim3(grid), dim3(PTHREADS), 0, ctx->stream, \
+        if (mode == 2) {                                                                                                    \
+            if constexpr (CC == 1 && QT == 0)                                                                               \
+                hipLaunchKernelGGL((gemv_planes_splitk_kernel<QT, RR, CC, 2, WW>), dim3(grid), dim3(PTHREADS), 0, ctx->stream, \
+                                   xm, quants, scales, om, K, N, fuse);                                                     \
+        } else if (fused)                                                                                                   \
+            hipLaunchKernelGGL((gemv_planes_splitk_kernel<QT, RR, CC, 1, WW>), dim3(grid), dim3(PTHREADS), 0, ctx->stream,  \
                                xm, quants, scales, om, K, N, fuse);                                                         \
         else                                                                                                                \
-            hipLaunchKernelGGL((gemv_planes_splitk_kernel<QT, RR, CC, false, WW>), dim3(grid), dim3(PTHREADS), 0, ctx->stream, \
+            hipLaunchKernelGGL((gemv_planes_splitk_kernel<QT, RR, CC, 0, WW>), dim3(grid), dim3(PTHREADS), 0, ctx->stream,  \
                                xm, quants, scales, om, K, N, fuse);                                                         \
     } while (0)
             if (wps <= 2) {
