@@ -6,6 +6,10 @@
 // from generated range tables.
 #include "tokenizer.h"
 
+#include <cctype>
+#include <cstdio>
+#include <queue>
+
 #include <algorithm>
 #include <cstdio>
 #include <cstring>
@@ -296,16 +300,22 @@ std::unique_ptr<BpeTokenizer> BpeTokenizer::from_tokenizer_json(const std::strin
     const Json *vocab = model->get("vocab"), *merges = model->get("merges");
     if ((mtype && *mtype != "BPE") || !vocab || vocab->kind != Json::Obj || !merges || merges->kind != Json::Arr)
         return refuse("model is not a BPE with \"vocab\" and \"merges\"");
+    // the SentencePiece-style family (Llama-2, TinyLlama, Mistral) says byte_fallback; the byte-level one does not
+    const bool spm = json_flag(*model, "byte_fallback");
     for (const char *key : {"unk_token", "continuing_subword_prefix", "end_of_word_suffix", "dropout"}) {
         const Json *v = model->get(key);
+        if (spm && std::string(key) == "unk_token") continue;
         if (v && v->kind != Json::Null && !(v->kind == Json::Str && v->str.empty()))
             return refuse(std::string("BPE option \"") + key + "\" is not supported");
     }
-    if (json_flag(*model, "byte_fallback") || json_flag(*model, "fuse_unk"))
-        return refuse("BPE byte_fallback / fuse_unk are not supported");
+    if (!spm && json_flag(*model, "fuse_unk")) return refuse("BPE fuse_unk without byte_fallback is not supported");
+    if (spm && (!json_flag(*model, "fuse_unk") || !json_str(*model, "unk_token")))
+        return refuse("BPE byte_fallback is supported with fuse_unk and an unk_token (the Llama-2 family)");
+    if (spm && json_flag(*model, "ignore_merges")) return refuse("BPE byte_fallback with ignore_merges is not supported");
 
     std::unique_ptr<BpeTokenizer> t(new BpeTokenizer());
     t->hf_decode_ = true;
+    t->spm_ = spm;
     t->ignore_merges_ = json_flag(*model, "ignore_merges");
     for (const auto &kv : vocab->obj) {
         if (kv.second.kind != Json::Num || kv.second.num < 0 || kv.second.num > 4294967295.0)
@@ -324,15 +334,59 @@ std::unique_ptr<BpeTokenizer> BpeTokenizer::from_tokenizer_json(const std::strin
         }
     }
     t->init_byte_alphabet();
+    if (spm) {
+        static const char U2581[] = "\xE2\x96\x81";  // U+2581, the stand-in for a space
+        t->unk_id_ = t->token_to_id(*json_str(*model, "unk_token"));
+        if (t->unk_id_ < 0) return refuse("unk_token is not in the vocabulary");
+        for (int b = 0; b < 256; b++) {
+            char name[8];
+            snprintf(name, sizeof(name), "<0x%02X>", b);
+            t->byte_ids_[b] = t->token_to_id(name);
+        }
+        // normaliser: Sequence[Prepend(U+2581), Replace(" " -> U+2581)]
+        const Json *nz = j.get("normalizer");
+        const Json *parts = nz && nz->kind == Json::Obj ? nz->get("normalizers") : nullptr;
+        bool ok = nz && nz->kind == Json::Obj && json_str(*nz, "type") && *json_str(*nz, "type") == "Sequence" && parts &&
+                  parts->kind == Json::Arr && parts->arr.size() == 2;
+        if (ok) {
+            const Json &pre = parts->arr[0], &rep = parts->arr[1];
+            const Json *pat = rep.kind == Json::Obj ? rep.get("pattern") : nullptr;
+            ok = pre.kind == Json::Obj && json_str(pre, "type") && *json_str(pre, "type") == "Prepend" && json_str(pre, "prepend") &&
+                 *json_str(pre, "prepend") == U2581 && rep.kind == Json::Obj && json_str(rep, "type") &&
+                 *json_str(rep, "type") == "Replace" && pat && pat->kind == Json::Obj && json_str(*pat, "String") &&
+                 *json_str(*pat, "String") == " " && json_str(rep, "content") && *json_str(rep, "content") == U2581;
+        }
+        if (!ok) return refuse("normalizer must be Sequence[Prepend(U+2581), Replace(\" \" -> U+2581)] for a byte_fallback BPE");
+        if (const Json *pt = j.get("pre_tokenizer"); pt && pt->kind != Json::Null)
+            return refuse("a byte_fallback BPE must have no pre-tokeniser");
+        // decoder: Sequence[Replace(U+2581 -> " "), ByteFallback, Fuse, Strip(" ", 1, 0)]
+        const Json *dec = j.get("decoder");
+        const Json *dparts = dec && dec->kind == Json::Obj ? dec->get("decoders") : nullptr;
+        ok = dec && dec->kind == Json::Obj && json_str(*dec, "type") && *json_str(*dec, "type") == "Sequence" && dparts &&
+             dparts->kind == Json::Arr && dparts->arr.size() == 4;
+        if (ok) {
+            const Json &d0 = dparts->arr[0], &d1 = dparts->arr[1], &d2 = dparts->arr[2], &d3 = dparts->arr[3];
+            auto type_is = [](const Json &e, const char *name) {
+                return e.kind == Json::Obj && json_str(e, "type") && *json_str(e, "type") == name;
+            };
+            const Json *pat = d0.kind == Json::Obj ? d0.get("pattern") : nullptr;
+            const Json *start = d3.kind == Json::Obj ? d3.get("start") : nullptr, *stop = d3.kind == Json::Obj ? d3.get("stop") : nullptr;
+            ok = type_is(d0, "Replace") && pat && pat->kind == Json::Obj && json_str(*pat, "String") && *json_str(*pat, "String") == U2581 &&
+                 json_str(d0, "content") && *json_str(d0, "content") == " " && type_is(d1, "ByteFallback") && type_is(d2, "Fuse") &&
+                 type_is(d3, "Strip") && json_str(d3, "content") && *json_str(d3, "content") == " " && start &&
+                 start->kind == Json::Num && start->num == 1 && stop && stop->kind == Json::Num && stop->num == 0;
+        }
+        if (!ok) return refuse("decoder must be Sequence[Replace(U+2581 -> \" \"), ByteFallback, Fuse, Strip(\" \", 1, 0)] for a byte_fallback BPE");
+    }
 
     // normaliser: none, or NFC (left to the caller)
-    if (const Json *nz = j.get("normalizer"); nz && nz->kind == Json::Obj) {
+    if (const Json *nz = j.get("normalizer"); !spm && nz && nz->kind == Json::Obj) {
         const std::string *ty = json_str(*nz, "type");
         if (!ty || *ty != "NFC") return refuse("normalizer " + (ty ? *ty : std::string("?")) + " is not supported (none or NFC)");
         t->wants_nfc_ = true;
     }
     // pre-tokeniser: Sequence[Split(pattern, Isolated), ByteLevel(use_regex = false)]
-    {
+    if (!spm) {
         const Json *pt = j.get("pre_tokenizer");
         std::vector<const Json *> parts;
         if (pt && pt->kind == Json::Obj) {
@@ -366,7 +420,7 @@ std::unique_ptr<BpeTokenizer> BpeTokenizer::from_tokenizer_json(const std::strin
         }
         if (!have_split || !have_bytes) return refuse("pre-tokeniser must be Split + ByteLevel");
     }
-    if (const Json *dec = j.get("decoder"); !dec || dec->kind != Json::Obj || !json_str(*dec, "type") || *json_str(*dec, "type") != "ByteLevel")
+    if (const Json *dec = j.get("decoder"); !spm && (!dec || dec->kind != Json::Obj || !json_str(*dec, "type") || *json_str(*dec, "type") != "ByteLevel"))
         return refuse("decoder must be ByteLevel");
 
     // added tokens
@@ -377,6 +431,8 @@ std::unique_ptr<BpeTokenizer> BpeTokenizer::from_tokenizer_json(const std::strin
             if (!id || id->kind != Json::Num || !content || content->empty()) return refuse("malformed added token");
             if (json_flag(a, "lstrip") || json_flag(a, "rstrip") || json_flag(a, "single_word"))
                 return refuse("added token \"" + *content + "\": lstrip / rstrip / single_word are not supported");
+            if (spm && json_flag(a, "normalized"))
+                return refuse("added token \"" + *content + "\": normalized added tokens are not supported with a byte_fallback BPE");
             t->added_.push_back(Added{*content, (uint32_t)id->num, json_flag(a, "special")});
         }
         std::stable_sort(t->added_.begin(), t->added_.end(),
@@ -457,7 +513,156 @@ std::vector<std::string> BpeTokenizer::bpe(const std::string &mapped) const {
     return word;
 }
 
+// The SentencePiece-style family as the `tokenizers` crate runs it (models/bpe: merge_word and Word::merge_all):
+// the normalised stretch - U+2581 in front, spaces replaced by U+2581 - is one word; a character that is a
+// vocabulary entry is a symbol, any other goes in as its UTF-8 bytes "<0xXX>" (or as the unknown token, runs of
+// which are fused, when a byte token is missing); then the adjacent pair with the lowest merge rank, leftmost
+// among equals, is merged until none is left. A heap of candidate pairs keeps this near-linear for long texts.
+void BpeTokenizer::encode_plain_spm(const char *text, size_t len, std::vector<uint32_t> *ids) const {
+    if (len == 0) return;
+    static const char U2581[] = "\xE2\x96\x81";
+    std::string norm(U2581);
+    for (size_t i = 0; i < len; i++) {
+        if (text[i] == ' ') norm += U2581;
+        else norm.push_back(text[i]);
+    }
+    struct Sym {
+        std::string s;
+        int64_t id;  // vocabulary id; merges look the strings up
+        int prev, next;
+        uint32_t ver;
+        bool alive;
+    };
+    std::vector<Sym> w;
+    auto push = [&](std::string str, int64_t id) {
+        Sym y{std::move(str), id, (int)w.size() - 1, -1, 0, true};
+        if (!w.empty()) w.back().next = (int)w.size();
+        w.push_back(std::move(y));
+    };
+    // An unknown character waits (fuse_unk: a run of them is one unknown token) until the next vocabulary character or
+    // the end of the word puts it in; byte tokens in between do not, exactly as the crate's merge_word has it.
+    bool unk_waits = false;
+    auto put_unk = [&]() {
+        if (unk_waits) push(decoder_.at((uint32_t)unk_id_), unk_id_);
+        unk_waits = false;
+    };
+    for (size_t i = 0; i < norm.size();) {
+        uint32_t cp;
+        size_t bad;
+        size_t n = utf8_at(reinterpret_cast<const unsigned char *>(norm.data()) + i, norm.size() - i, &cp, &bad);
+        if (!n) n = 1;  // ill-formed input: byte by byte (the caller hands valid UTF-8)
+        std::string ch(norm, i, n);
+        i += n;
+        auto it = encoder_.find(ch);
+        if (it != encoder_.end()) {
+            put_unk();
+            push(std::move(ch), it->second);
+            continue;
+        }
+        bool all = true;
+        for (unsigned char b : ch) all = all && byte_ids_[b] >= 0;
+        if (all) {
+            for (unsigned char b : ch) {
+                char name[8];
+                snprintf(name, sizeof(name), "<0x%02X>", (unsigned)b);
+                push(name, byte_ids_[b]);
+            }
+        } else {
+            unk_waits = true;
+        }
+    }
+    put_unk();
+    struct Cand {
+        uint32_t rank;
+        int left, right;
+        uint32_t lver, rver;
+    };
+    auto worse = [](const Cand &a, const Cand &b) { return a.rank != b.rank ? a.rank > b.rank : a.left > b.left; };
+    std::priority_queue<Cand, std::vector<Cand>, decltype(worse)> heap(worse);
+    std::string key;
+    auto offer = [&](int l) {
+        if (l < 0 || w[l].next < 0) return;
+        const int r = w[l].next;
+        key.assign(w[l].s);
+        key.push_back(' ');
+        key.append(w[r].s);
+        auto it = ranks_.find(key);
+        if (it != ranks_.end()) heap.push(Cand{it->second, l, r, w[l].ver, w[r].ver});
+    };
+    for (int i = 0; i + 1 < (int)w.size(); i++) offer(i);
+    while (!heap.empty()) {
+        const Cand c = heap.top();
+        heap.pop();
+        Sym &l = w[c.left], &r = w[c.right];
+        if (!l.alive || !r.alive || l.ver != c.lver || r.ver != c.rver || l.next != c.right) continue;  // a stale pair
+        l.s += r.s;
+        auto id = encoder_.find(l.s);
+        l.id = id == encoder_.end() ? -1 : (int64_t)id->second;
+        l.ver++;
+        r.alive = false;
+        l.next = r.next;
+        if (r.next >= 0) w[r.next].prev = c.left;
+        offer(l.prev);
+        offer(c.left);
+    }
+    for (int i = w.empty() ? -1 : 0; i >= 0; i = w[i].next)
+        if (w[i].id >= 0) ids->push_back((uint32_t)w[i].id);
+}
+
+// Decoder of that family: U+2581 back to spaces, runs of byte tokens to the text they spell (every byte of a run
+// that is not UTF-8 becomes U+FFFD), everything joined, one leading space dropped.
+std::string BpeTokenizer::decode_spm(const uint32_t *ids, size_t n, bool skip_special) const {
+    static const char U2581[] = "\xE2\x96\x81";
+    std::string out, run;
+    auto flush = [&]() {
+        if (run.empty()) return;
+        bool valid = true;
+        for (size_t i = 0; i < run.size() && valid;) {
+            uint32_t cp;
+            size_t bad;
+            const size_t m = utf8_at(reinterpret_cast<const unsigned char *>(run.data()) + i, run.size() - i, &cp, &bad);
+            valid = m != 0;
+            i += m ? m : 1;
+        }
+        if (valid) out += run;
+        else
+            for (size_t i = 0; i < run.size(); i++) out += "\xEF\xBF\xBD";
+        run.clear();
+    };
+    for (size_t k = 0; k < n; k++) {
+        auto it = decoder_.find(ids[k]);
+        if (it == decoder_.end()) continue;
+        if (skip_special) {
+            auto a = added_by_id_.find(ids[k]);
+            if (a != added_by_id_.end() && added_[a->second].special) continue;
+        }
+        const std::string &tok = it->second;
+        unsigned byte = 0;
+        if (tok.size() == 6 && tok.compare(0, 3, "<0x") == 0 && tok[5] == '>' && isxdigit((unsigned char)tok[3]) &&
+            isxdigit((unsigned char)tok[4]) && sscanf(tok.c_str() + 3, "%2x", &byte) == 1) {
+            run.push_back((char)byte);
+            continue;
+        }
+        flush();
+        for (size_t i = 0; i < tok.size();) {
+            if (tok.compare(i, 3, U2581) == 0) {
+                out.push_back(' ');
+                i += 3;
+            } else {
+                out.push_back(tok[i++]);
+            }
+        }
+    }
+    flush();
+    if (!out.empty() && out[0] == ' ') out.erase(0, 1);
+    return out;
+}
+
 void BpeTokenizer::encode_plain(const char *text, size_t len, std::vector<uint32_t> *ids) const {
+    if (spm_) {
+        encode_plain_spm(text, len, ids);
+        return;
+    }
     std::string mapped;
     for (const auto &piece : pre_tokenize(text, len, max_digits_)) {
         mapped.clear();
@@ -509,6 +714,7 @@ std::vector<uint32_t> BpeTokenizer::encode(const char *text, size_t len, bool ad
 }
 
 std::string BpeTokenizer::decode(const uint32_t *ids, size_t n, bool skip_special) const {
+    if (spm_) return decode_spm(ids, n, skip_special);
     std::string bytes, tok_bytes;
     for (size_t k = 0; k < n; k++) {
         auto it = decoder_.find(ids[k]);

@@ -1,5 +1,6 @@
-// Byte-level BPE tokenizer. Two sources: vocab.json + merges.txt, the reference's own Tokenizer
-// (src/tokenizer.rs:6-158); and a tokenizer.json of the byte-level BPE family (Qwen2/3, Llama-3), which the
+// BPE tokenizer. Sources: vocab.json + merges.txt, the reference's own byte-level Tokenizer
+// (src/tokenizer.rs:6-158); a tokenizer.json of the byte-level BPE family (Qwen2/3, Llama-3) or of the
+// SentencePiece-style BPE family (Llama-2, TinyLlama, Mistral: "\u2581" for spaces, byte fallback), which the
 // reference hands to the `tokenizers` crate (HfTokenizer, src/hf/tokenizer.rs:4-47). Host code only.
 #pragma once
 
@@ -19,8 +20,10 @@ public:
     // HfTokenizer::from_file (src/hf/tokenizer.rs:10-14) for the files this class can honour: model BPE
     // without unknown-token or byte fallback, ByteLevel pre-tokeniser and decoder behind a Split on the
     // Qwen2 or Llama-3 pattern, added tokens without strip or single-word flags, post-processor ByteLevel
-    // or TemplateProcessing. Anything else is refused with a message. An NFC normaliser is recorded
-    // (wants_nfc) and left to the caller: this class does not normalise.
+    // or TemplateProcessing. Or: model BPE with unk_token, fuse_unk and byte_fallback, normaliser
+    // Sequence[Prepend("\u2581"), Replace(" " -> "\u2581")], no pre-tokeniser, decoder Sequence[Replace("\u2581" -> " "),
+    // ByteFallback, Fuse, Strip(" ", 1, 0)] (the Llama-2 family). Anything else is refused with a message. An NFC
+    // normaliser is recorded (wants_nfc) and left to the caller: this class does not normalise.
     static std::unique_ptr<BpeTokenizer> from_tokenizer_json(const std::string &path, std::string *err);
     // reference encode (src/tokenizer.rs:119-144): pieces of the pre-tokeniser pattern, bytes mapped to
     // printable code points, merges by rank; pieces missing from the vocabulary are dropped. Added tokens
@@ -50,6 +53,13 @@ private:
     };
     void init_byte_alphabet();
     void encode_plain(const char *text, size_t len, std::vector<uint32_t> *ids) const;
+    // the SentencePiece-style family: the whole stretch is one word of characters (bytes where a character is not
+    // in the vocabulary), merged by rank
+    void encode_plain_spm(const char *text, size_t len, std::vector<uint32_t> *ids) const;
+    std::string decode_spm(const uint32_t *ids, size_t n, bool skip_special) const;
+    bool spm_ = false;            // SentencePiece-style family
+    int64_t unk_id_ = -1;
+    int64_t byte_ids_[256];       // ids of "<0x00>" .. "<0xFF>", -1 when absent
     std::vector<Added> added_;                         // longest content first
     std::unordered_map<uint32_t, size_t> added_by_id_;
     std::vector<uint32_t> prefix_ids_, suffix_ids_;    // post-processor template around a single sequence

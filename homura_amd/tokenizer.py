@@ -28,7 +28,8 @@ def pre_tokenize(text: str) -> list[str]:
 
 class Tokenizer:
     """reference Tokenizer (src/tokenizer.rs:6-158) over vocab.json + merges.txt; from_tokenizer_json gives
-    the reference's HfTokenizer (src/hf/tokenizer.rs:4-47) for byte-level BPE tokenizer.json files."""
+    the reference's HfTokenizer (src/hf/tokenizer.rs:4-47) for tokenizer.json files of the byte-level and the
+    SentencePiece-style (Llama-2) BPE families."""
 
     def __init__(self, vocab_json=None, merges_txt=None, *, tokenizer_json=None):
         self.lib = _ffi.load()

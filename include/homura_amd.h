@@ -563,7 +563,10 @@ const char *hm_version(void);
  * hm_tokenizer_open_json stands in for HfTokenizer::from_file (src/hf/tokenizer.rs:10-14), which hands a
  * tokenizer.json to the `tokenizers` crate (0.21.4 in the reference's Cargo.lock): it reads the files of
  * the byte-level BPE family (Qwen2/3, Llama-3: BPE model, Split on their pattern + ByteLevel, added
- * tokens, ByteLevel or TemplateProcessing post-processor) and refuses everything else with a message.
+ * tokens, ByteLevel or TemplateProcessing post-processor) and of the SentencePiece-style BPE family
+ * (Llama-2, TinyLlama, Mistral: BPE with unk_token, fuse_unk and byte_fallback, normaliser Prepend U+2581 +
+ * Replace " " by U+2581, no pre-tokeniser, decoder Replace / ByteFallback / Fuse / Strip), and refuses
+ * everything else with a message.
  * A file that asks for NFC normalisation is accepted and hm_tokenizer_wants_nfc says so: the caller
  * normalises the text, this library does not.
  * hm_tokenizer_open* return NULL and write a message into err. encode / decode return the full

@@ -2,7 +2,9 @@
 crate, 0.21.4 in its Cargo.lock) and the chat helpers (src/hf/chat.rs). The checker for the tokenizer is the
 `tokenizers` Python package, a binding of that same crate: each test writes a tokenizer.json with it (the
 reference's GPT-2 vocabulary and merges under the Qwen2 or the Llama-3 pre-tokeniser, with added tokens), loads
-the file into the library and compares ids and text. CPU only."""
+the file into the library and compares ids and text. The Llama-2 family (SentencePiece-style BPE with byte
+fallback: TinyLlama, Mistral) gets a vocabulary trained by the package on a few lines, since no file of that
+family is at hand. CPU only."""
 import json
 import random
 import sys
@@ -105,6 +107,120 @@ def test_ids_and_text_match_the_tokenizers_crate(tmp_path, family):
             assert mine.decode_raw(want_sp) == theirs.decode(want_sp, skip_special_tokens=False), repr(text)
         for token in ("<|im_end|>", "<|eot_id|>", "<think>", "Hello", "Ġworld", "no such token"):
             assert mine.token_to_id(token) == theirs.token_to_id(token)
+
+
+SPM_CORPUS = [
+    "The quick brown fox jumps over the lazy dog.", "Hello world, hello there, hello again!",
+    "A tokenizer turns text into numbers and numbers back into text.", "It's 2024: 3 + 4 = 7, and 12345 * 2 = 24690.",
+    "def main():\n    print('hello')\n    return 0", "caf\u00e9 na\u00efve r\u00e9sum\u00e9 \u00fcber stra\u00dfe",
+    "the the the and and of of to to in in is is that that it it", "    indented   text  with   runs  of   spaces",
+    "<s>[INST] What is the capital of France? [/INST] Paris.</s>", "one two three four five six seven eight nine ten",
+] * 3
+
+
+def _build_llama2(tmp_path, drop_bytes=()):
+    """A tokenizer.json laid out as Llama-2's: BPE with unk_token, fuse_unk and byte_fallback over a vocabulary of
+    pieces with U+2581 for spaces, no pre-tokeniser. `drop_bytes`: byte tokens left out of the vocabulary, so that
+    characters with those bytes come out as the unknown token."""
+    from tokenizers import Tokenizer, normalizers, trainers
+    from tokenizers.models import BPE
+    seed = Tokenizer(BPE())
+    seed.normalizer = normalizers.Sequence([normalizers.Prepend("\u2581"), normalizers.Replace(" ", "\u2581")])
+    seed.train_from_iterator(SPM_CORPUS, trainers.BpeTrainer(vocab_size=420, show_progress=False, special_tokens=[]))
+    trained = json.loads(seed.to_str())["model"]
+    pieces = sorted(trained["vocab"], key=trained["vocab"].get)
+    # two characters of the corpus go to bytes instead; pieces that spell a special token would take its place
+    pieces = [p for p in pieces if p not in ("\u00e9", "\u00df", "<unk>", "<s>", "</s>")]
+    merges = [m if isinstance(m, list) else m.split(" ") for m in trained["merges"]]
+    keep = set(pieces)
+    merges = [m for m in merges if m[0] in keep and m[1] in keep and m[0] + m[1] in keep]
+    names = ["<unk>", "<s>", "</s>"] + [f"<0x{b:02X}>" for b in range(256) if b not in drop_bytes] + pieces
+    vocab = {name: i for i, name in enumerate(names)}
+    special = [{"id": i, "content": c, "single_word": False, "lstrip": False, "rstrip": False, "normalized": False,
+                "special": True} for i, c in enumerate(["<unk>", "<s>", "</s>"])]
+    doc = {
+        "version": "1.0", "truncation": None, "padding": None, "added_tokens": special,
+        "normalizer": {"type": "Sequence", "normalizers": [
+            {"type": "Prepend", "prepend": "\u2581"},
+            {"type": "Replace", "pattern": {"String": " "}, "content": "\u2581"}]},
+        "pre_tokenizer": None,
+        "post_processor": {"type": "TemplateProcessing",
+                           "single": [{"SpecialToken": {"id": "<s>", "type_id": 0}}, {"Sequence": {"id": "A", "type_id": 0}}],
+                           "pair": [{"SpecialToken": {"id": "<s>", "type_id": 0}}, {"Sequence": {"id": "A", "type_id": 0}},
+                                    {"SpecialToken": {"id": "<s>", "type_id": 1}}, {"Sequence": {"id": "B", "type_id": 1}}],
+                           "special_tokens": {"<s>": {"id": "<s>", "ids": [1], "tokens": ["<s>"]}}},
+        "decoder": {"type": "Sequence", "decoders": [
+            {"type": "Replace", "pattern": {"String": "\u2581"}, "content": " "},
+            {"type": "ByteFallback"}, {"type": "Fuse"}, {"type": "Strip", "content": " ", "start": 1, "stop": 0}]},
+        "model": {"type": "BPE", "dropout": None, "unk_token": "<unk>", "continuing_subword_prefix": None,
+                  "end_of_word_suffix": None, "fuse_unk": True, "byte_fallback": True, "ignore_merges": False,
+                  "vocab": vocab, "merges": merges},
+    }
+    path = tmp_path / "llama2.json"
+    path.write_text(json.dumps(doc), encoding="utf-8")
+    return Tokenizer.from_file(str(path)), path
+
+
+SPM_TEXTS = TEXTS + SPM_CORPUS[:10] + [
+    "Hello</s>world", "<s>Hello</s> <s> again", " </s> ", "</s>", "<unk>known<unk>", "<0x0A> literal", "caf\u00e9\u00df\u00e9",
+    "\U0001f642\U0001f680 and \u65e5\u672c", "\U0001f642a\U0001f642\u00e9\U0001f680\U0001f680b", "\u2581 already \u2581\u2581 there",
+    "x" * 700 + " " + "the " * 300,
+]
+
+
+@pytest.mark.parametrize("drop_bytes", [(), tuple(range(0xF0, 0xF5)), (0x98, 0x99)], ids=["all_bytes", "no_f0_f4", "no_98_99"])
+def test_llama2_family_matches_the_tokenizers_crate(tmp_path, drop_bytes):
+    """Whole stretches between special tokens are one word; characters outside the vocabulary go in as byte tokens,
+    or as one fused unknown token where a byte token is missing; decoding undoes both."""
+    from homura_amd.tokenizer import Tokenizer
+    theirs, path = _build_llama2(tmp_path, drop_bytes)
+    rng = random.Random(11)
+    strays = [[rng.randrange(theirs.get_vocab_size()) for _ in range(rng.randint(1, 10))] for _ in range(200)]
+    strays += [[3 + 0xE6 - len([b for b in drop_bytes if b < 0xE6])], [1, 2, 0], []]
+    with Tokenizer.from_tokenizer_json(path) as mine:
+        assert mine.vocab_size == theirs.get_vocab_size(with_added_tokens=True)
+        seen_unk = seen_byte = False
+        for text in SPM_TEXTS + _random_texts(300, 13):
+            want = theirs.encode(text, add_special_tokens=False).ids
+            assert mine.encode(text) == want, repr(text)
+            seen_unk |= 0 in want and "<unk>" not in text
+            seen_byte |= any(3 <= i < 259 - len(drop_bytes) for i in want)
+            want_sp = theirs.encode(text, add_special_tokens=True).ids
+            assert mine.encode_with_special(text) == want_sp == [1] + want, repr(text)
+            assert mine.decode(want_sp) == theirs.decode(want_sp, skip_special_tokens=True), repr(text)
+            assert mine.decode_raw(want_sp) == theirs.decode(want_sp, skip_special_tokens=False), repr(text)
+        assert seen_byte and seen_unk == bool(drop_bytes)
+        for ids in strays:  # byte tokens that spell no UTF-8, in any company
+            assert mine.decode(ids) == theirs.decode(ids, skip_special_tokens=True), ids
+            assert mine.decode_raw(ids) == theirs.decode(ids, skip_special_tokens=False), ids
+        for token in ("<s>", "</s>", "<0x0A>", "\u2581the", "no such token"):
+            assert mine.token_to_id(token) == theirs.token_to_id(token)
+
+
+def test_llama2_family_files_outside_it_are_refused(tmp_path):
+    from homura_amd.tokenizer import Tokenizer
+    _, path = _build_llama2(tmp_path)
+    good = json.loads(path.read_text(encoding="utf-8"))
+
+    def refused(change, needle):
+        doc = json.loads(json.dumps(good))
+        change(doc)
+        p = tmp_path / "bad.json"
+        p.write_text(json.dumps(doc), encoding="utf-8")
+        with pytest.raises(ValueError) as e:
+            Tokenizer.from_tokenizer_json(p)
+        assert needle in str(e.value), str(e.value)
+
+    refused(lambda d: d["model"].__setitem__("fuse_unk", False), "fuse_unk")
+    refused(lambda d: d["model"].__setitem__("unk_token", None), "unk_token")
+    refused(lambda d: d["model"].__setitem__("unk_token", "<nope>"), "unk_token")
+    refused(lambda d: d["normalizer"]["normalizers"].pop(0), "normalizer")
+    refused(lambda d: d["normalizer"]["normalizers"][0].__setitem__("prepend", "_"), "normalizer")
+    refused(lambda d: d.__setitem__("normalizer", None), "normalizer")
+    refused(lambda d: d.__setitem__("pre_tokenizer", {"type": "Whitespace"}), "pre-tokeniser")
+    refused(lambda d: d["decoder"]["decoders"].pop(3), "decoder")
+    refused(lambda d: d["decoder"]["decoders"][3].__setitem__("start", 0), "decoder")
+    refused(lambda d: d["added_tokens"][1].__setitem__("normalized", True), "normalized")
 
 
 def test_template_prefix_only_with_special_tokens(tmp_path):
@@ -259,3 +375,22 @@ def test_stream_decoder_holds_back_split_characters(tmp_path):
                 out.append(piece)
                 prev = i
             assert "".join(out) == want
+
+
+def test_stream_decoder_on_the_llama2_family(tmp_path):
+    """The decoder of this family drops one leading space from whatever it is handed, so a token's text is what it
+    adds to the token before it (src/generate.rs:480-516); byte tokens of one character are held back together."""
+    from homura_amd.chat import StreamDecoder
+    from homura_amd.tokenizer import Tokenizer
+    theirs, path = _build_llama2(tmp_path)
+    with Tokenizer.from_tokenizer_json(path) as tok:
+        for text in ("Hello world, hello there", "the caf\u00e9 \U0001f642 is  over there \u65e5\u672c ok", " two  spaces"):
+            ids = tok.encode(text)
+            assert ids == theirs.encode(text, add_special_tokens=False).ids
+            sd, out, prev = StreamDecoder(tok), [], None
+            for i in ids:
+                piece = sd.push(i, prev)
+                assert "\ufffd" not in piece
+                out.append(piece)
+                prev = i
+            assert "".join(out) == text == tok.decode(ids)
