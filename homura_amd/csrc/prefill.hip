@@ -46,15 +46,32 @@ __global__ void split_rows_kernel(const float *__restrict__ x, uint16_t *__restr
 }
 
 // A GEMM result that was cut along K: the slices added in index order
-__device__ __forceinline__ float sum_parts(const float *__restrict__ p, size_t i, int parts, size_t stride) {
-    float v = p[i];
-    for (int s = 1; s < parts; s++) v += p[i + s * stride];
+// Sum of the K slices of a projection result, in slice order. Every slice is requested before the first is used:
+// a loop of loads waits for each in turn, eight trips to memory at eight slices.
+constexpr int MAX_SUM_PARTS = 8;
+template <int MAXP, class V>
+__device__ __forceinline__ V sum_parts_upto(const float *__restrict__ p, size_t i, int parts, size_t stride) {
+    V t[MAXP];
+#pragma unroll
+    for (int s = 0; s < MAXP; s++) t[s] = *reinterpret_cast<const V *>(p + i + (size_t)(s < parts ? s : 0) * stride);
+    V v = t[0];
+#pragma unroll
+    for (int s = 1; s < MAXP; s++)
+        if (s < parts) v += t[s];
     return v;
 }
+template <class V>
+__device__ __forceinline__ V sum_parts_as(const float *__restrict__ p, size_t i, int parts, size_t stride) {
+    if (parts == 1) return *reinterpret_cast<const V *>(p + i);
+    if (parts <= 2) return sum_parts_upto<2, V>(p, i, parts, stride);
+    if (parts <= 4) return sum_parts_upto<4, V>(p, i, parts, stride);
+    return sum_parts_upto<MAX_SUM_PARTS, V>(p, i, parts, stride);
+}
+__device__ __forceinline__ float sum_parts(const float *__restrict__ p, size_t i, int parts, size_t stride) {
+    return sum_parts_as<float>(p, i, parts, stride);
+}
 __device__ __forceinline__ f32x4 sum_parts4(const float *__restrict__ p, size_t i, int parts, size_t stride) {
-    f32x4 v = *reinterpret_cast<const f32x4 *>(p + i);
-    for (int s = 1; s < parts; s++) v += *reinterpret_cast<const f32x4 *>(p + i + s * stride);
-    return v;
+    return sum_parts_as<f32x4>(p, i, parts, stride);
 }
 
 // elements c .. c+3 of a split row
@@ -586,7 +603,7 @@ int rmsnorm_split_launch(hm_ctx *ctx, const float *d_x, const float *d_res, int 
     HM_REQUIRE(ctx, !q8k || dim % 256 == 0, "rmsnorm_split: Q8_K activations need dim %% 256 == 0 (dim=%d)", dim);
     HM_REQUIRE(ctx, d_x && d_w && (d_out_split || d_q8), "rmsnorm_split: NULL pointer");
     HM_REQUIRE(ctx, !d_q8 || (q8k && d_q8_scale && ((uintptr_t)d_q8 % 4) == 0), "rmsnorm_split: Q8_K rows need q8k, a scale buffer and 4-byte alignment");
-    HM_REQUIRE(ctx, rows > 0 && dim > 0 && dim % 4 == 0 && pieces >= 1 && pieces <= 3 && res_parts >= 1,
+    HM_REQUIRE(ctx, rows > 0 && dim > 0 && dim % 4 == 0 && pieces >= 1 && pieces <= 3 && res_parts >= 1 && res_parts <= MAX_SUM_PARTS,
                "rmsnorm_split: bad shape (dim %% 4 == 0 needed)");
     HM_REQUIRE(ctx, ((uintptr_t)d_x % 16) == 0 && ((uintptr_t)d_w % 16) == 0 && ((uintptr_t)d_out_split % 8) == 0 &&
                         ((uintptr_t)d_res % 16) == 0 && ((uintptr_t)d_resid_out % 16) == 0, "rmsnorm_split: misaligned buffer");
@@ -602,7 +619,7 @@ int silu_mul_split_launch(hm_ctx *ctx, const float *d_gu, int parts, uint16_t *d
     HM_REQUIRE(ctx, !q8k || inter % 256 == 0, "silu_mul_split: Q8_K activations need a width %% 256 == 0 (%d)", inter);
     HM_REQUIRE(ctx, d_gu && (d_out_split || d_q8), "silu_mul_split: NULL pointer");
     HM_REQUIRE(ctx, !d_q8 || (q8k && d_q8_scale && ((uintptr_t)d_q8 % 4) == 0), "silu_mul_split: Q8_K rows need q8k, a scale buffer and 4-byte alignment");
-    HM_REQUIRE(ctx, rows > 0 && inter > 0 && inter % 4 == 0 && pieces >= 1 && pieces <= 3 && parts >= 1,
+    HM_REQUIRE(ctx, rows > 0 && inter > 0 && inter % 4 == 0 && pieces >= 1 && pieces <= 3 && parts >= 1 && parts <= MAX_SUM_PARTS,
                "silu_mul_split: bad shape (intermediate size %% 4 == 0 needed)");
     HM_REQUIRE(ctx, ((uintptr_t)d_gu % 16) == 0 && ((uintptr_t)d_out_split % 8) == 0, "silu_mul_split: misaligned buffer");
     const size_t n = (size_t)rows * inter;
@@ -676,7 +693,7 @@ int quant_ints_launch(hm_ctx *ctx, int hm_dtype, const uint8_t *d_blocks, int N,
 
 int qkv_post_launch(hm_ctx *ctx, const QkvPostArgs &a) {
     HM_REQUIRE(ctx, a.qkv && a.cos_tab && a.sin_tab && a.kcache && a.vcache, "qkv_post: NULL pointer");
-    HM_REQUIRE(ctx, a.S > 0 && a.H > 0 && a.kvh > 0 && a.past >= 0 && a.parts >= 1, "qkv_post: bad shape");
+    HM_REQUIRE(ctx, a.S > 0 && a.H > 0 && a.kvh > 0 && a.past >= 0 && a.parts >= 1 && a.parts <= MAX_SUM_PARTS, "qkv_post: bad shape");
     HM_REQUIRE(ctx, a.hd >= 2 && a.hd <= 256 && a.hd % 2 == 0, "qkv_post: head_dim %d not supported", a.hd);
     HM_REQUIRE(ctx, (a.qw == nullptr) == (a.kw == nullptr), "qkv_post: q and k norm weights must come together");
     if (a.past + a.S > a.max_len)
