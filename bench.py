@@ -96,6 +96,7 @@ def main() -> int:
     ap.add_argument("--no-prefill", action="store_true", help="skip the prompt-pass measurement")
     ap.add_argument("--no-quantised", action="store_true", help="skip the decode measurements with quantised projections")
     ap.add_argument("--no-other-shapes", action="store_true", help="skip the decode measurements at the other listed models' shapes")
+    ap.add_argument("--no-long-cache", action="store_true", help="skip the decode measurements on caches of 4000 to 32000 rows")
     ap.add_argument("--no-kernel-configs", action="store_true",
                     help="skip the stand-alone kernel measurements (benchmark configurations 1, 3, 4, 5)")
     args = ap.parse_args()
@@ -332,6 +333,34 @@ def main() -> int:
                                   "kernel_launches_per_step": omdl.launches_per_step()}
                     omdl.close()
                 other_shapes[name] = entry
+        # The benchmarked model on longer caches: the whole-step launch keeps what fits in its wavefronts'
+        # registers and streams the further rows through its attention phase (instances for up to 1536, 2048,
+        # 4096 and 32768 live rows). Reported beside `value`.
+        long_cache = None
+        if not args.no_long_cache:
+            import dataclasses
+            import numpy as np
+            lcfg = dataclasses.replace(cfg, max_position_embeddings=32768)
+            lm = synth_model.build_model(ctx, lcfg, weights, 32768)
+            lm.set_graph(not args.no_graph)
+            long_cache = {"unit": "ms per token", "steps": 32,
+                          "what": "the benchmarked model (bf16, greedy, one launch per token) from caches of that many "
+                                  "rows: the 1024 synthetic rows repeated"}
+            for rows in (4000, 16300, 32000):
+                lkv = []
+                for a in kv:
+                    big = np.empty((1, a.shape[1], rows, a.shape[3]), dtype=np.float32)
+                    for r0 in range(0, rows, PREFILL):
+                        n = min(PREFILL, rows - r0)
+                        big[:, :, r0:r0 + n] = a[:, :, :n]
+                    lkv.append(big)
+                lm.init_kv_cache(lkv, rows)
+                del lkv
+                lm.bench_decode(int(prompt[0]), 8)
+                l_ms, _ = lm.bench_decode(int(prompt[1]), 32)
+                long_cache[str(rows)] = {"ms_per_step": round(l_ms / 32, 4), "value": round(32e3 / l_ms, 1),
+                                         "whole_step": bool(lm.whole_step()), "kernel_launches_per_step": lm.launches_per_step()}
+            lm.close()
         kernel_configs = None
         if not args.no_kernel_configs:
             from homura_amd import kernel_bench
@@ -382,6 +411,7 @@ def main() -> int:
         "prefill": prefill,
         "quantised_decode": quantised,
         "other_shapes": other_shapes,
+        "long_cache": long_cache,
         "event_ms_per_step": round(event_ms / args.steps, 4),
         "kernels": kernels,
         "kernel_configs": kernel_configs,
