@@ -1124,20 +1124,23 @@ __device__ __forceinline__ void compute_role(const FusedDecodeArgs &a, Lds<GE> &
                 }
             };
             // Rounds past the held ones (XR > 0: caches longer than the registers hold) are streamed inside
-            // the phase, two sets of PR rounds in turn: one is multiplied while the other is in flight.
+            // the phase through a ring of XD sets of PR rounds: one is multiplied while XD - 1 are in flight
+            // (they take the registers of the held rounds, which are dead by then). A request past the split's
+            // last round reads a valid row that nobody uses (kv_off), so the requests need no conditions.
+            constexpr int XD = 3;
             int npx = 0;
             if constexpr (GE::XR > 0) {
                 const int over = sp.cached - NR * NCW * RPI;
                 npx = over > 0 ? (over + PR * NCW * RPI - 1) / (PR * NCW * RPI) : 0;
             }
-            u32x4 kxa[PR], vxa[PR], kxb[PR], vxb[PR];
-            auto load_x = [&](u32x4 (&kx)[PR], u32x4 (&vx)[PR], const int r0) __attribute__((always_inline)) {
+            u32x4 kx[XD][PR], vx[XD][PR];
+            auto load_x = [&](u32x4 (&kxs)[PR], u32x4 (&vxs)[PR], const int r0) __attribute__((always_inline)) {
                 const uint16_t *kc = sm.lp[l].kcache, *vc = sm.lp[l].vcache;
 #pragma unroll
                 for (int i = 0; i < PR; i++) {
                     const size_t off = kv_off(r0 + i);
-                    kx[i] = ld128_global_stream(kc + off);
-                    vx[i] = ld128_global_stream(vc + off);
+                    kxs[i] = ld128_global_stream(kc + off);
+                    vxs[i] = ld128_global_stream(vc + off);
                 }
             };
 #pragma unroll
@@ -1146,22 +1149,28 @@ __device__ __forceinline__ void compute_role(const FusedDecodeArgs &a, Lds<GE> &
                 auto kk = [&](int i) { return s.kr[i0 + i]; };
                 auto vv = [&](int i) { return s.vr[i0 + i]; };
                 const bool last = ps == NPASS - 1 && npx == 0;
-                // the first streamed set goes out ahead of the last held pass, into registers of earlier rounds
+                // the first streamed sets go out ahead of the last held pass, into registers of earlier rounds
                 if constexpr (GE::XR > 0) {
-                    if (ps == NPASS - 1 && npx > 0) load_x(kxa, vxa, NR);
+                    if (ps == NPASS - 1 && npx > 0) {
+#pragma unroll
+                        for (int j = 0; j < XD - 1; j++) load_x(kx[j], vx[j], NR + j * PR);
+                    }
                 }
                 if (ps == 0) attn_pass(std::true_type{}, kk, vv, i0, last);
                 else attn_pass(std::false_type{}, kk, vv, i0, last);
             }
             if constexpr (GE::XR > 0) {
-                for (int x = 0; x < npx; x += 2) {
-                    if (x + 1 < npx) load_x(kxb, vxb, NR + (x + 1) * PR);
-                    attn_pass(std::false_type{}, [&](int i) { return kxa[i]; }, [&](int i) { return vxa[i]; }, NR + x * PR, x == npx - 1);
-                    if (x + 1 < npx) {
-                        if (x + 2 < npx) load_x(kxa, vxa, NR + (x + 2) * PR);
-                        attn_pass(std::false_type{}, [&](int i) { return kxb[i]; }, [&](int i) { return vxb[i]; }, NR + (x + 1) * PR, x + 1 == npx - 1);
+                // set x + j sits in ring slot j; the request that refills the slot freed last goes out first
+                auto ring_step = [&](auto self, auto jc, const int x) __attribute__((always_inline)) -> void {
+                    constexpr int j = decltype(jc)::value;
+                    load_x(kx[(j + XD - 1) % XD], vx[(j + XD - 1) % XD], NR + (x + j + XD - 1) * PR);
+                    attn_pass(std::false_type{}, [&](int i) { return kx[j][i]; }, [&](int i) { return vx[j][i]; },
+                              NR + (x + j) * PR, x + j == npx - 1);
+                    if constexpr (j + 1 < XD) {
+                        if (x + j + 1 < npx) self(self, std::integral_constant<int, j + 1>{}, x);
                     }
-                }
+                };
+                for (int x = 0; x < npx; x += XD) ring_step(ring_step, std::integral_constant<int, 0>{}, x);
             }
 #pragma unroll
             for (int g = 0; g < G; g++) {
