@@ -13,6 +13,9 @@ struct AttnArgs {
     // for max_len with a fixed chunk (workgroups past the live range exit at once).
     const DecodeState *state = nullptr;
     int fixed_chunk = 0;
+    // Decode-plan mode: rows the grid covers instead of max_len (0: max_len). The caller keeps
+    // state->pos + 1 within it: rows beyond would not be looked at.
+    int span = 0;
     // Fused prologue (decode plan, B == 1): when qkv_raw is set, q is ignored; the kernel applies
     // QK-norm + RoPE to the raw projection row and appends the new K/V row to the caches.
     const float *qkv_raw = nullptr;  // [H*hd | kvh*hd | kvh*hd]

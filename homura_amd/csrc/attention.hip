@@ -526,48 +526,109 @@ __global__ __launch_bounds__(ATT_THREADS) void gqa_decode_attn_stream_kernel(
     }
 }
 
-// Second half of the split attention: one workgroup of HD threads per (batch, query head)
-// folds that head's partial (o, max, sum) triples in ascending split order. A separate launch
-// instead of a "last workgroup to arrive" fold: the kernel boundary orders the partial writes,
-// so no device-scope fence (a full L2 write-back + invalidate on this chip) is needed.
-template <int HD, int G>
-__global__ __launch_bounds__(HD) void gqa_decode_fold_kernel(
+// Second half of the split attention: one workgroup per (batch, query head) folds that head's partial
+// (o, max, sum) triples. A separate launch instead of a "last workgroup to arrive" fold: the kernel boundary
+// orders the partial writes, so no device-scope fence (a full L2 write-back + invalidate on this chip) is needed.
+// The workgroup is SG groups of HD threads (thread = output element d of group sg). Group sg takes splits sg,
+// sg + SG, ... in ascending order against the maximum of its own splits, up to 32 loads a thread in flight; the
+// groups' (max, sum, o) then meet in LDS and are merged in group order. One group (grids of at most 32 splits) is the
+// plain ascending fold; a grid of hundreds of splits (tens of thousands of cached rows) folded by one group took
+// 57 us, longer than the attention itself.
+constexpr int FOLD_BATCH = 32;      // splits fetched per batch, all loads of a batch in flight together
+constexpr int FOLD_THREADS = 1024;  // of a workgroup with groups
+
+// GROUPS false: one group of HD threads (grids of at most FOLD_BATCH splits: a workgroup of 1024 threads costs about
+// 2 us more to start than one of 64 or 128). GROUPS true: FOLD_THREADS / HD groups; with few splits live (a grid
+// sized for a long cache with few rows in it yet) one group folds and the others leave at once.
+template <int HD, int G, bool GROUPS>
+__global__ __launch_bounds__(GROUPS ? FOLD_THREADS : HD) void gqa_decode_fold_kernel(
     float *__restrict__ out, const float *__restrict__ part_o, const float *__restrict__ part_ml,
     int kvh, int kv_len_arg, int chunk, const DecodeState *__restrict__ state) {
-    extern __shared__ float s_ml[];  // [nsplit][2] of this head
-    const int d = threadIdx.x;
+    constexpr int SGMAX = GROUPS ? FOLD_THREADS / HD : 1;
+    extern __shared__ float s_fold[];  // [SGMAX][HD + 2] group results, then [nsplit][2] (max, sum) of this head
+    const int d = GROUPS ? threadIdx.x % HD : threadIdx.x, sg = GROUPS ? threadIdx.x / HD : 0;
+    float *s_grp = s_fold, *s_ml = s_fold + SGMAX * (HD + 2);
     const int gi = blockIdx.x % G, kvhd = blockIdx.x / G, b = blockIdx.y;
     const int H = kvh * G;
     const int kv_len = state ? state->pos + 1 : kv_len_arg;
     const int nsplit = (kv_len + chunk - 1) / chunk;
     if (nsplit == 1) return;  // the attention kernel wrote the final result itself
+    const int SG = GROUPS && nsplit > FOLD_BATCH / 2 ? SGMAX : 1;
+    if (sg >= SG) return;
     const size_t pair = (size_t)b * kvh + kvhd;
     const float *ao = part_o + (pair * nsplit * G + gi) * HD + d;
     const float *aml = part_ml + (pair * nsplit * G + gi) * 2;
-    constexpr int FB = 32;  // splits fetched per batch, all loads of a batch in flight together
+    constexpr int FB = FOLD_BATCH;
     float o[FB];
 #pragma unroll
-    for (int u = 0; u < FB; u++) o[u] = u < nsplit ? ao[(size_t)u * G * HD] : 0.f;
-    for (int i = d; i < nsplit * 2; i += HD) s_ml[i] = aml[(size_t)(i >> 1) * G * 2 + (i & 1)];
+    for (int u = 0; u < FB; u++) {
+        const int sp = sg + u * SG;
+        o[u] = sp < nsplit ? ao[(size_t)sp * G * HD] : 0.f;
+    }
+    for (int i = threadIdx.x; i < nsplit * 2; i += SG * HD) s_ml[i] = aml[(size_t)(i >> 1) * G * 2 + (i & 1)];
     __syncthreads();
     float M = -INFINITY;
-    for (int s = 0; s < nsplit; s++) M = fmaxf(M, s_ml[s * 2]);
+    for (int sp = sg; sp < nsplit; sp += SG) M = fmaxf(M, s_ml[sp * 2]);
     float L = 0.f, O = 0.f;
-    for (int s0 = 0; s0 < nsplit; s0 += FB) {
-        if (s0 > 0) {
+    for (int u0 = 0; sg + u0 * SG < nsplit; u0 += FB) {
+        if (u0 > 0) {
 #pragma unroll
-            for (int u = 0; u < FB; u++) o[u] = s0 + u < nsplit ? ao[(size_t)(s0 + u) * G * HD] : 0.f;
+            for (int u = 0; u < FB; u++) {
+                const int sp = sg + (u0 + u) * SG;
+                o[u] = sp < nsplit ? ao[(size_t)sp * G * HD] : 0.f;
+            }
         }
 #pragma unroll
         for (int u = 0; u < FB; u++) {
-            if (s0 + u < nsplit) {
-                const float wgt = expf(s_ml[(s0 + u) * 2] - M);
-                L = fmaf(wgt, s_ml[(s0 + u) * 2 + 1], L);
+            const int sp = sg + (u0 + u) * SG;
+            if (sp < nsplit) {
+                const float wgt = expf(s_ml[sp * 2] - M);
+                L = fmaf(wgt, s_ml[sp * 2 + 1], L);
                 O = fmaf(wgt, o[u], O);
             }
         }
     }
-    out[((size_t)b * H + kvhd * G + gi) * HD + d] = O / L;
+    float *res = out + ((size_t)b * H + kvhd * G + gi) * HD + d;
+    if (SG == 1) {
+        *res = O / L;
+        return;
+    }
+    s_grp[sg * (HD + 2) + d] = O;
+    if (d == 0) {
+        s_grp[sg * (HD + 2) + HD] = M;
+        s_grp[sg * (HD + 2) + HD + 1] = L;
+    }
+    __syncthreads();
+    if (sg != 0) return;
+    float Mt = -INFINITY;
+    for (int g = 0; g < SG; g++) Mt = fmaxf(Mt, s_grp[g * (HD + 2) + HD]);
+    float Lt = 0.f, Ot = 0.f;
+    for (int g = 0; g < SG; g++) {
+        const float mg = s_grp[g * (HD + 2) + HD];
+        if (mg == -INFINITY) continue;  // a group without splits
+        const float wgt = expf(mg - Mt);
+        Lt = fmaf(wgt, s_grp[g * (HD + 2) + HD + 1], Lt);
+        Ot = fmaf(wgt, s_grp[g * (HD + 2) + d], Ot);
+    }
+    *res = Ot / Lt;
+}
+
+// nsplit: the grid's split count (what a call can ever have live)
+template <int HD, int G>
+int launch_fold(hm_ctx *ctx, const AttnArgs &a, const float *part_o, const float *part_ml, int nsplit, int chunk,
+                const DecodeState *state) {
+    const bool groups = nsplit > FOLD_BATCH;
+    const int sg = groups ? FOLD_THREADS / HD : 1;
+    const size_t fold_lds = ((size_t)sg * (HD + 2) + (size_t)nsplit * 2) * sizeof(float);
+    HM_REQUIRE(ctx, fold_lds <= 64 * 1024, "gqa_decode_attn: too many splits (%d)", nsplit);
+    if (groups)
+        hipLaunchKernelGGL((gqa_decode_fold_kernel<HD, G, true>), dim3(a.kvh * G, a.B), dim3(FOLD_THREADS), fold_lds,
+                           ctx->stream, a.out, part_o, part_ml, a.kvh, a.kv_len, chunk, state);
+    else
+        hipLaunchKernelGGL((gqa_decode_fold_kernel<HD, G, false>), dim3(a.kvh * G, a.B), dim3(HD), fold_lds, ctx->stream,
+                           a.out, part_o, part_ml, a.kvh, a.kv_len, chunk, state);
+    HM_LAUNCH_CHECK(ctx);
+    return HM_OK;
 }
 
 // KvCache::append_key / append_value (reference src/runtime.rs:521-568) with the cache in
@@ -616,11 +677,8 @@ int launch_attn(hm_ctx *ctx, const AttnArgs &a, int nsplit, int chunk) {
     }
     // nsplit is the grid's split count: 1 means no call can ever need a fold
     if (nsplit > 1 && a.phase != AttnArgs::SPLIT_ONLY) {
-        const size_t fold_lds = (size_t)nsplit * 2 * sizeof(float);
-        HM_REQUIRE(ctx, fold_lds <= 64 * 1024, "gqa_decode_attn: too many splits (%d)", nsplit);
-        hipLaunchKernelGGL((gqa_decode_fold_kernel<HD, G>), dim3(a.kvh * G, a.B), dim3(HD), fold_lds,
-                           ctx->stream, a.out, part_o, part_ml, a.kvh, a.kv_len, chunk, a.state);
-        HM_LAUNCH_CHECK(ctx);
+        const int rc = launch_fold<HD, G>(ctx, a, part_o, part_ml, nsplit, chunk, a.state);
+        if (rc != HM_OK) return rc;
     }
     return HM_OK;
 }
@@ -637,12 +695,8 @@ int launch_attn_stream(hm_ctx *ctx, const AttnArgs &a, int nsplit, int chunk) {
                        part_ml, a.kvh, a.max_len, a.kv_len, chunk, a.scale);
     HM_LAUNCH_CHECK(ctx);
     if (nsplit > 1) {
-        const size_t fold_lds = (size_t)nsplit * 2 * sizeof(float);
-        HM_REQUIRE(ctx, fold_lds <= 64 * 1024, "gqa_decode_attn: too many splits (%d)", nsplit);
-        hipLaunchKernelGGL((gqa_decode_fold_kernel<HD, G>), dim3(a.kvh * G, a.B), dim3(HD), fold_lds,
-                           ctx->stream, a.out, part_o, part_ml, a.kvh, a.kv_len, chunk,
-                           (const DecodeState *)nullptr);
-        HM_LAUNCH_CHECK(ctx);
+        const int rc = launch_fold<HD, G>(ctx, a, part_o, part_ml, nsplit, chunk, (const DecodeState *)nullptr);
+        if (rc != HM_OK) return rc;
     }
     return HM_OK;
 }
@@ -704,7 +758,8 @@ int gqa_decode_attn_launch(hm_ctx *ctx, const AttnArgs &a) {
     // A workgroup keeps its whole chunk in registers: 32..128 rows. Aim at about one workgroup
     // per CU over the rows that can be live.
     const int rows_step = 32;
-    const int span = a.state ? a.max_len : a.kv_len;  // rows the grid has to be able to cover
+    // rows the grid has to be able to cover
+    const int span = a.state ? (a.span > 0 && a.span < a.max_len ? a.span : a.max_len) : a.kv_len;
     int chunk = a.fixed_chunk;
     bool stepping = false;
     if (chunk <= 0) {

@@ -236,6 +236,10 @@ class ExecutionPlan {
     // Called before a step is enqueued or captured, with the KV cache in place (device tables that
     // depend on the cache's addresses are refreshed here, outside any capture).
     void set_pre_run(std::function<int()> fn) { pre_run_ = std::move(fn); }
+    // Rows the decode attention's grid covers in a recorded step (0: the cache's capacity). Whoever sets it keeps
+    // the live rows within it and drops the recorded step when it changes.
+    int attn_span() const { return attn_span_; }
+    void set_attn_span(int rows) { attn_span_ = rows; }
 
     // Per-kernel timing of one step (HOMURA_PROFILE analogue, reference src/runtime.rs:1849-1873):
     // HIP events around every device launch of a real decode step.
@@ -287,6 +291,7 @@ class ExecutionPlan {
     bool use_graph_ = false;
     bool whole_step_ = false;
     std::function<int()> pre_run_;
+    int attn_span_ = 0;
     hipGraph_t graph_ = nullptr;
     hipGraphExec_t graph_exec_ = nullptr;
 };

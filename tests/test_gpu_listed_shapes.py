@@ -81,3 +81,36 @@ def test_listed_shape_against_oracle(ctx, shape, fmt):
     want2 = np.concatenate([om.run_kv(ids[i:i + 1]) for i in range(2)])
     check(got2, want2, "steps behind the prompt", prompt=True)
     gm.close()
+
+
+@pytest.mark.parametrize("shape", ["qwen2.5-0.5b", "tinyllama-1.1b", "qwen2.5-1.5b", "smollm2-1.7b"])
+def test_listed_shape_on_longer_caches(ctx, shape):
+    """One launch per projection on caches of thousands of rows: the attention grid of the recorded step covers
+    the live rows rounded up to a power of two (2048 at least) and is recorded anew when they outgrow it; beyond
+    2048 rows a split takes 128 rows instead of 64 and the fold of the splits' partial results is shared out
+    over groups of threads. Decode steps across both borders (2048, 4096 live rows), eager and replayed from a
+    graph, against the oracle."""
+    cfg = dataclasses.replace(synth_model.listed_shape(shape, layers=2, vocab=1500), max_position_embeddings=16384)
+    weights = synth_model.synth_weights(cfg, 4343, DTYPE_BF16, has_qk_norm=False)
+    L = 9000
+    gm = synth_model.build_model(ctx, cfg, weights, L, DTYPE_BF16, has_qk_norm=False)
+    om = mf.build_oracle_model(cfg, weights, L, DTYPE_BF16, has_qk_norm=False)
+    assert not gm.whole_step()
+    gm.set_prefill_min(0)
+    ids = synth.token_ids(19, 12, cfg.vocab_size)
+    for rows in (2040, 4090, 8900):
+        kv = synth_model.synth_kv(cfg, 20 + rows, rows)
+        results = []
+        for graph in (False, True):
+            gm.set_graph(graph)
+            gm.init_kv_cache(kv, rows)
+            results.append(gm.run_kv(ids))
+            assert gm.kv_cache_len() == rows + len(ids)
+        mf.oracle_init_kv(om, kv)
+        want = np.concatenate([om.run_kv(ids[i:i + 1]) for i in range(len(ids))])
+        errs = [mf.rel_err(results[0][i], want[i]) for i in range(len(ids))]
+        say(f"{shape} from {rows} rows: rel err max {max(errs):.2e}")
+        assert max(errs) < 1e-2
+        assert np.array_equal(results[0], results[1])
+    gm.set_graph(False)
+    gm.close()

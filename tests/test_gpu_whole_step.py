@@ -278,7 +278,7 @@ def long_small(ctx):
 @pytest.mark.parametrize("rows", [4094, 4600, 5000, 6200, 9000, 12287, 20000, 32754])
 def test_rows_streamed_inside_the_attention_phase(long_small, rows):
     """More than 4096 live rows: a split's rows beyond the eight rounds held in registers are loaded inside
-    the attention phase, two rounds at a time in two alternating register sets. The lengths give a split one
+    the attention phase, two rounds at a time through a ring of three register sets. The lengths give a split one
     streamed row (4097 live rows: 129 a split), a partly filled round, an odd and an even number of
     passes, a split boundary that moves while tokens are appended, and the last round the instance
     serves (32768 rows). Logits against the oracle, tokens against the per-projection path."""
