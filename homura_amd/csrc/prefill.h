@@ -86,6 +86,9 @@ struct PrefillAttnArgs {
     int S = 0, H = 0, kvh = 0, hd = 0, max_len = 0, past = 0;
     float scale = 1.f;
     int pieces = 3;
+    // set by prefill_attn_launch when few query rows face a long cache: the keys are cut over gridDim.z
+    // workgroups, which leave their (O, max, sum) here for a second kernel to join
+    float *part_o = nullptr, *part_ml = nullptr;
 };
 int prefill_attn_launch(hm_ctx *ctx, const PrefillAttnArgs &a);
 

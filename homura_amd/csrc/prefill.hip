@@ -402,7 +402,10 @@ __global__ __launch_bounds__(A8_THREADS) void prefill_attn16_kernel(PrefillAttnA
     const int wg_end = a.past + min(a.S, q0 + AT_QROWS);
     const int wave_end = q0 + qw * 16 < a.S ? a.past + min(a.S, q0 + qw * 16 + 16) : 0;
     const int ntiles = (wg_end + A8_KEYS - 1) / A8_KEYS;
-    const int nrounds = (ntiles + KS - 1) / KS;
+    const int nrounds_all = (ntiles + KS - 1) / KS;
+    // the rounds of this workgroup: all of them, or its share when the keys are cut over gridDim.z workgroups
+    const int per_z = (nrounds_all + (int)gridDim.z - 1) / (int)gridDim.z;
+    const int r_begin = (int)blockIdx.z * per_z, nrounds = min(nrounds_all, r_begin + per_z);
     const int wave_first = a.past + min(q0 + qw * 16, a.S - 1);
 
     // This lane's part of a tile load: row dma_row of the tile, the chunk that belongs in slot dma_slot.
@@ -435,7 +438,7 @@ __global__ __launch_bounds__(A8_THREADS) void prefill_attn16_kernel(PrefillAttnA
             x0[ks] = *reinterpret_cast<const f32x4 *>(qp + 32 * ks);
             x1[ks] = *reinterpret_cast<const f32x4 *>(qp + 32 * ks + 4);
         }
-        request_round(0);
+        if (r_begin < nrounds) request_round(r_begin);  // (a tile load must not outlive the workgroup)
 #pragma unroll
         for (int ks = 0; ks < KSTEPS; ks++) {
             float f[8];
@@ -455,7 +458,7 @@ __global__ __launch_bounds__(A8_THREADS) void prefill_attn16_kernel(PrefillAttnA
     // transposing V reads: lane i of a group points at dims 4 (i % 4) .. + 3 of a 16-dim block, key 4 c4 + i / 4
     const int v_key = 4 * c4 + (l16 >> 2), v_sub = l16 & 3;
 
-    for (int r = 0; r < nrounds; r++) {
+    for (int r = r_begin; r < nrounds; r++) {
         // this round's tiles have landed for this wavefront (nothing else is in flight), then for everybody,
         // and everybody is done with the other set
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -557,7 +560,7 @@ __global__ __launch_bounds__(A8_THREADS) void prefill_attn16_kernel(PrefillAttnA
         for (int g = 1; g < KS; g++) {
             const float *other = xch + (size_t)((g - 1) * QW + qw) * PER_LANE * 64 + lane;
             const float m_o = other[(DB * 4) * 64], l_o = other[(DB * 4 + 1) * 64];
-            const float m_new = fmaxf(m_run, m_o);
+            const float m_new = fmaxf(fmaxf(m_run, m_o), -1e30f);  // (with the keys cut over workgroups group 0 may have seen none either)
             const float w_me = __builtin_amdgcn_exp2f(m_run - m_new), w_o = __builtin_amdgcn_exp2f(m_o - m_new);
             l_run = l_run * w_me + l_o * w_o;
             m_run = m_new;
@@ -569,8 +572,19 @@ __global__ __launch_bounds__(A8_THREADS) void prefill_attn16_kernel(PrefillAttnA
     }
     const float l_tot = quad_rows_sum(l_run);
     if (qrow >= a.S) return;
-    const float inv = 1.0f / l_tot;
     const int qd = a.H * HD;
+    if (a.part_o) {  // this workgroup's share of the keys: (O, max, sum) as they are
+        float *po = a.part_o + ((size_t)blockIdx.z * a.S + qrow) * qd + h * HD + 4 * c4;
+#pragma unroll
+        for (int db = 0; db < DB; db++) *reinterpret_cast<f32x4 *>(po + 16 * db) = acc_o[db];
+        if (c4 == 0) {
+            float *pm = a.part_ml + (((size_t)blockIdx.z * a.S + qrow) * a.H + h) * 2;
+            pm[0] = m_run;
+            pm[1] = l_tot;
+        }
+        return;
+    }
+    const float inv = 1.0f / l_tot;
     // value v of block db is d = 16 db + 4 c4 + v
 #pragma unroll
     for (int db = 0; db < DB; db++) {
@@ -589,6 +603,47 @@ __global__ __launch_bounds__(A8_THREADS) void prefill_attn16_kernel(PrefillAttnA
                 w.y = hi[p];
                 *reinterpret_cast<u32x2 *>(o16 + (size_t)p * qd) = w;
             }
+        }
+    }
+}
+
+// Joins the shares of prefill_attn16_kernel when the keys were cut over nz workgroups: four neighbouring outputs of
+// one (query row, head) per thread, the shares in index order against the largest reference point (scores are in
+// units of ln 2; a share that saw no visible key has max = -inf or the floor -1e30 and sum 0; share 0 sees key 0).
+template <int NP>
+__global__ __launch_bounds__(256) void prefill_attn_join_kernel(const float *__restrict__ part_o, const float *__restrict__ part_ml,
+                                                                int nz, int S, int H, int hd, float *__restrict__ out_f32,
+                                                                uint16_t *__restrict__ out_split) {
+    const size_t qd = (size_t)H * hd, e = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4;
+    if (e >= (size_t)S * qd) return;
+    const size_t qrow = e / qd;
+    const int col = (int)(e % qd), h = col / hd;
+    float m = -INFINITY;
+    for (int z = 0; z < nz; z++) m = fmaxf(m, part_ml[(((size_t)z * S + qrow) * H + h) * 2]);
+    float l = 0.f;
+    f32x4 o = {0.f, 0.f, 0.f, 0.f};
+    for (int z = 0; z < nz; z++) {
+        const float *pm = part_ml + (((size_t)z * S + qrow) * H + h) * 2;
+        const float w = __builtin_amdgcn_exp2f(pm[0] - m);
+        l = fmaf(w, pm[1], l);
+        const f32x4 oz = *reinterpret_cast<const f32x4 *>(part_o + ((size_t)z * S + qrow) * qd + col);
+#pragma unroll
+        for (int k = 0; k < 4; k++) o[k] = fmaf(w, oz[k], o[k]);
+    }
+    const float inv = 1.0f / l;
+    o = o * inv;
+    if (out_f32) *reinterpret_cast<f32x4 *>(out_f32 + qrow * qd + col) = o;
+    if (out_split) {
+        uint32_t lo[NP], hi[NP];
+        split_pair<NP>(o[0], o[1], lo);
+        split_pair<NP>(o[2], o[3], hi);
+        uint16_t *o16 = out_split + qrow * NP * qd + col;
+#pragma unroll
+        for (int p = 0; p < NP; p++) {
+            u32x2 w;
+            w.x = lo[p];
+            w.y = hi[p];
+            *reinterpret_cast<u32x2 *>(o16 + (size_t)p * qd) = w;
         }
     }
 }
@@ -726,7 +781,27 @@ int prefill_attn_launch(hm_ctx *ctx, const PrefillAttnArgs &a) {
         if (v == 1 || v == 2 || v == 4) ks = v;
     }
     const int qrows = 128 / ks;
-    const dim3 grid((unsigned)((a.S + qrows - 1) / qrows), (unsigned)a.H);
+    dim3 grid((unsigned)((a.S + qrows - 1) / qrows), (unsigned)a.H);
+    // Few query rows in front of a long cache (a chat turn behind a long conversation) leave most CUs without a
+    // workgroup while each workgroup walks every key: the keys are then cut over nz workgroups, eight rounds of
+    // tiles each at least, which leave their (O, max, sum) in the workspace for a second kernel to join.
+    PrefillAttnArgs b = a;
+    int nz = 1;
+    {
+        const long long wgs = (long long)grid.x * grid.y;
+        const int rounds = ((a.past + a.S + A8_KEYS - 1) / A8_KEYS + ks - 1) / ks;
+        nz = (int)std::min<long long>(std::min<long long>(32, ctx->num_cus / std::max<long long>(1, wgs)), rounds / 8);
+        const size_t per_z = (size_t)a.S * a.H * (a.hd + 2) * sizeof(float);
+        // (callers that carve scratch of their own from the workspace leave its first 16 MiB to the kernels)
+        const size_t room = std::min<size_t>(ctx->workspace_bytes, (size_t)16 << 20);
+        if (nz >= 2 && per_z * nz > room) nz = (int)(room / per_z);
+        if (nz < 2) nz = 1;
+        if (nz > 1) {
+            b.part_o = (float *)ctx->workspace;
+            b.part_ml = b.part_o + (size_t)nz * a.S * a.H * a.hd;
+            grid.z = (unsigned)nz;
+        }
+    }
     // two sets of ks pairs of 32-key tiles; the final exchange of the key groups wants
     // (ks - 1) * (128 / ks / 16) sets of (hd / 4 + 2) * 256 bytes
     const size_t lds = std::max<size_t>((size_t)2 * ks * 2 * A8_KEYS * a.hd * 2, (size_t)(ks - 1) * (8 / ks) * (a.hd / 4 + 2) * 256);
@@ -736,7 +811,7 @@ int prefill_attn_launch(hm_ctx *ctx, const PrefillAttnArgs &a) {
                                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
             HM_REQUIRE(ctx, e == hipSuccess, "prefill_attn: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));
         }
-        hipLaunchKernelGGL(kernel, grid, dim3(A8_THREADS), lds, ctx->stream, a);
+        hipLaunchKernelGGL(kernel, grid, dim3(A8_THREADS), lds, ctx->stream, b);
         return HM_OK;
     };
     int rc = HM_OK;
@@ -753,6 +828,17 @@ int prefill_attn_launch(hm_ctx *ctx, const PrefillAttnArgs &a) {
 #undef HM_AT_CASE
     if (rc != HM_OK) return rc;
     HM_LAUNCH_CHECK(ctx);
+    if (nz > 1) {
+        const size_t n4 = (size_t)a.S * a.H * a.hd / 4;
+        const dim3 jg((unsigned)((n4 + 255) / 256));
+        if (a.pieces == 3)
+            hipLaunchKernelGGL(prefill_attn_join_kernel<3>, jg, dim3(256), 0, ctx->stream, b.part_o, b.part_ml, nz, a.S, a.H, a.hd,
+                               a.out_f32, a.out_split);
+        else
+            hipLaunchKernelGGL(prefill_attn_join_kernel<2>, jg, dim3(256), 0, ctx->stream, b.part_o, b.part_ml, nz, a.S, a.H, a.hd,
+                               a.out_f32, a.out_split);
+        HM_LAUNCH_CHECK(ctx);
+    }
     return HM_OK;
 }
 

@@ -658,7 +658,11 @@ def test_attention_uniform_keys_give_mean_of_values(ctx):
     (1, 4, 2, 128, 64, 0),          # a single row
     (37, 14, 2, 64, 300, 33),       # g = 7, head_dim 64, nothing aligned
     (129, 4, 4, 64, 512, 64),       # MHA, one row into the second query block
-    (64, 12, 2, 128, 256, 191)])    # g = 6, the last key tile is a single key short of full
+    (64, 12, 2, 128, 256, 191),     # g = 6, the last key tile is a single key short of full
+    (8, 16, 8, 128, 9000, 8000),    # a chat turn behind a long conversation: the keys are cut over several workgroups
+    (40, 14, 2, 64, 5000, 4531),    # the same with g = 7, head_dim 64, nothing aligned
+    (48, 16, 8, 128, 16400, 16000),
+    (3, 4, 2, 128, 3000, 2900)])
 @pytest.mark.parametrize("key_groups", [0, 1, 2, 4])
 def test_gqa_prefill_attn(ctx, oracle, monkeypatch, S, H, kvh, hd, max_len, past, key_groups):
     """key_groups: how many wavefronts of a workgroup share a block of 32 query rows, each taking every
