@@ -83,18 +83,22 @@ def test_listed_shape_against_oracle(ctx, shape, fmt):
     gm.close()
 
 
-@pytest.mark.parametrize("shape", ["qwen2.5-0.5b", "tinyllama-1.1b", "qwen2.5-1.5b", "smollm2-1.7b"])
-def test_listed_shape_on_longer_caches(ctx, shape):
+@pytest.mark.parametrize("shape,fmt", [("qwen2.5-0.5b", "bf16"), ("tinyllama-1.1b", "bf16"), ("qwen2.5-1.5b", "bf16"),
+                                       ("smollm2-1.7b", "bf16"), ("qwen2.5-1.5b", "q8_0"), ("tinyllama-1.1b", "q4_0")])
+def test_listed_shape_on_longer_caches(ctx, shape, fmt):
     """One launch per projection on caches of thousands of rows: the attention grid of the recorded step covers
     the live rows rounded up to a power of two (2048 at least) and is recorded anew when they outgrow it; beyond
     2048 rows a split takes 128 rows instead of 64 and the fold of the splits' partial results is shared out
     over groups of threads. Decode steps across both borders (2048, 4096 live rows), eager and replayed from a
     graph, against the oracle."""
     cfg = dataclasses.replace(synth_model.listed_shape(shape, layers=2, vocab=1500), max_position_embeddings=16384)
-    weights = synth_model.synth_weights(cfg, 4343, DTYPE_BF16, has_qk_norm=False)
+    if fmt != "bf16":
+        cfg = dataclasses.replace(cfg, tie_word_embeddings=False)   # the quantised plan keeps an f32 LM head
+    wdt = FORMATS[fmt]
+    weights = synth_model.synth_weights(cfg, 4343, wdt, has_qk_norm=False)
     L = 9000
-    gm = synth_model.build_model(ctx, cfg, weights, L, DTYPE_BF16, has_qk_norm=False)
-    om = mf.build_oracle_model(cfg, weights, L, DTYPE_BF16, has_qk_norm=False)
+    gm = synth_model.build_model(ctx, cfg, weights, L, wdt, has_qk_norm=False)
+    om = mf.build_oracle_model(cfg, weights, L, wdt, has_qk_norm=False)
     assert not gm.whole_step()
     gm.set_prefill_min(0)
     ids = synth.token_ids(19, 12, cfg.vocab_size)
@@ -109,8 +113,13 @@ def test_listed_shape_on_longer_caches(ctx, shape):
         mf.oracle_init_kv(om, kv)
         want = np.concatenate([om.run_kv(ids[i:i + 1]) for i in range(len(ids))])
         errs = [mf.rel_err(results[0][i], want[i]) for i in range(len(ids))]
-        say(f"{shape} from {rows} rows: rel err max {max(errs):.2e}")
-        assert max(errs) < 1e-2
+        scale = max(np.abs(results[0][i] - want[i]).max() / np.abs(want[i]).max() for i in range(len(ids)))
+        say(f"{shape} {fmt} from {rows} rows: rel err max {max(errs):.2e}, of the logit scale {scale:.2e}")
+        # The Q4_0 TinyLlama of this test sits at 1e-4 of the logit scale on long caches (1e-6 at 70 rows, and
+        # 3e-6 for the others here), whichever Q4_0 kernels multiply (planes, cut rows, raw blocks) and however the
+        # attention grid is cut: its scores are large, and a softmax over thousands of rows turns their rounding
+        # into output error. A wrong split, span or fold gives errors of order 1.
+        assert max(errs) < (1e-2 if fmt == "bf16" else 3e-2) and scale < 1e-3
         assert np.array_equal(results[0], results[1])
     gm.set_graph(False)
     gm.close()
