@@ -345,7 +345,8 @@ def main() -> int:
             lm.set_graph(not args.no_graph)
             long_cache = {"unit": "ms per token", "steps": 32,
                           "what": "the benchmarked model (bf16, greedy, one launch per token) from caches of that many "
-                                  "rows: the 1024 synthetic rows repeated"}
+                                  "rows: the 1024 synthetic rows repeated; turn_of_32_tokens_ms: 32 tokens behind "
+                                  "that cache in one prompt pass"}
             for rows in (4000, 16300, 32000):
                 lkv = []
                 for a in kv:
@@ -355,11 +356,23 @@ def main() -> int:
                         big[:, :, r0:r0 + n] = a[:, :, :n]
                     lkv.append(big)
                 lm.init_kv_cache(lkv, rows)
-                del lkv
                 lm.bench_decode(int(prompt[0]), 8)
                 l_ms, _ = lm.bench_decode(int(prompt[1]), 32)
                 long_cache[str(rows)] = {"ms_per_step": round(l_ms / 32, 4), "value": round(32e3 / l_ms, 1),
                                          "whole_step": bool(lm.whole_step()), "kernel_launches_per_step": lm.launches_per_step()}
+                # a chat turn behind that cache: 32 tokens consumed in one prompt pass (wall clock around run_kv)
+                turn = synth.token_ids(seed + 0x300, 32, cfg.vocab_size)
+                best = None
+                for _ in range(3):
+                    lm.init_kv_cache(lkv, rows)
+                    ctx.sync()
+                    t0 = time.perf_counter()
+                    lm.run_kv(turn, want_logits=False)
+                    ctx.sync()
+                    dt = time.perf_counter() - t0
+                    best = dt if best is None or dt < best else best
+                long_cache[str(rows)]["turn_of_32_tokens_ms"] = round(best * 1e3, 3)
+                del lkv
             lm.close()
         kernel_configs = None
         if not args.no_kernel_configs:
