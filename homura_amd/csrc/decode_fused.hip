@@ -948,6 +948,10 @@ __device__ __forceinline__ void compute_role(const FusedDecodeArgs &a, Lds<GE> &
     // weight request): those instances request the down rows, the second half of the cache rows and the
     // Q|K|V rows one phase later, when the registers they land in have just been read for the last time.
     constexpr bool LATE = NR > 4;
+    // Their cache rows go out in four lots so that no phase start asks for much more than the CU keeps in flight
+    // (a wavefront that asks for more waits, with its phase's arithmetic behind it): the first rounds at the end of
+    // the attention phase, the rest of the first half with the O phase, the second half with gate|up and down.
+    constexpr int LATE_KV_P2 = LATE ? KV_CUT / 2 : 0, LATE_KV_P4 = LATE ? (NR - KV_CUT) / 2 : 0;
     {
         // the first layer's slice, in the order the loop re-requests it (the rest follows inside the loop)
         const FusedLayerPtrs lp = sm.lp[0];
@@ -1180,11 +1184,12 @@ __device__ __forceinline__ void compute_role(const FusedDecodeArgs &a, Lds<GE> &
             }
         }
         if (LATE) load_wq(nx, 0, GE::RQW);  // behind the arithmetic that needed the registers
+        if (LATE) load_kv(nx, 0, LATE_KV_P2);
         wg_barrier();
 
         // ── O projection rows (reference src/hf/emitter.rs:738-745) ──
         wg_barrier();
-        load_kv(nx, 0, KV_CUT);
+        load_kv(nx, LATE_KV_P2, KV_CUT);
         if (LATE) load_wd(sm.lp[l]);
         {
             using S = decltype(s.wo);
@@ -1201,6 +1206,7 @@ __device__ __forceinline__ void compute_role(const FusedDecodeArgs &a, Lds<GE> &
         // ── gate|up rows, SiLU(gate) * up (reference src/hf/emitter.rs:787-799) ──
         wg_barrier();
         if (!LATE) load_kv(nx, KV_CUT, NR);
+        if (LATE) load_kv(nx, KV_CUT, KV_CUT + LATE_KV_P4);
         load_wo(nx);
         {
             const float tot = ((sm.red[0] + sm.red[1]) + sm.red[2]) + sm.red[3];
@@ -1221,7 +1227,7 @@ __device__ __forceinline__ void compute_role(const FusedDecodeArgs &a, Lds<GE> &
         // ── down rows (reference src/hf/emitter.rs:801-804; the residual is added by the readers) ──
         wg_barrier();
         load_wg(nx, 0, WG_CUT);
-        if (LATE) load_kv(nx, KV_CUT, NR);
+        if (LATE) load_kv(nx, KV_CUT + LATE_KV_P4, NR);
         {
             using S = decltype(s.wd);
             float v[S::Q];
