@@ -334,7 +334,7 @@ def main() -> int:
                     omdl.close()
                 other_shapes[name] = entry
         # The benchmarked model on longer caches: the whole-step launch keeps what fits in its wavefronts'
-        # registers and streams the further rows through its attention phase (instances for up to 1536, 2048,
+        # registers and streams the further rows through its attention phase (instances for up to 1536, 2048, 3072,
         # 4096 and 32768 live rows). Reported beside `value`.
         long_cache = None
         if not args.no_long_cache:

@@ -1010,65 +1010,70 @@ __device__ __forceinline__ void compute_role(const FusedDecodeArgs &a, Lds<GE> &
 #pragma unroll
             for (int g = 0; g < G; g++) lds_x8(sm.qs[g], dl * 8, qv[g]);
             const bool with_new = sp.owner && cw == 0;  // the new row rides with wavefront 0 of the last split
-            // The rounds held in registers are taken PR at a time (their float forms would not fit beside the
-            // weight slices otherwise, and a spilled register is reloaded through the same in-order memory
-            // pipeline the weight requests wait in); passes after the first rescale what the earlier ones left.
-            // The new row rides with the last pass.
-            constexpr int PR = NR > 4 ? 2 : NR, NPASS = NR / PR;
+            // The rounds held in registers are taken PR at a time, at most four (the float forms of more would not
+            // fit beside the weight slices, and a spilled register is reloaded through the same in-order memory
+            // pipeline the weight requests wait in): one pass up to four rounds, two of three or of four beyond;
+            // passes after the first rescale what the earlier ones left. A pass costs its reductions and
+            // exponentials whatever its width: eight rounds as four passes of two took 0.519 ms a token at 4000 rows,
+            // as two of four 0.507. Streamed sets (below) stay two rounds wide, the ring holds three of them. The
+            // new row rides with the last pass.
+            constexpr int PR = NR == 6 ? 3 : (NR == 8 ? 4 : NR), NPASS = NR / PR;  // rounds a pass over the held rows
+            constexpr int PX = 2;                                                  // rounds a streamed set
             static_assert(NR % PR == 0, "row rounds are taken in equal passes");
             float m[G], lsum[G], acc[G][8];
-            // One pass: rounds i0 .. i0 + PR - 1 of the split, their rows handed over by kk(i) / vv(i).
-            auto attn_pass = [&](auto first_tag, auto kk, auto vv, const int i0, const bool last) __attribute__((always_inline)) {
+            // One pass: rounds i0 .. i0 + PW - 1 of the split, their rows handed over by kk(i) / vv(i).
+            auto attn_pass = [&](auto first_tag, auto width_tag, auto kk, auto vv, const int i0, const bool last) __attribute__((always_inline)) {
                 constexpr bool FIRST = decltype(first_tag)::value;
-                // slot PR is the new row (last pass only; elsewhere it is dead and multiplies zeros)
-                float kf[PR + 1][8];
+                constexpr int PW = decltype(width_tag)::value;  // rounds of this pass
+                // slot PW is the new row (last pass only; elsewhere it is dead and multiplies zeros)
+                float kf[PW + 1][8];
 #pragma unroll
-                for (int i = 0; i < PR; i++) unpack8f(kk(i), kf[i]);
-                if (last) lds_x8(sm.knew, dl * 8, kf[PR]);
+                for (int i = 0; i < PW; i++) unpack8f(kk(i), kf[i]);
+                if (last) lds_x8(sm.knew, dl * 8, kf[PW]);
                 else {
 #pragma unroll
-                    for (int e = 0; e < 8; e++) kf[PR][e] = 0.f;
+                    for (int e = 0; e < 8; e++) kf[PW][e] = 0.f;
                 }
-                float sc[G][PR + 1];
+                float sc[G][PW + 1];
 #pragma unroll
                 for (int g = 0; g < G; g++)
 #pragma unroll
-                    for (int i = 0; i <= PR; i++) sc[g][i] = 0.f;
+                    for (int i = 0; i <= PW; i++) sc[g][i] = 0.f;
 #pragma unroll
                 for (int e = 0; e < 8; e++)
 #pragma unroll
                     for (int g = 0; g < G; g++)
 #pragma unroll
-                        for (int i = 0; i <= PR; i++) sc[g][i] = fmaf(kf[i][e], qv[g][e], sc[g][i]);
+                        for (int i = 0; i <= PW; i++) sc[g][i] = fmaf(kf[i][e], qv[g][e], sc[g][i]);
                 // sums over the lanes of a row, all (head, row) chains side by side
 #pragma unroll
                 for (int g = 0; g < G; g++)
 #pragma unroll
-                    for (int i = 0; i <= PR; i++) sc[g][i] += dpp_move<0xB1, 0xF>(sc[g][i], 0.f);
+                    for (int i = 0; i <= PW; i++) sc[g][i] += dpp_move<0xB1, 0xF>(sc[g][i], 0.f);
 #pragma unroll
                 for (int g = 0; g < G; g++)
 #pragma unroll
-                    for (int i = 0; i <= PR; i++) sc[g][i] += dpp_move<0x4E, 0xF>(sc[g][i], 0.f);
+                    for (int i = 0; i <= PW; i++) sc[g][i] += dpp_move<0x4E, 0xF>(sc[g][i], 0.f);
 #pragma unroll
                 for (int g = 0; g < G; g++)
 #pragma unroll
-                    for (int i = 0; i <= PR; i++) sc[g][i] += dpp_move<0x141, 0xF>(sc[g][i], 0.f);
+                    for (int i = 0; i <= PW; i++) sc[g][i] += dpp_move<0x141, 0xF>(sc[g][i], 0.f);
                 if (LPR == 16) {
 #pragma unroll
                     for (int g = 0; g < G; g++)
 #pragma unroll
-                        for (int i = 0; i <= PR; i++) sc[g][i] += dpp_move<0x140, 0xF>(sc[g][i], 0.f);
+                        for (int i = 0; i <= PW; i++) sc[g][i] += dpp_move<0x140, 0xF>(sc[g][i], 0.f);
                 }
-                bool live[PR + 1];
+                bool live[PW + 1];
 #pragma unroll
-                for (int i = 0; i < PR; i++) live[i] = ((i0 + i) * NCW + cw) * RPI + sub < sp.cached;
-                live[PR] = last && with_new;
+                for (int i = 0; i < PW; i++) live[i] = ((i0 + i) * NCW + cw) * RPI + sub < sp.cached;
+                live[PW] = last && with_new;
                 float mp[G];
 #pragma unroll
                 for (int g = 0; g < G; g++) {
                     mp[g] = -INFINITY;
 #pragma unroll
-                    for (int i = 0; i <= PR; i++) {
+                    for (int i = 0; i <= PW; i++) {
                         sc[g][i] = live[i] ? sc[g][i] * a.scale : -INFINITY;
                         mp[g] = fmaxf(mp[g], sc[g][i]);
                     }
@@ -1090,14 +1095,14 @@ __device__ __forceinline__ void compute_role(const FusedDecodeArgs &a, Lds<GE> &
                         lsum[g] *= alpha[g];
                     }
                 }
-                float pr[G][PR + 1];
+                float pr[G][PW + 1];
 #pragma unroll
                 for (int g = 0; g < G; g++) {
 #pragma unroll
-                    for (int i = 0; i <= PR; i++) {
+                    for (int i = 0; i <= PW; i++) {
                         pr[g][i] = live[i] ? __expf(sc[g][i] - m[g]) : 0.f;
                         // a cache row is counted by the first of its lanes, the new row by lane 0
-                        if (i < PR ? dl == 0 : lane == 0) lsum[g] += pr[g][i];
+                        if (i < PW ? dl == 0 : lane == 0) lsum[g] += pr[g][i];
                     }
                 }
                 if (last) {
@@ -1113,43 +1118,43 @@ __device__ __forceinline__ void compute_role(const FusedDecodeArgs &a, Lds<GE> &
                         sm.wstat[cw][lane][1] = ll;
                     }
                 }
-                float vf[PR + 1][8];
+                float vf[PW + 1][8];
 #pragma unroll
-                for (int i = 0; i < PR; i++) unpack8f(vv(i), vf[i]);
-                if (last) lds_x8(sm.vnew, dl * 8, vf[PR]);
+                for (int i = 0; i < PW; i++) unpack8f(vv(i), vf[i]);
+                if (last) lds_x8(sm.vnew, dl * 8, vf[PW]);
                 else {
 #pragma unroll
-                    for (int e = 0; e < 8; e++) vf[PR][e] = 0.f;
+                    for (int e = 0; e < 8; e++) vf[PW][e] = 0.f;
                 }
 #pragma unroll
                 for (int g = 0; g < G; g++)
 #pragma unroll
                     for (int e = 0; e < 8; e++) acc[g][e] = FIRST ? 0.f : acc[g][e] * alpha[g];
 #pragma unroll
-                for (int i = 0; i <= PR; i++) {
+                for (int i = 0; i <= PW; i++) {
 #pragma unroll
                     for (int g = 0; g < G; g++) {
-                        const float p = (i < PR || sub == 0) ? pr[g][i] : 0.f;  // the new row: one row group only
+                        const float p = (i < PW || sub == 0) ? pr[g][i] : 0.f;  // the new row: one row group only
 #pragma unroll
                         for (int e = 0; e < 8; e++) acc[g][e] = fmaf(p, vf[i][e], acc[g][e]);
                     }
                 }
             };
             // Rounds past the held ones (XR > 0: caches longer than the registers hold) are streamed inside
-            // the phase through a ring of XD sets of PR rounds: one is multiplied while XD - 1 are in flight
+            // the phase through a ring of XD sets of PX rounds: one is multiplied while XD - 1 are in flight
             // (they take the registers of the held rounds, which are dead by then). A request past the split's
             // last round reads a valid row that nobody uses (kv_off), so the requests need no conditions.
             constexpr int XD = 3;
             int npx = 0;
             if constexpr (GE::XR > 0) {
                 const int over = sp.cached - NR * NCW * RPI;
-                npx = over > 0 ? (over + PR * NCW * RPI - 1) / (PR * NCW * RPI) : 0;
+                npx = over > 0 ? (over + PX * NCW * RPI - 1) / (PX * NCW * RPI) : 0;
             }
-            u32x4 kx[XD][PR], vx[XD][PR];
-            auto load_x = [&](u32x4 (&kxs)[PR], u32x4 (&vxs)[PR], const int r0) __attribute__((always_inline)) {
+            u32x4 kx[XD][PX], vx[XD][PX];
+            auto load_x = [&](u32x4 (&kxs)[PX], u32x4 (&vxs)[PX], const int r0) __attribute__((always_inline)) {
                 const uint16_t *kc = sm.lp[l].kcache, *vc = sm.lp[l].vcache;
 #pragma unroll
-                for (int i = 0; i < PR; i++) {
+                for (int i = 0; i < PX; i++) {
                     const size_t off = kv_off(r0 + i);
                     kxs[i] = ld128_global_stream(kc + off);
                     vxs[i] = ld128_global_stream(vc + off);
@@ -1165,19 +1170,19 @@ __device__ __forceinline__ void compute_role(const FusedDecodeArgs &a, Lds<GE> &
                 if constexpr (GE::XR > 0) {
                     if (ps == NPASS - 1 && npx > 0) {
 #pragma unroll
-                        for (int j = 0; j < XD - 1; j++) load_x(kx[j], vx[j], NR + j * PR);
+                        for (int j = 0; j < XD - 1; j++) load_x(kx[j], vx[j], NR + j * PX);
                     }
                 }
-                if (ps == 0) attn_pass(std::true_type{}, kk, vv, i0, last);
-                else attn_pass(std::false_type{}, kk, vv, i0, last);
+                if (ps == 0) attn_pass(std::true_type{}, std::integral_constant<int, PR>{}, kk, vv, i0, last);
+                else attn_pass(std::false_type{}, std::integral_constant<int, PR>{}, kk, vv, i0, last);
             }
             if constexpr (GE::XR > 0) {
                 // set x + j sits in ring slot j; the request that refills the slot freed last goes out first
                 auto ring_step = [&](auto self, auto jc, const int x) __attribute__((always_inline)) -> void {
                     constexpr int j = decltype(jc)::value;
-                    load_x(kx[(j + XD - 1) % XD], vx[(j + XD - 1) % XD], NR + (x + j + XD - 1) * PR);
-                    attn_pass(std::false_type{}, [&](int i) { return kx[j][i]; }, [&](int i) { return vx[j][i]; },
-                              NR + (x + j) * PR, x + j == npx - 1);
+                    load_x(kx[(j + XD - 1) % XD], vx[(j + XD - 1) % XD], NR + (x + j + XD - 1) * PX);
+                    attn_pass(std::false_type{}, std::integral_constant<int, PX>{}, [&](int i) { return kx[j][i]; }, [&](int i) { return vx[j][i]; },
+                              NR + (x + j) * PX, x + j == npx - 1);
                     if constexpr (j + 1 < XD) {
                         if (x + j + 1 < npx) self(self, std::integral_constant<int, j + 1>{}, x);
                     }
@@ -1850,6 +1855,11 @@ using GeoSmallQ = Geo<1024, 8, 4, 128, 1024, 64>;
 using GeoQwen3_0p6bShort = Geo<1024, 16, 8, 128, 3072, 256, 3>;
 using GeoSmallShort = Geo<512, 4, 2, 128, 1024, 64, 3>;
 using GeoSmallQShort = Geo<1024, 8, 4, 128, 1024, 64, 3>;
+// Six row rounds (3072 live rows): three attention passes instead of the four of the eight-round instances, and a
+// quarter fewer cache rows to ask for (Qwen3-0.6B, bf16: 0.453 against 0.468 ms a token at 2100 rows).
+using GeoQwen3_0p6bMid = Geo<1024, 16, 8, 128, 3072, 256, 6>;
+using GeoSmallMid = Geo<512, 4, 2, 128, 1024, 64, 6>;
+using GeoSmallQMid = Geo<1024, 8, 4, 128, 1024, 64, 6>;
 // The same shapes with eight row rounds: twice the live cache rows (4096) for 32 more registers a lane and an
 // attention phase twice as long; taken only by steps that the four-round instances do not serve.
 using GeoQwen3_0p6bLong = Geo<1024, 16, 8, 128, 3072, 256, 8>;
@@ -1887,12 +1897,15 @@ const Instance *find_instance(const FusedShape &s, int live_rows = 1) {
     static const Instance table[] = {
         instance<GeoQwen3_0p6bShort, FUSED_WF_K8>(), instance<GeoSmallQShort, FUSED_WF_K8>(),
         instance<GeoQwen3_0p6b, FUSED_WF_K8>(), instance<GeoSmallQ, FUSED_WF_K8>(),
+        instance<GeoQwen3_0p6bMid, FUSED_WF_K8>(), instance<GeoSmallQMid, FUSED_WF_K8>(),
         instance<GeoQwen3_0p6bLong, FUSED_WF_K8>(), instance<GeoSmallQLong, FUSED_WF_K8>(),
         instance<GeoQwen3_0p6bStream, FUSED_WF_K8>(), instance<GeoSmallQStream, FUSED_WF_K8>(),
         instance<GeoQwen3_0p6bShort, FUSED_WF_BF16>(), instance<GeoQwen3_0p6bShort, FUSED_WF_Q8_0>(), instance<GeoQwen3_0p6bShort, FUSED_WF_Q4_0>(),
         instance<GeoSmallShort, FUSED_WF_BF16>(),      instance<GeoSmallQShort, FUSED_WF_Q8_0>(),     instance<GeoSmallQShort, FUSED_WF_Q4_0>(),
         instance<GeoQwen3_0p6b, FUSED_WF_BF16>(), instance<GeoQwen3_0p6b, FUSED_WF_Q8_0>(), instance<GeoQwen3_0p6b, FUSED_WF_Q4_0>(),
         instance<GeoSmall, FUSED_WF_BF16>(),      instance<GeoSmallQ, FUSED_WF_Q8_0>(),     instance<GeoSmallQ, FUSED_WF_Q4_0>(),
+        instance<GeoQwen3_0p6bMid, FUSED_WF_BF16>(), instance<GeoQwen3_0p6bMid, FUSED_WF_Q8_0>(), instance<GeoQwen3_0p6bMid, FUSED_WF_Q4_0>(),
+        instance<GeoSmallMid, FUSED_WF_BF16>(),      instance<GeoSmallQMid, FUSED_WF_Q8_0>(),     instance<GeoSmallQMid, FUSED_WF_Q4_0>(),
         instance<GeoQwen3_0p6bLong, FUSED_WF_BF16>(), instance<GeoQwen3_0p6bLong, FUSED_WF_Q8_0>(), instance<GeoQwen3_0p6bLong, FUSED_WF_Q4_0>(),
         instance<GeoSmallLong, FUSED_WF_BF16>(),      instance<GeoSmallQLong, FUSED_WF_Q8_0>(),     instance<GeoSmallQLong, FUSED_WF_Q4_0>(),
         instance<GeoQwen3_0p6bStream, FUSED_WF_BF16>(), instance<GeoQwen3_0p6bStream, FUSED_WF_Q8_0>(), instance<GeoQwen3_0p6bStream, FUSED_WF_Q4_0>(),

@@ -379,7 +379,7 @@ int hm_model_set_graph(hm_model *m, int on);
  * (src/hf/emitter.rs:1016-1021). Served for bf16, all-Q8_0, all-Q4_0 and Q4_K / Q6_K (in any mix per
  * projection) models whose shape has a kernel instance (hm_model_whole_step_available); on by default then, and for bf16 models the same launch runs the
  * LM head and the greedy pick. The cache may be of any length: a step takes the instance of the kernel that
- * holds its live rows (1536, 2048, 4096 or 32768 of them; the smaller the faster; the last streams the rows beyond
+ * holds its live rows (1536, 2048, 3072, 4096 or 32768 of them; the smaller the faster; the last streams the rows beyond
  * 4096 inside its attention phase), beyond 32768 the per-projection path, chosen step by step. Results agree with the per-projection
  * path to f32 summation order.
  *

@@ -308,8 +308,8 @@ def test_rows_streamed_inside_the_attention_phase(long_small, rows):
 
 def test_cache_longer_than_the_kernel_serves_changes_over_and_back(ctx):
     """The whole-step launch holds a split's cache rows in registers: an instance with three row rounds serves
-    1536 live rows of this shape, one with four 2048, one with eight 4096 and, streaming further rounds inside
-    its attention phase, 32768. A model with a longer cache starts on the first, takes the next from the step
+    1536 live rows of this shape, one with four 2048, one with six 3072, one with eight 4096 and, streaming further
+    rounds inside its attention phase, 32768. A model with a longer cache starts on the first, takes the next from the step
     whose live rows exceed it, one launch per projection beyond 32768, and comes back after a cache reset; the
     steps on either side of each change give the oracle's logits and the per-projection path's tokens."""
     cfg = dataclasses.replace(synth_model.SMALL_WS, max_position_embeddings=65536)
@@ -321,7 +321,7 @@ def test_cache_longer_than_the_kernel_serves_changes_over_and_back(ctx):
     om = mf.build_oracle_model(cfg, weights, L)
     assert gm.whole_step_available() and gm.whole_step() and gm.launches_per_step() == 1
     ids = synth.token_ids(33, 14, cfg.vocab_size)
-    for rows, still_whole in ((1528, True), (2040, True), (4088, True), (32760, False)):
+    for rows, still_whole in ((1528, True), (2040, True), (3064, True), (4088, True), (32760, False)):
         kv = synth_model.synth_kv(cfg, 32 + rows, rows)
         for m in (gm, plain):
             m.set_prefill_min(0)
