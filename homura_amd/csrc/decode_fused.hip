@@ -951,11 +951,15 @@ __device__ __forceinline__ void compute_role(const FusedDecodeArgs &a, Lds<GE> &
     // (The K-quant form asks for half the bytes and was 2-3 % faster with the earlier lots: it keeps them.)
     constexpr bool K8_LOTS = WF == FUSED_WF_K8;
     constexpr int KV_CUT = NR / 2, WG_CUT = K8_LOTS ? 2 * GE::RGW / 3 : GE::RGW / 2;
-    // With more than four row rounds in registers a layer's slices and the next layer's cache rows do not
-    // all fit at once (a spilled value would come back through the memory pipeline, behind every outstanding
-    // weight request): those instances request the second half of the cache rows and the Q|K|V rows one phase
-    // later, when the registers they land in have just been read for the last time.
-    constexpr bool LATE = NR > 4;
+    // With eight row rounds in registers a layer's slices and the next layer's cache rows do not all fit at once
+    // (a spilled value would come back through the memory pipeline, behind every outstanding weight request): those
+    // instances request the second half of the cache rows and a quarter of the Q|K|V rows one phase later, when the
+    // registers they land in have just been read for the last time. (All Q|K|V rows at the start of the attention
+    // phase spill 20 to 192 bytes a lane in three of the eight instances; none of them there, as it was first
+    // built, costs 0.489 -> 0.507 ms a token at 4000 rows. Six rounds fit without any of this: 0.447 -> 0.421 ms
+    // at 2100 rows.)
+    constexpr bool LATE = NR > 6;
+    constexpr int WQ_EARLY = LATE ? 3 * GE::RQW / 4 : GE::RQW;  // Q|K|V rows of the next layer asked for at the start of the attention phase
     // Their cache rows go out in four lots so that no phase start asks for much more than the CU keeps in flight
     // (a wavefront that asks for more waits, with its phase's arithmetic behind it): the first rounds at the end of
     // the attention phase, the rest of the first half with the O phase, the second half with gate|up and down.
@@ -1004,7 +1008,7 @@ __device__ __forceinline__ void compute_role(const FusedDecodeArgs &a, Lds<GE> &
         //    Every wavefront leaves the (max, sum, P.V) of its own rows in LDS; the publishing threads
         //    merge the four. ──
         wg_barrier();
-        if (!LATE) load_wq(nx, 0, GE::RQW);
+        load_wq(nx, 0, WQ_EARLY);
         if (sp.split < sp.nsl) {
             float qv[G][8];
 #pragma unroll
@@ -1196,7 +1200,7 @@ __device__ __forceinline__ void compute_role(const FusedDecodeArgs &a, Lds<GE> &
                 *reinterpret_cast<f32x4 *>(dst + 4) = f32x4{acc[g][4], acc[g][5], acc[g][6], acc[g][7]};
             }
         }
-        if (LATE) load_wq(nx, 0, GE::RQW);  // behind the arithmetic that needed the registers
+        load_wq(nx, WQ_EARLY, GE::RQW);  // behind the arithmetic that needed the registers
         if (LATE) load_kv(nx, 0, LATE_KV_P2);
         wg_barrier();
 
